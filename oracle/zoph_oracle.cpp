@@ -1,0 +1,666 @@
+// CPU restatement of the Zoph_RNN stacked-LSTM forward path.
+//
+// THIS FILE IS TEST INFRASTRUCTURE.  It is the checker the HIP path is compared
+// with (tests, the smoke check, and the bench's cpu_baseline leg); nothing that
+// ships may call it.  It restates, on host arrays, the arithmetic of the
+// reference's forward kernels and cuBLAS call sites, citing the reference
+// file:line each function follows.  All matrices are column-major
+// (IDX2C, src/BZ_CUDA_UTIL.h:26); activations are H x minibatch.
+//
+// What pins each function (see tests/test_oracle_*.py): closed forms and
+// brute-force restatements in numpy float64, invariants (column sums, shift
+// invariance, linearity), and special cases that reduce to a textbook
+// routine.  The reference holds no golden vectors for this path and its
+// contractions run inside cuBLAS (summation order unknown), so no function
+// here is pinned by a reference-held vector: parity with the *reference* is
+// therefore "pinned by mathematics only" for every function in this file.
+//
+// Build: see oracle/Makefile (g++ -O2 -fopenmp -shared -fPIC).
+
+#include <algorithm>
+#include <cfloat>
+#include <cmath>
+#include <cstdint>
+#include <cstdlib>
+#include <cstring>
+#include <queue>
+#include <vector>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define IDX2C(i, j, ld) ((size_t)(j) * (size_t)(ld) + (size_t)(i))
+
+namespace {
+
+// ---------------------------------------------------------------------------
+// Contractions.  The reference calls cublasSgemm (src/BZ_CUDA_UTIL.h:691-696)
+// with alpha=1, beta=0.  acc64=1 accumulates in double and rounds once (the
+// "exact" value any fp32 summation order must be close to); acc64=0
+// accumulates in float (the timed CPU baseline).
+// ---------------------------------------------------------------------------
+template <typename Acc>
+void gemm_nn_t(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc) {
+  const int MB = 256, NB = 4;
+  const int nmb = (M + MB - 1) / MB;
+#pragma omp parallel for schedule(static)
+  for (int mb = 0; mb < nmb; ++mb) {
+    const int m0 = mb * MB;
+    const int mlen = std::min(MB, M - m0);
+    Acc acc[NB][MB];
+    for (int n0 = 0; n0 < N; n0 += NB) {
+      const int nlen = std::min(NB, N - n0);
+      for (int q = 0; q < nlen; ++q)
+        for (int i = 0; i < mlen; ++i) acc[q][i] = 0;
+      for (int k = 0; k < K; ++k) {
+        const float* a = A + IDX2C(m0, k, lda);
+        for (int q = 0; q < nlen; ++q) {
+          const Acc b = (Acc)B[IDX2C(k, n0 + q, ldb)];
+          Acc* ac = acc[q];
+          for (int i = 0; i < mlen; ++i) ac[i] += (Acc)a[i] * b;
+        }
+      }
+      for (int q = 0; q < nlen; ++q)
+        for (int i = 0; i < mlen; ++i) C[IDX2C(m0 + i, n0 + q, ldc)] = (float)acc[q][i];
+    }
+  }
+}
+
+// C(MxN) = A^T * B with A stored K x M (lda >= K): CUBLAS_OP_T on the first operand
+// (src/attention_node.hpp:195).
+template <typename Acc>
+void gemm_tn_t(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc) {
+#pragma omp parallel for schedule(static) collapse(2)
+  for (int n = 0; n < N; ++n)
+    for (int m = 0; m < M; ++m) {
+      const float* a = A + IDX2C(0, m, lda);
+      const float* b = B + IDX2C(0, n, ldb);
+      Acc s = 0;
+      for (int k = 0; k < K; ++k) s += (Acc)a[k] * (Acc)b[k];
+      C[IDX2C(m, n, ldc)] = (float)s;
+    }
+}
+
+void gemm_nn(int acc64, int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc) {
+  if (acc64)
+    gemm_nn_t<double>(M, N, K, A, lda, B, ldb, C, ldc);
+  else
+    gemm_nn_t<float>(M, N, K, A, lda, B, ldb, C, ldc);
+}
+void gemm_tn(int acc64, int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc) {
+  if (acc64)
+    gemm_tn_t<double>(M, N, K, A, lda, B, ldb, C, ldc);
+  else
+    gemm_tn_t<float>(M, N, K, A, lda, B, ldb, C, ldc);
+}
+
+// forward_sigmoid_kernel (float overload), src/custom_kernels.h:58-65.
+inline float sigmoid_f32(float v) { return 1.0f / (1.0f + expf(-1.0f * v)); }
+// forward_sigmoid_kernel_feed, src/custom_kernels.h:92-99: the literals are double, so the
+// expression is evaluated in double and rounded to float on the store.
+inline float sigmoid_via_f64(float v) { return (float)(1.0 / (1.0 + exp(-1.0 * (double)v))); }
+
+}  // namespace
+
+extern "C" {
+
+int orc_num_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
+
+void orc_set_num_threads(int n) {
+#ifdef _OPENMP
+  omp_set_num_threads(n);
+#else
+  (void)n;
+#endif
+}
+
+// vocab_to_01 + vocab_to_nonM1, src/custom_kernels.h:10-32, launched from
+// Input_To_Hidden_Layer::prep_GPU_vocab_indices (src/Input_To_Hidden_Layer.hpp:1199-1202).
+void orc_vocab_prep(const int* ids, int n, int* ids_nonneg, int* mask01) {
+  for (int i = 0; i < n; ++i) {
+    mask01[i] = (ids[i] == -1) ? 0 : 1;
+    ids_nonneg[i] = (ids[i] == -1) ? 0 : ids[i];
+  }
+}
+
+// vocab_softmax, src/custom_kernels.h:38-50 (in place on the ids, int and float masks).
+void orc_vocab_softmax(int* ids, int n, int* mask01, float* mask01f) {
+  for (int i = 0; i < n; ++i) {
+    if (ids[i] == -1) {
+      ids[i] = 0;
+      mask01[i] = 0;
+      mask01f[i] = 0.f;
+    } else {
+      mask01[i] = 1;
+      mask01f[i] = 1.f;
+    }
+  }
+}
+
+// sparse_lookup_kernel, src/custom_kernels.h:342-348: x[:,b] = W[:,ids[b]].
+void orc_embed_gather(const float* W, int H, int V, const int* ids, int mb, float* x) {
+  (void)V;
+  for (int b = 0; b < mb; ++b) memcpy(x + IDX2C(0, b, H), W + IDX2C(0, ids[b], H), sizeof(float) * (size_t)H);
+}
+
+void orc_gemm_nn(int acc64, int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc) {
+  gemm_nn(acc64, M, N, K, A, lda, B, ldb, C, ldc);
+}
+void orc_gemm_tn(int acc64, int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc) {
+  gemm_tn(acc64, M, N, K, A, lda, B, ldb, C, ldc);
+}
+
+// One LSTM node forward step.  LSTM_IH_Node::forward_prop_GPU (src/LSTM.hpp:76-421) and
+// LSTM_HH_Node::forward_prop_GPU (src/LSTM_HH.hpp:103-333).  Gate order i,f,c,o.
+//   M[g], Wh[g], Q[g]: H x H; b[g]: H; x, hprev, cprev, htild: H x mb; mask01: mb.
+//   Q == NULL or htild == NULL: the non-feed kernels (float sigmoid); else the *_feed kernels
+//   (third addend, sigmoid evaluated in double; src/LSTM.hpp:175-182).
+//   Outputs (each H x mb): gate_i, gate_f, gate_c (tanh), gate_o, c, h.  Any gate pointer may be NULL.
+void orc_lstm_step(int acc64, int H, int mb, const float* const* M, const float* const* Wh, const float* const* Q,
+                   const float* const* b, const float* x, const float* hprev, const float* cprev,
+                   const float* htild, const int* mask01, int clip_cell, float clip_threshold, float* gate_i,
+                   float* gate_f, float* gate_c, float* gate_o, float* c, float* h) {
+  const bool feed = (Q != nullptr && htild != nullptr);
+  const size_t n = (size_t)H * mb;
+  std::vector<float> t1(n), t2(n), t3(feed ? n : 0);
+  std::vector<float> gates[4];
+  for (int g = 0; g < 4; ++g) {
+    gates[g].resize(n);
+    // temp{1,3,5,7} = M_g x ; temp{2,4,6,8} = W_hg h_prev ; temp{9..12} = Q_g htild
+    gemm_nn(acc64, H, mb, H, M[g], H, x, H, t1.data(), H);
+    gemm_nn(acc64, H, mb, H, Wh[g], H, hprev, H, t2.data(), H);
+    if (feed) gemm_nn(acc64, H, mb, H, Q[g], H, htild, H, t3.data(), H);
+    for (int col = 0; col < mb; ++col)
+      for (int i = 0; i < H; ++i) {
+        const size_t ix = IDX2C(i, col, H);
+        float v;
+        if (feed)
+          v = t1[ix] + t2[ix] + t3[ix] + b[g][i];  // custom_kernels.h:96,132
+        else
+          v = t1[ix] + t2[ix] + b[g][i];  // custom_kernels.h:62,110
+        if (g == 2)
+          gates[g][ix] = tanhf(v);  // forward_tanh_kernel(_feed), custom_kernels.h:106-135
+        else
+          gates[g][ix] = feed ? sigmoid_via_f64(v) : sigmoid_f32(v);
+      }
+  }
+  for (int col = 0; col < mb; ++col)
+    for (int i = 0; i < H; ++i) {
+      const size_t ix = IDX2C(i, col, H);
+      // forward_c_t_kernel, custom_kernels.h:141-147
+      float cv = gates[1][ix] * cprev[ix] + gates[0][ix] * gates[2][ix];
+      if (clip_cell) {  // clip_mat_kernel, custom_kernels.h:2222-2231 (BZ_CUDA::clip_cell, src/LSTM.hpp:369-371)
+        if (cv > 0)
+          cv = (cv > clip_threshold) ? clip_threshold : cv;
+        else
+          cv = (cv < -clip_threshold) ? -clip_threshold : cv;
+      }
+      // forward_h_t_kernel, custom_kernels.h:162-168
+      float hv = gates[3][ix] * tanhf(cv);
+      // zero_c_t_and_h_t, custom_kernels.h:184-192
+      hv = hv * mask01[col];
+      cv = cv * mask01[col];
+      c[ix] = cv;
+      h[ix] = hv;
+    }
+  float* outs[4] = {gate_i, gate_f, gate_c, gate_o};
+  for (int g = 0; g < 4; ++g)
+    if (outs[g]) memcpy(outs[g], gates[g].data(), n * sizeof(float));
+}
+
+// Logits: D h + b_d.  cublasSgemm + matrix_bias_kernel (src/softmax.hpp:539-547, custom_kernels.h:787-794).
+void orc_softmax_logits(int acc64, const float* D, const float* b_d, int V, int H, const float* h, int mb,
+                        float* logits) {
+  gemm_nn(acc64, V, mb, H, D, V, h, H, logits, V);
+  for (int col = 0; col < mb; ++col)
+    for (int v = 0; v < V; ++v) logits[IDX2C(v, col, V)] = logits[IDX2C(v, col, V)] + b_d[v];
+}
+
+// outputdist_overflow_prevention_kernel, src/custom_kernels.h:503-577: per column, max, expf(x-max),
+// sum, divide.  emulate_tree=1 reproduces the kernel's summation order (256 strided partial sums, then a
+// binary tree, SOFTMAX_THREADS=256); emulate_tree=0 sums in double (the order-free value).
+void orc_softmax_dist(const float* logits, int V, int mb, int emulate_tree, float* prob) {
+  const int T = 256;
+#pragma omp parallel for schedule(static)
+  for (int col = 0; col < mb; ++col) {
+    const float* in = logits + IDX2C(0, col, V);
+    float* out = prob + IDX2C(0, col, V);
+    float mx = -FLT_MAX;
+    for (int v = 0; v < V; ++v)
+      if (mx < in[v]) mx = in[v];
+    if (emulate_tree) {
+      float buf[T];
+      for (int t = 0; t < T; ++t) buf[t] = 0.f;
+      for (int v = 0; v < V; ++v) {
+        const float z = expf(in[v] - mx);
+        buf[v % T] += z;
+        out[v] = z;
+      }
+      for (int stride = T / 2; stride > 0; stride >>= 1)
+        for (int t = 0; t < stride; ++t) buf[t] += buf[t + stride];
+      const float sum = buf[0];
+      for (int v = 0; v < V; ++v) out[v] = out[v] / sum;
+    } else {
+      double sum = 0;
+      for (int v = 0; v < V; ++v) {
+        const float z = expf(in[v] - mx);
+        out[v] = z;
+        sum += (double)z;
+      }
+      const float sumf = (float)sum;
+      for (int v = 0; v < V; ++v) out[v] = out[v] / sumf;
+    }
+  }
+}
+
+// outputdist_perplexity_kernel, src/custom_kernels.h:583-660: double log-probabilities,
+// log(exp(x-max)) - log(sum) per column.
+void orc_softmax_logprob_f64(const float* logits, int V, int mb, double* logp) {
+#pragma omp parallel for schedule(static)
+  for (int col = 0; col < mb; ++col) {
+    const float* in = logits + IDX2C(0, col, V);
+    double* out = logp + IDX2C(0, col, V);
+    double mx = -DBL_MAX;
+    for (int v = 0; v < V; ++v)
+      if (mx < (double)in[v]) mx = (double)in[v];
+    double sum = 0;
+    for (int v = 0; v < V; ++v) {
+      const double z = exp((double)in[v] - mx);
+      sum += z;
+      out[v] = z;
+    }
+    const double ls = log(sum);
+    for (int v = 0; v < V; ++v) out[v] = log(out[v]) - ls;
+  }
+}
+
+// softmax_layer::compute_loss_GPU, src/softmax.hpp:867-900: sum over unmasked columns of
+// logp[target[b], b].
+double orc_softmax_loss(const double* logp, int V, int mb, const int* target, const int* mask01) {
+  double loss = 0;
+  for (int b = 0; b < mb; ++b)
+    if (mask01[b] == 1) loss += logp[IDX2C(target[b], b, V)];
+  return loss;
+}
+
+// attention_node::forward_prop, src/attention_node.hpp:73-394 (single-source branch), with the kernels it
+// launches: tanh_kernel (custom_kernels.h:1567), sigmoid_kernel (:1583, double), alignment_pos_kernel (:1598),
+// lower_upper_kernel (:1608), create_indicies_kernel (:1650), load_in_hs_kernel (:1694),
+// elem_reduce_kernel_large (:1892), alignment_reduction_kernel (:1752), create_c_t_kernel (:1804),
+// tanh_att_forward_kernel (:1844), zero_h_t (:2212).
+//   hs_table: the longest_sent source-side top-layer states, table t at hs_table + t*H*mb
+//             (the reference keeps a pointer table d_total_hs_mat, src/attention_layer.hpp:106-160).
+//   batch_info: [0,mb) true source lengths S_b, [mb,2mb) left-pad offsets (src/fileHelper.h:499-500).
+//   outputs: h_tild H x mb; alignments and indices (2D+1) x mb laid out [b + mb*j]; p_t mb; c_ctx H x mb.
+void orc_attention_forward(int acc64, int H, int mb, int D, const float* W_a, const float* W_p, const float* v_p,
+                           const float* out_bias, const float* W_c1, const float* W_c2, const float* hs_table,
+                           const int* batch_info, const float* h_t, const int* mask01, float* h_tild,
+                           float* alignments, int* indices, float* p_t, float* c_ctx) {
+  const int W = 2 * D + 1;
+  const size_t n = (size_t)H * mb;
+  std::vector<float> tanh1(n), sigma1(mb), q(n), f1(n), f2(n);
+  std::vector<int> lower_upper(2 * (size_t)mb);
+  const float sigma_sq = (float)((D * D) / 4.0);  // attention_node.hpp:50
+
+  gemm_nn(acc64, H, mb, H, W_p, H, h_t, H, tanh1.data(), H);        // :132
+  for (size_t i = 0; i < n; ++i) tanh1[i] = tanhf(tanh1[i]);        // :141
+  gemm_nn(acc64, 1, mb, H, v_p, 1, tanh1.data(), H, sigma1.data(), 1);  // :147
+  for (int b = 0; b < mb; ++b) {
+    sigma1[b] = (float)(1.0 / (1.0 + exp(-1.0 * (double)sigma1[b])));  // sigmoid_kernel, double literals
+    p_t[b] = batch_info[b] * sigma1[b];                                // alignment_pos_kernel
+    const int ip = (int)p_t[b];
+    lower_upper[IDX2C(0, b, 2)] = (0 > ip - D) ? 0 : (ip - D);
+    lower_upper[IDX2C(1, b, 2)] = ((batch_info[b] - 1) < ip + D) ? (batch_info[b] - 1) : (ip + D);
+  }
+  for (int b = 0; b < mb; ++b) {  // create_indicies_kernel
+    int cur = lower_upper[IDX2C(0, b, 2)];
+    const int mx = lower_upper[IDX2C(1, b, 2)];
+    for (int j = 0; j < W; ++j) {
+      if (mask01[b] == 1) {
+        indices[IDX2C(b, j, mb)] = (cur > mx) ? -1 : cur;
+        cur++;
+      } else {
+        indices[IDX2C(b, j, mb)] = -1;
+      }
+    }
+  }
+  gemm_tn(acc64, H, mb, H, W_a, H, h_t, H, q.data(), H);  // :195, W_a^T h
+  // load_in_hs_kernel + elem_reduce_kernel_large: score over the gathered (or zero) source column.
+  auto hs_col = [&](int b, int j) -> const float* {
+    const int s = indices[IDX2C(b, j, mb)];
+    if (s == -1) return nullptr;
+    const int t = batch_info[b] - 1 - s + batch_info[mb + b];
+    return hs_table + (size_t)t * n + IDX2C(0, b, H);
+  };
+#pragma omp parallel for schedule(static)
+  for (int b = 0; b < mb; ++b)
+    for (int j = 0; j < W; ++j) {
+      const float* hs = hs_col(b, j);
+      if (acc64) {
+        double s = 0;
+        if (hs)
+          for (int k = 0; k < H; ++k) s += (double)hs[k] * (double)q[IDX2C(k, b, H)];
+        alignments[IDX2C(b, j, mb)] = (float)s;
+      } else {
+        float s = 0;
+        if (hs)
+          for (int k = 0; k < H; ++k) s += hs[k] * q[IDX2C(k, b, H)];
+        alignments[IDX2C(b, j, mb)] = s;
+      }
+    }
+  // alignment_reduction_kernel: note max_val starts at 0, not -inf.
+  for (int b = 0; b < mb; ++b) {
+    float sum = 0, max_val = 0;
+    for (int j = 0; j < W; ++j)
+      if (indices[IDX2C(b, j, mb)] != -1)
+        if (alignments[IDX2C(b, j, mb)] > max_val) max_val = alignments[IDX2C(b, j, mb)];
+    for (int j = 0; j < W; ++j) {
+      if (indices[IDX2C(b, j, mb)] != -1) {
+        alignments[IDX2C(b, j, mb)] = expf(alignments[IDX2C(b, j, mb)] - max_val);
+        sum += alignments[IDX2C(b, j, mb)];
+      } else {
+        alignments[IDX2C(b, j, mb)] = 0;
+      }
+    }
+    for (int j = 0; j < W; ++j) {
+      if (indices[IDX2C(b, j, mb)] != -1) {
+        const float d = p_t[b] - indices[IDX2C(b, j, mb)];
+        const float temp = expf((-1 * powf(d, 2.0f)) / (2 * sigma_sq));
+        if (sum != 0) alignments[IDX2C(b, j, mb)] = (alignments[IDX2C(b, j, mb)] / sum) * temp;
+      } else {
+        alignments[IDX2C(b, j, mb)] = 0;
+      }
+    }
+  }
+  // create_c_t_kernel: c[:,b] = sum_j a[b + mb*j] * hs[:, b + mb*j]
+#pragma omp parallel for schedule(static)
+  for (int b = 0; b < mb; ++b) {
+    for (int i = 0; i < H; ++i) c_ctx[IDX2C(i, b, H)] = 0;
+    for (int j = 0; j < W; ++j) {
+      const float* hs = hs_col(b, j);
+      if (!hs) continue;  // the gathered column is zero
+      const float a = alignments[IDX2C(b, j, mb)];
+      for (int i = 0; i < H; ++i) c_ctx[IDX2C(i, b, H)] += a * hs[i];
+    }
+  }
+  gemm_nn(acc64, H, mb, H, W_c1, H, c_ctx, H, f1.data(), H);  // :354
+  gemm_nn(acc64, H, mb, H, W_c2, H, h_t, H, f2.data(), H);    // :360
+  for (int b = 0; b < mb; ++b)
+    for (int i = 0; i < H; ++i) {
+      const size_t ix = IDX2C(i, b, H);
+      float v = tanhf(f1[ix] + f2[ix] + out_bias[i]);  // tanh_att_forward_kernel
+      v *= mask01[b];                                   // zero_h_t
+      h_tild[ix] = v;
+    }
+}
+
+// Column gather used by the decoder state shuffles: dst[:,i] = src[:,perm[i]]
+// (Input_To_Hidden_Layer::swap_states_decoding, src/Input_To_Hidden_Layer.hpp:1231-1242).
+void orc_gather_columns(const float* src, int H, const int* perm, int n, float* dst) {
+  for (int i = 0; i < n; ++i) memcpy(dst + IDX2C(0, i, H), src + IDX2C(0, perm[i], H), sizeof(float) * (size_t)H);
+}
+
+// transfer_decoding_states_GPU (src/Input_To_Hidden_Layer.hpp:1252-1266): broadcast one column to n columns.
+void orc_broadcast_column(const float* src_col, int H, int n, float* dst) {
+  for (int i = 0; i < n; ++i) memcpy(dst + IDX2C(0, i, H), src_col, sizeof(float) * (size_t)H);
+}
+
+}  // extern "C"
+
+// ---------------------------------------------------------------------------
+// Beam search.  decoder<dType> (src/decoder.h:162-1502), non-FSA path:
+// init_decoder (:1317-1355), expand_hypothesis_without_fsa (:1158-1315),
+// finish_current_hypotheses (:672-688), output_k_best_hypotheses (:1386-1413).
+// The two heaps are std::priority_queue with the reference's comparators
+// (pq_compare_functor / pq_global_compare_functor, :146-154) and the same
+// push order, so tie behaviour follows libstdc++ exactly as in the reference.
+// ---------------------------------------------------------------------------
+namespace {
+
+struct DecObj {
+  float val;
+  int vocab_index;
+};
+struct DecGlobalObj {
+  float val;
+  int beam_index;
+  int vocab_index;
+};
+struct PqCmp {
+  bool operator()(const DecObj& a, const DecObj& b) const { return a.val < b.val; }
+};
+struct PqGlobalCmp {
+  bool operator()(const DecGlobalObj& a, const DecGlobalObj& b) const { return a.val < b.val; }
+};
+struct Hypothesis {
+  std::vector<int> words;
+  float score;
+};
+
+struct OrcDecoder {
+  int beam, vocab, start_symbol, end_symbol, max_len;
+  float penalty, min_ratio;
+  int current_index;
+  std::vector<int> current_indices, new_indicies_changes;
+  std::vector<int> top_sentences, top_sentences_temp;  // beam x max_len, row-major here
+  std::vector<float> scores, scores_temp;
+  std::vector<Hypothesis> hypotheses;
+  std::priority_queue<DecObj, std::vector<DecObj>, PqCmp> pq;
+  std::priority_queue<DecGlobalObj, std::vector<DecGlobalObj>, PqGlobalCmp> pq_global;
+};
+
+}  // namespace
+
+extern "C" {
+
+void* orc_decoder_create(int beam, int vocab, int start_symbol, int end_symbol, int max_len, float min_ratio,
+                         float penalty) {
+  OrcDecoder* d = new OrcDecoder();
+  d->beam = beam;
+  d->vocab = vocab;
+  d->start_symbol = start_symbol;
+  d->end_symbol = end_symbol;
+  d->max_len = max_len;
+  d->min_ratio = min_ratio;
+  d->penalty = penalty;
+  d->current_indices.resize(beam);
+  d->new_indicies_changes.assign(beam, 0);
+  d->top_sentences.resize((size_t)beam * max_len);
+  d->top_sentences_temp.resize((size_t)beam * max_len);
+  d->scores.resize(beam);
+  d->scores_temp.resize(beam);
+  d->current_index = 0;
+  return d;
+}
+
+void orc_decoder_destroy(void* p) { delete (OrcDecoder*)p; }
+
+// init_decoder, src/decoder.h:1317-1355
+void orc_decoder_init(void* p) {
+  OrcDecoder* d = (OrcDecoder*)p;
+  d->current_index = 0;
+  std::fill(d->scores.begin(), d->scores.end(), 0.f);
+  d->hypotheses.clear();
+  for (int i = 0; i < d->beam; ++i) d->current_indices[i] = d->start_symbol;
+  std::fill(d->top_sentences.begin(), d->top_sentences.end(), d->start_symbol);
+}
+
+// expand_hypothesis_without_fsa, src/decoder.h:1158-1315.  outputdist: vocab x beam probabilities,
+// column-major (column = beam entry).
+void orc_decoder_expand(void* p, const float* outputdist, int index) {
+  OrcDecoder* d = (OrcDecoder*)p;
+  const int beam = d->beam, V = d->vocab, L = d->max_len;
+  int cols = beam;
+  if (index == 0) cols = 1;
+  while (!d->pq_global.empty()) d->pq_global.pop();
+  for (int i = 0; i < cols; ++i) {
+    while (!d->pq.empty()) d->pq.pop();
+    if (d->current_indices[i] == -1) break;
+    for (int j = 0; j < V; ++j) {
+      const float pr = outputdist[IDX2C(j, i, V)];
+      if ((int)d->pq.size() < beam + 1) {
+        d->pq.push(DecObj{-pr, j});
+      } else if (-pr < d->pq.top().val) {
+        d->pq.pop();
+        d->pq.push(DecObj{-pr, j});
+      }
+    }
+    while (!d->pq.empty()) {
+      DecObj t = d->pq.top();
+      d->pq.pop();
+      d->pq_global.push(DecGlobalObj{std::log(-t.val) + d->scores[i], i, t.vocab_index});
+    }
+  }
+  int i = 0;
+  while (i < beam) {
+    if (d->pq_global.empty()) {
+      for (int c = 0; c < L; ++c) d->top_sentences_temp[(size_t)i * L + c] = d->top_sentences[c];
+      d->top_sentences_temp[(size_t)i * L + d->current_index + 1] = d->start_symbol;
+      d->current_indices[i] = -1;
+      d->new_indicies_changes[i] = 0;
+      d->scores_temp[i] = 0;
+      i++;
+      continue;
+    }
+    DecGlobalObj t = d->pq_global.top();
+    d->pq_global.pop();
+    if (t.vocab_index != d->start_symbol) {
+      if (t.vocab_index == d->end_symbol) {
+        Hypothesis hy;
+        hy.words.assign(d->top_sentences.begin() + (size_t)t.beam_index * L,
+                        d->top_sentences.begin() + (size_t)t.beam_index * L + d->current_index + 2);
+        hy.words[d->current_index + 1] = d->end_symbol;
+        hy.score = t.val + d->penalty;
+        d->hypotheses.push_back(hy);
+      } else {
+        for (int c = 0; c < L; ++c)
+          d->top_sentences_temp[(size_t)i * L + c] = d->top_sentences[(size_t)t.beam_index * L + c];
+        d->top_sentences_temp[(size_t)i * L + d->current_index + 1] = t.vocab_index;
+        d->current_indices[i] = t.vocab_index;
+        d->new_indicies_changes[i] = t.beam_index;
+        d->scores_temp[i] = t.val + d->penalty;
+        i++;
+      }
+    }
+  }
+  d->top_sentences = d->top_sentences_temp;
+  d->scores = d->scores_temp;
+  d->current_index += 1;
+}
+
+// finish_current_hypotheses (non-FSA branch), src/decoder.h:672-688.
+void orc_decoder_finish(void* p, const float* outputdist) {
+  OrcDecoder* d = (OrcDecoder*)p;
+  const int L = d->max_len, V = d->vocab;
+  for (int i = 0; i < d->beam; ++i) {
+    if (d->current_indices[i] == -1) continue;
+    d->top_sentences[(size_t)i * L + d->current_index + 1] = d->end_symbol;
+    d->scores[i] += std::log(outputdist[IDX2C(1, i, V)]) + d->penalty;
+    Hypothesis hy;
+    hy.words.assign(d->top_sentences.begin() + (size_t)i * L,
+                    d->top_sentences.begin() + (size_t)i * L + d->current_index + 2);
+    hy.score = d->scores[i];
+    d->hypotheses.push_back(hy);
+  }
+  d->current_index += 1;
+}
+
+void orc_decoder_state(void* p, int* current_indices, int* new_indicies_changes, float* scores, int* top_sentences) {
+  OrcDecoder* d = (OrcDecoder*)p;
+  for (int i = 0; i < d->beam; ++i) {
+    if (current_indices) current_indices[i] = d->current_indices[i];
+    if (new_indicies_changes) new_indicies_changes[i] = d->new_indicies_changes[i];
+    if (scores) scores[i] = d->scores[i];
+  }
+  if (top_sentences) memcpy(top_sentences, d->top_sentences.data(), sizeof(int) * d->top_sentences.size());
+}
+
+int orc_decoder_current_index(void* p) { return ((OrcDecoder*)p)->current_index; }
+int orc_decoder_num_hypotheses(void* p) { return (int)((OrcDecoder*)p)->hypotheses.size(); }
+int orc_decoder_hypothesis(void* p, int i, int* words, int cap, float* score) {
+  OrcDecoder* d = (OrcDecoder*)p;
+  const Hypothesis& hy = d->hypotheses[i];
+  const int n = (int)hy.words.size();
+  for (int k = 0; k < n && k < cap; ++k) words[k] = hy.words[k];
+  *score = hy.score;
+  return n;
+}
+
+// output_k_best_hypotheses selection, src/decoder.h:1386-1413: indices (into the hypothesis list) of the
+// best num_hypotheses finished hypotheses with length/source_length > min_decoding_ratio, best first.
+int orc_decoder_k_best(void* p, int source_length, int num_hypotheses, int* out_idx) {
+  OrcDecoder* d = (OrcDecoder*)p;
+  struct KB {
+    float score;
+    float index;
+  };
+  struct KBCmp {
+    bool operator()(const KB& a, const KB& b) const { return a.score < b.score; }
+  };
+  std::priority_queue<KB, std::vector<KB>, KBCmp> best, best_temp;
+  for (size_t i = 0; i < d->hypotheses.size(); ++i) {
+    const float len_ratio = ((float)d->hypotheses[i].words.size()) / source_length;
+    if (len_ratio > d->min_ratio) {
+      if ((int)best.size() < num_hypotheses) {
+        best.push(KB{-d->hypotheses[i].score, (float)i});
+      } else if (-1 * best.top().score < d->hypotheses[i].score) {
+        best.pop();
+        best.push(KB{-d->hypotheses[i].score, (float)i});
+      }
+    }
+  }
+  while (!best.empty()) {
+    best_temp.push(KB{-1 * best.top().score, best.top().index});
+    best.pop();
+  }
+  int n = 0;
+  while (!best_temp.empty()) {
+    out_idx[n++] = (int)best_temp.top().index;
+    best_temp.pop();
+  }
+  return n;
+}
+
+// ---------------------------------------------------------------------------
+// Composite forward schedules (neuralMT_model::getError, src/model.hpp:1463-1802;
+// forward_prop_source, :2367-2452).  Used for end-to-end parity and as the timed CPU baseline.
+// ---------------------------------------------------------------------------
+
+// Stacked encoder / LM stack: for t in [0,T): layer 0 (embedding gather + IH node), then layers 1..L-1 (HH
+// nodes fed by the layer below at the same t).  Initial h,c per layer given (zeros for the LM / encoder,
+// src/model.hpp:1546-1551,1672-1683).
+//   weights[l][0..3]=M_g, [4..7]=Wh_g, [8..11]=b_g (gate order i,f,c,o); embed: H x V.
+//   ids_nonneg / mask01: time-major [b + t*mb] (src/fileHelper.h:488).
+//   h_all, c_all: L x T x (H*mb) (layer-major), every node's h_t and c_t.
+void orc_lstm_stack_forward(int acc64, int L, int H, int mb, int T, int V, const float* embed,
+                            const float* const* weights, const int* ids_nonneg, const int* mask01,
+                            const float* h0, const float* c0, int clip_cell, float clip_threshold, float* h_all,
+                            float* c_all) {
+  const size_t n = (size_t)H * mb;
+  std::vector<float> x(n);
+  for (int t = 0; t < T; ++t) {
+    for (int l = 0; l < L; ++l) {
+      const float* const* w = weights + (size_t)l * 12;
+      const float* in;
+      if (l == 0) {
+        orc_embed_gather(embed, H, V, ids_nonneg + (size_t)t * mb, mb, x.data());
+        in = x.data();
+      } else {
+        in = h_all + ((size_t)(l - 1) * T + t) * n;
+      }
+      const float* hp = (t == 0) ? h0 + (size_t)l * n : h_all + ((size_t)l * T + t - 1) * n;
+      const float* cp = (t == 0) ? c0 + (size_t)l * n : c_all + ((size_t)l * T + t - 1) * n;
+      orc_lstm_step(acc64, H, mb, w, w + 4, nullptr, w + 8, in, hp, cp, nullptr, mask01 + (size_t)t * mb,
+                    clip_cell, clip_threshold, nullptr, nullptr, nullptr, nullptr,
+                    c_all + ((size_t)l * T + t) * n, h_all + ((size_t)l * T + t) * n);
+    }
+  }
+}
+
+}  // extern "C"
