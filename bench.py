@@ -1,0 +1,258 @@
+#!/usr/bin/env python3
+"""Benchmark of the stacked-LSTM forward path on one MI355X.
+
+A step is one pass of the hot path over one batch of synthetic input.  The headline workload (config 2 of the
+baseline) is the 4-layer H=1000 encoder forward over a 128 x 50 minibatch with a 50 000-word vocabulary:
+embedding gather + four-gate contraction + fused cell for 200 layer-steps = 6400 tokens per step.  Inputs
+are resident in HBM before the timed region.  The config-3 decoder step (LSTM stack with feed-input,
+attention, full softmax) and the stand-alone HBM-bound kernels are measured in the same run and reported
+under "extra".
+
+Prints ONE JSON line on stdout.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "tests")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+import numpy as np  # noqa: E402
+
+PEAK_FP32_MFMA_TFLOPS = 157.3  # MI355X dense fp32 matrix peak
+PEAK_HBM_GBS = 8000.0          # MI355X HBM3E peak
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+class Uploaded:
+    """Keeps device arrays of one LSTM layer alive next to its packed weights."""
+
+    def __init__(self, ctx, ly):
+        self.H = ly["M"][0].shape[0]
+        self.M = [ctx.array(m) for m in ly["M"]]
+        self.Wh = [ctx.array(m) for m in ly["Wh"]]
+        self.b = [ctx.array(v) for v in ly["b"]]
+        self.Q = [ctx.array(m) for m in ly["Q"]] if "Q" in ly else None
+        self.w = ctx.lstm_pack(self.M, self.Wh, self.b, self.H, self.Q)
+
+
+def time_region(ctx, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    ctx.sync()
+    t0 = time.perf_counter()
+    ctx.timer_start()
+    for _ in range(steps):
+        fn()
+    ev_ms = ctx.timer_stop()
+    ctx.sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return wall_ms, ev_ms
+
+
+def bench_encoder(ctx, steps, warmup, H=1000, mb=128, T=50, V=50000, L=4):
+    from zoph_rnn_amd import synth
+    cfg = synth.encoder_config(H=H, mb=mb, T=T, V=V, L=L)
+    layers = [Uploaded(ctx, ly) for ly in cfg["layers"]]
+    d_embed = ctx.array(cfg["embed"])
+    ids = cfg["ids"]
+    d_nn, d_m = ctx.empty(ids.size, np.int32), ctx.empty(ids.size, np.int32)
+    ctx.vocab_prep(ctx.array(ids.reshape(-1)), ids.size, V, d_nn, d_m)
+    z = ctx.zeros((H, mb))
+    h_all = [ctx.empty((H * mb * T,)) for _ in range(L)]
+    c_all = [ctx.empty((H * mb * T,)) for _ in range(L)]
+    ws = [ly.w for ly in layers]
+
+    def step():
+        ctx.lstm_stack_forward(ws, d_embed, V, d_nn, d_m, T, mb, [z] * L, [z] * L, h_all, c_all)
+
+    wall_ms, ev_ms = time_region(ctx, step, steps, warmup)
+    launches = (T + L - 1) * steps            # one fused kernel launch per diagonal of the (layer, time) grid
+    flops_per_step = 2.0 * 4 * H * mb * (2 * H) * L * T
+    res = {"wall_ms": wall_ms, "event_ms": ev_ms, "tokens_per_step": mb * T, "launches_per_step": T + L - 1,
+           "flops_per_step": flops_per_step, "avg_launch_us": ev_ms * 1e3 / launches,
+           "flops_per_launch": flops_per_step / (T + L - 1)}
+    # keep references alive until here
+    res["_keep"] = (layers, d_embed, d_nn, d_m, z, h_all, c_all)
+    return res
+
+
+def bench_decoder_step(ctx, steps, warmup, H=1000, mb=128, S=50, V=50000, L=4, D=50):
+    """Config 3: gather, 4 LSTM layers (feed-input on layer 0), attention (D >= S: every source position has a
+    slot), full softmax to probabilities."""
+    from zoph_rnn_amd import capi, synth
+    c = synth.decoder_config(H=H, mb=mb, S=S, V=V, L=L)
+    layers = [Uploaded(ctx, ly) for ly in c["layers"]]
+    d_embed, d_ids = ctx.array(c["embed"]), ctx.array(c["ids"])
+    d_mask = ctx.array(np.ones(mb, np.int32))
+    d_hp = [ctx.array(a) for a in c["h_prev"]]
+    d_cp = [ctx.array(a) for a in c["c_prev"]]
+    d_htp = ctx.array(c["h_tild_prev"])
+    tables = [ctx.array(np.asfortranarray(c["hs"][t])) for t in range(S)]
+    aw = {k: ctx.array(v) for k, v in c["attn"].items()}
+    attn = ctx.attn_create(H, mb, D, aw["W_a"], aw["W_p"], aw["v_p"], aw["out_bias"], aw["W_c1"], aw["W_c2"], tables)
+    d_bi = ctx.array(c["batch_info"])
+    dD, dbd = ctx.array(c["D"]), ctx.array(c["b_d"])
+    d_x = ctx.empty((H, mb))
+    d_h = [ctx.empty((H, mb)) for _ in range(L)]
+    d_c = [ctx.empty((H, mb)) for _ in range(L)]
+    d_ht = ctx.empty((H, mb))
+    d_prob = ctx.empty((V, mb))
+
+    def lstm_part():
+        ctx.embed_gather(d_embed, H, V, d_ids, mb, d_x)
+        below = d_x
+        for l in range(L):
+            ctx.lstm_step(layers[l].w, below, d_hp[l], d_cp[l], d_mask, mb, d_h[l], d_c[l],
+                          d_htild=d_htp if l == 0 else None)
+            below = d_h[l]
+
+    def attn_part():
+        ctx.attn_step(attn, d_bi, d_h[L - 1], d_mask, d_ht)
+
+    def softmax_part():
+        ctx.softmax_forward(dD, dbd, V, H, d_ht, mb, capi.ZR_SOFTMAX_PROB, d_prob)
+
+    def step():
+        lstm_part()
+        attn_part()
+        softmax_part()
+
+    wall_ms, ev_ms = time_region(ctx, step, steps, warmup)
+    parts = {}
+    for name, fn in (("lstm_stack", lstm_part), ("attention", attn_part), ("softmax", softmax_part)):
+        _, ms = time_region(ctx, fn, steps, 1)
+        parts[name + "_us"] = round(ms * 1e3 / steps, 2)
+    flops = 2.0 * 4 * H * mb * (3 * H) + (L - 1) * 2.0 * 4 * H * mb * (2 * H) + 4 * 2.0 * H * H * mb + 2.0 * V * H * mb
+    res = {"ms_per_step": ev_ms / steps, "wall_ms_per_step": wall_ms / steps, "tokens_per_s": mb * steps / (ev_ms * 1e-3),
+           "gflop_per_step": flops / 1e9, "tflops": flops * steps / (ev_ms * 1e-3) / 1e12, "attention_D": D}
+    res.update(parts)
+    res["softmax_gemm_plus_normalise_tflops"] = round(2.0 * V * H * mb / (parts["softmax_us"] * 1e-6) / 1e12, 2)
+    ctx.attn_destroy(attn)
+    return res
+
+
+def bench_hbm_kernels(ctx, steps, H=1000, mb=128, V=50000):
+    """Stand-alone HBM-bound kernels at the benchmark shape: achieved GB/s of algorithmic bytes."""
+    from zoph_rnn_amd import synth
+    g = synth.rng(77, 1)
+    out = {}
+    # embedding gather for a whole 128 x 50 minibatch in one launch (6400 columns)
+    n = mb * 50
+    d_W = ctx.array(synth.uniform(g, (H, V)))
+    d_ids = ctx.array(synth.zipf_ids(g, (n,), V))
+    d_x = ctx.empty((H, n))
+    _, ms = time_region(ctx, lambda: ctx.embed_gather(d_W, H, V, d_ids, n, d_x), steps, 2)
+    bytes_ = 2.0 * n * H * 4 + n * 4
+    out["embed_gather"] = {"columns": n, "us": round(ms * 1e3 / steps, 2), "algorithmic_MB": round(bytes_ / 1e6, 3),
+                           "GBps": round(bytes_ * steps / (ms * 1e-3) / 1e9, 1)}
+    # fused gate kernel, one layer-step (4 pre-activation planes + c_prev in, c and h out)
+    d_pre = ctx.array(synth.uniform(g, (4 * H * mb,), -1, 1))
+    d_b = [ctx.array(synth.uniform(g, (H,))) for _ in range(4)]
+    d_cp = ctx.array(synth.uniform(g, (H, mb), -1, 1))
+    d_m = ctx.array(np.ones(mb, np.int32))
+    d_h, d_c = ctx.empty((H, mb)), ctx.empty((H, mb))
+    _, ms = time_region(ctx, lambda: ctx.lstm_gates(d_pre, d_b, d_cp, d_m, H, mb, d_h, d_c), steps, 2)
+    bytes_ = 7.0 * H * mb * 4 + 4 * H * 4 + mb * 4
+    out["lstm_gates"] = {"us": round(ms * 1e3 / steps, 2), "algorithmic_MB": round(bytes_ / 1e6, 3),
+                         "GBps": round(bytes_ * steps / (ms * 1e-3) / 1e9, 1)}
+    return out
+
+
+def cpu_baseline(H=1000, mb=128, V=50000, L=4, t_sample=20):
+    """The oracle (float accumulation, OpenMP) on a bounded sample of the headline workload: t_sample time steps
+    of the 4-layer encoder with the same shapes; per-token cost does not depend on T."""
+    import oracle_lib as o
+    from zoph_rnn_amd import synth
+    cfg = synth.encoder_config(H=H, mb=mb, T=t_sample, V=V, L=L)
+    nn, m = o.vocab_prep(cfg["ids"])
+    o.lstm_stack_forward(cfg["embed"], cfg["layers"], nn[:1], m[:1], acc64=False)  # warm-up (one time step)
+    reps = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        o.lstm_stack_forward(cfg["embed"], cfg["layers"], nn, m, acc64=False)
+        reps.append(time.perf_counter() - t0)
+    sec = sorted(reps)[1]
+    return {"value": round(mb * t_sample / sec, 1), "unit": "tokens/s", "cores": o.num_threads(), "kind": "port",
+            "sample": "%d of 50 time steps of the same 4-layer H=%d mb=%d encoder (3 repetitions, median; %.2f s each)"
+                      % (t_sample, H, mb, sec)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the config-3 and HBM-kernel measurements")
+    ap.add_argument("--lstm-tn", type=int, default=0)
+    ap.add_argument("--lstm-ks", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus %d is not supported (no cross-GPU path exists)" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+
+    from zoph_rnn_amd import capi
+    ctx = capi.Context(0)
+    if args.lstm_tn:
+        ctx.set_option(capi.ZR_OPT_LSTM_TN, args.lstm_tn)
+    if args.lstm_ks:
+        ctx.set_option(capi.ZR_OPT_LSTM_KSPLIT, args.lstm_ks)
+
+    enc = bench_encoder(ctx, args.steps, args.warmup)
+    enc.pop("_keep")
+    ms_per_step = enc["event_ms"] / args.steps
+    tokens_per_s = enc["tokens_per_step"] / (ms_per_step * 1e-3)
+    achieved_tflops = enc["flops_per_launch"] / (enc["avg_launch_us"] * 1e-6) / 1e12
+    log("encoder: %.3f ms/step (wall %.3f), %.0f tokens/s, %.1f TFLOP/s" %
+        (ms_per_step, enc["wall_ms"] / args.steps, tokens_per_s, achieved_tflops))
+
+    extra = {}
+    if not args.no_extra:
+        extra["config3_decoder_step"] = {k: (round(v, 4) if isinstance(v, float) else v)
+                                         for k, v in bench_decoder_step(ctx, args.steps, args.warmup).items()}
+        log("config3:", extra["config3_decoder_step"])
+        extra["hbm_kernels"] = bench_hbm_kernels(ctx, args.steps)
+        log("hbm kernels:", extra["hbm_kernels"])
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline()
+        log("cpu baseline:", cpu)
+    ctx.close()
+
+    line = {
+        "metric": "LSTM step tokens/sec on 1 GPU (4L H=1000 mb=128 V=50k) + % HBM/MFMA roofline",
+        "value": round(tokens_per_s, 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "config 2: 4-layer LSTM encoder forward, H=1000, minibatch 128, source length 50, "
+                               "vocab 50000 (Zipf ids), fp32; one step = 200 layer-steps = 6400 tokens",
+                   "tokens_per_step": enc["tokens_per_step"], "launches_per_step": enc["launches_per_step"]},
+        "roofline": {"bound": "mfma", "kernel": "lstm_fused_kernel", "achieved": round(achieved_tflops, 2),
+                     "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved_tflops / PEAK_FP32_MFMA_TFLOPS, 4),
+                     "traffic": None, "avg_launch_us": round(enc["avg_launch_us"], 2),
+                     "flops_per_launch": enc["flops_per_launch"]},
+        "cpu_baseline": cpu,
+        "extra": extra,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,218 @@
+/*
+ * zoph_rnn.h -- C-ABI of the MI355X (gfx950) implementation of Zoph_RNN's stacked-LSTM forward path.
+ *
+ * The reference (isi-nlp/Zoph_RNN) has no FFI: the path lives behind C++ template members compiled into one
+ * translation unit.  Each entry point below states which reference member / kernel / cuBLAS call site it
+ * replaces (paths relative to the reference root).  The C++ classes under zoph_rnn_amd/host/ keep the
+ * reference's class and member names and forward to these functions.
+ *
+ * Conventions
+ *   - every function returns 0 on success and a negative ZR_E* code on failure; zr_last_error() returns a
+ *     message for the calling thread.  Nothing here aborts the process (the reference exits on any CUDA
+ *     error, src/BZ_CUDA_UTIL.h:193-270).
+ *   - all matrices are column-major fp32 (IDX2C, src/BZ_CUDA_UTIL.h:26): activations are H x minibatch, the
+ *     embedding is H x V, the softmax matrix D is V x H.
+ *   - pointers named d_* are device pointers on the context's GPU, h_* are host pointers.
+ *   - a context owns one in-order HIP stream; calls on one context are asynchronous with respect to the host
+ *     and ordered with respect to each other.  A context is not re-entrant.
+ *   - gate order everywhere is i, f, c, o (the reference's temp1..8 / i_t, f_t, c_prime_t_tanh, o_t order).
+ */
+#ifndef ZOPH_RNN_H
+#define ZOPH_RNN_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ZR_OK 0
+#define ZR_EINVAL (-1)   /* bad argument (null pointer, non-positive size, unsupported shape) */
+#define ZR_EHIP (-2)     /* a HIP runtime call failed */
+#define ZR_ENOMEM (-3)   /* device allocation failed */
+#define ZR_EDATA (-4)    /* device-side data check failed (token id outside [0, V), ...) */
+
+typedef struct zr_ctx zr_ctx;
+typedef struct zr_lstm_weights zr_lstm_weights;
+typedef struct zr_beam zr_beam;
+
+/* ---- runtime ------------------------------------------------------------------------------------------ */
+
+/* Replaces layer_gpu_info::init / softmax_layer_gpu_info::init (src/gpu_info_struct.h:67-172: per-layer
+ * cudaSetDevice, 9+ streams, ~50 events, cublasCreate).  One in-order stream replaces the stream/event DAG. */
+int zr_ctx_create(int device, zr_ctx** out);
+int zr_ctx_destroy(zr_ctx* ctx);
+/* devSynchAll (src/BZ_CUDA_UTIL.h:977-987) followed by CUDA_GET_LAST_ERROR (:262-270): waits for the stream and
+ * reports launch errors and the device-side data flag (ZR_EDATA) instead of exiting. */
+int zr_ctx_sync(zr_ctx* ctx);
+/* Use a caller-owned hipStream_t (passed as void*) instead of the context's own; NULL restores the own stream. */
+int zr_ctx_set_stream(zr_ctx* ctx, void* hip_stream);
+/* Device-side timing of everything queued on the context's stream between the two calls (HIP events).  The
+ * reference brackets phases with host wall-clock Timer objects after devSynchAll (src/memory_util.h:87-124,
+ * src/model.hpp:2576-2686).  zr_timer_stop waits for the stream and returns milliseconds. */
+int zr_timer_start(zr_ctx* ctx);
+int zr_timer_stop(zr_ctx* ctx, float* h_ms);
+/* Tuning / mode switches: see ZR_OPT_* below. */
+int zr_ctx_set_option(zr_ctx* ctx, int option, int value);
+const char* zr_last_error(void);
+/* Library self-description: "gfx950 hip <build tag>". */
+const char* zr_version(void);
+
+#define ZR_OPT_LSTM_FUSED_EPILOGUE 1 /* 1 (default): gate maths in the GEMM epilogue; 0: GEMM then zr_lstm_gates */
+#define ZR_OPT_LSTM_TN 2             /* columns per workgroup / 32 for the fused LSTM kernel: 1, 2 or 4 (0 = auto) */
+#define ZR_OPT_GEMM_CFG 3            /* generic GEMM tile selection (0 = auto) */
+#define ZR_OPT_LSTM_KSPLIT 4         /* waves per workgroup splitting K in the fused LSTM kernel: 4 or 8 (0 = auto) */
+
+/* full_matrix_setup / cudaMalloc / cudaMemcpy / cudaMemset call sites (src/BZ_CUDA_UTIL.h:358-399 and the
+ * layer constructors, e.g. src/LSTM.hpp:23-42). */
+int zr_malloc(zr_ctx* ctx, size_t bytes, void** d_out);
+int zr_free(zr_ctx* ctx, void* d_ptr);
+int zr_h2d(zr_ctx* ctx, void* d_dst, const void* h_src, size_t bytes);
+int zr_d2h(zr_ctx* ctx, void* h_dst, const void* d_src, size_t bytes); /* synchronous with the stream */
+int zr_d2d(zr_ctx* ctx, void* d_dst, const void* d_src, size_t bytes);
+int zr_memset_zero(zr_ctx* ctx, void* d_dst, size_t bytes);
+
+/* ---- A1: index preparation ---------------------------------------------------------------------------- */
+
+/* vocab_to_01 + vocab_to_nonM1 (src/custom_kernels.h:10-32) as launched by
+ * Input_To_Hidden_Layer::prep_GPU_vocab_indices (src/Input_To_Hidden_Layer.hpp:1199-1202) and
+ * Hidden_To_Hidden_Layer::prep_GPU_vocab_indices (src/Hidden_To_Hidden_Layer.hpp:763).
+ * d_ids_nonneg or d_mask01 may be NULL.  vocab_size > 0 enables the [0,V) range check (flag read by zr_ctx_sync). */
+int zr_vocab_prep(zr_ctx* ctx, const int* d_ids, int n, int vocab_size, int* d_ids_nonneg, int* d_mask01);
+/* vocab_softmax (src/custom_kernels.h:38-50) from softmax_layer::prep_GPU_vocab_indices
+ * (src/softmax.hpp:926-947): in place -1 -> 0 plus int and float masks. */
+int zr_vocab_prep_softmax(zr_ctx* ctx, int* d_ids_inout, int n, int vocab_size, int* d_mask01, float* d_mask01_float);
+
+/* ---- A2: embedding-column gather ---------------------------------------------------------------------- */
+
+/* sparse_lookup_kernel (src/custom_kernels.h:342-348) from LSTM_IH_Node::forward_prop_GPU (src/LSTM.hpp:95):
+ * d_x[:,b] = d_W[:, d_ids[b]], bit-exact.  Ids outside [0,V) are clamped and raise the data flag. */
+int zr_embed_gather(zr_ctx* ctx, const float* d_W, int H, int V, const int* d_ids, int mb, float* d_x);
+
+/* ---- A3-A5: LSTM node forward -------------------------------------------------------------------------- */
+
+/* Packs one layer's parameters for zr_lstm_step.  Replaces the separate d_M_{i,f,c,o}, d_W_h{i,f,c,o},
+ * d_Q_{i,f,c,o}, d_b_{i,f,c,o} members read by the 8/12 cublasSgemm calls of one node
+ * (src/LSTM.hpp:140-339, src/LSTM_HH.hpp:148-271; members at src/Input_To_Hidden_Layer.h, src/Hidden_To_Hidden_Layer.h).
+ * d_M/d_Wh/d_Q/d_b: arrays of 4 device pointers in gate order i,f,c,o; d_Q may be NULL (no feed-input). */
+int zr_lstm_pack_weights(zr_ctx* ctx, const float* const d_M[4], const float* const d_Wh[4],
+                         const float* const d_Q[4], const float* const d_b[4], int H, zr_lstm_weights** out);
+int zr_lstm_weights_destroy(zr_ctx* ctx, zr_lstm_weights* w);
+
+/* One node forward step: LSTM_IH_Node::forward_prop_GPU after the gather (src/LSTM.hpp:133-399) and
+ * LSTM_HH_Node::forward_prop_GPU (src/LSTM_HH.hpp:103-333): the 8 (12 with feed-input) GEMMs, the four
+ * activation kernels (custom_kernels.h:58-135), forward_c_t_kernel (:141), clip_mat_kernel (:2222),
+ * forward_h_t_kernel (:162) and zero_c_t_and_h_t (:184) in one launch.
+ *   d_in:    x (IH node) or h_t of the layer below (HH node), H x mb
+ *   d_htild: NULL, or the previous attention output (feed-input; the reference skips it at index 0,
+ *            src/LSTM.hpp:154) -- requires weights packed with Q
+ *   clip_threshold <= 0 disables cell clipping (BZ_CUDA::clip_cell, src/BZ_CUDA_UTIL.h:107-108)
+ *   d_gates: NULL or 4 device pointers (i, f, c~, o; each H x mb) for callers that keep them (the reference's
+ *            node members d_i_t, d_f_t, d_c_prime_t_tanh, d_o_t)
+ *   d_h / d_c may alias d_hprev / d_cprev only if d_in != d_hprev (every output element is written once, after
+ *   all reads of the same element; other columns of h_prev are read by other workgroups, so in-place h is NOT
+ *   allowed; in-place c is). */
+int zr_lstm_step(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_in, const float* d_hprev,
+                 const float* d_cprev, const float* d_htild, const int* d_mask01, float clip_threshold, int mb,
+                 float* d_h, float* d_c, float* const d_gates[4]);
+
+/* The stand-alone fused gate kernel (the four activation kernels + c_t + clip + h_t + mask of the list above)
+ * on pre-activations that are already in memory: d_preact is 4 planes (i,f,c,o) of H x mb holding
+ * M x + W_h h (+ Q h~) without bias. */
+int zr_lstm_gates(zr_ctx* ctx, const float* d_preact, const float* const d_b[4], const float* d_cprev,
+                  const int* d_mask01, float clip_threshold, int H, int mb, float* d_h, float* d_c,
+                  float* const d_gates[4]);
+
+/* Whole stacked forward sweep (the time x layer loop of neuralMT_model::getError, src/model.hpp:1546-1621, and
+ * forward_prop_source, :2367-2452): layer 0 gathers its input from d_embed by token id, layer l>0 reads layer
+ * l-1's h_t.  Layers and time steps that do not depend on each other run in the same launch.
+ *   d_ids_nonneg, d_mask01: time-major [b + t*mb] (src/fileHelper.h:488), outputs of zr_vocab_prep
+ *   d_h0/d_c0: arrays of L device pointers (initial state per layer, H x mb) -- zeros for encoder / LM
+ *   d_h_all/d_c_all: arrays of L device pointers, each T*H*mb floats: node t's h_t at offset t*H*mb */
+int zr_lstm_stack_forward(zr_ctx* ctx, int L, const zr_lstm_weights* const layers[], const float* d_embed, int V,
+                          const int* d_ids_nonneg, const int* d_mask01, int T, int mb,
+                          const float* const d_h0[], const float* const d_c0[], float clip_threshold,
+                          float* const d_h_all[], float* const d_c_all[]);
+
+/* ---- dense contraction --------------------------------------------------------------------------------- */
+
+/* cublas_gemm_wrapper / cublasSgemm (src/BZ_CUDA_UTIL.h:691-696) with alpha = 1, beta = 0:
+ * C(M x N) = op(A) * B, trans_a = 0: A is M x K (lda >= M); trans_a = 1: A is K x M (lda >= K).  B is K x N. */
+int zr_gemm(zr_ctx* ctx, int trans_a, int M, int N, int K, const float* d_A, int lda, const float* d_B, int ldb,
+            float* d_C, int ldc);
+
+/* ---- A8/A9: output softmax ------------------------------------------------------------------------------ */
+
+#define ZR_SOFTMAX_PROB 0    /* probabilities: softmax_layer::get_distribution_GPU (src/softmax.hpp:514-632) */
+#define ZR_SOFTMAX_LOGPROB 1 /* natural-log probabilities, fp32 */
+
+/* D h + b_d on MFMA (cublasSgemm + matrix_bias_kernel, src/softmax.hpp:539-547) followed by the per-column
+ * max / exp / sum / normalise of outputdist_overflow_prevention_kernel (src/custom_kernels.h:503-577).
+ * d_out: V x mb.  d_logits_scratch: V x mb scratch for the logits, or NULL to use d_out in place. */
+int zr_softmax_forward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int mb,
+                       int mode, float* d_out, float* d_logits_scratch);
+/* softmax_layer::get_perplexity_GPU (src/softmax.hpp:636-692) with outputdist_perplexity_kernel
+ * (src/custom_kernels.h:583-660): double log-probabilities, V x mb. */
+int zr_softmax_logprob_f64(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int mb,
+                           double* d_logp, float* d_logits_scratch);
+/* softmax_layer::compute_loss_GPU (src/softmax.hpp:867-900): sum over unmasked columns of
+ * log p[target[b], b] (double), without materialising the V x mb log-probabilities.  Synchronous: *h_loss is
+ * valid on return.  d_logits_scratch: V x mb floats. */
+int zr_softmax_loss(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int mb,
+                    const int* d_target, const int* d_mask01, float* d_logits_scratch, double* h_loss);
+
+/* ---- A10: attention -------------------------------------------------------------------------------------- */
+
+/* attention_layer constructor (src/attention_layer.hpp:3-173): keeps the six parameter pointers (borrowed, not
+ * copied: d_W_a, d_W_p H x H; d_v_p H (stored 1 x H); d_out_bias H; d_W_c_p1, d_W_c_p2 H x H), uploads the
+ * source-state pointer table (d_total_hs_mat, :106-160) and allocates the node temporaries.
+ *   h_hs_table: host array of longest_sent device pointers; entry t = top-layer source h at source node t,
+ *               H x mb.  The tables are read at zr_attn_step time and must stay valid. */
+typedef struct zr_attn zr_attn;
+int zr_attn_create(zr_ctx* ctx, int H, int mb, int D, const float* d_W_a, const float* d_W_p, const float* d_v_p,
+                   const float* d_out_bias, const float* d_W_c1, const float* d_W_c2,
+                   const float* const* h_hs_table, int longest_sent, zr_attn** out);
+int zr_attn_destroy(zr_ctx* ctx, zr_attn* a);
+/* attention_node::forward_prop (src/attention_node.hpp:73-394), single-source branch: p_t, window, scores
+ * h_s . (W_a^T h), the reference's softmax (max initialised to 0) times the Gaussian prior, context and
+ * h~ = tanh(W_c1 c + W_c2 h + b) * mask.
+ *   d_batch_info: [0,mb) source lengths, [mb,2mb) left-pad offsets (src/fileHelper.h:499-500; uploaded by
+ *                 attention_layer::prep_minibatch_info, src/attention_layer.hpp:580-583)
+ *   outputs: d_htild H x mb (the node's d_final_temp_2); optional (NULL = internal): d_alignments and
+ *   d_indices ((2D+1) x mb, element [b + mb*j]), d_p_t (mb), d_c_ctx (H x mb). */
+int zr_attn_step(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, const float* d_h_t, const int* d_mask01,
+                 float* d_htild, float* d_alignments, int* d_indices, float* d_p_t, float* d_c_ctx);
+
+/* ---- A12: decoder state shuffles ------------------------------------------------------------------------- */
+
+/* swap_states_decoding (src/Input_To_Hidden_Layer.hpp:1231-1242, src/Hidden_To_Hidden_Layer.hpp:780-791):
+ * d_dst[:,i] = d_src[:, d_perm[i]] for i < n; d_dst must not alias d_src. */
+int zr_gather_columns(zr_ctx* ctx, const float* d_src, int H, const int* d_perm, int n, float* d_dst);
+/* transfer_decoding_states_GPU (src/Input_To_Hidden_Layer.hpp:1252-1266): one column to n columns. */
+int zr_broadcast_column(zr_ctx* ctx, const float* d_src_col, int H, int n, float* d_dst);
+
+/* ---- A13: beam search ------------------------------------------------------------------------------------ */
+
+/* decoder<dType> (src/decoder.h:162-1502), non-FSA path, for n_sent independent sentences decoded together
+ * (the reference decodes one sentence per pass; columns [s*beam, (s+1)*beam) belong to sentence s).
+ * start symbol 0, end symbol 1 (src/decoder.h:1325-1330). */
+int zr_beam_create(zr_ctx* ctx, int beam, int vocab, int n_sent, int max_len, float penalty, zr_beam** out);
+int zr_beam_destroy(zr_ctx* ctx, zr_beam* b);
+/* init_decoder (src/decoder.h:1317-1355) */
+int zr_beam_init(zr_ctx* ctx, zr_beam* b);
+/* expand_hypothesis_without_fsa (src/decoder.h:1158-1315) on device: d_prob is V x (n_sent*beam)
+ * probabilities.  Afterwards d_words (next input ids, -1 = dead slot) and d_backptr (new_indicies_changes)
+ * are valid, n_sent*beam ints each. */
+int zr_beam_expand(zr_ctx* ctx, zr_beam* b, const float* d_prob, int index, int* d_words, int* d_backptr);
+/* finish_current_hypotheses (src/decoder.h:672-688). */
+int zr_beam_finish(zr_ctx* ctx, zr_beam* b, const float* d_prob);
+/* Copies the finished hypotheses of sentence s to the host: returns their number (or a negative error);
+ * h_words is n x max_len (row-major, -1 padded), h_len and h_score have n entries; at most cap are copied. */
+int zr_beam_hypotheses(zr_ctx* ctx, zr_beam* b, int sentence, int cap, int* h_words, int* h_len, float* h_score);
+/* Current beam state of sentence s (top_sentences_scores, current_indices). */
+int zr_beam_state(zr_ctx* ctx, zr_beam* b, int sentence, float* h_scores, int* h_words);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ZOPH_RNN_H */

@@ -1,0 +1,465 @@
+"""Parity of the HIP path (through the C-ABI) against the CPU oracle on identical seeded inputs.
+
+Bars: gathers / index work bit-exact; fp32 activations, log-probs and attention weights within 1e-4 relative
+(|got - want| <= 1e-4 * max(|want|, 1e-2), see gpu_util.assert_close)."""
+import numpy as np
+import pytest
+
+import oracle_lib as o
+from gpu_util import Layer, assert_close, run_lstm_step
+from zoph_rnn_amd import capi, synth
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = capi.Context(0)
+    yield c
+    c.close()
+
+
+def U(g, shape, lo=-0.08, hi=0.08):
+    return synth.uniform(g, shape, lo, hi)
+
+
+# ------------------------------------------------------------------------------------------------ A1 / A2 / A12
+def test_vocab_prep_and_gather_bit_exact(ctx):
+    g = synth.rng(1, 10)
+    V, H = 97, 52
+    ids = g.integers(0, V, size=300).astype(np.int32)
+    ids[::7] = -1
+    d_ids = ctx.array(ids)
+    d_nn, d_m = ctx.empty(ids.shape, np.int32), ctx.empty(ids.shape, np.int32)
+    ctx.vocab_prep(d_ids, ids.size, V, d_nn, d_m)
+    ctx.sync()
+    nn, m = o.vocab_prep(ids)
+    assert np.array_equal(d_nn.get(), nn) and np.array_equal(d_m.get(), m)
+    d_mf = ctx.empty(ids.shape, np.float32)
+    ctx.vocab_prep_softmax(d_ids, ids.size, V, d_m, d_mf)
+    ctx.sync()
+    ids2, m2, mf2 = o.vocab_softmax(ids)
+    assert np.array_equal(d_ids.get(), ids2) and np.array_equal(d_m.get(), m2) and np.array_equal(d_mf.get(), mf2)
+    for Hh in (52, 51, 1000):  # 16-byte path, scalar path, full size
+        W = U(g, (Hh, V))
+        gids = np.array([0, V - 1, 5, 5, 0, 17] + list(g.integers(0, V, size=40)), np.int32)
+        d_x = ctx.empty((Hh, gids.size))
+        ctx.embed_gather(ctx.array(W), Hh, V, ctx.array(gids), gids.size, d_x)
+        ctx.sync()
+        assert d_x.get().tobytes() == o.embed_gather(W, gids).tobytes()
+
+
+def test_gather_out_of_range_id_is_reported_not_fatal(ctx):
+    W = np.asfortranarray(np.arange(12, dtype=np.float32).reshape(4, 3, order="F"))
+    d_x = ctx.empty((4, 2))
+    ctx.embed_gather(ctx.array(W), 4, 3, ctx.array(np.array([1, 7], np.int32)), 2, d_x)
+    with pytest.raises(capi.ZrError) as e:
+        ctx.sync()
+    assert e.value.code == -4
+    assert np.array_equal(d_x.get()[:, 0], W[:, 1]) and np.array_equal(d_x.get()[:, 1], W[:, 2])
+    ctx.sync()  # flag cleared
+
+
+def test_decoder_state_shuffles(ctx):
+    g = synth.rng(2, 10)
+    src = U(g, (1000, 12))
+    perm = np.array([3, 3, 0, 11, 5, 5, 5, 1, 2, 10, 9, 0], np.int32)
+    d_dst = ctx.empty((1000, 12))
+    ctx.gather_columns(ctx.array(src), 1000, ctx.array(perm), 12, d_dst)
+    ctx.sync()
+    assert d_dst.get().tobytes() == o.gather_columns(src, perm).tobytes()
+    ctx.broadcast_column(ctx.array(src[:, [4]]), 1000, 12, d_dst)
+    ctx.sync()
+    assert np.array_equal(d_dst.get(), np.repeat(src[:, [4]], 12, axis=1))
+
+
+# ------------------------------------------------------------------------------------------------ A3 contraction
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("M,N,K,trans", [(100, 8, 100, 0), (257, 33, 61, 0), (64, 128, 200, 1), (95, 7, 37, 1)])
+def test_gemm_tiles_and_tails(ctx, cfg, M, N, K, trans):
+    g = synth.rng(3, 100 * cfg + M)
+    A = U(g, (K, M) if trans else (M, K), -1, 1)
+    B = U(g, (K, N), -1, 1)
+    want = (A.T.astype(np.float64) if trans else A.astype(np.float64)) @ B.astype(np.float64)
+    dC = ctx.zeros((M, N))
+    ctx.set_option(capi.ZR_OPT_GEMM_CFG, cfg)
+    try:
+        ctx.gemm(trans, M, N, K, ctx.array(A), A.shape[0], ctx.array(B), K, dC, M)
+        ctx.sync()
+    finally:
+        ctx.set_option(capi.ZR_OPT_GEMM_CFG, 0)
+    # operands are U(-1,1): outputs have standard deviation sqrt(K)/3 and entries near zero are sums with
+    # cancellation, so the floor of the mixed bound is the output scale rather than 1e-2
+    assert_close(dC.get(), want, floor=float(np.sqrt(K) / 3), what="gemm cfg %d" % cfg)
+
+
+def test_gemm_padded_leading_dimensions(ctx):
+    g = synth.rng(4, 1)
+    M, N, K, lda, ldb, ldc = 70, 9, 44, 75, 47, 90  # ldb not a multiple of 4 -> scalar activation loads
+    A, B = U(g, (lda, K), -1, 1), U(g, (ldb, N), -1, 1)
+    C0 = np.full((ldc, N), 7.0, np.float32, order="F")
+    dC = ctx.array(C0)
+    ctx.gemm(0, M, N, K, ctx.array(A), lda, ctx.array(B), ldb, dC, ldc)
+    ctx.sync()
+    got = dC.get()
+    assert_close(got[:M], A[:M].astype(np.float64) @ B[:K].astype(np.float64), floor=float(np.sqrt(K) / 3),
+                 what="padded gemm")
+    assert np.all(got[M:] == 7.0)  # rows beyond M untouched
+
+
+def test_gemm_full_size_attention_shape(ctx):
+    g = synth.rng(5, 1)
+    A, B = U(g, (1000, 1000)), U(g, (1000, 128), -1, 1)
+    dC = ctx.empty((1000, 128))
+    ctx.gemm(0, 1000, 128, 1000, ctx.array(A), 1000, ctx.array(B), 1000, dC, 1000)
+    ctx.sync()
+    assert_close(dC.get(), o.gemm_nn(A, B), what="1000x128x1000")
+    ctx.gemm(1, 1000, 128, 1000, ctx.array(A), 1000, ctx.array(B), 1000, dC, 1000)
+    ctx.sync()
+    assert_close(dC.get(), o.gemm_tn(A, B), what="1000x128x1000 transposed")
+
+
+# ------------------------------------------------------------------------------------------------ A3-A5 LSTM node
+LSTM_SHAPES = [(32, 3), (100, 8), (72, 33), (250, 70)]
+
+
+@pytest.mark.parametrize("H,mb", LSTM_SHAPES)
+@pytest.mark.parametrize("tn,ks", [(0, 0), (1, 4), (1, 8), (2, 4), (2, 8), (4, 4)])
+def test_lstm_step_fused(ctx, H, mb, tn, ks):
+    g = synth.rng(6, H * 1000 + mb)
+    ly = synth.lstm_layer(g, H, forget_bias_one=True)
+    x, hp, cp = U(g, (H, mb), -1, 1), U(g, (H, mb), -1, 1), U(g, (H, mb), -1, 1)
+    mask = (g.random(mb) > 0.2).astype(np.int32)
+    layer = Layer(ctx, ly)
+    ctx.set_option(capi.ZR_OPT_LSTM_TN, tn)
+    ctx.set_option(capi.ZR_OPT_LSTM_KSPLIT, ks)
+    try:
+        got = run_lstm_step(ctx, layer, x, hp, cp, mask, want_gates=True)
+    finally:
+        ctx.set_option(capi.ZR_OPT_LSTM_TN, 0)
+        ctx.set_option(capi.ZR_OPT_LSTM_KSPLIT, 0)
+        layer.close()
+    want = o.lstm_step(ly["M"], ly["Wh"], ly["b"], x, hp, cp, mask)
+    for k in ("i", "f", "c_tilde", "o", "c", "h"):
+        assert_close(got[k], want[k], what="%s (H=%d mb=%d tn=%d ks=%d)" % (k, H, mb, tn, ks))
+    dead = mask == 0
+    assert np.all(got["h"][:, dead] == 0) and np.all(got["c"][:, dead] == 0)
+
+
+@pytest.mark.parametrize("fused", [1, 0])
+def test_lstm_step_feed_input_clip_and_unfused(ctx, fused):
+    g = synth.rng(7, fused)
+    H, mb = 100, 8
+    ly = synth.lstm_layer(g, H, feed_input=True)
+    x, hp, ht = U(g, (H, mb), -1, 1), U(g, (H, mb), -1, 1), U(g, (H, mb), -1, 1)
+    cp = U(g, (H, mb), -3, 3)
+    mask = np.array([1, 1, 0, 1, 1, 1, 0, 1], np.int32)
+    layer = Layer(ctx, ly)
+    ctx.set_option(capi.ZR_OPT_LSTM_FUSED_EPILOGUE, fused)
+    try:
+        got_feed = run_lstm_step(ctx, layer, x, hp, cp, mask, htild=ht, clip=0.6, want_gates=True)
+        got_plain = run_lstm_step(ctx, layer, x, hp, cp, mask)  # index 0: Q skipped although packed
+    finally:
+        ctx.set_option(capi.ZR_OPT_LSTM_FUSED_EPILOGUE, 1)
+        layer.close()
+    want_feed = o.lstm_step(ly["M"], ly["Wh"], ly["b"], x, hp, cp, mask, Q=ly["Q"], htild=ht, clip=0.6)
+    want_plain = o.lstm_step(ly["M"], ly["Wh"], ly["b"], x, hp, cp, mask)
+    for k in ("i", "f", "c_tilde", "o", "c", "h"):
+        assert_close(got_feed[k], want_feed[k], what="feed " + k)
+    assert np.all(np.abs(got_feed["c"]) <= 0.6)
+    assert_close(got_plain["h"], want_plain["h"], what="plain h")
+    assert_close(got_plain["c"], want_plain["c"], what="plain c")
+
+
+def test_lstm_gates_kernel_closed_forms(ctx):
+    """Stand-alone gate kernel on given pre-activations: zero pre-activations and saturation."""
+    H, mb = 1000, 16
+    g = synth.rng(8, 1)
+    cp = U(g, (H, mb), -2, 2)
+    zero_b = [ctx.zeros((H,)) for _ in range(4)]
+    dh, dc = ctx.empty((H, mb)), ctx.empty((H, mb))
+    ctx.lstm_gates(ctx.zeros((4 * H * mb,)), zero_b, ctx.array(cp), ctx.array(np.ones(mb, np.int32)), H, mb, dh, dc)
+    ctx.sync()
+    assert np.array_equal(dc.get(), 0.5 * cp)
+    assert_close(dh.get(), 0.5 * np.tanh(0.5 * cp.astype(np.float64)), what="h at zero pre-activation")
+    pre = np.concatenate([np.full(H * mb, v, np.float32) for v in (40.0, -40.0, 40.0, 40.0)])
+    ctx.lstm_gates(ctx.array(pre), zero_b, ctx.array(cp), ctx.array(np.ones(mb, np.int32)), H, mb, dh, dc)
+    ctx.sync()
+    assert np.all(dc.get() == 1.0) and np.allclose(dh.get(), np.tanh(1.0), atol=1e-6)
+
+
+def test_lstm_step_full_size_layer(ctx):
+    """One layer-step at the benchmark shape (H=1000, mb=128), with and without feed-input."""
+    g = synth.rng(9, 1)
+    H, mb = 1000, 128
+    ly = synth.lstm_layer(g, H, feed_input=True, forget_bias_one=True)
+    x, hp, cp, ht = (U(g, (H, mb), -0.08, 0.08), np.tanh(U(g, (H, mb), -1, 1)) * np.float32(0.5),
+                     U(g, (H, mb), -0.5, 0.5), np.tanh(U(g, (H, mb), -1, 1)))
+    mask = np.ones(mb, np.int32)
+    layer = Layer(ctx, ly)
+    try:
+        got = run_lstm_step(ctx, layer, x, hp, cp, mask)
+        got_feed = run_lstm_step(ctx, layer, x, hp, cp, mask, htild=ht)
+    finally:
+        layer.close()
+    want = o.lstm_step(ly["M"], ly["Wh"], ly["b"], x, hp, cp, mask)
+    want_feed = o.lstm_step(ly["M"], ly["Wh"], ly["b"], x, hp, cp, mask, Q=ly["Q"], htild=ht)
+    assert_close(got["h"], want["h"], what="h")
+    assert_close(got["c"], want["c"], what="c")
+    assert_close(got_feed["h"], want_feed["h"], what="h feed")
+    assert_close(got_feed["c"], want_feed["c"], what="c feed")
+
+
+# ------------------------------------------------------------------------------------------------ A6/A7/A11 stack
+def _run_stack(ctx, cfg_layers, embed, ids, h0=None, c0=None, clip=0.0):
+    H, V = embed.shape
+    T, mb = ids.shape
+    L = len(cfg_layers)
+    layers = [Layer(ctx, ly) for ly in cfg_layers]
+    d_ids = ctx.array(ids.reshape(-1))
+    d_nn, d_m = ctx.empty(ids.size, np.int32), ctx.empty(ids.size, np.int32)
+    ctx.vocab_prep(d_ids, ids.size, V, d_nn, d_m)
+    z = ctx.zeros((H, mb))
+    d_h0 = [ctx.array(h0[l]) if h0 is not None else z for l in range(L)]
+    d_c0 = [ctx.array(c0[l]) if c0 is not None else z for l in range(L)]
+    h_all = [ctx.empty((H * mb * T,)) for _ in range(L)]
+    c_all = [ctx.empty((H * mb * T,)) for _ in range(L)]
+    ctx.lstm_stack_forward([ly.w for ly in layers], ctx.array(embed), V, d_nn, d_m, T, mb, d_h0, d_c0, h_all, c_all,
+                           clip=clip)
+    ctx.sync()
+    hs = np.stack([a.get().reshape(T, mb, H).transpose(0, 2, 1) for a in h_all])
+    cs = np.stack([a.get().reshape(T, mb, H).transpose(0, 2, 1) for a in c_all])
+    for ly in layers:
+        ly.close()
+    return hs, cs
+
+
+def test_stack_forward_small_with_padding(ctx):
+    g = synth.rng(10, 1)
+    H, mb, T, V, L = 64, 5, 7, 211, 3
+    embed = U(g, (H, V))
+    layers = [synth.lstm_layer(g, H, forget_bias_one=True) for _ in range(L)]
+    ids = g.integers(0, V, size=(T, mb)).astype(np.int32)
+    ids[:3, 1] = -1  # left padding, as the source side is laid out
+    ids[:5, 4] = -1
+    hs, cs = _run_stack(ctx, layers, embed, ids)
+    nn, m = o.vocab_prep(ids)
+    want_h, want_c = o.lstm_stack_forward(embed, layers, nn, m)
+    assert_close(hs, want_h, what="stack h")
+    assert_close(cs, want_c, what="stack c")
+    assert np.all(hs[:, :3, :, 1] == 0) and np.all(cs[:, :5, :, 4] == 0)
+
+
+def test_config1_lm_forward_logprobs_and_loss(ctx):
+    """BASELINE config 1: 1-layer LM, H=100, mb=8, T=20, V=10000; per-step full log-probs and the summed loss."""
+    c = synth.config1()
+    H, mb, T, V = c["H"], c["mb"], c["T"], c["V"]
+    hs, _ = _run_stack(ctx, c["layers"], c["embed"], c["ids"])
+    nn, m = o.vocab_prep(c["ids"])
+    want_h, _ = o.lstm_stack_forward(c["embed"], c["layers"], nn, m)
+    assert_close(hs, want_h, what="LM h")
+    dD, dbd = ctx.array(c["D"]), ctx.array(c["b_d"])
+    d_logp, d_logp64, d_scr = ctx.empty((V, mb)), ctx.empty((V, mb), np.float64), ctx.empty((V, mb))
+    total, want_total = 0.0, 0.0
+    for t in range(T):
+        h_t = np.asfortranarray(hs[0, t])
+        d_h = ctx.array(h_t)
+        ctx.softmax_forward(dD, dbd, V, H, d_h, mb, capi.ZR_SOFTMAX_LOGPROB, d_logp)
+        ctx.softmax_logprob_f64(dD, dbd, V, H, d_h, mb, d_logp64, d_scr)
+        ctx.sync()
+        want = o.softmax_logprob_f64(o.softmax_logits(c["D"], c["b_d"], np.asfortranarray(want_h[0, t])))
+        assert_close(d_logp.get(), want, what="log-probs step %d" % t)
+        assert_close(d_logp64.get(), want, what="f64 log-probs step %d" % t)
+        tgt = c["targets"][t]
+        total += ctx.softmax_loss(dD, dbd, V, H, d_h, mb, ctx.array(tgt), ctx.array(np.ones(mb, np.int32)), d_scr)
+        want_total += o.softmax_loss(want, tgt, np.ones(mb, np.int32))
+    assert total == pytest.approx(want_total, rel=1e-5)
+
+
+# ------------------------------------------------------------------------------------------------ A8/A9 softmax
+@pytest.mark.parametrize("V,H,mb", [(211, 16, 6), (10000, 100, 8), (4099, 64, 33)])
+def test_softmax_prob_and_logprob(ctx, V, H, mb):
+    g = synth.rng(11, V)
+    D, bd, h = U(g, (V, H), -1, 1), U(g, (V,), -1, 1), U(g, (H, mb), -1, 1)
+    dD, dbd, dh = ctx.array(D), ctx.array(bd), ctx.array(h)
+    d_p, d_lp, d_scr = ctx.empty((V, mb)), ctx.empty((V, mb)), ctx.empty((V, mb))
+    ctx.softmax_forward(dD, dbd, V, H, dh, mb, capi.ZR_SOFTMAX_PROB, d_p, d_scr)
+    ctx.softmax_forward(dD, dbd, V, H, dh, mb, capi.ZR_SOFTMAX_LOGPROB, d_lp)  # in place on the logits
+    ctx.sync()
+    logits = o.softmax_logits(D, bd, h)
+    assert_close(d_scr.get(), logits, what="logits")
+    P = d_p.get()
+    assert_close(P, o.softmax_dist(logits), floor=1e-7, what="probabilities")
+    assert np.allclose(P.sum(axis=0, dtype=np.float64), 1.0, atol=1e-5)
+    assert np.array_equal(P.argmax(axis=0), logits.argmax(axis=0))
+    assert_close(d_lp.get(), o.softmax_logprob_f64(logits), what="log-probs")
+    # masked loss with out-of-order targets
+    tgt = g.integers(0, V, size=mb).astype(np.int32)
+    mask = (g.random(mb) > 0.3).astype(np.int32)
+    got = ctx.softmax_loss(dD, dbd, V, H, dh, mb, ctx.array(tgt), ctx.array(mask), d_scr)
+    assert got == pytest.approx(o.softmax_loss(o.softmax_logprob_f64(logits), tgt, mask), rel=1e-5, abs=1e-6)
+
+
+def test_softmax_extreme_logits_no_overflow(ctx):
+    V, H, mb = 512, 4, 3
+    D = np.zeros((V, H), np.float32, order="F")
+    D[:, 0] = np.where(np.arange(V) % 3 == 0, 80.0, -80.0)
+    h = np.zeros((H, mb), np.float32, order="F")
+    h[0, :] = [1.0, -1.0, 0.0]
+    d_p = ctx.empty((V, mb))
+    ctx.softmax_forward(ctx.array(D), ctx.zeros((V,)), V, H, ctx.array(h), mb, capi.ZR_SOFTMAX_PROB, d_p)
+    ctx.sync()
+    P = d_p.get()
+    assert np.all(np.isfinite(P)) and np.allclose(P.sum(axis=0, dtype=np.float64), 1.0, atol=1e-5)
+    assert np.allclose(P[:, 2], 1.0 / V)  # zero logits -> uniform
+
+
+def test_softmax_full_vocab_properties(ctx):
+    """V=50000, H=1000, mb=128 (the benchmark shape): size-independent properties plus an exact check of a
+    sampled set of columns against the oracle."""
+    g = synth.rng(12, 1)
+    V, H, mb = 50000, 1000, 128
+    D, bd = U(g, (V, H)), U(g, (V,))
+    h = np.tanh(U(g, (H, mb), -1, 1))
+    dD, dbd = ctx.array(D), ctx.array(bd)
+    d_p, d_scr = ctx.empty((V, mb)), ctx.empty((V, mb))
+    ctx.softmax_forward(dD, dbd, V, H, ctx.array(h), mb, capi.ZR_SOFTMAX_PROB, d_p, d_scr)
+    ctx.sync()
+    P, logits = d_p.get(), d_scr.get()
+    assert np.allclose(P.sum(axis=0, dtype=np.float64), 1.0, atol=1e-5)
+    assert np.array_equal(P.argmax(axis=0), logits.argmax(axis=0))
+    cols = [0, 31, 32, 77, 127]
+    want_logits = o.softmax_logits(D, bd, np.asfortranarray(h[:, cols]))
+    assert_close(logits[:, cols], want_logits, what="logits (sampled columns)")
+    assert_close(P[:, cols], o.softmax_dist(want_logits), floor=1e-7, what="probabilities (sampled columns)")
+
+
+# ------------------------------------------------------------------------------------------------ A10 attention
+def _run_attention(ctx, w, hs, batch_info, h_t, mask, D):
+    S, H, mb = hs.shape
+    tables = [ctx.array(np.asfortranarray(hs[t])) for t in range(S)]
+    dw = {k: ctx.array(v) for k, v in w.items()}
+    a = ctx.attn_create(H, mb, D, dw["W_a"], dw["W_p"], dw["v_p"], dw["out_bias"], dw["W_c1"], dw["W_c2"], tables)
+    Wn = 2 * D + 1
+    d_ht, d_al, d_ix, d_pt, d_cx = (ctx.empty((H, mb)), ctx.empty((mb, Wn)), ctx.empty((mb, Wn), np.int32),
+                                    ctx.empty((mb,)), ctx.empty((H, mb)))
+    ctx.attn_step(a, ctx.array(batch_info), ctx.array(h_t), ctx.array(mask), d_ht, d_al, d_ix, d_pt, d_cx)
+    ctx.sync()
+    out = {"h_tild": d_ht.get(), "alignments": d_al.get(), "indices": d_ix.get(), "p_t": d_pt.get(),
+           "c_ctx": d_cx.get()}
+    ctx.attn_destroy(a)
+    return out
+
+
+@pytest.mark.parametrize("H,mb,S,D", [(64, 6, 9, 2), (100, 8, 20, 10), (52, 33, 12, 12), (30, 5, 7, 3)])
+def test_attention_against_oracle(ctx, H, mb, S, D):
+    g = synth.rng(13, H + S)
+    w = synth.attention_weights(g, H)
+    for k in ("W_a", "W_p", "W_c1", "W_c2"):
+        w[k] = U(g, (H, H), -0.3, 0.3)
+    hs = (g.standard_normal(size=(S, H, mb), dtype=np.float32) * np.float32(0.5))
+    lens = g.integers(1, S + 1, size=mb).astype(np.int32)
+    lens[0] = S
+    batch_info = np.concatenate([lens, S - lens]).astype(np.int32)
+    mask = (g.random(mb) > 0.15).astype(np.int32)
+    h_t = U(g, (H, mb), -1, 1)
+    want = o.attention_forward(hs_table=hs, batch_info=batch_info, h_t=h_t, mask01=mask, D=D, **w)
+    got = _run_attention(ctx, w, hs, batch_info, h_t, mask, D)
+    assert_close(got["p_t"], want["p_t"], what="p_t")
+    # the window is floor(p_t) +- D: a p_t within rounding of an integer could legitimately move it
+    frac = want["p_t"] - np.floor(want["p_t"])
+    safe = (frac > 1e-4) & (frac < 1 - 1e-4)
+    assert safe.all(), "test inputs put p_t on an integer boundary; pick another seed"
+    assert np.array_equal(got["indices"], want["indices"])
+    assert_close(got["alignments"], want["alignments"], floor=1e-4, what="alignments")
+    assert_close(got["c_ctx"], want["c_ctx"], what="context")
+    assert_close(got["h_tild"], want["h_tild"], what="h_tild")
+    assert np.all(got["h_tild"][:, mask == 0] == 0)
+
+
+def test_attention_negative_scores_use_zero_initialised_max(ctx):
+    """All scores very negative: the reference's max starts at 0, exp underflows, the sum is 0 and the
+    alignments stay 0 (a -inf initialised max would give a normalised distribution instead)."""
+    H, mb, S, D = 8, 2, 5, 5
+    g = synth.rng(14, 1)
+    w = synth.attention_weights(g, H)
+    w["W_a"] = np.asfortranarray(-200.0 * np.eye(H, dtype=np.float32))
+    hs = np.ones((S, H, mb), np.float32)
+    h_t = np.ones((H, mb), np.float32, order="F")
+    bi = np.concatenate([np.full(mb, S, np.int32), np.zeros(mb, np.int32)])
+    got = _run_attention(ctx, w, hs, bi, h_t, np.ones(mb, np.int32), D)
+    want = o.attention_forward(hs_table=hs, batch_info=bi, h_t=h_t, mask01=np.ones(mb, np.int32), D=D, **w)
+    assert np.all(got["alignments"] == 0) and np.all(want["alignments"] == 0)
+    assert_close(got["h_tild"], want["h_tild"], what="h_tild")
+
+
+def test_config3_decoder_step_reduced_vocab(ctx):
+    """BASELINE config 3 wiring at H=1000, mb=128, S=50 with D=50 ("global") and D=10: LSTM stack with
+    feed-input on layer 0, attention on the top layer, softmax over a reduced vocabulary so that the oracle
+    finishes in seconds (the full-vocabulary softmax is covered by test_softmax_full_vocab_properties)."""
+    c = synth.decoder_config(V=2000)
+    H, mb, S, L, V = c["H"], c["mb"], c["S"], c["L"], c["V"]
+    mask = np.ones(mb, np.int32)
+    # oracle
+    x = o.embed_gather(c["embed"], c["ids"])
+    below, want_states = x, []
+    for l in range(L):
+        ly = c["layers"][l]
+        r = o.lstm_step(ly["M"], ly["Wh"], ly["b"], below, c["h_prev"][l], c["c_prev"][l], mask,
+                        Q=ly.get("Q"), htild=c["h_tild_prev"] if l == 0 else None)
+        want_states.append(r)
+        below = r["h"]
+    # HIP path
+    layers = [Layer(ctx, ly) for ly in c["layers"]]
+    d_x = ctx.empty((H, mb))
+    ctx.embed_gather(ctx.array(c["embed"]), H, V, ctx.array(c["ids"]), mb, d_x)
+    d_mask, d_ht_prev = ctx.array(mask), ctx.array(c["h_tild_prev"])
+    d_below, outs = d_x, []
+    for l in range(L):
+        d_h, d_c = ctx.empty((H, mb)), ctx.empty((H, mb))
+        ctx.lstm_step(layers[l].w, d_below, ctx.array(c["h_prev"][l]), ctx.array(c["c_prev"][l]), d_mask, mb, d_h,
+                      d_c, d_htild=d_ht_prev if l == 0 else None)
+        outs.append((d_h, d_c))
+        d_below = d_h
+    ctx.sync()
+    for l in range(L):
+        assert_close(outs[l][0].get(), want_states[l]["h"], what="layer %d h" % l)
+        assert_close(outs[l][1].get(), want_states[l]["c"], what="layer %d c" % l)
+    top_h = outs[-1][0].get()
+    for D in (50, 10):
+        want_att = o.attention_forward(hs_table=c["hs"], batch_info=c["batch_info"], h_t=top_h, mask01=mask, D=D,
+                                       **c["attn"])
+        got_att = _run_attention(ctx, c["attn"], c["hs"], c["batch_info"], top_h, mask, D)
+        frac = want_att["p_t"] - np.floor(want_att["p_t"])
+        safe = (frac > 1e-4) & (frac < 1 - 1e-4)
+        assert np.array_equal(got_att["indices"][safe], want_att["indices"][safe])
+        assert_close(got_att["alignments"][safe], want_att["alignments"][safe], floor=1e-4, what="alignments D=%d" % D)
+        assert_close(got_att["h_tild"][:, safe], want_att["h_tild"][:, safe], what="h_tild D=%d" % D)
+        if D == 50:  # every source position has a slot
+            assert np.all((want_att["indices"][:, :S] == np.arange(S)[None, :]))
+    d_lp = ctx.empty((V, mb))
+    ctx.softmax_forward(ctx.array(c["D"]), ctx.array(c["b_d"]), V, H, ctx.array(got_att["h_tild"]), mb,
+                        capi.ZR_SOFTMAX_LOGPROB, d_lp)
+    ctx.sync()
+    want_lp = o.softmax_logprob_f64(o.softmax_logits(c["D"], c["b_d"], got_att["h_tild"]))
+    assert_close(d_lp.get(), want_lp, what="log-probs")
+    for ly in layers:
+        ly.close()
+
+
+# ------------------------------------------------------------------------------------------------ error handling
+def test_bad_arguments_return_errors(ctx):
+    with pytest.raises(capi.ZrError) as e:
+        ctx.gemm(0, 0, 4, 4, 1, 1, 1, 1, 1, 1)
+    assert e.value.code == -1
+    with pytest.raises(capi.ZrError):
+        ctx.embed_gather(None, 8, 8, None, 4, None)
+    with pytest.raises(capi.ZrError):
+        ctx.lstm_step(None, 1, 1, 1, 1, 4, 1, 1)
+    g = synth.rng(15, 1)
+    layer = Layer(ctx, synth.lstm_layer(g, 16))
+    buf = ctx.zeros((16, 4))
+    with pytest.raises(capi.ZrError):  # feed-input requested on weights packed without Q
+        ctx.lstm_step(layer.w, buf, buf, buf, ctx.array(np.ones(4, np.int32)), 4, ctx.empty((16, 4)), ctx.empty((16, 4)),
+                      d_htild=buf)
+    layer.close()

@@ -1,0 +1,98 @@
+// Internal declarations shared by the HIP translation units of libzoph_rnn_hip.so.
+#ifndef ZR_INTERNAL_H
+#define ZR_INTERNAL_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/zoph_rnn.h"
+
+struct zr_ctx {
+  int device;
+  hipStream_t own_stream;
+  hipStream_t stream;  // the stream in use (own_stream or a caller-provided one)
+  int* d_flags;        // [0]: count of token ids seen outside [0, V); [1]: attention table index clamps
+  hipEvent_t ev_start, ev_stop;  // zr_timer_start / zr_timer_stop
+  // options
+  int lstm_fused;
+  int lstm_tn;
+  int lstm_ksplit;
+  int gemm_cfg;
+  // scratch owned by the context (grown on demand, never shrunk)
+  void* d_scratch;
+  size_t scratch_bytes;
+  void* d_scratch2;
+  size_t scratch2_bytes;
+};
+
+// error plumbing -------------------------------------------------------------------------------------------
+int zr_set_error(int code, const char* fmt, ...);
+
+#define ZR_CHECK_ARG(cond, ...)                  \
+  do {                                           \
+    if (!(cond)) return zr_set_error(ZR_EINVAL, __VA_ARGS__); \
+  } while (0)
+
+#define ZR_HIP(call)                                                                        \
+  do {                                                                                      \
+    hipError_t zr_e_ = (call);                                                              \
+    if (zr_e_ != hipSuccess)                                                                \
+      return zr_set_error(ZR_EHIP, "%s failed: %s (%s:%d)", #call, hipGetErrorString(zr_e_), \
+                          __FILE__, __LINE__);                                              \
+  } while (0)
+
+#define ZR_LAUNCH_CHECK(name)                                                                  \
+  do {                                                                                         \
+    hipError_t zr_e_ = hipGetLastError();                                                      \
+    if (zr_e_ != hipSuccess)                                                                   \
+      return zr_set_error(ZR_EHIP, "launch of %s failed: %s", name, hipGetErrorString(zr_e_)); \
+  } while (0)
+
+int zr_bind_device(zr_ctx* ctx);
+// Returns a context-owned scratch buffer of at least `bytes` (slot 0 or 1).
+int zr_ctx_scratch(zr_ctx* ctx, int slot, size_t bytes, void** out);
+
+// MFMA vector types ------------------------------------------------------------------------------------------
+typedef float zr_f32x16 __attribute__((ext_vector_type(16)));
+typedef float zr_f32x4 __attribute__((ext_vector_type(4)));
+
+// Generic multi-segment GEMM: C = sum_s op(A_s) * B_s, then an epilogue.  Up to 3 segments.
+enum ZrEpilogue {
+  ZR_EPI_STORE = 0,           // C = acc (+ bias[m] if bias)
+  ZR_EPI_TANH = 1,            // C = tanhf(acc)
+  ZR_EPI_TANH_BIAS_MASK = 2,  // C = tanhf(acc + bias[m]) * mask[n]
+  ZR_EPI_SOFTMAX_PARTIAL = 3  // C = acc + bias[m]; per (32-row block, n) partial (max, sum exp) -> partials
+};
+
+struct ZrGemmDesc {
+  int M, N;
+  int nseg;
+  int K[3];
+  const float* A[3];
+  int lda[3];
+  int trans_a;  // applies to every segment
+  const float* B[3];
+  int ldb[3];
+  float* C;
+  int ldc;
+  // batch (blockIdx.z): A/C/bias advance by these strides (elements); B is shared
+  int batch;
+  long long strideA, strideC, strideBias;
+  const float* bias;  // per row m (may be NULL)
+  const int* mask;    // per column n (ZR_EPI_TANH_BIAS_MASK)
+  int epilogue;
+  float* partials;  // ZR_EPI_SOFTMAX_PARTIAL: [ceil(M/32)][N][2] floats
+};
+
+int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d);
+// number of 32-row partial blocks the SOFTMAX_PARTIAL epilogue writes for M rows
+static inline int zr_softmax_partial_blocks(int M) { return (M + 31) / 32; }
+
+struct zr_lstm_weights {
+  int H;
+  int nseg;        // 2 (M, Wh) or 3 (+Q)
+  float* d_W;      // [nseg][4][H*H] column-major blocks
+  float* d_bias;   // [4][H]
+};
+
+#endif

@@ -1,0 +1,176 @@
+// fp32 MFMA contraction core for gfx950 (64-lane waves, v_mfma_f32_32x32x2_f32).
+//
+// Shape of the work: every GEMM on this path is  C(M x N) = W(M x K) * X(K x N)  with a large weight matrix W
+// streamed once, and a small activation matrix X (N = minibatch <= a few hundred columns).  Both are
+// column-major, so W is contiguous along M and X is contiguous along K.
+//
+// Operand mapping.  The instruction computes D(32x32) += a(32x2) * b(2x32); lane l supplies a[l%32][l/32]
+// and b[l/32][l%32], and holds D[8*(r/4) + 4*(l/32) + r%4][l%32] in accumulator register r.  We put the
+// ACTIVATIONS on the a side (D row = batch column n) and the WEIGHTS on the b side (D column = output row m):
+// then lane%32 indexes m, so the 32 lanes of a half-wave read 32 consecutive floats of a weight column
+// (one 128-byte line) and write 32 consecutive floats of an output column -- every weight load and every
+// output store is a full-line access, straight from/to registers, with no LDS transpose.
+//
+// K order.  Within a group of 8 consecutive k, lanes 0-31 take k0..k0+3 and lanes 32-63 take k0+4..k0+7, one k
+// per MFMA: the i-th MFMA of the group multiplies k0+i (half 0) and k0+4+i (half 1).  Any pairing of k values
+// is valid as long as both operands use the same one; this one lets each lane fetch its four activation
+// values of a group with a single 16-byte load along K.
+//
+// Split K.  KS waves of a workgroup may share one output tile and take the k-groups round-robin; their
+// partial tiles are summed through LDS in a fixed order (deterministic) before the epilogue runs.
+#ifndef ZR_MFMA_CORE_H
+#define ZR_MFMA_CORE_H
+
+#include "zr_internal.h"
+
+template <int TM, int TN>
+struct ZrFrag {
+  float x[TN][4];  // activations: x[tn][i] = X[k_i][n(tn, lane%32)]
+  float w[TM][4];  // weights:     w[tm][i] = W[m(tm, lane%32)][k_i]
+};
+
+// One K segment.  `wbase[tm]` points at this lane's weight row (NN: &W[row][0] with stride lda between k;
+// TRANS_A: &W^T storage of that row, contiguous in k).  `xcol[tn]` points at this lane's activation column.
+// Addresses are pre-clamped by the caller so that out-of-range rows/columns read valid memory.
+template <int TM, int TN, int KS, bool TRANS_A, bool VEC>
+__device__ __forceinline__ void zr_mma_segment(zr_f32x16 (&acc)[TM][TN], const float* const (&wbase)[TM],
+                                               long long lda, const float* const (&xcol)[TN], int K, int kslice,
+                                               int half) {
+  const int nfull = K >> 3;
+
+  auto load_full = [&](ZrFrag<TM, TN>& f, int g) {
+    const int k0 = g * 8 + 4 * half;
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+      if (VEC) {
+        const zr_f32x4 v = *(const zr_f32x4*)(xcol[tn] + k0);
+        f.x[tn][0] = v.x;
+        f.x[tn][1] = v.y;
+        f.x[tn][2] = v.z;
+        f.x[tn][3] = v.w;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) f.x[tn][i] = xcol[tn][k0 + i];
+      }
+    }
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+      if (TRANS_A) {
+        if (VEC) {
+          const zr_f32x4 v = *(const zr_f32x4*)(wbase[tm] + k0);
+          f.w[tm][0] = v.x;
+          f.w[tm][1] = v.y;
+          f.w[tm][2] = v.z;
+          f.w[tm][3] = v.w;
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) f.w[tm][i] = wbase[tm][k0 + i];
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) f.w[tm][i] = wbase[tm][(long long)(k0 + i) * lda];
+      }
+    }
+  };
+
+  auto mma = [&](const ZrFrag<TM, TN>& f) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.x[tn][i], f.w[tm][i], acc[tm][tn], 0, 0, 0);
+  };
+
+  ZrFrag<TM, TN> f0, f1;
+  int g = kslice;
+  if (g < nfull) {
+    load_full(f0, g);
+    while (true) {
+      const int g1 = g + KS;
+      if (g1 < nfull) load_full(f1, g1);
+      mma(f0);
+      if (g1 >= nfull) break;
+      const int g2 = g1 + KS;
+      if (g2 < nfull) load_full(f0, g2);
+      mma(f1);
+      if (g2 >= nfull) break;
+      g = g2;
+    }
+  }
+  // tail group (K not a multiple of 8): zero-filled, owned by the slice whose turn it is
+  if ((K & 7) != 0 && (nfull % KS) == kslice) {
+    const int k0 = nfull * 8 + 4 * half;
+    ZrFrag<TM, TN> f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int k = k0 + i;
+      const bool ok = k < K;
+      const int kc = ok ? k : K - 1;
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) {
+        const float v = xcol[tn][kc];
+        f.x[tn][i] = ok ? v : 0.0f;
+      }
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) {
+        const float v = TRANS_A ? wbase[tm][kc] : wbase[tm][(long long)kc * lda];
+        f.w[tm][i] = ok ? v : 0.0f;
+      }
+    }
+    mma(f);
+  }
+}
+
+// Sums the KS partial tiles of a workgroup and calls f(vals[TM], tn, r) once per (tn, r, lane) owned by the
+// calling thread, where vals[tm] is the finished accumulator register r of sub-tile (tm, tn) for this lane.
+// Every lane of a wave calls f with the same (tn, r) at the same time (wave-uniform control flow), and a
+// thread keeps its lane index, so the caller's mapping  m <- lane%32,  n <- 8*(r/4) + 4*(lane/32) + r%4  holds.
+// `red` is LDS of KS * TN*16 * 64 floats (unused when KS == 1).  All threads of the workgroup must call this.
+template <int TM, int TN, int KS, class F>
+__device__ __forceinline__ void zr_reduce_visit(zr_f32x16 (&acc)[TM][TN], float* red, int kslice, int lane, F f) {
+  if (KS == 1) {
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        float vals[TM];
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) vals[tm] = acc[tm][tn][r];
+        f(vals, tn, r);
+      }
+  } else {
+    constexpr int SLOTS = TN * 16;           // accumulator registers per sub-tile row of the tile
+    constexpr int PT = SLOTS / KS;           // slots finished by each wave
+    static_assert(SLOTS % KS == 0, "KS must divide TN*16");
+    float pre[TM][PT];
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+      __syncthreads();  // previous round's reads are done
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) red[((size_t)kslice * SLOTS + tn * 16 + r) * 64 + lane] = acc[tm][tn][r];
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < PT; ++i) {
+        const int slot = kslice + KS * i;
+        float s = 0.0f;
+#pragma unroll
+        for (int w = 0; w < KS; ++w) s += red[((size_t)w * SLOTS + slot) * 64 + lane];
+        pre[tm][i] = s;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < PT; ++i) {
+      const int slot = kslice + KS * i;
+      float vals[TM];
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) vals[tm] = pre[tm][i];
+      f(vals, slot / 16, slot % 16);
+    }
+  }
+}
+
+#endif

@@ -1,0 +1,211 @@
+// Context, error reporting and device memory helpers of the C-ABI.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "zr_internal.h"
+
+static thread_local char g_err[512] = "";
+
+int zr_set_error(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int zr_bind_device(zr_ctx* ctx) {
+  ZR_CHECK_ARG(ctx != nullptr, "null context");
+  ZR_HIP(hipSetDevice(ctx->device));
+  return ZR_OK;
+}
+
+int zr_ctx_scratch(zr_ctx* ctx, int slot, size_t bytes, void** out) {
+  void** buf = slot == 0 ? &ctx->d_scratch : &ctx->d_scratch2;
+  size_t* cap = slot == 0 ? &ctx->scratch_bytes : &ctx->scratch2_bytes;
+  if (*cap < bytes) {
+    // the old buffer may still be in use by queued kernels: drain the stream before releasing it
+    ZR_HIP(hipStreamSynchronize(ctx->stream));
+    if (*buf) ZR_HIP(hipFree(*buf));
+    *buf = nullptr;
+    *cap = 0;
+    size_t want = bytes + bytes / 4;
+    if (hipMalloc(buf, want) != hipSuccess) {
+      (void)hipGetLastError();
+      return zr_set_error(ZR_ENOMEM, "scratch allocation of %zu bytes failed", want);
+    }
+    *cap = want;
+  }
+  *out = *buf;
+  return ZR_OK;
+}
+
+extern "C" {
+
+const char* zr_last_error(void) { return g_err; }
+
+const char* zr_version(void) { return "gfx950 hip zoph_rnn_amd 0.1"; }
+
+int zr_ctx_create(int device, zr_ctx** out) {
+  ZR_CHECK_ARG(out != nullptr, "zr_ctx_create: out is null");
+  *out = nullptr;
+  int ndev = 0;
+  ZR_HIP(hipGetDeviceCount(&ndev));
+  ZR_CHECK_ARG(device >= 0 && device < ndev, "zr_ctx_create: device %d not in [0,%d)", device, ndev);
+  ZR_HIP(hipSetDevice(device));
+  zr_ctx* c = new zr_ctx();
+  memset(c, 0, sizeof(*c));
+  c->device = device;
+  hipError_t e = hipStreamCreate(&c->own_stream);  // default priority
+  if (e != hipSuccess) {
+    delete c;
+    return zr_set_error(ZR_EHIP, "hipStreamCreate failed: %s", hipGetErrorString(e));
+  }
+  c->stream = c->own_stream;
+  e = hipMalloc((void**)&c->d_flags, 4 * sizeof(int));
+  if (e != hipSuccess) {
+    (void)hipStreamDestroy(c->own_stream);
+    delete c;
+    return zr_set_error(ZR_ENOMEM, "flag allocation failed: %s", hipGetErrorString(e));
+  }
+  (void)hipMemset(c->d_flags, 0, 4 * sizeof(int));
+  c->lstm_fused = 1;
+  *out = c;
+  return ZR_OK;
+}
+
+int zr_ctx_destroy(zr_ctx* ctx) {
+  if (!ctx) return ZR_OK;
+  (void)hipSetDevice(ctx->device);
+  (void)hipStreamSynchronize(ctx->stream);
+  if (ctx->d_scratch) (void)hipFree(ctx->d_scratch);
+  if (ctx->d_scratch2) (void)hipFree(ctx->d_scratch2);
+  if (ctx->d_flags) (void)hipFree(ctx->d_flags);
+  if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
+  if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);
+  (void)hipStreamDestroy(ctx->own_stream);
+  delete ctx;
+  return ZR_OK;
+}
+
+int zr_ctx_sync(zr_ctx* ctx) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_HIP(hipStreamSynchronize(ctx->stream));
+  ZR_LAUNCH_CHECK("queued work");
+  int flags[4] = {0, 0, 0, 0};
+  ZR_HIP(hipMemcpy(flags, ctx->d_flags, sizeof(flags), hipMemcpyDeviceToHost));
+  if (flags[0] != 0 || flags[1] != 0) {
+    ZR_HIP(hipMemset(ctx->d_flags, 0, sizeof(flags)));
+    return zr_set_error(ZR_EDATA, "%d token id(s) outside [0, vocab) and %d source position(s) outside the "
+                        "attention table were clamped", flags[0], flags[1]);
+  }
+  return ZR_OK;
+}
+
+int zr_ctx_set_stream(zr_ctx* ctx, void* hip_stream) {
+  ZR_CHECK_ARG(ctx != nullptr, "null context");
+  ctx->stream = hip_stream ? (hipStream_t)hip_stream : ctx->own_stream;
+  return ZR_OK;
+}
+
+int zr_ctx_set_option(zr_ctx* ctx, int option, int value) {
+  ZR_CHECK_ARG(ctx != nullptr, "null context");
+  switch (option) {
+    case ZR_OPT_LSTM_FUSED_EPILOGUE:
+      ctx->lstm_fused = value ? 1 : 0;
+      return ZR_OK;
+    case ZR_OPT_LSTM_TN:
+      ZR_CHECK_ARG(value == 0 || value == 1 || value == 2 || value == 4, "ZR_OPT_LSTM_TN must be 0, 1, 2 or 4");
+      ctx->lstm_tn = value;
+      return ZR_OK;
+    case ZR_OPT_LSTM_KSPLIT:
+      ZR_CHECK_ARG(value == 0 || value == 4 || value == 8, "ZR_OPT_LSTM_KSPLIT must be 0, 4 or 8");
+      ctx->lstm_ksplit = value;
+      return ZR_OK;
+    case ZR_OPT_GEMM_CFG:
+      ZR_CHECK_ARG(value >= 0 && value <= 8, "ZR_OPT_GEMM_CFG out of range");
+      ctx->gemm_cfg = value;
+      return ZR_OK;
+    default:
+      return zr_set_error(ZR_EINVAL, "unknown option %d", option);
+  }
+}
+
+int zr_malloc(zr_ctx* ctx, size_t bytes, void** d_out) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(d_out != nullptr, "zr_malloc: out is null");
+  *d_out = nullptr;
+  if (bytes == 0) bytes = 4;
+  if (hipMalloc(d_out, bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    return zr_set_error(ZR_ENOMEM, "hipMalloc of %zu bytes failed", bytes);
+  }
+  return ZR_OK;
+}
+
+int zr_free(zr_ctx* ctx, void* d_ptr) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  if (!d_ptr) return ZR_OK;
+  ZR_HIP(hipStreamSynchronize(ctx->stream));
+  ZR_HIP(hipFree(d_ptr));
+  return ZR_OK;
+}
+
+int zr_h2d(zr_ctx* ctx, void* d_dst, const void* h_src, size_t bytes) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(bytes == 0 || (d_dst && h_src), "zr_h2d: null pointer");
+  if (bytes == 0) return ZR_OK;
+  // pageable host memory: the runtime stages the copy, and it is ordered after earlier work on the stream
+  ZR_HIP(hipMemcpyAsync(d_dst, h_src, bytes, hipMemcpyHostToDevice, ctx->stream));
+  ZR_HIP(hipStreamSynchronize(ctx->stream));
+  return ZR_OK;
+}
+
+int zr_d2h(zr_ctx* ctx, void* h_dst, const void* d_src, size_t bytes) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(bytes == 0 || (h_dst && d_src), "zr_d2h: null pointer");
+  if (bytes == 0) return ZR_OK;
+  ZR_HIP(hipMemcpyAsync(h_dst, d_src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+  ZR_HIP(hipStreamSynchronize(ctx->stream));
+  return ZR_OK;
+}
+
+int zr_d2d(zr_ctx* ctx, void* d_dst, const void* d_src, size_t bytes) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(bytes == 0 || (d_dst && d_src), "zr_d2d: null pointer");
+  if (bytes == 0) return ZR_OK;
+  ZR_HIP(hipMemcpyAsync(d_dst, d_src, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+  return ZR_OK;
+}
+
+}  // extern "C"
+
+// Stream timer: two HIP events on the context's stream (the reference wraps phases in host wall-clock Timer
+// objects after a device synchronise, src/memory_util.h:87-124).
+extern "C" int zr_timer_start(zr_ctx* ctx) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  if (!ctx->ev_start) {
+    ZR_HIP(hipEventCreate(&ctx->ev_start));
+    ZR_HIP(hipEventCreate(&ctx->ev_stop));
+  }
+  ZR_HIP(hipEventRecord(ctx->ev_start, ctx->stream));
+  return ZR_OK;
+}
+
+extern "C" int zr_timer_stop(zr_ctx* ctx, float* h_ms) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(ctx->ev_start != nullptr && h_ms != nullptr, "zr_timer_stop: no running timer or null output");
+  ZR_HIP(hipEventRecord(ctx->ev_stop, ctx->stream));
+  ZR_HIP(hipEventSynchronize(ctx->ev_stop));
+  ZR_HIP(hipEventElapsedTime(h_ms, ctx->ev_start, ctx->ev_stop));
+  return ZR_OK;
+}

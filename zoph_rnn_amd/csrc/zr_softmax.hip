@@ -1,0 +1,271 @@
+// Output softmax: logits on MFMA (bias and per-32-row (max, sum exp) partials fused into the GEMM epilogue),
+// then one read + one write of the V x mb matrix to normalise.
+#include <math.h>
+
+#include "zr_internal.h"
+
+namespace {
+
+// Combines the per-32-row partials of one column into (max, sum exp(x - max)).  One workgroup per column.
+__global__ void __launch_bounds__(256)
+softmax_colstats_kernel(const float* __restrict__ partials, int nblocks, int N, float* __restrict__ colstats) {
+  __shared__ float s_m[256];
+  __shared__ float s_s[256];
+  const int n = blockIdx.x;
+  const int tid = threadIdx.x;
+  float mx = -INFINITY;
+  for (int b = tid; b < nblocks; b += 256) mx = fmaxf(mx, partials[((size_t)b * N + n) * 2]);
+  s_m[tid] = mx;
+  __syncthreads();
+  for (int st = 128; st > 0; st >>= 1) {
+    if (tid < st) s_m[tid] = fmaxf(s_m[tid], s_m[tid + st]);
+    __syncthreads();
+  }
+  mx = s_m[0];
+  float sum = 0.0f;
+  for (int b = tid; b < nblocks; b += 256) {
+    const float* p = partials + ((size_t)b * N + n) * 2;
+    sum += p[1] * expf(p[0] - mx);
+  }
+  s_s[tid] = sum;
+  __syncthreads();
+  for (int st = 128; st > 0; st >>= 1) {
+    if (tid < st) s_s[tid] += s_s[tid + st];
+    __syncthreads();
+  }
+  if (tid == 0) {
+    colstats[2 * n] = mx;
+    colstats[2 * n + 1] = s_s[0];
+  }
+}
+
+// out = exp(x - max) / sum   (MODE 0)   or   (x - max) - log(sum)   (MODE 1).  16-byte accesses when VEC.
+template <int MODE, bool VEC>
+__global__ void __launch_bounds__(256)
+softmax_normalize_kernel(const float* in, float* out, int V, const float* __restrict__ colstats) {
+  const int n = blockIdx.y;
+  const float mx = colstats[2 * n];
+  const float sum = colstats[2 * n + 1];
+  const float inv = 1.0f / sum;
+  const float lsum = logf(sum);
+  const float* x = in + (size_t)n * V;
+  float* y = out + (size_t)n * V;
+  if (VEC) {
+    const int i4 = blockIdx.x * 256 + threadIdx.x;
+    if (i4 * 4 < V) {
+      zr_f32x4 v = ((const zr_f32x4*)x)[i4];
+      zr_f32x4 r;
+      if (MODE == 0) {
+        // expf(x - max) / sum, as the reference divides (custom_kernels.h:574-576)
+        r.x = expf(v.x - mx) / sum;
+        r.y = expf(v.y - mx) / sum;
+        r.z = expf(v.z - mx) / sum;
+        r.w = expf(v.w - mx) / sum;
+      } else {
+        r.x = (v.x - mx) - lsum;
+        r.y = (v.y - mx) - lsum;
+        r.z = (v.z - mx) - lsum;
+        r.w = (v.w - mx) - lsum;
+      }
+      ((zr_f32x4*)y)[i4] = r;
+    }
+  } else {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < V) y[i] = (MODE == 0) ? expf(x[i] - mx) / sum : (x[i] - mx) - lsum;
+  }
+  (void)inv;
+}
+
+// Double-precision column statistics straight from the logits (outputdist_perplexity_kernel accumulates in
+// double, reference: src/custom_kernels.h:583-660).  One workgroup per column, two passes over the column.
+__global__ void __launch_bounds__(256)
+softmax_colstats_f64_kernel(const float* __restrict__ logits, int V, double* __restrict__ colstats) {
+  __shared__ double s[256];
+  const int n = blockIdx.x;
+  const int tid = threadIdx.x;
+  const float* x = logits + (size_t)n * V;
+  double mx = -1.7976931348623157e308;
+  for (int i = tid; i < V; i += 256) mx = fmax(mx, (double)x[i]);
+  s[tid] = mx;
+  __syncthreads();
+  for (int st = 128; st > 0; st >>= 1) {
+    if (tid < st) s[tid] = fmax(s[tid], s[tid + st]);
+    __syncthreads();
+  }
+  mx = s[0];
+  __syncthreads();
+  double sum = 0.0;
+  for (int i = tid; i < V; i += 256) sum += exp((double)x[i] - mx);
+  s[tid] = sum;
+  __syncthreads();
+  for (int st = 128; st > 0; st >>= 1) {
+    if (tid < st) s[tid] += s[tid + st];
+    __syncthreads();
+  }
+  if (tid == 0) {
+    colstats[2 * n] = mx;
+    colstats[2 * n + 1] = log(s[0]);
+  }
+}
+
+__global__ void __launch_bounds__(256)
+softmax_logprob_f64_kernel(const float* __restrict__ logits, double* __restrict__ out, int V,
+                           const double* __restrict__ colstats) {
+  const int n = blockIdx.y;
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < V) out[(size_t)n * V + i] = ((double)logits[(size_t)n * V + i] - colstats[2 * n]) - colstats[2 * n + 1];
+}
+
+// loss = sum over unmasked columns of log p[target[b], b]; single workgroup, fixed summation order.
+__global__ void __launch_bounds__(256)
+softmax_loss_kernel(const float* __restrict__ logits, int V, int mb, const double* __restrict__ colstats,
+                    const int* __restrict__ target, const int* __restrict__ mask01, double* __restrict__ loss,
+                    int* __restrict__ flags) {
+  __shared__ double s[256];
+  const int tid = threadIdx.x;
+  double acc = 0.0;
+  for (int b = tid; b < mb; b += 256) {
+    if (mask01[b] == 1) {
+      int t = target[b];
+      if (t < 0 || t >= V) {
+        atomicAdd(&flags[0], 1);
+        t = t < 0 ? 0 : V - 1;
+      }
+      acc += ((double)logits[(size_t)b * V + t] - colstats[2 * b]) - colstats[2 * b + 1];
+    }
+  }
+  s[tid] = acc;
+  __syncthreads();
+  for (int st = 128; st > 0; st >>= 1) {
+    if (tid < st) s[tid] += s[tid + st];
+    __syncthreads();
+  }
+  if (tid == 0) loss[0] = s[0];
+}
+
+int logits_with_partials(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int mb,
+                         float* d_logits, float** partials_out, int* nblocks_out) {
+  const int nblocks = zr_softmax_partial_blocks(V);
+  void* scratch = nullptr;
+  // partials [nblocks][mb][2] followed by column stats (2 doubles per column, also used as 2 floats)
+  const size_t pbytes = sizeof(float) * 2 * (size_t)nblocks * mb;
+  int rc = zr_ctx_scratch(ctx, 1, pbytes + sizeof(double) * 2 * (size_t)mb + 64, &scratch);
+  if (rc) return rc;
+  ZrGemmDesc d = {};
+  d.M = V;
+  d.N = mb;
+  d.nseg = 1;
+  d.K[0] = H;
+  d.A[0] = d_D;
+  d.lda[0] = V;
+  d.B[0] = d_h;
+  d.ldb[0] = H;
+  d.C = d_logits;
+  d.ldc = V;
+  d.batch = 1;
+  d.bias = d_b_d;
+  d.epilogue = ZR_EPI_SOFTMAX_PARTIAL;
+  d.partials = (float*)scratch;
+  rc = zr_gemm_launch(ctx, d);
+  if (rc) return rc;
+  *partials_out = (float*)scratch;
+  *nblocks_out = nblocks;
+  return ZR_OK;
+}
+
+inline void* stats_ptr(float* partials, int nblocks, int mb) {
+  size_t off = sizeof(float) * 2 * (size_t)nblocks * mb;
+  off = (off + 63) & ~(size_t)63;
+  return (char*)partials + off;
+}
+
+int check_softmax_args(const char* who, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int mb) {
+  ZR_CHECK_ARG(V > 0 && H > 0 && mb > 0, "%s: V = %d, H = %d, mb = %d", who, V, H, mb);
+  ZR_CHECK_ARG(mb <= 65535, "%s: mb = %d exceeds 65535", who, mb);
+  ZR_CHECK_ARG(d_D && d_b_d && d_h, "%s: null pointer", who);
+  return ZR_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int zr_softmax_forward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int mb,
+                       int mode, float* d_out, float* d_logits_scratch) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  rc = check_softmax_args("zr_softmax_forward", d_D, d_b_d, V, H, d_h, mb);
+  if (rc) return rc;
+  ZR_CHECK_ARG(d_out != nullptr, "zr_softmax_forward: d_out is null");
+  ZR_CHECK_ARG(mode == ZR_SOFTMAX_PROB || mode == ZR_SOFTMAX_LOGPROB, "zr_softmax_forward: mode = %d", mode);
+  float* logits = d_logits_scratch ? d_logits_scratch : d_out;
+  float* partials = nullptr;
+  int nblocks = 0;
+  rc = logits_with_partials(ctx, d_D, d_b_d, V, H, d_h, mb, logits, &partials, &nblocks);
+  if (rc) return rc;
+  float* colstats = (float*)stats_ptr(partials, nblocks, mb);
+  softmax_colstats_kernel<<<mb, 256, 0, ctx->stream>>>(partials, nblocks, mb, colstats);
+  ZR_LAUNCH_CHECK("softmax_colstats_kernel");
+  const bool vec = (V % 4 == 0) && (((uintptr_t)logits & 15u) == 0) && (((uintptr_t)d_out & 15u) == 0);
+  if (vec) {
+    dim3 grid((V / 4 + 255) / 256, mb);
+    if (mode == ZR_SOFTMAX_PROB)
+      softmax_normalize_kernel<0, true><<<grid, 256, 0, ctx->stream>>>(logits, d_out, V, colstats);
+    else
+      softmax_normalize_kernel<1, true><<<grid, 256, 0, ctx->stream>>>(logits, d_out, V, colstats);
+  } else {
+    dim3 grid((V + 255) / 256, mb);
+    if (mode == ZR_SOFTMAX_PROB)
+      softmax_normalize_kernel<0, false><<<grid, 256, 0, ctx->stream>>>(logits, d_out, V, colstats);
+    else
+      softmax_normalize_kernel<1, false><<<grid, 256, 0, ctx->stream>>>(logits, d_out, V, colstats);
+  }
+  ZR_LAUNCH_CHECK("softmax_normalize_kernel");
+  return ZR_OK;
+}
+
+int zr_softmax_logprob_f64(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int mb,
+                           double* d_logp, float* d_logits_scratch) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  rc = check_softmax_args("zr_softmax_logprob_f64", d_D, d_b_d, V, H, d_h, mb);
+  if (rc) return rc;
+  ZR_CHECK_ARG(d_logp && d_logits_scratch, "zr_softmax_logprob_f64: null output or scratch");
+  float* partials = nullptr;
+  int nblocks = 0;
+  rc = logits_with_partials(ctx, d_D, d_b_d, V, H, d_h, mb, d_logits_scratch, &partials, &nblocks);
+  if (rc) return rc;
+  double* colstats = (double*)stats_ptr(partials, nblocks, mb);
+  softmax_colstats_f64_kernel<<<mb, 256, 0, ctx->stream>>>(d_logits_scratch, V, colstats);
+  ZR_LAUNCH_CHECK("softmax_colstats_f64_kernel");
+  dim3 grid((V + 255) / 256, mb);
+  softmax_logprob_f64_kernel<<<grid, 256, 0, ctx->stream>>>(d_logits_scratch, d_logp, V, colstats);
+  ZR_LAUNCH_CHECK("softmax_logprob_f64_kernel");
+  return ZR_OK;
+}
+
+int zr_softmax_loss(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int mb,
+                    const int* d_target, const int* d_mask01, float* d_logits_scratch, double* h_loss) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  rc = check_softmax_args("zr_softmax_loss", d_D, d_b_d, V, H, d_h, mb);
+  if (rc) return rc;
+  ZR_CHECK_ARG(d_target && d_mask01 && d_logits_scratch && h_loss, "zr_softmax_loss: null pointer");
+  float* partials = nullptr;
+  int nblocks = 0;
+  rc = logits_with_partials(ctx, d_D, d_b_d, V, H, d_h, mb, d_logits_scratch, &partials, &nblocks);
+  if (rc) return rc;
+  double* colstats = (double*)stats_ptr(partials, nblocks, mb);
+  softmax_colstats_f64_kernel<<<mb, 256, 0, ctx->stream>>>(d_logits_scratch, V, colstats);
+  ZR_LAUNCH_CHECK("softmax_colstats_f64_kernel");
+  // the loss cell lives in the partials area, which is dead once the column stats exist
+  double* d_loss = (double*)partials;
+  softmax_loss_kernel<<<1, 256, 0, ctx->stream>>>(d_logits_scratch, V, mb, colstats, d_target, d_mask01, d_loss,
+                                                  ctx->d_flags);
+  ZR_LAUNCH_CHECK("softmax_loss_kernel");
+  ZR_HIP(hipMemcpyAsync(h_loss, d_loss, sizeof(double), hipMemcpyDeviceToHost, ctx->stream));
+  ZR_HIP(hipStreamSynchronize(ctx->stream));
+  return ZR_OK;
+}
+
+}  // extern "C"
