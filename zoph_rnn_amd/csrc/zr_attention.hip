@@ -82,34 +82,39 @@ attn_score_kernel(const float* const* __restrict__ table, int longest_sent, cons
   if (lane == 0) align[slot] = acc;
 }
 
-// alignment_reduction_kernel (src/custom_kernels.h:1752-1794): one thread per column; max starts at 0.
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+// alignment_reduction_kernel (src/custom_kernels.h:1752-1794): the reference runs one thread per column; here
+// one wave per column with the window slots spread over the lanes.  The max starts at 0 as in the reference.
 __global__ void __launch_bounds__(64)
 attn_align_kernel(float* __restrict__ align, const int* __restrict__ indices, const float* __restrict__ p_t, int mb,
                   int W, float sigma_sq) {
-  const int b = blockIdx.x * 64 + threadIdx.x;
-  if (b >= mb) return;
-  float max_val = 0.0f, sum = 0.0f;
-  for (int j = 0; j < W; ++j)
+  const int b = blockIdx.x;
+  const int lane = threadIdx.x;
+  float max_val = 0.0f;
+  for (int j = lane; j < W; j += 64)
     if (indices[b + (size_t)mb * j] != -1) max_val = fmaxf(max_val, align[b + (size_t)mb * j]);
-  for (int j = 0; j < W; ++j) {
-    const size_t ix = b + (size_t)mb * j;
-    if (indices[ix] != -1) {
-      const float e = expf(align[ix] - max_val);
-      align[ix] = e;
-      sum += e;
-    } else {
-      align[ix] = 0.0f;
-    }
-  }
+  max_val = wave_max(max_val);
+  float sum = 0.0f;
+  for (int j = lane; j < W; j += 64)
+    if (indices[b + (size_t)mb * j] != -1) sum += expf(align[b + (size_t)mb * j] - max_val);
+  sum = wave_sum(sum);
   const float p = p_t[b];
-  for (int j = 0; j < W; ++j) {
+  for (int j = lane; j < W; j += 64) {
     const size_t ix = b + (size_t)mb * j;
     const int s_idx = indices[ix];
+    float a = 0.0f;
     if (s_idx != -1) {
+      a = expf(align[ix] - max_val);
       const float d = p - (float)s_idx;
       const float g = expf((-1.0f * d * d) / (2.0f * sigma_sq));
-      if (sum != 0.0f) align[ix] = (align[ix] / sum) * g;
+      if (sum != 0.0f) a = (a / sum) * g;
     }
+    align[ix] = a;
   }
 }
 
@@ -119,21 +124,44 @@ __global__ void __launch_bounds__(64)
 attn_context_kernel(const float* const* __restrict__ table, int longest_sent, const float* __restrict__ align,
                     const int* __restrict__ indices, const int* __restrict__ batch_info, int H, int mb, int W,
                     float* __restrict__ ctx_out) {
+  // The wave first compacts the valid slots of its column into LDS (source pointer + weight), so that the
+  // accumulation loop has no data-dependent branches and several 16-byte loads are in flight per lane.
+  constexpr int kMaxSlots = 512;
+  __shared__ const float* s_src[kMaxSlots];
+  __shared__ float s_a[kMaxSlots];
   const int b = blockIdx.y;
-  constexpr int WD = VEC ? 4 : 1;
-  const int i0 = (blockIdx.x * 64 + threadIdx.x) * WD;
-  if (i0 >= H) return;
+  const int lane = threadIdx.x;
   const int len = batch_info[b], off = batch_info[mb + b];
+  int nvalid = 0;
+  for (int j0 = 0; j0 < W; j0 += 64) {
+    const int j = j0 + lane;
+    int s_idx = -1;
+    if (j < W) s_idx = indices[b + (size_t)mb * j];
+    const bool valid = s_idx != -1;
+    const unsigned long long m = __ballot(valid);
+    if (valid) {
+      int t = len - 1 - s_idx + off;
+      t = t < 0 ? 0 : (t >= longest_sent ? longest_sent - 1 : t);
+      const int pos = nvalid + __popcll(m & ((1ull << lane) - 1ull));
+      if (pos < kMaxSlots) {
+        s_src[pos] = table[t] + (size_t)b * H;
+        s_a[pos] = align[b + (size_t)mb * j];
+      }
+    }
+    nvalid += __popcll(m);
+  }
+  if (nvalid > kMaxSlots) nvalid = kMaxSlots;  // host guarantees W <= kMaxSlots
+  __syncthreads();
+  constexpr int WD = VEC ? 4 : 1;
+  const int i0 = (blockIdx.x * 64 + lane) * WD;
+  if (i0 >= H) return;
   float acc[WD];
 #pragma unroll
   for (int q = 0; q < WD; ++q) acc[q] = 0.0f;
-  for (int j = 0; j < W; ++j) {
-    const int s_idx = indices[b + (size_t)mb * j];
-    if (s_idx == -1) continue;
-    int t = len - 1 - s_idx + off;
-    t = t < 0 ? 0 : (t >= longest_sent ? longest_sent - 1 : t);
-    const float a = align[b + (size_t)mb * j];
-    const float* hs = table[t] + (size_t)b * H + i0;
+#pragma unroll 4
+  for (int j = 0; j < nvalid; ++j) {
+    const float a = s_a[j];
+    const float* hs = s_src[j] + i0;
     if (VEC) {
       const zr_f32x4 v = *(const zr_f32x4*)hs;
       acc[0] += a * v.x;
@@ -165,6 +193,7 @@ int zr_attn_create(zr_ctx* ctx, int H, int mb, int D, const float* d_W_a, const 
   ZR_CHECK_ARG(H > 0 && mb > 0 && D >= 0 && longest_sent > 0, "zr_attn_create: H = %d, mb = %d, D = %d, longest_sent = %d",
                H, mb, D, longest_sent);
   ZR_CHECK_ARG(mb <= 65535, "zr_attn_create: mb = %d exceeds 65535", mb);
+  ZR_CHECK_ARG(2 * D + 1 <= 512, "zr_attn_create: attention width D = %d exceeds 255", D);
   ZR_CHECK_ARG(d_W_a && d_W_p && d_v_p && d_out_bias && d_W_c1 && d_W_c2 && h_hs_table, "zr_attn_create: null pointer");
   bool tables_aligned = true;
   for (int t = 0; t < longest_sent; ++t) {
@@ -271,7 +300,7 @@ int zr_attn_step(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, const float* 
                                                              H, mb, W, align, ctx->d_flags);
   ZR_LAUNCH_CHECK("attn_score_kernel");
   const float sigma_sq = (float)((D * D) / 4.0);  // attention_node.hpp:50
-  attn_align_kernel<<<(mb + 63) / 64, 64, 0, ctx->stream>>>(align, idx, pt, mb, W, sigma_sq);
+  attn_align_kernel<<<mb, 64, 0, ctx->stream>>>(align, idx, pt, mb, W, sigma_sq);
   ZR_LAUNCH_CHECK("attn_align_kernel");
   if (vec) {
     dim3 cg((H / 4 + 63) / 64, mb);

@@ -30,7 +30,7 @@ __global__ void __launch_bounds__(64 * KS * WPB) gemm_kernel(GemmArgs a) {
   __shared__ float red[KS > 1 ? WPB * KS * TN * 16 * 64 : 1];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction
   const int kslice = wave % KS;
   const int sub = wave / KS;  // which wave tile of the workgroup
   const int jl = lane & 31;
@@ -71,12 +71,18 @@ __global__ void __launch_bounds__(64 * KS * WPB) gemm_kernel(GemmArgs a) {
   for (int s = 0; s < a.nseg; ++s) {
     const float* A = a.A[s] + (long long)z * a.strideA;
     const float* wbase[TM];
+    unsigned woff[TM];
     const float* xcol[TN];
 #pragma unroll
-    for (int tm = 0; tm < TM; ++tm) wbase[tm] = TRANS_A ? A + (long long)rows[tm] * a.lda[s] : A + rows[tm];
+    for (int tm = 0; tm < TM; ++tm) {
+      wbase[tm] = A;
+      woff[tm] = TRANS_A ? (unsigned)((long long)rows[tm] * a.lda[s] + 4 * half)
+                         : (unsigned)(rows[tm] + 4LL * half * a.lda[s]);
+    }
 #pragma unroll
-    for (int tn = 0; tn < TN; ++tn) xcol[tn] = a.B[s] + (long long)cols[tn] * a.ldb[s];
-    zr_mma_segment<TM, TN, KS, TRANS_A, VEC>(acc, wbase, a.lda[s], xcol, a.K[s], kslice, half);
+    for (int tn = 0; tn < TN; ++tn) xcol[tn] = a.B[s] + (long long)cols[tn] * a.ldb[s] + 4 * half;
+    zr_mma_segment<TM, TN, KS, zr_prefetch_depth(TM, TN), TRANS_A, VEC>(acc, wbase, woff, a.lda[s], xcol, a.K[s],
+                                                                        kslice, half);
   }
 
   float* C = a.C + (long long)z * a.strideC;
@@ -177,6 +183,9 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
       ZR_CHECK_ARG(d.A[s] && d.B[s], "gemm: null operand in segment %d", s);
       ZR_CHECK_ARG(d.lda[s] >= (d.trans_a ? d.K[s] : d.M), "gemm: lda[%d] = %d too small", s, d.lda[s]);
       ZR_CHECK_ARG(d.ldb[s] >= d.K[s], "gemm: ldb[%d] = %d < K = %d", s, d.ldb[s], d.K[s]);
+      // per-lane weight offsets are 32-bit element indices
+      ZR_CHECK_ARG(d.trans_a ? ((long long)d.M * d.lda[s] + 8 < (1LL << 31)) : (d.M + 8LL * d.lda[s] < (1LL << 31)),
+                   "gemm: operand A of segment %d is too large for 32-bit offsets", s);
       ga.K[s] = d.K[s];
       ga.A[s] = d.A[s];
       ga.lda[s] = d.lda[s];

@@ -57,7 +57,7 @@ __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int kslice = tid >> 6;
+  const int kslice = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction
   const int jl = lane & 31;
   const int half = lane >> 5;
   const int H = L.H;
@@ -84,9 +84,13 @@ __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
   const long long HH = (long long)H * H;
   for (int s = 0; s < U.nseg; ++s) {
     const float* wbase[4];
+    unsigned woff[4];
     const float* xcol[TN];
 #pragma unroll
-    for (int g = 0; g < 4; ++g) wbase[g] = U.W + ((long long)s * 4 + g) * HH + jc;
+    for (int g = 0; g < 4; ++g) {
+      wbase[g] = U.W + ((long long)s * 4 + g) * HH;
+      woff[g] = (unsigned)(jc + 4 * half * H);
+    }
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) {
       long long c = cols[tn];
@@ -95,9 +99,10 @@ __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
         idv = idv < 0 ? 0 : (idv >= U.V ? U.V - 1 : idv);
         c = idv;
       }
-      xcol[tn] = U.in[s] + c * H;
+      xcol[tn] = U.in[s] + c * H + 4 * half;
     }
-    zr_mma_segment<4, TN, KS, false, VEC>(acc, wbase, (long long)H, xcol, H, kslice, half);
+    zr_mma_segment<4, TN, KS, zr_prefetch_depth(4, TN), false, VEC>(acc, wbase, woff, (long long)H, xcol, H, kslice,
+                                                                    half);
   }
 
   const float bi = U.bias[jc], bf = U.bias[H + jc], bc = U.bias[2 * H + jc], bo = U.bias[3 * H + jc];

@@ -16,6 +16,11 @@
 // is valid as long as both operands use the same one; this one lets each lane fetch its four activation
 // values of a group with a single 16-byte load along K.
 //
+// Latency.  The weights come from HBM / the memory-side cache, a microsecond or more away, while one k-group of
+// MFMAs lasts a fraction of that.  Operands are therefore fetched PF groups ahead into a ring of register
+// fragments (software pipeline); weight addresses are a wave-uniform base plus a fixed per-lane offset so the
+// address arithmetic stays on the scalar unit.
+//
 // Split K.  KS waves of a workgroup may share one output tile and take the k-groups round-robin; their
 // partial tiles are summed through LDS in a fixed order (deterministic) before the epilogue runs.
 #ifndef ZR_MFMA_CORE_H
@@ -23,52 +28,72 @@
 
 #include "zr_internal.h"
 
+// Prefetch distance in k-groups for a TM x TN sub-tile wave: as deep as the register budget of the fragment
+// ring allows (a fragment is 4*(TM+TN) registers).
+constexpr int zr_prefetch_depth(int tm, int tn) {
+#ifdef ZR_PF_OVERRIDE
+  return ZR_PF_OVERRIDE;
+#else
+  return 4 * (tm + tn) <= 20 ? 3 : (4 * (tm + tn) <= 24 ? 2 : 1);
+#endif
+}
+
 template <int TM, int TN>
 struct ZrFrag {
   float x[TN][4];  // activations: x[tn][i] = X[k_i][n(tn, lane%32)]
   float w[TM][4];  // weights:     w[tm][i] = W[m(tm, lane%32)][k_i]
 };
 
-// One K segment.  `wbase[tm]` points at this lane's weight row (NN: &W[row][0] with stride lda between k;
-// TRANS_A: &W^T storage of that row, contiguous in k).  `xcol[tn]` points at this lane's activation column.
-// Addresses are pre-clamped by the caller so that out-of-range rows/columns read valid memory.
-template <int TM, int TN, int KS, bool TRANS_A, bool VEC>
+// One K segment.
+//   wbase[tm]: wave-uniform pointer to the weight matrix of sub-tile tm
+//   woff[tm]:  this lane's fixed element offset into it:
+//                NN:      row + 4*half*lda      (element (row, k) at wbase[row + k*lda])
+//                TRANS_A: row*lda + 4*half      (element (row, k) at wbase[k + row*lda])
+//   xcol[tn]:  this lane's activation column, already advanced by 4*half
+// Rows / columns are pre-clamped by the caller so that out-of-range lanes read valid memory.
+// kslice must be wave-uniform.
+template <int TM, int TN, int KS, int PF, bool TRANS_A, bool VEC>
 __device__ __forceinline__ void zr_mma_segment(zr_f32x16 (&acc)[TM][TN], const float* const (&wbase)[TM],
-                                               long long lda, const float* const (&xcol)[TN], int K, int kslice,
-                                               int half) {
+                                               const unsigned (&woff)[TM], long long lda,
+                                               const float* const (&xcol)[TN], int K, int kslice, int half) {
   const int nfull = K >> 3;
+  constexpr int NS = PF + 1;
 
   auto load_full = [&](ZrFrag<TM, TN>& f, int g) {
-    const int k0 = g * 8 + 4 * half;
+    const int kg = g * 8;  // wave-uniform
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) {
       if (VEC) {
-        const zr_f32x4 v = *(const zr_f32x4*)(xcol[tn] + k0);
+        const zr_f32x4 v = *(const zr_f32x4*)(xcol[tn] + kg);
         f.x[tn][0] = v.x;
         f.x[tn][1] = v.y;
         f.x[tn][2] = v.z;
         f.x[tn][3] = v.w;
       } else {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) f.x[tn][i] = xcol[tn][k0 + i];
+        for (int i = 0; i < 4; ++i) f.x[tn][i] = xcol[tn][kg + i];
       }
     }
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) {
       if (TRANS_A) {
+        const float* p = wbase[tm] + kg;  // uniform
         if (VEC) {
-          const zr_f32x4 v = *(const zr_f32x4*)(wbase[tm] + k0);
+          const zr_f32x4 v = *(const zr_f32x4*)(p + woff[tm]);
           f.w[tm][0] = v.x;
           f.w[tm][1] = v.y;
           f.w[tm][2] = v.z;
           f.w[tm][3] = v.w;
         } else {
 #pragma unroll
-          for (int i = 0; i < 4; ++i) f.w[tm][i] = wbase[tm][k0 + i];
+          for (int i = 0; i < 4; ++i) f.w[tm][i] = p[woff[tm] + i];
         }
       } else {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) f.w[tm][i] = wbase[tm][(long long)(k0 + i) * lda];
+        for (int i = 0; i < 4; ++i) {
+          const float* p = wbase[tm] + (long long)(kg + i) * lda;  // uniform
+          f.w[tm][i] = p[woff[tm]];
+        }
       }
     }
   };
@@ -83,43 +108,55 @@ __device__ __forceinline__ void zr_mma_segment(zr_f32x16 (&acc)[TM][TN], const f
           acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.x[tn][i], f.w[tm][i], acc[tm][tn], 0, 0, 0);
   };
 
-  ZrFrag<TM, TN> f0, f1;
-  int g = kslice;
-  if (g < nfull) {
-    load_full(f0, g);
-    while (true) {
-      const int g1 = g + KS;
-      if (g1 < nfull) load_full(f1, g1);
-      mma(f0);
-      if (g1 >= nfull) break;
-      const int g2 = g1 + KS;
-      if (g2 < nfull) load_full(f0, g2);
-      mma(f1);
-      if (g2 >= nfull) break;
-      g = g2;
+  // The steady-state loop is free of branches: every stage issues the loads of the group PF stages ahead
+  // (group indices past the end are clamped to the last group: a few redundant loads of valid memory) and then
+  // multiplies the fragment loaded PF stages ago.  Keeping loads unconditional matters: with loads under
+  // branches the compiler cannot count how many younger loads are in flight and waits for all of them.
+  if (kslice < nfull) {
+    const int last = nfull - 1;
+    const int n_mine = (nfull - kslice + KS - 1) / KS;  // groups owned by this wave: kslice, kslice+KS, ...
+    ZrFrag<TM, TN> f[NS];
+#pragma unroll
+    for (int s = 0; s < PF; ++s) {
+      const int gl = kslice + s * KS;
+      load_full(f[s], gl < last ? gl : last);
     }
+    int it = 0;
+    for (; it + NS <= n_mine; it += NS) {
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        const int gl = kslice + (it + s + PF) * KS;
+        load_full(f[(s + PF) % NS], gl < last ? gl : last);
+        mma(f[s]);
+      }
+    }
+    // at most PF groups remain, all of them already loaded
+#pragma unroll
+    for (int s = 0; s < PF; ++s)
+      if (it + s < n_mine) mma(f[s]);
   }
   // tail group (K not a multiple of 8): zero-filled, owned by the slice whose turn it is
   if ((K & 7) != 0 && (nfull % KS) == kslice) {
-    const int k0 = nfull * 8 + 4 * half;
-    ZrFrag<TM, TN> f;
+    const int kg = nfull * 8;
+    ZrFrag<TM, TN> t;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int k = k0 + i;
+      const int k = kg + 4 * half + i;
       const bool ok = k < K;
-      const int kc = ok ? k : K - 1;
+      // xcol/woff already include this lane's 4*half: index relative to them
+      const int rel = ok ? kg + i : (K - 1) - 4 * half;
 #pragma unroll
       for (int tn = 0; tn < TN; ++tn) {
-        const float v = xcol[tn][kc];
-        f.x[tn][i] = ok ? v : 0.0f;
+        const float v = xcol[tn][rel];
+        t.x[tn][i] = ok ? v : 0.0f;
       }
 #pragma unroll
       for (int tm = 0; tm < TM; ++tm) {
-        const float v = TRANS_A ? wbase[tm][kc] : wbase[tm][(long long)kc * lda];
-        f.w[tm][i] = ok ? v : 0.0f;
+        const float v = TRANS_A ? wbase[tm][(long long)woff[tm] + rel] : wbase[tm][(long long)woff[tm] + (long long)rel * lda];
+        t.w[tm][i] = ok ? v : 0.0f;
       }
     }
-    mma(f);
+    mma(t);
   }
 }
 
