@@ -1,0 +1,133 @@
+"""Beam search on the device against the oracle's restatement of the reference decoder (std::priority_queue
+based, one sentence at a time).  Word ids and back-pointers must be bit-exact; scores within 1e-4 relative.
+Inputs are tie-free random distributions (exact ties follow libstdc++'s heap order in the reference, which
+the device path does not reproduce) plus one tie case whose outcome does not depend on that order."""
+import numpy as np
+import pytest
+
+import oracle_lib as o
+from zoph_rnn_amd import capi, synth
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = capi.Context(0)
+    yield c
+    c.close()
+
+
+def _random_dist(g, V, cols, peaky=2.0, eof_boost=0.0):
+    logits = g.standard_normal(size=(V, cols)) * peaky
+    logits[1, :] += eof_boost
+    e = np.exp(logits - logits.max(axis=0))
+    return np.asfortranarray((e / e.sum(axis=0)).astype(np.float32))
+
+
+def _decode_both(ctx, V, beam, n_sent, steps, max_len, penalty, seed, eof_boost):
+    g = synth.rng(seed, 21)
+    b = ctx.beam_create(beam, V, n_sent, max_len, penalty)
+    decs = [o.Decoder(beam, V, max_len, penalty=penalty) for _ in range(n_sent)]
+    d_words, d_back = ctx.empty(n_sent * beam, np.int32), ctx.empty(n_sent * beam, np.int32)
+    d_prob = ctx.empty((V, n_sent * beam))
+    for index in range(steps):
+        P = _random_dist(g, V, n_sent * beam, eof_boost=eof_boost)
+        d_prob.set(P)
+        ctx.beam_expand(b, d_prob, index, d_words, d_back)
+        ctx.sync()
+        words, back = d_words.get(), d_back.get()
+        for s in range(n_sent):
+            decs[s].expand(P[:, s * beam:(s + 1) * beam], index)
+            st = decs[s].state()
+            assert np.array_equal(words[s * beam:(s + 1) * beam], st["current_indices"]), (index, s)
+            assert np.array_equal(back[s * beam:(s + 1) * beam] - s * beam, st["new_indicies_changes"]), (index, s)
+            sc, w2 = ctx.beam_state(b, s, beam)
+            live = st["current_indices"] != -1
+            assert np.allclose(sc[live], st["scores"][live], rtol=1e-4, atol=1e-5)
+            assert np.array_equal(w2, st["current_indices"])
+    P = _random_dist(g, V, n_sent * beam)
+    d_prob.set(P)
+    ctx.beam_finish(b, d_prob)
+    ctx.sync()
+    for s in range(n_sent):
+        decs[s].finish(P[:, s * beam:(s + 1) * beam])
+        want = decs[s].hypotheses()
+        got, n = ctx.beam_hypotheses(b, s, cap=len(want) + 8, max_len=max_len)
+        assert n == len(want), (s, n, len(want))
+        for (gw, gs), (ww, ws) in zip(got, want):
+            assert np.array_equal(gw, ww)
+            assert gs == pytest.approx(ws, rel=1e-4, abs=1e-5)
+    ctx.beam_destroy(b)
+
+
+@pytest.mark.parametrize("V,beam,n_sent,steps", [(50, 4, 1, 6), (500, 12, 3, 8), (97, 3, 5, 10), (40, 1, 2, 5)])
+def test_beam_against_reference_rules(ctx, V, beam, n_sent, steps):
+    _decode_both(ctx, V, beam, n_sent, steps, max_len=steps + 4, penalty=0.0, seed=V + beam, eof_boost=0.0)
+
+
+def test_beam_with_frequent_eof_and_penalty(ctx):
+    """<EOF> made likely: hypotheses finish inside expand without consuming beam slots; a word penalty is added."""
+    _decode_both(ctx, 60, 5, 4, 7, max_len=12, penalty=0.3, seed=7, eof_boost=4.0)
+
+
+def test_beam_batching_does_not_change_a_sentence(ctx):
+    """16 sentences decoded together give, per sentence, what a single-sentence decode gives."""
+    V, beam, n_sent, steps, max_len = 300, 12, 16, 5, 10
+    g = synth.rng(31, 21)
+    Ps = [_random_dist(g, V, n_sent * beam) for _ in range(steps)]
+    d_words, d_back = ctx.empty(n_sent * beam, np.int32), ctx.empty(n_sent * beam, np.int32)
+    big = ctx.beam_create(beam, V, n_sent, max_len)
+    hist = []
+    for index, P in enumerate(Ps):
+        ctx.beam_expand(big, ctx.array(P), index, d_words, d_back)
+        ctx.sync()
+        hist.append((d_words.get().copy(), d_back.get().copy()))
+    d_w1, d_b1 = ctx.empty(beam, np.int32), ctx.empty(beam, np.int32)
+    for s in (0, 7, 15):
+        one = ctx.beam_create(beam, V, 1, max_len)
+        for index, P in enumerate(Ps):
+            ctx.beam_expand(one, ctx.array(np.asfortranarray(P[:, s * beam:(s + 1) * beam])), index, d_w1, d_b1)
+            ctx.sync()
+            assert np.array_equal(d_w1.get(), hist[index][0][s * beam:(s + 1) * beam])
+            assert np.array_equal(d_b1.get(), hist[index][1][s * beam:(s + 1) * beam] - s * beam)
+        ctx.beam_destroy(one)
+    ctx.beam_destroy(big)
+
+
+def test_beam_all_equal_probabilities(ctx):
+    """All probabilities equal: the kept words are 0..beam; <START> is skipped, <EOF> finishes, the remaining
+    slots are filled and the last one falls into the empty-heap branch -- a result that does not depend on the
+    order among the tied entries apart from which of the two equal survivors comes first."""
+    V, beam = 12, 3
+    b = ctx.beam_create(beam, V, 1, 6)
+    d_words, d_back = ctx.empty(beam, np.int32), ctx.empty(beam, np.int32)
+    ctx.beam_expand(b, ctx.array(np.full((V, beam), 0.125, np.float32, order="F")), 0, d_words, d_back)
+    ctx.sync()
+    w = d_words.get()
+    assert sorted(w[:2].tolist()) == [2, 3] and w[2] == -1
+    hyps, n = ctx.beam_hypotheses(b, 0, cap=4, max_len=6)
+    assert n == 1 and hyps[0][0].tolist() == [0, 1]
+    ctx.beam_destroy(b)
+
+
+def test_beam_full_vocab_shape(ctx):
+    """V=50000, beam 12, 16 sentences (192 columns): selection equals a full sort of every column."""
+    V, beam, n_sent = 50000, 12, 16
+    g = synth.rng(41, 21)
+    P = _random_dist(g, V, n_sent * beam, peaky=3.0)
+    b = ctx.beam_create(beam, V, n_sent, 8)
+    d_words, d_back = ctx.empty(n_sent * beam, np.int32), ctx.empty(n_sent * beam, np.int32)
+    d_prob = ctx.array(P)
+    for index in range(2):
+        ctx.beam_expand(b, d_prob, index, d_words, d_back)
+        ctx.sync()
+        words, back = d_words.get(), d_back.get()
+        for s in (0, 5, 15):
+            dec = o.Decoder(beam, V, 8)
+            for i2 in range(index + 1):
+                dec.expand(P[:, s * beam:(s + 1) * beam], i2)
+            st = dec.state()
+            assert np.array_equal(words[s * beam:(s + 1) * beam], st["current_indices"])
+            assert np.array_equal(back[s * beam:(s + 1) * beam] - s * beam, st["new_indicies_changes"])
+    ctx.beam_destroy(b)
