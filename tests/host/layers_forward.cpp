@@ -1,0 +1,193 @@
+// Drives the host-side layer classes (zoph_rnn_amd/host/zoph_layers.h) the way the reference's
+// neuralMT_model::getError does (src/model.hpp:1463-1802): index preparation, the source sweep, the target sweep
+// with attention + feed-input on the top target layer, and the per-step loss.  Weights come from a model file in
+// the reference's text layout.  Output (stdout): one line "loss <t> <value>" per target step, then the top-layer
+// output of every target step ("h <t> <H*mb floats>").
+//
+// usage: layers_forward <weights.txt> <ids.txt> H mb V L S T D
+//   ids.txt: S*mb source ids, T*mb target input ids, T*mb target output ids, 2*mb batch_info (time-major, -1 pads)
+//   S == 0: language model (no source, no attention).
+#include <cstdio>
+#include <fstream>
+#include <iostream>
+#include <vector>
+
+#include "../../zoph_rnn_amd/host/zoph_layers.h"
+
+int main(int argc, char** argv) {
+  if (argc != 10) {
+    std::fprintf(stderr, "usage: %s weights ids H mb V L S T D\n", argv[0]);
+    return 2;
+  }
+  const int H = atoi(argv[3]), mb = atoi(argv[4]), V = atoi(argv[5]), L = atoi(argv[6]), S = atoi(argv[7]),
+            T = atoi(argv[8]), D = atoi(argv[9]);
+  const bool seq2seq = S > 0;
+  const int longest = (S > T ? S : T);
+  std::vector<int> src(S * mb), tin(T * mb), tout(T * mb), binfo(2 * mb);
+  {
+    std::ifstream f(argv[2]);
+    for (auto& v : src) f >> v;
+    for (auto& v : tin) f >> v;
+    for (auto& v : tout) f >> v;
+    for (auto& v : binfo) f >> v;
+  }
+  layer_gpu_info gpu;
+  gpu.init(0);
+  neuralMT_model<precision> model;
+  global_params params;
+  params.LSTM_size = H;
+  params.minibatch_size = mb;
+  params.longest_sent = longest;
+  params.target_vocab_size = V;
+  params.source_vocab_size = V;
+  params.attent_params.attention_model = seq2seq;
+  params.attent_params.D = D;
+  params.attent_params.feed_input = seq2seq;
+
+  Input_To_Hidden_Layer<precision> input_layer_source, input_layer_target;
+  std::vector<Hidden_To_Hidden_Layer<precision>> source_hidden_layers(L - 1), target_hidden_layers(L - 1);
+  softmax_layer<precision> softmax_obj;
+  base_loss_layer<precision>* softmax = &softmax_obj;
+  softmax_obj.share_gpu(gpu);
+  softmax->init_loss_layer(&model, params);
+
+  if (seq2seq) {
+    input_layer_source.ih_layer_info.share(gpu);
+    input_layer_source.init_Input_To_Hidden_Layer(H, mb, V, longest, false, 0.f, false, 0.f, &model, 0, false, 0.f,
+                                                  false, false, nullptr, false, params, true);
+    for (int l = 0; l < L - 1; l++) {
+      source_hidden_layers[l].hh_layer_info.share(gpu);
+      source_hidden_layers[l].init_Hidden_To_Hidden_Layer(H, mb, longest, false, 0.f, false, 0.f, &model, 0, false,
+                                                           0.f, false, l);
+    }
+  }
+  input_layer_target.ih_layer_info.share(gpu);
+  input_layer_target.init_Input_To_Hidden_Layer(H, mb, V, longest, false, 0.f, false, 0.f, &model, 0, false, 0.f,
+                                                false, false, nullptr, false, params, false);
+  for (int l = 0; l < L - 1; l++) {
+    target_hidden_layers[l].hh_layer_info.share(gpu);
+    target_hidden_layers[l].init_Hidden_To_Hidden_Layer(H, mb, longest, false, 0.f, false, 0.f, &model, 0, false, 0.f,
+                                                         false, l);
+  }
+  // wiring of the layers (neuralMT_model::initModel, src/model.hpp:300-420): source layers feed upwards only,
+  // the top target layer feeds the softmax
+  auto wire = [&](Input_To_Hidden_Layer<precision>& in, std::vector<Hidden_To_Hidden_Layer<precision>>& hid,
+                  bool source_side) {
+    if (hid.empty()) {
+      in.upper_layer.init_upper_transfer_layer(true, false, source_side, softmax, nullptr);
+    } else {
+      in.upper_layer.init_upper_transfer_layer(false, false, source_side, nullptr, &hid[0]);
+      for (size_t l = 0; l + 1 < hid.size(); l++)
+        hid[l].upper_layer.init_upper_transfer_layer(false, false, source_side, nullptr, &hid[l + 1]);
+      hid.back().upper_layer.init_upper_transfer_layer(true, false, source_side, softmax, nullptr);
+    }
+  };
+  if (seq2seq) wire(input_layer_source, source_hidden_layers, true);
+  wire(input_layer_target, target_hidden_layers, false);
+
+  attention_layer<precision>* att = nullptr;
+  if (seq2seq) {
+    std::vector<const precision*> total_hs(longest);
+    for (int i = 0; i < longest; i++)
+      total_hs[i] = (L == 1) ? input_layer_source.nodes[i].d_h_t : source_hidden_layers[L - 2].nodes[i].d_h_t;
+    att = new attention_layer<precision>(H, mb, 0, D, longest, gpu, total_hs, true);
+    if (L == 1)
+      input_layer_target.init_attention(att);
+    else
+      target_hidden_layers[L - 2].init_attention(att);
+    input_layer_target.init_feed_input(L == 1 ? nullptr : &target_hidden_layers[L - 2], false);
+  }
+
+  // model file order (neuralMT_model::load_weights, src/model.hpp:2172-2241)
+  {
+    std::ifstream w(argv[1]);
+    if (seq2seq) {
+      input_layer_source.load_weights(w);
+      for (auto& l : source_hidden_layers) l.load_weights(w);
+    }
+    input_layer_target.load_weights(w);
+    for (auto& l : target_hidden_layers) l.load_weights(w);
+    softmax->load_weights(w);
+  }
+  // round trip through dump_weights: written next to the input as <weights>.dump
+  {
+    std::ofstream o(std::string(argv[1]) + ".dump");
+    o << std::setprecision(std::numeric_limits<precision>::digits10 + 2);
+    if (seq2seq) {
+      input_layer_source.dump_weights(o);
+      for (auto& l : source_hidden_layers) l.dump_weights(o);
+    }
+    input_layer_target.dump_weights(o);
+    for (auto& l : target_hidden_layers) l.dump_weights(o);
+    softmax->dump_weights(o);
+  }
+
+  // ---- getError schedule
+  if (seq2seq) {
+    input_layer_source.prep_GPU_vocab_indices(src.data(), nullptr, S, 0);
+    for (auto& l : source_hidden_layers) l.prep_GPU_vocab_indices(src.data(), S);
+    att->prep_minibatch_info(binfo.data());
+  }
+  input_layer_target.prep_GPU_vocab_indices(tin.data(), nullptr, T, 0);
+  for (auto& l : target_hidden_layers) l.prep_GPU_vocab_indices(tin.data(), T);
+  softmax->prep_GPU_vocab_indices(tout.data(), T);
+
+  for (int i = 0; i < S; i++) {
+    const int step = i * mb;
+    auto& n0 = input_layer_source.nodes[i];
+    n0.update_vectors_forward_GPU(input_layer_source.d_input_vocab_indices_full + step,
+                                  input_layer_source.d_input_vocab_indices_01_full + step,
+                                  i == 0 ? input_layer_source.d_init_hidden_vector : input_layer_source.nodes[i - 1].d_h_t,
+                                  i == 0 ? input_layer_source.d_init_cell_vector : input_layer_source.nodes[i - 1].d_c_t);
+    n0.forward_prop();
+    for (auto& l : source_hidden_layers) {
+      l.nodes[i].update_vectors_forward_GPU(l.d_input_vocab_indices_01_full + step,
+                                            i == 0 ? l.d_init_hidden_vector : l.nodes[i - 1].d_h_t,
+                                            i == 0 ? l.d_init_cell_vector : l.nodes[i - 1].d_c_t);
+      l.nodes[i].forward_prop();
+    }
+  }
+  std::vector<precision> host((size_t)H * mb);
+  std::cout << std::setprecision(9);
+  for (int i = 0; i < T; i++) {
+    const int step = i * mb;
+    precision *hp, *cp;
+    if (i > 0) {
+      hp = input_layer_target.nodes[i - 1].d_h_t;
+      cp = input_layer_target.nodes[i - 1].d_c_t;
+    } else if (seq2seq) {  // start from the encoder's last state (src/model.hpp:1714-1724)
+      hp = input_layer_source.nodes[S - 1].d_h_t;
+      cp = input_layer_source.nodes[S - 1].d_c_t;
+    } else {
+      hp = input_layer_target.d_init_hidden_vector;
+      cp = input_layer_target.d_init_cell_vector;
+    }
+    input_layer_target.nodes[i].update_vectors_forward_GPU(input_layer_target.d_input_vocab_indices_full + step,
+                                                           input_layer_target.d_input_vocab_indices_01_full + step, hp, cp);
+    input_layer_target.nodes[i].forward_prop();
+    for (size_t l = 0; l < target_hidden_layers.size(); l++) {
+      auto& ly = target_hidden_layers[l];
+      if (i > 0) {
+        hp = ly.nodes[i - 1].d_h_t;
+        cp = ly.nodes[i - 1].d_c_t;
+      } else if (seq2seq) {
+        hp = source_hidden_layers[l].nodes[S - 1].d_h_t;
+        cp = source_hidden_layers[l].nodes[S - 1].d_c_t;
+      } else {
+        hp = ly.d_init_hidden_vector;
+        cp = ly.d_init_cell_vector;
+      }
+      ly.nodes[i].update_vectors_forward_GPU(ly.d_input_vocab_indices_01_full + step, hp, cp);
+      ly.nodes[i].forward_prop();
+    }
+    softmax->backprop_prep_GPU(softmax->get_ht_ptr(i), step);
+    const double loss = softmax->compute_loss_GPU(i);
+    std::cout << "loss " << i << " " << std::setprecision(15) << loss << std::setprecision(9) << "\n";
+    ZOPH_CALL(zr_d2h(gpu.ctx, host.data(), softmax->get_ht_ptr(i), host.size() * sizeof(precision)));
+    std::cout << "h " << i;
+    for (precision v : host) std::cout << " " << v;
+    std::cout << "\n";
+  }
+  devSynchAll(gpu.ctx);
+  return 0;
+}

@@ -43,3 +43,16 @@ def build_hip(verbose=False, jobs=4):
 
 if __name__ == "__main__":
     print(build_hip(verbose=True, jobs=int(os.environ.get("JOBS", "4"))))
+
+
+def build_host_driver():
+    """C++ driver of the host-side layer classes (tests/host/layers_forward), plain g++ against the C-ABI."""
+    root = os.path.dirname(HERE)
+    src = os.path.join(root, "tests", "host", "layers_forward.cpp")
+    out = os.path.join(root, "tests", "host", "layers_forward")
+    cmd = [os.environ.get("CXX", "g++"), "-std=c++17", "-O1", "-Wall", "-o", out, src, "-L", HERE, "-lzoph_rnn_hip",
+           "-Wl,-rpath,$ORIGIN/../../zoph_rnn_amd"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("host driver build failed:\n" + r.stdout + r.stderr)
+    return out

@@ -13,8 +13,10 @@ __global__ void fill_zero_kernel(uint32_t* p, size_t n_words) {
 }
 
 // vocab_to_01 + vocab_to_nonM1 (reference: src/custom_kernels.h:10-32) in one pass.
-__global__ void vocab_prep_kernel(const int* __restrict__ ids, int n, int V, int* __restrict__ nonneg,
-                                  int* __restrict__ mask01, int* __restrict__ flags) {
+// `nonneg` may alias `ids` (in-place -1 -> 0, as the reference's input layer does): each element is read and
+// then written by the same thread, so neither pointer is declared restrict.
+__global__ void vocab_prep_kernel(const int* ids, int n, int V, int* nonneg, int* __restrict__ mask01,
+                                  int* __restrict__ flags) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
   const int stride = gridDim.x * blockDim.x;
   for (; i < n; i += stride) {

@@ -1,0 +1,862 @@
+// Host-side C++ classes that keep the names, public data members and forward-path member functions of the
+// reference's layer objects and forward every device operation to the C-ABI in include/zoph_rnn.h.
+//
+//   reference class (file)                                   here
+//   LSTM_IH_Node            (src/LSTM.h:19-106)              LSTM_IH_Node<float>
+//   LSTM_HH_Node            (src/LSTM_HH.h:19-102)           LSTM_HH_Node<float>
+//   Input_To_Hidden_Layer   (src/Input_To_Hidden_Layer.h:11) Input_To_Hidden_Layer<float>
+//   Hidden_To_Hidden_Layer  (src/Hidden_To_Hidden_Layer.h:12) Hidden_To_Hidden_Layer<float>
+//   softmax_layer           (src/softmax.h:14, base_loss.h)  softmax_layer<float> : base_loss_layer<float>
+//   attention_layer / node  (src/attention_layer.h:14, src/attention_node.h:11)
+//
+// Differences that follow from running on one GPU behind a C-ABI:
+//   - cublasHandle_t / cudaStream_t / cudaEvent_t members are replaced by one zr_ctx per layer_gpu_info; all
+//     layers of a model share one context (one in-order stream), so the reference's event wiring is not needed;
+//   - h_t is handed to the layer above by pointer (the reference's copy_h_t == false branch,
+//     src/LSTM.hpp:492-515) instead of a device-to-device copy;
+//   - only dType = float exists (typedef float precision, src/global_params.h:3);
+//   - back-propagation, gradient and update members are not provided (forward path only);
+//   - weights are initialised with std::mt19937 instead of boost::mt19937: the value stream differs, the
+//     distribution (uniform in [BZ_CUDA::lower, BZ_CUDA::upper], forget bias 1) is the same.
+// Like the reference, a failed device call prints the error and exits (src/BZ_CUDA_UTIL.h:193-201).
+#ifndef ZOPH_LAYERS_H
+#define ZOPH_LAYERS_H
+
+#include <cstdio>
+#include <cstdlib>
+#include <fstream>
+#include <iomanip>
+#include <limits>
+#include <random>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include "../../include/zoph_rnn.h"
+
+typedef float precision;  // src/global_params.h:3
+
+#define ZOPH_CALL(expr)                                                                    \
+  do {                                                                                     \
+    int zoph_rc_ = (expr);                                                                 \
+    if (zoph_rc_ != ZR_OK) {                                                               \
+      std::fprintf(stderr, "Error: %s failed (%d): %s\n", #expr, zoph_rc_, zr_last_error()); \
+      std::exit(EXIT_FAILURE);                                                             \
+    }                                                                                      \
+  } while (0)
+
+// Mutable globals of the reference that the forward path reads (src/BZ_CUDA_UTIL.h:59-159).
+namespace BZ_CUDA {
+inline bool clip_cell = false;
+inline precision cell_clip_threshold = 50;
+inline precision lower = -0.08f;
+inline precision upper = 0.08f;
+inline bool force_decode = false;
+inline std::mt19937 gen(1234);
+}  // namespace BZ_CUDA
+
+struct attention_params {  // src/global_params.h:8-22 (fields used by the forward path)
+  bool attention_model = false;
+  int D = 10;
+  bool feed_input = false;
+};
+
+struct global_params {  // src/global_params.h:61-299 (fields used by the forward path)
+  attention_params attent_params;
+  int LSTM_size = 100;
+  int minibatch_size = 8;
+  int longest_sent = 100;
+  int target_vocab_size = 0;
+  int source_vocab_size = 0;
+};
+
+template <typename dType>
+struct neuralMT_model {  // only the flags the layers consult (src/model.h:37-217)
+  bool train = false;
+  bool decode = false;
+  attention_params attent_params;
+};
+
+// One context per GPU (layer_gpu_info::init, src/gpu_info_struct.h:67-172).
+struct layer_gpu_info {
+  int device_number = 0;
+  zr_ctx* ctx = nullptr;
+  void init(int device) {
+    device_number = device;
+    ZOPH_CALL(zr_ctx_create(device, &ctx));
+  }
+  void share(const layer_gpu_info& other) { *this = other; }
+};
+typedef layer_gpu_info softmax_layer_gpu_info;
+typedef layer_gpu_info attention_layer_gpu_info;
+
+inline void devSynchAll(zr_ctx* ctx) { ZOPH_CALL(zr_ctx_sync(ctx)); }  // src/BZ_CUDA_UTIL.h:977-987
+
+// full_matrix_setup (src/BZ_CUDA_UTIL.h:358-364): device matrix filled U(lower, upper); the host copy is not kept.
+template <typename dType>
+void full_matrix_setup(zr_ctx* ctx, dType** h_ptr, dType** d_ptr, int rows, int cols) {
+  std::vector<dType> tmp((size_t)rows * cols);
+  std::uniform_real_distribution<double> dist(BZ_CUDA::lower, BZ_CUDA::upper);
+  for (auto& v : tmp) v = (dType)dist(BZ_CUDA::gen);
+  ZOPH_CALL(zr_malloc(ctx, tmp.size() * sizeof(dType), (void**)d_ptr));
+  ZOPH_CALL(zr_h2d(ctx, *d_ptr, tmp.data(), tmp.size() * sizeof(dType)));
+  if (h_ptr) *h_ptr = nullptr;
+}
+template <typename dType>
+void full_matrix_setup_0(zr_ctx* ctx, dType** d_ptr, int rows, int cols) {  // :381-399, zero filled
+  ZOPH_CALL(zr_malloc(ctx, (size_t)rows * cols * sizeof(dType), (void**)d_ptr));
+  ZOPH_CALL(zr_memset_zero(ctx, *d_ptr, (size_t)rows * cols * sizeof(dType)));
+}
+template <typename dType>
+void device_fill(zr_ctx* ctx, dType* d_ptr, size_t n, dType value) {
+  std::vector<dType> tmp(n, value);
+  ZOPH_CALL(zr_h2d(ctx, d_ptr, tmp.data(), n * sizeof(dType)));
+}
+
+// read_matrix_GPU / write_matrix_GPU (src/Eigen_Util.h:84-163): one matrix row per text line, a blank line after
+// the matrix, column-major on the device.
+template <typename dType>
+void read_matrix_GPU(zr_ctx* ctx, dType* d_mat, int rows, int cols, std::ifstream& input) {
+  std::vector<dType> tmp((size_t)rows * cols);
+  std::string line, tok;
+  for (int i = 0; i < rows; i++) {
+    std::getline(input, line);
+    std::istringstream iss(line, std::istringstream::in);
+    for (int j = 0; j < cols; j++) {
+      iss >> tok;
+      tmp[(size_t)j * rows + i] = (dType)std::stod(tok);
+    }
+  }
+  std::getline(input, line);
+  ZOPH_CALL(zr_h2d(ctx, d_mat, tmp.data(), tmp.size() * sizeof(dType)));
+}
+template <typename dType>
+void write_matrix_GPU(zr_ctx* ctx, dType* d_mat, int rows, int cols, std::ofstream& output) {
+  std::vector<dType> tmp((size_t)rows * cols);
+  ZOPH_CALL(zr_d2h(ctx, tmp.data(), d_mat, tmp.size() * sizeof(dType)));
+  for (int i = 0; i < rows; i++) {
+    for (int j = 0; j < cols; j++) {
+      output << tmp[(size_t)j * rows + i];
+      if (j != cols - 1) output << " ";
+    }
+    output << "\n";
+  }
+  output << "\n";
+}
+
+template <typename dType> class Input_To_Hidden_Layer;
+template <typename dType> class Hidden_To_Hidden_Layer;
+template <typename dType> class attention_layer;
+template <typename dType> class base_loss_layer;
+
+// src/transfer_layer.h:18-41
+template <typename dType>
+struct upper_transfer_layer {
+  bool upper_softmax = true;
+  bool copy_h_t = false;
+  bool source_side = true;
+  base_loss_layer<dType>* softmax = nullptr;
+  Hidden_To_Hidden_Layer<dType>* hidden_layer = nullptr;
+  void init_upper_transfer_layer(bool upper_softmax, bool copy_h_t, bool source_side, base_loss_layer<dType>* softmax,
+                                 Hidden_To_Hidden_Layer<dType>* hidden_layer) {
+    this->upper_softmax = upper_softmax;
+    this->copy_h_t = copy_h_t;
+    this->source_side = source_side;
+    this->softmax = softmax;
+    this->hidden_layer = hidden_layer;
+  }
+};
+
+// ------------------------------------------------------------------------------------------------ attention
+template <typename dType>
+class attention_node {  // src/attention_node.h:11-86
+ public:
+  int LSTM_size, minibatch_size, device_number, D, index;
+  bool feed_input;
+  attention_layer<dType>* attent_layer;
+  dType* d_h_t = nullptr;          // input: top-layer target hidden state
+  dType* d_final_temp_2 = nullptr; // output h~
+  dType* d_alignments = nullptr;
+  dType* d_p_t = nullptr;
+  dType* d_c_t = nullptr;
+  int* d_indicies = nullptr;
+  int** d_indicies_mask = nullptr;  // points at the owning LSTM node's 0/1 mask pointer
+  dType* d_lower_htild = nullptr;   // feed-input destination: next step's bottom node d_h_tild
+
+  attention_node(int LSTM_size, int minibatch_size, int device_number, int D, bool feed_input,
+                 attention_layer<dType>* attent_layer, int index);
+  void feed_input_init(dType* d_ptr_htild) { d_lower_htild = d_ptr_htild; }  // src/attention_node.hpp:56-60
+  void forward_prop();                                                         // src/attention_node.hpp:73-394
+};
+
+template <typename dType>
+class attention_layer {  // src/attention_layer.h:14-143
+ public:
+  attention_layer_gpu_info layer_info;
+  int LSTM_size, minibatch_size, device_number, D, longest_sent;
+  bool feed_input;
+  dType *d_W_a = nullptr, *d_W_p = nullptr, *d_v_p = nullptr, *d_output_bias = nullptr, *d_W_c_p1 = nullptr,
+        *d_W_c_p2 = nullptr;
+  int* d_batch_info = nullptr;
+  std::vector<const dType*> h_total_hs_mat;  // host copy of d_total_hs_mat (src/attention_layer.hpp:106-160)
+  zr_attn* attn = nullptr;
+  std::vector<attention_node<dType>> nodes;
+
+  // src/attention_layer.hpp:3-173.  total_hs: the source top-layer node states, entry t = node t's d_h_t.
+  attention_layer(int LSTM_size, int minibatch_size, int device_number, int D, int longest_sent,
+                  const layer_gpu_info& gpu, const std::vector<const dType*>& total_hs, bool feed_input) {
+    this->LSTM_size = LSTM_size;
+    this->minibatch_size = minibatch_size;
+    this->device_number = device_number;
+    this->D = D;
+    this->longest_sent = longest_sent;
+    this->feed_input = feed_input;
+    layer_info.share(gpu);
+    zr_ctx* ctx = layer_info.ctx;
+    dType* h = nullptr;
+    full_matrix_setup(ctx, &h, &d_W_a, LSTM_size, LSTM_size);
+    full_matrix_setup(ctx, &h, &d_W_p, LSTM_size, LSTM_size);
+    full_matrix_setup(ctx, &h, &d_v_p, 1, LSTM_size);
+    full_matrix_setup(ctx, &h, &d_output_bias, LSTM_size, 1);
+    full_matrix_setup(ctx, &h, &d_W_c_p1, LSTM_size, LSTM_size);
+    full_matrix_setup(ctx, &h, &d_W_c_p2, LSTM_size, LSTM_size);
+    ZOPH_CALL(zr_malloc(ctx, 2 * (size_t)minibatch_size * sizeof(int), (void**)&d_batch_info));
+    h_total_hs_mat = total_hs;
+    ZOPH_CALL(zr_attn_create(ctx, LSTM_size, minibatch_size, D, d_W_a, d_W_p, d_v_p, d_output_bias, d_W_c_p1, d_W_c_p2,
+                             h_total_hs_mat.data(), (int)h_total_hs_mat.size(), &attn));
+    for (int i = 0; i < longest_sent; i++)
+      nodes.push_back(attention_node<dType>(LSTM_size, minibatch_size, device_number, D, feed_input, this, i));
+  }
+  // src/attention_layer.hpp:580-583
+  void prep_minibatch_info(int* h_batch_info) {
+    ZOPH_CALL(zr_h2d(layer_info.ctx, d_batch_info, h_batch_info, 2 * (size_t)minibatch_size * sizeof(int)));
+  }
+  // weight order of the model file: W_a, W_p, v_p (LSTM_size x 1), output_bias, W_c_p1, W_c_p2
+  // (src/attention_layer.hpp:467-473)
+  void dump_weights(std::ofstream& output) {
+    zr_ctx* ctx = layer_info.ctx;
+    write_matrix_GPU(ctx, d_W_a, LSTM_size, LSTM_size, output);
+    write_matrix_GPU(ctx, d_W_p, LSTM_size, LSTM_size, output);
+    write_matrix_GPU(ctx, d_v_p, LSTM_size, 1, output);
+    write_matrix_GPU(ctx, d_output_bias, LSTM_size, 1, output);
+    write_matrix_GPU(ctx, d_W_c_p1, LSTM_size, LSTM_size, output);
+    write_matrix_GPU(ctx, d_W_c_p2, LSTM_size, LSTM_size, output);
+  }
+  void load_weights(std::ifstream& input) {
+    zr_ctx* ctx = layer_info.ctx;
+    read_matrix_GPU(ctx, d_W_a, LSTM_size, LSTM_size, input);
+    read_matrix_GPU(ctx, d_W_p, LSTM_size, LSTM_size, input);
+    read_matrix_GPU(ctx, d_v_p, LSTM_size, 1, input);
+    read_matrix_GPU(ctx, d_output_bias, LSTM_size, 1, input);
+    read_matrix_GPU(ctx, d_W_c_p1, LSTM_size, LSTM_size, input);
+    read_matrix_GPU(ctx, d_W_c_p2, LSTM_size, LSTM_size, input);
+  }
+};
+
+template <typename dType>
+attention_node<dType>::attention_node(int LSTM_size, int minibatch_size, int device_number, int D, bool feed_input,
+                                      attention_layer<dType>* attent_layer, int index) {
+  this->LSTM_size = LSTM_size;
+  this->minibatch_size = minibatch_size;
+  this->device_number = device_number;
+  this->D = D;
+  this->feed_input = feed_input;
+  this->attent_layer = attent_layer;
+  this->index = index;
+  zr_ctx* ctx = attent_layer->layer_info.ctx;
+  const size_t n = (size_t)LSTM_size * minibatch_size, w = (size_t)(2 * D + 1) * minibatch_size;
+  ZOPH_CALL(zr_malloc(ctx, n * sizeof(dType), (void**)&d_final_temp_2));
+  ZOPH_CALL(zr_malloc(ctx, n * sizeof(dType), (void**)&d_c_t));
+  ZOPH_CALL(zr_malloc(ctx, w * sizeof(dType), (void**)&d_alignments));
+  ZOPH_CALL(zr_malloc(ctx, w * sizeof(int), (void**)&d_indicies));
+  ZOPH_CALL(zr_malloc(ctx, (size_t)minibatch_size * sizeof(dType), (void**)&d_p_t));
+}
+
+template <typename dType>
+void attention_node<dType>::forward_prop() {
+  zr_ctx* ctx = attent_layer->layer_info.ctx;
+  ZOPH_CALL(zr_attn_step(ctx, attent_layer->attn, attent_layer->d_batch_info, d_h_t, *d_indicies_mask, d_final_temp_2,
+                         d_alignments, d_indicies, d_p_t, d_c_t));
+  // feed-input: h~ goes to the next time step's bottom node (src/attention_node.hpp:384-386)
+  if (feed_input && index != (attent_layer->longest_sent - 1) && d_lower_htild)
+    ZOPH_CALL(zr_d2d(ctx, d_lower_htild, d_final_temp_2, (size_t)LSTM_size * minibatch_size * sizeof(dType)));
+}
+
+// ------------------------------------------------------------------------------------------------ loss layer
+template <typename dType>
+class base_loss_layer {  // src/base_loss.h:13-64 (forward-path subset)
+ public:
+  virtual ~base_loss_layer() {}
+  virtual softmax_layer_gpu_info gpu_init(int device_number) = 0;
+  virtual void init_loss_layer(struct neuralMT_model<precision>* model, global_params& params) = 0;
+  virtual void forward_prop(int index) = 0;
+  virtual void backprop_prep_GPU(dType* d_h_t, int step) = 0;
+  virtual void backprop_prep_GPU_mgpu(int step) = 0;
+  virtual void prep_GPU_vocab_indices(int* h_output_vocab_indicies_target, int current_target_length) = 0;
+  virtual double compute_loss_GPU(int index) = 0;
+  virtual dType* get_ht_ptr(int index) = 0;
+  virtual void set_ht_ptr(int index, dType* d_h_t) = 0;
+  virtual void load_weights(std::ifstream& input) = 0;
+  virtual void dump_weights(std::ofstream& output) = 0;
+  virtual void get_distribution_GPU_decoder_wrapper() = 0;
+  virtual dType* get_dist_ptr() = 0;
+};
+
+template <typename dType>
+struct softmax_node {  // src/softmax_node.h:7-27
+  dType* d_outputdist = nullptr;
+  dType* d_h_t = nullptr;
+  int index = 0;
+};
+
+template <typename dType>
+class softmax_layer : public base_loss_layer<dType> {  // src/softmax.h:14-225
+ public:
+  softmax_layer_gpu_info s_layer_info;
+  int output_vocab_size = 0, LSTM_size = 0, minibatch_size = 0, longest_sent = 0;
+  dType *d_D = nullptr, *d_b_d = nullptr;
+  dType* d_outputdist = nullptr;       // V x minibatch probabilities (decoder path)
+  double* d_outputdist_perp = nullptr; // V x minibatch double log-probabilities (allocated on first use)
+  dType* d_logits = nullptr;           // scratch
+  dType* d_h_t = nullptr;
+  int *d_output_vocab_indices = nullptr, *d_output_vocab_indices_01 = nullptr;
+  dType* d_output_vocab_indices_01_float = nullptr;
+  int *d_output_vocab_indices_single = nullptr, *d_output_vocab_indices_01_single = nullptr;
+  std::vector<softmax_node<dType>> nodes;
+
+  softmax_layer_gpu_info gpu_init(int device_number) override {
+    if (!s_layer_info.ctx) s_layer_info.init(device_number);
+    return s_layer_info;
+  }
+  void share_gpu(const layer_gpu_info& gpu) { s_layer_info.share(gpu); }
+
+  // src/softmax.hpp:3-100: sizes come from params; D and b_d are U(lower, upper)
+  void init_loss_layer(struct neuralMT_model<precision>* /*model*/, global_params& params) override {
+    output_vocab_size = params.target_vocab_size;
+    LSTM_size = params.LSTM_size;
+    minibatch_size = params.minibatch_size;
+    longest_sent = params.longest_sent;
+    zr_ctx* ctx = s_layer_info.ctx;
+    dType* h = nullptr;
+    full_matrix_setup(ctx, &h, &d_D, output_vocab_size, LSTM_size);
+    full_matrix_setup(ctx, &h, &d_b_d, output_vocab_size, 1);
+    const size_t vm = (size_t)output_vocab_size * minibatch_size;
+    ZOPH_CALL(zr_malloc(ctx, vm * sizeof(dType), (void**)&d_outputdist));
+    ZOPH_CALL(zr_malloc(ctx, vm * sizeof(dType), (void**)&d_logits));
+    const size_t nt = (size_t)minibatch_size * longest_sent;
+    ZOPH_CALL(zr_malloc(ctx, nt * sizeof(int), (void**)&d_output_vocab_indices));
+    ZOPH_CALL(zr_malloc(ctx, nt * sizeof(int), (void**)&d_output_vocab_indices_01));
+    ZOPH_CALL(zr_malloc(ctx, nt * sizeof(dType), (void**)&d_output_vocab_indices_01_float));
+    nodes.resize(longest_sent);
+    for (int i = 0; i < longest_sent; i++) nodes[i].index = i;
+  }
+  // src/softmax.hpp:926-947
+  void prep_GPU_vocab_indices(int* h_output_vocab_indicies_target, int current_target_length) override {
+    zr_ctx* ctx = s_layer_info.ctx;
+    const int n = minibatch_size * current_target_length;
+    ZOPH_CALL(zr_h2d(ctx, d_output_vocab_indices, h_output_vocab_indicies_target, (size_t)n * sizeof(int)));
+    ZOPH_CALL(zr_vocab_prep_softmax(ctx, d_output_vocab_indices, n, output_vocab_size, d_output_vocab_indices_01,
+                                    d_output_vocab_indices_01_float));
+  }
+  // src/softmax.hpp:907-923
+  void backprop_prep_GPU(dType* d_h_t, int step) override {
+    this->d_h_t = d_h_t;
+    backprop_prep_GPU_mgpu(step);
+  }
+  void backprop_prep_GPU_mgpu(int step) override {
+    d_output_vocab_indices_single = d_output_vocab_indices + step;
+    d_output_vocab_indices_01_single = d_output_vocab_indices_01 + step;
+  }
+  // src/softmax.hpp:459-485: probabilities of node `index` (training-style forward; the node keeps its d_h_t)
+  void forward_prop(int index) override {
+    zr_ctx* ctx = s_layer_info.ctx;
+    if (!nodes[index].d_outputdist)
+      ZOPH_CALL(zr_malloc(ctx, (size_t)output_vocab_size * minibatch_size * sizeof(dType),
+                          (void**)&nodes[index].d_outputdist));
+    ZOPH_CALL(zr_softmax_forward(ctx, d_D, d_b_d, output_vocab_size, LSTM_size, nodes[index].d_h_t, minibatch_size,
+                                 ZR_SOFTMAX_PROB, nodes[index].d_outputdist, nullptr));
+  }
+  // src/softmax.hpp:867-900 (get_perplexity_GPU + the host-side sum)
+  double compute_loss_GPU(int index) override {
+    zr_ctx* ctx = s_layer_info.ctx;
+    dType* h = nodes[index].d_h_t ? nodes[index].d_h_t : d_h_t;
+    double loss = 0;
+    ZOPH_CALL(zr_softmax_loss(ctx, d_D, d_b_d, output_vocab_size, LSTM_size, h, minibatch_size,
+                              d_output_vocab_indices_single, d_output_vocab_indices_01_single, d_logits, &loss));
+    return loss;
+  }
+  // src/softmax.hpp:636-692: the full double log-probability matrix of d_h_t into d_outputdist_perp
+  void get_perplexity_GPU(dType* d_h_t_in, int /*index*/) {
+    zr_ctx* ctx = s_layer_info.ctx;
+    if (!d_outputdist_perp)
+      ZOPH_CALL(zr_malloc(ctx, (size_t)output_vocab_size * minibatch_size * sizeof(double), (void**)&d_outputdist_perp));
+    ZOPH_CALL(zr_softmax_logprob_f64(ctx, d_D, d_b_d, output_vocab_size, LSTM_size, d_h_t_in, minibatch_size,
+                                     d_outputdist_perp, d_logits));
+  }
+  dType* get_ht_ptr(int index) override { return nodes[index].d_h_t; }
+  void set_ht_ptr(int index, dType* d_h_t) override { nodes[index].d_h_t = d_h_t; }
+  // src/softmax.hpp:1028-1030
+  void get_distribution_GPU_decoder_wrapper() override {
+    ZOPH_CALL(zr_softmax_forward(s_layer_info.ctx, d_D, d_b_d, output_vocab_size, LSTM_size, d_h_t, minibatch_size,
+                                 ZR_SOFTMAX_PROB, d_outputdist, nullptr));
+  }
+  dType* get_dist_ptr() override { return d_outputdist; }
+  // src/softmax.hpp:310-323
+  void dump_weights(std::ofstream& output) override {
+    write_matrix_GPU(s_layer_info.ctx, d_D, output_vocab_size, LSTM_size, output);
+    write_matrix_GPU(s_layer_info.ctx, d_b_d, output_vocab_size, 1, output);
+  }
+  void load_weights(std::ifstream& input) override {
+    read_matrix_GPU(s_layer_info.ctx, d_D, output_vocab_size, LSTM_size, input);
+    read_matrix_GPU(s_layer_info.ctx, d_b_d, output_vocab_size, 1, input);
+  }
+};
+
+// ------------------------------------------------------------------------------------------------ LSTM nodes
+template <typename dType>
+class LSTM_HH_Node {  // src/LSTM_HH.h:19-102
+ public:
+  int minibatch_size, LSTM_size, index;
+  bool attention_model = false;
+  bool dropout;
+  dType dropout_rate;
+  Hidden_To_Hidden_Layer<dType>* model;
+  dType *d_o_t = nullptr, *d_c_t = nullptr, *d_f_t = nullptr, *d_c_prime_t_tanh = nullptr, *d_i_t = nullptr,
+        *d_h_t = nullptr;
+  int* d_input_vocab_indices_01 = nullptr;
+  dType *d_c_t_prev = nullptr, *d_h_t_prev = nullptr;
+  dType* d_h_t_below = nullptr;
+  dType* d_zeros = nullptr;
+
+  LSTM_HH_Node(int LSTM_size, int minibatch_size, Hidden_To_Hidden_Layer<dType>* m, int index, dType* d_zeros,
+               bool dropout, dType dropout_rate);
+  void update_vectors_forward_GPU(int* d_input_vocab_indices_01, dType* d_h_t_prev, dType* d_c_t_prev) {
+    this->d_h_t_prev = d_h_t_prev;
+    this->d_c_t_prev = d_c_t_prev;
+    this->d_input_vocab_indices_01 = d_input_vocab_indices_01;
+  }
+  void update_vectors_forward_decoder(int* d_input_vocab_indices_01) {
+    this->d_input_vocab_indices_01 = d_input_vocab_indices_01;
+  }
+  void forward_prop() { forward_prop_GPU(); }
+  void forward_prop_GPU();
+  void send_h_t_above();
+};
+
+template <typename dType>
+class LSTM_IH_Node {  // src/LSTM.h:19-106
+ public:
+  int minibatch_size, LSTM_size, index;
+  bool dropout;
+  dType dropout_rate;
+  bool attention_model = false;
+  bool feed_input = false;
+  Input_To_Hidden_Layer<dType>* model;
+  dType *d_o_t = nullptr, *d_c_t = nullptr, *d_f_t = nullptr, *d_c_prime_t_tanh = nullptr, *d_i_t = nullptr,
+        *d_h_t = nullptr, *d_sparse_lookup = nullptr;
+  int *d_input_vocab_indices = nullptr, *d_input_vocab_indices_01 = nullptr;
+  dType *d_c_t_prev = nullptr, *d_h_t_prev = nullptr;
+  dType* d_zeros = nullptr;
+  dType* d_h_tild = nullptr;
+
+  LSTM_IH_Node(int LSTM_size, int minibatch_size, int vocab_size, Input_To_Hidden_Layer<dType>* m, int index,
+               dType* d_zeros, bool dropout, dType dropout_rate);
+  void update_vectors_forward_GPU(int* d_input_vocab_indices, int* d_input_vocab_indices_01, dType* d_h_t_prev,
+                                  dType* d_c_t_prev) {
+    this->d_h_t_prev = d_h_t_prev;
+    this->d_c_t_prev = d_c_t_prev;
+    this->d_input_vocab_indices = d_input_vocab_indices;
+    this->d_input_vocab_indices_01 = d_input_vocab_indices_01;
+  }
+  void update_vectors_forward_decoder(int* d_input_vocab_indices, int* d_input_vocab_indices_01) {
+    this->d_input_vocab_indices = d_input_vocab_indices;
+    this->d_input_vocab_indices_01 = d_input_vocab_indices_01;
+  }
+  void forward_prop() { forward_prop_GPU(); }
+  void forward_prop_GPU();
+  void attention_extra();  // src/LSTM.hpp:533-539
+  void send_h_t_above();
+};
+
+// ------------------------------------------------------------------------------------------------ layers
+template <typename dType>
+class Hidden_To_Hidden_Layer {  // src/Hidden_To_Hidden_Layer.h:12-313
+ public:
+  layer_gpu_info hh_layer_info;
+  std::vector<LSTM_HH_Node<dType>> nodes;
+  dType *d_W_hi = nullptr, *d_W_hf = nullptr, *d_W_hc = nullptr, *d_W_ho = nullptr;
+  dType *d_b_i = nullptr, *d_b_f = nullptr, *d_b_c = nullptr, *d_b_o = nullptr;
+  dType *d_M_i = nullptr, *d_M_f = nullptr, *d_M_o = nullptr, *d_M_c = nullptr;
+  dType *d_init_hidden_vector = nullptr, *d_init_cell_vector = nullptr, *d_zeros = nullptr;
+  int *d_input_vocab_indices_01_full = nullptr, *d_input_vocab_indices_full = nullptr;
+  int LSTM_size = 0, minibatch_size = 0, longest_sent = 0, layer_number = -1;
+  neuralMT_model<precision>* model = nullptr;
+  upper_transfer_layer<dType> upper_layer;
+  attention_layer<dType>* attent_layer = nullptr;
+  zr_lstm_weights* packed = nullptr;  // repacked lazily after init / load_weights
+
+  // src/Hidden_To_Hidden_Layer.hpp:125-155 (and :4-112 for the device side)
+  void init_Hidden_To_Hidden_Layer(int LSTM_size, int minibatch_size, int longest_sent, bool /*debug_temp*/,
+                                   dType /*learning_rate*/, bool /*clip_gradients*/, dType /*norm_clip*/,
+                                   struct neuralMT_model<precision>* model, int /*seed*/, bool dropout,
+                                   dType dropout_rate, bool /*bi_dir*/, int layer_number) {
+    this->LSTM_size = LSTM_size;
+    this->minibatch_size = minibatch_size;
+    this->longest_sent = longest_sent;
+    this->model = model;
+    this->layer_number = layer_number;
+    zr_ctx* ctx = hh_layer_info.ctx;
+    dType* h = nullptr;
+    dType** mats[] = {&d_W_hi, &d_W_hf, &d_W_hc, &d_W_ho, &d_M_i, &d_M_f, &d_M_o, &d_M_c};
+    for (dType** m : mats) full_matrix_setup(ctx, &h, m, LSTM_size, LSTM_size);
+    dType** vecs[] = {&d_b_i, &d_b_f, &d_b_c, &d_b_o};
+    for (dType** v : vecs) full_matrix_setup(ctx, &h, v, LSTM_size, 1);
+    device_fill(ctx, d_b_f, LSTM_size, (dType)1);  // forget bias 1 (:31-34)
+    full_matrix_setup_0(ctx, &d_init_hidden_vector, LSTM_size, minibatch_size);
+    full_matrix_setup_0(ctx, &d_init_cell_vector, LSTM_size, minibatch_size);
+    full_matrix_setup_0(ctx, &d_zeros, LSTM_size, minibatch_size);
+    const size_t nt = (size_t)minibatch_size * longest_sent;
+    ZOPH_CALL(zr_malloc(ctx, nt * sizeof(int), (void**)&d_input_vocab_indices_full));
+    ZOPH_CALL(zr_malloc(ctx, nt * sizeof(int), (void**)&d_input_vocab_indices_01_full));
+    for (int i = 0; i < longest_sent; i++)
+      nodes.push_back(LSTM_HH_Node<dType>(LSTM_size, minibatch_size, this, i, d_zeros, dropout, dropout_rate));
+  }
+  void repack() {
+    zr_ctx* ctx = hh_layer_info.ctx;
+    if (packed) ZOPH_CALL(zr_lstm_weights_destroy(ctx, packed));
+    const dType* M[4] = {d_M_i, d_M_f, d_M_c, d_M_o};
+    const dType* Wh[4] = {d_W_hi, d_W_hf, d_W_hc, d_W_ho};
+    const dType* b[4] = {d_b_i, d_b_f, d_b_c, d_b_o};
+    ZOPH_CALL(zr_lstm_pack_weights(ctx, M, Wh, nullptr, b, LSTM_size, &packed));
+  }
+  // src/Hidden_To_Hidden_Layer.hpp:748-774
+  void prep_GPU_vocab_indices(int* h_input_vocab_indicies, int current_length) {
+    zr_ctx* ctx = hh_layer_info.ctx;
+    const int n = minibatch_size * current_length;
+    ZOPH_CALL(zr_h2d(ctx, d_input_vocab_indices_full, h_input_vocab_indicies, (size_t)n * sizeof(int)));
+    ZOPH_CALL(zr_vocab_prep(ctx, d_input_vocab_indices_full, n, 0, nullptr, d_input_vocab_indices_01_full));
+  }
+  // model-file order (src/Hidden_To_Hidden_Layer.hpp:669-692)
+  void dump_weights(std::ofstream& output) {
+    zr_ctx* ctx = hh_layer_info.ctx;
+    write_matrix_GPU(ctx, d_W_hi, LSTM_size, LSTM_size, output);
+    write_matrix_GPU(ctx, d_b_i, LSTM_size, 1, output);
+    write_matrix_GPU(ctx, d_W_hf, LSTM_size, LSTM_size, output);
+    write_matrix_GPU(ctx, d_b_f, LSTM_size, 1, output);
+    write_matrix_GPU(ctx, d_W_hc, LSTM_size, LSTM_size, output);
+    write_matrix_GPU(ctx, d_b_c, LSTM_size, 1, output);
+    write_matrix_GPU(ctx, d_W_ho, LSTM_size, LSTM_size, output);
+    write_matrix_GPU(ctx, d_b_o, LSTM_size, 1, output);
+    write_matrix_GPU(ctx, d_M_i, LSTM_size, LSTM_size, output);
+    write_matrix_GPU(ctx, d_M_f, LSTM_size, LSTM_size, output);
+    write_matrix_GPU(ctx, d_M_o, LSTM_size, LSTM_size, output);
+    write_matrix_GPU(ctx, d_M_c, LSTM_size, LSTM_size, output);
+    if (attent_layer) attent_layer->dump_weights(output);
+  }
+  void load_weights(std::ifstream& input) {
+    zr_ctx* ctx = hh_layer_info.ctx;
+    read_matrix_GPU(ctx, d_W_hi, LSTM_size, LSTM_size, input);
+    read_matrix_GPU(ctx, d_b_i, LSTM_size, 1, input);
+    read_matrix_GPU(ctx, d_W_hf, LSTM_size, LSTM_size, input);
+    read_matrix_GPU(ctx, d_b_f, LSTM_size, 1, input);
+    read_matrix_GPU(ctx, d_W_hc, LSTM_size, LSTM_size, input);
+    read_matrix_GPU(ctx, d_b_c, LSTM_size, 1, input);
+    read_matrix_GPU(ctx, d_W_ho, LSTM_size, LSTM_size, input);
+    read_matrix_GPU(ctx, d_b_o, LSTM_size, 1, input);
+    read_matrix_GPU(ctx, d_M_i, LSTM_size, LSTM_size, input);
+    read_matrix_GPU(ctx, d_M_f, LSTM_size, LSTM_size, input);
+    read_matrix_GPU(ctx, d_M_o, LSTM_size, LSTM_size, input);
+    read_matrix_GPU(ctx, d_M_c, LSTM_size, LSTM_size, input);
+    if (attent_layer) attent_layer->load_weights(input);
+    repack();
+  }
+  // src/Hidden_To_Hidden_Layer.hpp:780-791: reorder the columns of node 0's h and c by the beam back-pointers
+  void swap_states_decoding(const int* d_indicies, int /*index*/, dType* d_temp_swap_vals) {
+    zr_ctx* ctx = hh_layer_info.ctx;
+    const size_t bytes = (size_t)LSTM_size * minibatch_size * sizeof(dType);
+    ZOPH_CALL(zr_gather_columns(ctx, nodes[0].d_h_t, LSTM_size, d_indicies, minibatch_size, d_temp_swap_vals));
+    ZOPH_CALL(zr_d2d(ctx, nodes[0].d_h_t, d_temp_swap_vals, bytes));
+    ZOPH_CALL(zr_gather_columns(ctx, nodes[0].d_c_t, LSTM_size, d_indicies, minibatch_size, d_temp_swap_vals));
+    ZOPH_CALL(zr_d2d(ctx, nodes[0].d_c_t, d_temp_swap_vals, bytes));
+  }
+  // src/Hidden_To_Hidden_Layer.hpp:801-813: one source column replicated over the beam
+  void transfer_decoding_states_GPU(dType* d_h_t, dType* d_c_t) {
+    zr_ctx* ctx = hh_layer_info.ctx;
+    ZOPH_CALL(zr_broadcast_column(ctx, d_h_t, LSTM_size, minibatch_size, d_init_hidden_vector));
+    ZOPH_CALL(zr_broadcast_column(ctx, d_c_t, LSTM_size, minibatch_size, d_init_cell_vector));
+    nodes[0].d_h_t_prev = d_init_hidden_vector;
+    nodes[0].d_c_t_prev = d_init_cell_vector;
+  }
+  // src/Hidden_To_Hidden_Layer.hpp (init_attention): the top target layer owns the attention layer
+  void init_attention(attention_layer<dType>* layer) {
+    attent_layer = layer;
+    for (size_t i = 0; i < nodes.size(); i++) {
+      nodes[i].attention_model = true;
+      attent_layer->nodes[i].d_indicies_mask = &nodes[i].d_input_vocab_indices_01;
+      attent_layer->nodes[i].d_h_t = nodes[i].d_h_t;
+    }
+  }
+};
+
+template <typename dType>
+class Input_To_Hidden_Layer {  // src/Input_To_Hidden_Layer.h:11-368
+ public:
+  layer_gpu_info ih_layer_info;
+  std::vector<LSTM_IH_Node<dType>> nodes;
+  dType* d_W = nullptr;  // embedding, LSTM_size x input_vocab_size
+  dType *d_W_hi = nullptr, *d_W_hf = nullptr, *d_W_hc = nullptr, *d_W_ho = nullptr;
+  dType *d_b_i = nullptr, *d_b_f = nullptr, *d_b_c = nullptr, *d_b_o = nullptr;
+  dType *d_M_i = nullptr, *d_M_f = nullptr, *d_M_o = nullptr, *d_M_c = nullptr;
+  dType *d_Q_i = nullptr, *d_Q_f = nullptr, *d_Q_o = nullptr, *d_Q_c = nullptr;
+  dType *d_init_hidden_vector = nullptr, *d_init_cell_vector = nullptr, *d_zeros = nullptr;
+  int *d_input_vocab_indices_full = nullptr, *d_input_vocab_indices_01_full = nullptr;
+  int LSTM_size = 0, minibatch_size = 0, input_vocab_size = 0, longest_sent = 0;
+  bool feed_input = false;
+  neuralMT_model<precision>* model = nullptr;
+  upper_transfer_layer<dType> upper_layer;
+  attention_layer<dType>* attent_layer = nullptr;
+  zr_lstm_weights* packed = nullptr;
+
+  // src/Input_To_Hidden_Layer.hpp:171-202 (and :3-159 for the device side)
+  void init_Input_To_Hidden_Layer(int LSTM_size, int minibatch_size, int vocab_size, int longest_sent,
+                                  bool /*debug_temp*/, dType /*learning_rate*/, bool /*clip_gradients*/,
+                                  dType /*norm_clip*/, struct neuralMT_model<precision>* model, int /*seed*/,
+                                  bool dropout, dType dropout_rate, bool /*is_bi_dir*/, bool share_embeddings,
+                                  dType* d_embedding_ptr, bool /*combine_embeddings*/, global_params& /*params*/,
+                                  bool /*source*/) {
+    this->LSTM_size = LSTM_size;
+    this->minibatch_size = minibatch_size;
+    this->input_vocab_size = vocab_size;
+    this->longest_sent = longest_sent;
+    this->model = model;
+    zr_ctx* ctx = ih_layer_info.ctx;
+    dType* h = nullptr;
+    dType** mats[] = {&d_W_hi, &d_W_hf, &d_W_hc, &d_W_ho, &d_M_i, &d_M_f, &d_M_o, &d_M_c};
+    for (dType** m : mats) full_matrix_setup(ctx, &h, m, LSTM_size, LSTM_size);
+    dType** vecs[] = {&d_b_i, &d_b_f, &d_b_c, &d_b_o};
+    for (dType** v : vecs) full_matrix_setup(ctx, &h, v, LSTM_size, 1);
+    device_fill(ctx, d_b_f, LSTM_size, (dType)1);  // forget bias 1 (:33-36)
+    if (share_embeddings)
+      d_W = d_embedding_ptr;
+    else
+      full_matrix_setup(ctx, &h, &d_W, LSTM_size, vocab_size);
+    full_matrix_setup_0(ctx, &d_init_hidden_vector, LSTM_size, minibatch_size);
+    full_matrix_setup_0(ctx, &d_init_cell_vector, LSTM_size, minibatch_size);
+    full_matrix_setup_0(ctx, &d_zeros, LSTM_size, minibatch_size);
+    const size_t nt = (size_t)minibatch_size * longest_sent;
+    ZOPH_CALL(zr_malloc(ctx, nt * sizeof(int), (void**)&d_input_vocab_indices_full));
+    ZOPH_CALL(zr_malloc(ctx, nt * sizeof(int), (void**)&d_input_vocab_indices_01_full));
+    for (int i = 0; i < longest_sent; i++)
+      nodes.push_back(LSTM_IH_Node<dType>(LSTM_size, minibatch_size, vocab_size, this, i, d_zeros, dropout, dropout_rate));
+  }
+  void repack() {
+    zr_ctx* ctx = ih_layer_info.ctx;
+    if (packed) ZOPH_CALL(zr_lstm_weights_destroy(ctx, packed));
+    const dType* M[4] = {d_M_i, d_M_f, d_M_c, d_M_o};
+    const dType* Wh[4] = {d_W_hi, d_W_hf, d_W_hc, d_W_ho};
+    const dType* Q[4] = {d_Q_i, d_Q_f, d_Q_c, d_Q_o};
+    const dType* b[4] = {d_b_i, d_b_f, d_b_c, d_b_o};
+    ZOPH_CALL(zr_lstm_pack_weights(ctx, M, Wh, feed_input ? Q : nullptr, b, LSTM_size, &packed));
+  }
+  // src/Input_To_Hidden_Layer.hpp:1178-1225 (the *_Wgrad arguments serve the embedding gradient only)
+  void prep_GPU_vocab_indices(int* h_input_vocab_indicies, int* /*h_input_vocab_indicies_Wgrad*/, int current_length,
+                              int /*len_W*/) {
+    zr_ctx* ctx = ih_layer_info.ctx;
+    const int n = minibatch_size * current_length;
+    ZOPH_CALL(zr_h2d(ctx, d_input_vocab_indices_full, h_input_vocab_indicies, (size_t)n * sizeof(int)));
+    // mask first, then -1 -> 0 in place (vocab_to_01 then vocab_to_nonM1, :1199-1202)
+    ZOPH_CALL(zr_vocab_prep(ctx, d_input_vocab_indices_full, n, input_vocab_size, d_input_vocab_indices_full,
+                            d_input_vocab_indices_01_full));
+  }
+  // src/Input_To_Hidden_Layer.hpp:242-317: Q matrices and per-node d_h_tild; attention node i feeds node i+1
+  void init_feed_input(Hidden_To_Hidden_Layer<dType>* hidden_layer, bool /*multi_attention*/) {
+    zr_ctx* ctx = ih_layer_info.ctx;
+    feed_input = true;
+    dType* h = nullptr;
+    dType** mats[] = {&d_Q_i, &d_Q_f, &d_Q_o, &d_Q_c};
+    for (dType** m : mats) full_matrix_setup(ctx, &h, m, LSTM_size, LSTM_size);
+    attention_layer<dType>* att = hidden_layer ? hidden_layer->attent_layer : attent_layer;
+    for (size_t i = 0; i < nodes.size(); i++) nodes[i].attention_extra();
+    if (att)
+      for (size_t i = 0; i + 1 < nodes.size(); i++) att->nodes[i].feed_input_init(nodes[i + 1].d_h_tild);
+    repack();
+  }
+  void decoder_init_feed_input() {  // :300-317: decode keeps a single node; h~ is copied in by the driver
+    zr_ctx* ctx = ih_layer_info.ctx;
+    feed_input = true;
+    dType* h = nullptr;
+    dType** mats[] = {&d_Q_i, &d_Q_f, &d_Q_o, &d_Q_c};
+    for (dType** m : mats) full_matrix_setup(ctx, &h, m, LSTM_size, LSTM_size);
+    nodes[0].attention_extra();
+    repack();
+  }
+  void init_attention(attention_layer<dType>* layer) {
+    attent_layer = layer;
+    for (size_t i = 0; i < nodes.size(); i++) {
+      nodes[i].attention_model = true;
+      attent_layer->nodes[i].d_indicies_mask = &nodes[i].d_input_vocab_indices_01;
+      attent_layer->nodes[i].d_h_t = nodes[i].d_h_t;
+    }
+  }
+  // model-file order (src/Input_To_Hidden_Layer.hpp:1050-1159)
+  void dump_weights(std::ofstream& output) {
+    zr_ctx* ctx = ih_layer_info.ctx;
+    write_matrix_GPU(ctx, d_W_hi, LSTM_size, LSTM_size, output);
+    write_matrix_GPU(ctx, d_b_i, LSTM_size, 1, output);
+    write_matrix_GPU(ctx, d_W_hf, LSTM_size, LSTM_size, output);
+    write_matrix_GPU(ctx, d_b_f, LSTM_size, 1, output);
+    write_matrix_GPU(ctx, d_W_hc, LSTM_size, LSTM_size, output);
+    write_matrix_GPU(ctx, d_b_c, LSTM_size, 1, output);
+    write_matrix_GPU(ctx, d_W_ho, LSTM_size, LSTM_size, output);
+    write_matrix_GPU(ctx, d_b_o, LSTM_size, 1, output);
+    write_matrix_GPU(ctx, d_W, LSTM_size, input_vocab_size, output);
+    write_matrix_GPU(ctx, d_M_i, LSTM_size, LSTM_size, output);
+    write_matrix_GPU(ctx, d_M_f, LSTM_size, LSTM_size, output);
+    write_matrix_GPU(ctx, d_M_o, LSTM_size, LSTM_size, output);
+    write_matrix_GPU(ctx, d_M_c, LSTM_size, LSTM_size, output);
+    if (feed_input) {
+      write_matrix_GPU(ctx, d_Q_i, LSTM_size, LSTM_size, output);
+      write_matrix_GPU(ctx, d_Q_f, LSTM_size, LSTM_size, output);
+      write_matrix_GPU(ctx, d_Q_o, LSTM_size, LSTM_size, output);
+      write_matrix_GPU(ctx, d_Q_c, LSTM_size, LSTM_size, output);
+    }
+    if (attent_layer) attent_layer->dump_weights(output);
+  }
+  void load_weights(std::ifstream& input) {
+    zr_ctx* ctx = ih_layer_info.ctx;
+    read_matrix_GPU(ctx, d_W_hi, LSTM_size, LSTM_size, input);
+    read_matrix_GPU(ctx, d_b_i, LSTM_size, 1, input);
+    read_matrix_GPU(ctx, d_W_hf, LSTM_size, LSTM_size, input);
+    read_matrix_GPU(ctx, d_b_f, LSTM_size, 1, input);
+    read_matrix_GPU(ctx, d_W_hc, LSTM_size, LSTM_size, input);
+    read_matrix_GPU(ctx, d_b_c, LSTM_size, 1, input);
+    read_matrix_GPU(ctx, d_W_ho, LSTM_size, LSTM_size, input);
+    read_matrix_GPU(ctx, d_b_o, LSTM_size, 1, input);
+    read_matrix_GPU(ctx, d_W, LSTM_size, input_vocab_size, input);
+    read_matrix_GPU(ctx, d_M_i, LSTM_size, LSTM_size, input);
+    read_matrix_GPU(ctx, d_M_f, LSTM_size, LSTM_size, input);
+    read_matrix_GPU(ctx, d_M_o, LSTM_size, LSTM_size, input);
+    read_matrix_GPU(ctx, d_M_c, LSTM_size, LSTM_size, input);
+    if (feed_input) {
+      read_matrix_GPU(ctx, d_Q_i, LSTM_size, LSTM_size, input);
+      read_matrix_GPU(ctx, d_Q_f, LSTM_size, LSTM_size, input);
+      read_matrix_GPU(ctx, d_Q_o, LSTM_size, LSTM_size, input);
+      read_matrix_GPU(ctx, d_Q_c, LSTM_size, LSTM_size, input);
+    }
+    if (attent_layer) attent_layer->load_weights(input);
+    repack();
+  }
+  // src/Input_To_Hidden_Layer.hpp:1231-1242
+  void swap_states_decoding(const int* d_indicies, int /*index*/, dType* d_temp_swap_vals) {
+    zr_ctx* ctx = ih_layer_info.ctx;
+    const size_t bytes = (size_t)LSTM_size * minibatch_size * sizeof(dType);
+    ZOPH_CALL(zr_gather_columns(ctx, nodes[0].d_h_t, LSTM_size, d_indicies, minibatch_size, d_temp_swap_vals));
+    ZOPH_CALL(zr_d2d(ctx, nodes[0].d_h_t, d_temp_swap_vals, bytes));
+    ZOPH_CALL(zr_gather_columns(ctx, nodes[0].d_c_t, LSTM_size, d_indicies, minibatch_size, d_temp_swap_vals));
+    ZOPH_CALL(zr_d2d(ctx, nodes[0].d_c_t, d_temp_swap_vals, bytes));
+  }
+  // src/Input_To_Hidden_Layer.hpp:1252-1266
+  void transfer_decoding_states_GPU(dType* d_h_t, dType* d_c_t) {
+    zr_ctx* ctx = ih_layer_info.ctx;
+    ZOPH_CALL(zr_broadcast_column(ctx, d_h_t, LSTM_size, minibatch_size, d_init_hidden_vector));
+    ZOPH_CALL(zr_broadcast_column(ctx, d_c_t, LSTM_size, minibatch_size, d_init_cell_vector));
+    nodes[0].d_h_t_prev = d_init_hidden_vector;
+    nodes[0].d_c_t_prev = d_init_cell_vector;
+  }
+};
+
+// ------------------------------------------------------------------------------------------------ node bodies
+template <typename dType>
+LSTM_HH_Node<dType>::LSTM_HH_Node(int LSTM_size, int minibatch_size, Hidden_To_Hidden_Layer<dType>* m, int index,
+                                  dType* d_zeros, bool dropout, dType dropout_rate) {
+  model = m;
+  this->dropout = dropout;
+  this->dropout_rate = dropout_rate;
+  this->minibatch_size = minibatch_size;
+  this->LSTM_size = LSTM_size;
+  this->index = index;
+  this->d_zeros = d_zeros;
+  zr_ctx* ctx = m->hh_layer_info.ctx;
+  dType** bufs[] = {&d_o_t, &d_c_t, &d_f_t, &d_c_prime_t_tanh, &d_i_t, &d_h_t};  // init_LSTM_GPU, src/LSTM_HH.hpp:21-39
+  for (dType** b : bufs) full_matrix_setup_0(ctx, b, LSTM_size, minibatch_size);
+}
+
+template <typename dType>
+void LSTM_HH_Node<dType>::forward_prop_GPU() {  // src/LSTM_HH.hpp:103-333
+  zr_ctx* ctx = model->hh_layer_info.ctx;
+  if (!model->packed) model->repack();
+  dType* gates[4] = {d_i_t, d_f_t, d_c_prime_t_tanh, d_o_t};
+  ZOPH_CALL(zr_lstm_step(ctx, model->packed, d_h_t_below, d_h_t_prev, d_c_t_prev, nullptr, d_input_vocab_indices_01,
+                         BZ_CUDA::clip_cell ? BZ_CUDA::cell_clip_threshold : 0.0f, minibatch_size, d_h_t, d_c_t, gates));
+  send_h_t_above();
+}
+
+template <typename dType>
+void LSTM_HH_Node<dType>::send_h_t_above() {  // src/LSTM_HH.hpp:337-423, pointer-passing branch
+  int idx = (model->model && model->model->decode) ? 0 : index;
+  dType* out = d_h_t;
+  if (attention_model && model->attent_layer) {
+    model->attent_layer->nodes[idx].d_h_t = d_h_t;
+    model->attent_layer->nodes[idx].forward_prop();
+    out = model->attent_layer->nodes[idx].d_final_temp_2;
+  }
+  if (model->upper_layer.upper_softmax) {
+    if (!model->upper_layer.source_side && model->upper_layer.softmax) model->upper_layer.softmax->set_ht_ptr(idx, out);
+  } else if (model->upper_layer.hidden_layer) {
+    model->upper_layer.hidden_layer->nodes[idx].d_h_t_below = out;
+  }
+}
+
+template <typename dType>
+LSTM_IH_Node<dType>::LSTM_IH_Node(int LSTM_size, int minibatch_size, int /*vocab_size*/,
+                                  Input_To_Hidden_Layer<dType>* m, int index, dType* d_zeros, bool dropout,
+                                  dType dropout_rate) {
+  model = m;
+  this->dropout = dropout;
+  this->dropout_rate = dropout_rate;
+  this->minibatch_size = minibatch_size;
+  this->LSTM_size = LSTM_size;
+  this->index = index;
+  this->d_zeros = d_zeros;
+  zr_ctx* ctx = m->ih_layer_info.ctx;
+  dType** bufs[] = {&d_o_t, &d_c_t, &d_f_t, &d_c_prime_t_tanh, &d_i_t, &d_sparse_lookup, &d_h_t};  // src/LSTM.hpp:23-42
+  for (dType** b : bufs) full_matrix_setup_0(ctx, b, LSTM_size, minibatch_size);
+}
+
+template <typename dType>
+void LSTM_IH_Node<dType>::attention_extra() {
+  full_matrix_setup_0(model->ih_layer_info.ctx, &d_h_tild, LSTM_size, minibatch_size);
+  feed_input = true;
+}
+
+template <typename dType>
+void LSTM_IH_Node<dType>::forward_prop_GPU() {  // src/LSTM.hpp:76-421
+  zr_ctx* ctx = model->ih_layer_info.ctx;
+  if (!model->packed) model->repack();
+  ZOPH_CALL(zr_embed_gather(ctx, model->d_W, LSTM_size, model->input_vocab_size, d_input_vocab_indices, minibatch_size,
+                            d_sparse_lookup));
+  dType* gates[4] = {d_i_t, d_f_t, d_c_prime_t_tanh, d_o_t};
+  const bool use_q = feed_input && index != 0;  // src/LSTM.hpp:154
+  ZOPH_CALL(zr_lstm_step(ctx, model->packed, d_sparse_lookup, d_h_t_prev, d_c_t_prev, use_q ? d_h_tild : nullptr,
+                         d_input_vocab_indices_01, BZ_CUDA::clip_cell ? BZ_CUDA::cell_clip_threshold : 0.0f,
+                         minibatch_size, d_h_t, d_c_t, gates));
+  send_h_t_above();
+}
+
+template <typename dType>
+void LSTM_IH_Node<dType>::send_h_t_above() {  // src/LSTM.hpp:424-520, pointer-passing branch
+  int idx = (model->model && model->model->decode) ? 0 : index;
+  dType* out = d_h_t;
+  if (attention_model && model->attent_layer) {
+    model->attent_layer->nodes[idx].d_h_t = d_h_t;
+    model->attent_layer->nodes[idx].forward_prop();
+    out = model->attent_layer->nodes[idx].d_final_temp_2;
+  }
+  if (model->upper_layer.upper_softmax) {
+    if (!model->upper_layer.source_side && model->upper_layer.softmax) model->upper_layer.softmax->set_ht_ptr(idx, out);
+  } else if (model->upper_layer.hidden_layer) {
+    model->upper_layer.hidden_layer->nodes[idx].d_h_t_below = out;
+  }
+}
+
+#endif  // ZOPH_LAYERS_H
