@@ -463,3 +463,52 @@ def test_bad_arguments_return_errors(ctx):
         ctx.lstm_step(layer.w, buf, buf, buf, ctx.array(np.ones(4, np.int32)), 4, ctx.empty((16, 4)), ctx.empty((16, 4)),
                       d_htild=buf)
     layer.close()
+
+
+# ------------------------------------------------------------------------------------------------ split-K LSTM kernel
+@pytest.mark.parametrize("H,mb", [(32, 3), (100, 8), (72, 33), (252, 70), (1000, 128), (64, 150)])
+@pytest.mark.parametrize("kparts", [0, 1, 2, 3, 5])
+def test_lstm_step_lds_split_kernel(ctx, H, mb, kparts):
+    """The LDS / split-K kernel forced on every shape (it is picked automatically only for wide batches): odd chunk
+    counts, partial row tiles, partial column tiles, several K parts, with and without the feed-input segment."""
+    g = synth.rng(16, H * 1000 + mb + kparts)
+    ly = synth.lstm_layer(g, H, feed_input=True, forget_bias_one=True)
+    x, hp, cp, ht = U(g, (H, mb), -1, 1), U(g, (H, mb), -1, 1), U(g, (H, mb), -1, 1), U(g, (H, mb), -1, 1)
+    mask = (g.random(mb) > 0.2).astype(np.int32)
+    layer = Layer(ctx, ly)
+    ctx.set_option(capi.ZR_OPT_LSTM_KERNEL, 2)
+    ctx.set_option(capi.ZR_OPT_LSTM_KPARTS, kparts)
+    try:
+        got = run_lstm_step(ctx, layer, x, hp, cp, mask, want_gates=True)
+        got_feed = run_lstm_step(ctx, layer, x, hp, cp, mask, htild=ht, clip=0.7)
+        again = run_lstm_step(ctx, layer, x, hp, cp, mask, htild=ht, clip=0.7)
+    finally:
+        ctx.set_option(capi.ZR_OPT_LSTM_KERNEL, 0)
+        ctx.set_option(capi.ZR_OPT_LSTM_KPARTS, 0)
+        layer.close()
+    want = o.lstm_step(ly["M"], ly["Wh"], ly["b"], x, hp, cp, mask)
+    want_feed = o.lstm_step(ly["M"], ly["Wh"], ly["b"], x, hp, cp, mask, Q=ly["Q"], htild=ht, clip=0.7)
+    for k in ("i", "f", "c_tilde", "o", "c", "h"):
+        assert_close(got[k], want[k], what="%s (H=%d mb=%d kparts=%d)" % (k, H, mb, kparts))
+    assert_close(got_feed["h"], want_feed["h"], what="feed h")
+    assert_close(got_feed["c"], want_feed["c"], what="feed c")
+    # the cross-workgroup reduction adds partials in a fixed order: bit-identical from run to run
+    assert got_feed["h"].tobytes() == again["h"].tobytes() and got_feed["c"].tobytes() == again["c"].tobytes()
+
+
+def test_stack_forward_with_split_kernel_forced(ctx):
+    g = synth.rng(17, 1)
+    H, mb, T, V, L = 64, 5, 7, 211, 3
+    embed = U(g, (H, V))
+    layers = [synth.lstm_layer(g, H, forget_bias_one=True) for _ in range(L)]
+    ids = g.integers(0, V, size=(T, mb)).astype(np.int32)
+    ids[:3, 1] = -1
+    ctx.set_option(capi.ZR_OPT_LSTM_KERNEL, 2)
+    try:
+        hs, cs = _run_stack(ctx, layers, embed, ids)
+    finally:
+        ctx.set_option(capi.ZR_OPT_LSTM_KERNEL, 0)
+    nn, m = o.vocab_prep(ids)
+    want_h, want_c = o.lstm_stack_forward(embed, layers, nn, m)
+    assert_close(hs, want_h, what="stack h")
+    assert_close(cs, want_c, what="stack c")

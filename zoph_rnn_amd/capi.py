@@ -16,6 +16,8 @@ ZR_OPT_LSTM_FUSED_EPILOGUE = 1
 ZR_OPT_LSTM_TN = 2
 ZR_OPT_GEMM_CFG = 3
 ZR_OPT_LSTM_KSPLIT = 4
+ZR_OPT_LSTM_KERNEL = 5
+ZR_OPT_LSTM_KPARTS = 6
 ZR_SOFTMAX_PROB = 0
 ZR_SOFTMAX_LOGPROB = 1
 

@@ -7,6 +7,8 @@
 
 #include "../../include/zoph_rnn.h"
 
+#define ZR_MAX_COUNTERS 4096
+
 struct zr_ctx {
   int device;
   hipStream_t own_stream;
@@ -17,6 +19,9 @@ struct zr_ctx {
   int lstm_fused;
   int lstm_tn;
   int lstm_ksplit;
+  int lstm_kernel;   // 0 auto, 1 register-streaming kernel, 2 LDS / split-K kernel
+  int lstm_kparts;   // K parts per segment for the split-K kernel (0 auto)
+  int* d_counters;   // ZR_MAX_COUNTERS arrival counters, zero between launches
   int gemm_cfg;
   // scratch owned by the context (grown on demand, never shrunk)
   void* d_scratch;

@@ -35,6 +35,7 @@ struct LstmUnit {
 struct LstmLaunch {
   LstmUnit u[kMaxUnits];
   int n_units;
+  int nseg_max;             // largest nseg among the units
   int H, mb;
   float clip;
   int j_tiles, n_tiles;
@@ -126,6 +127,256 @@ __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
   });
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Second kernel: weights staged through LDS and shared by the waves of a workgroup, K split ACROSS workgroups.
+//
+// Why: with one 128-row x 64-column tile per CU and full K, every CU pulls (128 + 64) * K floats through its L1,
+// 384 MB per 4-node launch, and the kernel runs at the L1 fill rate (about 18 GB/s per CU) rather than at the MFMA
+// rate.  The traffic per CU is (rows + cols) * K for a fixed rows * cols * K of work, so it falls when a CU owns a
+// bigger tile over a shorter K range.  Here a workgroup owns 32 rows x 4 gates x (NWV * 32 * TN) columns -- all
+// 128 columns of the benchmark minibatch -- for one K segment (or a part of one): its NWV waves take 32*TN
+// columns each, share every weight chunk through LDS (read from L2 once per workgroup, 16-byte coalesced), and
+// fetch only their own activation columns.  The S = segments x parts workgroups of a tile write their partial
+// tiles to a scratch buffer; the last one to arrive (device-scope counter) adds the partials in split order --
+// the same order whoever is last, so results are deterministic -- and runs the gate/cell epilogue in registers.
+// ---------------------------------------------------------------------------------------------------------
+struct LstmLaunch2 {
+  LstmLaunch base;
+  int kparts;        // K parts per segment
+  int n_chunks;      // ceil(H / 32)
+  float* partials;   // [tile][split][wave][4*TN*16][64]
+  int* counters;     // [tile], zero between launches
+};
+
+template <int TN, int NWV>
+__global__ void __launch_bounds__(64 * NWV) lstm_lds_kernel(LstmLaunch2 P) {
+  constexpr int KC = 32;                       // k per chunk
+  constexpr int NTHR = 64 * NWV;
+  constexpr int F4_PER_CHUNK = KC * 4 * 8;     // float4 per weight chunk: 32 k x 4 gates x 8 (32 rows / 4)
+  constexpr int WLD = (F4_PER_CHUNK + NTHR - 1) / NTHR;  // float4 loads per thread per chunk
+  __shared__ zr_f32x4 Ws4[2][F4_PER_CHUNK];
+  __shared__ int s_last;
+  const LstmLaunch& L = P.base;
+  const int id = blockIdx.x;
+  const int r8 = id & 7;
+  const int q = id >> 3;
+  const int splits = L.nseg_max * P.kparts;
+  const int sp = q % splits;
+  const int tile = (q / splits) * 8 + r8;
+  const int n_tiles_total = L.n_units * L.j_tiles * L.n_tiles;
+  if (tile >= n_tiles_total) return;
+  const int nt = tile % L.n_tiles;
+  const int jt = (tile / L.n_tiles) % L.j_tiles;
+  const int unit = tile / (L.n_tiles * L.j_tiles);
+  const LstmUnit& U = L.u[unit];
+  const int seg = sp / P.kparts;
+  const int part = sp % P.kparts;
+  const bool seg_live = seg < U.nseg;  // units with fewer segments than the launch maximum contribute zeros
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int jl = lane & 31;
+  const int half = lane >> 5;
+  const int H = L.H;
+  const int j0 = jt * 32;
+  const int n0 = nt * (32 * TN * NWV) + wave * (32 * TN);
+  const int j = j0 + jl;
+
+  const int c_begin = (int)((long long)P.n_chunks * part / P.kparts);
+  const int c_end = (int)((long long)P.n_chunks * (part + 1) / P.kparts);
+
+  // this lane's activation columns (segment `seg`)
+  const float* xcol[TN];
+#pragma unroll
+  for (int tn = 0; tn < TN; ++tn) {
+    int c = n0 + tn * 32 + jl;
+    c = c < L.mb ? c : L.mb - 1;
+    long long col = c;
+    const int s_eff = seg_live ? seg : 0;
+    if (s_eff == 0 && U.gather_ids) {
+      int idv = U.gather_ids[c];
+      idv = idv < 0 ? 0 : (idv >= U.V ? U.V - 1 : idv);
+      col = idv;
+    }
+    xcol[tn] = U.in[s_eff] + col * H;
+  }
+  // this thread's share of a weight chunk: float4 index f -> (kk, gate, j4)
+  const float* wsrc[WLD];
+  bool wok_row[WLD];
+  int wkk[WLD];
+  const long long HH = (long long)H * H;
+#pragma unroll
+  for (int u = 0; u < WLD; ++u) {
+    const int f = tid + NTHR * u;
+    const int j4 = f & 7, g = (f >> 3) & 3, kk = f >> 5;
+    const int row = j0 + 4 * j4;
+    wok_row[u] = seg_live && (row < H) && (f < F4_PER_CHUNK);
+    wkk[u] = kk;
+    const int rowc = row < H ? row : H - 4;
+    wsrc[u] = U.W + ((long long)(seg_live ? seg : 0) * 4 + g) * HH + rowc;
+  }
+
+  zr_f32x16 acc[4][TN];
+#pragma unroll
+  for (int g = 0; g < 4; ++g)
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[g][tn][r] = 0.0f;
+
+  zr_f32x4 wreg[WLD];
+  zr_f32x4 xf[2][4][TN];
+
+  // All loads are unconditional with clamped addresses; invalid weights are zeroed by a select.  (Loads under
+  // branches stop the compiler from counting loads in flight and force full waits.)
+  auto gload = [&](int c, zr_f32x4 (&xdst)[4][TN]) {
+    const int cc = c < c_end ? c : c_end - 1;       // dummy chunk (odd chunk count): clamp, weights zeroed
+    const bool chunk_ok = c < c_end;
+#pragma unroll
+    for (int u = 0; u < WLD; ++u) {
+      const int k = cc * KC + wkk[u];
+      const int kc = k < H ? k : H - 1;
+      const zr_f32x4 v = *(const zr_f32x4*)(wsrc[u] + (long long)kc * H);
+      // zero by multiplication (weights are finite): a select would let the compiler skip the load under a
+      // branch, and loads under branches defeat its in-flight load counting
+      const float keep = (chunk_ok && wok_row[u] && (k < H)) ? 1.0f : 0.0f;
+      wreg[u].x = v.x * keep;
+      wreg[u].y = v.y * keep;
+      wreg[u].z = v.z * keep;
+      wreg[u].w = v.w * keep;
+    }
+#pragma unroll
+    for (int gq = 0; gq < 4; ++gq) {
+      // this lane multiplies k = kx .. kx+3; past the end of the column the matching weights are zero, so
+      // any valid address will do
+      int kx = cc * KC + 8 * gq + 4 * half;
+      kx = (kx + 4 <= H) ? kx : H - 4;
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) xdst[gq][tn] = *(const zr_f32x4*)(xcol[tn] + kx);
+    }
+  };
+  auto lds_store = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < WLD; ++u) {
+      const int f = tid + NTHR * u;
+      if (f < F4_PER_CHUNK) Ws4[buf][f] = wreg[u];
+    }
+  };
+  auto compute = [&](int buf, const zr_f32x4 (&xs)[4][TN]) {
+    // LDS -> register fragments one k-group ahead of the MFMAs that use them (16 weights per group per lane)
+    const float* Ws = (const float*)&Ws4[buf][0] + (4 * half * 4) * 32 + jl;
+    float wf[2][4][4];
+    auto lds_frag = [&](float (&dst)[4][4], int gq) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) dst[i][g] = Ws[((8 * gq + i) * 4 + g) * 32];
+    };
+    lds_frag(wf[0], 0);
+#pragma unroll
+    for (int gq = 0; gq < 4; ++gq) {
+      if (gq + 1 < 4) lds_frag(wf[(gq + 1) & 1], gq + 1);
+      // keep the LDS reads ahead of the MFMAs: left alone, the scheduler sinks each read to just before its use
+      // (shortest live range) and the matrix pipe idles for an LDS round trip every other instruction
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+          for (int tn = 0; tn < TN; ++tn)
+            acc[g][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(xs[gq][tn][i], wf[gq & 1][i][g], acc[g][tn], 0, 0, 0);
+    }
+  };
+
+  if (c_begin < c_end) {
+    gload(c_begin, xf[0]);
+    lds_store(0);
+    __syncthreads();
+    for (int c = c_begin; c < c_end; c += 2) {
+      // even stage: chunk c from buffer 0, prefetch c+1 into buffer 1
+      gload(c + 1, xf[1]);
+      compute(0, xf[0]);
+      lds_store(1);
+      __syncthreads();
+      // odd stage: chunk c+1 (all-zero weights if past the end) from buffer 1, prefetch c+2 into buffer 0
+      gload(c + 2, xf[0]);
+      compute(1, xf[1]);
+      lds_store(0);
+      __syncthreads();
+    }
+  }
+
+  const int jc = j < H ? j : H - 1;
+  const float bi = U.bias[jc], bf = U.bias[H + jc], bc = U.bias[2 * H + jc], bo = U.bias[3 * H + jc];
+  constexpr int SLOTS = 4 * TN * 16;
+  if (splits > 1) {
+    float* mine = P.partials + (((long long)tile * splits + sp) * NWV + wave) * (SLOTS * 64);
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          __hip_atomic_store(mine + ((g * TN + tn) * 16 + r) * 64 + lane, acc[g][tn][r], __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+    // The partials are written and read with device-scope atomic accesses (write-through / cache-bypassing on
+    // this multi-die part), so no L2 write-back + invalidate is needed to publish them -- a full device-scope
+    // fence here costs more than the whole K loop.  The workgroup-scope fence drains this wave's outstanding
+    // stores before the barrier; the counter increment after the barrier is a device-scope atomic.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    if (tid == 0) {
+      const int old = atomicAdd(&P.counters[tile], 1);
+      s_last = (old == splits - 1) ? 1 : 0;
+    }
+    __syncthreads();
+    if (!s_last) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    const float* base = P.partials + ((long long)tile * splits * NWV + wave) * (SLOTS * 64);
+    // split order k = 0, 1, ... for every finisher: the sum does not depend on which workgroup arrived last.
+    // All loads of one split are issued before any is consumed.
+    for (int k = 0; k < splits; ++k) {
+      const float* pk = base + (long long)k * NWV * (SLOTS * 64) + lane;
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) {
+          float t[16];
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            t[r] = __hip_atomic_load(pk + ((g * TN + tn) * 16 + r) * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[g][tn][r] = (k == 0) ? t[r] : acc[g][tn][r] + t[r];
+        }
+    }
+    if (tid == 0) __hip_atomic_store(&P.counters[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // next launch
+  }
+  if (j < H) {
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int n = n0 + tn * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+        if (n < L.mb) {
+          const long long ix = (long long)n * H + j;
+          float gi, gf, gc, go, c, h;
+          zr_lstm_cell(acc[0][tn][r] + bi, acc[1][tn][r] + bf, acc[2][tn][r] + bc, acc[3][tn][r] + bo, U.cprev[ix],
+                       (float)U.mask01[n], L.clip, gi, gf, gc, go, c, h);
+          U.c[ix] = c;
+          U.h[ix] = h;
+          if (U.gates[0]) {
+            U.gates[0][ix] = gi;
+            U.gates[1][ix] = gf;
+            U.gates[2][ix] = gc;
+            U.gates[3][ix] = go;
+          }
+        }
+      }
+  }
+}
+
 template <int TN, int KS>
 int launch_fused_v(zr_ctx* ctx, const LstmLaunch& L, bool vec) {
   const int groups = L.n_units * L.j_tiles;
@@ -138,9 +389,54 @@ int launch_fused_v(zr_ctx* ctx, const LstmLaunch& L, bool vec) {
   return ZR_OK;
 }
 
+template <int TN, int NWV>
+int launch_lds_v(zr_ctx* ctx, LstmLaunch& L) {
+  LstmLaunch2 P;
+  L.n_tiles = (L.mb + 32 * TN * NWV - 1) / (32 * TN * NWV);
+  const int tiles = L.n_units * L.j_tiles * L.n_tiles;
+  P.n_chunks = (L.H + 31) / 32;
+  int kparts = ctx->lstm_kparts;
+  if (kparts == 0) {
+    // about one workgroup per CU, not more: the finishing workgroup of a tile reads every partial, so its tail
+    // grows with the number of splits
+    kparts = 256 / (tiles * L.nseg_max);
+    if (kparts > 8) kparts = 8;
+  }
+  if (kparts > P.n_chunks) kparts = P.n_chunks;
+  if (kparts < 1) kparts = 1;
+  P.kparts = kparts;
+  const int splits = L.nseg_max * kparts;
+  void* scratch = nullptr;
+  const size_t bytes = sizeof(float) * (size_t)tiles * splits * NWV * (4 * TN * 16 * 64);
+  int rc = zr_ctx_scratch(ctx, 0, bytes, &scratch);
+  if (rc) return rc;
+  P.partials = (float*)scratch;
+  P.counters = ctx->d_counters;
+  P.base = L;
+  const int grid = ((tiles + 7) / 8) * 8 * splits;
+  lstm_lds_kernel<TN, NWV><<<grid, 64 * NWV, 0, ctx->stream>>>(P);
+  ZR_LAUNCH_CHECK("lstm_lds_kernel");
+  return ZR_OK;
+}
+
 int launch_fused(zr_ctx* ctx, LstmLaunch& L, bool vec) {
   L.j_tiles = (L.H + 31) / 32;
   const int n32 = (L.mb + 31) / 32;
+  L.nseg_max = 0;
+  for (int i = 0; i < L.n_units; ++i) L.nseg_max = L.u[i].nseg > L.nseg_max ? L.u[i].nseg : L.nseg_max;
+  // Kernel choice.  The register-streaming kernel needs no cross-workgroup reduction and wins whenever it can put
+  // a workgroup on (nearly) every CU -- a full diagonal of an encoder does.  A single node (a decoder step) gives
+  // it only ceil(H/32) * ceil(mb/64) workgroups; there the LDS / split-K kernel spreads the same node over ~256
+  // workgroups.  It needs 16-byte aligned operands and a batch wide enough for its 128-column tile.
+  int kernel = ctx->lstm_kernel;
+  if (kernel == 0) {
+    const long long wgs1 = (long long)L.n_units * L.j_tiles * ((n32 + 1) / 2);
+    kernel = (vec && n32 >= 3 && wgs1 < 200) ? 2 : 1;
+  }
+  if (kernel == 2 && vec && L.n_units * L.j_tiles * ((n32 + 3) / 4) <= ZR_MAX_COUNTERS) {
+    if (n32 > 4 && ctx->lstm_tn == 2) return launch_lds_v<2, 4>(ctx, L);
+    return launch_lds_v<1, 4>(ctx, L);
+  }
   int tn = ctx->lstm_tn;
   if (tn == 0) {
     // largest column tile that still yields at least one workgroup per CU

@@ -63,13 +63,14 @@ int zr_ctx_create(int device, zr_ctx** out) {
     return zr_set_error(ZR_EHIP, "hipStreamCreate failed: %s", hipGetErrorString(e));
   }
   c->stream = c->own_stream;
-  e = hipMalloc((void**)&c->d_flags, 4 * sizeof(int));
+  e = hipMalloc((void**)&c->d_flags, (4 + ZR_MAX_COUNTERS) * sizeof(int));
   if (e != hipSuccess) {
     (void)hipStreamDestroy(c->own_stream);
     delete c;
     return zr_set_error(ZR_ENOMEM, "flag allocation failed: %s", hipGetErrorString(e));
   }
-  (void)hipMemset(c->d_flags, 0, 4 * sizeof(int));
+  (void)hipMemset(c->d_flags, 0, (4 + ZR_MAX_COUNTERS) * sizeof(int));
+  c->d_counters = c->d_flags + 4;
   c->lstm_fused = 1;
   *out = c;
   return ZR_OK;
@@ -123,6 +124,14 @@ int zr_ctx_set_option(zr_ctx* ctx, int option, int value) {
     case ZR_OPT_LSTM_KSPLIT:
       ZR_CHECK_ARG(value == 0 || value == 4 || value == 8, "ZR_OPT_LSTM_KSPLIT must be 0, 4 or 8");
       ctx->lstm_ksplit = value;
+      return ZR_OK;
+    case ZR_OPT_LSTM_KERNEL:
+      ZR_CHECK_ARG(value >= 0 && value <= 2, "ZR_OPT_LSTM_KERNEL must be 0, 1 or 2");
+      ctx->lstm_kernel = value;
+      return ZR_OK;
+    case ZR_OPT_LSTM_KPARTS:
+      ZR_CHECK_ARG(value >= 0 && value <= 16, "ZR_OPT_LSTM_KPARTS must be in [0, 16]");
+      ctx->lstm_kparts = value;
       return ZR_OK;
     case ZR_OPT_GEMM_CFG:
       ZR_CHECK_ARG(value >= 0 && value <= 8, "ZR_OPT_GEMM_CFG out of range");
