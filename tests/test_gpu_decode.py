@@ -1,0 +1,117 @@
+"""End-to-end beam decode (BASELINE config 4 wiring at sizes the oracle finishes in seconds): encoder, then per step
+embedding gather -> LSTM stack with feed-input -> attention -> softmax -> device-side beam -> state reorder, for
+several sentences side by side, against one oracle decode per sentence (the reference decodes one sentence per
+pass).  Selected words and back-pointers must be identical at every step, hypotheses identical at the end."""
+import numpy as np
+import pytest
+
+import oracle_lib as o
+from zoph_rnn_amd import capi, driver, synth
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = capi.Context(0)
+    yield c
+    c.close()
+
+
+def _model(g, H, Vs, Vt, L):
+    m = {"src_embed": synth.uniform(g, (H, Vs), -0.5, 0.5), "tgt_embed": synth.uniform(g, (H, Vt), -0.5, 0.5),
+         "src_layers": [synth.lstm_layer(g, H, forget_bias_one=True) for _ in range(L)],
+         "tgt_layers": [synth.lstm_layer(g, H, feed_input=(l == 0), forget_bias_one=True) for l in range(L)],
+         "attn": synth.attention_weights(g, H),
+         # a peaked output distribution keeps candidate scores well separated (no near-ties for fp32 noise to flip)
+         "D_soft": synth.uniform(g, (Vt, H), -3.0, 3.0), "b_soft": synth.uniform(g, (Vt,), -1.0, 1.0)}
+    for ly in m["src_layers"] + m["tgt_layers"]:
+        for k in ("M", "Wh"):
+            ly[k] = [synth.uniform(g, (H, H), -0.3, 0.3) for _ in range(4)]
+    for k in ("W_a", "W_p", "W_c1", "W_c2"):
+        m["attn"][k] = synth.uniform(g, (H, H), -0.3, 0.3)
+    return m
+
+
+def _oracle_decode(m, src_col, src_len, S, beam, steps, D, penalty):
+    """One sentence, minibatch = beam, following forward_prop_source / forward_prop_target / swap_decoding_states."""
+    H, L, Vt = m["src_embed"].shape[0], len(m["src_layers"]), m["D_soft"].shape[0]
+    nn, mk = o.vocab_prep(src_col.reshape(S, 1))
+    hs, cs = o.lstm_stack_forward(m["src_embed"], m["src_layers"], nn, mk)
+    table = np.repeat(hs[L - 1], beam, axis=2)  # (S, H, beam)
+    hp = [np.repeat(np.asfortranarray(hs[l, S - 1]), beam, axis=1) for l in range(L)]
+    cp = [np.repeat(np.asfortranarray(cs[l, S - 1]), beam, axis=1) for l in range(L)]
+    binfo = np.concatenate([np.full(beam, src_len, np.int32), np.full(beam, S - src_len, np.int32)])
+    ones = np.ones(beam, np.int32)
+    dec = o.Decoder(beam, Vt, steps + 3, penalty=penalty)
+    words = np.zeros(beam, np.int32)
+    h_tild = None
+    hist, min_gap = [], np.inf
+
+    def forward(index):
+        nonlocal hp, cp, h_tild
+        below = o.embed_gather(m["tgt_embed"], np.maximum(words, 0))
+        newh, newc = [], []
+        for l in range(L):
+            ly = m["tgt_layers"][l]
+            feed = l == 0 and index > 0
+            r = o.lstm_step(ly["M"], ly["Wh"], ly["b"], below, hp[l], cp[l], ones, Q=ly["Q"] if feed else None,
+                            htild=h_tild if feed else None)
+            newh.append(r["h"])
+            newc.append(r["c"])
+            below = r["h"]
+        att = o.attention_forward(hs_table=table, batch_info=binfo, h_t=below, mask01=ones, D=D, **m["attn"])
+        P = o.softmax_dist(o.softmax_logits(m["D_soft"], m["b_soft"], att["h_tild"]))
+        return newh, newc, att, P
+
+    for index in range(steps):
+        newh, newc, att, P = forward(index)
+        # how close the closest pair of candidate scores is (the test is only meaningful without near-ties)
+        cols = 1 if index == 0 else beam
+        sc = dec.state()["scores"]
+        cand = np.sort(np.concatenate([np.log(np.sort(P[:, i])[-(beam + 2):]) + sc[i] for i in range(cols)]))
+        min_gap = min(min_gap, np.min(np.diff(cand)))
+        frac = att["p_t"] - np.floor(att["p_t"])
+        assert np.all((frac > 1e-4) & (frac < 1 - 1e-4)), "p_t on an integer boundary; pick another seed"
+        dec.expand(P, index)
+        st = dec.state()
+        words, back = st["current_indices"].copy(), st["new_indicies_changes"].copy()
+        hist.append((words.copy(), back.copy()))
+        hp = [np.asfortranarray(a[:, back]) for a in newh]
+        cp = [np.asfortranarray(a[:, back]) for a in newc]
+        h_tild = np.asfortranarray(att["h_tild"][:, back])
+    _, _, _, P = forward(steps)
+    dec.finish(P)
+    return hist, dec.hypotheses(), min_gap
+
+
+@pytest.mark.parametrize("H,L,beam,n_sent,S,steps,D", [(64, 2, 4, 3, 7, 6, 3), (48, 1, 3, 2, 5, 5, 10), (100, 3, 12, 2, 9, 4, 10)])
+def test_batched_beam_decode_matches_per_sentence_reference(ctx, H, L, beam, n_sent, S, steps, D):
+    g = synth.rng(61, H + beam)
+    Vs, Vt = 80, 400
+    m = _model(g, H, Vs, Vt, L)
+    lens = g.integers(max(2, S - 3), S + 1, size=n_sent).astype(np.int32)
+    lens[0] = S
+    src = g.integers(0, Vs, size=(S, n_sent)).astype(np.int32)
+    for s in range(n_sent):
+        src[:S - lens[s], s] = -1
+    w = driver.Seq2SeqWeights(ctx, m["src_embed"], m["src_layers"], m["tgt_embed"], m["tgt_layers"], m["attn"],
+                              m["D_soft"], m["b_soft"])
+    dec = driver.BeamDecode(ctx, w, beam, n_sent, S, steps, attention_D=D, penalty=0.0)
+    dec.encode(src, lens)
+    for _ in range(steps):
+        dec.step(record=True)
+    dec.finish()
+    for s in range(n_sent):
+        hist, hyps, gap = _oracle_decode(m, src[:, s], int(lens[s]), S, beam, steps, D, 0.0)
+        assert gap > 5e-6, "candidate scores nearly tie (gap %.2e): pick another seed" % gap
+        for index in range(steps):
+            gw, gb = dec.history[index]
+            assert np.array_equal(gw[s * beam:(s + 1) * beam], hist[index][0]), (s, index)
+            assert np.array_equal(gb[s * beam:(s + 1) * beam] - s * beam, hist[index][1]), (s, index)
+        got = dec.hypotheses(s)
+        assert len(got) == len(hyps)
+        for (gwords, gscore), (wwords, wscore) in zip(got, hyps):
+            assert np.array_equal(gwords, wwords)
+            assert gscore == pytest.approx(wscore, rel=1e-4, abs=1e-4)
+    dec.close()
