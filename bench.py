@@ -166,6 +166,42 @@ def bench_hbm_kernels(ctx, steps, H=1000, mb=128, V=50000):
     return out
 
 
+def bench_beam_decode(ctx, steps, H=1000, L=4, beam=12, n_sent=16, S=50, V=50000, D=10):
+    """Config 4: batched beam decode (16 sentences x beam 12 = 192 columns), per decode step: gather, 4 LSTM layers
+    with feed-input, attention (reference default width D=10), full softmax, device-side beam, state reorder."""
+    from zoph_rnn_amd import driver, synth
+    g = synth.rng(1234, 4)
+    src_layers = [synth.lstm_layer(g, H) for _ in range(L)]
+    tgt_layers = [synth.lstm_layer(g, H, feed_input=(l == 0)) for l in range(L)]
+    w = driver.Seq2SeqWeights(ctx, synth.uniform(g, (H, V)), src_layers, synth.uniform(g, (H, V)), tgt_layers,
+                              synth.attention_weights(g, H), synth.uniform(g, (V, H)), synth.uniform(g, (V,)))
+    dec = driver.BeamDecode(ctx, w, beam, n_sent, S, steps + 8, attention_D=D)
+    ctx.timer_start()
+    dec.encode(synth.zipf_ids(g, (S, n_sent), V), np.full(n_sent, S, np.int32))
+    enc_ms = ctx.timer_stop()
+    for _ in range(3):
+        dec.step()
+    _, ms = time_region(ctx, dec.step, steps, 0)
+    res = {"columns": beam * n_sent, "ms_per_decode_step": round(ms / steps, 4),
+           "hypotheses_per_s": round(beam * n_sent * steps / (ms * 1e-3), 1), "encode_ms": round(enc_ms, 3),
+           "attention_D": D}
+    dec.close()
+    return res
+
+
+def calibrate_copy(ctx, mbytes=64):
+    """A plain copy of known size (identity column gather: n*H*4 bytes read, n*H*4 bytes written) for scaling the
+    FETCH_SIZE / WRITE_SIZE counters."""
+    H = 1024
+    n = mbytes * 1024 * 1024 // (H * 4)
+    src, dst = ctx.zeros((H, n)), ctx.empty((H, n))
+    perm = ctx.array(np.arange(n, dtype=np.int32))
+    for _ in range(3):
+        ctx.gather_columns(src, H, perm, n, dst)
+    ctx.sync()
+    return {"kernel": "column_copy_kernel", "bytes_read": n * H * 4 + n * 4, "bytes_written": n * H * 4}
+
+
 def cpu_baseline(H=1000, mb=128, V=50000, L=4, t_sample=20):
     """The oracle (float accumulation, OpenMP) on a bounded sample of the headline workload: t_sample time steps
     of the 4-layer encoder with the same shapes; per-token cost does not depend on T."""
@@ -194,6 +230,8 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the config-3 and HBM-kernel measurements")
     ap.add_argument("--lstm-tn", type=int, default=0)
     ap.add_argument("--lstm-ks", type=int, default=0)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run a plain copy kernel of known size (for scaling HBM traffic counters) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (no cross-GPU path exists)" % args.gpus,
@@ -206,6 +244,11 @@ def main():
         ctx.set_option(capi.ZR_OPT_LSTM_TN, args.lstm_tn)
     if args.lstm_ks:
         ctx.set_option(capi.ZR_OPT_LSTM_KSPLIT, args.lstm_ks)
+
+    if args.calibrate_copy:
+        print(json.dumps(calibrate_copy(ctx)))
+        ctx.close()
+        return
 
     enc = bench_encoder(ctx, args.steps, args.warmup)
     enc.pop("_keep")
@@ -221,6 +264,8 @@ def main():
                                          for k, v in bench_decoder_step(ctx, args.steps, args.warmup).items()}
         log("config3:", extra["config3_decoder_step"])
         extra["hbm_kernels"] = bench_hbm_kernels(ctx, args.steps)
+        extra["config4_beam_decode"] = bench_beam_decode(ctx, args.steps)
+        log("config4:", extra["config4_beam_decode"])
         log("hbm kernels:", extra["hbm_kernels"])
     cpu = None
     if not args.no_cpu:

@@ -512,3 +512,21 @@ def test_stack_forward_with_split_kernel_forced(ctx):
     want_h, want_c = o.lstm_stack_forward(embed, layers, nn, m)
     assert_close(hs, want_h, what="stack h")
     assert_close(cs, want_c, what="stack c")
+
+
+@pytest.mark.parametrize("V,H,mb", [(4100, 100, 128), (5000, 72, 192), (4096, 36, 256), (6004, 1000, 100), (4360, 64, 300)])
+def test_softmax_large_vocab_lds_gemm_shapes(ctx, V, H, mb):
+    """Shapes that take the LDS-shared-weights GEMM (M >= 4096, N >= 96): row tails (V % 32 != 0), K tails
+    (H % 32 != 0, H % 8 != 0), 4-, 6- and 8-wave workgroups, more than one column tile."""
+    g = synth.rng(18, V + mb)
+    D, bd, h = U(g, (V, H), -0.5, 0.5), U(g, (V,), -1, 1), U(g, (H, mb), -1, 1)
+    d_lp, d_scr = ctx.empty((V, mb)), ctx.empty((V, mb))
+    ctx.softmax_forward(ctx.array(D), ctx.array(bd), V, H, ctx.array(h), mb, capi.ZR_SOFTMAX_LOGPROB, d_lp, d_scr)
+    ctx.sync()
+    logits = o.softmax_logits(D, bd, h)
+    assert_close(d_scr.get(), logits, floor=float(np.sqrt(H) * 0.3), what="logits")
+    assert_close(d_lp.get(), o.softmax_logprob_f64(logits), what="log-probs")
+    dC = ctx.empty((V, mb))
+    ctx.gemm(0, V, mb, H, ctx.array(D), V, ctx.array(h), H, dC, V)
+    ctx.sync()
+    assert_close(dC.get(), o.gemm_nn(D, h), floor=float(np.sqrt(H) * 0.3), what="plain gemm")

@@ -35,6 +35,8 @@ struct zr_beam {
   // per step scratch
   float* d_cand_p;          // [n_sent*beam][beam+1]
   int* d_cand_w;            // [n_sent*beam][beam+1]
+  float* d_part_p;          // [n_sent*beam][kChunks][beam+1] per-chunk candidates
+  int* d_part_w;
   void* d_block;            // the single allocation behind all of the above
 };
 
@@ -42,18 +44,30 @@ namespace {
 
 constexpr int KMAX = 32;  // beam + 1 <= KMAX
 
-// Per-column top-K: one workgroup per column.  Each thread keeps the K best of its strided share in
-// registers (sorted, descending; bubble insertion with static indexing), then K rounds of workgroup arg-max
-// over the thread heads produce the column's K best in descending order.
+// Per-column top-K in two stages.
+// Stage 1 (beam_topk_kernel): grid (kChunks, columns).  A workgroup scans its quarter of the column with 16-byte
+// loads; each thread keeps the K best of its share in registers (sorted, descending; bubble insertion with
+// static indexing, guarded by the thread's current K-th best so the common case is one compare), then K rounds
+// of workgroup arg-max over the thread heads emit the chunk's K best in descending order.
+// Stage 2 (beam_topk_merge_kernel): one wave per column merges the kChunks sorted lists.
+// Order everywhere: larger probability first, equal probabilities by lower word id.
+constexpr int kChunks = 4;
+
+__device__ __forceinline__ bool better(float pa, int wa, float pb, int wb) { return pa > pb || (pa == pb && wa < wb); }
+
 __global__ void __launch_bounds__(256)
-beam_topk_kernel(const float* __restrict__ prob, int V, int K, float* __restrict__ cand_p, int* __restrict__ cand_w) {
+beam_topk_kernel(const float* __restrict__ prob, int V, int K, float* __restrict__ part_p, int* __restrict__ part_w) {
   __shared__ float s_p[4];
   __shared__ int s_w[4];
-  __shared__ int s_owner[4];
-  const int col = blockIdx.x;
+  const int chunk = blockIdx.x;
+  const int col = blockIdx.y;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const float* p = prob + (size_t)col * V;
+  // chunk boundaries are multiples of 4 elements so that 16-byte loads stay aligned when V % 4 == 0
+  const int per = (((V + kChunks - 1) / kChunks) + 3) & ~3;
+  const int v_begin = chunk * per;
+  const int v_end = (v_begin + per < V) ? v_begin + per : V;
   float lp[KMAX];
   int lw[KMAX];
 #pragma unroll
@@ -61,19 +75,13 @@ beam_topk_kernel(const float* __restrict__ prob, int V, int K, float* __restrict
     lp[i] = -INFINITY;
     lw[i] = 0x7fffffff;
   }
-  for (int v = tid; v < V; v += 256) {
-    float x = p[v];
-    int xw = v;
-    // skip quickly when x does not beat this thread's K-th best (slot K-1; slots >= K stay -inf)
-    bool beats = false;
-#pragma unroll
-    for (int i = 0; i < KMAX; ++i)
-      if (i == K - 1) beats = x > lp[i];
-    if (!beats) continue;
+  float kth = -INFINITY;  // this thread's current K-th best
+  auto insert = [&](float x, int xw) {
+    // strict comparison: an equal, earlier (lower id) entry stays in front
 #pragma unroll
     for (int i = 0; i < KMAX; ++i) {
       if (i < K) {
-        const bool sw = x > lp[i];  // strict: an equal, earlier (lower id) entry stays in front
+        const bool sw = x > lp[i];
         const float tp = lp[i];
         const int tw = lw[i];
         lp[i] = sw ? x : tp;
@@ -81,6 +89,24 @@ beam_topk_kernel(const float* __restrict__ prob, int V, int K, float* __restrict
         x = sw ? tp : x;
         xw = sw ? tw : xw;
       }
+    }
+#pragma unroll
+    for (int i = 0; i < KMAX; ++i)
+      if (i == K - 1) kth = lp[i];
+  };
+  const bool vec = ((V & 3) == 0) && ((((uintptr_t)prob) & 15u) == 0);
+  if (vec) {
+    for (int v = v_begin + 4 * tid; v < v_end; v += 4 * 256) {
+      const zr_f32x4 q = *(const zr_f32x4*)(p + v);
+      if (q.x > kth) insert(q.x, v);
+      if (q.y > kth) insert(q.y, v + 1);
+      if (q.z > kth) insert(q.z, v + 2);
+      if (q.w > kth) insert(q.w, v + 3);
+    }
+  } else {
+    for (int v = v_begin + tid; v < v_end; v += 256) {
+      const float x = p[v];
+      if (x > kth) insert(x, v);
     }
   }
   int head = 0;  // index of this thread's best unconsumed entry
@@ -93,14 +119,13 @@ beam_topk_kernel(const float* __restrict__ prob, int V, int K, float* __restrict
         hp = lp[i];
         hw = lw[i];
       }
-    // arg-max over (p desc, word asc) across the wave, then across the 4 waves
     float bp = hp;
     int bw = hw;
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
       const float op = __shfl_xor(bp, off, 64);
       const int ow = __shfl_xor(bw, off, 64);
-      if (op > bp || (op == bp && ow < bw)) {
+      if (better(op, ow, bp, bw)) {
         bp = op;
         bw = ow;
       }
@@ -114,18 +139,68 @@ beam_topk_kernel(const float* __restrict__ prob, int V, int K, float* __restrict
     int gw = s_w[0];
 #pragma unroll
     for (int w = 1; w < 4; ++w)
-      if (s_p[w] > gp || (s_p[w] == gp && s_w[w] < gw)) {
+      if (better(s_p[w], s_w[w], gp, gw)) {
         gp = s_p[w];
         gw = s_w[w];
       }
-    if (hw == gw && hp == gp && gw != 0x7fffffff) head++;  // word ids are unique: exactly one owner
+    if (hw == gw && gw != 0x7fffffff) head++;  // word ids are unique: exactly one owner
     if (tid == 0) {
-      cand_p[(size_t)col * K + r] = gp;
-      cand_w[(size_t)col * K + r] = gw;
+      part_p[((size_t)col * kChunks + chunk) * K + r] = gp;
+      part_w[((size_t)col * kChunks + chunk) * K + r] = gw;
     }
     __syncthreads();
   }
-  (void)s_owner;
+}
+
+__global__ void __launch_bounds__(64)
+beam_topk_merge_kernel(const float* __restrict__ part_p, const int* __restrict__ part_w, int K,
+                       float* __restrict__ cand_p, int* __restrict__ cand_w) {
+  const int col = blockIdx.x;
+  const int lane = threadIdx.x;
+  const int n = kChunks * K;  // <= 128: two entries per lane
+  float p0 = -INFINITY, p1 = -INFINITY;
+  int w0 = 0x7fffffff, w1 = 0x7fffffff;
+  if (lane < n) {
+    p0 = part_p[(size_t)col * n + lane];
+    w0 = part_w[(size_t)col * n + lane];
+  }
+  if (lane + 64 < n) {
+    p1 = part_p[(size_t)col * n + lane + 64];
+    w1 = part_w[(size_t)col * n + lane + 64];
+  }
+  for (int r = 0; r < K; ++r) {
+    float bp = p0;
+    int bw = w0;
+    if (better(p1, w1, bp, bw)) {
+      bp = p1;
+      bw = w1;
+    }
+    const float mine_p = bp;
+    const int mine_w = bw;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float op = __shfl_xor(bp, off, 64);
+      const int ow = __shfl_xor(bw, off, 64);
+      if (better(op, ow, bp, bw)) {
+        bp = op;
+        bw = ow;
+      }
+    }
+    if (mine_w == bw && bw != 0x7fffffff) {  // the owner retires the winner
+      if (w0 == bw) {
+        p0 = -INFINITY;
+        w0 = 0x7fffffff;
+      } else {
+        p1 = -INFINITY;
+        w1 = 0x7fffffff;
+      }
+    }
+    (void)mine_p;
+    if (lane == 0) {
+      cand_p[(size_t)col * K + r] = bp;
+      cand_w[(size_t)col * K + r] = bw;
+    }
+  }
 }
 
 // Cross-column merge and bookkeeping for one sentence per workgroup (expand_hypothesis_without_fsa,
@@ -311,6 +386,7 @@ int zr_beam_create(zr_ctx* ctx, int beam, int vocab, int n_sent, int max_len, fl
   ZR_CHECK_ARG(out != nullptr, "zr_beam_create: out is null");
   *out = nullptr;
   ZR_CHECK_ARG(beam >= 1 && beam + 1 <= KMAX, "zr_beam_create: beam = %d not in [1, %d]", beam, KMAX - 1);
+  ZR_CHECK_ARG(n_sent * beam <= 65535, "zr_beam_create: more than 65535 columns");
   ZR_CHECK_ARG(vocab > beam + 1 && n_sent >= 1 && max_len >= 3, "zr_beam_create: vocab = %d, n_sent = %d, max_len = %d",
                vocab, n_sent, max_len);
   // the reference caps the beam at floor(sqrt(V)) (src/ensemble_factory.hpp:19-21)
@@ -335,6 +411,7 @@ int zr_beam_create(zr_ctx* ctx, int beam, int vocab, int n_sent, int max_len, fl
   const size_t o_hw = take((size_t)n_sent * b->hyp_cap * max_len * 4), o_hl = take((size_t)n_sent * b->hyp_cap * 4);
   const size_t o_hs = take((size_t)n_sent * b->hyp_cap * 4), o_hc = take((size_t)n_sent * 4);
   const size_t o_cp = take(nb * K * 4), o_cw = take(nb * K * 4);
+  const size_t o_pp = take(nb * 4 * K * 4), o_pw = take(nb * 4 * K * 4);  // kChunks = 4 lists per column
   char* base = nullptr;
   if (hipMalloc((void**)&base, off) != hipSuccess) {
     (void)hipGetLastError();
@@ -353,6 +430,8 @@ int zr_beam_create(zr_ctx* ctx, int beam, int vocab, int n_sent, int max_len, fl
   b->d_hyp_count = (int*)(base + o_hc);
   b->d_cand_p = (float*)(base + o_cp);
   b->d_cand_w = (int*)(base + o_cw);
+  b->d_part_p = (float*)(base + o_pp);
+  b->d_part_w = (int*)(base + o_pw);
   *out = b;
   return zr_beam_init(ctx, b);
 }
@@ -385,8 +464,12 @@ int zr_beam_expand(zr_ctx* ctx, zr_beam* b, const float* d_prob, int index, int*
   ZR_CHECK_ARG(index >= 0, "zr_beam_expand: index = %d", index);
   ZR_CHECK_ARG(b->current_index + 2 < b->max_len, "zr_beam_expand: hypotheses reached max_len = %d", b->max_len);
   const int K = b->beam + 1;
-  beam_topk_kernel<<<b->n_sent * b->beam, 256, 0, ctx->stream>>>(d_prob, b->vocab, K, b->d_cand_p, b->d_cand_w);
+  dim3 tgrid(kChunks, b->n_sent * b->beam);
+  beam_topk_kernel<<<tgrid, 256, 0, ctx->stream>>>(d_prob, b->vocab, K, b->d_part_p, b->d_part_w);
   ZR_LAUNCH_CHECK("beam_topk_kernel");
+  beam_topk_merge_kernel<<<b->n_sent * b->beam, 64, 0, ctx->stream>>>(b->d_part_p, b->d_part_w, K, b->d_cand_p,
+                                                                      b->d_cand_w);
+  ZR_LAUNCH_CHECK("beam_topk_merge_kernel");
   beam_merge_kernel<<<b->n_sent, 256, 0, ctx->stream>>>(b->beam, K, b->max_len, b->hyp_cap, b->penalty, index,
                                                         b->current_index, b->d_cand_p, b->d_cand_w, b->d_scores,
                                                         b->d_scores_tmp, b->d_words, b->d_sent, b->d_sent_tmp,

@@ -228,23 +228,16 @@ __global__ void __launch_bounds__(64 * NWV) lstm_lds_kernel(LstmLaunch2 P) {
   zr_f32x4 wreg[WLD];
   zr_f32x4 xf[2][4][TN];
 
-  // All loads are unconditional with clamped addresses; invalid weights are zeroed by a select.  (Loads under
-  // branches stop the compiler from counting loads in flight and force full waits.)
+  // All loads are unconditional with clamped addresses (loads under branches stop the compiler from counting
+  // loads in flight and force full waits).  gload only issues loads; out-of-range weights are zeroed by a
+  // multiplication in lds_store (weights are finite), so that nothing consumes a loaded value right after its load.
   auto gload = [&](int c, zr_f32x4 (&xdst)[4][TN]) {
-    const int cc = c < c_end ? c : c_end - 1;       // dummy chunk (odd chunk count): clamp, weights zeroed
-    const bool chunk_ok = c < c_end;
+    const int cc = c < c_end ? c : c_end - 1;  // dummy chunk (odd chunk count): clamped, zeroed at store time
 #pragma unroll
     for (int u = 0; u < WLD; ++u) {
       const int k = cc * KC + wkk[u];
       const int kc = k < H ? k : H - 1;
-      const zr_f32x4 v = *(const zr_f32x4*)(wsrc[u] + (long long)kc * H);
-      // zero by multiplication (weights are finite): a select would let the compiler skip the load under a
-      // branch, and loads under branches defeat its in-flight load counting
-      const float keep = (chunk_ok && wok_row[u] && (k < H)) ? 1.0f : 0.0f;
-      wreg[u].x = v.x * keep;
-      wreg[u].y = v.y * keep;
-      wreg[u].z = v.z * keep;
-      wreg[u].w = v.w * keep;
+      wreg[u] = *(const zr_f32x4*)(wsrc[u] + (long long)kc * H);
     }
 #pragma unroll
     for (int gq = 0; gq < 4; ++gq) {
@@ -256,11 +249,19 @@ __global__ void __launch_bounds__(64 * NWV) lstm_lds_kernel(LstmLaunch2 P) {
       for (int tn = 0; tn < TN; ++tn) xdst[gq][tn] = *(const zr_f32x4*)(xcol[tn] + kx);
     }
   };
-  auto lds_store = [&](int buf) {
+  auto lds_store = [&](int buf, int c) {
+    const bool chunk_ok = c < c_end;
+    const int cc = chunk_ok ? c : c_end - 1;
 #pragma unroll
     for (int u = 0; u < WLD; ++u) {
       const int f = tid + NTHR * u;
-      if (f < F4_PER_CHUNK) Ws4[buf][f] = wreg[u];
+      const float keep = (chunk_ok && wok_row[u] && (cc * KC + wkk[u]) < H) ? 1.0f : 0.0f;
+      zr_f32x4 v = wreg[u];
+      v.x *= keep;
+      v.y *= keep;
+      v.z *= keep;
+      v.w *= keep;
+      if (f < F4_PER_CHUNK) Ws4[buf][f] = v;
     }
   };
   auto compute = [&](int buf, const zr_f32x4 (&xs)[4][TN]) {
@@ -292,18 +293,18 @@ __global__ void __launch_bounds__(64 * NWV) lstm_lds_kernel(LstmLaunch2 P) {
 
   if (c_begin < c_end) {
     gload(c_begin, xf[0]);
-    lds_store(0);
+    lds_store(0, c_begin);
     __syncthreads();
     for (int c = c_begin; c < c_end; c += 2) {
       // even stage: chunk c from buffer 0, prefetch c+1 into buffer 1
       gload(c + 1, xf[1]);
       compute(0, xf[0]);
-      lds_store(1);
+      lds_store(1, c + 1);
       __syncthreads();
       // odd stage: chunk c+1 (all-zero weights if past the end) from buffer 1, prefetch c+2 into buffer 0
       gload(c + 2, xf[0]);
       compute(1, xf[1]);
-      lds_store(0);
+      lds_store(0, c + 2);
       __syncthreads();
     }
   }

@@ -134,7 +134,7 @@ int zr_ctx_set_option(zr_ctx* ctx, int option, int value) {
       ctx->lstm_kparts = value;
       return ZR_OK;
     case ZR_OPT_GEMM_CFG:
-      ZR_CHECK_ARG(value >= 0 && value <= 8, "ZR_OPT_GEMM_CFG out of range");
+      ZR_CHECK_ARG(value >= 0 && value <= 10, "ZR_OPT_GEMM_CFG out of range");
       ctx->gemm_cfg = value;
       return ZR_OK;
     default:
