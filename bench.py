@@ -190,16 +190,20 @@ def bench_beam_decode(ctx, steps, H=1000, L=4, beam=12, n_sent=16, S=50, V=50000
 
 
 def calibrate_copy(ctx, mbytes=64):
-    """A plain copy of known size (identity column gather: n*H*4 bytes read, n*H*4 bytes written) for scaling the
-    FETCH_SIZE / WRITE_SIZE counters."""
-    H = 1024
-    n = mbytes * 1024 * 1024 // (H * 4)
-    src, dst = ctx.zeros((H, n)), ctx.empty((H, n))
-    perm = ctx.array(np.arange(n, dtype=np.int32))
-    for _ in range(3):
-        ctx.gather_columns(src, H, perm, n, dst)
-    ctx.sync()
-    return {"kernel": "column_copy_kernel", "bytes_read": n * H * 4 + n * 4, "bytes_written": n * H * 4}
+    """Plain copies of known size (identity column gathers: n*H*4 bytes read, n*H*4 bytes written) for scaling the
+    FETCH_SIZE / WRITE_SIZE counters: one with 16-byte accesses (H = 1024, column_copy_kernel<true>) and one with
+    4-byte accesses (H = 1023, column_copy_kernel<false>), the access width of the MFMA kernels' weight loads."""
+    out = []
+    for H in (1024, 1023):
+        n = mbytes * 1024 * 1024 // (H * 4)
+        src, dst = ctx.zeros((H, n)), ctx.empty((H, n))
+        perm = ctx.array(np.arange(n, dtype=np.int32))
+        for _ in range(3):
+            ctx.gather_columns(src, H, perm, n, dst)
+        ctx.sync()
+        out.append({"kernel": "column_copy_kernel<%s>" % ("true" if H % 4 == 0 else "false"), "H": H, "columns": n,
+                    "KiB_read": (n * H * 4 + n * 4) / 1024.0, "KiB_written": n * H * 4 / 1024.0})
+    return out
 
 
 def cpu_baseline(H=1000, mb=128, V=50000, L=4, t_sample=20):

@@ -81,7 +81,7 @@ __global__ void __launch_bounds__(64 * KS * WPB) gemm_kernel(GemmArgs a) {
     }
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) xcol[tn] = a.B[s] + (long long)cols[tn] * a.ldb[s] + 4 * half;
-    zr_mma_segment<TM, TN, KS, zr_prefetch_depth(TM, TN), TRANS_A, VEC>(acc, wbase, woff, a.lda[s], xcol, a.K[s],
+    zr_mma_segment<TM, TN, KS, zr_prefetch_depth(TM, TN), TRANS_A ? ZR_A_TRANS : ZR_A_NN, VEC>(acc, wbase, woff, a.lda[s], xcol, a.K[s],
                                                                         kslice, half);
   }
 
@@ -89,7 +89,7 @@ __global__ void __launch_bounds__(64 * KS * WPB) gemm_kernel(GemmArgs a) {
   const float* bias = a.bias ? a.bias + (long long)z * a.strideBias : nullptr;
   float* redp = KS > 1 ? red + (size_t)sub * KS * TN * 16 * 64 : red;
 
-  zr_reduce_visit<TM, TN, KS>(acc, redp, kslice, lane, [&](const float(&vals)[TM], int tn, int r) {
+  zr_reduce_visit<TM, TN, KS>(acc, redp, kslice, lane, [&](const float(&vals)[TM], int tn, int r, int) {
     const int n = n0 + tn * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
     const bool n_ok = active && n < a.N;
 #pragma unroll

@@ -96,7 +96,11 @@ static inline int zr_softmax_partial_blocks(int M) { return (M + 31) / 32; }
 struct zr_lstm_weights {
   int H;
   int nseg;        // 2 (M, Wh) or 3 (+Q)
-  float* d_W;      // [nseg][4][H*H] column-major blocks
+  int ldw;         // H rounded up to 32: rows per packed k-block (rows >= H hold zeros)
+  int kp;          // H rounded up to 8: packed K extent (k >= H hold zeros)
+  // [nseg][4] matrices, each packed as [kp/4][ldw][4]: element (row, k) at ((k/4)*ldw + row)*4 + k%4.  A 32-row
+  // tile of four consecutive k is 512 contiguous, 128-byte aligned bytes, read with one 16-byte load per lane.
+  float* d_W;
   float* d_bias;   // [4][H]
 };
 

@@ -19,9 +19,11 @@ namespace {
 constexpr int kMaxUnits = 8;
 
 struct LstmUnit {
-  const float* W;           // [nseg][4][H*H]
+  const float* W;           // [nseg][4] packed matrices, [kp/4][ldw][4] each
   const float* bias;        // [4][H]
   const float* in[3];       // segment inputs, H x mb (ld = H)
+  const float* inp[3];      // optional copies of the same inputs packed as [H/4][mb][4] (null: use in[])
+  float* hp;                // optional: h is also written packed as [H/4][mb][4] for the units that consume it
   const int* gather_ids;    // non-null: column n of segment 0 is in[0] + ids[n]*H (embedding gather)
   const float* cprev;
   const int* mask01;
@@ -37,21 +39,37 @@ struct LstmLaunch {
   int n_units;
   int nseg_max;             // largest nseg among the units
   int H, mb;
+  int ldw, kp;              // packed weight extents: rows per k-block (H up to 32), K (H up to 8), zero filled
+  float* preact;            // non-null: store the four pre-activation sums ([4][H*mb], no bias) instead of the cell
   float clip;
   int j_tiles, n_tiles;
 };
 
+// Prefetch distance (k-groups) of the register-streaming kernel: a fragment is 4*(4+TN) registers and 4+TN
+// 16-byte loads; the accumulators take 64*TN registers of the 512 a wave may use at one wave per SIMD (KS = 4)
+// or of the 256 at two (KS = 8).
+constexpr int lstm_prefetch_depth(int tn, int ks) {
+#ifdef ZR_LSTM_PF
+  return ZR_LSTM_PF;
+#else
+  return ks > 4 ? (tn == 1 ? 5 : 2) : (tn == 1 ? 8 : (tn == 2 ? 6 : 1));
+#endif
+}
+
 template <int TN, int KS, bool VEC>
 __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
   __shared__ float red[KS * TN * 16 * 64];
-  // Workgroups that share a weight tile (same unit and row tile, different column tile) get ids that are
-  // congruent modulo 8, so the round-robin workgroup->XCD dispatch puts them on the same XCD and its L2.
+  // Workgroup ids congruent modulo 8 run on the same XCD (round-robin dispatch) and share its L2.  Each XCD gets
+  // a contiguous range of (unit, row tile) groups and every column tile of those groups: a weight tile is
+  // fetched from memory once however many column tiles read it, and an XCD touches the activations of one or
+  // two units only instead of all of them.
   const int id = blockIdx.x;
   const int r8 = id & 7;
   const int q = id >> 3;
   const int nt = q % L.n_tiles;
-  const int group = (q / L.n_tiles) * 8 + r8;
-  if (group >= L.n_units * L.j_tiles) return;
+  const int groups = L.n_units * L.j_tiles;
+  const int group = r8 * ((groups + 7) >> 3) + q / L.n_tiles;
+  if (q / L.n_tiles >= ((groups + 7) >> 3) || group >= groups) return;
   const int unit = group / L.j_tiles;
   const int jt = group % L.j_tiles;
   const LstmUnit& U = L.u[unit];
@@ -82,7 +100,21 @@ __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[g][tn][r] = 0.0f;
 
-  const long long HH = (long long)H * H;
+  // Epilogue operands are fetched now, ahead of the K loop, so that their memory latency is not paid after it.
+  constexpr int NV = zr_visit_count<TN, KS>();
+  const float bi = U.bias[jc], bf = U.bias[H + jc], bc = U.bias[2 * H + jc], bo = U.bias[3 * H + jc];
+  float cprev_v[NV], mask_v[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int slot = zr_visit_slot<KS>(kslice, i);
+    const int tn = slot >> 4, r = slot & 15;
+    int n = n0 + tn * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+    n = n < L.mb ? n : L.mb - 1;
+    cprev_v[i] = L.preact ? 0.0f : U.cprev[(long long)n * H + jc];
+    mask_v[i] = (float)U.mask01[n];
+  }
+
+  const long long HH = (long long)L.kp * L.ldw;
   for (int s = 0; s < U.nseg; ++s) {
     const float* wbase[4];
     unsigned woff[4];
@@ -90,7 +122,7 @@ __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       wbase[g] = U.W + ((long long)s * 4 + g) * HH;
-      woff[g] = (unsigned)(jc + 4 * half * H);
+      woff[g] = (unsigned)(4 * j + 4 * half * L.ldw);  // j < ldw: padded rows are zeros
     }
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) {
@@ -100,23 +132,30 @@ __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
         idv = idv < 0 ? 0 : (idv >= U.V ? U.V - 1 : idv);
         c = idv;
       }
-      xcol[tn] = U.in[s] + c * H + 4 * half;
+      xcol[tn] = (VEC && U.inp[s]) ? U.inp[s] + 4LL * cols[tn] + 4LL * half * L.mb : U.in[s] + c * H + 4 * half;
     }
-    zr_mma_segment<4, TN, KS, zr_prefetch_depth(4, TN), false, VEC>(acc, wbase, woff, (long long)H, xcol, H, kslice,
-                                                                    half);
+    zr_mma_segment<4, TN, KS, lstm_prefetch_depth(TN, KS), ZR_A_PACK4, VEC>(
+        acc, wbase, woff, (long long)L.ldw, xcol, H, kslice, half, (VEC && U.inp[s]) ? L.mb : 1);
   }
 
-  const float bi = U.bias[jc], bf = U.bias[H + jc], bc = U.bias[2 * H + jc], bo = U.bias[3 * H + jc];
   const bool j_ok = j < H;
-  zr_reduce_visit<4, TN, KS>(acc, red, kslice, lane, [&](const float(&z)[4], int tn, int r) {
+  zr_reduce_visit<4, TN, KS>(acc, red, kslice, lane, [&](const float(&z)[4], int tn, int r, int vi) {
     const int n = n0 + tn * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
     if (j_ok && n < L.mb) {
       const long long ix = (long long)n * H + j;
+      if (L.preact) {
+        const long long gs = (long long)H * L.mb;
+        L.preact[ix] = z[0];
+        L.preact[gs + ix] = z[1];
+        L.preact[2 * gs + ix] = z[2];
+        L.preact[3 * gs + ix] = z[3];
+        return;
+      }
       float gi, gf, gc, go, c, h;
-      zr_lstm_cell(z[0] + bi, z[1] + bf, z[2] + bc, z[3] + bo, U.cprev[ix], (float)U.mask01[n], L.clip, gi, gf, gc,
-                   go, c, h);
+      zr_lstm_cell(z[0] + bi, z[1] + bf, z[2] + bc, z[3] + bo, cprev_v[vi], mask_v[vi], L.clip, gi, gf, gc, go, c, h);
       U.c[ix] = c;
       U.h[ix] = h;
+      if (U.hp) U.hp[((long long)(j >> 2) * L.mb + n) * 4 + (j & 3)] = h;
       if (U.gates[0]) {
         U.gates[0][ix] = gi;
         U.gates[1][ix] = gf;
@@ -152,7 +191,7 @@ template <int TN, int NWV>
 __global__ void __launch_bounds__(64 * NWV) lstm_lds_kernel(LstmLaunch2 P) {
   constexpr int KC = 32;                       // k per chunk
   constexpr int NTHR = 64 * NWV;
-  constexpr int F4_PER_CHUNK = KC * 4 * 8;     // float4 per weight chunk: 32 k x 4 gates x 8 (32 rows / 4)
+  constexpr int F4_PER_CHUNK = (KC / 4) * 4 * 32;  // float4 per weight chunk: 8 k-blocks x 4 gates x 32 rows
   constexpr int WLD = (F4_PER_CHUNK + NTHR - 1) / NTHR;  // float4 loads per thread per chunk
   __shared__ zr_f32x4 Ws4[2][F4_PER_CHUNK];
   __shared__ int s_last;
@@ -162,9 +201,10 @@ __global__ void __launch_bounds__(64 * NWV) lstm_lds_kernel(LstmLaunch2 P) {
   const int q = id >> 3;
   const int splits = L.nseg_max * P.kparts;
   const int sp = q % splits;
-  const int tile = (q / splits) * 8 + r8;
   const int n_tiles_total = L.n_units * L.j_tiles * L.n_tiles;
-  if (tile >= n_tiles_total) return;
+  const int tiles_per_xcd = (n_tiles_total + 7) >> 3;  // contiguous tiles per XCD (ids congruent mod 8 share one)
+  const int tile = r8 * tiles_per_xcd + q / splits;
+  if (q / splits >= tiles_per_xcd || tile >= n_tiles_total) return;
   const int nt = tile % L.n_tiles;
   const int jt = (tile / L.n_tiles) % L.j_tiles;
   const int unit = tile / (L.n_tiles * L.j_tiles);
@@ -201,20 +241,20 @@ __global__ void __launch_bounds__(64 * NWV) lstm_lds_kernel(LstmLaunch2 P) {
     }
     xcol[tn] = U.in[s_eff] + col * H;
   }
-  // this thread's share of a weight chunk: float4 index f -> (kk, gate, j4)
+  // this thread's share of a weight chunk: float4 index f -> (k-block, gate, row); a float4 of the packed
+  // weights is four consecutive k of one row
   const float* wsrc[WLD];
   bool wok_row[WLD];
-  int wkk[WLD];
-  const long long HH = (long long)H * H;
+  int wkb[WLD];
+  const long long HH = (long long)L.kp * L.ldw;
+  const int kblocks = L.kp >> 2;
 #pragma unroll
   for (int u = 0; u < WLD; ++u) {
     const int f = tid + NTHR * u;
-    const int j4 = f & 7, g = (f >> 3) & 3, kk = f >> 5;
-    const int row = j0 + 4 * j4;
-    wok_row[u] = seg_live && (row < H) && (f < F4_PER_CHUNK);
-    wkk[u] = kk;
-    const int rowc = row < H ? row : H - 4;
-    wsrc[u] = U.W + ((long long)(seg_live ? seg : 0) * 4 + g) * HH + rowc;
+    const int row = f & 31, g = (f >> 5) & 3, kb = f >> 7;
+    wok_row[u] = seg_live && (f < F4_PER_CHUNK);  // rows >= H and k >= H of the packed weights are zeros
+    wkb[u] = kb;
+    wsrc[u] = U.W + ((long long)(seg_live ? seg : 0) * 4 + g) * HH + 4 * (j0 + row);
   }
 
   zr_f32x16 acc[4][TN];
@@ -235,9 +275,9 @@ __global__ void __launch_bounds__(64 * NWV) lstm_lds_kernel(LstmLaunch2 P) {
     const int cc = c < c_end ? c : c_end - 1;  // dummy chunk (odd chunk count): clamped, zeroed at store time
 #pragma unroll
     for (int u = 0; u < WLD; ++u) {
-      const int k = cc * KC + wkk[u];
-      const int kc = k < H ? k : H - 1;
-      wreg[u] = *(const zr_f32x4*)(wsrc[u] + (long long)kc * H);
+      const int kb = cc * (KC / 4) + wkb[u];
+      const int kbc = kb < kblocks ? kb : kblocks - 1;
+      wreg[u] = *(const zr_f32x4*)(wsrc[u] + (long long)kbc * (4 * L.ldw));
     }
 #pragma unroll
     for (int gq = 0; gq < 4; ++gq) {
@@ -255,7 +295,7 @@ __global__ void __launch_bounds__(64 * NWV) lstm_lds_kernel(LstmLaunch2 P) {
 #pragma unroll
     for (int u = 0; u < WLD; ++u) {
       const int f = tid + NTHR * u;
-      const float keep = (chunk_ok && wok_row[u] && (cc * KC + wkk[u]) < H) ? 1.0f : 0.0f;
+      const float keep = (chunk_ok && wok_row[u] && (cc * (KC / 4) + wkb[u]) < kblocks) ? 1.0f : 0.0f;
       zr_f32x4 v = wreg[u];
       v.x *= keep;
       v.y *= keep;
@@ -265,14 +305,19 @@ __global__ void __launch_bounds__(64 * NWV) lstm_lds_kernel(LstmLaunch2 P) {
     }
   };
   auto compute = [&](int buf, const zr_f32x4 (&xs)[4][TN]) {
-    // LDS -> register fragments one k-group ahead of the MFMAs that use them (16 weights per group per lane)
-    const float* Ws = (const float*)&Ws4[buf][0] + (4 * half * 4) * 32 + jl;
+    // LDS -> register fragments one k-group ahead of the MFMAs that use them: k-group gq is k-blocks 2*gq and
+    // 2*gq + 1, one per half-wave; a lane reads its row's four k of each gate with one 16-byte read
+    const zr_f32x4* Ws = &Ws4[buf][0] + half * 4 * 32 + jl;
     float wf[2][4][4];
     auto lds_frag = [&](float (&dst)[4][4], int gq) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) dst[i][g] = Ws[((8 * gq + i) * 4 + g) * 32];
+      for (int g = 0; g < 4; ++g) {
+        const zr_f32x4 v = Ws[(2 * gq * 4 + g) * 32];
+        dst[0][g] = v.x;
+        dst[1][g] = v.y;
+        dst[2][g] = v.z;
+        dst[3][g] = v.w;
+      }
     };
     lds_frag(wf[0], 0);
 #pragma unroll
@@ -367,6 +412,7 @@ __global__ void __launch_bounds__(64 * NWV) lstm_lds_kernel(LstmLaunch2 P) {
                        (float)U.mask01[n], L.clip, gi, gf, gc, go, c, h);
           U.c[ix] = c;
           U.h[ix] = h;
+          if (U.hp) U.hp[((long long)(j >> 2) * L.mb + n) * 4 + (j & 3)] = h;
           if (U.gates[0]) {
             U.gates[0][ix] = gi;
             U.gates[1][ix] = gf;
@@ -376,6 +422,19 @@ __global__ void __launch_bounds__(64 * NWV) lstm_lds_kernel(LstmLaunch2 P) {
         }
       }
   }
+}
+
+// One H x H column-major matrix (element (row, k) at src[row + k*H]) into the packed [kp/4][ldw][4] layout,
+// padding with zeros.  One thread per destination element.
+__global__ void __launch_bounds__(256) lstm_pack_kernel(const float* __restrict__ src, int H, int ldw, int kp,
+                                                        float* __restrict__ dst) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (long long)kp * ldw) return;
+  const int k4 = (int)(i & 3);
+  const long long t = i >> 2;
+  const int row = (int)(t % ldw);
+  const int k = (int)(t / ldw) * 4 + k4;
+  dst[i] = (row < H && k < H) ? src[row + (long long)k * H] : 0.0f;
 }
 
 template <int TN, int KS>
@@ -430,6 +489,7 @@ int launch_fused(zr_ctx* ctx, LstmLaunch& L, bool vec) {
   // it only ceil(H/32) * ceil(mb/64) workgroups; there the LDS / split-K kernel spreads the same node over ~256
   // workgroups.  It needs 16-byte aligned operands and a batch wide enough for its 128-column tile.
   int kernel = ctx->lstm_kernel;
+  if (L.preact) kernel = 1;  // only the register-streaming kernel stores raw pre-activations
   if (kernel == 0) {
     const long long wgs1 = (long long)L.n_units * L.j_tiles * ((n32 + 1) / 2);
     kernel = (vec && n32 >= 3 && wgs1 < 200) ? 2 : 1;
@@ -477,9 +537,13 @@ int zr_lstm_pack_weights(zr_ctx* ctx, const float* const d_M[4], const float* co
     ZR_CHECK_ARG(!d_Q || d_Q[g], "zr_lstm_pack_weights: null Q for gate %d", g);
   }
   const int nseg = d_Q ? 3 : 2;
-  const size_t HH = (size_t)H * H;
+  const int ldw = (H + 31) / 32 * 32;
+  const int kp = (H + 7) / 8 * 8;
+  const size_t HH = (size_t)kp * ldw;
   zr_lstm_weights* w = new zr_lstm_weights();
   w->H = H;
+  w->ldw = ldw;
+  w->kp = kp;
   w->nseg = nseg;
   w->d_W = nullptr;
   w->d_bias = nullptr;
@@ -493,13 +557,15 @@ int zr_lstm_pack_weights(zr_ctx* ctx, const float* const d_M[4], const float* co
   for (int g = 0; g < 4; ++g) {
     const float* segs[3] = {d_M[g], d_Wh[g], d_Q ? d_Q[g] : nullptr};
     for (int s = 0; s < nseg; ++s) {
-      hipError_t e = hipMemcpyAsync(w->d_W + ((size_t)s * 4 + g) * HH, segs[s], sizeof(float) * HH,
-                                    hipMemcpyDeviceToDevice, ctx->stream);
+      const long long total = (long long)HH;
+      lstm_pack_kernel<<<(unsigned)((total + 255) / 256), 256, 0, ctx->stream>>>(segs[s], H, ldw, kp,
+                                                                                 w->d_W + ((size_t)s * 4 + g) * HH);
+      hipError_t e = hipGetLastError();
       if (e != hipSuccess) {
         (void)hipFree(w->d_W);
         (void)hipFree(w->d_bias);
         delete w;
-        return zr_set_error(ZR_EHIP, "zr_lstm_pack_weights: copy failed: %s", hipGetErrorString(e));
+        return zr_set_error(ZR_EHIP, "zr_lstm_pack_weights: pack kernel failed: %s", hipGetErrorString(e));
       }
     }
     hipError_t e = hipMemcpyAsync(w->d_bias + (size_t)g * H, d_b[g], sizeof(float) * H, hipMemcpyDeviceToDevice,
@@ -541,40 +607,12 @@ int zr_lstm_step(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_in, const
   const int H = w->H;
   const int nseg = d_htild ? 3 : 2;
 
-  if (!ctx->lstm_fused) {
-    // reference-shaped two-phase path: pre-activations to memory (batched over the 4 gates), then the
-    // stand-alone fused gate kernel
-    void* pre = nullptr;
-    rc = zr_ctx_scratch(ctx, 0, sizeof(float) * 4 * (size_t)H * mb, &pre);
-    if (rc) return rc;
-    ZrGemmDesc d = {};
-    d.M = H;
-    d.N = mb;
-    d.nseg = nseg;
-    const float* ins[3] = {d_in, d_hprev, d_htild};
-    for (int s = 0; s < nseg; ++s) {
-      d.K[s] = H;
-      d.A[s] = w->d_W + (size_t)s * 4 * H * H;
-      d.lda[s] = H;
-      d.B[s] = ins[s];
-      d.ldb[s] = H;
-    }
-    d.C = (float*)pre;
-    d.ldc = H;
-    d.batch = 4;
-    d.strideA = (long long)H * H;
-    d.strideC = (long long)H * mb;
-    d.epilogue = ZR_EPI_STORE;
-    rc = zr_gemm_launch(ctx, d);
-    if (rc) return rc;
-    const float* b[4] = {w->d_bias, w->d_bias + H, w->d_bias + 2 * (size_t)H, w->d_bias + 3 * (size_t)H};
-    return zr_lstm_gates(ctx, (const float*)pre, b, d_cprev, d_mask01, clip_threshold, H, mb, d_h, d_c, d_gates);
-  }
-
   LstmLaunch L = {};
   L.n_units = 1;
   L.H = H;
   L.mb = mb;
+  L.ldw = w->ldw;
+  L.kp = w->kp;
   L.clip = clip_threshold;
   LstmUnit& U = L.u[0];
   U.W = w->d_W;
@@ -591,6 +629,18 @@ int zr_lstm_step(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_in, const
   U.nseg = nseg;
   U.V = 0;
   const bool vec = (H % 4 == 0) && aligned16(d_in) && aligned16(d_hprev) && (!d_htild || aligned16(d_htild));
+  if (!ctx->lstm_fused) {
+    // reference-shaped two-phase path: the four pre-activation sums go to memory, then the stand-alone fused gate
+    // kernel (the reference's element-wise kernels in one pass) adds the biases and runs the cell
+    void* pre = nullptr;
+    rc = zr_ctx_scratch(ctx, 1, sizeof(float) * 4 * (size_t)H * mb, &pre);
+    if (rc) return rc;
+    L.preact = (float*)pre;
+    rc = launch_fused(ctx, L, vec);
+    if (rc) return rc;
+    const float* b[4] = {w->d_bias, w->d_bias + H, w->d_bias + 2 * (size_t)H, w->d_bias + 3 * (size_t)H};
+    return zr_lstm_gates(ctx, (const float*)pre, b, d_cprev, d_mask01, clip_threshold, H, mb, d_h, d_c, d_gates);
+  }
   return launch_fused(ctx, L, vec);
 }
 
@@ -612,11 +662,24 @@ int zr_lstm_stack_forward(zr_ctx* ctx, int nl, const zr_lstm_weights* const laye
     vec = vec && aligned16(d_h0[l]) && aligned16(d_h_all[l]);
   }
   const size_t n = (size_t)H * mb;
+  // Every h is also written in a k-interleaved layout ([H/4][mb][4]) into a small ping-pong buffer per layer: its
+  // two consumers on the next diagonal, (l+1, t) and (l, t+1), then fetch activations with contiguous 16-byte
+  // loads.  The buffer written on diagonal d is read on d+1 only and overwritten on d+2.
+  float* hp_buf = nullptr;
+  if (vec && H % 8 == 0) {
+    void* p = nullptr;
+    rc = zr_ctx_scratch(ctx, 1, sizeof(float) * 2 * (size_t)nl * n, &p);
+    if (rc) return rc;
+    hp_buf = (float*)p;
+  }
+  auto hp_of = [&](int l, int d) { return hp_buf + ((size_t)(d & 1) * nl + l) * n; };
   // Diagonal wavefront: units (l, t) with l + t = d only depend on diagonal d-1.
   for (int d = 0; d < T + nl - 1; ++d) {
     LstmLaunch L = {};
     L.H = H;
     L.mb = mb;
+    L.ldw = layers[0]->ldw;
+    L.kp = layers[0]->kp;
     L.clip = clip_threshold;
     int nu = 0;
     for (int l = 0; l < nl; ++l) {
@@ -636,6 +699,10 @@ int zr_lstm_stack_forward(zr_ctx* ctx, int nl, const zr_lstm_weights* const laye
       }
       U.in[1] = (t == 0) ? d_h0[l] : d_h_all[l] + (size_t)(t - 1) * n;
       U.in[2] = nullptr;
+      U.inp[0] = (hp_buf && l > 0) ? hp_of(l - 1, d - 1) : nullptr;
+      U.inp[1] = (hp_buf && t > 0) ? hp_of(l, d - 1) : nullptr;
+      U.inp[2] = nullptr;
+      U.hp = hp_buf ? hp_of(l, d) : nullptr;
       U.cprev = (t == 0) ? d_c0[l] : d_c_all[l] + (size_t)(t - 1) * n;
       U.mask01 = d_mask01 + (size_t)t * mb;
       U.h = d_h_all[l] + (size_t)t * n;

@@ -38,6 +38,15 @@ constexpr int zr_prefetch_depth(int tm, int tn) {
 #endif
 }
 
+// How the weight operand is laid out in memory (element (row, k) of sub-tile tm):
+//   ZR_A_NN     column-major:  wbase[row + k*lda]                 one 4-byte load per k
+//   ZR_A_TRANS  row-major:     wbase[k + row*lda]                 one 16-byte load per 4 k (VEC)
+//   ZR_A_PACK4  k-interleaved: wbase[((k/4)*lda + row)*4 + k%4]   one 16-byte load per 4 k, and the 32 lanes of a
+//               half-wave read 512 contiguous bytes; K is padded to a multiple of 8 with zeros.  A wave can keep at
+//               most 63 vector-memory instructions in flight, so 16-byte loads let it keep four times the bytes of
+//               ZR_A_NN on the wire -- what hiding memory latency with one wave per SIMD needs.
+enum { ZR_A_NN = 0, ZR_A_TRANS = 1, ZR_A_PACK4 = 2 };
+
 template <int TM, int TN>
 struct ZrFrag {
   float x[TN][4];  // activations: x[tn][i] = X[k_i][n(tn, lane%32)]
@@ -47,15 +56,21 @@ struct ZrFrag {
 // One K segment.
 //   wbase[tm]: wave-uniform pointer to the weight matrix of sub-tile tm
 //   woff[tm]:  this lane's fixed element offset into it:
-//                NN:      row + 4*half*lda      (element (row, k) at wbase[row + k*lda])
-//                TRANS_A: row*lda + 4*half      (element (row, k) at wbase[k + row*lda])
+//                ZR_A_NN:     row + 4*half*lda
+//                ZR_A_TRANS:  row*lda + 4*half
+//                ZR_A_PACK4:  row*4 + 4*half*lda
 //   xcol[tn]:  this lane's activation column, already advanced by 4*half
+//   xstride:   element step of xcol per k: 1 for a plain column (X[k][n] at column base + k); mb for activations
+//              packed like ZR_A_PACK4 ([k/4][n][4], element step per k-block of 4 is 4*mb, so per k it is mb):
+//              then the 32 lanes of a half-wave read 512 contiguous bytes instead of 16 bytes from each of 32
+//              lines.  Packed activations require VEC and K % 8 == 0.
 // Rows / columns are pre-clamped by the caller so that out-of-range lanes read valid memory.
 // kslice must be wave-uniform.
-template <int TM, int TN, int KS, int PF, bool TRANS_A, bool VEC>
+template <int TM, int TN, int KS, int PF, int AMODE, bool VEC>
 __device__ __forceinline__ void zr_mma_segment(zr_f32x16 (&acc)[TM][TN], const float* const (&wbase)[TM],
                                                const unsigned (&woff)[TM], long long lda,
-                                               const float* const (&xcol)[TN], int K, int kslice, int half) {
+                                               const float* const (&xcol)[TN], int K, int kslice, int half,
+                                               int xstride = 1) {
   const int nfull = K >> 3;
   constexpr int NS = PF + 1;
 
@@ -64,7 +79,7 @@ __device__ __forceinline__ void zr_mma_segment(zr_f32x16 (&acc)[TM][TN], const f
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) {
       if (VEC) {
-        const zr_f32x4 v = *(const zr_f32x4*)(xcol[tn] + kg);
+        const zr_f32x4 v = *(const zr_f32x4*)(xcol[tn] + (long long)kg * xstride);
         f.x[tn][0] = v.x;
         f.x[tn][1] = v.y;
         f.x[tn][2] = v.z;
@@ -76,7 +91,14 @@ __device__ __forceinline__ void zr_mma_segment(zr_f32x16 (&acc)[TM][TN], const f
     }
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) {
-      if (TRANS_A) {
+      if (AMODE == ZR_A_PACK4) {
+        const float* p = wbase[tm] + (long long)kg * lda;  // uniform
+        const zr_f32x4 v = *(const zr_f32x4*)(p + woff[tm]);
+        f.w[tm][0] = v.x;
+        f.w[tm][1] = v.y;
+        f.w[tm][2] = v.z;
+        f.w[tm][3] = v.w;
+      } else if (AMODE == ZR_A_TRANS) {
         const float* p = wbase[tm] + kg;  // uniform
         if (VEC) {
           const zr_f32x4 v = *(const zr_f32x4*)(p + woff[tm]);
@@ -152,7 +174,10 @@ __device__ __forceinline__ void zr_mma_segment(zr_f32x16 (&acc)[TM][TN], const f
       }
 #pragma unroll
       for (int tm = 0; tm < TM; ++tm) {
-        const float v = TRANS_A ? wbase[tm][(long long)woff[tm] + rel] : wbase[tm][(long long)woff[tm] + (long long)rel * lda];
+        // ZR_A_PACK4: the padded tail block exists in memory, this lane's four values sit side by side
+        const float v = AMODE == ZR_A_PACK4   ? wbase[tm][(long long)kg * lda + woff[tm] + i]
+                        : AMODE == ZR_A_TRANS ? wbase[tm][(long long)woff[tm] + rel]
+                                              : wbase[tm][(long long)woff[tm] + (long long)rel * lda];
         t.w[tm][i] = ok ? v : 0.0f;
       }
     }
@@ -160,8 +185,16 @@ __device__ __forceinline__ void zr_mma_segment(zr_f32x16 (&acc)[TM][TN], const f
   }
 }
 
-// Sums the KS partial tiles of a workgroup and calls f(vals[TM], tn, r) once per (tn, r, lane) owned by the
-// calling thread, where vals[tm] is the finished accumulator register r of sub-tile (tm, tn) for this lane.
+// Number of visits zr_reduce_visit makes per thread, and the accumulator slot (tn*16 + r) of visit i: callers use
+// them to fetch epilogue operands (previous cell state, biases) before the K loop instead of after it.
+template <int TN, int KS>
+constexpr int zr_visit_count() { return KS == 1 ? TN * 16 : TN * 16 / KS; }
+template <int KS>
+__device__ __forceinline__ int zr_visit_slot(int kslice, int i) { return KS == 1 ? i : kslice + KS * i; }
+
+// Sums the KS partial tiles of a workgroup and calls f(vals[TM], tn, r, i) once per (tn, r, lane) owned by the
+// calling thread, where vals[tm] is the finished accumulator register r of sub-tile (tm, tn) for this lane and i
+// is the visit index (slot tn*16 + r == zr_visit_slot<KS>(kslice, i)).
 // Every lane of a wave calls f with the same (tn, r) at the same time (wave-uniform control flow), and a
 // thread keeps its lane index, so the caller's mapping  m <- lane%32,  n <- 8*(r/4) + 4*(lane/32) + r%4  holds.
 // `red` is LDS of KS * TN*16 * 64 floats (unused when KS == 1).  All threads of the workgroup must call this.
@@ -175,7 +208,7 @@ __device__ __forceinline__ void zr_reduce_visit(zr_f32x16 (&acc)[TM][TN], float*
         float vals[TM];
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) vals[tm] = acc[tm][tn][r];
-        f(vals, tn, r);
+        f(vals, tn, r, tn * 16 + r);
       }
   } else {
     constexpr int SLOTS = TN * 16;           // accumulator registers per sub-tile row of the tile
@@ -205,7 +238,7 @@ __device__ __forceinline__ void zr_reduce_visit(zr_f32x16 (&acc)[TM][TN], float*
       float vals[TM];
 #pragma unroll
       for (int tm = 0; tm < TM; ++tm) vals[tm] = pre[tm][i];
-      f(vals, slot / 16, slot % 16);
+      f(vals, slot / 16, slot % 16, i);
     }
   }
 }
