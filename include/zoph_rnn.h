@@ -146,6 +146,15 @@ int zr_gemm(zr_ctx* ctx, int trans_a, int M, int N, int K, const float* d_A, int
 
 /* ---- A8/A9: output softmax ------------------------------------------------------------------------------ */
 
+/* Optional preparation of an output layer for repeated use (no counterpart in the reference, which hands the raw
+ * V x H matrix d_D of softmax_layer, src/softmax.h:60, to cublasSgemm on every call): copies D into the layout the
+ * matrix cores read fastest (four consecutive k per row side by side, 32-row tiles 128-byte aligned; V*H*4 more
+ * bytes of device memory).  Afterwards every softmax entry point below that is given the same d_D, V and H uses the
+ * copy.  The copy is a snapshot: call again after changing D (it re-packs in place), and call zr_softmax_release
+ * before freeing d_D.  At most 8 matrices per context.  Results are the same with or without it. */
+int zr_softmax_prepare(zr_ctx* ctx, const float* d_D, int V, int H);
+int zr_softmax_release(zr_ctx* ctx, const float* d_D);
+
 #define ZR_SOFTMAX_PROB 0    /* probabilities: softmax_layer::get_distribution_GPU (src/softmax.hpp:514-632) */
 #define ZR_SOFTMAX_LOGPROB 1 /* natural-log probabilities, fp32 */
 

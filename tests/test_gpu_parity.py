@@ -277,11 +277,15 @@ def test_config1_lm_forward_logprobs_and_loss(ctx):
 
 
 # ------------------------------------------------------------------------------------------------ A8/A9 softmax
-@pytest.mark.parametrize("V,H,mb", [(211, 16, 6), (10000, 100, 8), (4099, 64, 33)])
-def test_softmax_prob_and_logprob(ctx, V, H, mb):
+@pytest.mark.parametrize("prepared", [False, True])
+@pytest.mark.parametrize("V,H,mb", [(211, 16, 6), (10000, 100, 8), (4099, 64, 33), (1003, 27, 70)])
+def test_softmax_prob_and_logprob(ctx, V, H, mb, prepared):
+    """prepared: the output matrix registered with zr_softmax_prepare (k-interleaved copy); same results."""
     g = synth.rng(11, V)
     D, bd, h = U(g, (V, H), -1, 1), U(g, (V,), -1, 1), U(g, (H, mb), -1, 1)
     dD, dbd, dh = ctx.array(D), ctx.array(bd), ctx.array(h)
+    if prepared:
+        ctx.softmax_prepare(dD, V, H)
     d_p, d_lp, d_scr = ctx.empty((V, mb)), ctx.empty((V, mb)), ctx.empty((V, mb))
     ctx.softmax_forward(dD, dbd, V, H, dh, mb, capi.ZR_SOFTMAX_PROB, d_p, d_scr)
     ctx.softmax_forward(dD, dbd, V, H, dh, mb, capi.ZR_SOFTMAX_LOGPROB, d_lp)  # in place on the logits
@@ -298,6 +302,18 @@ def test_softmax_prob_and_logprob(ctx, V, H, mb):
     mask = (g.random(mb) > 0.3).astype(np.int32)
     got = ctx.softmax_loss(dD, dbd, V, H, dh, mb, ctx.array(tgt), ctx.array(mask), d_scr)
     assert got == pytest.approx(o.softmax_loss(o.softmax_logprob_f64(logits), tgt, mask), rel=1e-5, abs=1e-6)
+    if prepared:
+        # re-packing after a change of D is picked up; releasing returns to the plain path
+        D2 = np.asfortranarray(-D)
+        dD.set(D2)
+        ctx.softmax_prepare(dD, V, H)
+        ctx.softmax_forward(dD, dbd, V, H, dh, mb, capi.ZR_SOFTMAX_LOGPROB, d_lp, d_scr)
+        ctx.sync()
+        assert_close(d_scr.get(), o.softmax_logits(D2, bd, h), what="logits after re-pack")
+        ctx.softmax_release(dD)
+        ctx.softmax_forward(dD, dbd, V, H, dh, mb, capi.ZR_SOFTMAX_LOGPROB, d_lp, d_scr)
+        ctx.sync()
+        assert_close(d_scr.get(), o.softmax_logits(D2, bd, h), what="logits after release")
 
 
 def test_softmax_extreme_logits_no_overflow(ctx):
@@ -314,7 +330,8 @@ def test_softmax_extreme_logits_no_overflow(ctx):
     assert np.allclose(P[:, 2], 1.0 / V)  # zero logits -> uniform
 
 
-def test_softmax_full_vocab_properties(ctx):
+@pytest.mark.parametrize("prepared", [False, True])
+def test_softmax_full_vocab_properties(ctx, prepared):
     """V=50000, H=1000, mb=128 (the benchmark shape): size-independent properties plus an exact check of a
     sampled set of columns against the oracle."""
     g = synth.rng(12, 1)
@@ -322,6 +339,8 @@ def test_softmax_full_vocab_properties(ctx):
     D, bd = U(g, (V, H)), U(g, (V,))
     h = np.tanh(U(g, (H, mb), -1, 1))
     dD, dbd = ctx.array(D), ctx.array(bd)
+    if prepared:
+        ctx.softmax_prepare(dD, V, H)
     d_p, d_scr = ctx.empty((V, mb)), ctx.empty((V, mb))
     ctx.softmax_forward(dD, dbd, V, H, ctx.array(h), mb, capi.ZR_SOFTMAX_PROB, d_p, d_scr)
     ctx.sync()
@@ -332,6 +351,8 @@ def test_softmax_full_vocab_properties(ctx):
     want_logits = o.softmax_logits(D, bd, np.asfortranarray(h[:, cols]))
     assert_close(logits[:, cols], want_logits, what="logits (sampled columns)")
     assert_close(P[:, cols], o.softmax_dist(want_logits), floor=1e-7, what="probabilities (sampled columns)")
+    if prepared:
+        ctx.softmax_release(dD)
 
 
 # ------------------------------------------------------------------------------------------------ A10 attention

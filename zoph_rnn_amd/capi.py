@@ -26,7 +26,7 @@ SYMBOLS = [
     "zr_ctx_create", "zr_ctx_destroy", "zr_ctx_sync", "zr_ctx_set_stream", "zr_ctx_set_option", "zr_last_error",
     "zr_version", "zr_timer_start", "zr_timer_stop", "zr_malloc", "zr_free", "zr_h2d", "zr_d2h", "zr_d2d", "zr_memset_zero", "zr_vocab_prep",
     "zr_vocab_prep_softmax", "zr_embed_gather", "zr_lstm_pack_weights", "zr_lstm_weights_destroy", "zr_lstm_step",
-    "zr_lstm_gates", "zr_lstm_stack_forward", "zr_gemm", "zr_softmax_forward", "zr_softmax_logprob_f64",
+    "zr_lstm_gates", "zr_lstm_stack_forward", "zr_gemm", "zr_softmax_prepare", "zr_softmax_release", "zr_softmax_forward", "zr_softmax_logprob_f64",
     "zr_softmax_loss", "zr_attn_create", "zr_attn_destroy", "zr_attn_step", "zr_gather_columns",
     "zr_broadcast_column", "zr_beam_create", "zr_beam_destroy", "zr_beam_init", "zr_beam_expand", "zr_beam_finish",
     "zr_beam_hypotheses", "zr_beam_state",
@@ -200,6 +200,12 @@ class Context:
                             _vp(d_B), C.c_int(ldb), _vp(d_C), C.c_int(ldc)))
 
     # ---- A8/A9
+    def softmax_prepare(self, d_D, V, H):
+        _chk(load().zr_softmax_prepare(self.h, _vp(d_D), C.c_int(V), C.c_int(H)))
+
+    def softmax_release(self, d_D):
+        _chk(load().zr_softmax_release(self.h, _vp(d_D)))
+
     def softmax_forward(self, d_D, d_b, V, H, d_h, mb, mode, d_out, d_scratch=None):
         _chk(load().zr_softmax_forward(self.h, _vp(d_D), _vp(d_b), C.c_int(V), C.c_int(H), _vp(d_h), C.c_int(mb),
                                        C.c_int(mode), _vp(d_out), _vp(d_scratch)))

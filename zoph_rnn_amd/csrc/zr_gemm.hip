@@ -22,31 +22,25 @@ struct GemmArgs {
   const int* mask;
   float* partials;
   int m_tiles, n_tiles;  // wave tiles along M and N
+  int b_pack4;           // B segments are k-interleaved copies: element (k, n) at ((k/4)*N + n)*4 + k%4
 };
 
-// Workgroup = 64*KS*WPB threads: WPB independent wave tiles, each shared by KS waves that split K.
-template <int TM, int TN, int KS, int WPB, bool TRANS_A, bool VEC, int EPI>
-__global__ void __launch_bounds__(64 * KS * WPB) gemm_kernel(GemmArgs a) {
-  __shared__ float red[KS > 1 ? WPB * KS * TN * 16 * 64 : 1];
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction
-  const int kslice = wave % KS;
-  const int sub = wave / KS;  // which wave tile of the workgroup
+// largest divisor c of nv with c * tm <= 32
+constexpr int stats_chunk(int nv, int tm) {
+  int best = 1;
+  for (int c = 1; c <= nv; ++c)
+    if (nv % c == 0 && c * tm <= 32) best = c;
+  return best;
+}
+
+// One output tile of 32*TM rows x 32*TN columns at (m0, n0), computed by the KS waves that call this together
+// (kslice = this wave's K slice, redp = their KS*TN*16*64 floats of LDS): all segments, the split-K sum and the
+// epilogue.  `active` false: same control flow (barriers), nothing stored.  PF = prefetch distance in k-groups.
+template <int TM, int TN, int KS, int AMODE, bool VEC, int EPI, int PF>
+__device__ __forceinline__ void gemm_tile(const GemmArgs& a, int m0, int n0, bool active, int z, float* redp,
+                                          int kslice, int lane) {
   const int jl = lane & 31;
   const int half = lane >> 5;
-  const int z = blockIdx.z;
-
-  // wave tile id -> (mt, nt), m fastest so that neighbouring waves stream neighbouring weight rows
-  long long tile = (long long)blockIdx.x * WPB + sub;
-  const long long ntiles = (long long)a.m_tiles * a.n_tiles;
-  const bool active = tile < ntiles;
-  if (!active) tile = ntiles - 1;  // keep the wave in step with the workgroup barriers; results discarded
-  const int mt = (int)(tile % a.m_tiles);
-  const int nt = (int)(tile / a.m_tiles);
-  const int m0 = mt * 32 * TM;
-  const int n0 = nt * 32 * TN;
-
   int rows[TM];
 #pragma unroll
   for (int tm = 0; tm < TM; ++tm) {
@@ -76,18 +70,96 @@ __global__ void __launch_bounds__(64 * KS * WPB) gemm_kernel(GemmArgs a) {
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) {
       wbase[tm] = A;
-      woff[tm] = TRANS_A ? (unsigned)((long long)rows[tm] * a.lda[s] + 4 * half)
-                         : (unsigned)(rows[tm] + 4LL * half * a.lda[s]);
+      woff[tm] = AMODE == ZR_A_PACK4   ? (unsigned)(4LL * rows[tm] + 4LL * half * a.lda[s])
+                 : AMODE == ZR_A_TRANS ? (unsigned)((long long)rows[tm] * a.lda[s] + 4 * half)
+                                       : (unsigned)(rows[tm] + 4LL * half * a.lda[s]);
     }
 #pragma unroll
-    for (int tn = 0; tn < TN; ++tn) xcol[tn] = a.B[s] + (long long)cols[tn] * a.ldb[s] + 4 * half;
-    zr_mma_segment<TM, TN, KS, zr_prefetch_depth(TM, TN), TRANS_A ? ZR_A_TRANS : ZR_A_NN, VEC>(acc, wbase, woff, a.lda[s], xcol, a.K[s],
-                                                                        kslice, half);
+    for (int tn = 0; tn < TN; ++tn)
+      xcol[tn] = (AMODE == ZR_A_PACK4 && a.b_pack4) ? a.B[s] + 4LL * cols[tn] + 4LL * half * a.N
+                                                   : a.B[s] + (long long)cols[tn] * a.ldb[s] + 4 * half;
+    zr_mma_segment<TM, TN, KS, PF, AMODE, VEC>(acc, wbase, woff, a.lda[s], xcol, a.K[s], kslice, half,
+                                               (AMODE == ZR_A_PACK4 && a.b_pack4) ? a.N : 1);
   }
 
   float* C = a.C + (long long)z * a.strideC;
   const float* bias = a.bias ? a.bias + (long long)z * a.strideBias : nullptr;
-  float* redp = KS > 1 ? red + (size_t)sub * KS * TN * 16 * 64 : red;
+
+  if (EPI == ZR_EPI_SOFTMAX_PARTIAL) {
+    // logits = acc + bias, plus (max, sum exp) of every 32-row block and column.  The values of all visits are
+    // collected first so that their cross-lane reductions run interleaved, then everything is stored.
+    float bias_v[TM];
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) bias_v[tm] = bias[rows[tm]];
+    auto store = [&](int n, int tm, bool okv, float val, float mxv, float sev) {
+      const int m = m0 + tm * 32 + jl;
+      if (okv) C[(long long)n * a.ldc + m] = val;
+      const int prow = (m0 >> 5) + tm;  // 32-row block index
+      if (jl == 0 && active && n < a.N && prow * 32 < a.M) {
+        float* p = a.partials + ((long long)prow * a.N + n) * 2;
+        p[0] = mxv;
+        p[1] = sev;
+      }
+    };
+    if (KS == 1) {
+      // four columns (accumulator registers) of every row sub-tile at a time
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+          float v[4 * TM], mx[4 * TM], se[4 * TM];
+          bool ok[4 * TM];
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm) {
+              const int n = n0 + tn * 32 + 8 * rg + 4 * half + i;
+              v[i * TM + tm] = acc[tm][tn][4 * rg + i] + bias_v[tm];
+              ok[i * TM + tm] = active && n < a.N && (m0 + tm * 32 + jl) < a.M;
+            }
+          zr_half_wave_softmax_stats<4 * TM>(v, ok, mx, se);
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm)
+              store(n0 + tn * 32 + 8 * rg + 4 * half + i, tm, ok[i * TM + tm], v[i * TM + tm], mx[i * TM + tm],
+                    se[i * TM + tm]);
+        }
+    } else {
+      constexpr int NV = zr_visit_count<TN, KS>();
+      float v[NV * TM];
+      bool ok[NV * TM];
+      int nn[NV];
+      zr_reduce_visit<TM, TN, KS>(acc, redp, kslice, lane, [&](const float(&vals)[TM], int tn, int r, int i) {
+        const int n = n0 + tn * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+        nn[i] = n;
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) {
+          v[i * TM + tm] = vals[tm] + bias_v[tm];
+          ok[i * TM + tm] = active && n < a.N && (m0 + tm * 32 + jl) < a.M;
+        }
+      });
+      // at most 32 butterflies at a time (register budget)
+      constexpr int CH = stats_chunk(NV, TM);
+#pragma unroll
+      for (int c0 = 0; c0 < NV; c0 += CH) {
+        float cv[CH * TM], cmx[CH * TM], cse[CH * TM];
+        bool cok[CH * TM];
+#pragma unroll
+        for (int j = 0; j < CH * TM; ++j) {
+          cv[j] = v[c0 * TM + j];
+          cok[j] = ok[c0 * TM + j];
+        }
+        zr_half_wave_softmax_stats<CH * TM>(cv, cok, cmx, cse);
+#pragma unroll
+        for (int i = 0; i < CH; ++i)
+#pragma unroll
+          for (int tm = 0; tm < TM; ++tm)
+            store(nn[c0 + i], tm, cok[i * TM + tm], cv[i * TM + tm], cmx[i * TM + tm], cse[i * TM + tm]);
+      }
+    }
+    return;
+  }
 
   zr_reduce_visit<TM, TN, KS>(acc, redp, kslice, lane, [&](const float(&vals)[TM], int tn, int r, int) {
     const int n = n0 + tn * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
@@ -104,31 +176,95 @@ __global__ void __launch_bounds__(64 * KS * WPB) gemm_kernel(GemmArgs a) {
         }
       } else if (EPI == ZR_EPI_TANH) {
         if (ok) C[(long long)n * a.ldc + m] = tanhf(v);
-      } else if (EPI == ZR_EPI_TANH_BIAS_MASK) {
+      } else {  // ZR_EPI_TANH_BIAS_MASK
         if (ok) C[(long long)n * a.ldc + m] = tanhf(v + bias[m]) * (float)a.mask[n];
-      } else {  // ZR_EPI_SOFTMAX_PARTIAL
-        if (ok) {
-          v += bias[m];
-          C[(long long)n * a.ldc + m] = v;
-        }
-        // (max, sum exp) over the 32 rows of this sub-tile for column n: reduce across the 32 lanes of a half
-        float mx = ok ? v : -INFINITY;
-#pragma unroll
-        for (int off = 16; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
-        float e = ok ? expf(v - mx) : 0.0f;
-#pragma unroll
-        for (int off = 16; off > 0; off >>= 1) e += __shfl_xor(e, off, 64);
-        const int prow = (m0 >> 5) + tm;  // 32-row block index
-        if (jl == 0 && n_ok && prow * 32 < a.M) {
-          float* p = a.partials + ((long long)prow * a.N + n) * 2;
-          p[0] = mx;
-          p[1] = e;
-        }
       }
     }
   });
 }
 
+// Workgroup = 64*KS*WPB threads: WPB independent wave tiles, each shared by KS waves that split K.
+// AMODE is the weight layout (ZR_A_NN / ZR_A_TRANS / ZR_A_PACK4).  The packed variant is built for two workgroups
+// per CU (at most 256 registers per wave): with several workgroups per CU in sequence, the prologue and epilogue
+// of one overlap the K loop of the other.
+template <int TM, int TN, int KS, int WPB, int AMODE, bool VEC, int EPI, int OCC = 1>
+__global__ void __launch_bounds__(64 * KS * WPB, OCC) gemm_kernel(GemmArgs a) {
+  __shared__ float red[KS > 1 ? WPB * KS * TN * 16 * 64 : 1];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction
+  const int kslice = wave % KS;
+  const int sub = wave / KS;  // which wave tile of the workgroup
+  const int jl = lane & 31;
+  const int half = lane >> 5;
+  const int z = blockIdx.z;
+
+  long long tile = (long long)blockIdx.x * WPB + sub;
+  const long long ntiles = (long long)a.m_tiles * a.n_tiles;
+  bool active = tile < ntiles;
+  int mt, nt;
+  if (AMODE == ZR_A_PACK4) {
+    // Workgroup ids congruent modulo 8 run on the same XCD.  Each XCD gets a contiguous range of row tiles and
+    // runs the column tiles of one row tile back to back, so a weight tile leaves memory once.
+    const int r8 = (int)(tile & 7);
+    const int q = (int)(tile >> 3);
+    const int mpx = (a.m_tiles + 7) >> 3;
+    nt = q % a.n_tiles;
+    mt = r8 * mpx + q / a.n_tiles;
+    active = (q / a.n_tiles < mpx) && (mt < a.m_tiles);
+    if (!active) mt = a.m_tiles - 1;
+  } else {
+    // wave tile id -> (mt, nt), m fastest so that neighbouring waves stream neighbouring weight rows
+    if (!active) tile = ntiles - 1;  // keep the wave in step with the workgroup barriers; results discarded
+    mt = (int)(tile % a.m_tiles);
+    nt = (int)(tile / a.m_tiles);
+  }
+  constexpr int PF = AMODE == ZR_A_PACK4 ? (OCC == 1 ? (TM + TN <= 4 ? 8 : 6) : (TM + TN == 4 ? 6 : 4))
+                                         : zr_prefetch_depth(TM, TN);
+  float* redp = KS > 1 ? red + (size_t)sub * KS * TN * 16 * 64 : red;
+  gemm_tile<TM, TN, KS, AMODE, VEC, EPI, PF>(a, mt * 32 * TM, nt * 32 * TN, active, z, redp, kslice, lane);
+}
+
+// Row-range variant for a tall weight matrix in the k-interleaved layout (the softmax logits: tens of thousands
+// of rows, a minibatch of columns).  With one tile per workgroup the number of workgroups is rarely a multiple of
+// the number of CUs and the last, partly filled round costs as much as a full one.  Here the grid is one
+// workgroup per CU (or fewer): each takes an equal share of the 32-row blocks (+-1) for one column tile and walks
+// it in passes of up to four blocks, so every CU finishes at about the same time and each weight element is
+// read by exactly one workgroup per column tile.
+template <int TN, int EPI>
+__global__ void __launch_bounds__(256) gemm_rows_kernel(GemmArgs a, int row_chunks) {
+  __shared__ float red[4 * TN * 16 * 64];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int kslice = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // ids congruent modulo 8 share an XCD: give each XCD a contiguous range of row chunks, column tiles adjacent
+  const int r8 = blockIdx.x & 7;
+  const int q = blockIdx.x >> 3;
+  const int cpx = (row_chunks + 7) >> 3;
+  const int nt = q % a.n_tiles;
+  const int chunk = r8 * cpx + q / a.n_tiles;
+  if (q / a.n_tiles >= cpx || chunk >= row_chunks) return;
+  const long long blocks = (a.M + 31) >> 5;
+  int b = (int)(blocks * chunk / row_chunks);
+  const int b_end = (int)(blocks * (chunk + 1) / row_chunks);
+  const int n0 = nt * 32 * TN;
+  // at most 192 accumulator registers per wave: four blocks per pass up to 96 columns, three at 128
+  constexpr int TMAX = TN <= 3 ? 4 : 3;
+  constexpr int PF4 = TN <= 2 ? 6 : (TN == 3 ? 4 : 3);
+  while (b < b_end) {
+    const int nb = b_end - b < TMAX ? b_end - b : TMAX;  // uniform over the workgroup
+    if (TMAX == 4 && nb == 4)
+      gemm_tile<TMAX, TN, 4, ZR_A_PACK4, true, EPI, PF4>(a, b * 32, n0, true, 0, red, kslice, lane);
+    else if (nb == 3)
+      gemm_tile<3, TN, 4, ZR_A_PACK4, true, EPI, PF4 + 1>(a, b * 32, n0, true, 0, red, kslice, lane);
+    else if (nb == 2)
+      gemm_tile<2, TN, 4, ZR_A_PACK4, true, EPI, PF4 + 2>(a, b * 32, n0, true, 0, red, kslice, lane);
+    else
+      gemm_tile<1, TN, 4, ZR_A_PACK4, true, EPI, PF4 + 2>(a, b * 32, n0, true, 0, red, kslice, lane);
+    b += nb;
+    __syncthreads();  // the next pass reuses the reduction buffer
+  }
+}
 
 // ---------------------------------------------------------------------------------------------------------
 // Large-M variant: weight rows staged through LDS and shared by all waves of the workgroup.
@@ -258,36 +394,50 @@ __global__ void __launch_bounds__(64 * NWV) gemm_lds_kernel(GemmArgs a) {
     __syncthreads();
   }
 
+  float bias_v[TMR];
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int n = n0 + 8 * (r >> 2) + 4 * half + (r & 3);
-    const bool n_ok = n < a.N;
+  for (int tm = 0; tm < TMR; ++tm) {
+    const int m = m0 + tm * 32 + jl;
+    bias_v[tm] = a.bias ? a.bias[m < M ? m : M - 1] : 0.0f;
+  }
+  if (EPI == ZR_EPI_STORE) {
 #pragma unroll
-    for (int tm = 0; tm < TMR; ++tm) {
-      const int m = m0 + tm * 32 + jl;
-      const bool ok = n_ok && m < M;
-      float v = acc[tm][r];
-      if (EPI == ZR_EPI_STORE) {
-        if (ok) {
-          if (a.bias) v += a.bias[m];
-          a.C[(long long)n * a.ldc + m] = v;
+    for (int r = 0; r < 16; ++r) {
+      const int n = n0 + 8 * (r >> 2) + 4 * half + (r & 3);
+#pragma unroll
+      for (int tm = 0; tm < TMR; ++tm) {
+        const int m = m0 + tm * 32 + jl;
+        if (n < a.N && m < M) a.C[(long long)n * a.ldc + m] = acc[tm][r] + bias_v[tm];
+      }
+    }
+  } else {  // ZR_EPI_SOFTMAX_PARTIAL: four columns (accumulator registers) of all row sub-tiles at a time
+#pragma unroll
+    for (int rg = 0; rg < 4; ++rg) {
+      float v[4 * TMR], mx[4 * TMR], se[4 * TMR];
+      bool ok[4 * TMR];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = n0 + 8 * rg + 4 * half + i;
+#pragma unroll
+        for (int tm = 0; tm < TMR; ++tm) {
+          v[i * TMR + tm] = acc[tm][4 * rg + i] + bias_v[tm];
+          ok[i * TMR + tm] = n < a.N && (m0 + tm * 32 + jl) < M;
         }
-      } else {  // ZR_EPI_SOFTMAX_PARTIAL
-        if (ok) {
-          v += a.bias[m];
-          a.C[(long long)n * a.ldc + m] = v;
-        }
-        float mx = ok ? v : -INFINITY;
+      }
+      zr_half_wave_softmax_stats<4 * TMR>(v, ok, mx, se);
 #pragma unroll
-        for (int off = 16; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
-        float e = ok ? expf(v - mx) : 0.0f;
+      for (int i = 0; i < 4; ++i) {
+        const int n = n0 + 8 * rg + 4 * half + i;
 #pragma unroll
-        for (int off = 16; off > 0; off >>= 1) e += __shfl_xor(e, off, 64);
-        const int prow = (m0 >> 5) + tm;
-        if (jl == 0 && n_ok && prow * 32 < M) {
-          float* p = a.partials + ((long long)prow * a.N + n) * 2;
-          p[0] = mx;
-          p[1] = e;
+        for (int tm = 0; tm < TMR; ++tm) {
+          const int m = m0 + tm * 32 + jl;
+          if (ok[i * TMR + tm]) a.C[(long long)n * a.ldc + m] = v[i * TMR + tm];
+          const int prow = (m0 >> 5) + tm;
+          if (jl == 0 && n < a.N && prow * 32 < M) {
+            float* p = a.partials + ((long long)prow * a.N + n) * 2;
+            p[0] = mx[i * TMR + tm];
+            p[1] = se[i * TMR + tm];
+          }
         }
       }
     }
@@ -320,23 +470,24 @@ int launch_lds_rows(zr_ctx* ctx, GemmArgs& ga, int epi) {
   return launch_lds<4, NWV>(ctx, ga, epi);
 }
 
-template <int TM, int TN, int KS, int WPB, bool TRANS_A, bool VEC>
+template <int TM, int TN, int KS, int WPB, int AMODE, bool VEC, int OCC = 1>
 int launch_epi(zr_ctx* ctx, const GemmArgs& ga, int batch, int epi) {
-  const long long ntiles = (long long)ga.m_tiles * ga.n_tiles;
+  long long ntiles = (long long)ga.m_tiles * ga.n_tiles;
+  if (AMODE == ZR_A_PACK4) ntiles = (long long)((ga.m_tiles + 7) / 8) * 8 * ga.n_tiles;  // XCD-major id space
   dim3 grid((unsigned)((ntiles + WPB - 1) / WPB), 1, batch);
   dim3 block(64 * KS * WPB);
   switch (epi) {
     case ZR_EPI_STORE:
-      gemm_kernel<TM, TN, KS, WPB, TRANS_A, VEC, ZR_EPI_STORE><<<grid, block, 0, ctx->stream>>>(ga);
+      gemm_kernel<TM, TN, KS, WPB, AMODE, VEC, ZR_EPI_STORE, OCC><<<grid, block, 0, ctx->stream>>>(ga);
       break;
     case ZR_EPI_TANH:
-      gemm_kernel<TM, TN, KS, WPB, TRANS_A, VEC, ZR_EPI_TANH><<<grid, block, 0, ctx->stream>>>(ga);
+      gemm_kernel<TM, TN, KS, WPB, AMODE, VEC, ZR_EPI_TANH, OCC><<<grid, block, 0, ctx->stream>>>(ga);
       break;
     case ZR_EPI_TANH_BIAS_MASK:
-      gemm_kernel<TM, TN, KS, WPB, TRANS_A, VEC, ZR_EPI_TANH_BIAS_MASK><<<grid, block, 0, ctx->stream>>>(ga);
+      gemm_kernel<TM, TN, KS, WPB, AMODE, VEC, ZR_EPI_TANH_BIAS_MASK, OCC><<<grid, block, 0, ctx->stream>>>(ga);
       break;
     default:
-      gemm_kernel<TM, TN, KS, WPB, TRANS_A, VEC, ZR_EPI_SOFTMAX_PARTIAL><<<grid, block, 0, ctx->stream>>>(ga);
+      gemm_kernel<TM, TN, KS, WPB, AMODE, VEC, ZR_EPI_SOFTMAX_PARTIAL, OCC><<<grid, block, 0, ctx->stream>>>(ga);
       break;
   }
   ZR_LAUNCH_CHECK("gemm_kernel");
@@ -348,14 +499,68 @@ int launch_cfg(zr_ctx* ctx, GemmArgs& ga, int batch, int epi, bool trans_a, bool
   ga.m_tiles = (ga.M + 32 * TM - 1) / (32 * TM);
   ga.n_tiles = (ga.N + 32 * TN - 1) / (32 * TN);
   if (trans_a) {
-    if (vec) return launch_epi<TM, TN, KS, WPB, true, true>(ctx, ga, batch, epi);
-    return launch_epi<TM, TN, KS, WPB, true, false>(ctx, ga, batch, epi);
+    if (vec) return launch_epi<TM, TN, KS, WPB, ZR_A_TRANS, true>(ctx, ga, batch, epi);
+    return launch_epi<TM, TN, KS, WPB, ZR_A_TRANS, false>(ctx, ga, batch, epi);
   }
-  if (vec) return launch_epi<TM, TN, KS, WPB, false, true>(ctx, ga, batch, epi);
-  return launch_epi<TM, TN, KS, WPB, false, false>(ctx, ga, batch, epi);
+  if (vec) return launch_epi<TM, TN, KS, WPB, ZR_A_NN, true>(ctx, ga, batch, epi);
+  return launch_epi<TM, TN, KS, WPB, ZR_A_NN, false>(ctx, ga, batch, epi);
+}
+
+// k-interleaved weights: one wave tile per workgroup, K split over its 4 waves
+template <int TM, int TN, int OCC>
+int launch_pack4(zr_ctx* ctx, GemmArgs& ga, int epi, bool vec) {
+  ga.m_tiles = (ga.M + 32 * TM - 1) / (32 * TM);
+  ga.n_tiles = (ga.N + 32 * TN - 1) / (32 * TN);
+  if (vec) return launch_epi<TM, TN, 4, 1, ZR_A_PACK4, true, OCC>(ctx, ga, 1, epi);
+  return launch_epi<TM, TN, 4, 1, ZR_A_PACK4, false, OCC>(ctx, ga, 1, epi);
+}
+
+// Activations X (K x N, column n at src + n*ld) into [K/4][N][4]; K % 4 == 0.  One thread per float4.
+__global__ void __launch_bounds__(256) pack4_x_kernel(const float* __restrict__ src, int K, int N, int ld,
+                                                      float* __restrict__ dst) {
+  const int i = blockIdx.x * 256 + threadIdx.x;  // float4 index in the source order: (n, k/4)
+  const int kb = K >> 2;
+  if (i >= kb * N) return;
+  const int n = i / kb, b = i - n * kb;
+  const zr_f32x4 v = *(const zr_f32x4*)(src + (long long)n * ld + 4 * b);
+  *(zr_f32x4*)(dst + ((long long)b * N + n) * 4) = v;
+}
+
+template <int TN>
+int launch_rows(zr_ctx* ctx, GemmArgs& ga, int epi, int n_tiles) {
+  ga.n_tiles = n_tiles;
+  ga.m_tiles = 0;
+  const int blocks = (ga.M + 31) / 32;
+  int row_chunks = 256 / n_tiles;  // one workgroup per CU
+  if (row_chunks > blocks) row_chunks = blocks;
+  const unsigned grid = (unsigned)((row_chunks + 7) / 8) * 8 * n_tiles;
+  if (epi == ZR_EPI_STORE)
+    gemm_rows_kernel<TN, ZR_EPI_STORE><<<grid, 256, 0, ctx->stream>>>(ga, row_chunks);
+  else
+    gemm_rows_kernel<TN, ZR_EPI_SOFTMAX_PARTIAL><<<grid, 256, 0, ctx->stream>>>(ga, row_chunks);
+  ZR_LAUNCH_CHECK("gemm_rows_kernel");
+  return ZR_OK;
+}
+
+__global__ void __launch_bounds__(256) pack4_kernel(const float* __restrict__ src, int M, int K, long long ld,
+                                                    int ldp, int kp, float* __restrict__ dst) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (long long)kp * ldp) return;
+  const int k4 = (int)(i & 3);
+  const long long t = i >> 2;
+  const int row = (int)(t % ldp);
+  const int k = (int)(t / ldp) * 4 + k4;
+  dst[i] = (row < M && k < K) ? src[row + (long long)k * ld] : 0.0f;
 }
 
 }  // namespace
+
+int zr_pack4_launch(zr_ctx* ctx, const float* src, int M, int K, long long ld, int ldp, int kp, float* dst) {
+  const long long total = (long long)kp * ldp;
+  pack4_kernel<<<(unsigned)((total + 255) / 256), 256, 0, ctx->stream>>>(src, M, K, ld, ldp, kp, dst);
+  ZR_LAUNCH_CHECK("pack4_kernel");
+  return ZR_OK;
+}
 
 int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
   ZR_CHECK_ARG(d.M > 0 && d.N > 0, "gemm: M = %d, N = %d", d.M, d.N);
@@ -373,6 +578,8 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
       ZR_CHECK_ARG(d.K[s] > 0, "gemm: K[%d] = %d", s, d.K[s]);
       ZR_CHECK_ARG(d.A[s] && d.B[s], "gemm: null operand in segment %d", s);
       ZR_CHECK_ARG(d.lda[s] >= (d.trans_a ? d.K[s] : d.M), "gemm: lda[%d] = %d too small", s, d.lda[s]);
+      ZR_CHECK_ARG(!d.a_pack4 || (!d.trans_a && d.batch == 1 && d.lda[s] % 32 == 0 && 4LL * d.lda[s] + 4LL * d.M < (1LL << 31)),
+                   "gemm: packed operand A of segment %d: needs no transpose, one batch, lda a multiple of 32", s);
       ZR_CHECK_ARG(d.ldb[s] >= d.K[s], "gemm: ldb[%d] = %d < K = %d", s, d.ldb[s], d.K[s]);
       // per-lane weight offsets are 32-bit element indices
       ZR_CHECK_ARG(d.trans_a ? ((long long)d.M * d.lda[s] + 8 < (1LL << 31)) : (d.M + 8LL * d.lda[s] < (1LL << 31)),
@@ -404,6 +611,46 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
   if (d.epilogue == ZR_EPI_TANH_BIAS_MASK) ZR_CHECK_ARG(d.bias && d.mask, "gemm: bias/mask required");
   if (d.epilogue == ZR_EPI_SOFTMAX_PARTIAL) ZR_CHECK_ARG(d.bias && d.partials, "gemm: bias/partials required");
 
+  ga.b_pack4 = 0;
+  if (d.a_pack4) {
+    // Activations too: a k-interleaved copy in scratch turns their loads (16 bytes from each of 32 lines per
+    // half-wave) into contiguous ones.  Worth a small extra kernel once the weight matrix is large.
+    bool xpack = vec && d.M >= 2048;
+    size_t xfloats = 0;
+    for (int s = 0; s < d.nseg; ++s) {
+      xpack = xpack && (d.K[s] % 8 == 0);
+      xfloats += (size_t)d.K[s] * d.N;
+    }
+    if (xpack) {
+      void* p = nullptr;
+      int rc = zr_ctx_scratch(ctx, 0, sizeof(float) * xfloats, &p);
+      if (rc) return rc;
+      float* xp = (float*)p;
+      for (int s = 0; s < d.nseg; ++s) {
+        const int f4 = (d.K[s] / 4) * d.N;
+        pack4_x_kernel<<<(f4 + 255) / 256, 256, 0, ctx->stream>>>(d.B[s], d.K[s], d.N, d.ldb[s], xp);
+        ZR_LAUNCH_CHECK("pack4_x_kernel");
+        ga.B[s] = xp;
+        xp += (size_t)d.K[s] * d.N;
+      }
+      ga.b_pack4 = 1;
+    }
+    // tall matrices: equal row ranges per CU, column tiles of equal width (at most 128 columns each)
+    if (vec && d.nseg == 1 && d.M >= 8192 && d.N > 32 && d.N <= 1024 && ctx->gemm_cfg != 11 &&
+        (d.epilogue == ZR_EPI_STORE || d.epilogue == ZR_EPI_SOFTMAX_PARTIAL)) {
+      const int n32 = (d.N + 31) / 32;
+      const int n_tiles = (n32 + 3) / 4;
+      const int tn = (n32 + n_tiles - 1) / n_tiles;
+      if (tn <= 2) return launch_rows<2>(ctx, ga, d.epilogue, n_tiles);
+      if (tn == 3) return launch_rows<3>(ctx, ga, d.epilogue, n_tiles);
+      return launch_rows<4>(ctx, ga, d.epilogue, n_tiles);
+    }
+    if (ctx->gemm_cfg == 12) return launch_pack4<4, 2, 1>(ctx, ga, d.epilogue, vec);
+    if (ctx->gemm_cfg == 13) return launch_pack4<2, 2, 1>(ctx, ga, d.epilogue, vec);
+    if (ctx->gemm_cfg == 14) return launch_pack4<2, 4, 1>(ctx, ga, d.epilogue, vec);
+    if (d.N <= 32) return launch_pack4<2, 1, 2>(ctx, ga, d.epilogue, vec);
+    return launch_pack4<2, 2, 2>(ctx, ga, d.epilogue, vec);
+  }
   // Large, untransposed, single-segment products with a wide batch (the softmax logits): LDS-shared weights.
   const bool lds_ok = !d.trans_a && d.nseg == 1 && d.batch == 1 && vec && (d.M % 4 == 0) && (d.lda[0] % 4 == 0) &&
                       (((uintptr_t)d.A[0] & 15u) == 0) && d.K[0] >= 8 && d.M >= 4096 && d.N >= 96 &&

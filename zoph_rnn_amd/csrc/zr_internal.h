@@ -8,6 +8,7 @@
 #include "../../include/zoph_rnn.h"
 
 #define ZR_MAX_COUNTERS 4096
+#define ZR_MAX_PACKED_D 8
 
 struct zr_ctx {
   int device;
@@ -28,6 +29,13 @@ struct zr_ctx {
   size_t scratch_bytes;
   void* d_scratch2;
   size_t scratch2_bytes;
+  // output-layer matrices registered with zr_softmax_prepare: the caller's D pointer -> its k-interleaved copy
+  struct PackedD {
+    const float* key;  // the caller's d_D (null: slot free)
+    int V, H;
+    int ldp;           // V rounded up to 32
+    float* d_pack;     // [ceil8(H)/4][ldp][4]
+  } packed_d[ZR_MAX_PACKED_D];
 };
 
 // error plumbing -------------------------------------------------------------------------------------------
@@ -76,6 +84,9 @@ struct ZrGemmDesc {
   const float* A[3];
   int lda[3];
   int trans_a;  // applies to every segment
+  // A is k-interleaved: element (m, k) at ((k/4)*lda + m)*4 + k%4, lda = M rounded up to 32, K padded to a multiple
+  // of 8, pads zero (see ZR_A_PACK4 in zr_mfma_core.h).  Single batch, no transpose.
+  int a_pack4;
   const float* B[3];
   int ldb[3];
   float* C;
@@ -90,6 +101,9 @@ struct ZrGemmDesc {
 };
 
 int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d);
+// Packs one M x K column-major matrix (leading dimension ld) into the k-interleaved layout [kp/4][ldp][4] with
+// zero padding (ldp >= M a multiple of 32, kp >= K a multiple of 8).  dst holds kp*ldp floats.
+int zr_pack4_launch(zr_ctx* ctx, const float* src, int M, int K, long long ld, int ldp, int kp, float* dst);
 // number of 32-row partial blocks the SOFTMAX_PARTIAL epilogue writes for M rows
 static inline int zr_softmax_partial_blocks(int M) { return (M + 31) / 32; }
 

@@ -424,19 +424,6 @@ __global__ void __launch_bounds__(64 * NWV) lstm_lds_kernel(LstmLaunch2 P) {
   }
 }
 
-// One H x H column-major matrix (element (row, k) at src[row + k*H]) into the packed [kp/4][ldw][4] layout,
-// padding with zeros.  One thread per destination element.
-__global__ void __launch_bounds__(256) lstm_pack_kernel(const float* __restrict__ src, int H, int ldw, int kp,
-                                                        float* __restrict__ dst) {
-  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
-  if (i >= (long long)kp * ldw) return;
-  const int k4 = (int)(i & 3);
-  const long long t = i >> 2;
-  const int row = (int)(t % ldw);
-  const int k = (int)(t / ldw) * 4 + k4;
-  dst[i] = (row < H && k < H) ? src[row + (long long)k * H] : 0.0f;
-}
-
 template <int TN, int KS>
 int launch_fused_v(zr_ctx* ctx, const LstmLaunch& L, bool vec) {
   const int groups = L.n_units * L.j_tiles;
@@ -557,15 +544,11 @@ int zr_lstm_pack_weights(zr_ctx* ctx, const float* const d_M[4], const float* co
   for (int g = 0; g < 4; ++g) {
     const float* segs[3] = {d_M[g], d_Wh[g], d_Q ? d_Q[g] : nullptr};
     for (int s = 0; s < nseg; ++s) {
-      const long long total = (long long)HH;
-      lstm_pack_kernel<<<(unsigned)((total + 255) / 256), 256, 0, ctx->stream>>>(segs[s], H, ldw, kp,
-                                                                                 w->d_W + ((size_t)s * 4 + g) * HH);
-      hipError_t e = hipGetLastError();
-      if (e != hipSuccess) {
+      if (zr_pack4_launch(ctx, segs[s], H, H, H, ldw, kp, w->d_W + ((size_t)s * 4 + g) * HH) != ZR_OK) {
         (void)hipFree(w->d_W);
         (void)hipFree(w->d_bias);
         delete w;
-        return zr_set_error(ZR_EHIP, "zr_lstm_pack_weights: pack kernel failed: %s", hipGetErrorString(e));
+        return ZR_EHIP;
       }
     }
     hipError_t e = hipMemcpyAsync(w->d_bias + (size_t)g * H, d_b[g], sizeof(float) * H, hipMemcpyDeviceToDevice,

@@ -243,4 +243,47 @@ __device__ __forceinline__ void zr_reduce_visit(zr_f32x16 (&acc)[TM][TN], float*
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// (max, sum of exp(v - max)) over the 32 lanes of each half-wave, for G independent values per lane at once.
+// In the MFMA output layout a half-wave holds the 32 rows of one output column, so this is the softmax partial
+// of a 32-row block.  The G butterflies are interleaved (a lone butterfly is a chain of ten dependent cross-lane
+// moves, each with the latency of an LDS round trip); the steps inside a 16-lane row are DPP moves on the
+// vector ALU, only the last one crosses rows.  Must be called by all 64 lanes.  Lanes with ok == false
+// contribute nothing; if no lane of a half is ok the result is (-inf, 0).
+// ---------------------------------------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float zr_dpp_move(float x) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, false));
+}
+
+template <int G>
+__device__ __forceinline__ void zr_half_wave_softmax_stats(const float (&v)[G], const bool (&ok)[G], float (&mx)[G],
+                                                           float (&se)[G]) {
+  // lane pairings: quad_perm(1,0,3,2), quad_perm(2,3,0,1), row_half_mirror, row_mirror, then lanes 16 apart
+#pragma unroll
+  for (int g = 0; g < G; ++g) mx[g] = ok[g] ? v[g] : -INFINITY;
+#pragma unroll
+  for (int g = 0; g < G; ++g) mx[g] = fmaxf(mx[g], zr_dpp_move<0xB1>(mx[g]));
+#pragma unroll
+  for (int g = 0; g < G; ++g) mx[g] = fmaxf(mx[g], zr_dpp_move<0x4E>(mx[g]));
+#pragma unroll
+  for (int g = 0; g < G; ++g) mx[g] = fmaxf(mx[g], zr_dpp_move<0x141>(mx[g]));
+#pragma unroll
+  for (int g = 0; g < G; ++g) mx[g] = fmaxf(mx[g], zr_dpp_move<0x140>(mx[g]));
+#pragma unroll
+  for (int g = 0; g < G; ++g) mx[g] = fmaxf(mx[g], __shfl_xor(mx[g], 16, 64));
+#pragma unroll
+  for (int g = 0; g < G; ++g) se[g] = ok[g] ? expf(v[g] - mx[g]) : 0.0f;
+#pragma unroll
+  for (int g = 0; g < G; ++g) se[g] += zr_dpp_move<0xB1>(se[g]);
+#pragma unroll
+  for (int g = 0; g < G; ++g) se[g] += zr_dpp_move<0x4E>(se[g]);
+#pragma unroll
+  for (int g = 0; g < G; ++g) se[g] += zr_dpp_move<0x141>(se[g]);
+#pragma unroll
+  for (int g = 0; g < G; ++g) se[g] += zr_dpp_move<0x140>(se[g]);
+#pragma unroll
+  for (int g = 0; g < G; ++g) se[g] += __shfl_xor(se[g], 16, 64);
+}
+
 #endif

@@ -83,6 +83,8 @@ int zr_ctx_destroy(zr_ctx* ctx) {
   if (ctx->d_scratch) (void)hipFree(ctx->d_scratch);
   if (ctx->d_scratch2) (void)hipFree(ctx->d_scratch2);
   if (ctx->d_flags) (void)hipFree(ctx->d_flags);
+  for (int i = 0; i < ZR_MAX_PACKED_D; ++i)
+    if (ctx->packed_d[i].d_pack) (void)hipFree(ctx->packed_d[i].d_pack);
   if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
   if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);
   (void)hipStreamDestroy(ctx->own_stream);
@@ -134,7 +136,7 @@ int zr_ctx_set_option(zr_ctx* ctx, int option, int value) {
       ctx->lstm_kparts = value;
       return ZR_OK;
     case ZR_OPT_GEMM_CFG:
-      ZR_CHECK_ARG(value >= 0 && value <= 10, "ZR_OPT_GEMM_CFG out of range");
+      ZR_CHECK_ARG(value >= 0 && value <= 14, "ZR_OPT_GEMM_CFG out of range");
       ctx->gemm_cfg = value;
       return ZR_OK;
     default:

@@ -158,6 +158,15 @@ int logits_with_partials(zr_ctx* ctx, const float* d_D, const float* d_b_d, int 
   d.K[0] = H;
   d.A[0] = d_D;
   d.lda[0] = V;
+  for (int i = 0; i < ZR_MAX_PACKED_D; ++i) {
+    const zr_ctx::PackedD& e = ctx->packed_d[i];
+    if (e.key == d_D && e.V == V && e.H == H) {  // registered with zr_softmax_prepare: use the MFMA-layout copy
+      d.A[0] = e.d_pack;
+      d.lda[0] = e.ldp;
+      d.a_pack4 = 1;
+      break;
+    }
+  }
   d.B[0] = d_h;
   d.ldb[0] = H;
   d.C = d_logits;
@@ -189,6 +198,58 @@ int check_softmax_args(const char* who, const float* d_D, const float* d_b_d, in
 }  // namespace
 
 extern "C" {
+
+int zr_softmax_prepare(zr_ctx* ctx, const float* d_D, int V, int H) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(d_D != nullptr && V > 0 && H > 0, "zr_softmax_prepare: d_D null or V = %d, H = %d", V, H);
+  const int ldp = (V + 31) / 32 * 32, kp = (H + 7) / 8 * 8;
+  ZR_CHECK_ARG(4LL * ldp + 4LL * V < (1LL << 31), "zr_softmax_prepare: V = %d too large", V);
+  int slot = -1;
+  for (int i = 0; i < ZR_MAX_PACKED_D; ++i)
+    if (ctx->packed_d[i].key == d_D) slot = i;
+  if (slot >= 0 && (ctx->packed_d[slot].V != V || ctx->packed_d[slot].H != H)) {
+    rc = zr_softmax_release(ctx, d_D);
+    if (rc) return rc;
+    slot = -1;
+  }
+  if (slot < 0) {
+    for (int i = 0; i < ZR_MAX_PACKED_D && slot < 0; ++i)
+      if (!ctx->packed_d[i].key) slot = i;
+    ZR_CHECK_ARG(slot >= 0, "zr_softmax_prepare: all %d slots are in use (zr_softmax_release one)", ZR_MAX_PACKED_D);
+    float* p = nullptr;
+    if (hipMalloc((void**)&p, sizeof(float) * (size_t)kp * ldp) != hipSuccess) {
+      (void)hipGetLastError();
+      return zr_set_error(ZR_ENOMEM, "zr_softmax_prepare: allocation of %zu bytes failed",
+                          sizeof(float) * (size_t)kp * ldp);
+    }
+    ctx->packed_d[slot].d_pack = p;
+    ctx->packed_d[slot].V = V;
+    ctx->packed_d[slot].H = H;
+    ctx->packed_d[slot].ldp = ldp;
+  }
+  rc = zr_pack4_launch(ctx, d_D, V, H, V, ldp, kp, ctx->packed_d[slot].d_pack);
+  if (rc) {
+    (void)hipFree(ctx->packed_d[slot].d_pack);
+    ctx->packed_d[slot] = zr_ctx::PackedD{};
+    return rc;
+  }
+  ctx->packed_d[slot].key = d_D;
+  return ZR_OK;
+}
+
+int zr_softmax_release(zr_ctx* ctx, const float* d_D) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  for (int i = 0; i < ZR_MAX_PACKED_D; ++i) {
+    if (ctx->packed_d[i].key == d_D && d_D) {
+      ZR_HIP(hipStreamSynchronize(ctx->stream));
+      (void)hipFree(ctx->packed_d[i].d_pack);
+      ctx->packed_d[i] = zr_ctx::PackedD{};
+    }
+  }
+  return ZR_OK;
+}
 
 int zr_softmax_forward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int mb,
                        int mode, float* d_out, float* d_logits_scratch) {

@@ -29,6 +29,7 @@ class Seq2SeqWeights:
         self.tgt = [self._pack(ly) for ly in tgt_layers]
         self.attn = {k: ctx.array(v, np.float32) for k, v in attn.items()}
         self.D_soft = ctx.array(D_soft, np.float32)
+        ctx.softmax_prepare(self.D_soft, self.Vt, self.H)
         self.b_soft = ctx.array(b_soft, np.float32)
 
     def _pack(self, ly):

@@ -349,6 +349,7 @@ class softmax_layer : public base_loss_layer<dType> {  // src/softmax.h:14-225
     ZOPH_CALL(zr_malloc(ctx, nt * sizeof(dType), (void**)&d_output_vocab_indices_01_float));
     nodes.resize(longest_sent);
     for (int i = 0; i < longest_sent; i++) nodes[i].index = i;
+    prepare_weights();
   }
   // src/softmax.hpp:926-947
   void prep_GPU_vocab_indices(int* h_output_vocab_indicies_target, int current_target_length) override {
@@ -409,7 +410,11 @@ class softmax_layer : public base_loss_layer<dType> {  // src/softmax.h:14-225
   void load_weights(std::ifstream& input) override {
     read_matrix_GPU(s_layer_info.ctx, d_D, output_vocab_size, LSTM_size, input);
     read_matrix_GPU(s_layer_info.ctx, d_b_d, output_vocab_size, 1, input);
+    prepare_weights();
   }
+  // No counterpart in the reference: snapshots d_D into the layout the matrix cores read fastest.  Called after
+  // init_loss_layer and load_weights; call again by hand after writing to d_D.
+  void prepare_weights() { ZOPH_CALL(zr_softmax_prepare(s_layer_info.ctx, d_D, output_vocab_size, LSTM_size)); }
 };
 
 // ------------------------------------------------------------------------------------------------ LSTM nodes
