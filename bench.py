@@ -26,6 +26,12 @@ import numpy as np  # noqa: E402
 PEAK_FP32_MFMA_TFLOPS = 157.3  # MI355X dense fp32 matrix peak
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E peak
 
+# HBM bytes per full-diagonal launch of lstm_fused_kernel on the headline workload, from two rocprofv3 --pmc runs
+# (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for a plain copy of
+# known size (bench.py --calibrate-copy): FETCH_SIZE 69122.6 KiB x 1.9704 + WRITE_SIZE 6000.0 KiB x 1.0000.
+# The summary of those runs is profiles/lstm_fused_kernel_config2_hbm_traffic.txt.
+LSTM_FUSED_FULL_DIAGONAL_TRAFFIC_BYTES = int((69122.6 * 1.9704 + 6000.0 * 1.0) * 1024)
+
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
@@ -82,6 +88,19 @@ def bench_encoder(ctx, steps, warmup, H=1000, mb=128, T=50, V=50000, L=4):
     # keep references alive until here
     res["_keep"] = (layers, d_embed, d_nn, d_m, z, h_all, c_all)
     return res
+
+
+def measure_full_diagonal_launch(ctx, steps, warmup, H=1000, mb=128, T=50, V=50000, L=4):
+    """Average duration of one full-diagonal launch of lstm_fused_kernel (L units: one node of every layer), the
+    launch that dominates the encoder sweep: a sweep over 2T time steps runs exactly T more of them than a sweep over
+    T (the ramp launches at both ends are the same), so the difference of the two event-timed regions / T is its
+    duration, launch gaps included."""
+    long_run = bench_encoder(ctx, steps, warmup, H=H, mb=mb, T=2 * T, V=V, L=L)
+    long_run.pop("_keep")
+    short_run = bench_encoder(ctx, steps, warmup, H=H, mb=mb, T=T, V=V, L=L)
+    short_run.pop("_keep")
+    us = (long_run["event_ms"] - short_run["event_ms"]) * 1e3 / (steps * T)
+    return us, L * 2.0 * 4 * H * mb * (2 * H)
 
 
 def bench_decoder_step(ctx, steps, warmup, H=1000, mb=128, S=50, V=50000, L=4, D=50):
@@ -259,9 +278,10 @@ def main():
     enc.pop("_keep")
     ms_per_step = enc["event_ms"] / args.steps
     tokens_per_s = enc["tokens_per_step"] / (ms_per_step * 1e-3)
-    achieved_tflops = enc["flops_per_launch"] / (enc["avg_launch_us"] * 1e-6) / 1e12
-    log("encoder: %.3f ms/step (wall %.3f), %.0f tokens/s, %.1f TFLOP/s" %
-        (ms_per_step, enc["wall_ms"] / args.steps, tokens_per_s, achieved_tflops))
+    launch_us, launch_flops = measure_full_diagonal_launch(ctx, max(2, args.steps // 4), 1)
+    achieved_tflops = launch_flops / (launch_us * 1e-6) / 1e12
+    log("encoder: %.3f ms/step (wall %.3f), %.0f tokens/s; full-diagonal launch %.2f us, %.1f TFLOP/s" %
+        (ms_per_step, enc["wall_ms"] / args.steps, tokens_per_s, launch_us, achieved_tflops))
 
     extra = {}
     if not args.no_extra:
@@ -296,8 +316,11 @@ def main():
                    "tokens_per_step": enc["tokens_per_step"], "launches_per_step": enc["launches_per_step"]},
         "roofline": {"bound": "mfma", "kernel": "lstm_fused_kernel", "achieved": round(achieved_tflops, 2),
                      "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved_tflops / PEAK_FP32_MFMA_TFLOPS, 4),
-                     "traffic": None, "avg_launch_us": round(enc["avg_launch_us"], 2),
-                     "flops_per_launch": enc["flops_per_launch"]},
+                     "traffic": LSTM_FUSED_FULL_DIAGONAL_TRAFFIC_BYTES, "traffic_unit": "bytes per launch",
+                     "launch": "full diagonal: 4 units (one node of each layer), 256 workgroups",
+                     "avg_launch_us": round(launch_us, 2), "flops_per_launch": launch_flops,
+                     "algorithmic_bytes_per_launch": 4 * (2 * 4 * 1000 * 1000 + 3 * 1000 * 128 + 2 * 1000 * 128) * 4,
+                     "whole_sweep_avg_launch_us": round(enc["avg_launch_us"], 2)},
         "cpu_baseline": cpu,
         "extra": extra,
     }
