@@ -100,6 +100,14 @@ int zr_embed_gather(zr_ctx* ctx, const float* d_W, int H, int V, const int* d_id
  * d_M/d_Wh/d_Q/d_b: arrays of 4 device pointers in gate order i,f,c,o; d_Q may be NULL (no feed-input). */
 int zr_lstm_pack_weights(zr_ctx* ctx, const float* const d_M[4], const float* const d_Wh[4],
                          const float* const d_Q[4], const float* const d_b[4], int H, zr_lstm_weights** out);
+/* Reduced-precision variant (no counterpart in the reference, whose only overloads are float and double,
+ * src/BZ_CUDA_UTIL.h:691-703): the eight / twelve matrices are stored as bf16 (round to nearest even; exact when the
+ * caller's values are already bf16-representable), biases stay fp32.  zr_lstm_step and zr_lstm_stack_forward take
+ * the result like any other packed layer: products run on the bf16 matrix cores with each fp32 activation split into
+ * two bf16 terms, accumulation and the cell state are fp32.  Against the fp32 path on the same (rounded) weights
+ * the results agree within 1e-4 relative.  Requires H % 16 == 0 and 16-byte aligned activations. */
+int zr_lstm_pack_weights_bf16(zr_ctx* ctx, const float* const d_M[4], const float* const d_Wh[4],
+                              const float* const d_Q[4], const float* const d_b[4], int H, zr_lstm_weights** out);
 int zr_lstm_weights_destroy(zr_ctx* ctx, zr_lstm_weights* w);
 
 /* One node forward step: LSTM_IH_Node::forward_prop_GPU after the gather (src/LSTM.hpp:133-399) and

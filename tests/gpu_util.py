@@ -26,17 +26,27 @@ def assert_close(got, want, rel=REL, floor=FLOOR, what=""):
                              % (what, int(bad.sum()), bad.size, i, got[i], want[i], err[i], bound[i]))
 
 
+def round_bf16(a):
+    """fp32 array rounded to the nearest bf16-representable value (ties to even), returned as fp32, same layout."""
+    a = np.asarray(a, dtype=np.float32)
+    if not (a.flags.c_contiguous or a.flags.f_contiguous):
+        a = np.ascontiguousarray(a)
+    u = a.view(np.uint32).astype(np.uint64)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+    return u.astype(np.uint32).view(np.float32)
+
+
 class Layer:
     """One LSTM layer's parameters on the device, packed for zr_lstm_step."""
 
-    def __init__(self, ctx, ly):
+    def __init__(self, ctx, ly, bf16=False):
         self.ctx = ctx
         self.H = ly["M"][0].shape[0]
         self.M = [ctx.array(m, np.float32) for m in ly["M"]]
         self.Wh = [ctx.array(m, np.float32) for m in ly["Wh"]]
         self.b = [ctx.array(v, np.float32) for v in ly["b"]]
         self.Q = [ctx.array(m, np.float32) for m in ly["Q"]] if "Q" in ly else None
-        self.w = ctx.lstm_pack(self.M, self.Wh, self.b, self.H, self.Q)
+        self.w = ctx.lstm_pack(self.M, self.Wh, self.b, self.H, self.Q, bf16=bf16)
 
     def close(self):
         self.ctx.lstm_weights_destroy(self.w)

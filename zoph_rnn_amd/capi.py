@@ -25,7 +25,7 @@ ZR_SOFTMAX_LOGPROB = 1
 SYMBOLS = [
     "zr_ctx_create", "zr_ctx_destroy", "zr_ctx_sync", "zr_ctx_set_stream", "zr_ctx_set_option", "zr_last_error",
     "zr_version", "zr_timer_start", "zr_timer_stop", "zr_malloc", "zr_free", "zr_h2d", "zr_d2h", "zr_d2d", "zr_memset_zero", "zr_vocab_prep",
-    "zr_vocab_prep_softmax", "zr_embed_gather", "zr_lstm_pack_weights", "zr_lstm_weights_destroy", "zr_lstm_step",
+    "zr_vocab_prep_softmax", "zr_embed_gather", "zr_lstm_pack_weights", "zr_lstm_pack_weights_bf16", "zr_lstm_weights_destroy", "zr_lstm_step",
     "zr_lstm_gates", "zr_lstm_stack_forward", "zr_gemm", "zr_softmax_prepare", "zr_softmax_release", "zr_softmax_forward", "zr_softmax_logprob_f64",
     "zr_softmax_loss", "zr_attn_create", "zr_attn_destroy", "zr_attn_step", "zr_gather_columns",
     "zr_broadcast_column", "zr_beam_create", "zr_beam_destroy", "zr_beam_init", "zr_beam_expand", "zr_beam_finish",
@@ -170,10 +170,11 @@ class Context:
         _chk(load().zr_embed_gather(self.h, _vp(d_W), C.c_int(H), C.c_int(V), _vp(d_ids), C.c_int(mb), _vp(d_x)))
 
     # ---- A3-A5
-    def lstm_pack(self, M, Wh, b, H, Q=None):
+    def lstm_pack(self, M, Wh, b, H, Q=None, bf16=False):
         w = C.c_void_p()
-        _chk(load().zr_lstm_pack_weights(self.h, _ptr_array(M), _ptr_array(Wh), _ptr_array(Q) if Q else None,
-                                         _ptr_array(b), C.c_int(H), C.byref(w)))
+        fn = load().zr_lstm_pack_weights_bf16 if bf16 else load().zr_lstm_pack_weights
+        _chk(fn(self.h, _ptr_array(M), _ptr_array(Wh), _ptr_array(Q) if Q else None, _ptr_array(b), C.c_int(H),
+                C.byref(w)))
         return w
 
     def lstm_weights_destroy(self, w):

@@ -553,7 +553,27 @@ __global__ void __launch_bounds__(256) pack4_kernel(const float* __restrict__ sr
   dst[i] = (row < M && k < K) ? src[row + (long long)k * ld] : 0.0f;
 }
 
+__global__ void __launch_bounds__(256) pack8_bf16_kernel(const float* __restrict__ src, int M, int K, long long ld,
+                                                         int ldp, int kp, unsigned short* __restrict__ dst) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (long long)kp * ldp) return;
+  const int k8 = (int)(i & 7);
+  const long long t = i >> 3;
+  const int row = (int)(t % ldp);
+  const int k = (int)(t / ldp) * 8 + k8;
+  const float v = (row < M && k < K) ? src[row + (long long)k * ld] : 0.0f;
+  dst[i] = __builtin_bit_cast(unsigned short, (__bf16)v);
+}
+
 }  // namespace
+
+int zr_pack8_bf16_launch(zr_ctx* ctx, const float* src, int M, int K, long long ld, int ldp, int kp,
+                         unsigned short* dst) {
+  const long long total = (long long)kp * ldp;
+  pack8_bf16_kernel<<<(unsigned)((total + 255) / 256), 256, 0, ctx->stream>>>(src, M, K, ld, ldp, kp, dst);
+  ZR_LAUNCH_CHECK("pack8_bf16_kernel");
+  return ZR_OK;
+}
 
 int zr_pack4_launch(zr_ctx* ctx, const float* src, int M, int K, long long ld, int ldp, int kp, float* dst) {
   const long long total = (long long)kp * ldp;

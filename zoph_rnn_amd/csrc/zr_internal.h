@@ -104,17 +104,22 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d);
 // Packs one M x K column-major matrix (leading dimension ld) into the k-interleaved layout [kp/4][ldp][4] with
 // zero padding (ldp >= M a multiple of 32, kp >= K a multiple of 8).  dst holds kp*ldp floats.
 int zr_pack4_launch(zr_ctx* ctx, const float* src, int M, int K, long long ld, int ldp, int kp, float* dst);
+// Same for the bf16 layout [kp/8][ldp][8] (round to nearest even); kp a multiple of 16.  dst holds kp*ldp elements.
+int zr_pack8_bf16_launch(zr_ctx* ctx, const float* src, int M, int K, long long ld, int ldp, int kp,
+                         unsigned short* dst);
 // number of 32-row partial blocks the SOFTMAX_PARTIAL epilogue writes for M rows
 static inline int zr_softmax_partial_blocks(int M) { return (M + 31) / 32; }
 
 struct zr_lstm_weights {
   int H;
   int nseg;        // 2 (M, Wh) or 3 (+Q)
+  int bf16;        // 0: fp32 matrices, k-interleaved by 4; 1: bf16 matrices, k-interleaved by 8
   int ldw;         // H rounded up to 32: rows per packed k-block (rows >= H hold zeros)
-  int kp;          // H rounded up to 8: packed K extent (k >= H hold zeros)
-  // [nseg][4] matrices, each packed as [kp/4][ldw][4]: element (row, k) at ((k/4)*ldw + row)*4 + k%4.  A 32-row
-  // tile of four consecutive k is 512 contiguous, 128-byte aligned bytes, read with one 16-byte load per lane.
-  float* d_W;
+  int kp;          // packed K extent: H rounded up to 8 (fp32) or 16 (bf16); k >= H hold zeros
+  // [nseg][4] matrices.  fp32: each [kp/4][ldw][4], element (row, k) at ((k/4)*ldw + row)*4 + k%4.
+  // bf16: each [kp/8][ldw][8], element (row, k) at ((k/8)*ldw + row)*8 + k%8 (2-byte elements).
+  // A 32-row tile of one k-block is 512 contiguous, 128-byte aligned bytes, read with one 16-byte load per lane.
+  void* d_W;
   float* d_bias;   // [4][H]
 };
 

@@ -19,7 +19,7 @@ namespace {
 constexpr int kMaxUnits = 8;
 
 struct LstmUnit {
-  const float* W;           // [nseg][4] packed matrices, [kp/4][ldw][4] each
+  const void* W;            // [nseg][4] packed matrices: fp32 [kp/4][ldw][4] or bf16 [kp/8][ldw][8] each
   const float* bias;        // [4][H]
   const float* in[3];       // segment inputs, H x mb (ld = H)
   const float* inp[3];      // optional copies of the same inputs packed as [H/4][mb][4] (null: use in[])
@@ -37,6 +37,7 @@ struct LstmUnit {
 struct LstmLaunch {
   LstmUnit u[kMaxUnits];
   int n_units;
+  int bf16;                 // the weights of every unit are bf16 (zr_lstm_weights::bf16)
   int nseg_max;             // largest nseg among the units
   int H, mb;
   int ldw, kp;              // packed weight extents: rows per k-block (H up to 32), K (H up to 8), zero filled
@@ -56,7 +57,7 @@ constexpr int lstm_prefetch_depth(int tn, int ks) {
 #endif
 }
 
-template <int TN, int KS, bool VEC>
+template <int TN, int KS, bool VEC, bool BF16 = false>
 __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
   __shared__ float red[KS * TN * 16 * 64];
   // Workgroup ids congruent modulo 8 run on the same XCD (round-robin dispatch) and share its L2.  Each XCD gets
@@ -114,28 +115,50 @@ __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
     mask_v[i] = (float)U.mask01[n];
   }
 
-  const long long HH = (long long)L.kp * L.ldw;
+  const long long HH = (long long)L.kp * L.ldw;  // elements per packed matrix
   for (int s = 0; s < U.nseg; ++s) {
-    const float* wbase[4];
-    unsigned woff[4];
-    const float* xcol[TN];
+    if constexpr (BF16) {
+      const unsigned short* wbase[4];
+      unsigned woff[4];
+      const float* xcol[TN];
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      wbase[g] = U.W + ((long long)s * 4 + g) * HH;
-      woff[g] = (unsigned)(4 * j + 4 * half * L.ldw);  // j < ldw: padded rows are zeros
-    }
-#pragma unroll
-    for (int tn = 0; tn < TN; ++tn) {
-      long long c = cols[tn];
-      if (s == 0 && U.gather_ids) {
-        int idv = U.gather_ids[cols[tn]];
-        idv = idv < 0 ? 0 : (idv >= U.V ? U.V - 1 : idv);
-        c = idv;
+      for (int g = 0; g < 4; ++g) {
+        wbase[g] = (const unsigned short*)U.W + ((long long)s * 4 + g) * HH;
+        woff[g] = (unsigned)(8 * j + 8 * half * L.ldw);
       }
-      xcol[tn] = (VEC && U.inp[s]) ? U.inp[s] + 4LL * cols[tn] + 4LL * half * L.mb : U.in[s] + c * H + 4 * half;
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) {
+        long long c = cols[tn];
+        if (s == 0 && U.gather_ids) {
+          int idv = U.gather_ids[cols[tn]];
+          idv = idv < 0 ? 0 : (idv >= U.V ? U.V - 1 : idv);
+          c = idv;
+        }
+        xcol[tn] = U.in[s] + c * H + 8 * half;
+      }
+      zr_mma_segment_bf16<4, TN, KS, (TN == 1 ? 6 : 4)>(acc, wbase, woff, (long long)L.ldw, xcol, H, kslice);
+    } else {
+      const float* wbase[4];
+      unsigned woff[4];
+      const float* xcol[TN];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        wbase[g] = (const float*)U.W + ((long long)s * 4 + g) * HH;
+        woff[g] = (unsigned)(4 * j + 4 * half * L.ldw);  // j < ldw: padded rows are zeros
+      }
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) {
+        long long c = cols[tn];
+        if (s == 0 && U.gather_ids) {
+          int idv = U.gather_ids[cols[tn]];
+          idv = idv < 0 ? 0 : (idv >= U.V ? U.V - 1 : idv);
+          c = idv;
+        }
+        xcol[tn] = (VEC && U.inp[s]) ? U.inp[s] + 4LL * cols[tn] + 4LL * half * L.mb : U.in[s] + c * H + 4 * half;
+      }
+      zr_mma_segment<4, TN, KS, lstm_prefetch_depth(TN, KS), ZR_A_PACK4, VEC>(
+          acc, wbase, woff, (long long)L.ldw, xcol, H, kslice, half, (VEC && U.inp[s]) ? L.mb : 1);
     }
-    zr_mma_segment<4, TN, KS, lstm_prefetch_depth(TN, KS), ZR_A_PACK4, VEC>(
-        acc, wbase, woff, (long long)L.ldw, xcol, H, kslice, half, (VEC && U.inp[s]) ? L.mb : 1);
   }
 
   const bool j_ok = j < H;
@@ -254,7 +277,7 @@ __global__ void __launch_bounds__(64 * NWV) lstm_lds_kernel(LstmLaunch2 P) {
     const int row = f & 31, g = (f >> 5) & 3, kb = f >> 7;
     wok_row[u] = seg_live && (f < F4_PER_CHUNK);  // rows >= H and k >= H of the packed weights are zeros
     wkb[u] = kb;
-    wsrc[u] = U.W + ((long long)(seg_live ? seg : 0) * 4 + g) * HH + 4 * (j0 + row);
+    wsrc[u] = (const float*)U.W + ((long long)(seg_live ? seg : 0) * 4 + g) * HH + 4 * (j0 + row);
   }
 
   zr_f32x16 acc[4][TN];
@@ -428,6 +451,15 @@ template <int TN, int KS>
 int launch_fused_v(zr_ctx* ctx, const LstmLaunch& L, bool vec) {
   const int groups = L.n_units * L.j_tiles;
   const int grid = ((groups + 7) / 8) * 8 * L.n_tiles;
+  if (L.bf16) {
+    if constexpr (KS == 4 && TN <= 2) {
+      lstm_fused_kernel<TN, KS, true, true><<<grid, 64 * KS, 0, ctx->stream>>>(L);
+      ZR_LAUNCH_CHECK("lstm_fused_kernel (bf16 weights)");
+      return ZR_OK;
+    } else {
+      return zr_set_error(ZR_EINVAL, "bf16 weights: no kernel for column tile %d, K split %d", TN, KS);
+    }
+  }
   if (vec)
     lstm_fused_kernel<TN, KS, true><<<grid, 64 * KS, 0, ctx->stream>>>(L);
   else
@@ -475,6 +507,12 @@ int launch_fused(zr_ctx* ctx, LstmLaunch& L, bool vec) {
   // a workgroup on (nearly) every CU -- a full diagonal of an encoder does.  A single node (a decoder step) gives
   // it only ceil(H/32) * ceil(mb/64) workgroups; there the LDS / split-K kernel spreads the same node over ~256
   // workgroups.  It needs 16-byte aligned operands and a batch wide enough for its 128-column tile.
+  if (L.bf16) {
+    ZR_CHECK_ARG(vec && L.H % 16 == 0, "bf16 weights need H %% 16 == 0 and 16-byte aligned activations (H = %d)", L.H);
+    const long long wg2 = (long long)L.n_units * L.j_tiles * ((n32 + 1) / 2);
+    L.n_tiles = (n32 >= 2 && wg2 >= 200) ? (n32 + 1) / 2 : n32;
+    return (n32 >= 2 && wg2 >= 200) ? launch_fused_v<2, 4>(ctx, L, vec) : launch_fused_v<1, 4>(ctx, L, vec);
+  }
   int kernel = ctx->lstm_kernel;
   if (L.preact) kernel = 1;  // only the register-streaming kernel stores raw pre-activations
   if (kernel == 0) {
@@ -511,40 +549,47 @@ inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
 extern "C" {
 
-int zr_lstm_pack_weights(zr_ctx* ctx, const float* const d_M[4], const float* const d_Wh[4],
-                         const float* const d_Q[4], const float* const d_b[4], int H, zr_lstm_weights** out) {
+static int pack_weights(zr_ctx* ctx, const char* who, bool bf16, const float* const d_M[4],
+                        const float* const d_Wh[4], const float* const d_Q[4], const float* const d_b[4], int H,
+                        zr_lstm_weights** out) {
   int rc = zr_bind_device(ctx);
   if (rc) return rc;
-  ZR_CHECK_ARG(out != nullptr, "zr_lstm_pack_weights: out is null");
+  ZR_CHECK_ARG(out != nullptr, "%s: out is null", who);
   *out = nullptr;
-  ZR_CHECK_ARG(H > 0, "zr_lstm_pack_weights: H = %d", H);
-  ZR_CHECK_ARG(d_M && d_Wh && d_b, "zr_lstm_pack_weights: null pointer array");
+  ZR_CHECK_ARG(H > 0, "%s: H = %d", who, H);
+  ZR_CHECK_ARG(!bf16 || H % 16 == 0, "%s: H = %d is not a multiple of 16", who, H);
+  ZR_CHECK_ARG(d_M && d_Wh && d_b, "%s: null pointer array", who);
   for (int g = 0; g < 4; ++g) {
-    ZR_CHECK_ARG(d_M[g] && d_Wh[g] && d_b[g], "zr_lstm_pack_weights: null matrix for gate %d", g);
-    ZR_CHECK_ARG(!d_Q || d_Q[g], "zr_lstm_pack_weights: null Q for gate %d", g);
+    ZR_CHECK_ARG(d_M[g] && d_Wh[g] && d_b[g], "%s: null matrix for gate %d", who, g);
+    ZR_CHECK_ARG(!d_Q || d_Q[g], "%s: null Q for gate %d", who, g);
   }
   const int nseg = d_Q ? 3 : 2;
   const int ldw = (H + 31) / 32 * 32;
-  const int kp = (H + 7) / 8 * 8;
+  const int kp = bf16 ? (H + 15) / 16 * 16 : (H + 7) / 8 * 8;
   const size_t HH = (size_t)kp * ldw;
+  const size_t esize = bf16 ? sizeof(unsigned short) : sizeof(float);
   zr_lstm_weights* w = new zr_lstm_weights();
   w->H = H;
+  w->bf16 = bf16 ? 1 : 0;
   w->ldw = ldw;
   w->kp = kp;
   w->nseg = nseg;
   w->d_W = nullptr;
   w->d_bias = nullptr;
-  if (hipMalloc((void**)&w->d_W, sizeof(float) * HH * 4 * nseg) != hipSuccess ||
+  if (hipMalloc((void**)&w->d_W, esize * HH * 4 * nseg) != hipSuccess ||
       hipMalloc((void**)&w->d_bias, sizeof(float) * 4 * (size_t)H) != hipSuccess) {
     (void)hipGetLastError();
     if (w->d_W) (void)hipFree(w->d_W);
     delete w;
-    return zr_set_error(ZR_ENOMEM, "zr_lstm_pack_weights: allocation failed (H = %d, nseg = %d)", H, nseg);
+    return zr_set_error(ZR_ENOMEM, "%s: allocation failed (H = %d, nseg = %d)", who, H, nseg);
   }
   for (int g = 0; g < 4; ++g) {
     const float* segs[3] = {d_M[g], d_Wh[g], d_Q ? d_Q[g] : nullptr};
     for (int s = 0; s < nseg; ++s) {
-      if (zr_pack4_launch(ctx, segs[s], H, H, H, ldw, kp, w->d_W + ((size_t)s * 4 + g) * HH) != ZR_OK) {
+      const size_t off = ((size_t)s * 4 + g) * HH;
+      rc = bf16 ? zr_pack8_bf16_launch(ctx, segs[s], H, H, H, ldw, kp, (unsigned short*)w->d_W + off)
+                : zr_pack4_launch(ctx, segs[s], H, H, H, ldw, kp, (float*)w->d_W + off);
+      if (rc != ZR_OK) {
         (void)hipFree(w->d_W);
         (void)hipFree(w->d_bias);
         delete w;
@@ -557,11 +602,21 @@ int zr_lstm_pack_weights(zr_ctx* ctx, const float* const d_M[4], const float* co
       (void)hipFree(w->d_W);
       (void)hipFree(w->d_bias);
       delete w;
-      return zr_set_error(ZR_EHIP, "zr_lstm_pack_weights: bias copy failed: %s", hipGetErrorString(e));
+      return zr_set_error(ZR_EHIP, "%s: bias copy failed: %s", who, hipGetErrorString(e));
     }
   }
   *out = w;
   return ZR_OK;
+}
+
+int zr_lstm_pack_weights(zr_ctx* ctx, const float* const d_M[4], const float* const d_Wh[4],
+                         const float* const d_Q[4], const float* const d_b[4], int H, zr_lstm_weights** out) {
+  return pack_weights(ctx, "zr_lstm_pack_weights", false, d_M, d_Wh, d_Q, d_b, H, out);
+}
+
+int zr_lstm_pack_weights_bf16(zr_ctx* ctx, const float* const d_M[4], const float* const d_Wh[4],
+                              const float* const d_Q[4], const float* const d_b[4], int H, zr_lstm_weights** out) {
+  return pack_weights(ctx, "zr_lstm_pack_weights_bf16", true, d_M, d_Wh, d_Q, d_b, H, out);
 }
 
 int zr_lstm_weights_destroy(zr_ctx* ctx, zr_lstm_weights* w) {
@@ -596,6 +651,7 @@ int zr_lstm_step(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_in, const
   L.mb = mb;
   L.ldw = w->ldw;
   L.kp = w->kp;
+  L.bf16 = w->bf16;
   L.clip = clip_threshold;
   LstmUnit& U = L.u[0];
   U.W = w->d_W;
@@ -641,6 +697,7 @@ int zr_lstm_stack_forward(zr_ctx* ctx, int nl, const zr_lstm_weights* const laye
   bool vec = (H > 0) && (H % 4 == 0) && aligned16(d_embed);
   for (int l = 0; l < nl; ++l) {
     ZR_CHECK_ARG(layers[l] && layers[l]->H == H, "zr_lstm_stack_forward: layer %d missing or of different size", l);
+    ZR_CHECK_ARG(layers[l]->bf16 == layers[0]->bf16, "zr_lstm_stack_forward: layers mix fp32 and bf16 weights");
     ZR_CHECK_ARG(d_h0[l] && d_c0[l] && d_h_all[l] && d_c_all[l], "zr_lstm_stack_forward: null state for layer %d", l);
     vec = vec && aligned16(d_h0[l]) && aligned16(d_h_all[l]);
   }
@@ -649,7 +706,7 @@ int zr_lstm_stack_forward(zr_ctx* ctx, int nl, const zr_lstm_weights* const laye
   // two consumers on the next diagonal, (l+1, t) and (l, t+1), then fetch activations with contiguous 16-byte
   // loads.  The buffer written on diagonal d is read on d+1 only and overwritten on d+2.
   float* hp_buf = nullptr;
-  if (vec && H % 8 == 0) {
+  if (vec && H % 8 == 0 && !layers[0]->bf16) {
     void* p = nullptr;
     rc = zr_ctx_scratch(ctx, 1, sizeof(float) * 2 * (size_t)nl * n, &p);
     if (rc) return rc;
@@ -663,6 +720,7 @@ int zr_lstm_stack_forward(zr_ctx* ctx, int nl, const zr_lstm_weights* const laye
     L.mb = mb;
     L.ldw = layers[0]->ldw;
     L.kp = layers[0]->kp;
+    L.bf16 = layers[0]->bf16;
     L.clip = clip_threshold;
     int nu = 0;
     for (int l = 0; l < nl; ++l) {

@@ -286,4 +286,111 @@ __device__ __forceinline__ void zr_half_wave_softmax_stats(const float (&v)[G], 
   for (int g = 0; g < G; ++g) se[g] += __shfl_xor(se[g], 16, 64);
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// bf16-weight variant of the contraction core (v_mfma_f32_32x32x16_bf16, 16 k per instruction).
+//
+// Weights are stored as bf16, k-interleaved in blocks of 8: element (row, k) at ((k/8)*lda + row)*8 + k%8 (lda =
+// rows rounded up to 32, K a multiple of 16, pads zero), so a lane's operand for one instruction -- 8 consecutive k
+// of its row -- is one 16-byte load and a half-wave reads 512 contiguous bytes.  Half-wave 0 takes k0..k0+7,
+// half-wave 1 k0+8..k0+15.
+// Activations stay fp32 in memory.  Each value is split in registers into two bf16 terms, x = hi + lo with
+// hi = bf16(x) and lo = bf16(x - hi), and both are multiplied with the same weight operand: the products are exact
+// in fp32, accumulation is fp32, and the only error beyond an fp32 contraction is the 2^-17 relative residue of
+// the split.  Two bf16 instructions replace eight fp32 ones.
+//   woff[tm]:  8*row + 8*half*lda   (bf16 elements)
+//   xcol[tn]:  this lane's activation column advanced by 8*half
+// ---------------------------------------------------------------------------------------------------------
+enum { ZR_A_PACK8_BF16 = 3 };
+typedef __bf16 zr_bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 zr_bf16x2 __attribute__((ext_vector_type(2)));
+typedef unsigned zr_u32x4 __attribute__((ext_vector_type(4)));
+
+// (x0, x1) -> packed bf16 pairs hi and lo with x = hi + lo up to 2^-17 |x|
+__device__ __forceinline__ void zr_split_bf16_pair(float x0, float x1, unsigned& hi, unsigned& lo) {
+  zr_bf16x2 h;
+  h[0] = (__bf16)x0;
+  h[1] = (__bf16)x1;
+  const unsigned hu = __builtin_bit_cast(unsigned, h);
+  const float h0 = __uint_as_float(hu << 16), h1 = __uint_as_float(hu & 0xFFFF0000u);
+  zr_bf16x2 l;
+  l[0] = (__bf16)(x0 - h0);
+  l[1] = (__bf16)(x1 - h1);
+  hi = hu;
+  lo = __builtin_bit_cast(unsigned, l);
+}
+
+template <int TM, int TN>
+struct ZrFragBf16 {
+  zr_f32x4 x[TN][2];  // 8 consecutive k of this lane's column
+  zr_u32x4 w[TM];     // 8 consecutive k of this lane's row, bf16
+};
+
+template <int TM, int TN, int KS, int PF>
+__device__ __forceinline__ void zr_mma_segment_bf16(zr_f32x16 (&acc)[TM][TN], const unsigned short* const (&wbase)[TM],
+                                                    const unsigned (&woff)[TM], long long lda,
+                                                    const float* const (&xcol)[TN], int K, int kslice) {
+  const int nfull = K >> 4;  // K % 16 == 0 (checked by the host code)
+  constexpr int NS = PF + 1;
+
+  auto load_full = [&](ZrFragBf16<TM, TN>& f, int g) {
+    const int kg = g * 16;  // wave-uniform
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+      f.x[tn][0] = *(const zr_f32x4*)(xcol[tn] + kg);
+      f.x[tn][1] = *(const zr_f32x4*)(xcol[tn] + kg + 4);
+    }
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+      const unsigned short* p = wbase[tm] + (long long)kg * lda;  // uniform
+      f.w[tm] = *(const zr_u32x4*)(p + woff[tm]);
+    }
+  };
+
+  auto mma = [&](const ZrFragBf16<TM, TN>& f) {
+    zr_bf16x8 w[TM];
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) w[tm] = __builtin_bit_cast(zr_bf16x8, f.w[tm]);
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+      unsigned h0, h1, h2, h3, l0, l1, l2, l3;
+      zr_split_bf16_pair(f.x[tn][0].x, f.x[tn][0].y, h0, l0);
+      zr_split_bf16_pair(f.x[tn][0].z, f.x[tn][0].w, h1, l1);
+      zr_split_bf16_pair(f.x[tn][1].x, f.x[tn][1].y, h2, l2);
+      zr_split_bf16_pair(f.x[tn][1].z, f.x[tn][1].w, h3, l3);
+      const zr_u32x4 hi = {h0, h1, h2, h3}, lo = {l0, l1, l2, l3};
+      const zr_bf16x8 xh = __builtin_bit_cast(zr_bf16x8, hi), xl = __builtin_bit_cast(zr_bf16x8, lo);
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xh, w[tm], acc[tm][tn], 0, 0, 0);
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xl, w[tm], acc[tm][tn], 0, 0, 0);
+    }
+  };
+
+  // same branch-free software pipeline as zr_mma_segment
+  if (kslice < nfull) {
+    const int last = nfull - 1;
+    const int n_mine = (nfull - kslice + KS - 1) / KS;
+    ZrFragBf16<TM, TN> f[NS];
+#pragma unroll
+    for (int s = 0; s < PF; ++s) {
+      const int gl = kslice + s * KS;
+      load_full(f[s], gl < last ? gl : last);
+    }
+    int it = 0;
+    for (; it + NS <= n_mine; it += NS) {
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        const int gl = kslice + (it + s + PF) * KS;
+        load_full(f[(s + PF) % NS], gl < last ? gl : last);
+        mma(f[s]);
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < PF; ++s)
+      if (it + s < n_mine) mma(f[s]);
+  }
+}
+
 #endif
