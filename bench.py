@@ -40,13 +40,13 @@ def log(*a):
 class Uploaded:
     """Keeps device arrays of one LSTM layer alive next to its packed weights."""
 
-    def __init__(self, ctx, ly):
+    def __init__(self, ctx, ly, bf16=False):
         self.H = ly["M"][0].shape[0]
         self.M = [ctx.array(m) for m in ly["M"]]
         self.Wh = [ctx.array(m) for m in ly["Wh"]]
         self.b = [ctx.array(v) for v in ly["b"]]
         self.Q = [ctx.array(m) for m in ly["Q"]] if "Q" in ly else None
-        self.w = ctx.lstm_pack(self.M, self.Wh, self.b, self.H, self.Q)
+        self.w = ctx.lstm_pack(self.M, self.Wh, self.b, self.H, self.Q, bf16=bf16)
 
 
 def time_region(ctx, fn, steps, warmup):
@@ -103,12 +103,12 @@ def measure_full_diagonal_launch(ctx, steps, warmup, H=1000, mb=128, T=50, V=500
     return us, L * 2.0 * 4 * H * mb * (2 * H)
 
 
-def bench_decoder_step(ctx, steps, warmup, H=1000, mb=128, S=50, V=50000, L=4, D=50):
+def bench_decoder_step(ctx, steps, warmup, H=1000, mb=128, S=50, V=50000, L=4, D=50, bf16=False):
     """Config 3: gather, 4 LSTM layers (feed-input on layer 0), attention (D >= S: every source position has a
     slot), full softmax to probabilities."""
     from zoph_rnn_amd import capi, synth
     c = synth.decoder_config(H=H, mb=mb, S=S, V=V, L=L)
-    layers = [Uploaded(ctx, ly) for ly in c["layers"]]
+    layers = [Uploaded(ctx, ly, bf16=bf16) for ly in c["layers"]]
     d_embed, d_ids = ctx.array(c["embed"]), ctx.array(c["ids"])
     d_mask = ctx.array(np.ones(mb, np.int32))
     d_hp = [ctx.array(a) for a in c["h_prev"]]
@@ -119,7 +119,9 @@ def bench_decoder_step(ctx, steps, warmup, H=1000, mb=128, S=50, V=50000, L=4, D
     attn = ctx.attn_create(H, mb, D, aw["W_a"], aw["W_p"], aw["v_p"], aw["out_bias"], aw["W_c1"], aw["W_c2"], tables)
     d_bi = ctx.array(c["batch_info"])
     dD, dbd = ctx.array(c["D"]), ctx.array(c["b_d"])
-    ctx.softmax_prepare(dD, V, H)  # one-time snapshot of D in the matrix cores' layout, outside the timed region
+    ctx.softmax_prepare(dD, V, H, bf16=bf16)  # one-time snapshot of D in the matrix cores' layout, not timed
+    if bf16:
+        ctx.attn_use_bf16_weights(attn)
     d_x = ctx.empty((H, mb))
     d_h = [ctx.empty((H, mb)) for _ in range(L)]
     d_c = [ctx.empty((H, mb)) for _ in range(L)]
@@ -156,6 +158,7 @@ def bench_decoder_step(ctx, steps, warmup, H=1000, mb=128, S=50, V=50000, L=4, D
     res.update(parts)
     res["softmax_gemm_plus_normalise_tflops"] = round(2.0 * V * H * mb / (parts["softmax_us"] * 1e-6) / 1e12, 2)
     ctx.attn_destroy(attn)
+    ctx.softmax_release(dD)
     return res
 
 
@@ -288,6 +291,10 @@ def main():
         extra["config3_decoder_step"] = {k: (round(v, 4) if isinstance(v, float) else v)
                                          for k, v in bench_decoder_step(ctx, args.steps, args.warmup).items()}
         log("config3:", extra["config3_decoder_step"])
+        c5 = bench_decoder_step(ctx, max(3, args.steps // 2), 2, H=2000, mb=256, V=80000, bf16=True)
+        c5["weights"] = "bf16 storage (LSTM, attention projections, output layer), fp32 activations split in two bf16 terms, fp32 accumulation"
+        extra["config5_decoder_step_bf16_weights"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in c5.items()}
+        log("config5:", extra["config5_decoder_step_bf16_weights"])
         extra["hbm_kernels"] = bench_hbm_kernels(ctx, args.steps)
         extra["config4_beam_decode"] = bench_beam_decode(ctx, args.steps)
         log("config4:", extra["config4_beam_decode"])

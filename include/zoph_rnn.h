@@ -161,6 +161,9 @@ int zr_gemm(zr_ctx* ctx, int trans_a, int M, int N, int K, const float* d_A, int
  * copy.  The copy is a snapshot: call again after changing D (it re-packs in place), and call zr_softmax_release
  * before freeing d_D.  At most 8 matrices per context.  Results are the same with or without it. */
 int zr_softmax_prepare(zr_ctx* ctx, const float* d_D, int V, int H);
+/* Same, with the copy stored as bf16 (round to nearest even; half the bytes to stream): the reduced-precision
+ * variant of the output layer, see zr_lstm_pack_weights_bf16 for the arithmetic.  Requires H % 16 == 0. */
+int zr_softmax_prepare_bf16(zr_ctx* ctx, const float* d_D, int V, int H);
 int zr_softmax_release(zr_ctx* ctx, const float* d_D);
 
 #define ZR_SOFTMAX_PROB 0    /* probabilities: softmax_layer::get_distribution_GPU (src/softmax.hpp:514-632) */
@@ -192,6 +195,11 @@ typedef struct zr_attn zr_attn;
 int zr_attn_create(zr_ctx* ctx, int H, int mb, int D, const float* d_W_a, const float* d_W_p, const float* d_v_p,
                    const float* d_out_bias, const float* d_W_c1, const float* d_W_c2,
                    const float* const* h_hs_table, int longest_sent, zr_attn** out);
+/* Reduced-precision variant (no counterpart in the reference): snapshots W_a, W_p, W_c_p1 and W_c_p2 as bf16 in the
+ * matrix cores' layout; later zr_attn_step calls multiply with the snapshots (bf16 matrix cores, fp32 activations
+ * split in two bf16 terms, fp32 accumulation).  v_p, the bias and everything element-wise stay fp32.  Call again
+ * after changing the matrices.  Requires H % 16 == 0. */
+int zr_attn_use_bf16_weights(zr_ctx* ctx, zr_attn* a);
 int zr_attn_destroy(zr_ctx* ctx, zr_attn* a);
 /* attention_node::forward_prop (src/attention_node.hpp:73-394), single-source branch: p_t, window, scores
  * h_s . (W_a^T h), the reference's softmax (max initialised to 0) times the Gaussian prior, context and

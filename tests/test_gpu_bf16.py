@@ -146,3 +146,160 @@ def test_config5_shape_lstm_node(ctx):
     close(got["c"][:, cols], want["c"], "config-5 node c")
     assert np.all(np.isfinite(got["h"])) and np.all(np.abs(got["h"]) <= 1.0)
     layer.close()
+
+
+@pytest.mark.parametrize("V,H,mb", [(211, 16, 6), (1003, 48, 70), (4099, 64, 33), (9000, 112, 130), (8200, 96, 200)])
+def test_softmax_bf16_output_layer(ctx, V, H, mb):
+    """Output matrix registered as bf16 (zr_softmax_prepare_bf16): logits, probabilities, log-probs and the loss
+    against the oracle on the bf16-rounded matrix; covers the generic tiles (V < 8192) and the row-range kernel."""
+    g = synth.rng(77, V + mb)
+    D = np.asfortranarray(round_bf16(U(g, (V, H), -0.5, 0.5)))
+    bd, h = U(g, (V,), -1, 1), U(g, (H, mb), -1, 1)
+    dD, dbd, dh = ctx.array(D), ctx.array(bd), ctx.array(h)
+    ctx.softmax_prepare(dD, V, H, bf16=True)
+    d_p, d_lp, d_scr = ctx.empty((V, mb)), ctx.empty((V, mb)), ctx.empty((V, mb))
+    ctx.softmax_forward(dD, dbd, V, H, dh, mb, capi.ZR_SOFTMAX_PROB, d_p, d_scr)
+    ctx.softmax_forward(dD, dbd, V, H, dh, mb, capi.ZR_SOFTMAX_LOGPROB, d_lp)
+    ctx.sync()
+    logits = o.softmax_logits(D, bd, h)
+    close(d_scr.get(), logits, "logits")
+    P = d_p.get()
+    assert_close(P, o.softmax_dist(logits), floor=1e-6, what="probabilities")
+    assert np.allclose(P.sum(axis=0, dtype=np.float64), 1.0, atol=1e-5)
+    close(d_lp.get(), o.softmax_logprob_f64(logits), "log-probs")
+    tgt = g.integers(0, V, size=mb).astype(np.int32)
+    mask = (g.random(mb) > 0.3).astype(np.int32)
+    got = ctx.softmax_loss(dD, dbd, V, H, dh, mb, ctx.array(tgt), ctx.array(mask), d_scr)
+    assert got == pytest.approx(o.softmax_loss(o.softmax_logprob_f64(logits), tgt, mask), rel=1e-5, abs=1e-4)
+    ctx.softmax_release(dD)
+
+
+def test_config5_shape_output_layer(ctx):
+    """V=80000, H=2000, minibatch 256 with a bf16 output matrix: column sums, arg-max consistency and sampled columns."""
+    g = synth.rng(78, 1)
+    V, H, mb = 80000, 2000, 256
+    D = np.asfortranarray(round_bf16(U(g, (V, H), -0.08, 0.08)))
+    bd = U(g, (V,), -0.08, 0.08)
+    h = np.tanh(U(g, (H, mb), -1, 1))
+    dD, dbd = ctx.array(D), ctx.array(bd)
+    ctx.softmax_prepare(dD, V, H, bf16=True)
+    d_p, d_scr = ctx.empty((V, mb)), ctx.empty((V, mb))
+    ctx.softmax_forward(dD, dbd, V, H, ctx.array(h), mb, capi.ZR_SOFTMAX_PROB, d_p, d_scr)
+    ctx.sync()
+    P, logits = d_p.get(), d_scr.get()
+    assert np.allclose(P.sum(axis=0, dtype=np.float64), 1.0, atol=1e-5)
+    assert np.array_equal(P.argmax(axis=0), logits.argmax(axis=0))
+    cols = [0, 63, 64, 200, 255]
+    want = o.softmax_logits(D, bd, np.asfortranarray(h[:, cols]))
+    close(logits[:, cols], want, "config-5 logits (sampled columns)")
+    assert_close(P[:, cols], o.softmax_dist(want), floor=1e-7, what="config-5 probabilities (sampled columns)")
+    ctx.softmax_release(dD)
+
+
+def _run_attention_bf16(ctx, w, hs, batch_info, h_t, mask, D):
+    S, H, mb = hs.shape
+    tables = [ctx.array(np.asfortranarray(hs[t])) for t in range(S)]
+    dw = {k: ctx.array(v) for k, v in w.items()}
+    a = ctx.attn_create(H, mb, D, dw["W_a"], dw["W_p"], dw["v_p"], dw["out_bias"], dw["W_c1"], dw["W_c2"], tables)
+    ctx.attn_use_bf16_weights(a)
+    Wn = 2 * D + 1
+    d_ht, d_al, d_ix, d_pt, d_cx = (ctx.empty((H, mb)), ctx.empty((mb, Wn)), ctx.empty((mb, Wn), np.int32),
+                                    ctx.empty((mb,)), ctx.empty((H, mb)))
+    ctx.attn_step(a, ctx.array(batch_info), ctx.array(h_t), ctx.array(mask), d_ht, d_al, d_ix, d_pt, d_cx)
+    ctx.sync()
+    out = {"h_tild": d_ht.get(), "alignments": d_al.get(), "indices": d_ix.get(), "p_t": d_pt.get(),
+           "c_ctx": d_cx.get()}
+    ctx.attn_destroy(a)
+    return out
+
+
+@pytest.mark.parametrize("H,mb,S,D", [(64, 6, 9, 2), (96, 40, 20, 10), (48, 33, 12, 12)])
+def test_attention_bf16_weights(ctx, H, mb, S, D):
+    g = synth.rng(79, H + S)
+    w = synth.attention_weights(g, H)
+    for k in ("W_a", "W_p", "W_c1", "W_c2"):
+        w[k] = np.asfortranarray(round_bf16(U(g, (H, H), -0.3, 0.3)))
+    hs = (g.standard_normal(size=(S, H, mb), dtype=np.float32) * np.float32(0.5))
+    lens = g.integers(1, S + 1, size=mb).astype(np.int32)
+    lens[0] = S
+    batch_info = np.concatenate([lens, S - lens]).astype(np.int32)
+    mask = (g.random(mb) > 0.15).astype(np.int32)
+    h_t = U(g, (H, mb), -1, 1)
+    want = o.attention_forward(hs_table=hs, batch_info=batch_info, h_t=h_t, mask01=mask, D=D, **w)
+    got = _run_attention_bf16(ctx, w, hs, batch_info, h_t, mask, D)
+    frac = want["p_t"] - np.floor(want["p_t"])
+    safe = (frac > 1e-3) & (frac < 1 - 1e-3)  # the window is floor(p_t) +- D: skip columns on an integer boundary
+    assert safe.sum() >= mb // 2
+    close(got["p_t"], want["p_t"], "p_t")
+    assert np.array_equal(got["indices"][safe], want["indices"][safe])
+    assert_close(got["alignments"][safe], want["alignments"][safe], floor=1e-3, what="alignments")
+    close(got["c_ctx"][:, safe], want["c_ctx"][:, safe], "context")
+    close(got["h_tild"][:, safe], want["h_tild"][:, safe], "h_tild")
+    assert np.all(got["h_tild"][:, mask == 0] == 0)
+
+
+def test_config5_decoder_step_reduced_vocab(ctx):
+    """BASELINE config 5 wiring (bf16 weights everywhere a matrix is streamed: 4 LSTM layers with feed-input,
+    attention projections, output layer) at H=2000, minibatch 256, S=50; vocabulary reduced to 2000 and 48 of the
+    256 columns checked against the oracle so that it finishes in seconds."""
+    c = synth.decoder_config(H=2000, mb=256, V=2000)
+    H, mb, S, L, V = c["H"], c["mb"], c["S"], c["L"], c["V"]
+    rb = lambda m: np.asfortranarray(round_bf16(m))
+    for ly in c["layers"]:
+        for k in ("M", "Wh", "Q"):
+            if k in ly:
+                ly[k] = [rb(m) for m in ly[k]]
+    for k in ("W_a", "W_p", "W_c1", "W_c2"):
+        c["attn"][k] = rb(c["attn"][k])
+    c["D"] = rb(c["D"])
+    mask = np.ones(mb, np.int32)
+    cols = np.arange(0, mb, 16)[:16].tolist() + list(range(224, 256))
+    sub = lambda a: np.asfortranarray(a[:, cols])
+    # HIP path, all 256 columns
+    layers = [Layer(ctx, ly, bf16=True) for ly in c["layers"]]
+    d_x = ctx.empty((H, mb))
+    ctx.embed_gather(ctx.array(c["embed"]), H, V, ctx.array(c["ids"]), mb, d_x)
+    d_mask, d_ht_prev = ctx.array(mask), ctx.array(c["h_tild_prev"])
+    d_below, outs = d_x, []
+    for l in range(L):
+        d_h, d_c = ctx.empty((H, mb)), ctx.empty((H, mb))
+        ctx.lstm_step(layers[l].w, d_below, ctx.array(c["h_prev"][l]), ctx.array(c["c_prev"][l]), d_mask, mb, d_h,
+                      d_c, d_htild=d_ht_prev if l == 0 else None)
+        outs.append((d_h, d_c))
+        d_below = d_h
+    ctx.sync()
+    # oracle on the sampled columns, layer by layer from the HIP path's own inputs
+    below = sub(o.embed_gather(c["embed"], c["ids"]))
+    for l in range(L):
+        ly = c["layers"][l]
+        r = o.lstm_step(ly["M"], ly["Wh"], ly["b"], below, sub(c["h_prev"][l]), sub(c["c_prev"][l]), mask[cols],
+                        Q=ly.get("Q"), htild=sub(c["h_tild_prev"]) if l == 0 else None)
+        close(outs[l][0].get()[:, cols], r["h"], "layer %d h" % l)
+        close(outs[l][1].get()[:, cols], r["c"], "layer %d c" % l)
+        below = sub(outs[l][0].get())
+    top_h = outs[-1][0].get()
+    D = 50
+    got_att = _run_attention_bf16(ctx, c["attn"], c["hs"], c["batch_info"], top_h, mask, D)
+    bi = c["batch_info"]
+    want_att = o.attention_forward(hs_table=np.ascontiguousarray(c["hs"][:, :, cols]),
+                                   batch_info=np.concatenate([bi[:mb][cols], bi[mb:][cols]]).astype(np.int32),
+                                   h_t=sub(top_h), mask01=mask[cols], D=D, **c["attn"])
+    frac = want_att["p_t"] - np.floor(want_att["p_t"])
+    safe = (frac > 1e-3) & (frac < 1 - 1e-3)
+    sel = np.array(cols)[safe]
+    assert np.array_equal(got_att["indices"][sel], want_att["indices"][safe])
+    assert_close(got_att["alignments"][sel], want_att["alignments"][safe], floor=1e-3, what="alignments")
+    # The scores are dot products of 2000 source-state values of size 0.5 with q = W_a^T h, so the 1e-5 absolute
+    # noise of q becomes 2e-4 on a score and on the alignment weights built from it: behind the alignment softmax
+    # the stated bound is 1e-4 absolute (1e-4 relative with a floor of 1).
+    assert_close(got_att["h_tild"][:, sel], want_att["h_tild"][:, safe], floor=1.0, what="h_tild")
+    dD = ctx.array(c["D"])
+    ctx.softmax_prepare(dD, V, H, bf16=True)
+    d_lp = ctx.empty((V, mb))
+    ctx.softmax_forward(dD, ctx.array(c["b_d"]), V, H, ctx.array(got_att["h_tild"]), mb, capi.ZR_SOFTMAX_LOGPROB, d_lp)
+    ctx.sync()
+    want_lp = o.softmax_logprob_f64(o.softmax_logits(c["D"], c["b_d"], sub(got_att["h_tild"])))
+    close(d_lp.get()[:, cols], want_lp, "log-probs")
+    ctx.softmax_release(dD)
+    for ly in layers:
+        ly.close()

@@ -26,8 +26,8 @@ SYMBOLS = [
     "zr_ctx_create", "zr_ctx_destroy", "zr_ctx_sync", "zr_ctx_set_stream", "zr_ctx_set_option", "zr_last_error",
     "zr_version", "zr_timer_start", "zr_timer_stop", "zr_malloc", "zr_free", "zr_h2d", "zr_d2h", "zr_d2d", "zr_memset_zero", "zr_vocab_prep",
     "zr_vocab_prep_softmax", "zr_embed_gather", "zr_lstm_pack_weights", "zr_lstm_pack_weights_bf16", "zr_lstm_weights_destroy", "zr_lstm_step",
-    "zr_lstm_gates", "zr_lstm_stack_forward", "zr_gemm", "zr_softmax_prepare", "zr_softmax_release", "zr_softmax_forward", "zr_softmax_logprob_f64",
-    "zr_softmax_loss", "zr_attn_create", "zr_attn_destroy", "zr_attn_step", "zr_gather_columns",
+    "zr_lstm_gates", "zr_lstm_stack_forward", "zr_gemm", "zr_softmax_prepare", "zr_softmax_prepare_bf16", "zr_softmax_release", "zr_softmax_forward", "zr_softmax_logprob_f64",
+    "zr_softmax_loss", "zr_attn_create", "zr_attn_use_bf16_weights", "zr_attn_destroy", "zr_attn_step", "zr_gather_columns",
     "zr_broadcast_column", "zr_beam_create", "zr_beam_destroy", "zr_beam_init", "zr_beam_expand", "zr_beam_finish",
     "zr_beam_hypotheses", "zr_beam_state",
 ]
@@ -201,8 +201,9 @@ class Context:
                             _vp(d_B), C.c_int(ldb), _vp(d_C), C.c_int(ldc)))
 
     # ---- A8/A9
-    def softmax_prepare(self, d_D, V, H):
-        _chk(load().zr_softmax_prepare(self.h, _vp(d_D), C.c_int(V), C.c_int(H)))
+    def softmax_prepare(self, d_D, V, H, bf16=False):
+        fn = load().zr_softmax_prepare_bf16 if bf16 else load().zr_softmax_prepare
+        _chk(fn(self.h, _vp(d_D), C.c_int(V), C.c_int(H)))
 
     def softmax_release(self, d_D):
         _chk(load().zr_softmax_release(self.h, _vp(d_D)))
@@ -228,6 +229,9 @@ class Context:
         _chk(load().zr_attn_create(self.h, C.c_int(H), C.c_int(mb), C.c_int(D), _vp(W_a), _vp(W_p), _vp(v_p),
                                    _vp(out_bias), _vp(W_c1), _vp(W_c2), tab, C.c_int(len(hs_tables)), C.byref(a)))
         return a
+
+    def attn_use_bf16_weights(self, a):
+        _chk(load().zr_attn_use_bf16_weights(self.h, a))
 
     def attn_destroy(self, a):
         _chk(load().zr_attn_destroy(self.h, a))

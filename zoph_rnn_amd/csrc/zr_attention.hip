@@ -15,6 +15,9 @@ struct zr_attn {
   const float** d_table;                                   // device copy of the pointer table
   float *d_tanh1, *d_q, *d_align, *d_pt, *d_ctx;
   int* d_idx;
+  // zr_attn_use_bf16_weights: owned bf16 k-interleaved snapshots of W_p, W_a^T, W_c1, W_c2 ([H/8][ldp][8] each)
+  unsigned short* d_bf16;
+  int ldp;
 };
 
 namespace {
@@ -212,6 +215,8 @@ int zr_attn_create(zr_ctx* ctx, int H, int mb, int D, const float* d_W_a, const 
   a->out_bias = d_out_bias;
   a->W_c1 = d_W_c1;
   a->W_c2 = d_W_c2;
+  a->d_bf16 = nullptr;
+  a->ldp = 0;
   const size_t n = (size_t)H * mb, W = 2 * (size_t)D + 1;
   // one allocation: table | tanh1 | q | ctx | align | p_t | idx
   const size_t tbytes = (sizeof(float*) * longest_sent + 255) & ~(size_t)255;
@@ -241,11 +246,36 @@ int zr_attn_create(zr_ctx* ctx, int H, int mb, int D, const float* d_W_a, const 
   return ZR_OK;
 }
 
+int zr_attn_use_bf16_weights(zr_ctx* ctx, zr_attn* a) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(a != nullptr, "zr_attn_use_bf16_weights: attention object is null");
+  const int H = a->H;
+  ZR_CHECK_ARG(H % 16 == 0, "zr_attn_use_bf16_weights: H = %d is not a multiple of 16", H);
+  const int ldp = (H + 31) / 32 * 32;
+  const size_t per = (size_t)H * ldp;
+  if (!a->d_bf16) {
+    if (hipMalloc((void**)&a->d_bf16, sizeof(unsigned short) * 4 * per) != hipSuccess) {
+      (void)hipGetLastError();
+      a->d_bf16 = nullptr;
+      return zr_set_error(ZR_ENOMEM, "zr_attn_use_bf16_weights: allocation failed");
+    }
+  }
+  a->ldp = ldp;
+  const float* src[4] = {a->W_p, a->W_a, a->W_c1, a->W_c2};
+  for (int i = 0; i < 4; ++i) {
+    rc = zr_pack8_bf16_launch(ctx, src[i], H, H, H, ldp, H, a->d_bf16 + i * per, i == 1 ? 1 : 0);  // W_a transposed
+    if (rc) return rc;
+  }
+  return ZR_OK;
+}
+
 int zr_attn_destroy(zr_ctx* ctx, zr_attn* a) {
   if (!a) return ZR_OK;
   int rc = zr_bind_device(ctx);
   if (rc) return rc;
   ZR_HIP(hipStreamSynchronize(ctx->stream));
+  if (a->d_bf16) (void)hipFree(a->d_bf16);
   (void)hipFree((void*)a->d_table);
   delete a;
   return ZR_OK;
@@ -269,8 +299,14 @@ int zr_attn_step(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, const float* 
   g.N = mb;
   g.nseg = 1;
   g.K[0] = H;
+  const size_t per = (size_t)H * a->ldp;
   g.A[0] = a->W_p;
   g.lda[0] = H;
+  if (a->d_bf16) {
+    g.A[0] = (const float*)a->d_bf16;
+    g.lda[0] = a->ldp;
+    g.a_pack = 2;
+  }
   g.B[0] = d_h_t;
   g.ldb[0] = H;
   g.C = a->d_tanh1;
@@ -284,6 +320,10 @@ int zr_attn_step(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, const float* 
   // q = W_a^T h  (:195)
   g.A[0] = a->W_a;
   g.trans_a = 1;
+  if (a->d_bf16) {
+    g.A[0] = (const float*)(a->d_bf16 + per);  // already transposed
+    g.trans_a = 0;
+  }
   g.C = a->d_q;
   g.epilogue = ZR_EPI_STORE;
   rc = zr_gemm_launch(ctx, g);
@@ -325,6 +365,12 @@ int zr_attn_step(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, const float* 
   o.K[1] = H;
   o.A[1] = a->W_c2;
   o.lda[1] = H;
+  if (a->d_bf16) {
+    o.A[0] = (const float*)(a->d_bf16 + 2 * per);
+    o.A[1] = (const float*)(a->d_bf16 + 3 * per);
+    o.lda[0] = o.lda[1] = a->ldp;
+    o.a_pack = 2;
+  }
   o.B[1] = d_h_t;
   o.ldb[1] = H;
   o.C = d_htild;

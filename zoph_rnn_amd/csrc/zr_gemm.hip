@@ -63,23 +63,37 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& a, int m0, int n0, boo
       for (int r = 0; r < 16; ++r) acc[tm][tn][r] = 0.0f;
 
   for (int s = 0; s < a.nseg; ++s) {
-    const float* A = a.A[s] + (long long)z * a.strideA;
-    const float* wbase[TM];
-    unsigned woff[TM];
-    const float* xcol[TN];
+    if constexpr (AMODE == ZR_A_PACK8_BF16) {
+      const unsigned short* wbase[TM];
+      unsigned woff[TM];
+      const float* xcol[TN];
 #pragma unroll
-    for (int tm = 0; tm < TM; ++tm) {
-      wbase[tm] = A;
-      woff[tm] = AMODE == ZR_A_PACK4   ? (unsigned)(4LL * rows[tm] + 4LL * half * a.lda[s])
-                 : AMODE == ZR_A_TRANS ? (unsigned)((long long)rows[tm] * a.lda[s] + 4 * half)
-                                       : (unsigned)(rows[tm] + 4LL * half * a.lda[s]);
+      for (int tm = 0; tm < TM; ++tm) {
+        wbase[tm] = (const unsigned short*)a.A[s];
+        woff[tm] = (unsigned)(8LL * rows[tm] + 8LL * half * a.lda[s]);
+      }
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) xcol[tn] = a.B[s] + (long long)cols[tn] * a.ldb[s] + 8 * half;
+      zr_mma_segment_bf16<TM, TN, KS, PF>(acc, wbase, woff, a.lda[s], xcol, a.K[s], kslice);
+    } else {
+      const float* A = a.A[s] + (long long)z * a.strideA;
+      const float* wbase[TM];
+      unsigned woff[TM];
+      const float* xcol[TN];
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) {
+        wbase[tm] = A;
+        woff[tm] = AMODE == ZR_A_PACK4   ? (unsigned)(4LL * rows[tm] + 4LL * half * a.lda[s])
+                   : AMODE == ZR_A_TRANS ? (unsigned)((long long)rows[tm] * a.lda[s] + 4 * half)
+                                         : (unsigned)(rows[tm] + 4LL * half * a.lda[s]);
+      }
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn)
+        xcol[tn] = (AMODE == ZR_A_PACK4 && a.b_pack4) ? a.B[s] + 4LL * cols[tn] + 4LL * half * a.N
+                                                     : a.B[s] + (long long)cols[tn] * a.ldb[s] + 4 * half;
+      zr_mma_segment<TM, TN, KS, PF, AMODE, VEC>(acc, wbase, woff, a.lda[s], xcol, a.K[s], kslice, half,
+                                                 (AMODE == ZR_A_PACK4 && a.b_pack4) ? a.N : 1);
     }
-#pragma unroll
-    for (int tn = 0; tn < TN; ++tn)
-      xcol[tn] = (AMODE == ZR_A_PACK4 && a.b_pack4) ? a.B[s] + 4LL * cols[tn] + 4LL * half * a.N
-                                                   : a.B[s] + (long long)cols[tn] * a.ldb[s] + 4 * half;
-    zr_mma_segment<TM, TN, KS, PF, AMODE, VEC>(acc, wbase, woff, a.lda[s], xcol, a.K[s], kslice, half,
-                                               (AMODE == ZR_A_PACK4 && a.b_pack4) ? a.N : 1);
   }
 
   float* C = a.C + (long long)z * a.strideC;
@@ -203,7 +217,7 @@ __global__ void __launch_bounds__(64 * KS * WPB, OCC) gemm_kernel(GemmArgs a) {
   const long long ntiles = (long long)a.m_tiles * a.n_tiles;
   bool active = tile < ntiles;
   int mt, nt;
-  if (AMODE == ZR_A_PACK4) {
+  if (AMODE == ZR_A_PACK4 || AMODE == ZR_A_PACK8_BF16) {
     // Workgroup ids congruent modulo 8 run on the same XCD.  Each XCD gets a contiguous range of row tiles and
     // runs the column tiles of one row tile back to back, so a weight tile leaves memory once.
     const int r8 = (int)(tile & 7);
@@ -219,8 +233,9 @@ __global__ void __launch_bounds__(64 * KS * WPB, OCC) gemm_kernel(GemmArgs a) {
     mt = (int)(tile % a.m_tiles);
     nt = (int)(tile / a.m_tiles);
   }
-  constexpr int PF = AMODE == ZR_A_PACK4 ? (OCC == 1 ? (TM + TN <= 4 ? 8 : 6) : (TM + TN == 4 ? 6 : 4))
-                                         : zr_prefetch_depth(TM, TN);
+  constexpr int PF = AMODE == ZR_A_PACK8_BF16 ? 4
+                     : AMODE == ZR_A_PACK4    ? (OCC == 1 ? (TM + TN <= 4 ? 8 : 6) : (TM + TN == 4 ? 6 : 4))
+                                              : zr_prefetch_depth(TM, TN);
   float* redp = KS > 1 ? red + (size_t)sub * KS * TN * 16 * 64 : red;
   gemm_tile<TM, TN, KS, AMODE, VEC, EPI, PF>(a, mt * 32 * TM, nt * 32 * TN, active, z, redp, kslice, lane);
 }
@@ -231,7 +246,7 @@ __global__ void __launch_bounds__(64 * KS * WPB, OCC) gemm_kernel(GemmArgs a) {
 // workgroup per CU (or fewer): each takes an equal share of the 32-row blocks (+-1) for one column tile and walks
 // it in passes of up to four blocks, so every CU finishes at about the same time and each weight element is
 // read by exactly one workgroup per column tile.
-template <int TN, int EPI>
+template <int TN, int EPI, int AMODE = ZR_A_PACK4>
 __global__ void __launch_bounds__(256) gemm_rows_kernel(GemmArgs a, int row_chunks) {
   __shared__ float red[4 * TN * 16 * 64];
   const int tid = threadIdx.x;
@@ -250,17 +265,17 @@ __global__ void __launch_bounds__(256) gemm_rows_kernel(GemmArgs a, int row_chun
   const int n0 = nt * 32 * TN;
   // at most 192 accumulator registers per wave: four blocks per pass up to 96 columns, three at 128
   constexpr int TMAX = TN <= 3 ? 4 : 3;
-  constexpr int PF4 = TN <= 2 ? 6 : (TN == 3 ? 4 : 3);
+  constexpr int PF4 = AMODE == ZR_A_PACK8_BF16 ? 2 : (TN <= 2 ? 6 : (TN == 3 ? 4 : 3));
   while (b < b_end) {
     const int nb = b_end - b < TMAX ? b_end - b : TMAX;  // uniform over the workgroup
     if (TMAX == 4 && nb == 4)
-      gemm_tile<TMAX, TN, 4, ZR_A_PACK4, true, EPI, PF4>(a, b * 32, n0, true, 0, red, kslice, lane);
+      gemm_tile<TMAX, TN, 4, AMODE, true, EPI, PF4>(a, b * 32, n0, true, 0, red, kslice, lane);
     else if (nb == 3)
-      gemm_tile<3, TN, 4, ZR_A_PACK4, true, EPI, PF4 + 1>(a, b * 32, n0, true, 0, red, kslice, lane);
+      gemm_tile<3, TN, 4, AMODE, true, EPI, PF4 + 1>(a, b * 32, n0, true, 0, red, kslice, lane);
     else if (nb == 2)
-      gemm_tile<2, TN, 4, ZR_A_PACK4, true, EPI, PF4 + 2>(a, b * 32, n0, true, 0, red, kslice, lane);
+      gemm_tile<2, TN, 4, AMODE, true, EPI, PF4 + 2>(a, b * 32, n0, true, 0, red, kslice, lane);
     else
-      gemm_tile<1, TN, 4, ZR_A_PACK4, true, EPI, PF4 + 2>(a, b * 32, n0, true, 0, red, kslice, lane);
+      gemm_tile<1, TN, 4, AMODE, true, EPI, PF4 + 2>(a, b * 32, n0, true, 0, red, kslice, lane);
     b += nb;
     __syncthreads();  // the next pass reuses the reduction buffer
   }
@@ -473,7 +488,8 @@ int launch_lds_rows(zr_ctx* ctx, GemmArgs& ga, int epi) {
 template <int TM, int TN, int KS, int WPB, int AMODE, bool VEC, int OCC = 1>
 int launch_epi(zr_ctx* ctx, const GemmArgs& ga, int batch, int epi) {
   long long ntiles = (long long)ga.m_tiles * ga.n_tiles;
-  if (AMODE == ZR_A_PACK4) ntiles = (long long)((ga.m_tiles + 7) / 8) * 8 * ga.n_tiles;  // XCD-major id space
+  if (AMODE == ZR_A_PACK4 || AMODE == ZR_A_PACK8_BF16)
+    ntiles = (long long)((ga.m_tiles + 7) / 8) * 8 * ga.n_tiles;  // XCD-major id space
   dim3 grid((unsigned)((ntiles + WPB - 1) / WPB), 1, batch);
   dim3 block(64 * KS * WPB);
   switch (epi) {
@@ -526,7 +542,7 @@ __global__ void __launch_bounds__(256) pack4_x_kernel(const float* __restrict__ 
   *(zr_f32x4*)(dst + ((long long)b * N + n) * 4) = v;
 }
 
-template <int TN>
+template <int TN, int AMODE = ZR_A_PACK4>
 int launch_rows(zr_ctx* ctx, GemmArgs& ga, int epi, int n_tiles) {
   ga.n_tiles = n_tiles;
   ga.m_tiles = 0;
@@ -535,9 +551,9 @@ int launch_rows(zr_ctx* ctx, GemmArgs& ga, int epi, int n_tiles) {
   if (row_chunks > blocks) row_chunks = blocks;
   const unsigned grid = (unsigned)((row_chunks + 7) / 8) * 8 * n_tiles;
   if (epi == ZR_EPI_STORE)
-    gemm_rows_kernel<TN, ZR_EPI_STORE><<<grid, 256, 0, ctx->stream>>>(ga, row_chunks);
+    gemm_rows_kernel<TN, ZR_EPI_STORE, AMODE><<<grid, 256, 0, ctx->stream>>>(ga, row_chunks);
   else
-    gemm_rows_kernel<TN, ZR_EPI_SOFTMAX_PARTIAL><<<grid, 256, 0, ctx->stream>>>(ga, row_chunks);
+    gemm_rows_kernel<TN, ZR_EPI_SOFTMAX_PARTIAL, AMODE><<<grid, 256, 0, ctx->stream>>>(ga, row_chunks);
   ZR_LAUNCH_CHECK("gemm_rows_kernel");
   return ZR_OK;
 }
@@ -554,23 +570,23 @@ __global__ void __launch_bounds__(256) pack4_kernel(const float* __restrict__ sr
 }
 
 __global__ void __launch_bounds__(256) pack8_bf16_kernel(const float* __restrict__ src, int M, int K, long long ld,
-                                                         int ldp, int kp, unsigned short* __restrict__ dst) {
+                                                         int ldp, int kp, unsigned short* __restrict__ dst, int trans) {
   const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
   if (i >= (long long)kp * ldp) return;
   const int k8 = (int)(i & 7);
   const long long t = i >> 3;
   const int row = (int)(t % ldp);
   const int k = (int)(t / ldp) * 8 + k8;
-  const float v = (row < M && k < K) ? src[row + (long long)k * ld] : 0.0f;
+  const float v = (row < M && k < K) ? (trans ? src[k + (long long)row * ld] : src[row + (long long)k * ld]) : 0.0f;
   dst[i] = __builtin_bit_cast(unsigned short, (__bf16)v);
 }
 
 }  // namespace
 
 int zr_pack8_bf16_launch(zr_ctx* ctx, const float* src, int M, int K, long long ld, int ldp, int kp,
-                         unsigned short* dst) {
+                         unsigned short* dst, int trans) {
   const long long total = (long long)kp * ldp;
-  pack8_bf16_kernel<<<(unsigned)((total + 255) / 256), 256, 0, ctx->stream>>>(src, M, K, ld, ldp, kp, dst);
+  pack8_bf16_kernel<<<(unsigned)((total + 255) / 256), 256, 0, ctx->stream>>>(src, M, K, ld, ldp, kp, dst, trans);
   ZR_LAUNCH_CHECK("pack8_bf16_kernel");
   return ZR_OK;
 }
@@ -598,8 +614,9 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
       ZR_CHECK_ARG(d.K[s] > 0, "gemm: K[%d] = %d", s, d.K[s]);
       ZR_CHECK_ARG(d.A[s] && d.B[s], "gemm: null operand in segment %d", s);
       ZR_CHECK_ARG(d.lda[s] >= (d.trans_a ? d.K[s] : d.M), "gemm: lda[%d] = %d too small", s, d.lda[s]);
-      ZR_CHECK_ARG(!d.a_pack4 || (!d.trans_a && d.batch == 1 && d.lda[s] % 32 == 0 && 4LL * d.lda[s] + 4LL * d.M < (1LL << 31)),
+      ZR_CHECK_ARG(!d.a_pack || (!d.trans_a && d.batch == 1 && d.lda[s] % 32 == 0 && 8LL * d.lda[s] + 8LL * d.M < (1LL << 31)),
                    "gemm: packed operand A of segment %d: needs no transpose, one batch, lda a multiple of 32", s);
+      ZR_CHECK_ARG(d.a_pack != 2 || d.K[s] % 16 == 0, "gemm: bf16 operand A needs K %% 16 == 0 (K[%d] = %d)", s, d.K[s]);
       ZR_CHECK_ARG(d.ldb[s] >= d.K[s], "gemm: ldb[%d] = %d < K = %d", s, d.ldb[s], d.K[s]);
       // per-lane weight offsets are 32-bit element indices
       ZR_CHECK_ARG(d.trans_a ? ((long long)d.M * d.lda[s] + 8 < (1LL << 31)) : (d.M + 8LL * d.lda[s] < (1LL << 31)),
@@ -632,7 +649,27 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
   if (d.epilogue == ZR_EPI_SOFTMAX_PARTIAL) ZR_CHECK_ARG(d.bias && d.partials, "gemm: bias/partials required");
 
   ga.b_pack4 = 0;
-  if (d.a_pack4) {
+  if (d.a_pack == 2) {
+    ZR_CHECK_ARG(vec, "gemm: bf16 operand A needs 16-byte aligned activations with ldb %% 4 == 0");
+    if (d.nseg == 1 && d.M >= 8192 && d.N > 32 && d.N <= 1024 &&
+        (d.epilogue == ZR_EPI_STORE || d.epilogue == ZR_EPI_SOFTMAX_PARTIAL)) {
+      const int n32 = (d.N + 31) / 32;
+      const int n_tiles = (n32 + 3) / 4;
+      const int tn = (n32 + n_tiles - 1) / n_tiles;
+      if (tn <= 2) return launch_rows<2, ZR_A_PACK8_BF16>(ctx, ga, d.epilogue, n_tiles);
+      if (tn == 3) return launch_rows<3, ZR_A_PACK8_BF16>(ctx, ga, d.epilogue, n_tiles);
+      return launch_rows<4, ZR_A_PACK8_BF16>(ctx, ga, d.epilogue, n_tiles);
+    }
+    if (d.N <= 32) {
+      ga.m_tiles = (ga.M + 63) / 64;
+      ga.n_tiles = (ga.N + 31) / 32;
+      return launch_epi<2, 1, 4, 1, ZR_A_PACK8_BF16, true, 2>(ctx, ga, 1, d.epilogue);
+    }
+    ga.m_tiles = (ga.M + 63) / 64;
+    ga.n_tiles = (ga.N + 63) / 64;
+    return launch_epi<2, 2, 4, 1, ZR_A_PACK8_BF16, true, 2>(ctx, ga, 1, d.epilogue);
+  }
+  if (d.a_pack) {
     // Activations too: a k-interleaved copy in scratch turns their loads (16 bytes from each of 32 lines per
     // half-wave) into contiguous ones.  Worth a small extra kernel once the weight matrix is large.
     bool xpack = vec && d.M >= 2048;

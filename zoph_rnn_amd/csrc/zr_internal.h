@@ -34,7 +34,8 @@ struct zr_ctx {
     const float* key;  // the caller's d_D (null: slot free)
     int V, H;
     int ldp;           // V rounded up to 32
-    float* d_pack;     // [ceil8(H)/4][ldp][4]
+    int bf16;          // 0: d_pack is fp32 [ceil8(H)/4][ldp][4]; 1: bf16 [H/8][ldp][8]
+    void* d_pack;
   } packed_d[ZR_MAX_PACKED_D];
 };
 
@@ -84,9 +85,12 @@ struct ZrGemmDesc {
   const float* A[3];
   int lda[3];
   int trans_a;  // applies to every segment
-  // A is k-interleaved: element (m, k) at ((k/4)*lda + m)*4 + k%4, lda = M rounded up to 32, K padded to a multiple
-  // of 8, pads zero (see ZR_A_PACK4 in zr_mfma_core.h).  Single batch, no transpose.
-  int a_pack4;
+  // 1: A is k-interleaved fp32: element (m, k) at ((k/4)*lda + m)*4 + k%4, lda = M rounded up to 32, K padded to
+  //    a multiple of 8, pads zero (ZR_A_PACK4 in zr_mfma_core.h).
+  // 2: A is k-interleaved bf16 (2-byte elements behind the float pointer): element (m, k) at
+  //    ((k/8)*lda + m)*8 + k%8, K a multiple of 16 (ZR_A_PACK8_BF16).
+  // Single batch, no transpose.
+  int a_pack;
   const float* B[3];
   int ldb[3];
   float* C;
@@ -105,8 +109,9 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d);
 // zero padding (ldp >= M a multiple of 32, kp >= K a multiple of 8).  dst holds kp*ldp floats.
 int zr_pack4_launch(zr_ctx* ctx, const float* src, int M, int K, long long ld, int ldp, int kp, float* dst);
 // Same for the bf16 layout [kp/8][ldp][8] (round to nearest even); kp a multiple of 16.  dst holds kp*ldp elements.
+// trans != 0: the source holds the transpose (element (row, k) at src[k + row*ld]).
 int zr_pack8_bf16_launch(zr_ctx* ctx, const float* src, int M, int K, long long ld, int ldp, int kp,
-                         unsigned short* dst);
+                         unsigned short* dst, int trans = 0);
 // number of 32-row partial blocks the SOFTMAX_PARTIAL epilogue writes for M rows
 static inline int zr_softmax_partial_blocks(int M) { return (M + 31) / 32; }
 

@@ -161,9 +161,9 @@ int logits_with_partials(zr_ctx* ctx, const float* d_D, const float* d_b_d, int 
   for (int i = 0; i < ZR_MAX_PACKED_D; ++i) {
     const zr_ctx::PackedD& e = ctx->packed_d[i];
     if (e.key == d_D && e.V == V && e.H == H) {  // registered with zr_softmax_prepare: use the MFMA-layout copy
-      d.A[0] = e.d_pack;
+      d.A[0] = (const float*)e.d_pack;
       d.lda[0] = e.ldp;
-      d.a_pack4 = 1;
+      d.a_pack = e.bf16 ? 2 : 1;
       break;
     }
   }
@@ -199,16 +199,19 @@ int check_softmax_args(const char* who, const float* d_D, const float* d_b_d, in
 
 extern "C" {
 
-int zr_softmax_prepare(zr_ctx* ctx, const float* d_D, int V, int H) {
+static int softmax_prepare(zr_ctx* ctx, const char* who, const float* d_D, int V, int H, bool bf16) {
   int rc = zr_bind_device(ctx);
   if (rc) return rc;
-  ZR_CHECK_ARG(d_D != nullptr && V > 0 && H > 0, "zr_softmax_prepare: d_D null or V = %d, H = %d", V, H);
-  const int ldp = (V + 31) / 32 * 32, kp = (H + 7) / 8 * 8;
-  ZR_CHECK_ARG(4LL * ldp + 4LL * V < (1LL << 31), "zr_softmax_prepare: V = %d too large", V);
+  ZR_CHECK_ARG(d_D != nullptr && V > 0 && H > 0, "%s: d_D null or V = %d, H = %d", who, V, H);
+  ZR_CHECK_ARG(!bf16 || H % 16 == 0, "%s: H = %d is not a multiple of 16", who, H);
+  const int ldp = (V + 31) / 32 * 32, kp = bf16 ? H : (H + 7) / 8 * 8;
+  ZR_CHECK_ARG(8LL * ldp + 8LL * V < (1LL << 31), "%s: V = %d too large", who, V);
+  const size_t bytes = (bf16 ? sizeof(unsigned short) : sizeof(float)) * (size_t)kp * ldp;
   int slot = -1;
   for (int i = 0; i < ZR_MAX_PACKED_D; ++i)
     if (ctx->packed_d[i].key == d_D) slot = i;
-  if (slot >= 0 && (ctx->packed_d[slot].V != V || ctx->packed_d[slot].H != H)) {
+  if (slot >= 0 && (ctx->packed_d[slot].V != V || ctx->packed_d[slot].H != H ||
+                    ctx->packed_d[slot].bf16 != (bf16 ? 1 : 0))) {
     rc = zr_softmax_release(ctx, d_D);
     if (rc) return rc;
     slot = -1;
@@ -216,19 +219,20 @@ int zr_softmax_prepare(zr_ctx* ctx, const float* d_D, int V, int H) {
   if (slot < 0) {
     for (int i = 0; i < ZR_MAX_PACKED_D && slot < 0; ++i)
       if (!ctx->packed_d[i].key) slot = i;
-    ZR_CHECK_ARG(slot >= 0, "zr_softmax_prepare: all %d slots are in use (zr_softmax_release one)", ZR_MAX_PACKED_D);
-    float* p = nullptr;
-    if (hipMalloc((void**)&p, sizeof(float) * (size_t)kp * ldp) != hipSuccess) {
+    ZR_CHECK_ARG(slot >= 0, "%s: all %d slots are in use (zr_softmax_release one)", who, ZR_MAX_PACKED_D);
+    void* p = nullptr;
+    if (hipMalloc(&p, bytes) != hipSuccess) {
       (void)hipGetLastError();
-      return zr_set_error(ZR_ENOMEM, "zr_softmax_prepare: allocation of %zu bytes failed",
-                          sizeof(float) * (size_t)kp * ldp);
+      return zr_set_error(ZR_ENOMEM, "%s: allocation of %zu bytes failed", who, bytes);
     }
     ctx->packed_d[slot].d_pack = p;
     ctx->packed_d[slot].V = V;
     ctx->packed_d[slot].H = H;
     ctx->packed_d[slot].ldp = ldp;
+    ctx->packed_d[slot].bf16 = bf16 ? 1 : 0;
   }
-  rc = zr_pack4_launch(ctx, d_D, V, H, V, ldp, kp, ctx->packed_d[slot].d_pack);
+  rc = bf16 ? zr_pack8_bf16_launch(ctx, d_D, V, H, V, ldp, kp, (unsigned short*)ctx->packed_d[slot].d_pack)
+            : zr_pack4_launch(ctx, d_D, V, H, V, ldp, kp, (float*)ctx->packed_d[slot].d_pack);
   if (rc) {
     (void)hipFree(ctx->packed_d[slot].d_pack);
     ctx->packed_d[slot] = zr_ctx::PackedD{};
@@ -236,6 +240,14 @@ int zr_softmax_prepare(zr_ctx* ctx, const float* d_D, int V, int H) {
   }
   ctx->packed_d[slot].key = d_D;
   return ZR_OK;
+}
+
+int zr_softmax_prepare(zr_ctx* ctx, const float* d_D, int V, int H) {
+  return softmax_prepare(ctx, "zr_softmax_prepare", d_D, V, H, false);
+}
+
+int zr_softmax_prepare_bf16(zr_ctx* ctx, const float* d_D, int V, int H) {
+  return softmax_prepare(ctx, "zr_softmax_prepare_bf16", d_D, V, H, true);
 }
 
 int zr_softmax_release(zr_ctx* ctx, const float* d_D) {
