@@ -8,6 +8,7 @@
 //   ids.txt: S*mb source ids, T*mb target input ids, T*mb target output ids, 2*mb batch_info (time-major, -1 pads)
 //   S == 0: language model (no source, no attention).
 #include <cstdio>
+#include <cstdlib>
 #include <fstream>
 #include <iostream>
 #include <vector>
@@ -31,6 +32,7 @@ int main(int argc, char** argv) {
     for (auto& v : tout) f >> v;
     for (auto& v : binfo) f >> v;
   }
+  if (const char* e = std::getenv("ZOPH_BF16_WEIGHTS")) BZ_CUDA::bf16_weights = (e[0] == '1');
   layer_gpu_info gpu;
   gpu.init(0);
   neuralMT_model<precision> model;

@@ -53,6 +53,10 @@ inline precision lower = -0.08f;
 inline precision upper = 0.08f;
 inline bool force_decode = false;
 inline std::mt19937 gen(1234);
+// No counterpart in the reference: when set before the layers are initialised / loaded, every matrix the matrix cores
+// stream (LSTM M / W_h / Q, attention W_a / W_p / W_c, softmax D) is snapshotted as bf16; the fp32 members stay as
+// the caller's copy.  Requires LSTM_size % 16 == 0.
+inline bool bf16_weights = false;
 }  // namespace BZ_CUDA
 
 struct attention_params {  // src/global_params.h:8-22 (fields used by the forward path)
@@ -224,6 +228,7 @@ class attention_layer {  // src/attention_layer.h:14-143
     h_total_hs_mat = total_hs;
     ZOPH_CALL(zr_attn_create(ctx, LSTM_size, minibatch_size, D, d_W_a, d_W_p, d_v_p, d_output_bias, d_W_c_p1, d_W_c_p2,
                              h_total_hs_mat.data(), (int)h_total_hs_mat.size(), &attn));
+    if (BZ_CUDA::bf16_weights) ZOPH_CALL(zr_attn_use_bf16_weights(ctx, attn));
     for (int i = 0; i < longest_sent; i++)
       nodes.push_back(attention_node<dType>(LSTM_size, minibatch_size, device_number, D, feed_input, this, i));
   }
@@ -250,6 +255,7 @@ class attention_layer {  // src/attention_layer.h:14-143
     read_matrix_GPU(ctx, d_output_bias, LSTM_size, 1, input);
     read_matrix_GPU(ctx, d_W_c_p1, LSTM_size, LSTM_size, input);
     read_matrix_GPU(ctx, d_W_c_p2, LSTM_size, LSTM_size, input);
+    if (BZ_CUDA::bf16_weights && attn) ZOPH_CALL(zr_attn_use_bf16_weights(ctx, attn));
   }
 };
 
@@ -414,7 +420,12 @@ class softmax_layer : public base_loss_layer<dType> {  // src/softmax.h:14-225
   }
   // No counterpart in the reference: snapshots d_D into the layout the matrix cores read fastest.  Called after
   // init_loss_layer and load_weights; call again by hand after writing to d_D.
-  void prepare_weights() { ZOPH_CALL(zr_softmax_prepare(s_layer_info.ctx, d_D, output_vocab_size, LSTM_size)); }
+  void prepare_weights() {
+    if (BZ_CUDA::bf16_weights)
+      ZOPH_CALL(zr_softmax_prepare_bf16(s_layer_info.ctx, d_D, output_vocab_size, LSTM_size));
+    else
+      ZOPH_CALL(zr_softmax_prepare(s_layer_info.ctx, d_D, output_vocab_size, LSTM_size));
+  }
 };
 
 // ------------------------------------------------------------------------------------------------ LSTM nodes
@@ -532,7 +543,10 @@ class Hidden_To_Hidden_Layer {  // src/Hidden_To_Hidden_Layer.h:12-313
     const dType* M[4] = {d_M_i, d_M_f, d_M_c, d_M_o};
     const dType* Wh[4] = {d_W_hi, d_W_hf, d_W_hc, d_W_ho};
     const dType* b[4] = {d_b_i, d_b_f, d_b_c, d_b_o};
-    ZOPH_CALL(zr_lstm_pack_weights(ctx, M, Wh, nullptr, b, LSTM_size, &packed));
+    if (BZ_CUDA::bf16_weights)
+      ZOPH_CALL(zr_lstm_pack_weights_bf16(ctx, M, Wh, nullptr, b, LSTM_size, &packed));
+    else
+      ZOPH_CALL(zr_lstm_pack_weights(ctx, M, Wh, nullptr, b, LSTM_size, &packed));
   }
   // src/Hidden_To_Hidden_Layer.hpp:748-774
   void prep_GPU_vocab_indices(int* h_input_vocab_indicies, int current_length) {
@@ -661,7 +675,10 @@ class Input_To_Hidden_Layer {  // src/Input_To_Hidden_Layer.h:11-368
     const dType* Wh[4] = {d_W_hi, d_W_hf, d_W_hc, d_W_ho};
     const dType* Q[4] = {d_Q_i, d_Q_f, d_Q_c, d_Q_o};
     const dType* b[4] = {d_b_i, d_b_f, d_b_c, d_b_o};
-    ZOPH_CALL(zr_lstm_pack_weights(ctx, M, Wh, feed_input ? Q : nullptr, b, LSTM_size, &packed));
+    if (BZ_CUDA::bf16_weights)
+      ZOPH_CALL(zr_lstm_pack_weights_bf16(ctx, M, Wh, feed_input ? Q : nullptr, b, LSTM_size, &packed));
+    else
+      ZOPH_CALL(zr_lstm_pack_weights(ctx, M, Wh, feed_input ? Q : nullptr, b, LSTM_size, &packed));
   }
   // src/Input_To_Hidden_Layer.hpp:1178-1225 (the *_Wgrad arguments serve the embedding gradient only)
   void prep_GPU_vocab_indices(int* h_input_vocab_indicies, int* /*h_input_vocab_indicies_Wgrad*/, int current_length,
