@@ -41,8 +41,19 @@ def build_hip(verbose=False, jobs=4):
     return LIB
 
 
-if __name__ == "__main__":
-    print(build_hip(verbose=True, jobs=int(os.environ.get("JOBS", "4"))))
+
+
+def build_force_decode():
+    """The force-decode / perplexity driver over text files (zoph_rnn_amd/host/force_decode), plain g++ against the
+    C-ABI."""
+    src = os.path.join(HERE, "host", "force_decode.cpp")
+    out = os.path.join(HERE, "host", "force_decode")
+    cmd = [os.environ.get("CXX", "g++"), "-std=c++17", "-O1", "-Wall", "-o", out, src, "-L", HERE, "-lzoph_rnn_hip",
+           "-Wl,-rpath,$ORIGIN/.."]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("force_decode build failed:\n" + r.stdout + r.stderr)
+    return out
 
 
 def build_host_driver():
@@ -56,3 +67,7 @@ def build_host_driver():
     if r.returncode != 0:
         raise RuntimeError("host driver build failed:\n" + r.stdout + r.stderr)
     return out
+
+
+if __name__ == "__main__":
+    print(build_hip(verbose=True, jobs=int(os.environ.get("JOBS", "4"))))

@@ -1,0 +1,563 @@
+// Model files, integerized data files and the forward (force-decode / perplexity) schedule on top of the layer
+// classes of zoph_layers.h.
+//
+//  * model_file_info, read_model_file_info, write_model_file_info: the text model file of the reference -- header
+//    line, vocabulary blocks between "====" lines, then the matrices (written by src/input_file_prep.h:304-357 and
+//    src/add_model_info.h:7-23, skipped over by neuralMT_model::load_weights, src/model.hpp:2172-2195).
+//  * integerize_parallel_text / integerize_target_text: raw tokenised text -> the 4-lines-per-sentence integer file
+//    (src/input_file_prep.h:403-500 for source/target pairs, :1590-1670 for the sequence model): vocabulary lookup
+//    with <UNK>, source reversed and left padded with -1, target input <START> + words, target output words + <EOF>,
+//    right padded with -1, padding per minibatch.
+//  * minibatch_reader: file_helper::read_minibatch (src/fileHelper.h:367-518) -- fills the time-major host arrays
+//    idx[b + t*minibatch] and batch_info.
+//  * forward_model: the layers wired as neuralMT_model::initModel does (src/model.hpp:300-420), load_weights /
+//    dump_weights in file order (src/model.hpp:2172-2241, 2058-2070), getError(GPU) (src/model.hpp:1463-1802) and
+//    get_perplexity with the force-decode output of one log-probability line per minibatch (src/model.hpp:2281-2355).
+#ifndef ZOPH_MODEL_H
+#define ZOPH_MODEL_H
+
+#include <algorithm>
+#include <cmath>
+#include <fstream>
+#include <functional>
+#include <iomanip>
+#include <limits>
+#include <map>
+#include <sstream>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "zoph_layers.h"
+
+struct model_file_info {
+  int num_layers = 1, LSTM_size = 0, target_vocab_size = 0, source_vocab_size = 0;
+  bool attention_model = false, feed_input = false, multi_source = false, combine_LSTM = false, char_cnn = false;
+  bool LM = false;                         // sequence model: no source side, one vocabulary block
+  std::vector<std::string> source_vocab;   // index -> word ("<UNK>" at 0)
+  std::vector<std::string> target_vocab;   // index -> word ("<START>", "<EOF>", "<UNK>" at 0, 1, 2)
+};
+
+inline bool zoph_is_separator(const std::string& s) { return s.size() > 3 && s[0] == '=' && s[1] == '=' && s[2] == '='; }
+
+// Reads the header and the vocabulary block(s) and leaves the stream at the first matrix.  Returns false and
+// fills err on a malformed file or a model kind the forward path does not cover.
+inline bool read_model_file_info(std::istream& in, bool LM, model_file_info& info, std::string& err) {
+  std::string line;
+  if (!std::getline(in, line)) {
+    err = "empty model file";
+    return false;
+  }
+  std::vector<std::string> f;
+  {
+    std::istringstream iss(line);
+    std::string w;
+    while (iss >> w) f.push_back(w);
+  }
+  // 9 fields after training (add_model_info); 3 or 4 straight after data preparation
+  if (f.size() != 9 && f.size() != 4 && f.size() != 3) {
+    err = "model header has " + std::to_string(f.size()) + " fields (expected 9, 4 or 3)";
+    return false;
+  }
+  try {
+    info.num_layers = std::stoi(f[0]);
+    info.LSTM_size = std::stoi(f[1]);
+    info.target_vocab_size = std::stoi(f[2]);
+    info.source_vocab_size = f.size() >= 4 ? std::stoi(f[3]) : 0;
+    if (f.size() == 9) {
+      info.attention_model = std::stoi(f[4]) != 0;
+      info.feed_input = std::stoi(f[5]) != 0;
+      info.multi_source = std::stoi(f[6]) != 0;
+      info.combine_LSTM = std::stoi(f[7]) != 0;
+      info.char_cnn = std::stoi(f[8]) != 0;
+    }
+  } catch (const std::exception&) {
+    err = "model header is not numeric: " + line;
+    return false;
+  }
+  info.LM = LM;
+  if (info.multi_source || info.char_cnn) {
+    err = "multi-source and character-CNN models are outside the forward path built here";
+    return false;
+  }
+  if (info.num_layers < 1 || info.LSTM_size < 1 || info.target_vocab_size < 3) {
+    err = "implausible model header: " + line;
+    return false;
+  }
+  if (!std::getline(in, line) || !zoph_is_separator(line)) {
+    err = "missing separator after the model header";
+    return false;
+  }
+  auto read_block = [&](std::vector<std::string>& vocab, const char* what) {
+    while (std::getline(in, line)) {
+      if (zoph_is_separator(line)) return true;
+      std::istringstream iss(line);
+      long long id;
+      std::string word;
+      if (!(iss >> id >> word) || id != (long long)vocab.size()) {
+        err = std::string("bad ") + what + " vocabulary line: " + line;
+        return false;
+      }
+      vocab.push_back(word);
+    }
+    err = std::string("unterminated ") + what + " vocabulary block";
+    return false;
+  };
+  info.source_vocab.clear();
+  info.target_vocab.clear();
+  if (!LM && !read_block(info.source_vocab, "source")) return false;
+  if (!read_block(info.target_vocab, "target")) return false;
+  if ((int)info.target_vocab.size() != info.target_vocab_size ||
+      (!LM && (int)info.source_vocab.size() != info.source_vocab_size)) {
+    err = "vocabulary blocks do not match the sizes in the header";
+    return false;
+  }
+  return true;
+}
+
+inline void write_model_file_info(std::ostream& out, const model_file_info& info) {
+  const char* sep = "==========================================================\n";
+  out << info.num_layers << " " << info.LSTM_size << " " << info.target_vocab_size << " " << info.source_vocab_size
+      << " " << (int)info.attention_model << " " << (int)info.feed_input << " " << (int)info.multi_source << " "
+      << (int)info.combine_LSTM << " " << (int)info.char_cnn << "\n";
+  out << sep;
+  if (!info.LM) {
+    for (size_t i = 0; i < info.source_vocab.size(); i++) out << i << " " << info.source_vocab[i] << "\n";
+    out << sep;
+  }
+  for (size_t i = 0; i < info.target_vocab.size(); i++) out << i << " " << info.target_vocab[i] << "\n";
+  out << sep;
+}
+
+// ------------------------------------------------------------------------------------------------ integerization
+inline std::vector<std::string> zoph_split_words(const std::string& line) {
+  std::istringstream iss(line);
+  std::vector<std::string> w;
+  std::string t;
+  while (iss >> t) w.push_back(t);
+  return w;
+}
+
+struct integerized_sentence {
+  std::vector<int> src, minus_two, tgt_in, tgt_out;
+};
+
+inline void zoph_write_int_line(std::ostream& out, const std::vector<int>& v) {
+  for (int x : v) out << x << " ";
+  out << "\n";
+}
+
+// Source / target text (one sentence per line, same number of lines) -> the integer file.  Sentences longer than
+// longest_sent - 2 words on either side are an error here (the reference's force-decode path refuses them too).
+// Returns the number of sentence pairs written, or -1 with err set.  total_target_words counts the target output
+// tokens (words + <EOF>), the denominator of the perplexity.
+inline int integerize_parallel_text(const model_file_info& info, const std::string& source_path,
+                                    const std::string& target_path, const std::string& out_path, int minibatch_size,
+                                    int longest_sent, long long& total_target_words, std::string& err) {
+  std::ifstream fs(source_path), ft(target_path);
+  if (!fs || !ft) {
+    err = "cannot open " + (fs ? target_path : source_path);
+    return -1;
+  }
+  std::unordered_map<std::string, int> smap, tmap;
+  for (size_t i = 0; i < info.source_vocab.size(); i++) smap[info.source_vocab[i]] = (int)i;
+  for (size_t i = 0; i < info.target_vocab.size(); i++) tmap[info.target_vocab[i]] = (int)i;
+  const int src_unk = smap.count("<UNK>") ? smap["<UNK>"] : 0;
+  const int tgt_unk = tmap.count("<UNK>") ? tmap["<UNK>"] : (tmap.count("<UNK>NULL") ? tmap["<UNK>NULL"] : 2);
+  std::vector<integerized_sentence> data;
+  std::string ls, lt;
+  total_target_words = 0;
+  while (std::getline(fs, ls)) {
+    if (!std::getline(ft, lt)) {
+      err = "target file has fewer lines than the source file";
+      return -1;
+    }
+    const auto sw = zoph_split_words(ls), tw = zoph_split_words(lt);
+    if ((int)sw.size() > longest_sent - 2 || (int)tw.size() > longest_sent - 2 || sw.empty() || tw.empty()) {
+      err = "sentence pair " + std::to_string(data.size() + 1) + " is empty or longer than longest_sent - 2";
+      return -1;
+    }
+    integerized_sentence s;
+    for (const auto& w : sw) s.src.push_back(smap.count(w) ? smap[w] : src_unk);
+    std::reverse(s.src.begin(), s.src.end());
+    s.minus_two.assign(s.src.size(), -2);
+    for (const auto& w : tw) s.tgt_in.push_back(tmap.count(w) ? tmap[w] : tgt_unk);
+    s.tgt_out = s.tgt_in;
+    s.tgt_in.insert(s.tgt_in.begin(), 0);  // <START>
+    s.tgt_out.push_back(1);                // <EOF>
+    total_target_words += (long long)s.tgt_out.size();
+    data.push_back(s);
+  }
+  if (std::getline(ft, lt) && !zoph_split_words(lt).empty()) {
+    err = "target file has more lines than the source file";
+    return -1;
+  }
+  for (size_t base = 0; base < data.size(); base += minibatch_size) {
+    const size_t end = std::min(data.size(), base + (size_t)minibatch_size);
+    size_t max_s = 0, max_t = 0;
+    for (size_t i = base; i < end; i++) {
+      max_s = std::max(max_s, data[i].src.size());
+      max_t = std::max(max_t, data[i].tgt_in.size());
+    }
+    for (size_t i = base; i < end; i++) {
+      auto& d = data[i];
+      d.src.insert(d.src.begin(), max_s - d.src.size(), -1);  // source: left padded
+      d.minus_two.insert(d.minus_two.begin(), max_s - d.minus_two.size(), -1);
+      d.tgt_in.resize(max_t, -1);                             // target: right padded
+      d.tgt_out.resize(max_t, -1);
+    }
+  }
+  std::ofstream out(out_path);
+  if (!out) {
+    err = "cannot write " + out_path;
+    return -1;
+  }
+  for (const auto& d : data) {
+    zoph_write_int_line(out, d.src);
+    zoph_write_int_line(out, d.minus_two);
+    zoph_write_int_line(out, d.tgt_in);
+    zoph_write_int_line(out, d.tgt_out);
+  }
+  return (int)data.size();
+}
+
+// Sequence-model variant (target side only): two empty lines, then target input and output; every sentence of a
+// minibatch is padded to one MORE than the longest (the reference pads `while size <= max`,
+// src/input_file_prep.h:1622-1627), which adds a fully masked last step.
+inline int integerize_target_text(const model_file_info& info, const std::string& target_path,
+                                  const std::string& out_path, int minibatch_size, int longest_sent,
+                                  long long& total_target_words, std::string& err) {
+  std::ifstream ft(target_path);
+  if (!ft) {
+    err = "cannot open " + target_path;
+    return -1;
+  }
+  std::unordered_map<std::string, int> tmap;
+  for (size_t i = 0; i < info.target_vocab.size(); i++) tmap[info.target_vocab[i]] = (int)i;
+  const int tgt_unk = tmap.count("<UNK>") ? tmap["<UNK>"] : 2;
+  std::vector<integerized_sentence> data;
+  std::string lt;
+  total_target_words = 0;
+  while (std::getline(ft, lt)) {
+    const auto tw = zoph_split_words(lt);
+    if (tw.empty() || (int)tw.size() > longest_sent - 3) {
+      err = "sentence " + std::to_string(data.size() + 1) + " is empty or longer than longest_sent - 3";
+      return -1;
+    }
+    integerized_sentence s;
+    for (const auto& w : tw) s.tgt_in.push_back(tmap.count(w) ? tmap[w] : tgt_unk);
+    s.tgt_out = s.tgt_in;
+    s.tgt_in.insert(s.tgt_in.begin(), 0);
+    s.tgt_out.push_back(1);
+    total_target_words += (long long)s.tgt_out.size();
+    data.push_back(s);
+  }
+  for (size_t base = 0; base < data.size(); base += minibatch_size) {
+    const size_t end = std::min(data.size(), base + (size_t)minibatch_size);
+    size_t max_t = 0;
+    for (size_t i = base; i < end; i++) max_t = std::max(max_t, data[i].tgt_in.size());
+    for (size_t i = base; i < end; i++) {
+      data[i].tgt_in.resize(max_t + 1, -1);
+      data[i].tgt_out.resize(max_t + 1, -1);
+    }
+  }
+  std::ofstream out(out_path);
+  if (!out) {
+    err = "cannot write " + out_path;
+    return -1;
+  }
+  for (const auto& d : data) {
+    out << "\n\n";
+    zoph_write_int_line(out, d.tgt_in);
+    zoph_write_int_line(out, d.tgt_out);
+  }
+  return (int)data.size();
+}
+
+// ------------------------------------------------------------------------------------------------ minibatch reader
+struct minibatch_reader {
+  int minibatch_size = 1, longest_sent = 100;
+  bool LM = false;
+  std::ifstream input_file;
+  // time-major host arrays, idx[b + t*minibatch_size], as the layers' prep_GPU_vocab_indices expect them
+  std::vector<int> h_input_vocab_indicies_source, h_output_vocab_indicies_source, h_input_vocab_indicies_target,
+      h_output_vocab_indicies_target, h_batch_info;
+  int current_source_length = 0, current_target_length = 0;
+  int sentences_in_minibatch = 0;  // fewer than minibatch_size at the end of the file (the rest is padding)
+  int words_in_minibatch = 0;
+
+  bool open(const std::string& path, int minibatch, int longest, bool lm) {
+    minibatch_size = minibatch;
+    longest_sent = longest;
+    LM = lm;
+    input_file.open(path);
+    const size_t n = (size_t)minibatch * longest;
+    h_input_vocab_indicies_source.assign(n, -1);
+    h_output_vocab_indicies_source.assign(n, -1);
+    h_input_vocab_indicies_target.assign(n, -1);
+    h_output_vocab_indicies_target.assign(n, -1);
+    h_batch_info.assign(2 * (size_t)minibatch, 0);
+    return (bool)input_file;
+  }
+
+  static std::vector<int> ints(const std::string& line) {
+    std::istringstream iss(line);
+    std::vector<int> v;
+    std::string w;
+    while (iss >> w) v.push_back(std::stoi(w));
+    return v;
+  }
+
+  // Reads up to minibatch_size sentences (4 lines each).  Returns false when nothing was left.  A short last
+  // minibatch is completed with fully padded (-1) columns, which contribute nothing to the loss.
+  bool read_minibatch(std::string& err) {
+    std::vector<std::vector<int>> si, so, ti, to;
+    std::string a, b, c, d;
+    while ((int)si.size() < minibatch_size && std::getline(input_file, a)) {
+      if (!std::getline(input_file, b) || !std::getline(input_file, c) || !std::getline(input_file, d)) {
+        err = "integer file ends in the middle of a sentence (4 lines per sentence)";
+        return false;
+      }
+      si.push_back(ints(a));
+      so.push_back(ints(b));
+      ti.push_back(ints(c));
+      to.push_back(ints(d));
+    }
+    sentences_in_minibatch = (int)si.size();
+    if (si.empty()) return false;
+    current_source_length = (int)si.back().size();
+    current_target_length = (int)ti.back().size();
+    for (size_t i = 0; i < si.size(); i++) {
+      if ((int)si[i].size() != current_source_length || (int)ti[i].size() != current_target_length ||
+          to[i].size() != ti[i].size()) {
+        err = "sentences of one minibatch differ in padded length (was the file made for another minibatch size?)";
+        return false;
+      }
+    }
+    if (current_source_length > longest_sent || current_target_length > longest_sent) {
+      err = "a sentence is longer than longest_sent";
+      return false;
+    }
+    words_in_minibatch = 0;
+    for (int i = 0; i < minibatch_size; i++) {
+      const bool real = i < (int)si.size();
+      int len = 0;
+      for (int j = 0; j < current_source_length; j++) {
+        const int v = real ? si[i][j] : -1;
+        if (v != -1) len++;
+        h_input_vocab_indicies_source[i + (size_t)j * minibatch_size] = v;
+        h_output_vocab_indicies_source[i + (size_t)j * minibatch_size] = real && j < (int)so[i].size() ? so[i][j] : -1;
+      }
+      // a padding column still needs one readable source position for the attention window
+      h_batch_info[i] = real ? len : (current_source_length > 0 ? 1 : 0);
+      h_batch_info[i + minibatch_size] = current_source_length - h_batch_info[i];
+      for (int j = 0; j < current_target_length; j++) {
+        h_input_vocab_indicies_target[i + (size_t)j * minibatch_size] = real ? ti[i][j] : -1;
+        h_output_vocab_indicies_target[i + (size_t)j * minibatch_size] = real ? to[i][j] : -1;
+        if (real && to[i][j] != -1) words_in_minibatch++;
+      }
+    }
+    return true;
+  }
+};
+
+// ------------------------------------------------------------------------------------------------ the model
+template <typename dType>
+class forward_model {
+ public:
+  model_file_info info;
+  global_params params;
+  layer_gpu_info gpu;
+  neuralMT_model<precision> flags;
+  Input_To_Hidden_Layer<dType> input_layer_source, input_layer_target;
+  std::vector<Hidden_To_Hidden_Layer<dType>> source_hidden_layers, target_hidden_layers;
+  softmax_layer<dType> softmax_obj;
+  base_loss_layer<dType>* softmax = nullptr;
+  attention_layer<dType>* att = nullptr;
+
+  // neuralMT_model::initModel (src/model.hpp:35-420) for the forward path on one device.  attention_D: the window
+  // half-width; the model file does not store it and the reference's decoder uses its default of 10.
+  void initModel(const layer_gpu_info& g, const model_file_info& mi, int minibatch_size, int longest_sent,
+                 int attention_D = 10) {
+    gpu = g;
+    info = mi;
+    const bool seq2seq = !mi.LM;
+    const int H = mi.LSTM_size, L = mi.num_layers;
+    params.LSTM_size = H;
+    params.minibatch_size = minibatch_size;
+    params.longest_sent = longest_sent;
+    params.target_vocab_size = mi.target_vocab_size;
+    params.source_vocab_size = mi.source_vocab_size;
+    params.attent_params.attention_model = seq2seq && mi.attention_model;
+    params.attent_params.D = attention_D;
+    params.attent_params.feed_input = seq2seq && mi.attention_model && mi.feed_input;
+    flags.attent_params = params.attent_params;
+    source_hidden_layers.resize(seq2seq ? L - 1 : 0);
+    target_hidden_layers.resize(L - 1);
+    softmax = &softmax_obj;
+    softmax_obj.share_gpu(gpu);
+    softmax->init_loss_layer(&flags, params);
+    if (seq2seq) {
+      input_layer_source.ih_layer_info.share(gpu);
+      input_layer_source.init_Input_To_Hidden_Layer(H, minibatch_size, mi.source_vocab_size, longest_sent, false, 0.f,
+                                                    false, 0.f, &flags, 0, false, 0.f, false, false, nullptr, false,
+                                                    params, true);
+      for (int l = 0; l < L - 1; l++) {
+        source_hidden_layers[l].hh_layer_info.share(gpu);
+        source_hidden_layers[l].init_Hidden_To_Hidden_Layer(H, minibatch_size, longest_sent, false, 0.f, false, 0.f,
+                                                             &flags, 0, false, 0.f, false, l);
+      }
+    }
+    input_layer_target.ih_layer_info.share(gpu);
+    input_layer_target.init_Input_To_Hidden_Layer(H, minibatch_size, mi.target_vocab_size, longest_sent, false, 0.f,
+                                                  false, 0.f, &flags, 0, false, 0.f, false, false, nullptr, false,
+                                                  params, false);
+    for (int l = 0; l < L - 1; l++) {
+      target_hidden_layers[l].hh_layer_info.share(gpu);
+      target_hidden_layers[l].init_Hidden_To_Hidden_Layer(H, minibatch_size, longest_sent, false, 0.f, false, 0.f,
+                                                           &flags, 0, false, 0.f, false, l);
+    }
+    auto wire = [&](Input_To_Hidden_Layer<dType>& in, std::vector<Hidden_To_Hidden_Layer<dType>>& hid, bool source) {
+      if (hid.empty()) {
+        in.upper_layer.init_upper_transfer_layer(true, false, source, softmax, nullptr);
+      } else {
+        in.upper_layer.init_upper_transfer_layer(false, false, source, nullptr, &hid[0]);
+        for (size_t l = 0; l + 1 < hid.size(); l++)
+          hid[l].upper_layer.init_upper_transfer_layer(false, false, source, nullptr, &hid[l + 1]);
+        hid.back().upper_layer.init_upper_transfer_layer(true, false, source, softmax, nullptr);
+      }
+    };
+    if (seq2seq) wire(input_layer_source, source_hidden_layers, true);
+    wire(input_layer_target, target_hidden_layers, false);
+    if (params.attent_params.attention_model) {
+      std::vector<const dType*> total_hs(longest_sent);
+      for (int i = 0; i < longest_sent; i++)
+        total_hs[i] = (L == 1) ? input_layer_source.nodes[i].d_h_t : source_hidden_layers[L - 2].nodes[i].d_h_t;
+      att = new attention_layer<dType>(H, minibatch_size, 0, attention_D, longest_sent, gpu, total_hs,
+                                       params.attent_params.feed_input);
+      if (L == 1)
+        input_layer_target.init_attention(att);
+      else
+        target_hidden_layers[L - 2].init_attention(att);
+      if (params.attent_params.feed_input)
+        input_layer_target.init_feed_input(L == 1 ? nullptr : &target_hidden_layers[L - 2], false);
+    }
+  }
+
+  // matrices only: the stream must stand at the first matrix (after read_model_file_info)
+  void load_weights(std::ifstream& w) {
+    if (!info.LM) {
+      input_layer_source.load_weights(w);
+      for (auto& l : source_hidden_layers) l.load_weights(w);
+    }
+    input_layer_target.load_weights(w);
+    for (auto& l : target_hidden_layers) l.load_weights(w);
+    softmax->load_weights(w);
+  }
+  // header, vocabulary blocks and matrices: a complete model file
+  void dump_weights(std::ofstream& o, bool with_header = true) {
+    if (with_header) write_model_file_info(o, info);
+    o << std::setprecision(std::numeric_limits<dType>::digits10 + 2);
+    if (!info.LM) {
+      input_layer_source.dump_weights(o);
+      for (auto& l : source_hidden_layers) l.dump_weights(o);
+    }
+    input_layer_target.dump_weights(o);
+    for (auto& l : target_hidden_layers) l.dump_weights(o);
+    softmax->dump_weights(o);
+  }
+
+  // neuralMT_model::getError(GPU = true), src/model.hpp:1463-1802: natural-log probability of the minibatch's
+  // target words.  per_step, if given, is called after each target step with (step, loss of the step).
+  double getError(minibatch_reader& mb, const std::function<void(int, double)>& per_step = nullptr) {
+    const bool seq2seq = !info.LM;
+    const int S = seq2seq ? mb.current_source_length : 0, T = mb.current_target_length;
+    const int mbs = params.minibatch_size;
+    if (seq2seq) {
+      input_layer_source.prep_GPU_vocab_indices(mb.h_input_vocab_indicies_source.data(), nullptr, S, 0);
+      for (auto& l : source_hidden_layers) l.prep_GPU_vocab_indices(mb.h_input_vocab_indicies_source.data(), S);
+      if (att) att->prep_minibatch_info(mb.h_batch_info.data());
+    }
+    input_layer_target.prep_GPU_vocab_indices(mb.h_input_vocab_indicies_target.data(), nullptr, T, 0);
+    for (auto& l : target_hidden_layers) l.prep_GPU_vocab_indices(mb.h_input_vocab_indicies_target.data(), T);
+    softmax->prep_GPU_vocab_indices(mb.h_output_vocab_indicies_target.data(), T);
+
+    for (int i = 0; i < S; i++) {
+      const int step = i * mbs;
+      auto& n0 = input_layer_source.nodes[i];
+      n0.update_vectors_forward_GPU(
+          input_layer_source.d_input_vocab_indices_full + step, input_layer_source.d_input_vocab_indices_01_full + step,
+          i == 0 ? input_layer_source.d_init_hidden_vector : input_layer_source.nodes[i - 1].d_h_t,
+          i == 0 ? input_layer_source.d_init_cell_vector : input_layer_source.nodes[i - 1].d_c_t);
+      n0.forward_prop();
+      for (auto& l : source_hidden_layers) {
+        l.nodes[i].update_vectors_forward_GPU(l.d_input_vocab_indices_01_full + step,
+                                              i == 0 ? l.d_init_hidden_vector : l.nodes[i - 1].d_h_t,
+                                              i == 0 ? l.d_init_cell_vector : l.nodes[i - 1].d_c_t);
+        l.nodes[i].forward_prop();
+      }
+    }
+    double total = 0;
+    for (int i = 0; i < T; i++) {
+      const int step = i * mbs;
+      dType *hp, *cp;
+      if (i > 0) {
+        hp = input_layer_target.nodes[i - 1].d_h_t;
+        cp = input_layer_target.nodes[i - 1].d_c_t;
+      } else if (seq2seq) {  // start from the encoder's last state (src/model.hpp:1714-1724)
+        hp = input_layer_source.nodes[S - 1].d_h_t;
+        cp = input_layer_source.nodes[S - 1].d_c_t;
+      } else {
+        hp = input_layer_target.d_init_hidden_vector;
+        cp = input_layer_target.d_init_cell_vector;
+      }
+      input_layer_target.nodes[i].update_vectors_forward_GPU(input_layer_target.d_input_vocab_indices_full + step,
+                                                             input_layer_target.d_input_vocab_indices_01_full + step,
+                                                             hp, cp);
+      input_layer_target.nodes[i].forward_prop();
+      for (size_t l = 0; l < target_hidden_layers.size(); l++) {
+        auto& ly = target_hidden_layers[l];
+        if (i > 0) {
+          hp = ly.nodes[i - 1].d_h_t;
+          cp = ly.nodes[i - 1].d_c_t;
+        } else if (seq2seq) {
+          hp = source_hidden_layers[l].nodes[S - 1].d_h_t;
+          cp = source_hidden_layers[l].nodes[S - 1].d_c_t;
+        } else {
+          hp = ly.d_init_hidden_vector;
+          cp = ly.d_init_cell_vector;
+        }
+        ly.nodes[i].update_vectors_forward_GPU(ly.d_input_vocab_indices_01_full + step, hp, cp);
+        ly.nodes[i].forward_prop();
+      }
+      softmax->backprop_prep_GPU(softmax->get_ht_ptr(i), step);
+      const double loss = softmax->compute_loss_GPU(i);
+      total += loss;
+      if (per_step) per_step(i, loss);
+    }
+    return total;
+  }
+
+  // neuralMT_model::get_perplexity (src/model.hpp:2281-2355): one getError per minibatch; with force_decode the
+  // minibatch's log-probability (natural log) goes to fd_stream, one line per minibatch.  Returns the perplexity
+  // 2^(-log2 P(data) / total_target_words).
+  double get_perplexity(const std::string& int_file, long long total_target_words, std::ostream* fd_stream,
+                        double& log_prob_total, std::string& err) {
+    minibatch_reader reader;
+    if (!reader.open(int_file, params.minibatch_size, params.longest_sent, info.LM)) {
+      err = "cannot open " + int_file;
+      return -1;
+    }
+    log_prob_total = 0;
+    while (reader.read_minibatch(err)) {
+      const double lp = getError(reader);
+      if (fd_stream) *fd_stream << std::setprecision(15) << lp << "\n";
+      log_prob_total += lp;
+    }
+    if (!err.empty()) return -1;
+    const double bits = log_prob_total / std::log(2.0);
+    return std::pow(2.0, -bits / (double)total_target_words);
+  }
+};
+
+#endif
