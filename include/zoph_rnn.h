@@ -60,7 +60,11 @@ const char* zr_version(void);
 
 #define ZR_OPT_LSTM_FUSED_EPILOGUE 1 /* 1 (default): gate maths in the GEMM epilogue; 0: GEMM then zr_lstm_gates */
 #define ZR_OPT_LSTM_TN 2             /* columns per workgroup / 32 for the fused LSTM kernel: 1, 2 or 4 (0 = auto) */
-#define ZR_OPT_GEMM_CFG 3            /* generic GEMM tile selection (0 = auto) */
+#define ZR_OPT_GEMM_CFG 3            /* generic GEMM tile selection, for tuning runs (0 = auto).  Plain weights: 1..8 =
+                                        wave tiles 64x128, 32x128, 32x64, 32x32, 32x32 K/4, 32x32 K/8, 64x64, 32x64 K/4;
+                                        9 = LDS-shared rows, 10 = LDS-shared rows with 128-row tiles.  Prepared
+                                        (k-interleaved) weights: 11 = one tile per workgroup instead of row ranges,
+                                        12..14 = tiles 128x64, 64x64, 64x128 at one workgroup per CU */
 #define ZR_OPT_LSTM_KSPLIT 4         /* waves per workgroup splitting K in the fused LSTM kernel: 4 or 8 (0 = auto) */
 #define ZR_OPT_LSTM_KERNEL 5         /* 0 auto; 1: weights streamed to registers, K split inside the workgroup;
                                         2: weights through LDS, K split across workgroups */
