@@ -1,0 +1,100 @@
+"""The beam-search translation driver (zoph_rnn_amd/host/beam_decode) end to end: model file and source text in,
+k-best hypotheses out, against one oracle decode per sentence (the reference decodes one sentence per pass).  Covers
+the C++ beam_decoder (encoder sweep, state replication, feed-input, attention, device-side beam, state reorder),
+grouping by source length, the step cap min(1.5 * source length, longest_sent - 2) and the k-best selection."""
+import numpy as np
+import pytest
+
+import model_files_util as mf
+from test_gpu_decode import _model, _oracle_decode
+from test_gpu_host_layers import _write_hh, _write_ih, _write_matrix
+from zoph_rnn_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _parse_blocks(text):
+    sents, cur = [], None
+    lines = text.split("\n")
+    i = 0
+    while i < len(lines):
+        ln = lines[i]
+        if ln.startswith("-----"):
+            cur = []
+            sents.append(cur)
+        elif ln.startswith("-Score:"):
+            score = float(ln.split()[1])
+            words = [int(x) for x in lines[i + 1].split()]
+            cur.append((words, score))
+            i += 1
+        i += 1
+    return sents
+
+
+@pytest.mark.parametrize("L,beam,batch", [(2, 4, 3), (1, 3, 8)])
+def test_beam_decode_cli_matches_per_sentence_oracle(tmp_path, L, beam, batch):
+    g = synth.rng(95, L + beam)
+    H, D, longest, K = 64, 3, 24, 3
+    src_vocab = ["<UNK>"] + mf.make_vocab(79, "s")
+    tgt_vocab = ["<START>", "<EOF>", "<UNK>"] + mf.make_vocab(397, "t")
+    Vs, Vt = len(src_vocab), len(tgt_vocab)
+    m = _model(g, H, Vs, Vt, L)
+    model = tmp_path / "model.nn"
+    with open(model, "w") as f:
+        mf.write_header(f, L, H, tgt_vocab, src_vocab, True, True)
+        _write_ih(f, m["src_layers"][0], m["src_embed"])
+        for ly in m["src_layers"][1:]:
+            _write_hh(f, ly)
+        _write_ih(f, m["tgt_layers"][0], m["tgt_embed"], m["attn"] if L == 1 else None)
+        for i, ly in enumerate(m["tgt_layers"][1:]):
+            _write_hh(f, ly, m["attn"] if i == L - 2 else None)
+        _write_matrix(f, m["D_soft"])
+        _write_matrix(f, m["b_soft"].reshape(-1, 1))
+    # sentences of three different lengths, interleaved, with unknown words
+    lens = [5, 7, 5, 4, 7, 5, 4]
+    src = [mf.random_sentences(g, src_vocab, 1, n, n)[0] for n in lens]
+    sp, out = tmp_path / "src.txt", tmp_path / "out.txt"
+    sp.write_text("".join(" ".join(s) + "\n" for s in src))
+    r = mf.run_program("beam_decode", ["--beam", beam, "--batch", batch, "--longest-sent", longest, "--attention-width",
+                                       D, "--num-best", K, "--print-score", "--ids", model, sp, out])
+    assert r.returncode == 0, r.stderr[-2000:]
+    got = _parse_blocks(out.read_text())
+    assert len(got) == len(src)
+    smap = {w: i for i, w in enumerate(src_vocab)}
+    for s, words in enumerate(src):
+        ids = np.array([smap.get(w, 0) for w in words][::-1], np.int32)
+        S = len(ids)
+        steps = min(int(1.5 * S), longest - 2)
+        _, hyps, gap = _oracle_decode(m, ids, S, S, beam, steps, D, 0.0)
+        assert gap > 5e-6, "candidate scores nearly tie (gap %.2e): pick another seed" % gap
+        keep = [(w, sc) for (w, sc) in hyps if len(w) / S > 0.5]
+        keep.sort(key=lambda t: -t[1])
+        want = keep[:K]
+        assert len(got[s]) == len(want), (s, len(got[s]), len(want))
+        for (gw, gs), (ww, ws) in zip(got[s], want):
+            assert gw == list(ww), (s, gw, list(ww))
+            assert gs == pytest.approx(ws, rel=1e-4, abs=1e-4)
+
+
+def test_beam_decode_cli_default_output_is_words(tmp_path):
+    g = synth.rng(96, 1)
+    H, L = 48, 1
+    src_vocab = ["<UNK>"] + mf.make_vocab(30, "s")
+    tgt_vocab = ["<START>", "<EOF>", "<UNK>"] + mf.make_vocab(100, "t")
+    m = _model(g, H, len(src_vocab), len(tgt_vocab), L)
+    model = tmp_path / "model.nn"
+    with open(model, "w") as f:
+        mf.write_header(f, L, H, tgt_vocab, src_vocab, True, True)
+        _write_ih(f, m["src_layers"][0], m["src_embed"])
+        _write_ih(f, m["tgt_layers"][0], m["tgt_embed"], m["attn"])
+        _write_matrix(f, m["D_soft"])
+        _write_matrix(f, m["b_soft"].reshape(-1, 1))
+    src = mf.random_sentences(g, src_vocab, 5, 3, 6)
+    sp, out = tmp_path / "src.txt", tmp_path / "out.txt"
+    sp.write_text("".join(" ".join(s) + "\n" for s in src))
+    r = mf.run_program("beam_decode", ["--beam", 3, "--batch", 2, "--longest-sent", 20, model, sp, out])
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = out.read_text().split("\n")[:-1]
+    assert len(lines) == len(src)
+    for ln in lines:
+        assert all(w in tgt_vocab[2:] for w in ln.split())  # words, no <START> / <EOF>

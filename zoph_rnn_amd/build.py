@@ -43,17 +43,26 @@ def build_hip(verbose=False, jobs=4):
 
 
 
-def build_force_decode():
-    """The force-decode / perplexity driver over text files (zoph_rnn_amd/host/force_decode), plain g++ against the
-    C-ABI."""
-    src = os.path.join(HERE, "host", "force_decode.cpp")
-    out = os.path.join(HERE, "host", "force_decode")
+def _build_host_program(name):
+    src = os.path.join(HERE, "host", name + ".cpp")
+    out = os.path.join(HERE, "host", name)
     cmd = [os.environ.get("CXX", "g++"), "-std=c++17", "-O1", "-Wall", "-o", out, src, "-L", HERE, "-lzoph_rnn_hip",
            "-Wl,-rpath,$ORIGIN/.."]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
-        raise RuntimeError("force_decode build failed:\n" + r.stdout + r.stderr)
+        raise RuntimeError(name + " build failed:\n" + r.stdout + r.stderr)
     return out
+
+
+def build_force_decode():
+    """The force-decode / perplexity driver over text files (zoph_rnn_amd/host/force_decode), plain g++ against the
+    C-ABI."""
+    return _build_host_program("force_decode")
+
+
+def build_beam_decode():
+    """The beam-search translation driver over text files (zoph_rnn_amd/host/beam_decode)."""
+    return _build_host_program("beam_decode")
 
 
 def build_host_driver():

@@ -1,0 +1,159 @@
+// Beam-search translation driver over text files: what `ZOPH_RNN --decode` does for one model
+// (ensemble_factory::decode_file_batch, src/ensemble_factory.hpp:583-765; k-best selection and output
+// decoder::output_k_best_hypotheses, src/decoder.h:1386-1480), on the MI355X path, several sentences at a time.
+//
+//   beam_decode [options] model.nn source.txt output.txt
+//
+// source.txt holds one tokenised sentence per line.  Sentences are integerized with the model's source vocabulary
+// (reversed, <UNK> for unknown words), grouped by source length (sentences decoded side by side must have one
+// length, so that every sentence gets exactly the number of steps the reference would give it: min(max-ratio *
+// source length, longest-sent - 2)) and written in input order.
+// Default output: the best hypothesis of each sentence as words, one line per sentence, <START> / <EOF> stripped.
+// With --num-best K > 1 or --print-score: the reference's block layout, a line of dashes per sentence, then per
+// hypothesis an optional "-Score: s" line and the hypothesis (ids with --ids, <START> and <EOF> included, as the
+// reference's integer output; words otherwise).
+//
+// Options: --beam B (12)  --batch N (16 sentences side by side)  --longest-sent L (100)  --attention-width D (10)
+//          --penalty P (0)  --min-ratio R (0.5)  --max-ratio R (1.5)  --num-best K (1)  --print-score  --ids  --bf16
+#include <cstdio>
+#include <cstdlib>
+#include <iostream>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "zoph_model.h"
+
+static int usage(const char* argv0) {
+  std::fprintf(stderr,
+               "usage: %s [--beam B] [--batch N] [--longest-sent L] [--attention-width D] [--penalty P]\n"
+               "          [--min-ratio R] [--max-ratio R] [--num-best K] [--print-score] [--ids] [--bf16]\n"
+               "          model.nn source.txt output.txt\n",
+               argv0);
+  return 2;
+}
+
+int main(int argc, char** argv) {
+  int beam = 12, batch = 16, longest = 100, D = 10, num_best = 1;
+  double penalty = 0, min_ratio = 0.5, max_ratio = 1.5;
+  bool print_score = false, ids_out = false, bf16 = false;
+  std::vector<std::string> pos;
+  for (int i = 1; i < argc; i++) {
+    const std::string a = argv[i];
+    auto geti = [&](int& dst) {
+      if (i + 1 >= argc) return false;
+      dst = std::atoi(argv[++i]);
+      return dst > 0;
+    };
+    auto getd = [&](double& dst) {
+      if (i + 1 >= argc) return false;
+      dst = std::atof(argv[++i]);
+      return true;
+    };
+    if (a == "--beam") { if (!geti(beam)) return usage(argv[0]); }
+    else if (a == "--batch") { if (!geti(batch)) return usage(argv[0]); }
+    else if (a == "--longest-sent") { if (!geti(longest)) return usage(argv[0]); }
+    else if (a == "--attention-width") { if (!geti(D)) return usage(argv[0]); }
+    else if (a == "--num-best") { if (!geti(num_best)) return usage(argv[0]); }
+    else if (a == "--penalty") { if (!getd(penalty)) return usage(argv[0]); }
+    else if (a == "--min-ratio") { if (!getd(min_ratio)) return usage(argv[0]); }
+    else if (a == "--max-ratio") { if (!getd(max_ratio)) return usage(argv[0]); }
+    else if (a == "--print-score") print_score = true;
+    else if (a == "--ids") ids_out = true;
+    else if (a == "--bf16") bf16 = true;
+    else if (a.rfind("--", 0) == 0) return usage(argv[0]);
+    else pos.push_back(a);
+  }
+  if (pos.size() != 3 || beam > 31) return usage(argv[0]);
+
+  std::ifstream model(pos[0]);
+  if (!model) {
+    std::fprintf(stderr, "cannot open %s\n", pos[0].c_str());
+    return 1;
+  }
+  model_file_info info;
+  std::string err;
+  if (!read_model_file_info(model, false, info, err)) {
+    std::fprintf(stderr, "%s: %s\n", pos[0].c_str(), err.c_str());
+    return 1;
+  }
+  // integerize the source side: vocabulary lookup, reversed (src/input_file_prep.h:405-416)
+  std::unordered_map<std::string, int> smap;
+  for (size_t i = 0; i < info.source_vocab.size(); i++) smap[info.source_vocab[i]] = (int)i;
+  const int unk = smap.count("<UNK>") ? smap["<UNK>"] : 0;
+  std::ifstream src(pos[1]);
+  if (!src) {
+    std::fprintf(stderr, "cannot open %s\n", pos[1].c_str());
+    return 1;
+  }
+  std::vector<std::vector<int>> sents;
+  std::string line;
+  while (std::getline(src, line)) {
+    std::vector<int> v;
+    for (const auto& w : zoph_split_words(line)) v.push_back(smap.count(w) ? smap[w] : unk);
+    std::reverse(v.begin(), v.end());
+    if (v.empty() || (int)v.size() > longest - 2) {
+      std::fprintf(stderr, "source sentence %zu is empty or longer than longest-sent - 2\n", sents.size() + 1);
+      return 1;
+    }
+    sents.push_back(v);
+  }
+  std::map<int, std::vector<int>> by_len;  // source length -> sentence numbers, in input order
+  for (size_t i = 0; i < sents.size(); i++) by_len[(int)sents[i].size()].push_back((int)i);
+
+  BZ_CUDA::bf16_weights = bf16;
+  layer_gpu_info gpu;
+  gpu.init(0);
+  forward_model<precision> m;
+  m.initModel(gpu, info, 1, longest, D);
+  m.load_weights(model);
+  beam_decoder<precision> dec(m, beam, batch, longest, D, penalty);
+  dec.min_decoding_ratio = min_ratio;
+  dec.max_decoding_ratio = max_ratio;
+
+  std::vector<std::vector<decoded_hypothesis>> results(sents.size());
+  for (const auto& kv : by_len) {
+    const auto& idx = kv.second;
+    for (size_t base = 0; base < idx.size(); base += batch) {
+      std::vector<std::vector<int>> group;
+      for (size_t j = base; j < std::min(idx.size(), base + (size_t)batch); j++) group.push_back(sents[idx[j]]);
+      std::vector<std::vector<decoded_hypothesis>> out;
+      dec.decode_batch(group, num_best, out);
+      for (size_t j = 0; j < group.size(); j++) results[idx[base + j]] = out[j];
+    }
+  }
+
+  std::ofstream out(pos[2]);
+  if (!out) {
+    std::fprintf(stderr, "cannot write %s\n", pos[2].c_str());
+    return 1;
+  }
+  auto put = [&](const decoded_hypothesis& h, bool strip) {
+    bool first = true;
+    for (int w : h.words) {
+      if (strip && (w == 0 || w == 1)) continue;
+      if (!first) out << " ";
+      first = false;
+      if (ids_out)
+        out << w;
+      else
+        out << (w >= 0 && w < (int)info.target_vocab.size() ? info.target_vocab[w] : "<UNK>");
+    }
+    out << "\n";
+  };
+  const bool blocks = num_best > 1 || print_score;
+  for (const auto& r : results) {
+    if (!blocks) {
+      if (r.empty()) out << "\n"; else put(r[0], true);
+      continue;
+    }
+    out << "------------------------------------------------\n";
+    for (const auto& h : r) {
+      if (print_score) out << "-Score: " << h.score << "\n";
+      put(h, false);
+    }
+    out << "\n";
+  }
+  std::cout << "Sentences: " << sents.size() << "\n";
+  return 0;
+}

@@ -18,6 +18,8 @@
 
 #include <algorithm>
 #include <cmath>
+#include <cstdio>
+#include <cstdlib>
 #include <fstream>
 #include <functional>
 #include <iomanip>
@@ -557,6 +559,220 @@ class forward_model {
     if (!err.empty()) return -1;
     const double bits = log_prob_total / std::log(2.0);
     return std::pow(2.0, -bits / (double)total_target_words);
+  }
+};
+
+// ------------------------------------------------------------------------------------------------ beam decoding
+// Batched beam-search decode on top of a loaded forward_model: what ensemble_factory::decode_file_batch
+// (src/ensemble_factory.hpp:583-765) does with decoder_model_wrapper::forward_prop_source / forward_prop_target /
+// swap_decoding_states (src/decoder_model_wrapper.hpp, src/model.hpp:2367-2726) and decoder<dType>
+// (src/decoder.h:1158-1413), for n_sent sentences of equal source length side by side.  Columns
+// [s*beam, (s+1)*beam) of every LSTM_size x (n_sent*beam) activation belong to sentence s; the probabilities feed the
+// device-side beam directly, so nothing vocabulary-sized is copied to the host.  As in the reference's decode path
+// every column runs with mask 1 and a dead beam slot (-1) is fed as word 0.
+struct decoded_hypothesis {
+  std::vector<int> words;  // target ids, <START> ... <EOF>
+  float score = 0;
+};
+
+template <typename dType>
+class beam_decoder {
+ public:
+  forward_model<dType>& m;
+  zr_ctx* ctx;
+  int beam, n_sent, cols, longest_sent, D, H, L, Vs, Vt;
+  double penalty, min_decoding_ratio = 0.5, max_decoding_ratio = 1.5;
+  bool attention, feed_input;
+  zr_attn* attn = nullptr;
+  zr_beam* bm = nullptr;
+  std::vector<dType*> tables;                 // longest_sent source top-layer states, H x cols
+  std::vector<dType*> h[2], c[2];             // ping-pong: previous / new state per layer
+  dType *h_tild[2] = {nullptr, nullptr}, *x = nullptr, *prob = nullptr, *zeros = nullptr;
+  std::vector<dType*> enc_h, enc_c;           // encoder sweep outputs per layer, longest_sent * H * n_sent
+  int *d_words = nullptr, *d_words_nn = nullptr, *d_back = nullptr, *d_ones = nullptr, *d_batch_info = nullptr,
+      *d_src = nullptr, *d_src_nn = nullptr, *d_src_mask = nullptr, *d_rep = nullptr;
+  std::vector<const zr_lstm_weights*> src_w, tgt_w;
+
+  template <typename T>
+  T* dmalloc(size_t n) {
+    T* p = nullptr;
+    ZOPH_CALL(zr_malloc(ctx, n * sizeof(T), (void**)&p));
+    return p;
+  }
+
+  beam_decoder(forward_model<dType>& model, int beam, int n_sent, int longest_sent, int attention_D, double penalty)
+      : m(model), ctx(model.gpu.ctx), beam(beam), n_sent(n_sent), cols(beam * n_sent), longest_sent(longest_sent),
+        D(attention_D), penalty(penalty) {
+    if (m.info.LM) {
+      std::fprintf(stderr, "beam_decoder: a sequence model has no source side to decode from\n");
+      std::exit(EXIT_FAILURE);
+    }
+    H = m.info.LSTM_size;
+    L = m.info.num_layers;
+    Vs = m.info.source_vocab_size;
+    Vt = m.info.target_vocab_size;
+    attention = m.params.attent_params.attention_model;
+    feed_input = m.params.attent_params.feed_input;
+    m.input_layer_source.repack();
+    m.input_layer_target.repack();
+    src_w.push_back(m.input_layer_source.packed);
+    tgt_w.push_back(m.input_layer_target.packed);
+    for (int l = 0; l + 1 < L; l++) {
+      m.source_hidden_layers[l].repack();
+      m.target_hidden_layers[l].repack();
+      src_w.push_back(m.source_hidden_layers[l].packed);
+      tgt_w.push_back(m.target_hidden_layers[l].packed);
+    }
+    const size_t n = (size_t)H * cols;
+    for (int i = 0; i < 2; i++) {
+      for (int l = 0; l < L; l++) {
+        h[i].push_back(dmalloc<dType>(n));
+        c[i].push_back(dmalloc<dType>(n));
+      }
+      h_tild[i] = dmalloc<dType>(n);
+    }
+    x = dmalloc<dType>(n);
+    prob = dmalloc<dType>((size_t)Vt * cols);
+    zeros = dmalloc<dType>((size_t)H * n_sent);
+    ZOPH_CALL(zr_memset_zero(ctx, zeros, (size_t)H * n_sent * sizeof(dType)));
+    for (int l = 0; l < L; l++) {
+      enc_h.push_back(dmalloc<dType>((size_t)longest_sent * H * n_sent));
+      enc_c.push_back(dmalloc<dType>((size_t)longest_sent * H * n_sent));
+    }
+    d_words = dmalloc<int>(cols);
+    d_words_nn = dmalloc<int>(cols);
+    d_back = dmalloc<int>(cols);
+    d_ones = dmalloc<int>(cols);
+    d_batch_info = dmalloc<int>(2 * (size_t)cols);
+    d_src = dmalloc<int>((size_t)longest_sent * n_sent);
+    d_src_nn = dmalloc<int>((size_t)longest_sent * n_sent);
+    d_src_mask = dmalloc<int>((size_t)longest_sent * n_sent);
+    d_rep = dmalloc<int>(cols);
+    std::vector<int> ones(cols, 1), rep(cols);
+    for (int i = 0; i < cols; i++) rep[i] = i / beam;
+    ZOPH_CALL(zr_h2d(ctx, d_ones, ones.data(), cols * sizeof(int)));
+    ZOPH_CALL(zr_h2d(ctx, d_rep, rep.data(), cols * sizeof(int)));
+    if (attention) {
+      std::vector<const dType*> tp;
+      for (int t = 0; t < longest_sent; t++) {
+        tables.push_back(dmalloc<dType>(n));
+        tp.push_back(tables.back());
+      }
+      auto* a = m.att;
+      ZOPH_CALL(zr_attn_create(ctx, H, cols, D, a->d_W_a, a->d_W_p, a->d_v_p, a->d_output_bias, a->d_W_c_p1,
+                               a->d_W_c_p2, tp.data(), longest_sent, &attn));
+      if (BZ_CUDA::bf16_weights) ZOPH_CALL(zr_attn_use_bf16_weights(ctx, attn));
+    }
+    ZOPH_CALL(zr_beam_create(ctx, beam, Vt, n_sent, longest_sent + 3, (float)penalty, &bm));
+  }
+
+  // forward_prop_target (src/model.hpp:2573-2688): state half p -> half q, probabilities into prob
+  void forward_target(int p, int step_index) {
+    const int q = 1 - p;
+    ZOPH_CALL(zr_vocab_prep(ctx, d_words, cols, Vt, d_words_nn, nullptr));
+    ZOPH_CALL(zr_embed_gather(ctx, m.input_layer_target.d_W, H, Vt, d_words_nn, cols, x));
+    const dType* below = x;
+    for (int l = 0; l < L; l++) {
+      const dType* feed = (l == 0 && feed_input && step_index > 0) ? h_tild[p] : nullptr;
+      ZOPH_CALL(zr_lstm_step(ctx, tgt_w[l], below, h[p][l], c[p][l], feed, d_ones, 0.0f, cols, h[q][l], c[q][l], nullptr));
+      below = h[q][l];
+    }
+    const dType* top = below;
+    if (attention) {
+      ZOPH_CALL(zr_attn_step(ctx, attn, d_batch_info, below, d_ones, h_tild[q], nullptr, nullptr, nullptr, nullptr));
+      top = h_tild[q];
+    }
+    ZOPH_CALL(zr_softmax_forward(ctx, m.softmax_obj.d_D, m.softmax_obj.d_b_d, Vt, H, top, cols, ZR_SOFTMAX_PROB, prob,
+                                 nullptr));
+  }
+
+  // Decodes up to n_sent sentences whose integerized sources (reversed, no padding) all have the same length S.
+  // out[s] receives the num_best best finished hypotheses of sentence s, best first
+  // (decoder::output_k_best_hypotheses, src/decoder.h:1386-1413).
+  void decode_batch(const std::vector<std::vector<int>>& sources, int num_best,
+                    std::vector<std::vector<decoded_hypothesis>>& out) {
+    const int real = (int)sources.size();
+    const int S = (int)sources[0].size();
+    if (real < 1 || real > n_sent || S < 1 || S > longest_sent) {
+      std::fprintf(stderr, "beam_decoder::decode_batch: %d sentences of source length %d do not fit\n", real, S);
+      std::exit(EXIT_FAILURE);
+    }
+    // time-major ids; a short batch is completed with copies of its first sentence (results ignored)
+    std::vector<int> ids((size_t)S * n_sent);
+    for (int s = 0; s < n_sent; s++) {
+      const auto& src = sources[s < real ? s : 0];
+      if ((int)src.size() != S) {
+        std::fprintf(stderr, "beam_decoder::decode_batch: sentences of one batch must have one source length\n");
+        std::exit(EXIT_FAILURE);
+      }
+      for (int t = 0; t < S; t++) ids[s + (size_t)t * n_sent] = src[t];
+    }
+    ZOPH_CALL(zr_h2d(ctx, d_src, ids.data(), ids.size() * sizeof(int)));
+    ZOPH_CALL(zr_vocab_prep(ctx, d_src, (int)ids.size(), Vs, d_src_nn, d_src_mask));
+    std::vector<const dType*> z(L, zeros);
+    ZOPH_CALL(zr_lstm_stack_forward(ctx, L, src_w.data(), m.input_layer_source.d_W, Vs, d_src_nn, d_src_mask, S, n_sent,
+                                    z.data(), z.data(), 0.0f, enc_h.data(), enc_c.data()));
+    // every sentence's states replicated over its beam columns (forward_prop_source, src/model.hpp:2394-2445, and
+    // transfer_decoding_states_GPU for the final state of each layer)
+    const size_t hn = (size_t)H * n_sent;
+    if (attention)
+      for (int t = 0; t < S; t++) ZOPH_CALL(zr_gather_columns(ctx, enc_h[L - 1] + t * hn, H, d_rep, cols, tables[t]));
+    for (int l = 0; l < L; l++) {
+      ZOPH_CALL(zr_gather_columns(ctx, enc_h[l] + (S - 1) * hn, H, d_rep, cols, h[0][l]));
+      ZOPH_CALL(zr_gather_columns(ctx, enc_c[l] + (S - 1) * hn, H, d_rep, cols, c[0][l]));
+    }
+    std::vector<int> binfo(2 * (size_t)cols);
+    for (int i = 0; i < cols; i++) {
+      binfo[i] = S;  // unpadded sources of equal length: full length, no offset
+      binfo[i + cols] = 0;
+    }
+    ZOPH_CALL(zr_h2d(ctx, d_batch_info, binfo.data(), binfo.size() * sizeof(int)));
+    std::vector<int> start(cols, 0);  // <START>
+    ZOPH_CALL(zr_h2d(ctx, d_words, start.data(), cols * sizeof(int)));
+    ZOPH_CALL(zr_beam_init(ctx, bm));
+
+    const int steps = std::min((int)(max_decoding_ratio * S), longest_sent - 2);
+    int p = 0, index = 0;
+    for (; index < steps; index++) {
+      forward_target(p, index);
+      ZOPH_CALL(zr_beam_expand(ctx, bm, prob, index, d_words, d_back));
+      // swap_decoding_states + target_copy_prev_states (src/model.hpp:2691-2726)
+      const int q = 1 - p;
+      for (int l = 0; l < L; l++) {
+        ZOPH_CALL(zr_gather_columns(ctx, h[q][l], H, d_back, cols, h[p][l]));
+        ZOPH_CALL(zr_gather_columns(ctx, c[q][l], H, d_back, cols, c[p][l]));
+      }
+      if (attention) ZOPH_CALL(zr_gather_columns(ctx, h_tild[q], H, d_back, cols, h_tild[p]));
+    }
+    // one last step and forced <EOF> on every live hypothesis (src/ensemble_factory.hpp:727-743)
+    forward_target(p, index);
+    ZOPH_CALL(zr_beam_finish(ctx, bm, prob));
+    ZOPH_CALL(zr_ctx_sync(ctx));
+
+    out.assign(real, {});
+    const int cap = 4 * beam * (steps + 2), max_len = longest_sent + 3;
+    std::vector<int> words((size_t)cap * max_len), lens(cap);
+    std::vector<float> scores(cap);
+    for (int s = 0; s < real; s++) {
+      int n = zr_beam_hypotheses(ctx, bm, s, cap, words.data(), lens.data(), scores.data());
+      if (n < 0) {
+        std::fprintf(stderr, "zr_beam_hypotheses failed: %s\n", zr_last_error());
+        std::exit(EXIT_FAILURE);
+      }
+      n = std::min(n, cap);
+      // output_k_best_hypotheses: length ratio filter, then the num_best best scores, best first
+      std::vector<int> order;
+      for (int i = 0; i < n; i++)
+        if ((float)lens[i] / (float)S > (float)min_decoding_ratio) order.push_back(i);
+      std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return scores[a] > scores[b]; });
+      if ((int)order.size() > num_best) order.resize(num_best);
+      for (int i : order) {
+        decoded_hypothesis hyp;
+        hyp.words.assign(words.begin() + (size_t)i * max_len, words.begin() + (size_t)i * max_len + lens[i]);
+        hyp.score = scores[i];
+        out[s].push_back(hyp);
+      }
+    }
   }
 };
 
