@@ -664,3 +664,170 @@ void orc_lstm_stack_forward(int acc64, int L, int H, int mb, int T, int V, const
 }
 
 }  // extern "C"
+
+// ---------------------------------------------------------------------------------------------------------
+// Backward pass (training).  Gradients are those of the LOG-LIKELIHOOD (the reference ascends: its softmax error
+// is D^T (onehot - p), src/softmax.hpp:700-712, and update_weights adds learning_rate * gradient, :232-300).
+// ---------------------------------------------------------------------------------------------------------
+namespace {
+
+// C(MxN) = A * B^T with A stored M x K and B stored N x K (cublasSgemm OP_N, OP_T: the weight-gradient products,
+// e.g. src/LSTM.hpp:1026-1100).  Always double accumulation.
+void gemm_nt64(int M, int N, int K, const float* A, int lda, const float* B, int ldb, double* C, int ldc, bool add) {
+#pragma omp parallel for schedule(static) collapse(2)
+  for (int n = 0; n < N; ++n)
+    for (int m = 0; m < M; ++m) {
+      double s = 0;
+      for (int k = 0; k < K; ++k) s += (double)A[IDX2C(m, k, lda)] * (double)B[IDX2C(n, k, ldb)];
+      if (add)
+        C[IDX2C(m, n, ldc)] += s;
+      else
+        C[IDX2C(m, n, ldc)] = s;
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+// One node's element-wise backward.  d_ERRt_ct_kernel, d_ERRnTOt_ot_kernel, d_ERRnTOt_ft_it_kernel,
+// d_ERRnTOt_tanhcpt_kernel and zero_columns_kernel (src/custom_kernels.h:199-262), in the order of
+// LSTM_IH_Node::back_prop_GPU (src/LSTM.hpp:542-700).
+//   err_h: d_ERRnTOtp1_ht + d_ERRt_ht, the total error arriving at h_t; err_c_next: d_ERRnTOtp1_ct.
+//   gates i, f, c~ (tanh), o and c_t, c_{t-1} as saved by the forward step.
+//   Outputs: dgate[4] = error at the four PRE-activations (the reference's d_ERRnTOt_it, _ft, _tanhcpt, _ot), gate
+//   order i,f,c,o; err_cprev = error passed to c_{t-1} (d_ERRnTOt_ct * f_t).
+void orc_lstm_step_backward(int H, int mb, const float* gi, const float* gf, const float* gc, const float* go,
+                            const float* c, const float* cprev, const int* mask01, const float* err_h,
+                            const float* err_c_next, float* dgate_i, float* dgate_f, float* dgate_c, float* dgate_o,
+                            float* err_cprev) {
+  for (int col = 0; col < mb; ++col)
+    for (int i = 0; i < H; ++i) {
+      const size_t ix = IDX2C(i, col, H);
+      const float m = (float)mask01[col];
+      const float eh = err_h[ix] * m;  // zero_columns_kernel on d_ERRnTOt_ht
+      const float th = tanhf(c[ix]);
+      const float errt_ct = eh * go[ix] * (1.0f - th * th);                      // d_ERRt_ct_kernel
+      const float ec = ((err_c_next ? err_c_next[ix] : 0.0f) + errt_ct) * m;     // d_ERRnTOt_ct, zero_columns_kernel
+      dgate_o[ix] = eh * th * go[ix] * (1.0f - go[ix]);                           // d_ERRnTOt_ot_kernel
+      dgate_f[ix] = ec * cprev[ix] * gf[ix] * (1.0f - gf[ix]);                    // d_ERRnTOt_ft_it_kernel
+      dgate_i[ix] = ec * gc[ix] * gi[ix] * (1.0f - gi[ix]);                       // d_ERRnTOt_ft_it_kernel
+      dgate_c[ix] = ec * gi[ix] * (1.0f - gc[ix] * gc[ix]);                       // d_ERRnTOt_tanhcpt_kernel
+      err_cprev[ix] = ec * gf[ix];                                                // elementwise_mult (:750-760)
+    }
+}
+
+// Forward sweep with saved gates, then back-propagation through time of the stacked LSTM (no attention, no dropout):
+// the loops of neuralMT_model::compute_gradients (src/model.hpp:1823-2000) over LSTM_IH_Node / LSTM_HH_Node
+// back_prop_GPU and compute_gradients_GPU (src/LSTM.hpp:542-1270, src/LSTM_HH.hpp:336-900).
+//   weights as in orc_lstm_stack_forward.  err_top: T x (H*mb), error arriving at the top layer's h_t from the
+//   loss layer (d_ERRt_ht).  err_hT / err_cT: L x (H*mb) errors arriving at the last time step from beyond (NULL = 0).
+//   Outputs (double accumulation, rounded once): grads[l][0..3] = dM_g, [4..7] = dWh_g (H x H), [8..11] = db_g (H);
+//   d_embed: H x V dense (zero where no token hit); err_h0 / err_c0: L x (H*mb) errors at the initial states.
+void orc_lstm_stack_backward(int L, int H, int mb, int T, int V, const float* embed, const float* const* weights,
+                             const int* ids_nonneg, const int* mask01, const float* h0, const float* c0,
+                             const float* err_top, const float* err_hT, const float* err_cT, float* const* grads,
+                             float* d_embed, float* err_h0, float* err_c0) {
+  const size_t n = (size_t)H * mb;
+  const size_t LT = (size_t)L * T;
+  std::vector<float> h_all(LT * n), c_all(LT * n), g_all(LT * 4 * n), x_all((size_t)T * n);
+  // forward, keeping the gates
+  for (int t = 0; t < T; ++t)
+    for (int l = 0; l < L; ++l) {
+      const float* const* w = weights + (size_t)l * 12;
+      const float* in;
+      if (l == 0) {
+        orc_embed_gather(embed, H, V, ids_nonneg + (size_t)t * mb, mb, x_all.data() + (size_t)t * n);
+        in = x_all.data() + (size_t)t * n;
+      } else {
+        in = h_all.data() + ((size_t)(l - 1) * T + t) * n;
+      }
+      const float* hp = (t == 0) ? h0 + (size_t)l * n : h_all.data() + ((size_t)l * T + t - 1) * n;
+      const float* cp = (t == 0) ? c0 + (size_t)l * n : c_all.data() + ((size_t)l * T + t - 1) * n;
+      float* g = g_all.data() + ((size_t)l * T + t) * 4 * n;
+      orc_lstm_step(1, H, mb, w, w + 4, nullptr, w + 8, in, hp, cp, nullptr, mask01 + (size_t)t * mb, 0, 0.0f, g,
+                    g + n, g + 2 * n, g + 3 * n, c_all.data() + ((size_t)l * T + t) * n,
+                    h_all.data() + ((size_t)l * T + t) * n);
+    }
+  // backward
+  std::vector<double> acc((size_t)L * 8 * H * H, 0.0), accb((size_t)L * 4 * H, 0.0), acce((size_t)H * V, 0.0);
+  std::vector<float> eh_next((size_t)L * n, 0.0f), ec_next((size_t)L * n, 0.0f);  // from t+1, per layer
+  if (err_hT) memcpy(eh_next.data(), err_hT, sizeof(float) * L * n);
+  if (err_cT) memcpy(ec_next.data(), err_cT, sizeof(float) * L * n);
+  std::vector<float> below(n), eh(n), dg(4 * n), ecp(n), tmp(n);
+  for (int t = T - 1; t >= 0; --t) {
+    std::fill(below.begin(), below.end(), 0.0f);
+    for (int l = L - 1; l >= 0; --l) {
+      const float* const* w = weights + (size_t)l * 12;
+      const float* g = g_all.data() + ((size_t)l * T + t) * 4 * n;
+      const float* cp = (t == 0) ? c0 + (size_t)l * n : c_all.data() + ((size_t)l * T + t - 1) * n;
+      const float* hp = (t == 0) ? h0 + (size_t)l * n : h_all.data() + ((size_t)l * T + t - 1) * n;
+      const float* in = (l == 0) ? x_all.data() + (size_t)t * n : h_all.data() + ((size_t)(l - 1) * T + t) * n;
+      // total error at h_t: from t+1 plus from above (the loss layer for the top layer)
+      const float* from_above = (l == L - 1) ? err_top + (size_t)t * n : below.data();
+      for (size_t i = 0; i < n; ++i) eh[i] = eh_next[(size_t)l * n + i] + from_above[i];
+      orc_lstm_step_backward(H, mb, g, g + n, g + 2 * n, g + 3 * n, c_all.data() + ((size_t)l * T + t) * n, cp,
+                             mask01 + (size_t)t * mb, eh.data(), ec_next.data() + (size_t)l * n, dg.data(),
+                             dg.data() + n, dg.data() + 2 * n, dg.data() + 3 * n, ecp.data());
+      memcpy(ec_next.data() + (size_t)l * n, ecp.data(), sizeof(float) * n);
+      // errors to h_{t-1} and to the layer below: sum over the gates of W^T dgate
+      std::fill(eh_next.begin() + (size_t)l * n, eh_next.begin() + (size_t)(l + 1) * n, 0.0f);
+      std::fill(below.begin(), below.end(), 0.0f);
+      for (int q = 0; q < 4; ++q) {
+        gemm_tn(1, H, mb, H, w[4 + q], H, dg.data() + (size_t)q * n, H, tmp.data(), H);
+        for (size_t i = 0; i < n; ++i) eh_next[(size_t)l * n + i] += tmp[i];
+        gemm_tn(1, H, mb, H, w[q], H, dg.data() + (size_t)q * n, H, tmp.data(), H);
+        for (size_t i = 0; i < n; ++i) below[i] += tmp[i];
+        // weight gradients: dM_g += dgate x^T, dWh_g += dgate h_{t-1}^T, db_g += row sums
+        gemm_nt64(H, H, mb, dg.data() + (size_t)q * n, H, in, H, acc.data() + ((size_t)l * 8 + q) * H * H, H, true);
+        gemm_nt64(H, H, mb, dg.data() + (size_t)q * n, H, hp, H, acc.data() + ((size_t)l * 8 + 4 + q) * H * H, H, true);
+        for (int col = 0; col < mb; ++col)
+          for (int i = 0; i < H; ++i) accb[((size_t)l * 4 + q) * H + i] += dg[(size_t)q * n + IDX2C(i, col, H)];
+      }
+      if (l == 0) {  // sparse embedding gradient (W_gradient kernels, src/custom_kernels.h:1297-1390), dense here
+        for (int col = 0; col < mb; ++col) {
+          if (mask01[(size_t)t * mb + col] != 1) continue;
+          const int id = ids_nonneg[(size_t)t * mb + col];
+          for (int i = 0; i < H; ++i) acce[IDX2C(i, id, H)] += below[IDX2C(i, col, H)];
+        }
+      }
+    }
+  }
+  for (int l = 0; l < L; ++l) {
+    for (int q = 0; q < 8; ++q)
+      for (size_t i = 0; i < (size_t)H * H; ++i) grads[(size_t)l * 12 + q][i] = (float)acc[((size_t)l * 8 + q) * H * H + i];
+    for (int q = 0; q < 4; ++q)
+      for (int i = 0; i < H; ++i) grads[(size_t)l * 12 + 8 + q][i] = (float)accb[((size_t)l * 4 + q) * H + i];
+  }
+  for (size_t i = 0; i < (size_t)H * V; ++i) d_embed[i] = (float)acce[i];
+  memcpy(err_h0, eh_next.data(), sizeof(float) * L * n);
+  memcpy(err_c0, ec_next.data(), sizeof(float) * L * n);
+}
+
+// Loss-layer backward for one step: softmax_layer::get_h_t_gradient_GPU, compute_D_gradient_GPU and
+// compute_b_d_gradient_GPU (src/softmax.hpp:700-860).  With p = softmax(D h + b) per column and e = onehot(target) - p
+// on unmasked columns (0 on masked ones):  err_h = D^T e (H x mb),  dD += e h^T (V x H),  db += row sums of e.
+// dD / db accumulate (double) across calls when `add` is set.
+void orc_softmax_backward(const float* D, const float* b_d, int V, int H, const float* h, int mb, const int* target,
+                          const int* mask01, int add, float* err_h, double* dD, double* db) {
+  std::vector<float> logits((size_t)V * mb), e((size_t)V * mb);
+  std::vector<double> logp((size_t)V * mb);
+  orc_softmax_logits(1, D, b_d, V, H, h, mb, logits.data());
+  orc_softmax_logprob_f64(logits.data(), V, mb, logp.data());
+  for (int col = 0; col < mb; ++col)
+    for (int v = 0; v < V; ++v) {
+      const size_t ix = IDX2C(v, col, V);
+      double val = -exp(logp[ix]);
+      if (v == target[col]) val += 1.0;
+      e[ix] = mask01[col] == 1 ? (float)val : 0.0f;
+    }
+  gemm_tn(1, H, mb, V, D, V, e.data(), V, err_h, H);
+  gemm_nt64(V, H, mb, e.data(), V, h, H, dD, V, add != 0);
+  for (int v = 0; v < V; ++v) {
+    double s = 0;
+    for (int col = 0; col < mb; ++col) s += e[IDX2C(v, col, V)];
+    db[v] = add ? db[v] + s : s;
+  }
+}
+
+}  // extern "C"

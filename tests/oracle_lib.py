@@ -299,3 +299,84 @@ class Decoder:
         idx = np.empty(max(num_hypotheses, 1), dtype=np.int32)
         n = lib().orc_decoder_k_best(self.h, source_length, num_hypotheses, _p(idx, i32p))
         return idx[:n].copy()
+
+
+def lstm_step_backward(gates, c, cprev, mask01, err_h, err_c_next=None):
+    """gates: dict with i, f, c_tilde, o (H x mb).  Returns dgate dict (i, f, c, o pre-activation errors) and
+    err_cprev."""
+    gi, gf, gc, go = (F(gates[k]) for k in ("i", "f", "c_tilde", "o"))
+    c, cprev, err_h = F(c), F(cprev), F(err_h)
+    H, mb = c.shape
+    mask01 = np.ascontiguousarray(mask01, dtype=np.int32)
+    ecn = F(err_c_next) if err_c_next is not None else None
+    outs = [np.empty((H, mb), dtype=np.float32, order="F") for _ in range(5)]
+    lib().orc_lstm_step_backward(C.c_int(H), C.c_int(mb), _p(gi), _p(gf), _p(gc), _p(go), _p(c), _p(cprev),
+                                 _p(mask01, i32p), _p(err_h), _p(ecn) if ecn is not None else None,
+                                 *[_p(a) for a in outs])
+    return {"i": outs[0], "f": outs[1], "c": outs[2], "o": outs[3]}, outs[4]
+
+
+def lstm_stack_backward(embed, layers, ids_nonneg, mask01, err_top, h0=None, c0=None, err_hT=None, err_cT=None):
+    """Back-propagation through time of the stacked LSTM (gradients of a loss whose derivative with respect to the top
+    layer's h_t is err_top[t], H x mb each).  Returns (grads, d_embed, err_h0, err_c0): grads[l] = dict with dM, dWh
+    (lists of 4 H x H) and db (list of 4 H); d_embed H x V; err_h0 / err_c0 lists of L (H x mb)."""
+    embed = F(embed)
+    H, V = embed.shape
+    ids_nonneg = np.ascontiguousarray(ids_nonneg, dtype=np.int32)
+    mask01 = np.ascontiguousarray(mask01, dtype=np.int32)
+    T, mb = ids_nonneg.shape
+    L = len(layers)
+    n = H * mb
+    keep = []
+    wptrs = (f32p * (12 * L))()
+    gptrs = (f32p * (12 * L))()
+    gmats = []
+    for l, ly in enumerate(layers):
+        mats = [F(m) for m in ly["M"]] + [F(m) for m in ly["Wh"]] + \
+               [np.ascontiguousarray(v, dtype=np.float32) for v in ly["b"]]
+        keep.append(mats)
+        gl = [np.zeros((H, H), dtype=np.float32, order="F") for _ in range(8)] + \
+             [np.zeros(H, dtype=np.float32) for _ in range(4)]
+        gmats.append(gl)
+        for j in range(12):
+            wptrs[12 * l + j] = _p(mats[j])
+            gptrs[12 * l + j] = _p(gl[j])
+
+    def flat(arrs):
+        if arrs is None:
+            return np.zeros(L * n, dtype=np.float32)
+        return np.concatenate([F(a).reshape(-1, order="F") for a in arrs])
+
+    h0f, c0f = flat(h0), flat(c0)
+    ehT = flat(err_hT) if err_hT is not None else None
+    ecT = flat(err_cT) if err_cT is not None else None
+    et = np.concatenate([F(err_top[t]).reshape(-1, order="F") for t in range(T)])
+    d_embed = np.zeros((H, V), dtype=np.float32, order="F")
+    eh0, ec0 = np.empty(L * n, dtype=np.float32), np.empty(L * n, dtype=np.float32)
+    lib().orc_lstm_stack_backward(C.c_int(L), C.c_int(H), C.c_int(mb), C.c_int(T), C.c_int(V), _p(embed), wptrs,
+                                  _p(ids_nonneg, i32p), _p(mask01, i32p), _p(h0f), _p(c0f), _p(et),
+                                  _p(ehT) if ehT is not None else None, _p(ecT) if ecT is not None else None, gptrs,
+                                  _p(d_embed), _p(eh0), _p(ec0))
+    grads = [{"dM": gl[0:4], "dWh": gl[4:8], "db": gl[8:12]} for gl in gmats]
+    unflat = lambda f: [f[l * n:(l + 1) * n].reshape(H, mb, order="F") for l in range(L)]
+    return grads, d_embed, unflat(eh0), unflat(ec0)
+
+
+def softmax_backward(D, b_d, h, target, mask01, dD=None, db=None):
+    """Returns err_h (H x mb), dD (V x H, float64), db (V, float64); dD / db given: accumulated into."""
+    D, h = F(D), F(h)
+    V, H = D.shape
+    mb = h.shape[1]
+    b_d = np.ascontiguousarray(b_d, dtype=np.float32)
+    target = np.ascontiguousarray(target, dtype=np.int32)
+    mask01 = np.ascontiguousarray(mask01, dtype=np.int32)
+    add = dD is not None
+    if add:
+        assert dD.flags.f_contiguous and dD.dtype == np.float64 and db.dtype == np.float64, "dD must be column-major f64"
+    if not add:
+        dD = np.zeros((V, H), dtype=np.float64, order="F")
+        db = np.zeros(V, dtype=np.float64)
+    err_h = np.empty((H, mb), dtype=np.float32, order="F")
+    lib().orc_softmax_backward(_p(D), _p(b_d), C.c_int(V), C.c_int(H), _p(h), C.c_int(mb), _p(target, i32p),
+                               _p(mask01, i32p), C.c_int(int(add)), _p(err_h), _p(dD, f64p), _p(db, f64p))
+    return err_h, dD, db
