@@ -244,6 +244,71 @@ int zr_beam_hypotheses(zr_ctx* ctx, zr_beam* b, int sentence, int cap, int* h_wo
 /* Current beam state of sentence s (top_sentences_scores, current_indices). */
 int zr_beam_state(zr_ctx* ctx, zr_beam* b, int sentence, float* h_scores, int* h_words);
 
+/* ---- F4: training backward (stacked LSTM and output layer; no attention, no dropout) ------------------------ */
+
+/* zr_lstm_stack_forward that also keeps every node's gate activations for the backward pass (the reference's nodes
+ * keep d_i_t, d_f_t, d_c_prime_t_tanh, d_o_t; src/LSTM.h:30-60).  d_gates_all: L pointers, each T*4*H*mb floats;
+ * gate g (order i, f, c~, o) of node t at offset (t*4 + g)*H*mb.  An entry may be NULL (that layer's gates are not
+ * kept). */
+int zr_lstm_stack_forward_train(zr_ctx* ctx, int L, const zr_lstm_weights* const layers[], const float* d_embed, int V,
+                                const int* d_ids_nonneg, const int* d_mask01, int T, int mb,
+                                const float* const d_h0[], const float* const d_c0[], float clip_threshold,
+                                float* const d_h_all[], float* const d_c_all[], float* const d_gates_all[]);
+
+/* Backward-side copy of one layer's matrices: M_g and W_hg stacked over the four gates as 4H x H matrices (rows
+ * g*H + j), the operands of the error products d_ERRnTOt_htM1 = sum_g W_hg^T err_g and d_ERRnTOt_h_Below =
+ * sum_g M_g^T err_g (src/LSTM_HH.hpp:470-560).  Call zr_lstm_train_refresh after the weights change. */
+typedef struct zr_lstm_train zr_lstm_train;
+int zr_lstm_train_create(zr_ctx* ctx, const float* const d_M[4], const float* const d_Wh[4], int H, zr_lstm_train** out);
+int zr_lstm_train_refresh(zr_ctx* ctx, zr_lstm_train* w, const float* const d_M[4], const float* const d_Wh[4]);
+int zr_lstm_train_destroy(zr_ctx* ctx, zr_lstm_train* w);
+/* 4H x H stacked matrix -> four H x H matrices (gate order i, f, c, o), e.g. the reference's d_M_i_grad ... */
+int zr_unstack_gates(zr_ctx* ctx, const float* d_stack, int H, float* const d_out[4]);
+
+/* Back-propagation through time over the whole (layer, time) grid: LSTM_IH_Node / LSTM_HH_Node::back_prop_GPU
+ * (src/LSTM.hpp:542-900, src/LSTM_HH.hpp:336-640) in the order of neuralMT_model::compute_gradients
+ * (src/model.hpp:1823-2000), errors only (weight gradients: zr_lstm_weight_gradients).
+ *   d_c0, d_c_all, d_gates_all: as given to / written by zr_lstm_stack_forward_train.
+ *   d_err_top: T*H*mb, the loss layer's error at the top layer's h_t (d_ERRt_ht).
+ *   d_err_hT / d_err_cT: L pointers (or NULL, or NULL entries): errors arriving at the last step from beyond.
+ *   Outputs: d_dgates_all[l]: 4H x (T*mb) column-major, the errors at the four pre-activations of every node
+ *   (element (g*H + j, t*mb + b)); d_err_below0: T*H*mb, the error at layer 0's input (NULL: not wanted);
+ *   d_err_h0 / d_err_c0: L pointers, errors at the initial states. */
+int zr_lstm_stack_backward(zr_ctx* ctx, int L, const zr_lstm_train* const layers[], int T, int mb,
+                           const int* d_mask01, const float* const d_c0[], const float* const d_c_all[],
+                           const float* const d_gates_all[], const float* d_err_top, const float* const d_err_hT[],
+                           const float* const d_err_cT[], float* const d_dgates_all[], float* d_err_below0,
+                           float* const d_err_h0[], float* const d_err_c0[]);
+
+/* One layer's weight gradients from the kept errors: compute_gradients_GPU (src/LSTM.hpp:1000-1270) summed over
+ * all nodes in one product each.  d_in_all: the layer's inputs, H x (T*mb) (the layer below's h, or the gathered
+ * embedding columns); d_h0, d_h_all: the layer's own initial state and outputs.
+ * d_dM_stack, d_dWh_stack: 4H x H stacked gradients (zr_unstack_gates splits them); d_db: 4H. */
+int zr_lstm_weight_gradients(zr_ctx* ctx, int H, int T, int mb, const float* d_dgates, const float* d_in_all,
+                             const float* d_h0, const float* d_h_all, float* d_dM_stack, float* d_dWh_stack,
+                             float* d_db);
+
+/* Embedding gradient (the sparse W gradient kernels, src/custom_kernels.h:1297-1390): d_dW[:, id[k]] += d_err[:, k]
+ * for the n unmasked positions; d_dW is H x V and is accumulated into (zero it first).  Uses float atomics, like
+ * the reference: the summation order within a column is not fixed. */
+int zr_embed_gradient(zr_ctx* ctx, int H, int V, const float* d_err, const int* d_ids_nonneg, const int* d_mask01,
+                      int n, float* d_dW);
+
+/* Loss-layer backward for n columns at once (all time steps of a minibatch, n = T*mb <= 65535):
+ * get_h_t_gradient_GPU, compute_D_gradient_GPU, compute_b_d_gradient_GPU (src/softmax.hpp:700-860).
+ *   d_h: H x n; d_target (-1 already mapped to 0) and d_mask01: n ints (zr_vocab_prep_softmax).
+ *   d_prob_scratch: V x n.  Outputs: d_err_h H x n (= D^T (onehot - p), 0 on masked columns), d_dD V x H,
+ *   d_db V (overwritten, not accumulated: pass every column of the minibatch in one call). */
+int zr_softmax_backward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int n,
+                        const int* d_target, const int* d_mask01, float* d_prob_scratch, float* d_err_h, float* d_dD,
+                        float* d_db);
+
+/* update_weights (src/softmax.hpp:232-300, src/Hidden_To_Hidden_Layer.hpp update_weights_GPU): the gradient is
+ * scaled (the reference divides by the minibatch size), clipped to norm_clip in L2 norm if norm_clip > 0
+ * (norm_clip_GPU_v2), and ADDED: W += learning_rate * clip(scale * grad). */
+int zr_sgd_update(zr_ctx* ctx, float* d_W, const float* d_grad, long long n, float scale, float norm_clip,
+                  float learning_rate);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,205 @@
+"""Training backward on the GPU (stacked LSTM + output layer) against the oracle, whose backward restatement is
+pinned by torch autograd in tests/test_oracle_backward_pins.py.  fp32 tolerance: 1e-4 relative with an absolute
+floor scaled to the size of the sums involved (stated per check)."""
+import numpy as np
+import pytest
+
+import oracle_lib as o
+from gpu_util import Layer, assert_close
+from zoph_rnn_amd import capi, synth
+
+pytestmark = pytest.mark.gpu
+U = synth.uniform
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = capi.Context(0)
+    yield c
+    c.close()
+
+
+class TrainLayer(Layer):
+    def __init__(self, ctx, ly):
+        super().__init__(ctx, ly)
+        self.t = ctx.lstm_train_create(self.M, self.Wh, self.H)
+
+    def close(self):
+        self.ctx.lstm_train_destroy(self.t)
+        super().close()
+
+
+def _unstack(ctx, d_stack, H):
+    outs = [ctx.empty((H, H)) for _ in range(4)]
+    ctx.unstack_gates(d_stack, H, outs)
+    ctx.sync()
+    return [a.get() for a in outs]
+
+
+def _gpu_stack_backward(ctx, embed, layers_np, ids, h0, c0, err_top, err_hT, err_cT):
+    H, V = embed.shape
+    T, mb = ids.shape
+    L = len(layers_np)
+    n = H * mb
+    layers = [TrainLayer(ctx, ly) for ly in layers_np]
+    d_embed = ctx.array(embed)
+    d_nn, d_m = ctx.empty(ids.size, np.int32), ctx.empty(ids.size, np.int32)
+    ctx.vocab_prep(ctx.array(ids.reshape(-1)), ids.size, V, d_nn, d_m)
+    d_h0, d_c0 = [ctx.array(a) for a in h0], [ctx.array(a) for a in c0]
+    h_all = [ctx.empty((n * T,)) for _ in range(L)]
+    c_all = [ctx.empty((n * T,)) for _ in range(L)]
+    g_all = [ctx.empty((4 * n * T,)) for _ in range(L)]
+    ctx.lstm_stack_forward_train([ly.w for ly in layers], d_embed, V, d_nn, d_m, T, mb, d_h0, d_c0, h_all, c_all, g_all)
+    d_err_top = ctx.array(np.concatenate([np.asfortranarray(e).reshape(-1, order="F") for e in err_top]))
+    dg_all = [ctx.empty((4 * n * T,)) for _ in range(L)]
+    eh0, ec0 = [ctx.empty((H, mb)) for _ in range(L)], [ctx.empty((H, mb)) for _ in range(L)]
+    d_below0 = ctx.empty((n * T,))
+    ctx.lstm_stack_backward([ly.t for ly in layers], T, mb, d_m, d_c0, c_all, g_all, d_err_top, dg_all, eh0, ec0,
+                            err_hT=[ctx.array(a) for a in err_hT] if err_hT else None,
+                            err_cT=[ctx.array(a) for a in err_cT] if err_cT else None, d_err_below0=d_below0)
+    # weight gradients, layer by layer
+    x_all = ctx.empty((n * T,))
+    ctx.embed_gather(d_embed, H, V, d_nn, T * mb, x_all)
+    grads = []
+    for l in range(L):
+        dM, dWh, db = ctx.empty((4 * H, H)), ctx.empty((4 * H, H)), ctx.empty((4 * H,))
+        ctx.lstm_weight_gradients(H, T, mb, dg_all[l], x_all if l == 0 else h_all[l - 1], d_h0[l], h_all[l], dM, dWh, db)
+        grads.append({"dM": _unstack(ctx, dM, H), "dWh": _unstack(ctx, dWh, H), "db": list(db.get().reshape(4, H))})
+    d_dW = ctx.zeros((H, V))
+    ctx.embed_gradient(H, V, d_below0, d_nn, d_m, T * mb, d_dW)
+    ctx.sync()
+    out = (grads, d_dW.get(), [a.get() for a in eh0], [a.get() for a in ec0])
+    for ly in layers:
+        ly.close()
+    return out
+
+
+@pytest.mark.parametrize("L,H,mb,T,V,pad,tail", [(1, 32, 8, 5, 40, False, False), (3, 48, 33, 7, 90, True, True),
+                                                 (2, 100, 20, 6, 150, True, True), (4, 64, 130, 4, 200, True, False)])
+def test_stack_backward_and_gradients(ctx, L, H, mb, T, V, pad, tail):
+    g = synth.rng(111, L * 1000 + H + mb)
+    embed = U(g, (H, V), -0.5, 0.5)
+    layers = [synth.lstm_layer(g, H) for _ in range(L)]
+    for ly in layers:
+        ly["M"] = [U(g, (H, H), -0.2, 0.2) for _ in range(4)]
+        ly["Wh"] = [U(g, (H, H), -0.2, 0.2) for _ in range(4)]
+    ids = g.integers(0, V, size=(T, mb)).astype(np.int32)
+    if pad:
+        ids[:2, 1] = -1
+        ids[T - 2:, 2] = -1
+        ids[:, 5] = -1  # a fully padded column
+    nn, mask = o.vocab_prep(ids)
+    h0 = [U(g, (H, mb), -0.5, 0.5) for _ in range(L)]
+    c0 = [U(g, (H, mb), -0.5, 0.5) for _ in range(L)]
+    err_top = [U(g, (H, mb), -1, 1) for _ in range(T)]
+    err_hT = [U(g, (H, mb), -1, 1) for _ in range(L)] if tail else None
+    err_cT = [U(g, (H, mb), -1, 1) for _ in range(L)] if tail else None
+    want_g, want_e, want_eh0, want_ec0 = o.lstm_stack_backward(embed, layers, nn, mask, err_top, h0, c0, err_hT, err_cT)
+    got_g, got_e, got_eh0, got_ec0 = _gpu_stack_backward(ctx, embed, layers, ids, h0, c0, err_top, err_hT, err_cT)
+    # errors are sums of up to 4H products of size ~0.2 x ~1: floor 0.05 as for the forward activations;
+    # weight gradients are sums over T*mb samples of products of size ~1: floor scaled with sqrt(T*mb)
+    wfloor = 0.05 * np.sqrt(T * mb)
+    for l in range(L):
+        assert_close(got_eh0[l], want_eh0[l], what="err_h0 layer %d" % l)
+        assert_close(got_ec0[l], want_ec0[l], what="err_c0 layer %d" % l)
+        for q in range(4):
+            assert_close(got_g[l]["dM"][q], want_g[l]["dM"][q], floor=wfloor, what="dM layer %d gate %d" % (l, q))
+            assert_close(got_g[l]["dWh"][q], want_g[l]["dWh"][q], floor=wfloor, what="dWh layer %d gate %d" % (l, q))
+            assert_close(got_g[l]["db"][q], want_g[l]["db"][q], floor=wfloor, what="db layer %d gate %d" % (l, q))
+    assert_close(got_e, want_e, floor=0.05 * np.sqrt(T), what="embedding gradient")
+    used = set(int(v) for v in ids[ids >= 0])
+    unused = [v for v in range(V) if v not in used]
+    assert np.all(got_e[:, unused] == 0)
+
+
+@pytest.mark.parametrize("V,H,n", [(211, 16, 6), (1003, 48, 70), (5000, 64, 160)])
+def test_softmax_backward(ctx, V, H, n):
+    g = synth.rng(112, V)
+    D, bd, h = U(g, (V, H), -0.5, 0.5), U(g, (V,), -1, 1), U(g, (H, n), -1, 1)
+    target = g.integers(0, V, size=n).astype(np.int32)
+    mask = (g.random(n) > 0.2).astype(np.int32)
+    d_scr, d_eh, d_dD, d_db = ctx.empty((V, n)), ctx.empty((H, n)), ctx.empty((V, H)), ctx.empty((V,))
+    ctx.softmax_backward(ctx.array(D), ctx.array(bd), V, H, ctx.array(h), n, ctx.array(target), ctx.array(mask), d_scr,
+                         d_eh, d_dD, d_db)
+    ctx.sync()
+    want_eh, want_dD, want_db = o.softmax_backward(D, bd, h, target, mask)
+    assert_close(d_eh.get(), want_eh, what="err_h")
+    assert_close(d_dD.get(), want_dD, floor=0.05 * np.sqrt(n), what="dD")
+    assert_close(d_db.get(), want_db, floor=0.05 * np.sqrt(n), what="db")
+    assert np.all(d_eh.get()[:, mask == 0] == 0)
+
+
+@pytest.mark.parametrize("n,clip", [(1000, 0.0), (100000, 5.0), (100000, 1e6), (37, 0.5)])
+def test_sgd_update(ctx, n, clip):
+    g = synth.rng(113, n)
+    W, G = U(g, (n,), -1, 1), U(g, (n,), -3, 3)
+    scale, lr = 1.0 / 8, 0.7
+    dW = ctx.array(W)
+    ctx.sgd_update(dW, ctx.array(G), n, scale, clip, lr)
+    ctx.sync()
+    gs = G.astype(np.float64) * scale
+    norm = np.sqrt((gs * gs).sum())
+    coef = clip / norm if (clip > 0 and norm > clip) else 1.0
+    want = W + lr * coef * gs
+    assert np.allclose(dW.get(), want, rtol=1e-5, atol=1e-6)
+    if clip > 0 and norm > clip:
+        assert np.sqrt((((dW.get() - W) / lr) ** 2).sum()) == pytest.approx(clip, rel=1e-4)
+
+
+def test_language_model_training_step_gradients(ctx):
+    """BASELINE config 1 shape (1-layer LM, H=100, minibatch 8, T=20, V=10000): the full gradient of the summed
+    log-likelihood -- output layer, LSTM matrices and biases, embedding -- from one forward/backward pass."""
+    c = synth.config1()
+    H, mb, T, V = c["H"], c["mb"], c["T"], c["V"]
+    L = len(c["layers"])
+    n = H * mb
+    ids, tgt_ids = c["ids"], c["targets"]
+    nn, mask = o.vocab_prep(ids)
+    # oracle: forward, per-step loss-layer backward (accumulated), then back-propagation through time
+    hs, _ = o.lstm_stack_forward(c["embed"], c["layers"], nn, mask)
+    dD = np.zeros((V, H), np.float64, order="F")
+    db = np.zeros(V, np.float64)
+    err_top = []
+    for t in range(T):
+        e, dD, db = o.softmax_backward(c["D"], c["b_d"], np.asfortranarray(hs[L - 1, t]), tgt_ids[t], np.ones(mb, np.int32),
+                                       dD, db)
+        err_top.append(e)
+    want_g, want_e, _, _ = o.lstm_stack_backward(c["embed"], c["layers"], nn, mask, err_top)
+    # GPU
+    layers = [TrainLayer(ctx, ly) for ly in c["layers"]]
+    d_embed = ctx.array(c["embed"])
+    d_nn, d_m = ctx.empty(ids.size, np.int32), ctx.empty(ids.size, np.int32)
+    ctx.vocab_prep(ctx.array(ids.reshape(-1)), ids.size, V, d_nn, d_m)
+    z = ctx.zeros((H, mb))
+    h_all, c_all, g_all = ([ctx.empty((n * T,)) for _ in range(L)] for _ in range(3))
+    g_all = [ctx.empty((4 * n * T,)) for _ in range(L)]
+    ctx.lstm_stack_forward_train([ly.w for ly in layers], d_embed, V, d_nn, d_m, T, mb, [z] * L, [z] * L, h_all, c_all,
+                                 g_all)
+    dDg, dbg = ctx.empty((V, H)), ctx.empty((V,))
+    d_err_top, d_scr = ctx.empty((n * T,)), ctx.empty((V, T * mb))
+    ones = ctx.array(np.ones(T * mb, np.int32))
+    ctx.softmax_backward(ctx.array(c["D"]), ctx.array(c["b_d"]), V, H, h_all[L - 1], T * mb,
+                         ctx.array(tgt_ids.reshape(-1).astype(np.int32)), ones, d_scr, d_err_top, dDg, dbg)
+    dg_all = [ctx.empty((4 * n * T,)) for _ in range(L)]
+    eh0, ec0 = [ctx.empty((H, mb)) for _ in range(L)], [ctx.empty((H, mb)) for _ in range(L)]
+    d_below0 = ctx.empty((n * T,))
+    ctx.lstm_stack_backward([ly.t for ly in layers], T, mb, d_m, [z] * L, c_all, g_all, d_err_top, dg_all, eh0, ec0,
+                            d_err_below0=d_below0)
+    x_all = ctx.empty((n * T,))
+    ctx.embed_gather(d_embed, H, V, d_nn, T * mb, x_all)
+    dM, dWh, dbl = ctx.empty((4 * H, H)), ctx.empty((4 * H, H)), ctx.empty((4 * H,))
+    ctx.lstm_weight_gradients(H, T, mb, dg_all[0], x_all, z, h_all[0], dM, dWh, dbl)
+    d_dW = ctx.zeros((H, V))
+    ctx.embed_gradient(H, V, d_below0, d_nn, d_m, T * mb, d_dW)
+    ctx.sync()
+    fl = 0.05 * np.sqrt(T * mb)
+    assert_close(dDg.get(), dD, floor=fl * 0.1, what="dD")
+    assert_close(dbg.get(), db, floor=fl * 0.1, what="db_d")
+    gM, gWh = _unstack(ctx, dM, H), _unstack(ctx, dWh, H)
+    for q in range(4):
+        assert_close(gM[q], want_g[0]["dM"][q], floor=fl * 0.1, what="dM gate %d" % q)
+        assert_close(gWh[q], want_g[0]["dWh"][q], floor=fl * 0.1, what="dWh gate %d" % q)
+        assert_close(dbl.get().reshape(4, H)[q], want_g[0]["db"][q], floor=fl * 0.1, what="db gate %d" % q)
+    assert_close(d_dW.get(), want_e, floor=0.05, what="embedding gradient")
+    for ly in layers:
+        ly.close()

@@ -30,6 +30,9 @@ SYMBOLS = [
     "zr_softmax_loss", "zr_attn_create", "zr_attn_use_bf16_weights", "zr_attn_destroy", "zr_attn_step", "zr_gather_columns",
     "zr_broadcast_column", "zr_beam_create", "zr_beam_destroy", "zr_beam_init", "zr_beam_expand", "zr_beam_finish",
     "zr_beam_hypotheses", "zr_beam_state",
+    "zr_lstm_stack_forward_train", "zr_lstm_train_create", "zr_lstm_train_refresh", "zr_lstm_train_destroy",
+    "zr_unstack_gates", "zr_lstm_stack_backward", "zr_lstm_weight_gradients", "zr_embed_gradient",
+    "zr_softmax_backward", "zr_sgd_update",
 ]
 
 _lib = None
@@ -199,6 +202,56 @@ class Context:
     def gemm(self, trans_a, M, N, K, d_A, lda, d_B, ldb, d_C, ldc):
         _chk(load().zr_gemm(self.h, C.c_int(trans_a), C.c_int(M), C.c_int(N), C.c_int(K), _vp(d_A), C.c_int(lda),
                             _vp(d_B), C.c_int(ldb), _vp(d_C), C.c_int(ldc)))
+
+    # ---- F4: training backward
+    def lstm_stack_forward_train(self, layers, d_embed, V, d_ids, d_mask, T, mb, h0, c0, h_all, c_all, gates_all,
+                                 clip=0.0):
+        L = len(layers)
+        larr = (C.c_void_p * L)(*[w.value for w in layers])
+        _chk(load().zr_lstm_stack_forward_train(self.h, C.c_int(L), larr, _vp(d_embed), C.c_int(V), _vp(d_ids),
+                                                _vp(d_mask), C.c_int(T), C.c_int(mb), _ptr_array(h0), _ptr_array(c0),
+                                                C.c_float(clip), _ptr_array(h_all), _ptr_array(c_all),
+                                                _ptr_array(gates_all)))
+
+    def lstm_train_create(self, M, Wh, H):
+        w = C.c_void_p()
+        _chk(load().zr_lstm_train_create(self.h, _ptr_array(M), _ptr_array(Wh), C.c_int(H), C.byref(w)))
+        return w
+
+    def lstm_train_refresh(self, w, M, Wh):
+        _chk(load().zr_lstm_train_refresh(self.h, w, _ptr_array(M), _ptr_array(Wh)))
+
+    def lstm_train_destroy(self, w):
+        _chk(load().zr_lstm_train_destroy(self.h, w))
+
+    def unstack_gates(self, d_stack, H, outs):
+        _chk(load().zr_unstack_gates(self.h, _vp(d_stack), C.c_int(H), _ptr_array(outs)))
+
+    def lstm_stack_backward(self, layers, T, mb, d_mask, c0, c_all, gates_all, d_err_top, dgates_all, err_h0, err_c0,
+                            err_hT=None, err_cT=None, d_err_below0=None):
+        L = len(layers)
+        larr = (C.c_void_p * L)(*[w.value for w in layers])
+        _chk(load().zr_lstm_stack_backward(self.h, C.c_int(L), larr, C.c_int(T), C.c_int(mb), _vp(d_mask),
+                                           _ptr_array(c0), _ptr_array(c_all), _ptr_array(gates_all), _vp(d_err_top),
+                                           _ptr_array(err_hT) if err_hT else None,
+                                           _ptr_array(err_cT) if err_cT else None, _ptr_array(dgates_all),
+                                           _vp(d_err_below0), _ptr_array(err_h0), _ptr_array(err_c0)))
+
+    def lstm_weight_gradients(self, H, T, mb, d_dgates, d_in_all, d_h0, d_h_all, d_dM, d_dWh, d_db):
+        _chk(load().zr_lstm_weight_gradients(self.h, C.c_int(H), C.c_int(T), C.c_int(mb), _vp(d_dgates), _vp(d_in_all),
+                                             _vp(d_h0), _vp(d_h_all), _vp(d_dM), _vp(d_dWh), _vp(d_db)))
+
+    def embed_gradient(self, H, V, d_err, d_ids, d_mask, n, d_dW):
+        _chk(load().zr_embed_gradient(self.h, C.c_int(H), C.c_int(V), _vp(d_err), _vp(d_ids), _vp(d_mask), C.c_int(n),
+                                      _vp(d_dW)))
+
+    def softmax_backward(self, d_D, d_b, V, H, d_h, n, d_target, d_mask, d_scratch, d_err_h, d_dD, d_db):
+        _chk(load().zr_softmax_backward(self.h, _vp(d_D), _vp(d_b), C.c_int(V), C.c_int(H), _vp(d_h), C.c_int(n),
+                                        _vp(d_target), _vp(d_mask), _vp(d_scratch), _vp(d_err_h), _vp(d_dD), _vp(d_db)))
+
+    def sgd_update(self, d_W, d_grad, n, scale, norm_clip, lr):
+        _chk(load().zr_sgd_update(self.h, _vp(d_W), _vp(d_grad), C.c_longlong(n), C.c_float(scale), C.c_float(norm_clip),
+                                  C.c_float(lr)))
 
     # ---- A8/A9
     def softmax_prepare(self, d_D, V, H, bf16=False):

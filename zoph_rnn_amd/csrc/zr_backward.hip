@@ -1,0 +1,460 @@
+// Training backward for the stacked LSTM and the output layer (no attention, no dropout).
+//
+// Gradients are those of the log-likelihood, as in the reference (its loss layer's error is D^T (onehot - p),
+// src/softmax.hpp:700-712; update_weights adds learning_rate * gradient, :232-300).
+//
+// What is different from the reference's schedule (src/LSTM.hpp:542-1270, src/LSTM_HH.hpp:336-900):
+//  * the element-wise error kernels of a node (d_ERRt_ct_kernel, d_ERRnTOt_ot_kernel, d_ERRnTOt_ft_it_kernel x2,
+//    d_ERRnTOt_tanhcpt_kernel, zero_columns_kernel x2, three cublas geam additions; src/custom_kernels.h:199-262)
+//    are one kernel that reads the saved gates once and writes the four pre-activation errors once;
+//  * the eight W^T * error products of a node are one batched product against the gate matrices stacked as
+//    4H x H (error to h_{t-1} and error to the layer below share the right-hand side);
+//  * the weight gradients are not accumulated step by step (8 rank-mb updates of H x H matrices per node, each a
+//    full read-modify-write of the matrix): every node's pre-activation errors are kept (4H x T*mb per layer, a
+//    few hundred MB) and each gradient is ONE product with K = T * mb after the sweep.
+#include <math.h>
+
+#include "zr_internal.h"
+
+struct zr_lstm_train {
+  int H;
+  float* d_stack;  // [2][4H x H] column-major: Wh stacked over the gates (rows g*H + j), then M
+};
+
+namespace {
+
+inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+__global__ void __launch_bounds__(256) stack_gates_kernel(const float* __restrict__ g0, const float* __restrict__ g1,
+                                                          const float* __restrict__ g2, const float* __restrict__ g3,
+                                                          int H, float* __restrict__ dst) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;  // over the 4H x H destination
+  if (i >= 4LL * H * H) return;
+  const int r = (int)(i % (4 * H));
+  const int k = (int)(i / (4 * H));
+  const int g = r / H, j = r - g * H;
+  const float* src = g == 0 ? g0 : (g == 1 ? g1 : (g == 2 ? g2 : g3));
+  dst[i] = src[j + (long long)k * H];
+}
+
+__global__ void __launch_bounds__(256) unstack_gates_kernel(const float* __restrict__ src, int H, float* __restrict__ g0,
+                                                            float* __restrict__ g1, float* __restrict__ g2,
+                                                            float* __restrict__ g3) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= 4LL * H * H) return;
+  const int r = (int)(i % (4 * H));
+  const int k = (int)(i / (4 * H));
+  const int g = r / H, j = r - g * H;
+  float* dst = g == 0 ? g0 : (g == 1 ? g1 : (g == 2 ? g2 : g3));
+  dst[j + (long long)k * H] = src[i];
+}
+
+// One node: total error at h_t (from above + from t+1), cell error, the four pre-activation errors, error to c_{t-1}.
+//   gates: [4][H*mb] (i, f, c~, o) of the node; dg: the node's 4H x mb block of the layer's error matrix
+//   (element (g*H + j, b) at dg[b*4H + g*H + j]); ec: in = error arriving at c_t from t+1 (or null at the last step),
+//   out = error for c_{t-1} (may alias).
+__global__ void __launch_bounds__(256) lstm_node_backward_kernel(
+    const float* __restrict__ gates, const float* __restrict__ c, const float* __restrict__ cprev,
+    const int* __restrict__ mask01, const float* __restrict__ err_above, const float* __restrict__ err_next,
+    const float* ec_in, float* ec_out, int H, int mb, float* __restrict__ dg) {
+  const int b = blockIdx.y;
+  const int j = blockIdx.x * 256 + threadIdx.x;
+  if (j >= H) return;
+  const size_t n = (size_t)H * mb, ix = (size_t)b * H + j;
+  const float m = (float)mask01[b];
+  float eh = 0.0f;
+  if (err_above) eh += err_above[ix];
+  if (err_next) eh += err_next[ix];
+  eh *= m;
+  const float gi = gates[ix], gf = gates[n + ix], gc = gates[2 * n + ix], go = gates[3 * n + ix];
+  const float th = tanhf(c[ix]);
+  const float errt_ct = eh * go * (1.0f - th * th);
+  const float ec = ((ec_in ? ec_in[ix] : 0.0f) + errt_ct) * m;
+  float* d = dg + (size_t)b * 4 * H + j;
+  d[0] = ec * gc * gi * (1.0f - gi);
+  d[H] = ec * cprev[ix] * gf * (1.0f - gf);
+  d[2 * (size_t)H] = ec * gi * (1.0f - gc * gc);
+  d[3 * (size_t)H] = eh * th * go * (1.0f - go);
+  ec_out[ix] = ec * gf;
+}
+
+// dst (cols x rows, column-major with leading dimension ldd, starting at row offset row0) = src^T, src rows x cols
+// column-major (ld = rows): dst[row0 + c + r*ldd] = src[r + c*rows].  32 x 32 tiles through LDS.
+__global__ void __launch_bounds__(256) transpose_kernel(const float* __restrict__ src, int rows, int cols,
+                                                        float* __restrict__ dst, long long ldd, int row0) {
+  __shared__ float tile[32][33];
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+  const int r0 = blockIdx.x * 32, c0 = blockIdx.y * 32;
+  for (int i = ty; i < 32; i += 8) {
+    const int r = r0 + tx, cc = c0 + i;
+    tile[i][tx] = (r < rows && cc < cols) ? src[r + (long long)cc * rows] : 0.0f;
+  }
+  __syncthreads();
+  for (int i = ty; i < 32; i += 8) {
+    const int cc = c0 + tx, r = r0 + i;
+    if (r < rows && cc < cols) dst[row0 + cc + (long long)r * ldd] = tile[tx][i];
+  }
+}
+
+// out[r] = sum over the n columns of a (rows x n, column-major).  One wave per 64 rows; fixed order.
+__global__ void __launch_bounds__(64) row_sum_kernel(const float* __restrict__ a, int rows, long long n,
+                                                     float* __restrict__ out) {
+  const int r = blockIdx.x * 64 + threadIdx.x;
+  if (r >= rows) return;
+  float s = 0.0f;
+  for (long long k = 0; k < n; ++k) s += a[r + k * rows];
+  out[r] = s;
+}
+
+// Embedding gradient: column id[k] of dW += err column k for every unmasked position.  Float atomics: the order of
+// the additions into one column is not fixed (the reference's sparse W gradient kernels use atomicAdd as well).
+__global__ void __launch_bounds__(256) embed_grad_kernel(const float* __restrict__ err, const int* __restrict__ ids,
+                                                         const int* __restrict__ mask01, int H, int V,
+                                                         float* __restrict__ dW) {
+  const int k = blockIdx.y;
+  if (mask01[k] != 1) return;
+  const int j = blockIdx.x * 256 + threadIdx.x;
+  if (j >= H) return;
+  int id = ids[k];
+  id = id < 0 ? 0 : (id >= V ? V - 1 : id);
+  atomicAdd(&dW[(size_t)id * H + j], err[(size_t)k * H + j]);
+}
+
+// p (V x n probabilities) -> e = onehot(target) - p on unmasked columns, 0 on masked ones, in place.
+__global__ void __launch_bounds__(256) softmax_error_kernel(float* __restrict__ p, int V, const int* __restrict__ target,
+                                                            const int* __restrict__ mask01) {
+  const int col = blockIdx.y;
+  const int v = blockIdx.x * 256 + threadIdx.x;
+  if (v >= V) return;
+  const size_t ix = (size_t)col * V + v;
+  float e = 0.0f;
+  if (mask01[col] == 1) e = (v == target[col] ? 1.0f : 0.0f) - p[ix];
+  p[ix] = e;
+}
+
+// sum of squares, two deterministic stages
+__global__ void __launch_bounds__(256) sumsq_partial_kernel(const float* __restrict__ g, long long n,
+                                                            double* __restrict__ partial) {
+  __shared__ double s[256];
+  double acc = 0.0;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) {
+    const double v = g[i];
+    acc += v * v;
+  }
+  s[threadIdx.x] = acc;
+  __syncthreads();
+  for (int st = 128; st > 0; st >>= 1) {
+    if ((int)threadIdx.x < st) s[threadIdx.x] += s[threadIdx.x + st];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) partial[blockIdx.x] = s[0];
+}
+
+// W += lr * coef * scale * g, with coef = norm_clip / ||scale * g|| when that norm exceeds norm_clip (> 0), else 1
+__global__ void __launch_bounds__(256) sgd_apply_kernel(float* __restrict__ W, const float* __restrict__ g, long long n,
+                                                        float scale, float norm_clip, float lr,
+                                                        const double* __restrict__ partial, int n_partial) {
+  __shared__ float coef_s;
+  if (threadIdx.x == 0) {
+    float coef = 1.0f;
+    if (norm_clip > 0.0f) {
+      double ss = 0.0;
+      for (int i = 0; i < n_partial; ++i) ss += partial[i];
+      const float norm = (float)sqrt(ss) * fabsf(scale);
+      if (norm > norm_clip) coef = norm_clip / norm;
+    }
+    coef_s = coef;
+  }
+  __syncthreads();
+  const float f = lr * coef_s * scale;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) W[i] += f * g[i];
+}
+
+int transpose_launch(zr_ctx* ctx, const float* src, int rows, int cols, float* dst, long long ldd, int row0) {
+  dim3 grid((rows + 31) / 32, (cols + 31) / 32);
+  transpose_kernel<<<grid, 256, 0, ctx->stream>>>(src, rows, cols, dst, ldd, row0);
+  ZR_LAUNCH_CHECK("transpose_kernel");
+  return ZR_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int zr_lstm_train_create(zr_ctx* ctx, const float* const d_M[4], const float* const d_Wh[4], int H,
+                         zr_lstm_train** out) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(out != nullptr, "zr_lstm_train_create: out is null");
+  *out = nullptr;
+  ZR_CHECK_ARG(H > 0 && d_M && d_Wh, "zr_lstm_train_create: H = %d or null pointer array", H);
+  for (int g = 0; g < 4; ++g) ZR_CHECK_ARG(d_M[g] && d_Wh[g], "zr_lstm_train_create: null matrix for gate %d", g);
+  zr_lstm_train* w = new zr_lstm_train();
+  w->H = H;
+  w->d_stack = nullptr;
+  const size_t per = 4 * (size_t)H * H;
+  if (hipMalloc((void**)&w->d_stack, sizeof(float) * 2 * per) != hipSuccess) {
+    (void)hipGetLastError();
+    delete w;
+    return zr_set_error(ZR_ENOMEM, "zr_lstm_train_create: allocation failed (H = %d)", H);
+  }
+  *out = w;
+  return zr_lstm_train_refresh(ctx, w, d_M, d_Wh);
+}
+
+int zr_lstm_train_refresh(zr_ctx* ctx, zr_lstm_train* w, const float* const d_M[4], const float* const d_Wh[4]) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(w && d_M && d_Wh, "zr_lstm_train_refresh: null pointer");
+  const int H = w->H;
+  const size_t per = 4 * (size_t)H * H;
+  const unsigned grid = (unsigned)((per + 255) / 256);
+  stack_gates_kernel<<<grid, 256, 0, ctx->stream>>>(d_Wh[0], d_Wh[1], d_Wh[2], d_Wh[3], H, w->d_stack);
+  ZR_LAUNCH_CHECK("stack_gates_kernel");
+  stack_gates_kernel<<<grid, 256, 0, ctx->stream>>>(d_M[0], d_M[1], d_M[2], d_M[3], H, w->d_stack + per);
+  ZR_LAUNCH_CHECK("stack_gates_kernel");
+  return ZR_OK;
+}
+
+int zr_lstm_train_destroy(zr_ctx* ctx, zr_lstm_train* w) {
+  if (!w) return ZR_OK;
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_HIP(hipStreamSynchronize(ctx->stream));
+  if (w->d_stack) (void)hipFree(w->d_stack);
+  delete w;
+  return ZR_OK;
+}
+
+int zr_unstack_gates(zr_ctx* ctx, const float* d_stack, int H, float* const d_out[4]) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(d_stack && d_out && H > 0, "zr_unstack_gates: null pointer or H = %d", H);
+  for (int g = 0; g < 4; ++g) ZR_CHECK_ARG(d_out[g] != nullptr, "zr_unstack_gates: d_out[%d] is null", g);
+  const size_t per = 4 * (size_t)H * H;
+  unstack_gates_kernel<<<(unsigned)((per + 255) / 256), 256, 0, ctx->stream>>>(d_stack, H, d_out[0], d_out[1], d_out[2],
+                                                                               d_out[3]);
+  ZR_LAUNCH_CHECK("unstack_gates_kernel");
+  return ZR_OK;
+}
+
+int zr_lstm_stack_backward(zr_ctx* ctx, int nl, const zr_lstm_train* const layers[], int T, int mb,
+                           const int* d_mask01, const float* const d_c0[], const float* const d_c_all[],
+                           const float* const d_gates_all[], const float* d_err_top, const float* const d_err_hT[],
+                           const float* const d_err_cT[], float* const d_dgates_all[], float* d_err_below0,
+                           float* const d_err_h0[], float* const d_err_c0[]) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(nl > 0 && nl <= 16 && T > 0 && mb > 0, "zr_lstm_stack_backward: L = %d, T = %d, mb = %d", nl, T, mb);
+  ZR_CHECK_ARG(mb <= 65535, "zr_lstm_stack_backward: mb = %d exceeds 65535", mb);
+  ZR_CHECK_ARG(layers && d_mask01 && d_c0 && d_c_all && d_gates_all && d_err_top && d_dgates_all && d_err_h0 &&
+                   d_err_c0,
+               "zr_lstm_stack_backward: null pointer");
+  const int H = layers[0] ? layers[0]->H : 0;
+  for (int l = 0; l < nl; ++l) {
+    ZR_CHECK_ARG(layers[l] && layers[l]->H == H, "zr_lstm_stack_backward: layer %d missing or of different size", l);
+    ZR_CHECK_ARG(d_c0[l] && d_c_all[l] && d_gates_all[l] && d_dgates_all[l] && d_err_h0[l] && d_err_c0[l],
+                 "zr_lstm_stack_backward: null buffer for layer %d", l);
+  }
+  const size_t n = (size_t)H * mb;
+  // work: per layer [2][H x mb] = (error to h_{t-1}, error to the layer below), the two outputs of the batched
+  // product; the cell error lives in d_err_c0[l] (updated in place step by step)
+  void* scratch = nullptr;
+  rc = zr_ctx_scratch(ctx, 1, sizeof(float) * 2 * n * nl, &scratch);
+  if (rc) return rc;
+  float* work = (float*)scratch;
+  for (int l = 0; l < nl; ++l) {
+    if (d_err_hT && d_err_hT[l])
+      ZR_HIP(hipMemcpyAsync(work + (size_t)l * 2 * n, d_err_hT[l], sizeof(float) * n, hipMemcpyDeviceToDevice, ctx->stream));
+    else
+      ZR_HIP(hipMemsetAsync(work + (size_t)l * 2 * n, 0, sizeof(float) * n, ctx->stream));
+    if (d_err_cT && d_err_cT[l])
+      ZR_HIP(hipMemcpyAsync(d_err_c0[l], d_err_cT[l], sizeof(float) * n, hipMemcpyDeviceToDevice, ctx->stream));
+    else
+      ZR_HIP(hipMemsetAsync(d_err_c0[l], 0, sizeof(float) * n, ctx->stream));
+  }
+  const size_t per = 4 * (size_t)H * H;
+  dim3 egrid((H + 255) / 256, mb);
+  for (int t = T - 1; t >= 0; --t) {
+    for (int l = nl - 1; l >= 0; --l) {
+      float* w_l = work + (size_t)l * 2 * n;
+      const float* above = (l == nl - 1) ? d_err_top + (size_t)t * n : work + (size_t)(l + 1) * 2 * n + n;
+      float* dg = d_dgates_all[l] + (size_t)t * 4 * n;
+      const float* cprev = (t == 0) ? d_c0[l] : d_c_all[l] + (size_t)(t - 1) * n;
+      lstm_node_backward_kernel<<<egrid, 256, 0, ctx->stream>>>(d_gates_all[l] + (size_t)t * 4 * n,
+                                                                d_c_all[l] + (size_t)t * n, cprev,
+                                                                d_mask01 + (size_t)t * mb, above, w_l, d_err_c0[l],
+                                                                d_err_c0[l], H, mb, dg);
+      ZR_LAUNCH_CHECK("lstm_node_backward_kernel");
+      // (error to h_{t-1}, error to below) = (Wh_stack^T, M_stack^T) * dg : one batched product, shared right side
+      ZrGemmDesc g = {};
+      g.M = H;
+      g.N = mb;
+      g.nseg = 1;
+      g.K[0] = 4 * H;
+      g.A[0] = layers[l]->d_stack;
+      g.lda[0] = 4 * H;
+      g.trans_a = 1;
+      g.B[0] = dg;
+      g.ldb[0] = 4 * H;
+      g.C = w_l;
+      g.ldc = H;
+      g.batch = 2;
+      g.strideA = (long long)per;
+      g.strideC = (long long)n;
+      g.epilogue = ZR_EPI_STORE;
+      rc = zr_gemm_launch(ctx, g);
+      if (rc) return rc;
+      if (l == 0 && d_err_below0)
+        ZR_HIP(hipMemcpyAsync(d_err_below0 + (size_t)t * n, w_l + n, sizeof(float) * n, hipMemcpyDeviceToDevice,
+                              ctx->stream));
+    }
+  }
+  for (int l = 0; l < nl; ++l)
+    ZR_HIP(hipMemcpyAsync(d_err_h0[l], work + (size_t)l * 2 * n, sizeof(float) * n, hipMemcpyDeviceToDevice, ctx->stream));
+  return ZR_OK;
+}
+
+int zr_lstm_weight_gradients(zr_ctx* ctx, int H, int T, int mb, const float* d_dgates, const float* d_in_all,
+                             const float* d_h0, const float* d_h_all, float* d_dM_stack, float* d_dWh_stack,
+                             float* d_db) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(H > 0 && T > 0 && mb > 0, "zr_lstm_weight_gradients: H = %d, T = %d, mb = %d", H, T, mb);
+  ZR_CHECK_ARG(d_dgates && d_in_all && d_h0 && d_h_all && d_dM_stack && d_dWh_stack && d_db,
+               "zr_lstm_weight_gradients: null pointer");
+  const long long K = (long long)T * mb;
+  ZR_CHECK_ARG(K < (1LL << 31) / 4, "zr_lstm_weight_gradients: T * mb = %lld too large", K);
+  void* scratch = nullptr;
+  rc = zr_ctx_scratch(ctx, 0, sizeof(float) * (size_t)K * H, &scratch);  // the transposed right-hand side, K x H
+  if (rc) return rc;
+  float* xt = (float*)scratch;
+  ZrGemmDesc g = {};
+  g.M = 4 * H;
+  g.N = H;
+  g.nseg = 1;
+  g.K[0] = (int)K;
+  g.A[0] = d_dgates;
+  g.lda[0] = 4 * H;
+  g.B[0] = xt;
+  g.ldb[0] = (int)K;
+  g.ldc = 4 * H;
+  g.batch = 1;
+  g.epilogue = ZR_EPI_STORE;
+  // dM = dgates * in^T
+  rc = transpose_launch(ctx, d_in_all, H, (int)K, xt, K, 0);
+  if (rc) return rc;
+  g.C = d_dM_stack;
+  rc = zr_gemm_launch(ctx, g);
+  if (rc) return rc;
+  // dWh = dgates * [h0, h_1 .. h_{T-1}]^T
+  rc = transpose_launch(ctx, d_h0, H, mb, xt, K, 0);
+  if (rc) return rc;
+  if (T > 1) {
+    rc = transpose_launch(ctx, d_h_all, H, (int)(K - mb), xt, K, mb);
+    if (rc) return rc;
+  }
+  g.C = d_dWh_stack;
+  rc = zr_gemm_launch(ctx, g);
+  if (rc) return rc;
+  row_sum_kernel<<<(4 * H + 63) / 64, 64, 0, ctx->stream>>>(d_dgates, 4 * H, K, d_db);
+  ZR_LAUNCH_CHECK("row_sum_kernel");
+  return ZR_OK;
+}
+
+int zr_embed_gradient(zr_ctx* ctx, int H, int V, const float* d_err, const int* d_ids_nonneg, const int* d_mask01,
+                      int n, float* d_dW) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(H > 0 && V > 0 && n >= 0 && n <= 65535 * 64, "zr_embed_gradient: H = %d, V = %d, n = %d", H, V, n);
+  if (n == 0) return ZR_OK;
+  ZR_CHECK_ARG(d_err && d_ids_nonneg && d_mask01 && d_dW, "zr_embed_gradient: null pointer");
+  for (int base = 0; base < n; base += 65535) {
+    const int cnt = n - base < 65535 ? n - base : 65535;
+    dim3 grid((H + 255) / 256, cnt);
+    embed_grad_kernel<<<grid, 256, 0, ctx->stream>>>(d_err + (size_t)base * H, d_ids_nonneg + base, d_mask01 + base, H, V,
+                                                     d_dW);
+    ZR_LAUNCH_CHECK("embed_grad_kernel");
+  }
+  return ZR_OK;
+}
+
+int zr_softmax_backward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int n,
+                        const int* d_target, const int* d_mask01, float* d_prob_scratch, float* d_err_h, float* d_dD,
+                        float* d_db) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(V > 0 && H > 0 && n > 0 && n <= 65535, "zr_softmax_backward: V = %d, H = %d, n = %d", V, H, n);
+  ZR_CHECK_ARG(d_D && d_b_d && d_h && d_target && d_mask01 && d_prob_scratch && d_err_h && d_dD && d_db,
+               "zr_softmax_backward: null pointer");
+  rc = zr_softmax_forward(ctx, d_D, d_b_d, V, H, d_h, n, ZR_SOFTMAX_PROB, d_prob_scratch, nullptr);
+  if (rc) return rc;
+  dim3 egrid((V + 255) / 256, n);
+  softmax_error_kernel<<<egrid, 256, 0, ctx->stream>>>(d_prob_scratch, V, d_target, d_mask01);
+  ZR_LAUNCH_CHECK("softmax_error_kernel");
+  // err_h = D^T e
+  ZrGemmDesc g = {};
+  g.M = H;
+  g.N = n;
+  g.nseg = 1;
+  g.K[0] = V;
+  g.A[0] = d_D;
+  g.lda[0] = V;
+  g.trans_a = 1;
+  g.B[0] = d_prob_scratch;
+  g.ldb[0] = V;
+  g.C = d_err_h;
+  g.ldc = H;
+  g.batch = 1;
+  g.epilogue = ZR_EPI_STORE;
+  rc = zr_gemm_launch(ctx, g);
+  if (rc) return rc;
+  // dD = e h^T : right-hand side h^T as an n x H column-major matrix
+  void* scratch = nullptr;
+  rc = zr_ctx_scratch(ctx, 0, sizeof(float) * (size_t)n * H, &scratch);
+  if (rc) return rc;
+  float* ht = (float*)scratch;
+  rc = transpose_launch(ctx, d_h, H, n, ht, n, 0);
+  if (rc) return rc;
+  ZrGemmDesc w = {};
+  w.M = V;
+  w.N = H;
+  w.nseg = 1;
+  w.K[0] = n;
+  w.A[0] = d_prob_scratch;
+  w.lda[0] = V;
+  w.B[0] = ht;
+  w.ldb[0] = n;
+  w.C = d_dD;
+  w.ldc = V;
+  w.batch = 1;
+  w.epilogue = ZR_EPI_STORE;
+  rc = zr_gemm_launch(ctx, w);
+  if (rc) return rc;
+  row_sum_kernel<<<(V + 63) / 64, 64, 0, ctx->stream>>>(d_prob_scratch, V, n, d_db);
+  ZR_LAUNCH_CHECK("row_sum_kernel");
+  return ZR_OK;
+}
+
+int zr_sgd_update(zr_ctx* ctx, float* d_W, const float* d_grad, long long n, float scale, float norm_clip,
+                  float learning_rate) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(n >= 0 && (n == 0 || (d_W && d_grad)), "zr_sgd_update: null pointer or n = %lld", n);
+  if (n == 0) return ZR_OK;
+  const int n_partial = 256;
+  void* scratch = nullptr;
+  rc = zr_ctx_scratch(ctx, 1, sizeof(double) * n_partial, &scratch);
+  if (rc) return rc;
+  if (norm_clip > 0.0f) {
+    sumsq_partial_kernel<<<n_partial, 256, 0, ctx->stream>>>(d_grad, n, (double*)scratch);
+    ZR_LAUNCH_CHECK("sumsq_partial_kernel");
+  }
+  const long long blocks = (n + 255) / 256;
+  sgd_apply_kernel<<<(unsigned)(blocks < 2048 ? blocks : 2048), 256, 0, ctx->stream>>>(
+      d_W, d_grad, n, scale, norm_clip, learning_rate, (const double*)scratch, n_partial);
+  ZR_LAUNCH_CHECK("sgd_apply_kernel");
+  return ZR_OK;
+}
+
+}  // extern "C"

@@ -687,6 +687,14 @@ int zr_lstm_stack_forward(zr_ctx* ctx, int nl, const zr_lstm_weights* const laye
                           const int* d_ids_nonneg, const int* d_mask01, int T, int mb,
                           const float* const d_h0[], const float* const d_c0[], float clip_threshold,
                           float* const d_h_all[], float* const d_c_all[]) {
+  return zr_lstm_stack_forward_train(ctx, nl, layers, d_embed, V, d_ids_nonneg, d_mask01, T, mb, d_h0, d_c0,
+                                     clip_threshold, d_h_all, d_c_all, nullptr);
+}
+
+int zr_lstm_stack_forward_train(zr_ctx* ctx, int nl, const zr_lstm_weights* const layers[], const float* d_embed,
+                                int V, const int* d_ids_nonneg, const int* d_mask01, int T, int mb,
+                                const float* const d_h0[], const float* const d_c0[], float clip_threshold,
+                                float* const d_h_all[], float* const d_c_all[], float* const d_gates_all[]) {
   int rc = zr_bind_device(ctx);
   if (rc) return rc;
   ZR_CHECK_ARG(nl > 0 && T > 0 && mb > 0 && V > 0, "zr_lstm_stack_forward: L = %d, T = %d, mb = %d, V = %d", nl, T,
@@ -748,7 +756,8 @@ int zr_lstm_stack_forward(zr_ctx* ctx, int nl, const zr_lstm_weights* const laye
       U.mask01 = d_mask01 + (size_t)t * mb;
       U.h = d_h_all[l] + (size_t)t * n;
       U.c = d_c_all[l] + (size_t)t * n;
-      for (int g = 0; g < 4; ++g) U.gates[g] = nullptr;
+      for (int g = 0; g < 4; ++g)
+        U.gates[g] = (d_gates_all && d_gates_all[l]) ? d_gates_all[l] + ((size_t)t * 4 + g) * n : nullptr;
       U.nseg = 2;
       if (nu == kMaxUnits) {
         L.n_units = nu;
