@@ -162,6 +162,79 @@ def bench_decoder_step(ctx, steps, warmup, H=1000, mb=128, S=50, V=50000, L=4, D
     return res
 
 
+def bench_training_step(ctx, steps, H=1000, mb=128, T=50, V=50000, L=4, lr=0.5, norm_clip=5.0):
+    """A language-model training step at the headline shape: forward sweep keeping the gates, output-layer backward
+    over all T*mb columns, back-propagation through time, weight / bias / embedding gradients and the clipped SGD
+    update of every parameter (no attention, no dropout)."""
+    from zoph_rnn_amd import synth
+    cfg = synth.encoder_config(H=H, mb=mb, T=T, V=V, L=L)
+    g = synth.rng(synth.SEED, 7)
+    layers = [Uploaded(ctx, ly) for ly in cfg["layers"]]
+    trains = [ctx.lstm_train_create(ly.M, ly.Wh, H) for ly in layers]
+    d_embed = ctx.array(cfg["embed"])
+    ids = cfg["ids"]
+    n, N = H * mb, T * mb
+    d_nn, d_m = ctx.empty(ids.size, np.int32), ctx.empty(ids.size, np.int32)
+    ctx.vocab_prep(ctx.array(ids.reshape(-1)), ids.size, V, d_nn, d_m)
+    dD, dbd = ctx.array(synth.uniform(g, (V, H))), ctx.array(synth.uniform(g, (V,)))
+    ctx.softmax_prepare(dD, V, H)
+    d_tgt = ctx.array(synth.zipf_ids(g, (N,), V).astype(np.int32))
+    z = ctx.zeros((H, mb))
+    h_all = [ctx.empty((n * T,)) for _ in range(L)]
+    c_all = [ctx.empty((n * T,)) for _ in range(L)]
+    g_all = [ctx.empty((4 * n * T,)) for _ in range(L)]
+    dg_all = [ctx.empty((4 * n * T,)) for _ in range(L)]
+    eh0, ec0 = [ctx.empty((H, mb)) for _ in range(L)], [ctx.empty((H, mb)) for _ in range(L)]
+    d_err_top, d_below0, x_all = ctx.empty((n * T,)), ctx.empty((n * T,)), ctx.empty((n * T,))
+    d_scr, g_D, g_bd, g_W = ctx.empty((V, N)), ctx.empty((V, H)), ctx.empty((V,)), ctx.zeros((H, V))
+    g_M = [ctx.empty((4 * H, H)) for _ in range(L)]
+    g_Wh = [ctx.empty((4 * H, H)) for _ in range(L)]
+    g_b = [ctx.empty((4 * H,)) for _ in range(L)]
+    u_M = [[ctx.empty((H, H)) for _ in range(4)] for _ in range(L)]
+    u_Wh = [[ctx.empty((H, H)) for _ in range(4)] for _ in range(L)]
+    ws = [ly.w for ly in layers]
+    sc = 1.0 / mb
+
+    def step():
+        ctx.lstm_stack_forward_train(ws, d_embed, V, d_nn, d_m, T, mb, [z] * L, [z] * L, h_all, c_all, g_all)
+        ctx.softmax_backward(dD, dbd, V, H, h_all[L - 1], N, d_tgt, d_m, d_scr, d_err_top, g_D, g_bd)
+        ctx.lstm_stack_backward(trains, T, mb, d_m, [z] * L, c_all, g_all, d_err_top, dg_all, eh0, ec0,
+                                d_err_below0=d_below0)
+        ctx.embed_gather(d_embed, H, V, d_nn, N, x_all)
+        for l in range(L):
+            ctx.lstm_weight_gradients(H, T, mb, dg_all[l], x_all if l == 0 else h_all[l - 1], z, h_all[l], g_M[l], g_Wh[l],
+                                      g_b[l])
+        ctx.memset_zero(g_W)
+        ctx.embed_gradient(H, V, d_below0, d_nn, d_m, N, g_W)
+        # update_weights: every parameter, then refresh the forward / backward copies of the matrices
+        ctx.sgd_update(dD, g_D, V * H, sc, norm_clip, lr)
+        ctx.sgd_update(dbd, g_bd, V, sc, norm_clip, lr)
+        ctx.sgd_update(d_embed, g_W, H * V, sc, norm_clip, lr)
+        for l in range(L):
+            ctx.unstack_gates(g_M[l], H, u_M[l])
+            ctx.unstack_gates(g_Wh[l], H, u_Wh[l])
+            for q in range(4):
+                ctx.sgd_update(layers[l].M[q], u_M[l][q], H * H, sc, norm_clip, lr)
+                ctx.sgd_update(layers[l].Wh[q], u_Wh[l][q], H * H, sc, norm_clip, lr)
+                ctx.sgd_update(layers[l].b[q], g_b[l].at(q * H), H, sc, norm_clip, lr)
+            ctx.lstm_weights_destroy(layers[l].w)
+            layers[l].w = ctx.lstm_pack(layers[l].M, layers[l].Wh, layers[l].b, H)
+            ws[l] = layers[l].w
+            ctx.lstm_train_refresh(trains[l], layers[l].M, layers[l].Wh)
+        ctx.softmax_prepare(dD, V, H)
+
+    wall_ms, ev_ms = time_region(ctx, step, steps, 1)
+    flops = 3 * 2.0 * 4 * H * N * (2 * H) * L + 3 * 2.0 * V * H * N  # forward + two backward products of each size
+    res = {"ms_per_step": round(ev_ms / steps, 3), "tokens_per_s": round(N * steps / (ev_ms * 1e-3), 1),
+           "tflops": round(flops * steps / (ev_ms * 1e-3) / 1e12, 1), "gflop_per_step": round(flops / 1e9, 1),
+           "what": "4-layer H=%d LM, minibatch %d x %d steps, vocabulary %d: forward, backward, gradients, clipped SGD"
+                   % (H, mb, T, V)}
+    ctx.softmax_release(dD)
+    for t in trains:
+        ctx.lstm_train_destroy(t)
+    return res
+
+
 def bench_hbm_kernels(ctx, steps, H=1000, mb=128, V=50000):
     """Stand-alone HBM-bound kernels at the benchmark shape: achieved GB/s of algorithmic bytes."""
     from zoph_rnn_amd import synth
@@ -257,6 +330,8 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the config-3 and HBM-kernel measurements")
     ap.add_argument("--lstm-tn", type=int, default=0)
     ap.add_argument("--lstm-ks", type=int, default=0)
+    ap.add_argument("--training-only", action="store_true",
+                    help="only run the language-model training step measurement (for profiling) and exit")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain copy kernel of known size (for scaling HBM traffic counters) and exit")
     args = ap.parse_args()
@@ -274,6 +349,10 @@ def main():
 
     if args.calibrate_copy:
         print(json.dumps(calibrate_copy(ctx)))
+        ctx.close()
+        return
+    if args.training_only:
+        print(json.dumps(bench_training_step(ctx, max(2, args.steps // 6))))
         ctx.close()
         return
 
@@ -295,6 +374,8 @@ def main():
         c5["weights"] = "bf16 storage (LSTM, attention projections, output layer), fp32 activations split in two bf16 terms, fp32 accumulation"
         extra["config5_decoder_step_bf16_weights"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in c5.items()}
         log("config5:", extra["config5_decoder_step_bf16_weights"])
+        extra["lm_training_step"] = bench_training_step(ctx, max(2, args.steps // 6))
+        log("training step:", extra["lm_training_step"])
         extra["hbm_kernels"] = bench_hbm_kernels(ctx, args.steps)
         extra["config4_beam_decode"] = bench_beam_decode(ctx, args.steps)
         log("config4:", extra["config4_beam_decode"])

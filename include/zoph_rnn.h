@@ -255,8 +255,8 @@ int zr_lstm_stack_forward_train(zr_ctx* ctx, int L, const zr_lstm_weights* const
                                 const float* const d_h0[], const float* const d_c0[], float clip_threshold,
                                 float* const d_h_all[], float* const d_c_all[], float* const d_gates_all[]);
 
-/* Backward-side copy of one layer's matrices: M_g and W_hg stacked over the four gates as 4H x H matrices (rows
- * g*H + j), the operands of the error products d_ERRnTOt_htM1 = sum_g W_hg^T err_g and d_ERRnTOt_h_Below =
+/* Backward-side copy of one layer's matrices: M_g and W_hg stacked over the four gates and transposed (H x 4H,
+ * element (k, g*H + j) = W_g[j][k]), the operands of the error products d_ERRnTOt_htM1 = sum_g W_hg^T err_g and d_ERRnTOt_h_Below =
  * sum_g M_g^T err_g (src/LSTM_HH.hpp:470-560).  Call zr_lstm_train_refresh after the weights change. */
 typedef struct zr_lstm_train zr_lstm_train;
 int zr_lstm_train_create(zr_ctx* ctx, const float* const d_M[4], const float* const d_Wh[4], int H, zr_lstm_train** out);

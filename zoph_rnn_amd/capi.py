@@ -161,6 +161,9 @@ class Context:
     def zeros(self, shape, dtype=np.float32):
         return DeviceArray(self, shape, dtype, zero=True)
 
+    def memset_zero(self, d_arr):
+        _chk(load().zr_memset_zero(self.h, C.c_void_p(d_arr.ptr), C.c_size_t((d_arr.nbytes + 3) // 4 * 4)))
+
     # ---- A1
     def vocab_prep(self, d_ids, n, vocab, d_nonneg, d_mask):
         _chk(load().zr_vocab_prep(self.h, _vp(d_ids), C.c_int(n), C.c_int(vocab), _vp(d_nonneg), _vp(d_mask)))

@@ -18,7 +18,9 @@
 
 struct zr_lstm_train {
   int H;
-  float* d_stack;  // [2][4H x H] column-major: Wh stacked over the gates (rows g*H + j), then M
+  // [2][H x 4H] column-major: the TRANSPOSE of Wh stacked over the gates, then of M: element (k, g*H + j) = W_g[j][k].
+  // The error products sum_g W_g^T err_g are then plain products with contiguous weight rows.
+  float* d_stack;
 };
 
 namespace {
@@ -28,13 +30,21 @@ inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 __global__ void __launch_bounds__(256) stack_gates_kernel(const float* __restrict__ g0, const float* __restrict__ g1,
                                                           const float* __restrict__ g2, const float* __restrict__ g3,
                                                           int H, float* __restrict__ dst) {
-  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;  // over the 4H x H destination
-  if (i >= 4LL * H * H) return;
-  const int r = (int)(i % (4 * H));
-  const int k = (int)(i / (4 * H));
-  const int g = r / H, j = r - g * H;
+  // dst: H x 4H column-major, dst[k + (g*H + j)*H] = W_g[j + k*H]; 32 x 32 tiles through LDS
+  __shared__ float tile[32][33];
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  const int g = blockIdx.z;
   const float* src = g == 0 ? g0 : (g == 1 ? g1 : (g == 2 ? g2 : g3));
-  dst[i] = src[j + (long long)k * H];
+  const int j0 = blockIdx.x * 32, k0 = blockIdx.y * 32;
+  for (int i = ty; i < 32; i += 8) {
+    const int j = j0 + tx, k = k0 + i;
+    tile[i][tx] = (j < H && k < H) ? src[j + (long long)k * H] : 0.0f;
+  }
+  __syncthreads();
+  for (int i = ty; i < 32; i += 8) {
+    const int k = k0 + tx, j = j0 + i;
+    if (j < H && k < H) dst[k + ((long long)g * H + j) * H] = tile[tx][i];
+  }
 }
 
 __global__ void __launch_bounds__(256) unstack_gates_kernel(const float* __restrict__ src, int H, float* __restrict__ g0,
@@ -96,13 +106,24 @@ __global__ void __launch_bounds__(256) transpose_kernel(const float* __restrict_
   }
 }
 
-// out[r] = sum over the n columns of a (rows x n, column-major).  One wave per 64 rows; fixed order.
-__global__ void __launch_bounds__(64) row_sum_kernel(const float* __restrict__ a, int rows, long long n,
-                                                     float* __restrict__ out) {
+// Row sums of a (rows x n, column-major) in two stages with a fixed summation order: stage 1 sums column chunk
+// blockIdx.y for 64 rows per wave into partial[chunk][rows]; stage 2 adds the chunks.
+__global__ void __launch_bounds__(64) row_sum_partial_kernel(const float* __restrict__ a, int rows, long long n,
+                                                             long long chunk, float* __restrict__ partial) {
+  const int r = blockIdx.x * 64 + threadIdx.x;
+  if (r >= rows) return;
+  const long long k0 = (long long)blockIdx.y * chunk;
+  const long long k1 = k0 + chunk < n ? k0 + chunk : n;
+  float s = 0.0f;
+  for (long long k = k0; k < k1; ++k) s += a[r + k * rows];
+  partial[(size_t)blockIdx.y * rows + r] = s;
+}
+__global__ void __launch_bounds__(64) row_sum_final_kernel(const float* __restrict__ partial, int rows, int chunks,
+                                                           float* __restrict__ out) {
   const int r = blockIdx.x * 64 + threadIdx.x;
   if (r >= rows) return;
   float s = 0.0f;
-  for (long long k = 0; k < n; ++k) s += a[r + k * rows];
+  for (int c = 0; c < chunks; ++c) s += partial[(size_t)c * rows + r];
   out[r] = s;
 }
 
@@ -170,6 +191,20 @@ __global__ void __launch_bounds__(256) sgd_apply_kernel(float* __restrict__ W, c
   for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) W[i] += f * g[i];
 }
 
+int row_sum_launch(zr_ctx* ctx, const float* a, int rows, long long n, float* out) {
+  const long long chunk = 64;
+  const int chunks = (int)((n + chunk - 1) / chunk);
+  void* scratch = nullptr;
+  int rc = zr_ctx_scratch(ctx, 0, sizeof(float) * (size_t)chunks * rows, &scratch);
+  if (rc) return rc;
+  dim3 grid((rows + 63) / 64, chunks);
+  row_sum_partial_kernel<<<grid, 64, 0, ctx->stream>>>(a, rows, n, chunk, (float*)scratch);
+  ZR_LAUNCH_CHECK("row_sum_partial_kernel");
+  row_sum_final_kernel<<<(rows + 63) / 64, 64, 0, ctx->stream>>>((const float*)scratch, rows, chunks, out);
+  ZR_LAUNCH_CHECK("row_sum_final_kernel");
+  return ZR_OK;
+}
+
 int transpose_launch(zr_ctx* ctx, const float* src, int rows, int cols, float* dst, long long ldd, int row0) {
   dim3 grid((rows + 31) / 32, (cols + 31) / 32);
   transpose_kernel<<<grid, 256, 0, ctx->stream>>>(src, rows, cols, dst, ldd, row0);
@@ -208,7 +243,7 @@ int zr_lstm_train_refresh(zr_ctx* ctx, zr_lstm_train* w, const float* const d_M[
   ZR_CHECK_ARG(w && d_M && d_Wh, "zr_lstm_train_refresh: null pointer");
   const int H = w->H;
   const size_t per = 4 * (size_t)H * H;
-  const unsigned grid = (unsigned)((per + 255) / 256);
+  dim3 grid((H + 31) / 32, (H + 31) / 32, 4);
   stack_gates_kernel<<<grid, 256, 0, ctx->stream>>>(d_Wh[0], d_Wh[1], d_Wh[2], d_Wh[3], H, w->d_stack);
   ZR_LAUNCH_CHECK("stack_gates_kernel");
   stack_gates_kernel<<<grid, 256, 0, ctx->stream>>>(d_M[0], d_M[1], d_M[2], d_M[3], H, w->d_stack + per);
@@ -293,8 +328,7 @@ int zr_lstm_stack_backward(zr_ctx* ctx, int nl, const zr_lstm_train* const layer
       g.nseg = 1;
       g.K[0] = 4 * H;
       g.A[0] = layers[l]->d_stack;
-      g.lda[0] = 4 * H;
-      g.trans_a = 1;
+      g.lda[0] = H;
       g.B[0] = dg;
       g.ldb[0] = 4 * H;
       g.C = w_l;
@@ -357,9 +391,7 @@ int zr_lstm_weight_gradients(zr_ctx* ctx, int H, int T, int mb, const float* d_d
   g.C = d_dWh_stack;
   rc = zr_gemm_launch(ctx, g);
   if (rc) return rc;
-  row_sum_kernel<<<(4 * H + 63) / 64, 64, 0, ctx->stream>>>(d_dgates, 4 * H, K, d_db);
-  ZR_LAUNCH_CHECK("row_sum_kernel");
-  return ZR_OK;
+  return row_sum_launch(ctx, d_dgates, 4 * H, K, d_db);
 }
 
 int zr_embed_gradient(zr_ctx* ctx, int H, int V, const float* d_err, const int* d_ids_nonneg, const int* d_mask01,
@@ -392,28 +424,36 @@ int zr_softmax_backward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V
   dim3 egrid((V + 255) / 256, n);
   softmax_error_kernel<<<egrid, 256, 0, ctx->stream>>>(d_prob_scratch, V, d_target, d_mask01);
   ZR_LAUNCH_CHECK("softmax_error_kernel");
-  // err_h = D^T e
+  // err_h = D^T e, computed as (e^T D)^T: with e^T as the left operand the product is tall (n rows) with contiguous
+  // rows, the shape the large-matrix kernels are built for; the two transposes move 2 x V*n + 2 x n*H floats.
+  void *s0 = nullptr, *s1 = nullptr;
+  rc = zr_ctx_scratch(ctx, 1, sizeof(float) * (size_t)V * n, &s1);
+  if (rc) return rc;
+  rc = zr_ctx_scratch(ctx, 0, sizeof(float) * (size_t)n * H, &s0);
+  if (rc) return rc;
+  float* et = (float*)s1;   // n x V
+  float* ct = (float*)s0;   // n x H
+  rc = transpose_launch(ctx, d_prob_scratch, V, n, et, n, 0);
+  if (rc) return rc;
   ZrGemmDesc g = {};
-  g.M = H;
-  g.N = n;
+  g.M = n;
+  g.N = H;
   g.nseg = 1;
   g.K[0] = V;
-  g.A[0] = d_D;
-  g.lda[0] = V;
-  g.trans_a = 1;
-  g.B[0] = d_prob_scratch;
+  g.A[0] = et;
+  g.lda[0] = n;
+  g.B[0] = d_D;
   g.ldb[0] = V;
-  g.C = d_err_h;
-  g.ldc = H;
+  g.C = ct;
+  g.ldc = n;
   g.batch = 1;
   g.epilogue = ZR_EPI_STORE;
   rc = zr_gemm_launch(ctx, g);
   if (rc) return rc;
-  // dD = e h^T : right-hand side h^T as an n x H column-major matrix
-  void* scratch = nullptr;
-  rc = zr_ctx_scratch(ctx, 0, sizeof(float) * (size_t)n * H, &scratch);
+  rc = transpose_launch(ctx, ct, n, H, d_err_h, H, 0);
   if (rc) return rc;
-  float* ht = (float*)scratch;
+  // dD = e h^T : right-hand side h^T as an n x H column-major matrix
+  float* ht = (float*)s0;  // the product above has been queued: the buffer is free again in stream order
   rc = transpose_launch(ctx, d_h, H, n, ht, n, 0);
   if (rc) return rc;
   ZrGemmDesc w = {};
@@ -431,9 +471,7 @@ int zr_softmax_backward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V
   w.epilogue = ZR_EPI_STORE;
   rc = zr_gemm_launch(ctx, w);
   if (rc) return rc;
-  row_sum_kernel<<<(V + 63) / 64, 64, 0, ctx->stream>>>(d_prob_scratch, V, n, d_db);
-  ZR_LAUNCH_CHECK("row_sum_kernel");
-  return ZR_OK;
+  return row_sum_launch(ctx, d_prob_scratch, V, n, d_db);
 }
 
 int zr_sgd_update(zr_ctx* ctx, float* d_W, const float* d_grad, long long n, float scale, float norm_clip,

@@ -710,7 +710,7 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
   }
   // Large, untransposed, single-segment products with a wide batch (the softmax logits): LDS-shared weights.
   const bool lds_ok = !d.trans_a && d.nseg == 1 && d.batch == 1 && vec && (d.M % 4 == 0) && (d.lda[0] % 4 == 0) &&
-                      (((uintptr_t)d.A[0] & 15u) == 0) && d.K[0] >= 8 && d.M >= 4096 && d.N >= 96 &&
+                      (((uintptr_t)d.A[0] & 15u) == 0) && d.K[0] >= 8 && d.M >= 2048 && d.N >= 96 &&
                       (d.epilogue == ZR_EPI_STORE || d.epilogue == ZR_EPI_SOFTMAX_PARTIAL);
   if (lds_ok && ctx->gemm_cfg == 10) return launch_lds<4, 4>(ctx, ga, d.epilogue);
   if (lds_ok && (ctx->gemm_cfg == 0 || ctx->gemm_cfg == 9)) {
