@@ -147,7 +147,7 @@ def test_sgd_update(ctx, n, clip):
 
 
 def test_language_model_training_step_gradients(ctx):
-    """BASELINE config 1 shape (1-layer LM, H=100, minibatch 8, T=20, V=10000): the full gradient of the summed
+    """benchmark configuration 1 shape (1-layer LM, H=100, minibatch 8, T=20, V=10000): the full gradient of the summed
     log-likelihood -- output layer, LSTM matrices and biases, embedding -- from one forward/backward pass."""
     c = synth.config1()
     H, mb, T, V = c["H"], c["mb"], c["T"], c["V"]

@@ -1,4 +1,4 @@
-"""Reduced-precision weights (BASELINE config 5: weights stored as bf16, fp32 accumulation, fp32 cell state).
+"""Reduced-precision weights (benchmark configuration 5: weights stored as bf16, fp32 accumulation, fp32 cell state).
 
 The reference has no reduced-precision path, so the bar is the oracle (double accumulation) run on the SAME
 bf16-rounded weights: that isolates what the HIP path adds on top of the storage format -- the two-term bf16 split of
@@ -239,7 +239,7 @@ def test_attention_bf16_weights(ctx, H, mb, S, D):
 
 
 def test_config5_decoder_step_reduced_vocab(ctx):
-    """BASELINE config 5 wiring (bf16 weights everywhere a matrix is streamed: 4 LSTM layers with feed-input,
+    """benchmark configuration 5 wiring (bf16 weights everywhere a matrix is streamed: 4 LSTM layers with feed-input,
     attention projections, output layer) at H=2000, minibatch 256, S=50; vocabulary reduced to 2000 and 48 of the
     256 columns checked against the oracle so that it finishes in seconds."""
     c = synth.decoder_config(H=2000, mb=256, V=2000)

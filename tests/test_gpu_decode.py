@@ -1,4 +1,4 @@
-"""End-to-end beam decode (BASELINE config 4 wiring at sizes the oracle finishes in seconds): encoder, then per step
+"""End-to-end beam decode (benchmark configuration 4 wiring at sizes the oracle finishes in seconds): encoder, then per step
 embedding gather -> LSTM stack with feed-input -> attention -> softmax -> device-side beam -> state reorder, for
 several sentences side by side, against one oracle decode per sentence (the reference decodes one sentence per
 pass).  Selected words and back-pointers must be identical at every step, hypotheses identical at the end."""

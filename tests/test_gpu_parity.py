@@ -251,7 +251,7 @@ def test_stack_forward_small_with_padding(ctx):
 
 
 def test_config1_lm_forward_logprobs_and_loss(ctx):
-    """BASELINE config 1: 1-layer LM, H=100, mb=8, T=20, V=10000; per-step full log-probs and the summed loss."""
+    """benchmark configuration 1: 1-layer LM, H=100, mb=8, T=20, V=10000; per-step full log-probs and the summed loss."""
     c = synth.config1()
     H, mb, T, V = c["H"], c["mb"], c["T"], c["V"]
     hs, _ = _run_stack(ctx, c["layers"], c["embed"], c["ids"])
@@ -415,7 +415,7 @@ def test_attention_negative_scores_use_zero_initialised_max(ctx):
 
 
 def test_config3_decoder_step_reduced_vocab(ctx):
-    """BASELINE config 3 wiring at H=1000, mb=128, S=50 with D=50 ("global") and D=10: LSTM stack with
+    """benchmark configuration 3 wiring at H=1000, mb=128, S=50 with D=50 ("global") and D=10: LSTM stack with
     feed-input on layer 0, attention on the top layer, softmax over a reduced vocabulary so that the oracle
     finishes in seconds (the full-vocabulary softmax is covered by test_softmax_full_vocab_properties)."""
     c = synth.decoder_config(V=2000)
