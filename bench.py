@@ -270,8 +270,6 @@ def bench_hbm_kernels(ctx, steps, H=1000, mb=128, V=50000):
     bytes_ = 7.0 * H * mbL * 4 + 4 * H * 4 + mbL * 4
     out["lstm_gates_6400_columns"] = {"us": round(ms * 1e3 / steps, 2), "algorithmic_MB": round(bytes_ / 1e6, 3),
                                       "GBps": round(bytes_ * steps / (ms * 1e-3) / 1e9, 1)}
-    # softmax without the product: zero weights make the logits the bias, so the V x mb normalisation dominates
-    # (column statistics + one read and one write of the V x mb matrix; the 12.8 GFLOP product is still issued)
     return out
 
 
