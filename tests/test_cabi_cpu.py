@@ -43,6 +43,20 @@ def test_null_context_and_bad_arguments_return_errors():
     assert lib.zr_ctx_create(0, None) == -1
     assert lib.zr_embed_gather(None, None, 8, 8, None, 1, None) == -1  # V checked before the context is touched
     assert lib.zr_gemm(None, 0, 4, 4, 4, None, 4, None, 4, None, 4) == -1
+    # entry points added later follow the same convention: a null context is an argument error, never a crash
+    assert lib.zr_softmax_prepare(None, None, 10, 8) == -1
+    assert lib.zr_softmax_prepare_bf16(None, None, 10, 8) == -1
+    assert lib.zr_softmax_release(None, None) == -1
+    assert lib.zr_attn_use_bf16_weights(None, None) == -1
+    assert lib.zr_lstm_pack_weights_bf16(None, None, None, None, None, 16, None) == -1
+    assert lib.zr_lstm_train_create(None, None, None, 8, None) == -1
+    assert lib.zr_unstack_gates(None, None, 8, None) == -1
+    assert lib.zr_lstm_stack_backward(None, 1, None, 1, 1, None, None, None, None, None, None, None, None, None, None,
+                                      None) == -1
+    assert lib.zr_lstm_weight_gradients(None, 8, 1, 1, None, None, None, None, None, None, None) == -1
+    assert lib.zr_embed_gradient(None, 8, 8, None, None, None, 1, None) == -1
+    assert lib.zr_softmax_backward(None, None, None, 8, 8, None, 1, None, None, None, None, None, None) == -1
+    assert lib.zr_sgd_update(None, None, None, C.c_longlong(4), C.c_float(1), C.c_float(0), C.c_float(0.1)) == -1
 
 
 def test_context_creation_without_gpu_fails_cleanly():
