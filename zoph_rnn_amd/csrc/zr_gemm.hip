@@ -23,6 +23,9 @@ struct GemmArgs {
   float* partials;
   int m_tiles, n_tiles;  // wave tiles along M and N
   int b_pack4;           // B segments are k-interleaved copies: element (k, n) at ((k/4)*N + n)*4 + k%4
+  // bf16 weights: B[s] is the bf16 "hi" array and Blo[s] the "lo" array of the split activations, both
+  // k-interleaved by 8 ([K/8][N][8]); see zr_split_pack_x_kernel
+  const unsigned short* Blo[3];
 };
 
 // largest divisor c of nv with c * tm <= 32
@@ -72,9 +75,14 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& a, int m0, int n0, boo
         wbase[tm] = (const unsigned short*)a.A[s];
         woff[tm] = (unsigned)(8LL * rows[tm] + 8LL * half * a.lda[s]);
       }
+      const unsigned short* xlo[TN];
 #pragma unroll
-      for (int tn = 0; tn < TN; ++tn) xcol[tn] = a.B[s] + (long long)cols[tn] * a.ldb[s] + 8 * half;
-      zr_mma_segment_bf16<TM, TN, KS, PF>(acc, wbase, woff, a.lda[s], xcol, a.K[s], kslice);
+      for (int tn = 0; tn < TN; ++tn) {
+        const long long off = 8LL * (cols[tn] + (long long)half * a.N);
+        xcol[tn] = (const float*)((const unsigned short*)a.B[s] + off);
+        xlo[tn] = a.Blo[s] + off;
+      }
+      zr_mma_segment_bf16<TM, TN, KS, PF, true>(acc, wbase, woff, a.lda[s], xcol, a.K[s], kslice, xlo, a.N);
     } else {
       const float* A = a.A[s] + (long long)z * a.strideA;
       const float* wbase[TM];
@@ -558,6 +566,28 @@ int launch_rows(zr_ctx* ctx, GemmArgs& ga, int epi, int n_tiles) {
   return ZR_OK;
 }
 
+// Activations X (K x N fp32, column n at src + n*ld, K % 8 == 0) -> two bf16 arrays hi and lo with x = hi + lo up
+// to 2^-16 |x|, each k-interleaved by 8: element (k, n) at ((k/8)*N + n)*8 + k%8.  One thread per 8 values.
+__global__ void __launch_bounds__(256) zr_split_pack_x_kernel(const float* __restrict__ src, int K, int N, int ld,
+                                                              unsigned short* __restrict__ hi,
+                                                              unsigned short* __restrict__ lo) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  const int kb = K >> 3;
+  if (i >= kb * N) return;
+  const int n = i / kb, b = i - n * kb;
+  const zr_f32x4 v0 = *(const zr_f32x4*)(src + (long long)n * ld + 8 * b);
+  const zr_f32x4 v1 = *(const zr_f32x4*)(src + (long long)n * ld + 8 * b + 4);
+  zr_u32x4 h, l;
+  unsigned a, c;
+  zr_split_bf16_pair(v0.x, v0.y, a, c); h.x = a; l.x = c;
+  zr_split_bf16_pair(v0.z, v0.w, a, c); h.y = a; l.y = c;
+  zr_split_bf16_pair(v1.x, v1.y, a, c); h.z = a; l.z = c;
+  zr_split_bf16_pair(v1.z, v1.w, a, c); h.w = a; l.w = c;
+  const long long o = ((long long)b * N + n) * 8;
+  *(zr_u32x4*)(hi + o) = h;
+  *(zr_u32x4*)(lo + o) = l;
+}
+
 __global__ void __launch_bounds__(256) pack4_kernel(const float* __restrict__ src, int M, int K, long long ld,
                                                     int ldp, int kp, float* __restrict__ dst) {
   const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
@@ -588,6 +618,14 @@ int zr_pack8_bf16_launch(zr_ctx* ctx, const float* src, int M, int K, long long 
   const long long total = (long long)kp * ldp;
   pack8_bf16_kernel<<<(unsigned)((total + 255) / 256), 256, 0, ctx->stream>>>(src, M, K, ld, ldp, kp, dst, trans);
   ZR_LAUNCH_CHECK("pack8_bf16_kernel");
+  return ZR_OK;
+}
+
+int zr_split_pack_x_launch(zr_ctx* ctx, const float* src, int K, int N, int ld, unsigned short* hi,
+                           unsigned short* lo) {
+  const int n8 = (K / 8) * N;
+  zr_split_pack_x_kernel<<<(n8 + 255) / 256, 256, 0, ctx->stream>>>(src, K, N, ld, hi, lo);
+  ZR_LAUNCH_CHECK("zr_split_pack_x_kernel");
   return ZR_OK;
 }
 
@@ -649,8 +687,27 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
   if (d.epilogue == ZR_EPI_SOFTMAX_PARTIAL) ZR_CHECK_ARG(d.bias && d.partials, "gemm: bias/partials required");
 
   ga.b_pack4 = 0;
+  for (int s = 0; s < 3; ++s) ga.Blo[s] = nullptr;
   if (d.a_pack == 2) {
     ZR_CHECK_ARG(vec, "gemm: bf16 operand A needs 16-byte aligned activations with ldb %% 4 == 0");
+    {
+      // split the fp32 activations into bf16 hi + lo once, k-interleaved, instead of in every workgroup's K loop
+      size_t elems = 0;
+      for (int s = 0; s < d.nseg; ++s) elems += (size_t)d.K[s] * d.N;
+      void* p = nullptr;
+      int rc = zr_ctx_scratch(ctx, 0, sizeof(unsigned short) * 2 * elems, &p);
+      if (rc) return rc;
+      unsigned short* hi = (unsigned short*)p;
+      for (int s = 0; s < d.nseg; ++s) {
+        const size_t e = (size_t)d.K[s] * d.N;
+        const int n8 = (d.K[s] / 8) * d.N;
+        zr_split_pack_x_kernel<<<(n8 + 255) / 256, 256, 0, ctx->stream>>>(d.B[s], d.K[s], d.N, d.ldb[s], hi, hi + e);
+        ZR_LAUNCH_CHECK("zr_split_pack_x_kernel");
+        ga.B[s] = (const float*)hi;
+        ga.Blo[s] = hi + e;
+        hi += 2 * e;
+      }
+    }
     if (d.nseg == 1 && d.M >= 8192 && d.N > 32 && d.N <= 1024 &&
         (d.epilogue == ZR_EPI_STORE || d.epilogue == ZR_EPI_SOFTMAX_PARTIAL)) {
       const int n32 = (d.N + 31) / 32;

@@ -109,6 +109,10 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d);
 // zero padding (ldp >= M a multiple of 32, kp >= K a multiple of 8).  dst holds kp*ldp floats.
 int zr_pack4_launch(zr_ctx* ctx, const float* src, int M, int K, long long ld, int ldp, int kp, float* dst);
 // Same for the bf16 layout [kp/8][ldp][8] (round to nearest even); kp a multiple of 16.  dst holds kp*ldp elements.
+// Activations X (K x N fp32, column-major with leading dimension ld, K % 8 == 0) split into bf16 hi + lo arrays
+// (K*N elements each), both k-interleaved by 8.
+int zr_split_pack_x_launch(zr_ctx* ctx, const float* src, int K, int N, int ld, unsigned short* hi,
+                           unsigned short* lo);
 // trans != 0: the source holds the transpose (element (row, k) at src[k + row*ld]).
 int zr_pack8_bf16_launch(zr_ctx* ctx, const float* src, int M, int K, long long ld, int ldp, int kp,
                          unsigned short* dst, int trans = 0);

@@ -23,6 +23,8 @@ struct LstmUnit {
   const float* bias;        // [4][H]
   const float* in[3];       // segment inputs, H x mb (ld = H)
   const float* inp[3];      // optional copies of the same inputs packed as [H/4][mb][4] (null: use in[])
+  const unsigned short* inp_lo[3];  // bf16 weights: inp[] then holds the bf16 "hi" half of the split inputs
+                                    // ([H/8][mb][8]) and inp_lo[] the "lo" half
   float* hp;                // optional: h is also written packed as [H/4][mb][4] for the units that consume it
   const int* gather_ids;    // non-null: column n of segment 0 is in[0] + ids[n]*H (embedding gather)
   const float* cprev;
@@ -57,7 +59,7 @@ constexpr int lstm_prefetch_depth(int tn, int ks) {
 #endif
 }
 
-template <int TN, int KS, bool VEC, bool BF16 = false>
+template <int TN, int KS, bool VEC, bool BF16 = false, bool XPK = false>
 __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
   __shared__ float red[KS * TN * 16 * 64];
   // Workgroup ids congruent modulo 8 run on the same XCD (round-robin dispatch) and share its L2.  Each XCD gets
@@ -136,7 +138,19 @@ __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
         }
         xcol[tn] = U.in[s] + c * H + 8 * half;
       }
-      zr_mma_segment_bf16<4, TN, KS, (TN == 1 ? 6 : 4)>(acc, wbase, woff, (long long)L.ldw, xcol, H, kslice);
+      if constexpr (XPK) {
+        const unsigned short* xlo[TN];
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) {
+          const long long off = 8LL * (cols[tn] + (long long)half * L.mb);
+          xcol[tn] = (const float*)((const unsigned short*)U.inp[s] + off);
+          xlo[tn] = U.inp_lo[s] + off;
+        }
+        zr_mma_segment_bf16<4, TN, KS, (TN == 1 ? 6 : 4), true>(acc, wbase, woff, (long long)L.ldw, xcol, H, kslice,
+                                                                 xlo, L.mb);
+      } else {
+        zr_mma_segment_bf16<4, TN, KS, (TN == 1 ? 6 : 4)>(acc, wbase, woff, (long long)L.ldw, xcol, H, kslice);
+      }
     } else {
       const float* wbase[4];
       unsigned woff[4];
@@ -453,7 +467,13 @@ int launch_fused_v(zr_ctx* ctx, const LstmLaunch& L, bool vec) {
   const int grid = ((groups + 7) / 8) * 8 * L.n_tiles;
   if (L.bf16) {
     if constexpr (KS == 4 && TN <= 2) {
-      lstm_fused_kernel<TN, KS, true, true><<<grid, 64 * KS, 0, ctx->stream>>>(L);
+      bool xpk = true;  // every segment of every unit has pre-split inputs
+      for (int i = 0; i < L.n_units; ++i)
+        for (int s2 = 0; s2 < L.u[i].nseg; ++s2) xpk = xpk && L.u[i].inp[s2] && L.u[i].inp_lo[s2];
+      if (xpk)
+        lstm_fused_kernel<TN, KS, true, true, true><<<grid, 64 * KS, 0, ctx->stream>>>(L);
+      else
+        lstm_fused_kernel<TN, KS, true, true><<<grid, 64 * KS, 0, ctx->stream>>>(L);
       ZR_LAUNCH_CHECK("lstm_fused_kernel (bf16 weights)");
       return ZR_OK;
     } else {
@@ -668,6 +688,21 @@ int zr_lstm_step(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_in, const
   U.nseg = nseg;
   U.V = 0;
   const bool vec = (H % 4 == 0) && aligned16(d_in) && aligned16(d_hprev) && (!d_htild || aligned16(d_htild));
+  if (w->bf16 && vec) {
+    // split the fp32 inputs into bf16 hi + lo once per node, k-interleaved, instead of in every workgroup's K loop
+    void* p = nullptr;
+    const size_t e = (size_t)H * mb;
+    rc = zr_ctx_scratch(ctx, 0, sizeof(unsigned short) * 2 * e * nseg, &p);
+    if (rc) return rc;
+    unsigned short* hi = (unsigned short*)p;
+    for (int s = 0; s < nseg; ++s) {
+      rc = zr_split_pack_x_launch(ctx, U.in[s], H, mb, H, hi, hi + e);
+      if (rc) return rc;
+      U.inp[s] = (const float*)hi;
+      U.inp_lo[s] = hi + e;
+      hi += 2 * e;
+    }
+  }
   if (!ctx->lstm_fused) {
     // reference-shaped two-phase path: the four pre-activation sums go to memory, then the stand-alone fused gate
     // kernel (the reference's element-wise kernels in one pass) adds the biases and runs the cell

@@ -299,6 +299,9 @@ __device__ __forceinline__ void zr_half_wave_softmax_stats(const float (&v)[G], 
 // the split.  Two bf16 instructions replace eight fp32 ones.
 //   woff[tm]:  8*row + 8*half*lda   (bf16 elements)
 //   xcol[tn]:  this lane's activation column advanced by 8*half
+// XPK: the activations were split and packed beforehand (zr_split_pack_x_kernel): two bf16 arrays hi and lo, each
+// k-interleaved like the weights ([K/8][N][8]); xcol[tn] / xlo[tn] then point at this lane's first block
+// (base + 8*(col + half*N)), xstride = N, and the loop body has no conversion arithmetic and only contiguous loads.
 // ---------------------------------------------------------------------------------------------------------
 enum { ZR_A_PACK8_BF16 = 3 };
 typedef __bf16 zr_bf16x8 __attribute__((ext_vector_type(8)));
@@ -321,14 +324,15 @@ __device__ __forceinline__ void zr_split_bf16_pair(float x0, float x1, unsigned&
 
 template <int TM, int TN>
 struct ZrFragBf16 {
-  zr_f32x4 x[TN][2];  // 8 consecutive k of this lane's column
+  zr_f32x4 x[TN][2];  // 8 consecutive k of this lane's column as fp32, or (XPK) [0] = hi and [1] = lo bf16 octets
   zr_u32x4 w[TM];     // 8 consecutive k of this lane's row, bf16
 };
 
-template <int TM, int TN, int KS, int PF>
+template <int TM, int TN, int KS, int PF, bool XPK = false>
 __device__ __forceinline__ void zr_mma_segment_bf16(zr_f32x16 (&acc)[TM][TN], const unsigned short* const (&wbase)[TM],
                                                     const unsigned (&woff)[TM], long long lda,
-                                                    const float* const (&xcol)[TN], int K, int kslice) {
+                                                    const float* const (&xcol)[TN], int K, int kslice,
+                                                    const unsigned short* const* xlo = nullptr, int xstride = 0) {
   const int nfull = K >> 4;  // K % 16 == 0 (checked by the host code)
   constexpr int NS = PF + 1;
 
@@ -336,8 +340,14 @@ __device__ __forceinline__ void zr_mma_segment_bf16(zr_f32x16 (&acc)[TM][TN], co
     const int kg = g * 16;  // wave-uniform
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) {
-      f.x[tn][0] = *(const zr_f32x4*)(xcol[tn] + kg);
-      f.x[tn][1] = *(const zr_f32x4*)(xcol[tn] + kg + 4);
+      if (XPK) {
+        const long long off = (long long)kg * xstride;  // bf16 elements; uniform
+        f.x[tn][0] = *(const zr_f32x4*)((const unsigned short*)xcol[tn] + off);
+        f.x[tn][1] = *(const zr_f32x4*)(xlo[tn] + off);
+      } else {
+        f.x[tn][0] = *(const zr_f32x4*)(xcol[tn] + kg);
+        f.x[tn][1] = *(const zr_f32x4*)(xcol[tn] + kg + 4);
+      }
     }
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) {
@@ -352,6 +362,16 @@ __device__ __forceinline__ void zr_mma_segment_bf16(zr_f32x16 (&acc)[TM][TN], co
     for (int tm = 0; tm < TM; ++tm) w[tm] = __builtin_bit_cast(zr_bf16x8, f.w[tm]);
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) {
+      if (XPK) {
+        const zr_bf16x8 ph = __builtin_bit_cast(zr_bf16x8, f.x[tn][0]), pl = __builtin_bit_cast(zr_bf16x8, f.x[tn][1]);
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ph, w[tm], acc[tm][tn], 0, 0, 0);
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pl, w[tm], acc[tm][tn], 0, 0, 0);
+        continue;
+      }
       unsigned h0, h1, h2, h3, l0, l1, l2, l3;
       zr_split_bf16_pair(f.x[tn][0].x, f.x[tn][0].y, h0, l0);
       zr_split_bf16_pair(f.x[tn][0].z, f.x[tn][0].w, h1, l1);
