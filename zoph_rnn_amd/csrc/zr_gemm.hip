@@ -227,9 +227,10 @@ __global__ void __launch_bounds__(64 * KS * WPB, OCC) gemm_kernel(GemmArgs a) {
   int mt, nt;
   if (AMODE == ZR_A_PACK4 || AMODE == ZR_A_PACK8_BF16) {
     // Workgroup ids congruent modulo 8 run on the same XCD.  Each XCD gets a contiguous range of row tiles and
-    // runs the column tiles of one row tile back to back, so a weight tile leaves memory once.
-    const int r8 = (int)(tile & 7);
-    const int q = (int)(tile >> 3);
+    // runs the column tiles of one row tile back to back (in neighbouring waves of a workgroup when WPB > 1), so a
+    // weight tile leaves memory once.
+    const int r8 = (int)(blockIdx.x & 7);
+    const int q = (int)(blockIdx.x >> 3) * WPB + sub;   // wave-tile slot within the XCD's range
     const int mpx = (a.m_tiles + 7) >> 3;
     nt = q % a.n_tiles;
     mt = r8 * mpx + q / a.n_tiles;
@@ -496,9 +497,12 @@ int launch_lds_rows(zr_ctx* ctx, GemmArgs& ga, int epi) {
 template <int TM, int TN, int KS, int WPB, int AMODE, bool VEC, int OCC = 1>
 int launch_epi(zr_ctx* ctx, const GemmArgs& ga, int batch, int epi) {
   long long ntiles = (long long)ga.m_tiles * ga.n_tiles;
-  if (AMODE == ZR_A_PACK4 || AMODE == ZR_A_PACK8_BF16)
-    ntiles = (long long)((ga.m_tiles + 7) / 8) * 8 * ga.n_tiles;  // XCD-major id space
   dim3 grid((unsigned)((ntiles + WPB - 1) / WPB), 1, batch);
+  if (AMODE == ZR_A_PACK4 || AMODE == ZR_A_PACK8_BF16) {
+    // XCD-major id space: 8 ranges of ceil(m_tiles/8) row tiles x n_tiles wave tiles, WPB wave tiles per workgroup
+    const long long per_xcd = (long long)((ga.m_tiles + 7) / 8) * ga.n_tiles;
+    grid.x = (unsigned)(((per_xcd + WPB - 1) / WPB) * 8);
+  }
   dim3 block(64 * KS * WPB);
   switch (epi) {
     case ZR_EPI_STORE:
