@@ -1,0 +1,64 @@
+// Test driver: SGD steps of model_trainer (zoph_rnn_amd/host/zoph_model.h) on the minibatches of an integerized file.
+//   train_step [--sequence] model.nn data.int minibatch longest_sent learning_rate norm_clip steps
+// Every step trains on the next minibatch of the file (wrapping around) and prints "loss <step> <log-likelihood>";
+// the updated model is written to <model.nn>.trained as a complete model file.
+#include <cstdio>
+#include <cstdlib>
+#include <iostream>
+#include <string>
+#include <vector>
+
+#include "../../zoph_rnn_amd/host/zoph_model.h"
+
+int main(int argc, char** argv) {
+  bool LM = false;
+  std::vector<std::string> pos;
+  for (int i = 1; i < argc; i++) {
+    if (std::string(argv[i]) == "--sequence")
+      LM = true;
+    else
+      pos.push_back(argv[i]);
+  }
+  if (pos.size() != 7) {
+    std::fprintf(stderr, "usage: %s [--sequence] model.nn data.int minibatch longest_sent learning_rate norm_clip steps\n", argv[0]);
+    return 2;
+  }
+  const int minibatch = std::atoi(pos[2].c_str()), longest = std::atoi(pos[3].c_str()), steps = std::atoi(pos[6].c_str());
+  const float lr = (float)std::atof(pos[4].c_str()), clip = (float)std::atof(pos[5].c_str());
+  std::ifstream model(pos[0]);
+  model_file_info info;
+  std::string err;
+  if (!model || !read_model_file_info(model, LM, info, err)) {
+    std::fprintf(stderr, "%s: %s\n", pos[0].c_str(), err.c_str());
+    return 1;
+  }
+  layer_gpu_info gpu;
+  gpu.init(0);
+  forward_model<precision> m;
+  m.initModel(gpu, info, minibatch, longest, 10);
+  m.load_weights(model);
+  model_trainer<precision> trainer(m);
+  minibatch_reader reader;
+  if (!reader.open(pos[1], minibatch, longest, LM)) {
+    std::fprintf(stderr, "cannot open %s\n", pos[1].c_str());
+    return 1;
+  }
+  std::cout << std::setprecision(15);
+  for (int s = 0; s < steps; s++) {
+    if (!reader.read_minibatch(err)) {
+      if (!err.empty()) {
+        std::fprintf(stderr, "%s\n", err.c_str());
+        return 1;
+      }
+      reader.input_file.clear();
+      reader.input_file.seekg(0, std::ios::beg);
+      if (!reader.read_minibatch(err)) return 1;
+    }
+    const double loss = trainer.train_minibatch(reader, lr, clip);
+    std::cout << "loss " << s << " " << loss << "\n";
+  }
+  devSynchAll(gpu.ctx);
+  std::ofstream out(pos[0] + ".trained");
+  m.dump_weights(out);
+  return 0;
+}

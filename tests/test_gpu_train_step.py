@@ -1,0 +1,209 @@
+"""model_trainer (zoph_rnn_amd/host/zoph_model.h) end to end through tests/host/train_step: SGD steps on minibatches
+of an integerized file, the updated model file compared with the same steps computed by the oracle (forward, loss
+layer backward accumulated over the time steps, stack backward, 1/minibatch scaling, per-matrix norm clipping and
+the ascent update in numpy).  The oracle's backward is pinned by torch autograd in tests/test_oracle_backward_pins.py.
+Tolerance: 1e-4 of the largest weight change of each matrix plus 1e-6 absolute (the file holds 8 significant digits)."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+import model_files_util as mf
+import oracle_lib as o
+from test_gpu_force_decode import _time_major
+from test_gpu_host_layers import _write_hh, _write_ih, _write_matrix
+from zoph_rnn_amd import synth
+
+pytestmark = pytest.mark.gpu
+DRIVER = os.path.join(mf.ROOT, "tests", "host", "train_step")
+
+
+def _write_model(path, m, tgt_vocab, src_vocab, lm):
+    L, H = len(m["tgt_layers"]), m["emb_t"].shape[0]
+    with open(path, "w") as f:
+        mf.write_header(f, L, H, tgt_vocab, src_vocab, False, False, lm=lm)
+        if not lm:
+            _write_ih(f, m["src_layers"][0], m["emb_s"])
+            for ly in m["src_layers"][1:]:
+                _write_hh(f, ly)
+        _write_ih(f, m["tgt_layers"][0], m["emb_t"])
+        for ly in m["tgt_layers"][1:]:
+            _write_hh(f, ly)
+        _write_matrix(f, m["D"])
+        _write_matrix(f, m["b_d"].reshape(-1, 1))
+
+
+def _read_model(path, n_head, L, H, Vs, Vt, lm):
+    """The dumped file back into the dictionary layout of _write_model (same matrix order)."""
+    vals = np.array(" ".join(open(path).read().split("\n")[n_head:]).split(), dtype=np.float64)
+    pos = [0]
+
+    def take(r, c):
+        a = vals[pos[0]:pos[0] + r * c].reshape(r, c)
+        pos[0] += r * c
+        return a
+
+    def layer(V):
+        ly = {"M": [None] * 4, "Wh": [None] * 4, "b": [None] * 4}
+        for g in range(4):
+            ly["Wh"][g] = take(H, H)
+            ly["b"][g] = take(H, 1).reshape(-1)
+        emb = take(H, V) if V else None
+        for g in (0, 1, 3, 2):
+            ly["M"][g] = take(H, H)
+        return ly, emb
+
+    m = {}
+    for side, V in (("src", Vs), ("tgt", Vt)):
+        if side == "src" and lm:
+            continue
+        first, emb = layer(V)
+        m["emb_" + side[0]] = emb
+        m[side + "_layers"] = [first] + [layer(0)[0] for _ in range(L - 1)]
+    m["D"] = take(Vt, H)
+    m["b_d"] = take(Vt, 1).reshape(-1)
+    assert pos[0] == vals.size
+    return m
+
+
+def _clip_update(W, grad, mb, clip, lr, clipped):
+    g = np.asarray(grad, np.float64) / mb
+    norm = np.sqrt((g * g).sum())
+    clipped.append(bool(norm > clip))
+    if norm > clip:
+        g = g * (clip / norm)
+    return (np.asarray(W, np.float64) + lr * g).astype(np.float32)
+
+
+def _oracle_step(m, chunk, mb, lm, lr, clip, clipped):
+    """One training step on the oracle; updates m in place and returns the log-likelihood before the update."""
+    L = len(m["tgt_layers"])
+    if lm:
+        tin, tout = _time_major([c[0] for c in chunk], mb), _time_major([c[1] for c in chunk], mb)
+        h0 = c0 = None
+    else:
+        src, tin, tout = (_time_major([c[k] for c in chunk], mb) for k in (0, 2, 3))
+        S = src.shape[0]
+        nn_s, m_s = o.vocab_prep(src)
+        hs_src, cs_src = o.lstm_stack_forward(m["emb_s"], m["src_layers"], nn_s, m_s)
+        h0 = [np.asfortranarray(hs_src[l, S - 1]) for l in range(L)]
+        c0 = [np.asfortranarray(cs_src[l, S - 1]) for l in range(L)]
+    T = tin.shape[0]
+    nn_t, m_t = o.vocab_prep(tin)
+    hs, _ = o.lstm_stack_forward(m["emb_t"], m["tgt_layers"], nn_t, m_t, h0=h0, c0=c0)
+    tgt, tmask, _ = o.vocab_softmax(tout)
+    Vt, H = m["D"].shape
+    dD, dbd = np.zeros((Vt, H), np.float64, order="F"), np.zeros(Vt, np.float64)
+    err_top, loss = [], 0.0
+    for t in range(T):
+        h = np.asfortranarray(hs[L - 1, t])
+        loss += o.softmax_loss(o.softmax_logprob_f64(o.softmax_logits(m["D"], m["b_d"], h)), tgt[t], tmask[t])
+        e, dD, dbd = o.softmax_backward(m["D"], m["b_d"], h, tgt[t], tmask[t], dD, dbd)
+        err_top.append(e)
+    g_t, dW_t, eh0, ec0 = o.lstm_stack_backward(m["emb_t"], m["tgt_layers"], nn_t, m_t, err_top, h0=h0, c0=c0)
+    sides = [("t", "tgt_layers", g_t, dW_t)]
+    if not lm:
+        zero_top = [np.zeros((H, mb), np.float32) for _ in range(S)]
+        g_s, dW_s, _, _ = o.lstm_stack_backward(m["emb_s"], m["src_layers"], nn_s, m_s, zero_top, err_hT=eh0, err_cT=ec0)
+        sides.append(("s", "src_layers", g_s, dW_s))
+    up = lambda W, g: _clip_update(W, g, mb, clip, lr, clipped)
+    m["D"], m["b_d"] = up(m["D"], dD), up(m["b_d"], dbd)
+    for s, key, grads, dW in sides:
+        m["emb_" + s] = up(m["emb_" + s], dW)
+        for ly, gr in zip(m[key], grads):
+            for k, gk in (("M", "dM"), ("Wh", "dWh"), ("b", "db")):
+                ly[k] = [up(ly[k][g], gr[gk][g]) for g in range(4)]
+    return loss
+
+
+def _compare(name, got, want, orig):
+    d_got, d_want = np.asarray(got, np.float64) - orig, np.asarray(want, np.float64) - orig
+    tol = 1e-4 * np.abs(d_want).max() + 1e-6
+    err = np.abs(d_got - d_want).max()
+    assert err <= tol, "%s: weight change off by %.3g (bound %.3g, largest change %.3g)" % (
+        name, err, tol, np.abs(d_want).max())
+
+
+@pytest.mark.parametrize("lm,L,H,mb,steps,clip", [(True, 2, 32, 4, 1, 0.4), (False, 2, 48, 3, 1, 0.25),
+                                                  (False, 1, 32, 5, 3, 5.0), (True, 3, 64, 8, 2, 1.0)])
+def test_train_steps_match_oracle(tmp_path, lm, L, H, mb, steps, clip):
+    if not os.path.exists(DRIVER):
+        pytest.fail("tests/host/train_step is not built: run `python __graft_entry__.py build`")
+    g = synth.rng(131, L * 100 + H + mb)
+    lr, longest = 0.5, 16
+    src_vocab = ["<UNK>"] + mf.make_vocab(40, "s")
+    tgt_vocab = ["<START>", "<EOF>", "<UNK>"] + mf.make_vocab(50, "t")
+    Vs, Vt = len(src_vocab), len(tgt_vocab)
+    m = {"emb_t": synth.uniform(g, (H, Vt), -0.5, 0.5),
+         "tgt_layers": [synth.lstm_layer(g, H, forget_bias_one=True) for _ in range(L)],
+         "D": synth.uniform(g, (Vt, H), -0.5, 0.5), "b_d": synth.uniform(g, (Vt,), -0.5, 0.5)}
+    if not lm:
+        m["emb_s"] = synth.uniform(g, (H, Vs), -0.5, 0.5)
+        m["src_layers"] = [synth.lstm_layer(g, H, forget_bias_one=True) for _ in range(L)]
+    model = tmp_path / "model.nn"
+    _write_model(model, m, tgt_vocab, src_vocab, lm)
+    n_head = 1 + (2 if lm else 3) + (0 if lm else Vs) + Vt
+    orig = _read_model(model, n_head, L, H, Vs, Vt, lm)
+    n_sent = 2 * mb
+    tgt = mf.random_sentences(g, tgt_vocab, n_sent, 1, 8)
+    data_path = tmp_path / "data.int"
+    if lm:
+        data = mf.integerize_targets(tgt, tgt_vocab, mb)
+        rows = [[[], [], d[0], d[1]] for d in data]
+    else:
+        src = mf.random_sentences(g, src_vocab, n_sent, 2, 9)
+        data = mf.integerize_pairs(src, tgt, src_vocab, tgt_vocab, mb)
+        rows = data
+    with open(data_path, "w") as f:
+        for r in rows:
+            for k in range(4):
+                f.write(" ".join(str(v) for v in r[k]) + "\n")
+    args = (["--sequence"] if lm else []) + [str(model), str(data_path), str(mb), str(longest), str(lr), str(clip),
+                                             str(steps)]
+    r = subprocess.run([DRIVER] + args, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    got_loss = [float(ln.split()[2]) for ln in r.stdout.splitlines() if ln.startswith("loss")]
+    chunks = [data[i:i + mb] for i in range(0, len(data), mb)]
+    clipped, want_loss = [], []
+    for s in range(steps):
+        want_loss.append(_oracle_step(m, chunks[s % len(chunks)], mb, lm, lr, clip, clipped))
+    assert len(got_loss) == steps
+    for a, b in zip(got_loss, want_loss):
+        assert a == pytest.approx(b, rel=1e-4, abs=1e-4)
+    if clip < 5.0:
+        assert any(clipped) and not all(clipped), "pick norm_clip so that both branches of the clipping run"
+    new = _read_model(str(model) + ".trained", n_head, L, H, Vs, Vt, lm)
+    _compare("D", new["D"], m["D"], orig["D"])
+    _compare("b_d", new["b_d"], m["b_d"], orig["b_d"])
+    for s, key in (("t", "tgt_layers"),) + (() if lm else (("s", "src_layers"),)):
+        _compare("embedding " + s, new["emb_" + s], m["emb_" + s], orig["emb_" + s])
+        for l in range(L):
+            for k in ("M", "Wh", "b"):
+                for gate in range(4):
+                    _compare("%s layer %d %s[%d]" % (key, l, k, gate), new[key][l][k][gate], m[key][l][k][gate],
+                             orig[key][l][k][gate])
+
+
+def test_repeated_steps_on_one_minibatch_raise_its_likelihood(tmp_path):
+    """Property check without the oracle: gradient ASCENT on the log-likelihood, so training on the same minibatch
+    again and again must raise it."""
+    g = synth.rng(132, 0)
+    H, L, mb = 64, 2, 6
+    tgt_vocab = ["<START>", "<EOF>", "<UNK>"] + mf.make_vocab(80, "w")
+    Vt = len(tgt_vocab)
+    m = {"emb_t": synth.uniform(g, (H, Vt), -0.1, 0.1),
+         "tgt_layers": [synth.lstm_layer(g, H, forget_bias_one=True) for _ in range(L)],
+         "D": synth.uniform(g, (Vt, H), -0.1, 0.1), "b_d": synth.uniform(g, (Vt,), -0.1, 0.1)}
+    model = tmp_path / "lm.nn"
+    _write_model(model, m, tgt_vocab, [], True)
+    data = mf.integerize_targets(mf.random_sentences(g, tgt_vocab, mb, 3, 9), tgt_vocab, mb)
+    with open(tmp_path / "data.int", "w") as f:
+        for d in data:
+            f.write("\n\n" + " ".join(map(str, d[0])) + "\n" + " ".join(map(str, d[1])) + "\n")
+    r = subprocess.run([DRIVER, "--sequence", str(model), str(tmp_path / "data.int"), str(mb), "16", "0.2", "5", "12"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    loss = [float(ln.split()[2]) for ln in r.stdout.splitlines() if ln.startswith("loss")]
+    assert len(loss) == 12 and all(b > a for a, b in zip(loss, loss[1:])), [round(v, 2) for v in loss]
+    assert loss[-1] > loss[0] + 0.1 * abs(loss[0])

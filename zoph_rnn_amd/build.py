@@ -66,15 +66,18 @@ def build_beam_decode():
 
 
 def build_host_driver():
-    """C++ driver of the host-side layer classes (tests/host/layers_forward), plain g++ against the C-ABI."""
+    """C++ test drivers of the host-side classes (tests/host/layers_forward, tests/host/train_step), plain g++
+    against the C-ABI."""
     root = os.path.dirname(HERE)
-    src = os.path.join(root, "tests", "host", "layers_forward.cpp")
-    out = os.path.join(root, "tests", "host", "layers_forward")
-    cmd = [os.environ.get("CXX", "g++"), "-std=c++17", "-O1", "-Wall", "-o", out, src, "-L", HERE, "-lzoph_rnn_hip",
-           "-Wl,-rpath,$ORIGIN/../../zoph_rnn_amd"]
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError("host driver build failed:\n" + r.stdout + r.stderr)
+    out = None
+    for name in ("train_step", "layers_forward"):
+        src = os.path.join(root, "tests", "host", name + ".cpp")
+        out = os.path.join(root, "tests", "host", name)
+        cmd = [os.environ.get("CXX", "g++"), "-std=c++17", "-O1", "-Wall", "-o", out, src, "-L", HERE,
+               "-lzoph_rnn_hip", "-Wl,-rpath,$ORIGIN/../../zoph_rnn_amd"]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("host driver build failed:\n" + r.stdout + r.stderr)
     return out
 
 

@@ -562,6 +562,190 @@ class forward_model {
   }
 };
 
+// ------------------------------------------------------------------------------------------------ training
+// One SGD step on a minibatch for models without attention (language models and plain encoder-decoder models):
+// neuralMT_model::compute_gradients (src/model.hpp:1823-2000) followed by update_weights (:2002-2040), written
+// against the stack-level training entry points of the library instead of node-by-node back_prop_GPU calls.
+// Gradients are those of the log-likelihood and are ADDED (the reference ascends), scaled by 1/minibatch_size and
+// clipped per matrix to norm_clip in L2 norm (norm_clip_GPU_v2), as the reference does without --global-clip.
+template <typename dType>
+class model_trainer {
+ public:
+  forward_model<dType>& m;
+  zr_ctx* ctx;
+  int H, L, mb, longest, Vs, Vt;
+  bool seq2seq;
+  struct side {
+    std::vector<zr_lstm_train*> train;
+    std::vector<dType*> h_all, c_all, g_all, dg_all, eh0, ec0, dM, dWh, db;
+    dType *below0 = nullptr, *x_all = nullptr, *dW = nullptr;
+    int *d_ids = nullptr, *d_nn = nullptr, *d_mask = nullptr;
+  } src, tgt;
+  dType *zeros = nullptr, *err_top = nullptr, *prob = nullptr, *dD = nullptr, *dbd = nullptr, *unst[4] = {};
+  int *d_tout = nullptr, *d_tmask = nullptr;
+  float* d_tmaskf = nullptr;
+
+  template <typename T>
+  T* dmalloc(size_t n) {
+    T* p = nullptr;
+    ZOPH_CALL(zr_malloc(ctx, n * sizeof(T), (void**)&p));
+    return p;
+  }
+  template <typename LayerT>
+  static void gate_ptrs(LayerT& ly, const dType* M[4], const dType* Wh[4]) {
+    M[0] = ly.d_M_i; M[1] = ly.d_M_f; M[2] = ly.d_M_c; M[3] = ly.d_M_o;
+    Wh[0] = ly.d_W_hi; Wh[1] = ly.d_W_hf; Wh[2] = ly.d_W_hc; Wh[3] = ly.d_W_ho;
+  }
+  void init_side(side& s, Input_To_Hidden_Layer<dType>& in, std::vector<Hidden_To_Hidden_Layer<dType>>& hid, int V) {
+    const size_t n = (size_t)H * mb, nT = n * longest;
+    for (int l = 0; l < L; l++) {
+      const dType *M[4], *Wh[4];
+      if (l == 0) gate_ptrs(in, M, Wh); else gate_ptrs(hid[l - 1], M, Wh);
+      zr_lstm_train* t = nullptr;
+      ZOPH_CALL(zr_lstm_train_create(ctx, M, Wh, H, &t));
+      s.train.push_back(t);
+      s.h_all.push_back(dmalloc<dType>(nT));
+      s.c_all.push_back(dmalloc<dType>(nT));
+      s.g_all.push_back(dmalloc<dType>(4 * nT));
+      s.dg_all.push_back(dmalloc<dType>(4 * nT));
+      s.eh0.push_back(dmalloc<dType>(n));
+      s.ec0.push_back(dmalloc<dType>(n));
+      s.dM.push_back(dmalloc<dType>(4 * (size_t)H * H));
+      s.dWh.push_back(dmalloc<dType>(4 * (size_t)H * H));
+      s.db.push_back(dmalloc<dType>(4 * (size_t)H));
+    }
+    s.below0 = dmalloc<dType>(nT);
+    s.x_all = dmalloc<dType>(nT);
+    s.dW = dmalloc<dType>((size_t)H * V);
+    s.d_ids = dmalloc<int>((size_t)mb * longest);
+    s.d_nn = dmalloc<int>((size_t)mb * longest);
+    s.d_mask = dmalloc<int>((size_t)mb * longest);
+  }
+
+  explicit model_trainer(forward_model<dType>& model) : m(model), ctx(model.gpu.ctx) {
+    if (m.params.attent_params.attention_model) {
+      std::fprintf(stderr, "model_trainer: the backward pass of the attention layer is not built\n");
+      std::exit(EXIT_FAILURE);
+    }
+    H = m.info.LSTM_size;
+    L = m.info.num_layers;
+    mb = m.params.minibatch_size;
+    longest = m.params.longest_sent;
+    Vs = m.info.source_vocab_size;
+    Vt = m.info.target_vocab_size;
+    seq2seq = !m.info.LM;
+    if ((long long)mb * longest > 65535) {
+      std::fprintf(stderr, "model_trainer: minibatch_size * longest_sent must not exceed 65535\n");
+      std::exit(EXIT_FAILURE);
+    }
+    if (seq2seq) init_side(src, m.input_layer_source, m.source_hidden_layers, Vs);
+    init_side(tgt, m.input_layer_target, m.target_hidden_layers, Vt);
+    const size_t n = (size_t)H * mb;
+    zeros = dmalloc<dType>(n);
+    ZOPH_CALL(zr_memset_zero(ctx, zeros, n * sizeof(dType)));
+    err_top = dmalloc<dType>(n * longest);
+    prob = dmalloc<dType>((size_t)Vt * mb * longest);
+    dD = dmalloc<dType>((size_t)Vt * H);
+    dbd = dmalloc<dType>(Vt);
+    for (auto& u : unst) u = dmalloc<dType>((size_t)H * H);
+    d_tout = dmalloc<int>((size_t)mb * longest);
+    d_tmask = dmalloc<int>((size_t)mb * longest);
+    d_tmaskf = dmalloc<float>((size_t)mb * longest);
+  }
+
+  void forward_side(side& s, Input_To_Hidden_Layer<dType>& in, std::vector<Hidden_To_Hidden_Layer<dType>>& hid,
+                    const int* h_ids, int T, int V, const std::vector<const dType*>& h0, const std::vector<const dType*>& c0) {
+    ZOPH_CALL(zr_h2d(ctx, s.d_ids, h_ids, (size_t)T * mb * sizeof(int)));
+    ZOPH_CALL(zr_vocab_prep(ctx, s.d_ids, T * mb, V, s.d_nn, s.d_mask));
+    std::vector<const zr_lstm_weights*> w;
+    if (!in.packed) in.repack();
+    w.push_back(in.packed);
+    for (auto& l : hid) {
+      if (!l.packed) l.repack();
+      w.push_back(l.packed);
+    }
+    ZOPH_CALL(zr_lstm_stack_forward_train(ctx, L, w.data(), in.d_W, V, s.d_nn, s.d_mask, T, mb, h0.data(), c0.data(), 0.0f,
+                                          s.h_all.data(), s.c_all.data(), s.g_all.data()));
+  }
+
+  template <typename LayerT>
+  void update_layer(LayerT& ly, side& s, int l, float scale, float norm_clip, float lr) {
+    const size_t hh = (size_t)H * H;
+    dType* M[4] = {ly.d_M_i, ly.d_M_f, ly.d_M_c, ly.d_M_o};
+    dType* Wh[4] = {ly.d_W_hi, ly.d_W_hf, ly.d_W_hc, ly.d_W_ho};
+    dType* b[4] = {ly.d_b_i, ly.d_b_f, ly.d_b_c, ly.d_b_o};
+    ZOPH_CALL(zr_unstack_gates(ctx, s.dM[l], H, unst));
+    for (int g = 0; g < 4; g++) ZOPH_CALL(zr_sgd_update(ctx, M[g], unst[g], (long long)hh, scale, norm_clip, lr));
+    ZOPH_CALL(zr_unstack_gates(ctx, s.dWh[l], H, unst));
+    for (int g = 0; g < 4; g++) ZOPH_CALL(zr_sgd_update(ctx, Wh[g], unst[g], (long long)hh, scale, norm_clip, lr));
+    for (int g = 0; g < 4; g++) ZOPH_CALL(zr_sgd_update(ctx, b[g], s.db[l] + (size_t)g * H, H, scale, norm_clip, lr));
+    ly.repack();
+    const dType *Mc[4], *Whc[4];
+    gate_ptrs(ly, Mc, Whc);
+    ZOPH_CALL(zr_lstm_train_refresh(ctx, s.train[l], Mc, Whc));
+  }
+
+  void backward_side(side& s, Input_To_Hidden_Layer<dType>& in, std::vector<Hidden_To_Hidden_Layer<dType>>& hid, int T,
+                     int V, const std::vector<const dType*>& h0, const std::vector<const dType*>& c0, const dType* top,
+                     const std::vector<const dType*>* ehT, const std::vector<const dType*>* ecT) {
+    std::vector<const dType*> c_all(s.c_all.begin(), s.c_all.end()), g_all(s.g_all.begin(), s.g_all.end());
+    ZOPH_CALL(zr_lstm_stack_backward(ctx, L, s.train.data(), T, mb, s.d_mask, c0.data(), c_all.data(), g_all.data(), top,
+                                     ehT ? ehT->data() : nullptr, ecT ? ecT->data() : nullptr, s.dg_all.data(),
+                                     s.below0, s.eh0.data(), s.ec0.data()));
+    ZOPH_CALL(zr_embed_gather(ctx, in.d_W, H, V, s.d_nn, T * mb, s.x_all));
+    for (int l = 0; l < L; l++)
+      ZOPH_CALL(zr_lstm_weight_gradients(ctx, H, T, mb, s.dg_all[l], l == 0 ? s.x_all : s.h_all[l - 1], h0[l],
+                                         s.h_all[l], s.dM[l], s.dWh[l], s.db[l]));
+    ZOPH_CALL(zr_memset_zero(ctx, s.dW, (size_t)H * V * sizeof(dType)));
+    ZOPH_CALL(zr_embed_gradient(ctx, H, V, s.below0, s.d_nn, s.d_mask, T * mb, s.dW));
+  }
+
+  // Forward, backward and update on the minibatch the reader holds.  Returns the minibatch's log-likelihood (natural
+  // log) under the weights BEFORE the update.
+  double train_minibatch(minibatch_reader& r, float learning_rate, float norm_clip) {
+    const int S = seq2seq ? r.current_source_length : 0, T = r.current_target_length;
+    const size_t n = (size_t)H * mb;
+    std::vector<const dType*> z(L, zeros);
+    std::vector<const dType*> th0 = z, tc0 = z;
+    if (seq2seq) {
+      forward_side(src, m.input_layer_source, m.source_hidden_layers, r.h_input_vocab_indicies_source.data(), S, Vs, z, z);
+      for (int l = 0; l < L; l++) {  // the decoder starts from the encoder's last state (src/model.hpp:1714-1724)
+        th0[l] = src.h_all[l] + (size_t)(S - 1) * n;
+        tc0[l] = src.c_all[l] + (size_t)(S - 1) * n;
+      }
+    }
+    forward_side(tgt, m.input_layer_target, m.target_hidden_layers, r.h_input_vocab_indicies_target.data(), T, Vt, th0, tc0);
+    // loss layer over all T * mb columns at once
+    ZOPH_CALL(zr_h2d(ctx, d_tout, r.h_output_vocab_indicies_target.data(), (size_t)T * mb * sizeof(int)));
+    ZOPH_CALL(zr_vocab_prep_softmax(ctx, d_tout, T * mb, Vt, d_tmask, d_tmaskf));
+    auto& sm = m.softmax_obj;
+    double loss = 0;
+    ZOPH_CALL(zr_softmax_loss(ctx, sm.d_D, sm.d_b_d, Vt, H, tgt.h_all[L - 1], T * mb, d_tout, d_tmask, prob, &loss));
+    ZOPH_CALL(zr_softmax_backward(ctx, sm.d_D, sm.d_b_d, Vt, H, tgt.h_all[L - 1], T * mb, d_tout, d_tmask, prob, err_top,
+                                  dD, dbd));
+    backward_side(tgt, m.input_layer_target, m.target_hidden_layers, T, Vt, th0, tc0, err_top, nullptr, nullptr);
+    if (seq2seq) {
+      // no attention: the encoder receives error only through its final states
+      ZOPH_CALL(zr_memset_zero(ctx, err_top, (size_t)S * n * sizeof(dType)));
+      std::vector<const dType*> ehT(tgt.eh0.begin(), tgt.eh0.end()), ecT(tgt.ec0.begin(), tgt.ec0.end());
+      backward_side(src, m.input_layer_source, m.source_hidden_layers, S, Vs, z, z, err_top, &ehT, &ecT);
+    }
+    // update_weights
+    const float scale = 1.0f / (float)mb;
+    ZOPH_CALL(zr_sgd_update(ctx, sm.d_D, dD, (long long)Vt * H, scale, norm_clip, learning_rate));
+    ZOPH_CALL(zr_sgd_update(ctx, sm.d_b_d, dbd, Vt, scale, norm_clip, learning_rate));
+    sm.prepare_weights();
+    auto update_side = [&](side& s, Input_To_Hidden_Layer<dType>& in, std::vector<Hidden_To_Hidden_Layer<dType>>& hid, int V) {
+      ZOPH_CALL(zr_sgd_update(ctx, in.d_W, s.dW, (long long)H * V, scale, norm_clip, learning_rate));
+      update_layer(in, s, 0, scale, norm_clip, learning_rate);
+      for (int l = 1; l < L; l++) update_layer(hid[l - 1], s, l, scale, norm_clip, learning_rate);
+    };
+    update_side(tgt, m.input_layer_target, m.target_hidden_layers, Vt);
+    if (seq2seq) update_side(src, m.input_layer_source, m.source_hidden_layers, Vs);
+    return loss;
+  }
+};
+
 // ------------------------------------------------------------------------------------------------ beam decoding
 // Batched beam-search decode on top of a loaded forward_model: what ensemble_factory::decode_file_batch
 // (src/ensemble_factory.hpp:583-765) does with decoder_model_wrapper::forward_prop_source / forward_prop_target /
