@@ -288,6 +288,25 @@ int zr_lstm_weight_gradients(zr_ctx* ctx, int H, int T, int mb, const float* d_d
                              const float* d_h0, const float* d_h_all, float* d_dM_stack, float* d_dWh_stack,
                              float* d_db);
 
+/* One node of the same computation, for callers that drive the (layer, time) grid themselves as the reference's
+ * layer classes do: the error part of LSTM_IH_Node::back_prop_GPU / LSTM_HH_Node::back_prop_GPU
+ * (src/LSTM.hpp:542-960, src/LSTM_HH.hpp:452-700).
+ *   d_gates: the node's saved i, f, c~, o (H x mb each); d_c, d_c_prev: c_t, c_{t-1}.
+ *   d_err_above: error at h_t from the layer above or the loss layer (d_d_ERRt_ht; NULL = none);
+ *   d_err_h_next / d_err_c_next: errors arriving from step t+1 (d_d_ERRnTOtp1_ht / _ct; NULL = none).
+ *   Outputs: d_dgates 4H x mb (rows g*H + j; the reference's d_d_ERRnTOt_it, _ft, _tanhcpt, _ot stacked),
+ *   d_err_h_prev, d_err_c_prev (d_d_ERRnTOt_htM1 / _ctM1; d_err_c_prev may alias d_err_c_next),
+ *   d_err_below (d_d_ERRnTOt_h_Below; NULL = not wanted; fastest when it is d_err_h_prev + H*mb). */
+int zr_lstm_node_backward(zr_ctx* ctx, const zr_lstm_train* layer, int mb, const float* const d_gates[4],
+                          const float* d_c, const float* d_c_prev, const int* d_mask01, const float* d_err_above,
+                          const float* d_err_h_next, const float* d_err_c_next, float* d_dgates, float* d_err_h_prev,
+                          float* d_err_c_prev, float* d_err_below);
+/* compute_gradients_GPU of one node (src/LSTM.hpp:963-1270, src/LSTM_HH.hpp:700-900): the rank-mb updates
+ * dM += dgates in^T, dWh += dgates h_{t-1}^T, db += row sums, ACCUMULATED into the stacked 4H x H / 4H gradients
+ * (zero them at the start of a minibatch).  d_in: the node's input (embedding columns or the h_t below), H x mb. */
+int zr_lstm_node_gradients(zr_ctx* ctx, int H, int mb, const float* d_dgates, const float* d_in, const float* d_h_prev,
+                           float* d_dM_stack, float* d_dWh_stack, float* d_db);
+
 /* Embedding gradient (the sparse W gradient kernels, src/custom_kernels.h:1297-1390): d_dW[:, id[k]] += d_err[:, k]
  * for the n unmasked positions; d_dW is H x V and is accumulated into (zero it first).  Uses float atomics, like
  * the reference: the summation order within a column is not fixed. */
@@ -302,6 +321,11 @@ int zr_embed_gradient(zr_ctx* ctx, int H, int V, const float* d_err, const int* 
 int zr_softmax_backward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int n,
                         const int* d_target, const int* d_mask01, float* d_prob_scratch, float* d_err_h, float* d_dD,
                         float* d_db);
+/* The same with d_dD and d_db ADDED to: one call per time step (softmax_layer::back_prop1 / back_prop2,
+ * src/softmax.hpp:600-700), gradients zeroed at the start of the minibatch. */
+int zr_softmax_backward_accumulate(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h,
+                                   int n, const int* d_target, const int* d_mask01, float* d_prob_scratch,
+                                   float* d_err_h, float* d_dD, float* d_db);
 
 /* update_weights (src/softmax.hpp:232-300, src/Hidden_To_Hidden_Layer.hpp update_weights_GPU): the gradient is
  * scaled (the reference divides by the minibatch size), clipped to norm_clip in L2 norm if norm_clip > 0

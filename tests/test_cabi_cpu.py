@@ -57,6 +57,11 @@ def test_null_context_and_bad_arguments_return_errors():
     assert lib.zr_embed_gradient(None, 8, 8, None, None, None, 1, None) == -1
     assert lib.zr_softmax_backward(None, None, None, 8, 8, None, 1, None, None, None, None, None, None) == -1
     assert lib.zr_sgd_update(None, None, None, C.c_longlong(4), C.c_float(1), C.c_float(0), C.c_float(0.1)) == -1
+    assert lib.zr_lstm_node_backward(None, None, 1, None, None, None, None, None, None, None, None, None, None,
+                                     None) == -1
+    assert lib.zr_lstm_node_gradients(None, 8, 1, None, None, None, None, None, None) == -1
+    assert lib.zr_softmax_backward_accumulate(None, None, None, 8, 8, None, 1, None, None, None, None, None,
+                                              None) == -1
 
 
 def test_context_creation_without_gpu_fails_cleanly():

@@ -203,3 +203,115 @@ def test_language_model_training_step_gradients(ctx):
     assert_close(d_dW.get(), want_e, floor=0.05, what="embedding gradient")
     for ly in layers:
         ly.close()
+
+
+@pytest.mark.parametrize("L,H,mb,T,V,adjacent", [(2, 48, 9, 5, 60, True), (3, 64, 40, 4, 80, False)])
+def test_node_by_node_backward_matches_oracle(ctx, L, H, mb, T, V, adjacent):
+    """The reference's own schedule through the node-level entry points: per node the error step
+    (zr_lstm_node_backward), then its gradient accumulation (zr_lstm_node_gradients), newest step first and top layer
+    first.  adjacent: the two error outputs share one buffer (the single batched product) or not (scratch + copies)."""
+    g = synth.rng(114, L * 100 + mb)
+    embed = U(g, (H, V), -0.5, 0.5)
+    layers_np = [synth.lstm_layer(g, H) for _ in range(L)]
+    for ly in layers_np:
+        ly["M"] = [U(g, (H, H), -0.2, 0.2) for _ in range(4)]
+        ly["Wh"] = [U(g, (H, H), -0.2, 0.2) for _ in range(4)]
+    ids = g.integers(0, V, size=(T, mb)).astype(np.int32)
+    ids[:2, 1] = -1
+    ids[T - 1:, 2] = -1
+    nn, mask = o.vocab_prep(ids)
+    h0 = [U(g, (H, mb), -0.5, 0.5) for _ in range(L)]
+    c0 = [U(g, (H, mb), -0.5, 0.5) for _ in range(L)]
+    err_top = [U(g, (H, mb), -1, 1) for _ in range(T)]
+    want_g, want_e, want_eh0, want_ec0 = o.lstm_stack_backward(embed, layers_np, nn, mask, err_top, h0, c0)
+    n = H * mb
+    layers = [TrainLayer(ctx, ly) for ly in layers_np]
+    d_embed = ctx.array(embed)
+    d_nn, d_m = ctx.empty(ids.size, np.int32), ctx.empty(ids.size, np.int32)
+    ctx.vocab_prep(ctx.array(ids.reshape(-1)), ids.size, V, d_nn, d_m)
+    d_h0, d_c0 = [ctx.array(a) for a in h0], [ctx.array(a) for a in c0]
+    h_all = [ctx.empty((n * T,)) for _ in range(L)]
+    c_all = [ctx.empty((n * T,)) for _ in range(L)]
+    g_all = [ctx.empty((4 * n * T,)) for _ in range(L)]
+    ctx.lstm_stack_forward_train([ly.w for ly in layers], d_embed, V, d_nn, d_m, T, mb, d_h0, d_c0, h_all, c_all, g_all)
+    x_all = ctx.empty((n * T,))
+    ctx.embed_gather(d_embed, H, V, d_nn, T * mb, x_all)
+    d_top = [ctx.array(e) for e in err_top]
+    f4 = np.dtype(np.float32).itemsize
+    dM = [ctx.zeros((4 * H, H)) for _ in range(L)]
+    dWh = [ctx.zeros((4 * H, H)) for _ in range(L)]
+    db = [ctx.zeros((4 * H,)) for _ in range(L)]
+    d_dW = ctx.zeros((H, V))
+    dg = ctx.empty((4 * H, mb))
+    if adjacent:
+        pair = [ctx.zeros((2 * n,)) for _ in range(L)]  # (error to h_{t-1}, error to below) per layer
+        eh = [p.ptr for p in pair]
+        below = [p.ptr + n * f4 for p in pair]
+    else:
+        eh_a, below_a = [ctx.zeros((n,)) for _ in range(L)], [ctx.zeros((n,)) for _ in range(L)]
+        eh, below = [a.ptr for a in eh_a], [a.ptr for a in below_a]
+    ec = [ctx.zeros((n,)) for _ in range(L)]
+    for t in range(T - 1, -1, -1):
+        for l in range(L - 1, -1, -1):
+            gt = g_all[l].ptr + t * 4 * n * f4
+            gates = [gt + k * n * f4 for k in range(4)]
+            c_t = c_all[l].ptr + t * n * f4
+            c_prev = d_c0[l].ptr if t == 0 else c_all[l].ptr + (t - 1) * n * f4
+            h_prev = d_h0[l].ptr if t == 0 else h_all[l].ptr + (t - 1) * n * f4
+            above = d_top[t].ptr if l == L - 1 else below[l + 1]
+            last = t == T - 1
+            ctx.lstm_node_backward(layers[l].t, mb, gates, c_t, c_prev, d_m.ptr + t * mb * 4, above,
+                                   None if last else eh[l], None if last else ec[l], dg, eh[l], ec[l], below[l])
+            d_in = x_all.ptr + t * n * f4 if l == 0 else h_all[l - 1].ptr + t * n * f4
+            ctx.lstm_node_gradients(H, mb, dg, d_in, h_prev, dM[l], dWh[l], db[l])
+            if l == 0:
+                ctx.embed_gradient(H, V, below[0], d_nn.ptr + t * mb * 4, d_m.ptr + t * mb * 4, mb, d_dW)
+    ctx.sync()
+    wfloor = 0.05 * np.sqrt(T * mb)
+    got = lambda p: ctx_get(ctx, p, (H, mb))
+    for l in range(L):
+        assert_close(got(eh[l]), want_eh0[l], what="err_h0 layer %d" % l)
+        assert_close(ec[l].get().reshape(H, mb, order="F"), want_ec0[l], what="err_c0 layer %d" % l)
+        gM, gWh, gb = _unstack(ctx, dM[l], H), _unstack(ctx, dWh[l], H), db[l].get().reshape(4, H)
+        for q in range(4):
+            assert_close(gM[q], want_g[l]["dM"][q], floor=wfloor, what="dM layer %d gate %d" % (l, q))
+            assert_close(gWh[q], want_g[l]["dWh"][q], floor=wfloor, what="dWh layer %d gate %d" % (l, q))
+            assert_close(gb[q], want_g[l]["db"][q], floor=wfloor, what="db layer %d gate %d" % (l, q))
+    assert_close(d_dW.get(), want_e, floor=0.05 * np.sqrt(T), what="embedding gradient")
+    for ly in layers:
+        ly.close()
+
+
+def ctx_get(ctx, ptr, shape):
+    """Device memory at a raw address as a column-major host array."""
+    import ctypes
+    flat = np.empty(int(np.prod(shape)), np.float32)
+    rc = capi.load().zr_d2h(ctx.h, flat.ctypes.data_as(ctypes.c_void_p), ctypes.c_void_p(int(ptr)),
+                            ctypes.c_size_t(flat.nbytes))
+    assert rc == 0
+    return flat.reshape(shape, order="F")
+
+
+@pytest.mark.parametrize("V,H,mb,T", [(301, 32, 7, 4), (2000, 64, 48, 3)])
+def test_softmax_backward_step_by_step_accumulates(ctx, V, H, mb, T):
+    """One zr_softmax_backward_accumulate call per time step adds up to the all-columns call and to the oracle."""
+    g = synth.rng(115, V)
+    D, bd = U(g, (V, H), -0.5, 0.5), U(g, (V,), -1, 1)
+    hs = [U(g, (H, mb), -1, 1) for _ in range(T)]
+    tg = [g.integers(0, V, size=mb).astype(np.int32) for _ in range(T)]
+    mk = [(g.random(mb) > 0.2).astype(np.int32) for _ in range(T)]
+    dD, db = np.zeros((V, H), np.float64, order="F"), np.zeros(V, np.float64)
+    want_e = []
+    for t in range(T):
+        e, dD, db = o.softmax_backward(D, bd, hs[t], tg[t], mk[t], dD, db)
+        want_e.append(e)
+    d_D, d_b = ctx.array(D), ctx.array(bd)
+    d_dD, d_db, d_scr = ctx.zeros((V, H)), ctx.zeros((V,)), ctx.empty((V, mb))
+    for t in range(T):
+        d_e = ctx.empty((H, mb))
+        ctx.softmax_backward(d_D, d_b, V, H, ctx.array(hs[t]), mb, ctx.array(tg[t]), ctx.array(mk[t]), d_scr, d_e, d_dD,
+                             d_db, accumulate=True)
+        ctx.sync()
+        assert_close(d_e.get(), want_e[t], what="err_h step %d" % t)
+    assert_close(d_dD.get(), dD, floor=0.05 * np.sqrt(T * mb), what="dD")
+    assert_close(d_db.get(), db, floor=0.05 * np.sqrt(T * mb), what="db")

@@ -32,7 +32,8 @@ SYMBOLS = [
     "zr_beam_hypotheses", "zr_beam_state",
     "zr_lstm_stack_forward_train", "zr_lstm_train_create", "zr_lstm_train_refresh", "zr_lstm_train_destroy",
     "zr_unstack_gates", "zr_lstm_stack_backward", "zr_lstm_weight_gradients", "zr_embed_gradient",
-    "zr_softmax_backward", "zr_sgd_update",
+    "zr_softmax_backward", "zr_sgd_update", "zr_lstm_node_backward", "zr_lstm_node_gradients",
+    "zr_softmax_backward_accumulate",
 ]
 
 _lib = None
@@ -244,12 +245,24 @@ class Context:
         _chk(load().zr_lstm_weight_gradients(self.h, C.c_int(H), C.c_int(T), C.c_int(mb), _vp(d_dgates), _vp(d_in_all),
                                              _vp(d_h0), _vp(d_h_all), _vp(d_dM), _vp(d_dWh), _vp(d_db)))
 
+    def lstm_node_backward(self, layer, mb, gates, d_c, d_c_prev, d_mask, d_err_above, d_err_h_next, d_err_c_next,
+                           d_dgates, d_err_h_prev, d_err_c_prev, d_err_below=None):
+        _chk(load().zr_lstm_node_backward(self.h, layer, C.c_int(mb), _ptr_array(gates), _vp(d_c), _vp(d_c_prev),
+                                          _vp(d_mask), _vp(d_err_above), _vp(d_err_h_next), _vp(d_err_c_next),
+                                          _vp(d_dgates), _vp(d_err_h_prev), _vp(d_err_c_prev), _vp(d_err_below)))
+
+    def lstm_node_gradients(self, H, mb, d_dgates, d_in, d_h_prev, d_dM, d_dWh, d_db):
+        _chk(load().zr_lstm_node_gradients(self.h, C.c_int(H), C.c_int(mb), _vp(d_dgates), _vp(d_in), _vp(d_h_prev),
+                                           _vp(d_dM), _vp(d_dWh), _vp(d_db)))
+
     def embed_gradient(self, H, V, d_err, d_ids, d_mask, n, d_dW):
         _chk(load().zr_embed_gradient(self.h, C.c_int(H), C.c_int(V), _vp(d_err), _vp(d_ids), _vp(d_mask), C.c_int(n),
                                       _vp(d_dW)))
 
-    def softmax_backward(self, d_D, d_b, V, H, d_h, n, d_target, d_mask, d_scratch, d_err_h, d_dD, d_db):
-        _chk(load().zr_softmax_backward(self.h, _vp(d_D), _vp(d_b), C.c_int(V), C.c_int(H), _vp(d_h), C.c_int(n),
+    def softmax_backward(self, d_D, d_b, V, H, d_h, n, d_target, d_mask, d_scratch, d_err_h, d_dD, d_db,
+                         accumulate=False):
+        fn = load().zr_softmax_backward_accumulate if accumulate else load().zr_softmax_backward
+        _chk(fn(self.h, _vp(d_D), _vp(d_b), C.c_int(V), C.c_int(H), _vp(d_h), C.c_int(n),
                                         _vp(d_target), _vp(d_mask), _vp(d_scratch), _vp(d_err_h), _vp(d_dD), _vp(d_db)))
 
     def sgd_update(self, d_W, d_grad, n, scale, norm_clip, lr):

@@ -60,23 +60,24 @@ __global__ void __launch_bounds__(256) unstack_gates_kernel(const float* __restr
 }
 
 // One node: total error at h_t (from above + from t+1), cell error, the four pre-activation errors, error to c_{t-1}.
-//   gates: [4][H*mb] (i, f, c~, o) of the node; dg: the node's 4H x mb block of the layer's error matrix
+//   g_i, g_f, g_c, g_o: the node's saved gate activations (H x mb each); dg: the node's 4H x mb block of the layer's error matrix
 //   (element (g*H + j, b) at dg[b*4H + g*H + j]); ec: in = error arriving at c_t from t+1 (or null at the last step),
 //   out = error for c_{t-1} (may alias).
 __global__ void __launch_bounds__(256) lstm_node_backward_kernel(
-    const float* __restrict__ gates, const float* __restrict__ c, const float* __restrict__ cprev,
+    const float* __restrict__ g_i, const float* __restrict__ g_f, const float* __restrict__ g_c,
+    const float* __restrict__ g_o, const float* __restrict__ c, const float* __restrict__ cprev,
     const int* __restrict__ mask01, const float* __restrict__ err_above, const float* __restrict__ err_next,
     const float* ec_in, float* ec_out, int H, int mb, float* __restrict__ dg) {
   const int b = blockIdx.y;
   const int j = blockIdx.x * 256 + threadIdx.x;
   if (j >= H) return;
-  const size_t n = (size_t)H * mb, ix = (size_t)b * H + j;
+  const size_t ix = (size_t)b * H + j;
   const float m = (float)mask01[b];
   float eh = 0.0f;
   if (err_above) eh += err_above[ix];
   if (err_next) eh += err_next[ix];
   eh *= m;
-  const float gi = gates[ix], gf = gates[n + ix], gc = gates[2 * n + ix], go = gates[3 * n + ix];
+  const float gi = g_i[ix], gf = g_f[ix], gc = g_c[ix], go = g_o[ix];
   const float th = tanhf(c[ix]);
   const float errt_ct = eh * go * (1.0f - th * th);
   const float ec = ((ec_in ? ec_in[ix] : 0.0f) + errt_ct) * m;
@@ -119,12 +120,12 @@ __global__ void __launch_bounds__(64) row_sum_partial_kernel(const float* __rest
   partial[(size_t)blockIdx.y * rows + r] = s;
 }
 __global__ void __launch_bounds__(64) row_sum_final_kernel(const float* __restrict__ partial, int rows, int chunks,
-                                                           float* __restrict__ out) {
+                                                           float* __restrict__ out, int accumulate) {
   const int r = blockIdx.x * 64 + threadIdx.x;
   if (r >= rows) return;
   float s = 0.0f;
   for (int c = 0; c < chunks; ++c) s += partial[(size_t)c * rows + r];
-  out[r] = s;
+  out[r] = accumulate ? out[r] + s : s;
 }
 
 // Embedding gradient: column id[k] of dW += err column k for every unmasked position.  Float atomics: the order of
@@ -191,7 +192,7 @@ __global__ void __launch_bounds__(256) sgd_apply_kernel(float* __restrict__ W, c
   for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) W[i] += f * g[i];
 }
 
-int row_sum_launch(zr_ctx* ctx, const float* a, int rows, long long n, float* out) {
+int row_sum_launch(zr_ctx* ctx, const float* a, int rows, long long n, float* out, int accumulate = 0) {
   const long long chunk = 64;
   const int chunks = (int)((n + chunk - 1) / chunk);
   void* scratch = nullptr;
@@ -200,7 +201,8 @@ int row_sum_launch(zr_ctx* ctx, const float* a, int rows, long long n, float* ou
   dim3 grid((rows + 63) / 64, chunks);
   row_sum_partial_kernel<<<grid, 64, 0, ctx->stream>>>(a, rows, n, chunk, (float*)scratch);
   ZR_LAUNCH_CHECK("row_sum_partial_kernel");
-  row_sum_final_kernel<<<(rows + 63) / 64, 64, 0, ctx->stream>>>((const float*)scratch, rows, chunks, out);
+  row_sum_final_kernel<<<(rows + 63) / 64, 64, 0, ctx->stream>>>((const float*)scratch, rows, chunks, out,
+                                                                           accumulate);
   ZR_LAUNCH_CHECK("row_sum_final_kernel");
   return ZR_OK;
 }
@@ -316,7 +318,8 @@ int zr_lstm_stack_backward(zr_ctx* ctx, int nl, const zr_lstm_train* const layer
       const float* above = (l == nl - 1) ? d_err_top + (size_t)t * n : work + (size_t)(l + 1) * 2 * n + n;
       float* dg = d_dgates_all[l] + (size_t)t * 4 * n;
       const float* cprev = (t == 0) ? d_c0[l] : d_c_all[l] + (size_t)(t - 1) * n;
-      lstm_node_backward_kernel<<<egrid, 256, 0, ctx->stream>>>(d_gates_all[l] + (size_t)t * 4 * n,
+      const float* gt = d_gates_all[l] + (size_t)t * 4 * n;
+      lstm_node_backward_kernel<<<egrid, 256, 0, ctx->stream>>>(gt, gt + n, gt + 2 * n, gt + 3 * n,
                                                                 d_c_all[l] + (size_t)t * n, cprev,
                                                                 d_mask01 + (size_t)t * mb, above, w_l, d_err_c0[l],
                                                                 d_err_c0[l], H, mb, dg);
@@ -349,13 +352,13 @@ int zr_lstm_stack_backward(zr_ctx* ctx, int nl, const zr_lstm_train* const layer
   return ZR_OK;
 }
 
-int zr_lstm_weight_gradients(zr_ctx* ctx, int H, int T, int mb, const float* d_dgates, const float* d_in_all,
-                             const float* d_h0, const float* d_h_all, float* d_dM_stack, float* d_dWh_stack,
-                             float* d_db) {
+static int weight_gradients(zr_ctx* ctx, int H, int T, int mb, const float* d_dgates, const float* d_in_all,
+                            const float* d_h0, const float* d_h_all, float* d_dM_stack, float* d_dWh_stack,
+                            float* d_db, int accumulate) {
   int rc = zr_bind_device(ctx);
   if (rc) return rc;
   ZR_CHECK_ARG(H > 0 && T > 0 && mb > 0, "zr_lstm_weight_gradients: H = %d, T = %d, mb = %d", H, T, mb);
-  ZR_CHECK_ARG(d_dgates && d_in_all && d_h0 && d_h_all && d_dM_stack && d_dWh_stack && d_db,
+  ZR_CHECK_ARG(d_dgates && d_in_all && d_h0 && (d_h_all || T == 1) && d_dM_stack && d_dWh_stack && d_db,
                "zr_lstm_weight_gradients: null pointer");
   const long long K = (long long)T * mb;
   ZR_CHECK_ARG(K < (1LL << 31) / 4, "zr_lstm_weight_gradients: T * mb = %lld too large", K);
@@ -375,6 +378,7 @@ int zr_lstm_weight_gradients(zr_ctx* ctx, int H, int T, int mb, const float* d_d
   g.ldc = 4 * H;
   g.batch = 1;
   g.epilogue = ZR_EPI_STORE;
+  g.accumulate = accumulate;
   // dM = dgates * in^T
   rc = transpose_launch(ctx, d_in_all, H, (int)K, xt, K, 0);
   if (rc) return rc;
@@ -391,7 +395,70 @@ int zr_lstm_weight_gradients(zr_ctx* ctx, int H, int T, int mb, const float* d_d
   g.C = d_dWh_stack;
   rc = zr_gemm_launch(ctx, g);
   if (rc) return rc;
-  return row_sum_launch(ctx, d_dgates, 4 * H, K, d_db);
+  return row_sum_launch(ctx, d_dgates, 4 * H, K, d_db, accumulate);
+}
+
+int zr_lstm_weight_gradients(zr_ctx* ctx, int H, int T, int mb, const float* d_dgates, const float* d_in_all,
+                             const float* d_h0, const float* d_h_all, float* d_dM_stack, float* d_dWh_stack,
+                             float* d_db) {
+  return weight_gradients(ctx, H, T, mb, d_dgates, d_in_all, d_h0, d_h_all, d_dM_stack, d_dWh_stack, d_db, 0);
+}
+
+int zr_lstm_node_gradients(zr_ctx* ctx, int H, int mb, const float* d_dgates, const float* d_in, const float* d_h_prev,
+                           float* d_dM_stack, float* d_dWh_stack, float* d_db) {
+  return weight_gradients(ctx, H, 1, mb, d_dgates, d_in, d_h_prev, nullptr, d_dM_stack, d_dWh_stack, d_db, 1);
+}
+
+int zr_lstm_node_backward(zr_ctx* ctx, const zr_lstm_train* layer, int mb, const float* const d_gates[4],
+                          const float* d_c, const float* d_c_prev, const int* d_mask01, const float* d_err_above,
+                          const float* d_err_h_next, const float* d_err_c_next, float* d_dgates, float* d_err_h_prev,
+                          float* d_err_c_prev, float* d_err_below) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(layer && mb > 0 && mb <= 65535, "zr_lstm_node_backward: null layer or mb = %d", mb);
+  ZR_CHECK_ARG(d_gates && d_gates[0] && d_gates[1] && d_gates[2] && d_gates[3] && d_c && d_c_prev && d_mask01 &&
+                   d_dgates && d_err_h_prev && d_err_c_prev,
+               "zr_lstm_node_backward: null pointer");
+  const int H = layer->H;
+  const size_t n = (size_t)H * mb;
+  dim3 egrid((H + 255) / 256, mb);
+  lstm_node_backward_kernel<<<egrid, 256, 0, ctx->stream>>>(d_gates[0], d_gates[1], d_gates[2], d_gates[3], d_c,
+                                                            d_c_prev, d_mask01, d_err_above, d_err_h_next,
+                                                            d_err_c_next, d_err_c_prev, H, mb, d_dgates);
+  ZR_LAUNCH_CHECK("lstm_node_backward_kernel");
+  // the two error products share their right-hand side: one batched launch when the outputs are adjacent
+  // (d_err_below == d_err_h_prev + H*mb), else through a scratch pair and two copies
+  float* out = d_err_h_prev;
+  const bool adjacent = d_err_below == d_err_h_prev + n;
+  if (!adjacent) {
+    void* scratch = nullptr;
+    rc = zr_ctx_scratch(ctx, 1, sizeof(float) * 2 * n, &scratch);
+    if (rc) return rc;
+    out = (float*)scratch;
+  }
+  ZrGemmDesc g = {};
+  g.M = H;
+  g.N = mb;
+  g.nseg = 1;
+  g.K[0] = 4 * H;
+  g.A[0] = layer->d_stack;
+  g.lda[0] = H;
+  g.B[0] = d_dgates;
+  g.ldb[0] = 4 * H;
+  g.C = out;
+  g.ldc = H;
+  g.batch = d_err_below ? 2 : 1;
+  g.strideA = 4LL * H * H;
+  g.strideC = (long long)n;
+  g.epilogue = ZR_EPI_STORE;
+  rc = zr_gemm_launch(ctx, g);
+  if (rc) return rc;
+  if (!adjacent) {
+    ZR_HIP(hipMemcpyAsync(d_err_h_prev, out, sizeof(float) * n, hipMemcpyDeviceToDevice, ctx->stream));
+    if (d_err_below)
+      ZR_HIP(hipMemcpyAsync(d_err_below, out + n, sizeof(float) * n, hipMemcpyDeviceToDevice, ctx->stream));
+  }
+  return ZR_OK;
 }
 
 int zr_embed_gradient(zr_ctx* ctx, int H, int V, const float* d_err, const int* d_ids_nonneg, const int* d_mask01,
@@ -411,9 +478,9 @@ int zr_embed_gradient(zr_ctx* ctx, int H, int V, const float* d_err, const int* 
   return ZR_OK;
 }
 
-int zr_softmax_backward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int n,
-                        const int* d_target, const int* d_mask01, float* d_prob_scratch, float* d_err_h, float* d_dD,
-                        float* d_db) {
+static int softmax_backward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int n,
+                            const int* d_target, const int* d_mask01, float* d_prob_scratch, float* d_err_h,
+                            float* d_dD, float* d_db, int accumulate) {
   int rc = zr_bind_device(ctx);
   if (rc) return rc;
   ZR_CHECK_ARG(V > 0 && H > 0 && n > 0 && n <= 65535, "zr_softmax_backward: V = %d, H = %d, n = %d", V, H, n);
@@ -433,25 +500,39 @@ int zr_softmax_backward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V
   if (rc) return rc;
   float* et = (float*)s1;   // n x V
   float* ct = (float*)s0;   // n x H
-  rc = transpose_launch(ctx, d_prob_scratch, V, n, et, n, 0);
-  if (rc) return rc;
   ZrGemmDesc g = {};
-  g.M = n;
-  g.N = H;
   g.nseg = 1;
   g.K[0] = V;
-  g.A[0] = et;
-  g.lda[0] = n;
-  g.B[0] = d_D;
-  g.ldb[0] = V;
-  g.C = ct;
-  g.ldc = n;
   g.batch = 1;
   g.epilogue = ZR_EPI_STORE;
-  rc = zr_gemm_launch(ctx, g);
-  if (rc) return rc;
-  rc = transpose_launch(ctx, ct, n, H, d_err_h, H, 0);
-  if (rc) return rc;
+  if (n >= 1024) {
+    rc = transpose_launch(ctx, d_prob_scratch, V, n, et, n, 0);
+    if (rc) return rc;
+    g.M = n;
+    g.N = H;
+    g.A[0] = et;
+    g.lda[0] = n;
+    g.B[0] = d_D;
+    g.ldb[0] = V;
+    g.C = ct;
+    g.ldc = n;
+    rc = zr_gemm_launch(ctx, g);
+    if (rc) return rc;
+    rc = transpose_launch(ctx, ct, n, H, d_err_h, H, 0);
+    if (rc) return rc;
+  } else {  // few columns (one time step): D^T e directly
+    g.M = H;
+    g.N = n;
+    g.trans_a = 1;
+    g.A[0] = d_D;
+    g.lda[0] = V;
+    g.B[0] = d_prob_scratch;
+    g.ldb[0] = V;
+    g.C = d_err_h;
+    g.ldc = H;
+    rc = zr_gemm_launch(ctx, g);
+    if (rc) return rc;
+  }
   // dD = e h^T : right-hand side h^T as an n x H column-major matrix
   float* ht = (float*)s0;  // the product above has been queued: the buffer is free again in stream order
   rc = transpose_launch(ctx, d_h, H, n, ht, n, 0);
@@ -469,9 +550,22 @@ int zr_softmax_backward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V
   w.ldc = V;
   w.batch = 1;
   w.epilogue = ZR_EPI_STORE;
+  w.accumulate = accumulate;
   rc = zr_gemm_launch(ctx, w);
   if (rc) return rc;
-  return row_sum_launch(ctx, d_prob_scratch, V, n, d_db);
+  return row_sum_launch(ctx, d_prob_scratch, V, n, d_db, accumulate);
+}
+
+int zr_softmax_backward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int n,
+                        const int* d_target, const int* d_mask01, float* d_prob_scratch, float* d_err_h, float* d_dD,
+                        float* d_db) {
+  return softmax_backward(ctx, d_D, d_b_d, V, H, d_h, n, d_target, d_mask01, d_prob_scratch, d_err_h, d_dD, d_db, 0);
+}
+
+int zr_softmax_backward_accumulate(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h,
+                                   int n, const int* d_target, const int* d_mask01, float* d_prob_scratch,
+                                   float* d_err_h, float* d_dD, float* d_db) {
+  return softmax_backward(ctx, d_D, d_b_d, V, H, d_h, n, d_target, d_mask01, d_prob_scratch, d_err_h, d_dD, d_db, 1);
 }
 
 int zr_sgd_update(zr_ctx* ctx, float* d_W, const float* d_grad, long long n, float scale, float norm_clip,

@@ -26,6 +26,7 @@ struct GemmArgs {
   // bf16 weights: B[s] is the bf16 "hi" array and Blo[s] the "lo" array of the split activations, both
   // k-interleaved by 8 ([K/8][N][8]); see zr_split_pack_x_kernel
   const unsigned short* Blo[3];
+  int accum;  // ZR_EPI_STORE only: C += result instead of C = result
 };
 
 // largest divisor c of nv with c * tm <= 32
@@ -194,7 +195,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& a, int m0, int n0, boo
       if (EPI == ZR_EPI_STORE) {
         if (ok) {
           if (bias) v += bias[m];
-          C[(long long)n * a.ldc + m] = v;
+          float* cp = C + (long long)n * a.ldc + m;
+          *cp = a.accum ? *cp + v : v;
         }
       } else if (EPI == ZR_EPI_TANH) {
         if (ok) C[(long long)n * a.ldc + m] = tanhf(v);
@@ -431,7 +433,11 @@ __global__ void __launch_bounds__(64 * NWV) gemm_lds_kernel(GemmArgs a) {
 #pragma unroll
       for (int tm = 0; tm < TMR; ++tm) {
         const int m = m0 + tm * 32 + jl;
-        if (n < a.N && m < M) a.C[(long long)n * a.ldc + m] = acc[tm][r] + bias_v[tm];
+        if (n < a.N && m < M) {
+          float* cp = a.C + (long long)n * a.ldc + m;
+          const float v = acc[tm][r] + bias_v[tm];
+          *cp = a.accum ? *cp + v : v;
+        }
       }
     }
   } else {  // ZR_EPI_SOFTMAX_PARTIAL: four columns (accumulator registers) of all row sub-tiles at a time
@@ -687,7 +693,9 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
   ga.bias = d.bias;
   ga.mask = d.mask;
   ga.partials = d.partials;
+  ga.accum = d.accumulate;
   if (d.epilogue == ZR_EPI_TANH_BIAS_MASK) ZR_CHECK_ARG(d.bias && d.mask, "gemm: bias/mask required");
+  ZR_CHECK_ARG(!d.accumulate || d.epilogue == ZR_EPI_STORE, "gemm: accumulate needs the plain store epilogue");
   if (d.epilogue == ZR_EPI_SOFTMAX_PARTIAL) ZR_CHECK_ARG(d.bias && d.partials, "gemm: bias/partials required");
 
   ga.b_pack4 = 0;

@@ -102,6 +102,7 @@ struct ZrGemmDesc {
   const int* mask;    // per column n (ZR_EPI_TANH_BIAS_MASK)
   int epilogue;
   float* partials;  // ZR_EPI_SOFTMAX_PARTIAL: [ceil(M/32)][N][2] floats
+  int accumulate;   // ZR_EPI_STORE only: C += product (+ bias) instead of C = ...
 };
 
 int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d);
