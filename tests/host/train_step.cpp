@@ -1,7 +1,9 @@
 // Test driver: SGD steps of model_trainer (zoph_rnn_amd/host/zoph_model.h) on the minibatches of an integerized file.
-//   train_step [--sequence] model.nn data.int minibatch longest_sent learning_rate norm_clip steps
+//   train_step [--sequence] [--node-level] model.nn data.int minibatch longest_sent learning_rate norm_clip steps
 // Every step trains on the next minibatch of the file (wrapping around) and prints "loss <step> <log-likelihood>";
-// the updated model is written to <model.nn>.trained as a complete model file.
+// the updated model is written to <model.nn>.trained as a complete model file.  --node-level: the step is
+// forward_model::compute_gradients, i.e. the layer objects' own back_prop_GPU / update_weights members in the
+// reference's node-by-node order, instead of model_trainer's stack-level calls.
 #include <cstdio>
 #include <cstdlib>
 #include <iostream>
@@ -11,16 +13,18 @@
 #include "../../zoph_rnn_amd/host/zoph_model.h"
 
 int main(int argc, char** argv) {
-  bool LM = false;
+  bool LM = false, node_level = false;
   std::vector<std::string> pos;
   for (int i = 1; i < argc; i++) {
     if (std::string(argv[i]) == "--sequence")
       LM = true;
+    else if (std::string(argv[i]) == "--node-level")
+      node_level = true;
     else
       pos.push_back(argv[i]);
   }
   if (pos.size() != 7) {
-    std::fprintf(stderr, "usage: %s [--sequence] model.nn data.int minibatch longest_sent learning_rate norm_clip steps\n", argv[0]);
+    std::fprintf(stderr, "usage: %s [--sequence] [--node-level] model.nn data.int minibatch longest_sent learning_rate norm_clip steps\n", argv[0]);
     return 2;
   }
   const int minibatch = std::atoi(pos[2].c_str()), longest = std::atoi(pos[3].c_str()), steps = std::atoi(pos[6].c_str());
@@ -35,9 +39,12 @@ int main(int argc, char** argv) {
   layer_gpu_info gpu;
   gpu.init(0);
   forward_model<precision> m;
+  m.params.learning_rate = lr;
+  m.params.norm_clip = clip;
+  m.params.clip_gradient = clip > 0;
   m.initModel(gpu, info, minibatch, longest, 10);
   m.load_weights(model);
-  model_trainer<precision> trainer(m);
+  model_trainer<precision>* trainer = node_level ? nullptr : new model_trainer<precision>(m);
   minibatch_reader reader;
   if (!reader.open(pos[1], minibatch, longest, LM)) {
     std::fprintf(stderr, "cannot open %s\n", pos[1].c_str());
@@ -54,7 +61,13 @@ int main(int argc, char** argv) {
       reader.input_file.seekg(0, std::ios::beg);
       if (!reader.read_minibatch(err)) return 1;
     }
-    const double loss = trainer.train_minibatch(reader, lr, clip);
+    double loss;
+    if (node_level) {
+      loss = m.getError(reader);
+      m.compute_gradients(reader);
+    } else {
+      loss = trainer->train_minibatch(reader, lr, clip);
+    }
     std::cout << "loss " << s << " " << loss << "\n";
   }
   devSynchAll(gpu.ctx);

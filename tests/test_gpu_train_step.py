@@ -125,9 +125,12 @@ def _compare(name, got, want, orig):
         name, err, tol, np.abs(d_want).max())
 
 
+@pytest.mark.parametrize("node_level", [False, True])
 @pytest.mark.parametrize("lm,L,H,mb,steps,clip", [(True, 2, 32, 4, 1, 0.4), (False, 2, 48, 3, 1, 0.25),
                                                   (False, 1, 32, 5, 3, 5.0), (True, 3, 64, 8, 2, 1.0)])
-def test_train_steps_match_oracle(tmp_path, lm, L, H, mb, steps, clip):
+def test_train_steps_match_oracle(tmp_path, lm, L, H, mb, steps, clip, node_level):
+    """node_level: the same steps through the layer objects' back_prop_GPU / update_weights members
+    (forward_model::compute_gradients) instead of model_trainer."""
     if not os.path.exists(DRIVER):
         pytest.fail("tests/host/train_step is not built: run `python __graft_entry__.py build`")
     g = synth.rng(131, L * 100 + H + mb)
@@ -159,7 +162,7 @@ def test_train_steps_match_oracle(tmp_path, lm, L, H, mb, steps, clip):
         for r in rows:
             for k in range(4):
                 f.write(" ".join(str(v) for v in r[k]) + "\n")
-    args = (["--sequence"] if lm else []) + [str(model), str(data_path), str(mb), str(longest), str(lr), str(clip),
+    args = (["--sequence"] if lm else []) + (["--node-level"] if node_level else []) + [str(model), str(data_path), str(mb), str(longest), str(lr), str(clip),
                                              str(steps)]
     r = subprocess.run([DRIVER] + args, capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, r.stderr[-2000:]

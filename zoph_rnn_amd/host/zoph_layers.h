@@ -15,7 +15,11 @@
 //   - h_t is handed to the layer above by pointer (the reference's copy_h_t == false branch,
 //     src/LSTM.hpp:492-515) instead of a device-to-device copy;
 //   - only dType = float exists (typedef float precision, src/global_params.h:3);
-//   - back-propagation, gradient and update members are not provided (forward path only);
+//   - back-propagation members exist for the LSTM layers and the softmax (backprop_prep_GPU, back_prop_GPU,
+//     compute_gradients_GPU, clear_gradients, update_weights; back_prop1 / back_prop2); the attention layer, dropout
+//     and feed-input have none.  Gradients of the four gate matrices are kept stacked (4H x H, gate order i, f, c, o)
+//     in d_M_grad_stack / d_W_h_grad_stack / d_b_grad_stack; the reference's d_M_i_grad ... members are filled from
+//     them by update_weights().  Training buffers are allocated by clear_gradients(true), not by the init calls;
 //   - weights are initialised with std::mt19937 instead of boost::mt19937: the value stream differs, the
 //     distribution (uniform in [BZ_CUDA::lower, BZ_CUDA::upper], forget bias 1) is the same.
 // Like the reference, a failed device call prints the error and exits (src/BZ_CUDA_UTIL.h:193-201).
@@ -65,8 +69,11 @@ struct attention_params {  // src/global_params.h:8-22 (fields used by the forwa
   bool feed_input = false;
 };
 
-struct global_params {  // src/global_params.h:61-299 (fields used by the forward path)
+struct global_params {  // src/global_params.h:61-299 (fields the layers use)
   attention_params attent_params;
+  bool clip_gradient = true;
+  precision norm_clip = 5.0f;
+  precision learning_rate = 0.5f;
   int LSTM_size = 100;
   int minibatch_size = 8;
   int longest_sent = 100;
@@ -169,6 +176,23 @@ struct upper_transfer_layer {
     this->softmax = softmax;
     this->hidden_layer = hidden_layer;
   }
+};
+
+// src/transfer_layer.h:38-55
+template <typename dType>
+struct lower_transfer_layer {
+  bool lower_input = true;     // the layer below is the input layer (else a hidden layer)
+  bool copy_d_Err_ht = false;  // one GPU: the error is handed down by pointer
+  Input_To_Hidden_Layer<dType>* input_layer = nullptr;
+  Hidden_To_Hidden_Layer<dType>* hidden_layer = nullptr;
+  void init_lower_transfer_layer(bool lower_input, bool copy_d_Err_ht, Input_To_Hidden_Layer<dType>* input_layer,
+                                 Hidden_To_Hidden_Layer<dType>* hidden_layer) {
+    this->lower_input = lower_input;
+    this->copy_d_Err_ht = copy_d_Err_ht;
+    this->input_layer = input_layer;
+    this->hidden_layer = hidden_layer;
+  }
+  inline void send_error(int index, dType* d_err);  // node `index` of the layer below takes d_err as its d_d_ERRt_ht
 };
 
 // ------------------------------------------------------------------------------------------------ attention
@@ -296,6 +320,13 @@ class base_loss_layer {  // src/base_loss.h:13-64 (forward-path subset)
   virtual softmax_layer_gpu_info gpu_init(int device_number) = 0;
   virtual void init_loss_layer(struct neuralMT_model<precision>* model, global_params& params) = 0;
   virtual void forward_prop(int index) = 0;
+  virtual void back_prop1(int index) = 0;
+  virtual void back_prop2(int index) = 0;
+  virtual void clear_gradients() = 0;
+  virtual void update_weights() = 0;
+  virtual void update_learning_rate(dType learning_rate) = 0;
+  virtual void init_lower_transfer_layer(bool lower_input, bool copy_d_Err_ht, Input_To_Hidden_Layer<dType>* input_layer,
+                                         Hidden_To_Hidden_Layer<dType>* hidden_layer) = 0;
   virtual void backprop_prep_GPU(dType* d_h_t, int step) = 0;
   virtual void backprop_prep_GPU_mgpu(int step) = 0;
   virtual void prep_GPU_vocab_indices(int* h_output_vocab_indicies_target, int current_target_length) = 0;
@@ -312,6 +343,7 @@ template <typename dType>
 struct softmax_node {  // src/softmax_node.h:7-27
   dType* d_outputdist = nullptr;
   dType* d_h_t = nullptr;
+  dType* d_d_ERRt_ht = nullptr;  // error at h_t of this step (allocated on first use by back_prop1)
   int index = 0;
 };
 
@@ -329,6 +361,10 @@ class softmax_layer : public base_loss_layer<dType> {  // src/softmax.h:14-225
   dType* d_output_vocab_indices_01_float = nullptr;
   int *d_output_vocab_indices_single = nullptr, *d_output_vocab_indices_01_single = nullptr;
   std::vector<softmax_node<dType>> nodes;
+  dType *d_D_grad = nullptr, *d_b_d_grad = nullptr;  // allocated by the first clear_gradients()
+  bool clip_gradients = true;
+  dType norm_clip = 5, learning_rate = 0.5f;
+  lower_transfer_layer<dType> lower_layer;
 
   softmax_layer_gpu_info gpu_init(int device_number) override {
     if (!s_layer_info.ctx) s_layer_info.init(device_number);
@@ -342,6 +378,9 @@ class softmax_layer : public base_loss_layer<dType> {  // src/softmax.h:14-225
     LSTM_size = params.LSTM_size;
     minibatch_size = params.minibatch_size;
     longest_sent = params.longest_sent;
+    clip_gradients = params.clip_gradient;
+    norm_clip = params.norm_clip;
+    learning_rate = params.learning_rate;
     zr_ctx* ctx = s_layer_info.ctx;
     dType* h = nullptr;
     full_matrix_setup(ctx, &h, &d_D, output_vocab_size, LSTM_size);
@@ -400,6 +439,45 @@ class softmax_layer : public base_loss_layer<dType> {  // src/softmax.h:14-225
     ZOPH_CALL(zr_softmax_logprob_f64(ctx, d_D, d_b_d, output_vocab_size, LSTM_size, d_h_t_in, minibatch_size,
                                      d_outputdist_perp, d_logits));
   }
+  // ---- training (src/softmax.hpp:232-300, 600-860)
+  void init_lower_transfer_layer(bool lower_input, bool copy_d_Err_ht, Input_To_Hidden_Layer<dType>* input_layer,
+                                 Hidden_To_Hidden_Layer<dType>* hidden_layer) override {
+    lower_layer.init_lower_transfer_layer(lower_input, copy_d_Err_ht, input_layer, hidden_layer);
+  }
+  void clear_gradients() override {
+    zr_ctx* ctx = s_layer_info.ctx;
+    const size_t vh = (size_t)output_vocab_size * LSTM_size;
+    if (!d_D_grad) {
+      ZOPH_CALL(zr_malloc(ctx, vh * sizeof(dType), (void**)&d_D_grad));
+      ZOPH_CALL(zr_malloc(ctx, (size_t)output_vocab_size * sizeof(dType), (void**)&d_b_d_grad));
+    }
+    ZOPH_CALL(zr_memset_zero(ctx, d_D_grad, vh * sizeof(dType)));
+    ZOPH_CALL(zr_memset_zero(ctx, d_b_d_grad, (size_t)output_vocab_size * sizeof(dType)));
+  }
+  // back_prop1: the error at h_t of step `index` (get_h_t_gradient_GPU), handed to the layer below.  The D and b_d
+  // gradient terms of the step (compute_D_gradient_GPU, compute_b_d_gradient_GPU -- back_prop2 in the reference) come
+  // out of the same library call, so they are accumulated here and back_prop2 has nothing left to do.  The step's
+  // distribution is recomputed from nodes[index].d_h_t; backprop_prep_GPU(_, index * minibatch_size) must precede.
+  void back_prop1(int index) override {
+    zr_ctx* ctx = s_layer_info.ctx;
+    if (!d_D_grad) clear_gradients();
+    if (!nodes[index].d_d_ERRt_ht) full_matrix_setup_0(ctx, &nodes[index].d_d_ERRt_ht, LSTM_size, minibatch_size);
+    dType* h = nodes[index].d_h_t ? nodes[index].d_h_t : d_h_t;
+    ZOPH_CALL(zr_softmax_backward_accumulate(ctx, d_D, d_b_d, output_vocab_size, LSTM_size, h, minibatch_size,
+                                             d_output_vocab_indices_single, d_output_vocab_indices_01_single,
+                                             d_logits, nodes[index].d_d_ERRt_ht, d_D_grad, d_b_d_grad));
+    lower_layer.send_error(index, nodes[index].d_d_ERRt_ht);
+  }
+  void back_prop2(int /*index*/) override {}
+  // scale by 1 / minibatch_size, clip each gradient to norm_clip in L2 norm, add (gradient ascent on log-likelihood)
+  void update_weights() override {
+    zr_ctx* ctx = s_layer_info.ctx;
+    const float scale = 1.0f / (float)minibatch_size, clip = clip_gradients ? norm_clip : 0.0f;
+    ZOPH_CALL(zr_sgd_update(ctx, d_D, d_D_grad, (long long)output_vocab_size * LSTM_size, scale, clip, learning_rate));
+    ZOPH_CALL(zr_sgd_update(ctx, d_b_d, d_b_d_grad, output_vocab_size, scale, clip, learning_rate));
+    prepare_weights();
+  }
+  void update_learning_rate(dType lr) override { learning_rate = lr; }
   dType* get_ht_ptr(int index) override { return nodes[index].d_h_t; }
   void set_ht_ptr(int index, dType* d_h_t) override { nodes[index].d_h_t = d_h_t; }
   // src/softmax.hpp:1028-1030
@@ -429,6 +507,65 @@ class softmax_layer : public base_loss_layer<dType> {  // src/softmax.h:14-225
 };
 
 // ------------------------------------------------------------------------------------------------ LSTM nodes
+// Training-side members both LSTM layer classes carry (the reference declares them in each class:
+// src/Hidden_To_Hidden_Layer.h:143-233, src/Input_To_Hidden_Layer.h).  Nothing here is allocated until
+// clear_gradients(true) runs.
+template <typename dType>
+struct lstm_layer_training {
+  zr_lstm_train* train_weights = nullptr;  // transposed, gate-stacked snapshot of M and W_h for the error products
+  dType *d_M_grad_stack = nullptr, *d_W_h_grad_stack = nullptr, *d_b_grad_stack = nullptr;  // 4H x H, 4H x H, 4H
+  dType *d_W_hi_grad = nullptr, *d_W_hf_grad = nullptr, *d_W_hc_grad = nullptr, *d_W_ho_grad = nullptr;
+  dType *d_M_i_grad = nullptr, *d_M_f_grad = nullptr, *d_M_o_grad = nullptr, *d_M_c_grad = nullptr;
+  dType *d_b_i_grad = nullptr, *d_b_f_grad = nullptr, *d_b_c_grad = nullptr, *d_b_o_grad = nullptr;
+  // errors of the node being processed; d_d_ERRnTOt_h_Below sits directly behind d_d_ERRnTOt_htM1
+  dType *d_d_ERRnTOt_htM1 = nullptr, *d_d_ERRnTOt_h_Below = nullptr, *d_d_ERRnTOt_ctM1 = nullptr;
+  dType* d_d_ERRnTOt_gates = nullptr;  // 4H x minibatch: the reference's d_d_ERRnTOt_it, _ft, _tanhcpt, _ot stacked
+  dType *d_init_d_ERRnTOtp1_ht = nullptr, *d_init_d_ERRnTOtp1_ct = nullptr;  // zeros for the last time step
+  dType learning_rate = 0.5f, norm_clip = 5;
+  bool clip_gradients = true;
+  lower_transfer_layer<dType> lower_layer;
+
+  void alloc_training(zr_ctx* ctx, int H, int mb) {
+    const size_t hh = (size_t)H * H, n = (size_t)H * mb;
+    full_matrix_setup_0(ctx, &d_M_grad_stack, 4 * H, H);
+    full_matrix_setup_0(ctx, &d_W_h_grad_stack, 4 * H, H);
+    full_matrix_setup_0(ctx, &d_b_grad_stack, 4 * H, 1);
+    dType** mats[] = {&d_W_hi_grad, &d_W_hf_grad, &d_W_hc_grad, &d_W_ho_grad, &d_M_i_grad, &d_M_f_grad, &d_M_c_grad, &d_M_o_grad};
+    for (dType** m : mats) ZOPH_CALL(zr_malloc(ctx, hh * sizeof(dType), (void**)m));
+    d_b_i_grad = d_b_grad_stack;
+    d_b_f_grad = d_b_grad_stack + H;
+    d_b_c_grad = d_b_grad_stack + 2 * (size_t)H;
+    d_b_o_grad = d_b_grad_stack + 3 * (size_t)H;
+    full_matrix_setup_0(ctx, &d_d_ERRnTOt_htM1, H, 2 * mb);
+    d_d_ERRnTOt_h_Below = d_d_ERRnTOt_htM1 + n;
+    full_matrix_setup_0(ctx, &d_d_ERRnTOt_ctM1, H, mb);
+    full_matrix_setup_0(ctx, &d_d_ERRnTOt_gates, 4 * H, mb);
+    full_matrix_setup_0(ctx, &d_init_d_ERRnTOtp1_ht, H, mb);
+    full_matrix_setup_0(ctx, &d_init_d_ERRnTOtp1_ct, H, mb);
+  }
+  void zero_gradients(zr_ctx* ctx, int H) {
+    ZOPH_CALL(zr_memset_zero(ctx, d_M_grad_stack, 4 * (size_t)H * H * sizeof(dType)));
+    ZOPH_CALL(zr_memset_zero(ctx, d_W_h_grad_stack, 4 * (size_t)H * H * sizeof(dType)));
+    ZOPH_CALL(zr_memset_zero(ctx, d_b_grad_stack, 4 * (size_t)H * sizeof(dType)));
+  }
+  // scale_gradients + norm_clip_GPU_v2 per matrix + update_params (src/Hidden_To_Hidden_Layer.hpp:497-560): every
+  // matrix and bias vector is scaled by 1 / minibatch_size, clipped on its own, and added
+  void apply_gradients(zr_ctx* ctx, int H, int mb, dType* const M[4], dType* const Wh[4], dType* const b[4]) {
+    const float scale = 1.0f / (float)mb, clip = clip_gradients ? (float)norm_clip : 0.0f;
+    const long long hh = (long long)H * H;
+    dType* gM[4] = {d_M_i_grad, d_M_f_grad, d_M_c_grad, d_M_o_grad};
+    dType* gWh[4] = {d_W_hi_grad, d_W_hf_grad, d_W_hc_grad, d_W_ho_grad};
+    dType* gb[4] = {d_b_i_grad, d_b_f_grad, d_b_c_grad, d_b_o_grad};
+    ZOPH_CALL(zr_unstack_gates(ctx, d_M_grad_stack, H, gM));
+    ZOPH_CALL(zr_unstack_gates(ctx, d_W_h_grad_stack, H, gWh));
+    for (int g = 0; g < 4; g++) {
+      ZOPH_CALL(zr_sgd_update(ctx, M[g], gM[g], hh, scale, clip, learning_rate));
+      ZOPH_CALL(zr_sgd_update(ctx, Wh[g], gWh[g], hh, scale, clip, learning_rate));
+      ZOPH_CALL(zr_sgd_update(ctx, b[g], gb[g], H, scale, clip, learning_rate));
+    }
+  }
+};
+
 template <typename dType>
 class LSTM_HH_Node {  // src/LSTM_HH.h:19-102
  public:
@@ -443,9 +580,17 @@ class LSTM_HH_Node {  // src/LSTM_HH.h:19-102
   dType *d_c_t_prev = nullptr, *d_h_t_prev = nullptr;
   dType* d_h_t_below = nullptr;
   dType* d_zeros = nullptr;
+  // errors arriving from step t+1 and from above (NULL: none); set by backprop_prep_GPU / the layer above
+  dType *d_d_ERRnTOtp1_ht = nullptr, *d_d_ERRnTOtp1_ct = nullptr, *d_d_ERRt_ht = nullptr;
 
   LSTM_HH_Node(int LSTM_size, int minibatch_size, Hidden_To_Hidden_Layer<dType>* m, int index, dType* d_zeros,
                bool dropout, dType dropout_rate);
+  void backprop_prep_GPU(dType* d_d_ERRnTOtp1_ht, dType* d_d_ERRnTOtp1_ct) {  // src/LSTM_HH.hpp:430-434
+    this->d_d_ERRnTOtp1_ht = d_d_ERRnTOtp1_ht;
+    this->d_d_ERRnTOtp1_ct = d_d_ERRnTOtp1_ct;
+  }
+  void back_prop_GPU(int index);     // src/LSTM_HH.hpp:452-700
+  void compute_gradients_GPU();      // src/LSTM_HH.hpp:700-900
   void update_vectors_forward_GPU(int* d_input_vocab_indices_01, dType* d_h_t_prev, dType* d_c_t_prev) {
     this->d_h_t_prev = d_h_t_prev;
     this->d_c_t_prev = d_c_t_prev;
@@ -474,9 +619,16 @@ class LSTM_IH_Node {  // src/LSTM.h:19-106
   dType *d_c_t_prev = nullptr, *d_h_t_prev = nullptr;
   dType* d_zeros = nullptr;
   dType* d_h_tild = nullptr;
+  dType *d_d_ERRnTOtp1_ht = nullptr, *d_d_ERRnTOtp1_ct = nullptr, *d_d_ERRt_ht = nullptr;
 
   LSTM_IH_Node(int LSTM_size, int minibatch_size, int vocab_size, Input_To_Hidden_Layer<dType>* m, int index,
                dType* d_zeros, bool dropout, dType dropout_rate);
+  void backprop_prep_GPU(dType* d_d_ERRnTOtp1_ht, dType* d_d_ERRnTOtp1_ct) {  // src/LSTM.hpp:523-530
+    this->d_d_ERRnTOtp1_ht = d_d_ERRnTOtp1_ht;
+    this->d_d_ERRnTOtp1_ct = d_d_ERRnTOtp1_ct;
+  }
+  void back_prop_GPU(int index);     // src/LSTM.hpp:542-960
+  void compute_gradients_GPU();      // src/LSTM.hpp:963-1270
   void update_vectors_forward_GPU(int* d_input_vocab_indices, int* d_input_vocab_indices_01, dType* d_h_t_prev,
                                   dType* d_c_t_prev) {
     this->d_h_t_prev = d_h_t_prev;
@@ -496,7 +648,7 @@ class LSTM_IH_Node {  // src/LSTM.h:19-106
 
 // ------------------------------------------------------------------------------------------------ layers
 template <typename dType>
-class Hidden_To_Hidden_Layer {  // src/Hidden_To_Hidden_Layer.h:12-313
+class Hidden_To_Hidden_Layer : public lstm_layer_training<dType> {  // src/Hidden_To_Hidden_Layer.h:12-313
  public:
   layer_gpu_info hh_layer_info;
   std::vector<LSTM_HH_Node<dType>> nodes;
@@ -513,9 +665,12 @@ class Hidden_To_Hidden_Layer {  // src/Hidden_To_Hidden_Layer.h:12-313
 
   // src/Hidden_To_Hidden_Layer.hpp:125-155 (and :4-112 for the device side)
   void init_Hidden_To_Hidden_Layer(int LSTM_size, int minibatch_size, int longest_sent, bool /*debug_temp*/,
-                                   dType /*learning_rate*/, bool /*clip_gradients*/, dType /*norm_clip*/,
+                                   dType learning_rate, bool clip_gradients, dType norm_clip,
                                    struct neuralMT_model<precision>* model, int /*seed*/, bool dropout,
                                    dType dropout_rate, bool /*bi_dir*/, int layer_number) {
+    this->learning_rate = learning_rate;
+    this->clip_gradients = clip_gradients;
+    this->norm_clip = norm_clip;
     this->LSTM_size = LSTM_size;
     this->minibatch_size = minibatch_size;
     this->longest_sent = longest_sent;
@@ -548,6 +703,33 @@ class Hidden_To_Hidden_Layer {  // src/Hidden_To_Hidden_Layer.h:12-313
     else
       ZOPH_CALL(zr_lstm_pack_weights(ctx, M, Wh, nullptr, b, LSTM_size, &packed));
   }
+  // ---- training.  clear_gradients(true) allocates the training buffers (src/Hidden_To_Hidden_Layer.hpp:158-232
+  // allocates them in the init call) and zeroes; clear_gradients(false) zeroes (:283-316).
+  void clear_gradients(bool init) {
+    zr_ctx* ctx = hh_layer_info.ctx;
+    if (init || !this->train_weights) {
+      if (!this->train_weights) {
+        this->alloc_training(ctx, LSTM_size, minibatch_size);
+        const dType* M[4] = {d_M_i, d_M_f, d_M_c, d_M_o};
+        const dType* Wh[4] = {d_W_hi, d_W_hf, d_W_hc, d_W_ho};
+        ZOPH_CALL(zr_lstm_train_create(ctx, M, Wh, LSTM_size, &this->train_weights));
+      }
+    }
+    this->zero_gradients(ctx, LSTM_size);
+  }
+  void clear_gradients_GPU(bool init) { clear_gradients(init); }
+  // src/Hidden_To_Hidden_Layer.hpp:497-560, then the snapshots the kernels read are rebuilt
+  void update_weights() {
+    zr_ctx* ctx = hh_layer_info.ctx;
+    dType* M[4] = {d_M_i, d_M_f, d_M_c, d_M_o};
+    dType* Wh[4] = {d_W_hi, d_W_hf, d_W_hc, d_W_ho};
+    dType* b[4] = {d_b_i, d_b_f, d_b_c, d_b_o};
+    this->apply_gradients(ctx, LSTM_size, minibatch_size, M, Wh, b);
+    repack();
+    ZOPH_CALL(zr_lstm_train_refresh(ctx, this->train_weights, M, Wh));
+  }
+  void update_weights_GPU() { update_weights(); }
+  void update_learning_rate(dType lr) { this->learning_rate = lr; }
   // src/Hidden_To_Hidden_Layer.hpp:748-774
   void prep_GPU_vocab_indices(int* h_input_vocab_indicies, int current_length) {
     zr_ctx* ctx = hh_layer_info.ctx;
@@ -618,7 +800,7 @@ class Hidden_To_Hidden_Layer {  // src/Hidden_To_Hidden_Layer.h:12-313
 };
 
 template <typename dType>
-class Input_To_Hidden_Layer {  // src/Input_To_Hidden_Layer.h:11-368
+class Input_To_Hidden_Layer : public lstm_layer_training<dType> {  // src/Input_To_Hidden_Layer.h:11-368
  public:
   layer_gpu_info ih_layer_info;
   std::vector<LSTM_IH_Node<dType>> nodes;
@@ -638,11 +820,14 @@ class Input_To_Hidden_Layer {  // src/Input_To_Hidden_Layer.h:11-368
 
   // src/Input_To_Hidden_Layer.hpp:171-202 (and :3-159 for the device side)
   void init_Input_To_Hidden_Layer(int LSTM_size, int minibatch_size, int vocab_size, int longest_sent,
-                                  bool /*debug_temp*/, dType /*learning_rate*/, bool /*clip_gradients*/,
-                                  dType /*norm_clip*/, struct neuralMT_model<precision>* model, int /*seed*/,
+                                  bool /*debug_temp*/, dType learning_rate, bool clip_gradients,
+                                  dType norm_clip, struct neuralMT_model<precision>* model, int /*seed*/,
                                   bool dropout, dType dropout_rate, bool /*is_bi_dir*/, bool share_embeddings,
                                   dType* d_embedding_ptr, bool /*combine_embeddings*/, global_params& /*params*/,
                                   bool /*source*/) {
+    this->learning_rate = learning_rate;
+    this->clip_gradients = clip_gradients;
+    this->norm_clip = norm_clip;
     this->LSTM_size = LSTM_size;
     this->minibatch_size = minibatch_size;
     this->input_vocab_size = vocab_size;
@@ -680,6 +865,37 @@ class Input_To_Hidden_Layer {  // src/Input_To_Hidden_Layer.h:11-368
     else
       ZOPH_CALL(zr_lstm_pack_weights(ctx, M, Wh, feed_input ? Q : nullptr, b, LSTM_size, &packed));
   }
+  // ---- training: as in Hidden_To_Hidden_Layer plus the embedding gradient d_W_grad (dense LSTM_size x vocabulary;
+  // the reference keeps the same matrix and touches only the minibatch's columns, src/custom_kernels.h:1346-1368)
+  dType* d_W_grad = nullptr;
+  void clear_gradients(bool init) {
+    zr_ctx* ctx = ih_layer_info.ctx;
+    if (init || !this->train_weights) {
+      if (!this->train_weights) {
+        this->alloc_training(ctx, LSTM_size, minibatch_size);
+        full_matrix_setup_0(ctx, &d_W_grad, LSTM_size, input_vocab_size);
+        const dType* M[4] = {d_M_i, d_M_f, d_M_c, d_M_o};
+        const dType* Wh[4] = {d_W_hi, d_W_hf, d_W_hc, d_W_ho};
+        ZOPH_CALL(zr_lstm_train_create(ctx, M, Wh, LSTM_size, &this->train_weights));
+      }
+    }
+    this->zero_gradients(ctx, LSTM_size);
+    ZOPH_CALL(zr_memset_zero(ctx, d_W_grad, (size_t)LSTM_size * input_vocab_size * sizeof(dType)));
+  }
+  void clear_gradients_GPU(bool init) { clear_gradients(init); }
+  void update_weights() {  // src/Input_To_Hidden_Layer.hpp:690-790
+    zr_ctx* ctx = ih_layer_info.ctx;
+    dType* M[4] = {d_M_i, d_M_f, d_M_c, d_M_o};
+    dType* Wh[4] = {d_W_hi, d_W_hf, d_W_hc, d_W_ho};
+    dType* b[4] = {d_b_i, d_b_f, d_b_c, d_b_o};
+    ZOPH_CALL(zr_sgd_update(ctx, d_W, d_W_grad, (long long)LSTM_size * input_vocab_size, 1.0f / (float)minibatch_size,
+                            this->clip_gradients ? (float)this->norm_clip : 0.0f, this->learning_rate));
+    this->apply_gradients(ctx, LSTM_size, minibatch_size, M, Wh, b);
+    repack();
+    ZOPH_CALL(zr_lstm_train_refresh(ctx, this->train_weights, M, Wh));
+  }
+  void update_weights_GPU() { update_weights(); }
+  void update_learning_rate(dType lr) { this->learning_rate = lr; }
   // src/Input_To_Hidden_Layer.hpp:1178-1225 (the *_Wgrad arguments serve the embedding gradient only)
   void prep_GPU_vocab_indices(int* h_input_vocab_indicies, int* /*h_input_vocab_indicies_Wgrad*/, int current_length,
                               int /*len_W*/) {
@@ -879,6 +1095,67 @@ void LSTM_IH_Node<dType>::send_h_t_above() {  // src/LSTM.hpp:424-520, pointer-p
   } else if (model->upper_layer.hidden_layer) {
     model->upper_layer.hidden_layer->nodes[idx].d_h_t_below = out;
   }
+}
+
+// ------------------------------------------------------------------------------------------------ backward
+template <typename dType>
+void lower_transfer_layer<dType>::send_error(int index, dType* d_err) {
+  if (lower_input) {
+    if (input_layer) input_layer->nodes[index].d_d_ERRt_ht = d_err;
+  } else if (hidden_layer) {
+    hidden_layer->nodes[index].d_d_ERRt_ht = d_err;
+  }
+}
+
+// One node of back-propagation through time.  The reference runs nine element-wise kernels and eight products per
+// node; here the node is one element-wise kernel and one batched product (zr_lstm_node_backward), followed by the
+// node's share of the weight gradients.  The errors for step t-1 land in the layer's d_d_ERRnTOt_htM1 / _ctM1, which
+// the driver passes to the next backprop_prep_GPU call, and the error for the layer below is handed down by pointer.
+template <typename dType>
+void LSTM_HH_Node<dType>::back_prop_GPU(int index) {
+  zr_ctx* ctx = model->hh_layer_info.ctx;
+  if (!model->train_weights) model->clear_gradients(true);
+  const dType* gates[4] = {d_i_t, d_f_t, d_c_prime_t_tanh, d_o_t};
+  ZOPH_CALL(zr_lstm_node_backward(ctx, model->train_weights, minibatch_size, gates, d_c_t, d_c_t_prev,
+                                  d_input_vocab_indices_01, d_d_ERRt_ht, d_d_ERRnTOtp1_ht, d_d_ERRnTOtp1_ct,
+                                  model->d_d_ERRnTOt_gates, model->d_d_ERRnTOt_htM1, model->d_d_ERRnTOt_ctM1,
+                                  model->d_d_ERRnTOt_h_Below));
+  compute_gradients_GPU();
+  model->lower_layer.send_error(index, model->d_d_ERRnTOt_h_Below);
+}
+
+template <typename dType>
+void LSTM_HH_Node<dType>::compute_gradients_GPU() {
+  ZOPH_CALL(zr_lstm_node_gradients(model->hh_layer_info.ctx, LSTM_size, minibatch_size, model->d_d_ERRnTOt_gates,
+                                   d_h_t_below, d_h_t_prev, model->d_M_grad_stack, model->d_W_h_grad_stack,
+                                   model->d_b_grad_stack));
+}
+
+template <typename dType>
+void LSTM_IH_Node<dType>::back_prop_GPU(int /*index*/) {
+  zr_ctx* ctx = model->ih_layer_info.ctx;
+  if (feed_input) {
+    std::fprintf(stderr, "Error: back-propagation through the feed-input connection is not built\n");
+    std::exit(EXIT_FAILURE);
+  }
+  if (!model->train_weights) model->clear_gradients(true);
+  const dType* gates[4] = {d_i_t, d_f_t, d_c_prime_t_tanh, d_o_t};
+  ZOPH_CALL(zr_lstm_node_backward(ctx, model->train_weights, minibatch_size, gates, d_c_t, d_c_t_prev,
+                                  d_input_vocab_indices_01, d_d_ERRt_ht, d_d_ERRnTOtp1_ht, d_d_ERRnTOtp1_ct,
+                                  model->d_d_ERRnTOt_gates, model->d_d_ERRnTOt_htM1, model->d_d_ERRnTOt_ctM1,
+                                  model->d_d_ERRnTOt_h_Below));
+  compute_gradients_GPU();
+}
+
+template <typename dType>
+void LSTM_IH_Node<dType>::compute_gradients_GPU() {
+  zr_ctx* ctx = model->ih_layer_info.ctx;
+  ZOPH_CALL(zr_lstm_node_gradients(ctx, LSTM_size, minibatch_size, model->d_d_ERRnTOt_gates, d_sparse_lookup,
+                                   d_h_t_prev, model->d_M_grad_stack, model->d_W_h_grad_stack, model->d_b_grad_stack));
+  // the sparse W gradient (src/custom_kernels.h:353-378): the error at the node's input, added into the columns of
+  // the minibatch's words
+  ZOPH_CALL(zr_embed_gradient(ctx, LSTM_size, model->input_vocab_size, model->d_d_ERRnTOt_h_Below,
+                              d_input_vocab_indices, d_input_vocab_indices_01, minibatch_size, model->d_W_grad));
 }
 
 #endif  // ZOPH_LAYERS_H

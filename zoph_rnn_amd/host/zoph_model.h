@@ -401,32 +401,40 @@ class forward_model {
     softmax->init_loss_layer(&flags, params);
     if (seq2seq) {
       input_layer_source.ih_layer_info.share(gpu);
-      input_layer_source.init_Input_To_Hidden_Layer(H, minibatch_size, mi.source_vocab_size, longest_sent, false, 0.f,
-                                                    false, 0.f, &flags, 0, false, 0.f, false, false, nullptr, false,
-                                                    params, true);
+      input_layer_source.init_Input_To_Hidden_Layer(H, minibatch_size, mi.source_vocab_size, longest_sent, false,
+                                                    params.learning_rate, params.clip_gradient, params.norm_clip,
+                                                    &flags, 0, false, 0.f, false, false, nullptr, false, params, true);
       for (int l = 0; l < L - 1; l++) {
         source_hidden_layers[l].hh_layer_info.share(gpu);
-        source_hidden_layers[l].init_Hidden_To_Hidden_Layer(H, minibatch_size, longest_sent, false, 0.f, false, 0.f,
-                                                             &flags, 0, false, 0.f, false, l);
+        source_hidden_layers[l].init_Hidden_To_Hidden_Layer(H, minibatch_size, longest_sent, false, params.learning_rate,
+                                                             params.clip_gradient, params.norm_clip, &flags, 0, false,
+                                                             0.f, false, l);
       }
     }
     input_layer_target.ih_layer_info.share(gpu);
-    input_layer_target.init_Input_To_Hidden_Layer(H, minibatch_size, mi.target_vocab_size, longest_sent, false, 0.f,
-                                                  false, 0.f, &flags, 0, false, 0.f, false, false, nullptr, false,
-                                                  params, false);
+    input_layer_target.init_Input_To_Hidden_Layer(H, minibatch_size, mi.target_vocab_size, longest_sent, false,
+                                                  params.learning_rate, params.clip_gradient, params.norm_clip, &flags,
+                                                  0, false, 0.f, false, false, nullptr, false, params, false);
     for (int l = 0; l < L - 1; l++) {
       target_hidden_layers[l].hh_layer_info.share(gpu);
-      target_hidden_layers[l].init_Hidden_To_Hidden_Layer(H, minibatch_size, longest_sent, false, 0.f, false, 0.f,
-                                                           &flags, 0, false, 0.f, false, l);
+      target_hidden_layers[l].init_Hidden_To_Hidden_Layer(H, minibatch_size, longest_sent, false, params.learning_rate,
+                                                           params.clip_gradient, params.norm_clip, &flags, 0, false,
+                                                           0.f, false, l);
     }
+    // upper transfer (h_t upwards) and lower transfer (error downwards) wiring, src/model.hpp:191-290
     auto wire = [&](Input_To_Hidden_Layer<dType>& in, std::vector<Hidden_To_Hidden_Layer<dType>>& hid, bool source) {
       if (hid.empty()) {
         in.upper_layer.init_upper_transfer_layer(true, false, source, softmax, nullptr);
+        if (!source) softmax->init_lower_transfer_layer(true, false, &in, nullptr);
       } else {
         in.upper_layer.init_upper_transfer_layer(false, false, source, nullptr, &hid[0]);
-        for (size_t l = 0; l + 1 < hid.size(); l++)
+        hid[0].lower_layer.init_lower_transfer_layer(true, false, &in, nullptr);
+        for (size_t l = 0; l + 1 < hid.size(); l++) {
           hid[l].upper_layer.init_upper_transfer_layer(false, false, source, nullptr, &hid[l + 1]);
+          hid[l + 1].lower_layer.init_lower_transfer_layer(false, false, nullptr, &hid[l]);
+        }
         hid.back().upper_layer.init_upper_transfer_layer(true, false, source, softmax, nullptr);
+        if (!source) softmax->init_lower_transfer_layer(false, false, nullptr, &hid.back());
       }
     };
     if (seq2seq) wire(input_layer_source, source_hidden_layers, true);
@@ -472,6 +480,12 @@ class forward_model {
   // neuralMT_model::getError(GPU = true), src/model.hpp:1463-1802: natural-log probability of the minibatch's
   // target words.  per_step, if given, is called after each target step with (step, loss of the step).
   double getError(minibatch_reader& mb, const std::function<void(int, double)>& per_step = nullptr) {
+    return forward_pass(mb, true, per_step);
+  }
+
+  // The forward half shared by getError and compute_gradients: every node of the (layer, time) grid in the
+  // reference's order; with_loss adds the loss layer's log-probability of every step.
+  double forward_pass(minibatch_reader& mb, bool with_loss, const std::function<void(int, double)>& per_step = nullptr) {
     const bool seq2seq = !info.LM;
     const int S = seq2seq ? mb.current_source_length : 0, T = mb.current_target_length;
     const int mbs = params.minibatch_size;
@@ -532,12 +546,83 @@ class forward_model {
         ly.nodes[i].update_vectors_forward_GPU(ly.d_input_vocab_indices_01_full + step, hp, cp);
         ly.nodes[i].forward_prop();
       }
+      if (!with_loss) continue;
       softmax->backprop_prep_GPU(softmax->get_ht_ptr(i), step);
       const double loss = softmax->compute_loss_GPU(i);
       total += loss;
       if (per_step) per_step(i, loss);
     }
     return total;
+  }
+
+  // neuralMT_model::compute_gradients (src/model.hpp:813-1230) for models without attention, through the layer
+  // objects' own members in the reference's order: forward over the grid, then per target step (last first) the loss
+  // layer's back_prop1 and the nodes' backprop_prep_GPU / back_prop_GPU from the top layer down, then the source side
+  // started from the errors the target side left at its first step, then update_weights and clear_gradients.
+  void compute_gradients(minibatch_reader& mb) {
+    if (params.attent_params.attention_model) {
+      std::fprintf(stderr, "compute_gradients: the backward pass of the attention layer is not built\n");
+      std::exit(EXIT_FAILURE);
+    }
+    const bool seq2seq = !info.LM;
+    const int S = seq2seq ? mb.current_source_length : 0, T = mb.current_target_length;
+    const int mbs = params.minibatch_size;
+    if (!trained_before) {
+      clear_gradients(true);
+      trained_before = true;
+    }
+    forward_pass(mb, false);
+    for (int i = T - 1; i >= 0; i--) {
+      const bool last = i == T - 1;
+      softmax->backprop_prep_GPU(softmax->get_ht_ptr(i), i * mbs);
+      softmax->back_prop1(i);
+      for (int j = (int)target_hidden_layers.size() - 1; j >= 0; j--) {
+        auto& ly = target_hidden_layers[j];
+        ly.nodes[i].backprop_prep_GPU(last ? ly.d_init_d_ERRnTOtp1_ht : ly.d_d_ERRnTOt_htM1,
+                                      last ? ly.d_init_d_ERRnTOtp1_ct : ly.d_d_ERRnTOt_ctM1);
+        ly.nodes[i].back_prop_GPU(i);
+      }
+      auto& in = input_layer_target;
+      in.nodes[i].backprop_prep_GPU(last ? in.d_init_d_ERRnTOtp1_ht : in.d_d_ERRnTOt_htM1,
+                                    last ? in.d_init_d_ERRnTOtp1_ct : in.d_d_ERRnTOt_ctM1);
+      in.nodes[i].back_prop_GPU(i);
+      softmax->back_prop2(i);
+    }
+    for (int i = S - 1; i >= 0; i--) {
+      const bool last = i == S - 1;  // the source's last step continues from the target's first (:1097-1126)
+      for (int j = (int)source_hidden_layers.size() - 1; j >= 0; j--) {
+        auto& ly = source_hidden_layers[j];
+        ly.nodes[i].backprop_prep_GPU(last ? target_hidden_layers[j].d_d_ERRnTOt_htM1 : ly.d_d_ERRnTOt_htM1,
+                                      last ? target_hidden_layers[j].d_d_ERRnTOt_ctM1 : ly.d_d_ERRnTOt_ctM1);
+        ly.nodes[i].back_prop_GPU(i);
+      }
+      auto& in = input_layer_source;
+      in.nodes[i].backprop_prep_GPU(last ? input_layer_target.d_d_ERRnTOt_htM1 : in.d_d_ERRnTOt_htM1,
+                                    last ? input_layer_target.d_d_ERRnTOt_ctM1 : in.d_d_ERRnTOt_ctM1);
+      in.nodes[i].back_prop_GPU(i);
+    }
+    update_weights();
+    clear_gradients(false);
+  }
+  bool trained_before = false;
+
+  void clear_gradients(bool init) {  // src/model.hpp:1431-1460
+    if (!info.LM) {
+      input_layer_source.clear_gradients(init);
+      for (auto& l : source_hidden_layers) l.clear_gradients(init);
+    }
+    input_layer_target.clear_gradients(init);
+    for (auto& l : target_hidden_layers) l.clear_gradients(init);
+    softmax->clear_gradients();
+  }
+  void update_weights() {  // src/model.hpp:1845-1955, per-matrix clipping (no global norm)
+    softmax->update_weights();
+    if (!info.LM) {
+      input_layer_source.update_weights();
+      for (auto& l : source_hidden_layers) l.update_weights();
+    }
+    input_layer_target.update_weights();
+    for (auto& l : target_hidden_layers) l.update_weights();
   }
 
   // neuralMT_model::get_perplexity (src/model.hpp:2281-2355): one getError per minibatch; with force_decode the
