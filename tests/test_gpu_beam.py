@@ -131,3 +131,57 @@ def test_beam_full_vocab_shape(ctx):
             assert np.array_equal(words[s * beam:(s + 1) * beam], st["current_indices"])
             assert np.array_equal(back[s * beam:(s + 1) * beam] - s * beam, st["new_indicies_changes"])
     ctx.beam_destroy(b)
+
+
+def _expand_given(ctx, Ps, beam, n_sent, max_len):
+    """beam_expand over the given distributions against the oracle decoder, word ids and back-pointers bit-exact."""
+    V = Ps[0].shape[0]
+    b = ctx.beam_create(beam, V, n_sent, max_len, 0.0)
+    decs = [o.Decoder(beam, V, max_len) for _ in range(n_sent)]
+    d_words, d_back = ctx.empty(n_sent * beam, np.int32), ctx.empty(n_sent * beam, np.int32)
+    for index, P in enumerate(Ps):
+        ctx.beam_expand(b, ctx.array(P), index, d_words, d_back)
+        ctx.sync()
+        words, back = d_words.get(), d_back.get()
+        for s in range(n_sent):
+            decs[s].expand(P[:, s * beam:(s + 1) * beam], index)
+            st = decs[s].state()
+            assert np.array_equal(words[s * beam:(s + 1) * beam], st["current_indices"]), (index, s)
+            assert np.array_equal(back[s * beam:(s + 1) * beam] - s * beam, st["new_indicies_changes"]), (index, s)
+    ctx.beam_destroy(b)
+
+
+@pytest.mark.parametrize("V,beam", [(40003, 12), (16384, 5), (16385, 31), (70000, 20)])
+def test_beam_selection_on_adversarial_layouts(ctx, V, beam):
+    """Layouts chosen against the selection kernel's structure (one workgroup per 16384 words, each thread holding
+    words 4t..4t+3 of every 1024): the largest values all inside one thread's share, at chunk boundaries, in the
+    ragged tail, and values that fall steadily with the word id; vocabulary sizes that are not multiples of 4 take the scalar-load path."""
+    g = synth.rng(43, V)
+    n_sent = 2
+    cols = n_sent * beam
+    # distinct small values: a random permutation of an evenly spaced grid in every column
+    base = np.stack([g.permutation(V) for _ in range(cols)], axis=1) * (1e-3 / V) + 1e-4
+    P = []
+    a = base.copy()                                    # step 0: big values in thread 5's words of chunk 0
+    idx = np.array([4 * 5 + c + 1024 * i for i in range(16) for c in range(4)])
+    idx = idx[(idx > 1) & (idx < V)]
+    a[idx, :] += 1.0 + g.random((idx.size, cols))
+    P.append(a)
+    a = base.copy()                                    # step 1: big values around chunk boundaries and the tail
+    edge = np.array([v for v in (16383, 16384, 16385, 32767, 32768, V - 1, V - 2, V - 3, 2, 3) if 1 < v < V])
+    a[edge, :] += 1.0 + g.random((edge.size, cols))
+    P.append(a)
+    a = base.copy()                                    # step 2: values falling with the word id
+    a += np.exp(-np.arange(V) / 200.0)[:, None] * (1.0 + 0.01 * np.arange(cols))[None, :]
+    P.append(a)
+    a = base.copy()                                    # step 3: in every wave of chunk 0, `beam` threads whose whole
+    ts = [w * 64 + j for w in range(4) for j in range(beam)]   # share is large: the list built from the wave-level
+    idx = np.array([4 * t + c + 1024 * i for t in ts for i in range(16) for c in range(4)])  # bound overflows
+    idx = idx[(idx > 1) & (idx < V)]
+    a[idx, :] = 1.0 + np.stack([g.permutation(idx.size) for _ in range(cols)], axis=1) / idx.size
+    P.append(a)
+    Ps = [np.asfortranarray((p / p.sum(axis=0)).astype(np.float32)) for p in P]
+    for p in Ps:  # the oracle comparison needs tie-free columns at the top
+        top = np.sort(p, axis=0)[-(beam + 2):]
+        assert np.all(np.diff(top, axis=0) > 0)
+    _expand_given(ctx, Ps, beam, n_sent, max_len=8)

@@ -35,7 +35,7 @@ struct zr_beam {
   // per step scratch
   float* d_cand_p;          // [n_sent*beam][beam+1]
   int* d_cand_w;            // [n_sent*beam][beam+1]
-  float* d_part_p;          // [n_sent*beam][kChunks][beam+1] per-chunk candidates
+  float* d_part_p;          // [n_sent*beam][chunks][beam+1] per-chunk candidates of the first top-K stage
   int* d_part_w;
   void* d_block;            // the single allocation behind all of the above
 };
@@ -44,161 +44,185 @@ namespace {
 
 constexpr int KMAX = 32;  // beam + 1 <= KMAX
 
-// Per-column top-K in two stages.
-// Stage 1 (beam_topk_kernel): grid (kChunks, columns).  A workgroup scans its quarter of the column with 16-byte
-// loads; each thread keeps the K best of its share in registers (sorted, descending; bubble insertion with
-// static indexing, guarded by the thread's current K-th best so the common case is one compare), then K rounds
-// of workgroup arg-max over the thread heads emit the chunk's K best in descending order.
-// Stage 2 (beam_topk_merge_kernel): one wave per column merges the kChunks sorted lists.
-// Order everywhere: larger probability first, equal probabilities by lower word id.
-constexpr int kChunks = 4;
+// Per-column top-K in two stages, both built on one total order: key = (probability as an order-preserving 32-bit
+// pattern) << 32 | (0x7fffffff - word id).  Larger key = larger probability, equal probabilities by lower word id;
+// keys of distinct words are distinct, so there are no ties to break anywhere.  Key 0 marks "no element" (a NaN
+// probability is treated the same way and is never selected).
+//
+// Stage 1 (beam_topk_kernel): grid (chunks, columns).  A workgroup takes up to kTopkChunk consecutive words of a
+// column into registers with 16-byte loads (one pass over HBM, no value-dependent work per element).  The K-th
+// largest of a set of per-thread maxima, tau, is a lower bound of the chunk's K-th largest key, so the chunk's K best
+// are among the elements with key >= tau; those are appended to a list in LDS.  tau is first taken per wave (64
+// broadcast reads from LDS) and the largest of the four used; should the list overflow, tau is recomputed over all 256 maxima:
+// then at most K-1 threads have a maximum above tau, each holds 4*kTopkE4 elements, and one thread's maximum equals
+// tau, so the list cannot exceed (K-1)*4*kTopkE4 + 1 entries whatever the data.  Each listed element then counts the
+// listed keys above its own: that count is its rank, and ranks below K are written out in place.
+// Stage 2 (beam_topk_merge_kernel): one workgroup per column ranks the chunks' K-lists the same way.
+constexpr int kTopkE4 = 16;                        // 16-byte loads per thread
+constexpr int kTopkChunk = 256 * 4 * kTopkE4;      // words per workgroup
+constexpr int kTopkCap = (KMAX - 1) * 4 * kTopkE4 + 64;  // candidate list capacity
+constexpr int kMaxChunks = 64;                     // vocabulary up to kMaxChunks * kTopkChunk words
 
-__device__ __forceinline__ bool better(float pa, int wa, float pb, int wb) { return pa > pb || (pa == pb && wa < wb); }
+__device__ __forceinline__ unsigned long long topk_key(float p, int w) {
+  unsigned u = __float_as_uint(p);
+  u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+  if (p != p) return 0ull;
+  return ((unsigned long long)u << 32) | (unsigned)(0x7fffffff - w);
+}
+__device__ __forceinline__ void topk_unkey(unsigned long long key, float& p, int& w) {
+  if (key == 0ull) {
+    p = -INFINITY;
+    w = 0x7fffffff;
+    return;
+  }
+  unsigned u = (unsigned)(key >> 32);
+  u = (u & 0x80000000u) ? (u & 0x7fffffffu) : ~u;
+  p = __uint_as_float(u);
+  w = 0x7fffffff - (int)(unsigned)(key & 0xffffffffu);
+}
 
 __global__ void __launch_bounds__(256)
-beam_topk_kernel(const float* __restrict__ prob, int V, int K, float* __restrict__ part_p, int* __restrict__ part_w) {
-  __shared__ float s_p[4];
-  __shared__ int s_w[4];
+beam_topk_kernel(const float* __restrict__ prob, int V, int K, int n_chunks, float* __restrict__ part_p,
+                 int* __restrict__ part_w) {
+  __shared__ unsigned long long s_max[256];
+  __shared__ unsigned long long s_cand[kTopkCap];
+  __shared__ unsigned long long s_tau_wave[4];
+  __shared__ unsigned long long s_tau;
+  __shared__ int s_count;
   const int chunk = blockIdx.x;
   const int col = blockIdx.y;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const float* p = prob + (size_t)col * V;
-  // chunk boundaries are multiples of 4 elements so that 16-byte loads stay aligned when V % 4 == 0
-  const int per = (((V + kChunks - 1) / kChunks) + 3) & ~3;
-  const int v_begin = chunk * per;
-  const int v_end = (v_begin + per < V) ? v_begin + per : V;
-  float lp[KMAX];
-  int lw[KMAX];
-#pragma unroll
-  for (int i = 0; i < KMAX; ++i) {
-    lp[i] = -INFINITY;
-    lw[i] = 0x7fffffff;
-  }
-  float kth = -INFINITY;  // this thread's current K-th best
-  auto insert = [&](float x, int xw) {
-    // strict comparison: an equal, earlier (lower id) entry stays in front
-#pragma unroll
-    for (int i = 0; i < KMAX; ++i) {
-      if (i < K) {
-        const bool sw = x > lp[i];
-        const float tp = lp[i];
-        const int tw = lw[i];
-        lp[i] = sw ? x : tp;
-        lw[i] = sw ? xw : tw;
-        x = sw ? tp : x;
-        xw = sw ? tw : xw;
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < KMAX; ++i)
-      if (i == K - 1) kth = lp[i];
-  };
+  const int v_begin = chunk * kTopkChunk;
+  const int v_end = (v_begin + kTopkChunk < V) ? v_begin + kTopkChunk : V;
+  if (tid == 0) s_count = 0;
+  // element e = 4*i + c of this thread is word v_begin + 4*(tid + 256*i) + c; words past the end read as -inf,
+  // and -inf (like NaN) is never selected
+  float x[4 * kTopkE4];
   const bool vec = ((V & 3) == 0) && ((((uintptr_t)prob) & 15u) == 0);
-  if (vec) {
-    for (int v = v_begin + 4 * tid; v < v_end; v += 4 * 256) {
-      const zr_f32x4 q = *(const zr_f32x4*)(p + v);
-      if (q.x > kth) insert(q.x, v);
-      if (q.y > kth) insert(q.y, v + 1);
-      if (q.z > kth) insert(q.z, v + 2);
-      if (q.w > kth) insert(q.w, v + 3);
-    }
-  } else {
-    for (int v = v_begin + tid; v < v_end; v += 256) {
-      const float x = p[v];
-      if (x > kth) insert(x, v);
+#pragma unroll
+  for (int i = 0; i < kTopkE4; ++i) {
+    const int v = v_begin + 4 * (tid + 256 * i);
+    if (vec) {
+      const bool ok = v + 3 < v_end;
+      const zr_f32x4 q = *(const zr_f32x4*)(p + (ok ? v : 0));
+      x[4 * i] = ok ? q.x : -INFINITY;
+      x[4 * i + 1] = ok ? q.y : -INFINITY;
+      x[4 * i + 2] = ok ? q.z : -INFINITY;
+      x[4 * i + 3] = ok ? q.w : -INFINITY;
+    } else {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const float q = p[v + c < v_end ? v + c : 0];
+        x[4 * i + c] = v + c < v_end ? q : -INFINITY;
+      }
     }
   }
-  int head = 0;  // index of this thread's best unconsumed entry
-  for (int r = 0; r < K; ++r) {
-    float hp = -INFINITY;
-    int hw = 0x7fffffff;
+  // this thread's best element: words are visited in ascending order, so a strict comparison keeps the lowest id
+  float bm = -INFINITY;
+  int bv = 0x7fffffff;
 #pragma unroll
-    for (int i = 0; i < KMAX; ++i)
-      if (i == head) {
-        hp = lp[i];
-        hw = lw[i];
-      }
-    float bp = hp;
-    int bw = hw;
+  for (int i = 0; i < kTopkE4; ++i)
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-      const float op = __shfl_xor(bp, off, 64);
-      const int ow = __shfl_xor(bw, off, 64);
-      if (better(op, ow, bp, bw)) {
-        bp = op;
-        bw = ow;
+    for (int c = 0; c < 4; ++c)
+      if (x[4 * i + c] > bm) {
+        bm = x[4 * i + c];
+        bv = v_begin + 4 * (tid + 256 * i) + c;
       }
+  const unsigned long long mine = bm > -INFINITY ? topk_key(bm, bv) : 0ull;
+  s_max[tid] = mine;
+  __syncthreads();
+  // First bound: the K-th largest maximum inside each wave (its 64 entries of s_max, broadcast reads), then the
+  // largest of the four.
+  {
+    const unsigned long long* wmax = s_max + 64 * wave;
+    int rank = 0;
+#pragma unroll 16
+    for (int j = 0; j < 64; ++j) {
+      const unsigned long long o = wmax[j];
+      rank += (o > mine || (o == mine && j < lane)) ? 1 : 0;
     }
-    if (lane == 0) {
-      s_p[wave] = bp;
-      s_w[wave] = bw;
+    if (rank == K - 1) s_tau_wave[wave] = mine;
+  }
+  __syncthreads();
+  unsigned long long tau = s_tau_wave[0];
+#pragma unroll
+  for (int w = 1; w < 4; ++w) tau = s_tau_wave[w] > tau ? s_tau_wave[w] : tau;
+  auto collect = [&](unsigned long long t) {
+    if (mine >= t && mine != 0ull) {
+      float tp;
+      int tw;
+      topk_unkey(t, tp, tw);
+#pragma unroll
+      for (int i = 0; i < kTopkE4; ++i)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const float q = x[4 * i + c];
+          if (q >= tp) {  // rare: the full test and the append sit behind one comparison per element
+            const int v = v_begin + 4 * (tid + 256 * i) + c;
+            if (q > -INFINITY && (q > tp || v <= tw)) {
+              const int pos = atomicAdd(&s_count, 1);
+              if (pos < kTopkCap) s_cand[pos] = topk_key(q, v);
+            }
+          }
+        }
     }
+  };
+  collect(tau);
+  __syncthreads();
+  if (s_count > kTopkCap) {
+    // The wave-level bound let too many elements through (possible only when several waves hold threads whose whole
+    // share is large).  The K-th largest of all 256 maxima bounds the list by (K-1) * 4*kTopkE4 + 1 whatever the data.
+    int rank = 0;
+    for (int j = 0; j < 256; ++j) {
+      const unsigned long long o = s_max[j];
+      rank += (o > mine || (o == mine && j < tid)) ? 1 : 0;
+    }
+    if (rank == K - 1) s_tau = mine;
     __syncthreads();
-    float gp = s_p[0];
-    int gw = s_w[0];
-#pragma unroll
-    for (int w = 1; w < 4; ++w)
-      if (better(s_p[w], s_w[w], gp, gw)) {
-        gp = s_p[w];
-        gw = s_w[w];
-      }
-    if (hw == gw && gw != 0x7fffffff) head++;  // word ids are unique: exactly one owner
-    if (tid == 0) {
-      part_p[((size_t)col * kChunks + chunk) * K + r] = gp;
-      part_w[((size_t)col * kChunks + chunk) * K + r] = gw;
-    }
+    if (tid == 0) s_count = 0;
     __syncthreads();
+    collect(s_tau);
+    __syncthreads();
+  }
+  const int n = s_count < kTopkCap ? s_count : kTopkCap;
+  float* out_p = part_p + ((size_t)col * n_chunks + chunk) * K;
+  int* out_w = part_w + ((size_t)col * n_chunks + chunk) * K;
+  for (int a = tid; a < n; a += 256) {
+    const unsigned long long ka = s_cand[a];
+    int rank = 0;
+#pragma unroll 8
+    for (int b = 0; b < n; ++b) rank += s_cand[b] > ka ? 1 : 0;
+    if (rank < K) topk_unkey(ka, out_p[rank], out_w[rank]);
+  }
+  if (tid < K && tid >= n) {  // fewer than K words in the chunk
+    out_p[tid] = -INFINITY;
+    out_w[tid] = 0x7fffffff;
   }
 }
 
-__global__ void __launch_bounds__(64)
-beam_topk_merge_kernel(const float* __restrict__ part_p, const int* __restrict__ part_w, int K,
+__global__ void __launch_bounds__(256)
+beam_topk_merge_kernel(const float* __restrict__ part_p, const int* __restrict__ part_w, int K, int n_chunks,
                        float* __restrict__ cand_p, int* __restrict__ cand_w) {
+  __shared__ unsigned long long s_key[kMaxChunks * KMAX];
   const int col = blockIdx.x;
-  const int lane = threadIdx.x;
-  const int n = kChunks * K;  // <= 128: two entries per lane
-  float p0 = -INFINITY, p1 = -INFINITY;
-  int w0 = 0x7fffffff, w1 = 0x7fffffff;
-  if (lane < n) {
-    p0 = part_p[(size_t)col * n + lane];
-    w0 = part_w[(size_t)col * n + lane];
-  }
-  if (lane + 64 < n) {
-    p1 = part_p[(size_t)col * n + lane + 64];
-    w1 = part_w[(size_t)col * n + lane + 64];
-  }
-  for (int r = 0; r < K; ++r) {
-    float bp = p0;
-    int bw = w0;
-    if (better(p1, w1, bp, bw)) {
-      bp = p1;
-      bw = w1;
+  const int tid = threadIdx.x;
+  const int n = n_chunks * K;
+  for (int a = tid; a < n; a += 256)
+    s_key[a] = topk_key(part_p[(size_t)col * n + a], part_w[(size_t)col * n + a]);  // (-inf, 0x7fffffff) -> lowest
+  __syncthreads();
+  for (int a = tid; a < n; a += 256) {
+    const unsigned long long ka = s_key[a];
+    int rank = 0;
+#pragma unroll 8
+    for (int b = 0; b < n; ++b) {
+      const unsigned long long kb = s_key[b];
+      rank += (kb > ka || (kb == ka && b < a)) ? 1 : 0;  // fillers share one key: order them by position
     }
-    const float mine_p = bp;
-    const int mine_w = bw;
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-      const float op = __shfl_xor(bp, off, 64);
-      const int ow = __shfl_xor(bw, off, 64);
-      if (better(op, ow, bp, bw)) {
-        bp = op;
-        bw = ow;
-      }
-    }
-    if (mine_w == bw && bw != 0x7fffffff) {  // the owner retires the winner
-      if (w0 == bw) {
-        p0 = -INFINITY;
-        w0 = 0x7fffffff;
-      } else {
-        p1 = -INFINITY;
-        w1 = 0x7fffffff;
-      }
-    }
-    (void)mine_p;
-    if (lane == 0) {
-      cand_p[(size_t)col * K + r] = bp;
-      cand_w[(size_t)col * K + r] = bw;
+    if (rank < K) {
+      cand_p[(size_t)col * K + rank] = part_p[(size_t)col * n + a];
+      cand_w[(size_t)col * K + rank] = part_w[(size_t)col * n + a];
     }
   }
 }
@@ -215,6 +239,9 @@ beam_merge_kernel(int beam, int K, int max_len, int hyp_cap, float penalty, int 
   __shared__ int c_col[MAXC];
   __shared__ int c_word[MAXC];
   __shared__ int c_order[MAXC];
+  // one sortable key per candidate: value (order-preserving bit pattern) above, then (column, rank within column)
+  // inverted, so that a larger key comes first and equal values go by (column, better rank)
+  __shared__ unsigned long long c_key[MAXC];
   __shared__ int s_ncand;
   __shared__ int s_parent[KMAX];   // parent column of each new beam slot (-1: empty-heap filler)
   __shared__ int s_word[KMAX];
@@ -229,35 +256,34 @@ beam_merge_kernel(int beam, int K, int max_len, int hyp_cap, float penalty, int 
   int* st = sent + (size_t)s * beam * max_len;
   int* stt = sent_tmp + (size_t)s * beam * max_len;
 
-  if (tid == 0) {
-    // live columns: all of them, or column 0 only at the first step; stop at the first dead slot (:1188-1191)
-    int cols = (index == 0) ? 1 : beam;
-    int n = 0;
-    for (int i = 0; i < cols; ++i) {
-      if (wd[i] == -1) break;
-      // the reference pops its per-column heap in ascending probability and pushes into the global heap
-      for (int r = K - 1; r >= 0; --r) {
-        const size_t ci = ((size_t)s * beam + i) * K + r;
-        c_val[n] = logf(cand_p[ci]) + sc[i];
-        c_col[n] = i;
-        c_word[n] = cand_w[ci];
-        ++n;
-      }
-    }
-    s_ncand = n;
+  // live columns: all of them, or column 0 only at the first step; stop at the first dead slot (:1188-1191)
+  if (tid < 64) {  // beam < 64: one ballot over the slots finds the first dead one
+    const int all = (index == 0) ? 1 : beam;
+    const unsigned long long dead = __ballot(tid < all && wd[tid] == -1);
+    if (tid == 0) s_ncand = (dead ? __builtin_ctzll(dead) : all) * K;
+  }
+  __syncthreads();
+  const int live = s_ncand / K;
+  // candidate a = i*K + q of live column i: the reference pops its per-column heap in ascending probability and
+  // pushes into the global heap, so q counts ranks from the worst (rank K-1) to the best (rank 0)
+  for (int a = tid; a < live * K; a += 256) {
+    const int i = a / K, r = K - 1 - a % K;
+    const size_t ci = ((size_t)s * beam + i) * K + r;
+    c_val[a] = logf(cand_p[ci]) + sc[i];
+    c_col[a] = i;
+    c_word[a] = cand_w[ci];
+    unsigned u = __float_as_uint(c_val[a]);
+    u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+    c_key[a] = ((unsigned long long)u << 32) | (unsigned)(0x7fffffff - (i * K + r));
   }
   __syncthreads();
   const int n = s_ncand;
-  // rank = number of candidates that come before this one: larger value first, then (column, better rank)
+  // rank = number of candidates that come before this one
   for (int a = tid; a < n; a += 256) {
-    const float va = c_val[a];
-    const int ka = c_col[a] * K + (K - 1 - (a % K));  // (column, rank within column) key
+    const unsigned long long ka = c_key[a];
     int rank = 0;
-    for (int b = 0; b < n; ++b) {
-      const float vb = c_val[b];
-      const int kb = c_col[b] * K + (K - 1 - (b % K));
-      if (vb > va || (vb == va && kb < ka)) ++rank;
-    }
+#pragma unroll 8
+    for (int b = 0; b < n; ++b) rank += c_key[b] > ka ? 1 : 0;
     c_order[rank] = a;
   }
   __syncthreads();
@@ -302,34 +328,25 @@ beam_merge_kernel(int beam, int K, int max_len, int hyp_cap, float penalty, int 
       hyp_score[(size_t)s * hyp_cap + h] = s_fin_score[f];
     }
   }
-  // new beam rows
-  for (int i = 0; i < beam; ++i) {
+  // new beam rows into the other sentence buffer (the host swaps the two after the launch): slot i continues its
+  // parent's words [0, current_index] with its own word.  One flat loop over (slot, position), so that the loads of
+  // all rows are in flight together; positions past current_index + 1 are never read.
+  const int lim = current_index + 2 < max_len ? current_index + 2 : max_len;
+  for (int e = tid; e < beam * lim; e += 256) {
+    const int i = e / lim, c = e % lim;
     const int parent = s_parent[i];
-    const int* src = st + (size_t)(parent < 0 ? 0 : parent) * max_len;
-    int* dst = stt + (size_t)i * max_len;
-    for (int c = tid; c < max_len; c += 256) {
-      int v = src[c];
-      if (c == current_index + 1) v = (parent < 0) ? 0 : s_word[i];
-      dst[c] = v;
-    }
+    int v = st[(size_t)(parent < 0 ? 0 : parent) * max_len + c];
+    if (c == current_index + 1) v = (parent < 0) ? 0 : s_word[i];
+    stt[(size_t)i * max_len + c] = v;
   }
-  __syncthreads();
   if (tid < beam) {
     const int parent = s_parent[tid];
-    scores_tmp[(size_t)s * beam + tid] = s_score[tid];
     out_words[(size_t)s * beam + tid] = s_word[tid];
     out_backptr[(size_t)s * beam + tid] = s * beam + (parent < 0 ? 0 : parent);
-  }
-  __syncthreads();
-  if (tid < beam) {
-    sc[tid] = scores_tmp[(size_t)s * beam + tid];
+    sc[tid] = s_score[tid];  // s_score was filled from the old scores before the last barrier
     wd[tid] = s_word[tid];
   }
-  if (tid == 0) {
-    const int total = base + nfin;
-    hyp_count[s] = total;  // may exceed hyp_cap: the host reports the overflow
-  }
-  for (int c = tid; c < beam * max_len; c += 256) st[c] = stt[c];
+  if (tid == 0) hyp_count[s] = base + nfin;  // may exceed hyp_cap: the host reports the overflow
 }
 
 // finish_current_hypotheses, non-FSA branch (src/decoder.h:672-688)
@@ -387,6 +404,7 @@ int zr_beam_create(zr_ctx* ctx, int beam, int vocab, int n_sent, int max_len, fl
   *out = nullptr;
   ZR_CHECK_ARG(beam >= 1 && beam + 1 <= KMAX, "zr_beam_create: beam = %d not in [1, %d]", beam, KMAX - 1);
   ZR_CHECK_ARG(n_sent * beam <= 65535, "zr_beam_create: more than 65535 columns");
+  ZR_CHECK_ARG(vocab <= kMaxChunks * kTopkChunk, "zr_beam_create: vocab = %d exceeds %d", vocab, kMaxChunks * kTopkChunk);
   ZR_CHECK_ARG(vocab > beam + 1 && n_sent >= 1 && max_len >= 3, "zr_beam_create: vocab = %d, n_sent = %d, max_len = %d",
                vocab, n_sent, max_len);
   // the reference caps the beam at floor(sqrt(V)) (src/ensemble_factory.hpp:19-21)
@@ -411,7 +429,8 @@ int zr_beam_create(zr_ctx* ctx, int beam, int vocab, int n_sent, int max_len, fl
   const size_t o_hw = take((size_t)n_sent * b->hyp_cap * max_len * 4), o_hl = take((size_t)n_sent * b->hyp_cap * 4);
   const size_t o_hs = take((size_t)n_sent * b->hyp_cap * 4), o_hc = take((size_t)n_sent * 4);
   const size_t o_cp = take(nb * K * 4), o_cw = take(nb * K * 4);
-  const size_t o_pp = take(nb * 4 * K * 4), o_pw = take(nb * 4 * K * 4);  // kChunks = 4 lists per column
+  const size_t n_chunks = ((size_t)vocab + kTopkChunk - 1) / kTopkChunk;  // K-lists per column from the first stage
+  const size_t o_pp = take(nb * n_chunks * K * 4), o_pw = take(nb * n_chunks * K * 4);
   char* base = nullptr;
   if (hipMalloc((void**)&base, off) != hipSuccess) {
     (void)hipGetLastError();
@@ -464,11 +483,12 @@ int zr_beam_expand(zr_ctx* ctx, zr_beam* b, const float* d_prob, int index, int*
   ZR_CHECK_ARG(index >= 0, "zr_beam_expand: index = %d", index);
   ZR_CHECK_ARG(b->current_index + 2 < b->max_len, "zr_beam_expand: hypotheses reached max_len = %d", b->max_len);
   const int K = b->beam + 1;
-  dim3 tgrid(kChunks, b->n_sent * b->beam);
-  beam_topk_kernel<<<tgrid, 256, 0, ctx->stream>>>(d_prob, b->vocab, K, b->d_part_p, b->d_part_w);
+  const int n_chunks = (b->vocab + kTopkChunk - 1) / kTopkChunk;
+  dim3 tgrid(n_chunks, b->n_sent * b->beam);
+  beam_topk_kernel<<<tgrid, 256, 0, ctx->stream>>>(d_prob, b->vocab, K, n_chunks, b->d_part_p, b->d_part_w);
   ZR_LAUNCH_CHECK("beam_topk_kernel");
-  beam_topk_merge_kernel<<<b->n_sent * b->beam, 64, 0, ctx->stream>>>(b->d_part_p, b->d_part_w, K, b->d_cand_p,
-                                                                      b->d_cand_w);
+  beam_topk_merge_kernel<<<b->n_sent * b->beam, 256, 0, ctx->stream>>>(b->d_part_p, b->d_part_w, K, n_chunks,
+                                                                       b->d_cand_p, b->d_cand_w);
   ZR_LAUNCH_CHECK("beam_topk_merge_kernel");
   beam_merge_kernel<<<b->n_sent, 256, 0, ctx->stream>>>(b->beam, K, b->max_len, b->hyp_cap, b->penalty, index,
                                                         b->current_index, b->d_cand_p, b->d_cand_w, b->d_scores,
@@ -476,6 +496,9 @@ int zr_beam_expand(zr_ctx* ctx, zr_beam* b, const float* d_prob, int index, int*
                                                         b->d_hyp_words, b->d_hyp_len, b->d_hyp_score, b->d_hyp_count,
                                                         d_words, d_backptr);
   ZR_LAUNCH_CHECK("beam_merge_kernel");
+  int* t = b->d_sent;  // the kernel wrote the new rows into d_sent_tmp
+  b->d_sent = b->d_sent_tmp;
+  b->d_sent_tmp = t;
   b->current_index += 1;
   return ZR_OK;
 }
