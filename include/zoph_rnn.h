@@ -220,6 +220,12 @@ int zr_attn_step(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, const float* 
 /* swap_states_decoding (src/Input_To_Hidden_Layer.hpp:1231-1242, src/Hidden_To_Hidden_Layer.hpp:780-791):
  * d_dst[:,i] = d_src[:, d_perm[i]] for i < n; d_dst must not alias d_src. */
 int zr_gather_columns(zr_ctx* ctx, const float* d_src, int H, const int* d_perm, int n, float* d_dst);
+/* The same reorder for n_arrays (<= 32) matrices of H rows in one launch: neuralMT_model::swap_decoding_states
+ * (src/model.hpp:2704-2726) calls swap_states_decoding once per layer for h and c and reorders h~; each of those is
+ * a sub-microsecond copy, so they share a kernel.  d_perm[i] must lie in [0, n_src_cols) (checked on the device,
+ * reported by zr_ctx_sync). */
+int zr_gather_columns_multi(zr_ctx* ctx, int n_arrays, const float* const d_src[], int H, const int* d_perm,
+                            int n_src_cols, int n, float* const d_dst[]);
 /* transfer_decoding_states_GPU (src/Input_To_Hidden_Layer.hpp:1252-1266): one column to n columns. */
 int zr_broadcast_column(zr_ctx* ctx, const float* d_src_col, int H, int n, float* d_dst);
 

@@ -71,6 +71,19 @@ def test_decoder_state_shuffles(ctx):
     ctx.broadcast_column(ctx.array(src[:, [4]]), 1000, 12, d_dst)
     ctx.sync()
     assert np.array_equal(d_dst.get(), np.repeat(src[:, [4]], 12, axis=1))
+    # every state matrix of a decode step in one launch: bit-equal to one gather per matrix
+    for Hh in (1000, 50, 33):  # 16-byte path, and two heights that take the scalar path
+        srcs = [U(g, (Hh, 12)) for _ in range(9)]
+        dsts = [ctx.empty((Hh, 12)) for _ in range(9)]
+        ctx.gather_columns_multi([ctx.array(a) for a in srcs], Hh, ctx.array(perm), 12, 12, dsts)
+        ctx.sync()
+        for a, d in zip(srcs, dsts):
+            assert d.get().tobytes() == o.gather_columns(a, perm).tobytes()
+    bad = ctx.array(np.array([0, 12, 3], np.int32))  # 12 is out of range: clamped, reported at the next sync
+    ctx.gather_columns_multi([ctx.array(srcs[0])], 33, bad, 12, 3, [ctx.empty((33, 3))])
+    with pytest.raises(capi.ZrError):
+        ctx.sync()
+    ctx.sync()
 
 
 # ------------------------------------------------------------------------------------------------ A3 contraction

@@ -33,7 +33,7 @@ SYMBOLS = [
     "zr_lstm_stack_forward_train", "zr_lstm_train_create", "zr_lstm_train_refresh", "zr_lstm_train_destroy",
     "zr_unstack_gates", "zr_lstm_stack_backward", "zr_lstm_weight_gradients", "zr_embed_gradient",
     "zr_softmax_backward", "zr_sgd_update", "zr_lstm_node_backward", "zr_lstm_node_gradients",
-    "zr_softmax_backward_accumulate",
+    "zr_softmax_backward_accumulate", "zr_gather_columns_multi",
 ]
 
 _lib = None
@@ -312,6 +312,10 @@ class Context:
     # ---- A12
     def gather_columns(self, d_src, H, d_perm, n, d_dst):
         _chk(load().zr_gather_columns(self.h, _vp(d_src), C.c_int(H), _vp(d_perm), C.c_int(n), _vp(d_dst)))
+
+    def gather_columns_multi(self, srcs, H, d_perm, n_src_cols, n, dsts):
+        _chk(load().zr_gather_columns_multi(self.h, C.c_int(len(srcs)), _ptr_array(srcs), C.c_int(H), _vp(d_perm),
+                                            C.c_int(n_src_cols), C.c_int(n), _ptr_array(dsts)))
 
     def broadcast_column(self, d_src_col, H, n, d_dst):
         _chk(load().zr_broadcast_column(self.h, _vp(d_src_col), C.c_int(H), C.c_int(n), _vp(d_dst)))

@@ -74,6 +74,33 @@ column_copy_kernel(const float* __restrict__ src, int H, int V, const int* __res
   }
 }
 
+// The same copy for up to kMaxMulti arrays at once (blockIdx.z picks the array): the per-layer state reorders of a
+// decode step are each far too small to fill the chip, so they share one launch.
+constexpr int kMaxMulti = 32;
+struct MultiCopy {
+  const float* src[kMaxMulti];
+  float* dst[kMaxMulti];
+};
+template <bool VEC>
+__global__ void __launch_bounds__(64)
+multi_column_copy_kernel(MultiCopy a, int H, const int* __restrict__ col_ids, int n_src_cols, int* __restrict__ flags) {
+  const int col = blockIdx.y;
+  int sc = col_ids[col];
+  if (sc < 0 || sc >= n_src_cols) {
+    if (threadIdx.x == 0 && blockIdx.x == 0 && blockIdx.z == 0) atomicAdd(&flags[0], 1);
+    sc = sc < 0 ? 0 : n_src_cols - 1;
+  }
+  const float* s = a.src[blockIdx.z] + (size_t)sc * H;
+  float* d = a.dst[blockIdx.z] + (size_t)col * H;
+  if (VEC) {
+    const int i4 = blockIdx.x * 64 + threadIdx.x;
+    if (i4 * 4 < H) ((zr_f32x4*)d)[i4] = ((const zr_f32x4*)s)[i4];
+  } else {
+    const int i = blockIdx.x * 64 + threadIdx.x;
+    if (i < H) d[i] = s[i];
+  }
+}
+
 // Fused gate kernel: the reference's forward_sigmoid_kernel x3, forward_tanh_kernel, forward_c_t_kernel,
 // clip_mat_kernel, forward_h_t_kernel and zero_c_t_and_h_t (src/custom_kernels.h:58-192, 2222-2231) in one
 // pass: 4 pre-activation reads + c_prev read, c and h written once.
@@ -212,6 +239,38 @@ int zr_gather_columns(zr_ctx* ctx, const float* d_src, int H, const int* d_perm,
   ZR_CHECK_ARG(n == 0 || d_perm, "zr_gather_columns: d_perm is null");
   ZR_CHECK_ARG(d_src != d_dst || n == 0, "zr_gather_columns: d_dst must not alias d_src");
   return column_copy(ctx, "zr_gather_columns", d_src, H, 0, d_perm, 0, n, d_dst);
+}
+
+int zr_gather_columns_multi(zr_ctx* ctx, int n_arrays, const float* const d_src[], int H, const int* d_perm,
+                            int n_src_cols, int n, float* const d_dst[]) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(n_arrays >= 0 && n_arrays <= kMaxMulti, "zr_gather_columns_multi: %d arrays (at most %d)", n_arrays,
+               kMaxMulti);
+  ZR_CHECK_ARG(H > 0 && n >= 0 && n <= 65535 && n_src_cols > 0, "zr_gather_columns_multi: H = %d, n = %d, %d source columns",
+               H, n, n_src_cols);
+  if (n_arrays == 0 || n == 0) return ZR_OK;
+  ZR_CHECK_ARG(d_src && d_dst && d_perm, "zr_gather_columns_multi: null pointer");
+  MultiCopy a;
+  bool vec = H % 4 == 0;
+  for (int i = 0; i < kMaxMulti; ++i) {
+    a.src[i] = i < n_arrays ? d_src[i] : nullptr;
+    a.dst[i] = i < n_arrays ? d_dst[i] : nullptr;
+    if (i < n_arrays) {
+      ZR_CHECK_ARG(d_src[i] && d_dst[i], "zr_gather_columns_multi: array %d is null", i);
+      ZR_CHECK_ARG(d_src[i] != d_dst[i], "zr_gather_columns_multi: array %d: d_dst must not alias d_src", i);
+      vec = vec && aligned16(d_src[i]) && aligned16(d_dst[i]);
+    }
+  }
+  if (vec) {
+    dim3 grid((H / 4 + 63) / 64, n, n_arrays);
+    multi_column_copy_kernel<true><<<grid, 64, 0, ctx->stream>>>(a, H, d_perm, n_src_cols, ctx->d_flags);
+  } else {
+    dim3 grid((H + 63) / 64, n, n_arrays);
+    multi_column_copy_kernel<false><<<grid, 64, 0, ctx->stream>>>(a, H, d_perm, n_src_cols, ctx->d_flags);
+  }
+  ZR_LAUNCH_CHECK("multi_column_copy_kernel");
+  return ZR_OK;
 }
 
 int zr_broadcast_column(zr_ctx* ctx, const float* d_src_col, int H, int n, float* d_dst) {

@@ -118,10 +118,8 @@ class BeamDecode:
         # swap_decoding_states + target_copy_prev_states (src/model.hpp:2691-2726): the new state, permuted, becomes
         # the previous state of the next step
         p, q = self.cur, 1 - self.cur
-        for l in range(L):
-            ctx.gather_columns(self.h[q][l], H, self.d_back, cols, self.h[p][l])
-            ctx.gather_columns(self.c[q][l], H, self.d_back, cols, self.c[p][l])
-        ctx.gather_columns(self.h_tild[q], H, self.d_back, cols, self.h_tild[p])
+        ctx.gather_columns_multi(self.h[q] + self.c[q] + [self.h_tild[q]], H, self.d_back, cols, cols,
+                                 self.h[p] + self.c[p] + [self.h_tild[p]])
         self.step_index += 1
         if record:
             ctx.sync()

@@ -1007,11 +1007,15 @@ class beam_decoder {
       ZOPH_CALL(zr_beam_expand(ctx, bm, prob, index, d_words, d_back));
       // swap_decoding_states + target_copy_prev_states (src/model.hpp:2691-2726)
       const int q = 1 - p;
-      for (int l = 0; l < L; l++) {
-        ZOPH_CALL(zr_gather_columns(ctx, h[q][l], H, d_back, cols, h[p][l]));
-        ZOPH_CALL(zr_gather_columns(ctx, c[q][l], H, d_back, cols, c[p][l]));
+      std::vector<const dType*> from(h[q].begin(), h[q].end());
+      from.insert(from.end(), c[q].begin(), c[q].end());
+      std::vector<dType*> to(h[p].begin(), h[p].end());
+      to.insert(to.end(), c[p].begin(), c[p].end());
+      if (attention) {
+        from.push_back(h_tild[q]);
+        to.push_back(h_tild[p]);
       }
-      if (attention) ZOPH_CALL(zr_gather_columns(ctx, h_tild[q], H, d_back, cols, h_tild[p]));
+      ZOPH_CALL(zr_gather_columns_multi(ctx, (int)from.size(), from.data(), H, d_back, cols, cols, to.data()));
     }
     // one last step and forced <EOF> on every live hypothesis (src/ensemble_factory.hpp:727-743)
     forward_target(p, index);
