@@ -28,9 +28,9 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E peak
 
 # HBM bytes per full-diagonal launch of lstm_fused_kernel on the headline workload, from two rocprofv3 --pmc runs
 # (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for a plain copy of
-# known size (bench.py --calibrate-copy): FETCH_SIZE 69122.6 KiB x 1.9704 + WRITE_SIZE 6000.0 KiB x 1.0000.
+# known size (bench.py --calibrate-copy): FETCH_SIZE 69128.2 KiB x 1.9707 + WRITE_SIZE 6000.0 KiB x 1.0000.
 # The summary of those runs is profiles/lstm_fused_kernel_config2_hbm_traffic.txt.
-LSTM_FUSED_FULL_DIAGONAL_TRAFFIC_BYTES = int((69122.6 * 1.9704 + 6000.0 * 1.0) * 1024)
+LSTM_FUSED_FULL_DIAGONAL_TRAFFIC_BYTES = int((69128.2 * 1.9707 + 6000.0 * 1.0) * 1024)
 
 
 def log(*a):
@@ -296,6 +296,31 @@ def bench_beam_decode(ctx, steps, H=1000, L=4, beam=12, n_sent=16, S=50, V=50000
     return res
 
 
+def vendor_sgemm_reference(iters=50):
+    """Not part of the product path: times the vendor library's fp32 GEMM (through torch.bmm) on the shapes of the two
+    main products -- the four node products of a full encoder diagonal and the config-3 output-layer logits -- as a
+    yardstick for the hand-written kernels, which in addition fuse the gate / cell and the soft-max partial epilogues."""
+    import torch
+    torch.backends.cuda.matmul.allow_tf32 = False
+    out = {}
+    for name, (b, m, n, k) in {"encoder_full_diagonal_4x(4000x128x2000)": (4, 4000, 128, 2000),
+                               "config3_logits_50000x128x1000": (1, 50000, 128, 1000)}.items():
+        a = torch.randn(b, m, k, device="cuda:0", dtype=torch.float32)
+        x = torch.randn(b, k, n, device="cuda:0", dtype=torch.float32)
+        for _ in range(5):
+            torch.bmm(a, x)
+        torch.cuda.synchronize()
+        t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0.record()
+        for _ in range(iters):
+            torch.bmm(a, x)
+        t1.record()
+        torch.cuda.synchronize()
+        us = t0.elapsed_time(t1) * 1e3 / iters
+        out[name] = {"us": round(us, 2), "tflops": round(2.0 * b * m * n * k / us / 1e6, 1)}
+    return out
+
+
 def calibrate_copy(ctx, mbytes=64):
     """Plain copies of known size (identity column gathers: n*H*4 bytes read, n*H*4 bytes written) for scaling the
     FETCH_SIZE / WRITE_SIZE counters: one with 16-byte accesses (H = 1024, column_copy_kernel<true>) and one with
@@ -343,6 +368,8 @@ def main():
     ap.add_argument("--lstm-ks", type=int, default=0)
     ap.add_argument("--training-only", action="store_true",
                     help="only run the language-model training step measurement (for profiling) and exit")
+    ap.add_argument("--vendor-gemm", action="store_true",
+                    help="only time the vendor library's fp32 GEMM on the main products' shapes (a yardstick) and exit")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain copy kernel of known size (for scaling HBM traffic counters) and exit")
     args = ap.parse_args()
@@ -350,6 +377,10 @@ def main():
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (no cross-GPU path exists)" % args.gpus,
               file=sys.stderr)
         sys.exit(2)
+
+    if args.vendor_gemm:
+        print(json.dumps(vendor_sgemm_reference()))
+        return
 
     from zoph_rnn_amd import capi
     ctx = capi.Context(0)

@@ -24,7 +24,6 @@ struct zr_beam {
   int current_index;        // host copy; the reference's decoder::current_index
   // device state, per sentence
   float* d_scores;          // [n_sent][beam]
-  float* d_scores_tmp;
   int* d_words;             // [n_sent][beam] current_indices (-1 = dead slot)
   int* d_sent;              // [n_sent][beam][max_len] top_sentences
   int* d_sent_tmp;
@@ -231,7 +230,7 @@ beam_topk_merge_kernel(const float* __restrict__ part_p, const int* __restrict__
 // src/decoder.h:1214-1315).
 __global__ void __launch_bounds__(256)
 beam_merge_kernel(int beam, int K, int max_len, int hyp_cap, float penalty, int index, int current_index,
-                  const float* __restrict__ cand_p, const int* __restrict__ cand_w, float* scores, float* scores_tmp,
+                  const float* __restrict__ cand_p, const int* __restrict__ cand_w, float* scores,
                   int* words, int* sent, int* sent_tmp, int* hyp_words, int* hyp_len, float* hyp_score,
                   int* hyp_count, int* out_words, int* out_backptr) {
   constexpr int MAXC = KMAX * KMAX;
@@ -424,7 +423,7 @@ int zr_beam_create(zr_ctx* ctx, int beam, int vocab, int n_sent, int max_len, fl
     off += (bytes + 255) & ~(size_t)255;
     return o;
   };
-  const size_t o_scores = take(nb * 4), o_scores_tmp = take(nb * 4), o_words = take(nb * 4);
+  const size_t o_scores = take(nb * 4), o_words = take(nb * 4);
   const size_t o_sent = take(nb * max_len * 4), o_sent_tmp = take(nb * max_len * 4);
   const size_t o_hw = take((size_t)n_sent * b->hyp_cap * max_len * 4), o_hl = take((size_t)n_sent * b->hyp_cap * 4);
   const size_t o_hs = take((size_t)n_sent * b->hyp_cap * 4), o_hc = take((size_t)n_sent * 4);
@@ -439,7 +438,6 @@ int zr_beam_create(zr_ctx* ctx, int beam, int vocab, int n_sent, int max_len, fl
   }
   b->d_block = base;
   b->d_scores = (float*)(base + o_scores);
-  b->d_scores_tmp = (float*)(base + o_scores_tmp);
   b->d_words = (int*)(base + o_words);
   b->d_sent = (int*)(base + o_sent);
   b->d_sent_tmp = (int*)(base + o_sent_tmp);
@@ -492,7 +490,7 @@ int zr_beam_expand(zr_ctx* ctx, zr_beam* b, const float* d_prob, int index, int*
   ZR_LAUNCH_CHECK("beam_topk_merge_kernel");
   beam_merge_kernel<<<b->n_sent, 256, 0, ctx->stream>>>(b->beam, K, b->max_len, b->hyp_cap, b->penalty, index,
                                                         b->current_index, b->d_cand_p, b->d_cand_w, b->d_scores,
-                                                        b->d_scores_tmp, b->d_words, b->d_sent, b->d_sent_tmp,
+                                                        b->d_words, b->d_sent, b->d_sent_tmp,
                                                         b->d_hyp_words, b->d_hyp_len, b->d_hyp_score, b->d_hyp_count,
                                                         d_words, d_backptr);
   ZR_LAUNCH_CHECK("beam_merge_kernel");

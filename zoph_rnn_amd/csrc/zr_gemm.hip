@@ -219,8 +219,6 @@ __global__ void __launch_bounds__(64 * KS * WPB, OCC) gemm_kernel(GemmArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction
   const int kslice = wave % KS;
   const int sub = wave / KS;  // which wave tile of the workgroup
-  const int jl = lane & 31;
-  const int half = lane >> 5;
   const int z = blockIdx.z;
 
   long long tile = (long long)blockIdx.x * WPB + sub;
