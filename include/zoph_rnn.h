@@ -327,6 +327,12 @@ int zr_embed_gradient(zr_ctx* ctx, int H, int V, const float* d_err, const int* 
 int zr_softmax_backward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int n,
                         const int* d_target, const int* d_mask01, float* d_prob_scratch, float* d_err_h, float* d_dD,
                         float* d_db);
+/* The same plus the minibatch's log-likelihood, sum over unmasked columns of log((double) p[target]) as the
+ * reference's train_perplexity_kernel forms it from the float probabilities (src/custom_kernels.h:478-488,
+ * src/softmax.hpp:616-619): no second logits product for the loss.  Waits for the stream (h_loss is host memory). */
+int zr_softmax_backward_loss(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int n,
+                             const int* d_target, const int* d_mask01, float* d_prob_scratch, float* d_err_h,
+                             float* d_dD, float* d_db, double* h_loss);
 /* The same with d_dD and d_db ADDED to: one call per time step (softmax_layer::back_prop1 / back_prop2,
  * src/softmax.hpp:600-700), gradients zeroed at the start of the minibatch. */
 int zr_softmax_backward_accumulate(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h,

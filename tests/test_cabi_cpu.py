@@ -61,6 +61,8 @@ def test_null_context_and_bad_arguments_return_errors():
                                      None) == -1
     assert lib.zr_lstm_node_gradients(None, 8, 1, None, None, None, None, None, None) == -1
     assert lib.zr_gather_columns_multi(None, 1, None, 8, None, 4, 4, None) == -1
+    assert lib.zr_softmax_backward_loss(None, None, None, 8, 8, None, 1, None, None, None, None, None, None,
+                                        None) == -1
     assert lib.zr_softmax_backward_accumulate(None, None, None, 8, 8, None, 1, None, None, None, None, None,
                                               None) == -1
 

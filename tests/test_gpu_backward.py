@@ -127,6 +127,12 @@ def test_softmax_backward(ctx, V, H, n):
     assert_close(d_dD.get(), want_dD, floor=0.05 * np.sqrt(n), what="dD")
     assert_close(d_db.get(), want_db, floor=0.05 * np.sqrt(n), what="db")
     assert np.all(d_eh.get()[:, mask == 0] == 0)
+    # the variant that also returns the log-likelihood of the columns, formed from the float probabilities
+    loss = ctx.softmax_backward_loss(ctx.array(D), ctx.array(bd), V, H, ctx.array(h), n, ctx.array(target),
+                                     ctx.array(mask), d_scr, d_eh, d_dD, d_db)
+    want_loss = o.softmax_loss(o.softmax_logprob_f64(o.softmax_logits(D, bd, h)), target, mask)
+    assert loss == pytest.approx(want_loss, rel=1e-5, abs=1e-5)
+    assert_close(d_dD.get(), want_dD, floor=0.05 * np.sqrt(n), what="dD (loss variant)")
 
 
 @pytest.mark.parametrize("n,clip", [(1000, 0.0), (100000, 5.0), (100000, 1e6), (37, 0.5)])

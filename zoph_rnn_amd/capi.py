@@ -33,7 +33,7 @@ SYMBOLS = [
     "zr_lstm_stack_forward_train", "zr_lstm_train_create", "zr_lstm_train_refresh", "zr_lstm_train_destroy",
     "zr_unstack_gates", "zr_lstm_stack_backward", "zr_lstm_weight_gradients", "zr_embed_gradient",
     "zr_softmax_backward", "zr_sgd_update", "zr_lstm_node_backward", "zr_lstm_node_gradients",
-    "zr_softmax_backward_accumulate", "zr_gather_columns_multi",
+    "zr_softmax_backward_accumulate", "zr_gather_columns_multi", "zr_softmax_backward_loss",
 ]
 
 _lib = None
@@ -264,6 +264,14 @@ class Context:
         fn = load().zr_softmax_backward_accumulate if accumulate else load().zr_softmax_backward
         _chk(fn(self.h, _vp(d_D), _vp(d_b), C.c_int(V), C.c_int(H), _vp(d_h), C.c_int(n),
                                         _vp(d_target), _vp(d_mask), _vp(d_scratch), _vp(d_err_h), _vp(d_dD), _vp(d_db)))
+
+    def softmax_backward_loss(self, d_D, d_b, V, H, d_h, n, d_target, d_mask, d_scratch, d_err_h, d_dD, d_db):
+        """softmax_backward plus the log-likelihood of the n columns (returned)."""
+        loss = C.c_double(0.0)
+        _chk(load().zr_softmax_backward_loss(self.h, _vp(d_D), _vp(d_b), C.c_int(V), C.c_int(H), _vp(d_h), C.c_int(n),
+                                             _vp(d_target), _vp(d_mask), _vp(d_scratch), _vp(d_err_h), _vp(d_dD),
+                                             _vp(d_db), C.byref(loss)))
+        return loss.value
 
     def sgd_update(self, d_W, d_grad, n, scale, norm_clip, lr):
         _chk(load().zr_sgd_update(self.h, _vp(d_W), _vp(d_grad), C.c_longlong(n), C.c_float(scale), C.c_float(norm_clip),

@@ -89,6 +89,24 @@ __global__ void __launch_bounds__(256) lstm_node_backward_kernel(
   ec_out[ix] = ec * gf;
 }
 
+// Sum over the unmasked columns of log((double) p[target, column]): train_perplexity_kernel
+// (src/custom_kernels.h:478-488), one workgroup, fixed summation order.
+__global__ void __launch_bounds__(256) train_logprob_kernel(const float* __restrict__ prob, int V, int n,
+                                                            const int* __restrict__ target,
+                                                            const int* __restrict__ mask01, double* __restrict__ out) {
+  __shared__ double part[256];
+  double s = 0.0;
+  for (int i = threadIdx.x; i < n; i += 256)
+    if (mask01[i] == 1) s += log((double)prob[(size_t)i * V + target[i]]);
+  part[threadIdx.x] = s;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if ((int)threadIdx.x < w) part[threadIdx.x] += part[threadIdx.x + w];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) out[0] = part[0];
+}
+
 // dst (cols x rows, column-major with leading dimension ldd, starting at row offset row0) = src^T, src rows x cols
 // column-major (ld = rows): dst[row0 + c + r*ldd] = src[r + c*rows].  32 x 32 tiles through LDS.
 __global__ void __launch_bounds__(256) transpose_kernel(const float* __restrict__ src, int rows, int cols,
@@ -480,7 +498,7 @@ int zr_embed_gradient(zr_ctx* ctx, int H, int V, const float* d_err, const int* 
 
 static int softmax_backward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int n,
                             const int* d_target, const int* d_mask01, float* d_prob_scratch, float* d_err_h,
-                            float* d_dD, float* d_db, int accumulate) {
+                            float* d_dD, float* d_db, int accumulate, double* h_loss = nullptr) {
   int rc = zr_bind_device(ctx);
   if (rc) return rc;
   ZR_CHECK_ARG(V > 0 && H > 0 && n > 0 && n <= 65535, "zr_softmax_backward: V = %d, H = %d, n = %d", V, H, n);
@@ -488,16 +506,23 @@ static int softmax_backward(zr_ctx* ctx, const float* d_D, const float* d_b_d, i
                "zr_softmax_backward: null pointer");
   rc = zr_softmax_forward(ctx, d_D, d_b_d, V, H, d_h, n, ZR_SOFTMAX_PROB, d_prob_scratch, nullptr);
   if (rc) return rc;
-  dim3 egrid((V + 255) / 256, n);
-  softmax_error_kernel<<<egrid, 256, 0, ctx->stream>>>(d_prob_scratch, V, d_target, d_mask01);
-  ZR_LAUNCH_CHECK("softmax_error_kernel");
   // err_h = D^T e, computed as (e^T D)^T: with e^T as the left operand the product is tall (n rows) with contiguous
   // rows, the shape the large-matrix kernels are built for; the two transposes move 2 x V*n + 2 x n*H floats.
   void *s0 = nullptr, *s1 = nullptr;
   rc = zr_ctx_scratch(ctx, 1, sizeof(float) * (size_t)V * n, &s1);
   if (rc) return rc;
-  rc = zr_ctx_scratch(ctx, 0, sizeof(float) * (size_t)n * H, &s0);
+  rc = zr_ctx_scratch(ctx, 0, sizeof(float) * (size_t)n * H + sizeof(double), &s0);
   if (rc) return rc;
+  if (h_loss) {
+    // before the probabilities are turned into errors.  The cell is the head of scratch 0; the copy out is queued
+    // ahead of the kernels that reuse that buffer, and waited for at the end of this call.
+    train_logprob_kernel<<<1, 256, 0, ctx->stream>>>(d_prob_scratch, V, n, d_target, d_mask01, (double*)s0);
+    ZR_LAUNCH_CHECK("train_logprob_kernel");
+    ZR_HIP(hipMemcpyAsync(h_loss, s0, sizeof(double), hipMemcpyDeviceToHost, ctx->stream));
+  }
+  dim3 egrid((V + 255) / 256, n);
+  softmax_error_kernel<<<egrid, 256, 0, ctx->stream>>>(d_prob_scratch, V, d_target, d_mask01);
+  ZR_LAUNCH_CHECK("softmax_error_kernel");
   float* et = (float*)s1;   // n x V
   float* ct = (float*)s0;   // n x H
   ZrGemmDesc g = {};
@@ -553,13 +578,24 @@ static int softmax_backward(zr_ctx* ctx, const float* d_D, const float* d_b_d, i
   w.accumulate = accumulate;
   rc = zr_gemm_launch(ctx, w);
   if (rc) return rc;
-  return row_sum_launch(ctx, d_prob_scratch, V, n, d_db, accumulate);
+  rc = row_sum_launch(ctx, d_prob_scratch, V, n, d_db, accumulate);
+  if (rc) return rc;
+  if (h_loss) ZR_HIP(hipStreamSynchronize(ctx->stream));
+  return ZR_OK;
 }
 
 int zr_softmax_backward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int n,
                         const int* d_target, const int* d_mask01, float* d_prob_scratch, float* d_err_h, float* d_dD,
                         float* d_db) {
   return softmax_backward(ctx, d_D, d_b_d, V, H, d_h, n, d_target, d_mask01, d_prob_scratch, d_err_h, d_dD, d_db, 0);
+}
+
+int zr_softmax_backward_loss(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int n,
+                             const int* d_target, const int* d_mask01, float* d_prob_scratch, float* d_err_h,
+                             float* d_dD, float* d_db, double* h_loss) {
+  ZR_CHECK_ARG(h_loss != nullptr, "zr_softmax_backward_loss: h_loss is null");
+  return softmax_backward(ctx, d_D, d_b_d, V, H, d_h, n, d_target, d_mask01, d_prob_scratch, d_err_h, d_dD, d_db, 0,
+                          h_loss);
 }
 
 int zr_softmax_backward_accumulate(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h,

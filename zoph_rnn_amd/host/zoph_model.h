@@ -804,10 +804,9 @@ class model_trainer {
     ZOPH_CALL(zr_h2d(ctx, d_tout, r.h_output_vocab_indicies_target.data(), (size_t)T * mb * sizeof(int)));
     ZOPH_CALL(zr_vocab_prep_softmax(ctx, d_tout, T * mb, Vt, d_tmask, d_tmaskf));
     auto& sm = m.softmax_obj;
-    double loss = 0;
-    ZOPH_CALL(zr_softmax_loss(ctx, sm.d_D, sm.d_b_d, Vt, H, tgt.h_all[L - 1], T * mb, d_tout, d_tmask, prob, &loss));
-    ZOPH_CALL(zr_softmax_backward(ctx, sm.d_D, sm.d_b_d, Vt, H, tgt.h_all[L - 1], T * mb, d_tout, d_tmask, prob, err_top,
-                                  dD, dbd));
+    double loss = 0;  // from the same probabilities the error is formed from (train_perplexity_kernel)
+    ZOPH_CALL(zr_softmax_backward_loss(ctx, sm.d_D, sm.d_b_d, Vt, H, tgt.h_all[L - 1], T * mb, d_tout, d_tmask, prob,
+                                       err_top, dD, dbd, &loss));
     backward_side(tgt, m.input_layer_target, m.target_hidden_layers, T, Vt, th0, tc0, err_top, nullptr, nullptr);
     if (seq2seq) {
       // no attention: the encoder receives error only through its final states
