@@ -395,12 +395,19 @@ __global__ void __launch_bounds__(64 * NWV) gemm_lds_kernel(GemmArgs a) {
 #pragma unroll
     for (int gq = 0; gq < 4; ++gq) {
       if (gq + 1 < 4) lds_frag(wf[(gq + 1) & 1], gq + 1);
-      __builtin_amdgcn_sched_barrier(0);  // keep the LDS reads ahead of the MFMAs that consume them
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int tm = 0; tm < TMR; ++tm)
           acc[tm] = __builtin_amdgcn_mfma_f32_32x32x2f32(xs[gq][i], wf[gq & 1][i][tm], acc[tm], 0, 0, 0);
+      // issue order within this group: one LDS read of the next fragment behind each MFMA, so that the reads hide
+      // under the matrix pipe instead of stalling it in a burst (and never slide down to just before their use)
+#pragma unroll
+      for (int j = 0; j < 4 * TMR; ++j) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
 

@@ -161,6 +161,9 @@ int logits_with_partials(zr_ctx* ctx, const float* d_D, const float* d_b_d, int 
   for (int i = 0; i < ZR_MAX_PACKED_D; ++i) {
     const zr_ctx::PackedD& e = ctx->packed_d[i];
     if (e.key == d_D && e.V == V && e.H == H) {  // registered with zr_softmax_prepare: use the MFMA-layout copy
+      // ... unless the batch is thousands of columns wide (all time steps of a training minibatch at once): there
+      // the LDS-staged kernel on the plain matrix is faster than the register-streaming one on the fp32 copy
+      if (!e.bf16 && mb > 1024) break;
       d.A[0] = (const float*)e.d_pack;
       d.lda[0] = e.ldp;
       d.a_pack = e.bf16 ? 2 : 1;
