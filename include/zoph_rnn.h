@@ -67,8 +67,9 @@ const char* zr_version(void);
                                         12..14 = tiles 128x64, 64x64, 64x128 at one workgroup per CU */
 #define ZR_OPT_LSTM_KSPLIT 4         /* waves per workgroup splitting K in the fused LSTM kernel: 4 or 8 (0 = auto) */
 #define ZR_OPT_LSTM_KERNEL 5         /* 0 auto; 1: weights streamed to registers, K split inside the workgroup;
-                                        2: weights through LDS, K split across workgroups */
-#define ZR_OPT_LSTM_KPARTS 6         /* kernel 2: K parts per weight segment (0 = auto) */
+                                        2: weights through LDS, K split across workgroups;
+                                        3: weights streamed to registers, K split inside and across workgroups */
+#define ZR_OPT_LSTM_KPARTS 6         /* kernels 2 and 3: K parts per weight segment (0 = auto) */
 
 /* full_matrix_setup / cudaMalloc / cudaMemcpy / cudaMemset call sites (src/BZ_CUDA_UTIL.h:358-399 and the
  * layer constructors, e.g. src/LSTM.hpp:23-42). */

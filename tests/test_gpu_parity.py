@@ -530,6 +530,36 @@ def test_lstm_step_lds_split_kernel(ctx, H, mb, kparts):
     assert got_feed["h"].tobytes() == again["h"].tobytes() and got_feed["c"].tobytes() == again["c"].tobytes()
 
 
+@pytest.mark.parametrize("H,mb", [(32, 3), (104, 8), (72, 33), (256, 70), (1000, 128), (64, 150), (1000, 192), (1000, 12)])
+@pytest.mark.parametrize("kparts", [0, 2, 3, 5])
+def test_lstm_step_register_kernel_split_across_workgroups(ctx, H, mb, kparts):
+    """The register-streaming kernel with K divided over several workgroups per tile (H % 8 == 0): column tiles of 32,
+    64 and 96, uneven K parts, partial row and column tiles, two and three weight segments; a request for more parts
+    than k-groups falls back to another kernel and must still be right."""
+    g = synth.rng(19, H * 1000 + mb + kparts)
+    ly = synth.lstm_layer(g, H, feed_input=True, forget_bias_one=True)
+    x, hp, cp, ht = U(g, (H, mb), -1, 1), U(g, (H, mb), -1, 1), U(g, (H, mb), -1, 1), U(g, (H, mb), -1, 1)
+    mask = (g.random(mb) > 0.2).astype(np.int32)
+    layer = Layer(ctx, ly)
+    ctx.set_option(capi.ZR_OPT_LSTM_KERNEL, 3)
+    ctx.set_option(capi.ZR_OPT_LSTM_KPARTS, kparts)
+    try:
+        got = run_lstm_step(ctx, layer, x, hp, cp, mask, want_gates=True)
+        got_feed = run_lstm_step(ctx, layer, x, hp, cp, mask, htild=ht, clip=0.7)
+        again = run_lstm_step(ctx, layer, x, hp, cp, mask, htild=ht, clip=0.7)
+    finally:
+        ctx.set_option(capi.ZR_OPT_LSTM_KERNEL, 0)
+        ctx.set_option(capi.ZR_OPT_LSTM_KPARTS, 0)
+        layer.close()
+    want = o.lstm_step(ly["M"], ly["Wh"], ly["b"], x, hp, cp, mask)
+    want_feed = o.lstm_step(ly["M"], ly["Wh"], ly["b"], x, hp, cp, mask, Q=ly["Q"], htild=ht, clip=0.7)
+    for k in ("i", "f", "c_tilde", "o", "c", "h"):
+        assert_close(got[k], want[k], what="%s (H=%d mb=%d kparts=%d)" % (k, H, mb, kparts))
+    assert_close(got_feed["h"], want_feed["h"], what="feed h")
+    assert_close(got_feed["c"], want_feed["c"], what="feed c")
+    assert got_feed["h"].tobytes() == again["h"].tobytes() and got_feed["c"].tobytes() == again["c"].tobytes()
+
+
 def test_stack_forward_with_split_kernel_forced(ctx):
     g = synth.rng(17, 1)
     H, mb, T, V, L = 64, 5, 7, 211, 3

@@ -46,6 +46,10 @@ struct LstmLaunch {
   float* preact;            // non-null: store the four pre-activation sums ([4][H*mb], no bias) instead of the cell
   float clip;
   int j_tiles, n_tiles;
+  // K split ACROSS workgroups (SPLIT variant of lstm_fused_kernel): blockIdx.y = part of every segment's K range
+  int kparts;
+  float* partials;   // [tile][part][visit][gate][thread]
+  int* counters;     // [tile], zero between launches
 };
 
 // Prefetch distance (k-groups) of the register-streaming kernel: a fragment is 4*(4+TN) registers and 4+TN
@@ -55,13 +59,17 @@ constexpr int lstm_prefetch_depth(int tn, int ks) {
 #ifdef ZR_LSTM_PF
   return ZR_LSTM_PF;
 #else
-  return ks > 4 ? (tn == 1 ? 5 : 2) : (tn == 1 ? 8 : (tn == 2 ? 6 : 1));
+  return ks > 4 ? (tn == 1 ? 5 : 2) : (tn == 1 ? 8 : (tn == 2 ? 6 : (tn == 3 ? 3 : 1)));
 #endif
 }
 
-template <int TN, int KS, bool VEC, bool BF16 = false, bool XPK = false>
+// SPLIT: the K range of every segment is also divided over gridDim.y workgroups (a single node cannot fill the chip
+// with whole-K tiles).  Each writes its tile of partial sums; the last to arrive at the tile's counter adds the parts
+// in part order -- the same order whoever is last, so results do not depend on timing -- and runs the cell epilogue.
+template <int TN, int KS, bool VEC, bool BF16 = false, bool XPK = false, bool SPLIT = false>
 __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
   __shared__ float red[KS * TN * 16 * 64];
+  __shared__ int s_last;
   // Workgroup ids congruent modulo 8 run on the same XCD (round-robin dispatch) and share its L2.  Each XCD gets
   // a contiguous range of (unit, row tile) groups and every column tile of those groups: a weight tile is
   // fetched from memory once however many column tiles read it, and an XCD touches the activations of one or
@@ -170,13 +178,26 @@ __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
         }
         xcol[tn] = (VEC && U.inp[s]) ? U.inp[s] + 4LL * cols[tn] + 4LL * half * L.mb : U.in[s] + c * H + 4 * half;
       }
-      zr_mma_segment<4, TN, KS, lstm_prefetch_depth(TN, KS), ZR_A_PACK4, VEC>(
-          acc, wbase, woff, (long long)L.ldw, xcol, H, kslice, half, (VEC && U.inp[s]) ? L.mb : 1);
+      const int xstride = (VEC && U.inp[s]) ? L.mb : 1;
+      if constexpr (SPLIT) {
+        // this workgroup's share of the segment: k-groups [g0, g1) of H / 8 (H % 8 == 0 on this path)
+        const int groups = H >> 3, part = blockIdx.y;
+        const int g0 = (int)((long long)groups * part / L.kparts), g1 = (int)((long long)groups * (part + 1) / L.kparts);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) wbase[g] += (long long)g0 * 8 * L.ldw;
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) xcol[tn] += (long long)g0 * 8 * xstride;
+        zr_mma_segment<4, TN, KS, lstm_prefetch_depth(TN, KS), ZR_A_PACK4, VEC>(
+            acc, wbase, woff, (long long)L.ldw, xcol, (g1 - g0) * 8, kslice, half, xstride);
+      } else {
+        zr_mma_segment<4, TN, KS, lstm_prefetch_depth(TN, KS), ZR_A_PACK4, VEC>(
+            acc, wbase, woff, (long long)L.ldw, xcol, H, kslice, half, xstride);
+      }
     }
   }
 
   const bool j_ok = j < H;
-  zr_reduce_visit<4, TN, KS>(acc, red, kslice, lane, [&](const float(&z)[4], int tn, int r, int vi) {
+  auto finish = [&](const float(&z)[4], int tn, int r, int vi) {
     const int n = n0 + tn * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
     if (j_ok && n < L.mb) {
       const long long ix = (long long)n * H + j;
@@ -200,7 +221,52 @@ __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
         U.gates[3][ix] = go;
       }
     }
-  });
+  };
+  if constexpr (!SPLIT) {
+    zr_reduce_visit<4, TN, KS>(acc, red, kslice, lane, finish);
+  } else {
+    constexpr int NTHR = 64 * KS;
+    const int tile = group * L.n_tiles + nt;
+    const int parts = L.kparts, part = blockIdx.y;
+    // partial tile of this workgroup: [visit][gate][thread], written and read with device-scope relaxed atomics
+    // (cache-bypassing on this multi-die part), published by the counter increment behind the barrier
+    float* mine = L.partials + ((long long)tile * parts + part) * (NV * 4 * NTHR) + tid;
+    zr_reduce_visit<4, TN, KS>(acc, red, kslice, lane, [&](const float(&z)[4], int, int, int vi) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+        __hip_atomic_store(mine + (vi * 4 + g) * NTHR, z[g], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    });
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    if (tid == 0) {
+      const int old = atomicAdd(&L.counters[tile], 1);
+      s_last = (old == parts - 1) ? 1 : 0;
+    }
+    __syncthreads();
+    if (!s_last) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    const float* base = L.partials + (long long)tile * parts * (NV * 4 * NTHR) + tid;
+    float sum[NV][4];
+    for (int p = 0; p < parts; ++p) {  // part order 0, 1, ... for every finisher
+      const float* pp = base + (long long)p * (NV * 4 * NTHR);
+      float t[NV][4];
+#pragma unroll
+      for (int vi = 0; vi < NV; ++vi)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+          t[vi][g] = __hip_atomic_load(pp + (vi * 4 + g) * NTHR, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+      for (int vi = 0; vi < NV; ++vi)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) sum[vi][g] = (p == 0) ? t[vi][g] : sum[vi][g] + t[vi][g];
+    }
+    if (tid == 0) __hip_atomic_store(&L.counters[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // next launch
+#pragma unroll
+    for (int vi = 0; vi < NV; ++vi) {
+      const int slot = zr_visit_slot<KS>(kslice, vi);
+      finish(sum[vi], slot >> 4, slot & 15, vi);
+    }
+  }
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -488,6 +554,24 @@ int launch_fused_v(zr_ctx* ctx, const LstmLaunch& L, bool vec) {
   return ZR_OK;
 }
 
+// Register-streaming kernel with K also split across `parts` workgroups per tile (SPLIT variant).
+template <int TN>
+int launch_fused_split(zr_ctx* ctx, LstmLaunch& L, int parts) {
+  const int groups = L.n_units * L.j_tiles;
+  const long long tiles = (long long)groups * L.n_tiles;
+  constexpr int NV = zr_visit_count<TN, 4>();
+  void* scratch = nullptr;
+  int rc = zr_ctx_scratch(ctx, 0, sizeof(float) * (size_t)tiles * parts * NV * 4 * 256, &scratch);
+  if (rc) return rc;
+  L.kparts = parts;
+  L.partials = (float*)scratch;
+  L.counters = ctx->d_counters;
+  dim3 grid((unsigned)(((groups + 7) / 8) * 8 * L.n_tiles), (unsigned)parts);
+  lstm_fused_kernel<TN, 4, true, false, false, true><<<grid, 256, 0, ctx->stream>>>(L);
+  ZR_LAUNCH_CHECK("lstm_fused_kernel (K split across workgroups)");
+  return ZR_OK;
+}
+
 template <int TN, int NWV>
 int launch_lds_v(zr_ctx* ctx, LstmLaunch& L) {
   LstmLaunch2 P;
@@ -525,8 +609,8 @@ int launch_fused(zr_ctx* ctx, LstmLaunch& L, bool vec) {
   for (int i = 0; i < L.n_units; ++i) L.nseg_max = L.u[i].nseg > L.nseg_max ? L.u[i].nseg : L.nseg_max;
   // Kernel choice.  The register-streaming kernel needs no cross-workgroup reduction and wins whenever it can put
   // a workgroup on (nearly) every CU -- a full diagonal of an encoder does.  A single node (a decoder step) gives
-  // it only ceil(H/32) * ceil(mb/64) workgroups; there the LDS / split-K kernel spreads the same node over ~256
-  // workgroups.  It needs 16-byte aligned operands and a batch wide enough for its 128-column tile.
+  // it only ceil(H/32) * ceil(mb/64) workgroups; there K is split across workgroups too: by the same kernel's SPLIT
+  // variant when H % 8 == 0, else by the LDS kernel (which needs a batch wide enough for its 128-column tile).
   if (L.bf16) {
     ZR_CHECK_ARG(vec && L.H % 16 == 0, "bf16 weights need H %% 16 == 0 and 16-byte aligned activations (H = %d)", L.H);
     const long long wg2 = (long long)L.n_units * L.j_tiles * ((n32 + 1) / 2);
@@ -535,10 +619,31 @@ int launch_fused(zr_ctx* ctx, LstmLaunch& L, bool vec) {
   }
   int kernel = ctx->lstm_kernel;
   if (L.preact) kernel = 1;  // only the register-streaming kernel stores raw pre-activations
-  if (kernel == 0) {
-    const long long wgs1 = (long long)L.n_units * L.j_tiles * ((n32 + 1) / 2);
-    kernel = (vec && n32 >= 3 && wgs1 < 200) ? 2 : 1;
+  // A launch that cannot put a whole-K tile on most CUs (a decoder node, the first and last diagonals of an encoder)
+  // divides K across workgroups as well.
+  const long long wgs_whole_k = (long long)L.n_units * L.j_tiles * ((n32 + 1) / 2);
+  if (kernel == 0 && vec && (L.H & 7) == 0 && wgs_whole_k < 200) kernel = 3;
+  if (kernel == 3 && vec && (L.H & 7) == 0) {
+    // widest column tile that divides the batch's 32-column blocks evenly, then as many K parts as fill the chip
+    const int tn = (n32 % 3 == 0) ? 3 : (n32 >= 2 ? 2 : 1);
+    L.n_tiles = (n32 + tn - 1) / tn;
+    const long long tiles = (long long)L.n_units * L.j_tiles * L.n_tiles;
+    int parts = ctx->lstm_kparts;
+    if (parts == 0) {
+      parts = (int)((256 + tiles / 2) / tiles);
+      const int max_parts = (L.H >> 3) / 16;  // at least 16 k-groups per part (4 per wave)
+      if (parts > max_parts) parts = max_parts;
+      if (parts > 8) parts = 8;
+    }
+    if (parts >= 2 && tiles <= ZR_MAX_COUNTERS && parts <= (L.H >> 3)) {
+      if (tn == 3) return launch_fused_split<3>(ctx, L, parts);
+      if (tn == 2) return launch_fused_split<2>(ctx, L, parts);
+      return launch_fused_split<1>(ctx, L, parts);
+    }
+    kernel = ctx->lstm_kernel == 3 ? 0 : ctx->lstm_kernel;  // no useful split for this shape
   }
+  if (kernel == 3) kernel = 0;  // needs 16-byte aligned operands and H % 8 == 0
+  if (kernel == 0) kernel = (vec && n32 >= 3 && wgs_whole_k < 200) ? 2 : 1;
   if (kernel == 2 && vec && L.n_units * L.j_tiles * ((n32 + 3) / 4) <= ZR_MAX_COUNTERS) {
     if (n32 > 4 && ctx->lstm_tn == 2) return launch_lds_v<2, 4>(ctx, L);
     return launch_lds_v<1, 4>(ctx, L);

@@ -128,7 +128,7 @@ int zr_ctx_set_option(zr_ctx* ctx, int option, int value) {
       ctx->lstm_ksplit = value;
       return ZR_OK;
     case ZR_OPT_LSTM_KERNEL:
-      ZR_CHECK_ARG(value >= 0 && value <= 2, "ZR_OPT_LSTM_KERNEL must be 0, 1 or 2");
+      ZR_CHECK_ARG(value >= 0 && value <= 3, "ZR_OPT_LSTM_KERNEL must be 0, 1, 2 or 3");
       ctx->lstm_kernel = value;
       return ZR_OK;
     case ZR_OPT_LSTM_KPARTS:
