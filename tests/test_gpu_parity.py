@@ -291,9 +291,13 @@ def test_config1_lm_forward_logprobs_and_loss(ctx):
 
 # ------------------------------------------------------------------------------------------------ A8/A9 softmax
 @pytest.mark.parametrize("prepared", [False, True])
-@pytest.mark.parametrize("V,H,mb", [(211, 16, 6), (10000, 100, 8), (4099, 64, 33), (1003, 27, 70)])
+@pytest.mark.parametrize("V,H,mb", [(211, 16, 6), (10000, 100, 8), (4099, 64, 33), (1003, 27, 70), (8300, 40, 128),
+                                    (8400, 24, 100), (16500, 32, 192), (9000, 16, 40)])
 def test_softmax_prob_and_logprob(ctx, V, H, mb, prepared):
-    """prepared: the output matrix registered with zr_softmax_prepare (k-interleaved copy); same results."""
+    """prepared: the output matrix registered with zr_softmax_prepare (k-interleaved copy); same results.  The shapes
+    with more than 8192 rows take the row-range kernel when prepared: 260-516 blocks of 32 rows over 128 or 256
+    workgroups, so a few blocks are left over and dealt out in 32-column pieces (column tiles of 128, 96 and 64, the
+    last column tile partly filled)."""
     g = synth.rng(11, V)
     D, bd, h = U(g, (V, H), -1, 1), U(g, (V,), -1, 1), U(g, (H, mb), -1, 1)
     dD, dbd, dh = ctx.array(D), ctx.array(bd), ctx.array(h)

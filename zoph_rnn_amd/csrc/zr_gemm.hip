@@ -252,9 +252,10 @@ __global__ void __launch_bounds__(64 * KS * WPB, OCC) gemm_kernel(GemmArgs a) {
 // Row-range variant for a tall weight matrix in the k-interleaved layout (the softmax logits: tens of thousands
 // of rows, a minibatch of columns).  With one tile per workgroup the number of workgroups is rarely a multiple of
 // the number of CUs and the last, partly filled round costs as much as a full one.  Here the grid is one
-// workgroup per CU (or fewer): each takes an equal share of the 32-row blocks (+-1) for one column tile and walks
-// it in passes of up to four blocks, so every CU finishes at about the same time and each weight element is
-// read by exactly one workgroup per column tile.
+// workgroup per CU (or fewer): each takes an equal share of the 32-row blocks for one column tile and walks it in
+// passes of up to four blocks; the few blocks that do not divide evenly are split into 32-column pieces over the
+// workgroups.  Every CU finishes at about the same time and each weight element is read by exactly one workgroup
+// per column tile (by up to TN for the left-over blocks).
 template <int TN, int EPI, int AMODE = ZR_A_PACK4>
 __global__ void __launch_bounds__(256) gemm_rows_kernel(GemmArgs a, int row_chunks) {
   __shared__ float red[4 * TN * 16 * 64];
@@ -268,9 +269,15 @@ __global__ void __launch_bounds__(256) gemm_rows_kernel(GemmArgs a, int row_chun
   const int nt = q % a.n_tiles;
   const int chunk = r8 * cpx + q / a.n_tiles;
   if (q / a.n_tiles >= cpx || chunk >= row_chunks) return;
-  const long long blocks = (a.M + 31) >> 5;
-  int b = (int)(blocks * chunk / row_chunks);
-  const int b_end = (int)(blocks * (chunk + 1) / row_chunks);
+  // Every chunk takes the same number of 32-row blocks; the blocks left over (fewer than row_chunks) are dealt out
+  // afterwards in 32-column pieces, one piece per workgroup, so that no workgroup carries a whole extra block.
+  // (Only when that is at most one piece per workgroup; with more left over, shares of +-1 block cost less.)
+  const int blocks = (a.M + 31) >> 5;
+  const int per_chunk = blocks / row_chunks;
+  const int left = blocks - per_chunk * row_chunks;
+  const bool pieces = left * TN <= row_chunks;
+  int b = pieces ? chunk * per_chunk : (int)((long long)blocks * chunk / row_chunks);
+  const int b_end = pieces ? b + per_chunk : (int)((long long)blocks * (chunk + 1) / row_chunks);
   const int n0 = nt * 32 * TN;
   // at most 192 accumulator registers per wave: four blocks per pass up to 96 columns, three at 128
   constexpr int TMAX = TN <= 3 ? 4 : 3;
@@ -287,6 +294,12 @@ __global__ void __launch_bounds__(256) gemm_rows_kernel(GemmArgs a, int row_chun
       gemm_tile<1, TN, 4, AMODE, true, EPI, PF4 + 2>(a, b * 32, n0, true, 0, red, kslice, lane);
     b += nb;
     __syncthreads();  // the next pass reuses the reduction buffer
+  }
+  for (int u = chunk; pieces && u < left * TN; u += row_chunks) {
+    const int blk = per_chunk * row_chunks + u / TN, sub = u % TN;
+    if (n0 + sub * 32 < a.N)
+      gemm_tile<1, 1, 4, AMODE, true, EPI, PF4 + 2>(a, blk * 32, n0 + sub * 32, true, 0, red, kslice, lane);
+    __syncthreads();
   }
 }
 
