@@ -640,7 +640,8 @@ int launch_fused(zr_ctx* ctx, LstmLaunch& L, bool vec) {
       if (tn == 2) return launch_fused_split<2>(ctx, L, parts);
       return launch_fused_split<1>(ctx, L, parts);
     }
-    kernel = ctx->lstm_kernel == 3 ? 0 : ctx->lstm_kernel;  // no useful split for this shape
+    // no useful split for this shape (e.g. 192 whole-K tiles): one tile per CU on most CUs beats the LDS kernel
+    kernel = 1;
   }
   if (kernel == 3) kernel = 0;  // needs 16-byte aligned operands and H % 8 == 0
   if (kernel == 0) kernel = (vec && n32 >= 3 && wgs_whole_k < 200) ? 2 : 1;
