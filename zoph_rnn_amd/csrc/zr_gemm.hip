@@ -780,11 +780,12 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
       ga.b_pack4 = 1;
     }
     // tall matrices: equal row ranges per CU, column tiles of equal width (at most 128 columns each)
-    if (vec && d.nseg == 1 && d.M >= 8192 && d.N > 32 && d.N <= 1024 && ctx->gemm_cfg != 11 &&
+    if (vec && d.nseg == 1 && d.M >= 8192 && d.N <= 1024 && ctx->gemm_cfg != 11 &&
         (d.epilogue == ZR_EPI_STORE || d.epilogue == ZR_EPI_SOFTMAX_PARTIAL)) {
       const int n32 = (d.N + 31) / 32;
       const int n_tiles = (n32 + 3) / 4;
       const int tn = (n32 + n_tiles - 1) / n_tiles;
+      if (tn == 1) return launch_rows<1>(ctx, ga, d.epilogue, n_tiles);
       if (tn <= 2) return launch_rows<2>(ctx, ga, d.epilogue, n_tiles);
       if (tn == 3) return launch_rows<3>(ctx, ga, d.epilogue, n_tiles);
       return launch_rows<4>(ctx, ga, d.epilogue, n_tiles);
