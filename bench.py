@@ -421,6 +421,9 @@ def main():
         extra["hbm_kernels"] = bench_hbm_kernels(ctx, args.steps)
         extra["config4_beam_decode"] = bench_beam_decode(ctx, args.steps)
         log("config4:", extra["config4_beam_decode"])
+        # the reference decodes one sentence per pass: the same step with 12 columns
+        extra["config4_single_sentence_beam12"] = bench_beam_decode(ctx, args.steps, n_sent=1)
+        log("config4, one sentence:", extra["config4_single_sentence_beam12"])
         log("hbm kernels:", extra["hbm_kernels"])
     cpu = None
     if not args.no_cpu:
