@@ -148,7 +148,8 @@ def test_config5_shape_lstm_node(ctx):
     layer.close()
 
 
-@pytest.mark.parametrize("V,H,mb", [(211, 16, 6), (1003, 48, 70), (4099, 64, 33), (9000, 112, 130), (8200, 96, 200)])
+@pytest.mark.parametrize("V,H,mb", [(211, 16, 6), (1003, 48, 70), (4099, 64, 33), (9000, 112, 130), (8200, 96, 200),
+                                    (8300, 16, 97), (12000, 48, 128), (9000, 32, 300), (40000, 64, 256)])
 def test_softmax_bf16_output_layer(ctx, V, H, mb):
     """Output matrix registered as bf16 (zr_softmax_prepare_bf16): logits, probabilities, log-probs and the loss
     against the oracle on the bf16-rounded matrix; covers the generic tiles (V < 8192) and the row-range kernel."""

@@ -651,10 +651,11 @@ int launch_fused(zr_ctx* ctx, LstmLaunch& L, bool vec) {
   }
   int tn = ctx->lstm_tn;
   if (tn == 0) {
-    // largest column tile that still yields at least one workgroup per CU
+    // 64-column tiles once they occupy more than half the CUs: 32-column tiles would then need two rounds of
+    // workgroups, which costs more than one round of the wider tile
     tn = 1;
     const int groups = L.n_units * L.j_tiles;
-    if (n32 >= 2 && (long long)groups * ((n32 + 1) / 2) >= 256) tn = 2;
+    if (n32 >= 2 && (long long)groups * ((n32 + 1) / 2) > 128) tn = 2;
   }
   if (tn > n32) tn = n32 >= 2 ? 2 : 1;
   if (tn == 4 && n32 < 4) tn = 2;
