@@ -70,6 +70,11 @@ const char* zr_version(void);
                                         2: weights through LDS, K split across workgroups;
                                         3: weights streamed to registers, K split inside and across workgroups */
 #define ZR_OPT_LSTM_KPARTS 6         /* kernels 2 and 3: K parts per weight segment (0 = auto) */
+#define ZR_OPT_LSTM_SWEEP 7          /* zr_lstm_stack_forward as ONE launch whose workgroups hand h to each other
+                                        through device memory: 0 auto (when they fill most of the device and are all
+                                        resident at once), 1 never (one launch per diagonal), 2 whenever they fit */
+#define ZR_OPT_LSTM_SWEEP_SPIN 8     /* polls a workgroup of that launch spends on one wait before it gives up
+                                        (0 = default, about a second); giving up is reported by zr_ctx_sync */
 
 /* full_matrix_setup / cudaMalloc / cudaMemcpy / cudaMemset call sites (src/BZ_CUDA_UTIL.h:358-399 and the
  * layer constructors, e.g. src/LSTM.hpp:23-42). */

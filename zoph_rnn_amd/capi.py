@@ -18,6 +18,8 @@ ZR_OPT_GEMM_CFG = 3
 ZR_OPT_LSTM_KSPLIT = 4
 ZR_OPT_LSTM_KERNEL = 5
 ZR_OPT_LSTM_KPARTS = 6
+ZR_OPT_LSTM_SWEEP = 7
+ZR_OPT_LSTM_SWEEP_SPIN = 8
 ZR_SOFTMAX_PROB = 0
 ZR_SOFTMAX_LOGPROB = 1
 

@@ -14,7 +14,8 @@ struct zr_ctx {
   int device;
   hipStream_t own_stream;
   hipStream_t stream;  // the stream in use (own_stream or a caller-provided one)
-  int* d_flags;        // [0]: count of token ids seen outside [0, V); [1]: attention table index clamps
+  int* d_flags;        // [0]: count of token ids seen outside [0, V); [1]: attention table index clamps;
+                       // [2]: a workgroup of the whole-sweep LSTM kernel abandoned a wait
   hipEvent_t ev_start, ev_stop;  // zr_timer_start / zr_timer_stop
   // options
   int lstm_fused;
@@ -23,6 +24,10 @@ struct zr_ctx {
   int lstm_kernel;   // 0 auto, 1 register-streaming kernel, 2 LDS / split-K kernel
   int lstm_kparts;   // K parts per segment for the split-K kernel (0 auto)
   int* d_counters;   // ZR_MAX_COUNTERS arrival counters, zero between launches
+  int lstm_sweep;    // whole-sweep LSTM kernel: 0 auto, 1 never, 2 whenever the launch fits on the device
+  int sweep_spin;    // polls before a waiting workgroup of that kernel gives up (0: default)
+  int cu_count;      // compute units of the device (filled with sweep_capacity)
+  int sweep_capacity[3];  // resident workgroups of lstm_sweep_kernel<TN> (0: not asked yet, -1: unknown)
   int gemm_cfg;
   // scratch owned by the context (grown on demand, never shrunk)
   void* d_scratch;

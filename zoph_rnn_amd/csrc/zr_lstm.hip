@@ -236,8 +236,7 @@ __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
       for (int g = 0; g < 4; ++g)
         __hip_atomic_store(mine + (vi * 4 + g) * NTHR, z[g], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     });
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __syncthreads();
+    zr_publish_barrier();
     if (tid == 0) {
       const int old = atomicAdd(&L.counters[tile], 1);
       s_last = (old == parts - 1) ? 1 : 0;
@@ -472,10 +471,9 @@ __global__ void __launch_bounds__(64 * NWV) lstm_lds_kernel(LstmLaunch2 P) {
                              __HIP_MEMORY_SCOPE_AGENT);
     // The partials are written and read with device-scope atomic accesses (write-through / cache-bypassing on
     // this multi-die part), so no L2 write-back + invalidate is needed to publish them -- a full device-scope
-    // fence here costs more than the whole K loop.  The workgroup-scope fence drains this wave's outstanding
-    // stores before the barrier; the counter increment after the barrier is a device-scope atomic.
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __syncthreads();
+    // fence here costs more than the whole K loop.  Every wave waits for its own stores to complete before the
+    // barrier; the counter increment after the barrier is a device-scope atomic.
+    zr_publish_barrier();
     if (tid == 0) {
       const int old = atomicAdd(&P.counters[tile], 1);
       s_last = (old == splits - 1) ? 1 : 0;
@@ -524,6 +522,226 @@ __global__ void __launch_bounds__(64 * NWV) lstm_lds_kernel(LstmLaunch2 P) {
           }
         }
       }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Whole-sweep kernel: ONE launch runs every (layer, time step) node of a stacked forward pass.
+//
+// A workgroup owns the same tile -- 32 hidden rows x 32*TN batch columns of one layer -- at every time step and loops
+// over t itself.  Node (l, t) needs h of (l-1, t) and of (l, t-1), each produced by the j_tiles workgroups that own
+// the same batch columns of that layer: every (layer, column tile) has an arrival counter in device memory that its
+// producers bump once per time step, and a consumer waits until the counter reaches (steps needed) * j_tiles.  The
+// layers settle into a skewed pipeline: the input from below is consumed first and the recurrent input second, so the
+// hand-over latency of a layer's own h hides behind half a K loop, and a layer never waits for the layer above it.
+// Compared with one launch per diagonal this removes, per step, the launch, the drain of the slowest tile and the
+// refill of the operand pipeline from a cold start; the cell state never leaves registers.
+//
+// Hand-over through memory: h is written twice, to the caller's array (plain stores, visible at kernel end) and to a
+// k-interleaved copy [H/4][mb][4] per (layer, t) that the consumers read.  The chip's eight dies have one L2 each.
+// The copy is written with device-scope stores (written through to memory); every wave waits for its stores to
+// complete, then a workgroup barrier, then one thread bumps the counter.  A consumer polls the counter with
+// device-scope loads and reads the copy with ordinary loads.  Those cannot hit a stale line as long as no line is
+// cached before it was written: caches are clean when the kernel starts, every line of a copy is read only after
+// the wait for its producers, and with mb % 8 == 0 a 128-byte line (8 columns x 4 rows) has one producer.  For other
+// minibatch sizes lines straddle producers, and the consumers invalidate their caches after every wait instead
+// (device-scope acquire), which costs about 4 % at the benchmark shape.
+//
+// Operand fetch: buffer loads (descriptor base + scalar offset advancing with k + fixed 32-bit lane offset), so the K
+// loop holds no vector instruction other than the MFMAs; see zr_mma_segment_u.
+//
+// Progress: the launch must be wholly resident (the host checks grid <= CUs x resident workgroups per CU), then the
+// dependency graph is acyclic and every wait ends.  Every wait is bounded all the same: a workgroup that runs out of
+// polls marks every counter, which releases all other waiters, raises the status flag and leaves; the others leave
+// at their next wait.
+// ---------------------------------------------------------------------------------------------------------
+constexpr int kSweepGaveUp = 1 << 28;  // bit set in every counter by a workgroup that stopped waiting
+constexpr int kSweepCtrStride = 32;    // ints between counters: one 128-byte line each
+
+struct LstmSweep {
+  const float* W[kMaxUnits];     // per layer: [2][4] packed fp32 matrices
+  const float* bias[kMaxUnits];  // per layer: [4][H]
+  const float* h0[kMaxUnits];
+  const float* c0[kMaxUnits];
+  float* h_all[kMaxUnits];
+  float* c_all[kMaxUnits];
+  float* gates_all[kMaxUnits];   // null: gates not kept
+  const float* embed;
+  const int* ids;                // [T][mb], already non-negative
+  const int* mask01;             // [T][mb]
+  float* hp;                     // [nl][T] k-interleaved copies of h, H*mb floats each
+  int* counters;                 // [nl][n_tiles] at kSweepCtrStride, zero at launch
+  int* status;                   // set to 1 when a wait was abandoned
+  int nl, T, V, H, mb, ldw, kp, j_tiles, n_tiles;
+  float clip;
+  int spin_limit;
+  int fence;   // 1: consumers invalidate their caches after every wait (see lstm_sweep_kernel)
+};
+
+// All threads of the workgroup call this.  False: leave the kernel.
+__device__ __forceinline__ bool sweep_wait(const LstmSweep& P, int* ctr, int target, int* s_go) {
+  if (threadIdx.x == 0) {
+    int v = __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (int spins = 0; v < target && spins < P.spin_limit; ++spins) {
+      __builtin_amdgcn_s_sleep(8);
+      v = __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    const bool ok = v >= target && !(v & kSweepGaveUp);
+    if (!ok) {
+      if (!(v & kSweepGaveUp)) {
+        const int n = P.nl * P.n_tiles;
+        for (int i = 0; i < n; ++i) atomicOr(P.counters + i * kSweepCtrStride, kSweepGaveUp);
+      }
+      __hip_atomic_store(P.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    *s_go = ok ? 1 : 0;
+  }
+  __syncthreads();
+  const bool go = *s_go != 0;
+  if (go && P.fence) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  return go;
+}
+
+template <int TN>
+__global__ void __launch_bounds__(256) lstm_sweep_kernel(LstmSweep P) {
+  constexpr int KS = 4;
+  __shared__ float red[KS * TN * 16 * 64];
+  __shared__ int s_go[2];
+  // same die-aware placement as lstm_fused_kernel, with one unit per layer
+  const int id = blockIdx.x;
+  const int r8 = id & 7;
+  const int q = id >> 3;
+  const int nt = q % P.n_tiles;
+  const int groups = P.nl * P.j_tiles;
+  const int group = r8 * ((groups + 7) >> 3) + q / P.n_tiles;
+  if (q / P.n_tiles >= ((groups + 7) >> 3) || group >= groups) return;
+  const int l = group / P.j_tiles;
+  const int jt = group % P.j_tiles;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int kslice = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int H = P.H, mb = P.mb;
+  const int j0 = jt * 32;
+  const int n0 = nt * 32 * TN;
+  const long long n_el = (long long)H * mb;
+  constexpr int NV = zr_visit_count<TN, KS>();
+  // batch column of visit i of a lane in half-wave `half`, clamped
+  auto visit_col = [&](int i, int half) {
+    const int slot = zr_visit_slot<KS>(kslice, i);
+    const int tn = slot >> 4, r = slot & 15;
+    const int n = n0 + tn * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+    return n < mb ? n : mb - 1;
+  };
+  auto clamp_col = [&](int c) { return c < mb ? c : mb - 1; };
+  auto clamp_id = [&](int v) { return v < 0 ? 0 : (v >= P.V ? P.V - 1 : v); };
+
+  const float* bias = P.bias[l];
+  float bi, bf, bc, bo;
+  float c_state[NV];  // cell state of this thread's outputs, carried from step to step
+  int idv[TN];        // layer 0: embedding column of each batch column, fetched one step ahead
+  {
+    const int jl = lane & 31, half = lane >> 5;
+    const int jc = j0 + jl < H ? j0 + jl : H - 1;
+    bi = bias[jc], bf = bias[H + jc], bc = bias[2 * H + jc], bo = bias[3 * H + jc];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) c_state[i] = P.c0[l][(long long)visit_col(i, half) * H + jc];
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) idv[tn] = (l == 0) ? clamp_id(P.ids[clamp_col(n0 + tn * 32 + jl)]) : 0;
+  }
+
+  const long long HH = (long long)P.kp * P.ldw;
+  const float* Wl = P.W[l];
+  int* my_ctr = P.counters + (l * P.n_tiles + nt) * kSweepCtrStride;
+  int* below_ctr = P.counters + ((l > 0 ? l - 1 : 0) * P.n_tiles + nt) * kSweepCtrStride;
+  float* hp_mine = P.hp + (long long)l * P.T * n_el;
+  const float* hp_below = P.hp + (long long)(l > 0 ? l - 1 : 0) * P.T * n_el;
+  float* gates = P.gates_all[l];
+
+  for (int t = 0; t < P.T; ++t) {
+    // Everything that depends on the lane is derived afresh in each time step from a lane index the compiler cannot
+    // see through: hoisted out of the loop, the per-lane addresses of both K loops would have to stay in registers
+    // through all of it, and the kernel has none to spare.
+    int lane_t = lane;
+    asm volatile("" : "+v"(lane_t));
+    const int jl = lane_t & 31, half = lane_t >> 5;
+    const int j = j0 + jl;
+    const bool j_ok = j < H;
+    int cols[TN];
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) cols[tn] = clamp_col(n0 + tn * 32 + jl);
+    const unsigned woffb = 16u * (unsigned)(j + half * P.ldw);
+    int idn[TN];
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+      const int tt = t + 1 < P.T ? t + 1 : t;
+      idn[tn] = (l == 0) ? clamp_id(P.ids[(long long)tt * mb + cols[tn]]) : 0;
+    }
+
+    zr_f32x16 acc[4][TN];
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[g][tn][r] = 0.0f;
+
+    for (int s = 0; s < 2; ++s) {
+      // segment 0: input from below (h of (l-1, t), or the embedding columns); segment 1: h of (l, t-1)
+      const bool packed = (s == 0) ? (l > 0) : (t > 0);
+      if (packed) {
+        int* ctr = (s == 0) ? below_ctr : my_ctr;
+        const int target = ((s == 0) ? t + 1 : t) * P.j_tiles;
+        if (!sweep_wait(P, ctr, target, &s_go[s])) return;
+      }
+      unsigned wsoff[4];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) wsoff[g] = (unsigned)(((long long)s * 4 + g) * HH * 4);
+      const float* xp = (s == 0) ? hp_below + (long long)t * n_el : hp_mine + (long long)(t > 0 ? t - 1 : 0) * n_el;
+      const float* xu = (s == 0) ? P.embed : P.h0[l];
+      unsigned xoffb[TN];
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) {
+        const unsigned c = (s == 0) ? (unsigned)idv[tn] : (unsigned)cols[tn];
+        xoffb[tn] = packed ? 16u * ((unsigned)cols[tn] + (unsigned)(half * mb)) : 4u * (c * (unsigned)H + 4u * half);
+      }
+      zr_mma_segment_u<4, TN, KS, lstm_prefetch_depth(TN, KS)>(
+          acc, zr_make_rsrc(Wl), wsoff, woffb, 32u * (unsigned)P.ldw, zr_make_rsrc(packed ? xp : xu), xoffb,
+          packed ? 32u * (unsigned)mb : 32u, H, kslice);
+    }
+
+    // the column masks are fetched here, behind the K loops, and arrive while the partial tiles are being summed
+    float mask_v[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) mask_v[i] = (float)P.mask01[(long long)t * mb + visit_col(i, half)];
+    float* h_out = P.h_all[l] + (long long)t * n_el;
+    float* c_out = P.c_all[l] + (long long)t * n_el;
+    float* hp_out = hp_mine + (long long)t * n_el;
+    zr_reduce_visit<4, TN, KS>(acc, red, kslice, lane, [&](const float(&z)[4], int tn, int r, int vi) {
+      const int n = n0 + tn * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+      float gi, gf, gc, go, c, h;
+      zr_lstm_cell(z[0] + bi, z[1] + bf, z[2] + bc, z[3] + bo, c_state[vi], mask_v[vi], P.clip, gi, gf, gc, go, c, h);
+      c_state[vi] = c;
+      if (j_ok && n < mb) {
+        const long long ix = (long long)n * H + j;
+        c_out[ix] = c;
+        h_out[ix] = h;
+        __hip_atomic_store(hp_out + ((long long)(j >> 2) * mb + n) * 4 + (j & 3), h, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+        if (gates) {
+          float* gt = gates + (long long)t * 4 * n_el + ix;
+          gt[0] = gi;
+          gt[n_el] = gf;
+          gt[2 * n_el] = gc;
+          gt[3 * n_el] = go;
+        }
+      }
+    });
+    // publish this step: every wave's stores have completed before the barrier, then one arrival per workgroup
+    zr_publish_barrier();
+    if (tid == 0) atomicAdd(my_ctr, 1);
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) idv[tn] = idn[tn];
   }
 }
 
@@ -668,6 +886,32 @@ int launch_fused(zr_ctx* ctx, LstmLaunch& L, bool vec) {
   if (tn == 1) return ks == 8 ? launch_fused_v<1, 8>(ctx, L, vec) : launch_fused_v<1, 4>(ctx, L, vec);
   if (tn == 2) return ks == 8 ? launch_fused_v<2, 8>(ctx, L, vec) : launch_fused_v<2, 4>(ctx, L, vec);
   return launch_fused_v<4, 4>(ctx, L, vec);
+}
+
+
+// Resident workgroups of lstm_sweep_kernel<TN> the device can hold at once (0: unknown / query failed).
+template <int TN>
+int sweep_capacity(zr_ctx* ctx) {
+  int& cached = ctx->sweep_capacity[TN];
+  if (cached == 0) {
+    int cus = 0, per_cu = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, ctx->device) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lstm_sweep_kernel<TN>, 256, 0) != hipSuccess) {
+      (void)hipGetLastError();
+      cached = -1;
+    } else {
+      ctx->cu_count = cus;
+      cached = cus * per_cu > 0 ? cus * per_cu : -1;
+    }
+  }
+  return cached > 0 ? cached : 0;
+}
+
+template <int TN>
+int launch_sweep_v(zr_ctx* ctx, LstmSweep& P, int grid) {
+  lstm_sweep_kernel<TN><<<grid, 256, 0, ctx->stream>>>(P);
+  ZR_LAUNCH_CHECK("lstm_sweep_kernel");
+  return ZR_OK;
 }
 
 inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
@@ -852,6 +1096,63 @@ int zr_lstm_stack_forward_train(zr_ctx* ctx, int nl, const zr_lstm_weights* cons
     vec = vec && aligned16(d_h0[l]) && aligned16(d_h_all[l]);
   }
   const size_t n = (size_t)H * mb;
+  // One launch for the whole sweep when its workgroups -- one tile of one layer each, kept for all T steps -- fill
+  // most of the chip and fit on it together; otherwise one launch per diagonal.
+  if (vec && H % 8 == 0 && !layers[0]->bf16 && ctx->lstm_fused && ctx->lstm_sweep != 1 && nl <= kMaxUnits) {
+    const int j_tiles = (H + 31) / 32, n32 = (mb + 31) / 32;
+    const int groups = nl * j_tiles;
+    const int padded = (groups + 7) / 8 * 8;
+    int tn = 0;
+    if ((long long)padded * n32 <= sweep_capacity<1>(ctx)) tn = 1;
+    else if ((long long)padded * ((n32 + 1) / 2) <= sweep_capacity<2>(ctx)) tn = 2;
+    const int n_tiles = tn ? (n32 + tn - 1) / tn : 0;
+    const long long tiles = (long long)groups * n_tiles;
+    const bool fills = tn && tiles * 10 >= 6LL * ctx->cu_count;
+    // the kernel addresses its operands as descriptor base + 32-bit byte offsets
+    const long long lim = 1LL << 32;
+    const bool offsets_fit = (long long)V * H * 4 < lim && (long long)n * 4 < lim &&
+                             8LL * layers[0]->kp * layers[0]->ldw * 4 < lim;
+    if (tn && offsets_fit && (fills || ctx->lstm_sweep == 2) && nl * n_tiles <= 512 &&
+        (long long)T * j_tiles < kSweepGaveUp) {
+      LstmSweep P = {};
+      const size_t ctr_bytes = sizeof(int) * 512 * kSweepCtrStride;
+      void* p = nullptr;
+      rc = zr_ctx_scratch(ctx, 1, ctr_bytes + sizeof(float) * (size_t)nl * T * n, &p);
+      if (rc) return rc;
+      P.counters = (int*)p;
+      P.hp = (float*)((char*)p + ctr_bytes);
+      rc = zr_memset_zero(ctx, P.counters, sizeof(int) * (size_t)nl * n_tiles * kSweepCtrStride);
+      if (rc) return rc;
+      for (int l = 0; l < nl; ++l) {
+        P.W[l] = (const float*)layers[l]->d_W;
+        P.bias[l] = layers[l]->d_bias;
+        P.h0[l] = d_h0[l];
+        P.c0[l] = d_c0[l];
+        P.h_all[l] = d_h_all[l];
+        P.c_all[l] = d_c_all[l];
+        P.gates_all[l] = d_gates_all ? d_gates_all[l] : nullptr;
+      }
+      P.embed = d_embed;
+      P.ids = d_ids_nonneg;
+      P.mask01 = d_mask01;
+      P.status = ctx->d_flags + 2;
+      P.nl = nl;
+      P.T = T;
+      P.V = V;
+      P.H = H;
+      P.mb = mb;
+      P.ldw = layers[0]->ldw;
+      P.kp = layers[0]->kp;
+      P.j_tiles = j_tiles;
+      P.n_tiles = n_tiles;
+      P.clip = clip_threshold;
+      P.spin_limit = ctx->sweep_spin > 0 ? ctx->sweep_spin : (1 << 20);
+      // Without the invalidation a consumer relies on never having cached a line before its producer wrote it: true
+      // when no 128-byte line of the k-interleaved copies is shared between two producers, i.e. mb % 8 == 0.
+      P.fence = (mb % 8 == 0) ? 0 : 1;
+      return tn == 1 ? launch_sweep_v<1>(ctx, P, padded * n_tiles) : launch_sweep_v<2>(ctx, P, padded * n_tiles);
+    }
+  }
   // Every h is also written in a k-interleaved layout ([H/4][mb][4]) into a small ping-pong buffer per layer: its
   // two consumers on the next diagonal, (l+1, t) and (l, t+1), then fetch activations with contiguous 16-byte
   // loads.  The buffer written on diagonal d is read on d+1 only and overwritten on d+2.

@@ -66,7 +66,10 @@ struct ZrFrag {
 //              lines.  Packed activations require VEC and K % 8 == 0.
 // Rows / columns are pre-clamped by the caller so that out-of-range lanes read valid memory.
 // kslice must be wave-uniform.
-template <int TM, int TN, int KS, int PF, int AMODE, bool VEC>
+// PIN: stages are fenced off from each other for the instruction scheduler (each stage's loads stay next to its own
+// MFMAs).  Needed where the scheduler would otherwise gather the loads of a whole ring revolution at its end, which
+// drains the ring once per revolution.
+template <int TM, int TN, int KS, int PF, int AMODE, bool VEC, bool PIN = false>
 __device__ __forceinline__ void zr_mma_segment(zr_f32x16 (&acc)[TM][TN], const float* const (&wbase)[TM],
                                                const unsigned (&woff)[TM], long long lda,
                                                const float* const (&xcol)[TN], int K, int kslice, int half,
@@ -150,6 +153,18 @@ __device__ __forceinline__ void zr_mma_segment(zr_f32x16 (&acc)[TM][TN], const f
         const int gl = kslice + (it + s + PF) * KS;
         load_full(f[(s + PF) % NS], gl < last ? gl : last);
         mma(f[s]);
+        if (PIN) {
+          // one load, then its share of the stage's MFMAs: a run of back-to-back loads holds the wave's issue slot
+          // for longer than one MFMA lasts and leaves the matrix pipe idle behind it
+          constexpr int NL = TM + TN, NM = 4 * TM * TN;
+#pragma unroll
+          for (int q = 0; q < NL; ++q) {
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, NM / NL, 0);
+          }
+          __builtin_amdgcn_sched_group_barrier(0x008, NM - NL * (NM / NL), 0);
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
     }
     // at most PF groups remain, all of them already loaded
@@ -183,6 +198,94 @@ __device__ __forceinline__ void zr_mma_segment(zr_f32x16 (&acc)[TM][TN], const f
     }
     mma(t);
   }
+}
+
+// Variant of zr_mma_segment for k-interleaved weights and 16-byte activation loads that fetches through buffer
+// descriptors: an address is descriptor base (scalar registers) + a scalar byte offset that advances with k + a 32-bit
+// per-lane byte offset that stays fixed through the segment, so a load needs no vector address arithmetic at all
+// (64-bit vector adds would compete with the MFMAs for the vector issue slot).  Stages are pinned for the scheduler
+// (see PIN above).
+//   wrsrc:    descriptor over the TM weight sub-tiles' matrices; wsoff[tm] = byte offset of sub-tile tm's matrix
+//   woffb:    this lane's byte offset into every weight sub-tile: 4 * (4*row + 4*half*lda)
+//   xrsrc:    descriptor over the activations
+//   xoffb[tn]: this lane's byte offset of its column, 4*half included
+//   wstep / xstep: bytes per k-group of 8 (weights: 32*lda; activations: 32 for a plain column, 32*mb k-interleaved)
+// Every offset sum must stay below 4 GiB (the host checks the extents).
+typedef unsigned zr_u32x4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t zr_make_rsrc(const void* base) {
+  // raw buffer, no bounds limit to speak of, 32-bit data format (descriptor word 3 for this GPU family)
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0xFFFFFFFF, 0x00020000);
+}
+
+template <int TM, int TN, int KS, int PF>
+__device__ __forceinline__ void zr_mma_segment_u(zr_f32x16 (&acc)[TM][TN], __amdgpu_buffer_rsrc_t wrsrc,
+                                                 const unsigned (&wsoff)[TM], unsigned woffb, unsigned wstep,
+                                                 __amdgpu_buffer_rsrc_t xrsrc, const unsigned (&xoffb)[TN],
+                                                 unsigned xstep, int K, int kslice) {
+  const int nfull = K >> 3;  // K % 8 == 0
+  constexpr int NS = PF + 1;
+  auto load_full = [&](ZrFrag<TM, TN>& f, int g) {
+    const unsigned ug = (unsigned)g;  // wave-uniform
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+      const zr_u32x4v v = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, (int)xoffb[tn], (int)(ug * xstep), 0);
+      f.x[tn][0] = __uint_as_float(v.x);
+      f.x[tn][1] = __uint_as_float(v.y);
+      f.x[tn][2] = __uint_as_float(v.z);
+      f.x[tn][3] = __uint_as_float(v.w);
+    }
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+      const zr_u32x4v v = __builtin_amdgcn_raw_buffer_load_b128(wrsrc, (int)woffb, (int)(wsoff[tm] + ug * wstep), 0);
+      f.w[tm][0] = __uint_as_float(v.x);
+      f.w[tm][1] = __uint_as_float(v.y);
+      f.w[tm][2] = __uint_as_float(v.z);
+      f.w[tm][3] = __uint_as_float(v.w);
+    }
+  };
+  auto mma = [&](const ZrFrag<TM, TN>& f) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.x[tn][i], f.w[tm][i], acc[tm][tn], 0, 0, 0);
+  };
+  if (kslice < nfull) {
+    const int last = nfull - 1;
+    const int n_mine = (nfull - kslice + KS - 1) / KS;
+    ZrFrag<TM, TN> f[NS];
+#pragma unroll
+    for (int s = 0; s < PF; ++s) {
+      const int gl = kslice + s * KS;
+      load_full(f[s], gl < last ? gl : last);
+    }
+    int it = 0;
+    for (; it + NS <= n_mine; it += NS) {
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        const int gl = kslice + (it + s + PF) * KS;
+        load_full(f[(s + PF) % NS], gl < last ? gl : last);
+        mma(f[s]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < PF; ++s)
+      if (it + s < n_mine) mma(f[s]);
+  }
+}
+
+// Workgroup barrier that also publishes: when it returns, every store any thread of the workgroup issued before it
+// has completed (device-scope write-through stores have reached memory), so one thread may then announce the
+// workgroup's data to other workgroups with a device-scope atomic.  A workgroup-scope release fence alone only keeps
+// the compiler from sinking the stores; it does not make a wave wait for the acknowledgements of stores in flight,
+// hence the explicit vmcnt(0) (s_waitcnt operand: vmcnt = 0, expcnt and lgkmcnt at their maxima = no wait).
+__device__ __forceinline__ void zr_publish_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  __syncthreads();
 }
 
 // Number of visits zr_reduce_visit makes per thread, and the accumulator slot (tn*16 + r) of visit i: callers use

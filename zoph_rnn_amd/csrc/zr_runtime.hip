@@ -99,6 +99,12 @@ int zr_ctx_sync(zr_ctx* ctx) {
   ZR_LAUNCH_CHECK("queued work");
   int flags[4] = {0, 0, 0, 0};
   ZR_HIP(hipMemcpy(flags, ctx->d_flags, sizeof(flags), hipMemcpyDeviceToHost));
+  if (flags[2] != 0) {
+    ZR_HIP(hipMemset(ctx->d_flags, 0, sizeof(flags)));
+    return zr_set_error(ZR_EHIP, "a whole-sweep LSTM launch gave up waiting for another workgroup: the outputs of "
+                        "zr_lstm_stack_forward since the last zr_ctx_sync are incomplete (ZR_OPT_LSTM_SWEEP = 1 "
+                        "selects one launch per diagonal)");
+  }
   if (flags[0] != 0 || flags[1] != 0) {
     ZR_HIP(hipMemset(ctx->d_flags, 0, sizeof(flags)));
     return zr_set_error(ZR_EDATA, "%d token id(s) outside [0, vocab) and %d source position(s) outside the "
@@ -134,6 +140,14 @@ int zr_ctx_set_option(zr_ctx* ctx, int option, int value) {
     case ZR_OPT_LSTM_KPARTS:
       ZR_CHECK_ARG(value >= 0 && value <= 16, "ZR_OPT_LSTM_KPARTS must be in [0, 16]");
       ctx->lstm_kparts = value;
+      return ZR_OK;
+    case ZR_OPT_LSTM_SWEEP:
+      ZR_CHECK_ARG(value >= 0 && value <= 2, "ZR_OPT_LSTM_SWEEP must be 0, 1 or 2");
+      ctx->lstm_sweep = value;
+      return ZR_OK;
+    case ZR_OPT_LSTM_SWEEP_SPIN:
+      ZR_CHECK_ARG(value >= 0, "ZR_OPT_LSTM_SWEEP_SPIN must not be negative");
+      ctx->sweep_spin = value;
       return ZR_OK;
     case ZR_OPT_GEMM_CFG:
       ZR_CHECK_ARG(value >= 0 && value <= 14, "ZR_OPT_GEMM_CFG out of range");
