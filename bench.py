@@ -26,11 +26,11 @@ import numpy as np  # noqa: E402
 PEAK_FP32_MFMA_TFLOPS = 157.3  # MI355X dense fp32 matrix peak
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E peak
 
-# HBM bytes per full-diagonal launch of lstm_fused_kernel on the headline workload, from two rocprofv3 --pmc runs
-# (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for a plain copy of
-# known size (bench.py --calibrate-copy): FETCH_SIZE 69128.2 KiB x 1.9707 + WRITE_SIZE 6000.0 KiB x 1.0000.
-# The summary of those runs is profiles/lstm_fused_kernel_config2_hbm_traffic.txt.
-LSTM_FUSED_FULL_DIAGONAL_TRAFFIC_BYTES = int((69128.2 * 1.9707 + 6000.0 * 1.0) * 1024)
+# HBM bytes per launch of lstm_sweep_kernel on the headline workload, from two rocprofv3 --pmc runs (FETCH_SIZE, then
+# WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for a plain copy of known size
+# (bench.py --calibrate-copy): FETCH_SIZE 0 KiB x 1.0 + WRITE_SIZE 0 KiB x 1.0.
+# The summary of those runs is profiles/lstm_sweep_kernel_config2_hbm_traffic.txt.
+LSTM_SWEEP_TRAFFIC_BYTES = None
 
 
 def log(*a):
@@ -80,21 +80,20 @@ def bench_encoder(ctx, steps, warmup, H=1000, mb=128, T=50, V=50000, L=4):
         ctx.lstm_stack_forward(ws, d_embed, V, d_nn, d_m, T, mb, [z] * L, [z] * L, h_all, c_all)
 
     wall_ms, ev_ms = time_region(ctx, step, steps, warmup)
-    launches = (T + L - 1) * steps            # one fused kernel launch per diagonal of the (layer, time) grid
+    # one lstm_sweep_kernel launch per step (preceded by a sub-microsecond counter-clearing fill)
     flops_per_step = 2.0 * 4 * H * mb * (2 * H) * L * T
-    res = {"wall_ms": wall_ms, "event_ms": ev_ms, "tokens_per_step": mb * T, "launches_per_step": T + L - 1,
-           "flops_per_step": flops_per_step, "avg_launch_us": ev_ms * 1e3 / launches,
-           "flops_per_launch": flops_per_step / (T + L - 1)}
+    res = {"wall_ms": wall_ms, "event_ms": ev_ms, "tokens_per_step": mb * T, "launches_per_step": 1,
+           "flops_per_step": flops_per_step, "avg_launch_us": ev_ms * 1e3 / steps,
+           "flops_per_launch": flops_per_step}
     # keep references alive until here
     res["_keep"] = (layers, d_embed, d_nn, d_m, z, h_all, c_all)
     return res
 
 
-def measure_full_diagonal_launch(ctx, steps, warmup, H=1000, mb=128, T=50, V=50000, L=4):
-    """Average duration of one full-diagonal launch of lstm_fused_kernel (L units: one node of every layer), the
-    launch that dominates the encoder sweep: a sweep over 2T time steps runs exactly T more of them than a sweep over
-    T (the ramp launches at both ends are the same), so the difference of the two event-timed regions / T is its
-    duration, launch gaps included."""
+def measure_steady_state_step(ctx, steps, warmup, H=1000, mb=128, T=50, V=50000, L=4):
+    """Time one more time step adds to a sweep (L nodes, one of every layer) once the layers run as a pipeline: a sweep
+    over 2T time steps has T more of them than a sweep over T and the same fill and drain, so the difference of the
+    two event-timed regions / T is that time."""
     long_run = bench_encoder(ctx, steps, warmup, H=H, mb=mb, T=2 * T, V=V, L=L)
     long_run.pop("_keep")
     short_run = bench_encoder(ctx, steps, warmup, H=H, mb=mb, T=T, V=V, L=L)
@@ -366,6 +365,9 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the config-3 and HBM-kernel measurements")
     ap.add_argument("--lstm-tn", type=int, default=0)
     ap.add_argument("--lstm-ks", type=int, default=0)
+    ap.add_argument("--sweep-only", action="store_true",
+                    help="run only the headline encoder sweep (one kernel launch per step) and print its time: the "
+                         "command the rocprofv3 summaries under profiles/ are made with")
     ap.add_argument("--training-only", action="store_true",
                     help="only run the language-model training step measurement (for profiling) and exit")
     ap.add_argument("--vendor-gemm", action="store_true",
@@ -393,6 +395,12 @@ def main():
         print(json.dumps(calibrate_copy(ctx)))
         ctx.close()
         return
+    if args.sweep_only:
+        enc = bench_encoder(ctx, args.steps, args.warmup)
+        enc.pop("_keep")
+        print(json.dumps({"ms_per_step": enc["event_ms"] / args.steps, "steps": args.steps}))
+        ctx.close()
+        return
     if args.training_only:
         print(json.dumps(bench_training_step(ctx, max(2, args.steps // 6))))
         ctx.close()
@@ -402,10 +410,18 @@ def main():
     enc.pop("_keep")
     ms_per_step = enc["event_ms"] / args.steps
     tokens_per_s = enc["tokens_per_step"] / (ms_per_step * 1e-3)
-    launch_us, launch_flops = measure_full_diagonal_launch(ctx, max(2, args.steps // 4), 1)
-    achieved_tflops = launch_flops / (launch_us * 1e-6) / 1e12
-    log("encoder: %.3f ms/step (wall %.3f), %.0f tokens/s; full-diagonal launch %.2f us, %.1f TFLOP/s" %
-        (ms_per_step, enc["wall_ms"] / args.steps, tokens_per_s, launch_us, achieved_tflops))
+    launch_us = enc["avg_launch_us"]
+    achieved_tflops = enc["flops_per_launch"] / (launch_us * 1e-6) / 1e12
+    step_us, step_flops = measure_steady_state_step(ctx, max(2, args.steps // 4), 1)
+    log("encoder: %.3f ms/step (wall %.3f), %.0f tokens/s = %.1f TFLOP/s over the launch; one more time step costs "
+        "%.2f us = %.1f TFLOP/s" % (ms_per_step, enc["wall_ms"] / args.steps, tokens_per_s, achieved_tflops, step_us,
+                                    step_flops / (step_us * 1e-6) / 1e12))
+    # the same sweep as one launch per diagonal of the (layer, time) grid, for comparison
+    ctx.set_option(capi.ZR_OPT_LSTM_SWEEP, 1)
+    diag = bench_encoder(ctx, args.steps, args.warmup)
+    diag.pop("_keep")
+    ctx.set_option(capi.ZR_OPT_LSTM_SWEEP, 0)
+    log("encoder with one launch per diagonal: %.3f ms/step" % (diag["event_ms"] / args.steps))
 
     extra = {}
     if not args.no_extra:
@@ -447,13 +463,16 @@ def main():
         "config": {"workload": "config 2: 4-layer LSTM encoder forward, H=1000, minibatch 128, source length 50, "
                                "vocab 50000 (Zipf ids), fp32; one step = 200 layer-steps = 6400 tokens",
                    "tokens_per_step": enc["tokens_per_step"], "launches_per_step": enc["launches_per_step"]},
-        "roofline": {"bound": "mfma", "kernel": "lstm_fused_kernel", "achieved": round(achieved_tflops, 2),
+        "roofline": {"bound": "mfma", "kernel": "lstm_sweep_kernel", "achieved": round(achieved_tflops, 2),
                      "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved_tflops / PEAK_FP32_MFMA_TFLOPS, 4),
-                     "traffic": LSTM_FUSED_FULL_DIAGONAL_TRAFFIC_BYTES, "traffic_unit": "bytes per launch",
-                     "launch": "full diagonal: 4 units (one node of each layer), 256 workgroups",
-                     "avg_launch_us": round(launch_us, 2), "flops_per_launch": launch_flops,
-                     "algorithmic_bytes_per_launch": 4 * (2 * 4 * 1000 * 1000 + 3 * 1000 * 128 + 2 * 1000 * 128) * 4,
-                     "whole_sweep_avg_launch_us": round(enc["avg_launch_us"], 2)},
+                     "traffic": LSTM_SWEEP_TRAFFIC_BYTES, "traffic_unit": "bytes per launch",
+                     "launch": "whole sweep: 4 layers x 50 time steps = 200 nodes, 256 workgroups resident throughout "
+                               "(the pipeline of layers fills and drains inside the launch)",
+                     "avg_launch_us": round(launch_us, 2), "flops_per_launch": enc["flops_per_launch"],
+                     "algorithmic_bytes_per_launch": 200 * (2 * 4 * 1000 * 1000 + 3 * 1000 * 128 + 2 * 1000 * 128) * 4,
+                     "steady_state_step_us": round(step_us, 2),
+                     "steady_state_tflops": round(step_flops / (step_us * 1e-6) / 1e12, 2),
+                     "one_launch_per_diagonal_ms_per_step": round(diag["event_ms"] / args.steps, 4)},
         "cpu_baseline": cpu,
         "extra": extra,
     }

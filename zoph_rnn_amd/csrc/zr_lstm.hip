@@ -46,6 +46,7 @@ struct LstmLaunch {
   float* preact;            // non-null: store the four pre-activation sums ([4][H*mb], no bias) instead of the cell
   float clip;
   int j_tiles, n_tiles;
+  int buf_ok;               // host: H % 8 == 0 and every operand array is below 4 GiB (buffer-load variants)
   // K split ACROSS workgroups (SPLIT variant of lstm_fused_kernel): blockIdx.y = part of every segment's K range
   int kparts;
   float* partials;   // [tile][part][visit][gate][thread]
@@ -66,7 +67,9 @@ constexpr int lstm_prefetch_depth(int tn, int ks) {
 // SPLIT: the K range of every segment is also divided over gridDim.y workgroups (a single node cannot fill the chip
 // with whole-K tiles).  Each writes its tile of partial sums; the last to arrive at the tile's counter adds the parts
 // in part order -- the same order whoever is last, so results do not depend on timing -- and runs the cell epilogue.
-template <int TN, int KS, bool VEC, bool BF16 = false, bool XPK = false, bool SPLIT = false>
+// BUF: operands are fetched with buffer loads (zr_mma_segment_u): fp32 weights, 16-byte aligned activations,
+// H % 8 == 0 and every operand array below 4 GiB (the host checks).
+template <int TN, int KS, bool VEC, bool BF16 = false, bool XPK = false, bool SPLIT = false, bool BUF = false>
 __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
   __shared__ float red[KS * TN * 16 * 64];
   __shared__ int s_last;
@@ -159,6 +162,32 @@ __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
       } else {
         zr_mma_segment_bf16<4, TN, KS, (TN == 1 ? 6 : 4)>(acc, wbase, woff, (long long)L.ldw, xcol, H, kslice);
       }
+    } else if constexpr (BUF) {
+      // k-groups [g0, g1) of this segment (all of them unless K is also split across workgroups)
+      int g0 = 0, g1 = H >> 3;
+      if constexpr (SPLIT) {
+        const int groups = H >> 3, part = blockIdx.y;
+        g0 = (int)((long long)groups * part / L.kparts);
+        g1 = (int)((long long)groups * (part + 1) / L.kparts);
+      }
+      unsigned wsoff[4], xoffb[TN];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) wsoff[g] = (unsigned)((((long long)s * 4 + g) * HH + (long long)g0 * 8 * L.ldw) * 4);
+      const unsigned woffb = 16u * (unsigned)(j + half * L.ldw);
+      const bool packed = U.inp[s] != nullptr;
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) {
+        unsigned c = (unsigned)cols[tn];
+        if (s == 0 && U.gather_ids) {
+          int idv = U.gather_ids[cols[tn]];
+          c = (unsigned)(idv < 0 ? 0 : (idv >= U.V ? U.V - 1 : idv));
+        }
+        xoffb[tn] = packed ? 16u * ((unsigned)cols[tn] + (unsigned)(half * L.mb)) : 4u * (c * (unsigned)H + 4u * half);
+      }
+      const float* xb = packed ? U.inp[s] + (long long)g0 * 8 * L.mb : U.in[s] + g0 * 8;
+      zr_mma_segment_u<4, TN, KS, lstm_prefetch_depth(TN, KS)>(acc, zr_make_rsrc(U.W), wsoff, woffb, 32u * (unsigned)L.ldw,
+                                                               zr_make_rsrc(xb), xoffb,
+                                                               packed ? 32u * (unsigned)L.mb : 32u, (g1 - g0) * 8, kslice);
     } else {
       const float* wbase[4];
       unsigned woff[4];
@@ -764,7 +793,9 @@ int launch_fused_v(zr_ctx* ctx, const LstmLaunch& L, bool vec) {
       return zr_set_error(ZR_EINVAL, "bf16 weights: no kernel for column tile %d, K split %d", TN, KS);
     }
   }
-  if (vec)
+  if (vec && L.buf_ok)
+    lstm_fused_kernel<TN, KS, true, false, false, false, true><<<grid, 64 * KS, 0, ctx->stream>>>(L);
+  else if (vec)
     lstm_fused_kernel<TN, KS, true><<<grid, 64 * KS, 0, ctx->stream>>>(L);
   else
     lstm_fused_kernel<TN, KS, false><<<grid, 64 * KS, 0, ctx->stream>>>(L);
@@ -785,7 +816,10 @@ int launch_fused_split(zr_ctx* ctx, LstmLaunch& L, int parts) {
   L.partials = (float*)scratch;
   L.counters = ctx->d_counters;
   dim3 grid((unsigned)(((groups + 7) / 8) * 8 * L.n_tiles), (unsigned)parts);
-  lstm_fused_kernel<TN, 4, true, false, false, true><<<grid, 256, 0, ctx->stream>>>(L);
+  if (L.buf_ok)
+    lstm_fused_kernel<TN, 4, true, false, false, true, true><<<grid, 256, 0, ctx->stream>>>(L);
+  else
+    lstm_fused_kernel<TN, 4, true, false, false, true><<<grid, 256, 0, ctx->stream>>>(L);
   ZR_LAUNCH_CHECK("lstm_fused_kernel (K split across workgroups)");
   return ZR_OK;
 }
@@ -825,6 +859,13 @@ int launch_fused(zr_ctx* ctx, LstmLaunch& L, bool vec) {
   const int n32 = (L.mb + 31) / 32;
   L.nseg_max = 0;
   for (int i = 0; i < L.n_units; ++i) L.nseg_max = L.u[i].nseg > L.nseg_max ? L.u[i].nseg : L.nseg_max;
+  {
+    const long long lim = 1LL << 32;
+    bool ok = vec && !L.bf16 && (L.H & 7) == 0 && (long long)L.H * L.mb * 4 < lim &&
+              4LL * L.nseg_max * L.kp * L.ldw * 4 < lim;
+    for (int i = 0; i < L.n_units; ++i) ok = ok && (!L.u[i].gather_ids || (long long)L.u[i].V * L.H * 4 < lim);
+    L.buf_ok = ok ? 1 : 0;
+  }
   // Kernel choice.  The register-streaming kernel needs no cross-workgroup reduction and wins whenever it can put
   // a workgroup on (nearly) every CU -- a full diagonal of an encoder does.  A single node (a decoder step) gives
   // it only ceil(H/32) * ceil(mb/64) workgroups; there K is split across workgroups too: by the same kernel's SPLIT

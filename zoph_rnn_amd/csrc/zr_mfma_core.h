@@ -204,7 +204,7 @@ __device__ __forceinline__ void zr_mma_segment(zr_f32x16 (&acc)[TM][TN], const f
 // descriptors: an address is descriptor base (scalar registers) + a scalar byte offset that advances with k + a 32-bit
 // per-lane byte offset that stays fixed through the segment, so a load needs no vector address arithmetic at all
 // (64-bit vector adds would compete with the MFMAs for the vector issue slot).  Stages are pinned for the scheduler
-// (see PIN above).
+// (see PIN above) and, inside a stage, the loads are spread evenly among the MFMAs.
 //   wrsrc:    descriptor over the TM weight sub-tiles' matrices; wsoff[tm] = byte offset of sub-tile tm's matrix
 //   woffb:    this lane's byte offset into every weight sub-tile: 4 * (4*row + 4*half*lda)
 //   xrsrc:    descriptor over the activations
@@ -268,6 +268,17 @@ __device__ __forceinline__ void zr_mma_segment_u(zr_f32x16 (&acc)[TM][TN], __amd
         const int gl = kslice + (it + s + PF) * KS;
         load_full(f[(s + PF) % NS], gl < last ? gl : last);
         mma(f[s]);
+        {
+          // one load, then its share of the stage's MFMAs: a load issued while the matrix pipe works costs nothing,
+          // a run of loads leaves the pipe idle for as long as their issue takes
+          constexpr int NL = TM + TN, NM = 4 * TM * TN, PER = NM / NL;
+#pragma unroll
+          for (int q = 0; q < NL; ++q) {
+            __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);  // MFMA
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);    // vector memory read
+          }
+          __builtin_amdgcn_sched_group_barrier(0x008, NM - NL * PER, 0);
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
