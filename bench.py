@@ -28,9 +28,9 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E peak
 
 # HBM bytes per launch of lstm_sweep_kernel on the headline workload, from two rocprofv3 --pmc runs (FETCH_SIZE, then
 # WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for a plain copy of known size
-# (bench.py --calibrate-copy): FETCH_SIZE 0 KiB x 1.0 + WRITE_SIZE 0 KiB x 1.0.
+# (bench.py --calibrate-copy): FETCH_SIZE 3397743.8 KiB x 1.9706 + WRITE_SIZE 401518.3 KiB x 1.0000.
 # The summary of those runs is profiles/lstm_sweep_kernel_config2_hbm_traffic.txt.
-LSTM_SWEEP_TRAFFIC_BYTES = None
+LSTM_SWEEP_TRAFFIC_BYTES = int((3397743.8 * 1.9706 + 401518.3 * 1.0) * 1024)
 
 
 def log(*a):
