@@ -146,7 +146,10 @@ int zr_lstm_gates(zr_ctx* ctx, const float* d_preact, const float* const d_b[4],
 
 /* Whole stacked forward sweep (the time x layer loop of neuralMT_model::getError, src/model.hpp:1546-1621, and
  * forward_prop_source, :2367-2452): layer 0 gathers its input from d_embed by token id, layer l>0 reads layer
- * l-1's h_t.  Layers and time steps that do not depend on each other run in the same launch.
+ * l-1's h_t.  Nodes that do not depend on each other run side by side: either the whole sweep is ONE launch whose
+ * workgroups keep their tile of one layer for all T steps and hand h_t to each other through device memory (taken
+ * when they fill most of the GPU and are all resident at once; see ZR_OPT_LSTM_SWEEP), or one launch per diagonal
+ * l + t = d.  The single launch keeps its hand-over buffer and arrival counters in the context's scratch memory.
  *   d_ids_nonneg, d_mask01: time-major [b + t*mb] (src/fileHelper.h:488), outputs of zr_vocab_prep
  *   d_h0/d_c0: arrays of L device pointers (initial state per layer, H x mb) -- zeros for encoder / LM
  *   d_h_all/d_c_all: arrays of L device pointers, each T*H*mb floats: node t's h_t at offset t*H*mb */

@@ -614,6 +614,53 @@ def test_stack_forward_whole_sweep_launch(ctx, H, mb, T, L):
     assert np.all(out[2][0][:, :2, :, 1] == 0) and np.all(out[2][1][:, : T - 1, :, mb - 1] == 0)
 
 
+def test_whole_sweep_launch_keeps_gates_for_training(ctx):
+    """zr_lstm_stack_forward_train through the single-launch sweep: every node's four gate activations, h and c against
+    the oracle's node-by-node forward pass."""
+    g = synth.rng(22, 1)
+    H, mb, T, V, L = 96, 24, 5, 131, 2
+    embed = U(g, (H, V))
+    layers_np = [synth.lstm_layer(g, H, forget_bias_one=True) for _ in range(L)]
+    ids = g.integers(0, V, size=(T, mb)).astype(np.int32)
+    ids[:2, 3] = -1
+    n = H * mb
+    layers = [Layer(ctx, ly) for ly in layers_np]
+    d_nn, d_m = ctx.empty(ids.size, np.int32), ctx.empty(ids.size, np.int32)
+    ctx.vocab_prep(ctx.array(ids.reshape(-1)), ids.size, V, d_nn, d_m)
+    z = ctx.zeros((H, mb))
+    h_all = [ctx.empty((n * T,)) for _ in range(L)]
+    c_all = [ctx.empty((n * T,)) for _ in range(L)]
+    g_all = [ctx.empty((4 * n * T,)) for _ in range(L)]
+    ctx.set_option(capi.ZR_OPT_LSTM_SWEEP, 2)
+    try:
+        ctx.lstm_stack_forward_train([ly.w for ly in layers], ctx.array(embed), V, d_nn, d_m, T, mb, [z] * L, [z] * L,
+                                     h_all, c_all, g_all)
+        ctx.sync()
+    finally:
+        ctx.set_option(capi.ZR_OPT_LSTM_SWEEP, 0)
+    nn, m = o.vocab_prep(ids)
+    zero = np.zeros((H, mb), np.float32)
+    below = None
+    for l, ly in enumerate(layers_np):
+        hp, cp = zero, zero
+        outs = []
+        got_h = h_all[l].get().reshape(T, mb, H).transpose(0, 2, 1)
+        got_c = c_all[l].get().reshape(T, mb, H).transpose(0, 2, 1)
+        got_g = g_all[l].get().reshape(T, 4, mb, H).transpose(0, 1, 3, 2)
+        for t in range(T):
+            x = np.asfortranarray(embed[:, nn[t]]) if l == 0 else below[t]
+            want = o.lstm_step(ly["M"], ly["Wh"], ly["b"], x, hp, cp, m[t])
+            for gi, k in enumerate(("i", "f", "c_tilde", "o")):
+                assert_close(got_g[t, gi], want[k], what="gate %s layer %d step %d" % (k, l, t))
+            assert_close(got_h[t], want["h"], what="h layer %d step %d" % (l, t))
+            assert_close(got_c[t], want["c"], what="c layer %d step %d" % (l, t))
+            hp, cp = want["h"], want["c"]
+            outs.append(want["h"])
+        below = outs
+    for ly in layers:
+        ly.close()
+
+
 def test_whole_sweep_launch_back_to_back_with_different_inputs(ctx):
     """Two sweeps of the same shape with different data, back to back through the same hand-over buffers: the second
     must not see anything of the first (mb % 8 == 0: the consumers do not invalidate their caches inside the launch)."""

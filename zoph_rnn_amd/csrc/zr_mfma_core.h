@@ -66,10 +66,7 @@ struct ZrFrag {
 //              lines.  Packed activations require VEC and K % 8 == 0.
 // Rows / columns are pre-clamped by the caller so that out-of-range lanes read valid memory.
 // kslice must be wave-uniform.
-// PIN: stages are fenced off from each other for the instruction scheduler (each stage's loads stay next to its own
-// MFMAs).  Needed where the scheduler would otherwise gather the loads of a whole ring revolution at its end, which
-// drains the ring once per revolution.
-template <int TM, int TN, int KS, int PF, int AMODE, bool VEC, bool PIN = false>
+template <int TM, int TN, int KS, int PF, int AMODE, bool VEC>
 __device__ __forceinline__ void zr_mma_segment(zr_f32x16 (&acc)[TM][TN], const float* const (&wbase)[TM],
                                                const unsigned (&woff)[TM], long long lda,
                                                const float* const (&xcol)[TN], int K, int kslice, int half,
@@ -153,18 +150,6 @@ __device__ __forceinline__ void zr_mma_segment(zr_f32x16 (&acc)[TM][TN], const f
         const int gl = kslice + (it + s + PF) * KS;
         load_full(f[(s + PF) % NS], gl < last ? gl : last);
         mma(f[s]);
-        if (PIN) {
-          // one load, then its share of the stage's MFMAs: a run of back-to-back loads holds the wave's issue slot
-          // for longer than one MFMA lasts and leaves the matrix pipe idle behind it
-          constexpr int NL = TM + TN, NM = 4 * TM * TN;
-#pragma unroll
-          for (int q = 0; q < NL; ++q) {
-            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, NM / NL, 0);
-          }
-          __builtin_amdgcn_sched_group_barrier(0x008, NM - NL * (NM / NL), 0);
-          __builtin_amdgcn_sched_barrier(0);
-        }
       }
     }
     // at most PF groups remain, all of them already loaded
@@ -203,8 +188,10 @@ __device__ __forceinline__ void zr_mma_segment(zr_f32x16 (&acc)[TM][TN], const f
 // Variant of zr_mma_segment for k-interleaved weights and 16-byte activation loads that fetches through buffer
 // descriptors: an address is descriptor base (scalar registers) + a scalar byte offset that advances with k + a 32-bit
 // per-lane byte offset that stays fixed through the segment, so a load needs no vector address arithmetic at all
-// (64-bit vector adds would compete with the MFMAs for the vector issue slot).  Stages are pinned for the scheduler
-// (see PIN above) and, inside a stage, the loads are spread evenly among the MFMAs.
+// (64-bit vector adds would compete with the MFMAs for the vector issue slot).  The stages of the ring are fenced
+// off from each other for the instruction scheduler -- left alone it gathers the loads of a whole ring revolution
+// at its end, which drains the ring once per revolution -- and, inside a stage, the loads are spread evenly among
+// the MFMAs.
 //   wrsrc:    descriptor over the TM weight sub-tiles' matrices; wsoff[tm] = byte offset of sub-tile tm's matrix
 //   woffb:    this lane's byte offset into every weight sub-tile: 4 * (4*row + 4*half*lda)
 //   xrsrc:    descriptor over the activations
