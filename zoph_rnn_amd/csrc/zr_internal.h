@@ -68,6 +68,8 @@ int zr_set_error(int code, const char* fmt, ...);
   } while (0)
 
 int zr_bind_device(zr_ctx* ctx);
+// Number of contexts of this process that are alive on `device`.
+int zr_live_contexts(int device);
 // Returns a context-owned scratch buffer of at least `bytes` (slot 0 or 1).
 int zr_ctx_scratch(zr_ctx* ctx, int slot, size_t bytes, void** out);
 

@@ -1148,7 +1148,10 @@ int zr_lstm_stack_forward_train(zr_ctx* ctx, int nl, const zr_lstm_weights* cons
     else if ((long long)padded * ((n32 + 1) / 2) <= sweep_capacity<2>(ctx)) tn = 2;
     const int n_tiles = tn ? (n32 + tn - 1) / tn : 0;
     const long long tiles = (long long)groups * n_tiles;
-    const bool fills = tn && tiles * 10 >= 6LL * ctx->cu_count;
+    // Left to itself the library takes the single launch only when it fills most of the chip and this is the only
+    // context on the device: two such launches from two streams could each hold part of the CUs and wait for the
+    // rest (their bounded waits would end it, with an error).
+    const bool fills = tn && tiles * 10 >= 6LL * ctx->cu_count && zr_live_contexts(ctx->device) == 1;
     // the kernel addresses its operands as descriptor base + 32-bit byte offsets
     const long long lim = 1LL << 32;
     const bool offsets_fit = (long long)V * H * 4 < lim && (long long)n * 4 < lim &&

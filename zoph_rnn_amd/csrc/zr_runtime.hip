@@ -3,9 +3,16 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
+
 #include "zr_internal.h"
 
 static thread_local char g_err[512] = "";
+
+// live contexts per device in this process (zr_live_contexts)
+static std::atomic<int> g_live[64];
+
+int zr_live_contexts(int device) { return (device >= 0 && device < 64) ? g_live[device].load() : 2; }
 
 int zr_set_error(int code, const char* fmt, ...) {
   va_list ap;
@@ -72,6 +79,7 @@ int zr_ctx_create(int device, zr_ctx** out) {
   (void)hipMemset(c->d_flags, 0, (4 + ZR_MAX_COUNTERS) * sizeof(int));
   c->d_counters = c->d_flags + 4;
   c->lstm_fused = 1;
+  if (device < 64) g_live[device].fetch_add(1);
   *out = c;
   return ZR_OK;
 }
@@ -88,6 +96,7 @@ int zr_ctx_destroy(zr_ctx* ctx) {
   if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
   if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);
   (void)hipStreamDestroy(ctx->own_stream);
+  if (ctx->device >= 0 && ctx->device < 64) g_live[ctx->device].fetch_sub(1);
   delete ctx;
   return ZR_OK;
 }
