@@ -561,8 +561,9 @@ __global__ void __launch_bounds__(64 * NWV) lstm_lds_kernel(LstmLaunch2 P) {
 // over t itself.  Node (l, t) needs h of (l-1, t) and of (l, t-1), each produced by the j_tiles workgroups that own
 // the same batch columns of that layer: every (layer, column tile) has an arrival counter in device memory that its
 // producers bump once per time step, and a consumer waits until the counter reaches (steps needed) * j_tiles.  The
-// layers settle into a skewed pipeline: the input from below is consumed first and the recurrent input second, so the
-// hand-over latency of a layer's own h hides behind half a K loop, and a layer never waits for the layer above it.
+// layers settle into a skewed pipeline: a layer above the first consumes its recurrent input first and the input from
+// below second, so it trails the layer below by half a step and that hand-over hides behind half a K loop; a layer
+// never waits for the layer above it.
 // Compared with one launch per diagonal this removes, per step, the launch, the drain of the slowest tile and the
 // refill of the operand pipeline from a cold start; the cell state never leaves registers.
 //
@@ -715,8 +716,13 @@ __global__ void __launch_bounds__(256) lstm_sweep_kernel(LstmSweep P) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[g][tn][r] = 0.0f;
 
-    for (int s = 0; s < 2; ++s) {
-      // segment 0: input from below (h of (l-1, t), or the embedding columns); segment 1: h of (l, t-1)
+    for (int q = 0; q < 2; ++q) {
+      // segment 0: input from below (h of (l-1, t), or the embedding columns); segment 1: h of (l, t-1).  Layers above
+      // the first take the recurrent segment first: it only needs the layer's own previous step, so a layer can trail
+      // the one below it by half a step instead of a whole one (the pipeline of layers fills and drains in half the
+      // time) and the wait for the layer below hides behind half a K loop.  The order is fixed per layer, so the
+      // summation order, and with it every bit of the result, does not depend on timing.
+      const int s = (l > 0) ? 1 - q : q;
       const bool packed = (s == 0) ? (l > 0) : (t > 0);
       if (packed) {
         int* ctr = (s == 0) ? below_ctr : my_ctr;
