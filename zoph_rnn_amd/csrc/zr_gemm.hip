@@ -311,8 +311,9 @@ __global__ void __launch_bounds__(256) gemm_rows_kernel(GemmArgs a, int row_chun
 // parked in LDS (double buffered, one barrier per chunk) and multiplied by every wave, while each wave fetches
 // only its own 32 activation columns.  Against one 32x32 tile per wave this cuts the bytes pulled through the
 // CU's L1 per flop by about TMR, which is what limited the softmax-logits GEMM (V x H times H x mb).
-// Loads are unconditional with clamped addresses (see zr_mfma_core.h on why); out-of-range weights are zeroed
-// by multiplication.  Requires: no transpose, one K segment, M, lda, ldb multiples of 4, 16-byte aligned bases.
+// Loads are unconditional (see zr_mfma_core.h on why) buffer loads whose descriptors end at the last valid element,
+// so out-of-range weights read as zeros.  Requires: no transpose, one K segment, K a multiple of 8, M, lda, ldb
+// multiples of 4, 16-byte aligned bases, both operands below 4 GiB.
 // ---------------------------------------------------------------------------------------------------------
 template <int TMR, int NWV, int EPI>
 __global__ void __launch_bounds__(64 * NWV) gemm_lds_kernel(GemmArgs a) {
@@ -337,20 +338,25 @@ __global__ void __launch_bounds__(64 * NWV) gemm_lds_kernel(GemmArgs a) {
 
   int col = n0 + jl;
   col = col < a.N ? col : a.N - 1;
-  const float* xcol = a.B[0] + (long long)col * a.ldb[0];
+  // Operands come through buffer descriptors: address = base + a scalar byte offset that advances with the chunk +
+  // a per-thread byte offset fixed for the whole loop, so the loop holds no vector address arithmetic.  The
+  // descriptors end exactly at the last valid element: a read past it (the K tail of the last chunk, the dummy chunk
+  // of an odd chunk count) returns zeros, which is what those weights must be.  Rows past M are clamped to valid
+  // rows instead; what they produce lands in output rows that are never stored.  Requires K % 8 == 0 (host-checked).
+  const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float*>(A), 0, (int)(unsigned)((((long long)K - 1) * lda + M) * 4), 0x00020000);
+  const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float*>(a.B[0]), 0, (int)(unsigned)((((long long)a.N - 1) * a.ldb[0] + K) * 4), 0x00020000);
+  const unsigned xoffb = 4u * ((unsigned)col * (unsigned)a.ldb[0] + 4u * (unsigned)half);
 
-  const float* wsrc[WLD];
-  float wkeep[WLD];
-  int wkk[WLD];
+  unsigned woffb[WLD];
 #pragma unroll
   for (int u = 0; u < WLD; ++u) {
     const int f = tid + NTHR * u;
     const int fc = f < F4 ? f : F4 - 1;
     const int j4 = fc & 7, tm = (fc >> 3) % TMR, kk = fc / (8 * TMR);
     const int row = m0 + 32 * tm + 4 * j4;
-    wkeep[u] = (row < M && f < F4) ? 1.0f : 0.0f;
-    wkk[u] = kk;
-    wsrc[u] = A + (row < M ? row : M - 4);
+    woffb[u] = 4u * ((unsigned)(row < M ? row : M - 4) + (unsigned)kk * (unsigned)lda);
   }
 
   zr_f32x16 acc[TMR];
@@ -359,38 +365,35 @@ __global__ void __launch_bounds__(64 * NWV) gemm_lds_kernel(GemmArgs a) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[tm][r] = 0.0f;
 
-  zr_f32x4 wreg[WLD];
+  zr_u32x4v wreg[WLD];
   zr_f32x4 xf[2][4];
-  // gload only issues loads (raw values stay in registers while the current chunk is multiplied); the zeroing of
-  // out-of-range weights happens in lds_store, so that no instruction consumes a loaded value right after its
-  // load and several loads stay in flight.
+  // gload only issues loads (the values stay in registers while the current chunk is multiplied) so that several
+  // loads stay in flight.
   auto gload = [&](int c, zr_f32x4 (&xdst)[4]) {
-    const int cc = c < n_chunks ? c : n_chunks - 1;
+    const unsigned wso = (unsigned)c * (unsigned)(KC * 4) * (unsigned)lda;
 #pragma unroll
-    for (int u = 0; u < WLD; ++u) {
-      const int k = cc * KC + wkk[u];
-      const int kc = k < K ? k : K - 1;
-      wreg[u] = *(const zr_f32x4*)(wsrc[u] + (long long)kc * lda);
-    }
+    for (int u = 0; u < WLD; ++u)  // the scalar-offset operand is exempt from the range check: add it on the vector side
+      wreg[u] = __builtin_amdgcn_raw_buffer_load_b128(wrsrc, (int)(woffb[u] + wso), 0, 0);
 #pragma unroll
     for (int gq = 0; gq < 4; ++gq) {
-      int kx = cc * KC + 8 * gq + 4 * half;
-      kx = (kx + 4 <= K) ? kx : K - 4;
-      xdst[gq] = *(const zr_f32x4*)(xcol + kx);
+      int kx = c * KC + 8 * gq;
+      kx = kx + 8 <= K ? kx : K - 8;  // wave-uniform: the weights of the k values this replaces are zeros
+      const zr_u32x4v v = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, (int)(xoffb + (unsigned)kx * 4u), 0, 0);
+      xdst[gq].x = __uint_as_float(v.x);
+      xdst[gq].y = __uint_as_float(v.y);
+      xdst[gq].z = __uint_as_float(v.z);
+      xdst[gq].w = __uint_as_float(v.w);
     }
   };
-  auto lds_store = [&](int buf, int c) {
-    const float chunk_keep = c < n_chunks ? 1.0f : 0.0f;  // dummy chunk of an odd chunk count: all zeros
-    const int cc = c < n_chunks ? c : n_chunks - 1;
+  auto lds_store = [&](int buf, int) {
 #pragma unroll
     for (int u = 0; u < WLD; ++u) {
       const int f = tid + NTHR * u;
-      const float keep = ((cc * KC + wkk[u]) < K ? wkeep[u] : 0.0f) * chunk_keep;
-      zr_f32x4 v = wreg[u];
-      v.x *= keep;
-      v.y *= keep;
-      v.z *= keep;
-      v.w *= keep;
+      zr_f32x4 v;
+      v.x = __uint_as_float(wreg[u].x);
+      v.y = __uint_as_float(wreg[u].y);
+      v.z = __uint_as_float(wreg[u].z);
+      v.w = __uint_as_float(wreg[u].w);
       if (f < F4) Ws4[buf][f] = v;
     }
   };
@@ -798,7 +801,8 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
   }
   // Large, untransposed, single-segment products with a wide batch (the softmax logits): LDS-shared weights.
   const bool lds_ok = !d.trans_a && d.nseg == 1 && d.batch == 1 && vec && (d.M % 4 == 0) && (d.lda[0] % 4 == 0) &&
-                      (((uintptr_t)d.A[0] & 15u) == 0) && d.K[0] >= 8 && d.M >= 2048 && d.N >= 96 &&
+                      (((uintptr_t)d.A[0] & 15u) == 0) && d.K[0] >= 8 && d.K[0] % 8 == 0 && d.M >= 2048 && d.N >= 96 &&
+                      ((long long)d.K[0] + 64) * d.lda[0] * 4 < (1LL << 32) && (long long)d.N * d.ldb[0] * 4 < (1LL << 32) &&
                       (d.epilogue == ZR_EPI_STORE || d.epilogue == ZR_EPI_SOFTMAX_PARTIAL);
   if (lds_ok && ctx->gemm_cfg == 10) return launch_lds<4, 4>(ctx, ga, d.epilogue);
   if (lds_ok && (ctx->gemm_cfg == 0 || ctx->gemm_cfg == 9)) {
