@@ -49,6 +49,28 @@ def test_vocab_prep_and_gather_bit_exact(ctx):
         assert d_x.get().tobytes() == o.embed_gather(W, gids).tobytes()
 
 
+@pytest.mark.parametrize("Hh,n", [(1000, 1500), (260, 1024), (2052, 1100), (4, 2000)])
+def test_gather_many_columns_bit_exact(ctx, Hh, n):
+    """1024 columns and more take the one-wave-per-column kernel: column lengths below, at and above one 1024-float
+    pass, duplicates, first and last column of the table."""
+    g = synth.rng(23, Hh + n)
+    V = 777
+    W = U(g, (Hh, V))
+    ids = g.integers(0, V, size=n).astype(np.int32)
+    ids[:4] = [0, V - 1, 5, 5]
+    d_x = ctx.empty((Hh, n))
+    ctx.embed_gather(ctx.array(W), Hh, V, ctx.array(ids), n, d_x)
+    ctx.sync()
+    assert d_x.get().tobytes() == o.embed_gather(W, ids).tobytes()
+    bad = ids.copy()
+    bad[n // 2] = V + 3
+    ctx.embed_gather(ctx.array(W), Hh, V, ctx.array(bad), n, d_x)
+    with pytest.raises(capi.ZrError):
+        ctx.sync()
+    want = o.embed_gather(W, np.minimum(bad, V - 1))
+    assert d_x.get().tobytes() == want.tobytes()
+
+
 def test_gather_out_of_range_id_is_reported_not_fatal(ctx):
     W = np.asfortranarray(np.arange(12, dtype=np.float32).reshape(4, 3, order="F"))
     d_x = ctx.empty((4, 2))

@@ -74,6 +74,37 @@ column_copy_kernel(const float* __restrict__ src, int H, int V, const int* __res
   }
 }
 
+// Many columns: a 64-lane wave copies one whole column, four 16-byte loads in flight per lane before the first store
+// (a quarter of the workgroups of column_copy_kernel and four times the bytes in flight per wave).
+__global__ void __launch_bounds__(256)
+column_copy_wide_kernel(const float* __restrict__ src, int H, int V, const int* __restrict__ col_ids, int fixed_col,
+                        int n_cols, float* __restrict__ dst, int* __restrict__ flags) {
+  const int col = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (col >= n_cols) return;
+  const int lane = threadIdx.x & 63;
+  int sc = col_ids ? col_ids[col] : fixed_col;
+  if (V > 0 && (sc < 0 || sc >= V)) {
+    if (lane == 0) atomicAdd(&flags[0], 1);
+    sc = sc < 0 ? 0 : V - 1;
+  }
+  const zr_f32x4* s = (const zr_f32x4*)(src + (size_t)sc * H);
+  zr_f32x4* d = (zr_f32x4*)(dst + (size_t)col * H);
+  const int n4 = H >> 2;
+  for (int base = 0; base < n4; base += 256) {
+    zr_f32x4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int i4 = base + u * 64 + lane;
+      v[u] = s[i4 < n4 ? i4 : n4 - 1];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int i4 = base + u * 64 + lane;
+      if (i4 < n4) d[i4] = v[u];
+    }
+  }
+}
+
 // The same copy for up to kMaxMulti arrays at once (blockIdx.z picks the array): the per-layer state reorders of a
 // decode step are each far too small to fill the chip, so they share one launch.
 constexpr int kMaxMulti = 32;
@@ -218,7 +249,9 @@ static int column_copy(zr_ctx* ctx, const char* who, const float* src, int H, in
   ZR_CHECK_ARG(n <= 65535, "%s: at most 65535 columns per call (got %d)", who, n);
   if (n == 0) return ZR_OK;
   const bool vec = (H % 4 == 0) && aligned16(src) && aligned16(dst);
-  if (vec) {
+  if (vec && n >= 1024) {
+    column_copy_wide_kernel<<<(n + 3) / 4, 256, 0, ctx->stream>>>(src, H, V, ids, fixed_col, n, dst, ctx->d_flags);
+  } else if (vec) {
     dim3 grid((H / 4 + 63) / 64, n);
     column_copy_kernel<true><<<grid, 64, 0, ctx->stream>>>(src, H, V, ids, fixed_col, dst, ctx->d_flags);
   } else {
