@@ -21,6 +21,10 @@ struct zr_lstm_train {
   // [2][H x 4H] column-major: the TRANSPOSE of Wh stacked over the gates, then of M: element (k, g*H + j) = W_g[j][k].
   // The error products sum_g W_g^T err_g are then plain products with contiguous weight rows.
   float* d_stack;
+  // the same two matrices in the matrix cores' k-interleaved layout ([kp/4][ldp][4], ldp = H rounded up to 32,
+  // kp = 4H rounded up to 8), kp*ldp floats each: the operand of the whole-grid backward sweep
+  float* d_stack_pack;
+  int ldp, kp;
 };
 
 namespace {
@@ -87,6 +91,42 @@ __global__ void __launch_bounds__(256) lstm_node_backward_kernel(
   d[2 * (size_t)H] = ec * gi * (1.0f - gc * gc);
   d[3 * (size_t)H] = eh * th * go * (1.0f - go);
   ec_out[ix] = ec * gf;
+}
+
+// The same for up to 8 independent nodes in one launch (blockIdx.z picks the node).
+struct NodeBackwardGroup {
+  const float* gates[8];      // node's four gate planes, H*mb apart
+  const float* c[8];
+  const float* cprev[8];
+  const int* mask01[8];
+  const float* err_above[8];  // may be null
+  const float* err_next[8];   // may be null
+  float* ec[8];               // cell error, updated in place
+  float* dg[8];
+};
+__global__ void __launch_bounds__(256) lstm_node_backward_group_kernel(NodeBackwardGroup G, int H, int mb) {
+  const int u = blockIdx.z;
+  const int b = blockIdx.y;
+  const int j = blockIdx.x * 256 + threadIdx.x;
+  if (j >= H) return;
+  const size_t n = (size_t)H * mb;
+  const size_t ix = (size_t)b * H + j;
+  const float m = (float)G.mask01[u][b];
+  float eh = 0.0f;
+  if (G.err_above[u]) eh += G.err_above[u][ix];
+  if (G.err_next[u]) eh += G.err_next[u][ix];
+  eh *= m;
+  const float* gt = G.gates[u];
+  const float gi = gt[ix], gf = gt[n + ix], gc = gt[2 * n + ix], go = gt[3 * n + ix];
+  const float th = tanhf(G.c[u][ix]);
+  const float errt_ct = eh * go * (1.0f - th * th);
+  const float ec = (G.ec[u][ix] + errt_ct) * m;
+  float* d = G.dg[u] + (size_t)b * 4 * H + j;
+  d[0] = ec * gc * gi * (1.0f - gi);
+  d[H] = ec * G.cprev[u][ix] * gf * (1.0f - gf);
+  d[2 * (size_t)H] = ec * gi * (1.0f - gc * gc);
+  d[3 * (size_t)H] = eh * th * go * (1.0f - go);
+  G.ec[u][ix] = ec * gf;
 }
 
 // Sum over the unmasked columns of log((double) p[target, column]): train_perplexity_kernel
@@ -247,9 +287,14 @@ int zr_lstm_train_create(zr_ctx* ctx, const float* const d_M[4], const float* co
   zr_lstm_train* w = new zr_lstm_train();
   w->H = H;
   w->d_stack = nullptr;
+  w->d_stack_pack = nullptr;
+  w->ldp = (H + 31) / 32 * 32;
+  w->kp = (4 * H + 7) / 8 * 8;
   const size_t per = 4 * (size_t)H * H;
-  if (hipMalloc((void**)&w->d_stack, sizeof(float) * 2 * per) != hipSuccess) {
+  if (hipMalloc((void**)&w->d_stack, sizeof(float) * 2 * per) != hipSuccess ||
+      hipMalloc((void**)&w->d_stack_pack, sizeof(float) * 2 * (size_t)w->kp * w->ldp) != hipSuccess) {
     (void)hipGetLastError();
+    if (w->d_stack) (void)hipFree(w->d_stack);
     delete w;
     return zr_set_error(ZR_ENOMEM, "zr_lstm_train_create: allocation failed (H = %d)", H);
   }
@@ -268,6 +313,11 @@ int zr_lstm_train_refresh(zr_ctx* ctx, zr_lstm_train* w, const float* const d_M[
   ZR_LAUNCH_CHECK("stack_gates_kernel");
   stack_gates_kernel<<<grid, 256, 0, ctx->stream>>>(d_M[0], d_M[1], d_M[2], d_M[3], H, w->d_stack + per);
   ZR_LAUNCH_CHECK("stack_gates_kernel");
+  for (int z = 0; z < 2; ++z) {
+    rc = zr_pack4_launch(ctx, w->d_stack + z * per, H, 4 * H, H, w->ldp, w->kp,
+                         w->d_stack_pack + (size_t)z * w->kp * w->ldp);
+    if (rc) return rc;
+  }
   return ZR_OK;
 }
 
@@ -277,6 +327,7 @@ int zr_lstm_train_destroy(zr_ctx* ctx, zr_lstm_train* w) {
   if (rc) return rc;
   ZR_HIP(hipStreamSynchronize(ctx->stream));
   if (w->d_stack) (void)hipFree(w->d_stack);
+  if (w->d_stack_pack) (void)hipFree(w->d_stack_pack);
   delete w;
   return ZR_OK;
 }
@@ -312,61 +363,90 @@ int zr_lstm_stack_backward(zr_ctx* ctx, int nl, const zr_lstm_train* const layer
                  "zr_lstm_stack_backward: null buffer for layer %d", l);
   }
   const size_t n = (size_t)H * mb;
-  // work: per layer [2][H x mb] = (error to h_{t-1}, error to the layer below), the two outputs of the batched
-  // product; the cell error lives in d_err_c0[l] (updated in place step by step)
+  // The grid is walked by anti-diagonals d = l + t, highest first: node (l, t) needs the errors of (l+1, t) and
+  // (l, t+1), both on diagonal d+1, so the nodes of a diagonal are independent and share two launches (the gate
+  // derivatives of all of them, then all their error products as one grouped GEMM).
+  // work: two sets (diagonal parity) of per-layer [2][H x mb] = (error to h_{t-1}, error to the layer below): a
+  // node reads what diagonal d+1 wrote into the other set while its neighbours on diagonal d write this one.  The
+  // cell error lives in d_err_c0[l] (updated in place step by step; one node per layer and diagonal touches it).
   void* scratch = nullptr;
-  rc = zr_ctx_scratch(ctx, 1, sizeof(float) * 2 * n * nl, &scratch);
+  rc = zr_ctx_scratch(ctx, 1, sizeof(float) * 4 * n * nl, &scratch);
   if (rc) return rc;
   float* work = (float*)scratch;
+  auto wk = [&](int d, int l) { return work + ((size_t)(d & 1) * nl + l) * 2 * n; };
   for (int l = 0; l < nl; ++l) {
+    // node (l, T-1) is on diagonal l + T - 1 and reads its "next step" error from the set of diagonal l + T
+    float* first = wk(l + T, l);
     if (d_err_hT && d_err_hT[l])
-      ZR_HIP(hipMemcpyAsync(work + (size_t)l * 2 * n, d_err_hT[l], sizeof(float) * n, hipMemcpyDeviceToDevice, ctx->stream));
-    else
-      ZR_HIP(hipMemsetAsync(work + (size_t)l * 2 * n, 0, sizeof(float) * n, ctx->stream));
+      ZR_HIP(hipMemcpyAsync(first, d_err_hT[l], sizeof(float) * n, hipMemcpyDeviceToDevice, ctx->stream));
+    else {
+      rc = zr_memset_zero(ctx, first, sizeof(float) * n);
+      if (rc) return rc;
+    }
     if (d_err_cT && d_err_cT[l])
       ZR_HIP(hipMemcpyAsync(d_err_c0[l], d_err_cT[l], sizeof(float) * n, hipMemcpyDeviceToDevice, ctx->stream));
-    else
-      ZR_HIP(hipMemsetAsync(d_err_c0[l], 0, sizeof(float) * n, ctx->stream));
+    else {
+      rc = zr_memset_zero(ctx, d_err_c0[l], sizeof(float) * n);
+      if (rc) return rc;
+    }
   }
-  const size_t per = 4 * (size_t)H * H;
-  dim3 egrid((H + 255) / 256, mb);
-  for (int t = T - 1; t >= 0; --t) {
-    for (int l = nl - 1; l >= 0; --l) {
-      float* w_l = work + (size_t)l * 2 * n;
-      const float* above = (l == nl - 1) ? d_err_top + (size_t)t * n : work + (size_t)(l + 1) * 2 * n + n;
-      float* dg = d_dgates_all[l] + (size_t)t * 4 * n;
-      const float* cprev = (t == 0) ? d_c0[l] : d_c_all[l] + (size_t)(t - 1) * n;
-      const float* gt = d_gates_all[l] + (size_t)t * 4 * n;
-      lstm_node_backward_kernel<<<egrid, 256, 0, ctx->stream>>>(gt, gt + n, gt + 2 * n, gt + 3 * n,
-                                                                d_c_all[l] + (size_t)t * n, cprev,
-                                                                d_mask01 + (size_t)t * mb, above, w_l, d_err_c0[l],
-                                                                d_err_c0[l], H, mb, dg);
-      ZR_LAUNCH_CHECK("lstm_node_backward_kernel");
-      // (error to h_{t-1}, error to below) = (Wh_stack^T, M_stack^T) * dg : one batched product, shared right side
+  const bool packed_ok = (H % 4 == 0) && layers[0]->d_stack_pack != nullptr;
+  for (int d = nl + T - 2; d >= 0; --d) {
+    for (int lhi = nl - 1; lhi >= 0; lhi -= 8) {  // at most 8 nodes per launch
+      NodeBackwardGroup G = {};
       ZrGemmDesc g = {};
+      int nu = 0;
+      for (int l = lhi; l >= 0 && l > lhi - 8; --l) {
+        const int t = d - l;
+        if (t < 0 || t >= T) continue;
+        float* w_l = wk(d, l);
+        G.gates[nu] = d_gates_all[l] + (size_t)t * 4 * n;
+        G.c[nu] = d_c_all[l] + (size_t)t * n;
+        G.cprev[nu] = (t == 0) ? d_c0[l] : d_c_all[l] + (size_t)(t - 1) * n;
+        G.mask01[nu] = d_mask01 + (size_t)t * mb;
+        G.err_above[nu] = (l == nl - 1) ? d_err_top + (size_t)t * n : wk(d + 1, l + 1) + n;
+        G.err_next[nu] = wk(d + 1, l);
+        G.ec[nu] = d_err_c0[l];
+        G.dg[nu] = d_dgates_all[l] + (size_t)t * 4 * n;
+        g.gA[nu] = packed_ok ? layers[l]->d_stack_pack : layers[l]->d_stack;
+        g.gB[nu] = G.dg[nu];
+        g.gC[nu] = w_l;
+        ++nu;
+      }
+      if (nu == 0) continue;
+      dim3 egrid((H + 255) / 256, mb, nu);
+      lstm_node_backward_group_kernel<<<egrid, 256, 0, ctx->stream>>>(G, H, mb);
+      ZR_LAUNCH_CHECK("lstm_node_backward_group_kernel");
+      // (error to h_{t-1}, error to below) = (Wh_stack^T, M_stack^T) * dg for every node: batch of 2 inside a group
+      g.groups = nu;
       g.M = H;
       g.N = mb;
       g.nseg = 1;
       g.K[0] = 4 * H;
-      g.A[0] = layers[l]->d_stack;
-      g.lda[0] = H;
-      g.B[0] = dg;
       g.ldb[0] = 4 * H;
-      g.C = w_l;
       g.ldc = H;
       g.batch = 2;
-      g.strideA = (long long)per;
       g.strideC = (long long)n;
       g.epilogue = ZR_EPI_STORE;
+      if (packed_ok) {
+        g.a_pack = 1;
+        g.lda[0] = layers[0]->ldp;
+        g.strideA = (long long)layers[0]->kp * layers[0]->ldp;
+      } else {
+        g.lda[0] = H;
+        g.strideA = 4LL * H * H;
+      }
       rc = zr_gemm_launch(ctx, g);
       if (rc) return rc;
-      if (l == 0 && d_err_below0)
-        ZR_HIP(hipMemcpyAsync(d_err_below0 + (size_t)t * n, w_l + n, sizeof(float) * n, hipMemcpyDeviceToDevice,
-                              ctx->stream));
     }
+    const int t0 = d;  // layer 0's node on this diagonal
+    if (d_err_below0 && t0 < T)
+      ZR_HIP(hipMemcpyAsync(d_err_below0 + (size_t)t0 * n, wk(d, 0) + n, sizeof(float) * n, hipMemcpyDeviceToDevice,
+                            ctx->stream));
   }
+  // node (l, 0) is on diagonal l
   for (int l = 0; l < nl; ++l)
-    ZR_HIP(hipMemcpyAsync(d_err_h0[l], work + (size_t)l * 2 * n, sizeof(float) * n, hipMemcpyDeviceToDevice, ctx->stream));
+    ZR_HIP(hipMemcpyAsync(d_err_h0[l], wk(l, l), sizeof(float) * n, hipMemcpyDeviceToDevice, ctx->stream));
   return ZR_OK;
 }
 

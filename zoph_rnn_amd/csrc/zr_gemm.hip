@@ -27,6 +27,11 @@ struct GemmArgs {
   // k-interleaved by 8 ([K/8][N][8]); see zr_split_pack_x_kernel
   const unsigned short* Blo[3];
   int accum;  // ZR_EPI_STORE only: C += result instead of C = result
+  // groups > 0: blockIdx.z = group * batch + batch index; the group picks A, B and C from these tables
+  int groups, batch;
+  const float* gA[8];
+  const float* gB[8];
+  float* gC[8];
 };
 
 // largest divisor c of nv with c * tm <= 32
@@ -66,6 +71,18 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& a, int m0, int n0, boo
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[tm][tn][r] = 0.0f;
 
+  // several problems in one launch: the group picks the operands, z becomes the batch index inside the group
+  const float* grpA = nullptr;
+  const float* grpB = nullptr;
+  float* grpC = nullptr;
+  if (a.groups) {
+    const int grp = z / a.batch;
+    z -= grp * a.batch;
+    grpA = a.gA[grp];
+    grpB = a.gB[grp];
+    grpC = a.gC[grp];
+  }
+
   for (int s = 0; s < a.nseg; ++s) {
     if constexpr (AMODE == ZR_A_PACK8_BF16) {
       const unsigned short* wbase[TM];
@@ -85,7 +102,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& a, int m0, int n0, boo
       }
       zr_mma_segment_bf16<TM, TN, KS, PF, true>(acc, wbase, woff, a.lda[s], xcol, a.K[s], kslice, xlo, a.N);
     } else {
-      const float* A = a.A[s] + (long long)z * a.strideA;
+      const float* A = (grpA ? grpA : a.A[s]) + (long long)z * a.strideA;
+      const float* Bs = grpB ? grpB : a.B[s];
       const float* wbase[TM];
       unsigned woff[TM];
       const float* xcol[TN];
@@ -98,14 +116,14 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& a, int m0, int n0, boo
       }
 #pragma unroll
       for (int tn = 0; tn < TN; ++tn)
-        xcol[tn] = (AMODE == ZR_A_PACK4 && a.b_pack4) ? a.B[s] + 4LL * cols[tn] + 4LL * half * a.N
-                                                     : a.B[s] + (long long)cols[tn] * a.ldb[s] + 4 * half;
+        xcol[tn] = (AMODE == ZR_A_PACK4 && a.b_pack4) ? Bs + 4LL * cols[tn] + 4LL * half * a.N
+                                                     : Bs + (long long)cols[tn] * a.ldb[s] + 4 * half;
       zr_mma_segment<TM, TN, KS, PF, AMODE, VEC>(acc, wbase, woff, a.lda[s], xcol, a.K[s], kslice, half,
                                                  (AMODE == ZR_A_PACK4 && a.b_pack4) ? a.N : 1);
     }
   }
 
-  float* C = a.C + (long long)z * a.strideC;
+  float* C = (grpC ? grpC : a.C) + (long long)z * a.strideC;
   const float* bias = a.bias ? a.bias + (long long)z * a.strideBias : nullptr;
 
   if (EPI == ZR_EPI_SOFTMAX_PARTIAL) {
@@ -563,11 +581,11 @@ int launch_cfg(zr_ctx* ctx, GemmArgs& ga, int batch, int epi, bool trans_a, bool
 
 // k-interleaved weights: one wave tile per workgroup, K split over its 4 waves
 template <int TM, int TN, int OCC>
-int launch_pack4(zr_ctx* ctx, GemmArgs& ga, int epi, bool vec) {
+int launch_pack4(zr_ctx* ctx, GemmArgs& ga, int epi, bool vec, int zcount) {
   ga.m_tiles = (ga.M + 32 * TM - 1) / (32 * TM);
   ga.n_tiles = (ga.N + 32 * TN - 1) / (32 * TN);
-  if (vec) return launch_epi<TM, TN, 4, 1, ZR_A_PACK4, true, OCC>(ctx, ga, 1, epi);
-  return launch_epi<TM, TN, 4, 1, ZR_A_PACK4, false, OCC>(ctx, ga, 1, epi);
+  if (vec) return launch_epi<TM, TN, 4, 1, ZR_A_PACK4, true, OCC>(ctx, ga, zcount, epi);
+  return launch_epi<TM, TN, 4, 1, ZR_A_PACK4, false, OCC>(ctx, ga, zcount, epi);
 }
 
 // Activations X (K x N, column n at src + n*ld) into [K/4][N][4]; K % 4 == 0.  One thread per float4.
@@ -670,9 +688,24 @@ int zr_pack4_launch(zr_ctx* ctx, const float* src, int M, int K, long long ld, i
 int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
   ZR_CHECK_ARG(d.M > 0 && d.N > 0, "gemm: M = %d, N = %d", d.M, d.N);
   ZR_CHECK_ARG(d.nseg >= 1 && d.nseg <= 3, "gemm: nseg = %d", d.nseg);
-  ZR_CHECK_ARG(d.C != nullptr && d.ldc >= d.M, "gemm: C null or ldc %d < M %d", d.ldc, d.M);
+  ZR_CHECK_ARG((d.groups > 0 || d.C != nullptr) && d.ldc >= d.M, "gemm: C null or ldc %d < M %d", d.ldc, d.M);
   ZR_CHECK_ARG(d.batch >= 1 && d.batch <= 65535, "gemm: batch = %d", d.batch);
+  ZR_CHECK_ARG(d.groups >= 0 && d.groups <= 8, "gemm: groups = %d", d.groups);
+  if (d.groups > 0) {
+    ZR_CHECK_ARG(d.nseg == 1 && d.epilogue == ZR_EPI_STORE && !d.bias && d.a_pack != 2 && d.batch * d.groups <= 65535,
+                 "gemm: grouped problems take one segment, the plain store epilogue, no bias and fp32 operands");
+    for (int g = 0; g < d.groups; ++g)
+      ZR_CHECK_ARG(d.gA[g] && d.gB[g] && d.gC[g], "gemm: null operand in group %d", g);
+  }
   GemmArgs ga;
+  ga.groups = d.groups;
+  ga.batch = d.batch;
+  for (int g = 0; g < 8; ++g) {
+    ga.gA[g] = g < d.groups ? d.gA[g] : nullptr;
+    ga.gB[g] = g < d.groups ? d.gB[g] : nullptr;
+    ga.gC[g] = g < d.groups ? d.gC[g] : nullptr;
+  }
+  const int zcount = d.batch * (d.groups > 0 ? d.groups : 1);  // grid depth
   ga.M = d.M;
   ga.N = d.N;
   ga.nseg = d.nseg;
@@ -681,10 +714,11 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
   for (int s = 0; s < 3; ++s) {
     if (s < d.nseg) {
       ZR_CHECK_ARG(d.K[s] > 0, "gemm: K[%d] = %d", s, d.K[s]);
-      ZR_CHECK_ARG(d.A[s] && d.B[s], "gemm: null operand in segment %d", s);
+      ZR_CHECK_ARG(d.groups > 0 || (d.A[s] && d.B[s]), "gemm: null operand in segment %d", s);
       ZR_CHECK_ARG(d.lda[s] >= (d.trans_a ? d.K[s] : d.M), "gemm: lda[%d] = %d too small", s, d.lda[s]);
-      ZR_CHECK_ARG(!d.a_pack || (!d.trans_a && d.batch == 1 && d.lda[s] % 32 == 0 && 8LL * d.lda[s] + 8LL * d.M < (1LL << 31)),
-                   "gemm: packed operand A of segment %d: needs no transpose, one batch, lda a multiple of 32", s);
+      ZR_CHECK_ARG(!d.a_pack || (!d.trans_a && (d.batch == 1 || d.a_pack == 1) && d.lda[s] % 32 == 0 &&
+                                 8LL * d.lda[s] + 8LL * d.M < (1LL << 31)),
+                   "gemm: packed operand A of segment %d: needs no transpose, lda a multiple of 32 (bf16: one batch)", s);
       ZR_CHECK_ARG(d.a_pack != 2 || d.K[s] % 16 == 0, "gemm: bf16 operand A needs K %% 16 == 0 (K[%d] = %d)", s, d.K[s]);
       ZR_CHECK_ARG(d.ldb[s] >= d.K[s], "gemm: ldb[%d] = %d < K = %d", s, d.ldb[s], d.K[s]);
       // per-lane weight offsets are 32-bit element indices
@@ -696,7 +730,11 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
       ga.B[s] = d.B[s];
       ga.ldb[s] = d.ldb[s];
       vec = vec && (d.ldb[s] % 4 == 0) && (((uintptr_t)d.B[s] & 15u) == 0);
-      if (d.trans_a) vec = vec && (d.lda[s] % 4 == 0) && (((uintptr_t)d.A[s] & 15u) == 0) && (d.strideA % 4 == 0);
+      for (int g = 0; g < d.groups; ++g) vec = vec && (((uintptr_t)d.gB[g] & 15u) == 0);
+      if (d.trans_a) {
+        vec = vec && (d.lda[s] % 4 == 0) && (((uintptr_t)d.A[s] & 15u) == 0) && (d.strideA % 4 == 0);
+        for (int g = 0; g < d.groups; ++g) vec = vec && (((uintptr_t)d.gA[g] & 15u) == 0);
+      }
       flops += 2LL * d.M * d.N * d.K[s];
     } else {
       ga.K[s] = 0;
@@ -762,7 +800,7 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
   if (d.a_pack) {
     // Activations too: a k-interleaved copy in scratch turns their loads (16 bytes from each of 32 lines per
     // half-wave) into contiguous ones.  Worth a small extra kernel once the weight matrix is large.
-    bool xpack = vec && d.M >= 2048;
+    bool xpack = vec && d.M >= 2048 && d.groups == 0;
     size_t xfloats = 0;
     for (int s = 0; s < d.nseg; ++s) {
       xpack = xpack && (d.K[s] % 8 == 0);
@@ -783,7 +821,7 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
       ga.b_pack4 = 1;
     }
     // tall matrices: equal row ranges per CU, column tiles of equal width (at most 128 columns each)
-    if (vec && d.nseg == 1 && d.M >= 8192 && d.N <= 1024 && ctx->gemm_cfg != 11 &&
+    if (vec && d.nseg == 1 && zcount == 1 && d.M >= 8192 && d.N <= 1024 && ctx->gemm_cfg != 11 &&
         (d.epilogue == ZR_EPI_STORE || d.epilogue == ZR_EPI_SOFTMAX_PARTIAL)) {
       const int n32 = (d.N + 31) / 32;
       const int n_tiles = (n32 + 3) / 4;
@@ -793,14 +831,14 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
       if (tn == 3) return launch_rows<3>(ctx, ga, d.epilogue, n_tiles);
       return launch_rows<4>(ctx, ga, d.epilogue, n_tiles);
     }
-    if (ctx->gemm_cfg == 12) return launch_pack4<4, 2, 1>(ctx, ga, d.epilogue, vec);
-    if (ctx->gemm_cfg == 13) return launch_pack4<2, 2, 1>(ctx, ga, d.epilogue, vec);
-    if (ctx->gemm_cfg == 14) return launch_pack4<2, 4, 1>(ctx, ga, d.epilogue, vec);
-    if (d.N <= 32) return launch_pack4<2, 1, 2>(ctx, ga, d.epilogue, vec);
-    return launch_pack4<2, 2, 2>(ctx, ga, d.epilogue, vec);
+    if (ctx->gemm_cfg == 12) return launch_pack4<4, 2, 1>(ctx, ga, d.epilogue, vec, zcount);
+    if (ctx->gemm_cfg == 13) return launch_pack4<2, 2, 1>(ctx, ga, d.epilogue, vec, zcount);
+    if (ctx->gemm_cfg == 14) return launch_pack4<2, 4, 1>(ctx, ga, d.epilogue, vec, zcount);
+    if (d.N <= 32) return launch_pack4<2, 1, 2>(ctx, ga, d.epilogue, vec, zcount);
+    return launch_pack4<2, 2, 2>(ctx, ga, d.epilogue, vec, zcount);
   }
   // Large, untransposed, single-segment products with a wide batch (the softmax logits): LDS-shared weights.
-  const bool lds_ok = !d.trans_a && d.nseg == 1 && d.batch == 1 && vec && (d.M % 4 == 0) && (d.lda[0] % 4 == 0) &&
+  const bool lds_ok = !d.trans_a && d.nseg == 1 && zcount == 1 && vec && (d.M % 4 == 0) && (d.lda[0] % 4 == 0) &&
                       (((uintptr_t)d.A[0] & 15u) == 0) && d.K[0] >= 8 && d.K[0] % 8 == 0 && d.M >= 2048 && d.N >= 96 &&
                       ((long long)d.K[0] + 64) * d.lda[0] * 4 < (1LL << 32) && (long long)d.N * d.ldb[0] * 4 < (1LL << 32) &&
                       (d.epilogue == ZR_EPI_STORE || d.epilogue == ZR_EPI_SOFTMAX_PARTIAL);
@@ -816,7 +854,7 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
   const bool trans_a = d.trans_a != 0;
   int cfg = ctx->gemm_cfg;
   if (cfg == 0) {
-    const long long sub32 = (long long)((d.M + 31) / 32) * ((d.N + 31) / 32) * d.batch;  // 32x32 output blocks
+    const long long sub32 = (long long)((d.M + 31) / 32) * ((d.N + 31) / 32) * zcount;  // 32x32 output blocks
     if (sub32 >= 8 * 2048)
       cfg = 1;  // 64 x 128 wave tiles
     else if (sub32 >= 4 * 2048)
@@ -833,21 +871,21 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
   (void)flops;
   switch (cfg) {
     case 1:
-      return launch_cfg<2, 4, 1, 4>(ctx, ga, d.batch, d.epilogue, trans_a, vec);
+      return launch_cfg<2, 4, 1, 4>(ctx, ga, zcount, d.epilogue, trans_a, vec);
     case 2:
-      return launch_cfg<1, 4, 1, 4>(ctx, ga, d.batch, d.epilogue, trans_a, vec);
+      return launch_cfg<1, 4, 1, 4>(ctx, ga, zcount, d.epilogue, trans_a, vec);
     case 3:
-      return launch_cfg<1, 2, 1, 4>(ctx, ga, d.batch, d.epilogue, trans_a, vec);
+      return launch_cfg<1, 2, 1, 4>(ctx, ga, zcount, d.epilogue, trans_a, vec);
     case 4:
-      return launch_cfg<1, 1, 1, 4>(ctx, ga, d.batch, d.epilogue, trans_a, vec);
+      return launch_cfg<1, 1, 1, 4>(ctx, ga, zcount, d.epilogue, trans_a, vec);
     case 5:
-      return launch_cfg<1, 1, 4, 1>(ctx, ga, d.batch, d.epilogue, trans_a, vec);
+      return launch_cfg<1, 1, 4, 1>(ctx, ga, zcount, d.epilogue, trans_a, vec);
     case 6:
-      return launch_cfg<1, 1, 8, 1>(ctx, ga, d.batch, d.epilogue, trans_a, vec);
+      return launch_cfg<1, 1, 8, 1>(ctx, ga, zcount, d.epilogue, trans_a, vec);
     case 7:
-      return launch_cfg<2, 2, 1, 4>(ctx, ga, d.batch, d.epilogue, trans_a, vec);
+      return launch_cfg<2, 2, 1, 4>(ctx, ga, zcount, d.epilogue, trans_a, vec);
     default:
-      return launch_cfg<1, 2, 4, 1>(ctx, ga, d.batch, d.epilogue, trans_a, vec);
+      return launch_cfg<1, 2, 4, 1>(ctx, ga, zcount, d.epilogue, trans_a, vec);
   }
 }
 

@@ -110,6 +110,13 @@ struct ZrGemmDesc {
   int epilogue;
   float* partials;  // ZR_EPI_SOFTMAX_PARTIAL: [ceil(M/32)][N][2] floats
   int accumulate;   // ZR_EPI_STORE only: C += product (+ bias) instead of C = ...
+  // groups > 0: that many independent problems of the same shape in one launch (at most 8; one segment, plain store
+  // epilogue, no bias): problem g multiplies gA[g] (instead of A[0]) with gB[g] (instead of B[0]) into gC[g]
+  // (instead of C); lda/ldb/ldc, the batch count and its strides apply inside every problem.
+  int groups;
+  const float* gA[8];
+  const float* gB[8];
+  float* gC[8];
 };
 
 int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d);
