@@ -28,9 +28,9 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E peak
 
 # HBM bytes per launch of lstm_sweep_kernel on the headline workload, from two rocprofv3 --pmc runs (FETCH_SIZE, then
 # WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for a plain copy of known size
-# (bench.py --calibrate-copy): FETCH_SIZE 3397743.8 KiB x 1.9706 + WRITE_SIZE 401518.3 KiB x 1.0000.
+# (bench.py --calibrate-copy): FETCH_SIZE 3394327.1 KiB x 1.9855 + WRITE_SIZE 400528.6 KiB x 1.0000.
 # The summary of those runs is profiles/lstm_sweep_kernel_config2_hbm_traffic.txt.
-LSTM_SWEEP_TRAFFIC_BYTES = int((3397743.8 * 1.9706 + 401518.3 * 1.0) * 1024)
+LSTM_SWEEP_TRAFFIC_BYTES = int((3394327.1 * 1.9855 + 400528.6 * 1.0) * 1024)
 
 
 def log(*a):
@@ -322,8 +322,8 @@ def vendor_sgemm_reference(iters=50):
 
 def calibrate_copy(ctx, mbytes=64):
     """Plain copies of known size (identity column gathers: n*H*4 bytes read, n*H*4 bytes written) for scaling the
-    FETCH_SIZE / WRITE_SIZE counters: one with 16-byte accesses (H = 1024, column_copy_kernel<true>) and one with
-    4-byte accesses (H = 1023, column_copy_kernel<false>), the access width of the MFMA kernels' weight loads."""
+    FETCH_SIZE / WRITE_SIZE counters: one with 16-byte accesses (H = 1024, column_copy_wide_kernel) and one with
+    4-byte accesses (H = 1023, column_copy_kernel<false>)."""
     out = []
     for H in (1024, 1023):
         n = mbytes * 1024 * 1024 // (H * 4)
@@ -332,7 +332,7 @@ def calibrate_copy(ctx, mbytes=64):
         for _ in range(3):
             ctx.gather_columns(src, H, perm, n, dst)
         ctx.sync()
-        out.append({"kernel": "column_copy_kernel<%s>" % ("true" if H % 4 == 0 else "false"), "H": H, "columns": n,
+        out.append({"kernel": "column_copy_wide_kernel" if H % 4 == 0 else "column_copy_kernel<false>", "H": H, "columns": n,
                     "KiB_read": (n * H * 4 + n * 4) / 1024.0, "KiB_written": n * H * 4 / 1024.0})
     return out
 
