@@ -73,7 +73,8 @@ const char* zr_version(void);
 #define ZR_OPT_LSTM_SWEEP 7          /* zr_lstm_stack_forward as ONE launch whose workgroups hand h to each other
                                         through device memory: 0 auto (when they fill most of the device, are all
                                         resident at once and the context is the process's only one on its device),
-                                        1 never (one launch per diagonal), 2 whenever they fit */
+                                        1 never (one launch per diagonal), 2 whenever they fit.  The environment
+                                        variable ZR_LSTM_SWEEP presets this option for every context created */
 #define ZR_OPT_LSTM_SWEEP_SPIN 8     /* polls a workgroup of that launch spends on one wait before it gives up
                                         (0 = default, about a second); giving up is reported by zr_ctx_sync */
 

@@ -1,6 +1,7 @@
 // Context, error reporting and device memory helpers of the C-ABI.
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <atomic>
@@ -79,6 +80,12 @@ int zr_ctx_create(int device, zr_ctx** out) {
   (void)hipMemset(c->d_flags, 0, (4 + ZR_MAX_COUNTERS) * sizeof(int));
   c->d_counters = c->d_flags + 4;
   c->lstm_fused = 1;
+  // ZR_LSTM_SWEEP in the environment presets ZR_OPT_LSTM_SWEEP for every context of the process (0, 1 or 2): lets a
+  // whole program, e.g. a test run, be put on one path or the other without touching its code
+  if (const char* e = getenv("ZR_LSTM_SWEEP")) {
+    const int v = atoi(e);
+    if (v >= 0 && v <= 2) c->lstm_sweep = v;
+  }
   if (device < 64) g_live[device].fetch_add(1);
   *out = c;
   return ZR_OK;
