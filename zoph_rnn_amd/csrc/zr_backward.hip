@@ -103,6 +103,7 @@ struct NodeBackwardGroup {
   const float* err_next[8];   // may be null
   float* ec[8];               // cell error, updated in place
   float* dg[8];
+  float* dgp[8];              // non-null: second copy of dg, k-interleaved [4H/4][mb][4] (the grouped product's right side)
 };
 __global__ void __launch_bounds__(256) lstm_node_backward_group_kernel(NodeBackwardGroup G, int H, int mb) {
   const int u = blockIdx.z;
@@ -122,10 +123,21 @@ __global__ void __launch_bounds__(256) lstm_node_backward_group_kernel(NodeBackw
   const float errt_ct = eh * go * (1.0f - th * th);
   const float ec = (G.ec[u][ix] + errt_ct) * m;
   float* d = G.dg[u] + (size_t)b * 4 * H + j;
-  d[0] = ec * gc * gi * (1.0f - gi);
-  d[H] = ec * G.cprev[u][ix] * gf * (1.0f - gf);
-  d[2 * (size_t)H] = ec * gi * (1.0f - gc * gc);
-  d[3 * (size_t)H] = eh * th * go * (1.0f - go);
+  const float di = ec * gc * gi * (1.0f - gi), df = ec * G.cprev[u][ix] * gf * (1.0f - gf);
+  const float dc = ec * gi * (1.0f - gc * gc), dob = eh * th * go * (1.0f - go);
+  d[0] = di;
+  d[H] = df;
+  d[2 * (size_t)H] = dc;
+  d[3 * (size_t)H] = dob;
+  if (G.dgp[u]) {
+    // row k = g*H + j of the 4H x mb matrix, column b
+    float* p = G.dgp[u];
+    const size_t k0 = (size_t)j, k1 = (size_t)H + j, k2 = 2 * (size_t)H + j, k3 = 3 * (size_t)H + j;
+    p[((k0 >> 2) * mb + b) * 4 + (k0 & 3)] = di;
+    p[((k1 >> 2) * mb + b) * 4 + (k1 & 3)] = df;
+    p[((k2 >> 2) * mb + b) * 4 + (k2 & 3)] = dc;
+    p[((k3 >> 2) * mb + b) * 4 + (k3 & 3)] = dob;
+  }
   G.ec[u][ix] = ec * gf;
 }
 
@@ -369,10 +381,13 @@ int zr_lstm_stack_backward(zr_ctx* ctx, int nl, const zr_lstm_train* const layer
   // work: two sets (diagonal parity) of per-layer [2][H x mb] = (error to h_{t-1}, error to the layer below): a
   // node reads what diagonal d+1 wrote into the other set while its neighbours on diagonal d write this one.  The
   // cell error lives in d_err_c0[l] (updated in place step by step; one node per layer and diagonal touches it).
+  const bool packed_ok = (H % 4 == 0) && layers[0]->d_stack_pack != nullptr;
+  const bool bpack = packed_ok && (H % 2 == 0);  // K = 4H must be a multiple of 8
   void* scratch = nullptr;
-  rc = zr_ctx_scratch(ctx, 1, sizeof(float) * 4 * n * nl, &scratch);
+  rc = zr_ctx_scratch(ctx, 1, sizeof(float) * (4 * n * nl + (bpack ? 8 * 4 * n : 0)), &scratch);
   if (rc) return rc;
   float* work = (float*)scratch;
+  float* dgp_buf = work + 4 * n * nl;  // k-interleaved copies of the gate errors of the diagonal in flight
   auto wk = [&](int d, int l) { return work + ((size_t)(d & 1) * nl + l) * 2 * n; };
   for (int l = 0; l < nl; ++l) {
     // node (l, T-1) is on diagonal l + T - 1 and reads its "next step" error from the set of diagonal l + T
@@ -390,7 +405,6 @@ int zr_lstm_stack_backward(zr_ctx* ctx, int nl, const zr_lstm_train* const layer
       if (rc) return rc;
     }
   }
-  const bool packed_ok = (H % 4 == 0) && layers[0]->d_stack_pack != nullptr;
   for (int d = nl + T - 2; d >= 0; --d) {
     for (int lhi = nl - 1; lhi >= 0; lhi -= 8) {  // at most 8 nodes per launch
       NodeBackwardGroup G = {};
@@ -408,8 +422,9 @@ int zr_lstm_stack_backward(zr_ctx* ctx, int nl, const zr_lstm_train* const layer
         G.err_next[nu] = wk(d + 1, l);
         G.ec[nu] = d_err_c0[l];
         G.dg[nu] = d_dgates_all[l] + (size_t)t * 4 * n;
+        G.dgp[nu] = bpack ? dgp_buf + (size_t)nu * 4 * n : nullptr;
         g.gA[nu] = packed_ok ? layers[l]->d_stack_pack : layers[l]->d_stack;
-        g.gB[nu] = G.dg[nu];
+        g.gB[nu] = bpack ? G.dgp[nu] : G.dg[nu];
         g.gC[nu] = w_l;
         ++nu;
       }
@@ -430,6 +445,7 @@ int zr_lstm_stack_backward(zr_ctx* ctx, int nl, const zr_lstm_train* const layer
       g.epilogue = ZR_EPI_STORE;
       if (packed_ok) {
         g.a_pack = 1;
+        g.b_packed = bpack ? 1 : 0;
         g.lda[0] = layers[0]->ldp;
         g.strideA = (long long)layers[0]->kp * layers[0]->ldp;
       } else {

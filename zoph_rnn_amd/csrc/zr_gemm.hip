@@ -800,7 +800,13 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
   if (d.a_pack) {
     // Activations too: a k-interleaved copy in scratch turns their loads (16 bytes from each of 32 lines per
     // half-wave) into contiguous ones.  Worth a small extra kernel once the weight matrix is large.
-    bool xpack = vec && d.M >= 2048 && d.groups == 0;
+    if (d.b_packed) {
+      ZR_CHECK_ARG(d.a_pack == 1 && vec, "gemm: a k-interleaved B needs a k-interleaved fp32 A and 16-byte alignment");
+      for (int s = 0; s < d.nseg; ++s)
+        ZR_CHECK_ARG(d.K[s] % 8 == 0, "gemm: a k-interleaved B needs K %% 8 == 0 (K[%d] = %d)", s, d.K[s]);
+      ga.b_pack4 = 1;
+    }
+    bool xpack = vec && d.M >= 2048 && d.groups == 0 && !d.b_packed;
     size_t xfloats = 0;
     for (int s = 0; s < d.nseg; ++s) {
       xpack = xpack && (d.K[s] % 8 == 0);

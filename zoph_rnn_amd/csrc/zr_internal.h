@@ -113,6 +113,8 @@ struct ZrGemmDesc {
   // groups > 0: that many independent problems of the same shape in one launch (at most 8; one segment, plain store
   // epilogue, no bias): problem g multiplies gA[g] (instead of A[0]) with gB[g] (instead of B[0]) into gC[g]
   // (instead of C); lda/ldb/ldc, the batch count and its strides apply inside every problem.
+  int b_packed;  // with a_pack == 1: B (and every gB) is already k-interleaved, element (k, n) at ((k/4)*N + n)*4 + k%4
+                 // (K a multiple of 8, 16-byte aligned); ldb is ignored
   int groups;
   const float* gA[8];
   const float* gB[8];
