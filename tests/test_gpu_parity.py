@@ -684,23 +684,45 @@ def test_whole_sweep_launch_keeps_gates_for_training(ctx):
 
 
 def test_whole_sweep_launch_back_to_back_with_different_inputs(ctx):
-    """Two sweeps of the same shape with different data, back to back through the same hand-over buffers: the second
-    must not see anything of the first (mb % 8 == 0: the consumers do not invalidate their caches inside the launch)."""
+    """Sweeps of the same shape with different token ids and initial states, queued back to back through the same
+    hand-over buffers with nothing but the counter-clearing fill between them (the whole hand-over buffer, 1.5 MB, stays
+    cache resident): a later sweep must not see anything of an earlier one (mb % 8 == 0: the consumers do not
+    invalidate their caches inside the launch)."""
     H, mb, T, V, L = 256, 64, 6, 211, 4
+    g = synth.rng(21, 1)
+    embed = U(g, (H, V))
+    layers_np = [synth.lstm_layer(g, H, forget_bias_one=True) for _ in range(L)]
+    layers = [Layer(ctx, ly) for ly in layers_np]
+    d_embed = ctx.array(embed)
+    n = H * mb
+    runs = []
+    for seed in range(4):
+        ids = g.integers(0, V, size=(T, mb)).astype(np.int32)
+        h0 = [np.tanh(U(g, (H, mb), -1, 1)) for _ in range(L)]
+        c0 = [U(g, (H, mb), -0.5, 0.5) for _ in range(L)]
+        d_nn, d_m = ctx.empty(ids.size, np.int32), ctx.empty(ids.size, np.int32)
+        ctx.vocab_prep(ctx.array(ids.reshape(-1)), ids.size, V, d_nn, d_m)
+        runs.append(dict(ids=ids, h0=h0, c0=c0, d_nn=d_nn, d_m=d_m, d_h0=[ctx.array(a) for a in h0],
+                         d_c0=[ctx.array(a) for a in c0], h_all=[ctx.empty((n * T,)) for _ in range(L)],
+                         c_all=[ctx.empty((n * T,)) for _ in range(L)]))
+    ctx.sync()
     ctx.set_option(capi.ZR_OPT_LSTM_SWEEP, 2)
     try:
-        for seed in (1, 2, 3):
-            g = synth.rng(21, seed)
-            embed = U(g, (H, V))
-            layers = [synth.lstm_layer(g, H, forget_bias_one=True) for _ in range(L)]
-            ids = g.integers(0, V, size=(T, mb)).astype(np.int32)
-            hs, cs = _run_stack(ctx, layers, embed, ids)
-            nn, m = o.vocab_prep(ids)
-            want_h, want_c = o.lstm_stack_forward(embed, layers, nn, m)
-            assert_close(hs, want_h, what="stack h (run %d)" % seed)
-            assert_close(cs, want_c, what="stack c (run %d)" % seed)
+        for r in runs:  # queued without a synchronisation or any other work in between
+            ctx.lstm_stack_forward([ly.w for ly in layers], d_embed, V, r["d_nn"], r["d_m"], T, mb, r["d_h0"], r["d_c0"],
+                                   r["h_all"], r["c_all"])
+        ctx.sync()
     finally:
         ctx.set_option(capi.ZR_OPT_LSTM_SWEEP, 0)
+    for i, r in enumerate(runs):
+        nn, m = o.vocab_prep(r["ids"])
+        want_h, want_c = o.lstm_stack_forward(embed, layers_np, nn, m, h0=r["h0"], c0=r["c0"])
+        hs = np.stack([a.get().reshape(T, mb, H).transpose(0, 2, 1) for a in r["h_all"]])
+        cs = np.stack([a.get().reshape(T, mb, H).transpose(0, 2, 1) for a in r["c_all"]])
+        assert_close(hs, want_h, what="stack h (run %d)" % i)
+        assert_close(cs, want_c, what="stack c (run %d)" % i)
+    for ly in layers:
+        ly.close()
 
 
 def test_whole_sweep_launch_abandoned_wait_is_reported(ctx):
