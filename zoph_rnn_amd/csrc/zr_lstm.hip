@@ -889,8 +889,13 @@ int launch_fused(zr_ctx* ctx, LstmLaunch& L, bool vec) {
   const long long wgs_whole_k = (long long)L.n_units * L.j_tiles * ((n32 + 1) / 2);
   if (kernel == 0 && vec && (L.H & 7) == 0 && wgs_whole_k < 200) kernel = 3;
   if (kernel == 3 && vec && (L.H & 7) == 0) {
-    // widest column tile that divides the batch's 32-column blocks evenly, then as many K parts as fill the chip
-    const int tn = (n32 % 3 == 0) ? 3 : (n32 >= 2 ? 2 : 1);
+    // 32-column tiles and as few K parts as fill the chip: measured on four decoder nodes of H = 1000 against wider
+    // tiles with more parts, 119 us against 138 at 128 columns, 88 against 117 at 64 (a short K range per workgroup
+    // never gets its operand pipeline going, and the cross-workgroup sum grows with the parts); when the tiles alone
+    // fill the chip no split is made at all (167 against 181 us at 192 columns, 172 against 191 at 256)
+    int tn = 1;
+    if (ctx->lstm_tn == 2 && n32 >= 2) tn = 2;                   // tuning runs
+    if (ctx->lstm_tn == 4 && n32 % 3 == 0) tn = 3;
     L.n_tiles = (n32 + tn - 1) / tn;
     const long long tiles = (long long)L.n_units * L.j_tiles * L.n_tiles;
     int parts = ctx->lstm_kparts;
