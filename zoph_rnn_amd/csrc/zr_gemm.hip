@@ -869,6 +869,8 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
       cfg = 3;  // 32 x 64
     else if (sub32 >= 1024)
       cfg = 4;  // 32 x 32
+    else if (sub32 <= 256 && d.K[0] >= 512)
+      cfg = 6;  // 32 x 32, K split over 8 waves: at most one tile per CU, the K loop is all there is to shorten
     else
       cfg = 5;  // 32 x 32, K split over 4 waves
     if (d.N <= 32 && cfg < 4) cfg = 4;
