@@ -28,9 +28,9 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E peak
 
 # HBM bytes per launch of lstm_sweep_kernel on the headline workload, from two rocprofv3 --pmc runs (FETCH_SIZE, then
 # WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for a plain copy of known size
-# (bench.py --calibrate-copy): FETCH_SIZE 3394301.0 KiB x 1.9855 + WRITE_SIZE 400487.9 KiB x 1.0000.
+# (bench.py --calibrate-copy): FETCH_SIZE 3394177.9 KiB x 1.9854 + WRITE_SIZE 400563.6 KiB x 1.0000.
 # The summary of those runs is profiles/lstm_sweep_kernel_config2_hbm_traffic.txt.
-LSTM_SWEEP_TRAFFIC_BYTES = int((3394301.0 * 1.9855 + 400487.9 * 1.0) * 1024)
+LSTM_SWEEP_TRAFFIC_BYTES = int((3394177.9 * 1.9854 + 400563.6 * 1.0) * 1024)
 
 
 def log(*a):

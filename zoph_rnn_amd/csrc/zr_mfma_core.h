@@ -204,14 +204,38 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t zr_make_rsrc(const void* base)
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0xFFFFFFFF, 0x00020000);
 }
 
+// The weight halves of the first PF ring stages of a segment, issued ahead of time (zr_mma_segment_u with WPRE then
+// fetches only the activation halves in its prologue): weights depend on nothing, so a caller that must wait for its
+// activations can have them in flight during the wait.
 template <int TM, int TN, int KS, int PF>
+__device__ __forceinline__ void zr_preload_w(ZrFrag<TM, TN> (&f)[PF + 1], __amdgpu_buffer_rsrc_t wrsrc,
+                                             const unsigned (&wsoff)[TM], unsigned woffb, unsigned wstep, int K,
+                                             int kslice) {
+  const int last = (K >> 3) - 1;
+#pragma unroll
+  for (int s = 0; s < PF; ++s) {
+    int gl = kslice + s * KS;
+    gl = gl < last ? gl : last;
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+      const zr_u32x4v v =
+          __builtin_amdgcn_raw_buffer_load_b128(wrsrc, (int)woffb, (int)(wsoff[tm] + (unsigned)gl * wstep), 0);
+      f[s].w[tm][0] = __uint_as_float(v.x);
+      f[s].w[tm][1] = __uint_as_float(v.y);
+      f[s].w[tm][2] = __uint_as_float(v.z);
+      f[s].w[tm][3] = __uint_as_float(v.w);
+    }
+  }
+}
+
+template <int TM, int TN, int KS, int PF, bool WPRE = false>
 __device__ __forceinline__ void zr_mma_segment_u(zr_f32x16 (&acc)[TM][TN], __amdgpu_buffer_rsrc_t wrsrc,
                                                  const unsigned (&wsoff)[TM], unsigned woffb, unsigned wstep,
                                                  __amdgpu_buffer_rsrc_t xrsrc, const unsigned (&xoffb)[TN],
-                                                 unsigned xstep, int K, int kslice) {
+                                                 unsigned xstep, int K, int kslice, ZrFrag<TM, TN> (&f)[PF + 1]) {
   const int nfull = K >> 3;  // K % 8 == 0
   constexpr int NS = PF + 1;
-  auto load_full = [&](ZrFrag<TM, TN>& f, int g) {
+  auto load_x = [&](ZrFrag<TM, TN>& f, int g) {
     const unsigned ug = (unsigned)g;  // wave-uniform
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) {
@@ -221,6 +245,10 @@ __device__ __forceinline__ void zr_mma_segment_u(zr_f32x16 (&acc)[TM][TN], __amd
       f.x[tn][2] = __uint_as_float(v.z);
       f.x[tn][3] = __uint_as_float(v.w);
     }
+  };
+  auto load_full = [&](ZrFrag<TM, TN>& f, int g) {
+    const unsigned ug = (unsigned)g;  // wave-uniform
+    load_x(f, g);
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) {
       const zr_u32x4v v = __builtin_amdgcn_raw_buffer_load_b128(wrsrc, (int)woffb, (int)(wsoff[tm] + ug * wstep), 0);
@@ -242,11 +270,13 @@ __device__ __forceinline__ void zr_mma_segment_u(zr_f32x16 (&acc)[TM][TN], __amd
   if (kslice < nfull) {
     const int last = nfull - 1;
     const int n_mine = (nfull - kslice + KS - 1) / KS;
-    ZrFrag<TM, TN> f[NS];
 #pragma unroll
     for (int s = 0; s < PF; ++s) {
       const int gl = kslice + s * KS;
-      load_full(f[s], gl < last ? gl : last);
+      if (WPRE)
+        load_x(f[s], gl < last ? gl : last);
+      else
+        load_full(f[s], gl < last ? gl : last);
     }
     int it = 0;
     for (; it + NS <= n_mine; it += NS) {
@@ -273,6 +303,16 @@ __device__ __forceinline__ void zr_mma_segment_u(zr_f32x16 (&acc)[TM][TN], __amd
     for (int s = 0; s < PF; ++s)
       if (it + s < n_mine) mma(f[s]);
   }
+}
+
+// The same with a ring of its own (no weights fetched ahead).
+template <int TM, int TN, int KS, int PF>
+__device__ __forceinline__ void zr_mma_segment_u(zr_f32x16 (&acc)[TM][TN], __amdgpu_buffer_rsrc_t wrsrc,
+                                                 const unsigned (&wsoff)[TM], unsigned woffb, unsigned wstep,
+                                                 __amdgpu_buffer_rsrc_t xrsrc, const unsigned (&xoffb)[TN],
+                                                 unsigned xstep, int K, int kslice) {
+  ZrFrag<TM, TN> f[PF + 1];
+  zr_mma_segment_u<TM, TN, KS, PF, false>(acc, wrsrc, wsoff, woffb, wstep, xrsrc, xoffb, xstep, K, kslice, f);
 }
 
 // Workgroup barrier that also publishes: when it returns, every store any thread of the workgroup issued before it
