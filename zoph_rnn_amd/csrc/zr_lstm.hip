@@ -635,7 +635,7 @@ __device__ __forceinline__ bool sweep_wait(const LstmSweep& P, int* ctr, int tar
 template <int TN>
 __global__ void __launch_bounds__(256) lstm_sweep_kernel(LstmSweep P) {
   constexpr int KS = 4;
-  __shared__ float red[KS * TN * 16 * 64];
+  __shared__ __align__(16) float red[KS * 4 * TN * 16 * 64];  // all partial tiles of the workgroup at once
   __shared__ int s_go[2];
   // same die-aware placement as lstm_fused_kernel, with one unit per layer
   const int id = blockIdx.x;
@@ -658,7 +658,7 @@ __global__ void __launch_bounds__(256) lstm_sweep_kernel(LstmSweep P) {
   constexpr int NV = zr_visit_count<TN, KS>();
   // batch column of visit i of a lane in half-wave `half`, clamped
   auto visit_col = [&](int i, int half) {
-    const int slot = zr_visit_slot<KS>(kslice, i);
+    const int slot = zr_wide_visit_slot<KS>(kslice, i);
     const int tn = slot >> 4, r = slot & 15;
     const int n = n0 + tn * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
     return n < mb ? n : mb - 1;
@@ -760,7 +760,7 @@ __global__ void __launch_bounds__(256) lstm_sweep_kernel(LstmSweep P) {
     float* h_out = P.h_all[l] + (long long)t * n_el;
     float* c_out = P.c_all[l] + (long long)t * n_el;
     float* hp_out = hp_mine + (long long)t * n_el;
-    zr_reduce_visit<4, TN, KS>(acc, red, kslice, lane, [&](const float(&z)[4], int tn, int r, int vi) {
+    zr_reduce_visit_wide<4, TN, KS>(acc, red, kslice, lane, [&](const float(&z)[4], int tn, int r, int vi) {
       const int n = n0 + tn * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
       float gi, gf, gc, go, c, h;
       zr_lstm_cell(z[0] + bi, z[1] + bf, z[2] + bc, z[3] + bo, c_state[vi], mask_v[vi], P.clip, gi, gf, gc, go, c, h);

@@ -384,6 +384,53 @@ __device__ __forceinline__ void zr_reduce_visit(zr_f32x16 (&acc)[TM][TN], float*
   }
 }
 
+// The same reduction in ONE round, for kernels that own a whole CU's LDS: every wave writes all TM*TN of its partial
+// tiles (16-byte stores, four consecutive accumulator registers of a lane each), one barrier, and every wave sums
+// the KS copies of the groups of four it finishes (16-byte loads; the sum runs over the waves in the same order as
+// in zr_reduce_visit, so both give the same bits).  Against TM rounds of write-barrier-read this saves 2*TM - 2
+// barriers with their exposed LDS latency and three quarters of the LDS instructions.  `red` holds
+// KS * TM * TN*16 * 64 floats, 16-byte aligned (128 KB for TM=4, TN=2, KS=4).  Visit i of wave `kslice` is
+// accumulator slot zr_wide_visit_slot<KS>(kslice, i); otherwise the contract is zr_reduce_visit's.
+template <int KS>
+__device__ __forceinline__ int zr_wide_visit_slot(int kslice, int i) { return (kslice + KS * (i >> 2)) * 4 + (i & 3); }
+
+template <int TM, int TN, int KS, class F>
+__device__ __forceinline__ void zr_reduce_visit_wide(zr_f32x16 (&acc)[TM][TN], float* red, int kslice, int lane, F f) {
+  constexpr int G4 = TN * 4;   // groups of four accumulator registers per sub-tile row of the tile
+  constexpr int PG = G4 / KS;  // groups finished by each wave
+  static_assert(KS > 1 && G4 % KS == 0, "KS must divide TN*4");
+  zr_f32x4* red4 = (zr_f32x4*)red;
+  __syncthreads();  // the previous use of `red` is over
+#pragma unroll
+  for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+    for (int g4 = 0; g4 < G4; ++g4) {
+      zr_f32x4 v;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) v[c] = acc[tm][g4 >> 2][(g4 & 3) * 4 + c];
+      red4[((kslice * TM + tm) * G4 + g4) * 64 + lane] = v;
+    }
+  __syncthreads();
+  zr_f32x4 pre[TM][PG];
+#pragma unroll
+  for (int i4 = 0; i4 < PG; ++i4)
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+      zr_f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int w = 0; w < KS; ++w) sum += red4[((w * TM + tm) * G4 + kslice + KS * i4) * 64 + lane];
+      pre[tm][i4] = sum;
+    }
+#pragma unroll
+  for (int i = 0; i < PG * 4; ++i) {
+    const int slot = zr_wide_visit_slot<KS>(kslice, i);
+    float vals[TM];
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) vals[tm] = pre[tm][i >> 2][i & 3];
+    f(vals, slot >> 4, slot & 15, i);
+  }
+}
+
 // ---------------------------------------------------------------------------------------------------------
 // (max, sum of exp(v - max)) over the 32 lanes of each half-wave, for G independent values per lane at once.
 // In the MFMA output layout a half-wave holds the 32 rows of one output column, so this is the softmax partial
