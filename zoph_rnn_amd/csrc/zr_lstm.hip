@@ -760,29 +760,38 @@ __global__ void __launch_bounds__(256) lstm_sweep_kernel(LstmSweep P) {
     float* h_out = P.h_all[l] + (long long)t * n_el;
     float* c_out = P.c_all[l] + (long long)t * n_el;
     float* hp_out = hp_mine + (long long)t * n_el;
+    // Only the k-interleaved copy of h, which the waiting workgroups read, goes out before the arrival is published;
+    // the outputs nobody waits for (h, c and the gate values kept for training) are held in registers and stored
+    // after it, so that their write latency overlaps the next step instead of sitting in front of the publish.
+    float h_v[NV], g_v[4][NV];
     zr_reduce_visit_wide<4, TN, KS>(acc, red, kslice, lane, [&](const float(&z)[4], int tn, int r, int vi) {
       const int n = n0 + tn * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-      float gi, gf, gc, go, c, h;
-      zr_lstm_cell(z[0] + bi, z[1] + bf, z[2] + bc, z[3] + bo, c_state[vi], mask_v[vi], P.clip, gi, gf, gc, go, c, h);
+      float c;
+      zr_lstm_cell(z[0] + bi, z[1] + bf, z[2] + bc, z[3] + bo, c_state[vi], mask_v[vi], P.clip, g_v[0][vi], g_v[1][vi],
+                   g_v[2][vi], g_v[3][vi], c, h_v[vi]);
       c_state[vi] = c;
-      if (j_ok && n < mb) {
-        const long long ix = (long long)n * H + j;
-        c_out[ix] = c;
-        h_out[ix] = h;
-        __hip_atomic_store(hp_out + ((long long)(j >> 2) * mb + n) * 4 + (j & 3), h, __ATOMIC_RELAXED,
+      if (j_ok && n < mb)
+        __hip_atomic_store(hp_out + ((long long)(j >> 2) * mb + n) * 4 + (j & 3), h_v[vi], __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_AGENT);
-        if (gates) {
-          float* gt = gates + (long long)t * 4 * n_el + ix;
-          gt[0] = gi;
-          gt[n_el] = gf;
-          gt[2 * n_el] = gc;
-          gt[3 * n_el] = go;
-        }
-      }
     });
     // publish this step: every wave's stores have completed before the barrier, then one arrival per workgroup
     zr_publish_barrier();
     if (tid == 0) atomicAdd(my_ctr, 1);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int slot = zr_wide_visit_slot<KS>(kslice, i);
+      const int n = n0 + (slot >> 4) * 32 + 8 * ((slot & 15) >> 2) + 4 * half + (slot & 3);
+      if (j_ok && n < mb) {
+        const long long ix = (long long)n * H + j;
+        c_out[ix] = c_state[i];
+        h_out[ix] = h_v[i];
+        if (gates) {
+          float* gt = gates + (long long)t * 4 * n_el + ix;
+#pragma unroll
+          for (int g = 0; g < 4; ++g) gt[g * n_el] = g_v[g][i];
+        }
+      }
+    }
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) idv[tn] = idn[tn];
   }
