@@ -71,8 +71,23 @@ constexpr int lstm_prefetch_depth(int tn, int ks) {
 // H % 8 == 0 and every operand array below 4 GiB (the host checks).
 template <int TN, int KS, bool VEC, bool BF16 = false, bool XPK = false, bool SPLIT = false, bool BUF = false>
 __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
-  __shared__ float red[KS * TN * 16 * 64];
+  // Four waves at up to 64 columns (one workgroup per CU at these register counts anyway) sum their partial tiles in
+  // one LDS round, which takes all 16 sub-tiles of every wave at once; the other shapes go gate by gate.
+  constexpr bool WIDE = KS == 4 && TN <= 2 && !BF16;
+  __shared__ __align__(16) float red[(WIDE ? 4 : 1) * KS * TN * 16 * 64];
   __shared__ int s_last;
+  auto visit_slot = [&](int kslice_, int i) {
+    if constexpr (WIDE)
+      return zr_wide_visit_slot<KS>(kslice_, i);
+    else
+      return zr_visit_slot<KS>(kslice_, i);
+  };
+  auto reduce_visit = [&](zr_f32x16(&acc_)[4][TN], int kslice_, int lane_, auto f) {
+    if constexpr (WIDE)
+      zr_reduce_visit_wide<4, TN, KS>(acc_, red, kslice_, lane_, f);
+    else
+      zr_reduce_visit<4, TN, KS>(acc_, red, kslice_, lane_, f);
+  };
   // Workgroup ids congruent modulo 8 run on the same XCD (round-robin dispatch) and share its L2.  Each XCD gets
   // a contiguous range of (unit, row tile) groups and every column tile of those groups: a weight tile is
   // fetched from memory once however many column tiles read it, and an XCD touches the activations of one or
@@ -120,7 +135,7 @@ __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
   float cprev_v[NV], mask_v[NV];
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
-    const int slot = zr_visit_slot<KS>(kslice, i);
+    const int slot = visit_slot(kslice, i);
     const int tn = slot >> 4, r = slot & 15;
     int n = n0 + tn * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
     n = n < L.mb ? n : L.mb - 1;
@@ -252,7 +267,7 @@ __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
     }
   };
   if constexpr (!SPLIT) {
-    zr_reduce_visit<4, TN, KS>(acc, red, kslice, lane, finish);
+    reduce_visit(acc, kslice, lane, finish);
   } else {
     constexpr int NTHR = 64 * KS;
     const int tile = group * L.n_tiles + nt;
@@ -260,7 +275,7 @@ __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
     // partial tile of this workgroup: [visit][gate][thread], written and read with device-scope relaxed atomics
     // (cache-bypassing on this multi-die part), published by the counter increment behind the barrier
     float* mine = L.partials + ((long long)tile * parts + part) * (NV * 4 * NTHR) + tid;
-    zr_reduce_visit<4, TN, KS>(acc, red, kslice, lane, [&](const float(&z)[4], int, int, int vi) {
+    reduce_visit(acc, kslice, lane, [&](const float(&z)[4], int, int, int vi) {
 #pragma unroll
       for (int g = 0; g < 4; ++g)
         __hip_atomic_store(mine + (vi * 4 + g) * NTHR, z[g], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -291,7 +306,7 @@ __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
     if (tid == 0) __hip_atomic_store(&L.counters[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // next launch
 #pragma unroll
     for (int vi = 0; vi < NV; ++vi) {
-      const int slot = zr_visit_slot<KS>(kslice, vi);
+      const int slot = visit_slot(kslice, vi);
       finish(sum[vi], slot >> 4, slot & 15, vi);
     }
   }
