@@ -727,6 +727,48 @@ def test_whole_sweep_launch_back_to_back_with_different_inputs(ctx):
         ly.close()
 
 
+@pytest.mark.parametrize("H,mb,T,L", [(200, 70, 20, 3), (256, 64, 12, 4)])
+def test_whole_sweep_launch_many_repetitions_identical(ctx, H, mb, T, L):
+    """The same sweep 400 times in a row: the order of the sums is fixed, so whatever the timing of the hand-overs
+    between workgroups, every repetition gives the first one's bits (checked every 50 launches), the first one agrees
+    with the oracle, and no wait is ever abandoned (zr_ctx_sync would report it).  mb = 70 takes the waits that
+    invalidate the caches, mb = 64 the ones that do not."""
+    g = synth.rng(23, H + mb)
+    V = 257
+    embed = U(g, (H, V))
+    layers_np = [synth.lstm_layer(g, H, forget_bias_one=True) for _ in range(L)]
+    layers = [Layer(ctx, ly) for ly in layers_np]
+    ids = g.integers(0, V, size=(T, mb)).astype(np.int32)
+    ids[:3, 2] = -1
+    d_embed = ctx.array(embed)
+    d_nn, d_m = ctx.empty(ids.size, np.int32), ctx.empty(ids.size, np.int32)
+    ctx.vocab_prep(ctx.array(ids.reshape(-1)), ids.size, V, d_nn, d_m)
+    z = ctx.zeros((H, mb))
+    h_all = [ctx.empty((H * mb * T,)) for _ in range(L)]
+    c_all = [ctx.empty((H * mb * T,)) for _ in range(L)]
+    first = None
+    ctx.set_option(capi.ZR_OPT_LSTM_SWEEP, 2)
+    try:
+        for i in range(400):
+            ctx.lstm_stack_forward([ly.w for ly in layers], d_embed, V, d_nn, d_m, T, mb, [z] * L, [z] * L, h_all, c_all)
+            if i % 50 == 0 or i == 399:
+                ctx.sync()
+                got = [a.get().tobytes() for a in h_all + c_all]
+                if first is None:
+                    first = got
+                    nn, m = o.vocab_prep(ids)
+                    want_h, want_c = o.lstm_stack_forward(embed, layers_np, nn, m)
+                    hs = np.stack([a.get().reshape(T, mb, H).transpose(0, 2, 1) for a in h_all])
+                    cs = np.stack([a.get().reshape(T, mb, H).transpose(0, 2, 1) for a in c_all])
+                    assert_close(hs, want_h, what="stack h")
+                    assert_close(cs, want_c, what="stack c")
+                assert got == first, "repetition %d differs from the first" % i
+    finally:
+        ctx.set_option(capi.ZR_OPT_LSTM_SWEEP, 0)
+    for ly in layers:
+        ly.close()
+
+
 def test_whole_sweep_launch_abandoned_wait_is_reported(ctx):
     """With a single poll per wait the upper layers give up at once: every workgroup still leaves the kernel, and
     zr_ctx_sync reports the incomplete sweep; the next sweep with the default limit is complete again."""
