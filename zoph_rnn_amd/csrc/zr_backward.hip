@@ -177,6 +177,35 @@ __global__ void __launch_bounds__(256) transpose_kernel(const float* __restrict_
   }
 }
 
+// The same with 64 x 64 tiles and 16-byte accesses on both sides, for rows, cols, ldd and row0 multiples of 4 and
+// 16-byte aligned bases (a thread reads four consecutive rows of a source column and writes four consecutive
+// columns, which are consecutive in dst, of a source row).
+__global__ void __launch_bounds__(256) transpose_wide_kernel(const float* __restrict__ src, int rows, int cols,
+                                                             float* __restrict__ dst, long long ldd, int row0) {
+  __shared__ float tile[64][65];
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;  // 16 x 16
+  const int r0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = r0 + 4 * tx, cl = ty + 16 * i, cc = c0 + cl;
+    zr_f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (r < rows && cc < cols) v = *(const zr_f32x4*)(src + r + (long long)cc * rows);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) tile[cl][4 * tx + k] = v[k];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int rl = ty + 16 * i, r = r0 + rl, cc = c0 + 4 * tx;
+    if (r < rows && cc < cols) {
+      zr_f32x4 v;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) v[k] = tile[4 * tx + k][rl];
+      *(zr_f32x4*)(dst + row0 + cc + (long long)r * ldd) = v;
+    }
+  }
+}
+
 // Row sums of a (rows x n, column-major) in two stages with a fixed summation order: stage 1 sums column chunk
 // blockIdx.y for 64 rows per wave into partial[chunk][rows]; stage 2 adds the chunks.
 __global__ void __launch_bounds__(64) row_sum_partial_kernel(const float* __restrict__ a, int rows, long long n,
@@ -188,6 +217,18 @@ __global__ void __launch_bounds__(64) row_sum_partial_kernel(const float* __rest
   float s = 0.0f;
   for (long long k = k0; k < k1; ++k) s += a[r + k * rows];
   partial[(size_t)blockIdx.y * rows + r] = s;
+}
+// The same sums in the same order, four consecutive rows per thread with 16-byte loads (rows % 4 == 0, a 16-byte
+// aligned): 256 rows per wave.
+__global__ void __launch_bounds__(64) row_sum_partial_wide_kernel(const float* __restrict__ a, int rows, long long n,
+                                                                  long long chunk, float* __restrict__ partial) {
+  const int r = (blockIdx.x * 64 + threadIdx.x) * 4;
+  if (r >= rows) return;
+  const long long k0 = (long long)blockIdx.y * chunk;
+  const long long k1 = k0 + chunk < n ? k0 + chunk : n;
+  zr_f32x4 s = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (long long k = k0; k < k1; ++k) s += *(const zr_f32x4*)(a + r + k * rows);
+  *(zr_f32x4*)(partial + (size_t)blockIdx.y * rows + r) = s;
 }
 __global__ void __launch_bounds__(64) row_sum_final_kernel(const float* __restrict__ partial, int rows, int chunks,
                                                            float* __restrict__ out, int accumulate) {
@@ -213,15 +254,28 @@ __global__ void __launch_bounds__(256) embed_grad_kernel(const float* __restrict
 }
 
 // p (V x n probabilities) -> e = onehot(target) - p on unmasked columns, 0 on masked ones, in place.
+// VEC: four consecutive rows per thread with 16-byte accesses (V % 4 == 0, p 16-byte aligned).
+template <bool VEC>
 __global__ void __launch_bounds__(256) softmax_error_kernel(float* __restrict__ p, int V, const int* __restrict__ target,
                                                             const int* __restrict__ mask01) {
   const int col = blockIdx.y;
-  const int v = blockIdx.x * 256 + threadIdx.x;
-  if (v >= V) return;
-  const size_t ix = (size_t)col * V + v;
-  float e = 0.0f;
-  if (mask01[col] == 1) e = (v == target[col] ? 1.0f : 0.0f) - p[ix];
-  p[ix] = e;
+  const bool on = mask01[col] == 1;
+  const int tg = target[col];
+  if (VEC) {
+    const int v = (blockIdx.x * 256 + threadIdx.x) * 4;
+    if (v >= V) return;
+    zr_f32x4* q = (zr_f32x4*)(p + (size_t)col * V + v);
+    const zr_f32x4 x = *q;
+    zr_f32x4 e;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) e[c] = on ? (v + c == tg ? 1.0f : 0.0f) - x[c] : 0.0f;
+    *q = e;
+  } else {
+    const int v = blockIdx.x * 256 + threadIdx.x;
+    if (v >= V) return;
+    const size_t ix = (size_t)col * V + v;
+    p[ix] = on ? (v == tg ? 1.0f : 0.0f) - p[ix] : 0.0f;
+  }
 }
 
 // sum of squares, two deterministic stages
@@ -268,8 +322,13 @@ int row_sum_launch(zr_ctx* ctx, const float* a, int rows, long long n, float* ou
   void* scratch = nullptr;
   int rc = zr_ctx_scratch(ctx, 0, sizeof(float) * (size_t)chunks * rows, &scratch);
   if (rc) return rc;
-  dim3 grid((rows + 63) / 64, chunks);
-  row_sum_partial_kernel<<<grid, 64, 0, ctx->stream>>>(a, rows, n, chunk, (float*)scratch);
+  if (rows % 4 == 0 && aligned16(a) && aligned16(scratch)) {
+    dim3 grid((rows / 4 + 63) / 64, chunks);
+    row_sum_partial_wide_kernel<<<grid, 64, 0, ctx->stream>>>(a, rows, n, chunk, (float*)scratch);
+  } else {
+    dim3 grid((rows + 63) / 64, chunks);
+    row_sum_partial_kernel<<<grid, 64, 0, ctx->stream>>>(a, rows, n, chunk, (float*)scratch);
+  }
   ZR_LAUNCH_CHECK("row_sum_partial_kernel");
   row_sum_final_kernel<<<(rows + 63) / 64, 64, 0, ctx->stream>>>((const float*)scratch, rows, chunks, out,
                                                                            accumulate);
@@ -278,8 +337,13 @@ int row_sum_launch(zr_ctx* ctx, const float* a, int rows, long long n, float* ou
 }
 
 int transpose_launch(zr_ctx* ctx, const float* src, int rows, int cols, float* dst, long long ldd, int row0) {
-  dim3 grid((rows + 31) / 32, (cols + 31) / 32);
-  transpose_kernel<<<grid, 256, 0, ctx->stream>>>(src, rows, cols, dst, ldd, row0);
+  if (rows % 4 == 0 && cols % 4 == 0 && ldd % 4 == 0 && row0 % 4 == 0 && aligned16(src) && aligned16(dst)) {
+    dim3 grid((rows + 63) / 64, (cols + 63) / 64);
+    transpose_wide_kernel<<<grid, 256, 0, ctx->stream>>>(src, rows, cols, dst, ldd, row0);
+  } else {
+    dim3 grid((rows + 31) / 32, (cols + 31) / 32);
+    transpose_kernel<<<grid, 256, 0, ctx->stream>>>(src, rows, cols, dst, ldd, row0);
+  }
   ZR_LAUNCH_CHECK("transpose_kernel");
   return ZR_OK;
 }
@@ -616,8 +680,13 @@ static int softmax_backward(zr_ctx* ctx, const float* d_D, const float* d_b_d, i
     ZR_LAUNCH_CHECK("train_logprob_kernel");
     ZR_HIP(hipMemcpyAsync(h_loss, s0, sizeof(double), hipMemcpyDeviceToHost, ctx->stream));
   }
-  dim3 egrid((V + 255) / 256, n);
-  softmax_error_kernel<<<egrid, 256, 0, ctx->stream>>>(d_prob_scratch, V, d_target, d_mask01);
+  if (V % 4 == 0 && aligned16(d_prob_scratch)) {
+    dim3 egrid((V / 4 + 255) / 256, n);
+    softmax_error_kernel<true><<<egrid, 256, 0, ctx->stream>>>(d_prob_scratch, V, d_target, d_mask01);
+  } else {
+    dim3 egrid((V + 255) / 256, n);
+    softmax_error_kernel<false><<<egrid, 256, 0, ctx->stream>>>(d_prob_scratch, V, d_target, d_mask01);
+  }
   ZR_LAUNCH_CHECK("softmax_error_kernel");
   float* et = (float*)s1;   // n x V
   float* ct = (float*)s0;   // n x H
