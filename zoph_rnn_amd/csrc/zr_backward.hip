@@ -278,18 +278,32 @@ __global__ void __launch_bounds__(256) softmax_error_kernel(float* __restrict__ 
   }
 }
 
-// sum of squares, two deterministic stages
-__global__ void __launch_bounds__(256) sumsq_partial_kernel(const float* __restrict__ g, long long n,
-                                                            double* __restrict__ partial) {
-  __shared__ double s[256];
+// sum of squares, two deterministic stages.  1024 threads per block and 16-byte loads (when g is 16-byte aligned)
+// keep enough bytes in flight to stream a large gradient at memory speed from only gridDim.x = 256 blocks, the
+// number of partial sums the second stage adds up in a fixed order.
+__global__ void __launch_bounds__(1024) sumsq_partial_kernel(const float* __restrict__ g, long long n, int vec,
+                                                             double* __restrict__ partial) {
+  __shared__ double s[1024];
   double acc = 0.0;
-  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) {
+  const long long tid = (long long)blockIdx.x * 1024 + threadIdx.x, nthr = (long long)gridDim.x * 1024;
+  long long done = 0;
+  if (vec) {
+    const long long n4 = n >> 2;
+    const zr_f32x4* g4 = (const zr_f32x4*)g;
+    for (long long i = tid; i < n4; i += nthr) {
+      const zr_f32x4 v = g4[i];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) acc += (double)v[c] * (double)v[c];
+    }
+    done = n4 << 2;
+  }
+  for (long long i = done + tid; i < n; i += nthr) {
     const double v = g[i];
     acc += v * v;
   }
   s[threadIdx.x] = acc;
   __syncthreads();
-  for (int st = 128; st > 0; st >>= 1) {
+  for (int st = 512; st > 0; st >>= 1) {
     if ((int)threadIdx.x < st) s[threadIdx.x] += s[threadIdx.x + st];
     __syncthreads();
   }
@@ -780,7 +794,7 @@ int zr_sgd_update(zr_ctx* ctx, float* d_W, const float* d_grad, long long n, flo
   rc = zr_ctx_scratch(ctx, 1, sizeof(double) * n_partial, &scratch);
   if (rc) return rc;
   if (norm_clip > 0.0f) {
-    sumsq_partial_kernel<<<n_partial, 256, 0, ctx->stream>>>(d_grad, n, (double*)scratch);
+    sumsq_partial_kernel<<<n_partial, 1024, 0, ctx->stream>>>(d_grad, n, aligned16(d_grad) ? 1 : 0, (double*)scratch);
     ZR_LAUNCH_CHECK("sumsq_partial_kernel");
   }
   const long long blocks = (n + 255) / 256;
