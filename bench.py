@@ -30,7 +30,7 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E peak
 # WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for a plain copy of known size
 # (bench.py --calibrate-copy): FETCH_SIZE 3394177.9 KiB x 1.9854 + WRITE_SIZE 400563.6 KiB x 1.0000.
 # The summary of those runs is profiles/lstm_sweep_kernel_config2_hbm_traffic.txt.
-LSTM_SWEEP_TRAFFIC_BYTES = int((3393108.9 * 1.98545 + 401504.6 * 1.0) * 1024)
+LSTM_SWEEP_TRAFFIC_BYTES = int((3393158.5 * 1.98548 + 401142.5 * 1.0) * 1024)
 
 
 def log(*a):
