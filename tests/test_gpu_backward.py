@@ -112,7 +112,7 @@ def test_stack_backward_and_gradients(ctx, L, H, mb, T, V, pad, tail):
     assert np.all(got_e[:, unused] == 0)
 
 
-@pytest.mark.parametrize("V,H,n", [(211, 16, 6), (1003, 48, 70), (5000, 64, 160)])
+@pytest.mark.parametrize("V,H,n", [(211, 16, 6), (1003, 48, 70), (5000, 64, 160), (1000, 32, 1056), (1003, 40, 1030)])
 def test_softmax_backward(ctx, V, H, n):
     g = synth.rng(112, V)
     D, bd, h = U(g, (V, H), -0.5, 0.5), U(g, (V,), -1, 1), U(g, (H, n), -1, 1)
