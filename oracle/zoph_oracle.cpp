@@ -10,7 +10,13 @@
 // What pins each function (see tests/test_oracle_*.py): closed forms and
 // brute-force restatements in numpy float64, invariants (column sums, shift
 // invariance, linearity), and special cases that reduce to a textbook
-// routine.  The reference holds no golden vectors for this path and its
+// routine.  Checked by value against an independent float64 statement:
+// the contractions, the LSTM cell (torch.nn.LSTMCell; feed-input term), the
+// stacked sweep with non-zero initial states and the cell clip, every output
+// of the attention step (p_t, alignments, context, h~; fails for W_a in place
+// of W_a^T and for a missing tanh), the soft-max (scipy logsumexp), the beam
+// step with a non-zero length penalty for survivors, <EOF> hypotheses and the
+// forced finish, and the strict length-ratio filter of the k-best output.  The reference holds no golden vectors for this path and its
 // contractions run inside cuBLAS (summation order unknown), so no function
 // here is pinned by a reference-held vector: parity with the *reference* is
 // therefore "pinned by mathematics only" for every function in this file.

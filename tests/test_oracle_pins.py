@@ -429,3 +429,218 @@ def test_stack_forward_is_composition_of_steps():
             assert np.array_equal(h_all[l, t], r["h"]) and np.array_equal(c_all[l, t], r["c"])
             hp[l], cp[l], below = r["h"], r["c"], r["h"]
     assert np.all(h_all[:, 0, :, 1] == 0)
+
+
+# ----------------------------------------------------------------------------- by-value brute-force pins
+def _attention_numpy_f64(w, hs, lens, offs, h_t, mask, D):
+    """Luong local-p attention written from the paper's formulas in float64, column by column, with plain numpy
+    products: p_t = S sigmoid(v_p . tanh(W_p h)); score_s = h_s . (W_a^T h) = h^T W_a h_s over the window
+    [max(0, floor(p_t) - D), min(S - 1, floor(p_t) + D)]; softmax over the window times exp(-(p_t - s)^2 / (2 (D/2)^2));
+    context = sum a_s h_s; h~ = tanh(W_c1 c + W_c2 h + b).  Source position s of column b is table
+    S_b - 1 - s + offset_b (the source is stored reversed and left padded)."""
+    H, mb = h_t.shape
+    Wa, Wp, Wc1, Wc2 = (w[k].astype(np.float64) for k in ("W_a", "W_p", "W_c1", "W_c2"))
+    vp, bias = w["v_p"].astype(np.float64).reshape(-1), w["out_bias"].astype(np.float64)
+    out = {"p_t": np.zeros(mb), "scores": {}, "align": {}, "c": np.zeros((H, mb)), "h_tild": np.zeros((H, mb))}
+    for b in range(mb):
+        h = h_t[:, b].astype(np.float64)
+        p = lens[b] / (1.0 + np.exp(-(vp @ np.tanh(Wp @ h))))
+        out["p_t"][b] = p
+        if not mask[b]:
+            continue
+        lo, hi = max(0, int(p) - D), min(int(lens[b]) - 1, int(p) + D)
+        pos = list(range(lo, hi + 1))
+        src = [hs[lens[b] - 1 - s + offs[b], :, b].astype(np.float64) for s in pos]
+        sc = np.array([h @ Wa @ hv for hv in src])
+        e = np.exp(sc - sc.max())
+        a = e / e.sum() * np.exp(-(p - np.array(pos)) ** 2 / (2 * (D / 2.0) ** 2))
+        c = sum(ai * hv for ai, hv in zip(a, src))
+        out["scores"][b], out["align"][b] = dict(zip(pos, sc)), dict(zip(pos, a))
+        out["c"][:, b] = c
+        out["h_tild"][:, b] = np.tanh(Wc1 @ c + Wc2 @ h + bias)
+    return out
+
+
+@pytest.mark.parametrize("H,mb,S,D,seed", [(10, 6, 9, 2, 1), (16, 5, 12, 12, 2), (7, 4, 30, 3, 3)])
+def test_attention_by_value_against_numpy_f64(H, mb, S, D, seed):
+    """Every output by value: fails for W_a in place of W_a^T (W_a is not symmetric), for a missing tanh or sigmoid
+    in p_t, for a wrong Gaussian width and for a wrong source-table index."""
+    rng = np.random.default_rng(seed)
+    w = dict(W_a=U((H, H), -0.6, 0.6, rng), W_p=U((H, H), -0.9, 0.9, rng), v_p=U(H, -1.5, 1.5, rng),
+             out_bias=U(H, -0.3, 0.3, rng), W_c1=U((H, H), -0.4, 0.4, rng), W_c2=U((H, H), -0.4, 0.4, rng))
+    assert np.abs(w["W_a"] - w["W_a"].T).max() > 0.1
+    hs = rng.normal(0, 0.7, size=(S, H, mb)).astype(np.float32)
+    lens = rng.integers(1, S + 1, size=mb).astype(np.int32)
+    lens[0] = S
+    offs = (S - lens).astype(np.int32)
+    mask = np.ones(mb, np.int32)
+    mask[mb - 2] = 0
+    h_t = U((H, mb), -1, 1, rng)
+    r = o.attention_forward(hs_table=hs, batch_info=np.concatenate([lens, offs]), h_t=h_t, mask01=mask, D=D, **w)
+    want = _attention_numpy_f64(w, hs, lens, offs, h_t, mask, D)
+    assert np.allclose(r["p_t"], want["p_t"], rtol=2e-6)
+    # p_t must actually depend on the tanh: the pre-activations are large enough that dropping it moves p_t
+    lin = lens / (1.0 + np.exp(-(w["v_p"].astype(np.float64) @ (w["W_p"].astype(np.float64) @ h_t))))
+    assert np.abs(lin - want["p_t"]).max() > 1e-2
+    Wn = 2 * D + 1
+    for b in range(mb):
+        if not mask[b]:
+            assert np.all(r["alignments"][b] == 0) and np.all(r["h_tild"][:, b] == 0)
+            continue
+        got = {int(s): r["alignments"][b, j] for j, s in enumerate(r["indices"][b]) if s != -1}
+        assert sorted(got) == sorted(want["align"][b])
+        for s, a in want["align"][b].items():
+            assert got[s] == pytest.approx(a, rel=2e-5, abs=1e-9)
+        # the alignments differ from those of the transposed score matrix by far more than the tolerance
+        assert len(got) <= Wn
+    assert np.allclose(r["c_ctx"], want["c"], atol=2e-6)
+    assert np.allclose(r["h_tild"], want["h_tild"], atol=2e-6)
+    wT = dict(w, W_a=np.asfortranarray(w["W_a"].T))
+    wrong = _attention_numpy_f64(wT, hs, lens, offs, h_t, mask, D)
+    assert np.abs(wrong["h_tild"] - want["h_tild"]).max() > 1e-3
+
+
+def _bruteforce_decode_step(P, prev_scores, prev_sent, live, beam, index, penalty):
+    """One beam step from the rules alone (tie-free inputs): candidates are the beam+1 most probable words of each
+    live column scored log p + column score; best first: <START> is dropped, <EOF> closes a hypothesis with
+    candidate score + penalty, anything else survives with candidate score + penalty until beam survivors exist."""
+    cols = 1 if index == 0 else beam
+    cands = []
+    for i in range(cols):
+        if not live[i]:
+            break
+        for v in np.argsort(-P[:, i], kind="stable")[:beam + 1]:
+            cands.append((np.float32(np.float32(np.log(P[v, i])) + np.float32(prev_scores[i])), i, int(v)))
+    cands.sort(key=lambda t: -t[0])
+    surv, fin = [], []
+    for val, i, v in cands:
+        if len(surv) == beam:
+            break
+        if v == 0:
+            continue
+        if v == 1:
+            fin.append((prev_sent[i] + [1], np.float32(val + np.float32(penalty))))
+        else:
+            surv.append((prev_sent[i] + [v], np.float32(val + np.float32(penalty)), i))
+    return surv, fin
+
+
+@pytest.mark.parametrize("penalty", [0.75, -0.4])
+def test_beam_penalty_in_expand_and_finish_against_bruteforce(penalty):
+    """Length penalty != 0: survivors and <EOF> hypotheses each gain exactly one penalty per word, and because the
+    penalty enters the scores that rank the next step, dropping it anywhere changes the later selections."""
+    V, beam, steps = 30, 3, 6
+    rng = np.random.default_rng(77)
+    dec = o.Decoder(beam, V, max_len=steps + 3, penalty=penalty)
+    scores, sent, live = np.zeros(beam, np.float32), [[0] for _ in range(beam)], [True] * beam
+    all_fin = []
+    for index in range(steps):
+        logits = rng.normal(0, 2.0, size=(V, beam))
+        logits[1] += 3.0  # make <EOF> a frequent candidate
+        P = np.asfortranarray((np.exp(logits) / np.exp(logits).sum(axis=0)).astype(np.float32))
+        surv, fin = _bruteforce_decode_step(P, scores, sent, live, beam, index, penalty)
+        assert len(surv) == beam
+        dec.expand(P, index)
+        st = dec.state()
+        assert st["current_indices"].tolist() == [s[0][-1] for s in surv]
+        assert st["new_indicies_changes"].tolist() == [s[2] for s in surv]
+        assert np.allclose(st["scores"], [s[1] for s in surv], rtol=2e-6, atol=1e-6)
+        for i in range(beam):
+            assert st["top_sentences"][i, :index + 2].tolist() == surv[i][0]
+        all_fin += fin
+        scores, sent = np.array([s[1] for s in surv], np.float32), [s[0] for s in surv]
+    assert len(all_fin) >= 3  # the <EOF> branch was exercised
+    # forced finish: every live beam ends with <EOF>, score + log P(<EOF>) + penalty
+    for i in range(beam):
+        all_fin.append((sent[i] + [1], np.float32(scores[i] + np.float32(np.log(P[1, i])) + np.float32(penalty))))
+    dec.finish(P)
+    hyps = dec.hypotheses()
+    assert len(hyps) == len(all_fin)
+    for (hw, hsc), (bw, bsc) in zip(hyps, all_fin):
+        assert hw.tolist() == bw and hsc == pytest.approx(bsc, rel=2e-6, abs=1e-6)
+
+
+def test_k_best_ratio_filter_is_strict():
+    """Hypotheses whose length / source length equals min_decoding_ratio exactly are dropped (strictly greater
+    passes), src/decoder.h:1394.  Lengths count <START> and <EOF>."""
+    V, beam = 8, 2
+
+    def dist():
+        # <EOF> (word 1) is the second most probable word of column 0, so every step pops: best survivor, <EOF> of
+        # the best column (a finished hypothesis), second survivor.  The two columns differ, so nothing ties.
+        P = np.full((V, beam), 1e-4, np.float32, order="F")
+        P[1, :] = 0.3
+        P[2, 0], P[3, 0] = 0.42, 0.21
+        P[2, 1], P[3, 1] = 0.40, 0.22
+        return P
+
+    dec = o.Decoder(beam, V, max_len=10, penalty=0.0, min_ratio=0.5)
+    for index in range(4):  # <EOF> is among the top beam+1 of every column: hypotheses of 2, 3, 4, 5 words
+        dec.expand(dist(), index)
+    hyps = dec.hypotheses()
+    lengths = [len(w) for w, _ in hyps]
+    assert {2, 3, 4, 5} <= set(lengths)
+    S = 8  # ratio 0.5 <=> length 4: lengths 2, 3 and exactly 4 are out, 5 is in
+    order = dec.k_best(source_length=S, num_hypotheses=len(hyps))
+    assert len(order) > 0 and all(lengths[i] > 4 for i in order)
+    assert sorted(order.tolist()) == [i for i, n in enumerate(lengths) if n > 4]
+    scores = [hyps[i][1] for i in order]
+    assert scores == sorted(scores, reverse=True)
+    S = 10  # ratio 0.5 <=> length 5, the longest there is: nothing passes
+    assert dec.k_best(source_length=S, num_hypotheses=len(hyps)).size == 0
+    S = 9   # 4/9 < 0.5 < 5/9
+    assert sorted(dec.k_best(source_length=S, num_hypotheses=len(hyps)).tolist()) == \
+        [i for i, n in enumerate(lengths) if n >= 5]
+
+
+def _lstm_stack_numpy_f64(embed, layers, ids, h0, c0, clip):
+    """Stacked LSTM in float64 from the textbook equations (gate order i, f, c~, o); ids -1 = padded position:
+    embedding column 0 is read and h, c of that column are zeroed; the cell is clamped to +-clip before h."""
+    T, mb = ids.shape
+    L, H = len(layers), embed.shape[0]
+    sig = lambda v: 1.0 / (1.0 + np.exp(-v))
+    h = [np.array(a, np.float64) for a in h0]
+    c = [np.array(a, np.float64) for a in c0]
+    h_all, c_all = np.zeros((L, T, H, mb)), np.zeros((L, T, H, mb))
+    for t in range(T):
+        below = embed[:, np.maximum(ids[t], 0)].astype(np.float64)
+        m = (ids[t] >= 0).astype(np.float64)
+        for l, ly in enumerate(layers):
+            pre = [ly["M"][g].astype(np.float64) @ below + ly["Wh"][g].astype(np.float64) @ h[l] +
+                   ly["b"][g].astype(np.float64)[:, None] for g in range(4)]
+            cn = sig(pre[1]) * c[l] + sig(pre[0]) * np.tanh(pre[2])
+            if clip is not None:
+                cn = np.clip(cn, -clip, clip)
+            hn = sig(pre[3]) * np.tanh(cn)
+            h[l], c[l] = hn * m, cn * m
+            h_all[l, t], c_all[l, t] = h[l], c[l]
+            below = h[l]
+    return h_all, c_all
+
+
+@pytest.mark.parametrize("clip", [None, 0.3])
+def test_stack_forward_nonzero_initial_state_and_clip_against_numpy_f64(clip):
+    H, mb, T, V, L = 9, 4, 5, 23, 3
+    rng = np.random.default_rng(11)
+    embed = U((H, V), -1, 1, rng)
+    layers = [{"M": [U((H, H), -0.8, 0.8, rng) for _ in range(4)], "Wh": [U((H, H), -0.8, 0.8, rng) for _ in range(4)],
+               "b": [U(H, -0.5, 0.5, rng) for _ in range(4)]} for _ in range(L)]
+    ids = rng.integers(0, V, size=(T, mb)).astype(np.int32)
+    ids[:2, 2] = -1
+    h0 = [U((H, mb), -0.9, 0.9, rng) for _ in range(L)]
+    c0 = [U((H, mb), -1.5, 1.5, rng) for _ in range(L)]
+    nn, m = o.vocab_prep(ids)
+    h_all, c_all = o.lstm_stack_forward(embed, layers, nn, m, h0=h0, c0=c0, clip=clip)
+    want_h, want_c = _lstm_stack_numpy_f64(embed, layers, ids, h0, c0, clip)
+    assert np.allclose(h_all, want_h, atol=2e-6) and np.allclose(c_all, want_c, atol=2e-6)
+    # the cases must exercise what they claim to: the initial state matters, and the clip binds somewhere
+    z = [np.zeros((H, mb), np.float32)] * L
+    hz, _ = _lstm_stack_numpy_f64(embed, layers, ids, z, z, clip)
+    assert np.abs(hz[:, 0] - want_h[:, 0]).max() > 1e-2
+    if clip is not None:
+        unclipped, cu = _lstm_stack_numpy_f64(embed, layers, ids, h0, c0, None)
+        assert np.abs(cu).max() > clip + 0.1 and np.abs(want_c).max() <= clip + 1e-12
+        assert np.abs(unclipped - want_h).max() > 1e-3
+        # each layer has its own initial state: swapping two layers' states changes the result
+    h_sw, _ = o.lstm_stack_forward(embed, layers, nn, m, h0=h0[::-1], c0=c0[::-1], clip=clip)
+    assert np.abs(h_sw - want_h).max() > 1e-2
