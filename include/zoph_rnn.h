@@ -189,6 +189,16 @@ int zr_softmax_release(zr_ctx* ctx, const float* d_D);
  * d_out: V x mb.  d_logits_scratch: V x mb scratch for the logits, or NULL to use d_out in place. */
 int zr_softmax_forward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int mb,
                        int mode, float* d_out, float* d_logits_scratch);
+/* zr_softmax_forward for callers that cannot allocate device memory (code under HIP graph capture, serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments, same kernels and
+ * bit-identical results, but the product's scratch memory (the activations re-laid-out for the matrix cores and the
+ * per-32-row partial column statistics) lives in a 32 MiB array that is part of the library's device image on every
+ * GPU it runs on, so the call itself allocates and frees nothing.  Limits (ZR_EINVAL beyond them, message in
+ * zr_last_error): H*mb*4 <= 8 MiB and ceil(V/32)*mb*8 + 16*mb + 64 <= 24 MiB -- e.g. V = 80000 with 256 columns
+ * of H = 2000 fits, 6400 columns of V = 50000 do not.  Every call on one GPU shares that GPU's array: calls that overlap
+ * on one GPU (two contexts, two streams) race; calls on one context are ordered by its stream and safe. */
+int zr_softmax_forward_static(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h,
+                              int mb, int mode, float* d_out, float* d_logits_scratch);
 /* softmax_layer::get_perplexity_GPU (src/softmax.hpp:636-692) with outputdist_perplexity_kernel
  * (src/custom_kernels.h:583-660): double log-probabilities, V x mb. */
 int zr_softmax_logprob_f64(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int mb,

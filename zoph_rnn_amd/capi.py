@@ -36,6 +36,7 @@ SYMBOLS = [
     "zr_unstack_gates", "zr_lstm_stack_backward", "zr_lstm_weight_gradients", "zr_embed_gradient",
     "zr_softmax_backward", "zr_sgd_update", "zr_lstm_node_backward", "zr_lstm_node_gradients",
     "zr_softmax_backward_accumulate", "zr_gather_columns_multi", "zr_softmax_backward_loss",
+    "zr_softmax_forward_static",
 ]
 
 _lib = None
@@ -287,9 +288,11 @@ class Context:
     def softmax_release(self, d_D):
         _chk(load().zr_softmax_release(self.h, _vp(d_D)))
 
-    def softmax_forward(self, d_D, d_b, V, H, d_h, mb, mode, d_out, d_scratch=None):
-        _chk(load().zr_softmax_forward(self.h, _vp(d_D), _vp(d_b), C.c_int(V), C.c_int(H), _vp(d_h), C.c_int(mb),
-                                       C.c_int(mode), _vp(d_out), _vp(d_scratch)))
+    def softmax_forward(self, d_D, d_b, V, H, d_h, mb, mode, d_out, d_scratch=None, static=False):
+        """static=True: the allocation-free entry point (scratch in the library's static device array)."""
+        fn = load().zr_softmax_forward_static if static else load().zr_softmax_forward
+        _chk(fn(self.h, _vp(d_D), _vp(d_b), C.c_int(V), C.c_int(H), _vp(d_h), C.c_int(mb),
+                C.c_int(mode), _vp(d_out), _vp(d_scratch)))
 
     def softmax_logprob_f64(self, d_D, d_b, V, H, d_h, mb, d_logp, d_scratch):
         _chk(load().zr_softmax_logprob_f64(self.h, _vp(d_D), _vp(d_b), C.c_int(V), C.c_int(H), _vp(d_h), C.c_int(mb),

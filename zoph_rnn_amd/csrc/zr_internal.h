@@ -34,6 +34,12 @@ struct zr_ctx {
   size_t scratch_bytes;
   void* d_scratch2;
   size_t scratch2_bytes;
+  // the device's statically allocated scratch array (zr_runtime.hip), resolved when the context is created
+  void* d_static_scratch;
+  // while set, zr_ctx_scratch hands out these fixed buffers (slot 0 / slot 1) and never allocates
+  int fixed_scratch;
+  void* d_fixed[2];
+  size_t fixed_bytes[2];
   // output-layer matrices registered with zr_softmax_prepare: the caller's D pointer -> its k-interleaved copy
   struct PackedD {
     const float* key;  // the caller's d_D (null: slot free)
@@ -72,6 +78,10 @@ int zr_bind_device(zr_ctx* ctx);
 int zr_live_contexts(int device);
 // Returns a context-owned scratch buffer of at least `bytes` (slot 0 or 1).
 int zr_ctx_scratch(zr_ctx* ctx, int slot, size_t bytes, void** out);
+// Size of the statically allocated device scratch array every GPU holds for the allocation-free entry point, and
+// how that entry point divides it between the two scratch slots.
+#define ZR_STATIC_SCRATCH_BYTES (32u << 20)
+#define ZR_STATIC_SCRATCH_SLOT0_BYTES (8u << 20)
 
 // MFMA vector types ------------------------------------------------------------------------------------------
 typedef float zr_f32x16 __attribute__((ext_vector_type(16)));

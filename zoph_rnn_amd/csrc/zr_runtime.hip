@@ -5,8 +5,31 @@
 #include <string.h>
 
 #include <atomic>
+#include <mutex>
 
 #include "zr_internal.h"
+
+// Scratch memory of the allocation-free entry point (zr_softmax_forward_static): every GPU the library runs on holds
+// its own copy of this array until the process ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress; the device address differs per GPU and is looked up once per device, with that device
+// current (static_scratch_address), and only that address is ever passed to kernels.
+static __device__ __align__(256) unsigned char scratch[ZR_STATIC_SCRATCH_BYTES];
+static void* g_static_scratch[64];
+static std::mutex g_static_scratch_mu;
+
+// Device address of `scratch` on the current device (which must be `device`).
+static int static_scratch_address(int device, void** out) {
+  std::lock_guard<std::mutex> lock(g_static_scratch_mu);
+  if (device < 0 || device >= 64) return zr_set_error(ZR_EINVAL, "device %d has no static scratch slot", device);
+  if (!g_static_scratch[device]) {
+    void* ptr = nullptr;
+    ZR_HIP(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)));
+    if (!ptr) return zr_set_error(ZR_EHIP, "hipGetSymbolAddress returned a null address for the static scratch array");
+    g_static_scratch[device] = ptr;
+  }
+  *out = g_static_scratch[device];
+  return ZR_OK;
+}
 
 static thread_local char g_err[512] = "";
 
@@ -30,6 +53,14 @@ int zr_bind_device(zr_ctx* ctx) {
 }
 
 int zr_ctx_scratch(zr_ctx* ctx, int slot, size_t bytes, void** out) {
+  if (ctx->fixed_scratch) {
+    if (bytes > ctx->fixed_bytes[slot])
+      return zr_set_error(ZR_EINVAL, "this call needs %zu bytes of scratch memory (%s) but the allocation-free entry "
+                          "point has %zu: use the allocating entry point for this size", bytes,
+                          slot == 0 ? "re-laid-out activations" : "partial column statistics", ctx->fixed_bytes[slot]);
+    *out = ctx->d_fixed[slot];
+    return ZR_OK;
+  }
   void** buf = slot == 0 ? &ctx->d_scratch : &ctx->d_scratch2;
   size_t* cap = slot == 0 ? &ctx->scratch_bytes : &ctx->scratch2_bytes;
   if (*cap < bytes) {
@@ -79,6 +110,15 @@ int zr_ctx_create(int device, zr_ctx** out) {
   }
   (void)hipMemset(c->d_flags, 0, (4 + ZR_MAX_COUNTERS) * sizeof(int));
   c->d_counters = c->d_flags + 4;
+  {
+    const int rc = static_scratch_address(device, &c->d_static_scratch);
+    if (rc) {
+      (void)hipFree(c->d_flags);
+      (void)hipStreamDestroy(c->own_stream);
+      delete c;
+      return rc;
+    }
+  }
   c->lstm_fused = 1;
   // ZR_LSTM_SWEEP in the environment presets ZR_OPT_LSTM_SWEEP for every context of the process (0, 1 or 2): lets a
   // whole program, e.g. a test run, be put on one path or the other without touching its code

@@ -300,6 +300,22 @@ int zr_softmax_forward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V,
   return ZR_OK;
 }
 
+// zr_softmax_forward on the device's statically allocated scratch array: same kernels, no allocation.  The array is
+// split into the two buffers the product needs (re-laid-out activations, then partial column statistics + column
+// statistics); both are fully written before they are read, so nothing has to be cleared between calls.
+int zr_softmax_forward_static(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int mb,
+                              int mode, float* d_out, float* d_logits_scratch) {
+  ZR_CHECK_ARG(ctx != nullptr && ctx->d_static_scratch != nullptr, "zr_softmax_forward_static: null context");
+  ctx->fixed_scratch = 1;
+  ctx->d_fixed[0] = ctx->d_static_scratch;
+  ctx->fixed_bytes[0] = ZR_STATIC_SCRATCH_SLOT0_BYTES;
+  ctx->d_fixed[1] = (char*)ctx->d_static_scratch + ZR_STATIC_SCRATCH_SLOT0_BYTES;
+  ctx->fixed_bytes[1] = ZR_STATIC_SCRATCH_BYTES - ZR_STATIC_SCRATCH_SLOT0_BYTES;
+  const int rc = zr_softmax_forward(ctx, d_D, d_b_d, V, H, d_h, mb, mode, d_out, d_logits_scratch);
+  ctx->fixed_scratch = 0;
+  return rc;
+}
+
 int zr_softmax_logprob_f64(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int mb,
                            double* d_logp, float* d_logits_scratch) {
   int rc = zr_bind_device(ctx);
