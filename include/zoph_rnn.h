@@ -54,6 +54,18 @@ int zr_timer_start(zr_ctx* ctx);
 int zr_timer_stop(zr_ctx* ctx, float* h_ms);
 /* Tuning / mode switches: see ZR_OPT_* below. */
 int zr_ctx_set_option(zr_ctx* ctx, int option, int value);
+/* State of the context that a caller may want to look at (no counterpart in the reference):
+ *   ZR_QUERY_LSTM_STACK_PATH: which schedule the last zr_lstm_stack_forward(_train) call on this context took --
+ *     0 none yet, ZR_LSTM_STACK_PATH_SWEEP (one launch for the whole sweep) or ZR_LSTM_STACK_PATH_DIAGONALS (one
+ *     launch per diagonal).  Does not wait.
+ *   ZR_QUERY_LSTM_SWEEP_ABANDONED: waits for the stream; 1 if a single-launch sweep since the last look gave up a wait
+ *     (its outputs were then overwritten with NaN; run the sweep again with ZR_OPT_LSTM_SWEEP = 1), else 0.  Clears
+ *     the flag, so a following zr_ctx_sync no longer reports it. */
+int zr_ctx_query(zr_ctx* ctx, int what, int* h_value);
+#define ZR_QUERY_LSTM_STACK_PATH 1
+#define ZR_QUERY_LSTM_SWEEP_ABANDONED 2
+#define ZR_LSTM_STACK_PATH_SWEEP 1
+#define ZR_LSTM_STACK_PATH_DIAGONALS 2
 const char* zr_last_error(void);
 /* Library self-description: "gfx950 hip <build tag>". */
 const char* zr_version(void);
@@ -72,7 +84,8 @@ const char* zr_version(void);
 #define ZR_OPT_LSTM_KPARTS 6         /* kernels 2 and 3: K parts per weight segment (0 = auto) */
 #define ZR_OPT_LSTM_SWEEP 7          /* zr_lstm_stack_forward as ONE launch whose workgroups hand h to each other
                                         through device memory: 0 auto (when they fill most of the device, are all
-                                        resident at once and the context is the process's only one on its device),
+                                        resident at once, the context is the process's only one on its device and
+                                        runs on its own stream),
                                         1 never (one launch per diagonal), 2 whenever they fit.  The environment
                                         variable ZR_LSTM_SWEEP presets this option for every context created */
 #define ZR_OPT_LSTM_SWEEP_SPIN 8     /* polls a workgroup of that launch spends on one wait before it gives up

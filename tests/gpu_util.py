@@ -26,6 +26,15 @@ def assert_close(got, want, rel=REL, floor=FLOOR, what=""):
                              % (what, int(bad.sum()), bad.size, i, got[i], want[i], err[i], bound[i]))
 
 
+def magnitude_floor(want):
+    """Floor for assert_close on products of operands much larger than the model's own (tests that draw U(-0.5, 0.5)
+    matrices against U(-1, 1) activations reach logits of +-28 at H = 1000): fp32 accumulation noise is about
+    eps * sqrt(K) times the size of the PARTIAL sums, which follow the largest entries of the result, not the entry
+    being compared, so the near-zero floor scales with the largest magnitude: 0.05 * max(1, max |want|).  With
+    max |want| <= 1 this is the ordinary floor."""
+    return FLOOR * max(1.0, float(np.max(np.abs(want))))
+
+
 def round_bf16(a):
     """fp32 array rounded to the nearest bf16-representable value (ties to even), returned as fp32, same layout."""
     a = np.asarray(a, dtype=np.float32)

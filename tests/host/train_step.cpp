@@ -1,9 +1,11 @@
 // Test driver: SGD steps of model_trainer (zoph_rnn_amd/host/zoph_model.h) on the minibatches of an integerized file.
-//   train_step [--sequence] [--node-level] model.nn data.int minibatch longest_sent learning_rate norm_clip steps
+//   train_step [--sequence] [--node-level] [--abandon-sweeps] model.nn data.int minibatch longest_sent learning_rate norm_clip steps
 // Every step trains on the next minibatch of the file (wrapping around) and prints "loss <step> <log-likelihood>";
 // the updated model is written to <model.nn>.trained as a complete model file.  --node-level: the step is
 // forward_model::compute_gradients, i.e. the layer objects' own back_prop_GPU / update_weights members in the
-// reference's node-by-node order, instead of model_trainer's stack-level calls.
+// reference's node-by-node order, instead of model_trainer's stack-level calls.  --abandon-sweeps: the forward pass is
+// forced onto the single-launch sweep with a wait limit of one poll, so its workgroups give up (and leave the kernel
+// normally); model_trainer must notice and repeat the forward pass; prints "abandoned <count>" at the end.
 #include <cstdio>
 #include <cstdlib>
 #include <iostream>
@@ -13,13 +15,15 @@
 #include "../../zoph_rnn_amd/host/zoph_model.h"
 
 int main(int argc, char** argv) {
-  bool LM = false, node_level = false;
+  bool LM = false, node_level = false, abandon = false;
   std::vector<std::string> pos;
   for (int i = 1; i < argc; i++) {
     if (std::string(argv[i]) == "--sequence")
       LM = true;
     else if (std::string(argv[i]) == "--node-level")
       node_level = true;
+    else if (std::string(argv[i]) == "--abandon-sweeps")
+      abandon = true;
     else
       pos.push_back(argv[i]);
   }
@@ -45,6 +49,11 @@ int main(int argc, char** argv) {
   m.initModel(gpu, info, minibatch, longest, 10);
   m.load_weights(model);
   model_trainer<precision>* trainer = node_level ? nullptr : new model_trainer<precision>(m);
+  if (abandon && trainer) {
+    ZOPH_CALL(zr_ctx_set_option(gpu.ctx, ZR_OPT_LSTM_SWEEP, 2));
+    ZOPH_CALL(zr_ctx_set_option(gpu.ctx, ZR_OPT_LSTM_SWEEP_SPIN, 1));
+    trainer->lstm_sweep_option = 2;
+  }
   minibatch_reader reader;
   if (!reader.open(pos[1], minibatch, longest, LM)) {
     std::fprintf(stderr, "cannot open %s\n", pos[1].c_str());
@@ -70,6 +79,7 @@ int main(int argc, char** argv) {
     }
     std::cout << "loss " << s << " " << loss << "\n";
   }
+  if (trainer) std::cout << "abandoned " << trainer->abandoned_sweeps << "\n";
   devSynchAll(gpu.ctx);
   std::ofstream out(pos[0] + ".trained");
   m.dump_weights(out);

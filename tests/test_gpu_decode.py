@@ -66,14 +66,17 @@ def _oracle_decode(m, src_col, src_len, S, beam, steps, D, penalty):
 
     for index in range(steps):
         newh, newc, att, P = forward(index)
-        # how close the closest pair of candidate scores is (the test is only meaningful without near-ties)
+        # how close the closest pair of candidate scores is among those the step can pop (the test is only meaningful
+        # without near-ties there; further down the list the order of candidates has no effect on anything)
         cols = 1 if index == 0 else beam
         sc = dec.state()["scores"]
-        cand = np.sort(np.concatenate([np.log(np.sort(P[:, i])[-(beam + 2):]) + sc[i] for i in range(cols)]))
-        min_gap = min(min_gap, np.min(np.diff(cand)))
+        cand = np.sort(np.concatenate([np.log(np.sort(P[:, i])[-(beam + 2):]) + sc[i] for i in range(cols)]))[::-1]
+        n_hyp_before = len(dec.hypotheses())
         frac = att["p_t"] - np.floor(att["p_t"])
         assert np.all((frac > 1e-4) & (frac < 1 - 1e-4)), "p_t on an integer boundary; pick another seed"
         dec.expand(P, index)
+        popped = beam + (len(dec.hypotheses()) - n_hyp_before) + 2  # survivors + <EOF> hypotheses (+ a <START>) + next
+        min_gap = min(min_gap, np.min(-np.diff(cand[:popped + 1])))
         st = dec.state()
         words, back = st["current_indices"].copy(), st["new_indicies_changes"].copy()
         hist.append((words.copy(), back.copy()))
@@ -114,4 +117,53 @@ def test_batched_beam_decode_matches_per_sentence_reference(ctx, H, L, beam, n_s
         for (gwords, gscore), (wwords, wscore) in zip(got, hyps):
             assert np.array_equal(gwords, wwords)
             assert gscore == pytest.approx(wscore, rel=1e-4, abs=1e-4)
+    dec.close()
+
+
+def test_config4_beam_decode_at_full_size(ctx):
+    """Benchmark configuration 4 at its real shape: 4 layers, H = 1000, beam 12 x 16 sentences = 192 live columns,
+    source length 50, both vocabularies 50 000, attention window D = 50 (every source position has a slot), feed-input.
+    Six decode steps and the forced finish; three of the sixteen sentences (first, middle, last: different source
+    lengths) are decoded one at a time by the oracle, as the reference does, and every selected word, back-pointer
+    and finished hypothesis must be identical.  LSTM and attention weights have the benchmark's U(-0.08, 0.08) range;
+    the output matrix is drawn wider so that candidate scores are separated by far more than fp32 noise."""
+    H, L, beam, n_sent, S, steps, D = 1000, 4, 12, 16, 50, 6, 50
+    Vs = Vt = 50000
+    g = synth.rng(64, 4)
+    m = {"src_embed": synth.uniform(g, (H, Vs)), "tgt_embed": synth.uniform(g, (H, Vt), -0.5, 0.5),
+         "src_layers": [synth.lstm_layer(g, H, forget_bias_one=True) for _ in range(L)],
+         "tgt_layers": [synth.lstm_layer(g, H, feed_input=(l == 0), forget_bias_one=True) for l in range(L)],
+         "attn": synth.attention_weights(g, H),
+         "D_soft": synth.uniform(g, (Vt, H), -0.5, 0.5), "b_soft": synth.uniform(g, (Vt,), -1.0, 1.0)}
+    lens = g.integers(S - 12, S + 1, size=n_sent).astype(np.int32)
+    lens[0] = S
+    src = synth.zipf_ids(g, (S, n_sent), Vs)
+    for s in range(n_sent):
+        src[:S - lens[s], s] = -1
+    w = driver.Seq2SeqWeights(ctx, m["src_embed"], m["src_layers"], m["tgt_embed"], m["tgt_layers"], m["attn"],
+                              m["D_soft"], m["b_soft"])
+    dec = driver.BeamDecode(ctx, w, beam, n_sent, S, steps, attention_D=D, penalty=0.0)
+    dec.encode(src, lens)
+    for _ in range(steps):
+        dec.step(record=True)
+    dec.finish()
+    checked = 0
+    for s in (0, n_sent // 2, n_sent - 1):
+        hist, hyps, gap = _oracle_decode(m, src[:, s], int(lens[s]), S, beam, steps, D, 0.0)
+        assert gap > 5e-6, "candidate scores nearly tie (gap %.2e): pick another seed" % gap
+        for index in range(steps):
+            gw, gb = dec.history[index]
+            assert np.array_equal(gw[s * beam:(s + 1) * beam], hist[index][0]), (s, index)
+            assert np.array_equal(gb[s * beam:(s + 1) * beam] - s * beam, hist[index][1]), (s, index)
+        got = dec.hypotheses(s)
+        assert len(got) == len(hyps) and len(got) >= beam
+        for (gwords, gscore), (wwords, wscore) in zip(got, hyps):
+            assert np.array_equal(gwords, wwords)
+            assert gscore == pytest.approx(wscore, rel=1e-4, abs=1e-4)
+        checked += 1
+    assert checked == 3
+    # every sentence's words lie in the vocabulary and no beam slot died (192 live hypotheses throughout)
+    for index in range(steps):
+        gw, gb = dec.history[index]
+        assert np.all((gw >= 2) & (gw < Vt)) and np.all((gb // beam) == np.repeat(np.arange(n_sent), beam))
     dec.close()

@@ -125,10 +125,17 @@ def _compare(name, got, want, orig):
         name, err, tol, np.abs(d_want).max())
 
 
+def test_abandoned_forward_sweep_is_repeated_before_the_update(tmp_path):
+    """The forward sweeps are made to give up their waits (one poll allowed; every workgroup still leaves the kernel
+    normally): model_trainer must see it, run the forward pass again with one launch per diagonal, and end with the
+    oracle's weights -- nothing of the abandoned sweep's outputs may reach them."""
+    test_train_steps_match_oracle(tmp_path, True, 3, 64, 8, 2, 1.0, False, abandon=True)
+
+
 @pytest.mark.parametrize("node_level", [False, True])
 @pytest.mark.parametrize("lm,L,H,mb,steps,clip", [(True, 2, 32, 4, 1, 0.4), (False, 2, 48, 3, 1, 0.25),
                                                   (False, 1, 32, 5, 3, 5.0), (True, 3, 64, 8, 2, 1.0)])
-def test_train_steps_match_oracle(tmp_path, lm, L, H, mb, steps, clip, node_level):
+def test_train_steps_match_oracle(tmp_path, lm, L, H, mb, steps, clip, node_level, abandon=False):
     """node_level: the same steps through the layer objects' back_prop_GPU / update_weights members
     (forward_model::compute_gradients) instead of model_trainer."""
     if not os.path.exists(DRIVER):
@@ -162,11 +169,15 @@ def test_train_steps_match_oracle(tmp_path, lm, L, H, mb, steps, clip, node_leve
         for r in rows:
             for k in range(4):
                 f.write(" ".join(str(v) for v in r[k]) + "\n")
-    args = (["--sequence"] if lm else []) + (["--node-level"] if node_level else []) + [str(model), str(data_path), str(mb), str(longest), str(lr), str(clip),
+    args = (["--sequence"] if lm else []) + (["--node-level"] if node_level else []) + \
+        (["--abandon-sweeps"] if abandon else []) + [str(model), str(data_path), str(mb), str(longest), str(lr), str(clip),
                                              str(steps)]
     r = subprocess.run([DRIVER] + args, capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, r.stderr[-2000:]
     got_loss = [float(ln.split()[2]) for ln in r.stdout.splitlines() if ln.startswith("loss")]
+    if abandon:
+        n_abandoned = [int(ln.split()[1]) for ln in r.stdout.splitlines() if ln.startswith("abandoned")]
+        assert n_abandoned == [steps], "every step's forward sweep should have been abandoned and repeated"
     chunks = [data[i:i + mb] for i in range(0, len(data), mb)]
     clipped, want_loss = [], []
     for s in range(steps):

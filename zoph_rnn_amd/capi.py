@@ -20,6 +20,10 @@ ZR_OPT_LSTM_KERNEL = 5
 ZR_OPT_LSTM_KPARTS = 6
 ZR_OPT_LSTM_SWEEP = 7
 ZR_OPT_LSTM_SWEEP_SPIN = 8
+ZR_QUERY_LSTM_STACK_PATH = 1
+ZR_QUERY_LSTM_SWEEP_ABANDONED = 2
+ZR_LSTM_STACK_PATH_SWEEP = 1
+ZR_LSTM_STACK_PATH_DIAGONALS = 2
 ZR_SOFTMAX_PROB = 0
 ZR_SOFTMAX_LOGPROB = 1
 
@@ -36,7 +40,7 @@ SYMBOLS = [
     "zr_unstack_gates", "zr_lstm_stack_backward", "zr_lstm_weight_gradients", "zr_embed_gradient",
     "zr_softmax_backward", "zr_sgd_update", "zr_lstm_node_backward", "zr_lstm_node_gradients",
     "zr_softmax_backward_accumulate", "zr_gather_columns_multi", "zr_softmax_backward_loss",
-    "zr_softmax_forward_static",
+    "zr_softmax_forward_static", "zr_ctx_query",
 ]
 
 _lib = None
@@ -152,6 +156,11 @@ class Context:
         ms = C.c_float()
         _chk(load().zr_timer_stop(self.h, C.byref(ms)))
         return ms.value
+
+    def query(self, what):
+        v = C.c_int(0)
+        _chk(load().zr_ctx_query(self.h, C.c_int(what), C.byref(v)))
+        return v.value
 
     def set_option(self, opt, value):
         _chk(load().zr_ctx_set_option(self.h, C.c_int(opt), C.c_int(value)))

@@ -248,6 +248,7 @@ beam_merge_kernel(int beam, int K, int max_len, int hyp_cap, float penalty, int 
   __shared__ int s_fin_parent[MAXC];
   __shared__ float s_fin_score[MAXC];
   __shared__ int s_nfin;
+  __shared__ int s_base;  // finished hypotheses of the sentence before this step
   const int s = blockIdx.x;
   const int tid = threadIdx.x;
   float* sc = scores + (size_t)s * beam;
@@ -311,11 +312,14 @@ beam_merge_kernel(int beam, int K, int max_len, int hyp_cap, float penalty, int 
       }
     }
     s_nfin = nfin;
+    // read here, by the thread that updates it at the end, and handed on through shared memory: a wave that came late
+    // to a load of its own could otherwise see the updated count
+    s_base = hyp_count[s];
   }
   __syncthreads();
   // finished hypotheses: parent's words [0, current_index+1) then <EOF>
   const int nfin = s_nfin;
-  const int base = hyp_count[s];
+  const int base = s_base;
   for (int f = 0; f < nfin; ++f) {
     const int h = base + f;
     if (h >= hyp_cap) break;

@@ -991,10 +991,39 @@ int sweep_capacity(zr_ctx* ctx) {
   return cached > 0 ? cached : 0;
 }
 
+// Runs right behind lstm_sweep_kernel.  A sweep whose workgroups gave up a wait leaves part of h_all / c_all
+// unwritten; whatever is queued behind it on the stream would read stale memory.  When the status flag is up this
+// kernel overwrites every output of the sweep with NaN, so that nothing downstream can pass for a result; when it
+// is down (always, in practice) every workgroup reads one word and leaves.
+struct SweepPoison {
+  float* out[3 * kMaxUnits];  // h_all, c_all and (where kept) gates_all of every layer
+  long long count[3 * kMaxUnits];
+  int n_out;
+  const int* status;
+};
+
+__global__ void __launch_bounds__(256) lstm_sweep_poison_kernel(SweepPoison P) {
+  if (__hip_atomic_load(P.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0) return;
+  const float nan = __builtin_nanf("");
+  const long long stride = (long long)gridDim.x * 256;
+  for (int a = 0; a < P.n_out; ++a)
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < P.count[a]; i += stride) P.out[a][i] = nan;
+}
+
 template <int TN>
 int launch_sweep_v(zr_ctx* ctx, LstmSweep& P, int grid) {
   lstm_sweep_kernel<TN><<<grid, 256, 0, ctx->stream>>>(P);
   ZR_LAUNCH_CHECK("lstm_sweep_kernel");
+  SweepPoison Q = {};
+  const long long per = (long long)P.T * P.H * P.mb;
+  for (int l = 0; l < P.nl; ++l) {
+    Q.out[Q.n_out] = P.h_all[l], Q.count[Q.n_out++] = per;
+    Q.out[Q.n_out] = P.c_all[l], Q.count[Q.n_out++] = per;
+    if (P.gates_all[l]) Q.out[Q.n_out] = P.gates_all[l], Q.count[Q.n_out++] = 4 * per;
+  }
+  Q.status = P.status;
+  lstm_sweep_poison_kernel<<<512, 256, 0, ctx->stream>>>(Q);
+  ZR_LAUNCH_CHECK("lstm_sweep_poison_kernel");
   return ZR_OK;
 }
 
@@ -1194,7 +1223,9 @@ int zr_lstm_stack_forward_train(zr_ctx* ctx, int nl, const zr_lstm_weights* cons
     // Left to itself the library takes the single launch only when it fills most of the chip and this is the only
     // context on the device: two such launches from two streams could each hold part of the CUs and wait for the
     // rest (their bounded waits would end it, with an error).
-    const bool fills = tn && tiles * 10 >= 6LL * ctx->cu_count && zr_live_contexts(ctx->device) == 1;
+    // Nor on a caller-provided stream: the caller's other streams may hold compute units for as long as they like.
+    const bool fills = tn && tiles * 10 >= 6LL * ctx->cu_count && zr_live_contexts(ctx->device) == 1 &&
+                       ctx->stream == ctx->own_stream;
     // the kernel addresses its operands as descriptor base + 32-bit byte offsets
     const long long lim = 1LL << 32;
     const bool offsets_fit = (long long)V * H * 4 < lim && (long long)n * 4 < lim &&
@@ -1237,12 +1268,14 @@ int zr_lstm_stack_forward_train(zr_ctx* ctx, int nl, const zr_lstm_weights* cons
       // Without the invalidation a consumer relies on never having cached a line before its producer wrote it: true
       // when no 128-byte line of the k-interleaved copies is shared between two producers, i.e. mb % 8 == 0.
       P.fence = (mb % 8 == 0) ? 0 : 1;
+      ctx->last_stack_path = ZR_LSTM_STACK_PATH_SWEEP;
       return tn == 1 ? launch_sweep_v<1>(ctx, P, padded * n_tiles) : launch_sweep_v<2>(ctx, P, padded * n_tiles);
     }
   }
   // Every h is also written in a k-interleaved layout ([H/4][mb][4]) into a small ping-pong buffer per layer: its
   // two consumers on the next diagonal, (l+1, t) and (l, t+1), then fetch activations with contiguous 16-byte
   // loads.  The buffer written on diagonal d is read on d+1 only and overwritten on d+2.
+  ctx->last_stack_path = ZR_LSTM_STACK_PATH_DIAGONALS;
   float* hp_buf = nullptr;
   if (vec && H % 8 == 0 && !layers[0]->bf16) {
     void* p = nullptr;

@@ -169,6 +169,28 @@ int zr_ctx_sync(zr_ctx* ctx) {
   return ZR_OK;
 }
 
+int zr_ctx_query(zr_ctx* ctx, int what, int* h_value) {
+  ZR_CHECK_ARG(ctx != nullptr, "null context");
+  ZR_CHECK_ARG(h_value != nullptr, "zr_ctx_query: h_value is null");
+  switch (what) {
+    case ZR_QUERY_LSTM_STACK_PATH:
+      *h_value = ctx->last_stack_path;
+      return ZR_OK;
+    case ZR_QUERY_LSTM_SWEEP_ABANDONED: {
+      int rc = zr_bind_device(ctx);
+      if (rc) return rc;
+      ZR_HIP(hipStreamSynchronize(ctx->stream));
+      int flag = 0;
+      ZR_HIP(hipMemcpy(&flag, ctx->d_flags + 2, sizeof(int), hipMemcpyDeviceToHost));
+      if (flag != 0) ZR_HIP(hipMemset(ctx->d_flags + 2, 0, sizeof(int)));
+      *h_value = flag != 0 ? 1 : 0;
+      return ZR_OK;
+    }
+    default:
+      return zr_set_error(ZR_EINVAL, "zr_ctx_query: unknown item %d", what);
+  }
+}
+
 int zr_ctx_set_stream(zr_ctx* ctx, void* hip_stream) {
   ZR_CHECK_ARG(ctx != nullptr, "null context");
   ctx->stream = hip_stream ? (hipStream_t)hip_stream : ctx->own_stream;

@@ -53,6 +53,16 @@ typedef float precision;  // src/global_params.h:3
 namespace BZ_CUDA {
 inline bool clip_cell = false;
 inline precision cell_clip_threshold = 50;
+// With clip_cell set the reference also clamps the back-propagated errors to +-error_clip_threshold
+// (src/LSTM.hpp:792,888; src/LSTM_HH.hpp:665,756,774).  The backward kernels here have no such clamp, so the backward
+// members refuse to run with clip_cell set rather than return gradients that differ from the reference's.
+inline void refuse_backward_with_clip_cell(const char* who) {
+  if (clip_cell) {
+    std::fprintf(stderr, "Error: %s: the backward pass does not clamp errors (BZ_CUDA::error_clip_threshold) and "
+                 "cannot run with BZ_CUDA::clip_cell set\n", who);
+    std::exit(EXIT_FAILURE);
+  }
+}
 inline precision lower = -0.08f;
 inline precision upper = 0.08f;
 inline bool force_decode = false;
@@ -1113,6 +1123,7 @@ void lower_transfer_layer<dType>::send_error(int index, dType* d_err) {
 // the driver passes to the next backprop_prep_GPU call, and the error for the layer below is handed down by pointer.
 template <typename dType>
 void LSTM_HH_Node<dType>::back_prop_GPU(int index) {
+  BZ_CUDA::refuse_backward_with_clip_cell("LSTM_HH_Node::back_prop_GPU");
   zr_ctx* ctx = model->hh_layer_info.ctx;
   if (!model->train_weights) model->clear_gradients(true);
   const dType* gates[4] = {d_i_t, d_f_t, d_c_prime_t_tanh, d_o_t};
@@ -1133,6 +1144,7 @@ void LSTM_HH_Node<dType>::compute_gradients_GPU() {
 
 template <typename dType>
 void LSTM_IH_Node<dType>::back_prop_GPU(int /*index*/) {
+  BZ_CUDA::refuse_backward_with_clip_cell("LSTM_IH_Node::back_prop_GPU");
   zr_ctx* ctx = model->ih_layer_info.ctx;
   if (feed_input) {
     std::fprintf(stderr, "Error: back-propagation through the feed-input connection is not built\n");

@@ -708,6 +708,7 @@ class model_trainer {
   }
 
   explicit model_trainer(forward_model<dType>& model) : m(model), ctx(model.gpu.ctx) {
+    BZ_CUDA::refuse_backward_with_clip_cell("model_trainer");
     if (m.params.attent_params.attention_model) {
       std::fprintf(stderr, "model_trainer: the backward pass of the attention layer is not built\n");
       std::exit(EXIT_FAILURE);
@@ -785,6 +786,9 @@ class model_trainer {
     ZOPH_CALL(zr_embed_gradient(ctx, H, V, s.below0, s.d_nn, s.d_mask, T * mb, s.dW));
   }
 
+  int lstm_sweep_option = 0;  // the context's ZR_OPT_LSTM_SWEEP setting, restored after a repeated forward pass
+  int abandoned_sweeps = 0;   // forward passes that had to be repeated (see train_minibatch)
+
   // Forward, backward and update on the minibatch the reader holds.  Returns the minibatch's log-likelihood (natural
   // log) under the weights BEFORE the update.
   double train_minibatch(minibatch_reader& r, float learning_rate, float norm_clip) {
@@ -792,21 +796,35 @@ class model_trainer {
     const size_t n = (size_t)H * mb;
     std::vector<const dType*> z(L, zeros);
     std::vector<const dType*> th0 = z, tc0 = z;
-    if (seq2seq) {
-      forward_side(src, m.input_layer_source, m.source_hidden_layers, r.h_input_vocab_indicies_source.data(), S, Vs, z, z);
-      for (int l = 0; l < L; l++) {  // the decoder starts from the encoder's last state (src/model.hpp:1714-1724)
-        th0[l] = src.h_all[l] + (size_t)(S - 1) * n;
-        tc0[l] = src.c_all[l] + (size_t)(S - 1) * n;
-      }
-    }
-    forward_side(tgt, m.input_layer_target, m.target_hidden_layers, r.h_input_vocab_indicies_target.data(), T, Vt, th0, tc0);
-    // loss layer over all T * mb columns at once
-    ZOPH_CALL(zr_h2d(ctx, d_tout, r.h_output_vocab_indicies_target.data(), (size_t)T * mb * sizeof(int)));
-    ZOPH_CALL(zr_vocab_prep_softmax(ctx, d_tout, T * mb, Vt, d_tmask, d_tmaskf));
     auto& sm = m.softmax_obj;
     double loss = 0;  // from the same probabilities the error is formed from (train_perplexity_kernel)
-    ZOPH_CALL(zr_softmax_backward_loss(ctx, sm.d_D, sm.d_b_d, Vt, H, tgt.h_all[L - 1], T * mb, d_tout, d_tmask, prob,
-                                       err_top, dD, dbd, &loss));
+    auto forward_and_loss = [&]() {
+      if (seq2seq) {
+        forward_side(src, m.input_layer_source, m.source_hidden_layers, r.h_input_vocab_indicies_source.data(), S, Vs, z, z);
+        for (int l = 0; l < L; l++) {  // the decoder starts from the encoder's last state (src/model.hpp:1714-1724)
+          th0[l] = src.h_all[l] + (size_t)(S - 1) * n;
+          tc0[l] = src.c_all[l] + (size_t)(S - 1) * n;
+        }
+      }
+      forward_side(tgt, m.input_layer_target, m.target_hidden_layers, r.h_input_vocab_indicies_target.data(), T, Vt, th0, tc0);
+      // loss layer over all T * mb columns at once
+      ZOPH_CALL(zr_h2d(ctx, d_tout, r.h_output_vocab_indicies_target.data(), (size_t)T * mb * sizeof(int)));
+      ZOPH_CALL(zr_vocab_prep_softmax(ctx, d_tout, T * mb, Vt, d_tmask, d_tmaskf));
+      ZOPH_CALL(zr_softmax_backward_loss(ctx, sm.d_D, sm.d_b_d, Vt, H, tgt.h_all[L - 1], T * mb, d_tout, d_tmask, prob,
+                                         err_top, dD, dbd, &loss));
+    };
+    forward_and_loss();
+    // A single-launch forward sweep that gave up a wait (another process or stream holding compute units) leaves NaN
+    // in its outputs; nothing of it may reach the weights.  The loss call above has already waited for the stream, so
+    // the look costs one small copy.  Run the forward pass again with one launch per diagonal, which cannot stall.
+    int gave_up = 0;
+    ZOPH_CALL(zr_ctx_query(ctx, ZR_QUERY_LSTM_SWEEP_ABANDONED, &gave_up));
+    if (gave_up) {
+      ++abandoned_sweeps;
+      ZOPH_CALL(zr_ctx_set_option(ctx, ZR_OPT_LSTM_SWEEP, 1));
+      forward_and_loss();
+      ZOPH_CALL(zr_ctx_set_option(ctx, ZR_OPT_LSTM_SWEEP, lstm_sweep_option));
+    }
     backward_side(tgt, m.input_layer_target, m.target_hidden_layers, T, Vt, th0, tc0, err_top, nullptr, nullptr);
     if (seq2seq) {
       // no attention: the encoder receives error only through its final states
