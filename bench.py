@@ -121,6 +121,8 @@ def bench_decoder_step(ctx, steps, warmup, H=1000, mb=128, S=50, V=50000, L=4, D
     ctx.softmax_prepare(dD, V, H, bf16=bf16)  # one-time snapshot of D in the matrix cores' layout, not timed
     if bf16:
         ctx.attn_use_bf16_weights(attn)
+    else:
+        ctx.attn_prepare(attn)  # one-time snapshot of the four attention matrices, like the output layer's: not timed
     d_x = ctx.empty((H, mb))
     d_h = [ctx.empty((H, mb)) for _ in range(L)]
     d_c = [ctx.empty((H, mb)) for _ in range(L)]

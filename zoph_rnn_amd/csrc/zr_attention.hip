@@ -18,6 +18,11 @@ struct zr_attn {
   // zr_attn_use_bf16_weights: owned bf16 k-interleaved snapshots of W_p, W_a^T, W_c1, W_c2 ([H/8][ldp][8] each)
   unsigned short* d_bf16;
   int ldp;
+  // zr_attn_prepare: owned fp32 k-interleaved snapshots ([kp/4][ldp32][4] each) of W_p, W_a^T, W_c1, W_c2 in that
+  // order, and the raw (pre-tanh) W_p h product next to q
+  float* d_pack32;
+  int ldp32, kp32;
+  float *d_hpack, *d_cpack;  // k-interleaved copies ([H/4][mb][4]) of h_t and of the context (inside d_pack32's block)
 };
 
 namespace {
@@ -182,6 +187,241 @@ attn_context_kernel(const float* const* __restrict__ table, int longest_sent, co
     o[0] = acc[0];
 }
 
+__device__ __forceinline__ float block_sum_256(float v, float* s_red, int tid) {
+  v = wave_sum(v);
+  __syncthreads();  // the previous use of s_red is over
+  if ((tid & 63) == 0) s_red[tid >> 6] = v;
+  __syncthreads();
+  return s_red[0] + s_red[1] + s_red[2] + s_red[3];
+}
+
+// Everything of the attention step between the two projections and the output product, for one batch column per
+// workgroup: p_t and the window (attn_window_kernel; `pre` holds W_p h BEFORE the tanh), the scores h_s . q of the
+// valid window slots (attn_score_kernel), the reference's max-starts-at-0 softmax times the Gaussian
+// (attn_align_kernel) and the context vector (attn_context_kernel).  The valid source columns come from memory once,
+// for the scores; the context pass a few microseconds later finds them in the L2 the workgroup's CU sits behind.
+// Requires H % 4 == 0 and 16-byte aligned source tables, pre, q and ctx_out; W <= 512.
+__global__ void __launch_bounds__(256)
+attn_fused_kernel(const float* const* __restrict__ table, int longest_sent, const float* __restrict__ pre,
+                  const float* __restrict__ q, const float* __restrict__ v_p, const int* __restrict__ batch_info,
+                  const int* __restrict__ mask01, int H, int mb, int D, float sigma_sq, float* __restrict__ p_t,
+                  int* __restrict__ indices, float* __restrict__ align, float* __restrict__ ctx_out,
+                  float* __restrict__ ctx_pack, int* __restrict__ flags) {
+  constexpr int kMaxSlots = 512;
+  __shared__ float s_red[4];
+  __shared__ float s_val[kMaxSlots];         // scores, then alignment weights, of the valid slots
+  __shared__ const float* s_src[kMaxSlots];  // source column of each valid slot
+  const int b = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int W = 2 * D + 1;
+  const int H4 = H >> 2;
+  // p_t = S * sigmoid(v_p . tanh(W_p h)), sigmoid in double as the reference's sigmoid_kernel
+  float part = 0.0f;
+  for (int k4 = tid; k4 < H4; k4 += 256) {
+    const zr_f32x4 t = ((const zr_f32x4*)(pre + (size_t)b * H))[k4];
+    const zr_f32x4 v = ((const zr_f32x4*)v_p)[k4];
+    part += v.x * tanhf(t.x) + v.y * tanhf(t.y) + v.z * tanhf(t.z) + v.w * tanhf(t.w);
+  }
+  const float sdot = block_sum_256(part, s_red, tid);
+  const float sig = (float)(1.0 / (1.0 + exp(-1.0 * (double)sdot)));
+  const int len = batch_info[b], off = batch_info[mb + b];
+  const float p = (float)len * sig;
+  const int ip = (int)p;
+  const int lo = (0 > ip - D) ? 0 : (ip - D);
+  const int hi = ((len - 1) < ip + D) ? (len - 1) : (ip + D);
+  const bool live = mask01[b] == 1;
+  int nvalid = live ? hi - lo + 1 : 0;
+  nvalid = nvalid < 0 ? 0 : (nvalid > W ? W : nvalid);
+  if (tid == 0) p_t[b] = p;
+  for (int j = tid; j < W; j += 256) {
+    indices[b + (size_t)mb * j] = j < nvalid ? lo + j : -1;
+    if (j < nvalid) {
+      int t = len - 1 - (lo + j) + off;
+      if (t < 0 || t >= longest_sent) {
+        atomicAdd(&flags[1], 1);
+        t = t < 0 ? 0 : longest_sent - 1;
+      }
+      s_src[j] = table[t] + (size_t)b * H;
+    }
+  }
+  __syncthreads();
+  // scores: the slots go round the four waves, two at a time per wave so that their loads overlap
+  {
+    const zr_f32x4* qc = (const zr_f32x4*)(q + (size_t)b * H);
+    for (int j = wave * 2; j < nvalid; j += 8) {
+      const bool two = j + 1 < nvalid;
+      const zr_f32x4* h0 = (const zr_f32x4*)s_src[j];
+      const zr_f32x4* h1 = (const zr_f32x4*)s_src[two ? j + 1 : j];
+      float a0 = 0.0f, a1 = 0.0f;
+      for (int k4 = lane; k4 < H4; k4 += 64) {
+        const zr_f32x4 c = qc[k4];
+        const zr_f32x4 x0 = h0[k4];
+        const zr_f32x4 x1 = h1[k4];
+        a0 += x0.x * c.x + x0.y * c.y + x0.z * c.z + x0.w * c.w;
+        a1 += x1.x * c.x + x1.y * c.y + x1.z * c.z + x1.w * c.w;
+      }
+      a0 = wave_sum(a0);
+      a1 = wave_sum(a1);
+      if (lane == 0) {
+        s_val[j] = a0;
+        if (two) s_val[j + 1] = a1;
+      }
+    }
+  }
+  __syncthreads();
+  // alignment weights (alignment_reduction_kernel, src/custom_kernels.h:1752-1794): the maximum starts at 0
+  if (wave == 0) {
+    float max_val = 0.0f;
+    for (int j = lane; j < nvalid; j += 64) max_val = fmaxf(max_val, s_val[j]);
+    max_val = wave_max(max_val);
+    float sum = 0.0f;
+    for (int j = lane; j < nvalid; j += 64) sum += expf(s_val[j] - max_val);
+    sum = wave_sum(sum);
+    for (int j = lane; j < W; j += 64) {
+      float a = 0.0f;
+      if (j < nvalid) {
+        a = expf(s_val[j] - max_val);
+        const float d = p - (float)(lo + j);
+        const float g = expf((-1.0f * d * d) / (2.0f * sigma_sq));
+        if (sum != 0.0f) a = (a / sum) * g;
+        s_val[j] = a;
+      }
+      align[b + (size_t)mb * j] = a;
+    }
+  }
+  __syncthreads();
+  // context: c[:, b] = sum_j a_j h_s(slot j), four rows per thread, four slots in flight
+  for (int k4 = tid; k4 < H4; k4 += 256) {
+    zr_f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    int j = 0;
+    for (; j + 4 <= nvalid; j += 4) {
+      const zr_f32x4 x0 = ((const zr_f32x4*)s_src[j])[k4];
+      const zr_f32x4 x1 = ((const zr_f32x4*)s_src[j + 1])[k4];
+      const zr_f32x4 x2 = ((const zr_f32x4*)s_src[j + 2])[k4];
+      const zr_f32x4 x3 = ((const zr_f32x4*)s_src[j + 3])[k4];
+      acc += s_val[j] * x0;
+      acc += s_val[j + 1] * x1;
+      acc += s_val[j + 2] * x2;
+      acc += s_val[j + 3] * x3;
+    }
+    for (; j < nvalid; ++j) acc += s_val[j] * ((const zr_f32x4*)s_src[j])[k4];
+    ((zr_f32x4*)(ctx_out + (size_t)b * H))[k4] = acc;
+    if (ctx_pack) ((zr_f32x4*)ctx_pack)[(size_t)k4 * mb + b] = acc;
+  }
+}
+
+// Sum over the 64 lanes of each of N values held one per register: lanes end up with the totals in all lanes.
+template <int N>
+__device__ __forceinline__ void wave_sum_many(float (&v)[N]) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1)
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] += __shfl_xor(v[i], off, 64);
+}
+
+// attn_fused_kernel for H <= 1024 and at most MAXS window slots: every thread owns four consecutive rows and keeps
+// them, for every valid slot, in registers -- all loads of a column's source states are in flight together, the
+// scores are formed from the registers, and so is the context, so the source states are read exactly once and nothing
+// is read twice.  Also writes the context k-interleaved ([H/4][mb][4]) for the output product when ctx_pack is given.
+template <int MAXS>
+__global__ void __launch_bounds__(256)
+attn_fused_reg_kernel(const float* const* __restrict__ table, int longest_sent, const float* __restrict__ pre,
+                      const float* __restrict__ q, const float* __restrict__ v_p, const int* __restrict__ batch_info,
+                      const int* __restrict__ mask01, int H, int mb, int D, float sigma_sq, float* __restrict__ p_t,
+                      int* __restrict__ indices, float* __restrict__ align, float* __restrict__ ctx_out,
+                      float* __restrict__ ctx_pack, int* __restrict__ flags) {
+  __shared__ float s_red[4];
+  __shared__ float s_part[4][MAXS];
+  __shared__ float s_val[MAXS];
+  __shared__ const float* s_src[MAXS];
+  const int b = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int W = 2 * D + 1;
+  const int H4 = H >> 2;
+  const bool mine = tid < H4;
+  const int k4 = mine ? tid : 0;
+  float part = 0.0f;
+  if (mine) {
+    const zr_f32x4 t = ((const zr_f32x4*)(pre + (size_t)b * H))[k4];
+    const zr_f32x4 v = ((const zr_f32x4*)v_p)[k4];
+    part = v.x * tanhf(t.x) + v.y * tanhf(t.y) + v.z * tanhf(t.z) + v.w * tanhf(t.w);
+  }
+  const zr_f32x4 qv = ((const zr_f32x4*)(q + (size_t)b * H))[k4];
+  const float sdot = block_sum_256(part, s_red, tid);
+  const float sig = (float)(1.0 / (1.0 + exp(-1.0 * (double)sdot)));
+  const int len = batch_info[b], off = batch_info[mb + b];
+  const float p = (float)len * sig;
+  const int ip = (int)p;
+  const int lo = (0 > ip - D) ? 0 : (ip - D);
+  const int hi = ((len - 1) < ip + D) ? (len - 1) : (ip + D);
+  const bool live = mask01[b] == 1;
+  int nvalid = live ? hi - lo + 1 : 0;
+  nvalid = nvalid < 0 ? 0 : (nvalid > W ? W : nvalid);
+  nvalid = nvalid > MAXS ? MAXS : nvalid;  // the host picks MAXS >= min(W, longest_sent)
+  if (tid == 0) p_t[b] = p;
+  for (int j = tid; j < W; j += 256) indices[b + (size_t)mb * j] = j < nvalid ? lo + j : -1;
+  if (tid < nvalid) {
+    int t = len - 1 - (lo + tid) + off;
+    if (t < 0 || t >= longest_sent) {
+      atomicAdd(&flags[1], 1);
+      t = t < 0 ? 0 : longest_sent - 1;
+    }
+    s_src[tid] = table[t] + (size_t)b * H;
+  }
+  __syncthreads();
+  zr_f32x4 x[MAXS];
+#pragma unroll
+  for (int j = 0; j < MAXS; ++j) {
+    x[j] = zr_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    if (j < nvalid && mine) x[j] = ((const zr_f32x4*)s_src[j])[k4];
+  }
+  // partial scores of this thread's four rows, summed over the wave in batches of 16 slots, then over the four waves
+#pragma unroll
+  for (int j0 = 0; j0 < MAXS; j0 += 16) {
+    if (j0 < nvalid) {  // uniform over the workgroup
+      float d[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) d[i] = x[j0 + i].x * qv.x + x[j0 + i].y * qv.y + x[j0 + i].z * qv.z + x[j0 + i].w * qv.w;
+      wave_sum_many<16>(d);
+      float dl = d[0];  // lane i keeps slot j0 + i
+#pragma unroll
+      for (int i = 1; i < 16; ++i) dl = lane == i ? d[i] : dl;
+      if (lane < 16) s_part[wave][j0 + lane] = dl;
+    }
+  }
+  __syncthreads();
+  if (wave == 0) {
+    // alignment_reduction_kernel (src/custom_kernels.h:1752-1794): the maximum starts at 0
+    float sc = 0.0f;
+    const bool v = lane < nvalid;
+    if (MAXS <= 64) {
+      if (v) sc = (s_part[0][lane] + s_part[1][lane]) + (s_part[2][lane] + s_part[3][lane]);
+      const float max_val = wave_max(v ? fmaxf(sc, 0.0f) : 0.0f);
+      const float e = v ? expf(sc - max_val) : 0.0f;
+      const float sum = wave_sum(e);
+      float a = 0.0f;
+      if (v) {
+        const float dd = p - (float)(lo + lane);
+        const float g = expf((-1.0f * dd * dd) / (2.0f * sigma_sq));
+        a = sum != 0.0f ? (e / sum) * g : e;
+        s_val[lane] = a;
+      }
+      for (int j = lane; j < W; j += 64) align[b + (size_t)mb * j] = j == lane ? a : 0.0f;
+    }
+  }
+  __syncthreads();
+  if (mine) {
+    zr_f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int j = 0; j < MAXS; ++j)
+      if (j < nvalid) acc += s_val[j] * x[j];
+    ((zr_f32x4*)(ctx_out + (size_t)b * H))[k4] = acc;
+    if (ctx_pack) ((zr_f32x4*)ctx_pack)[(size_t)k4 * mb + b] = acc;
+  }
+}
+
 }  // namespace
 
 extern "C" {
@@ -217,6 +457,8 @@ int zr_attn_create(zr_ctx* ctx, int H, int mb, int D, const float* d_W_a, const 
   a->W_c2 = d_W_c2;
   a->d_bf16 = nullptr;
   a->ldp = 0;
+  a->d_pack32 = nullptr;
+  a->ldp32 = a->kp32 = 0;
   const size_t n = (size_t)H * mb, W = 2 * (size_t)D + 1;
   // one allocation: table | tanh1 | q | ctx | align | p_t | idx
   const size_t tbytes = (sizeof(float*) * longest_sent + 255) & ~(size_t)255;
@@ -270,12 +512,42 @@ int zr_attn_use_bf16_weights(zr_ctx* ctx, zr_attn* a) {
   return ZR_OK;
 }
 
+int zr_attn_prepare(zr_ctx* ctx, zr_attn* a) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(a != nullptr, "zr_attn_prepare: attention object is null");
+  const int H = a->H;
+  const int ldp = (H + 31) / 32 * 32, kp = (H + 7) / 8 * 8;
+  const size_t per = (size_t)kp * ldp;
+  if (!a->d_pack32) {
+    if (hipMalloc((void**)&a->d_pack32, sizeof(float) * (4 * per + 2 * (size_t)H * a->mb)) != hipSuccess) {
+      (void)hipGetLastError();
+      a->d_pack32 = nullptr;
+      return zr_set_error(ZR_ENOMEM, "zr_attn_prepare: allocation failed");
+    }
+  }
+  a->ldp32 = ldp;
+  a->kp32 = kp;
+  // the context's copy first, h_t's right behind it: together they are the k-interleaved [c; h_t] (2H x mb) that the
+  // output product multiplies with [W_c1 | W_c2], whose snapshots are neighbours as well
+  a->d_cpack = a->d_pack32 + 4 * per;
+  a->d_hpack = a->d_cpack + (size_t)H * a->mb;
+  rc = zr_pack4_launch(ctx, a->W_p, H, H, H, ldp, kp, a->d_pack32);
+  if (rc) return rc;
+  rc = zr_pack4_trans_launch(ctx, a->W_a, H, H, H, ldp, kp, a->d_pack32 + per);  // W_a^T
+  if (rc) return rc;
+  rc = zr_pack4_launch(ctx, a->W_c1, H, H, H, ldp, kp, a->d_pack32 + 2 * per);
+  if (rc) return rc;
+  return zr_pack4_launch(ctx, a->W_c2, H, H, H, ldp, kp, a->d_pack32 + 3 * per);
+}
+
 int zr_attn_destroy(zr_ctx* ctx, zr_attn* a) {
   if (!a) return ZR_OK;
   int rc = zr_bind_device(ctx);
   if (rc) return rc;
   ZR_HIP(hipStreamSynchronize(ctx->stream));
   if (a->d_bf16) (void)hipFree(a->d_bf16);
+  if (a->d_pack32) (void)hipFree(a->d_pack32);
   (void)hipFree((void*)a->d_table);
   delete a;
   return ZR_OK;
@@ -292,6 +564,91 @@ int zr_attn_step(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, const float* 
   int* idx = d_indices ? d_indices : a->d_idx;
   float* pt = d_p_t ? d_p_t : a->d_pt;
   float* cctx = d_c_ctx ? d_c_ctx : a->d_ctx;
+
+  const bool fast = a->d_pack32 && !a->d_bf16 && (H % 4 == 0) && a->tables_aligned && (((uintptr_t)cctx & 15u) == 0) &&
+                    (((uintptr_t)d_h_t & 15u) == 0);
+  if (fast) {
+    // Three launches.  (1) W_p h (before the tanh) and q = W_a^T h as one batch of two products on the k-interleaved
+    // snapshots; d_tanh1 and d_q are neighbours in the object's allocation (stride H*mb).
+    const size_t per = (size_t)a->kp32 * a->ldp32;
+    ZrGemmDesc g = {};
+    g.M = H;
+    g.N = mb;
+    g.nseg = 1;
+    g.K[0] = H;
+    g.A[0] = a->d_pack32;
+    g.lda[0] = a->ldp32;
+    g.a_pack = 1;
+    // with H % 8 == 0 the products read k-interleaved activations (contiguous 16-byte loads instead of 16 bytes from
+    // each of 32 lines per half-wave): h_t is re-laid-out once for both products, the context is written that way
+    const bool bp = H % 8 == 0;
+    if (bp) {
+      rc = zr_pack4_x_launch(ctx, d_h_t, H, mb, H, a->d_hpack);
+      if (rc) return rc;
+    }
+    g.B[0] = bp ? a->d_hpack : d_h_t;
+    g.b_packed = bp ? 1 : 0;
+    g.ldb[0] = H;
+    g.C = a->d_tanh1;
+    g.ldc = H;
+    g.batch = 2;
+    g.strideA = (long long)per;
+    g.strideC = (long long)H * mb;
+    g.epilogue = ZR_EPI_STORE;
+    rc = zr_gemm_launch(ctx, g);
+    if (rc) return rc;
+    // (2) p_t, window, scores, alignment weights and context, one workgroup per column
+    const float sigma_sq = (float)((D * D) / 4.0);  // attention_node.hpp:50
+    float* cpack = bp ? a->d_cpack : nullptr;
+    const int max_slots = W < a->longest_sent ? W : a->longest_sent;
+    if (H <= 1024 && max_slots <= 16)
+      attn_fused_reg_kernel<16><<<mb, 256, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_tanh1, a->d_q, a->v_p,
+                                                             d_batch_info, d_mask01, H, mb, D, sigma_sq, pt, idx, align,
+                                                             cctx, cpack, ctx->d_flags);
+    else if (H <= 1024 && max_slots <= 32)
+      attn_fused_reg_kernel<32><<<mb, 256, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_tanh1, a->d_q, a->v_p,
+                                                             d_batch_info, d_mask01, H, mb, D, sigma_sq, pt, idx, align,
+                                                             cctx, cpack, ctx->d_flags);
+    else if (H <= 1024 && max_slots <= 64)
+      attn_fused_reg_kernel<64><<<mb, 256, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_tanh1, a->d_q, a->v_p,
+                                                             d_batch_info, d_mask01, H, mb, D, sigma_sq, pt, idx, align,
+                                                             cctx, cpack, ctx->d_flags);
+    else
+      attn_fused_kernel<<<mb, 256, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_tanh1, a->d_q, a->v_p,
+                                                     d_batch_info, d_mask01, H, mb, D, sigma_sq, pt, idx, align, cctx,
+                                                     cpack, ctx->d_flags);
+    ZR_LAUNCH_CHECK("attn_fused_kernel");
+    // (3) h~ = tanh(W_c1 c + W_c2 h + b) * mask
+    ZrGemmDesc o = {};
+    o.M = H;
+    o.N = mb;
+    o.a_pack = 1;
+    o.A[0] = a->d_pack32 + 2 * per;
+    o.lda[0] = o.lda[1] = a->ldp32;
+    if (bp) {
+      // one K loop of 2H over [W_c1 | W_c2] and [c; h_t] (H % 8 == 0: no padding between the halves of either operand),
+      // so the second half's operands are already on their way while the first half is multiplied
+      o.nseg = 1;
+      o.K[0] = 2 * H;
+      o.B[0] = a->d_cpack;
+      o.b_packed = 1;
+      o.ldb[0] = 2 * H;
+    } else {
+      o.nseg = 2;
+      o.K[0] = o.K[1] = H;
+      o.A[1] = a->d_pack32 + 3 * per;
+      o.B[0] = cctx;
+      o.B[1] = d_h_t;
+      o.ldb[0] = o.ldb[1] = H;
+    }
+    o.C = d_htild;
+    o.ldc = H;
+    o.batch = 1;
+    o.bias = a->out_bias;
+    o.mask = d_mask01;
+    o.epilogue = ZR_EPI_TANH_BIAS_MASK;
+    return zr_gemm_launch(ctx, o);
+  }
 
   // tanh(W_p h)  (reference: attention_node.hpp:132-141)
   ZrGemmDesc g = {};

@@ -45,7 +45,9 @@ constexpr int stats_chunk(int nv, int tm) {
 // One output tile of 32*TM rows x 32*TN columns at (m0, n0), computed by the KS waves that call this together
 // (kslice = this wave's K slice, redp = their KS*TN*16*64 floats of LDS): all segments, the split-K sum and the
 // epilogue.  `active` false: same control flow (barriers), nothing stored.  PF = prefetch distance in k-groups.
-template <int TM, int TN, int KS, int AMODE, bool VEC, int EPI, int PF>
+// BUF (k-interleaved fp32 operands on both sides, K % 8 == 0, every row and column of the tile in range, operands below
+// 4 GiB): the K loop fetches through buffer descriptors with the pinned schedule of zr_mma_segment_u.
+template <int TM, int TN, int KS, int AMODE, bool VEC, int EPI, int PF, bool BUF = false>
 __device__ __forceinline__ void gemm_tile(const GemmArgs& a, int m0, int n0, bool active, int z, float* redp,
                                           int kslice, int lane) {
   const int jl = lane & 31;
@@ -83,8 +85,25 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& a, int m0, int n0, boo
     grpC = a.gC[grp];
   }
 
+  // epilogue operands go out ahead of the K loop
+  const float* bias = a.bias ? a.bias + (long long)z * a.strideBias : nullptr;
+  float bias_v[TM];
+  if (EPI == ZR_EPI_SOFTMAX_PARTIAL) {
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) bias_v[tm] = bias[rows[tm]];
+  }
+
   for (int s = 0; s < a.nseg; ++s) {
-    if constexpr (AMODE == ZR_A_PACK8_BF16) {
+    if constexpr (BUF) {
+      unsigned wsoff[TM], xoffb[TN];
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) wsoff[tm] = 512u * (unsigned)tm;  // 32 rows of 16 bytes
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) xoffb[tn] = 16u * (unsigned)(n0 + tn * 32 + jl + half * a.N);
+      const unsigned woffb = 16u * (unsigned)(m0 + jl + half * (int)a.lda[s]);
+      zr_mma_segment_u<TM, TN, KS, PF>(acc, zr_make_rsrc(a.A[s]), wsoff, woffb, 32u * (unsigned)a.lda[s],
+                                       zr_make_rsrc(a.B[s]), xoffb, 32u * (unsigned)a.N, a.K[s], kslice);
+    } else if constexpr (AMODE == ZR_A_PACK8_BF16) {
       const unsigned short* wbase[TM];
       unsigned woff[TM];
       const float* xcol[TN];
@@ -124,22 +143,17 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& a, int m0, int n0, boo
   }
 
   float* C = (grpC ? grpC : a.C) + (long long)z * a.strideC;
-  const float* bias = a.bias ? a.bias + (long long)z * a.strideBias : nullptr;
 
   if (EPI == ZR_EPI_SOFTMAX_PARTIAL) {
     // logits = acc + bias, plus (max, sum exp) of every 32-row block and column.  The values of all visits are
     // collected first so that their cross-lane reductions run interleaved, then everything is stored.
-    float bias_v[TM];
-#pragma unroll
-    for (int tm = 0; tm < TM; ++tm) bias_v[tm] = bias[rows[tm]];
     auto store = [&](int n, int tm, bool okv, float val, float mxv, float sev) {
       const int m = m0 + tm * 32 + jl;
       if (okv) C[(long long)n * a.ldc + m] = val;
       const int prow = (m0 >> 5) + tm;  // 32-row block index
       if (jl == 0 && active && n < a.N && prow * 32 < a.M) {
-        float* p = a.partials + ((long long)prow * a.N + n) * 2;
-        p[0] = mxv;
-        p[1] = sev;
+        typedef float zr_f32x2 __attribute__((ext_vector_type(2)));
+        *(zr_f32x2*)(a.partials + ((long long)n * ((a.M + 31) >> 5) + prow) * 2) = zr_f32x2{mxv, sev};
       }
     };
     if (KS == 1) {
@@ -318,6 +332,35 @@ __global__ void __launch_bounds__(256) gemm_rows_kernel(GemmArgs a, int row_chun
     if (n0 + sub * 32 < a.N)
       gemm_tile<1, 1, 4, AMODE, true, EPI, PF4 + 2>(a, blk * 32, n0 + sub * 32, true, 0, red, kslice, lane);
     __syncthreads();
+  }
+}
+
+// Tall weight matrix (k-interleaved) times a minibatch that is a multiple of 128 columns wide, balanced over the
+// CUs without a persistent loop.  One 64-row x 128-column tile per workgroup runs at the best rate this core reaches
+// (all 512 registers of a wave: 128 accumulators and a six-deep operand ring), but the number of such tiles is rarely a
+// multiple of the number of CUs, and a last, mostly empty round costs as much as a full one.  So only as many
+// 64-row tiles as fill whole rounds are taken that way (workgroups [0, n_big)); the rows left over go to the
+// workgroups behind them as 32 x 32 tiles, which the hardware hands out as the CUs run dry, and whose round lasts an
+// eighth of a big one.  Workgroup ids congruent modulo 8 share an XCD: each XCD takes a contiguous range of big row
+// tiles and the column tiles of one row tile run side by side on it.
+template <int EPI>
+__global__ void __launch_bounds__(256) gemm_tall_kernel(GemmArgs a, int big_rows, int n_col_tiles, int n_big) {
+  __shared__ float red[4 * 4 * 16 * 64];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int kslice = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int bid = blockIdx.x;
+  if (bid < n_big) {
+    const int r8 = bid & 7, q = bid >> 3;
+    const int mpx = big_rows >> 3;  // big_rows is a multiple of 8
+    const int nt = q % n_col_tiles;
+    const int mt = r8 * mpx + q / n_col_tiles;
+    gemm_tile<2, 4, 4, ZR_A_PACK4, true, EPI, 6, true>(a, mt * 64, nt * 128, true, 0, red, kslice, lane);
+  } else {
+    const int idx = bid - n_big;
+    const int n32 = (a.N + 31) >> 5;
+    const int blk = big_rows * 2 + idx / n32;
+    gemm_tile<1, 1, 4, ZR_A_PACK4, true, EPI, 8>(a, blk * 32, (idx % n32) * 32, true, 0, red, kslice, lane);
   }
 }
 
@@ -503,7 +546,7 @@ __global__ void __launch_bounds__(64 * NWV) gemm_lds_kernel(GemmArgs a) {
           if (ok[i * TMR + tm]) a.C[(long long)n * a.ldc + m] = v[i * TMR + tm];
           const int prow = (m0 >> 5) + tm;
           if (jl == 0 && n < a.N && prow * 32 < M) {
-            float* p = a.partials + ((long long)prow * a.N + n) * 2;
+            float* p = a.partials + ((long long)n * ((a.M + 31) >> 5) + prow) * 2;
             p[0] = mx[i * TMR + tm];
             p[1] = se[i * TMR + tm];
           }
@@ -615,6 +658,35 @@ int launch_rows(zr_ctx* ctx, GemmArgs& ga, int epi, int n_tiles) {
   return ZR_OK;
 }
 
+// gemm_tall_kernel: N a multiple of 128, fp32 k-interleaved A.  Returns false when the shape is better served by the
+// row-range kernel (too many rows would be left to the small tiles).
+bool launch_tall(zr_ctx* ctx, GemmArgs& ga, int epi, int* rc) {
+  const int blocks = (ga.M + 31) / 32;
+  const int n_col_tiles = ga.N / 128;
+  const int n32 = ga.N / 32;
+  const long long row_tiles = blocks / 2;  // whole 64-row tiles
+  // as many big row tiles as fill whole rounds of 256 workgroups, a multiple of 8 of them
+  long long big_rows = (row_tiles * n_col_tiles / 256) * 256 / n_col_tiles;
+  big_rows = big_rows / 8 * 8;
+  const long long small = (long long)(blocks - 2 * big_rows) * n32;
+  const bool offsets_fit = (long long)ga.K[0] * ga.lda[0] * 4 + 4096 < (1LL << 32) && (long long)ga.K[0] * ga.N * 4 < (1LL << 32);
+  if (big_rows == 0 || small > 1024 || !offsets_fit) {
+    // the left-over rows would be more than four rounds of small tiles: run whole big tiles to the end instead when
+    // that wastes less than a third of a round, else leave the shape to the row-range kernel
+    return false;
+  }
+  ga.m_tiles = ga.n_tiles = 0;
+  const int n_big = (int)(big_rows * n_col_tiles);
+  const unsigned grid = (unsigned)(n_big + small);
+  if (epi == ZR_EPI_STORE)
+    gemm_tall_kernel<ZR_EPI_STORE><<<grid, 256, 0, ctx->stream>>>(ga, (int)big_rows, n_col_tiles, n_big);
+  else
+    gemm_tall_kernel<ZR_EPI_SOFTMAX_PARTIAL><<<grid, 256, 0, ctx->stream>>>(ga, (int)big_rows, n_col_tiles, n_big);
+  hipError_t e = hipGetLastError();
+  *rc = e == hipSuccess ? ZR_OK : zr_set_error(ZR_EHIP, "launch of gemm_tall_kernel failed: %s", hipGetErrorString(e));
+  return true;
+}
+
 // Activations X (K x N fp32, column n at src + n*ld, K % 8 == 0) -> two bf16 arrays hi and lo with x = hi + lo up
 // to 2^-16 |x|, each k-interleaved by 8: element (k, n) at ((k/8)*N + n)*8 + k%8.  One thread per 8 values.
 __global__ void __launch_bounds__(256) zr_split_pack_x_kernel(const float* __restrict__ src, int K, int N, int ld,
@@ -646,6 +718,18 @@ __global__ void __launch_bounds__(256) pack4_kernel(const float* __restrict__ sr
   const int row = (int)(t % ldp);
   const int k = (int)(t / ldp) * 4 + k4;
   dst[i] = (row < M && k < K) ? src[row + (long long)k * ld] : 0.0f;
+}
+
+// The same for the TRANSPOSE of the source: element (row, k) of the packed matrix is src[k + row*ld].
+__global__ void __launch_bounds__(256) pack4_trans_kernel(const float* __restrict__ src, int M, int K, long long ld,
+                                                          int ldp, int kp, float* __restrict__ dst) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (long long)kp * ldp) return;
+  const int k4 = (int)(i & 3);
+  const long long t = i >> 2;
+  const int row = (int)(t % ldp);
+  const int k = (int)(t / ldp) * 4 + k4;
+  dst[i] = (row < M && k < K) ? src[k + (long long)row * ld] : 0.0f;
 }
 
 __global__ void __launch_bounds__(256) pack8_bf16_kernel(const float* __restrict__ src, int M, int K, long long ld,
@@ -682,6 +766,20 @@ int zr_pack4_launch(zr_ctx* ctx, const float* src, int M, int K, long long ld, i
   const long long total = (long long)kp * ldp;
   pack4_kernel<<<(unsigned)((total + 255) / 256), 256, 0, ctx->stream>>>(src, M, K, ld, ldp, kp, dst);
   ZR_LAUNCH_CHECK("pack4_kernel");
+  return ZR_OK;
+}
+
+int zr_pack4_x_launch(zr_ctx* ctx, const float* src, int K, int N, int ld, float* dst) {
+  const int f4 = (K / 4) * N;
+  pack4_x_kernel<<<(f4 + 255) / 256, 256, 0, ctx->stream>>>(src, K, N, ld, dst);
+  ZR_LAUNCH_CHECK("pack4_x_kernel");
+  return ZR_OK;
+}
+
+int zr_pack4_trans_launch(zr_ctx* ctx, const float* src, int M, int K, long long ld, int ldp, int kp, float* dst) {
+  const long long total = (long long)kp * ldp;
+  pack4_trans_kernel<<<(unsigned)((total + 255) / 256), 256, 0, ctx->stream>>>(src, M, K, ld, ldp, kp, dst);
+  ZR_LAUNCH_CHECK("pack4_trans_kernel");
   return ZR_OK;
 }
 
@@ -830,12 +928,30 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
     if (vec && d.nseg == 1 && zcount == 1 && d.M >= 8192 && d.N <= 1024 && ctx->gemm_cfg != 11 &&
         (d.epilogue == ZR_EPI_STORE || d.epilogue == ZR_EPI_SOFTMAX_PARTIAL)) {
       const int n32 = (d.N + 31) / 32;
+      if (d.N % 128 == 0 && ga.b_pack4 && ctx->gemm_cfg == 0) {
+        int rc = ZR_OK;
+        if (launch_tall(ctx, ga, d.epilogue, &rc)) return rc;
+      }
       const int n_tiles = (n32 + 3) / 4;
       const int tn = (n32 + n_tiles - 1) / n_tiles;
       if (tn == 1) return launch_rows<1>(ctx, ga, d.epilogue, n_tiles);
       if (tn <= 2) return launch_rows<2>(ctx, ga, d.epilogue, n_tiles);
       if (tn == 3) return launch_rows<3>(ctx, ga, d.epilogue, n_tiles);
       return launch_rows<4>(ctx, ga, d.epilogue, n_tiles);
+    }
+    // Small outputs (the attention projections: about a thousand rows by a minibatch of columns): 32 x 32 tiles with K
+    // split over the eight waves of a workgroup, so that a few hundred workgroups share the chip and each wave's chain
+    // of dependent matrix instructions is short.
+    {
+      const long long t32 = (long long)((d.M + 31) / 32) * ((d.N + 31) / 32) * zcount;
+      long long ktot = 0;
+      for (int s = 0; s < d.nseg; ++s) ktot += d.K[s];
+      if (ctx->gemm_cfg == 0 && d.groups == 0 && t32 <= 768 && ktot >= 512) {
+        ga.m_tiles = (ga.M + 31) / 32;
+        ga.n_tiles = (ga.N + 31) / 32;
+        if (vec) return launch_epi<1, 1, 8, 1, ZR_A_PACK4, true, 1>(ctx, ga, zcount, d.epilogue);
+        return launch_epi<1, 1, 8, 1, ZR_A_PACK4, false, 1>(ctx, ga, zcount, d.epilogue);
+      }
     }
     if (ctx->gemm_cfg == 12) return launch_pack4<4, 2, 1>(ctx, ga, d.epilogue, vec, zcount);
     if (ctx->gemm_cfg == 13) return launch_pack4<2, 2, 1>(ctx, ga, d.epilogue, vec, zcount);

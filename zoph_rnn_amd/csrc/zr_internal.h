@@ -93,7 +93,7 @@ enum ZrEpilogue {
   ZR_EPI_STORE = 0,           // C = acc (+ bias[m] if bias)
   ZR_EPI_TANH = 1,            // C = tanhf(acc)
   ZR_EPI_TANH_BIAS_MASK = 2,  // C = tanhf(acc + bias[m]) * mask[n]
-  ZR_EPI_SOFTMAX_PARTIAL = 3  // C = acc + bias[m]; per (32-row block, n) partial (max, sum exp) -> partials
+  ZR_EPI_SOFTMAX_PARTIAL = 3  // C = acc + bias[m]; per (n, 32-row block) partial (max, sum exp) -> partials
 };
 
 struct ZrGemmDesc {
@@ -119,7 +119,7 @@ struct ZrGemmDesc {
   const float* bias;  // per row m (may be NULL)
   const int* mask;    // per column n (ZR_EPI_TANH_BIAS_MASK)
   int epilogue;
-  float* partials;  // ZR_EPI_SOFTMAX_PARTIAL: [ceil(M/32)][N][2] floats
+  float* partials;  // ZR_EPI_SOFTMAX_PARTIAL: [N][ceil(M/32)][2] floats (contiguous per column)
   int accumulate;   // ZR_EPI_STORE only: C += product (+ bias) instead of C = ...
   // groups > 0: that many independent problems of the same shape in one launch (at most 8; one segment, plain store
   // epilogue, no bias): problem g multiplies gA[g] (instead of A[0]) with gB[g] (instead of B[0]) into gC[g]
@@ -136,6 +136,11 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d);
 // Packs one M x K column-major matrix (leading dimension ld) into the k-interleaved layout [kp/4][ldp][4] with
 // zero padding (ldp >= M a multiple of 32, kp >= K a multiple of 8).  dst holds kp*ldp floats.
 int zr_pack4_launch(zr_ctx* ctx, const float* src, int M, int K, long long ld, int ldp, int kp, float* dst);
+// Activations X (K x N fp32, column n at src + n*ld, K % 4 == 0, 16-byte aligned) into the k-interleaved layout
+// [K/4][N][4] (element (k, n) at ((k/4)*N + n)*4 + k%4).
+int zr_pack4_x_launch(zr_ctx* ctx, const float* src, int K, int N, int ld, float* dst);
+// The same from the transpose: element (row, k) of the packed matrix is src[k + row*ld].
+int zr_pack4_trans_launch(zr_ctx* ctx, const float* src, int M, int K, long long ld, int ldp, int kp, float* dst);
 // Same for the bf16 layout [kp/8][ldp][8] (round to nearest even); kp a multiple of 16.  dst holds kp*ldp elements.
 // Activations X (K x N fp32, column-major with leading dimension ld, K % 8 == 0) split into bf16 hi + lo arrays
 // (K*N elements each), both k-interleaved by 8.

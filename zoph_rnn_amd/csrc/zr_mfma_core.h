@@ -460,8 +460,10 @@ __device__ __forceinline__ void zr_half_wave_softmax_stats(const float (&v)[G], 
   for (int g = 0; g < G; ++g) mx[g] = fmaxf(mx[g], zr_dpp_move<0x140>(mx[g]));
 #pragma unroll
   for (int g = 0; g < G; ++g) mx[g] = fmaxf(mx[g], __shfl_xor(mx[g], 16, 64));
+  // hardware base-2 exponential (one ulp) of (v - max) * log2(e): relative error below 1e-7 * |v - max|, far inside
+  // what the sums of these terms are used for
 #pragma unroll
-  for (int g = 0; g < G; ++g) se[g] = ok[g] ? expf(v[g] - mx[g]) : 0.0f;
+  for (int g = 0; g < G; ++g) se[g] = ok[g] ? __builtin_amdgcn_exp2f((v[g] - mx[g]) * 1.4426950408889634f) : 0.0f;
 #pragma unroll
   for (int g = 0; g < G; ++g) se[g] += zr_dpp_move<0xB1>(se[g]);
 #pragma unroll

@@ -6,36 +6,58 @@
 
 namespace {
 
-// Combines the per-32-row partials of one column into (max, sum exp(x - max)).  One workgroup per column.
+// Folds the per-32-row partials of one column ([N][nblocks][2] floats: contiguous per column, nblocks
+// (max, sum exp(x - max)) pairs) into the column's (max, sum).  One workgroup per column; every thread folds its pairs
+// into one running pair -- eight loads at a time, all in flight together -- then the threads' pairs are folded
+// across the wave and the four waves, always in the same order.
+__device__ __forceinline__ void softmax_fold(float& m, float& sm, float pm, float ps) {
+  const float mn = fmaxf(m, pm);
+  sm = (m == mn ? sm : sm * expf(m - mn)) + (pm == mn ? ps : ps * expf(pm - mn));
+  m = mn;
+}
+
 __global__ void __launch_bounds__(256)
-softmax_colstats_kernel(const float* __restrict__ partials, int nblocks, int N, float* __restrict__ colstats) {
-  __shared__ float s_m[256];
-  __shared__ float s_s[256];
+softmax_colstats_kernel(const float* __restrict__ partials, int nblocks, float* __restrict__ colstats) {
+  typedef float zr_f32x2 __attribute__((ext_vector_type(2)));
+  __shared__ float s_m[4], s_s[4];
   const int n = blockIdx.x;
   const int tid = threadIdx.x;
-  float mx = -INFINITY;
-  for (int b = tid; b < nblocks; b += 256) mx = fmaxf(mx, partials[((size_t)b * N + n) * 2]);
-  s_m[tid] = mx;
+  const int lane = tid & 63, wave = tid >> 6;
+  const zr_f32x2* pp = (const zr_f32x2*)(partials + (size_t)n * nblocks * 2);
+  float mx = -INFINITY, sum = 0.0f;
+  for (int b0 = 0; b0 < nblocks; b0 += 2048) {
+    zr_f32x2 pr[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int b = b0 + tid + 256 * u;
+      pr[u] = zr_f32x2{-INFINITY, 0.0f};
+      if (b < nblocks) pr[u] = pp[b];
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) softmax_fold(mx, sum, pr[u].x, pr[u].y);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float om = __shfl_xor(mx, off, 64), os = __shfl_xor(sum, off, 64);
+    // both partners add in the same order, so every lane ends with the same bits
+    float a_m = (lane & off) ? om : mx, a_s = (lane & off) ? os : sum;
+    const float b_m = (lane & off) ? mx : om, b_s = (lane & off) ? sum : os;
+    softmax_fold(a_m, a_s, b_m, b_s);
+    mx = a_m;
+    sum = a_s;
+  }
+  if (lane == 0) {
+    s_m[wave] = mx;
+    s_s[wave] = sum;
+  }
   __syncthreads();
-  for (int st = 128; st > 0; st >>= 1) {
-    if (tid < st) s_m[tid] = fmaxf(s_m[tid], s_m[tid + st]);
-    __syncthreads();
-  }
-  mx = s_m[0];
-  float sum = 0.0f;
-  for (int b = tid; b < nblocks; b += 256) {
-    const float* p = partials + ((size_t)b * N + n) * 2;
-    sum += p[1] * expf(p[0] - mx);
-  }
-  s_s[tid] = sum;
-  __syncthreads();
-  for (int st = 128; st > 0; st >>= 1) {
-    if (tid < st) s_s[tid] += s_s[tid + st];
-    __syncthreads();
-  }
   if (tid == 0) {
+    mx = s_m[0];
+    sum = s_s[0];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) softmax_fold(mx, sum, s_m[w], s_s[w]);
     colstats[2 * n] = mx;
-    colstats[2 * n + 1] = s_s[0];
+    colstats[2 * n + 1] = sum;
   }
 }
 
@@ -46,7 +68,6 @@ softmax_normalize_kernel(const float* in, float* out, int V, const float* __rest
   const int n = blockIdx.y;
   const float mx = colstats[2 * n];
   const float sum = colstats[2 * n + 1];
-  const float inv = 1.0f / sum;
   const float lsum = logf(sum);
   const float* x = in + (size_t)n * V;
   float* y = out + (size_t)n * V;
@@ -73,7 +94,6 @@ softmax_normalize_kernel(const float* in, float* out, int V, const float* __rest
     const int i = blockIdx.x * 256 + threadIdx.x;
     if (i < V) y[i] = (MODE == 0) ? expf(x[i] - mx) / sum : (x[i] - mx) - lsum;
   }
-  (void)inv;
 }
 
 // Double-precision column statistics straight from the logits (outputdist_perplexity_kernel accumulates in
@@ -147,7 +167,7 @@ int logits_with_partials(zr_ctx* ctx, const float* d_D, const float* d_b_d, int 
                          float* d_logits, float** partials_out, int* nblocks_out) {
   const int nblocks = zr_softmax_partial_blocks(V);
   void* scratch = nullptr;
-  // partials [nblocks][mb][2] followed by column stats (2 doubles per column, also used as 2 floats)
+  // partials [mb][nblocks][2] followed by column stats (2 doubles per column, also used as 2 floats)
   const size_t pbytes = sizeof(float) * 2 * (size_t)nblocks * mb;
   int rc = zr_ctx_scratch(ctx, 1, pbytes + sizeof(double) * 2 * (size_t)mb + 64, &scratch);
   if (rc) return rc;
@@ -280,7 +300,7 @@ int zr_softmax_forward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V,
   rc = logits_with_partials(ctx, d_D, d_b_d, V, H, d_h, mb, logits, &partials, &nblocks);
   if (rc) return rc;
   float* colstats = (float*)stats_ptr(partials, nblocks, mb);
-  softmax_colstats_kernel<<<mb, 256, 0, ctx->stream>>>(partials, nblocks, mb, colstats);
+  softmax_colstats_kernel<<<mb, 256, 0, ctx->stream>>>(partials, nblocks, colstats);
   ZR_LAUNCH_CHECK("softmax_colstats_kernel");
   const bool vec = (V % 4 == 0) && (((uintptr_t)logits & 15u) == 0) && (((uintptr_t)d_out & 15u) == 0);
   if (vec) {

@@ -54,6 +54,7 @@ class BeamDecode:
         self.tables = [ctx.empty((H, cols)) for _ in range(src_len)]
         self.attn = ctx.attn_create(H, cols, attention_D, w.attn["W_a"], w.attn["W_p"], w.attn["v_p"],
                                     w.attn["out_bias"], w.attn["W_c1"], w.attn["W_c2"], self.tables)
+        ctx.attn_prepare(self.attn)
         self.bm = ctx.beam_create(beam, w.Vt, n_sent, self.max_len, penalty)
         self.h = [[ctx.empty((H, cols)) for _ in range(L)] for _ in range(2)]  # ping-pong: previous / new state
         self.c = [[ctx.empty((H, cols)) for _ in range(L)] for _ in range(2)]

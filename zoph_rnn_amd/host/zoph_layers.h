@@ -262,7 +262,10 @@ class attention_layer {  // src/attention_layer.h:14-143
     h_total_hs_mat = total_hs;
     ZOPH_CALL(zr_attn_create(ctx, LSTM_size, minibatch_size, D, d_W_a, d_W_p, d_v_p, d_output_bias, d_W_c_p1, d_W_c_p2,
                              h_total_hs_mat.data(), (int)h_total_hs_mat.size(), &attn));
-    if (BZ_CUDA::bf16_weights) ZOPH_CALL(zr_attn_use_bf16_weights(ctx, attn));
+    if (BZ_CUDA::bf16_weights)
+      ZOPH_CALL(zr_attn_use_bf16_weights(ctx, attn));
+    else
+      ZOPH_CALL(zr_attn_prepare(ctx, attn));
     for (int i = 0; i < longest_sent; i++)
       nodes.push_back(attention_node<dType>(LSTM_size, minibatch_size, device_number, D, feed_input, this, i));
   }
@@ -289,7 +292,12 @@ class attention_layer {  // src/attention_layer.h:14-143
     read_matrix_GPU(ctx, d_output_bias, LSTM_size, 1, input);
     read_matrix_GPU(ctx, d_W_c_p1, LSTM_size, LSTM_size, input);
     read_matrix_GPU(ctx, d_W_c_p2, LSTM_size, LSTM_size, input);
-    if (BZ_CUDA::bf16_weights && attn) ZOPH_CALL(zr_attn_use_bf16_weights(ctx, attn));
+    if (attn) {  // the snapshots follow the matrices
+      if (BZ_CUDA::bf16_weights)
+        ZOPH_CALL(zr_attn_use_bf16_weights(ctx, attn));
+      else
+        ZOPH_CALL(zr_attn_prepare(ctx, attn));
+    }
   }
 };
 

@@ -947,7 +947,10 @@ class beam_decoder {
       auto* a = m.att;
       ZOPH_CALL(zr_attn_create(ctx, H, cols, D, a->d_W_a, a->d_W_p, a->d_v_p, a->d_output_bias, a->d_W_c_p1,
                                a->d_W_c_p2, tp.data(), longest_sent, &attn));
-      if (BZ_CUDA::bf16_weights) ZOPH_CALL(zr_attn_use_bf16_weights(ctx, attn));
+      if (BZ_CUDA::bf16_weights)
+        ZOPH_CALL(zr_attn_use_bf16_weights(ctx, attn));
+      else
+        ZOPH_CALL(zr_attn_prepare(ctx, attn));
     }
     ZOPH_CALL(zr_beam_create(ctx, beam, Vt, n_sent, longest_sent + 3, (float)penalty, &bm));
   }
