@@ -152,6 +152,14 @@ int zr_lstm_step(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_in, const
                  const float* d_cprev, const float* d_htild, const int* d_mask01, float clip_threshold, int mb,
                  float* d_h, float* d_c, float* const d_gates[4]);
 
+/* The same node with the embedding lookup folded in: LSTM_IH_Node::forward_prop_GPU as a whole, sparse_lookup_kernel
+ * included (src/LSTM.hpp:95 and :133-399).  Column b of the node's input is d_embed[:, d_ids_nonneg[b]] (d_embed is
+ * H x V), read straight from the embedding by the product's own loads; no H x mb copy of the looked-up columns is
+ * made.  Ids outside [0, V) are clamped and raise the data flag, as in zr_embed_gather. */
+int zr_lstm_step_embed(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_embed, int V, const int* d_ids_nonneg,
+                       const float* d_hprev, const float* d_cprev, const float* d_htild, const int* d_mask01,
+                       float clip_threshold, int mb, float* d_h, float* d_c, float* const d_gates[4]);
+
 /* The stand-alone fused gate kernel (the four activation kernels + c_t + clip + h_t + mask of the list above)
  * on pre-activations that are already in memory: d_preact is 4 planes (i,f,c,o) of H x mb holding
  * M x + W_h h (+ Q h~) without bias. */

@@ -598,6 +598,44 @@ def test_lstm_step_register_kernel_split_across_workgroups(ctx, H, mb, kparts):
     assert got_feed["h"].tobytes() == again["h"].tobytes() and got_feed["c"].tobytes() == again["c"].tobytes()
 
 
+@pytest.mark.parametrize("H,mb,feed,fused", [(64, 5, False, 1), (1000, 128, True, 1), (200, 70, True, 1), (72, 33, False, 0),
+                                            (36, 12, True, 1)])
+def test_lstm_step_with_embedding_lookup_folded_in(ctx, H, mb, feed, fused):
+    """zr_lstm_step_embed (the node reads its input columns from the embedding by token id) against the gather followed
+    by zr_lstm_step -- bit for bit, the same kernel reads the same numbers -- and against the oracle; duplicate ids,
+    first and last column of the embedding, a masked column; also through the two-phase path (fused = 0)."""
+    g = synth.rng(29, H + mb)
+    V = 977
+    ly = synth.lstm_layer(g, H, feed_input=feed, forget_bias_one=True)
+    embed = U(g, (H, V), -1, 1)
+    ids = g.integers(0, V, size=mb).astype(np.int32)
+    ids[0], ids[mb - 1] = 0, V - 1
+    if mb > 3:
+        ids[2] = ids[1]
+    hp, cp, ht = U(g, (H, mb), -1, 1), U(g, (H, mb), -1, 1), U(g, (H, mb), -1, 1)
+    mask = np.ones(mb, np.int32)
+    mask[mb // 2] = 0
+    layer = Layer(ctx, ly)
+    d_embed, d_ids, d_mask = ctx.array(embed), ctx.array(ids), ctx.array(mask)
+    d_hp, d_cp, d_ht = ctx.array(hp), ctx.array(cp), ctx.array(ht) if feed else None
+    h1, c1, h2, c2, x = (ctx.empty((H, mb)) for _ in range(5))
+    ctx.set_option(capi.ZR_OPT_LSTM_FUSED_EPILOGUE, fused)
+    try:
+        ctx.lstm_step_embed(layer.w, d_embed, V, d_ids, d_hp, d_cp, d_mask, mb, h1, c1, d_htild=d_ht, clip=0.8)
+        ctx.embed_gather(d_embed, H, V, d_ids, mb, x)
+        ctx.lstm_step(layer.w, x, d_hp, d_cp, d_mask, mb, h2, c2, d_htild=d_ht, clip=0.8)
+        ctx.sync()
+    finally:
+        ctx.set_option(capi.ZR_OPT_LSTM_FUSED_EPILOGUE, 1)
+        layer.close()
+    assert h1.get().tobytes() == h2.get().tobytes() and c1.get().tobytes() == c2.get().tobytes()
+    want = o.lstm_step(ly["M"], ly["Wh"], ly["b"], o.embed_gather(embed, ids), hp, cp, mask, Q=ly.get("Q"),
+                       htild=ht if feed else None, clip=0.8)
+    assert_close(h1.get(), want["h"], what="h")
+    assert_close(c1.get(), want["c"], what="c")
+    assert np.all(h1.get()[:, mb // 2] == 0)
+
+
 def test_stack_forward_with_split_kernel_forced(ctx):
     g = synth.rng(17, 1)
     H, mb, T, V, L = 64, 5, 7, 211, 3

@@ -40,7 +40,7 @@ SYMBOLS = [
     "zr_unstack_gates", "zr_lstm_stack_backward", "zr_lstm_weight_gradients", "zr_embed_gradient",
     "zr_softmax_backward", "zr_sgd_update", "zr_lstm_node_backward", "zr_lstm_node_gradients",
     "zr_softmax_backward_accumulate", "zr_gather_columns_multi", "zr_softmax_backward_loss",
-    "zr_softmax_forward_static", "zr_ctx_query", "zr_attn_prepare",
+    "zr_softmax_forward_static", "zr_ctx_query", "zr_attn_prepare", "zr_lstm_step_embed",
 ]
 
 _lib = None
@@ -203,6 +203,12 @@ class Context:
         _chk(load().zr_lstm_step(self.h, w, _vp(d_in), _vp(d_hprev), _vp(d_cprev), _vp(d_htild), _vp(d_mask),
                                  C.c_float(clip), C.c_int(mb), _vp(d_h), _vp(d_c),
                                  _ptr_array(gates) if gates else None))
+
+    def lstm_step_embed(self, w, d_embed, V, d_ids, d_hprev, d_cprev, d_mask, mb, d_h, d_c, d_htild=None, clip=0.0,
+                        gates=None):
+        _chk(load().zr_lstm_step_embed(self.h, w, _vp(d_embed), C.c_int(V), _vp(d_ids), _vp(d_hprev), _vp(d_cprev),
+                                       _vp(d_htild), _vp(d_mask), C.c_float(clip), C.c_int(mb), _vp(d_h), _vp(d_c),
+                                       _ptr_array(gates) if gates else None))
 
     def lstm_gates(self, d_preact, b, d_cprev, d_mask, H, mb, d_h, d_c, clip=0.0, gates=None):
         _chk(load().zr_lstm_gates(self.h, _vp(d_preact), _ptr_array(b), _vp(d_cprev), _vp(d_mask), C.c_float(clip),

@@ -1114,9 +1114,29 @@ int zr_lstm_weights_destroy(zr_ctx* ctx, zr_lstm_weights* w) {
   return ZR_OK;
 }
 
+static int lstm_step_impl(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_in, const int* d_gather_ids, int V,
+                          const float* d_hprev, const float* d_cprev, const float* d_htild, const int* d_mask01,
+                          float clip_threshold, int mb, float* d_h, float* d_c, float* const d_gates[4]);
+
 int zr_lstm_step(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_in, const float* d_hprev,
                  const float* d_cprev, const float* d_htild, const int* d_mask01, float clip_threshold, int mb,
                  float* d_h, float* d_c, float* const d_gates[4]) {
+  return lstm_step_impl(ctx, w, d_in, nullptr, 0, d_hprev, d_cprev, d_htild, d_mask01, clip_threshold, mb, d_h, d_c,
+                        d_gates);
+}
+
+int zr_lstm_step_embed(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_embed, int V, const int* d_ids_nonneg,
+                       const float* d_hprev, const float* d_cprev, const float* d_htild, const int* d_mask01,
+                       float clip_threshold, int mb, float* d_h, float* d_c, float* const d_gates[4]) {
+  ZR_CHECK_ARG(V > 0 && d_ids_nonneg != nullptr, "zr_lstm_step_embed: V = %d or null token ids", V);
+  return lstm_step_impl(ctx, w, d_embed, d_ids_nonneg, V, d_hprev, d_cprev, d_htild, d_mask01, clip_threshold, mb, d_h,
+                        d_c, d_gates);
+}
+
+// d_gather_ids non-null: d_in is the H x V embedding and column b of the input is d_in[:, d_gather_ids[b]].
+static int lstm_step_impl(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_in, const int* d_gather_ids, int V,
+                          const float* d_hprev, const float* d_cprev, const float* d_htild, const int* d_mask01,
+                          float clip_threshold, int mb, float* d_h, float* d_c, float* const d_gates[4]) {
   int rc = zr_bind_device(ctx);
   if (rc) return rc;
   ZR_CHECK_ARG(w != nullptr, "zr_lstm_step: weights are null");
@@ -1128,6 +1148,17 @@ int zr_lstm_step(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_in, const
     for (int g = 0; g < 4; ++g) ZR_CHECK_ARG(d_gates[g] != nullptr, "zr_lstm_step: d_gates[%d] is null", g);
   const int H = w->H;
   const int nseg = d_htild ? 3 : 2;
+  if (d_gather_ids && (w->bf16 || !ctx->lstm_fused)) {
+    // these paths re-lay-out or re-read their inputs as whole matrices: gather the columns first
+    void* x = nullptr;
+    rc = zr_ctx_scratch(ctx, 1, sizeof(float) * (size_t)H * mb * (ctx->lstm_fused ? 1 : 5), &x);
+    if (rc) return rc;
+    float* xg = (float*)x + (ctx->lstm_fused ? 0 : 4 * (size_t)H * mb);  // behind the pre-activation planes
+    rc = zr_embed_gather(ctx, d_in, H, V, d_gather_ids, mb, xg);
+    if (rc) return rc;
+    d_in = xg;
+    d_gather_ids = nullptr;
+  }
 
   LstmLaunch L = {};
   L.n_units = 1;
@@ -1143,14 +1174,14 @@ int zr_lstm_step(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_in, const
   U.in[0] = d_in;
   U.in[1] = d_hprev;
   U.in[2] = d_htild;
-  U.gather_ids = nullptr;
+  U.gather_ids = d_gather_ids;
   U.cprev = d_cprev;
   U.mask01 = d_mask01;
   U.h = d_h;
   U.c = d_c;
   for (int g = 0; g < 4; ++g) U.gates[g] = d_gates ? d_gates[g] : nullptr;
   U.nseg = nseg;
-  U.V = 0;
+  U.V = d_gather_ids ? V : 0;
   const bool vec = (H % 4 == 0) && aligned16(d_in) && aligned16(d_hprev) && (!d_htild || aligned16(d_htild));
   if (w->bf16 && vec) {
     // split the fp32 inputs into bf16 hi + lo once per node, k-interleaved, instead of in every workgroup's K loop

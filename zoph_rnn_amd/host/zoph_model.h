@@ -959,11 +959,13 @@ class beam_decoder {
   void forward_target(int p, int step_index) {
     const int q = 1 - p;
     ZOPH_CALL(zr_vocab_prep(ctx, d_words, cols, Vt, d_words_nn, nullptr));
-    ZOPH_CALL(zr_embed_gather(ctx, m.input_layer_target.d_W, H, Vt, d_words_nn, cols, x));
-    const dType* below = x;
-    for (int l = 0; l < L; l++) {
-      const dType* feed = (l == 0 && feed_input && step_index > 0) ? h_tild[p] : nullptr;
-      ZOPH_CALL(zr_lstm_step(ctx, tgt_w[l], below, h[p][l], c[p][l], feed, d_ones, 0.0f, cols, h[q][l], c[q][l], nullptr));
+    // layer 0 looks its input columns up in the embedding itself (sparse lookup folded into the node)
+    const dType* feed = (feed_input && step_index > 0) ? h_tild[p] : nullptr;
+    ZOPH_CALL(zr_lstm_step_embed(ctx, tgt_w[0], m.input_layer_target.d_W, Vt, d_words_nn, h[p][0], c[p][0], feed, d_ones,
+                                 0.0f, cols, h[q][0], c[q][0], nullptr));
+    const dType* below = h[q][0];
+    for (int l = 1; l < L; l++) {
+      ZOPH_CALL(zr_lstm_step(ctx, tgt_w[l], below, h[p][l], c[p][l], nullptr, d_ones, 0.0f, cols, h[q][l], c[q][l], nullptr));
       below = h[q][l];
     }
     const dType* top = below;
