@@ -264,6 +264,13 @@ int zr_attn_destroy(zr_ctx* ctx, zr_attn* a);
 int zr_attn_step(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, const float* d_h_t, const int* d_mask01,
                  float* d_htild, float* d_alignments, int* d_indices, float* d_p_t, float* d_c_ctx);
 
+/* get_viterbi_alignment_kernel (src/custom_kernels.h:1623-1635, launched by attention_node::forward_prop when
+ * BZ_CUDA::unk_replacement is set, src/attention_node.hpp:225-234): d_viterbi[b] = source position of the window slot
+ * with the largest alignment weight of column b (first of equal maxima; -1 for a masked column), from the alignments
+ * and window indices of the last zr_attn_step.  d_alignments / d_indices: what was passed to zr_attn_step, or NULL for
+ * the object's internal arrays. */
+int zr_attn_viterbi(zr_ctx* ctx, const zr_attn* a, const float* d_alignments, const int* d_indices, int* d_viterbi);
+
 /* ---- A12: decoder state shuffles ------------------------------------------------------------------------- */
 
 /* swap_states_decoding (src/Input_To_Hidden_Layer.hpp:1231-1242, src/Hidden_To_Hidden_Layer.hpp:780-791):

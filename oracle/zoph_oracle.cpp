@@ -406,6 +406,22 @@ void orc_attention_forward(int acc64, int H, int mb, int D, const float* W_a, co
     }
 }
 
+// get_viterbi_alignment_kernel, src/custom_kernels.h:1623-1635: for every column the window index of the largest
+// alignment weight; the running maximum starts at -1 and only a strictly larger weight replaces it.
+void orc_attention_viterbi(const float* alignments, const int* indices, int D, int mb, int* out) {
+  for (int b = 0; b < mb; ++b) {
+    float max_val = -1;
+    int max_index = -1;
+    for (int i = 0; i < 2 * D + 1; ++i) {
+      if (max_val < alignments[IDX2C(b, i, mb)]) {
+        max_val = alignments[IDX2C(b, i, mb)];
+        max_index = indices[IDX2C(b, i, mb)];
+      }
+    }
+    out[b] = max_index;
+  }
+}
+
 // Column gather used by the decoder state shuffles: dst[:,i] = src[:,perm[i]]
 // (Input_To_Hidden_Layer::swap_states_decoding, src/Input_To_Hidden_Layer.hpp:1231-1242).
 void orc_gather_columns(const float* src, int H, const int* perm, int n, float* dst) {

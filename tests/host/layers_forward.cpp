@@ -2,7 +2,11 @@
 // neuralMT_model::getError does (src/model.hpp:1463-1802): index preparation, the source sweep, the target sweep
 // with attention + feed-input on the top target layer, and the per-step loss.  Weights come from a model file in
 // the reference's text layout.  Output (stdout): one line "loss <t> <value>" per target step, then the top-layer
-// output of every target step ("h <t> <H*mb floats>").
+// output of every target step ("h <t> <H*mb floats>").  With a source side the members that take the reference's own
+// parameter lists are exercised too: the layers' init_attention(device, D, feed_input, model, params), then at the end
+// a decode-time attention layer set up with init_att_decoder on copies of the source states (its one node re-runs the
+// last target step with every column unmasked: "dec_h <H*mb floats>", "viterbi <mb ints>") and
+// swap_states_decoding with a host index vector ("swap_before" / "swap_after", the first target node's h).
 //
 // usage: layers_forward <weights.txt> <ids.txt> H mb V L S T D
 //   ids.txt: S*mb source ids, T*mb target input ids, T*mb target output ids, 2*mb batch_info (time-major, -1 pads)
@@ -89,14 +93,18 @@ int main(int argc, char** argv) {
 
   attention_layer<precision>* att = nullptr;
   if (seq2seq) {
-    std::vector<const precision*> total_hs(longest);
+    // as neuralMT_model::initModel does (src/model.hpp:330-345): the top target layer builds the attention layer from
+    // the model's source states
+    model.source_top_h_t.resize(longest);
     for (int i = 0; i < longest; i++)
-      total_hs[i] = (L == 1) ? input_layer_source.nodes[i].d_h_t : source_hidden_layers[L - 2].nodes[i].d_h_t;
-    att = new attention_layer<precision>(H, mb, 0, D, longest, gpu, total_hs, true);
-    if (L == 1)
-      input_layer_target.init_attention(att);
-    else
-      target_hidden_layers[L - 2].init_attention(att);
+      model.source_top_h_t[i] = (L == 1) ? input_layer_source.nodes[i].d_h_t : source_hidden_layers[L - 2].nodes[i].d_h_t;
+    if (L == 1) {
+      input_layer_target.init_attention(0, D, true, &model, params);
+      att = input_layer_target.attent_layer;
+    } else {
+      target_hidden_layers[L - 2].init_attention(0, D, true, &model, params);
+      att = target_hidden_layers[L - 2].attent_layer;
+    }
     input_layer_target.init_feed_input(L == 1 ? nullptr : &target_hidden_layers[L - 2], false);
   }
 
@@ -187,6 +195,50 @@ int main(int argc, char** argv) {
     std::cout << "loss " << i << " " << std::setprecision(15) << loss << std::setprecision(9) << "\n";
     ZOPH_CALL(zr_d2h(gpu.ctx, host.data(), softmax->get_ht_ptr(i), host.size() * sizeof(precision)));
     std::cout << "h " << i;
+    for (precision v : host) std::cout << " " << v;
+    std::cout << "\n";
+  }
+  if (seq2seq && !BZ_CUDA::bf16_weights) {
+    // decode-time attention layer (neuralMT_model::initModel_decoding, src/model.hpp:560-583): copies of the source
+    // states, one node, every column unmasked
+    BZ_CUDA::unk_replacement = true;
+    const size_t n = (size_t)H * mb;
+    for (int i = 0; i < longest; i++) {
+      precision* p = nullptr;
+      ZOPH_CALL(zr_malloc(gpu.ctx, n * sizeof(precision), (void**)&p));
+      ZOPH_CALL(zr_d2d(gpu.ctx, p, model.source_top_h_t[i], n * sizeof(precision)));
+      model.top_source_states.push_back(p);
+    }
+    attention_layer<precision> decoder_att_layer;
+    std::vector<precision*> none;
+    cublasHandle_t handle = gpu.ctx;
+    decoder_att_layer.init_att_decoder(H, mb, 0, D, longest, handle, &model, false, model.top_source_states, false, none);
+    precision* src_w[] = {att->d_W_a, att->d_W_p, att->d_v_p, att->d_output_bias, att->d_W_c_p1, att->d_W_c_p2};
+    precision* dst_w[] = {decoder_att_layer.d_W_a, decoder_att_layer.d_W_p, decoder_att_layer.d_v_p,
+                          decoder_att_layer.d_output_bias, decoder_att_layer.d_W_c_p1, decoder_att_layer.d_W_c_p2};
+    const size_t sizes[] = {(size_t)H * H, (size_t)H * H, (size_t)H, (size_t)H, (size_t)H * H, (size_t)H * H};
+    for (int i = 0; i < 6; i++) ZOPH_CALL(zr_d2d(gpu.ctx, dst_w[i], src_w[i], sizes[i] * sizeof(precision)));
+    ZOPH_CALL(zr_attn_prepare(gpu.ctx, decoder_att_layer.attn));
+    decoder_att_layer.prep_minibatch_info(binfo.data());
+    decoder_att_layer.nodes[0].d_h_t = (L == 1) ? input_layer_target.nodes[T - 1].d_h_t : target_hidden_layers[L - 2].nodes[T - 1].d_h_t;
+    decoder_att_layer.nodes[0].forward_prop();
+    ZOPH_CALL(zr_d2h(gpu.ctx, host.data(), decoder_att_layer.nodes[0].d_final_temp_2, host.size() * sizeof(precision)));
+    std::cout << "dec_h";
+    for (precision v : host) std::cout << " " << v;
+    std::cout << "\nviterbi";
+    for (int v : BZ_CUDA::viterbi_alignments) std::cout << " " << v;
+    std::cout << "\n";
+    // swap_states_decoding with a host-side index vector, as the reference's decoder passes it
+    std::vector<int> order(mb);
+    for (int b = 0; b < mb; b++) order[b] = (b * 3 + 1) % mb;
+    precision* d_temp = nullptr;
+    ZOPH_CALL(zr_malloc(gpu.ctx, n * sizeof(precision), (void**)&d_temp));
+    ZOPH_CALL(zr_d2h(gpu.ctx, host.data(), input_layer_target.nodes[0].d_h_t, host.size() * sizeof(precision)));
+    std::cout << "swap_before";
+    for (precision v : host) std::cout << " " << v;
+    input_layer_target.swap_states_decoding(order, 0, d_temp);
+    ZOPH_CALL(zr_d2h(gpu.ctx, host.data(), input_layer_target.nodes[0].d_h_t, host.size() * sizeof(precision)));
+    std::cout << "\nswap_after";
     for (precision v : host) std::cout << " " << v;
     std::cout << "\n";
   }

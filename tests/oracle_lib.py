@@ -198,6 +198,15 @@ def attention_forward(W_a, W_p, v_p, out_bias, W_c1, W_c2, hs_table, batch_info,
     return out
 
 
+def attention_viterbi(alignments, indices):
+    """alignments, indices: (mb, 2D+1) arrays laid out [b + mb*j] (column-major)."""
+    al, ix = F(alignments), F(indices, np.int32)
+    mb, Wn = al.shape
+    out = np.empty(mb, dtype=np.int32)
+    lib().orc_attention_viterbi(_p(al), _p(ix, i32p), C.c_int((Wn - 1) // 2), C.c_int(mb), _p(out, i32p))
+    return out
+
+
 def pack_hs_table(hs_table):
     """(S, H, mb) logical array -> flat float32 buffer of S column-major H x mb tables."""
     hs_table = np.asarray(hs_table, dtype=np.float32)

@@ -81,6 +81,10 @@ def _run_driver(tmp_path, weights_writer, ids_blocks, H, mb, V, L, S, T, D, bf16
             losses[int(p[1])] = float(p[2])
         elif p[0] == "h":
             hs[int(p[1])] = np.array(p[2:], dtype=np.float32).reshape(H, mb, order="F")
+        elif p[0] in ("dec_h", "swap_before", "swap_after"):
+            hs[p[0]] = np.array(p[1:], dtype=np.float32).reshape(H, mb, order="F")
+        elif p[0] == "viterbi":
+            hs["viterbi"] = np.array(p[1:], dtype=np.int32)
     # dump_weights must reproduce the file it loaded (same order, same layout)
     dumped = np.array(open(wpath + ".dump").read().split(), dtype=np.float64)
     loaded = np.array(open(wpath).read().split(), dtype=np.float64)
@@ -186,3 +190,12 @@ def test_seq2seq_attention_feed_input_through_layer_classes(tmp_path, L, bf16):
         assert_close(hs[t], att["h_tild"], floor=1.0 if bf16 else 5e-2, what="h_tild step %d" % t)
         lp = o.softmax_logprob_f64(o.softmax_logits(Dm, bd, att["h_tild"]))
         assert losses[t] == pytest.approx(o.softmax_loss(lp, tgt[t], tmask[t]), rel=1e-4 if bf16 else 1e-5, abs=1e-6)
+    if not bf16:
+        # the decode-time attention layer (init_att_decoder, one node, all columns unmasked) on the last step's top h
+        ones = np.ones(mb, np.int32)
+        dec = o.attention_forward(hs_table=table, batch_info=binfo, h_t=below, mask01=ones, D=D, **attn)
+        assert_close(hs["dec_h"], dec["h_tild"], what="decode-time attention layer h_tild")
+        assert hs["viterbi"].tolist() == o.attention_viterbi(dec["alignments"], dec["indices"]).tolist()
+        # swap_states_decoding with a host index vector: column i <- column (3 i + 1) mod mb
+        order = [(b * 3 + 1) % mb for b in range(mb)]
+        assert np.array_equal(hs["swap_after"], hs["swap_before"][:, order])

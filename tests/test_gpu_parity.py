@@ -448,6 +448,55 @@ def test_attention_against_oracle(ctx, H, mb, S, D, prepared):
     assert np.all(got["h_tild"][:, mask == 0] == 0)
 
 
+@pytest.mark.parametrize("mb,D", [(7, 4), (130, 50), (3, 255)])
+def test_attention_viterbi_alignment_bit_exact(ctx, mb, D):
+    """zr_attn_viterbi against the oracle on crafted weights: ties (first maximum wins), all-zero live columns, masked
+    columns and short windows; then on the alignments of a real attention step."""
+    g = synth.rng(31, mb + D)
+    Wn = 2 * D + 1
+    al = np.asfortranarray(g.random((mb, Wn), dtype=np.float32))
+    ix = np.asfortranarray(g.integers(0, 300, size=(mb, Wn)).astype(np.int32))
+    al[1, 2] = al[1, Wn - 1] = 2.0
+    al[2, :] = 0.0
+    al[0, :], ix[0, :] = 0.0, -1
+    if mb > 5:
+        al[5, 5:], ix[5, 5:] = 0.0, -1
+        al[6, 70 % Wn] = al[6, 3] = 3.0  # tie across lanes: lower slot wins
+    H = 8
+    tables = [ctx.zeros((H, mb))]
+    z = ctx.zeros((H, H))
+    a = ctx.attn_create(H, mb, D, z, z, ctx.zeros((H,)), ctx.zeros((H,)), z, z, tables)
+    d_out = ctx.empty((mb,), np.int32)
+    ctx.attn_viterbi(a, ctx.array(al), ctx.array(ix), d_out)
+    ctx.sync()
+    assert d_out.get().tolist() == o.attention_viterbi(al, ix).tolist()
+    ctx.attn_destroy(a)
+
+
+def test_attention_viterbi_after_a_step(ctx):
+    H, mb, S, D = 64, 9, 12, 3
+    g = synth.rng(32, 1)
+    w = synth.attention_weights(g, H)
+    hs = (g.standard_normal(size=(S, H, mb), dtype=np.float32) * np.float32(0.5))
+    lens = g.integers(2, S + 1, size=mb).astype(np.int32)
+    bi = np.concatenate([lens, S - lens]).astype(np.int32)
+    mask = np.ones(mb, np.int32)
+    mask[4] = 0
+    h_t = U(g, (H, mb), -1, 1)
+    tables = [ctx.array(np.asfortranarray(hs[t])) for t in range(S)]
+    dw = {k: ctx.array(v) for k, v in w.items()}
+    a = ctx.attn_create(H, mb, D, dw["W_a"], dw["W_p"], dw["v_p"], dw["out_bias"], dw["W_c1"], dw["W_c2"], tables)
+    ctx.attn_prepare(a)
+    d_ht, d_out = ctx.empty((H, mb)), ctx.empty((mb,), np.int32)
+    ctx.attn_step(a, ctx.array(bi), ctx.array(h_t), ctx.array(mask), d_ht)  # internal alignment / index arrays
+    ctx.attn_viterbi(a, None, None, d_out)
+    ctx.sync()
+    want = o.attention_forward(hs_table=hs, batch_info=bi, h_t=h_t, mask01=mask, D=D, **w)
+    assert d_out.get().tolist() == o.attention_viterbi(want["alignments"], want["indices"]).tolist()
+    assert d_out.get()[4] == -1
+    ctx.attn_destroy(a)
+
+
 @pytest.mark.parametrize("prepared", [False, True])
 def test_attention_negative_scores_use_zero_initialised_max(ctx, prepared):
     """All scores very negative: the reference's max starts at 0, exp underflows, the sum is 0 and the

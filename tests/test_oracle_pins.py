@@ -644,3 +644,20 @@ def test_stack_forward_nonzero_initial_state_and_clip_against_numpy_f64(clip):
         # each layer has its own initial state: swapping two layers' states changes the result
     h_sw, _ = o.lstm_stack_forward(embed, layers, nn, m, h0=h0[::-1], c0=c0[::-1], clip=clip)
     assert np.abs(h_sw - want_h).max() > 1e-2
+
+
+def test_attention_viterbi_first_maximum_wins():
+    """Independent statement: numpy argmax returns the first maximum, the rule of a scan that only replaces on a
+    strictly larger weight; a masked column (all weights 0, all indices -1) reports -1."""
+    rng = np.random.default_rng(9)
+    mb, D = 7, 4
+    Wn = 2 * D + 1
+    al = np.asfortranarray(rng.random((mb, Wn)).astype(np.float32))
+    ix = np.asfortranarray(rng.integers(0, 40, size=(mb, Wn)).astype(np.int32))
+    al[1, 2] = al[1, 6] = 2.0           # tie: slot 2 wins
+    al[3, :] = 0.0                      # all zero, live column: first slot's index
+    al[4, :], ix[4, :] = 0.0, -1        # masked column
+    al[5, 5:], ix[5, 5:] = 0.0, -1      # short window: tail slots empty
+    want = [int(ix[b, int(np.argmax(al[b]))]) for b in range(mb)]
+    assert want[1] == ix[1, 2] and want[3] == ix[3, 0] and want[4] == -1
+    assert o.attention_viterbi(al, ix).tolist() == want

@@ -40,7 +40,7 @@ SYMBOLS = [
     "zr_unstack_gates", "zr_lstm_stack_backward", "zr_lstm_weight_gradients", "zr_embed_gradient",
     "zr_softmax_backward", "zr_sgd_update", "zr_lstm_node_backward", "zr_lstm_node_gradients",
     "zr_softmax_backward_accumulate", "zr_gather_columns_multi", "zr_softmax_backward_loss",
-    "zr_softmax_forward_static", "zr_ctx_query", "zr_attn_prepare", "zr_lstm_step_embed",
+    "zr_softmax_forward_static", "zr_ctx_query", "zr_attn_prepare", "zr_lstm_step_embed", "zr_attn_viterbi",
 ]
 
 _lib = None
@@ -329,6 +329,9 @@ class Context:
 
     def attn_use_bf16_weights(self, a):
         _chk(load().zr_attn_use_bf16_weights(self.h, a))
+
+    def attn_viterbi(self, a, d_align, d_idx, d_out):
+        _chk(load().zr_attn_viterbi(self.h, a, _vp(d_align), _vp(d_idx), _vp(d_out)))
 
     def attn_prepare(self, a):
         _chk(load().zr_attn_prepare(self.h, a))

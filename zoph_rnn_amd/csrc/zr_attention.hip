@@ -311,6 +311,37 @@ attn_fused_kernel(const float* const* __restrict__ table, int longest_sent, cons
   }
 }
 
+// get_viterbi_alignment_kernel (src/custom_kernels.h:1623-1635): per column, the source position of the window slot with
+// the largest alignment weight.  The reference scans the slots in order with a running maximum that starts at -1 and
+// is replaced only by a strictly larger weight, so the first of equal maxima wins, and a column whose weights are all
+// zero reports the index of its first slot (-1 when the column is masked).  One wave per column: every lane scans its
+// slots in order, then the lanes' (weight, slot) pairs are merged, larger weight first and lower slot on a tie.
+__global__ void __launch_bounds__(64)
+attn_viterbi_kernel(const float* __restrict__ align, const int* __restrict__ indices, int mb, int W,
+                    int* __restrict__ out) {
+  const int b = blockIdx.x;
+  const int lane = threadIdx.x;
+  float best = -1.0f;
+  int slot = 0x7fffffff;
+  for (int j = lane; j < W; j += 64) {
+    const float a = align[b + (size_t)mb * j];
+    if (best < a) {
+      best = a;
+      slot = j;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ob = __shfl_xor(best, off, 64);
+    const int os = __shfl_xor(slot, off, 64);
+    if (ob > best || (ob == best && os < slot)) {
+      best = ob;
+      slot = os;
+    }
+  }
+  if (lane == 0) out[b] = slot == 0x7fffffff ? -1 : indices[b + (size_t)mb * slot];
+}
+
 // Sum over the 64 lanes of each of N values held one per register: lanes end up with the totals in all lanes.
 template <int N>
 __device__ __forceinline__ void wave_sum_many(float (&v)[N]) {
@@ -509,6 +540,17 @@ int zr_attn_use_bf16_weights(zr_ctx* ctx, zr_attn* a) {
     rc = zr_pack8_bf16_launch(ctx, src[i], H, H, H, ldp, H, a->d_bf16 + i * per, i == 1 ? 1 : 0);  // W_a transposed
     if (rc) return rc;
   }
+  return ZR_OK;
+}
+
+int zr_attn_viterbi(zr_ctx* ctx, const zr_attn* a, const float* d_alignments, const int* d_indices, int* d_viterbi) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(a != nullptr && d_viterbi != nullptr, "zr_attn_viterbi: null attention object or output");
+  const float* al = d_alignments ? d_alignments : a->d_align;
+  const int* ix = d_indices ? d_indices : a->d_idx;
+  attn_viterbi_kernel<<<a->mb, 64, 0, ctx->stream>>>(al, ix, a->mb, 2 * a->D + 1, d_viterbi);
+  ZR_LAUNCH_CHECK("attn_viterbi_kernel");
   return ZR_OK;
 }
 

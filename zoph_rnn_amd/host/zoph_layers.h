@@ -66,6 +66,8 @@ inline void refuse_backward_with_clip_cell(const char* who) {
 inline precision lower = -0.08f;
 inline precision upper = 0.08f;
 inline bool force_decode = false;
+inline bool unk_replacement = false;          // src/BZ_CUDA_UTIL.h:78: attention nodes also report Viterbi alignments
+inline std::vector<int> viterbi_alignments;   // src/BZ_CUDA_UTIL.h:82: per beam column, filled by attention_node::forward_prop
 inline std::mt19937 gen(1234);
 // No counterpart in the reference: when set before the layers are initialised / loaded, every matrix the matrix cores
 // stream (LSTM M / W_h / Q, attention W_a / W_p / W_c, softmax D) is snapshotted as bf16; the fp32 members stay as
@@ -91,11 +93,22 @@ struct global_params {  // src/global_params.h:61-299 (fields the layers use)
   int source_vocab_size = 0;
 };
 
+// The reference passes a cublasHandle_t& into the attention layer's constructors (src/attention_layer.h:118-119,143-144);
+// the handle of this library is the context, which owns the stream the layer's work is queued on.
+typedef zr_ctx* cublasHandle_t;
+
 template <typename dType>
-struct neuralMT_model {  // only the flags the layers consult (src/model.h:37-217)
+struct neuralMT_model {  // only what the layers consult (src/model.h:37-217)
   bool train = false;
   bool decode = false;
   attention_params attent_params;
+  // What attention_layer's constructor reads from the model (src/attention_layer.hpp:106-160): the source side's
+  // top-layer node states, entry t = d_h_t of node t of the last source layer (model->source_hidden_layers.back().nodes[t]
+  // or model->input_layer_source.nodes[t] in the reference).  The owner of the layers fills it before constructing the
+  // attention layer.
+  std::vector<const dType*> source_top_h_t;
+  // src/model.h:107: the decoder's copies of the source states, one LSTM_size x beam matrix per source position
+  std::vector<dType*> top_source_states;
 };
 
 // One context per GPU (layer_gpu_info::init, src/gpu_info_struct.h:67-172).
@@ -238,11 +251,64 @@ class attention_layer {  // src/attention_layer.h:14-143
   int* d_batch_info = nullptr;
   std::vector<const dType*> h_total_hs_mat;  // host copy of d_total_hs_mat (src/attention_layer.hpp:106-160)
   zr_attn* attn = nullptr;
+  int* d_viterbi_alignments = nullptr;  // minibatch_size ints, allocated when BZ_CUDA::unk_replacement is set
+  int* d_ones_minibatch_int = nullptr;  // init_att_decoder: the decode path runs every column with mask 1
+  neuralMT_model<dType>* model = nullptr;
   std::vector<attention_node<dType>> nodes;
+
+  attention_layer() {}
+
+  // The reference's own parameter list (src/attention_layer.h:118-119, body src/attention_layer.hpp:3-173).  `handle`
+  // is the context (cublasHandle_t above); the source states come from model->source_top_h_t.  Gradient clipping
+  // parameters are accepted and unused (this layer has no backward pass); dropout and the second source side of a
+  // multi-source model are not built and are refused.
+  attention_layer(int LSTM_size, int minibatch_size, int device_number, int D, int longest_sent, cublasHandle_t& handle,
+                  neuralMT_model<dType>* model, bool feed_input, bool /*clip_gradients*/, dType /*norm_clip*/,
+                  bool dropout, dType /*dropout_rate*/, global_params& /*params*/, bool bi_side) {
+    if (dropout || bi_side || !model || (int)model->source_top_h_t.size() < longest_sent) {
+      std::fprintf(stderr, "Error: attention_layer: dropout and multi-source attention are not built, and the model "
+                   "must list its %d source top-layer states in source_top_h_t\n", longest_sent);
+      std::exit(EXIT_FAILURE);
+    }
+    layer_gpu_info gpu;
+    gpu.device_number = device_number;
+    gpu.ctx = handle;
+    this->model = model;
+    setup(LSTM_size, minibatch_size, device_number, D, longest_sent, gpu, model->source_top_h_t, feed_input, longest_sent);
+  }
 
   // src/attention_layer.hpp:3-173.  total_hs: the source top-layer node states, entry t = node t's d_h_t.
   attention_layer(int LSTM_size, int minibatch_size, int device_number, int D, int longest_sent,
                   const layer_gpu_info& gpu, const std::vector<const dType*>& total_hs, bool feed_input) {
+    setup(LSTM_size, minibatch_size, device_number, D, longest_sent, gpu, total_hs, feed_input, longest_sent);
+  }
+
+  // The decode-time layer (src/attention_layer.h:143-144, body src/attention_layer.hpp:176-259): minibatch = beam, ONE
+  // node whose mask is all ones, source states read from top_source_states (the decoder's LSTM_size x beam copies,
+  // src/model.hpp:565-583).  feed_input is always false here as in the reference: the decode driver moves h~ itself.
+  // multi_attention_v2 is not built.
+  void init_att_decoder(int LSTM_size, int beam_size, int device_number, int D, int longest_sent, cublasHandle_t& handle,
+                        neuralMT_model<dType>* model, bool feed_input, std::vector<dType*>& top_source_states,
+                        bool multi_attention_v2, std::vector<dType*>& /*top_source_states_v2*/) {
+    if (multi_attention_v2 || (int)top_source_states.size() < longest_sent) {
+      std::fprintf(stderr, "Error: init_att_decoder: multi_attention_v2 is not built, and top_source_states must hold "
+                   "%d matrices\n", longest_sent);
+      std::exit(EXIT_FAILURE);
+    }
+    layer_gpu_info gpu;
+    gpu.device_number = device_number;
+    gpu.ctx = handle;
+    this->model = model;
+    std::vector<const dType*> total_hs(top_source_states.begin(), top_source_states.begin() + longest_sent);
+    setup(LSTM_size, beam_size, device_number, D, longest_sent, gpu, total_hs, feed_input, 1);
+    std::vector<int> ones((size_t)beam_size, 1);
+    ZOPH_CALL(zr_malloc(gpu.ctx, ones.size() * sizeof(int), (void**)&d_ones_minibatch_int));
+    ZOPH_CALL(zr_h2d(gpu.ctx, d_ones_minibatch_int, ones.data(), ones.size() * sizeof(int)));
+    nodes[0].d_indicies_mask = &d_ones_minibatch_int;
+  }
+
+  void setup(int LSTM_size, int minibatch_size, int device_number, int D, int longest_sent, const layer_gpu_info& gpu,
+             const std::vector<const dType*>& total_hs, bool feed_input, int n_nodes) {
     this->LSTM_size = LSTM_size;
     this->minibatch_size = minibatch_size;
     this->device_number = device_number;
@@ -266,7 +332,11 @@ class attention_layer {  // src/attention_layer.h:14-143
       ZOPH_CALL(zr_attn_use_bf16_weights(ctx, attn));
     else
       ZOPH_CALL(zr_attn_prepare(ctx, attn));
-    for (int i = 0; i < longest_sent; i++)
+    if (BZ_CUDA::unk_replacement) {  // src/attention_layer.hpp:252-255
+      ZOPH_CALL(zr_malloc(ctx, (size_t)minibatch_size * sizeof(int), (void**)&d_viterbi_alignments));
+      BZ_CUDA::viterbi_alignments.assign((size_t)minibatch_size, -1);
+    }
+    for (int i = 0; i < n_nodes; i++)
       nodes.push_back(attention_node<dType>(LSTM_size, minibatch_size, device_number, D, feed_input, this, i));
   }
   // src/attention_layer.hpp:580-583
@@ -325,6 +395,12 @@ void attention_node<dType>::forward_prop() {
   zr_ctx* ctx = attent_layer->layer_info.ctx;
   ZOPH_CALL(zr_attn_step(ctx, attent_layer->attn, attent_layer->d_batch_info, d_h_t, *d_indicies_mask, d_final_temp_2,
                          d_alignments, d_indicies, d_p_t, d_c_t));
+  if (BZ_CUDA::unk_replacement && attent_layer->d_viterbi_alignments) {  // src/attention_node.hpp:225-234
+    ZOPH_CALL(zr_attn_viterbi(ctx, attent_layer->attn, d_alignments, d_indicies, attent_layer->d_viterbi_alignments));
+    BZ_CUDA::viterbi_alignments.resize((size_t)minibatch_size);
+    ZOPH_CALL(zr_d2h(ctx, BZ_CUDA::viterbi_alignments.data(), attent_layer->d_viterbi_alignments,
+                     (size_t)minibatch_size * sizeof(int)));
+  }
   // feed-input: h~ goes to the next time step's bottom node (src/attention_node.hpp:384-386)
   if (feed_input && index != (attent_layer->longest_sent - 1) && d_lower_htild)
     ZOPH_CALL(zr_d2d(ctx, d_lower_htild, d_final_temp_2, (size_t)LSTM_size * minibatch_size * sizeof(dType)));
@@ -664,6 +740,24 @@ class LSTM_IH_Node {  // src/LSTM.h:19-106
   void send_h_t_above();
 };
 
+// Device copy of a host index vector for swap_states_decoding: the reference hands over an Eigen vector
+// (const Eigen::MatrixBase<Derived>&, src/Input_To_Hidden_Layer.h:345); anything indexable with (i) or [i] that holds
+// minibatch_size entries is accepted here.
+namespace zoph_detail {
+template <typename V>
+auto index_at(const V& v, int i, int) -> decltype((int)v(i)) { return (int)v(i); }
+template <typename V>
+auto index_at(const V& v, int i, long) -> decltype((int)v[i]) { return (int)v[i]; }
+template <typename V>
+inline int* upload_indices(zr_ctx* ctx, const V& indicies, int n, int** d_cache) {
+  std::vector<int> h((size_t)n);
+  for (int i = 0; i < n; i++) h[(size_t)i] = index_at(indicies, i, 0);
+  if (!*d_cache) ZOPH_CALL(zr_malloc(ctx, (size_t)n * sizeof(int), (void**)d_cache));
+  ZOPH_CALL(zr_h2d(ctx, *d_cache, h.data(), (size_t)n * sizeof(int)));
+  return *d_cache;
+}
+}  // namespace zoph_detail
+
 // ------------------------------------------------------------------------------------------------ layers
 template <typename dType>
 class Hidden_To_Hidden_Layer : public lstm_layer_training<dType> {  // src/Hidden_To_Hidden_Layer.h:12-313
@@ -806,6 +900,13 @@ class Hidden_To_Hidden_Layer : public lstm_layer_training<dType> {  // src/Hidde
     nodes[0].d_h_t_prev = d_init_hidden_vector;
     nodes[0].d_c_t_prev = d_init_cell_vector;
   }
+  // the reference's own parameter list (src/Hidden_To_Hidden_Layer.h:282): a host-side index vector
+  int* d_swap_indices = nullptr;
+  template <typename IndexVector>
+  void swap_states_decoding(const IndexVector& indicies, int index, dType* d_temp_swap_vals) {
+    swap_states_decoding((const int*)zoph_detail::upload_indices(hh_layer_info.ctx, indicies, minibatch_size, &d_swap_indices),
+                         index, d_temp_swap_vals);
+  }
   // src/Hidden_To_Hidden_Layer.hpp (init_attention): the top target layer owns the attention layer
   void init_attention(attention_layer<dType>* layer) {
     attent_layer = layer;
@@ -814,6 +915,14 @@ class Hidden_To_Hidden_Layer : public lstm_layer_training<dType> {  // src/Hidde
       attent_layer->nodes[i].d_indicies_mask = &nodes[i].d_input_vocab_indices_01;
       attent_layer->nodes[i].d_h_t = nodes[i].d_h_t;
     }
+  }
+  // The reference's own parameter list (src/Hidden_To_Hidden_Layer.h:290, body src/Hidden_To_Hidden_Layer.hpp:160-186):
+  // the layer builds its attention layer itself, from the model's source states (model->source_top_h_t).
+  void init_attention(int device_number, int D, bool feed_input, neuralMT_model<dType>* model, global_params& params) {
+    cublasHandle_t handle = hh_layer_info.ctx;
+    init_attention(new attention_layer<dType>(LSTM_size, minibatch_size, device_number, D, longest_sent, handle, model,
+                                              feed_input, this->clip_gradients, this->norm_clip, false, (dType)0, params,
+                                              false));
   }
 };
 
@@ -953,6 +1062,21 @@ class Input_To_Hidden_Layer : public lstm_layer_training<dType> {  // src/Input_
       attent_layer->nodes[i].d_indicies_mask = &nodes[i].d_input_vocab_indices_01;
       attent_layer->nodes[i].d_h_t = nodes[i].d_h_t;
     }
+  }
+  // The reference's own parameter list (src/Input_To_Hidden_Layer.h:353, body src/Input_To_Hidden_Layer.hpp:230-260):
+  // the layer builds its attention layer itself, from the model's source states (model->source_top_h_t).
+  void init_attention(int device_number, int D, bool feed_input, neuralMT_model<dType>* model, global_params& params) {
+    cublasHandle_t handle = ih_layer_info.ctx;
+    init_attention(new attention_layer<dType>(LSTM_size, minibatch_size, device_number, D, longest_sent, handle, model,
+                                              feed_input, this->clip_gradients, this->norm_clip, false, (dType)0, params,
+                                              false));
+  }
+  // the reference's own parameter list (src/Input_To_Hidden_Layer.h:345): a host-side index vector
+  int* d_swap_indices = nullptr;
+  template <typename IndexVector>
+  void swap_states_decoding(const IndexVector& indicies, int index, dType* d_temp_swap_vals) {
+    swap_states_decoding((const int*)zoph_detail::upload_indices(ih_layer_info.ctx, indicies, minibatch_size, &d_swap_indices),
+                         index, d_temp_swap_vals);
   }
   // model-file order (src/Input_To_Hidden_Layer.hpp:1050-1159)
   void dump_weights(std::ofstream& output) {

@@ -440,15 +440,17 @@ class forward_model {
     if (seq2seq) wire(input_layer_source, source_hidden_layers, true);
     wire(input_layer_target, target_hidden_layers, false);
     if (params.attent_params.attention_model) {
-      std::vector<const dType*> total_hs(longest_sent);
+      // the top target layer builds the attention layer from the model's source states, as in the reference
+      // (src/model.hpp:330-345: init_attention(device, D, feed_input, this, params))
+      flags.source_top_h_t.resize(longest_sent);
       for (int i = 0; i < longest_sent; i++)
-        total_hs[i] = (L == 1) ? input_layer_source.nodes[i].d_h_t : source_hidden_layers[L - 2].nodes[i].d_h_t;
-      att = new attention_layer<dType>(H, minibatch_size, 0, attention_D, longest_sent, gpu, total_hs,
-                                       params.attent_params.feed_input);
+        flags.source_top_h_t[i] = (L == 1) ? input_layer_source.nodes[i].d_h_t : source_hidden_layers[L - 2].nodes[i].d_h_t;
+      params.attent_params.D = attention_D;
       if (L == 1)
-        input_layer_target.init_attention(att);
+        input_layer_target.init_attention(0, attention_D, params.attent_params.feed_input, &flags, params);
       else
-        target_hidden_layers[L - 2].init_attention(att);
+        target_hidden_layers[L - 2].init_attention(0, attention_D, params.attent_params.feed_input, &flags, params);
+      att = (L == 1) ? input_layer_target.attent_layer : target_hidden_layers[L - 2].attent_layer;
       if (params.attent_params.feed_input)
         input_layer_target.init_feed_input(L == 1 ? nullptr : &target_hidden_layers[L - 2], false);
     }
