@@ -51,16 +51,22 @@ constexpr int KMAX = 32;  // beam + 1 <= KMAX
 // Stage 1 (beam_topk_kernel): grid (chunks, columns).  A workgroup takes up to kTopkChunk consecutive words of a
 // column into registers with 16-byte loads (one pass over HBM, no value-dependent work per element).  The K-th
 // largest of a set of per-thread maxima, tau, is a lower bound of the chunk's K-th largest key, so the chunk's K best
-// are among the elements with key >= tau; those are appended to a list in LDS.  tau is first taken per wave (64
-// broadcast reads from LDS) and the largest of the four used; should the list overflow, tau is recomputed over all 256 maxima:
-// then at most K-1 threads have a maximum above tau, each holds 4*kTopkE4 elements, and one thread's maximum equals
-// tau, so the list cannot exceed (K-1)*4*kTopkE4 + 1 entries whatever the data.  Each listed element then counts the
+// are among the elements with key >= tau; those are appended to a list in LDS.  tau is first taken per wave on the
+// probabilities alone (a cross-lane sort of the 64 thread maxima) and the largest of the four used; should the list
+// overflow, tau is recomputed over all 256 maxima as full keys: then at most K-1 threads have a maximum above tau, each
+// holds 4*E4 elements, and one thread's maximum equals tau, so the list cannot exceed (K-1)*4*E4 + 1 entries whatever
+// the data.  Each listed element then counts the
 // listed keys above its own: that count is its rank, and ranks below K are written out in place.
 // Stage 2 (beam_topk_merge_kernel): one workgroup per column ranks the chunks' K-lists the same way.
-constexpr int kTopkE4 = 16;                        // 16-byte loads per thread
-constexpr int kTopkChunk = 256 * 4 * kTopkE4;      // words per workgroup
-constexpr int kTopkCap = (KMAX - 1) * 4 * kTopkE4 + 64;  // candidate list capacity
-constexpr int kMaxChunks = 64;                     // vocabulary up to kMaxChunks * kTopkChunk words
+// Words per workgroup = 1024 * E4 (E4 16-byte loads per thread).  8192-word chunks measured best at 192 columns of
+// 50 000 words (12.9 us against 14.2 with 16384 and 18.6 with 4096: every workgroup of the launch is resident at once
+// and they load, then select, in step, so what counts is the length of one workgroup's chain of phases);
+// vocabularies beyond kMaxChunks small chunks take the large ones.
+constexpr int kTopkE4Small = 8, kTopkE4Large = 16;
+constexpr int kMaxChunks = 64;                     // K-lists per column the merge stage holds
+constexpr int topk_chunk(int e4) { return 256 * 4 * e4; }
+constexpr int topk_cap(int e4) { return (KMAX - 1) * 4 * e4 + 64; }  // candidate list capacity
+inline int topk_e4_for(int vocab) { return vocab > kMaxChunks * topk_chunk(kTopkE4Small) ? kTopkE4Large : kTopkE4Small; }
 
 __device__ __forceinline__ unsigned long long topk_key(float p, int w) {
   unsigned u = __float_as_uint(p);
@@ -80,9 +86,11 @@ __device__ __forceinline__ void topk_unkey(unsigned long long key, float& p, int
   w = 0x7fffffff - (int)(unsigned)(key & 0xffffffffu);
 }
 
+template <int kTopkE4>
 __global__ void __launch_bounds__(256)
 beam_topk_kernel(const float* __restrict__ prob, int V, int K, int n_chunks, float* __restrict__ part_p,
                  int* __restrict__ part_w) {
+  constexpr int kTopkChunk = topk_chunk(kTopkE4), kTopkCap = topk_cap(kTopkE4);
   __shared__ unsigned long long s_max[256];
   __shared__ unsigned long long s_cand[kTopkCap];
   __shared__ unsigned long long s_tau_wave[4];
@@ -118,41 +126,38 @@ beam_topk_kernel(const float* __restrict__ prob, int V, int K, int n_chunks, flo
       }
     }
   }
-  // this thread's best element: words are visited in ascending order, so a strict comparison keeps the lowest id
+  // The kernel is bound by vector instructions, not by memory: everything per element is kept to a compare or less.
+  // This thread's largest probability (NaN never wins a maximum), as an order-preserving 32-bit pattern; 0 = none.
   float bm = -INFINITY;
-  int bv = 0x7fffffff;
 #pragma unroll
-  for (int i = 0; i < kTopkE4; ++i)
-#pragma unroll
-    for (int c = 0; c < 4; ++c)
-      if (x[4 * i + c] > bm) {
-        bm = x[4 * i + c];
-        bv = v_begin + 4 * (tid + 256 * i) + c;
-      }
-  const unsigned long long mine = bm > -INFINITY ? topk_key(bm, bv) : 0ull;
-  s_max[tid] = mine;
-  __syncthreads();
-  // First bound: the K-th largest maximum inside each wave (its 64 entries of s_max, broadcast reads), then the
-  // largest of the four.
+  for (int i = 0; i < kTopkE4; ++i) bm = fmaxf(bm, fmaxf(fmaxf(x[4 * i], x[4 * i + 1]), fmaxf(x[4 * i + 2], x[4 * i + 3])));
+  const unsigned mu = bm > -INFINITY ? (unsigned)(topk_key(bm, 0) >> 32) : 0u;
+  // First bound, on the probabilities alone: the K-th largest thread maximum inside each wave (a bitonic sort of the
+  // 64 lanes' values, 21 exchange steps), then the largest of the four waves' bounds.  The K-th largest of any set of
+  // group maxima is a lower bound of the chunk's K-th largest element, so everything at or above it is listed -- with
+  // equal probabilities around the bound that is a few more elements than the exact rule needs, and if the list
+  // overflows the exact bound below takes over.
   {
-    const unsigned long long* wmax = s_max + 64 * wave;
-    int rank = 0;
-#pragma unroll 16
-    for (int j = 0; j < 64; ++j) {
-      const unsigned long long o = wmax[j];
-      rank += (o > mine || (o == mine && j < lane)) ? 1 : 0;
-    }
-    if (rank == K - 1) s_tau_wave[wave] = mine;
+    unsigned v = mu;
+#pragma unroll
+    for (int k = 2; k <= 64; k <<= 1)
+#pragma unroll
+      for (int j = k >> 1; j > 0; j >>= 1) {
+        const unsigned o = (unsigned)__shfl_xor((int)v, j, 64);
+        const bool keep_max = ((lane & j) == 0) == ((lane & k) == 0);
+        v = keep_max ? (v > o ? v : o) : (v < o ? v : o);
+      }
+    if (lane == K - 1) s_tau_wave[wave] = (unsigned long long)v << 32;  // lowest key of that probability
   }
   __syncthreads();
   unsigned long long tau = s_tau_wave[0];
 #pragma unroll
   for (int w = 1; w < 4; ++w) tau = s_tau_wave[w] > tau ? s_tau_wave[w] : tau;
   auto collect = [&](unsigned long long t) {
-    if (mine >= t && mine != 0ull) {
-      float tp;
-      int tw;
-      topk_unkey(t, tp, tw);
+    float tp;
+    int tw;
+    topk_unkey(t, tp, tw);
+    if (bm >= tp && mu != 0u) {
 #pragma unroll
       for (int i = 0; i < kTopkE4; ++i)
 #pragma unroll
@@ -171,8 +176,18 @@ beam_topk_kernel(const float* __restrict__ prob, int V, int K, int n_chunks, flo
   collect(tau);
   __syncthreads();
   if (s_count > kTopkCap) {
-    // The wave-level bound let too many elements through (possible only when several waves hold threads whose whole
-    // share is large).  The K-th largest of all 256 maxima bounds the list by (K-1) * 4*kTopkE4 + 1 whatever the data.
+    // The wave-level bound let too many elements through (several waves holding threads whose whole share is large, or
+    // many equal probabilities at the bound).  The K-th largest of all 256 thread maxima as full keys (probability,
+    // then lower word id) bounds the list by (K-1) * 4*kTopkE4 + 1 entries whatever the data.
+    int bv = 0x7fffffff;
+#pragma unroll
+    for (int i = kTopkE4 - 1; i >= 0; --i)
+#pragma unroll
+      for (int c = 3; c >= 0; --c)
+        if (x[4 * i + c] == bm) bv = v_begin + 4 * (tid + 256 * i) + c;  // descending scan: the lowest id stays
+    const unsigned long long mine = mu != 0u ? topk_key(bm, bv) : 0ull;
+    s_max[tid] = mine;
+    __syncthreads();
     int rank = 0;
     for (int j = 0; j < 256; ++j) {
       const unsigned long long o = s_max[j];
@@ -407,7 +422,9 @@ int zr_beam_create(zr_ctx* ctx, int beam, int vocab, int n_sent, int max_len, fl
   *out = nullptr;
   ZR_CHECK_ARG(beam >= 1 && beam + 1 <= KMAX, "zr_beam_create: beam = %d not in [1, %d]", beam, KMAX - 1);
   ZR_CHECK_ARG(n_sent * beam <= 65535, "zr_beam_create: more than 65535 columns");
-  ZR_CHECK_ARG(vocab <= kMaxChunks * kTopkChunk, "zr_beam_create: vocab = %d exceeds %d", vocab, kMaxChunks * kTopkChunk);
+  ZR_CHECK_ARG(vocab <= kMaxChunks * topk_chunk(kTopkE4Large), "zr_beam_create: vocab = %d exceeds %d", vocab,
+               kMaxChunks * topk_chunk(kTopkE4Large));
+  const int kTopkChunk = topk_chunk(topk_e4_for(vocab));
   ZR_CHECK_ARG(vocab > beam + 1 && n_sent >= 1 && max_len >= 3, "zr_beam_create: vocab = %d, n_sent = %d, max_len = %d",
                vocab, n_sent, max_len);
   // the reference caps the beam at floor(sqrt(V)) (src/ensemble_factory.hpp:19-21)
@@ -485,9 +502,13 @@ int zr_beam_expand(zr_ctx* ctx, zr_beam* b, const float* d_prob, int index, int*
   ZR_CHECK_ARG(index >= 0, "zr_beam_expand: index = %d", index);
   ZR_CHECK_ARG(b->current_index + 2 < b->max_len, "zr_beam_expand: hypotheses reached max_len = %d", b->max_len);
   const int K = b->beam + 1;
-  const int n_chunks = (b->vocab + kTopkChunk - 1) / kTopkChunk;
+  const int e4 = topk_e4_for(b->vocab);
+  const int n_chunks = (b->vocab + topk_chunk(e4) - 1) / topk_chunk(e4);
   dim3 tgrid(n_chunks, b->n_sent * b->beam);
-  beam_topk_kernel<<<tgrid, 256, 0, ctx->stream>>>(d_prob, b->vocab, K, n_chunks, b->d_part_p, b->d_part_w);
+  if (e4 == kTopkE4Small)
+    beam_topk_kernel<kTopkE4Small><<<tgrid, 256, 0, ctx->stream>>>(d_prob, b->vocab, K, n_chunks, b->d_part_p, b->d_part_w);
+  else
+    beam_topk_kernel<kTopkE4Large><<<tgrid, 256, 0, ctx->stream>>>(d_prob, b->vocab, K, n_chunks, b->d_part_p, b->d_part_w);
   ZR_LAUNCH_CHECK("beam_topk_kernel");
   beam_topk_merge_kernel<<<b->n_sent * b->beam, 256, 0, ctx->stream>>>(b->d_part_p, b->d_part_w, K, n_chunks,
                                                                        b->d_cand_p, b->d_cand_w);
