@@ -151,9 +151,27 @@ def _expand_given(ctx, Ps, beam, n_sent, max_len):
     ctx.beam_destroy(b)
 
 
-@pytest.mark.parametrize("V,beam", [(40003, 12), (16384, 5), (16385, 31), (70000, 20)])
+@pytest.mark.parametrize("V", [20000, 8192 * 3 + 5, 600000])
+def test_beam_all_equal_probabilities_large_vocab(ctx, V):
+    """Every word equally probable, over several chunks of the selection kernel (and, at 600 000 words, over its large
+    chunks): the probability-only bound of the first stage lets every element through, the candidate list overflows
+    and the exact bound takes over.  Equal probabilities rank by lower word id, so the beam + 1 kept words are
+    0..beam: <START> is skipped, <EOF> finishes a hypothesis, words 2..beam survive and the last slot stays empty."""
+    beam = 12
+    b = ctx.beam_create(beam, V, 1, 6)
+    d_words, d_back = ctx.empty(beam, np.int32), ctx.empty(beam, np.int32)
+    ctx.beam_expand(b, ctx.array(np.full((V, beam), np.float32(1.0 / V), np.float32, order="F")), 0, d_words, d_back)
+    ctx.sync()
+    w = d_words.get()
+    assert sorted(w[:beam - 1].tolist()) == list(range(2, beam + 1)) and w[beam - 1] == -1
+    hyps, n = ctx.beam_hypotheses(b, 0, cap=4, max_len=6)
+    assert n == 1 and hyps[0][0].tolist() == [0, 1]
+    ctx.beam_destroy(b)
+
+
+@pytest.mark.parametrize("V,beam", [(40003, 12), (16384, 5), (16385, 31), (70000, 20), (8193, 12)])
 def test_beam_selection_on_adversarial_layouts(ctx, V, beam):
-    """Layouts chosen against the selection kernel's structure (one workgroup per 16384 words, each thread holding
+    """Layouts chosen against the selection kernel's structure (one workgroup per 8192 or 16384 words, each thread holding
     words 4t..4t+3 of every 1024): the largest values all inside one thread's share, at chunk boundaries, in the
     ragged tail, and values that fall steadily with the word id; vocabulary sizes that are not multiples of 4 take the scalar-load path."""
     g = synth.rng(43, V)
@@ -168,7 +186,8 @@ def test_beam_selection_on_adversarial_layouts(ctx, V, beam):
     a[idx, :] += 1.0 + g.random((idx.size, cols))
     P.append(a)
     a = base.copy()                                    # step 1: big values around chunk boundaries and the tail
-    edge = np.array([v for v in (16383, 16384, 16385, 32767, 32768, V - 1, V - 2, V - 3, 2, 3) if 1 < v < V])
+    edge = np.array([v for v in (8191, 8192, 16383, 16384, 16385, 32767, 32768, V - 1, V - 2, V - 3, 2, 3)
+                     if 1 < v < V and (v > 8192 or V < 16384)])  # (the 8192 boundary only in the case added for it)
     a[edge, :] += 1.0 + g.random((edge.size, cols))
     P.append(a)
     a = base.copy()                                    # step 2: values falling with the word id
