@@ -432,6 +432,15 @@ def main():
         c5["weights"] = "bf16 storage (LSTM, attention projections, output layer), fp32 activations split in two bf16 terms, fp32 accumulation"
         extra["config5_decoder_step_bf16_weights"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in c5.items()}
         log("config5:", extra["config5_decoder_step_bf16_weights"])
+        from zoph_rnn_amd import capi as _capi
+        ctx.set_option(_capi.ZR_OPT_BF16_ACTIVATION_TERMS, 1)
+        try:
+            c5s = bench_decoder_step(ctx, max(3, args.steps // 2), 2, H=2000, mb=256, V=80000, bf16=True)
+        finally:
+            ctx.set_option(_capi.ZR_OPT_BF16_ACTIVATION_TERMS, 2)
+        c5s["weights"] = "bf16 storage, activations rounded to bf16 once (single-term mode), fp32 accumulation"
+        extra["config5_decoder_step_bf16_single_term"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in c5s.items()}
+        log("config5 single-term:", extra["config5_decoder_step_bf16_single_term"])
         extra["lm_training_step"] = bench_training_step(ctx, max(2, args.steps // 6))
         log("training step:", extra["lm_training_step"])
         extra["hbm_kernels"] = bench_hbm_kernels(ctx, args.steps)

@@ -91,6 +91,12 @@ const char* zr_version(void);
 #define ZR_OPT_LSTM_SWEEP_SPIN 8     /* polls a workgroup of that launch spends on one wait before it gives up
                                         (0 = default, about a second); giving up is reported by zr_ctx_sync */
 
+#define ZR_OPT_BF16_ACTIVATION_TERMS 9 /* products against bf16 weights (zr_lstm_pack_weights_bf16, zr_softmax_prepare_bf16,
+                                        zr_attn_use_bf16_weights): 2 (default) = every fp32 activation enters as two
+                                        bf16 terms (hi + lo: fp32-level accuracy, two matrix instructions per 16 k);
+                                        1 = activations rounded to bf16 once (relative error 2^-9 per activation, half
+                                        the matrix instructions and half the activation operand traffic) */
+
 /* full_matrix_setup / cudaMalloc / cudaMemcpy / cudaMemset call sites (src/BZ_CUDA_UTIL.h:358-399 and the
  * layer constructors, e.g. src/LSTM.hpp:23-42). */
 int zr_malloc(zr_ctx* ctx, size_t bytes, void** d_out);

@@ -304,3 +304,126 @@ def test_config5_decoder_step_reduced_vocab(ctx):
     ctx.softmax_release(dD)
     for ly in layers:
         ly.close()
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Single-term mode (ZR_OPT_BF16_ACTIVATION_TERMS = 1): every activation entering a product against bf16 weights is
+# rounded to bf16 once (round to nearest even) instead of being split into hi + lo.  Products of two bf16 numbers are
+# exact in fp32, so the mode has a sharp contract: it computes what the fp32 path computes on bf16-ROUNDED ACTIVATIONS
+# (and the same rounded weights), to the accumulation tolerance of the two-term mode.  Against the unrounded
+# activations the results move by about 2^-9 * |w| * |x| * sqrt(K) per pre-activation; the stated bound for h and the
+# logits at the benchmark's value ranges is 1e-2 absolute.
+# ---------------------------------------------------------------------------------------------------------------
+def _rb(a):
+    return np.asfortranarray(round_bf16(a))
+
+
+@pytest.fixture()
+def single_term(ctx):
+    ctx.set_option(capi.ZR_OPT_BF16_ACTIVATION_TERMS, 1)
+    yield ctx
+    ctx.set_option(capi.ZR_OPT_BF16_ACTIVATION_TERMS, 2)
+
+
+@pytest.mark.parametrize("H,mb,feed", [(64, 33, False), (112, 64, True), (496, 70, True), (2000, 256, True)])
+def test_single_term_lstm_step_is_the_fp32_path_on_rounded_activations(single_term, H, mb, feed):
+    ctx = single_term
+    g = synth.rng(91, H + mb)
+    ly, _ = _rounded_layer(g, H, feed)
+    x, hp, cp = U(g, (H, mb), -1, 1), U(g, (H, mb), -1, 1), U(g, (H, mb), -1, 1)
+    ht = U(g, (H, mb), -1, 1) if feed else None
+    mask = (g.random(mb) > 0.2).astype(np.int32)
+    layer = Layer(ctx, ly, bf16=True)
+    got = run_lstm_step(ctx, layer, x, hp, cp, mask, htild=ht, want_gates=True)
+    layer.close()
+    cols = np.arange(mb) if H < 1000 else np.array([0, 31, 32, 100, 255])
+    sub = lambda a: np.asfortranarray(a[:, cols])
+    # the cell state is not an operand of any product: it stays fp32
+    want = o.lstm_step(ly["M"], ly["Wh"], ly["b"], _rb(sub(x)), _rb(sub(hp)), sub(cp), mask[cols],
+                       Q=ly.get("Q") if feed else None, htild=_rb(sub(ht)) if feed else None)
+    for k in ("i", "f", "c_tilde", "o", "c", "h"):
+        close(got[k][:, cols], want[k], "single-term lstm %s" % k)
+    # and it is NOT the two-term result: the rounding of the activations is visible, inside the stated bound
+    exact = o.lstm_step(ly["M"], ly["Wh"], ly["b"], sub(x), sub(hp), sub(cp), mask[cols],
+                        Q=ly.get("Q") if feed else None, htild=sub(ht) if feed else None)
+    dev = np.abs(got["h"][:, cols].astype(np.float64) - exact["h"]).max()
+    assert 1e-6 < dev < 1e-2, dev
+
+
+@pytest.mark.parametrize("V,H,mb", [(1003, 48, 70), (9000, 112, 130), (12000, 48, 128), (40000, 64, 256)])
+def test_single_term_output_layer_is_the_fp32_path_on_rounded_activations(single_term, V, H, mb):
+    ctx = single_term
+    g = synth.rng(92, V + mb)
+    D = _rb(U(g, (V, H), -0.5, 0.5))
+    bd, h = U(g, (V,), -1, 1), U(g, (H, mb), -1, 1)
+    dD, dbd = ctx.array(D), ctx.array(bd)
+    ctx.softmax_prepare(dD, V, H, bf16=True)
+    d_lp, d_scr = ctx.empty((V, mb)), ctx.empty((V, mb))
+    ctx.softmax_forward(dD, dbd, V, H, ctx.array(h), mb, capi.ZR_SOFTMAX_LOGPROB, d_lp, d_scr)
+    ctx.sync()
+    ctx.softmax_release(dD)
+    logits = o.softmax_logits(D, bd, _rb(h))
+    close(d_scr.get(), logits, "single-term logits")
+    close(d_lp.get(), o.softmax_logprob_f64(logits), "single-term log-probs")
+    dev = np.abs(d_scr.get().astype(np.float64) - o.softmax_logits(D, bd, h)).max()
+    assert 1e-6 < dev < 2e-2, dev
+
+
+def test_single_term_stack_rounds_every_product_input(single_term):
+    """zr_lstm_stack_forward with bf16 weights in single-term mode against the oracle composed node by node with the
+    inputs of every product (embedding column or h from below, h from the step before) rounded to bf16 on use; what
+    is stored (h, c) stays fp32."""
+    ctx = single_term
+    H, mb, T, V, L = 96, 40, 5, 300, 2
+    cfg = synth.encoder_config(H=H, mb=mb, T=T, V=V, L=L)
+    for ly in cfg["layers"]:
+        for k in ("M", "Wh"):
+            ly[k] = [_rb(m) for m in ly[k]]
+    layers = [Layer(ctx, ly, bf16=True) for ly in cfg["layers"]]
+    ids = cfg["ids"]
+    d_nn, d_m = ctx.empty(ids.size, np.int32), ctx.empty(ids.size, np.int32)
+    ctx.vocab_prep(ctx.array(ids.reshape(-1)), ids.size, V, d_nn, d_m)
+    z = ctx.zeros((H, mb))
+    h_all = [ctx.empty((H * mb * T,)) for _ in range(L)]
+    c_all = [ctx.empty((H * mb * T,)) for _ in range(L)]
+    ctx.lstm_stack_forward([ly.w for ly in layers], ctx.array(cfg["embed"]), V, d_nn, d_m, T, mb, [z] * L, [z] * L,
+                           h_all, c_all)
+    ctx.sync()
+    nn, m = o.vocab_prep(ids)
+    hp = [np.zeros((H, mb), np.float32, order="F") for _ in range(L)]
+    cp = [np.zeros((H, mb), np.float32, order="F") for _ in range(L)]
+    for t in range(T):
+        below = o.embed_gather(cfg["embed"], nn[t])
+        for l in range(L):
+            ly = cfg["layers"][l]
+            r = o.lstm_step(ly["M"], ly["Wh"], ly["b"], _rb(below), _rb(hp[l]), cp[l], m[t])
+            got_h = h_all[l].get().reshape(T, mb, H).transpose(0, 2, 1)[t]
+            got_c = c_all[l].get().reshape(T, mb, H).transpose(0, 2, 1)[t]
+            close(got_h, r["h"], "single-term stack h layer %d step %d" % (l, t))
+            close(got_c, r["c"], "single-term stack c layer %d step %d" % (l, t))
+            # follow the device's own values so that the comparison of later nodes is not a comparison of drifts
+            hp[l], cp[l], below = np.asfortranarray(got_h), np.asfortranarray(got_c), np.asfortranarray(got_h)
+    for ly in layers:
+        ly.close()
+
+
+def test_single_term_attention_within_stated_bound(single_term):
+    """Attention with bf16 snapshots in single-term mode: window indices identical, h~ within the stated 1e-2."""
+    ctx = single_term
+    H, mb, S, D = 256, 40, 20, 10
+    g = synth.rng(93, 1)
+    w = synth.attention_weights(g, H)
+    for k in ("W_a", "W_p", "W_c1", "W_c2"):
+        w[k] = _rb(w[k])
+    hs = (g.standard_normal(size=(S, H, mb), dtype=np.float32) * np.float32(0.1))
+    lens = g.integers(3, S + 1, size=mb).astype(np.int32)
+    bi = np.concatenate([lens, S - lens]).astype(np.int32)
+    mask = np.ones(mb, np.int32)
+    h_t = U(g, (H, mb), -1, 1)
+    got = _run_attention_bf16(ctx, w, hs, bi, h_t, mask, D)
+    want = o.attention_forward(hs_table=hs, batch_info=bi, h_t=h_t, mask01=mask, D=D, **w)
+    frac = want["p_t"] - np.floor(want["p_t"])
+    safe = (frac > 2e-2) & (frac < 1 - 2e-2)
+    assert safe.sum() > mb // 2
+    assert np.array_equal(got["indices"][safe], want["indices"][safe])
+    assert np.abs(got["h_tild"][:, safe] - want["h_tild"][:, safe]).max() < 1e-2

@@ -20,6 +20,7 @@ ZR_OPT_LSTM_KERNEL = 5
 ZR_OPT_LSTM_KPARTS = 6
 ZR_OPT_LSTM_SWEEP = 7
 ZR_OPT_LSTM_SWEEP_SPIN = 8
+ZR_OPT_BF16_ACTIVATION_TERMS = 9
 ZR_QUERY_LSTM_STACK_PATH = 1
 ZR_QUERY_LSTM_SWEEP_ABANDONED = 2
 ZR_LSTM_STACK_PATH_SWEEP = 1

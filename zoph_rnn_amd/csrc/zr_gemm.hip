@@ -103,7 +103,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& a, int m0, int n0, boo
       const unsigned woffb = 16u * (unsigned)(m0 + jl + half * (int)a.lda[s]);
       zr_mma_segment_u<TM, TN, KS, PF>(acc, zr_make_rsrc(a.A[s]), wsoff, woffb, 32u * (unsigned)a.lda[s],
                                        zr_make_rsrc(a.B[s]), xoffb, 32u * (unsigned)a.N, a.K[s], kslice);
-    } else if constexpr (AMODE == ZR_A_PACK8_BF16) {
+    } else if constexpr (zr_is_bf16_mode(AMODE)) {
       const unsigned short* wbase[TM];
       unsigned woff[TM];
       const float* xcol[TN];
@@ -119,7 +119,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& a, int m0, int n0, boo
         xcol[tn] = (const float*)((const unsigned short*)a.B[s] + off);
         xlo[tn] = a.Blo[s] + off;
       }
-      zr_mma_segment_bf16<TM, TN, KS, PF, true>(acc, wbase, woff, a.lda[s], xcol, a.K[s], kslice, xlo, a.N);
+      zr_mma_segment_bf16<TM, TN, KS, PF, true, AMODE == ZR_A_PACK8_BF16>(acc, wbase, woff, a.lda[s], xcol, a.K[s], kslice,
+                                                                          xlo, a.N);
     } else {
       const float* A = (grpA ? grpA : a.A[s]) + (long long)z * a.strideA;
       const float* Bs = grpB ? grpB : a.B[s];
@@ -257,7 +258,7 @@ __global__ void __launch_bounds__(64 * KS * WPB, OCC) gemm_kernel(GemmArgs a) {
   const long long ntiles = (long long)a.m_tiles * a.n_tiles;
   bool active = tile < ntiles;
   int mt, nt;
-  if (AMODE == ZR_A_PACK4 || AMODE == ZR_A_PACK8_BF16) {
+  if (AMODE == ZR_A_PACK4 || zr_is_bf16_mode(AMODE)) {
     // Workgroup ids congruent modulo 8 run on the same XCD.  Each XCD gets a contiguous range of row tiles and
     // runs the column tiles of one row tile back to back (in neighbouring waves of a workgroup when WPB > 1), so a
     // weight tile leaves memory once.
@@ -274,7 +275,7 @@ __global__ void __launch_bounds__(64 * KS * WPB, OCC) gemm_kernel(GemmArgs a) {
     mt = (int)(tile % a.m_tiles);
     nt = (int)(tile / a.m_tiles);
   }
-  constexpr int PF = AMODE == ZR_A_PACK8_BF16 ? 4
+  constexpr int PF = zr_is_bf16_mode(AMODE) ? 4
                      : AMODE == ZR_A_PACK4    ? (OCC == 1 ? (TM + TN <= 4 ? 8 : 6) : (TM + TN == 4 ? 6 : 4))
                                               : zr_prefetch_depth(TM, TN);
   float* redp = KS > 1 ? red + (size_t)sub * KS * TN * 16 * 64 : red;
@@ -313,7 +314,7 @@ __global__ void __launch_bounds__(256) gemm_rows_kernel(GemmArgs a, int row_chun
   const int n0 = nt * 32 * TN;
   // at most 192 accumulator registers per wave: four blocks per pass up to 96 columns, three at 128
   constexpr int TMAX = TN <= 3 ? 4 : 3;
-  constexpr int PF4 = AMODE == ZR_A_PACK8_BF16 ? 2 : (TN <= 2 ? 6 : (TN == 3 ? 4 : 3));
+  constexpr int PF4 = zr_is_bf16_mode(AMODE) ? 2 : (TN <= 2 ? 6 : (TN == 3 ? 4 : 3));
   while (b < b_end) {
     const int nb = b_end - b < TMAX ? b_end - b : TMAX;  // uniform over the workgroup
     if (TMAX == 4 && nb == 4)
@@ -586,7 +587,7 @@ template <int TM, int TN, int KS, int WPB, int AMODE, bool VEC, int OCC = 1>
 int launch_epi(zr_ctx* ctx, const GemmArgs& ga, int batch, int epi) {
   long long ntiles = (long long)ga.m_tiles * ga.n_tiles;
   dim3 grid((unsigned)((ntiles + WPB - 1) / WPB), 1, batch);
-  if (AMODE == ZR_A_PACK4 || AMODE == ZR_A_PACK8_BF16) {
+  if (AMODE == ZR_A_PACK4 || zr_is_bf16_mode(AMODE)) {
     // XCD-major id space: 8 ranges of ceil(m_tiles/8) row tiles x n_tiles wave tiles, WPB wave tiles per workgroup
     const long long per_xcd = (long long)((ga.m_tiles + 7) / 8) * ga.n_tiles;
     grid.x = (unsigned)(((per_xcd + WPB - 1) / WPB) * 8);
@@ -706,7 +707,7 @@ __global__ void __launch_bounds__(256) zr_split_pack_x_kernel(const float* __res
   zr_split_bf16_pair(v1.z, v1.w, a, c); h.w = a; l.w = c;
   const long long o = ((long long)b * N + n) * 8;
   *(zr_u32x4*)(hi + o) = h;
-  *(zr_u32x4*)(lo + o) = l;
+  if (lo) *(zr_u32x4*)(lo + o) = l;  // null: single-term mode, the residues are dropped
 }
 
 __global__ void __launch_bounds__(256) pack4_kernel(const float* __restrict__ src, int M, int K, long long ld,
@@ -859,6 +860,7 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
   for (int s = 0; s < 3; ++s) ga.Blo[s] = nullptr;
   if (d.a_pack == 2) {
     ZR_CHECK_ARG(vec, "gemm: bf16 operand A needs 16-byte aligned activations with ldb %% 4 == 0");
+    const bool one_term = ctx->bf16_terms == 1;
     {
       // split the fp32 activations into bf16 hi + lo once, k-interleaved, instead of in every workgroup's K loop
       size_t elems = 0;
@@ -870,10 +872,12 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
       for (int s = 0; s < d.nseg; ++s) {
         const size_t e = (size_t)d.K[s] * d.N;
         const int n8 = (d.K[s] / 8) * d.N;
-        zr_split_pack_x_kernel<<<(n8 + 255) / 256, 256, 0, ctx->stream>>>(d.B[s], d.K[s], d.N, d.ldb[s], hi, hi + e);
+        const bool lo = !one_term;
+        zr_split_pack_x_kernel<<<(n8 + 255) / 256, 256, 0, ctx->stream>>>(d.B[s], d.K[s], d.N, d.ldb[s], hi,
+                                                                          lo ? hi + e : nullptr);
         ZR_LAUNCH_CHECK("zr_split_pack_x_kernel");
         ga.B[s] = (const float*)hi;
-        ga.Blo[s] = hi + e;
+        ga.Blo[s] = lo ? hi + e : nullptr;
         hi += 2 * e;
       }
     }
@@ -882,6 +886,11 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
       const int n32 = (d.N + 31) / 32;
       const int n_tiles = (n32 + 3) / 4;
       const int tn = (n32 + n_tiles - 1) / n_tiles;
+      if (one_term) {
+        if (tn <= 2) return launch_rows<2, ZR_A_PACK8_BF16_1T>(ctx, ga, d.epilogue, n_tiles);
+        if (tn == 3) return launch_rows<3, ZR_A_PACK8_BF16_1T>(ctx, ga, d.epilogue, n_tiles);
+        return launch_rows<4, ZR_A_PACK8_BF16_1T>(ctx, ga, d.epilogue, n_tiles);
+      }
       if (tn <= 2) return launch_rows<2, ZR_A_PACK8_BF16>(ctx, ga, d.epilogue, n_tiles);
       if (tn == 3) return launch_rows<3, ZR_A_PACK8_BF16>(ctx, ga, d.epilogue, n_tiles);
       return launch_rows<4, ZR_A_PACK8_BF16>(ctx, ga, d.epilogue, n_tiles);
@@ -889,10 +898,12 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
     if (d.N <= 32) {
       ga.m_tiles = (ga.M + 63) / 64;
       ga.n_tiles = (ga.N + 31) / 32;
+      if (one_term) return launch_epi<2, 1, 4, 1, ZR_A_PACK8_BF16_1T, true, 2>(ctx, ga, 1, d.epilogue);
       return launch_epi<2, 1, 4, 1, ZR_A_PACK8_BF16, true, 2>(ctx, ga, 1, d.epilogue);
     }
     ga.m_tiles = (ga.M + 63) / 64;
     ga.n_tiles = (ga.N + 63) / 64;
+    if (one_term) return launch_epi<2, 2, 4, 1, ZR_A_PACK8_BF16_1T, true, 2>(ctx, ga, 1, d.epilogue);
     return launch_epi<2, 2, 4, 1, ZR_A_PACK8_BF16, true, 2>(ctx, ga, 1, d.epilogue);
   }
   if (d.a_pack) {

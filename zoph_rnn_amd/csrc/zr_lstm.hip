@@ -40,6 +40,7 @@ struct LstmLaunch {
   LstmUnit u[kMaxUnits];
   int n_units;
   int bf16;                 // the weights of every unit are bf16 (zr_lstm_weights::bf16)
+  int bf16_single;          // bf16 weights: activations enter as one bf16 term instead of two
   int nseg_max;             // largest nseg among the units
   int H, mb;
   int ldw, kp;              // packed weight extents: rows per k-block (H up to 32), K (H up to 8), zero filled
@@ -69,7 +70,8 @@ constexpr int lstm_prefetch_depth(int tn, int ks) {
 // in part order -- the same order whoever is last, so results do not depend on timing -- and runs the cell epilogue.
 // BUF: operands are fetched with buffer loads (zr_mma_segment_u): fp32 weights, 16-byte aligned activations,
 // H % 8 == 0 and every operand array below 4 GiB (the host checks).
-template <int TN, int KS, bool VEC, bool BF16 = false, bool XPK = false, bool SPLIT = false, bool BUF = false>
+template <int TN, int KS, bool VEC, bool BF16 = false, bool XPK = false, bool SPLIT = false, bool BUF = false,
+          bool ONE_TERM = false>
 __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
   // Four waves at up to 64 columns (one workgroup per CU at these register counts anyway) sum their partial tiles in
   // one LDS round, which takes all 16 sub-tiles of every wave at once; the other shapes go gate by gate.
@@ -172,10 +174,12 @@ __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
           xcol[tn] = (const float*)((const unsigned short*)U.inp[s] + off);
           xlo[tn] = U.inp_lo[s] + off;
         }
-        zr_mma_segment_bf16<4, TN, KS, (TN == 1 ? 6 : 4), true>(acc, wbase, woff, (long long)L.ldw, xcol, H, kslice,
-                                                                 xlo, L.mb);
+        // ONE_TERM: single-term mode, activations rounded to bf16 once (no lo array)
+        zr_mma_segment_bf16<4, TN, KS, (TN == 1 ? 6 : 4), true, !ONE_TERM>(acc, wbase, woff, (long long)L.ldw, xcol, H,
+                                                                            kslice, xlo, L.mb);
       } else {
-        zr_mma_segment_bf16<4, TN, KS, (TN == 1 ? 6 : 4)>(acc, wbase, woff, (long long)L.ldw, xcol, H, kslice);
+        zr_mma_segment_bf16<4, TN, KS, (TN == 1 ? 6 : 4), false, !ONE_TERM>(acc, wbase, woff, (long long)L.ldw, xcol, H,
+                                                                             kslice);
       }
     } else if constexpr (BUF) {
       // k-groups [g0, g1) of this segment (all of them unless K is also split across workgroups)
@@ -820,9 +824,13 @@ int launch_fused_v(zr_ctx* ctx, const LstmLaunch& L, bool vec) {
     if constexpr (KS == 4 && TN <= 2) {
       bool xpk = true;  // every segment of every unit has pre-split inputs
       for (int i = 0; i < L.n_units; ++i)
-        for (int s2 = 0; s2 < L.u[i].nseg; ++s2) xpk = xpk && L.u[i].inp[s2] && L.u[i].inp_lo[s2];
-      if (xpk)
+        for (int s2 = 0; s2 < L.u[i].nseg; ++s2) xpk = xpk && L.u[i].inp[s2];  // (inp_lo null: single-term mode)
+      if (xpk && L.bf16_single)
+        lstm_fused_kernel<TN, KS, true, true, true, false, false, true><<<grid, 64 * KS, 0, ctx->stream>>>(L);
+      else if (xpk)
         lstm_fused_kernel<TN, KS, true, true, true><<<grid, 64 * KS, 0, ctx->stream>>>(L);
+      else if (L.bf16_single)
+        lstm_fused_kernel<TN, KS, true, true, false, false, false, true><<<grid, 64 * KS, 0, ctx->stream>>>(L);
       else
         lstm_fused_kernel<TN, KS, true, true><<<grid, 64 * KS, 0, ctx->stream>>>(L);
       ZR_LAUNCH_CHECK("lstm_fused_kernel (bf16 weights)");
@@ -1167,6 +1175,7 @@ static int lstm_step_impl(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_
   L.ldw = w->ldw;
   L.kp = w->kp;
   L.bf16 = w->bf16;
+  L.bf16_single = ctx->bf16_terms == 1;
   L.clip = clip_threshold;
   LstmUnit& U = L.u[0];
   U.W = w->d_W;
@@ -1191,10 +1200,11 @@ static int lstm_step_impl(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_
     if (rc) return rc;
     unsigned short* hi = (unsigned short*)p;
     for (int s = 0; s < nseg; ++s) {
-      rc = zr_split_pack_x_launch(ctx, U.in[s], H, mb, H, hi, hi + e);
+      const bool lo = ctx->bf16_terms != 1;
+      rc = zr_split_pack_x_launch(ctx, U.in[s], H, mb, H, hi, lo ? hi + e : nullptr);
       if (rc) return rc;
       U.inp[s] = (const float*)hi;
-      U.inp_lo[s] = hi + e;
+      U.inp_lo[s] = lo ? hi + e : nullptr;
       hi += 2 * e;
     }
   }
@@ -1323,6 +1333,7 @@ int zr_lstm_stack_forward_train(zr_ctx* ctx, int nl, const zr_lstm_weights* cons
     L.ldw = layers[0]->ldw;
     L.kp = layers[0]->kp;
     L.bf16 = layers[0]->bf16;
+    L.bf16_single = ctx->bf16_terms == 1;
     L.clip = clip_threshold;
     int nu = 0;
     for (int l = 0; l < nl; ++l) {

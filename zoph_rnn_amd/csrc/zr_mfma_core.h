@@ -493,7 +493,9 @@ __device__ __forceinline__ void zr_half_wave_softmax_stats(const float (&v)[G], 
 // k-interleaved like the weights ([K/8][N][8]); xcol[tn] / xlo[tn] then point at this lane's first block
 // (base + 8*(col + half*N)), xstride = N, and the loop body has no conversion arithmetic and only contiguous loads.
 // ---------------------------------------------------------------------------------------------------------
-enum { ZR_A_PACK8_BF16 = 3 };
+// ZR_A_PACK8_BF16_1T: the same weight layout in single-term mode (activations rounded to bf16 once, no lo array)
+enum { ZR_A_PACK8_BF16 = 3, ZR_A_PACK8_BF16_1T = 4 };
+constexpr bool zr_is_bf16_mode(int amode) { return amode == ZR_A_PACK8_BF16 || amode == ZR_A_PACK8_BF16_1T; }
 typedef __bf16 zr_bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 zr_bf16x2 __attribute__((ext_vector_type(2)));
 typedef unsigned zr_u32x4 __attribute__((ext_vector_type(4)));
@@ -518,7 +520,9 @@ struct ZrFragBf16 {
   zr_u32x4 w[TM];     // 8 consecutive k of this lane's row, bf16
 };
 
-template <int TM, int TN, int KS, int PF, bool XPK = false>
+// LO = false (with XPK): single-term mode -- only the hi halves are fetched and multiplied: every activation is
+// rounded to bf16 once (relative error 2^-9), half the matrix instructions and half the activation operand traffic.
+template <int TM, int TN, int KS, int PF, bool XPK = false, bool LO = true>
 __device__ __forceinline__ void zr_mma_segment_bf16(zr_f32x16 (&acc)[TM][TN], const unsigned short* const (&wbase)[TM],
                                                     const unsigned (&woff)[TM], long long lda,
                                                     const float* const (&xcol)[TN], int K, int kslice,
@@ -533,7 +537,7 @@ __device__ __forceinline__ void zr_mma_segment_bf16(zr_f32x16 (&acc)[TM][TN], co
       if (XPK) {
         const long long off = (long long)kg * xstride;  // bf16 elements; uniform
         f.x[tn][0] = *(const zr_f32x4*)((const unsigned short*)xcol[tn] + off);
-        f.x[tn][1] = *(const zr_f32x4*)(xlo[tn] + off);
+        if (LO) f.x[tn][1] = *(const zr_f32x4*)(xlo[tn] + off);
       } else {
         f.x[tn][0] = *(const zr_f32x4*)(xcol[tn] + kg);
         f.x[tn][1] = *(const zr_f32x4*)(xcol[tn] + kg + 4);
@@ -557,9 +561,11 @@ __device__ __forceinline__ void zr_mma_segment_bf16(zr_f32x16 (&acc)[TM][TN], co
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm)
           acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ph, w[tm], acc[tm][tn], 0, 0, 0);
+        if (LO) {
 #pragma unroll
-        for (int tm = 0; tm < TM; ++tm)
-          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pl, w[tm], acc[tm][tn], 0, 0, 0);
+          for (int tm = 0; tm < TM; ++tm)
+            acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pl, w[tm], acc[tm][tn], 0, 0, 0);
+        }
         continue;
       }
       unsigned h0, h1, h2, h3, l0, l1, l2, l3;
@@ -572,9 +578,11 @@ __device__ __forceinline__ void zr_mma_segment_bf16(zr_f32x16 (&acc)[TM][TN], co
 #pragma unroll
       for (int tm = 0; tm < TM; ++tm)
         acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xh, w[tm], acc[tm][tn], 0, 0, 0);
+      if (LO) {
 #pragma unroll
-      for (int tm = 0; tm < TM; ++tm)
-        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xl, w[tm], acc[tm][tn], 0, 0, 0);
+        for (int tm = 0; tm < TM; ++tm)
+          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xl, w[tm], acc[tm][tn], 0, 0, 0);
+      }
     }
   };
 
