@@ -246,8 +246,18 @@ def bench_hbm_kernels(ctx, steps, H=1000, mb=128, V=50000):
     d_x = ctx.empty((H, n))
     _, ms = time_region(ctx, lambda: ctx.embed_gather(d_W, H, V, d_ids, n, d_x), steps, 2)
     bytes_ = 2.0 * n * H * 4 + n * 4
+    ids_host = synth.zipf_ids(synth.rng(77, 2), (n,), V)
+    unique = int(np.unique(ids_host).size)
     out["embed_gather"] = {"columns": n, "us": round(ms * 1e3 / steps, 2), "algorithmic_MB": round(bytes_ / 1e6, 3),
-                           "GBps": round(bytes_ * steps / (ms * 1e-3) / 1e9, 1)}
+                           "GBps": round(bytes_ * steps / (ms * 1e-3) / 1e9, 1), "cache_assisted": True,
+                           "note": "Zipf(1.1) ids repeat: repeated columns are served by the caches, so this is a rate "
+                                   "of algorithmic bytes, not of HBM bytes; see embed_gather_unique_ids"}
+    # the same gather with 6400 DISTINCT columns: every byte read comes from memory
+    d_uid = ctx.array(synth.rng(77, 3).permutation(V)[:n].astype(np.int32))
+    _, ms = time_region(ctx, lambda: ctx.embed_gather(d_W, H, V, d_uid, n, d_x), steps, 2)
+    out["embed_gather_unique_ids"] = {"columns": n, "us": round(ms * 1e3 / steps, 2), "algorithmic_MB": round(bytes_ / 1e6, 3),
+                                      "GBps": round(bytes_ * steps / (ms * 1e-3) / 1e9, 1), "cache_assisted": False}
+    del unique
     # fused gate kernel, one layer-step (4 pre-activation planes + c_prev in, c and h out)
     d_pre = ctx.array(synth.uniform(g, (4 * H * mb,), -1, 1))
     d_b = [ctx.array(synth.uniform(g, (H,))) for _ in range(4)]
@@ -372,6 +382,10 @@ def main():
                     help="only run the language-model training step measurement (for profiling) and exit")
     ap.add_argument("--vendor-gemm", action="store_true",
                     help="only time the vendor library's fp32 GEMM on the main products' shapes (a yardstick) and exit")
+    ap.add_argument("--hbm-kernels-only", action="store_true",
+                    help="only run the HBM-bound kernels at the benchmark shapes (embedding gather and fused gates over "
+                         "6400 columns with unique token ids, a config-3 decoder step, a config-4 decode step) a few "
+                         "times and exit: the command the counter summaries of those kernels under profiles/ are made with")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain copy kernel of known size (for scaling HBM traffic counters) and exit")
     args = ap.parse_args()
@@ -393,6 +407,14 @@ def main():
 
     if args.calibrate_copy:
         print(json.dumps(calibrate_copy(ctx)))
+        ctx.close()
+        return
+    if args.hbm_kernels_only:
+        n = max(2, min(args.steps, 5))
+        out = {"hbm_kernels": bench_hbm_kernels(ctx, n),
+               "config3_decoder_step": {k: v for k, v in bench_decoder_step(ctx, n, 1).items() if k.endswith("_us")},
+               "config4_beam_decode": bench_beam_decode(ctx, n)}
+        print(json.dumps(out))
         ctx.close()
         return
     if args.sweep_only:
