@@ -130,10 +130,8 @@ def bench_decoder_step(ctx, steps, warmup, H=1000, mb=128, S=50, V=50000, L=4, D
     d_prob = ctx.empty((V, mb))
 
     def lstm_part():
-        # layer 0 looks its input columns up in the embedding itself (sparse lookup folded into the node)
-        ctx.lstm_step_embed(layers[0].w, d_embed, V, d_ids, d_hp[0], d_cp[0], d_mask, mb, d_h[0], d_c[0], d_htild=d_htp)
-        for l in range(1, L):
-            ctx.lstm_step(layers[l].w, d_h[l - 1], d_hp[l], d_cp[l], d_mask, mb, d_h[l], d_c[l])
+        # all layers of the step in one call; layer 0 looks its input columns up in the embedding itself
+        ctx.lstm_decoder_step([ly.w for ly in layers], d_embed, V, d_ids, d_hp, d_cp, d_mask, mb, d_h, d_c, d_htild=d_htp)
 
     def attn_part():
         ctx.attn_step(attn, d_bi, d_h[L - 1], d_mask, d_ht)

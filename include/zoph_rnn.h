@@ -55,17 +55,20 @@ int zr_timer_stop(zr_ctx* ctx, float* h_ms);
 /* Tuning / mode switches: see ZR_OPT_* below. */
 int zr_ctx_set_option(zr_ctx* ctx, int option, int value);
 /* State of the context that a caller may want to look at (no counterpart in the reference):
- *   ZR_QUERY_LSTM_STACK_PATH: which schedule the last zr_lstm_stack_forward(_train) call on this context took --
- *     0 none yet, ZR_LSTM_STACK_PATH_SWEEP (one launch for the whole sweep) or ZR_LSTM_STACK_PATH_DIAGONALS (one
- *     launch per diagonal).  Does not wait.
- *   ZR_QUERY_LSTM_SWEEP_ABANDONED: waits for the stream; 1 if a single-launch sweep since the last look gave up a wait
- *     (its outputs were then overwritten with NaN; run the sweep again with ZR_OPT_LSTM_SWEEP = 1), else 0.  Clears
+ *   ZR_QUERY_LSTM_STACK_PATH: which schedule the last zr_lstm_stack_forward(_train) or zr_lstm_decoder_step call on
+ *     this context took -- 0 none yet, ZR_LSTM_STACK_PATH_SWEEP (one launch for the whole sweep),
+ *     ZR_LSTM_STACK_PATH_DIAGONALS (one launch per diagonal), ZR_LSTM_STACK_PATH_STEP_SINGLE_LAUNCH or
+ *     ZR_LSTM_STACK_PATH_STEP_PER_LAYER (zr_lstm_decoder_step).  Does not wait.
+ *   ZR_QUERY_LSTM_SWEEP_ABANDONED: waits for the stream; 1 if a single-launch sweep or decoder step since the last look
+ *     gave up a wait (its outputs were then overwritten with NaN; run it again with ZR_OPT_LSTM_SWEEP = 1), else 0.  Clears
  *     the flag, so a following zr_ctx_sync no longer reports it. */
 int zr_ctx_query(zr_ctx* ctx, int what, int* h_value);
 #define ZR_QUERY_LSTM_STACK_PATH 1
 #define ZR_QUERY_LSTM_SWEEP_ABANDONED 2
 #define ZR_LSTM_STACK_PATH_SWEEP 1
 #define ZR_LSTM_STACK_PATH_DIAGONALS 2
+#define ZR_LSTM_STACK_PATH_STEP_SINGLE_LAUNCH 3 /* zr_lstm_decoder_step: all layers in one launch */
+#define ZR_LSTM_STACK_PATH_STEP_PER_LAYER 4     /* zr_lstm_decoder_step: one launch per layer */
 const char* zr_last_error(void);
 /* Library self-description: "gfx950 hip <build tag>". */
 const char* zr_version(void);
@@ -165,6 +168,21 @@ int zr_lstm_step(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_in, const
 int zr_lstm_step_embed(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_embed, int V, const int* d_ids_nonneg,
                        const float* d_hprev, const float* d_cprev, const float* d_htild, const int* d_mask01,
                        float clip_threshold, int mb, float* d_h, float* d_c, float* const d_gates[4]);
+
+/* One decoder time step through all L layers: the LSTM part of neuralMT_model::forward_prop_target
+ * (src/model.hpp:2573-2640) -- layer 0 is zr_lstm_step_embed on the current words (with d_htild, the previous step's
+ * attention output, through Q when feed-input is on: src/LSTM.hpp:154-164), layer l > 0 is zr_lstm_step on this
+ * step's h of layer l-1 (src/LSTM_HH.hpp:148-317).  The layers of one step form a chain, but the W_h and Q products
+ * only read the previous step: when two workgroups per state tile fit on the device at once the whole step is ONE
+ * launch, in which half of the workgroups stream those products for all layers while the other half walk up the
+ * chain (same conditions, option and give-up reporting as the single-launch sweep: ZR_OPT_LSTM_SWEEP,
+ * ZR_QUERY_LSTM_SWEEP_ABANDONED); otherwise one launch per layer.  Both give the same h and c to rounding.
+ *   d_hprev / d_cprev / d_h / d_c: arrays of L device pointers (H x mb each).  No d_h[l] may alias another d_h, any
+ *   d_hprev[m] or d_htild; d_c[l] may alias d_cprev[l]. */
+int zr_lstm_decoder_step(zr_ctx* ctx, int L, const zr_lstm_weights* const layers[], const float* d_embed, int V,
+                         const int* d_ids_nonneg, const float* const d_hprev[], const float* const d_cprev[],
+                         const float* d_htild, const int* d_mask01, float clip_threshold, int mb,
+                         float* const d_h[], float* const d_c[]);
 
 /* The stand-alone fused gate kernel (the four activation kernels + c_t + clip + h_t + mask of the list above)
  * on pre-activations that are already in memory: d_preact is 4 planes (i,f,c,o) of H x mb holding

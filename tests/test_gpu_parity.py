@@ -685,6 +685,123 @@ def test_lstm_step_with_embedding_lookup_folded_in(ctx, H, mb, feed, fused):
     assert np.all(h1.get()[:, mb // 2] == 0)
 
 
+def _decoder_step_case(g, H, mb, L, feed, V=977):
+    layers = [synth.lstm_layer(g, H, feed_input=(feed and l == 0), forget_bias_one=True) for l in range(L)]
+    embed = U(g, (H, V), -1, 1)
+    ids = g.integers(0, V, size=mb).astype(np.int32)
+    ids[0], ids[mb - 1] = 0, V - 1
+    if mb > 3:
+        ids[2] = ids[1]
+    hp = [U(g, (H, mb), -1, 1) for _ in range(L)]
+    cp = [U(g, (H, mb), -1, 1) for _ in range(L)]
+    ht = U(g, (H, mb), -1, 1) if feed else None
+    mask = np.ones(mb, np.int32)
+    mask[mb // 2] = 0
+    return layers, embed, ids, hp, cp, ht, mask
+
+
+def _run_decoder_step(ctx, case, V=977, clip=0.8, expect_path=None):
+    layers, embed, ids, hp, cp, ht, mask = case
+    H, mb = hp[0].shape
+    L = len(layers)
+    lys = [Layer(ctx, ly) for ly in layers]
+    try:
+        d_h = [ctx.zeros((H, mb)) for _ in range(L)]
+        d_c = [ctx.zeros((H, mb)) for _ in range(L)]
+        ctx.lstm_decoder_step([ly.w for ly in lys], ctx.array(embed), V, ctx.array(ids), [ctx.array(a) for a in hp],
+                              [ctx.array(a) for a in cp], ctx.array(mask), mb, d_h, d_c,
+                              d_htild=ctx.array(ht) if ht is not None else None, clip=clip)
+        if expect_path is not None:
+            assert ctx.query(capi.ZR_QUERY_LSTM_STACK_PATH) == expect_path
+        abandoned = ctx.query(capi.ZR_QUERY_LSTM_SWEEP_ABANDONED)
+        ctx.sync()
+        return [a.get() for a in d_h], [a.get() for a in d_c], abandoned
+    finally:
+        for ly in lys:
+            ly.close()
+
+
+def _oracle_decoder_step(case, clip=0.8):
+    layers, embed, ids, hp, cp, ht, mask = case
+    hs, cs = [], []
+    x = o.embed_gather(embed, ids)
+    for l, ly in enumerate(layers):
+        r = o.lstm_step(ly["M"], ly["Wh"], ly["b"], x, hp[l], cp[l], mask, Q=ly.get("Q") if l == 0 else None,
+                        htild=ht if l == 0 else None, clip=clip)
+        hs.append(r["h"])
+        cs.append(r["c"])
+        x = r["h"]
+    return hs, cs
+
+
+@pytest.mark.parametrize("H,mb,L,feed", [(64, 5, 3, True), (1000, 128, 4, True), (200, 70, 2, True), (72, 33, 1, False),
+                                         (128, 128, 4, False), (256, 192, 4, True), (1000, 12, 4, True),
+                                         (104, 40, 8, False)])
+def test_decoder_step_all_layers_in_one_launch(ctx, H, mb, L, feed):
+    """zr_lstm_decoder_step as ONE launch (two resident workgroups per state tile: one streams the W_h / Q products of
+    every layer, the other walks up the chain of layers) against the oracle's node-by-node step and against one launch
+    per layer: feed-input on layer 0, duplicate and extreme ids, a masked column, cell clipping, row and column tails,
+    a batch width that is not a multiple of 8 (consumers then invalidate their caches), one to eight layers."""
+    g = synth.rng(31, H + mb + L)
+    case = _decoder_step_case(g, H, mb, L, feed)
+    ctx.set_option(capi.ZR_OPT_LSTM_SWEEP, 2)
+    try:
+        h1, c1, gave_up = _run_decoder_step(ctx, case, expect_path=capi.ZR_LSTM_STACK_PATH_STEP_SINGLE_LAUNCH)
+        ctx.set_option(capi.ZR_OPT_LSTM_SWEEP, 1)
+        h2, c2, _ = _run_decoder_step(ctx, case, expect_path=capi.ZR_LSTM_STACK_PATH_STEP_PER_LAYER)
+    finally:
+        ctx.set_option(capi.ZR_OPT_LSTM_SWEEP, 0)
+    assert gave_up == 0
+    want_h, want_c = _oracle_decoder_step(case)
+    for l in range(L):
+        assert_close(h1[l], want_h[l], what="h of layer %d" % l)
+        assert_close(c1[l], want_c[l], what="c of layer %d" % l)
+        assert_close(h2[l], want_h[l], what="h of layer %d, per-layer launches" % l)
+        assert_close(c2[l], want_c[l], what="c of layer %d, per-layer launches" % l)
+        assert np.all(h1[l][:, mb // 2] == 0) and np.all(c1[l][:, mb // 2] == 0)
+
+
+def test_decoder_step_picks_the_single_launch_at_benchmark_size_and_repeats_bit_for_bit(ctx):
+    """H = 1000, 128 columns, 4 layers with feed-input: left to itself the library takes the single launch (it fills
+    the device); two runs give the same bits (the two partial sums of a tile are always added in the same order)."""
+    g = synth.rng(32, 1)
+    case = _decoder_step_case(g, 1000, 128, 4, True)
+    h1, c1, a1 = _run_decoder_step(ctx, case, expect_path=capi.ZR_LSTM_STACK_PATH_STEP_SINGLE_LAUNCH)
+    h2, c2, a2 = _run_decoder_step(ctx, case, expect_path=capi.ZR_LSTM_STACK_PATH_STEP_SINGLE_LAUNCH)
+    assert a1 == 0 and a2 == 0
+    for l in range(4):
+        assert h1[l].tobytes() == h2[l].tobytes() and c1[l].tobytes() == c2[l].tobytes()
+
+
+def test_decoder_step_single_launch_abandoned_wait_is_reported(ctx):
+    """With a single poll per wait the layers above the first give up at once: every workgroup still leaves the kernel,
+    the query reports it, the unfinished outputs hold NaN, and the next step with the default limit is complete again
+    (the last workgroup out of the abandoned launch returned the counters to zero)."""
+    g = synth.rng(33, 1)
+    case = _decoder_step_case(g, 128, 40, 3, True)
+    ctx.set_option(capi.ZR_OPT_LSTM_SWEEP, 2)
+    ctx.set_option(capi.ZR_OPT_LSTM_SWEEP_SPIN, 1)
+    try:
+        h1, c1, gave_up = _run_decoder_step(ctx, case, expect_path=capi.ZR_LSTM_STACK_PATH_STEP_SINGLE_LAUNCH)
+        assert gave_up == 1
+        # what the abandoned step did not finish holds NaN, what it did finish is right; the top layer cannot be complete
+        want_h, want_c = _oracle_decoder_step(case)
+        assert np.isnan(h1[-1]).any() and np.isnan(c1[-1]).any()
+        for got, want in zip(h1 + c1, want_h + want_c):
+            done = ~np.isnan(got)
+            assert_close(np.where(done, got, 0.0), np.where(done, want, 0.0), what="finished part of an abandoned step")
+        ctx.set_option(capi.ZR_OPT_LSTM_SWEEP_SPIN, 0)
+        h2, c2, gave_up = _run_decoder_step(ctx, case, expect_path=capi.ZR_LSTM_STACK_PATH_STEP_SINGLE_LAUNCH)
+        assert gave_up == 0
+    finally:
+        ctx.set_option(capi.ZR_OPT_LSTM_SWEEP, 0)
+        ctx.set_option(capi.ZR_OPT_LSTM_SWEEP_SPIN, 0)
+    want_h, want_c = _oracle_decoder_step(case)
+    for l in range(3):
+        assert_close(h2[l], want_h[l], what="h of layer %d" % l)
+        assert_close(c2[l], want_c[l], what="c of layer %d" % l)
+
+
 def test_stack_forward_with_split_kernel_forced(ctx):
     g = synth.rng(17, 1)
     H, mb, T, V, L = 64, 5, 7, 211, 3

@@ -25,6 +25,8 @@ ZR_QUERY_LSTM_STACK_PATH = 1
 ZR_QUERY_LSTM_SWEEP_ABANDONED = 2
 ZR_LSTM_STACK_PATH_SWEEP = 1
 ZR_LSTM_STACK_PATH_DIAGONALS = 2
+ZR_LSTM_STACK_PATH_STEP_SINGLE_LAUNCH = 3
+ZR_LSTM_STACK_PATH_STEP_PER_LAYER = 4
 ZR_SOFTMAX_PROB = 0
 ZR_SOFTMAX_LOGPROB = 1
 
@@ -41,7 +43,7 @@ SYMBOLS = [
     "zr_unstack_gates", "zr_lstm_stack_backward", "zr_lstm_weight_gradients", "zr_embed_gradient",
     "zr_softmax_backward", "zr_sgd_update", "zr_lstm_node_backward", "zr_lstm_node_gradients",
     "zr_softmax_backward_accumulate", "zr_gather_columns_multi", "zr_softmax_backward_loss",
-    "zr_softmax_forward_static", "zr_ctx_query", "zr_attn_prepare", "zr_lstm_step_embed", "zr_attn_viterbi",
+    "zr_softmax_forward_static", "zr_ctx_query", "zr_attn_prepare", "zr_lstm_step_embed", "zr_attn_viterbi", "zr_lstm_decoder_step",
 ]
 
 _lib = None
@@ -210,6 +212,13 @@ class Context:
         _chk(load().zr_lstm_step_embed(self.h, w, _vp(d_embed), C.c_int(V), _vp(d_ids), _vp(d_hprev), _vp(d_cprev),
                                        _vp(d_htild), _vp(d_mask), C.c_float(clip), C.c_int(mb), _vp(d_h), _vp(d_c),
                                        _ptr_array(gates) if gates else None))
+
+    def lstm_decoder_step(self, layers, d_embed, V, d_ids, hprev, cprev, d_mask, mb, h, c, d_htild=None, clip=0.0):
+        L = len(layers)
+        larr = (C.c_void_p * L)(*[w.value for w in layers])
+        _chk(load().zr_lstm_decoder_step(self.h, C.c_int(L), larr, _vp(d_embed), C.c_int(V), _vp(d_ids),
+                                         _ptr_array(hprev), _ptr_array(cprev), _vp(d_htild), _vp(d_mask),
+                                         C.c_float(clip), C.c_int(mb), _ptr_array(h), _ptr_array(c)))
 
     def lstm_gates(self, d_preact, b, d_cprev, d_mask, H, mb, d_h, d_c, clip=0.0, gates=None):
         _chk(load().zr_lstm_gates(self.h, _vp(d_preact), _ptr_array(b), _vp(d_cprev), _vp(d_mask), C.c_float(clip),

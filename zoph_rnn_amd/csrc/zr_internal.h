@@ -28,6 +28,7 @@ struct zr_ctx {
   int sweep_spin;    // polls before a waiting workgroup of that kernel gives up (0: default)
   int cu_count;      // compute units of the device (filled with sweep_capacity)
   int sweep_capacity[3];  // resident workgroups of lstm_sweep_kernel<TN> (0: not asked yet, -1: unknown)
+  int stack_step_capacity;  // the same for lstm_decoder_stack_kernel<1>
   int gemm_cfg;
   int bf16_terms;       // bf16-weight products: 2 (default, 0 = 2) = activations as two bf16 terms, 1 = rounded to bf16 once
   int last_stack_path;  // ZR_LSTM_STACK_PATH_* of the last zr_lstm_stack_forward(_train) call (0: none yet)

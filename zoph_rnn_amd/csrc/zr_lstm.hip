@@ -816,6 +816,281 @@ __global__ void __launch_bounds__(256) lstm_sweep_kernel(LstmSweep P) {
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// One decoder time step through ALL layers in one launch (the LSTM part of neuralMT_model::forward_prop_target,
+// src/model.hpp:2573-2640: layer 0 on the embedding column of the current word, the previous step's attention output
+// through Q when feed-input is on, layer l > 0 on h_t of layer l-1).
+//
+// A time step is a chain: layer l cannot start its M_l . h_t^{l-1} product before layer l-1 has finished, and one
+// layer is too little work for the chip, so one launch per layer runs four short launches back to back, each with its
+// own launch gap, ramp-up, cross-workgroup sum and tail.  But more than half of the step's products do not depend on
+// the step at all: W_h . h_{t-1} of every layer and Q . h~_{t-1} read only the previous step.  Here every
+// 32-row x 32*TN-column tile of the state has TWO resident workgroups for the whole step:
+//   role 1 streams the products that depend on nothing -- W_h^l . h_{t-1}^l for l = 0, 1, ... (and the upper part of
+//          Q's K range) -- never waits, and leaves each layer's partial pre-activation tile in device memory;
+//   role 0 computes M_0 . x (x gathered from the embedding) and the lower part of Q's K range, then for each layer:
+//          takes role 1's partial tile, adds it to its own sums (own + role 1's: one fixed order, so the result does
+//          not depend on timing), runs the gate / cell epilogue, writes h and c, publishes a k-interleaved copy of
+//          h for the layer above, and goes on to M_{l+1} . h_t^l as soon as all row tiles of its column tile have
+//          arrived (the weights of that product are already in flight while it waits).
+// (Four workgroups per tile at two per compute unit -- the chain sharing each compute unit with the backlog of
+// independent products -- measured slower: 115 us against 106 at H = 1000, 128 columns, 4 layers; the epilogues and
+// hand-overs of the chain take three times as long next to a wave that keeps the matrix pipe busy.)
+// Hand-over, progress and bounded waits are those of lstm_sweep_kernel: device-scope stores and counters, a launch that
+// must be wholly resident (the host checks), waits that give up after a poll limit, mark every counter and raise the
+// status flag.  A finishing workgroup that gives up leaves NaN in the part of h and c it did not finish.  The last
+// workgroup to leave returns the counters to zero for the next launch.
+// ---------------------------------------------------------------------------------------------------------
+struct LstmDecStack {
+  const float* W[kMaxUnits];      // per layer: [nseg][4] packed fp32 matrices
+  const float* bias[kMaxUnits];   // per layer: [4][H]
+  const float* hprev[kMaxUnits];
+  const float* cprev[kMaxUnits];
+  float* h[kMaxUnits];
+  float* c[kMaxUnits];
+  const float* in0;               // layer 0 input: the H x V embedding when ids is set, else H x mb columns
+  const int* ids;                 // [mb], already non-negative (null: in0 holds the columns themselves)
+  const float* htild;             // previous attention output for layer 0's Q segment (null: none)
+  const int* mask01;              // [mb]
+  float* hp;                      // [nl] k-interleaved copies of h, H*mb floats each
+  float* partials;                // [nl][tile][visit][gate][thread]: role 1's sums
+  int* counters;                  // [nl][tiles] tile flags, then [nl][n_tiles] layer counters at kSweepCtrStride
+  int n_counters;                 // ints in `counters` (all of them are marked when a wait is abandoned)
+  int* departures;                // workgroups that have left the kernel (zero at launch)
+  int* status;
+  int nl, V, H, mb, ldw, kp, j_tiles, n_tiles;
+  float clip;
+  int spin_limit;
+  int fence;                      // as in LstmSweep
+};
+
+// All threads of the workgroup call this.  False: leave the kernel.
+__device__ __forceinline__ bool stack_wait(const LstmDecStack& P, int* ctr, int target, int* s_go) {
+  if (threadIdx.x == 0) {
+    int v = __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (int spins = 0; v < target && spins < P.spin_limit; ++spins) {
+      __builtin_amdgcn_s_sleep(2);
+      v = __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    const bool ok = v >= target && !(v & kSweepGaveUp);
+    if (!ok) {
+      if (!(v & kSweepGaveUp))
+        for (int i = 0; i < P.n_counters; ++i) atomicOr(P.counters + i, kSweepGaveUp);
+      __hip_atomic_store(P.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    *s_go = ok ? 1 : 0;
+  }
+  __syncthreads();
+  const bool go = *s_go != 0;
+  if (go && P.fence) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  return go;
+}
+
+template <int TN>
+__global__ void __launch_bounds__(256) lstm_decoder_stack_kernel(LstmDecStack P) {
+  constexpr int KS = 4;
+  constexpr int PF = lstm_prefetch_depth(TN, KS);
+  constexpr int NV = zr_visit_count<TN, KS>();
+  __shared__ __align__(16) float red[KS * 4 * TN * 16 * 64];
+  __shared__ int s_go[3];
+  const int tid = threadIdx.x;
+
+  auto work = [&]() {
+    // die-aware placement as in lstm_fused_kernel; both roles of a tile land on the same die (gridDim.x % 8 == 0)
+    const int id = blockIdx.x;
+    const int r8 = id & 7;
+    const int q8 = id >> 3;
+    const int nt = q8 % P.n_tiles;
+    const int per_die = (P.j_tiles + 7) >> 3;
+    const int jt = r8 * per_die + q8 / P.n_tiles;
+    if (q8 / P.n_tiles >= per_die || jt >= P.j_tiles) return;
+    const int role = blockIdx.y;
+
+    const int lane = tid & 63;
+    const int kslice = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int H = P.H, mb = P.mb;
+    const int j0 = jt * 32;
+    const int n0 = nt * 32 * TN;
+    const long long n_el = (long long)H * mb;
+    const long long HH = (long long)P.kp * P.ldw;
+    const int kgroups = H >> 3;
+    // Q's K range: role 0 takes 9/16 of it, so that role 1's sums of layer 0 (which still have to travel) are there
+    // when role 0 comes for them
+    const int q_split = (kgroups * 9) >> 4;
+    const int tiles = P.j_tiles * P.n_tiles;
+    const int tile = jt * P.n_tiles + nt;
+    int* layer_ctr = P.counters + P.nl * tiles;
+    auto visit_col = [&](int i, int half) {
+      const int slot = zr_wide_visit_slot<KS>(kslice, i);
+      const int tn = slot >> 4, r = slot & 15;
+      const int n = n0 + tn * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+      return n < mb ? n : mb - 1;
+    };
+
+    // A finishing workgroup that abandons a wait in layer l0 leaves NaN in its tile of h and c from that layer up
+    // (role 1 never waits): whatever of the step's outputs was not finished cannot pass for a result.
+    auto abandon = [&](int l0) {
+      const float nan = __builtin_nanf("");
+      for (int l = l0; l < P.nl; ++l)
+        for (int e = tid; e < 32 * 32 * TN; e += 256) {
+          const int j = j0 + (e & 31), n = n0 + (e >> 5);
+          if (j < H && n < mb) P.h[l][(long long)n * H + j] = nan, P.c[l][(long long)n * H + j] = nan;
+        }
+    };
+    for (int l = 0; l < P.nl; ++l) {
+      // per-lane values are derived afresh in every layer (see lstm_sweep_kernel)
+      int lane_t = lane;
+      asm volatile("" : "+v"(lane_t));
+      const int jl = lane_t & 31, half = lane_t >> 5;
+      const int j = j0 + jl;
+      const bool j_ok = j < H;
+      const int jc = j_ok ? j : H - 1;
+      int cols[TN];
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) {
+        const int c = n0 + tn * 32 + jl;
+        cols[tn] = c < mb ? c : mb - 1;
+      }
+      const unsigned woffb = 16u * (unsigned)(j + half * P.ldw);
+
+      // epilogue operands of the finishing role go out ahead of the K loops
+      float bi = 0.0f, bf = 0.0f, bc = 0.0f, bo = 0.0f, cprev_v[NV], mask_v[NV];
+#pragma unroll
+      for (int i = 0; i < NV; ++i) cprev_v[i] = 0.0f, mask_v[i] = 0.0f;
+      if (role == 0) {
+        const float* bias = P.bias[l];
+        bi = bias[jc], bf = bias[H + jc], bc = bias[2 * H + jc], bo = bias[3 * H + jc];
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+          const int n = visit_col(i, half);
+          cprev_v[i] = P.cprev[l][(long long)n * H + jc];
+          mask_v[i] = (float)P.mask01[n];
+        }
+      }
+
+      zr_f32x16 acc[4][TN];
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[g][tn][r] = 0.0f;
+
+      const int nq = (l == 0 && P.htild) ? 2 : 1;
+      for (int q = 0; q < nq; ++q) {
+        // q = 0: this role's own matrix (0 = M, 1 = W_h) over all of K; q = 1: its part of Q's K range
+        const int s = (q == 1) ? 2 : role;
+        int g0 = 0, g1 = kgroups;
+        if (q == 1) {
+          g0 = role ? q_split : 0;
+          g1 = role ? kgroups : q_split;
+        }
+        const int K = (g1 - g0) * 8;
+        const bool packed = role == 0 && q == 0 && l > 0;
+        unsigned wsoff[4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) wsoff[g] = (unsigned)((((long long)s * 4 + g) * HH + (long long)g0 * 8 * P.ldw) * 4);
+        ZrFrag<4, TN> ring[PF + 1];
+        const __amdgpu_buffer_rsrc_t wrsrc = zr_make_rsrc(P.W[l]);
+        zr_preload_w<4, TN, KS, PF>(ring, wrsrc, wsoff, woffb, 32u * (unsigned)P.ldw, K, kslice);
+        if (packed) {
+          if (!stack_wait(P, layer_ctr + ((l - 1) * P.n_tiles + nt) * kSweepCtrStride, P.j_tiles, &s_go[0])) {
+            abandon(l);
+            return;
+          }
+        }
+        const float* xb;
+        unsigned xoffb[TN];
+        if (packed) {
+          xb = P.hp + (long long)(l - 1) * n_el;
+#pragma unroll
+          for (int tn = 0; tn < TN; ++tn) xoffb[tn] = 16u * ((unsigned)cols[tn] + (unsigned)(half * mb));
+        } else {
+          xb = (q == 1) ? P.htild + g0 * 8 : (role == 1 ? P.hprev[l] : P.in0);
+          const bool gather = q == 0 && role == 0 && P.ids != nullptr;
+#pragma unroll
+          for (int tn = 0; tn < TN; ++tn) {
+            unsigned c = (unsigned)cols[tn];
+            if (gather) {
+              const int v = P.ids[cols[tn]];
+              c = (unsigned)(v < 0 ? 0 : (v >= P.V ? P.V - 1 : v));
+            }
+            xoffb[tn] = 4u * (c * (unsigned)H + 4u * half);
+          }
+        }
+        zr_mma_segment_u<4, TN, KS, PF, true>(acc, wrsrc, wsoff, woffb, 32u * (unsigned)P.ldw, zr_make_rsrc(xb), xoffb,
+                                              packed ? 32u * (unsigned)mb : 32u, K, kslice, ring);
+      }
+
+      float* part = P.partials + ((long long)l * tiles + tile) * (NV * 4 * 256) + tid;
+      int* flag = P.counters + l * tiles + tile;
+      if (role == 1) {
+        zr_reduce_visit_wide<4, TN, KS>(acc, red, kslice, lane, [&](const float(&z)[4], int, int, int vi) {
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+            __hip_atomic_store(part + (vi * 4 + g) * 256, z[g], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        });
+        zr_publish_barrier();
+        if (tid == 0) atomicAdd(flag, 1);
+        continue;
+      }
+
+      // role 0: the other role's sums (normally long there), fetched while this workgroup's partial tiles are summed
+      if (!stack_wait(P, flag, 1, &s_go[1])) {
+        abandon(l);
+        return;
+      }
+      float other[NV][4];
+#pragma unroll
+      for (int vi = 0; vi < NV; ++vi)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+          other[vi][g] = __hip_atomic_load(part + (vi * 4 + g) * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const bool hand_on = l + 1 < P.nl;
+      float* hp_out = P.hp + (long long)l * n_el;
+      float h_v[NV], c_v[NV];
+      zr_reduce_visit_wide<4, TN, KS>(acc, red, kslice, lane, [&](const float(&z)[4], int tn, int r, int vi) {
+        const int n = n0 + tn * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+        float gi, gf, gc, go;
+        zr_lstm_cell((z[0] + other[vi][0]) + bi, (z[1] + other[vi][1]) + bf, (z[2] + other[vi][2]) + bc,
+                     (z[3] + other[vi][3]) + bo, cprev_v[vi], mask_v[vi], P.clip, gi, gf, gc, go, c_v[vi], h_v[vi]);
+        if (hand_on && j_ok && n < mb)
+          __hip_atomic_store(hp_out + ((long long)(j >> 2) * mb + n) * 4 + (j & 3), h_v[vi], __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+      });
+      if (hand_on) {
+        zr_publish_barrier();
+        if (tid == 0) atomicAdd(layer_ctr + (l * P.n_tiles + nt) * kSweepCtrStride, 1);
+      }
+      float* h_out = P.h[l];
+      float* c_out = P.c[l];
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const int slot = zr_wide_visit_slot<KS>(kslice, i);
+        const int n = n0 + (slot >> 4) * 32 + 8 * ((slot & 15) >> 2) + 4 * half + (slot & 3);
+        if (j_ok && n < mb) {
+          const long long ix = (long long)n * H + j;
+          c_out[ix] = c_v[i];
+          h_out[ix] = h_v[i];
+        }
+      }
+    }
+  };
+  work();
+
+  // Departure.  The last workgroup out returns the counters to zero for the next launch.
+  __syncthreads();
+  if (tid == 0) {
+    const int total = (int)(gridDim.x * gridDim.y);
+    const int before = __hip_atomic_fetch_add(P.departures, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s_go[2] = before == total - 1 ? 1 : 0;
+  }
+  __syncthreads();
+  if (!s_go[2]) return;
+  for (int i = tid; i < P.n_counters; i += 256) __hip_atomic_store(P.counters + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (tid == 0) __hip_atomic_store(P.departures, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 template <int TN, int KS>
 int launch_fused_v(zr_ctx* ctx, const LstmLaunch& L, bool vec) {
   const int groups = L.n_units * L.j_tiles;
@@ -1035,6 +1310,23 @@ int launch_sweep_v(zr_ctx* ctx, LstmSweep& P, int grid) {
   return ZR_OK;
 }
 
+// Resident workgroups of lstm_decoder_stack_kernel<1> the device can hold at once (0: unknown / query failed).
+int stack_step_capacity(zr_ctx* ctx) {
+  int& cached = ctx->stack_step_capacity;
+  if (cached == 0) {
+    int cus = 0, per_cu = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, ctx->device) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lstm_decoder_stack_kernel<1>, 256, 0) != hipSuccess) {
+      (void)hipGetLastError();
+      cached = -1;
+    } else {
+      ctx->cu_count = cus;
+      cached = cus * per_cu > 0 ? cus * per_cu : -1;
+    }
+  }
+  return cached > 0 ? cached : 0;
+}
+
 inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
 }  // namespace
@@ -1221,6 +1513,99 @@ static int lstm_step_impl(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_
     return zr_lstm_gates(ctx, (const float*)pre, b, d_cprev, d_mask01, clip_threshold, H, mb, d_h, d_c, d_gates);
   }
   return launch_fused(ctx, L, vec);
+}
+
+int zr_lstm_decoder_step(zr_ctx* ctx, int nl, const zr_lstm_weights* const layers[], const float* d_embed, int V,
+                         const int* d_ids_nonneg, const float* const d_hprev[], const float* const d_cprev[],
+                         const float* d_htild, const int* d_mask01, float clip_threshold, int mb,
+                         float* const d_h[], float* const d_c[]) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(nl > 0 && nl <= kMaxUnits && mb > 0 && V > 0, "zr_lstm_decoder_step: L = %d, mb = %d, V = %d", nl, mb, V);
+  ZR_CHECK_ARG(layers && d_embed && d_ids_nonneg && d_hprev && d_cprev && d_mask01 && d_h && d_c,
+               "zr_lstm_decoder_step: null pointer");
+  const int H = layers[0] ? layers[0]->H : 0;
+  bool vec = (H > 0) && (H % 4 == 0) && aligned16(d_embed) && (!d_htild || aligned16(d_htild));
+  for (int l = 0; l < nl; ++l) {
+    ZR_CHECK_ARG(layers[l] && layers[l]->H == H, "zr_lstm_decoder_step: layer %d missing or of different size", l);
+    ZR_CHECK_ARG(layers[l]->bf16 == layers[0]->bf16, "zr_lstm_decoder_step: layers mix fp32 and bf16 weights");
+    ZR_CHECK_ARG(d_hprev[l] && d_cprev[l] && d_h[l] && d_c[l], "zr_lstm_decoder_step: null state for layer %d", l);
+    ZR_CHECK_ARG(d_h[l] != d_htild, "zr_lstm_decoder_step: d_h[%d] aliases d_htild", l);
+    for (int m = 0; m < nl; ++m)
+      ZR_CHECK_ARG(d_h[l] != d_hprev[m] && (l == m || d_h[l] != d_h[m]),
+                   "zr_lstm_decoder_step: d_h[%d] aliases another state array", l);
+    vec = vec && aligned16(d_hprev[l]);
+  }
+  ZR_CHECK_ARG(!d_htild || layers[0]->nseg == 3, "zr_lstm_decoder_step: d_htild given but layer 0 was packed without Q");
+  const size_t n = (size_t)H * mb;
+
+  // One launch for the whole step when two workgroups per tile fit on the device together (the same conditions as the
+  // single-launch sweep of zr_lstm_stack_forward); otherwise one node after the other.
+  if (vec && H % 8 == 0 && H >= 64 && !layers[0]->bf16 && ctx->lstm_fused && ctx->lstm_sweep != 1) {
+    const int j_tiles = (H + 31) / 32, n_tiles = (mb + 31) / 32;
+    const int padded = (j_tiles + 7) / 8 * 8;
+    const long long tiles = (long long)j_tiles * n_tiles;
+    const long long wgs = 2LL * padded * n_tiles;
+    const int cap = stack_step_capacity(ctx);
+    const bool fills = wgs * 10 >= 6LL * ctx->cu_count && zr_live_contexts(ctx->device) == 1 &&
+                       ctx->stream == ctx->own_stream;
+    const long long lim = 1LL << 32;
+    const bool offsets_fit = (long long)V * H * 4 < lim && (long long)n * 4 < lim &&
+                             12LL * layers[0]->kp * layers[0]->ldw * 4 < lim;
+    const long long n_counters = nl * tiles + (long long)nl * n_tiles * kSweepCtrStride;
+    if (cap > 0 && wgs <= cap && offsets_fit && n_counters < ZR_MAX_COUNTERS && (fills || ctx->lstm_sweep == 2)) {
+      constexpr int NV = zr_visit_count<1, 4>();
+      LstmDecStack P = {};
+      void* p = nullptr;
+      const size_t hp_bytes = sizeof(float) * (size_t)nl * n;
+      rc = zr_ctx_scratch(ctx, 1, hp_bytes + sizeof(float) * (size_t)nl * tiles * NV * 4 * 256, &p);
+      if (rc) return rc;
+      P.hp = (float*)p;
+      P.partials = (float*)((char*)p + hp_bytes);
+      P.counters = ctx->d_counters;
+      P.n_counters = (int)n_counters;
+      P.departures = ctx->d_counters + (ZR_MAX_COUNTERS - 1);
+      for (int l = 0; l < nl; ++l) {
+        P.W[l] = (const float*)layers[l]->d_W;
+        P.bias[l] = layers[l]->d_bias;
+        P.hprev[l] = d_hprev[l];
+        P.cprev[l] = d_cprev[l];
+        P.h[l] = d_h[l];
+        P.c[l] = d_c[l];
+      }
+      P.in0 = d_embed;
+      P.ids = d_ids_nonneg;
+      P.htild = d_htild;
+      P.mask01 = d_mask01;
+      P.status = ctx->d_flags + 2;
+      P.nl = nl;
+      P.V = V;
+      P.H = H;
+      P.mb = mb;
+      P.ldw = layers[0]->ldw;
+      P.kp = layers[0]->kp;
+      P.j_tiles = j_tiles;
+      P.n_tiles = n_tiles;
+      P.clip = clip_threshold;
+      P.spin_limit = ctx->sweep_spin > 0 ? ctx->sweep_spin : (1 << 20);
+      P.fence = (mb % 8 == 0) ? 0 : 1;
+      ctx->last_stack_path = ZR_LSTM_STACK_PATH_STEP_SINGLE_LAUNCH;
+      lstm_decoder_stack_kernel<1><<<dim3((unsigned)(padded * n_tiles), 2u), 256, 0, ctx->stream>>>(P);
+      ZR_LAUNCH_CHECK("lstm_decoder_stack_kernel");
+      return ZR_OK;
+    }
+  }
+  ctx->last_stack_path = ZR_LSTM_STACK_PATH_STEP_PER_LAYER;
+  for (int l = 0; l < nl; ++l) {
+    if (l == 0)
+      rc = lstm_step_impl(ctx, layers[0], d_embed, d_ids_nonneg, V, d_hprev[0], d_cprev[0], d_htild, d_mask01,
+                          clip_threshold, mb, d_h[0], d_c[0], nullptr);
+    else
+      rc = lstm_step_impl(ctx, layers[l], d_h[l - 1], nullptr, 0, d_hprev[l], d_cprev[l], nullptr, d_mask01,
+                          clip_threshold, mb, d_h[l], d_c[l], nullptr);
+    if (rc) return rc;
+  }
+  return ZR_OK;
 }
 
 int zr_lstm_stack_forward(zr_ctx* ctx, int nl, const zr_lstm_weights* const layers[], const float* d_embed, int V,

@@ -101,12 +101,9 @@ class BeamDecode:
         p, q = self.cur, 1 - self.cur
         ctx.vocab_prep(self.d_words, cols, w.Vt, self.d_words_nn, None)
         feed = self.h_tild[p] if self.step_index > 0 else None
-        ctx.lstm_step_embed(w.tgt[0], w.tgt_embed, w.Vt, self.d_words_nn, self.h[p][0], self.c[p][0], self.d_ones, cols,
-                            self.h[q][0], self.c[q][0], d_htild=feed)
-        below = self.h[q][0]
-        for l in range(1, L):
-            ctx.lstm_step(w.tgt[l], below, self.h[p][l], self.c[p][l], self.d_ones, cols, self.h[q][l], self.c[q][l])
-            below = self.h[q][l]
+        ctx.lstm_decoder_step(w.tgt, w.tgt_embed, w.Vt, self.d_words_nn, self.h[p], self.c[p], self.d_ones, cols,
+                              self.h[q], self.c[q], d_htild=feed)
+        below = self.h[q][L - 1]
         ctx.attn_step(self.attn, self.d_batch_info, below, self.d_ones, self.h_tild[q])
         ctx.softmax_forward(w.D_soft, w.b_soft, w.Vt, H, self.h_tild[q], cols, capi.ZR_SOFTMAX_PROB, self.prob)
 

@@ -880,6 +880,7 @@ class beam_decoder {
   int *d_words = nullptr, *d_words_nn = nullptr, *d_back = nullptr, *d_ones = nullptr, *d_batch_info = nullptr,
       *d_src = nullptr, *d_src_nn = nullptr, *d_src_mask = nullptr, *d_rep = nullptr;
   std::vector<const zr_lstm_weights*> src_w, tgt_w;
+  int abandoned_launches = 0;  // batches decoded a second time because a single-launch sweep or step gave up a wait
 
   template <typename T>
   T* dmalloc(size_t n) {
@@ -961,15 +962,12 @@ class beam_decoder {
   void forward_target(int p, int step_index) {
     const int q = 1 - p;
     ZOPH_CALL(zr_vocab_prep(ctx, d_words, cols, Vt, d_words_nn, nullptr));
-    // layer 0 looks its input columns up in the embedding itself (sparse lookup folded into the node)
+    // all layers of the step in one call; layer 0 looks its input columns up in the embedding itself
     const dType* feed = (feed_input && step_index > 0) ? h_tild[p] : nullptr;
-    ZOPH_CALL(zr_lstm_step_embed(ctx, tgt_w[0], m.input_layer_target.d_W, Vt, d_words_nn, h[p][0], c[p][0], feed, d_ones,
-                                 0.0f, cols, h[q][0], c[q][0], nullptr));
-    const dType* below = h[q][0];
-    for (int l = 1; l < L; l++) {
-      ZOPH_CALL(zr_lstm_step(ctx, tgt_w[l], below, h[p][l], c[p][l], nullptr, d_ones, 0.0f, cols, h[q][l], c[q][l], nullptr));
-      below = h[q][l];
-    }
+    std::vector<const dType*> hp(h[p].begin(), h[p].end()), cp(c[p].begin(), c[p].end());
+    ZOPH_CALL(zr_lstm_decoder_step(ctx, L, tgt_w.data(), m.input_layer_target.d_W, Vt, d_words_nn, hp.data(), cp.data(),
+                                   feed, d_ones, 0.0f, cols, h[q].data(), c[q].data()));
+    const dType* below = h[q][L - 1];
     const dType* top = below;
     if (attention) {
       ZOPH_CALL(zr_attn_step(ctx, attn, d_batch_info, below, d_ones, h_tild[q], nullptr, nullptr, nullptr, nullptr));
@@ -1044,6 +1042,18 @@ class beam_decoder {
     // one last step and forced <EOF> on every live hypothesis (src/ensemble_factory.hpp:727-743)
     forward_target(p, index);
     ZOPH_CALL(zr_beam_finish(ctx, bm, prob));
+    {
+      // A single-launch encoder sweep or decoder step that gave up a wait left NaN in its outputs: the batch is
+      // decoded again with one launch per node (and so is every later batch of this decoder).
+      int abandoned = 0;
+      ZOPH_CALL(zr_ctx_query(ctx, ZR_QUERY_LSTM_SWEEP_ABANDONED, &abandoned));
+      if (abandoned) {
+        abandoned_launches++;
+        ZOPH_CALL(zr_ctx_set_option(ctx, ZR_OPT_LSTM_SWEEP, 1));
+        decode_batch(sources, num_best, out);
+        return;
+      }
+    }
     ZOPH_CALL(zr_ctx_sync(ctx));
 
     out.assign(real, {});
