@@ -422,6 +422,169 @@ void orc_attention_viterbi(const float* alignments, const int* indices, int D, i
   }
 }
 
+// attention_node::back_prop, src/attention_node.hpp:398-669 (single-source branch), with the kernels it launches:
+// zero_h_t (custom_kernels.h:2212), tanh_grad_kernel (:1835), error_alignments_kernel_large (:1968),
+// error_hs_ct_kernel_large (:2179), error_pt_kernel (:2006), att_vp_error (:2040), grad_W_p_kernel (:2051),
+// get_ht_scalings_Wa_grad_kernel (:2094), scale_ht_kernel (:2114), copy_errors_source (:2142), and its cuBLAS calls.
+// The values the reference caches in the forward pass (tanh_1, sigma_1, W_a^T h, the gathered source columns and the
+// Gaussian factors d_cached_exp) are recomputed here from h_t, p_t and the indices with the forward pass's formulas.
+//   h_t:        the h_t the forward pass read (after the attention layer's dropout, where that is on)
+//   err_htild:  error with respect to h~ (the caller has already added the feed-input error of the next step, :416)
+//   outputs:    err_h_t (H x mb, overwritten; before the dropout of :647); err_hs_table (same layout as hs_table, +=);
+//               dW_a, dW_p, dW_c1, dW_c2 (H x H), dv_p, dbias (H), all += as in the reference (beta = 1)
+void orc_attention_backward(int H, int mb, int D, const float* W_a, const float* W_p, const float* v_p,
+                            const float* W_c1, const float* W_c2, const float* hs_table, const int* batch_info,
+                            const float* h_t, const int* mask01, const float* h_tild, const float* alignments,
+                            const int* indices, const float* p_t, const float* c_ctx, const float* err_htild,
+                            float* err_h_t, float* err_hs_table, float* dW_a, float* dW_p, float* dv_p, float* dbias,
+                            float* dW_c1, float* dW_c2) {
+  const int W = 2 * D + 1;
+  const size_t n = (size_t)H * mb;
+  const float sigma_sq = (float)((D * D) / 4.0);
+  std::vector<float> e(n), err_ct(n), err_ht(n), tanh1(n), sigma1(mb), q(n), temp1(n), hs_sum(n, 0.0f), tmp(n);
+  std::vector<float> err_as((size_t)W * mb), err_pt(mb), scal((size_t)W * mb), gauss((size_t)W * mb);
+  auto hs_index = [&](int b, int j) -> long long {
+    const int s = indices[IDX2C(b, j, mb)];
+    if (s == -1) return -1;
+    const int t = batch_info[b] - 1 - s + batch_info[mb + b];
+    return (long long)((size_t)t * n + IDX2C(0, b, H));
+  };
+  // C (H x H) += A (H x mb) * B^T (B is H x mb): cublas gemm N,T with beta = 1, accumulated in double per element
+  auto outer_acc = [&](const float* A, const float* B, float* C) {
+#pragma omp parallel for schedule(static)
+    for (int j = 0; j < H; ++j)
+      for (int i = 0; i < H; ++i) {
+        double sum = 0;
+        for (int b = 0; b < mb; ++b) sum += (double)A[IDX2C(i, b, H)] * (double)B[IDX2C(j, b, H)];
+        C[IDX2C(i, j, H)] += (float)sum;
+      }
+  };
+  for (int b = 0; b < mb; ++b)
+    for (int i = 0; i < H; ++i) {
+      const size_t ix = IDX2C(i, b, H);
+      const float v = err_htild[ix] * mask01[b];            // zero_h_t
+      e[ix] = v * (1 - h_tild[ix] * h_tild[ix]);            // tanh_grad_kernel on d_final_temp_2
+    }
+  outer_acc(e.data(), c_ctx, dW_c1);                         // :437
+  outer_acc(e.data(), h_t, dW_c2);                           // :443
+  for (int i = 0; i < H; ++i) {                              // :456, gemv with the ones vector
+    double sum = 0;
+    for (int b = 0; b < mb; ++b) sum += e[IDX2C(i, b, H)];
+    dbias[i] += (float)sum;
+  }
+  gemm_tn(1, H, mb, H, W_c1, H, e.data(), H, err_ct.data(), H);  // :464
+  gemm_tn(1, H, mb, H, W_c2, H, e.data(), H, err_ht.data(), H);  // :476
+  // error_alignments_kernel_large and error_hs_ct_kernel_large
+  for (int b = 0; b < mb; ++b)
+    for (int j = 0; j < W; ++j) {
+      const long long at = hs_index(b, j);
+      double sum = 0;
+      if (at >= 0) {
+        const float a = alignments[IDX2C(b, j, mb)];
+        for (int i = 0; i < H; ++i) {
+          sum += (double)err_ct[IDX2C(i, b, H)] * (double)hs_table[at + i];
+          err_hs_table[at + i] += err_ct[IDX2C(i, b, H)] * a;
+        }
+      }
+      err_as[IDX2C(j, b, W)] = (float)sum;
+    }
+  // error_pt_kernel
+  for (int b = 0; b < mb; ++b) {
+    double sum = 0;
+    for (int j = 0; j < W; ++j)
+      sum += (double)(err_as[IDX2C(j, b, W)] * alignments[IDX2C(b, j, mb)] *
+                      ((indices[IDX2C(b, j, mb)] - p_t[b]) / sigma_sq));
+    err_pt[b] = (float)sum;
+  }
+  // forward values again: tanh_1, sigma_1 (attention_node.hpp:132-150)
+  gemm_nn(1, H, mb, H, W_p, H, h_t, H, tanh1.data(), H);
+  for (size_t i = 0; i < n; ++i) tanh1[i] = tanhf(tanh1[i]);
+  gemm_nn(1, 1, mb, H, v_p, 1, tanh1.data(), H, sigma1.data(), 1);
+  for (int b = 0; b < mb; ++b) sigma1[b] = (float)(1.0 / (1.0 + exp(-1.0 * (double)sigma1[b])));
+  // att_vp_error, then the gemv into v_p_grad (:536)
+  for (int b = 0; b < mb; ++b)
+    for (int i = 0; i < H; ++i)
+      temp1[IDX2C(i, b, H)] = err_pt[b] * sigma1[b] * (1 - sigma1[b]) * batch_info[b] * tanh1[IDX2C(i, b, H)];
+  for (int i = 0; i < H; ++i) {
+    double sum = 0;
+    for (int b = 0; b < mb; ++b) sum += temp1[IDX2C(i, b, H)];
+    dv_p[i] += (float)sum;
+  }
+  // grad_W_p_kernel, the outer product into W_p_grad (:545) and W_p^T temp into the error of h_t (:551, beta = 1)
+  for (int b = 0; b < mb; ++b)
+    for (int i = 0; i < H; ++i) {
+      const size_t ix = IDX2C(i, b, H);
+      temp1[ix] = err_pt[b] * batch_info[b] * v_p[i] * sigma1[b] * (1 - sigma1[b]) * (1 - tanh1[ix] * tanh1[ix]);
+    }
+  outer_acc(temp1.data(), h_t, dW_p);
+  gemm_tn(1, H, mb, H, W_p, H, temp1.data(), H, tmp.data(), H);
+  for (size_t i = 0; i < n; ++i) err_ht[i] += tmp[i];
+  // get_ht_scalings_Wa_grad_kernel; d_cached_exp as alignment_reduction_kernel leaves it (1 on empty slots)
+  for (int b = 0; b < mb; ++b)
+    for (int j = 0; j < W; ++j) {
+      const int s = indices[IDX2C(b, j, mb)];
+      float g = 1;
+      if (s != -1) {
+        const float d = p_t[b] - s;
+        g = expf((-1 * powf(d, 2.0f)) / (2 * sigma_sq));
+      }
+      gauss[IDX2C(j, b, W)] = g;
+    }
+  for (int b = 0; b < mb; ++b)
+    for (int j = 0; j < W; ++j) {
+      const float aj = alignments[IDX2C(b, j, mb)], gj = gauss[IDX2C(j, b, W)];
+      float v = err_as[IDX2C(j, b, W)] * aj * (1 - aj / gj);
+      for (int k = 0; k < W; ++k)
+        if (k != j) v += -1 * err_as[IDX2C(k, b, W)] * alignments[IDX2C(b, k, mb)] * aj / gj;
+      scal[IDX2C(j, b, W)] = v;
+    }
+  // the loop of :580-601: h_s_sum += scaling * h_s; error of h_s += scaling * (W_a^T h)
+  gemm_tn(1, H, mb, H, W_a, H, h_t, H, q.data(), H);
+  for (int b = 0; b < mb; ++b)
+    for (int j = 0; j < W; ++j) {
+      const long long at = hs_index(b, j);
+      if (at < 0) continue;  // the gathered column is zero and copy_errors_source skips the slot
+      const float sc = scal[IDX2C(j, b, W)];
+      for (int i = 0; i < H; ++i) {
+        hs_sum[IDX2C(i, b, H)] += hs_table[at + i] * sc;
+        err_hs_table[at + i] += q[IDX2C(i, b, H)] * sc;
+      }
+    }
+  outer_acc(h_t, hs_sum.data(), dW_a);                              // :632
+  gemm_nn(1, H, mb, H, W_a, H, hs_sum.data(), H, tmp.data(), H);    // :636, beta = 1
+  for (size_t i = 0; i < n; ++i) err_h_t[i] = err_ht[i] + tmp[i];
+}
+
+// dropout_kernel, src/custom_kernels.h:1556-1560: `rate` is the probability of KEEPING a value, `uniform` the
+// numbers curandGenerateUniform left in the mask array.
+void orc_dropout(const float* uniform, float rate, float* x, size_t n) {
+  for (size_t i = 0; i < n; ++i) x[i] = (uniform[i] < rate) * (1 / rate) * x[i];
+}
+
+// The feed-input part of LSTM_IH_Node::back_prop_GPU and compute_gradients_GPU (src/LSTM.hpp:804-866, under
+// `feed_input && index != 0`, and the Q gradient products :1014-1050): error of h~_{t-1} = sum_g Q_g^T d_g, and
+// Q_g_grad += d_g h~^T.
+//   dgates: the four pre-activation errors stacked as [4H] x mb (i, f, c~, o); Q, dQ: four H x H matrices each
+void orc_lstm_feed_backward(int H, int mb, const float* const* Q, const float* dgates, const float* htild,
+                            float* err_htild, float* const* dQ) {
+  const size_t n = (size_t)H * mb;
+  std::vector<float> dg(n), tmp(n);
+  for (size_t i = 0; i < n; ++i) err_htild[i] = 0;
+  for (int g = 0; g < 4; ++g) {
+    for (int b = 0; b < mb; ++b)
+      for (int i = 0; i < H; ++i) dg[IDX2C(i, b, H)] = dgates[IDX2C(g * H + i, b, 4 * H)];
+    gemm_tn(1, H, mb, H, Q[g], H, dg.data(), H, tmp.data(), H);
+    for (size_t i = 0; i < n; ++i) err_htild[i] += tmp[i];
+#pragma omp parallel for schedule(static)
+    for (int j = 0; j < H; ++j)
+      for (int i = 0; i < H; ++i) {
+        double sum = 0;
+        for (int b = 0; b < mb; ++b) sum += (double)dg[IDX2C(i, b, H)] * (double)htild[IDX2C(j, b, H)];
+        dQ[g][IDX2C(i, j, H)] += (float)sum;
+      }
+  }
+}
+
 // Column gather used by the decoder state shuffles: dst[:,i] = src[:,perm[i]]
 // (Input_To_Hidden_Layer::swap_states_decoding, src/Input_To_Hidden_Layer.hpp:1231-1242).
 void orc_gather_columns(const float* src, int H, const int* perm, int n, float* dst) {

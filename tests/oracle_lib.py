@@ -198,6 +198,53 @@ def attention_forward(W_a, W_p, v_p, out_bias, W_c1, W_c2, hs_table, batch_info,
     return out
 
 
+def attention_backward(W_a, W_p, v_p, W_c1, W_c2, hs_table, batch_info, h_t, mask01, fwd, err_htild, D, grads=None,
+                       err_hs=None):
+    """fwd: the dictionary attention_forward returned for the same inputs.  Returns (err_h_t, err_hs, grads); err_hs
+    (S, H, mb) and grads {"W_a", "W_p", "v_p", "bias", "W_c1", "W_c2"} are accumulated into when given."""
+    W_a, W_p, W_c1, W_c2, h_t, err_htild = F(W_a), F(W_p), F(W_c1), F(W_c2), F(h_t), F(err_htild)
+    H, mb = h_t.shape
+    v_p = np.ascontiguousarray(v_p, dtype=np.float32).reshape(-1)
+    hs = pack_hs_table(hs_table)
+    S = np.asarray(hs_table).shape[0]
+    batch_info = np.ascontiguousarray(batch_info, dtype=np.int32)
+    mask01 = np.ascontiguousarray(mask01, dtype=np.int32)
+    if grads is None:
+        grads = {k: np.zeros((H, H), np.float32, order="F") for k in ("W_a", "W_p", "W_c1", "W_c2")}
+        grads["v_p"] = np.zeros(H, np.float32)
+        grads["bias"] = np.zeros(H, np.float32)
+    ehs = np.zeros(S * H * mb, np.float32) if err_hs is None else pack_hs_table(err_hs)
+    err_h_t = np.empty((H, mb), dtype=np.float32, order="F")
+    lib().orc_attention_backward(C.c_int(H), C.c_int(mb), C.c_int(D), _p(W_a), _p(W_p), _p(v_p), _p(W_c1), _p(W_c2),
+                                 _p(hs), _p(batch_info, i32p), _p(h_t), _p(mask01, i32p), _p(F(fwd["h_tild"])),
+                                 _p(F(fwd["alignments"])), _p(F(fwd["indices"], np.int32), i32p), _p(F(fwd["p_t"])),
+                                 _p(F(fwd["c_ctx"])), _p(err_htild), _p(err_h_t), _p(ehs), _p(grads["W_a"]),
+                                 _p(grads["W_p"]), _p(grads["v_p"]), _p(grads["bias"]), _p(grads["W_c1"]),
+                                 _p(grads["W_c2"]))
+    err_hs_out = np.stack([ehs[t * H * mb:(t + 1) * H * mb].reshape(H, mb, order="F") for t in range(S)])
+    return err_h_t, err_hs_out, grads
+
+
+def dropout(uniform, rate, x):
+    """dropout_kernel: x * (uniform < rate) / rate; returns a new array."""
+    x = F(x).copy(order="F")
+    u = F(uniform)
+    assert u.shape == x.shape
+    lib().orc_dropout(_p(u), C.c_float(rate), _p(x), C.c_size_t(x.size))
+    return x
+
+
+def lstm_feed_backward(Q, dgates, htild, dQ=None):
+    """dgates: (4H, mb) stacked pre-activation errors.  Returns (err_htild, dQ list of four H x H)."""
+    dgates, htild = F(dgates), F(htild)
+    H, mb = htild.shape
+    Qs = [F(q) for q in Q]
+    dQ = [np.zeros((H, H), np.float32, order="F") for _ in range(4)] if dQ is None else [F(q) for q in dQ]
+    err = np.empty((H, mb), dtype=np.float32, order="F")
+    lib().orc_lstm_feed_backward(C.c_int(H), C.c_int(mb), _pp(Qs), _p(dgates), _p(htild), _p(err), _pp(dQ))
+    return err, dQ
+
+
 def attention_viterbi(alignments, indices):
     """alignments, indices: (mb, 2D+1) arrays laid out [b + mb*j] (column-major)."""
     al, ix = F(alignments), F(indices, np.int32)

@@ -137,3 +137,102 @@ def test_softmax_backward_matches_torch_and_finite_differences(V, H, mb):
     # accumulation across calls
     _, dD2, db2 = o.softmax_backward(D, b, h, target, mask, dD.copy(order="F"), db.copy())
     assert np.allclose(dD2, 2 * dD) and np.allclose(db2, 2 * db)
+
+
+def _torch_attention(w, hs, lens, offs, h_t, mask, D, err_htild):
+    """Luong local-p attention from the paper's formulas in torch float64, column by column (window positions are
+    integers and carry no gradient); the scalar is <err_htild, h~>.  Returns the leaf tensors with their gradients."""
+    td = lambda a: torch.tensor(np.asarray(a, dtype=np.float64), requires_grad=True)
+    W = {k: td(w[k]) for k in ("W_a", "W_p", "W_c1", "W_c2")}
+    W["v_p"], W["out_bias"] = td(np.asarray(w["v_p"]).reshape(-1)), td(w["out_bias"])
+    HS, Ht = td(hs), td(h_t)
+    H, mb = h_t.shape
+    loss = torch.zeros((), dtype=torch.float64)
+    for b in range(mb):
+        if not mask[b]:
+            continue
+        h = Ht[:, b]
+        p = float(lens[b]) * torch.sigmoid(W["v_p"] @ torch.tanh(W["W_p"] @ h))
+        ip = int(p.item())
+        pos = list(range(max(0, ip - D), min(int(lens[b]) - 1, ip + D) + 1))
+        src = torch.stack([HS[int(lens[b]) - 1 - s + int(offs[b]), :, b] for s in pos])  # window x H
+        sc = src @ (W["W_a"].T @ h)
+        a = torch.softmax(sc, 0) * torch.exp(-(p - torch.tensor(pos, dtype=torch.float64)) ** 2 / (2 * (D / 2.0) ** 2))
+        c = a @ src
+        ht = torch.tanh(W["W_c1"] @ c + W["W_c2"] @ h + W["out_bias"])
+        loss = loss + (torch.tensor(np.asarray(err_htild[:, b], np.float64)) * ht).sum()
+    loss.backward()
+    return W, HS, Ht
+
+
+@pytest.mark.parametrize("H,mb,S,D,seed", [(10, 6, 9, 2, 1), (16, 5, 12, 12, 2), (7, 4, 30, 3, 3), (12, 3, 5, 1, 4)])
+def test_attention_backward_matches_torch_autograd(H, mb, S, D, seed):
+    """Every output of the attention backward by value against autograd: the error of h_t, of every source state, and
+    the six weight gradients; short sources, a window cut at both ends, a masked column.  A dropped term (the Gaussian's
+    derivative through p_t, the soft-max Jacobian's off-diagonal part, the W_p path into h_t) moves the result by far
+    more than the tolerance."""
+    rng = np.random.default_rng(seed)
+    w = dict(W_a=U(rng, (H, H), -0.6, 0.6), W_p=U(rng, (H, H), -0.9, 0.9), v_p=U(rng, (H,), -1.5, 1.5),
+             out_bias=U(rng, (H,), -0.3, 0.3), W_c1=U(rng, (H, H), -0.4, 0.4), W_c2=U(rng, (H, H), -0.4, 0.4))
+    hs = rng.normal(0, 0.7, size=(S, H, mb)).astype(np.float32)
+    lens = rng.integers(1, S + 1, size=mb).astype(np.int32)
+    lens[0] = S
+    offs = (S - lens).astype(np.int32)
+    mask = np.ones(mb, np.int32)
+    mask[mb - 2] = 0
+    h_t = U(rng, (H, mb), -1, 1)
+    err = U(rng, (H, mb), -1, 1)
+    binfo = np.concatenate([lens, offs])
+    fwd = o.attention_forward(hs_table=hs, batch_info=binfo, h_t=h_t, mask01=mask, D=D, **w)
+    # gradients accumulate: start them from a non-zero value and check the increment
+    g0 = {k: np.asfortranarray(U(rng, (H, H), -1, 1)) for k in ("W_a", "W_p", "W_c1", "W_c2")}
+    g0["v_p"], g0["bias"] = U(rng, (H,), -1, 1), U(rng, (H,), -1, 1)
+    ehs0 = rng.normal(0, 1, size=(S, H, mb)).astype(np.float32)
+    grads = {k: v.copy(order="F") for k, v in g0.items()}
+    err_h, err_hs, grads = o.attention_backward(w["W_a"], w["W_p"], w["v_p"], w["W_c1"], w["W_c2"], hs, binfo, h_t, mask,
+                                                fwd, err, D, grads=grads, err_hs=ehs0)
+    W, HS, Ht = _torch_attention(w, hs, lens, offs, h_t, mask, D, err)
+
+    def close(got, want, what):
+        want = np.asarray(want, np.float64)
+        tol = 2e-5 * max(1.0, np.abs(want).max())
+        assert np.abs(np.asarray(got, np.float64) - want).max() <= tol, what
+
+    close(err_h, Ht.grad.numpy(), "error of h_t")
+    close(err_hs - ehs0, HS.grad.numpy(), "error of the source states")
+    for k, t in (("W_a", "W_a"), ("W_p", "W_p"), ("W_c1", "W_c1"), ("W_c2", "W_c2"), ("v_p", "v_p"), ("bias", "out_bias")):
+        close(grads[k] - g0[k], W[t].grad.numpy(), "gradient of " + k)
+    # the terms a plausible mistake drops are large here
+    assert np.abs(W["W_p"].grad.numpy()).max() > 1e-3 and np.abs(W["W_a"].grad.numpy()).max() > 1e-3
+    assert np.all(err_h[:, mb - 2] == 0)
+
+
+def test_dropout_keeps_with_probability_rate_and_rescales():
+    """dropout_kernel: `rate` is the KEEP probability; kept values are divided by it, the others become 0."""
+    rng = np.random.default_rng(5)
+    x = U(rng, (7, 5), -2, 2)
+    u = rng.random((7, 5)).astype(np.float32)
+    u[0, 0], u[1, 0] = 0.3, np.float32(0.29999998)
+    got = o.dropout(u, 0.3, x)
+    want = np.where(u < np.float32(0.3), x * (np.float32(1) / np.float32(0.3)), 0).astype(np.float32)
+    assert np.array_equal(got, want)  # (a dropped negative value is -0, which equals 0)
+    assert got[0, 0] == 0 and got[1, 0] != 0  # strict comparison
+
+
+def test_lstm_feed_backward_matches_torch_autograd():
+    """z_g = Q_g h~ enters gate g's pre-activation: with d_g the pre-activation errors, the error of h~ is
+    sum_g Q_g^T d_g and Q_g's gradient d_g h~^T."""
+    rng = np.random.default_rng(6)
+    H, mb = 9, 4
+    Q = [U(rng, (H, H), -1, 1) for _ in range(4)]
+    ht = U(rng, (H, mb), -1, 1)
+    dg = U(rng, (4 * H, mb), -1, 1)
+    dQ0 = [np.asfortranarray(U(rng, (H, H), -1, 1)) for _ in range(4)]
+    err, dQ = o.lstm_feed_backward(Q, dg, ht, dQ=[q.copy(order="F") for q in dQ0])
+    tQ = [torch.tensor(q.astype(np.float64), requires_grad=True) for q in Q]
+    th = torch.tensor(ht.astype(np.float64), requires_grad=True)
+    loss = sum((torch.tensor(dg[g * H:(g + 1) * H].astype(np.float64)) * (tQ[g] @ th)).sum() for g in range(4))
+    loss.backward()
+    assert np.abs(err - th.grad.numpy()).max() < 1e-5
+    for g in range(4):
+        assert np.abs(dQ[g] - dQ0[g] - tQ[g].grad.numpy()).max() < 1e-5
