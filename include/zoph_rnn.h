@@ -393,6 +393,43 @@ int zr_lstm_node_backward(zr_ctx* ctx, const zr_lstm_train* layer, int mb, const
 int zr_lstm_node_gradients(zr_ctx* ctx, int H, int mb, const float* d_dgates, const float* d_in, const float* d_h_prev,
                            float* d_dM_stack, float* d_dWh_stack, float* d_db);
 
+/* The feed-input part of a bottom-layer node's backward (LSTM_IH_Node::back_prop_GPU under `feed_input && index != 0`,
+ * src/LSTM.hpp:804-866, and the Q gradient products of compute_gradients_GPU, :1014-1050):
+ *   d_err_htild (d_ERRnTOt_h_tild, H x mb, overwritten) = sum_g Q_g^T dgates_g -- the error the previous step's
+ *     attention node adds to its own (src/attention_node.hpp:416);
+ *   d_dQ_stack (4H x H, stacked over the gates like zr_lstm_node_gradients' outputs, ACCUMULATED) += dgates h~^T.
+ *   d_dgates: the node's stacked pre-activation errors (output of zr_lstm_node_backward); d_htild: the node's d_h_tild. */
+int zr_lstm_feed_backward(zr_ctx* ctx, const float* const d_Q[4], int H, int mb, const float* d_dgates,
+                          const float* d_htild, float* d_err_htild, float* d_dQ_stack);
+
+/* attention_node::back_prop (src/attention_node.hpp:398-669, single-source branch) with its kernels (zero_h_t,
+ * tanh_grad_kernel, error_alignments_kernel_large, error_hs_ct_kernel_large, error_pt_kernel, att_vp_error,
+ * grad_W_p_kernel, get_ht_scalings_Wa_grad_kernel, scale_ht_kernel, copy_errors_source: src/custom_kernels.h:1835,
+ * 1968-2196, 2212).  What the reference caches in the forward pass (tanh_1, sigma_1, W_a^T h, the Gaussian factors)
+ * is computed again from d_h_t, d_p_t and d_indices.
+ *   d_h_t: the h_t the forward step read (d_h_t_att: after the layer's dropout where that is on);
+ *   d_h_tild, d_alignments, d_indices, d_p_t, d_c_t: outputs of that zr_attn_step call;
+ *   d_err_htild: error of h~ (d_d_ERRt_ht_tild; the caller has added the feed-input error, :416);
+ *   d_err_h_t (H x mb, overwritten): error of h_t (d_ERRnTOt_ht_p1, before the dropout of :647); may be d_err_htild;
+ *   grads: the layer's six gradient arrays, ACCUMULATED into (beta = 1 in the reference);
+ *   the errors of the source states are ADDED into the arrays registered with zr_attn_set_error_tables, entry t for
+ *   the source position stored in hs table t (d_total_hs_error, src/attention_layer.hpp:106-160). */
+typedef struct zr_attn_grads {
+  float *d_W_a, *d_W_p, *d_v_p, *d_out_bias, *d_W_c1, *d_W_c2;
+} zr_attn_grads;
+int zr_attn_set_error_tables(zr_ctx* ctx, zr_attn* a, float* const* h_err_tables, int n);
+int zr_attn_backward(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, const float* d_h_t, const int* d_mask01,
+                     const float* d_h_tild, const float* d_alignments, const int* d_indices, const float* d_p_t,
+                     const float* d_c_t, const float* d_err_htild, float* d_err_h_t, const zr_attn_grads* grads);
+
+/* dropout_kernel (src/custom_kernels.h:1556-1560; forward call sites src/LSTM.hpp:118, src/LSTM_HH.hpp:124,
+ * src/attention_node.hpp:105, src/softmax.hpp:477, backward :647, src/LSTM_HH.hpp:674, src/softmax.hpp:746):
+ * x = (uniform < keep_rate) * (1 / keep_rate) * x, in place; keep_rate is the probability of KEEPING a value. */
+int zr_dropout_apply(zr_ctx* ctx, const float* d_uniform, float keep_rate, float* d_x, long long n);
+/* Fills d_out with n uniform numbers in (0, 1], a pure function of (seed, call, index): the stand-in for
+ * curandGenerateUniform (src/BZ_CUDA_UTIL.h:793-795), whose stream cannot be reproduced. */
+int zr_uniform_fill(zr_ctx* ctx, unsigned long long seed, unsigned long long call, float* d_out, long long n);
+
 /* Embedding gradient (the sparse W gradient kernels, src/custom_kernels.h:1297-1390): d_dW[:, id[k]] += d_err[:, k]
  * for the n unmasked positions; d_dW is H x V and is accumulated into (zero it first).  Uses float atomics, like
  * the reference: the summation order within a column is not fixed. */

@@ -321,3 +321,103 @@ def test_softmax_backward_step_by_step_accumulates(ctx, V, H, mb, T):
         assert_close(d_e.get(), want_e[t], what="err_h step %d" % t)
     assert_close(d_dD.get(), dD, floor=0.05 * np.sqrt(T * mb), what="dD")
     assert_close(d_db.get(), db, floor=0.05 * np.sqrt(T * mb), what="db")
+
+
+@pytest.mark.parametrize("H,mb,S,D", [(64, 6, 9, 2), (100, 8, 20, 10), (52, 33, 12, 12), (30, 5, 7, 3), (300, 70, 40, 50),
+                                      (1000, 16, 30, 10)])
+def test_attention_backward_against_oracle(ctx, H, mb, S, D):
+    """zr_attn_backward (attention_node::back_prop) against the oracle, whose restatement is pinned by torch autograd:
+    the error of h_t, the error added to every source state, and the six weight gradients, all accumulated on top of
+    non-zero starting values; short sources, windows cut at both ends, masked columns, row tails."""
+    g = synth.rng(41, H + S)
+    w = synth.attention_weights(g, H)
+    if H <= 128:
+        for k in ("W_a", "W_p", "W_c1", "W_c2"):
+            w[k] = U(g, (H, H), -0.3, 0.3)
+    hs = (g.standard_normal(size=(S, H, mb), dtype=np.float32) * np.float32(0.5 if H <= 128 else 0.1))
+    lens = g.integers(1, S + 1, size=mb).astype(np.int32)
+    lens[0] = S
+    batch_info = np.concatenate([lens, S - lens]).astype(np.int32)
+    mask = (g.random(mb) > 0.15).astype(np.int32)
+    mask[0] = 1
+    h_t = U(g, (H, mb), -1, 1)
+    err = U(g, (H, mb), -1, 1)
+    fwd = o.attention_forward(hs_table=hs, batch_info=batch_info, h_t=h_t, mask01=mask, D=D, **w)
+    g0 = {k: np.asfortranarray(U(g, (H, H), -0.5, 0.5)) for k in ("W_a", "W_p", "W_c1", "W_c2")}
+    g0["v_p"], g0["bias"] = U(g, (H,), -0.5, 0.5), U(g, (H,), -0.5, 0.5)
+    ehs0 = (g.standard_normal(size=(S, H, mb), dtype=np.float32) * np.float32(0.5))
+    want_eh, want_ehs, want_g = o.attention_backward(w["W_a"], w["W_p"], w["v_p"], w["W_c1"], w["W_c2"], hs, batch_info,
+                                                     h_t, mask, fwd, err, D,
+                                                     grads={k: v.copy(order="F") for k, v in g0.items()}, err_hs=ehs0)
+    # the library's own forward outputs feed its backward, as in training
+    tables = [ctx.array(np.asfortranarray(hs[t])) for t in range(S)]
+    etables = [ctx.array(np.asfortranarray(ehs0[t])) for t in range(S)]
+    dw = {k: ctx.array(v) for k, v in w.items()}
+    a = ctx.attn_create(H, mb, D, dw["W_a"], dw["W_p"], dw["v_p"], dw["out_bias"], dw["W_c1"], dw["W_c2"], tables)
+    ctx.attn_set_error_tables(a, etables)
+    Wn = 2 * D + 1
+    d_ht, d_al, d_ix, d_pt, d_cx = (ctx.empty((H, mb)), ctx.empty((mb, Wn)), ctx.empty((mb, Wn), np.int32),
+                                    ctx.empty((mb,)), ctx.empty((H, mb)))
+    d_bi, d_h, d_m = ctx.array(batch_info), ctx.array(h_t), ctx.array(mask)
+    ctx.attn_step(a, d_bi, d_h, d_m, d_ht, d_al, d_ix, d_pt, d_cx)
+    d_g = [ctx.array(g0[k]) for k in ("W_a", "W_p", "v_p", "bias", "W_c1", "W_c2")]
+    d_err, d_eh = ctx.array(err), ctx.empty((H, mb))
+    ctx.attn_backward(a, d_bi, d_h, d_m, d_ht, d_al, d_ix, d_pt, d_cx, d_err, d_eh, d_g)
+    ctx.sync()
+    assert np.array_equal(d_ix.get(), fwd["indices"])
+    assert_close(d_eh.get(), want_eh, what="error of h_t")
+    for t in range(S):
+        assert_close(etables[t].get(), want_ehs[t], what="error of source state %d" % t)
+    for d, k in zip(d_g, ("W_a", "W_p", "v_p", "bias", "W_c1", "W_c2")):
+        assert_close(d.get().reshape(want_g[k].shape, order="F"), want_g[k], what="gradient of " + k)
+    assert np.all(d_eh.get()[:, mask == 0] == 0)
+    # in place: the error of h_t may overwrite the error of h~ (the reference copies it there, :654)
+    for d, k in zip(d_g, ("W_a", "W_p", "v_p", "bias", "W_c1", "W_c2")):
+        d.set(g0[k])
+    ctx.attn_backward(a, d_bi, d_h, d_m, d_ht, d_al, d_ix, d_pt, d_cx, d_err, d_err, d_g)
+    ctx.sync()
+    assert d_err.get().tobytes() == d_eh.get().tobytes()
+    ctx.attn_destroy(a)
+
+
+@pytest.mark.parametrize("n,rate", [(1000, 0.8), (70001, 0.3), (5, 1.0)])
+def test_dropout_apply_bit_exact_and_uniform_fill(ctx, n, rate):
+    """dropout_kernel on given uniform numbers: bit for bit the oracle's; the library's own uniform numbers lie in
+    (0, 1], repeat for the same (seed, call) and differ for another call, with the mean and keep fraction of a uniform
+    sample."""
+    g = synth.rng(43, n)
+    x = U(g, (n,), -2, 2)
+    u = g.random(n, dtype=np.float32)
+    d_x, d_u = ctx.array(x), ctx.array(u)
+    ctx.dropout_apply(d_u, rate, d_x, n)
+    ctx.sync()
+    assert np.array_equal(d_x.get(), o.dropout(u, rate, x))
+    a, b, c = ctx.empty((n,)), ctx.empty((n,)), ctx.empty((n,))
+    ctx.uniform_fill(1234, 7, a, n)
+    ctx.uniform_fill(1234, 7, b, n)
+    ctx.uniform_fill(1234, 8, c, n)
+    ctx.sync()
+    ua, uc = a.get(), c.get()
+    assert ua.tobytes() == b.get().tobytes() and not np.array_equal(ua, uc)
+    assert ua.min() > 0 and ua.max() <= 1
+    if n >= 1000:
+        assert abs(ua.mean() - 0.5) < 4 * 0.2887 / np.sqrt(n)
+        assert abs((ua < 0.3).mean() - 0.3) < 4 * np.sqrt(0.21 / n)
+        assert abs(np.corrcoef(ua[:-1], ua[1:])[0, 1]) < 5 / np.sqrt(n)
+
+
+@pytest.mark.parametrize("H,mb", [(48, 9), (100, 33), (1000, 16)])
+def test_lstm_feed_backward_against_oracle(ctx, H, mb):
+    g = synth.rng(44, H)
+    Q = [U(g, (H, H), -0.3, 0.3) for _ in range(4)]
+    ht = U(g, (H, mb), -1, 1)
+    dg = U(g, (4 * H, mb), -1, 1)
+    dQ0 = U(g, (4 * H, H), -0.5, 0.5)
+    want_err, want_dQ = o.lstm_feed_backward(Q, dg, ht, dQ=[np.asfortranarray(dQ0[k * H:(k + 1) * H]) for k in range(4)])
+    d_err, d_dQ = ctx.empty((H, mb)), ctx.array(dQ0)
+    ctx.lstm_feed_backward([ctx.array(q) for q in Q], H, mb, ctx.array(dg), ctx.array(ht), d_err, d_dQ)
+    ctx.sync()
+    assert_close(d_err.get(), want_err, what="error of h~")
+    got = d_dQ.get()
+    for k in range(4):
+        assert_close(got[k * H:(k + 1) * H], want_dQ[k], what="gradient of Q[%d]" % k)

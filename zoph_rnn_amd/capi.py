@@ -43,7 +43,8 @@ SYMBOLS = [
     "zr_unstack_gates", "zr_lstm_stack_backward", "zr_lstm_weight_gradients", "zr_embed_gradient",
     "zr_softmax_backward", "zr_sgd_update", "zr_lstm_node_backward", "zr_lstm_node_gradients",
     "zr_softmax_backward_accumulate", "zr_gather_columns_multi", "zr_softmax_backward_loss",
-    "zr_softmax_forward_static", "zr_ctx_query", "zr_attn_prepare", "zr_lstm_step_embed", "zr_attn_viterbi", "zr_lstm_decoder_step",
+    "zr_softmax_forward_static", "zr_ctx_query", "zr_attn_prepare", "zr_lstm_step_embed", "zr_attn_viterbi", "zr_lstm_decoder_step", "zr_lstm_feed_backward", "zr_attn_set_error_tables",
+    "zr_attn_backward", "zr_dropout_apply", "zr_uniform_fill",
 ]
 
 _lib = None
@@ -272,6 +273,26 @@ class Context:
     def lstm_weight_gradients(self, H, T, mb, d_dgates, d_in_all, d_h0, d_h_all, d_dM, d_dWh, d_db):
         _chk(load().zr_lstm_weight_gradients(self.h, C.c_int(H), C.c_int(T), C.c_int(mb), _vp(d_dgates), _vp(d_in_all),
                                              _vp(d_h0), _vp(d_h_all), _vp(d_dM), _vp(d_dWh), _vp(d_db)))
+
+    def lstm_feed_backward(self, Q, H, mb, d_dgates, d_htild, d_err_htild, d_dQ_stack):
+        _chk(load().zr_lstm_feed_backward(self.h, _ptr_array(Q), C.c_int(H), C.c_int(mb), _vp(d_dgates), _vp(d_htild),
+                                          _vp(d_err_htild), _vp(d_dQ_stack)))
+
+    def attn_set_error_tables(self, attn, tables):
+        _chk(load().zr_attn_set_error_tables(self.h, attn, _ptr_array(tables), C.c_int(len(tables))))
+
+    def attn_backward(self, attn, d_batch_info, d_h_t, d_mask, d_h_tild, d_align, d_idx, d_p_t, d_c_t, d_err_htild,
+                      d_err_h_t, grads):
+        """grads: six device arrays in the order W_a, W_p, v_p, out_bias, W_c1, W_c2 (accumulated into)."""
+        g = _ptr_array(grads)  # zr_attn_grads: six pointers
+        _chk(load().zr_attn_backward(self.h, attn, _vp(d_batch_info), _vp(d_h_t), _vp(d_mask), _vp(d_h_tild), _vp(d_align),
+                                     _vp(d_idx), _vp(d_p_t), _vp(d_c_t), _vp(d_err_htild), _vp(d_err_h_t), g))
+
+    def dropout_apply(self, d_uniform, keep_rate, d_x, n):
+        _chk(load().zr_dropout_apply(self.h, _vp(d_uniform), C.c_float(keep_rate), _vp(d_x), C.c_longlong(n)))
+
+    def uniform_fill(self, seed, call, d_out, n):
+        _chk(load().zr_uniform_fill(self.h, C.c_ulonglong(seed), C.c_ulonglong(call), _vp(d_out), C.c_longlong(n)))
 
     def lstm_node_backward(self, layer, mb, gates, d_c, d_c_prev, d_mask, d_err_above, d_err_h_next, d_err_c_next,
                            d_dgates, d_err_h_prev, d_err_c_prev, d_err_below=None):

@@ -8,22 +8,6 @@
 
 #include "zr_internal.h"
 
-struct zr_attn {
-  int H, mb, D, longest_sent;
-  bool tables_aligned;  // every source table is 16-byte aligned
-  const float *W_a, *W_p, *v_p, *out_bias, *W_c1, *W_c2;  // borrowed device pointers
-  const float** d_table;                                   // device copy of the pointer table
-  float *d_tanh1, *d_q, *d_align, *d_pt, *d_ctx;
-  int* d_idx;
-  // zr_attn_use_bf16_weights: owned bf16 k-interleaved snapshots of W_p, W_a^T, W_c1, W_c2 ([H/8][ldp][8] each)
-  unsigned short* d_bf16;
-  int ldp;
-  // zr_attn_prepare: owned fp32 k-interleaved snapshots ([kp/4][ldp32][4] each) of W_p, W_a^T, W_c1, W_c2 in that
-  // order, and the raw (pre-tanh) W_p h product next to q
-  float* d_pack32;
-  int ldp32, kp32;
-  float *d_hpack, *d_cpack;  // k-interleaved copies ([H/4][mb][4]) of h_t and of the context (inside d_pack32's block)
-};
 
 namespace {
 
@@ -489,6 +473,7 @@ int zr_attn_create(zr_ctx* ctx, int H, int mb, int D, const float* d_W_a, const 
   a->d_bf16 = nullptr;
   a->ldp = 0;
   a->d_pack32 = nullptr;
+  a->d_err_table = nullptr;
   a->ldp32 = a->kp32 = 0;
   const size_t n = (size_t)H * mb, W = 2 * (size_t)D + 1;
   // one allocation: table | tanh1 | q | ctx | align | p_t | idx
@@ -590,6 +575,7 @@ int zr_attn_destroy(zr_ctx* ctx, zr_attn* a) {
   ZR_HIP(hipStreamSynchronize(ctx->stream));
   if (a->d_bf16) (void)hipFree(a->d_bf16);
   if (a->d_pack32) (void)hipFree(a->d_pack32);
+  if (a->d_err_table) (void)hipFree((void*)a->d_err_table);
   (void)hipFree((void*)a->d_table);
   delete a;
   return ZR_OK;

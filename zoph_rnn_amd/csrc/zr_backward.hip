@@ -1,4 +1,4 @@
-// Training backward for the stacked LSTM and the output layer (no attention, no dropout).
+// Training backward for the stacked LSTM, the output layer and the attention layer; dropout.
 //
 // Gradients are those of the log-likelihood, as in the reference (its loss layer's error is D^T (onehot - p),
 // src/softmax.hpp:700-712; update_weights adds learning_rate * gradient, :232-300).
@@ -330,6 +330,182 @@ __global__ void __launch_bounds__(256) sgd_apply_kernel(float* __restrict__ W, c
   for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) W[i] += f * g[i];
 }
 
+
+// ---- attention backward (attention_node::back_prop, src/attention_node.hpp:398-669) --------------------------------
+
+__device__ __forceinline__ float bwd_wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+// Sum over the 256 threads of a workgroup, in every thread.  `red` holds 4 floats.
+__device__ __forceinline__ float bwd_block_sum(float v, float* red) {
+  v = bwd_wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+// zero_h_t + tanh_grad_kernel (src/custom_kernels.h:2212, :1835): e = err * mask * (1 - h~^2)
+__global__ void __launch_bounds__(256) attn_bwd_e_kernel(const float* __restrict__ err, const float* __restrict__ htild,
+                                                         const int* __restrict__ mask01, int H, long long n,
+                                                         float* __restrict__ e) {
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) {
+    const float t = htild[i];
+    e[i] = err[i] * (float)mask01[i / H] * (1.0f - t * t);
+  }
+}
+
+// error_alignments_kernel_large + error_hs_ct_kernel_large (:1968, :2179), one workgroup per (window slot, column):
+// err_as[j + W*b] = <err_ct[:, b], h_s>, and the error of that source state += err_ct[:, b] * a.  Distinct slots of a
+// column are distinct source positions, so no two workgroups touch the same error column.
+__global__ void __launch_bounds__(256) attn_bwd_align_kernel(const float* __restrict__ err_ct,
+                                                             const float* const* __restrict__ table,
+                                                             float* const* __restrict__ err_table,
+                                                             const int* __restrict__ batch_info,
+                                                             const int* __restrict__ indices,
+                                                             const float* __restrict__ align, int H, int mb, int W,
+                                                             int longest, float* __restrict__ err_as) {
+  __shared__ float red[4];
+  const int j = blockIdx.x, b = blockIdx.y;
+  const int s = indices[b + (size_t)mb * j];
+  if (s == -1) {
+    if (threadIdx.x == 0) err_as[j + (size_t)W * b] = 0.0f;
+    return;
+  }
+  int t = batch_info[b] - 1 - s + batch_info[mb + b];
+  t = t < 0 ? 0 : (t >= longest ? longest - 1 : t);
+  const float* hs = table[t] + (size_t)b * H;
+  float* ehs = err_table[t] + (size_t)b * H;
+  const float* ec = err_ct + (size_t)b * H;
+  const float a = align[b + (size_t)mb * j];
+  float sum = 0.0f;
+  for (int i = threadIdx.x; i < H; i += 256) {
+    const float v = ec[i];
+    sum += v * hs[i];
+    ehs[i] += v * a;
+  }
+  sum = bwd_block_sum(sum, red);
+  if (threadIdx.x == 0) err_as[j + (size_t)W * b] = sum;
+}
+
+// Per column: sigma_1 again (sigmoid_kernel, double), error_pt_kernel (:2006), the factors of att_vp_error and
+// grad_W_p_kernel (:2040, :2051) that depend on the column only, and get_ht_scalings_Wa_grad_kernel (:2094) with the
+// Gaussian factors alignment_reduction_kernel caches (1 on empty slots).
+//   col[0][b] = err_pt * sig * (1 - sig) * S_b     (times tanh_1: the v_p gradient's summand)
+//   col[1][b] = err_pt * S_b,  col[2][b] = sig     (grad_W_p_kernel multiplies in the reference's order)
+__global__ void __launch_bounds__(64) attn_bwd_column_kernel(const float* __restrict__ tanh1,
+                                                             const float* __restrict__ v_p,
+                                                             const int* __restrict__ batch_info,
+                                                             const int* __restrict__ indices,
+                                                             const float* __restrict__ align,
+                                                             const float* __restrict__ p_t,
+                                                             const float* __restrict__ err_as, int H, int mb, int W,
+                                                             float sigma_sq, float* __restrict__ col,
+                                                             float* __restrict__ scal) {
+  const int b = blockIdx.x, lane = threadIdx.x;
+  float s = 0.0f;
+  for (int k = lane; k < H; k += 64) s += v_p[k] * tanh1[(size_t)b * H + k];
+  s = bwd_wave_sum(s);
+  const float sig = (float)(1.0 / (1.0 + exp(-1.0 * (double)s)));
+  const float p = p_t[b];
+  float ept = 0.0f, tot = 0.0f;  // tot = sum_k err_as[k] * a_k
+  for (int j = lane; j < W; j += 64) {
+    const float ea = err_as[j + (size_t)W * b] * align[b + (size_t)mb * j];
+    tot += ea;
+    ept += ea * (((float)indices[b + (size_t)mb * j] - p) / sigma_sq);
+  }
+  ept = bwd_wave_sum(ept);
+  tot = bwd_wave_sum(tot);
+  const float len = (float)batch_info[b];
+  if (lane == 0) {
+    col[b] = ept * sig * (1.0f - sig) * len;
+    col[mb + b] = ept * len;
+    col[2 * mb + b] = sig;
+  }
+  // scaling_j = err_as_j a_j (1 - a_j / g_j) - sum_{k != j} err_as_k a_k a_j / g_j  =  err_as_j a_j - (a_j / g_j) tot:
+  // the reference's sum with the j-th term folded in, O(W) per slot instead of O(W^2)
+  for (int j = lane; j < W; j += 64) {
+    const int sidx = indices[b + (size_t)mb * j];
+    float g = 1.0f;
+    if (sidx != -1) {
+      const float d = p - (float)sidx;
+      g = expf((-1.0f * d * d) / (2.0f * sigma_sq));
+    }
+    const float aj = align[b + (size_t)mb * j];
+    scal[j + (size_t)W * b] = err_as[j + (size_t)W * b] * aj - (aj / g) * tot;
+  }
+}
+
+// att_vp_error and grad_W_p_kernel (:2040, :2051) in one pass over tanh_1
+__global__ void __launch_bounds__(256) attn_bwd_vp_wp_kernel(const float* __restrict__ tanh1,
+                                                             const float* __restrict__ v_p,
+                                                             const float* __restrict__ col, int H, int mb, long long n,
+                                                             float* __restrict__ tv, float* __restrict__ tw) {
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) {
+    const int b = (int)(i / H), k = (int)(i % H);
+    const float t = tanh1[i], sig = col[2 * mb + b];
+    tv[i] = col[b] * t;
+    tw[i] = col[mb + b] * v_p[k] * sig * (1.0f - sig) * (1.0f - t * t);
+  }
+}
+
+// The loop of src/attention_node.hpp:580-601 for one column per workgroup: h_s_sum[:, b] = sum_j scaling_j h_s_j
+// (scale_ht_kernel + add_two_mats_kernel) and the error of h_s_j += scaling_j * (W_a^T h)[:, b] (copy_errors_source).
+__global__ void __launch_bounds__(256) attn_bwd_hs_kernel(const float* __restrict__ q,
+                                                          const float* const* __restrict__ table,
+                                                          float* const* __restrict__ err_table,
+                                                          const int* __restrict__ batch_info,
+                                                          const int* __restrict__ indices,
+                                                          const float* __restrict__ scal, int H, int mb, int W,
+                                                          int longest, float* __restrict__ hs_sum) {
+  const int b = blockIdx.x;
+  const int len = batch_info[b], off = batch_info[mb + b];
+  for (int i0 = 0; i0 < H; i0 += 256) {
+    const int i = i0 + threadIdx.x;
+    const bool ok = i < H;
+    const float qv = ok ? q[(size_t)b * H + i] : 0.0f;
+    float acc = 0.0f;
+    for (int j = 0; j < W; ++j) {
+      const int s = indices[b + (size_t)mb * j];
+      if (s == -1) continue;
+      int t = len - 1 - s + off;
+      t = t < 0 ? 0 : (t >= longest ? longest - 1 : t);
+      const float sc = scal[j + (size_t)W * b];
+      if (ok) {
+        acc += table[t][(size_t)b * H + i] * sc;
+        err_table[t][(size_t)b * H + i] += qv * sc;
+      }
+    }
+    if (ok) hs_sum[(size_t)b * H + i] = acc;
+  }
+}
+
+// dropout_kernel (src/custom_kernels.h:1556-1560)
+__global__ void __launch_bounds__(256) dropout_kernel(const float* __restrict__ uniform, float rate, float* __restrict__ x,
+                                                      long long n) {
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
+    x[i] = (float)(uniform[i] < rate) * (1.0f / rate) * x[i];
+}
+
+// Uniform numbers in (0, 1] from a counter-based generator (the reference fills its masks with curandGenerateUniform,
+// whose stream cannot be reproduced; what matters is that the numbers are uniform, independent of each other and a
+// pure function of (seed, call counter, index)): 32 bits of a 64-bit mix of the three, as (bits + 1) * 2^-32 rounded
+// to float -- curand's convention, which never returns 0.
+__global__ void __launch_bounds__(256) uniform_fill_kernel(unsigned long long seed, unsigned long long call,
+                                                           float* __restrict__ out, long long n) {
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) {
+    unsigned long long z = seed + 0x9E3779B97F4A7C15ULL * (call * 0x100000001B3ULL + (unsigned long long)i + 1ULL);
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ULL;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBULL;
+    z = z ^ (z >> 31);
+    const unsigned bits = (unsigned)(z >> 32);
+    float u = ((float)bits + 1.0f) * 2.3283064365386963e-10f;
+    out[i] = u > 1.0f ? 1.0f : u;
+  }
+}
+
 int row_sum_launch(zr_ctx* ctx, const float* a, int rows, long long n, float* out, int accumulate = 0) {
   const long long chunk = 64;
   const int chunks = (int)((n + chunk - 1) / chunk);
@@ -651,6 +827,200 @@ int zr_lstm_node_backward(zr_ctx* ctx, const zr_lstm_train* layer, int mb, const
       ZR_HIP(hipMemcpyAsync(d_err_below, out + n, sizeof(float) * n, hipMemcpyDeviceToDevice, ctx->stream));
   }
   return ZR_OK;
+}
+
+int zr_attn_set_error_tables(zr_ctx* ctx, zr_attn* a, float* const* h_err_tables, int n) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(a && h_err_tables, "zr_attn_set_error_tables: null pointer");
+  ZR_CHECK_ARG(n == a->longest_sent, "zr_attn_set_error_tables: %d tables, the layer has %d source positions", n,
+               a->longest_sent);
+  for (int t = 0; t < n; ++t) ZR_CHECK_ARG(h_err_tables[t] != nullptr, "zr_attn_set_error_tables: entry %d is null", t);
+  if (!a->d_err_table) {
+    if (hipMalloc((void**)&a->d_err_table, sizeof(float*) * n) != hipSuccess) {
+      (void)hipGetLastError();
+      a->d_err_table = nullptr;
+      return zr_set_error(ZR_ENOMEM, "zr_attn_set_error_tables: allocation failed");
+    }
+  }
+  ZR_HIP(hipStreamSynchronize(ctx->stream));
+  ZR_HIP(hipMemcpy((void*)a->d_err_table, h_err_tables, sizeof(float*) * n, hipMemcpyHostToDevice));
+  return ZR_OK;
+}
+
+int zr_attn_backward(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, const float* d_h_t, const int* d_mask01,
+                     const float* d_h_tild, const float* d_alignments, const int* d_indices, const float* d_p_t,
+                     const float* d_c_t, const float* d_err_htild, float* d_err_h_t, const zr_attn_grads* grads) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(a != nullptr, "zr_attn_backward: attention object is null");
+  ZR_CHECK_ARG(a->d_err_table != nullptr, "zr_attn_backward: call zr_attn_set_error_tables first");
+  ZR_CHECK_ARG(d_batch_info && d_h_t && d_mask01 && d_h_tild && d_alignments && d_indices && d_p_t && d_c_t &&
+                   d_err_htild && d_err_h_t && grads,
+               "zr_attn_backward: null pointer");
+  ZR_CHECK_ARG(grads->d_W_a && grads->d_W_p && grads->d_v_p && grads->d_out_bias && grads->d_W_c1 && grads->d_W_c2,
+               "zr_attn_backward: null gradient array");
+  ZR_CHECK_ARG(a->D >= 1, "zr_attn_backward: D = %d (the Gaussian's width D/2 must be positive)", a->D);
+  const int H = a->H, mb = a->mb, W = 2 * a->D + 1;
+  const size_t n = (size_t)H * mb;
+  const float sigma_sq = (float)((a->D * a->D) / 4.0);  // src/attention_node.hpp:50
+  void* scratch = nullptr;
+  rc = zr_ctx_scratch(ctx, 1, sizeof(float) * (6 * n + 2 * (size_t)W * mb + 3 * (size_t)mb), &scratch);
+  if (rc) return rc;
+  float* e = (float*)scratch;
+  float* err_ct = e + n;
+  float* tv = e + 2 * n;
+  float* tw = e + 3 * n;
+  float* hs_sum = e + 4 * n;
+  float* tr = e + 5 * n;  // a transposed right-hand side, mb x H
+  float* err_as = e + 6 * n;
+  float* scal = err_as + (size_t)W * mb;
+  float* col = scal + (size_t)W * mb;
+  const int eg = (int)((n + 255) / 256 < 2048 ? (n + 255) / 256 : 2048);
+
+  // C (H x H) += A (H x mb) * B^T for B H x mb (cuBLAS gemm N, T with beta = 1 in the reference)
+  auto outer_acc = [&](const float* A, const float* B, float* C) -> int {
+    int r = transpose_launch(ctx, B, H, mb, tr, mb, 0);
+    if (r) return r;
+    ZrGemmDesc g = {};
+    g.M = H;
+    g.N = H;
+    g.nseg = 1;
+    g.K[0] = mb;
+    g.A[0] = A;
+    g.lda[0] = H;
+    g.B[0] = tr;
+    g.ldb[0] = mb;
+    g.C = C;
+    g.ldc = H;
+    g.batch = 1;
+    g.epilogue = ZR_EPI_STORE;
+    g.accumulate = 1;
+    return zr_gemm_launch(ctx, g);
+  };
+  // C (H x mb) (+)= op(A) (H x H) * B (H x mb)
+  auto product = [&](const float* A, int trans, const float* B, float* C, int accumulate, int epilogue) -> int {
+    ZrGemmDesc g = {};
+    g.M = H;
+    g.N = mb;
+    g.nseg = 1;
+    g.K[0] = H;
+    g.A[0] = A;
+    g.lda[0] = H;
+    g.trans_a = trans;
+    g.B[0] = B;
+    g.ldb[0] = H;
+    g.C = C;
+    g.ldc = H;
+    g.batch = 1;
+    g.epilogue = epilogue;
+    g.accumulate = accumulate;
+    return zr_gemm_launch(ctx, g);
+  };
+
+  attn_bwd_e_kernel<<<eg, 256, 0, ctx->stream>>>(d_err_htild, d_h_tild, d_mask01, H, (long long)n, e);
+  ZR_LAUNCH_CHECK("attn_bwd_e_kernel");
+  if ((rc = outer_acc(e, d_c_t, grads->d_W_c1))) return rc;                     // :437
+  if ((rc = outer_acc(e, d_h_t, grads->d_W_c2))) return rc;                     // :443
+  if ((rc = row_sum_launch(ctx, e, H, mb, grads->d_out_bias, 1))) return rc;    // :456
+  if ((rc = product(a->W_c1, 1, e, err_ct, 0, ZR_EPI_STORE))) return rc;        // :464
+  if ((rc = product(a->W_c2, 1, e, d_err_h_t, 0, ZR_EPI_STORE))) return rc;     // :476
+  attn_bwd_align_kernel<<<dim3(W, mb), 256, 0, ctx->stream>>>(err_ct, a->d_table, a->d_err_table, d_batch_info, d_indices,
+                                                              d_alignments, H, mb, W, a->longest_sent, err_as);
+  ZR_LAUNCH_CHECK("attn_bwd_align_kernel");
+  if ((rc = product(a->W_p, 0, d_h_t, a->d_tanh1, 0, ZR_EPI_TANH))) return rc;  // tanh_1 of the forward pass again
+  attn_bwd_column_kernel<<<mb, 64, 0, ctx->stream>>>(a->d_tanh1, a->v_p, d_batch_info, d_indices, d_alignments, d_p_t,
+                                                     err_as, H, mb, W, sigma_sq, col, scal);
+  ZR_LAUNCH_CHECK("attn_bwd_column_kernel");
+  attn_bwd_vp_wp_kernel<<<eg, 256, 0, ctx->stream>>>(a->d_tanh1, a->v_p, col, H, mb, (long long)n, tv, tw);
+  ZR_LAUNCH_CHECK("attn_bwd_vp_wp_kernel");
+  if ((rc = row_sum_launch(ctx, tv, H, mb, grads->d_v_p, 1))) return rc;        // :536
+  if ((rc = outer_acc(tw, d_h_t, grads->d_W_p))) return rc;                     // :545
+  if ((rc = product(a->W_p, 1, tw, d_err_h_t, 1, ZR_EPI_STORE))) return rc;     // :551
+  if ((rc = product(a->W_a, 1, d_h_t, a->d_q, 0, ZR_EPI_STORE))) return rc;     // W_a^T h of the forward pass again
+  attn_bwd_hs_kernel<<<mb, 256, 0, ctx->stream>>>(a->d_q, a->d_table, a->d_err_table, d_batch_info, d_indices, scal, H, mb,
+                                                  W, a->longest_sent, hs_sum);
+  ZR_LAUNCH_CHECK("attn_bwd_hs_kernel");
+  if ((rc = outer_acc(d_h_t, hs_sum, grads->d_W_a))) return rc;                 // :632
+  return product(a->W_a, 0, hs_sum, d_err_h_t, 1, ZR_EPI_STORE);                // :636
+}
+
+int zr_dropout_apply(zr_ctx* ctx, const float* d_uniform, float keep_rate, float* d_x, long long n) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(d_uniform && d_x && n >= 0, "zr_dropout_apply: null pointer or n = %lld", n);
+  ZR_CHECK_ARG(keep_rate > 0.0f && keep_rate <= 1.0f, "zr_dropout_apply: keep rate %g not in (0, 1]", (double)keep_rate);
+  if (n == 0) return ZR_OK;
+  const int grid = (int)((n + 255) / 256 < 2048 ? (n + 255) / 256 : 2048);
+  dropout_kernel<<<grid, 256, 0, ctx->stream>>>(d_uniform, keep_rate, d_x, n);
+  ZR_LAUNCH_CHECK("dropout_kernel");
+  return ZR_OK;
+}
+
+int zr_uniform_fill(zr_ctx* ctx, unsigned long long seed, unsigned long long call, float* d_out, long long n) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(d_out && n >= 0, "zr_uniform_fill: null pointer or n = %lld", n);
+  if (n == 0) return ZR_OK;
+  const int grid = (int)((n + 255) / 256 < 2048 ? (n + 255) / 256 : 2048);
+  uniform_fill_kernel<<<grid, 256, 0, ctx->stream>>>(seed, call, d_out, n);
+  ZR_LAUNCH_CHECK("uniform_fill_kernel");
+  return ZR_OK;
+}
+
+int zr_lstm_feed_backward(zr_ctx* ctx, const float* const d_Q[4], int H, int mb, const float* d_dgates,
+                          const float* d_htild, float* d_err_htild, float* d_dQ_stack) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(H > 0 && mb > 0, "zr_lstm_feed_backward: H = %d, mb = %d", H, mb);
+  ZR_CHECK_ARG(d_Q && d_dgates && d_htild && d_err_htild && d_dQ_stack, "zr_lstm_feed_backward: null pointer");
+  for (int g = 0; g < 4; ++g) ZR_CHECK_ARG(d_Q[g] != nullptr, "zr_lstm_feed_backward: Q matrix %d is null", g);
+  // error of h~ = sum_g Q_g^T d_g (src/LSTM.hpp:804-857: four products and add_four_matrices_kernel)
+  for (int half = 0; half < 2; ++half) {
+    ZrGemmDesc g = {};
+    g.M = H;
+    g.N = mb;
+    g.nseg = 2;
+    for (int s = 0; s < 2; ++s) {
+      const int gate = 2 * half + s;
+      g.K[s] = H;
+      g.A[s] = d_Q[gate];
+      g.lda[s] = H;
+      g.B[s] = d_dgates + (size_t)gate * H;
+      g.ldb[s] = 4 * H;
+    }
+    g.trans_a = 1;
+    g.C = d_err_htild;
+    g.ldc = H;
+    g.batch = 1;
+    g.epilogue = ZR_EPI_STORE;
+    g.accumulate = half;
+    rc = zr_gemm_launch(ctx, g);
+    if (rc) return rc;
+  }
+  // Q gradients, stacked over the gates like the M and W_h gradients: dQ (4H x H) += dgates (4H x mb) * h~^T
+  // (src/LSTM.hpp:1014-1050)
+  void* scratch = nullptr;
+  rc = zr_ctx_scratch(ctx, 1, sizeof(float) * (size_t)H * mb, &scratch);
+  if (rc) return rc;
+  float* tr = (float*)scratch;
+  rc = transpose_launch(ctx, d_htild, H, mb, tr, mb, 0);
+  if (rc) return rc;
+  ZrGemmDesc w = {};
+  w.M = 4 * H;
+  w.N = H;
+  w.nseg = 1;
+  w.K[0] = mb;
+  w.A[0] = d_dgates;
+  w.lda[0] = 4 * H;
+  w.B[0] = tr;
+  w.ldb[0] = mb;
+  w.C = d_dQ_stack;
+  w.ldc = 4 * H;
+  w.batch = 1;
+  w.epilogue = ZR_EPI_STORE;
+  w.accumulate = 1;
+  return zr_gemm_launch(ctx, w);
 }
 
 int zr_embed_gradient(zr_ctx* ctx, int H, int V, const float* d_err, const int* d_ids_nonneg, const int* d_mask01,

@@ -167,4 +167,23 @@ struct zr_lstm_weights {
   float* d_bias;   // [4][H]
 };
 
+// The attention layer's handle (zr_attention.hip; the backward pass lives in zr_backward.hip).
+struct zr_attn {
+  int H, mb, D, longest_sent;
+  bool tables_aligned;  // every source table is 16-byte aligned
+  const float *W_a, *W_p, *v_p, *out_bias, *W_c1, *W_c2;  // borrowed device pointers
+  const float** d_table;                                   // device copy of the pointer table
+  float *d_tanh1, *d_q, *d_align, *d_pt, *d_ctx;
+  int* d_idx;
+  // zr_attn_use_bf16_weights: owned bf16 k-interleaved snapshots of W_p, W_a^T, W_c1, W_c2 ([H/8][ldp][8] each)
+  unsigned short* d_bf16;
+  int ldp;
+  // zr_attn_prepare: owned fp32 k-interleaved snapshots ([kp/4][ldp32][4] each) of W_p, W_a^T, W_c1, W_c2 in that
+  // order, and the raw (pre-tanh) W_p h product next to q
+  float* d_pack32;
+  int ldp32, kp32;
+  float *d_hpack, *d_cpack;  // k-interleaved copies ([H/4][mb][4]) of h_t and of the context (inside d_pack32's block)
+  float** d_err_table;       // zr_attn_set_error_tables: device copy of the source-state error pointers (null: none)
+};
+
 #endif
