@@ -108,6 +108,9 @@ int zr_h2d(zr_ctx* ctx, void* d_dst, const void* h_src, size_t bytes);
 int zr_d2h(zr_ctx* ctx, void* h_dst, const void* d_src, size_t bytes); /* synchronous with the stream */
 int zr_d2d(zr_ctx* ctx, void* d_dst, const void* d_src, size_t bytes);
 int zr_memset_zero(zr_ctx* ctx, void* d_dst, size_t bytes);
+/* d_dst[i] += d_src[i] (add_two_mats_kernel, src/custom_kernels.h:1818-1822; e.g. the feed-input error added to an
+ * attention node's error, src/attention_node.hpp:416). */
+int zr_add_inplace(zr_ctx* ctx, float* d_dst, const float* d_src, long long n);
 
 /* ---- A1: index preparation ---------------------------------------------------------------------------- */
 

@@ -1,11 +1,14 @@
 // Test driver: SGD steps of model_trainer (zoph_rnn_amd/host/zoph_model.h) on the minibatches of an integerized file.
-//   train_step [--sequence] [--node-level] [--abandon-sweeps] model.nn data.int minibatch longest_sent learning_rate norm_clip steps
+//   train_step [--sequence] [--node-level] [--abandon-sweeps] [--attention-D=N] [--dropout=KEEP_RATE] [--dropout-seed=S]
+//              model.nn data.int minibatch longest_sent learning_rate norm_clip steps
 // Every step trains on the next minibatch of the file (wrapping around) and prints "loss <step> <log-likelihood>";
 // the updated model is written to <model.nn>.trained as a complete model file.  --node-level: the step is
 // forward_model::compute_gradients, i.e. the layer objects' own back_prop_GPU / update_weights members in the
 // reference's node-by-node order, instead of model_trainer's stack-level calls.  --abandon-sweeps: the forward pass is
 // forced onto the single-launch sweep with a wait limit of one poll, so its workgroups give up (and leave the kernel
 // normally); model_trainer must notice and repeat the forward pass; prints "abandoned <count>" at the end.
+// Models with attention (and feed-input) and dropout train through the node-level path only; --attention-D sets the
+// window half-width (the model file does not store it), --dropout the probability of keeping a value.
 #include <cstdio>
 #include <cstdlib>
 #include <iostream>
@@ -16,9 +19,18 @@
 
 int main(int argc, char** argv) {
   bool LM = false, node_level = false, abandon = false;
+  int attention_D = 10;
+  float dropout_rate = 1.0f;
   std::vector<std::string> pos;
   for (int i = 1; i < argc; i++) {
-    if (std::string(argv[i]) == "--sequence")
+    const std::string a = argv[i];
+    if (a.rfind("--attention-D=", 0) == 0)
+      attention_D = std::atoi(a.c_str() + 14);
+    else if (a.rfind("--dropout=", 0) == 0)
+      dropout_rate = (float)std::atof(a.c_str() + 10);
+    else if (a.rfind("--dropout-seed=", 0) == 0)
+      BZ_CUDA::dropout_seed = std::strtoull(a.c_str() + 15, nullptr, 10);
+    else if (std::string(argv[i]) == "--sequence")
       LM = true;
     else if (std::string(argv[i]) == "--node-level")
       node_level = true;
@@ -46,7 +58,7 @@ int main(int argc, char** argv) {
   m.params.learning_rate = lr;
   m.params.norm_clip = clip;
   m.params.clip_gradient = clip > 0;
-  m.initModel(gpu, info, minibatch, longest, 10);
+  m.initModel(gpu, info, minibatch, longest, attention_D, dropout_rate);
   m.load_weights(model);
   model_trainer<precision>* trainer = node_level ? nullptr : new model_trainer<precision>(m);
   if (abandon && trainer) {

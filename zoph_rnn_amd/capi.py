@@ -44,7 +44,7 @@ SYMBOLS = [
     "zr_softmax_backward", "zr_sgd_update", "zr_lstm_node_backward", "zr_lstm_node_gradients",
     "zr_softmax_backward_accumulate", "zr_gather_columns_multi", "zr_softmax_backward_loss",
     "zr_softmax_forward_static", "zr_ctx_query", "zr_attn_prepare", "zr_lstm_step_embed", "zr_attn_viterbi", "zr_lstm_decoder_step", "zr_lstm_feed_backward", "zr_attn_set_error_tables",
-    "zr_attn_backward", "zr_dropout_apply", "zr_uniform_fill",
+    "zr_attn_backward", "zr_dropout_apply", "zr_uniform_fill", "zr_add_inplace",
 ]
 
 _lib = None
@@ -287,6 +287,9 @@ class Context:
         g = _ptr_array(grads)  # zr_attn_grads: six pointers
         _chk(load().zr_attn_backward(self.h, attn, _vp(d_batch_info), _vp(d_h_t), _vp(d_mask), _vp(d_h_tild), _vp(d_align),
                                      _vp(d_idx), _vp(d_p_t), _vp(d_c_t), _vp(d_err_htild), _vp(d_err_h_t), g))
+
+    def add_inplace(self, d_dst, d_src, n):
+        _chk(load().zr_add_inplace(self.h, _vp(d_dst), _vp(d_src), C.c_longlong(n)))
 
     def dropout_apply(self, d_uniform, keep_rate, d_x, n):
         _chk(load().zr_dropout_apply(self.h, _vp(d_uniform), C.c_float(keep_rate), _vp(d_x), C.c_longlong(n)))

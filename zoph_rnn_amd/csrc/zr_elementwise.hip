@@ -198,9 +198,27 @@ lstm_gates_kernel(const float* __restrict__ preact, const float* __restrict__ b_
 
 inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
+// add_two_mats_kernel (src/custom_kernels.h:1818-1822)
+__global__ void __launch_bounds__(256) add_inplace_kernel(float* __restrict__ dst, const float* __restrict__ src,
+                                                          long long n) {
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
+    dst[i] = dst[i] + src[i];
+}
+
 }  // namespace
 
 extern "C" {
+
+int zr_add_inplace(zr_ctx* ctx, float* d_dst, const float* d_src, long long n) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(n >= 0 && (n == 0 || (d_dst && d_src)), "zr_add_inplace: null pointer or n = %lld", n);
+  if (n == 0) return ZR_OK;
+  const int blocks = (int)((n + 255) / 256 < 2048 ? (n + 255) / 256 : 2048);
+  add_inplace_kernel<<<blocks, 256, 0, ctx->stream>>>(d_dst, d_src, n);
+  ZR_LAUNCH_CHECK("add_inplace_kernel");
+  return ZR_OK;
+}
 
 int zr_memset_zero(zr_ctx* ctx, void* d_dst, size_t bytes) {
   int rc = zr_bind_device(ctx);

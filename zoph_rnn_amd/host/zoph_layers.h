@@ -15,8 +15,9 @@
 //   - h_t is handed to the layer above by pointer (the reference's copy_h_t == false branch,
 //     src/LSTM.hpp:492-515) instead of a device-to-device copy;
 //   - only dType = float exists (typedef float precision, src/global_params.h:3);
-//   - back-propagation members exist for the LSTM layers and the softmax (backprop_prep_GPU, back_prop_GPU,
-//     compute_gradients_GPU, clear_gradients, update_weights; back_prop1 / back_prop2); the attention layer, dropout
+//   - back-propagation members exist for the LSTM layers, the softmax and the attention layer (backprop_prep_GPU,
+//     back_prop_GPU, compute_gradients_GPU, clear_gradients, update_weights; back_prop1 / back_prop2; back_prop),
+//     feed-input and dropout included; multi-source attention
 //     and feed-input have none.  Gradients of the four gate matrices are kept stacked (4H x H, gate order i, f, c, o)
 //     in d_M_grad_stack / d_W_h_grad_stack / d_b_grad_stack; the reference's d_M_i_grad ... members are filled from
 //     them by update_weights().  Training buffers are allocated by clear_gradients(true), not by the init calls;
@@ -73,6 +74,14 @@ inline std::mt19937 gen(1234);
 // stream (LSTM M / W_h / Q, attention W_a / W_p / W_c, softmax D) is snapshotted as bf16; the fp32 members stay as
 // the caller's copy.  Requires LSTM_size % 16 == 0.
 inline bool bf16_weights = false;
+// Dropout masks.  The reference fills them with curandGenerateUniform from per-layer generators; here a mask is
+// zr_uniform_fill(seed, call): seed = dropout_seed + dropout_minibatch (the owner of the layers counts the minibatches
+// it has trained on), call = dropout_call(stream, node index) with one stream number per layer.
+inline unsigned long long dropout_seed = 1234;
+inline unsigned long long dropout_minibatch = 0;
+inline unsigned long long dropout_call(int stream, int index) { return ((unsigned long long)stream << 24) | (unsigned)index; }
+enum { DROPOUT_STREAM_SOURCE_INPUT = 1, DROPOUT_STREAM_TARGET_INPUT = 2, DROPOUT_STREAM_SOURCE_HIDDEN = 16,
+       DROPOUT_STREAM_TARGET_HIDDEN = 48, DROPOUT_STREAM_ATTENTION = 96, DROPOUT_STREAM_SOFTMAX = 97 };
 }  // namespace BZ_CUDA
 
 struct attention_params {  // src/global_params.h:8-22 (fields used by the forward path)
@@ -91,6 +100,8 @@ struct global_params {  // src/global_params.h:61-299 (fields the layers use)
   int longest_sent = 100;
   int target_vocab_size = 0;
   int source_vocab_size = 0;
+  bool dropout = false;            // src/global_params.h:86-87
+  precision dropout_rate = 1.0f;   // probability of KEEPING a value
 };
 
 // The reference passes a cublasHandle_t& into the attention layer's constructors (src/attention_layer.h:118-119,143-144);
@@ -101,6 +112,7 @@ template <typename dType>
 struct neuralMT_model {  // only what the layers consult (src/model.h:37-217)
   bool train = false;
   bool decode = false;
+  bool grad_check_flag = false;  // src/model.h: dropout masks are kept instead of drawn afresh
   attention_params attent_params;
   // What attention_layer's constructor reads from the model (src/attention_layer.hpp:106-160): the source side's
   // top-layer node states, entry t = d_h_t of node t of the last source layer (model->source_hidden_layers.back().nodes[t]
@@ -233,11 +245,20 @@ class attention_node {  // src/attention_node.h:11-86
   int* d_indicies = nullptr;
   int** d_indicies_mask = nullptr;  // points at the owning LSTM node's 0/1 mask pointer
   dType* d_lower_htild = nullptr;   // feed-input destination: next step's bottom node d_h_tild
+  // training
+  bool dropout = false;
+  dType dropout_rate = 1;
+  dType* d_dropout_mask = nullptr;
+  dType* d_h_t_att = nullptr;              // the h_t the step read: d_h_t, or its dropped-out copy
+  dType* d_h_t_att_buf = nullptr;          // storage of that copy (dropout only)
+  dType* d_d_ERRt_ht_tild = nullptr;       // error of h~ in, error of h_t out: the owning LSTM node's d_d_ERRt_ht
+  dType* d_ERRtTOn_htild_below = nullptr;  // error of h~ arriving from the next step's bottom node (feed-input)
 
   attention_node(int LSTM_size, int minibatch_size, int device_number, int D, bool feed_input,
                  attention_layer<dType>* attent_layer, int index);
-  void feed_input_init(dType* d_ptr_htild) { d_lower_htild = d_ptr_htild; }  // src/attention_node.hpp:56-60
-  void forward_prop();                                                         // src/attention_node.hpp:73-394
+  void feed_input_init(dType* d_ptr_htild);  // src/attention_node.hpp:56-60
+  void forward_prop();                        // src/attention_node.hpp:73-394
+  void back_prop();                           // src/attention_node.hpp:398-669
 };
 
 template <typename dType>
@@ -255,25 +276,36 @@ class attention_layer {  // src/attention_layer.h:14-143
   int* d_ones_minibatch_int = nullptr;  // init_att_decoder: the decode path runs every column with mask 1
   neuralMT_model<dType>* model = nullptr;
   std::vector<attention_node<dType>> nodes;
+  // training (src/attention_layer.h:60-100; allocated by the first clear_gradients())
+  dType *d_W_a_grad = nullptr, *d_W_p_grad = nullptr, *d_v_p_grad = nullptr, *d_output_bias_grad = nullptr,
+        *d_W_c_p1_grad = nullptr, *d_W_c_p2_grad = nullptr;
+  std::vector<dType*> h_total_hs_error;  // d_total_hs_error: entry t receives the error of source state t
+  bool transfer_done = false;            // src/attention_layer.h: false until the last step's node has run backward
+  bool clip_gradients = true, dropout = false;
+  dType norm_clip = 5, learning_rate = 0.5f, dropout_rate = 1;
 
   attention_layer() {}
 
   // The reference's own parameter list (src/attention_layer.h:118-119, body src/attention_layer.hpp:3-173).  `handle`
-  // is the context (cublasHandle_t above); the source states come from model->source_top_h_t.  Gradient clipping
-  // parameters are accepted and unused (this layer has no backward pass); dropout and the second source side of a
-  // multi-source model are not built and are refused.
+  // is the context (cublasHandle_t above); the source states come from model->source_top_h_t.  The second source side
+  // of a multi-source model is not built and is refused.
   attention_layer(int LSTM_size, int minibatch_size, int device_number, int D, int longest_sent, cublasHandle_t& handle,
-                  neuralMT_model<dType>* model, bool feed_input, bool /*clip_gradients*/, dType /*norm_clip*/,
-                  bool dropout, dType /*dropout_rate*/, global_params& /*params*/, bool bi_side) {
-    if (dropout || bi_side || !model || (int)model->source_top_h_t.size() < longest_sent) {
-      std::fprintf(stderr, "Error: attention_layer: dropout and multi-source attention are not built, and the model "
-                   "must list its %d source top-layer states in source_top_h_t\n", longest_sent);
+                  neuralMT_model<dType>* model, bool feed_input, bool clip_gradients, dType norm_clip,
+                  bool dropout, dType dropout_rate, global_params& params, bool bi_side) {
+    if (bi_side || !model || (int)model->source_top_h_t.size() < longest_sent) {
+      std::fprintf(stderr, "Error: attention_layer: multi-source attention is not built, and the model must list its "
+                   "%d source top-layer states in source_top_h_t\n", longest_sent);
       std::exit(EXIT_FAILURE);
     }
     layer_gpu_info gpu;
     gpu.device_number = device_number;
     gpu.ctx = handle;
     this->model = model;
+    this->clip_gradients = clip_gradients;
+    this->norm_clip = norm_clip;
+    this->learning_rate = params.learning_rate;
+    this->dropout = dropout;
+    this->dropout_rate = dropout_rate;
     setup(LSTM_size, minibatch_size, device_number, D, longest_sent, gpu, model->source_top_h_t, feed_input, longest_sent);
   }
 
@@ -339,6 +371,46 @@ class attention_layer {  // src/attention_layer.h:14-143
     for (int i = 0; i < n_nodes; i++)
       nodes.push_back(attention_node<dType>(LSTM_size, minibatch_size, device_number, D, feed_input, this, i));
   }
+  // ---- training.  clear_gradients (src/attention_layer.hpp:262-300) zeroes the six gradients (allocating them and the
+  // source-state error arrays the first time) and the errors of the source states; the owner of the encoder's top
+  // layer hands error array t to that layer's node t as its error from above (the reference points d_total_hs_error at
+  // those nodes' d_d_ERRt_ht, src/attention_layer.hpp:106-160).
+  void clear_gradients() {
+    zr_ctx* ctx = layer_info.ctx;
+    const size_t hh = (size_t)LSTM_size * LSTM_size, n = (size_t)LSTM_size * minibatch_size;
+    if (!d_W_a_grad) {
+      dType** mats[] = {&d_W_a_grad, &d_W_p_grad, &d_W_c_p1_grad, &d_W_c_p2_grad};
+      for (dType** m : mats) ZOPH_CALL(zr_malloc(ctx, hh * sizeof(dType), (void**)m));
+      ZOPH_CALL(zr_malloc(ctx, (size_t)LSTM_size * sizeof(dType), (void**)&d_v_p_grad));
+      ZOPH_CALL(zr_malloc(ctx, (size_t)LSTM_size * sizeof(dType), (void**)&d_output_bias_grad));
+      h_total_hs_error.resize(h_total_hs_mat.size());
+      for (auto& e : h_total_hs_error) ZOPH_CALL(zr_malloc(ctx, n * sizeof(dType), (void**)&e));
+      ZOPH_CALL(zr_attn_set_error_tables(ctx, attn, h_total_hs_error.data(), (int)h_total_hs_error.size()));
+    }
+    dType* mats[] = {d_W_a_grad, d_W_p_grad, d_W_c_p1_grad, d_W_c_p2_grad};
+    for (dType* m : mats) ZOPH_CALL(zr_memset_zero(ctx, m, hh * sizeof(dType)));
+    ZOPH_CALL(zr_memset_zero(ctx, d_v_p_grad, (size_t)LSTM_size * sizeof(dType)));
+    ZOPH_CALL(zr_memset_zero(ctx, d_output_bias_grad, (size_t)LSTM_size * sizeof(dType)));
+    for (dType* e : h_total_hs_error) ZOPH_CALL(zr_memset_zero(ctx, e, n * sizeof(dType)));
+    transfer_done = false;
+  }
+  // scale_gradients, norm_clip_GPU_v2 per matrix, update_params (src/attention_layer.hpp:303-420); then the snapshots
+  // the forward kernels read are rebuilt
+  void update_weights() {
+    zr_ctx* ctx = layer_info.ctx;
+    const float scale = 1.0f / (float)minibatch_size, clip = clip_gradients ? (float)norm_clip : 0.0f;
+    const long long hh = (long long)LSTM_size * LSTM_size;
+    ZOPH_CALL(zr_sgd_update(ctx, d_W_a, d_W_a_grad, hh, scale, clip, learning_rate));
+    ZOPH_CALL(zr_sgd_update(ctx, d_W_p, d_W_p_grad, hh, scale, clip, learning_rate));
+    ZOPH_CALL(zr_sgd_update(ctx, d_v_p, d_v_p_grad, LSTM_size, scale, clip, learning_rate));
+    ZOPH_CALL(zr_sgd_update(ctx, d_output_bias, d_output_bias_grad, LSTM_size, scale, clip, learning_rate));
+    ZOPH_CALL(zr_sgd_update(ctx, d_W_c_p1, d_W_c_p1_grad, hh, scale, clip, learning_rate));
+    ZOPH_CALL(zr_sgd_update(ctx, d_W_c_p2, d_W_c_p2_grad, hh, scale, clip, learning_rate));
+    if (BZ_CUDA::bf16_weights)
+      ZOPH_CALL(zr_attn_use_bf16_weights(ctx, attn));
+    else
+      ZOPH_CALL(zr_attn_prepare(ctx, attn));
+  }
   // src/attention_layer.hpp:580-583
   void prep_minibatch_info(int* h_batch_info) {
     ZOPH_CALL(zr_h2d(layer_info.ctx, d_batch_info, h_batch_info, 2 * (size_t)minibatch_size * sizeof(int)));
@@ -381,6 +453,8 @@ attention_node<dType>::attention_node(int LSTM_size, int minibatch_size, int dev
   this->feed_input = feed_input;
   this->attent_layer = attent_layer;
   this->index = index;
+  this->dropout = attent_layer->dropout;
+  this->dropout_rate = attent_layer->dropout_rate;
   zr_ctx* ctx = attent_layer->layer_info.ctx;
   const size_t n = (size_t)LSTM_size * minibatch_size, w = (size_t)(2 * D + 1) * minibatch_size;
   ZOPH_CALL(zr_malloc(ctx, n * sizeof(dType), (void**)&d_final_temp_2));
@@ -391,10 +465,31 @@ attention_node<dType>::attention_node(int LSTM_size, int minibatch_size, int dev
 }
 
 template <typename dType>
+void attention_node<dType>::feed_input_init(dType* d_ptr_htild) {
+  d_lower_htild = d_ptr_htild;
+  full_matrix_setup_0(attent_layer->layer_info.ctx, &d_ERRtTOn_htild_below, LSTM_size, minibatch_size);
+}
+
+template <typename dType>
 void attention_node<dType>::forward_prop() {
   zr_ctx* ctx = attent_layer->layer_info.ctx;
-  ZOPH_CALL(zr_attn_step(ctx, attent_layer->attn, attent_layer->d_batch_info, d_h_t, *d_indicies_mask, d_final_temp_2,
-                         d_alignments, d_indicies, d_p_t, d_c_t));
+  const size_t n = (size_t)LSTM_size * minibatch_size;
+  d_h_t_att = d_h_t;
+  if (dropout && attent_layer->model && attent_layer->model->train) {  // src/attention_node.hpp:98-106
+    if (!d_dropout_mask) {
+      ZOPH_CALL(zr_malloc(ctx, n * sizeof(dType), (void**)&d_dropout_mask));
+      ZOPH_CALL(zr_malloc(ctx, n * sizeof(dType), (void**)&d_h_t_att_buf));
+    }
+    if (!attent_layer->model->grad_check_flag)
+      ZOPH_CALL(zr_uniform_fill(ctx, BZ_CUDA::dropout_seed + BZ_CUDA::dropout_minibatch,
+                                BZ_CUDA::dropout_call(BZ_CUDA::DROPOUT_STREAM_ATTENTION, index), d_dropout_mask,
+                                (long long)n));
+    ZOPH_CALL(zr_d2d(ctx, d_h_t_att_buf, d_h_t, n * sizeof(dType)));
+    ZOPH_CALL(zr_dropout_apply(ctx, d_dropout_mask, dropout_rate, d_h_t_att_buf, (long long)n));
+    d_h_t_att = d_h_t_att_buf;
+  }
+  ZOPH_CALL(zr_attn_step(ctx, attent_layer->attn, attent_layer->d_batch_info, d_h_t_att, *d_indicies_mask,
+                         d_final_temp_2, d_alignments, d_indicies, d_p_t, d_c_t));
   if (BZ_CUDA::unk_replacement && attent_layer->d_viterbi_alignments) {  // src/attention_node.hpp:225-234
     ZOPH_CALL(zr_attn_viterbi(ctx, attent_layer->attn, d_alignments, d_indicies, attent_layer->d_viterbi_alignments));
     BZ_CUDA::viterbi_alignments.resize((size_t)minibatch_size);
@@ -404,6 +499,26 @@ void attention_node<dType>::forward_prop() {
   // feed-input: h~ goes to the next time step's bottom node (src/attention_node.hpp:384-386)
   if (feed_input && index != (attent_layer->longest_sent - 1) && d_lower_htild)
     ZOPH_CALL(zr_d2d(ctx, d_lower_htild, d_final_temp_2, (size_t)LSTM_size * minibatch_size * sizeof(dType)));
+}
+
+// src/attention_node.hpp:398-669.  d_d_ERRt_ht_tild holds the error of h~ on entry (the loss layer's) and the error of
+// h_t on return, as in the reference (:654).
+template <typename dType>
+void attention_node<dType>::back_prop() {
+  zr_ctx* ctx = attent_layer->layer_info.ctx;
+  const long long n = (long long)LSTM_size * minibatch_size;
+  if (!attent_layer->d_W_a_grad) attent_layer->clear_gradients();
+  // the error the next step's bottom node sent through its Q matrices; the last step has none (:407-422)
+  if (feed_input && attent_layer->transfer_done && d_ERRtTOn_htild_below)
+    ZOPH_CALL(zr_add_inplace(ctx, d_d_ERRt_ht_tild, d_ERRtTOn_htild_below, n));
+  attent_layer->transfer_done = true;
+  zr_attn_grads g = {attent_layer->d_W_a_grad, attent_layer->d_W_p_grad, attent_layer->d_v_p_grad,
+                     attent_layer->d_output_bias_grad, attent_layer->d_W_c_p1_grad, attent_layer->d_W_c_p2_grad};
+  ZOPH_CALL(zr_attn_backward(ctx, attent_layer->attn, attent_layer->d_batch_info, d_h_t_att ? d_h_t_att : d_h_t,
+                             *d_indicies_mask, d_final_temp_2, d_alignments, d_indicies, d_p_t, d_c_t, d_d_ERRt_ht_tild,
+                             d_d_ERRt_ht_tild, &g));
+  if (dropout && d_dropout_mask && d_h_t_att == d_h_t_att_buf)  // :646-648
+    ZOPH_CALL(zr_dropout_apply(ctx, d_dropout_mask, dropout_rate, d_d_ERRt_ht_tild, n));
 }
 
 // ------------------------------------------------------------------------------------------------ loss layer
@@ -438,6 +553,7 @@ struct softmax_node {  // src/softmax_node.h:7-27
   dType* d_outputdist = nullptr;
   dType* d_h_t = nullptr;
   dType* d_d_ERRt_ht = nullptr;  // error at h_t of this step (allocated on first use by back_prop1)
+  dType *d_dropout_mask = nullptr, *d_h_t_drop = nullptr;  // dropout: the mask and the dropped-out copy of d_h_t
   int index = 0;
 };
 
@@ -459,6 +575,29 @@ class softmax_layer : public base_loss_layer<dType> {  // src/softmax.h:14-225
   bool clip_gradients = true;
   dType norm_clip = 5, learning_rate = 0.5f;
   lower_transfer_layer<dType> lower_layer;
+  // dropout on the layer's input, models without attention only (src/softmax.hpp:474-478, :745-747)
+  bool dropout = false;
+  dType dropout_rate = 1;
+  neuralMT_model<precision>* model = nullptr;
+  // the h_t of node `index` as the loss layer reads it in training: dropped out once per node and minibatch
+  dType* training_input(int index) {
+    dType* h = nodes[index].d_h_t ? nodes[index].d_h_t : d_h_t;
+    if (!(dropout && model && model->train && !model->attent_params.attention_model)) return h;
+    zr_ctx* ctx = s_layer_info.ctx;
+    const size_t n = (size_t)LSTM_size * minibatch_size;
+    auto& nd = nodes[index];
+    if (!nd.d_dropout_mask) {
+      ZOPH_CALL(zr_malloc(ctx, n * sizeof(dType), (void**)&nd.d_dropout_mask));
+      ZOPH_CALL(zr_malloc(ctx, n * sizeof(dType), (void**)&nd.d_h_t_drop));
+    }
+    if (!model->grad_check_flag)
+      ZOPH_CALL(zr_uniform_fill(ctx, BZ_CUDA::dropout_seed + BZ_CUDA::dropout_minibatch,
+                                BZ_CUDA::dropout_call(BZ_CUDA::DROPOUT_STREAM_SOFTMAX, index), nd.d_dropout_mask,
+                                (long long)n));
+    ZOPH_CALL(zr_d2d(ctx, nd.d_h_t_drop, h, n * sizeof(dType)));
+    ZOPH_CALL(zr_dropout_apply(ctx, nd.d_dropout_mask, dropout_rate, nd.d_h_t_drop, (long long)n));
+    return nd.d_h_t_drop;
+  }
 
   softmax_layer_gpu_info gpu_init(int device_number) override {
     if (!s_layer_info.ctx) s_layer_info.init(device_number);
@@ -467,7 +606,10 @@ class softmax_layer : public base_loss_layer<dType> {  // src/softmax.h:14-225
   void share_gpu(const layer_gpu_info& gpu) { s_layer_info.share(gpu); }
 
   // src/softmax.hpp:3-100: sizes come from params; D and b_d are U(lower, upper)
-  void init_loss_layer(struct neuralMT_model<precision>* /*model*/, global_params& params) override {
+  void init_loss_layer(struct neuralMT_model<precision>* model, global_params& params) override {
+    this->model = model;
+    dropout = params.dropout;
+    dropout_rate = params.dropout_rate;
     output_vocab_size = params.target_vocab_size;
     LSTM_size = params.LSTM_size;
     minibatch_size = params.minibatch_size;
@@ -556,10 +698,13 @@ class softmax_layer : public base_loss_layer<dType> {  // src/softmax.h:14-225
     zr_ctx* ctx = s_layer_info.ctx;
     if (!d_D_grad) clear_gradients();
     if (!nodes[index].d_d_ERRt_ht) full_matrix_setup_0(ctx, &nodes[index].d_d_ERRt_ht, LSTM_size, minibatch_size);
-    dType* h = nodes[index].d_h_t ? nodes[index].d_h_t : d_h_t;
+    dType* h = training_input(index);
     ZOPH_CALL(zr_softmax_backward_accumulate(ctx, d_D, d_b_d, output_vocab_size, LSTM_size, h, minibatch_size,
                                              d_output_vocab_indices_single, d_output_vocab_indices_01_single,
                                              d_logits, nodes[index].d_d_ERRt_ht, d_D_grad, d_b_d_grad));
+    if (h == nodes[index].d_h_t_drop && h)  // src/softmax.hpp:745-747
+      ZOPH_CALL(zr_dropout_apply(ctx, nodes[index].d_dropout_mask, dropout_rate, nodes[index].d_d_ERRt_ht,
+                                 (long long)LSTM_size * minibatch_size));
     lower_layer.send_error(index, nodes[index].d_d_ERRt_ht);
   }
   void back_prop2(int /*index*/) override {}
@@ -614,6 +759,10 @@ struct lstm_layer_training {
   // errors of the node being processed; d_d_ERRnTOt_h_Below sits directly behind d_d_ERRnTOt_htM1
   dType *d_d_ERRnTOt_htM1 = nullptr, *d_d_ERRnTOt_h_Below = nullptr, *d_d_ERRnTOt_ctM1 = nullptr;
   dType* d_d_ERRnTOt_gates = nullptr;  // 4H x minibatch: the reference's d_d_ERRnTOt_it, _ft, _tanhcpt, _ot stacked
+  // feed-input (bottom target layer only; allocated by alloc_feed_training)
+  dType* d_Q_grad_stack = nullptr;     // 4H x H
+  dType *d_Q_i_grad = nullptr, *d_Q_f_grad = nullptr, *d_Q_c_grad = nullptr, *d_Q_o_grad = nullptr;
+  dType* d_ERRnTOt_h_tild = nullptr;   // error of h~_{t-1} of the node being processed (first step: unused)
   dType *d_init_d_ERRnTOtp1_ht = nullptr, *d_init_d_ERRnTOtp1_ct = nullptr;  // zeros for the last time step
   dType learning_rate = 0.5f, norm_clip = 5;
   bool clip_gradients = true;
@@ -637,7 +786,21 @@ struct lstm_layer_training {
     full_matrix_setup_0(ctx, &d_init_d_ERRnTOtp1_ht, H, mb);
     full_matrix_setup_0(ctx, &d_init_d_ERRnTOtp1_ct, H, mb);
   }
+  void alloc_feed_training(zr_ctx* ctx, int H, int mb) {
+    full_matrix_setup_0(ctx, &d_Q_grad_stack, 4 * H, H);
+    dType** mats[] = {&d_Q_i_grad, &d_Q_f_grad, &d_Q_c_grad, &d_Q_o_grad};
+    for (dType** m : mats) ZOPH_CALL(zr_malloc(ctx, (size_t)H * H * sizeof(dType), (void**)m));
+    full_matrix_setup_0(ctx, &d_ERRnTOt_h_tild, H, mb);
+  }
+  // the Q matrices' share of update_weights (src/Input_To_Hidden_Layer.hpp:690-790)
+  void apply_feed_gradients(zr_ctx* ctx, int H, int mb, dType* const Q[4]) {
+    const float scale = 1.0f / (float)mb, clip = clip_gradients ? (float)norm_clip : 0.0f;
+    dType* gQ[4] = {d_Q_i_grad, d_Q_f_grad, d_Q_c_grad, d_Q_o_grad};
+    ZOPH_CALL(zr_unstack_gates(ctx, d_Q_grad_stack, H, gQ));
+    for (int g = 0; g < 4; g++) ZOPH_CALL(zr_sgd_update(ctx, Q[g], gQ[g], (long long)H * H, scale, clip, learning_rate));
+  }
   void zero_gradients(zr_ctx* ctx, int H) {
+    if (d_Q_grad_stack) ZOPH_CALL(zr_memset_zero(ctx, d_Q_grad_stack, 4 * (size_t)H * H * sizeof(dType)));
     ZOPH_CALL(zr_memset_zero(ctx, d_M_grad_stack, 4 * (size_t)H * H * sizeof(dType)));
     ZOPH_CALL(zr_memset_zero(ctx, d_W_h_grad_stack, 4 * (size_t)H * H * sizeof(dType)));
     ZOPH_CALL(zr_memset_zero(ctx, d_b_grad_stack, 4 * (size_t)H * sizeof(dType)));
@@ -674,6 +837,10 @@ class LSTM_HH_Node {  // src/LSTM_HH.h:19-102
   dType *d_c_t_prev = nullptr, *d_h_t_prev = nullptr;
   dType* d_h_t_below = nullptr;
   dType* d_zeros = nullptr;
+  // dropout (src/LSTM_HH.hpp:111-126): the node's input is a dropped-out copy of the state below.  The reference
+  // always copies the state below into the node; here it is read in place unless dropout is on.
+  dType *d_dropout_mask = nullptr, *d_h_t_below_drop = nullptr;
+  dType* d_input = nullptr;  // what the step read: d_h_t_below or d_h_t_below_drop
   // errors arriving from step t+1 and from above (NULL: none); set by backprop_prep_GPU / the layer above
   dType *d_d_ERRnTOtp1_ht = nullptr, *d_d_ERRnTOtp1_ct = nullptr, *d_d_ERRt_ht = nullptr;
 
@@ -713,6 +880,8 @@ class LSTM_IH_Node {  // src/LSTM.h:19-106
   dType *d_c_t_prev = nullptr, *d_h_t_prev = nullptr;
   dType* d_zeros = nullptr;
   dType* d_h_tild = nullptr;
+  dType* d_dropout_mask = nullptr;            // src/LSTM.hpp:39-41, :112-119
+  dType* d_ERRnTOt_h_tild_cpy = nullptr;      // where the error of h~_{t-1} goes: attention node t-1's d_ERRtTOn_htild_below
   dType *d_d_ERRnTOtp1_ht = nullptr, *d_d_ERRnTOtp1_ct = nullptr, *d_d_ERRt_ht = nullptr;
 
   LSTM_IH_Node(int LSTM_size, int minibatch_size, int vocab_size, Input_To_Hidden_Layer<dType>* m, int index,
@@ -921,8 +1090,8 @@ class Hidden_To_Hidden_Layer : public lstm_layer_training<dType> {  // src/Hidde
   void init_attention(int device_number, int D, bool feed_input, neuralMT_model<dType>* model, global_params& params) {
     cublasHandle_t handle = hh_layer_info.ctx;
     init_attention(new attention_layer<dType>(LSTM_size, minibatch_size, device_number, D, longest_sent, handle, model,
-                                              feed_input, this->clip_gradients, this->norm_clip, false, (dType)0, params,
-                                              false));
+                                              feed_input, this->clip_gradients, this->norm_clip, params.dropout,
+                                              params.dropout_rate, params, false));
   }
 };
 
@@ -1001,6 +1170,7 @@ class Input_To_Hidden_Layer : public lstm_layer_training<dType> {  // src/Input_
       if (!this->train_weights) {
         this->alloc_training(ctx, LSTM_size, minibatch_size);
         full_matrix_setup_0(ctx, &d_W_grad, LSTM_size, input_vocab_size);
+        if (feed_input) this->alloc_feed_training(ctx, LSTM_size, minibatch_size);
         const dType* M[4] = {d_M_i, d_M_f, d_M_c, d_M_o};
         const dType* Wh[4] = {d_W_hi, d_W_hf, d_W_hc, d_W_ho};
         ZOPH_CALL(zr_lstm_train_create(ctx, M, Wh, LSTM_size, &this->train_weights));
@@ -1018,6 +1188,10 @@ class Input_To_Hidden_Layer : public lstm_layer_training<dType> {  // src/Input_
     ZOPH_CALL(zr_sgd_update(ctx, d_W, d_W_grad, (long long)LSTM_size * input_vocab_size, 1.0f / (float)minibatch_size,
                             this->clip_gradients ? (float)this->norm_clip : 0.0f, this->learning_rate));
     this->apply_gradients(ctx, LSTM_size, minibatch_size, M, Wh, b);
+    if (feed_input && this->d_Q_grad_stack) {
+      dType* Q[4] = {d_Q_i, d_Q_f, d_Q_c, d_Q_o};
+      this->apply_feed_gradients(ctx, LSTM_size, minibatch_size, Q);
+    }
     repack();
     ZOPH_CALL(zr_lstm_train_refresh(ctx, this->train_weights, M, Wh));
   }
@@ -1043,7 +1217,10 @@ class Input_To_Hidden_Layer : public lstm_layer_training<dType> {  // src/Input_
     attention_layer<dType>* att = hidden_layer ? hidden_layer->attent_layer : attent_layer;
     for (size_t i = 0; i < nodes.size(); i++) nodes[i].attention_extra();
     if (att)
-      for (size_t i = 0; i + 1 < nodes.size(); i++) att->nodes[i].feed_input_init(nodes[i + 1].d_h_tild);
+      for (size_t i = 0; i + 1 < nodes.size(); i++) {
+        att->nodes[i].feed_input_init(nodes[i + 1].d_h_tild);
+        nodes[i + 1].d_ERRnTOt_h_tild_cpy = att->nodes[i].d_ERRtTOn_htild_below;  // :253, :272
+      }
     repack();
   }
   void decoder_init_feed_input() {  // :300-317: decode keeps a single node; h~ is copied in by the driver
@@ -1068,8 +1245,8 @@ class Input_To_Hidden_Layer : public lstm_layer_training<dType> {  // src/Input_
   void init_attention(int device_number, int D, bool feed_input, neuralMT_model<dType>* model, global_params& params) {
     cublasHandle_t handle = ih_layer_info.ctx;
     init_attention(new attention_layer<dType>(LSTM_size, minibatch_size, device_number, D, longest_sent, handle, model,
-                                              feed_input, this->clip_gradients, this->norm_clip, false, (dType)0, params,
-                                              false));
+                                              feed_input, this->clip_gradients, this->norm_clip, params.dropout,
+                                              params.dropout_rate, params, false));
   }
   // the reference's own parameter list (src/Input_To_Hidden_Layer.h:345): a host-side index vector
   int* d_swap_indices = nullptr;
@@ -1166,7 +1343,24 @@ void LSTM_HH_Node<dType>::forward_prop_GPU() {  // src/LSTM_HH.hpp:103-333
   zr_ctx* ctx = model->hh_layer_info.ctx;
   if (!model->packed) model->repack();
   dType* gates[4] = {d_i_t, d_f_t, d_c_prime_t_tanh, d_o_t};
-  ZOPH_CALL(zr_lstm_step(ctx, model->packed, d_h_t_below, d_h_t_prev, d_c_t_prev, nullptr, d_input_vocab_indices_01,
+  d_input = d_h_t_below;
+  if (dropout && model->model && model->model->train) {  // src/LSTM_HH.hpp:111-126
+    const size_t n = (size_t)LSTM_size * minibatch_size;
+    if (!d_dropout_mask) {
+      ZOPH_CALL(zr_malloc(ctx, n * sizeof(dType), (void**)&d_dropout_mask));
+      ZOPH_CALL(zr_malloc(ctx, n * sizeof(dType), (void**)&d_h_t_below_drop));
+    }
+    if (!model->model->grad_check_flag) {
+      const int stream = (model->upper_layer.source_side ? BZ_CUDA::DROPOUT_STREAM_SOURCE_HIDDEN
+                                                         : BZ_CUDA::DROPOUT_STREAM_TARGET_HIDDEN) + model->layer_number;
+      ZOPH_CALL(zr_uniform_fill(ctx, BZ_CUDA::dropout_seed + BZ_CUDA::dropout_minibatch,
+                                BZ_CUDA::dropout_call(stream, index), d_dropout_mask, (long long)n));
+    }
+    ZOPH_CALL(zr_d2d(ctx, d_h_t_below_drop, d_h_t_below, n * sizeof(dType)));
+    ZOPH_CALL(zr_dropout_apply(ctx, d_dropout_mask, dropout_rate, d_h_t_below_drop, (long long)n));
+    d_input = d_h_t_below_drop;
+  }
+  ZOPH_CALL(zr_lstm_step(ctx, model->packed, d_input, d_h_t_prev, d_c_t_prev, nullptr, d_input_vocab_indices_01,
                          BZ_CUDA::clip_cell ? BZ_CUDA::cell_clip_threshold : 0.0f, minibatch_size, d_h_t, d_c_t, gates));
   send_h_t_above();
 }
@@ -1215,6 +1409,17 @@ void LSTM_IH_Node<dType>::forward_prop_GPU() {  // src/LSTM.hpp:76-421
   if (!model->packed) model->repack();
   ZOPH_CALL(zr_embed_gather(ctx, model->d_W, LSTM_size, model->input_vocab_size, d_input_vocab_indices, minibatch_size,
                             d_sparse_lookup));
+  if (dropout && model->model && model->model->train) {  // src/LSTM.hpp:112-119
+    const size_t n = (size_t)LSTM_size * minibatch_size;
+    if (!d_dropout_mask) ZOPH_CALL(zr_malloc(ctx, n * sizeof(dType), (void**)&d_dropout_mask));
+    if (!model->model->grad_check_flag) {
+      const int stream = model->upper_layer.source_side ? BZ_CUDA::DROPOUT_STREAM_SOURCE_INPUT
+                                                        : BZ_CUDA::DROPOUT_STREAM_TARGET_INPUT;
+      ZOPH_CALL(zr_uniform_fill(ctx, BZ_CUDA::dropout_seed + BZ_CUDA::dropout_minibatch,
+                                BZ_CUDA::dropout_call(stream, index), d_dropout_mask, (long long)n));
+    }
+    ZOPH_CALL(zr_dropout_apply(ctx, d_dropout_mask, dropout_rate, d_sparse_lookup, (long long)n));
+  }
   dType* gates[4] = {d_i_t, d_f_t, d_c_prime_t_tanh, d_o_t};
   const bool use_q = feed_input && index != 0;  // src/LSTM.hpp:154
   ZOPH_CALL(zr_lstm_step(ctx, model->packed, d_sparse_lookup, d_h_t_prev, d_c_t_prev, use_q ? d_h_tild : nullptr,
@@ -1258,36 +1463,53 @@ void LSTM_HH_Node<dType>::back_prop_GPU(int index) {
   BZ_CUDA::refuse_backward_with_clip_cell("LSTM_HH_Node::back_prop_GPU");
   zr_ctx* ctx = model->hh_layer_info.ctx;
   if (!model->train_weights) model->clear_gradients(true);
+  if (attention_model && model->attent_layer) {  // src/LSTM_HH.hpp:470-482: the error of h~ becomes the error of h_t
+    auto& an = model->attent_layer->nodes[index];
+    an.d_d_ERRt_ht_tild = d_d_ERRt_ht;
+    an.back_prop();
+  }
   const dType* gates[4] = {d_i_t, d_f_t, d_c_prime_t_tanh, d_o_t};
   ZOPH_CALL(zr_lstm_node_backward(ctx, model->train_weights, minibatch_size, gates, d_c_t, d_c_t_prev,
                                   d_input_vocab_indices_01, d_d_ERRt_ht, d_d_ERRnTOtp1_ht, d_d_ERRnTOtp1_ct,
                                   model->d_d_ERRnTOt_gates, model->d_d_ERRnTOt_htM1, model->d_d_ERRnTOt_ctM1,
                                   model->d_d_ERRnTOt_h_Below));
   compute_gradients_GPU();
+  if (d_input == d_h_t_below_drop && d_dropout_mask)  // src/LSTM_HH.hpp:673-675
+    ZOPH_CALL(zr_dropout_apply(ctx, d_dropout_mask, dropout_rate, model->d_d_ERRnTOt_h_Below,
+                               (long long)LSTM_size * minibatch_size));
   model->lower_layer.send_error(index, model->d_d_ERRnTOt_h_Below);
 }
 
 template <typename dType>
 void LSTM_HH_Node<dType>::compute_gradients_GPU() {
   ZOPH_CALL(zr_lstm_node_gradients(model->hh_layer_info.ctx, LSTM_size, minibatch_size, model->d_d_ERRnTOt_gates,
-                                   d_h_t_below, d_h_t_prev, model->d_M_grad_stack, model->d_W_h_grad_stack,
-                                   model->d_b_grad_stack));
+                                   d_input ? d_input : d_h_t_below, d_h_t_prev, model->d_M_grad_stack,
+                                   model->d_W_h_grad_stack, model->d_b_grad_stack));
 }
 
 template <typename dType>
 void LSTM_IH_Node<dType>::back_prop_GPU(int /*index*/) {
   BZ_CUDA::refuse_backward_with_clip_cell("LSTM_IH_Node::back_prop_GPU");
   zr_ctx* ctx = model->ih_layer_info.ctx;
-  if (feed_input) {
-    std::fprintf(stderr, "Error: back-propagation through the feed-input connection is not built\n");
-    std::exit(EXIT_FAILURE);
-  }
   if (!model->train_weights) model->clear_gradients(true);
+  if (attention_model && model->attent_layer) {  // src/LSTM.hpp:587-599: a one-layer model's attention sits on this layer
+    auto& an = model->attent_layer->nodes[index];
+    an.d_d_ERRt_ht_tild = d_d_ERRt_ht;
+    an.back_prop();
+  }
   const dType* gates[4] = {d_i_t, d_f_t, d_c_prime_t_tanh, d_o_t};
   ZOPH_CALL(zr_lstm_node_backward(ctx, model->train_weights, minibatch_size, gates, d_c_t, d_c_t_prev,
                                   d_input_vocab_indices_01, d_d_ERRt_ht, d_d_ERRnTOtp1_ht, d_d_ERRnTOtp1_ct,
                                   model->d_d_ERRnTOt_gates, model->d_d_ERRnTOt_htM1, model->d_d_ERRnTOt_ctM1,
                                   model->d_d_ERRnTOt_h_Below));
+  if (feed_input && index != 0) {  // src/LSTM.hpp:804-866 and :1014-1050
+    const dType* Q[4] = {model->d_Q_i, model->d_Q_f, model->d_Q_c, model->d_Q_o};
+    ZOPH_CALL(zr_lstm_feed_backward(ctx, Q, LSTM_size, minibatch_size, model->d_d_ERRnTOt_gates, d_h_tild,
+                                    model->d_ERRnTOt_h_tild, model->d_Q_grad_stack));
+    if (d_ERRnTOt_h_tild_cpy)
+      ZOPH_CALL(zr_d2d(ctx, d_ERRnTOt_h_tild_cpy, model->d_ERRnTOt_h_tild,
+                       (size_t)LSTM_size * minibatch_size * sizeof(dType)));
+  }
   compute_gradients_GPU();
 }
 
@@ -1297,7 +1519,11 @@ void LSTM_IH_Node<dType>::compute_gradients_GPU() {
   ZOPH_CALL(zr_lstm_node_gradients(ctx, LSTM_size, minibatch_size, model->d_d_ERRnTOt_gates, d_sparse_lookup,
                                    d_h_t_prev, model->d_M_grad_stack, model->d_W_h_grad_stack, model->d_b_grad_stack));
   // the sparse W gradient (src/custom_kernels.h:353-378): the error at the node's input, added into the columns of
-  // the minibatch's words
+  // the minibatch's words; with dropout the error passes the node's mask first (W_small_dropout_gradient_kernel,
+  // src/LSTM.hpp:1196)
+  if (dropout && d_dropout_mask && model->model && model->model->train)
+    ZOPH_CALL(zr_dropout_apply(ctx, d_dropout_mask, dropout_rate, model->d_d_ERRnTOt_h_Below,
+                               (long long)LSTM_size * minibatch_size));
   ZOPH_CALL(zr_embed_gradient(ctx, LSTM_size, model->input_vocab_size, model->d_d_ERRnTOt_h_Below,
                               d_input_vocab_indices, d_input_vocab_indices_01, minibatch_size, model->d_W_grad));
 }

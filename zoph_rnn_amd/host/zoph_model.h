@@ -379,10 +379,15 @@ class forward_model {
 
   // neuralMT_model::initModel (src/model.hpp:35-420) for the forward path on one device.  attention_D: the window
   // half-width; the model file does not store it and the reference's decoder uses its default of 10.
+  // dropout_rate < 1: dropout with that probability of KEEPING a value, applied in compute_gradients only
+  // (global_params::dropout / dropout_rate, src/global_params.h:86-87).
   void initModel(const layer_gpu_info& g, const model_file_info& mi, int minibatch_size, int longest_sent,
-                 int attention_D = 10) {
+                 int attention_D = 10, float dropout_rate = 1.0f) {
     gpu = g;
     info = mi;
+    params.dropout = dropout_rate < 1.0f;
+    params.dropout_rate = dropout_rate;
+    const bool dr = params.dropout;
     const bool seq2seq = !mi.LM;
     const int H = mi.LSTM_size, L = mi.num_layers;
     params.LSTM_size = H;
@@ -403,23 +408,23 @@ class forward_model {
       input_layer_source.ih_layer_info.share(gpu);
       input_layer_source.init_Input_To_Hidden_Layer(H, minibatch_size, mi.source_vocab_size, longest_sent, false,
                                                     params.learning_rate, params.clip_gradient, params.norm_clip,
-                                                    &flags, 0, false, 0.f, false, false, nullptr, false, params, true);
+                                                    &flags, 0, dr, dropout_rate, false, false, nullptr, false, params, true);
       for (int l = 0; l < L - 1; l++) {
         source_hidden_layers[l].hh_layer_info.share(gpu);
         source_hidden_layers[l].init_Hidden_To_Hidden_Layer(H, minibatch_size, longest_sent, false, params.learning_rate,
-                                                             params.clip_gradient, params.norm_clip, &flags, 0, false,
-                                                             0.f, false, l);
+                                                             params.clip_gradient, params.norm_clip, &flags, 0, dr,
+                                                             dropout_rate, false, l);
       }
     }
     input_layer_target.ih_layer_info.share(gpu);
     input_layer_target.init_Input_To_Hidden_Layer(H, minibatch_size, mi.target_vocab_size, longest_sent, false,
                                                   params.learning_rate, params.clip_gradient, params.norm_clip, &flags,
-                                                  0, false, 0.f, false, false, nullptr, false, params, false);
+                                                  0, dr, dropout_rate, false, false, nullptr, false, params, false);
     for (int l = 0; l < L - 1; l++) {
       target_hidden_layers[l].hh_layer_info.share(gpu);
       target_hidden_layers[l].init_Hidden_To_Hidden_Layer(H, minibatch_size, longest_sent, false, params.learning_rate,
-                                                           params.clip_gradient, params.norm_clip, &flags, 0, false,
-                                                           0.f, false, l);
+                                                           params.clip_gradient, params.norm_clip, &flags, 0, dr,
+                                                           dropout_rate, false, l);
     }
     // upper transfer (h_t upwards) and lower transfer (error downwards) wiring, src/model.hpp:191-290
     auto wire = [&](Input_To_Hidden_Layer<dType>& in, std::vector<Hidden_To_Hidden_Layer<dType>>& hid, bool source) {
@@ -557,15 +562,13 @@ class forward_model {
     return total;
   }
 
-  // neuralMT_model::compute_gradients (src/model.hpp:813-1230) for models without attention, through the layer
-  // objects' own members in the reference's order: forward over the grid, then per target step (last first) the loss
-  // layer's back_prop1 and the nodes' backprop_prep_GPU / back_prop_GPU from the top layer down, then the source side
-  // started from the errors the target side left at its first step, then update_weights and clear_gradients.
+  // neuralMT_model::compute_gradients (src/model.hpp:813-1230) through the layer objects' own members in the
+  // reference's order: forward over the grid (training mode: dropout where it is on), then per target step (last
+  // first) the loss layer's back_prop1 and the nodes' backprop_prep_GPU / back_prop_GPU from the top layer down -- the
+  // top node runs its attention node's back_prop first, the bottom node sends the feed-input error to the previous
+  // step's attention node -- then the source side, started from the errors the target side left at its first step and
+  // with the attention layer's source-state errors arriving at its top layer, then update_weights and clear_gradients.
   void compute_gradients(minibatch_reader& mb) {
-    if (params.attent_params.attention_model) {
-      std::fprintf(stderr, "compute_gradients: the backward pass of the attention layer is not built\n");
-      std::exit(EXIT_FAILURE);
-    }
     const bool seq2seq = !info.LM;
     const int S = seq2seq ? mb.current_source_length : 0, T = mb.current_target_length;
     const int mbs = params.minibatch_size;
@@ -573,6 +576,7 @@ class forward_model {
       clear_gradients(true);
       trained_before = true;
     }
+    flags.train = true;
     forward_pass(mb, false);
     for (int i = T - 1; i >= 0; i--) {
       const bool last = i == T - 1;
@@ -592,6 +596,12 @@ class forward_model {
     }
     for (int i = S - 1; i >= 0; i--) {
       const bool last = i == S - 1;  // the source's last step continues from the target's first (:1097-1126)
+      if (att) {  // the error of source state i, collected by the attention nodes, arrives from above
+        if (source_hidden_layers.empty())
+          input_layer_source.nodes[i].d_d_ERRt_ht = att->h_total_hs_error[i];
+        else
+          source_hidden_layers.back().nodes[i].d_d_ERRt_ht = att->h_total_hs_error[i];
+      }
       for (int j = (int)source_hidden_layers.size() - 1; j >= 0; j--) {
         auto& ly = source_hidden_layers[j];
         ly.nodes[i].backprop_prep_GPU(last ? target_hidden_layers[j].d_d_ERRnTOt_htM1 : ly.d_d_ERRnTOt_htM1,
@@ -603,10 +613,28 @@ class forward_model {
                                     last ? input_layer_target.d_d_ERRnTOt_ctM1 : in.d_d_ERRnTOt_ctM1);
       in.nodes[i].back_prop_GPU(i);
     }
+    flags.train = false;
+    BZ_CUDA::dropout_minibatch++;
     update_weights();
     clear_gradients(false);
   }
   bool trained_before = false;
+  // learning rate and per-matrix norm clip (0: none) of every layer's update_weights
+  void set_training_rates(float learning_rate, float norm_clip) {
+    auto set = [&](auto& ly) {
+      ly.learning_rate = learning_rate;
+      ly.norm_clip = norm_clip;
+      ly.clip_gradients = norm_clip > 0;
+    };
+    if (!info.LM) {
+      set(input_layer_source);
+      for (auto& l : source_hidden_layers) set(l);
+    }
+    set(input_layer_target);
+    for (auto& l : target_hidden_layers) set(l);
+    set(softmax_obj);
+    if (att) set(*att);
+  }
 
   void clear_gradients(bool init) {  // src/model.hpp:1431-1460
     if (!info.LM) {
@@ -616,6 +644,7 @@ class forward_model {
     input_layer_target.clear_gradients(init);
     for (auto& l : target_hidden_layers) l.clear_gradients(init);
     softmax->clear_gradients();
+    if (att) att->clear_gradients();
   }
   void update_weights() {  // src/model.hpp:1845-1955, per-matrix clipping (no global norm)
     softmax->update_weights();
@@ -625,6 +654,7 @@ class forward_model {
     }
     input_layer_target.update_weights();
     for (auto& l : target_hidden_layers) l.update_weights();
+    if (att) att->update_weights();
   }
 
   // neuralMT_model::get_perplexity (src/model.hpp:2281-2355): one getError per minibatch; with force_decode the
@@ -650,9 +680,11 @@ class forward_model {
 };
 
 // ------------------------------------------------------------------------------------------------ training
-// One SGD step on a minibatch for models without attention (language models and plain encoder-decoder models):
-// neuralMT_model::compute_gradients (src/model.hpp:1823-2000) followed by update_weights (:2002-2040), written
-// against the stack-level training entry points of the library instead of node-by-node back_prop_GPU calls.
+// One SGD step on a minibatch: neuralMT_model::compute_gradients (src/model.hpp:1823-2000) followed by update_weights
+// (:2002-2040).  Models without attention and without dropout (language models and plain encoder-decoder models) go
+// through the stack-level training entry points of the library instead of node-by-node back_prop_GPU calls; models
+// with attention (feed-input makes every target step depend on the one before, so there is no sweep to batch) or
+// dropout go through forward_model::compute_gradients, the layer objects' own members.
 // Gradients are those of the log-likelihood and are ADDED (the reference ascends), scaled by 1/minibatch_size and
 // clipped per matrix to norm_clip in L2 norm (norm_clip_GPU_v2), as the reference does without --global-clip.
 template <typename dType>
@@ -711,10 +743,7 @@ class model_trainer {
 
   explicit model_trainer(forward_model<dType>& model) : m(model), ctx(model.gpu.ctx) {
     BZ_CUDA::refuse_backward_with_clip_cell("model_trainer");
-    if (m.params.attent_params.attention_model) {
-      std::fprintf(stderr, "model_trainer: the backward pass of the attention layer is not built\n");
-      std::exit(EXIT_FAILURE);
-    }
+    node_level = m.params.attent_params.attention_model || m.params.dropout;
     H = m.info.LSTM_size;
     L = m.info.num_layers;
     mb = m.params.minibatch_size;
@@ -722,6 +751,7 @@ class model_trainer {
     Vs = m.info.source_vocab_size;
     Vt = m.info.target_vocab_size;
     seq2seq = !m.info.LM;
+    if (node_level) return;
     if ((long long)mb * longest > 65535) {
       std::fprintf(stderr, "model_trainer: minibatch_size * longest_sent must not exceed 65535\n");
       std::exit(EXIT_FAILURE);
@@ -788,12 +818,19 @@ class model_trainer {
     ZOPH_CALL(zr_embed_gradient(ctx, H, V, s.below0, s.d_nn, s.d_mask, T * mb, s.dW));
   }
 
+  bool node_level = false;    // attention or dropout: the step runs through forward_model::compute_gradients
   int lstm_sweep_option = 0;  // the context's ZR_OPT_LSTM_SWEEP setting, restored after a repeated forward pass
   int abandoned_sweeps = 0;   // forward passes that had to be repeated (see train_minibatch)
 
   // Forward, backward and update on the minibatch the reader holds.  Returns the minibatch's log-likelihood (natural
   // log) under the weights BEFORE the update.
   double train_minibatch(minibatch_reader& r, float learning_rate, float norm_clip) {
+    if (node_level) {
+      m.set_training_rates(learning_rate, norm_clip);
+      const double ll = m.getError(r);
+      m.compute_gradients(r);
+      return ll;
+    }
     const int S = seq2seq ? r.current_source_length : 0, T = r.current_target_length;
     const size_t n = (size_t)H * mb;
     std::vector<const dType*> z(L, zeros);
