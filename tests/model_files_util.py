@@ -106,3 +106,66 @@ def random_sentences(g, vocab, n, min_len, max_len, oov_rate=0.1, oov_prefix="oo
                 words.append(vocab[int(g.integers(3, len(vocab)))])
         out.append(words)
     return out
+
+
+def parse_like_reference_script(path):
+    """A second, independent reading of a model file: the steps of the reference's own Python reader for models without
+    attention (scripts/load_model.py:8-20 read_matrix -- `rows` lines of numbers, then one empty line; :53-67 and
+    :121-135 the matrix order of the two layer kinds; :184-186 the loss layer; :264-277 a vocabulary block runs to the
+    next line that starts with "==="; :289-334 header, one separator line, source vocabulary unless the model is a
+    sequence model, target vocabulary, source layers, target layers, loss layer).  The script keys "sequence model" on
+    a three-field header; the current header always has nine fields and a zero source vocabulary instead.
+    Returns (header ints, source vocab or None, target vocab, source layers or None, target layers, D, b) with every layer
+    a dict of the script's parameter names."""
+    f = open(path)
+    head = [int(x) for x in f.readline().split()]
+    L, H, Vt, Vs = head[0], head[1], head[2], head[3]
+    lm = Vs == 0
+    f.readline()
+
+    def vocab():
+        out = {}
+        while True:
+            line = f.readline()
+            assert line, "file ended inside a vocabulary block"
+            if line.startswith("==="):
+                return out
+            idx, word = line.split()
+            out[int(idx)] = word
+
+    def matrix(rows, cols):
+        m = np.zeros((rows, cols))
+        for i in range(rows):
+            vals = [float(x) for x in f.readline().split()]
+            assert len(vals) == cols, "row of %d numbers where %d were expected" % (len(vals), cols)
+            m[i] = vals
+        assert f.readline().strip() == "", "a matrix must be followed by an empty line"
+        return m
+
+    def layer(V):
+        names = ["w_hi", "b_i", "w_hf", "b_f", "w_hc", "b_c", "w_ho", "b_o"] + (["w"] if V else []) + \
+                ["m_i", "m_f", "m_o", "m_c"]
+        out = {}
+        for nme in names:
+            out[nme] = matrix(H, V if nme == "w" else (1 if nme.startswith("b_") else H))
+        return out
+
+    src_vocab = None if lm else vocab()
+    tgt_vocab = vocab()
+    src_layers = None if lm else [layer(Vs)] + [layer(0) for _ in range(L - 1)]
+    tgt_layers = [layer(Vt)] + [layer(0) for _ in range(L - 1)]
+    D, b = matrix(Vt, H), matrix(Vt, 1)
+    assert f.read().strip() == "", "data left after the loss layer"
+    return head, src_vocab, tgt_vocab, src_layers, tgt_layers, D, b
+
+
+def check_layers_against_script_reading(layers_np, embed, parsed_layers):
+    """layers_np: the dictionaries the writers take (gate order i, f, c, o); parsed_layers: parse_like_reference_script's."""
+    gate = {"i": 0, "f": 1, "c": 2, "o": 3}
+    for l, (ly, got) in enumerate(zip(layers_np, parsed_layers)):
+        for g, k in gate.items():
+            assert np.allclose(got["w_h" + g], ly["Wh"][k], rtol=1e-6, atol=0), (l, "w_h" + g)
+            assert np.allclose(got["m_" + g], ly["M"][k], rtol=1e-6, atol=0), (l, "m_" + g)
+            assert np.allclose(got["b_" + g].reshape(-1), ly["b"][k], rtol=1e-6, atol=0), (l, "b_" + g)
+        if l == 0:
+            assert np.allclose(got["w"], embed, rtol=1e-6, atol=0)

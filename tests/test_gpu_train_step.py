@@ -221,3 +221,37 @@ def test_repeated_steps_on_one_minibatch_raise_its_likelihood(tmp_path):
     loss = [float(ln.split()[2]) for ln in r.stdout.splitlines() if ln.startswith("loss")]
     assert len(loss) == 12 and all(b > a for a, b in zip(loss, loss[1:])), [round(v, 2) for v in loss]
     assert loss[-1] > loss[0] + 0.1 * abs(loss[0])
+
+
+@pytest.mark.parametrize("lm,L", [(False, 2), (True, 1)])
+def test_model_file_dumped_by_the_layer_objects_reads_back_under_the_reference_scripts_layout(tmp_path, lm, L):
+    """The C++ side's writer (forward_model::dump_weights -> the layers' dump_weights members) against the second
+    description of the format, the reference's own Python reader restated in model_files_util.parse_like_reference_script:
+    a model is loaded and dumped again without a training step (steps = 0)."""
+    if not os.path.exists(DRIVER):
+        pytest.fail("tests/host/train_step is not built: run `python __graft_entry__.py build`")
+    g = synth.rng(133, L)
+    H, mb = 16, 2
+    src_vocab = ["<UNK>"] + mf.make_vocab(12, "s")
+    tgt_vocab = ["<START>", "<EOF>", "<UNK>"] + mf.make_vocab(14, "t")
+    Vs, Vt = len(src_vocab), len(tgt_vocab)
+    m = {"emb_t": synth.uniform(g, (H, Vt)), "tgt_layers": [synth.lstm_layer(g, H, forget_bias_one=True) for _ in range(L)],
+         "D": synth.uniform(g, (Vt, H)), "b_d": synth.uniform(g, (Vt,))}
+    if not lm:
+        m["emb_s"] = synth.uniform(g, (H, Vs))
+        m["src_layers"] = [synth.lstm_layer(g, H) for _ in range(L)]
+    model = tmp_path / "model.nn"
+    _write_model(model, m, tgt_vocab, src_vocab, lm)
+    data = tmp_path / "data.int"
+    data.write_text("")
+    args = (["--sequence"] if lm else []) + [str(model), str(data), str(mb), "8", "0.5", "5", "0"]
+    r = subprocess.run([DRIVER] + args, capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr[-2000:]
+    head, sv, tv, sl, tl, D, b = mf.parse_like_reference_script(str(model) + ".trained")
+    assert head[:4] == [L, H, Vt, 0 if lm else Vs]
+    assert tv == dict(enumerate(tgt_vocab))
+    if not lm:
+        assert sv == dict(enumerate(src_vocab))
+        mf.check_layers_against_script_reading(m["src_layers"], m["emb_s"], sl)
+    mf.check_layers_against_script_reading(m["tgt_layers"], m["emb_t"], tl)
+    assert np.allclose(D, m["D"], rtol=1e-6, atol=0) and np.allclose(b.reshape(-1), m["b_d"], rtol=1e-6, atol=0)

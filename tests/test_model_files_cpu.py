@@ -75,3 +75,44 @@ def test_too_long_sentence_is_an_error_not_a_truncation(tmp_path):
     sv, tv, src, tgt, model, sp, tp = _setup(tmp_path)
     r = mf.run_force_decode(["--integerize-only", "--longest-sent", 6, model, sp, tp, tmp_path / "o.txt"])
     assert r.returncode == 1 and "longer than longest_sent" in r.stderr
+
+
+@pytest.mark.parametrize("lm,L", [(False, 2), (True, 1), (False, 1)])
+def test_written_model_files_read_back_under_the_reference_scripts_layout(tmp_path, lm, L):
+    """The test-suite's model writer against a second description of the format: the reference's own Python reader for
+    models without attention (scripts/load_model.py), restated in model_files_util.parse_like_reference_script.  Pins
+    the separator and vocabulary lines, one matrix row per line, the empty line behind every matrix and the order of
+    the matrices of both layer kinds and the loss layer (gates are distinct random matrices, so a swapped pair fails)."""
+    from test_gpu_host_layers import _write_hh, _write_ih, _write_matrix
+    g = synth.rng(77, L + int(lm))
+    H = 6
+    src_vocab = ["<UNK>"] + mf.make_vocab(7, "s")
+    tgt_vocab = ["<START>", "<EOF>", "<UNK>"] + mf.make_vocab(9, "t")
+    Vs, Vt = len(src_vocab), len(tgt_vocab)
+    m = {"emb_t": synth.uniform(g, (H, Vt)), "tgt_layers": [synth.lstm_layer(g, H, forget_bias_one=True) for _ in range(L)],
+         "D": synth.uniform(g, (Vt, H)), "b_d": synth.uniform(g, (Vt,))}
+    if not lm:
+        m["emb_s"] = synth.uniform(g, (H, Vs))
+        m["src_layers"] = [synth.lstm_layer(g, H) for _ in range(L)]
+    path = tmp_path / "m.nn"
+    with open(path, "w") as f:
+        mf.write_header(f, L, H, tgt_vocab, src_vocab, False, False, lm=lm)
+        if not lm:
+            _write_ih(f, m["src_layers"][0], m["emb_s"])
+            for ly in m["src_layers"][1:]:
+                _write_hh(f, ly)
+        _write_ih(f, m["tgt_layers"][0], m["emb_t"])
+        for ly in m["tgt_layers"][1:]:
+            _write_hh(f, ly)
+        _write_matrix(f, m["D"])
+        _write_matrix(f, m["b_d"].reshape(-1, 1))
+    head, sv, tv, sl, tl, D, b = mf.parse_like_reference_script(path)
+    assert head[:4] == [L, H, Vt, 0 if lm else Vs]
+    assert tv == dict(enumerate(tgt_vocab))
+    if lm:
+        assert sv is None and sl is None
+    else:
+        assert sv == dict(enumerate(src_vocab))
+        mf.check_layers_against_script_reading(m["src_layers"], m["emb_s"], sl)
+    mf.check_layers_against_script_reading(m["tgt_layers"], m["emb_t"], tl)
+    assert np.allclose(D, m["D"], rtol=1e-7, atol=0) and np.allclose(b.reshape(-1), m["b_d"], rtol=1e-7, atol=0)
