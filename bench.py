@@ -140,9 +140,9 @@ def bench_decoder_step(ctx, steps, warmup, H=1000, mb=128, S=50, V=50000, L=4, D
         ctx.softmax_forward(dD, dbd, V, H, d_ht, mb, capi.ZR_SOFTMAX_PROB, d_prob)
 
     def step():
-        lstm_part()
-        attn_part()
-        softmax_part()
+        # forward_prop_target as one call: the three parts below with their hand-overs kept in the matrix cores' layout
+        ctx.decoder_step([ly.w for ly in layers], d_embed, V, d_ids, d_hp, d_cp, d_mask, mb, d_h, d_c, attn, d_bi, d_ht, dD,
+                         dbd, V, capi.ZR_SOFTMAX_PROB, d_prob, d_htild_prev=d_htp)
 
     wall_ms, ev_ms = time_region(ctx, step, steps, warmup)
     parts = {}

@@ -425,6 +425,21 @@ int zr_attn_backward(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, const flo
                      const float* d_h_tild, const float* d_alignments, const int* d_indices, const float* d_p_t,
                      const float* d_c_t, const float* d_err_htild, float* d_err_h_t, const zr_attn_grads* grads);
 
+/* One decoder time step from the current words to the output distribution: neuralMT_model::forward_prop_target
+ * (src/model.hpp:2573-2688) as one call -- zr_lstm_decoder_step, then zr_attn_step on the top layer's h_t (attn may be
+ * NULL: no attention), then zr_softmax_forward on h~ (or on the top h_t).  Same kernels and the same results as the three
+ * calls; what the call adds is that the activations handed from one stage to the next stay in the matrix cores'
+ * k-interleaved layout (the LSTM launch writes the top layer's h that way for the attention products, the attention
+ * output product writes h~ that way for the output layer), so the two re-layout launches between the stages go away.
+ *   V_in: rows of d_embed's vocabulary; V_out, d_D, d_b_d, mode, d_out: as in zr_softmax_forward;
+ *   d_alignments, d_indices, d_p_t, d_c_ctx: as in zr_attn_step (NULL: not wanted). */
+int zr_decoder_step(zr_ctx* ctx, int L, const zr_lstm_weights* const layers[], const float* d_embed, int V_in,
+                    const int* d_ids_nonneg, const float* const d_hprev[], const float* const d_cprev[],
+                    const float* d_htild_prev, const int* d_mask01, float clip_threshold, int mb, float* const d_h[],
+                    float* const d_c[], zr_attn* attn, const int* d_batch_info, float* d_htild, float* d_alignments,
+                    int* d_indices, float* d_p_t, float* d_c_ctx, const float* d_D, const float* d_b_d, int V_out,
+                    int mode, float* d_out);
+
 /* dropout_kernel (src/custom_kernels.h:1556-1560; forward call sites src/LSTM.hpp:118, src/LSTM_HH.hpp:124,
  * src/attention_node.hpp:105, src/softmax.hpp:477, backward :647, src/LSTM_HH.hpp:674, src/softmax.hpp:746):
  * x = (uniform < keep_rate) * (1 / keep_rate) * x, in place; keep_rate is the probability of KEEPING a value. */

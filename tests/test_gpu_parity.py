@@ -802,6 +802,65 @@ def test_decoder_step_single_launch_abandoned_wait_is_reported(ctx):
         assert_close(c2[l], want_c[l], what="c of layer %d" % l)
 
 
+@pytest.mark.parametrize("H,mb,L,S,D,V,prepared", [(1000, 128, 4, 20, 10, 5000, True), (64, 5, 2, 9, 3, 301, True),
+                                                   (1000, 128, 2, 12, 12, 2000, False), (100, 8, 1, 7, 2, 333, True),
+                                                   (256, 64, 3, 30, 50, 40000, True)])
+def test_decoder_step_as_one_call_matches_the_three_calls(ctx, H, mb, L, S, D, V, prepared):
+    """zr_decoder_step (forward_prop_target as one call, hand-overs kept in the matrix cores' layout) against
+    zr_lstm_decoder_step + zr_attn_step + zr_softmax_forward on the same inputs: the same kernels read the same numbers,
+    so every output is the same bit for bit -- with and without the prepared snapshots, with an LSTM stack that takes
+    the single launch and one that does not, with a layer size the packed layout does not cover."""
+    g = synth.rng(35, H + mb + L)
+    case = _decoder_step_case(g, H, mb, L, True, V=V)
+    layers, embed, ids, hp, cp, ht, mask = case
+    w = synth.attention_weights(g, H)
+    hs = (g.standard_normal(size=(S, H, mb), dtype=np.float32) * np.float32(0.1))
+    lens = g.integers(1, S + 1, size=mb).astype(np.int32)
+    binfo = np.concatenate([lens, S - lens]).astype(np.int32)
+    Dm, bd = U(g, (V, H)), U(g, (V,))
+    lys = [Layer(ctx, ly) for ly in layers]
+    tables = [ctx.array(np.asfortranarray(hs[t])) for t in range(S)]
+    dw = {k: ctx.array(v) for k, v in w.items()}
+    a = ctx.attn_create(H, mb, D, dw["W_a"], dw["W_p"], dw["v_p"], dw["out_bias"], dw["W_c1"], dw["W_c2"], tables)
+    dD, dbd = ctx.array(Dm), ctx.array(bd)
+    if prepared:
+        ctx.attn_prepare(a)
+        ctx.softmax_prepare(dD, V, H)
+    try:
+        d_embed, d_ids, d_mask, d_bi = ctx.array(embed), ctx.array(ids), ctx.array(mask), ctx.array(binfo)
+        d_hp, d_cp, d_htp = [ctx.array(x) for x in hp], [ctx.array(x) for x in cp], ctx.array(ht)
+        outs = []
+        for one_call in (False, True):
+            d_h = [ctx.zeros((H, mb)) for _ in range(L)]
+            d_c = [ctx.zeros((H, mb)) for _ in range(L)]
+            d_ht, d_p = ctx.zeros((H, mb)), ctx.zeros((V, mb))
+            if one_call:
+                ctx.decoder_step([ly.w for ly in lys], d_embed, V, d_ids, d_hp, d_cp, d_mask, mb, d_h, d_c, a, d_bi, d_ht, dD,
+                                 dbd, V, capi.ZR_SOFTMAX_PROB, d_p, d_htild_prev=d_htp, clip=0.8)
+            else:
+                ctx.lstm_decoder_step([ly.w for ly in lys], d_embed, V, d_ids, d_hp, d_cp, d_mask, mb, d_h, d_c,
+                                      d_htild=d_htp, clip=0.8)
+                ctx.attn_step(a, d_bi, d_h[L - 1], d_mask, d_ht)
+                ctx.softmax_forward(dD, dbd, V, H, d_ht, mb, capi.ZR_SOFTMAX_PROB, d_p)
+            ctx.sync()
+            outs.append([x.get() for x in d_h + d_c + [d_ht, d_p]])
+        for x, y in zip(*outs):
+            assert x.tobytes() == y.tobytes()
+        want_h, _ = _oracle_decoder_step(case)
+        assert_close(outs[1][L - 1], want_h[L - 1], what="top h")
+        att = o.attention_forward(hs_table=hs, batch_info=binfo, h_t=want_h[L - 1], mask01=mask, D=D, **w)
+        assert_close(outs[1][2 * L], att["h_tild"], what="h_tild")
+        cols = np.array([0, mb // 2, mb - 1])
+        want_p = o.softmax_dist(o.softmax_logits(Dm, bd, np.asfortranarray(att["h_tild"][:, cols])))
+        assert_close(outs[1][2 * L + 1][:, cols], want_p, floor=1e-7, what="probabilities (sampled columns)")
+    finally:
+        if prepared:
+            ctx.softmax_release(dD)
+        ctx.attn_destroy(a)
+        for ly in lys:
+            ly.close()
+
+
 def test_stack_forward_with_split_kernel_forced(ctx):
     g = synth.rng(17, 1)
     H, mb, T, V, L = 64, 5, 7, 211, 3

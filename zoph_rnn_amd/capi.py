@@ -43,7 +43,7 @@ SYMBOLS = [
     "zr_unstack_gates", "zr_lstm_stack_backward", "zr_lstm_weight_gradients", "zr_embed_gradient",
     "zr_softmax_backward", "zr_sgd_update", "zr_lstm_node_backward", "zr_lstm_node_gradients",
     "zr_softmax_backward_accumulate", "zr_gather_columns_multi", "zr_softmax_backward_loss",
-    "zr_softmax_forward_static", "zr_ctx_query", "zr_attn_prepare", "zr_lstm_step_embed", "zr_attn_viterbi", "zr_lstm_decoder_step", "zr_lstm_feed_backward", "zr_attn_set_error_tables",
+    "zr_softmax_forward_static", "zr_ctx_query", "zr_attn_prepare", "zr_lstm_step_embed", "zr_attn_viterbi", "zr_lstm_decoder_step", "zr_decoder_step", "zr_lstm_feed_backward", "zr_attn_set_error_tables",
     "zr_attn_backward", "zr_dropout_apply", "zr_uniform_fill", "zr_add_inplace",
 ]
 
@@ -220,6 +220,17 @@ class Context:
         _chk(load().zr_lstm_decoder_step(self.h, C.c_int(L), larr, _vp(d_embed), C.c_int(V), _vp(d_ids),
                                          _ptr_array(hprev), _ptr_array(cprev), _vp(d_htild), _vp(d_mask),
                                          C.c_float(clip), C.c_int(mb), _ptr_array(h), _ptr_array(c)))
+
+    def decoder_step(self, layers, d_embed, V_in, d_ids, hprev, cprev, d_mask, mb, h, c, attn, d_batch_info, d_htild, d_D,
+                     d_b_d, V_out, mode, d_out, d_htild_prev=None, clip=0.0, d_align=None, d_idx=None, d_pt=None,
+                     d_ctx=None):
+        L = len(layers)
+        larr = (C.c_void_p * L)(*[w.value for w in layers])
+        _chk(load().zr_decoder_step(self.h, C.c_int(L), larr, _vp(d_embed), C.c_int(V_in), _vp(d_ids), _ptr_array(hprev),
+                                    _ptr_array(cprev), _vp(d_htild_prev), _vp(d_mask), C.c_float(clip), C.c_int(mb),
+                                    _ptr_array(h), _ptr_array(c), attn, _vp(d_batch_info), _vp(d_htild), _vp(d_align),
+                                    _vp(d_idx), _vp(d_pt), _vp(d_ctx), _vp(d_D), _vp(d_b_d), C.c_int(V_out), C.c_int(mode),
+                                    _vp(d_out)))
 
     def lstm_gates(self, d_preact, b, d_cprev, d_mask, H, mb, d_h, d_c, clip=0.0, gates=None):
         _chk(load().zr_lstm_gates(self.h, _vp(d_preact), _ptr_array(b), _vp(d_cprev), _vp(d_mask), C.c_float(clip),

@@ -547,7 +547,7 @@ int zr_attn_prepare(zr_ctx* ctx, zr_attn* a) {
   const int ldp = (H + 31) / 32 * 32, kp = (H + 7) / 8 * 8;
   const size_t per = (size_t)kp * ldp;
   if (!a->d_pack32) {
-    if (hipMalloc((void**)&a->d_pack32, sizeof(float) * (4 * per + 2 * (size_t)H * a->mb)) != hipSuccess) {
+    if (hipMalloc((void**)&a->d_pack32, sizeof(float) * (4 * per + 3 * (size_t)H * a->mb)) != hipSuccess) {
       (void)hipGetLastError();
       a->d_pack32 = nullptr;
       return zr_set_error(ZR_ENOMEM, "zr_attn_prepare: allocation failed");
@@ -559,6 +559,7 @@ int zr_attn_prepare(zr_ctx* ctx, zr_attn* a) {
   // output product multiplies with [W_c1 | W_c2], whose snapshots are neighbours as well
   a->d_cpack = a->d_pack32 + 4 * per;
   a->d_hpack = a->d_cpack + (size_t)H * a->mb;
+  a->d_htpack = a->d_hpack + (size_t)H * a->mb;
   rc = zr_pack4_launch(ctx, a->W_p, H, H, H, ldp, kp, a->d_pack32);
   if (rc) return rc;
   rc = zr_pack4_trans_launch(ctx, a->W_a, H, H, H, ldp, kp, a->d_pack32 + per);  // W_a^T
@@ -581,8 +582,50 @@ int zr_attn_destroy(zr_ctx* ctx, zr_attn* a) {
   return ZR_OK;
 }
 
+static int attn_step_impl(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, const float* d_h_t, const int* d_mask01,
+                          float* d_htild, float* d_alignments, int* d_indices, float* d_p_t, float* d_c_ctx,
+                          bool h_packed, float* d_htild_pack);
+
 int zr_attn_step(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, const float* d_h_t, const int* d_mask01,
                  float* d_htild, float* d_alignments, int* d_indices, float* d_p_t, float* d_c_ctx) {
+  return attn_step_impl(ctx, a, d_batch_info, d_h_t, d_mask01, d_htild, d_alignments, d_indices, d_p_t, d_c_ctx, false,
+                        nullptr);
+}
+
+// True when zr_attn_step on these operands takes the path that reads a->d_hpack (and can write h~ k-interleaved).
+static bool attn_reads_packed_h(const zr_attn* a, const float* d_h_t, const float* d_c_ctx) {
+  const float* cctx = d_c_ctx ? d_c_ctx : a->d_ctx;
+  return a->d_pack32 && !a->d_bf16 && (a->H % 8 == 0) && a->tables_aligned && (((uintptr_t)cctx & 15u) == 0) &&
+         (((uintptr_t)d_h_t & 15u) == 0);
+}
+
+int zr_decoder_step(zr_ctx* ctx, int nl, const zr_lstm_weights* const layers[], const float* d_embed, int V_in,
+                    const int* d_ids_nonneg, const float* const d_hprev[], const float* const d_cprev[],
+                    const float* d_htild_prev, const int* d_mask01, float clip_threshold, int mb, float* const d_h[],
+                    float* const d_c[], zr_attn* attn, const int* d_batch_info, float* d_htild, float* d_alignments,
+                    int* d_indices, float* d_p_t, float* d_c_ctx, const float* d_D, const float* d_b_d, int V_out,
+                    int mode, float* d_out) {
+  ZR_CHECK_ARG(nl > 0 && d_h && d_D && d_b_d && d_out, "zr_decoder_step: null pointer or L = %d", nl);
+  ZR_CHECK_ARG(!attn || (attn->mb == mb && d_batch_info && d_htild), "zr_decoder_step: attention layer of another width, or "
+               "null batch info / h~");
+  const float* top = d_h[nl - 1];
+  const bool packed = attn && top && attn_reads_packed_h(attn, top, d_c_ctx);
+  int wrote = 0;
+  int rc = zr_lstm_decoder_step_packed(ctx, nl, layers, d_embed, V_in, d_ids_nonneg, d_hprev, d_cprev, d_htild_prev,
+                                       d_mask01, clip_threshold, mb, d_h, d_c, packed ? attn->d_hpack : nullptr, &wrote);
+  if (rc) return rc;
+  if (!attn)
+    return zr_softmax_forward_packed(ctx, d_D, d_b_d, V_out, layers[0]->H, top, nullptr, mb, mode, d_out, nullptr);
+  rc = attn_step_impl(ctx, attn, d_batch_info, top, d_mask01, d_htild, d_alignments, d_indices, d_p_t, d_c_ctx,
+                      packed && wrote, packed ? attn->d_htpack : nullptr);
+  if (rc) return rc;
+  return zr_softmax_forward_packed(ctx, d_D, d_b_d, V_out, attn->H, d_htild, packed ? attn->d_htpack : nullptr, mb, mode,
+                                   d_out, nullptr);
+}
+
+static int attn_step_impl(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, const float* d_h_t, const int* d_mask01,
+                          float* d_htild, float* d_alignments, int* d_indices, float* d_p_t, float* d_c_ctx,
+                          bool h_packed, float* d_htild_pack) {
   int rc = zr_bind_device(ctx);
   if (rc) return rc;
   ZR_CHECK_ARG(a != nullptr, "zr_attn_step: attention object is null");
@@ -610,7 +653,7 @@ int zr_attn_step(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, const float* 
     // with H % 8 == 0 the products read k-interleaved activations (contiguous 16-byte loads instead of 16 bytes from
     // each of 32 lines per half-wave): h_t is re-laid-out once for both products, the context is written that way
     const bool bp = H % 8 == 0;
-    if (bp) {
+    if (bp && !h_packed) {
       rc = zr_pack4_x_launch(ctx, d_h_t, H, mb, H, a->d_hpack);
       if (rc) return rc;
     }
@@ -670,6 +713,7 @@ int zr_attn_step(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, const float* 
       o.ldb[0] = o.ldb[1] = H;
     }
     o.C = d_htild;
+    o.Cpack = bp ? d_htild_pack : nullptr;
     o.ldc = H;
     o.batch = 1;
     o.bias = a->out_bias;

@@ -21,6 +21,7 @@ struct GemmArgs {
   const float* bias;
   const int* mask;
   float* partials;
+  float* Cpack;          // ZR_EPI_TANH_BIAS_MASK: second, k-interleaved copy of the result (null: none)
   int m_tiles, n_tiles;  // wave tiles along M and N
   int b_pack4;           // B segments are k-interleaved copies: element (k, n) at ((k/4)*N + n)*4 + k%4
   // bf16 weights: B[s] is the bf16 "hi" array and Blo[s] the "lo" array of the split activations, both
@@ -234,7 +235,11 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& a, int m0, int n0, boo
       } else if (EPI == ZR_EPI_TANH) {
         if (ok) C[(long long)n * a.ldc + m] = tanhf(v);
       } else {  // ZR_EPI_TANH_BIAS_MASK
-        if (ok) C[(long long)n * a.ldc + m] = tanhf(v + bias[m]) * (float)a.mask[n];
+        if (ok) {
+          const float t = tanhf(v + bias[m]) * (float)a.mask[n];
+          C[(long long)n * a.ldc + m] = t;
+          if (a.Cpack) a.Cpack[((long long)(m >> 2) * a.N + n) * 4 + (m & 3)] = t;
+        }
       }
     }
   });
@@ -851,6 +856,9 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
   ga.bias = d.bias;
   ga.mask = d.mask;
   ga.partials = d.partials;
+  ga.Cpack = d.Cpack;
+  ZR_CHECK_ARG(!d.Cpack || (d.epilogue == ZR_EPI_TANH_BIAS_MASK && d.batch <= 1 && d.groups == 0),
+               "gemm: a k-interleaved second result needs the tanh-bias-mask epilogue and a single problem");
   ga.accum = d.accumulate;
   if (d.epilogue == ZR_EPI_TANH_BIAS_MASK) ZR_CHECK_ARG(d.bias && d.mask, "gemm: bias/mask required");
   ZR_CHECK_ARG(!d.accumulate || d.epilogue == ZR_EPI_STORE, "gemm: accumulate needs the plain store epilogue");

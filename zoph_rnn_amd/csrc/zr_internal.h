@@ -122,6 +122,8 @@ struct ZrGemmDesc {
   const int* mask;    // per column n (ZR_EPI_TANH_BIAS_MASK)
   int epilogue;
   float* partials;  // ZR_EPI_SOFTMAX_PARTIAL: [N][ceil(M/32)][2] floats (contiguous per column)
+  float* Cpack;     // ZR_EPI_TANH_BIAS_MASK, single batch: the result is also stored k-interleaved, element (m, n) at
+                    // ((m/4)*N + n)*4 + m%4 -- the layout a following product with b_packed reads (null: not wanted)
   int accumulate;   // ZR_EPI_STORE only: C += product (+ bias) instead of C = ...
   // groups > 0: that many independent problems of the same shape in one launch (at most 8; one segment, plain store
   // epilogue, no bias): problem g multiplies gA[g] (instead of A[0]) with gB[g] (instead of B[0]) into gC[g]
@@ -167,6 +169,18 @@ struct zr_lstm_weights {
   float* d_bias;   // [4][H]
 };
 
+// Pieces of zr_decoder_step (zr_attention.hip): the three public calls with the hand-overs between them kept in the
+// k-interleaved layout.  d_hp_top (zr_lstm_decoder_step): where the top layer's h is also written as [H/4][mb][4];
+// *wrote_hp_top tells whether it was (only the single-launch path does).  h_packed (zr_attn_step): a->d_hpack already
+// holds that copy of d_h_t; d_htild_pack: h~ is also written k-interleaved there.  d_h_packed (zr_softmax_forward):
+// a k-interleaved copy of d_h, used when the registered matrix allows it.
+int zr_lstm_decoder_step_packed(zr_ctx* ctx, int nl, const zr_lstm_weights* const layers[], const float* d_embed, int V,
+                                const int* d_ids_nonneg, const float* const d_hprev[], const float* const d_cprev[],
+                                const float* d_htild, const int* d_mask01, float clip_threshold, int mb,
+                                float* const d_h[], float* const d_c[], float* d_hp_top, int* wrote_hp_top);
+int zr_softmax_forward_packed(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h,
+                              const float* d_h_packed, int mb, int mode, float* d_out, float* d_logits_scratch);
+
 // The attention layer's handle (zr_attention.hip; the backward pass lives in zr_backward.hip).
 struct zr_attn {
   int H, mb, D, longest_sent;
@@ -183,6 +197,7 @@ struct zr_attn {
   float* d_pack32;
   int ldp32, kp32;
   float *d_hpack, *d_cpack;  // k-interleaved copies ([H/4][mb][4]) of h_t and of the context (inside d_pack32's block)
+  float* d_htpack;           // the same of h~, written by the output product for zr_decoder_step (same block)
   float** d_err_table;       // zr_attn_set_error_tables: device copy of the source-state error pointers (null: none)
 };
 

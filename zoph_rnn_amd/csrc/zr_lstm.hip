@@ -853,6 +853,7 @@ struct LstmDecStack {
   const float* htild;             // previous attention output for layer 0's Q segment (null: none)
   const int* mask01;              // [mb]
   float* hp;                      // [nl] k-interleaved copies of h, H*mb floats each
+  float* hp_top;                  // optional: the top layer's h k-interleaved, for the caller's next product
   float* partials;                // [nl][tile][visit][gate][thread]: role 1's sums
   int* counters;                  // [nl][tiles] tile flags, then [nl][n_tiles] layer counters at kSweepCtrStride
   int n_counters;                 // ints in `counters` (all of them are marked when a wait is abandoned)
@@ -1064,6 +1065,7 @@ __global__ void __launch_bounds__(256) lstm_decoder_stack_kernel(LstmDecStack P)
       }
       float* h_out = P.h[l];
       float* c_out = P.c[l];
+      float* hp_top = hand_on ? nullptr : P.hp_top;
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
         const int slot = zr_wide_visit_slot<KS>(kslice, i);
@@ -1072,6 +1074,7 @@ __global__ void __launch_bounds__(256) lstm_decoder_stack_kernel(LstmDecStack P)
           const long long ix = (long long)n * H + j;
           c_out[ix] = c_v[i];
           h_out[ix] = h_v[i];
+          if (hp_top) hp_top[((long long)(j >> 2) * mb + n) * 4 + (j & 3)] = h_v[i];
         }
       }
     }
@@ -1519,6 +1522,17 @@ int zr_lstm_decoder_step(zr_ctx* ctx, int nl, const zr_lstm_weights* const layer
                          const int* d_ids_nonneg, const float* const d_hprev[], const float* const d_cprev[],
                          const float* d_htild, const int* d_mask01, float clip_threshold, int mb,
                          float* const d_h[], float* const d_c[]) {
+  return zr_lstm_decoder_step_packed(ctx, nl, layers, d_embed, V, d_ids_nonneg, d_hprev, d_cprev, d_htild, d_mask01,
+                                     clip_threshold, mb, d_h, d_c, nullptr, nullptr);
+}
+
+}  // extern "C"
+
+int zr_lstm_decoder_step_packed(zr_ctx* ctx, int nl, const zr_lstm_weights* const layers[], const float* d_embed, int V,
+                                const int* d_ids_nonneg, const float* const d_hprev[], const float* const d_cprev[],
+                                const float* d_htild, const int* d_mask01, float clip_threshold, int mb,
+                                float* const d_h[], float* const d_c[], float* d_hp_top, int* wrote_hp_top) {
+  if (wrote_hp_top) *wrote_hp_top = 0;
   int rc = zr_bind_device(ctx);
   if (rc) return rc;
   ZR_CHECK_ARG(nl > 0 && nl <= kMaxUnits && mb > 0 && V > 0, "zr_lstm_decoder_step: L = %d, mb = %d, V = %d", nl, mb, V);
@@ -1575,6 +1589,8 @@ int zr_lstm_decoder_step(zr_ctx* ctx, int nl, const zr_lstm_weights* const layer
       }
       P.in0 = d_embed;
       P.ids = d_ids_nonneg;
+      P.hp_top = d_hp_top;
+      if (wrote_hp_top && d_hp_top) *wrote_hp_top = 1;
       P.htild = d_htild;
       P.mask01 = d_mask01;
       P.status = ctx->d_flags + 2;
@@ -1607,6 +1623,8 @@ int zr_lstm_decoder_step(zr_ctx* ctx, int nl, const zr_lstm_weights* const layer
   }
   return ZR_OK;
 }
+
+extern "C" {
 
 int zr_lstm_stack_forward(zr_ctx* ctx, int nl, const zr_lstm_weights* const layers[], const float* d_embed, int V,
                           const int* d_ids_nonneg, const int* d_mask01, int T, int mb,

@@ -163,8 +163,10 @@ softmax_loss_kernel(const float* __restrict__ logits, int V, int mb, const doubl
   if (tid == 0) loss[0] = s[0];
 }
 
+// d_h_packed: optional k-interleaved copy of d_h ([H/4][mb][4]); used when the product runs on the registered fp32 copy
+// of D and H % 8 == 0 (the product then skips its own re-layout of d_h).
 int logits_with_partials(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int mb,
-                         float* d_logits, float** partials_out, int* nblocks_out) {
+                         float* d_logits, float** partials_out, int* nblocks_out, const float* d_h_packed = nullptr) {
   const int nblocks = zr_softmax_partial_blocks(V);
   void* scratch = nullptr;
   // partials [mb][nblocks][2] followed by column stats (2 doubles per column, also used as 2 floats)
@@ -192,6 +194,10 @@ int logits_with_partials(zr_ctx* ctx, const float* d_D, const float* d_b_d, int 
   }
   d.B[0] = d_h;
   d.ldb[0] = H;
+  if (d_h_packed && d.a_pack == 1 && H % 8 == 0 && (((uintptr_t)d_h_packed & 15u) == 0)) {
+    d.B[0] = d_h_packed;
+    d.b_packed = 1;
+  }
   d.C = d_logits;
   d.ldc = V;
   d.batch = 1;
@@ -288,6 +294,13 @@ int zr_softmax_release(zr_ctx* ctx, const float* d_D) {
 
 int zr_softmax_forward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int mb,
                        int mode, float* d_out, float* d_logits_scratch) {
+  return zr_softmax_forward_packed(ctx, d_D, d_b_d, V, H, d_h, nullptr, mb, mode, d_out, d_logits_scratch);
+}
+
+}  // extern "C"
+
+int zr_softmax_forward_packed(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h,
+                              const float* d_h_packed, int mb, int mode, float* d_out, float* d_logits_scratch) {
   int rc = zr_bind_device(ctx);
   if (rc) return rc;
   rc = check_softmax_args("zr_softmax_forward", d_D, d_b_d, V, H, d_h, mb);
@@ -297,7 +310,7 @@ int zr_softmax_forward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V,
   float* logits = d_logits_scratch ? d_logits_scratch : d_out;
   float* partials = nullptr;
   int nblocks = 0;
-  rc = logits_with_partials(ctx, d_D, d_b_d, V, H, d_h, mb, logits, &partials, &nblocks);
+  rc = logits_with_partials(ctx, d_D, d_b_d, V, H, d_h, mb, logits, &partials, &nblocks, d_h_packed);
   if (rc) return rc;
   float* colstats = (float*)stats_ptr(partials, nblocks, mb);
   softmax_colstats_kernel<<<mb, 256, 0, ctx->stream>>>(partials, nblocks, colstats);
@@ -319,6 +332,8 @@ int zr_softmax_forward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V,
   ZR_LAUNCH_CHECK("softmax_normalize_kernel");
   return ZR_OK;
 }
+
+extern "C" {
 
 // zr_softmax_forward on the device's statically allocated scratch array: same kernels, no allocation.  The array is
 // split into the two buffers the product needs (re-laid-out activations, then partial column statistics + column

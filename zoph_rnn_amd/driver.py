@@ -101,11 +101,9 @@ class BeamDecode:
         p, q = self.cur, 1 - self.cur
         ctx.vocab_prep(self.d_words, cols, w.Vt, self.d_words_nn, None)
         feed = self.h_tild[p] if self.step_index > 0 else None
-        ctx.lstm_decoder_step(w.tgt, w.tgt_embed, w.Vt, self.d_words_nn, self.h[p], self.c[p], self.d_ones, cols,
-                              self.h[q], self.c[q], d_htild=feed)
-        below = self.h[q][L - 1]
-        ctx.attn_step(self.attn, self.d_batch_info, below, self.d_ones, self.h_tild[q])
-        ctx.softmax_forward(w.D_soft, w.b_soft, w.Vt, H, self.h_tild[q], cols, capi.ZR_SOFTMAX_PROB, self.prob)
+        ctx.decoder_step(w.tgt, w.tgt_embed, w.Vt, self.d_words_nn, self.h[p], self.c[p], self.d_ones, cols, self.h[q],
+                         self.c[q], self.attn, self.d_batch_info, self.h_tild[q], w.D_soft, w.b_soft, w.Vt,
+                         capi.ZR_SOFTMAX_PROB, self.prob, d_htild_prev=feed)
 
     def step(self, record=False):
         """One decode step: forward, expand the beam, reorder the states by the back-pointers."""

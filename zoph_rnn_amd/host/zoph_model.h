@@ -999,19 +999,14 @@ class beam_decoder {
   void forward_target(int p, int step_index) {
     const int q = 1 - p;
     ZOPH_CALL(zr_vocab_prep(ctx, d_words, cols, Vt, d_words_nn, nullptr));
-    // all layers of the step in one call; layer 0 looks its input columns up in the embedding itself
+    // the whole step in one call: all LSTM layers (layer 0 looks its input columns up in the embedding itself), the
+    // attention step on the top layer's h_t, the output distribution of h~
     const dType* feed = (feed_input && step_index > 0) ? h_tild[p] : nullptr;
     std::vector<const dType*> hp(h[p].begin(), h[p].end()), cp(c[p].begin(), c[p].end());
-    ZOPH_CALL(zr_lstm_decoder_step(ctx, L, tgt_w.data(), m.input_layer_target.d_W, Vt, d_words_nn, hp.data(), cp.data(),
-                                   feed, d_ones, 0.0f, cols, h[q].data(), c[q].data()));
-    const dType* below = h[q][L - 1];
-    const dType* top = below;
-    if (attention) {
-      ZOPH_CALL(zr_attn_step(ctx, attn, d_batch_info, below, d_ones, h_tild[q], nullptr, nullptr, nullptr, nullptr));
-      top = h_tild[q];
-    }
-    ZOPH_CALL(zr_softmax_forward(ctx, m.softmax_obj.d_D, m.softmax_obj.d_b_d, Vt, H, top, cols, ZR_SOFTMAX_PROB, prob,
-                                 nullptr));
+    ZOPH_CALL(zr_decoder_step(ctx, L, tgt_w.data(), m.input_layer_target.d_W, Vt, d_words_nn, hp.data(), cp.data(), feed,
+                              d_ones, 0.0f, cols, h[q].data(), c[q].data(), attention ? attn : nullptr, d_batch_info,
+                              attention ? h_tild[q] : nullptr, nullptr, nullptr, nullptr, nullptr, m.softmax_obj.d_D,
+                              m.softmax_obj.d_b_d, Vt, ZR_SOFTMAX_PROB, prob));
   }
 
   // Decodes up to n_sent sentences whose integerized sources (reversed, no padding) all have the same length S.
