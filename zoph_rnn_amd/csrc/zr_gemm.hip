@@ -342,16 +342,24 @@ __global__ void __launch_bounds__(256) gemm_rows_kernel(GemmArgs a, int row_chun
 }
 
 // Tall weight matrix (k-interleaved) times a minibatch that is a multiple of 128 columns wide, balanced over the
-// CUs without a persistent loop.  One 64-row x 128-column tile per workgroup runs at the best rate this core reaches
-// (all 512 registers of a wave: 128 accumulators and a six-deep operand ring), but the number of such tiles is rarely a
-// multiple of the number of CUs, and a last, mostly empty round costs as much as a full one.  So only as many
+// CUs without a persistent loop.  A workgroup takes one 64-row x 128-column tile; two workgroups share a CU (256
+// registers each: 128 accumulators and a two-deep operand ring), so that the epilogue of one tile -- cross-wave sum,
+// soft-max partials, stores: a fifth of a tile's time -- and the ramp-up of the next overlap the other workgroup's K
+// loop instead of leaving the matrix pipe idle.  The number of such tiles is rarely a multiple of the number of CUs,
+// and a last, mostly empty round costs as much as a full one.  So only as many
 // 64-row tiles as fill whole rounds are taken that way (workgroups [0, n_big)); the rows left over go to the
 // workgroups behind them as 32 x 32 tiles, which the hardware hands out as the CUs run dry, and whose round lasts an
 // eighth of a big one.  Workgroup ids congruent modulo 8 share an XCD: each XCD takes a contiguous range of big row
 // tiles and the column tiles of one row tile run side by side on it.
+// Big tile of gemm_tall_kernel: 32*kTallTM rows x 32*kTallTN columns, operand ring kTallPF deep, kTallOcc workgroups
+// per CU.  Measured on the 50000 x 128 x 1000 logits product (kernel time, us): one workgroup per CU with a six-deep
+// ring (all 512 registers) 134-136; two per CU with a ring of two 119, of three 122, of one 122; 32 x 128 tiles at two
+// per CU 123; 64 x 64 tiles at three per CU 123.
+constexpr int kTallTM = 2, kTallTN = 4, kTallPF = 2, kTallOcc = 2;
 template <int EPI>
-__global__ void __launch_bounds__(256) gemm_tall_kernel(GemmArgs a, int big_rows, int n_col_tiles, int n_big) {
-  __shared__ float red[4 * 4 * 16 * 64];
+__global__ void __launch_bounds__(256, kTallOcc) gemm_tall_kernel(GemmArgs a, int big_rows, int n_col_tiles, int n_big) {
+  constexpr int TM = kTallTM, TN = kTallTN;
+  __shared__ float red[4 * TN * 16 * 64];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int kslice = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -361,11 +369,11 @@ __global__ void __launch_bounds__(256) gemm_tall_kernel(GemmArgs a, int big_rows
     const int mpx = big_rows >> 3;  // big_rows is a multiple of 8
     const int nt = q % n_col_tiles;
     const int mt = r8 * mpx + q / n_col_tiles;
-    gemm_tile<2, 4, 4, ZR_A_PACK4, true, EPI, 6, true>(a, mt * 64, nt * 128, true, 0, red, kslice, lane);
+    gemm_tile<TM, TN, 4, ZR_A_PACK4, true, EPI, kTallPF, true>(a, mt * 32 * TM, nt * 32 * TN, true, 0, red, kslice, lane);
   } else {
     const int idx = bid - n_big;
     const int n32 = (a.N + 31) >> 5;
-    const int blk = big_rows * 2 + idx / n32;
+    const int blk = big_rows * TM + idx / n32;
     gemm_tile<1, 1, 4, ZR_A_PACK4, true, EPI, 8>(a, blk * 32, (idx % n32) * 32, true, 0, red, kslice, lane);
   }
 }
@@ -667,14 +675,15 @@ int launch_rows(zr_ctx* ctx, GemmArgs& ga, int epi, int n_tiles) {
 // gemm_tall_kernel: N a multiple of 128, fp32 k-interleaved A.  Returns false when the shape is better served by the
 // row-range kernel (too many rows would be left to the small tiles).
 bool launch_tall(zr_ctx* ctx, GemmArgs& ga, int epi, int* rc) {
+  constexpr int TM = kTallTM, TN = kTallTN;
   const int blocks = (ga.M + 31) / 32;
-  const int n_col_tiles = ga.N / 128;
+  const int n_col_tiles = ga.N / (32 * TN);
   const int n32 = ga.N / 32;
-  const long long row_tiles = blocks / 2;  // whole 64-row tiles
+  const long long row_tiles = blocks / TM;  // whole big row tiles
   // as many big row tiles as fill whole rounds of 256 workgroups, a multiple of 8 of them
   long long big_rows = (row_tiles * n_col_tiles / 256) * 256 / n_col_tiles;
   big_rows = big_rows / 8 * 8;
-  const long long small = (long long)(blocks - 2 * big_rows) * n32;
+  const long long small = (long long)(blocks - TM * big_rows) * n32;
   const bool offsets_fit = (long long)ga.K[0] * ga.lda[0] * 4 + 4096 < (1LL << 32) && (long long)ga.K[0] * ga.N * 4 < (1LL << 32);
   if (big_rows == 0 || small > 1024 || !offsets_fit) {
     // the left-over rows would be more than four rounds of small tiles: run whole big tiles to the end instead when

@@ -656,7 +656,8 @@ __global__ void __launch_bounds__(256) lstm_sweep_kernel(LstmSweep P) {
   constexpr int KS = 4;
   __shared__ __align__(16) float red[KS * 4 * TN * 16 * 64];  // all partial tiles of the workgroup at once
   __shared__ int s_go[2];
-  // same die-aware placement as lstm_fused_kernel, with one unit per layer
+  // same die-aware placement as lstm_fused_kernel, with one unit per layer.  (Two workgroups per CU on 32-column tiles
+  // -- 512 workgroups for four layers of H = 1000 at 128 columns -- measured 2 % slower than one on 64-column tiles.)
   const int id = blockIdx.x;
   const int r8 = id & 7;
   const int q = id >> 3;
