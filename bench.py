@@ -153,6 +153,8 @@ def bench_decoder_step(ctx, steps, warmup, H=1000, mb=128, S=50, V=50000, L=4, D
     res = {"ms_per_step": ev_ms / steps, "wall_ms_per_step": wall_ms / steps, "tokens_per_s": mb * steps / (ev_ms * 1e-3),
            "gflop_per_step": flops / 1e9, "tflops": flops * steps / (ev_ms * 1e-3) / 1e12, "attention_D": D}
     res.update(parts)
+    if not bf16:
+        res["frac_of_fp32_matrix_peak"] = round(res["tflops"] / PEAK_FP32_MFMA_TFLOPS, 4)
     res["softmax_gemm_plus_normalise_tflops"] = round(2.0 * V * H * mb / (parts["softmax_us"] * 1e-6) / 1e12, 2)
     ctx.attn_destroy(attn)
     ctx.softmax_release(dD)
