@@ -317,12 +317,12 @@ def test_config1_lm_forward_logprobs_and_loss(ctx):
 # ------------------------------------------------------------------------------------------------ A8/A9 softmax
 @pytest.mark.parametrize("prepared", [False, True])
 @pytest.mark.parametrize("V,H,mb", [(211, 16, 6), (10000, 100, 8), (4099, 64, 33), (1003, 27, 70), (8300, 40, 128),
-                                    (8400, 24, 100), (16500, 32, 192), (9000, 16, 40)])
+                                    (8400, 24, 100), (16500, 32, 192), (9000, 16, 40), (9100, 24, 64), (8250, 16, 320)])
 def test_softmax_prob_and_logprob(ctx, V, H, mb, prepared):
     """prepared: the output matrix registered with zr_softmax_prepare (k-interleaved copy); same results.  The shapes
-    with more than 8192 rows take the row-range kernel when prepared: 260-516 blocks of 32 rows over 128 or 256
-    workgroups, so a few blocks are left over and dealt out in 32-column pieces (column tiles of 128, 96 and 64, the
-    last column tile partly filled)."""
+    with more than 8192 rows take the tall-matrix kernels when prepared: 64-row tiles of 128, 96 or 64 columns where
+    the minibatch is a multiple of those (128; 192; 64 and 320), row ranges with 32-column pieces otherwise (100 and
+    40 columns, the last column tile partly filled); the rows beyond the last full tile go to the small tiles."""
     g = synth.rng(11, V)
     D, bd, h = U(g, (V, H), -1, 1), U(g, (V,), -1, 1), U(g, (H, mb), -1, 1)
     dD, dbd, dh = ctx.array(D), ctx.array(bd), ctx.array(h)
@@ -857,6 +857,42 @@ def test_decoder_step_as_one_call_matches_the_three_calls(ctx, H, mb, L, S, D, V
         if prepared:
             ctx.softmax_release(dD)
         ctx.attn_destroy(a)
+        for ly in lys:
+            ly.close()
+
+
+def test_decoder_step_as_one_call_without_attention(ctx):
+    """zr_decoder_step with no attention layer: the output distribution is taken from the top layer's h_t; log-probability
+    mode; against the separate calls bit for bit."""
+    g = synth.rng(36, 1)
+    H, mb, L, V = 128, 40, 2, 777
+    case = _decoder_step_case(g, H, mb, L, False, V=V)
+    layers, embed, ids, hp, cp, _, mask = case
+    Dm, bd = U(g, (V, H)), U(g, (V,))
+    lys = [Layer(ctx, ly) for ly in layers]
+    try:
+        d_embed, d_ids, d_mask = ctx.array(embed), ctx.array(ids), ctx.array(mask)
+        d_hp, d_cp = [ctx.array(x) for x in hp], [ctx.array(x) for x in cp]
+        dD, dbd = ctx.array(Dm), ctx.array(bd)
+        outs = []
+        for one_call in (False, True):
+            d_h = [ctx.zeros((H, mb)) for _ in range(L)]
+            d_c = [ctx.zeros((H, mb)) for _ in range(L)]
+            d_p = ctx.zeros((V, mb))
+            if one_call:
+                ctx.decoder_step([ly.w for ly in lys], d_embed, V, d_ids, d_hp, d_cp, d_mask, mb, d_h, d_c, None, None, None,
+                                 dD, dbd, V, capi.ZR_SOFTMAX_LOGPROB, d_p, clip=0.8)
+            else:
+                ctx.lstm_decoder_step([ly.w for ly in lys], d_embed, V, d_ids, d_hp, d_cp, d_mask, mb, d_h, d_c, clip=0.8)
+                ctx.softmax_forward(dD, dbd, V, H, d_h[L - 1], mb, capi.ZR_SOFTMAX_LOGPROB, d_p)
+            ctx.sync()
+            outs.append([x.get() for x in d_h + d_c + [d_p]])
+        for x, y in zip(*outs):
+            assert x.tobytes() == y.tobytes()
+        want_h, _ = _oracle_decoder_step(case)
+        want_lp = o.softmax_logprob_f64(o.softmax_logits(Dm, bd, want_h[L - 1]))
+        assert_close(outs[1][2 * L], want_lp, what="log-probabilities")
+    finally:
         for ly in lys:
             ly.close()
 

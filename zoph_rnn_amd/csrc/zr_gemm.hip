@@ -351,14 +351,13 @@ __global__ void __launch_bounds__(256) gemm_rows_kernel(GemmArgs a, int row_chun
 // workgroups behind them as 32 x 32 tiles, which the hardware hands out as the CUs run dry, and whose round lasts an
 // eighth of a big one.  Workgroup ids congruent modulo 8 share an XCD: each XCD takes a contiguous range of big row
 // tiles and the column tiles of one row tile run side by side on it.
-// Big tile of gemm_tall_kernel: 32*kTallTM rows x 32*kTallTN columns, operand ring kTallPF deep, kTallOcc workgroups
-// per CU.  Measured on the 50000 x 128 x 1000 logits product (kernel time, us): one workgroup per CU with a six-deep
+// Big tile of gemm_tall_kernel: 32*TM rows x 32*TN columns, operand ring PF deep, OCC workgroups per CU.  Measured on the 50000 x 128 x 1000 logits product (kernel time, us): one workgroup per CU with a six-deep
 // ring (all 512 registers) 134-136; two per CU with a ring of two 119, of three 122, of one 122; 32 x 128 tiles at two
 // per CU 123; 64 x 64 tiles at three per CU 123.
-constexpr int kTallTM = 2, kTallTN = 4, kTallPF = 2, kTallOcc = 2;
-template <int EPI>
-__global__ void __launch_bounds__(256, kTallOcc) gemm_tall_kernel(GemmArgs a, int big_rows, int n_col_tiles, int n_big) {
-  constexpr int TM = kTallTM, TN = kTallTN;
+// Minibatches that are a multiple of 64 but not of 128 columns wide (192 beam columns) take 64 x 64 tiles at three
+// workgroups per CU.
+template <int EPI, int TM, int TN, int PF, int OCC>
+__global__ void __launch_bounds__(256, OCC) gemm_tall_kernel(GemmArgs a, int big_rows, int n_col_tiles, int n_big) {
   __shared__ float red[4 * TN * 16 * 64];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -369,7 +368,7 @@ __global__ void __launch_bounds__(256, kTallOcc) gemm_tall_kernel(GemmArgs a, in
     const int mpx = big_rows >> 3;  // big_rows is a multiple of 8
     const int nt = q % n_col_tiles;
     const int mt = r8 * mpx + q / n_col_tiles;
-    gemm_tile<TM, TN, 4, ZR_A_PACK4, true, EPI, kTallPF, true>(a, mt * 32 * TM, nt * 32 * TN, true, 0, red, kslice, lane);
+    gemm_tile<TM, TN, 4, ZR_A_PACK4, true, EPI, PF, true>(a, mt * 32 * TM, nt * 32 * TN, true, 0, red, kslice, lane);
   } else {
     const int idx = bid - n_big;
     const int n32 = (a.N + 31) >> 5;
@@ -674,8 +673,8 @@ int launch_rows(zr_ctx* ctx, GemmArgs& ga, int epi, int n_tiles) {
 
 // gemm_tall_kernel: N a multiple of 128, fp32 k-interleaved A.  Returns false when the shape is better served by the
 // row-range kernel (too many rows would be left to the small tiles).
-bool launch_tall(zr_ctx* ctx, GemmArgs& ga, int epi, int* rc) {
-  constexpr int TM = kTallTM, TN = kTallTN;
+template <int TM, int TN, int PF, int OCC>
+bool launch_tall_v(zr_ctx* ctx, GemmArgs& ga, int epi, int* rc) {
   const int blocks = (ga.M + 31) / 32;
   const int n_col_tiles = ga.N / (32 * TN);
   const int n32 = ga.N / 32;
@@ -686,20 +685,29 @@ bool launch_tall(zr_ctx* ctx, GemmArgs& ga, int epi, int* rc) {
   const long long small = (long long)(blocks - TM * big_rows) * n32;
   const bool offsets_fit = (long long)ga.K[0] * ga.lda[0] * 4 + 4096 < (1LL << 32) && (long long)ga.K[0] * ga.N * 4 < (1LL << 32);
   if (big_rows == 0 || small > 1024 || !offsets_fit) {
-    // the left-over rows would be more than four rounds of small tiles: run whole big tiles to the end instead when
-    // that wastes less than a third of a round, else leave the shape to the row-range kernel
+    // the left-over rows would be more than four rounds of small tiles: leave the shape to the row-range kernel
     return false;
   }
   ga.m_tiles = ga.n_tiles = 0;
   const int n_big = (int)(big_rows * n_col_tiles);
   const unsigned grid = (unsigned)(n_big + small);
   if (epi == ZR_EPI_STORE)
-    gemm_tall_kernel<ZR_EPI_STORE><<<grid, 256, 0, ctx->stream>>>(ga, (int)big_rows, n_col_tiles, n_big);
+    gemm_tall_kernel<ZR_EPI_STORE, TM, TN, PF, OCC><<<grid, 256, 0, ctx->stream>>>(ga, (int)big_rows, n_col_tiles, n_big);
   else
-    gemm_tall_kernel<ZR_EPI_SOFTMAX_PARTIAL><<<grid, 256, 0, ctx->stream>>>(ga, (int)big_rows, n_col_tiles, n_big);
+    gemm_tall_kernel<ZR_EPI_SOFTMAX_PARTIAL, TM, TN, PF, OCC><<<grid, 256, 0, ctx->stream>>>(ga, (int)big_rows, n_col_tiles,
+                                                                                            n_big);
   hipError_t e = hipGetLastError();
   *rc = e == hipSuccess ? ZR_OK : zr_set_error(ZR_EHIP, "launch of gemm_tall_kernel failed: %s", hipGetErrorString(e));
   return true;
+}
+
+// gemm_tall_kernel: N a multiple of 128, 96 or 64 (column tiles of that width: two workgroups per CU at 128, three
+// below), fp32 k-interleaved A.  Returns false when the shape is better served by the row-range kernel (too many rows
+// would be left to the small tiles).  Measured at 50000 x 192 x 1000: row ranges 201 us, 64 x 64 tiles 190, 64 x 96 182.
+bool launch_tall(zr_ctx* ctx, GemmArgs& ga, int epi, int* rc) {
+  if (ga.N % 128 == 0) return launch_tall_v<2, 4, 2, 2>(ctx, ga, epi, rc);
+  if (ga.N % 96 == 0) return launch_tall_v<2, 3, 2, 3>(ctx, ga, epi, rc);
+  return launch_tall_v<2, 2, 2, 3>(ctx, ga, epi, rc);
 }
 
 // Activations X (K x N fp32, column n at src + n*ld, K % 8 == 0) -> two bf16 arrays hi and lo with x = hi + lo up
@@ -956,7 +964,7 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
     if (vec && d.nseg == 1 && zcount == 1 && d.M >= 8192 && d.N <= 1024 && ctx->gemm_cfg != 11 &&
         (d.epilogue == ZR_EPI_STORE || d.epilogue == ZR_EPI_SOFTMAX_PARTIAL)) {
       const int n32 = (d.N + 31) / 32;
-      if (d.N % 128 == 0 && ga.b_pack4 && ctx->gemm_cfg == 0) {
+      if ((d.N % 64 == 0 || d.N % 96 == 0) && ga.b_pack4 && ctx->gemm_cfg == 0) {
         int rc = ZR_OK;
         if (launch_tall(ctx, ga, d.epilogue, &rc)) return rc;
       }
