@@ -99,6 +99,10 @@ const char* zr_version(void);
                                         bf16 terms (hi + lo: fp32-level accuracy, two matrix instructions per 16 k);
                                         1 = activations rounded to bf16 once (relative error 2^-9 per activation, half
                                         the matrix instructions and half the activation operand traffic) */
+#define ZR_OPT_LSTM_STEP_WAIT_EXTRA 10 /* for tests of the give-up path of zr_lstm_decoder_step's single launch: the
+                                        waits of a layer for the layer below expect this many arrivals more than there
+                                        will be, so each of them runs to ZR_OPT_LSTM_SWEEP_SPIN polls and gives up
+                                        whatever the timing (0 = off, the default) */
 
 /* full_matrix_setup / cudaMalloc / cudaMemcpy / cudaMemset call sites (src/BZ_CUDA_UTIL.h:358-399 and the
  * layer constructors, e.g. src/LSTM.hpp:23-42). */
@@ -231,10 +235,17 @@ int zr_softmax_release(zr_ctx* ctx, const float* d_D);
 
 #define ZR_SOFTMAX_PROB 0    /* probabilities: softmax_layer::get_distribution_GPU (src/softmax.hpp:514-632) */
 #define ZR_SOFTMAX_LOGPROB 1 /* natural-log probabilities, fp32 */
+/* The logits D h + b_d and, behind them, the column statistics of the reference's overflow-safe soft-max
+ * (src/custom_kernels.h:503-577): d_out holds V*mb + 2*mb floats, the V x mb logits followed by (max, sum of
+ * exp(x - max)) per column.  No normalised matrix is written: zr_beam_expand_logits / zr_beam_finish_logits form
+ * exp(x - max) / sum for the few entries a decode step needs, so the V x mb matrix is written once and read once per
+ * step instead of written twice and read twice.  d_logits_scratch must be NULL in this mode. */
+#define ZR_SOFTMAX_LOGITS 2
 
 /* D h + b_d on MFMA (cublasSgemm + matrix_bias_kernel, src/softmax.hpp:539-547) followed by the per-column
  * max / exp / sum / normalise of outputdist_overflow_prevention_kernel (src/custom_kernels.h:503-577).
- * d_out: V x mb.  d_logits_scratch: V x mb scratch for the logits, or NULL to use d_out in place. */
+ * d_out: V x mb (V*mb + 2*mb floats in mode ZR_SOFTMAX_LOGITS).  d_logits_scratch: V x mb scratch for the logits, or
+ * NULL to use d_out in place. */
 int zr_softmax_forward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int mb,
                        int mode, float* d_out, float* d_logits_scratch);
 /* zr_softmax_forward for callers that cannot allocate device memory (code under HIP graph capture, serving loops,
@@ -327,6 +338,15 @@ int zr_beam_init(zr_ctx* ctx, zr_beam* b);
 int zr_beam_expand(zr_ctx* ctx, zr_beam* b, const float* d_prob, int index, int* d_words, int* d_backptr);
 /* finish_current_hypotheses (src/decoder.h:672-688). */
 int zr_beam_finish(zr_ctx* ctx, zr_beam* b, const float* d_prob);
+/* zr_beam_expand / zr_beam_finish on the output of ZR_SOFTMAX_LOGITS: d_logits V x (n_sent*beam), d_colstats 2 floats
+ * per column (max, sum of exp(x - max)) -- d_out and d_out + V*cols of that call.  The per-column selection runs on the
+ * logits (the soft-max is monotonic within a column) and only the beam+1 selected entries of a column are normalised,
+ * with the same expression as the full matrix, so candidates, scores, words and back-pointers are those of
+ * zr_beam_expand on the probabilities; the one difference: two words whose logits differ but whose probabilities
+ * round to the same float rank by logit here and by word id there. */
+int zr_beam_expand_logits(zr_ctx* ctx, zr_beam* b, const float* d_logits, const float* d_colstats, int index,
+                          int* d_words, int* d_backptr);
+int zr_beam_finish_logits(zr_ctx* ctx, zr_beam* b, const float* d_logits, const float* d_colstats);
 /* Copies the finished hypotheses of sentence s to the host: returns their number (or a negative error);
  * h_words is n x max_len (row-major, -1 padded), h_len and h_score have n entries; at most cap are copied. */
 int zr_beam_hypotheses(zr_ctx* ctx, zr_beam* b, int sentence, int cap, int* h_words, int* h_len, float* h_score);

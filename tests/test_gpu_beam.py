@@ -204,3 +204,68 @@ def test_beam_selection_on_adversarial_layouts(ctx, V, beam):
         top = np.sort(p, axis=0)[-(beam + 2):]
         assert np.all(np.diff(top, axis=0) > 0)
     _expand_given(ctx, Ps, beam, n_sent, max_len=8)
+
+
+@pytest.mark.parametrize("V,H,beam,n_sent,prepared", [(5000, 32, 5, 3, False), (50000, 64, 12, 16, True),
+                                                      (8193, 16, 31, 2, False), (70001, 24, 7, 4, True)])
+def test_beam_on_logits_equals_beam_on_probabilities(ctx, V, H, beam, n_sent, prepared):
+    """ZR_SOFTMAX_LOGITS + zr_beam_expand_logits / zr_beam_finish_logits against ZR_SOFTMAX_PROB + zr_beam_expand /
+    zr_beam_finish on the same activations: the logits are the same bits, the column statistics are the column's maximum
+    and its sum of exp(x - max), and every word, back-pointer, beam score and finished hypothesis is identical, scores
+    to the bit (the selected entries are normalised with the expression the full matrix is normalised with).  <EOF> is
+    made likely so that hypotheses finish inside the steps."""
+    g = synth.rng(47, V + beam)
+    cols, steps, max_len = n_sent * beam, 5, 10
+    D = np.asfortranarray(g.uniform(-1, 1, size=(V, H)).astype(np.float32))
+    bd = g.uniform(-1, 1, size=V).astype(np.float32)
+    bd[1] += 3.0
+    dD, dbd = ctx.array(D), ctx.array(bd)
+    if prepared:
+        ctx.softmax_prepare(dD, V, H)
+    d_prob, d_scr = ctx.empty((V, cols)), ctx.empty((V, cols))
+    d_lg = ctx.empty((V * cols + 2 * cols,))
+    d_stats = d_lg.at(V * cols)
+    ba, bb = ctx.beam_create(beam, V, n_sent, max_len, 0.1), ctx.beam_create(beam, V, n_sent, max_len, 0.1)
+    wa, ka = ctx.empty(cols, np.int32), ctx.empty(cols, np.int32)
+    wb, kb = ctx.empty(cols, np.int32), ctx.empty(cols, np.int32)
+    for index in range(steps + 1):
+        h = np.asfortranarray(g.uniform(-1, 1, size=(H, cols)).astype(np.float32))
+        dh = ctx.array(h)
+        ctx.softmax_forward(dD, dbd, V, H, dh, cols, capi.ZR_SOFTMAX_PROB, d_prob, d_scr)
+        ctx.softmax_forward(dD, dbd, V, H, dh, cols, capi.ZR_SOFTMAX_LOGITS, d_lg)
+        ctx.sync()
+        out = d_lg.get()
+        lg, stats = out[:V * cols].reshape((V, cols), order="F"), out[V * cols:].reshape(cols, 2)
+        assert np.array_equal(lg, d_scr.get())
+        assert np.array_equal(stats[:, 0], lg.max(axis=0))
+        want_sum = np.exp(lg.astype(np.float64) - lg.max(axis=0).astype(np.float64)).sum(axis=0)
+        assert np.allclose(stats[:, 1], want_sum, rtol=2e-6, atol=0)
+        if index == steps:
+            ctx.beam_finish(ba, d_prob)
+            ctx.beam_finish_logits(bb, d_lg, d_stats)
+            break
+        ctx.beam_expand(ba, d_prob, index, wa, ka)
+        ctx.beam_expand_logits(bb, d_lg, d_stats, index, wb, kb)
+        ctx.sync()
+        assert np.array_equal(wa.get(), wb.get()), index
+        assert np.array_equal(ka.get(), kb.get()), index
+        for s in range(n_sent):
+            sa, xa = ctx.beam_state(ba, s, beam)
+            sb, xb = ctx.beam_state(bb, s, beam)
+            assert np.array_equal(xa, xb) and np.array_equal(sa[xa != -1], sb[xb != -1]), (index, s)
+    ctx.sync()
+    finished = 0
+    for s in range(n_sent):
+        ga, na = ctx.beam_hypotheses(ba, s, cap=256, max_len=max_len)
+        gb, nb = ctx.beam_hypotheses(bb, s, cap=256, max_len=max_len)
+        assert na == nb and na >= 1
+        for (w1, s1), (w2, s2) in zip(ga, gb):
+            assert np.array_equal(w1, w2) and s1 == s2
+        finished += na
+    assert finished > n_sent * beam  # some hypotheses finished inside the steps, not only at the forced end
+    with pytest.raises(capi.ZrError):
+        ctx.softmax_forward(dD, dbd, V, H, dh, cols, capi.ZR_SOFTMAX_LOGITS, d_lg, d_scr)
+    if prepared:
+        ctx.softmax_release(dD)
+    ctx.beam_destroy(ba)
+    ctx.beam_destroy(bb)

@@ -736,12 +736,15 @@ def _oracle_decoder_step(case, clip=0.8):
 
 @pytest.mark.parametrize("H,mb,L,feed", [(64, 5, 3, True), (1000, 128, 4, True), (200, 70, 2, True), (72, 33, 1, False),
                                          (128, 128, 4, False), (256, 192, 4, True), (1000, 12, 4, True),
-                                         (104, 40, 8, False)])
+                                         (104, 40, 8, False), (1000, 192, 4, True), (520, 200, 3, True),
+                                         (776, 250, 2, False)])
 def test_decoder_step_all_layers_in_one_launch(ctx, H, mb, L, feed):
     """zr_lstm_decoder_step as ONE launch (two resident workgroups per state tile: one streams the W_h / Q products of
     every layer, the other walks up the chain of layers) against the oracle's node-by-node step and against one launch
     per layer: feed-input on layer 0, duplicate and extreme ids, a masked column, cell clipping, row and column tails,
-    a batch width that is not a multiple of 8 (consumers then invalidate their caches), one to eight layers."""
+    a batch width that is not a multiple of 8 (consumers then invalidate their caches), one to eight layers.  The last
+    three shapes have more 32-column tiles than the device holds workgroup pairs for and take 64-column tiles (192
+    columns of H = 1000: the batched beam decode; a last column tile of 8 columns; exactly 256 workgroups)."""
     g = synth.rng(31, H + mb + L)
     case = _decoder_step_case(g, H, mb, L, feed)
     ctx.set_option(capi.ZR_OPT_LSTM_SWEEP, 2)
@@ -773,14 +776,17 @@ def test_decoder_step_picks_the_single_launch_at_benchmark_size_and_repeats_bit_
         assert h1[l].tobytes() == h2[l].tobytes() and c1[l].tobytes() == c2[l].tobytes()
 
 
-def test_decoder_step_single_launch_abandoned_wait_is_reported(ctx):
-    """With a single poll per wait the layers above the first give up at once: every workgroup still leaves the kernel,
-    the query reports it, the unfinished outputs hold NaN, and the next step with the default limit is complete again
-    (the last workgroup out of the abandoned launch returned the counters to zero)."""
+@pytest.mark.parametrize("H,mb,L", [(128, 40, 3), (128, 520, 3)])
+def test_decoder_step_single_launch_abandoned_wait_is_reported(ctx, H, mb, L):
+    """The waits for the layer below are told to expect one arrival more than will come and given 64 polls: the layers
+    above the first give up whatever the timing, every workgroup still leaves the kernel, the query reports it, the
+    unfinished outputs hold NaN, and the next step with the default settings is complete again (the last workgroup out
+    of the abandoned launch returned the counters to zero).  Both tile widths."""
     g = synth.rng(33, 1)
-    case = _decoder_step_case(g, 128, 40, 3, True)
+    case = _decoder_step_case(g, H, mb, L, True)
     ctx.set_option(capi.ZR_OPT_LSTM_SWEEP, 2)
-    ctx.set_option(capi.ZR_OPT_LSTM_SWEEP_SPIN, 1)
+    ctx.set_option(capi.ZR_OPT_LSTM_SWEEP_SPIN, 64)
+    ctx.set_option(capi.ZR_OPT_LSTM_STEP_WAIT_EXTRA, 1)
     try:
         h1, c1, gave_up = _run_decoder_step(ctx, case, expect_path=capi.ZR_LSTM_STACK_PATH_STEP_SINGLE_LAUNCH)
         assert gave_up == 1
@@ -791,13 +797,15 @@ def test_decoder_step_single_launch_abandoned_wait_is_reported(ctx):
             done = ~np.isnan(got)
             assert_close(np.where(done, got, 0.0), np.where(done, want, 0.0), what="finished part of an abandoned step")
         ctx.set_option(capi.ZR_OPT_LSTM_SWEEP_SPIN, 0)
+        ctx.set_option(capi.ZR_OPT_LSTM_STEP_WAIT_EXTRA, 0)
         h2, c2, gave_up = _run_decoder_step(ctx, case, expect_path=capi.ZR_LSTM_STACK_PATH_STEP_SINGLE_LAUNCH)
         assert gave_up == 0
     finally:
         ctx.set_option(capi.ZR_OPT_LSTM_SWEEP, 0)
         ctx.set_option(capi.ZR_OPT_LSTM_SWEEP_SPIN, 0)
+        ctx.set_option(capi.ZR_OPT_LSTM_STEP_WAIT_EXTRA, 0)
     want_h, want_c = _oracle_decoder_step(case)
-    for l in range(3):
+    for l in range(L):
         assert_close(h2[l], want_h[l], what="h of layer %d" % l)
         assert_close(c2[l], want_c[l], what="c of layer %d" % l)
 

@@ -21,6 +21,7 @@ ZR_OPT_LSTM_KPARTS = 6
 ZR_OPT_LSTM_SWEEP = 7
 ZR_OPT_LSTM_SWEEP_SPIN = 8
 ZR_OPT_BF16_ACTIVATION_TERMS = 9
+ZR_OPT_LSTM_STEP_WAIT_EXTRA = 10
 ZR_QUERY_LSTM_STACK_PATH = 1
 ZR_QUERY_LSTM_SWEEP_ABANDONED = 2
 ZR_LSTM_STACK_PATH_SWEEP = 1
@@ -29,6 +30,7 @@ ZR_LSTM_STACK_PATH_STEP_SINGLE_LAUNCH = 3
 ZR_LSTM_STACK_PATH_STEP_PER_LAYER = 4
 ZR_SOFTMAX_PROB = 0
 ZR_SOFTMAX_LOGPROB = 1
+ZR_SOFTMAX_LOGITS = 2  # d_out: V*mb logits followed by 2*mb column statistics (max, sum of exp(x - max))
 
 # every symbol include/zoph_rnn.h declares
 SYMBOLS = [
@@ -37,7 +39,7 @@ SYMBOLS = [
     "zr_vocab_prep_softmax", "zr_embed_gather", "zr_lstm_pack_weights", "zr_lstm_pack_weights_bf16", "zr_lstm_weights_destroy", "zr_lstm_step",
     "zr_lstm_gates", "zr_lstm_stack_forward", "zr_gemm", "zr_softmax_prepare", "zr_softmax_prepare_bf16", "zr_softmax_release", "zr_softmax_forward", "zr_softmax_logprob_f64",
     "zr_softmax_loss", "zr_attn_create", "zr_attn_use_bf16_weights", "zr_attn_destroy", "zr_attn_step", "zr_gather_columns",
-    "zr_broadcast_column", "zr_beam_create", "zr_beam_destroy", "zr_beam_init", "zr_beam_expand", "zr_beam_finish",
+    "zr_broadcast_column", "zr_beam_create", "zr_beam_destroy", "zr_beam_init", "zr_beam_expand", "zr_beam_finish", "zr_beam_expand_logits", "zr_beam_finish_logits",
     "zr_beam_hypotheses", "zr_beam_state",
     "zr_lstm_stack_forward_train", "zr_lstm_train_create", "zr_lstm_train_refresh", "zr_lstm_train_destroy",
     "zr_unstack_gates", "zr_lstm_stack_backward", "zr_lstm_weight_gradients", "zr_embed_gradient",
@@ -417,6 +419,13 @@ class Context:
 
     def beam_finish(self, b, d_prob):
         _chk(load().zr_beam_finish(self.h, b, _vp(d_prob)))
+
+    def beam_expand_logits(self, b, d_logits, d_colstats, index, d_words, d_backptr):
+        _chk(load().zr_beam_expand_logits(self.h, b, _vp(d_logits), _vp(d_colstats), C.c_int(index), _vp(d_words),
+                                          _vp(d_backptr)))
+
+    def beam_finish_logits(self, b, d_logits, d_colstats):
+        _chk(load().zr_beam_finish_logits(self.h, b, _vp(d_logits), _vp(d_colstats)))
 
     def beam_hypotheses(self, b, sentence, cap, max_len):
         words = np.full((cap, max_len), -1, dtype=np.int32)

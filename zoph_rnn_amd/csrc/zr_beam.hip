@@ -216,9 +216,11 @@ beam_topk_kernel(const float* __restrict__ prob, int V, int K, int n_chunks, flo
   }
 }
 
+// colstats (or null): the values are logits and (max, sum of exp(x - max)) per column turns the K selected ones into
+// probabilities, exp(x - max) / sum as the full normalisation forms them (src/custom_kernels.h:574-576).
 __global__ void __launch_bounds__(256)
 beam_topk_merge_kernel(const float* __restrict__ part_p, const int* __restrict__ part_w, int K, int n_chunks,
-                       float* __restrict__ cand_p, int* __restrict__ cand_w) {
+                       float* __restrict__ cand_p, int* __restrict__ cand_w, const float* __restrict__ colstats) {
   __shared__ unsigned long long s_key[kMaxChunks * KMAX];
   const int col = blockIdx.x;
   const int tid = threadIdx.x;
@@ -235,7 +237,9 @@ beam_topk_merge_kernel(const float* __restrict__ part_p, const int* __restrict__
       rank += (kb > ka || (kb == ka && b < a)) ? 1 : 0;  // fillers share one key: order them by position
     }
     if (rank < K) {
-      cand_p[(size_t)col * K + rank] = part_p[(size_t)col * n + a];
+      float v = part_p[(size_t)col * n + a];
+      if (colstats && v > -INFINITY) v = expf(v - colstats[2 * col]) / colstats[2 * col + 1];
+      cand_p[(size_t)col * K + rank] = v;
       cand_w[(size_t)col * K + rank] = part_w[(size_t)col * n + a];
     }
   }
@@ -370,8 +374,8 @@ beam_merge_kernel(int beam, int K, int max_len, int hyp_cap, float penalty, int 
 // finish_current_hypotheses, non-FSA branch (src/decoder.h:672-688)
 __global__ void __launch_bounds__(256)
 beam_finish_kernel(int beam, int V, int max_len, int hyp_cap, float penalty, int current_index,
-                   const float* __restrict__ prob, float* scores, const int* words, int* sent, int* hyp_words,
-                   int* hyp_len, float* hyp_score, int* hyp_count) {
+                   const float* __restrict__ prob, const float* __restrict__ colstats, float* scores, const int* words,
+                   int* sent, int* hyp_words, int* hyp_len, float* hyp_score, int* hyp_count) {
   const int s = blockIdx.x;
   const int tid = threadIdx.x;
   int base = hyp_count[s];
@@ -380,7 +384,9 @@ beam_finish_kernel(int beam, int V, int max_len, int hyp_cap, float penalty, int
   for (int i = 0; i < beam; ++i) {
     if (words[(size_t)s * beam + i] == -1) continue;
     int* row = sent + ((size_t)s * beam + i) * max_len;
-    const float sc = scores[(size_t)s * beam + i] + logf(prob[((size_t)s * beam + i) * V + 1]) + penalty;
+    float p_eof = prob[((size_t)s * beam + i) * V + 1];
+    if (colstats) p_eof = expf(p_eof - colstats[2 * (s * beam + i)]) / colstats[2 * (s * beam + i) + 1];  // logits
+    const float sc = scores[(size_t)s * beam + i] + logf(p_eof) + penalty;
     const int h = base + added;
     if (h < hyp_cap) {
       int* hw = hyp_words + ((size_t)s * hyp_cap + h) * max_len;
@@ -495,23 +501,25 @@ int zr_beam_init(zr_ctx* ctx, zr_beam* b) {
   return ZR_OK;
 }
 
-int zr_beam_expand(zr_ctx* ctx, zr_beam* b, const float* d_prob, int index, int* d_words, int* d_backptr) {
+// d_colstats null: d_values are probabilities; otherwise logits with their column statistics
+static int beam_expand_impl(zr_ctx* ctx, const char* who, zr_beam* b, const float* d_values, const float* d_colstats,
+                            int index, int* d_words, int* d_backptr) {
   int rc = zr_bind_device(ctx);
   if (rc) return rc;
-  ZR_CHECK_ARG(b && d_prob && d_words && d_backptr, "zr_beam_expand: null pointer");
-  ZR_CHECK_ARG(index >= 0, "zr_beam_expand: index = %d", index);
-  ZR_CHECK_ARG(b->current_index + 2 < b->max_len, "zr_beam_expand: hypotheses reached max_len = %d", b->max_len);
+  ZR_CHECK_ARG(b && d_values && d_words && d_backptr, "%s: null pointer", who);
+  ZR_CHECK_ARG(index >= 0, "%s: index = %d", who, index);
+  ZR_CHECK_ARG(b->current_index + 2 < b->max_len, "%s: hypotheses reached max_len = %d", who, b->max_len);
   const int K = b->beam + 1;
   const int e4 = topk_e4_for(b->vocab);
   const int n_chunks = (b->vocab + topk_chunk(e4) - 1) / topk_chunk(e4);
   dim3 tgrid(n_chunks, b->n_sent * b->beam);
   if (e4 == kTopkE4Small)
-    beam_topk_kernel<kTopkE4Small><<<tgrid, 256, 0, ctx->stream>>>(d_prob, b->vocab, K, n_chunks, b->d_part_p, b->d_part_w);
+    beam_topk_kernel<kTopkE4Small><<<tgrid, 256, 0, ctx->stream>>>(d_values, b->vocab, K, n_chunks, b->d_part_p, b->d_part_w);
   else
-    beam_topk_kernel<kTopkE4Large><<<tgrid, 256, 0, ctx->stream>>>(d_prob, b->vocab, K, n_chunks, b->d_part_p, b->d_part_w);
+    beam_topk_kernel<kTopkE4Large><<<tgrid, 256, 0, ctx->stream>>>(d_values, b->vocab, K, n_chunks, b->d_part_p, b->d_part_w);
   ZR_LAUNCH_CHECK("beam_topk_kernel");
   beam_topk_merge_kernel<<<b->n_sent * b->beam, 256, 0, ctx->stream>>>(b->d_part_p, b->d_part_w, K, n_chunks,
-                                                                       b->d_cand_p, b->d_cand_w);
+                                                                       b->d_cand_p, b->d_cand_w, d_colstats);
   ZR_LAUNCH_CHECK("beam_topk_merge_kernel");
   beam_merge_kernel<<<b->n_sent, 256, 0, ctx->stream>>>(b->beam, K, b->max_len, b->hyp_cap, b->penalty, index,
                                                         b->current_index, b->d_cand_p, b->d_cand_w, b->d_scores,
@@ -526,16 +534,36 @@ int zr_beam_expand(zr_ctx* ctx, zr_beam* b, const float* d_prob, int index, int*
   return ZR_OK;
 }
 
-int zr_beam_finish(zr_ctx* ctx, zr_beam* b, const float* d_prob) {
+static int beam_finish_impl(zr_ctx* ctx, const char* who, zr_beam* b, const float* d_values, const float* d_colstats) {
   int rc = zr_bind_device(ctx);
   if (rc) return rc;
-  ZR_CHECK_ARG(b && d_prob, "zr_beam_finish: null pointer");
+  ZR_CHECK_ARG(b && d_values, "%s: null pointer", who);
   beam_finish_kernel<<<b->n_sent, 256, 0, ctx->stream>>>(b->beam, b->vocab, b->max_len, b->hyp_cap, b->penalty,
-                                                         b->current_index, d_prob, b->d_scores, b->d_words, b->d_sent,
-                                                         b->d_hyp_words, b->d_hyp_len, b->d_hyp_score, b->d_hyp_count);
+                                                         b->current_index, d_values, d_colstats, b->d_scores, b->d_words,
+                                                         b->d_sent, b->d_hyp_words, b->d_hyp_len, b->d_hyp_score,
+                                                         b->d_hyp_count);
   ZR_LAUNCH_CHECK("beam_finish_kernel");
   b->current_index += 1;
   return ZR_OK;
+}
+
+int zr_beam_expand(zr_ctx* ctx, zr_beam* b, const float* d_prob, int index, int* d_words, int* d_backptr) {
+  return beam_expand_impl(ctx, "zr_beam_expand", b, d_prob, nullptr, index, d_words, d_backptr);
+}
+
+int zr_beam_expand_logits(zr_ctx* ctx, zr_beam* b, const float* d_logits, const float* d_colstats, int index,
+                          int* d_words, int* d_backptr) {
+  ZR_CHECK_ARG(d_colstats != nullptr, "zr_beam_expand_logits: d_colstats is null");
+  return beam_expand_impl(ctx, "zr_beam_expand_logits", b, d_logits, d_colstats, index, d_words, d_backptr);
+}
+
+int zr_beam_finish(zr_ctx* ctx, zr_beam* b, const float* d_prob) {
+  return beam_finish_impl(ctx, "zr_beam_finish", b, d_prob, nullptr);
+}
+
+int zr_beam_finish_logits(zr_ctx* ctx, zr_beam* b, const float* d_logits, const float* d_colstats) {
+  ZR_CHECK_ARG(d_colstats != nullptr, "zr_beam_finish_logits: d_colstats is null");
+  return beam_finish_impl(ctx, "zr_beam_finish_logits", b, d_logits, d_colstats);
 }
 
 int zr_beam_hypotheses(zr_ctx* ctx, zr_beam* b, int sentence, int cap, int* h_words, int* h_len, float* h_score) {

@@ -26,9 +26,10 @@ struct zr_ctx {
   int* d_counters;   // ZR_MAX_COUNTERS arrival counters, zero between launches
   int lstm_sweep;    // whole-sweep LSTM kernel: 0 auto, 1 never, 2 whenever the launch fits on the device
   int sweep_spin;    // polls before a waiting workgroup of that kernel gives up (0: default)
+  int step_wait_extra;  // arrivals the decoder step's layer waits expect beyond the real ones (tests of giving up)
   int cu_count;      // compute units of the device (filled with sweep_capacity)
   int sweep_capacity[3];  // resident workgroups of lstm_sweep_kernel<TN> (0: not asked yet, -1: unknown)
-  int stack_step_capacity;  // the same for lstm_decoder_stack_kernel<1>
+  int stack_step_capacity;  // the same for lstm_decoder_stack_kernel (the lesser of its two tile widths)
   int gemm_cfg;
   int bf16_terms;       // bf16-weight products: 2 (default, 0 = 2) = activations as two bf16 terms, 1 = rounded to bf16 once
   int last_stack_path;  // ZR_LSTM_STACK_PATH_* of the last zr_lstm_stack_forward(_train) call (0: none yet)

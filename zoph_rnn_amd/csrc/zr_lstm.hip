@@ -864,6 +864,7 @@ struct LstmDecStack {
   float clip;
   int spin_limit;
   int fence;                      // as in LstmSweep
+  int wait_extra;                 // arrivals a layer's wait for the layer below expects beyond the real ones (tests)
 };
 
 // All threads of the workgroup call this.  False: leave the kernel.
@@ -996,7 +997,8 @@ __global__ void __launch_bounds__(256) lstm_decoder_stack_kernel(LstmDecStack P)
         const __amdgpu_buffer_rsrc_t wrsrc = zr_make_rsrc(P.W[l]);
         zr_preload_w<4, TN, KS, PF>(ring, wrsrc, wsoff, woffb, 32u * (unsigned)P.ldw, K, kslice);
         if (packed) {
-          if (!stack_wait(P, layer_ctr + ((l - 1) * P.n_tiles + nt) * kSweepCtrStride, P.j_tiles, &s_go[0])) {
+          if (!stack_wait(P, layer_ctr + ((l - 1) * P.n_tiles + nt) * kSweepCtrStride, P.j_tiles + P.wait_extra,
+                          &s_go[0])) {
             abandon(l);
             return;
           }
@@ -1314,16 +1316,19 @@ int launch_sweep_v(zr_ctx* ctx, LstmSweep& P, int grid) {
   return ZR_OK;
 }
 
-// Resident workgroups of lstm_decoder_stack_kernel<1> the device can hold at once (0: unknown / query failed).
+// Resident workgroups of lstm_decoder_stack_kernel (either tile width) the device can hold at once (0: unknown /
+// query failed).
 int stack_step_capacity(zr_ctx* ctx) {
   int& cached = ctx->stack_step_capacity;
   if (cached == 0) {
-    int cus = 0, per_cu = 0;
+    int cus = 0, per_cu = 0, per_cu2 = 0;
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, ctx->device) != hipSuccess ||
-        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lstm_decoder_stack_kernel<1>, 256, 0) != hipSuccess) {
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lstm_decoder_stack_kernel<1>, 256, 0) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu2, lstm_decoder_stack_kernel<2>, 256, 0) != hipSuccess) {
       (void)hipGetLastError();
       cached = -1;
     } else {
+      per_cu = per_cu2 < per_cu ? per_cu2 : per_cu;
       ctx->cu_count = cus;
       cached = cus * per_cu > 0 ? cus * per_cu : -1;
     }
@@ -1557,11 +1562,15 @@ int zr_lstm_decoder_step_packed(zr_ctx* ctx, int nl, const zr_lstm_weights* cons
   // One launch for the whole step when two workgroups per tile fit on the device together (the same conditions as the
   // single-launch sweep of zr_lstm_stack_forward); otherwise one node after the other.
   if (vec && H % 8 == 0 && H >= 64 && !layers[0]->bf16 && ctx->lstm_fused && ctx->lstm_sweep != 1) {
-    const int j_tiles = (H + 31) / 32, n_tiles = (mb + 31) / 32;
+    const int j_tiles = (H + 31) / 32;
     const int padded = (j_tiles + 7) / 8 * 8;
+    const int cap = stack_step_capacity(ctx);
+    // 32-column tiles while two workgroups per tile fit on the device together, 64-column tiles beyond that (192 columns
+    // of H = 1000: 384 workgroups against 192)
+    const int tn = (2LL * padded * ((mb + 31) / 32) <= cap) ? 1 : 2;
+    const int n_tiles = (mb + 32 * tn - 1) / (32 * tn);
     const long long tiles = (long long)j_tiles * n_tiles;
     const long long wgs = 2LL * padded * n_tiles;
-    const int cap = stack_step_capacity(ctx);
     const bool fills = wgs * 10 >= 6LL * ctx->cu_count && zr_live_contexts(ctx->device) == 1 &&
                        ctx->stream == ctx->own_stream;
     const long long lim = 1LL << 32;
@@ -1569,7 +1578,7 @@ int zr_lstm_decoder_step_packed(zr_ctx* ctx, int nl, const zr_lstm_weights* cons
                              12LL * layers[0]->kp * layers[0]->ldw * 4 < lim;
     const long long n_counters = nl * tiles + (long long)nl * n_tiles * kSweepCtrStride;
     if (cap > 0 && wgs <= cap && offsets_fit && n_counters < ZR_MAX_COUNTERS && (fills || ctx->lstm_sweep == 2)) {
-      constexpr int NV = zr_visit_count<1, 4>();
+      const int NV = tn == 1 ? zr_visit_count<1, 4>() : zr_visit_count<2, 4>();
       LstmDecStack P = {};
       void* p = nullptr;
       const size_t hp_bytes = sizeof(float) * (size_t)nl * n;
@@ -1606,8 +1615,13 @@ int zr_lstm_decoder_step_packed(zr_ctx* ctx, int nl, const zr_lstm_weights* cons
       P.clip = clip_threshold;
       P.spin_limit = ctx->sweep_spin > 0 ? ctx->sweep_spin : (1 << 20);
       P.fence = (mb % 8 == 0) ? 0 : 1;
+      P.wait_extra = ctx->step_wait_extra;
       ctx->last_stack_path = ZR_LSTM_STACK_PATH_STEP_SINGLE_LAUNCH;
-      lstm_decoder_stack_kernel<1><<<dim3((unsigned)(padded * n_tiles), 2u), 256, 0, ctx->stream>>>(P);
+      const dim3 grid((unsigned)(padded * n_tiles), 2u);
+      if (tn == 1)
+        lstm_decoder_stack_kernel<1><<<grid, 256, 0, ctx->stream>>>(P);
+      else
+        lstm_decoder_stack_kernel<2><<<grid, 256, 0, ctx->stream>>>(P);
       ZR_LAUNCH_CHECK("lstm_decoder_stack_kernel");
       return ZR_OK;
     }

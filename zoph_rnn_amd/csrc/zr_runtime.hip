@@ -227,6 +227,10 @@ int zr_ctx_set_option(zr_ctx* ctx, int option, int value) {
       ZR_CHECK_ARG(value >= 0, "ZR_OPT_LSTM_SWEEP_SPIN must not be negative");
       ctx->sweep_spin = value;
       return ZR_OK;
+    case ZR_OPT_LSTM_STEP_WAIT_EXTRA:
+      ZR_CHECK_ARG(value >= 0 && value <= 1024, "ZR_OPT_LSTM_STEP_WAIT_EXTRA must be in [0, 1024]");
+      ctx->step_wait_extra = value;
+      return ZR_OK;
     case ZR_OPT_BF16_ACTIVATION_TERMS:
       ZR_CHECK_ARG(value == 1 || value == 2, "ZR_OPT_BF16_ACTIVATION_TERMS must be 1 or 2");
       ctx->bf16_terms = value;

@@ -61,10 +61,8 @@ softmax_colstats_kernel(const float* __restrict__ partials, int nblocks, float* 
   }
 }
 
-// out = exp(x - max) / sum   (MODE 0)   or   (x - max) - log(sum)   (MODE 1).  16-byte accesses when VEC, and then
-// each thread takes kNormUnroll of them 256 apart, all loaded before the first is used: one access per thread left
-// the kernel waiting on its own start-up and load latency (6272 workgroups of one load each at 50000 x 128: 26 us).
-constexpr int kNormUnroll = 4;
+// out = exp(x - max) / sum   (MODE 0)   or   (x - max) - log(sum)   (MODE 1).  16-byte accesses when VEC.  One access
+// per thread: four per thread, loaded before the first is used, measured slower (11.1 against 9.4 us at 50000 x 128).
 template <int MODE, bool VEC>
 __global__ void __launch_bounds__(256)
 softmax_normalize_kernel(const float* in, float* out, int V, const float* __restrict__ colstats) {
@@ -75,32 +73,23 @@ softmax_normalize_kernel(const float* in, float* out, int V, const float* __rest
   const float* x = in + (size_t)n * V;
   float* y = out + (size_t)n * V;
   if (VEC) {
-    const int base = blockIdx.x * (256 * kNormUnroll) + threadIdx.x;
-    const int n4 = V >> 2;
-    zr_f32x4 v[kNormUnroll];
-#pragma unroll
-    for (int u = 0; u < kNormUnroll; ++u) {
-      const int i4 = base + 256 * u;
-      v[u] = zr_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-      if (i4 < n4) v[u] = ((const zr_f32x4*)x)[i4];
-    }
-#pragma unroll
-    for (int u = 0; u < kNormUnroll; ++u) {
-      const int i4 = base + 256 * u;
+    const int i4 = blockIdx.x * 256 + threadIdx.x;
+    if (i4 * 4 < V) {
+      zr_f32x4 v = ((const zr_f32x4*)x)[i4];
       zr_f32x4 r;
       if (MODE == 0) {
         // expf(x - max) / sum, as the reference divides (custom_kernels.h:574-576)
-        r.x = expf(v[u].x - mx) / sum;
-        r.y = expf(v[u].y - mx) / sum;
-        r.z = expf(v[u].z - mx) / sum;
-        r.w = expf(v[u].w - mx) / sum;
+        r.x = expf(v.x - mx) / sum;
+        r.y = expf(v.y - mx) / sum;
+        r.z = expf(v.z - mx) / sum;
+        r.w = expf(v.w - mx) / sum;
       } else {
-        r.x = (v[u].x - mx) - lsum;
-        r.y = (v[u].y - mx) - lsum;
-        r.z = (v[u].z - mx) - lsum;
-        r.w = (v[u].w - mx) - lsum;
+        r.x = (v.x - mx) - lsum;
+        r.y = (v.y - mx) - lsum;
+        r.z = (v.z - mx) - lsum;
+        r.w = (v.w - mx) - lsum;
       }
-      if (i4 < n4) ((zr_f32x4*)y)[i4] = r;
+      ((zr_f32x4*)y)[i4] = r;
     }
   } else {
     const int i = blockIdx.x * 256 + threadIdx.x;
@@ -318,18 +307,25 @@ int zr_softmax_forward_packed(zr_ctx* ctx, const float* d_D, const float* d_b_d,
   rc = check_softmax_args("zr_softmax_forward", d_D, d_b_d, V, H, d_h, mb);
   if (rc) return rc;
   ZR_CHECK_ARG(d_out != nullptr, "zr_softmax_forward: d_out is null");
-  ZR_CHECK_ARG(mode == ZR_SOFTMAX_PROB || mode == ZR_SOFTMAX_LOGPROB, "zr_softmax_forward: mode = %d", mode);
-  float* logits = d_logits_scratch ? d_logits_scratch : d_out;
+  ZR_CHECK_ARG(mode == ZR_SOFTMAX_PROB || mode == ZR_SOFTMAX_LOGPROB || mode == ZR_SOFTMAX_LOGITS,
+               "zr_softmax_forward: mode = %d", mode);
+  const bool logits_only = mode == ZR_SOFTMAX_LOGITS;
+  ZR_CHECK_ARG(!logits_only || d_logits_scratch == nullptr,
+               "zr_softmax_forward: ZR_SOFTMAX_LOGITS writes the logits to d_out and takes no d_logits_scratch");
+  float* logits = (d_logits_scratch && !logits_only) ? d_logits_scratch : d_out;
   float* partials = nullptr;
   int nblocks = 0;
   rc = logits_with_partials(ctx, d_D, d_b_d, V, H, d_h, mb, logits, &partials, &nblocks, d_h_packed);
   if (rc) return rc;
-  float* colstats = (float*)stats_ptr(partials, nblocks, mb);
+  // ZR_SOFTMAX_LOGITS: the column statistics go behind the logits in the caller's buffer and no normalised matrix is
+  // written -- a consumer that needs only a few entries per column (the beam search) normalises those itself
+  float* colstats = logits_only ? d_out + (size_t)V * mb : (float*)stats_ptr(partials, nblocks, mb);
   softmax_colstats_kernel<<<mb, 256, 0, ctx->stream>>>(partials, nblocks, colstats);
   ZR_LAUNCH_CHECK("softmax_colstats_kernel");
+  if (logits_only) return ZR_OK;
   const bool vec = (V % 4 == 0) && (((uintptr_t)logits & 15u) == 0) && (((uintptr_t)d_out & 15u) == 0);
   if (vec) {
-    dim3 grid((V / 4 + 256 * kNormUnroll - 1) / (256 * kNormUnroll), mb);
+    dim3 grid((V / 4 + 255) / 256, mb);
     if (mode == ZR_SOFTMAX_PROB)
       softmax_normalize_kernel<0, true><<<grid, 256, 0, ctx->stream>>>(logits, d_out, V, colstats);
     else

@@ -892,8 +892,8 @@ class model_trainer {
 // (src/ensemble_factory.hpp:583-765) does with decoder_model_wrapper::forward_prop_source / forward_prop_target /
 // swap_decoding_states (src/decoder_model_wrapper.hpp, src/model.hpp:2367-2726) and decoder<dType>
 // (src/decoder.h:1158-1413), for n_sent sentences of equal source length side by side.  Columns
-// [s*beam, (s+1)*beam) of every LSTM_size x (n_sent*beam) activation belong to sentence s; the probabilities feed the
-// device-side beam directly, so nothing vocabulary-sized is copied to the host.  As in the reference's decode path
+// [s*beam, (s+1)*beam) of every LSTM_size x (n_sent*beam) activation belong to sentence s; the logits feed the
+// device-side beam directly (it normalises the entries it selects), so nothing vocabulary-sized is copied to the host.  As in the reference's decode path
 // every column runs with mask 1 and a dead beam slot (-1) is fed as word 0.
 struct decoded_hypothesis {
   std::vector<int> words;  // target ids, <START> ... <EOF>
@@ -912,7 +912,7 @@ class beam_decoder {
   zr_beam* bm = nullptr;
   std::vector<dType*> tables;                 // longest_sent source top-layer states, H x cols
   std::vector<dType*> h[2], c[2];             // ping-pong: previous / new state per layer
-  dType *h_tild[2] = {nullptr, nullptr}, *x = nullptr, *prob = nullptr, *zeros = nullptr;
+  dType *h_tild[2] = {nullptr, nullptr}, *x = nullptr, *logits = nullptr, *zeros = nullptr;
   std::vector<dType*> enc_h, enc_c;           // encoder sweep outputs per layer, longest_sent * H * n_sent
   int *d_words = nullptr, *d_words_nn = nullptr, *d_back = nullptr, *d_ones = nullptr, *d_batch_info = nullptr,
       *d_src = nullptr, *d_src_nn = nullptr, *d_src_mask = nullptr, *d_rep = nullptr;
@@ -958,7 +958,8 @@ class beam_decoder {
       h_tild[i] = dmalloc<dType>(n);
     }
     x = dmalloc<dType>(n);
-    prob = dmalloc<dType>((size_t)Vt * cols);
+    // logits, then two statistics per column (ZR_SOFTMAX_LOGITS): the beam normalises only what it selects
+    logits = dmalloc<dType>((size_t)Vt * cols + 2 * (size_t)cols);
     zeros = dmalloc<dType>((size_t)H * n_sent);
     ZOPH_CALL(zr_memset_zero(ctx, zeros, (size_t)H * n_sent * sizeof(dType)));
     for (int l = 0; l < L; l++) {
@@ -995,7 +996,7 @@ class beam_decoder {
     ZOPH_CALL(zr_beam_create(ctx, beam, Vt, n_sent, longest_sent + 3, (float)penalty, &bm));
   }
 
-  // forward_prop_target (src/model.hpp:2573-2688): state half p -> half q, probabilities into prob
+  // forward_prop_target (src/model.hpp:2573-2688): state half p -> half q, logits and column statistics into logits
   void forward_target(int p, int step_index) {
     const int q = 1 - p;
     ZOPH_CALL(zr_vocab_prep(ctx, d_words, cols, Vt, d_words_nn, nullptr));
@@ -1006,7 +1007,7 @@ class beam_decoder {
     ZOPH_CALL(zr_decoder_step(ctx, L, tgt_w.data(), m.input_layer_target.d_W, Vt, d_words_nn, hp.data(), cp.data(), feed,
                               d_ones, 0.0f, cols, h[q].data(), c[q].data(), attention ? attn : nullptr, d_batch_info,
                               attention ? h_tild[q] : nullptr, nullptr, nullptr, nullptr, nullptr, m.softmax_obj.d_D,
-                              m.softmax_obj.d_b_d, Vt, ZR_SOFTMAX_PROB, prob));
+                              m.softmax_obj.d_b_d, Vt, ZR_SOFTMAX_LOGITS, logits));
   }
 
   // Decodes up to n_sent sentences whose integerized sources (reversed, no padding) all have the same length S.
@@ -1058,7 +1059,7 @@ class beam_decoder {
     int p = 0, index = 0;
     for (; index < steps; index++) {
       forward_target(p, index);
-      ZOPH_CALL(zr_beam_expand(ctx, bm, prob, index, d_words, d_back));
+      ZOPH_CALL(zr_beam_expand_logits(ctx, bm, logits, logits + (size_t)Vt * cols, index, d_words, d_back));
       // swap_decoding_states + target_copy_prev_states (src/model.hpp:2691-2726)
       const int q = 1 - p;
       std::vector<const dType*> from(h[q].begin(), h[q].end());
@@ -1073,7 +1074,7 @@ class beam_decoder {
     }
     // one last step and forced <EOF> on every live hypothesis (src/ensemble_factory.hpp:727-743)
     forward_target(p, index);
-    ZOPH_CALL(zr_beam_finish(ctx, bm, prob));
+    ZOPH_CALL(zr_beam_finish_logits(ctx, bm, logits, logits + (size_t)Vt * cols));
     {
       // A single-launch encoder sweep or decoder step that gave up a wait left NaN in its outputs: the batch is
       // decoded again with one launch per node (and so is every later batch of this decoder).
