@@ -350,8 +350,12 @@ def test_single_term_lstm_step_is_the_fp32_path_on_rounded_activations(single_te
     assert 1e-6 < dev < 1e-2, dev
 
 
-@pytest.mark.parametrize("V,H,mb", [(1003, 48, 70), (9000, 112, 130), (12000, 48, 128), (40000, 64, 256)])
+@pytest.mark.parametrize("V,H,mb", [(1003, 48, 70), (9000, 112, 130), (12000, 48, 128), (40000, 64, 256),
+                                    (70000, 208, 256), (66000, 80, 128), (65570, 96, 256)])
 def test_single_term_output_layer_is_the_fp32_path_on_rounded_activations(single_term, V, H, mb):
+    """The last four shapes take the kernel that stages the activations through LDS (256 or 128 columns, K >= 64):
+    only column-split workgroups (40000 rows are fewer than one round of four-block workgroups); a full round plus
+    left-over blocks with K = 208 (three chunks and a quarter); 128 columns; a last 64-row block with 34 rows."""
     ctx = single_term
     g = synth.rng(92, V + mb)
     D = _rb(U(g, (V, H), -0.5, 0.5))
@@ -366,7 +370,7 @@ def test_single_term_output_layer_is_the_fp32_path_on_rounded_activations(single
     close(d_scr.get(), logits, "single-term logits")
     close(d_lp.get(), o.softmax_logprob_f64(logits), "single-term log-probs")
     dev = np.abs(d_scr.get().astype(np.float64) - o.softmax_logits(D, bd, h)).max()
-    assert 1e-6 < dev < 2e-2, dev
+    assert 1e-6 < dev < 2e-2 * max(1.0, np.sqrt(H / 64.0)), dev  # the rounding noise grows with sqrt(K)
 
 
 def test_single_term_stack_rounds_every_product_input(single_term):

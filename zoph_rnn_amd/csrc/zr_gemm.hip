@@ -35,12 +35,83 @@ struct GemmArgs {
   float* gC[8];
 };
 
+template <int... I>
+struct zr_int_seq {};
+template <int N, int... I>
+struct zr_make_int_seq_t : zr_make_int_seq_t<N - 1, N - 1, I...> {};
+template <int... I>
+struct zr_make_int_seq_t<0, I...> {
+  typedef zr_int_seq<I...> type;
+};
+template <int N>
+using zr_make_int_seq = typename zr_make_int_seq_t<N>::type;
+
 // largest divisor c of nv with c * tm <= 32
 constexpr int stats_chunk(int nv, int tm) {
   int best = 1;
   for (int c = 1; c <= nv; ++c)
     if (nv % c == 0 && c * tm <= 32) best = c;
   return best;
+}
+
+// Soft-max-partial epilogue of a wave that holds a whole 32*TM x 32*TN tile (no K split): logits = acc + bias stored to
+// C, and (max, sum exp) of every 32-row block and column to a.partials.  Four columns (accumulator registers) of every
+// row sub-tile at a time, so that their cross-lane reductions run interleaved.  One instantiation per 32-column block
+// (a loop over them is not unrolled at eight blocks, and an accumulator array indexed by a variable lives in memory).
+template <int TM, int TN, int TNI, bool FULL>
+__device__ __forceinline__ void softmax_partial_epilogue_block(const GemmArgs& a, float* C,
+                                                               const zr_f32x16 (&acc)[TM][TN], const float (&bias_v)[TM],
+                                                               int m0, int n0, bool active, int lane) {
+  const int jl = lane & 31;
+  const int half = lane >> 5;
+  auto store = [&](int n, int tm, bool okv, float val, float mxv, float sev) {
+    const int m = m0 + tm * 32 + jl;
+    if (FULL || okv) C[(long long)n * a.ldc + m] = val;
+    const int prow = (m0 >> 5) + tm;  // 32-row block index
+    if (jl == 0 && (FULL || (active && n < a.N && prow * 32 < a.M))) {
+      typedef float zr_f32x2 __attribute__((ext_vector_type(2)));
+      *(zr_f32x2*)(a.partials + ((long long)n * ((a.M + 31) >> 5) + prow) * 2) = zr_f32x2{mxv, sev};
+    }
+  };
+#pragma unroll
+  for (int rg = 0; rg < 4; ++rg) {
+    float v[4 * TM], mx[4 * TM], se[4 * TM];
+    bool ok[4 * TM];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) {
+        const int n = n0 + TNI * 32 + 8 * rg + 4 * half + i;
+        v[i * TM + tm] = acc[tm][TNI][4 * rg + i] + bias_v[tm];
+        ok[i * TM + tm] = FULL || (active && n < a.N && (m0 + tm * 32 + jl) < a.M);
+      }
+    zr_half_wave_softmax_stats<4 * TM>(v, ok, mx, se);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+        store(n0 + TNI * 32 + 8 * rg + 4 * half + i, tm, ok[i * TM + tm], v[i * TM + tm], mx[i * TM + tm],
+              se[i * TM + tm]);
+  }
+}
+
+template <int TM, int TN, bool FULL, int... TNI>
+__device__ __forceinline__ void softmax_partial_epilogue_blocks(const GemmArgs& a, float* C,
+                                                                const zr_f32x16 (&acc)[TM][TN], const float (&bias_v)[TM],
+                                                                int m0, int n0, bool active, int lane,
+                                                                zr_int_seq<TNI...>) {
+  (softmax_partial_epilogue_block<TM, TN, TNI, FULL>(a, C, acc, bias_v, m0, n0, active, lane), ...);
+}
+
+template <int TM, int TN>
+__device__ __forceinline__ void softmax_partial_epilogue(const GemmArgs& a, float* C, const zr_f32x16 (&acc)[TM][TN],
+                                                         const float (&bias_v)[TM], int m0, int n0, bool active,
+                                                         int lane) {
+  // FULL: the whole tile lies inside the matrix (uniform over the wave): no masks, no branches around the stores
+  if (active && m0 + 32 * TM <= a.M && n0 + 32 * TN <= a.N)
+    softmax_partial_epilogue_blocks<TM, TN, true>(a, C, acc, bias_v, m0, n0, active, lane, zr_make_int_seq<TN>{});
+  else
+    softmax_partial_epilogue_blocks<TM, TN, false>(a, C, acc, bias_v, m0, n0, active, lane, zr_make_int_seq<TN>{});
 }
 
 // One output tile of 32*TM rows x 32*TN columns at (m0, n0), computed by the KS waves that call this together
@@ -159,29 +230,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& a, int m0, int n0, boo
       }
     };
     if (KS == 1) {
-      // four columns (accumulator registers) of every row sub-tile at a time
-#pragma unroll
-      for (int tn = 0; tn < TN; ++tn)
-#pragma unroll
-        for (int rg = 0; rg < 4; ++rg) {
-          float v[4 * TM], mx[4 * TM], se[4 * TM];
-          bool ok[4 * TM];
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int tm = 0; tm < TM; ++tm) {
-              const int n = n0 + tn * 32 + 8 * rg + 4 * half + i;
-              v[i * TM + tm] = acc[tm][tn][4 * rg + i] + bias_v[tm];
-              ok[i * TM + tm] = active && n < a.N && (m0 + tm * 32 + jl) < a.M;
-            }
-          zr_half_wave_softmax_stats<4 * TM>(v, ok, mx, se);
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int tm = 0; tm < TM; ++tm)
-              store(n0 + tn * 32 + 8 * rg + 4 * half + i, tm, ok[i * TM + tm], v[i * TM + tm], mx[i * TM + tm],
-                    se[i * TM + tm]);
-        }
+      softmax_partial_epilogue<TM, TN>(a, C, acc, bias_v, m0, n0, active, lane);
     } else {
       constexpr int NV = zr_visit_count<TN, KS>();
       float v[NV * TM];
@@ -375,6 +424,218 @@ __global__ void __launch_bounds__(256, OCC) gemm_tall_kernel(GemmArgs a, int big
     const int blk = big_rows * TM + idx / n32;
     gemm_tile<1, 1, 4, ZR_A_PACK4, true, EPI, 8>(a, blk * 32, (idx % n32) * 32, true, 0, red, kslice, lane);
   }
+}
+
+// Soft-max-partial epilogue for accumulators held the other way round: lane = column (n0 + 32*tn + lane % 32),
+// register r = row m0 + 32*tm + 8*(r/4) + 4*(lane/32) + r%4.  A 32-row block's maximum and sum of exponentials are then
+// 15 in-lane operations and one exchange between the half-waves each (against five cross-lane stages per VALUE when a
+// lane holds one row), and a lane's four consecutive rows leave as one 16-byte store.  VEC: C + n*ldc is 16-byte aligned
+// for every column and the tile lies wholly inside the matrix.
+template <int TM, int TN, int TNI, bool VEC>
+__device__ __forceinline__ void softmax_partial_epilogue_t_block(const GemmArgs& a, const zr_f32x16 (&acc)[TM][TN], int m0,
+                                                                 int n0, int lane) {
+  const int jl = lane & 31, half = lane >> 5;
+  const int n = n0 + TNI * 32 + jl;
+  const int nblocks = (a.M + 31) >> 5;
+#pragma unroll
+  for (int tm = 0; tm < TM; ++tm) {
+    const int mb0 = m0 + tm * 32 + 4 * half;  // this lane's rows: mb0 + 8*q + i
+    float v[16];
+    bool ok[16];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      zr_f32x4 b4;
+      if (VEC) {
+        b4 = *(const zr_f32x4*)(a.bias + mb0 + 8 * q);
+      } else {
+        b4.x = a.bias[min(mb0 + 8 * q, a.M - 1)];
+        b4.y = a.bias[min(mb0 + 8 * q + 1, a.M - 1)];
+        b4.z = a.bias[min(mb0 + 8 * q + 2, a.M - 1)];
+        b4.w = a.bias[min(mb0 + 8 * q + 3, a.M - 1)];
+      }
+      v[4 * q] = acc[tm][TNI][4 * q] + b4.x;
+      v[4 * q + 1] = acc[tm][TNI][4 * q + 1] + b4.y;
+      v[4 * q + 2] = acc[tm][TNI][4 * q + 2] + b4.z;
+      v[4 * q + 3] = acc[tm][TNI][4 * q + 3] + b4.w;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ok[4 * q + i] = VEC || (mb0 + 8 * q + i < a.M && n < a.N);
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) mx = fmaxf(mx, ok[r] ? v[r] : -INFINITY);
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    float se = 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) se += ok[r] ? __builtin_amdgcn_exp2f((v[r] - mx) * 1.4426950408889634f) : 0.0f;
+    se += __shfl_xor(se, 32, 64);
+    float* cp = a.C + (long long)(n < a.N ? n : a.N - 1) * a.ldc + mb0;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (VEC) {
+        *(zr_f32x4*)(cp + 8 * q) = zr_f32x4{v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]};
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (ok[4 * q + i]) cp[8 * q + i] = v[4 * q + i];
+      }
+    }
+    const int prow = (m0 >> 5) + tm;
+    if (half == 0 && n < a.N && prow * 32 < a.M) {
+      typedef float zr_f32x2 __attribute__((ext_vector_type(2)));
+      *(zr_f32x2*)(a.partials + ((long long)n * nblocks + prow) * 2) = zr_f32x2{mx, se};
+    }
+  }
+}
+
+template <int TM, int TN, bool VEC, int... TNI>
+__device__ __forceinline__ void softmax_partial_epilogue_t_blocks(const GemmArgs& a, const zr_f32x16 (&acc)[TM][TN],
+                                                                  int m0, int n0, int lane, zr_int_seq<TNI...>) {
+  (softmax_partial_epilogue_t_block<TM, TN, TNI, VEC>(a, acc, m0, n0, lane), ...);
+}
+
+template <int TM, int TN>
+__device__ __forceinline__ void softmax_partial_epilogue_t(const GemmArgs& a, const zr_f32x16 (&acc)[TM][TN], int m0,
+                                                           int n0, int lane) {
+  const bool vec = m0 + 32 * TM <= a.M && n0 + 32 * TN <= a.N && (a.ldc & 3) == 0 && (m0 & 3) == 0 &&
+                   (((uintptr_t)a.C | (uintptr_t)a.bias) & 15u) == 0;  // uniform
+  if (vec)
+    softmax_partial_epilogue_t_blocks<TM, TN, true>(a, acc, m0, n0, lane, zr_make_int_seq<TN>{});
+  else
+    softmax_partial_epilogue_t_blocks<TM, TN, false>(a, acc, m0, n0, lane, zr_make_int_seq<TN>{});
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Tall bf16 weight matrix (k-interleaved by 8) times a minibatch of exactly 32*NB columns whose activations were
+// rounded to bf16 once (single-term mode), soft-max-partial epilogue: the output-layer product of the bf16 model.
+// In bf16 a 32 x 32 x 16 matrix instruction takes 32 cycles for two 1 KB operands, so a K loop that fetches both
+// operands of every wave from L2 is bound by that traffic, not by the matrix pipe.  Here
+//   * the activations go through LDS: per 64-k chunk the workgroup copies 8 k-groups x 32*NB columns (a contiguous
+//     4*NB KB of the packed array) into one of two LDS buffers, and every wave reads its operands from there;
+//   * the four waves of a workgroup take DIFFERENT rows (64 each) and ALL the columns, so a weight element is
+//     fetched by exactly one wave of the launch, straight into registers, one chunk ahead;
+//   * one barrier per chunk: the chunk after the current one is written into the other buffer before it.
+// 64 x 256 accumulators per wave are 256 registers, which leaves the launch at one workgroup per CU, and the number of
+// 64-row blocks is rarely a multiple of four per CU.  So only whole rounds of such workgroups are taken (ids below
+// n_main); every 64-row block left over goes to one further workgroup whose four waves split the columns instead
+// (the same staging; the weights of those few blocks are fetched by four waves each).
+// ---------------------------------------------------------------------------------------------------------
+template <int TM, int TNW, int NB, int CG>
+__device__ __forceinline__ void bf16_lds_tile(const GemmArgs& a, zr_u32x4* sB, int m0, int nb0, int tid) {
+  constexpr int STEPS = CG / 2;          // 16-k steps per chunk of CG k-groups of 8
+  constexpr int NP = NB * CG / 8;        // 4 KB pieces of the packed activations per chunk, one 16-byte load each
+  constexpr int N = 32 * NB;
+  const int lane = tid & 63, jl = lane & 31, half = lane >> 5;
+  int rows[TM];
+#pragma unroll
+  for (int tm = 0; tm < TM; ++tm) {
+    const int r = m0 + tm * 32 + jl;
+    rows[tm] = r < a.M ? r : a.M - 1;
+  }
+  zr_f32x16 acc[TM][TNW];
+#pragma unroll
+  for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+    for (int tn = 0; tn < TNW; ++tn)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[tm][tn][r] = 0.0f;
+
+  const unsigned lda16 = 16u * (unsigned)a.lda[0];
+  const int kgroups = a.K[0] >> 3;
+  const int nchunks = (kgroups + CG - 1) / CG;
+  const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(a.A[0]), 0,
+                                                                         (unsigned)kgroups * lda16, 0x00020000);
+  const __amdgpu_buffer_rsrc_t brsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(a.B[0]), 0,
+                                                                         (unsigned)kgroups * (16u * N), 0x00020000);
+  unsigned aoff[TM];
+#pragma unroll
+  for (int tm = 0; tm < TM; ++tm) aoff[tm] = 16u * (unsigned)rows[tm] + (unsigned)half * lda16;
+  const unsigned boff = 16u * (unsigned)tid;
+
+  // Both operands are fetched through descriptors that end at k = K, with the whole offset in the per-lane part (the
+  // part the bounds check looks at): the steps of the last chunk that lie past the end of K read zeros, so the loop needs
+  // neither a tail nor a branch around its matrix instructions (which would turn every accumulator into a merge of two
+  // values) nor selects behind its loads (which would make each load wait for its data where it is issued).
+  auto load_a = [&](zr_u32x4 (&ar)[STEPS][TM], int c) {
+#pragma unroll
+    for (int st = 0; st < STEPS; ++st) {
+      const unsigned koff = (unsigned)(c * CG + 2 * st) * lda16;  // uniform
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+        ar[st][tm] =
+            __builtin_bit_cast(zr_u32x4, __builtin_amdgcn_raw_buffer_load_b128(arsrc, (int)(aoff[tm] + koff), 0, 0));
+    }
+  };
+  auto load_b = [&](zr_u32x4 (&stg)[NP], int c) {
+#pragma unroll
+    for (int i = 0; i < NP; ++i)
+      stg[i] = __builtin_bit_cast(
+          zr_u32x4, __builtin_amdgcn_raw_buffer_load_b128(brsrc, (int)(boff + (unsigned)(c * NP + i) * 4096u), 0, 0));
+  };
+  auto store_b = [&](const zr_u32x4 (&stg)[NP], int buf) {
+#pragma unroll
+    for (int i = 0; i < NP; ++i) sB[buf * (CG * N) + i * 256 + tid] = stg[i];
+  };
+  auto compute = [&](const zr_u32x4 (&ar)[STEPS][TM], int buf) {
+    const zr_u32x4* sb = sB + buf * (CG * N) + half * N + nb0 * 32 + jl;
+    zr_u32x4 bq[2][TNW];
+#pragma unroll
+    for (int tn = 0; tn < TNW; ++tn) bq[0][tn] = sb[tn * 32];
+#pragma unroll
+    for (int st = 0; st < STEPS; ++st) {
+      if (st + 1 < STEPS) {
+#pragma unroll
+        for (int tn = 0; tn < TNW; ++tn) bq[(st + 1) & 1][tn] = sb[2 * (st + 1) * N + tn * 32];
+      }
+#pragma unroll
+      for (int tn = 0; tn < TNW; ++tn)
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+          // weights first: a lane ends up with one column and sixteen rows of each 32 x 32 block
+          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(zr_bf16x8, ar[st][tm]),
+                                                                __builtin_bit_cast(zr_bf16x8, bq[st & 1][tn]), acc[tm][tn],
+                                                                0, 0, 0);
+    }
+  };
+
+  // (Weights two chunks ahead, a ring of three register sets, measured no faster: 95.8 against 93.1 us at 65536 rows.)
+  zr_u32x4 ar0[STEPS][TM], ar1[STEPS][TM], stg[NP];
+  load_b(stg, 0);
+  load_a(ar0, 0);
+  store_b(stg, 0);
+  __syncthreads();
+  for (int c = 0; c < nchunks; c += 2) {
+    // the fetches for the next chunk go out before this chunk's matrix work and stay there (the scheduler would
+    // otherwise sink them to their first use, the LDS stores at the end of the chunk)
+    load_b(stg, c + 1);
+    load_a(ar1, c + 1);
+    __builtin_amdgcn_sched_barrier(0);
+    compute(ar0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    store_b(stg, 1);  // buffer 1 was last read in chunk c - 1, behind the barrier that ended it
+    __syncthreads();
+    load_b(stg, c + 2);
+    load_a(ar0, c + 2);
+    __builtin_amdgcn_sched_barrier(0);
+    compute(ar1, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    store_b(stg, 0);
+    __syncthreads();
+  }
+  softmax_partial_epilogue_t<TM, TNW>(a, acc, m0, nb0 * 32, lane);
+}
+
+template <int NB>
+__global__ void __launch_bounds__(256) gemm_bf16_lds_kernel(GemmArgs a, int n_main) {
+  // chunks of 64 k (128-k chunks for the column-split workgroups, whose matrix work per chunk is a quarter as long,
+  // measured slower: 41.6 against 38.0 us for the 226 left-over blocks of 80000 rows)
+  __shared__ zr_u32x4 sB[2 * 8 * 32 * NB];
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int bid = blockIdx.x;
+  if (bid < n_main)
+    bf16_lds_tile<2, NB, NB, 8>(a, sB, (bid * 4 + wave) * 64, 0, tid);
+  else
+    bf16_lds_tile<2, NB / 4, NB, 8>(a, sB, (n_main * 4 + (bid - n_main)) * 64, wave * (NB / 4), tid);
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -671,6 +932,19 @@ int launch_rows(zr_ctx* ctx, GemmArgs& ga, int epi, int n_tiles) {
   return ZR_OK;
 }
 
+// gemm_bf16_lds_kernel: whole rounds of four-block workgroups, one further workgroup per 64-row block left over.
+template <int NB>
+int launch_bf16_lds(zr_ctx* ctx, GemmArgs& ga) {
+  const int nb64 = (ga.M + 63) / 64;
+  const int cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
+  const int n_main = nb64 / (4 * cus) * cus;
+  const int rest = nb64 - 4 * n_main;
+  ga.m_tiles = ga.n_tiles = 0;
+  gemm_bf16_lds_kernel<NB><<<(unsigned)(n_main + rest), 256, 0, ctx->stream>>>(ga, n_main);
+  ZR_LAUNCH_CHECK("gemm_bf16_lds_kernel");
+  return ZR_OK;
+}
+
 // gemm_tall_kernel: N a multiple of 128, fp32 k-interleaved A.  Returns false when the shape is better served by the
 // row-range kernel (too many rows would be left to the small tiles).
 template <int TM, int TN, int PF, int OCC>
@@ -911,6 +1185,12 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
       const int n32 = (d.N + 31) / 32;
       const int n_tiles = (n32 + 3) / 4;
       const int tn = (n32 + n_tiles - 1) / n_tiles;
+      // single-term logits at 256 or 128 columns: activations through LDS, every weight element fetched by one wave
+      if (one_term && d.epilogue == ZR_EPI_SOFTMAX_PARTIAL && ctx->gemm_cfg == 0 && (d.N == 256 || d.N == 128) &&
+          d.K[0] >= 64 && (long long)(d.K[0] / 8 + 32) * d.lda[0] * 16 < (1LL << 32)) {
+        if (d.N == 256) return launch_bf16_lds<8>(ctx, ga);
+        return launch_bf16_lds<4>(ctx, ga);
+      }
       if (one_term) {
         if (tn <= 2) return launch_rows<2, ZR_A_PACK8_BF16_1T>(ctx, ga, d.epilogue, n_tiles);
         if (tn == 3) return launch_rows<3, ZR_A_PACK8_BF16_1T>(ctx, ga, d.epilogue, n_tiles);
