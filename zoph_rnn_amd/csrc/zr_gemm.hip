@@ -506,7 +506,8 @@ __device__ __forceinline__ void softmax_partial_epilogue_t(const GemmArgs& a, co
 
 // ---------------------------------------------------------------------------------------------------------
 // Tall bf16 weight matrix (k-interleaved by 8) times a minibatch of exactly 32*NB columns whose activations were
-// rounded to bf16 once (single-term mode), soft-max-partial epilogue: the output-layer product of the bf16 model.
+// rounded to bf16 once (single-term mode) or split into two bf16 terms, soft-max-partial epilogue: the output-layer
+// product of the bf16 model.
 // In bf16 a 32 x 32 x 16 matrix instruction takes 32 cycles for two 1 KB operands, so a K loop that fetches both
 // operands of every wave from L2 is bound by that traffic, not by the matrix pipe.  Here
 //   * the activations go through LDS: per 64-k chunk the workgroup copies 8 k-groups x 32*NB columns (a contiguous
@@ -519,11 +520,16 @@ __device__ __forceinline__ void softmax_partial_epilogue_t(const GemmArgs& a, co
 // n_main); every 64-row block left over goes to one further workgroup whose four waves split the columns instead
 // (the same staging; the weights of those few blocks are fetched by four waves each).
 // ---------------------------------------------------------------------------------------------------------
-template <int TM, int TNW, int NB, int CG>
+// LO: two-term mode -- the activations come as two bf16 arrays (hi and lo, see zr_split_pack_x_kernel) and every weight
+// operand is multiplied with both; a chunk is then 32 k of each, so that chunks hold the same matrix work in both modes.
+template <int TM, int TNW, int NB, int CG, bool LO>
 __device__ __forceinline__ void bf16_lds_tile(const GemmArgs& a, zr_u32x4* sB, int m0, int nb0, int tid) {
   constexpr int STEPS = CG / 2;          // 16-k steps per chunk of CG k-groups of 8
-  constexpr int NP = NB * CG / 8;        // 4 KB pieces of the packed activations per chunk, one 16-byte load each
+  constexpr int NT = LO ? 2 : 1;         // activation terms
+  constexpr int NP1 = NB * CG / 8;       // 4 KB pieces of one packed activation array per chunk, one 16-byte load each
+  constexpr int NP = NP1 * NT;
   constexpr int N = 32 * NB;
+  constexpr int BUF = NT * CG * N;       // 16-byte elements per LDS buffer: [term][k-group][column]
   const int lane = tid & 63, jl = lane & 31, half = lane >> 5;
   int rows[TM];
 #pragma unroll
@@ -546,6 +552,8 @@ __device__ __forceinline__ void bf16_lds_tile(const GemmArgs& a, zr_u32x4* sB, i
                                                                          (unsigned)kgroups * lda16, 0x00020000);
   const __amdgpu_buffer_rsrc_t brsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(a.B[0]), 0,
                                                                          (unsigned)kgroups * (16u * N), 0x00020000);
+  const __amdgpu_buffer_rsrc_t blrsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<unsigned short*>(LO ? a.Blo[0] : (const unsigned short*)a.B[0]), 0, (unsigned)kgroups * (16u * N), 0x00020000);
   unsigned aoff[TM];
 #pragma unroll
   for (int tm = 0; tm < TM; ++tm) aoff[tm] = 16u * (unsigned)rows[tm] + (unsigned)half * lda16;
@@ -567,32 +575,37 @@ __device__ __forceinline__ void bf16_lds_tile(const GemmArgs& a, zr_u32x4* sB, i
   };
   auto load_b = [&](zr_u32x4 (&stg)[NP], int c) {
 #pragma unroll
-    for (int i = 0; i < NP; ++i)
-      stg[i] = __builtin_bit_cast(
-          zr_u32x4, __builtin_amdgcn_raw_buffer_load_b128(brsrc, (int)(boff + (unsigned)(c * NP + i) * 4096u), 0, 0));
+    for (int i = 0; i < NP; ++i) {
+      const unsigned off = boff + (unsigned)(c * NP1 + i % NP1) * 4096u;
+      stg[i] = __builtin_bit_cast(zr_u32x4,
+                                  __builtin_amdgcn_raw_buffer_load_b128(i < NP1 ? brsrc : blrsrc, (int)off, 0, 0));
+    }
   };
   auto store_b = [&](const zr_u32x4 (&stg)[NP], int buf) {
 #pragma unroll
-    for (int i = 0; i < NP; ++i) sB[buf * (CG * N) + i * 256 + tid] = stg[i];
+    for (int i = 0; i < NP; ++i) sB[buf * BUF + i * 256 + tid] = stg[i];
   };
+  // one pass per (16-k step, term): the same weight operands against the hi octets, then against the lo octets
   auto compute = [&](const zr_u32x4 (&ar)[STEPS][TM], int buf) {
-    const zr_u32x4* sb = sB + buf * (CG * N) + half * N + nb0 * 32 + jl;
+    const zr_u32x4* sb = sB + buf * BUF + half * N + nb0 * 32 + jl;
+    constexpr int PASSES = STEPS * NT;
+    auto frag = [&](int ps, int tn) { return sb[(ps % NT) * (CG * N) + 2 * (ps / NT) * N + tn * 32]; };
     zr_u32x4 bq[2][TNW];
 #pragma unroll
-    for (int tn = 0; tn < TNW; ++tn) bq[0][tn] = sb[tn * 32];
+    for (int tn = 0; tn < TNW; ++tn) bq[0][tn] = frag(0, tn);
 #pragma unroll
-    for (int st = 0; st < STEPS; ++st) {
-      if (st + 1 < STEPS) {
+    for (int ps = 0; ps < PASSES; ++ps) {
+      if (ps + 1 < PASSES) {
 #pragma unroll
-        for (int tn = 0; tn < TNW; ++tn) bq[(st + 1) & 1][tn] = sb[2 * (st + 1) * N + tn * 32];
+        for (int tn = 0; tn < TNW; ++tn) bq[(ps + 1) & 1][tn] = frag(ps + 1, tn);
       }
 #pragma unroll
       for (int tn = 0; tn < TNW; ++tn)
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm)
           // weights first: a lane ends up with one column and sixteen rows of each 32 x 32 block
-          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(zr_bf16x8, ar[st][tm]),
-                                                                __builtin_bit_cast(zr_bf16x8, bq[st & 1][tn]), acc[tm][tn],
+          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(zr_bf16x8, ar[ps / NT][tm]),
+                                                                __builtin_bit_cast(zr_bf16x8, bq[ps & 1][tn]), acc[tm][tn],
                                                                 0, 0, 0);
     }
   };
@@ -624,18 +637,19 @@ __device__ __forceinline__ void bf16_lds_tile(const GemmArgs& a, zr_u32x4* sB, i
   softmax_partial_epilogue_t<TM, TNW>(a, acc, m0, nb0 * 32, lane);
 }
 
-template <int NB>
+template <int NB, bool LO>
 __global__ void __launch_bounds__(256) gemm_bf16_lds_kernel(GemmArgs a, int n_main) {
-  // chunks of 64 k (128-k chunks for the column-split workgroups, whose matrix work per chunk is a quarter as long,
-  // measured slower: 41.6 against 38.0 us for the 226 left-over blocks of 80000 rows)
+  // chunks of 64 k, or of 32 k in each of the two terms (128-k chunks for the column-split workgroups, whose matrix
+  // work per chunk is a quarter as long, measured slower: 41.6 against 38.0 us for the 226 left-over blocks of 80000 rows)
+  constexpr int CG = LO ? 4 : 8;
   __shared__ zr_u32x4 sB[2 * 8 * 32 * NB];
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int bid = blockIdx.x;
   if (bid < n_main)
-    bf16_lds_tile<2, NB, NB, 8>(a, sB, (bid * 4 + wave) * 64, 0, tid);
+    bf16_lds_tile<2, NB, NB, CG, LO>(a, sB, (bid * 4 + wave) * 64, 0, tid);
   else
-    bf16_lds_tile<2, NB / 4, NB, 8>(a, sB, (n_main * 4 + (bid - n_main)) * 64, wave * (NB / 4), tid);
+    bf16_lds_tile<2, NB / 4, NB, CG, LO>(a, sB, (n_main * 4 + (bid - n_main)) * 64, wave * (NB / 4), tid);
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -933,14 +947,14 @@ int launch_rows(zr_ctx* ctx, GemmArgs& ga, int epi, int n_tiles) {
 }
 
 // gemm_bf16_lds_kernel: whole rounds of four-block workgroups, one further workgroup per 64-row block left over.
-template <int NB>
+template <int NB, bool LO>
 int launch_bf16_lds(zr_ctx* ctx, GemmArgs& ga) {
   const int nb64 = (ga.M + 63) / 64;
   const int cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
   const int n_main = nb64 / (4 * cus) * cus;
   const int rest = nb64 - 4 * n_main;
   ga.m_tiles = ga.n_tiles = 0;
-  gemm_bf16_lds_kernel<NB><<<(unsigned)(n_main + rest), 256, 0, ctx->stream>>>(ga, n_main);
+  gemm_bf16_lds_kernel<NB, LO><<<(unsigned)(n_main + rest), 256, 0, ctx->stream>>>(ga, n_main);
   ZR_LAUNCH_CHECK("gemm_bf16_lds_kernel");
   return ZR_OK;
 }
@@ -1185,11 +1199,11 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
       const int n32 = (d.N + 31) / 32;
       const int n_tiles = (n32 + 3) / 4;
       const int tn = (n32 + n_tiles - 1) / n_tiles;
-      // single-term logits at 256 or 128 columns: activations through LDS, every weight element fetched by one wave
-      if (one_term && d.epilogue == ZR_EPI_SOFTMAX_PARTIAL && ctx->gemm_cfg == 0 && (d.N == 256 || d.N == 128) &&
-          d.K[0] >= 64 && (long long)(d.K[0] / 8 + 32) * d.lda[0] * 16 < (1LL << 32)) {
-        if (d.N == 256) return launch_bf16_lds<8>(ctx, ga);
-        return launch_bf16_lds<4>(ctx, ga);
+      // logits at 256 or 128 columns: activations through LDS, every weight element fetched by one wave
+      if (d.epilogue == ZR_EPI_SOFTMAX_PARTIAL && ctx->gemm_cfg == 0 && (d.N == 256 || d.N == 128) && d.K[0] >= 64 &&
+          (long long)(d.K[0] / 8 + 32) * d.lda[0] * 16 < (1LL << 32)) {
+        if (one_term) return d.N == 256 ? launch_bf16_lds<8, false>(ctx, ga) : launch_bf16_lds<4, false>(ctx, ga);
+        return d.N == 256 ? launch_bf16_lds<8, true>(ctx, ga) : launch_bf16_lds<4, true>(ctx, ga);
       }
       if (one_term) {
         if (tn <= 2) return launch_rows<2, ZR_A_PACK8_BF16_1T>(ctx, ga, d.epilogue, n_tiles);
