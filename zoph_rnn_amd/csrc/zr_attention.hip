@@ -513,7 +513,8 @@ int zr_attn_use_bf16_weights(zr_ctx* ctx, zr_attn* a) {
   const int ldp = (H + 31) / 32 * 32;
   const size_t per = (size_t)H * ldp;
   if (!a->d_bf16) {
-    if (hipMalloc((void**)&a->d_bf16, sizeof(unsigned short) * 4 * per) != hipSuccess) {
+    // the four matrices, then room for h_t as two bf16 terms (split once per step for its three products)
+    if (hipMalloc((void**)&a->d_bf16, sizeof(unsigned short) * (4 * per + 2 * (size_t)H * a->mb)) != hipSuccess) {
       (void)hipGetLastError();
       a->d_bf16 = nullptr;
       return zr_set_error(ZR_ENOMEM, "zr_attn_use_bf16_weights: allocation failed");
@@ -623,6 +624,33 @@ int zr_decoder_step(zr_ctx* ctx, int nl, const zr_lstm_weights* const layers[], 
                                    d_out, nullptr);
 }
 
+// Everything between the projections and the output product in one launch (d_tanh1 holds W_p h BEFORE the tanh, d_q
+// holds W_a^T h): the register-resident kernel up to H = 1024 and 64 window slots, the two-pass one beyond.
+static int launch_attn_middle(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, const int* d_mask01, float* pt, int* idx,
+                              float* align, float* cctx, float* cpack) {
+  const int H = a->H, mb = a->mb, D = a->D, W = 2 * D + 1;
+  const float sigma_sq = (float)((D * D) / 4.0);  // attention_node.hpp:50
+  const int max_slots = W < a->longest_sent ? W : a->longest_sent;
+  if (H <= 1024 && max_slots <= 16)
+    attn_fused_reg_kernel<16><<<mb, 256, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_tanh1, a->d_q, a->v_p,
+                                                           d_batch_info, d_mask01, H, mb, D, sigma_sq, pt, idx, align,
+                                                           cctx, cpack, ctx->d_flags);
+  else if (H <= 1024 && max_slots <= 32)
+    attn_fused_reg_kernel<32><<<mb, 256, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_tanh1, a->d_q, a->v_p,
+                                                           d_batch_info, d_mask01, H, mb, D, sigma_sq, pt, idx, align,
+                                                           cctx, cpack, ctx->d_flags);
+  else if (H <= 1024 && max_slots <= 64)
+    attn_fused_reg_kernel<64><<<mb, 256, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_tanh1, a->d_q, a->v_p,
+                                                           d_batch_info, d_mask01, H, mb, D, sigma_sq, pt, idx, align,
+                                                           cctx, cpack, ctx->d_flags);
+  else
+    attn_fused_kernel<<<mb, 256, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_tanh1, a->d_q, a->v_p, d_batch_info,
+                                                   d_mask01, H, mb, D, sigma_sq, pt, idx, align, cctx, cpack,
+                                                   ctx->d_flags);
+  ZR_LAUNCH_CHECK("attn_fused_kernel");
+  return ZR_OK;
+}
+
 static int attn_step_impl(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, const float* d_h_t, const int* d_mask01,
                           float* d_htild, float* d_alignments, int* d_indices, float* d_p_t, float* d_c_ctx,
                           bool h_packed, float* d_htild_pack) {
@@ -636,8 +664,8 @@ static int attn_step_impl(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, cons
   float* pt = d_p_t ? d_p_t : a->d_pt;
   float* cctx = d_c_ctx ? d_c_ctx : a->d_ctx;
 
-  const bool fast = a->d_pack32 && !a->d_bf16 && (H % 4 == 0) && a->tables_aligned && (((uintptr_t)cctx & 15u) == 0) &&
-                    (((uintptr_t)d_h_t & 15u) == 0);
+  const bool fast = a->d_pack32 && !a->d_bf16 && (H % 4 == 0) && a->tables_aligned &&
+                    ((((uintptr_t)cctx | (uintptr_t)d_h_t | (uintptr_t)a->v_p) & 15u) == 0);
   if (fast) {
     // Three launches.  (1) W_p h (before the tanh) and q = W_a^T h as one batch of two products on the k-interleaved
     // snapshots; d_tanh1 and d_q are neighbours in the object's allocation (stride H*mb).
@@ -669,26 +697,8 @@ static int attn_step_impl(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, cons
     rc = zr_gemm_launch(ctx, g);
     if (rc) return rc;
     // (2) p_t, window, scores, alignment weights and context, one workgroup per column
-    const float sigma_sq = (float)((D * D) / 4.0);  // attention_node.hpp:50
-    float* cpack = bp ? a->d_cpack : nullptr;
-    const int max_slots = W < a->longest_sent ? W : a->longest_sent;
-    if (H <= 1024 && max_slots <= 16)
-      attn_fused_reg_kernel<16><<<mb, 256, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_tanh1, a->d_q, a->v_p,
-                                                             d_batch_info, d_mask01, H, mb, D, sigma_sq, pt, idx, align,
-                                                             cctx, cpack, ctx->d_flags);
-    else if (H <= 1024 && max_slots <= 32)
-      attn_fused_reg_kernel<32><<<mb, 256, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_tanh1, a->d_q, a->v_p,
-                                                             d_batch_info, d_mask01, H, mb, D, sigma_sq, pt, idx, align,
-                                                             cctx, cpack, ctx->d_flags);
-    else if (H <= 1024 && max_slots <= 64)
-      attn_fused_reg_kernel<64><<<mb, 256, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_tanh1, a->d_q, a->v_p,
-                                                             d_batch_info, d_mask01, H, mb, D, sigma_sq, pt, idx, align,
-                                                             cctx, cpack, ctx->d_flags);
-    else
-      attn_fused_kernel<<<mb, 256, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_tanh1, a->d_q, a->v_p,
-                                                     d_batch_info, d_mask01, H, mb, D, sigma_sq, pt, idx, align, cctx,
-                                                     cpack, ctx->d_flags);
-    ZR_LAUNCH_CHECK("attn_fused_kernel");
+    rc = launch_attn_middle(ctx, a, d_batch_info, d_mask01, pt, idx, align, cctx, bp ? a->d_cpack : nullptr);
+    if (rc) return rc;
     // (3) h~ = tanh(W_c1 c + W_c2 h + b) * mask
     ZrGemmDesc o = {};
     o.M = H;
@@ -738,14 +748,32 @@ static int attn_step_impl(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, cons
   }
   g.B[0] = d_h_t;
   g.ldb[0] = H;
+  // bf16 weights: h_t enters three products (W_p, W_a^T, W_c2); it is split into its bf16 terms once, here
+  const unsigned short* h_hi = nullptr;
+  const unsigned short* h_lo = nullptr;
+  if (a->d_bf16 && (((uintptr_t)d_h_t & 15u) == 0)) {
+    unsigned short* hs = a->d_bf16 + 4 * per;
+    const bool two_terms = ctx->bf16_terms != 1;
+    rc = zr_split_pack_x_launch(ctx, d_h_t, H, mb, H, hs, two_terms ? hs + (size_t)H * mb : nullptr);
+    if (rc) return rc;
+    h_hi = hs;
+    h_lo = two_terms ? hs + (size_t)H * mb : nullptr;
+    g.Bhi[0] = h_hi;
+    g.Blo[0] = h_lo;
+  }
   g.C = a->d_tanh1;
   g.ldc = H;
   g.batch = 1;
-  g.epilogue = ZR_EPI_TANH;
+  // With 16-byte loads available the window, scores, alignment weights and context are one launch (which applies the
+  // tanh itself) instead of four: bf16 weights, or matrices not registered with zr_attn_prepare.
+  const bool vec = (H % 4 == 0) && a->tables_aligned && ((((uintptr_t)cctx | (uintptr_t)a->v_p) & 15u) == 0);
+  g.epilogue = vec ? ZR_EPI_STORE : ZR_EPI_TANH;
   rc = zr_gemm_launch(ctx, g);
   if (rc) return rc;
-  attn_window_kernel<<<mb, 64, 0, ctx->stream>>>(a->d_tanh1, a->v_p, d_batch_info, d_mask01, H, mb, D, pt, idx);
-  ZR_LAUNCH_CHECK("attn_window_kernel");
+  if (!vec) {
+    attn_window_kernel<<<mb, 64, 0, ctx->stream>>>(a->d_tanh1, a->v_p, d_batch_info, d_mask01, H, mb, D, pt, idx);
+    ZR_LAUNCH_CHECK("attn_window_kernel");
+  }
   // q = W_a^T h  (:195)
   g.A[0] = a->W_a;
   g.trans_a = 1;
@@ -757,30 +785,23 @@ static int attn_step_impl(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, cons
   g.epilogue = ZR_EPI_STORE;
   rc = zr_gemm_launch(ctx, g);
   if (rc) return rc;
-  // 16-byte loads need H % 4 == 0 and 16-byte aligned table / output bases (column offsets are multiples of H)
-  const bool vec = (H % 4 == 0) && a->tables_aligned && (((uintptr_t)cctx & 15u) == 0);
-  const long long slots = (long long)mb * W;
-  const unsigned sgrid = (unsigned)((slots + 3) / 4);
-  if (vec)
-    attn_score_kernel<true><<<sgrid, 256, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_q, idx, d_batch_info, H,
-                                                            mb, W, align, ctx->d_flags);
-  else
-    attn_score_kernel<false><<<sgrid, 256, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_q, idx, d_batch_info,
-                                                             H, mb, W, align, ctx->d_flags);
-  ZR_LAUNCH_CHECK("attn_score_kernel");
-  const float sigma_sq = (float)((D * D) / 4.0);  // attention_node.hpp:50
-  attn_align_kernel<<<mb, 64, 0, ctx->stream>>>(align, idx, pt, mb, W, sigma_sq);
-  ZR_LAUNCH_CHECK("attn_align_kernel");
   if (vec) {
-    dim3 cg((H / 4 + 63) / 64, mb);
-    attn_context_kernel<true><<<cg, 64, 0, ctx->stream>>>(a->d_table, a->longest_sent, align, idx, d_batch_info, H,
-                                                          mb, W, cctx);
+    rc = launch_attn_middle(ctx, a, d_batch_info, d_mask01, pt, idx, align, cctx, nullptr);
+    if (rc) return rc;
   } else {
+    const long long slots = (long long)mb * W;
+    const unsigned sgrid = (unsigned)((slots + 3) / 4);
+    attn_score_kernel<false><<<sgrid, 256, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_q, idx, d_batch_info, H,
+                                                             mb, W, align, ctx->d_flags);
+    ZR_LAUNCH_CHECK("attn_score_kernel");
+    const float sigma_sq = (float)((D * D) / 4.0);  // attention_node.hpp:50
+    attn_align_kernel<<<mb, 64, 0, ctx->stream>>>(align, idx, pt, mb, W, sigma_sq);
+    ZR_LAUNCH_CHECK("attn_align_kernel");
     dim3 cg((H + 63) / 64, mb);
-    attn_context_kernel<false><<<cg, 64, 0, ctx->stream>>>(a->d_table, a->longest_sent, align, idx, d_batch_info, H,
-                                                           mb, W, cctx);
+    attn_context_kernel<false><<<cg, 64, 0, ctx->stream>>>(a->d_table, a->longest_sent, align, idx, d_batch_info, H, mb,
+                                                           W, cctx);
+    ZR_LAUNCH_CHECK("attn_context_kernel");
   }
-  ZR_LAUNCH_CHECK("attn_context_kernel");
   // h~ = tanh(W_c1 c + W_c2 h + b) * mask  (:354-379) as one two-segment GEMM with a fused epilogue
   ZrGemmDesc o = {};
   o.M = H;
@@ -802,6 +823,8 @@ static int attn_step_impl(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, cons
   }
   o.B[1] = d_h_t;
   o.ldb[1] = H;
+  o.Bhi[1] = h_hi;
+  o.Blo[1] = h_lo;
   o.C = d_htild;
   o.ldc = H;
   o.batch = 1;

@@ -1020,6 +1020,44 @@ __global__ void __launch_bounds__(256) zr_split_pack_x_kernel(const float* __res
   if (lo) *(zr_u32x4*)(lo + o) = l;  // null: single-term mode, the residues are dropped
 }
 
+// The same for up to kSplitMultiMax matrices of one shape in one launch (blockIdx.y picks the matrix): a decoder step
+// splits the previous state of every layer, the previous attention output and the embedding columns of the current
+// words at its start, and each of them as a launch of its own costs more in launch latency than in work.  Matrix i goes
+// to hi + i*stride (lo + i*stride); ids (or null) turns matrix 0 into a gather, column n read from src[0] + ids[n]*ld
+// (ids outside [0, V) are clamped, as the gather kernel does).
+constexpr int kSplitMultiMax = 12;
+struct SplitMulti {
+  const float* src[kSplitMultiMax];
+  const int* ids;
+  int V;
+};
+__global__ void __launch_bounds__(256) zr_split_pack_multi_kernel(SplitMulti m, int K, int N, int ld,
+                                                                  unsigned short* __restrict__ hi,
+                                                                  unsigned short* __restrict__ lo, long long stride) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  const int kb = K >> 3;
+  if (i >= kb * N) return;
+  const int which = blockIdx.y;
+  const int n = i / kb, b = i - n * kb;
+  long long col = n;
+  if (which == 0 && m.ids) {
+    const int v = m.ids[n];
+    col = v < 0 ? 0 : (v >= m.V ? m.V - 1 : v);
+  }
+  const float* src = m.src[which] + col * ld + 8 * b;
+  const zr_f32x4 v0 = *(const zr_f32x4*)src;
+  const zr_f32x4 v1 = *(const zr_f32x4*)(src + 4);
+  zr_u32x4 h, l;
+  unsigned a, c;
+  zr_split_bf16_pair(v0.x, v0.y, a, c); h.x = a; l.x = c;
+  zr_split_bf16_pair(v0.z, v0.w, a, c); h.y = a; l.y = c;
+  zr_split_bf16_pair(v1.x, v1.y, a, c); h.z = a; l.z = c;
+  zr_split_bf16_pair(v1.z, v1.w, a, c); h.w = a; l.w = c;
+  const long long o = which * stride + ((long long)b * N + n) * 8;
+  *(zr_u32x4*)(hi + o) = h;
+  if (lo) *(zr_u32x4*)(lo + o) = l;
+}
+
 __global__ void __launch_bounds__(256) pack4_kernel(const float* __restrict__ src, int M, int K, long long ld,
                                                     int ldp, int kp, float* __restrict__ dst) {
   const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
@@ -1070,6 +1108,20 @@ int zr_split_pack_x_launch(zr_ctx* ctx, const float* src, int K, int N, int ld, 
   const int n8 = (K / 8) * N;
   zr_split_pack_x_kernel<<<(n8 + 255) / 256, 256, 0, ctx->stream>>>(src, K, N, ld, hi, lo);
   ZR_LAUNCH_CHECK("zr_split_pack_x_kernel");
+  return ZR_OK;
+}
+
+int zr_split_pack_multi_launch(zr_ctx* ctx, int n_src, const float* const* srcs, const int* d_ids, int V, int K, int N,
+                               int ld, unsigned short* hi, unsigned short* lo, long long stride) {
+  if (n_src < 1 || n_src > kSplitMultiMax) return zr_set_error(ZR_EINVAL, "split: %d matrices in one launch", n_src);
+  SplitMulti m = {};
+  for (int i = 0; i < n_src; ++i) m.src[i] = srcs[i];
+  m.ids = d_ids;
+  m.V = V;
+  const int n8 = (K / 8) * N;
+  zr_split_pack_multi_kernel<<<dim3((unsigned)((n8 + 255) / 256), (unsigned)n_src), 256, 0, ctx->stream>>>(m, K, N, ld, hi,
+                                                                                                          lo, stride);
+  ZR_LAUNCH_CHECK("zr_split_pack_multi_kernel");
   return ZR_OK;
 }
 
@@ -1186,6 +1238,11 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
         const size_t e = (size_t)d.K[s] * d.N;
         const int n8 = (d.K[s] / 8) * d.N;
         const bool lo = !one_term;
+        if (d.Bhi[s] && (one_term || d.Blo[s])) {  // the caller has split this segment already
+          ga.B[s] = (const float*)d.Bhi[s];
+          ga.Blo[s] = lo ? d.Blo[s] : nullptr;
+          continue;
+        }
         zr_split_pack_x_kernel<<<(n8 + 255) / 256, 256, 0, ctx->stream>>>(d.B[s], d.K[s], d.N, d.ldb[s], hi,
                                                                           lo ? hi + e : nullptr);
         ZR_LAUNCH_CHECK("zr_split_pack_x_kernel");

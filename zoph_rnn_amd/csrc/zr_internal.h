@@ -129,6 +129,10 @@ struct ZrGemmDesc {
   // groups > 0: that many independent problems of the same shape in one launch (at most 8; one segment, plain store
   // epilogue, no bias): problem g multiplies gA[g] (instead of A[0]) with gB[g] (instead of B[0]) into gC[g]
   // (instead of C); lda/ldb/ldc, the batch count and its strides apply inside every problem.
+  // a_pack == 2: segment s's activations already split and k-interleaved by 8 (zr_split_pack_x_launch's layout): the
+  // bf16 "hi" array, and the "lo" array in two-term mode (null entries: the launch splits B[s] itself)
+  const unsigned short* Bhi[3];
+  const unsigned short* Blo[3];
   int b_packed;  // with a_pack == 1: B (and every gB) is already k-interleaved, element (k, n) at ((k/4)*N + n)*4 + k%4
                  // (K a multiple of 8, 16-byte aligned); ldb is ignored
   int groups;
@@ -149,6 +153,10 @@ int zr_pack4_trans_launch(zr_ctx* ctx, const float* src, int M, int K, long long
 // Same for the bf16 layout [kp/8][ldp][8] (round to nearest even); kp a multiple of 16.  dst holds kp*ldp elements.
 // Activations X (K x N fp32, column-major with leading dimension ld, K % 8 == 0) split into bf16 hi + lo arrays
 // (K*N elements each), both k-interleaved by 8.
+// n_src (at most 12) K x N matrices split in one launch: matrix i to hi + i*stride (and lo + i*stride; lo null: single
+// term).  d_ids non-null: matrix 0 is gathered, column n read from srcs[0] + clamp(d_ids[n], 0, V-1)*ld.
+int zr_split_pack_multi_launch(zr_ctx* ctx, int n_src, const float* const* srcs, const int* d_ids, int V, int K, int N,
+                               int ld, unsigned short* hi, unsigned short* lo, long long stride);
 int zr_split_pack_x_launch(zr_ctx* ctx, const float* src, int K, int N, int ld, unsigned short* hi,
                            unsigned short* lo);
 // trans != 0: the source holds the transpose (element (row, k) at src[k + row*ld]).

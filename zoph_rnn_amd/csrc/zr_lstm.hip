@@ -1425,7 +1425,8 @@ int zr_lstm_weights_destroy(zr_ctx* ctx, zr_lstm_weights* w) {
 
 static int lstm_step_impl(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_in, const int* d_gather_ids, int V,
                           const float* d_hprev, const float* d_cprev, const float* d_htild, const int* d_mask01,
-                          float clip_threshold, int mb, float* d_h, float* d_c, float* const d_gates[4]);
+                          float clip_threshold, int mb, float* d_h, float* d_c, float* const d_gates[4],
+                          const unsigned short* const* pre_hi = nullptr, const unsigned short* const* pre_lo = nullptr);
 
 int zr_lstm_step(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_in, const float* d_hprev,
                  const float* d_cprev, const float* d_htild, const int* d_mask01, float clip_threshold, int mb,
@@ -1443,9 +1444,12 @@ int zr_lstm_step_embed(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_emb
 }
 
 // d_gather_ids non-null: d_in is the H x V embedding and column b of the input is d_in[:, d_gather_ids[b]].
+// pre_hi / pre_lo (or null; bf16 weights only): segment s's input already split into bf16 terms and k-interleaved by 8
+// (pre_lo[s] null in single-term mode); such a segment is neither gathered nor split here.
 static int lstm_step_impl(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_in, const int* d_gather_ids, int V,
                           const float* d_hprev, const float* d_cprev, const float* d_htild, const int* d_mask01,
-                          float clip_threshold, int mb, float* d_h, float* d_c, float* const d_gates[4]) {
+                          float clip_threshold, int mb, float* d_h, float* d_c, float* const d_gates[4],
+                          const unsigned short* const* pre_hi, const unsigned short* const* pre_lo) {
   int rc = zr_bind_device(ctx);
   if (rc) return rc;
   ZR_CHECK_ARG(w != nullptr, "zr_lstm_step: weights are null");
@@ -1457,6 +1461,9 @@ static int lstm_step_impl(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_
     for (int g = 0; g < 4; ++g) ZR_CHECK_ARG(d_gates[g] != nullptr, "zr_lstm_step: d_gates[%d] is null", g);
   const int H = w->H;
   const int nseg = d_htild ? 3 : 2;
+  const bool two_terms = ctx->bf16_terms != 1;
+  auto presplit = [&](int sg) { return w->bf16 && pre_hi && pre_hi[sg] && (!two_terms || (pre_lo && pre_lo[sg])); };
+  if (d_gather_ids && presplit(0)) d_gather_ids = nullptr;  // the split columns are the gathered ones
   if (d_gather_ids && (w->bf16 || !ctx->lstm_fused)) {
     // these paths re-lay-out or re-read their inputs as whole matrices: gather the columns first
     void* x = nullptr;
@@ -1501,7 +1508,12 @@ static int lstm_step_impl(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_
     if (rc) return rc;
     unsigned short* hi = (unsigned short*)p;
     for (int s = 0; s < nseg; ++s) {
-      const bool lo = ctx->bf16_terms != 1;
+      const bool lo = two_terms;
+      if (presplit(s)) {
+        U.inp[s] = (const float*)pre_hi[s];
+        U.inp_lo[s] = lo ? pre_lo[s] : nullptr;
+        continue;
+      }
       rc = zr_split_pack_x_launch(ctx, U.in[s], H, mb, H, hi, lo ? hi + e : nullptr);
       if (rc) return rc;
       U.inp[s] = (const float*)hi;
@@ -1627,6 +1639,41 @@ int zr_lstm_decoder_step_packed(zr_ctx* ctx, int nl, const zr_lstm_weights* cons
     }
   }
   ctx->last_stack_path = ZR_LSTM_STACK_PATH_STEP_PER_LAYER;
+  if (layers[0]->bf16 && vec && ctx->lstm_fused && nl + 2 <= 12) {
+    // bf16 weights: every product input enters as bf16 terms, k-interleaved.  Everything the step knows at its start --
+    // the embedding columns of the current words, h_{t-1} of every layer, the previous attention output -- is split in
+    // ONE launch (as launches of their own these nl + 2 small kernels, and the gather in front of the first, cost more
+    // in launch latency than in work); only h_t of the layer below is split between the layers.
+    const bool two_terms = ctx->bf16_terms != 1;
+    const size_t e = n;  // bf16 elements per array
+    void* p = nullptr;
+    rc = zr_ctx_scratch(ctx, 1, sizeof(unsigned short) * 2 * e * (size_t)(nl + 3), &p);
+    if (rc) return rc;
+    unsigned short* hi = (unsigned short*)p;
+    unsigned short* lo = hi + e * (size_t)(nl + 3);
+    const float* srcs[12];
+    int ns = 0;
+    srcs[ns++] = d_embed;  // matrix 0: gathered by the word ids
+    for (int l = 0; l < nl; ++l) srcs[ns++] = d_hprev[l];
+    if (d_htild) srcs[ns++] = d_htild;
+    rc = zr_split_pack_multi_launch(ctx, ns, srcs, d_ids_nonneg, V, H, mb, H, hi, two_terms ? lo : nullptr, (long long)e);
+    if (rc) return rc;
+    unsigned short* below_hi = hi + e * (size_t)(nl + 2);
+    unsigned short* below_lo = lo + e * (size_t)(nl + 2);
+    for (int l = 0; l < nl; ++l) {
+      const unsigned short* ph[3] = {l == 0 ? hi : below_hi, hi + e * (size_t)(1 + l), hi + e * (size_t)(1 + nl)};
+      const unsigned short* pl[3] = {l == 0 ? lo : below_lo, lo + e * (size_t)(1 + l), lo + e * (size_t)(1 + nl)};
+      if (l > 0) {
+        rc = zr_split_pack_x_launch(ctx, d_h[l - 1], H, mb, H, below_hi, two_terms ? below_lo : nullptr);
+        if (rc) return rc;
+      }
+      rc = lstm_step_impl(ctx, layers[l], l == 0 ? d_embed : d_h[l - 1], l == 0 ? d_ids_nonneg : nullptr, l == 0 ? V : 0,
+                          d_hprev[l], d_cprev[l], l == 0 ? d_htild : nullptr, d_mask01, clip_threshold, mb, d_h[l],
+                          d_c[l], nullptr, ph, two_terms ? pl : nullptr);
+      if (rc) return rc;
+    }
+    return ZR_OK;
+  }
   for (int l = 0; l < nl; ++l) {
     if (l == 0)
       rc = lstm_step_impl(ctx, layers[0], d_embed, d_ids_nonneg, V, d_hprev[0], d_cprev[0], d_htild, d_mask01,
