@@ -438,3 +438,78 @@ def test_single_term_attention_within_stated_bound(single_term):
     assert safe.sum() > mb // 2
     assert np.array_equal(got["indices"][safe], want["indices"][safe])
     assert np.abs(got["h_tild"][:, safe] - want["h_tild"][:, safe]).max() < 1e-2
+
+
+@pytest.mark.parametrize("terms", [2, 1])
+@pytest.mark.parametrize("H,mb,L,S,D,V,feed", [(112, 64, 3, 9, 3, 301, True), (496, 256, 2, 20, 10, 9000, True),
+                                               (64, 33, 1, 7, 2, 211, False)])
+def test_bf16_decoder_step_as_one_call_matches_the_separate_calls(ctx, H, mb, L, S, D, V, feed, terms):
+    """zr_decoder_step on bf16 weights (the step's known inputs -- embedding columns, h_{t-1} of every layer, the previous
+    attention output -- split into bf16 terms in one launch, h_t split once for the attention products) against one
+    zr_lstm_step_embed / zr_lstm_step per layer + zr_attn_step + zr_softmax_forward: the same kernels read the same
+    numbers, so every output is the same bit for bit, in both activation modes, with and without feed-input; and the
+    top h against the oracle on the rounded weights (and, in single-term mode, rounded product inputs)."""
+    ctx.set_option(capi.ZR_OPT_BF16_ACTIVATION_TERMS, terms)
+    g = synth.rng(93, H + mb + L)
+    lys_np = [_rounded_layer(g, H, feed and l == 0)[0] for l in range(L)]
+    embed = U(g, (H, V), -1, 1)
+    ids = g.integers(0, V, size=mb).astype(np.int32)
+    ids[0], ids[mb - 1] = 0, V - 1
+    hp = [U(g, (H, mb), -1, 1) for _ in range(L)]
+    cp = [U(g, (H, mb), -1, 1) for _ in range(L)]
+    ht = U(g, (H, mb), -1, 1) if feed else None
+    mask = np.ones(mb, np.int32)
+    mask[mb // 2] = 0
+    w = synth.attention_weights(g, H)
+    for k in ("W_a", "W_p", "W_c1", "W_c2"):
+        w[k] = np.asfortranarray(round_bf16(w[k]))
+    hs = (g.standard_normal(size=(S, H, mb), dtype=np.float32) * np.float32(0.1))
+    lens = g.integers(1, S + 1, size=mb).astype(np.int32)
+    binfo = np.concatenate([lens, S - lens]).astype(np.int32)
+    Dm, bd = np.asfortranarray(round_bf16(U(g, (V, H), -0.3, 0.3))), U(g, (V,))
+    lys = [Layer(ctx, ly, bf16=True) for ly in lys_np]
+    tables = [ctx.array(np.asfortranarray(hs[t])) for t in range(S)]
+    dw = {k: ctx.array(v) for k, v in w.items()}
+    a = ctx.attn_create(H, mb, D, dw["W_a"], dw["W_p"], dw["v_p"], dw["out_bias"], dw["W_c1"], dw["W_c2"], tables)
+    ctx.attn_use_bf16_weights(a)
+    dD, dbd = ctx.array(Dm), ctx.array(bd)
+    ctx.softmax_prepare(dD, V, H, bf16=True)
+    try:
+        d_embed, d_ids, d_mask, d_bi = ctx.array(embed), ctx.array(ids), ctx.array(mask), ctx.array(binfo)
+        d_hp, d_cp = [ctx.array(x) for x in hp], [ctx.array(x) for x in cp]
+        d_htp = ctx.array(ht) if feed else None
+        outs = []
+        for one_call in (False, True):
+            d_h = [ctx.zeros((H, mb)) for _ in range(L)]
+            d_c = [ctx.zeros((H, mb)) for _ in range(L)]
+            d_ht, d_p = ctx.zeros((H, mb)), ctx.zeros((V, mb))
+            if one_call:
+                ctx.decoder_step([ly.w for ly in lys], d_embed, V, d_ids, d_hp, d_cp, d_mask, mb, d_h, d_c, a, d_bi, d_ht, dD,
+                                 dbd, V, capi.ZR_SOFTMAX_PROB, d_p, d_htild_prev=d_htp)
+                assert ctx.query(capi.ZR_QUERY_LSTM_STACK_PATH) == capi.ZR_LSTM_STACK_PATH_STEP_PER_LAYER
+            else:
+                for l in range(L):
+                    if l == 0:
+                        ctx.lstm_step_embed(lys[0].w, d_embed, V, d_ids, d_hp[0], d_cp[0], d_mask, mb, d_h[0], d_c[0],
+                                            d_htild=d_htp)
+                    else:
+                        ctx.lstm_step(lys[l].w, d_h[l - 1], d_hp[l], d_cp[l], d_mask, mb, d_h[l], d_c[l])
+                ctx.attn_step(a, d_bi, d_h[L - 1], d_mask, d_ht)
+                ctx.softmax_forward(dD, dbd, V, H, d_ht, mb, capi.ZR_SOFTMAX_PROB, d_p)
+            ctx.sync()
+            outs.append([x.get() for x in d_h + d_c + [d_ht, d_p]])
+        for x, y in zip(*outs):
+            assert x.tobytes() == y.tobytes()
+        rnd = _rb if terms == 1 else (lambda z: z)
+        x = rnd(o.embed_gather(embed, ids))
+        for l, ly in enumerate(lys_np):
+            r = o.lstm_step(ly["M"], ly["Wh"], ly["b"], x, rnd(hp[l]), cp[l], mask, Q=ly.get("Q") if l == 0 else None,
+                            htild=rnd(ht) if (feed and l == 0) else None)
+            close(outs[1][l], r["h"], "h of layer %d" % l)
+            x = rnd(np.asfortranarray(outs[1][l]))
+    finally:
+        ctx.set_option(capi.ZR_OPT_BF16_ACTIVATION_TERMS, 2)
+        ctx.softmax_release(dD)
+        ctx.attn_destroy(a)
+        for ly in lys:
+            ly.close()
