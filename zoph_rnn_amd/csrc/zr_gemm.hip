@@ -522,7 +522,8 @@ __device__ __forceinline__ void softmax_partial_epilogue_t(const GemmArgs& a, co
 // ---------------------------------------------------------------------------------------------------------
 // LO: two-term mode -- the activations come as two bf16 arrays (hi and lo, see zr_split_pack_x_kernel) and every weight
 // operand is multiplied with both; a chunk is then 32 k of each, so that chunks hold the same matrix work in both modes.
-template <int TM, int TNW, int NB, int CG, bool LO>
+// PD: how many chunks ahead the fetches run (a ring of PD + 1 register sets).
+template <int TM, int TNW, int NB, int CG, bool LO, int PD>
 __device__ __forceinline__ void bf16_lds_tile(const GemmArgs& a, zr_u32x4* sB, int m0, int nb0, int tid) {
   constexpr int STEPS = CG / 2;          // 16-k steps per chunk of CG k-groups of 8
   constexpr int NT = LO ? 2 : 1;         // activation terms
@@ -610,46 +611,50 @@ __device__ __forceinline__ void bf16_lds_tile(const GemmArgs& a, zr_u32x4* sB, i
     }
   };
 
-  // (Weights two chunks ahead, a ring of three register sets, measured no faster: 95.8 against 93.1 us at 65536 rows.)
-  zr_u32x4 ar0[STEPS][TM], ar1[STEPS][TM], stg[NP];
-  load_b(stg, 0);
-  load_a(ar0, 0);
-  store_b(stg, 0);
+  // Ring of R = PD + 1 register sets for the weights and the staged activations.  One chunk ahead everywhere: two ahead
+  // measured no faster for the row-split workgroups (95.8 against 93.1 us at 65536 rows), three ahead no faster for the
+  // column-split ones (41.2 against 38.0 us for the 226 left-over blocks of 80000 rows), and neither did giving those
+  // two row blocks each (49.7 us) or 128-k chunks (41.6 us).
+  constexpr int R = PD + 1;
+  static_assert(R % 2 == 0, "the LDS buffer of a chunk is its index modulo 2, fixed inside the unrolled loop body");
+  zr_u32x4 ar[R][STEPS][TM], stg[R][NP];
+#pragma unroll
+  for (int k = 0; k < PD; ++k) {
+    load_b(stg[k], k);
+    load_a(ar[k], k);
+  }
+  store_b(stg[0], 0);
   __syncthreads();
-  for (int c = 0; c < nchunks; c += 2) {
-    // the fetches for the next chunk go out before this chunk's matrix work and stay there (the scheduler would
-    // otherwise sink them to their first use, the LDS stores at the end of the chunk)
-    load_b(stg, c + 1);
-    load_a(ar1, c + 1);
-    __builtin_amdgcn_sched_barrier(0);
-    compute(ar0, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    store_b(stg, 1);  // buffer 1 was last read in chunk c - 1, behind the barrier that ended it
-    __syncthreads();
-    load_b(stg, c + 2);
-    load_a(ar0, c + 2);
-    __builtin_amdgcn_sched_barrier(0);
-    compute(ar1, 1);
-    __builtin_amdgcn_sched_barrier(0);
-    store_b(stg, 0);
-    __syncthreads();
+  for (int c0 = 0; c0 < nchunks; c0 += R) {
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+      const int c = c0 + u;
+      // the fetches go out before this chunk's matrix work and stay there (the scheduler would otherwise sink them to
+      // their first use, the LDS stores at the end of a chunk)
+      load_b(stg[(u + PD) % R], c + PD);
+      load_a(ar[(u + PD) % R], c + PD);
+      __builtin_amdgcn_sched_barrier(0);
+      compute(ar[u], u & 1);
+      __builtin_amdgcn_sched_barrier(0);
+      store_b(stg[(u + 1) % R], (u + 1) & 1);  // that buffer was last read in chunk c - 1, behind the barrier that ended it
+      __syncthreads();
+    }
   }
   softmax_partial_epilogue_t<TM, TNW>(a, acc, m0, nb0 * 32, lane);
 }
 
 template <int NB, bool LO>
 __global__ void __launch_bounds__(256) gemm_bf16_lds_kernel(GemmArgs a, int n_main) {
-  // chunks of 64 k, or of 32 k in each of the two terms (128-k chunks for the column-split workgroups, whose matrix
-  // work per chunk is a quarter as long, measured slower: 41.6 against 38.0 us for the 226 left-over blocks of 80000 rows)
+  // chunks of 64 k, or of 32 k in each of the two terms
   constexpr int CG = LO ? 4 : 8;
   __shared__ zr_u32x4 sB[2 * 8 * 32 * NB];
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int bid = blockIdx.x;
   if (bid < n_main)
-    bf16_lds_tile<2, NB, NB, CG, LO>(a, sB, (bid * 4 + wave) * 64, 0, tid);
+    bf16_lds_tile<2, NB, NB, CG, LO, 1>(a, sB, (bid * 4 + wave) * 64, 0, tid);
   else
-    bf16_lds_tile<2, NB / 4, NB, CG, LO>(a, sB, (n_main * 4 + (bid - n_main)) * 64, wave * (NB / 4), tid);
+    bf16_lds_tile<2, NB / 4, NB, CG, LO, 1>(a, sB, (n_main * 4 + (bid - n_main)) * 64, wave * (NB / 4), tid);
 }
 
 // ---------------------------------------------------------------------------------------------------------
