@@ -511,18 +511,20 @@ __device__ __forceinline__ void softmax_partial_epilogue_t(const GemmArgs& a, co
 // In bf16 a 32 x 32 x 16 matrix instruction takes 32 cycles for two 1 KB operands, so a K loop that fetches both
 // operands of every wave from L2 is bound by that traffic, not by the matrix pipe.  Here
 //   * the activations go through LDS: per 64-k chunk the workgroup copies 8 k-groups x 32*NB columns (a contiguous
-//     4*NB KB of the packed array) into one of two LDS buffers, and every wave reads its operands from there;
+//     4*NB KB of the packed array) into one of two LDS buffers with loads that write LDS directly (no staging
+//     registers, no LDS store instructions), and every wave reads its operands from there;
 //   * the four waves of a workgroup take DIFFERENT rows (64 each) and ALL the columns, so a weight element is
 //     fetched by exactly one wave of the launch, straight into registers, one chunk ahead;
-//   * one barrier per chunk: the chunk after the current one is written into the other buffer before it.
+//   * one barrier per chunk, behind a wait for the chunk's fetches: the chunk after the current one lands in the other
+//     buffer while the current one is multiplied.
 // 64 x 256 accumulators per wave are 256 registers, which leaves the launch at one workgroup per CU, and the number of
 // 64-row blocks is rarely a multiple of four per CU.  So only whole rounds of such workgroups are taken (ids below
 // n_main); every 64-row block left over goes to one further workgroup whose four waves split the columns instead
 // (the same staging; the weights of those few blocks are fetched by four waves each).
 // ---------------------------------------------------------------------------------------------------------
 // LO: two-term mode -- the activations come as two bf16 arrays (hi and lo, see zr_split_pack_x_kernel) and every weight
-// operand is multiplied with both; a chunk is then 32 k of each, so that chunks hold the same matrix work in both modes.
-// PD: how many chunks ahead the fetches run (a ring of PD + 1 register sets).
+// operand is multiplied with both (a chunk then holds CG k-groups of each term).
+// PD: how many chunks ahead the weight fetches run (a ring of PD + 1 register sets; 1 with the LDS double buffer).
 template <int TM, int TNW, int NB, int CG, bool LO, int PD>
 __device__ __forceinline__ void bf16_lds_tile(const GemmArgs& a, zr_u32x4* sB, int m0, int nb0, int tid) {
   constexpr int STEPS = CG / 2;          // 16-k steps per chunk of CG k-groups of 8
@@ -574,17 +576,16 @@ __device__ __forceinline__ void bf16_lds_tile(const GemmArgs& a, zr_u32x4* sB, i
             __builtin_bit_cast(zr_u32x4, __builtin_amdgcn_raw_buffer_load_b128(arsrc, (int)(aoff[tm] + koff), 0, 0));
     }
   };
-  auto load_b = [&](zr_u32x4 (&stg)[NP], int c) {
+  // activations: straight from memory into LDS (each lane's 16 bytes land at the wave's base + 16 * lane)
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  auto load_b = [&](int c, int buf) {
 #pragma unroll
     for (int i = 0; i < NP; ++i) {
       const unsigned off = boff + (unsigned)(c * NP1 + i % NP1) * 4096u;
-      stg[i] = __builtin_bit_cast(zr_u32x4,
-                                  __builtin_amdgcn_raw_buffer_load_b128(i < NP1 ? brsrc : blrsrc, (int)off, 0, 0));
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(i < NP1 ? brsrc : blrsrc,
+                                               (__attribute__((address_space(3))) void*)(sB + buf * BUF + i * 256 + wave * 64),
+                                               16, (int)off, 0, 0, 0);
     }
-  };
-  auto store_b = [&](const zr_u32x4 (&stg)[NP], int buf) {
-#pragma unroll
-    for (int i = 0; i < NP; ++i) sB[buf * BUF + i * 256 + tid] = stg[i];
   };
   // one pass per (16-k step, term): the same weight operands against the hi octets, then against the lo octets
   auto compute = [&](const zr_u32x4 (&ar)[STEPS][TM], int buf) {
@@ -616,27 +617,24 @@ __device__ __forceinline__ void bf16_lds_tile(const GemmArgs& a, zr_u32x4* sB, i
   // column-split ones (41.2 against 38.0 us for the 226 left-over blocks of 80000 rows), and neither did giving those
   // two row blocks each (49.7 us) or 128-k chunks (41.6 us).
   constexpr int R = PD + 1;
-  static_assert(R % 2 == 0, "the LDS buffer of a chunk is its index modulo 2, fixed inside the unrolled loop body");
-  zr_u32x4 ar[R][STEPS][TM], stg[R][NP];
-#pragma unroll
-  for (int k = 0; k < PD; ++k) {
-    load_b(stg[k], k);
-    load_a(ar[k], k);
-  }
-  store_b(stg[0], 0);
+  static_assert(PD == 1, "the LDS double buffer is written one chunk ahead");
+  zr_u32x4 ar[R][STEPS][TM];
+  load_b(0, 0);
+  load_a(ar[0], 0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the LDS loads have landed
   __syncthreads();
   for (int c0 = 0; c0 < nchunks; c0 += R) {
 #pragma unroll
     for (int u = 0; u < R; ++u) {
       const int c = c0 + u;
-      // the fetches go out before this chunk's matrix work and stay there (the scheduler would otherwise sink them to
-      // their first use, the LDS stores at the end of a chunk)
-      load_b(stg[(u + PD) % R], c + PD);
-      load_a(ar[(u + PD) % R], c + PD);
+      // the fetches go out before this chunk's matrix work and stay there; the other LDS buffer was last read in chunk
+      // c - 1, behind the barrier that ended it
+      load_b(c + 1, (u + 1) & 1);
+      load_a(ar[(u + 1) % R], c + 1);
       __builtin_amdgcn_sched_barrier(0);
       compute(ar[u], u & 1);
       __builtin_amdgcn_sched_barrier(0);
-      store_b(stg[(u + 1) % R], (u + 1) & 1);  // that buffer was last read in chunk c - 1, behind the barrier that ended it
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
       __syncthreads();
     }
   }
@@ -645,9 +643,10 @@ __device__ __forceinline__ void bf16_lds_tile(const GemmArgs& a, zr_u32x4* sB, i
 
 template <int NB, bool LO>
 __global__ void __launch_bounds__(256) gemm_bf16_lds_kernel(GemmArgs a, int n_main) {
-  // chunks of 64 k, or of 32 k in each of the two terms
-  constexpr int CG = LO ? 4 : 8;
-  __shared__ zr_u32x4 sB[2 * 8 * 32 * NB];
+  // chunks of 64 k (of each term); measured at 80000 x 256 x 2000: 128-k chunks no faster in single-term mode (126 us
+  // either way), 32-k chunks of each term slower in two-term mode (212 against 195 us)
+  constexpr int CG = 8;
+  __shared__ zr_u32x4 sB[2 * (LO ? 2 : 1) * CG * 32 * NB];
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int bid = blockIdx.x;
