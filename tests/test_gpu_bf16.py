@@ -441,13 +441,16 @@ def test_single_term_attention_within_stated_bound(single_term):
 
 
 @pytest.mark.parametrize("terms", [2, 1])
-@pytest.mark.parametrize("H,mb,L,S,D,V,feed", [(112, 64, 3, 9, 3, 301, True), (496, 256, 2, 20, 10, 9000, True),
-                                               (64, 33, 1, 7, 2, 211, False)])
-def test_bf16_decoder_step_as_one_call_matches_the_separate_calls(ctx, H, mb, L, S, D, V, feed, terms):
+@pytest.mark.parametrize("H,mb,L,S,D,V,feed,attn_bf16", [(112, 64, 3, 9, 3, 301, True, True),
+                                                         (496, 256, 2, 20, 10, 9000, True, True),
+                                                         (64, 33, 1, 7, 2, 211, False, True),
+                                                         (112, 64, 2, 9, 3, 301, True, False)])
+def test_bf16_decoder_step_as_one_call_matches_the_separate_calls(ctx, H, mb, L, S, D, V, feed, attn_bf16, terms):
     """zr_decoder_step on bf16 weights (the step's known inputs -- embedding columns, h_{t-1} of every layer, the previous
     attention output -- split into bf16 terms in one launch, h_t split once for the attention products) against one
     zr_lstm_step_embed / zr_lstm_step per layer + zr_attn_step + zr_softmax_forward: the same kernels read the same
-    numbers, so every output is the same bit for bit, in both activation modes, with and without feed-input; and the
+    numbers, so every output is the same bit for bit, in both activation modes, with and without feed-input, and with an
+    fp32 attention layer (registered matrices) behind the bf16 LSTM layers, which must not be handed bf16 terms; and the
     top h against the oracle on the rounded weights (and, in single-term mode, rounded product inputs)."""
     ctx.set_option(capi.ZR_OPT_BF16_ACTIVATION_TERMS, terms)
     g = synth.rng(93, H + mb + L)
@@ -471,9 +474,12 @@ def test_bf16_decoder_step_as_one_call_matches_the_separate_calls(ctx, H, mb, L,
     tables = [ctx.array(np.asfortranarray(hs[t])) for t in range(S)]
     dw = {k: ctx.array(v) for k, v in w.items()}
     a = ctx.attn_create(H, mb, D, dw["W_a"], dw["W_p"], dw["v_p"], dw["out_bias"], dw["W_c1"], dw["W_c2"], tables)
-    ctx.attn_use_bf16_weights(a)
+    if attn_bf16:
+        ctx.attn_use_bf16_weights(a)
+    else:
+        ctx.attn_prepare(a)
     dD, dbd = ctx.array(Dm), ctx.array(bd)
-    ctx.softmax_prepare(dD, V, H, bf16=True)
+    ctx.softmax_prepare(dD, V, H, bf16=attn_bf16)
     try:
         d_embed, d_ids, d_mask, d_bi = ctx.array(embed), ctx.array(ids), ctx.array(mask), ctx.array(binfo)
         d_hp, d_cp = [ctx.array(x) for x in hp], [ctx.array(x) for x in cp]

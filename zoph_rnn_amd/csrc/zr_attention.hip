@@ -611,14 +611,21 @@ int zr_decoder_step(zr_ctx* ctx, int nl, const zr_lstm_weights* const layers[], 
                "null batch info / h~");
   const float* top = d_h[nl - 1];
   const bool packed = attn && top && attn_reads_packed_h(attn, top, d_c_ctx);
+  // bf16 weights on both sides: the top LSTM layer leaves h_t as bf16 terms in the attention layer's buffer
+  const bool split16 = attn && top && attn->d_bf16 && layers && layers[0] && layers[0]->bf16 &&
+                       layers[0]->H == attn->H && (((uintptr_t)top & 15u) == 0);
+  // (an fp32 attention layer behind bf16 LSTM layers, or the other way round, re-lays h_t out itself)
+  const bool pack32 = packed && layers && layers[0] && !layers[0]->bf16;
+  float* hand_over = pack32 ? attn->d_hpack
+                            : (split16 ? (float*)(attn->d_bf16 + 4 * (size_t)attn->H * attn->ldp) : nullptr);
   int wrote = 0;
   int rc = zr_lstm_decoder_step_packed(ctx, nl, layers, d_embed, V_in, d_ids_nonneg, d_hprev, d_cprev, d_htild_prev,
-                                       d_mask01, clip_threshold, mb, d_h, d_c, packed ? attn->d_hpack : nullptr, &wrote);
+                                       d_mask01, clip_threshold, mb, d_h, d_c, hand_over, &wrote);
   if (rc) return rc;
   if (!attn)
     return zr_softmax_forward_packed(ctx, d_D, d_b_d, V_out, layers[0]->H, top, nullptr, mb, mode, d_out, nullptr);
   rc = attn_step_impl(ctx, attn, d_batch_info, top, d_mask01, d_htild, d_alignments, d_indices, d_p_t, d_c_ctx,
-                      packed && wrote, packed ? attn->d_htpack : nullptr);
+                      (pack32 || split16) && wrote, packed ? attn->d_htpack : nullptr);
   if (rc) return rc;
   return zr_softmax_forward_packed(ctx, d_D, d_b_d, V_out, attn->H, d_htild, packed ? attn->d_htpack : nullptr, mb, mode,
                                    d_out, nullptr);
@@ -754,8 +761,10 @@ static int attn_step_impl(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, cons
   if (a->d_bf16 && (((uintptr_t)d_h_t & 15u) == 0)) {
     unsigned short* hs = a->d_bf16 + 4 * per;
     const bool two_terms = ctx->bf16_terms != 1;
-    rc = zr_split_pack_x_launch(ctx, d_h_t, H, mb, H, hs, two_terms ? hs + (size_t)H * mb : nullptr);
-    if (rc) return rc;
+    if (!h_packed) {  // (h_packed: the producer of h_t has left the terms there already)
+      rc = zr_split_pack_x_launch(ctx, d_h_t, H, mb, H, hs, two_terms ? hs + (size_t)H * mb : nullptr);
+      if (rc) return rc;
+    }
     h_hi = hs;
     h_lo = two_terms ? hs + (size_t)H * mb : nullptr;
     g.Bhi[0] = h_hi;

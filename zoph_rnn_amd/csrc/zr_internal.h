@@ -180,7 +180,8 @@ struct zr_lstm_weights {
 
 // Pieces of zr_decoder_step (zr_attention.hip): the three public calls with the hand-overs between them kept in the
 // k-interleaved layout.  d_hp_top (zr_lstm_decoder_step): where the top layer's h is also written as [H/4][mb][4];
-// *wrote_hp_top tells whether it was (only the single-launch path does).  h_packed (zr_attn_step): a->d_hpack already
+// *wrote_hp_top tells whether it was (only the single-launch path does).  With bf16 weights d_hp_top instead receives
+// the top layer's h as bf16 terms, k-interleaved by 8: H*mb hi terms, then (two-term mode) H*mb lo terms.  h_packed (zr_attn_step): a->d_hpack already
 // holds that copy of d_h_t; d_htild_pack: h~ is also written k-interleaved there.  d_h_packed (zr_softmax_forward):
 // a k-interleaved copy of d_h, used when the registered matrix allows it.
 int zr_lstm_decoder_step_packed(zr_ctx* ctx, int nl, const zr_lstm_weights* const layers[], const float* d_embed, int V,

@@ -26,6 +26,9 @@ struct LstmUnit {
   const unsigned short* inp_lo[3];  // bf16 weights: inp[] then holds the bf16 "hi" half of the split inputs
                                     // ([H/8][mb][8]) and inp_lo[] the "lo" half
   float* hp;                // optional: h is also written packed as [H/4][mb][4] for the units that consume it
+  unsigned short* hsplit_hi;  // optional: h is also written as bf16 terms, k-interleaved by 8 ([H/8][mb][8]), the layout
+  unsigned short* hsplit_lo;  // products against bf16 weights read (hsplit_lo null: single term); same rounding as
+                              // zr_split_pack_x_kernel
   const int* gather_ids;    // non-null: column n of segment 0 is in[0] + ids[n]*H (embedding gather)
   const float* cprev;
   const int* mask01;
@@ -262,6 +265,12 @@ __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
       U.c[ix] = c;
       U.h[ix] = h;
       if (U.hp) U.hp[((long long)(j >> 2) * L.mb + n) * 4 + (j & 3)] = h;
+      if (U.hsplit_hi) {
+        const __bf16 hb = (__bf16)h;
+        const long long o = ((long long)(j >> 3) * L.mb + n) * 8 + (j & 7);
+        U.hsplit_hi[o] = __builtin_bit_cast(unsigned short, hb);
+        if (U.hsplit_lo) U.hsplit_lo[o] = __builtin_bit_cast(unsigned short, (__bf16)(h - (float)hb));
+      }
       if (U.gates[0]) {
         U.gates[0][ix] = gi;
         U.gates[1][ix] = gf;
@@ -1426,7 +1435,8 @@ int zr_lstm_weights_destroy(zr_ctx* ctx, zr_lstm_weights* w) {
 static int lstm_step_impl(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_in, const int* d_gather_ids, int V,
                           const float* d_hprev, const float* d_cprev, const float* d_htild, const int* d_mask01,
                           float clip_threshold, int mb, float* d_h, float* d_c, float* const d_gates[4],
-                          const unsigned short* const* pre_hi = nullptr, const unsigned short* const* pre_lo = nullptr);
+                          const unsigned short* const* pre_hi = nullptr, const unsigned short* const* pre_lo = nullptr,
+                          unsigned short* out_hi = nullptr, unsigned short* out_lo = nullptr);
 
 int zr_lstm_step(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_in, const float* d_hprev,
                  const float* d_cprev, const float* d_htild, const int* d_mask01, float clip_threshold, int mb,
@@ -1445,11 +1455,13 @@ int zr_lstm_step_embed(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_emb
 
 // d_gather_ids non-null: d_in is the H x V embedding and column b of the input is d_in[:, d_gather_ids[b]].
 // pre_hi / pre_lo (or null; bf16 weights only): segment s's input already split into bf16 terms and k-interleaved by 8
-// (pre_lo[s] null in single-term mode); such a segment is neither gathered nor split here.
+// (pre_lo[s] null in single-term mode); such a segment is neither gathered nor split here.  out_hi / out_lo (or null):
+// h is also written in that form, for the product that reads it next.
 static int lstm_step_impl(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_in, const int* d_gather_ids, int V,
                           const float* d_hprev, const float* d_cprev, const float* d_htild, const int* d_mask01,
                           float clip_threshold, int mb, float* d_h, float* d_c, float* const d_gates[4],
-                          const unsigned short* const* pre_hi, const unsigned short* const* pre_lo) {
+                          const unsigned short* const* pre_hi, const unsigned short* const* pre_lo,
+                          unsigned short* out_hi, unsigned short* out_lo) {
   int rc = zr_bind_device(ctx);
   if (rc) return rc;
   ZR_CHECK_ARG(w != nullptr, "zr_lstm_step: weights are null");
@@ -1496,6 +1508,8 @@ static int lstm_step_impl(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_
   U.mask01 = d_mask01;
   U.h = d_h;
   U.c = d_c;
+  U.hsplit_hi = (ctx->lstm_fused && H % 8 == 0) ? out_hi : nullptr;
+  U.hsplit_lo = U.hsplit_hi ? out_lo : nullptr;
   for (int g = 0; g < 4; ++g) U.gates[g] = d_gates ? d_gates[g] : nullptr;
   U.nseg = nseg;
   U.V = d_gather_ids ? V : 0;
@@ -1658,20 +1672,28 @@ int zr_lstm_decoder_step_packed(zr_ctx* ctx, int nl, const zr_lstm_weights* cons
     if (d_htild) srcs[ns++] = d_htild;
     rc = zr_split_pack_multi_launch(ctx, ns, srcs, d_ids_nonneg, V, H, mb, H, hi, two_terms ? lo : nullptr, (long long)e);
     if (rc) return rc;
-    unsigned short* below_hi = hi + e * (size_t)(nl + 2);
-    unsigned short* below_lo = lo + e * (size_t)(nl + 2);
+    // h_t of a layer leaves its launch in both forms: fp32 for the caller and bf16 terms for the layer above (two
+    // buffers in turn: a launch reads one while it writes the other) or, from the top layer, for the caller's next
+    // product (d_hp_top: hi terms, then H*mb elements further the lo terms)
+    // (the second of the two is the embedding columns' slot, free once layer 0 has run)
+    unsigned short* below_hi[2] = {hi + e * (size_t)(nl + 2), hi};
+    unsigned short* below_lo[2] = {lo + e * (size_t)(nl + 2), lo};
+    unsigned short* top_hi = (unsigned short*)d_hp_top;
+    unsigned short* top_lo = top_hi ? top_hi + e : nullptr;
     for (int l = 0; l < nl; ++l) {
-      const unsigned short* ph[3] = {l == 0 ? hi : below_hi, hi + e * (size_t)(1 + l), hi + e * (size_t)(1 + nl)};
-      const unsigned short* pl[3] = {l == 0 ? lo : below_lo, lo + e * (size_t)(1 + l), lo + e * (size_t)(1 + nl)};
-      if (l > 0) {
-        rc = zr_split_pack_x_launch(ctx, d_h[l - 1], H, mb, H, below_hi, two_terms ? below_lo : nullptr);
-        if (rc) return rc;
-      }
+      const unsigned short* in_hi = l == 0 ? hi : below_hi[(l - 1) & 1];
+      const unsigned short* in_lo = l == 0 ? lo : below_lo[(l - 1) & 1];
+      const unsigned short* ph[3] = {in_hi, hi + e * (size_t)(1 + l), hi + e * (size_t)(1 + nl)};
+      const unsigned short* pl[3] = {in_lo, lo + e * (size_t)(1 + l), lo + e * (size_t)(1 + nl)};
+      const bool last = l == nl - 1;
+      unsigned short* oh = last ? top_hi : below_hi[l & 1];
+      unsigned short* ol = last ? top_lo : below_lo[l & 1];
       rc = lstm_step_impl(ctx, layers[l], l == 0 ? d_embed : d_h[l - 1], l == 0 ? d_ids_nonneg : nullptr, l == 0 ? V : 0,
                           d_hprev[l], d_cprev[l], l == 0 ? d_htild : nullptr, d_mask01, clip_threshold, mb, d_h[l],
-                          d_c[l], nullptr, ph, two_terms ? pl : nullptr);
+                          d_c[l], nullptr, ph, two_terms ? pl : nullptr, oh, two_terms ? ol : nullptr);
       if (rc) return rc;
     }
+    if (wrote_hp_top && top_hi) *wrote_hp_top = 1;
     return ZR_OK;
   }
   for (int l = 0; l < nl; ++l) {
