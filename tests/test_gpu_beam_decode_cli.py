@@ -98,3 +98,58 @@ def test_beam_decode_cli_default_output_is_words(tmp_path):
     assert len(lines) == len(src)
     for ln in lines:
         assert all(w in tgt_vocab[2:] for w in ln.split())  # words, no <START> / <EOF>
+
+
+def test_beam_decode_cli_with_bf16_weight_storage(tmp_path):
+    """--bf16: every streamed matrix (LSTM, attention, output layer) is stored as bf16 on the device and the decode runs
+    through the bf16 decoder step (the step's inputs split into bf16 terms in one launch, every LSTM node leaving its h as
+    bf16 terms for the next product).  The model's matrices are bf16-representable, so the storage is exact and the
+    fp32 oracle on the same matrices is the bar: same words, scores to 1e-4."""
+    from gpu_util import round_bf16
+    g = synth.rng(97, 3)
+    H, L, D, longest, K, beam = 64, 2, 3, 24, 2, 4
+    src_vocab = ["<UNK>"] + mf.make_vocab(79, "s")
+    tgt_vocab = ["<START>", "<EOF>", "<UNK>"] + mf.make_vocab(397, "t")
+    m = _model(g, H, len(src_vocab), len(tgt_vocab), L)
+    rb = lambda a: np.asfortranarray(round_bf16(a))
+    for ly in m["src_layers"] + m["tgt_layers"]:
+        for k in ("M", "Wh", "Q"):
+            if k in ly:
+                ly[k] = [rb(x) for x in ly[k]]
+    for k in ("W_a", "W_p", "W_c1", "W_c2"):
+        m["attn"][k] = rb(m["attn"][k])
+    m["D_soft"] = rb(m["D_soft"])
+    model = tmp_path / "model.nn"
+    with open(model, "w") as f:
+        mf.write_header(f, L, H, tgt_vocab, src_vocab, True, True)
+        _write_ih(f, m["src_layers"][0], m["src_embed"])
+        for ly in m["src_layers"][1:]:
+            _write_hh(f, ly)
+        _write_ih(f, m["tgt_layers"][0], m["tgt_embed"], None)
+        for i, ly in enumerate(m["tgt_layers"][1:]):
+            _write_hh(f, ly, m["attn"] if i == L - 2 else None)
+        _write_matrix(f, m["D_soft"])
+        _write_matrix(f, m["b_soft"].reshape(-1, 1))
+    lens = [5, 7, 5, 4, 7]
+    src = [mf.random_sentences(g, src_vocab, 1, n, n)[0] for n in lens]
+    sp, out = tmp_path / "src.txt", tmp_path / "out.txt"
+    sp.write_text("".join(" ".join(s) + "\n" for s in src))
+    r = mf.run_program("beam_decode", ["--bf16", "--beam", beam, "--batch", 3, "--longest-sent", longest,
+                                       "--attention-width", D, "--num-best", K, "--print-score", "--ids", model, sp, out])
+    assert r.returncode == 0, r.stderr[-2000:]
+    got = _parse_blocks(out.read_text())
+    assert len(got) == len(src)
+    smap = {w: i for i, w in enumerate(src_vocab)}
+    for s, words in enumerate(src):
+        ids = np.array([smap.get(w, 0) for w in words][::-1], np.int32)
+        S = len(ids)
+        steps = min(int(1.5 * S), longest - 2)
+        _, hyps, gap = _oracle_decode(m, ids, S, S, beam, steps, D, 0.0)
+        assert gap > 5e-5, "candidate scores nearly tie (gap %.2e): pick another seed" % gap
+        keep = [(w, sc) for (w, sc) in hyps if len(w) / S > 0.5]
+        keep.sort(key=lambda t: -t[1])
+        want = keep[:K]
+        assert len(got[s]) == len(want), (s, len(got[s]), len(want))
+        for (gw, gs), (ww, ws) in zip(got[s], want):
+            assert gw == list(ww), (s, gw, list(ww))
+            assert gs == pytest.approx(ws, rel=1e-4, abs=2e-4)
