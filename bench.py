@@ -80,9 +80,10 @@ def bench_encoder(ctx, steps, warmup, H=1000, mb=128, T=50, V=50000, L=4):
         ctx.lstm_stack_forward(ws, d_embed, V, d_nn, d_m, T, mb, [z] * L, [z] * L, h_all, c_all)
 
     wall_ms, ev_ms = time_region(ctx, step, steps, warmup)
-    # one lstm_sweep_kernel launch per step (preceded by a sub-microsecond counter-clearing fill)
+    # one lstm_sweep_kernel launch per step, between a counter-clearing fill in front of it and the check behind it that
+    # overwrites the outputs of a sweep that gave up a wait (4-5 us each, inside the timed region)
     flops_per_step = 2.0 * 4 * H * mb * (2 * H) * L * T
-    res = {"wall_ms": wall_ms, "event_ms": ev_ms, "tokens_per_step": mb * T, "launches_per_step": 1,
+    res = {"wall_ms": wall_ms, "event_ms": ev_ms, "tokens_per_step": mb * T, "launches_per_step": 3,
            "flops_per_step": flops_per_step, "avg_launch_us": ev_ms * 1e3 / steps,
            "flops_per_launch": flops_per_step}
     # keep references alive until here
