@@ -500,6 +500,26 @@ int zr_softmax_backward_accumulate(zr_ctx* ctx, const float* d_D, const float* d
 int zr_sgd_update(zr_ctx* ctx, float* d_W, const float* d_grad, long long n, float scale, float norm_clip,
                   float learning_rate);
 
+/* The reference's three ways of clipping a gradient before the update (src/main.cu:495-511): per matrix
+ * (--matrix-clip-gradients, norm_clip_GPU_v2, src/custom_kernels.h:1064-1078), over the whole model
+ * (--whole-clip-gradients, norm_clip_GPU_v2_p1 / _p2, :1083-1135) and per element (--ind-clip-gradients,
+ * clip_mat_kernel, :2220-2231). */
+#define ZR_CLIP_NONE 0
+#define ZR_CLIP_MATRIX_NORM 1
+#define ZR_CLIP_WHOLE_NORM 2
+#define ZR_CLIP_ELEMENT 3
+/* calculate_global_norm (src/Hidden_To_Hidden_Layer.hpp:241-335, src/model.hpp:1850-1892): adds the squared L2 norm of
+ * scale * grad to the double at d_sumsq (device memory; reset != 0 overwrites it instead, n == 0 with reset clears
+ * it).  The sum stays on the device: no copy to the host, no wait. */
+int zr_grad_sumsq_accumulate(zr_ctx* ctx, const float* d_grad, long long n, float scale, double* d_sumsq, int reset);
+/* W += learning_rate * clip(scale * grad) with clip chosen by clip_mode: ZR_CLIP_NONE; ZR_CLIP_MATRIX_NORM (what
+ * zr_sgd_update does with norm_clip = threshold); ZR_CLIP_WHOLE_NORM: shrunk by threshold / sqrt(*d_sumsq) when the
+ * norm accumulated over every gradient of the model exceeds threshold (update_global_params,
+ * src/Hidden_To_Hidden_Layer.hpp:353-382); ZR_CLIP_ELEMENT: every element of scale * grad clamped to +-threshold
+ * (src/Hidden_To_Hidden_Layer.hpp:503-517).  d_sumsq is read in ZR_CLIP_WHOLE_NORM only. */
+int zr_sgd_update_clipped(zr_ctx* ctx, float* d_W, const float* d_grad, long long n, float scale, int clip_mode,
+                          float threshold, const double* d_sumsq, float learning_rate);
+
 #ifdef __cplusplus
 }
 #endif

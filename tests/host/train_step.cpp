@@ -1,5 +1,5 @@
 // Test driver: SGD steps of model_trainer (zoph_rnn_amd/host/zoph_model.h) on the minibatches of an integerized file.
-//   train_step [--sequence] [--node-level] [--abandon-sweeps] [--attention-D=N] [--dropout=KEEP_RATE] [--dropout-seed=S]
+//   train_step [--sequence] [--node-level] [--abandon-sweeps] [--whole-clip | --ind-clip=T] [--attention-D=N] [--dropout=KEEP_RATE] [--dropout-seed=S]
 //              model.nn data.int minibatch longest_sent learning_rate norm_clip steps
 // Every step trains on the next minibatch of the file (wrapping around) and prints "loss <step> <log-likelihood>";
 // the updated model is written to <model.nn>.trained as a complete model file.  --node-level: the step is
@@ -7,6 +7,8 @@
 // reference's node-by-node order, instead of model_trainer's stack-level calls.  --abandon-sweeps: the forward pass is
 // forced onto the single-launch sweep with a wait limit of one poll, so its workgroups give up (and leave the kernel
 // normally); model_trainer must notice and repeat the forward pass; prints "abandoned <count>" at the end.
+// --whole-clip: norm_clip bounds the L2 norm of all gradients together (prints "global_norm <step> <norm>");
+// --ind-clip=THRESHOLD: every gradient element is clamped to +-THRESHOLD instead (norm_clip is then unused).
 // Models with attention (and feed-input) and dropout train through the node-level path only; --attention-D sets the
 // window half-width (the model file does not store it), --dropout the probability of keeping a value.
 #include <cstdio>
@@ -36,11 +38,17 @@ int main(int argc, char** argv) {
       node_level = true;
     else if (std::string(argv[i]) == "--abandon-sweeps")
       abandon = true;
+    else if (a == "--whole-clip")  // --whole-clip-gradients of the reference: norm_clip bounds the whole model's norm
+      BZ_CUDA::global_clip_flag = true;
+    else if (a.rfind("--ind-clip=", 0) == 0) {  // --ind-clip-gradients: every element clamped to +-threshold
+      BZ_CUDA::individual_grad_clip = true;
+      BZ_CUDA::ind_norm_clip_thres = (float)std::atof(a.c_str() + 11);
+    }
     else
       pos.push_back(argv[i]);
   }
   if (pos.size() != 7) {
-    std::fprintf(stderr, "usage: %s [--sequence] [--node-level] model.nn data.int minibatch longest_sent learning_rate norm_clip steps\n", argv[0]);
+    std::fprintf(stderr, "usage: %s [--sequence] [--node-level] [--whole-clip | --ind-clip=THRESHOLD] model.nn data.int minibatch longest_sent learning_rate norm_clip steps\n", argv[0]);
     return 2;
   }
   const int minibatch = std::atoi(pos[2].c_str()), longest = std::atoi(pos[3].c_str()), steps = std::atoi(pos[6].c_str());
@@ -57,7 +65,7 @@ int main(int argc, char** argv) {
   forward_model<precision> m;
   m.params.learning_rate = lr;
   m.params.norm_clip = clip;
-  m.params.clip_gradient = clip > 0;
+  m.params.clip_gradient = clip > 0 && !BZ_CUDA::global_clip_flag && !BZ_CUDA::individual_grad_clip;
   m.initModel(gpu, info, minibatch, longest, attention_D, dropout_rate);
   m.load_weights(model);
   model_trainer<precision>* trainer = node_level ? nullptr : new model_trainer<precision>(m);
@@ -90,6 +98,7 @@ int main(int argc, char** argv) {
       loss = trainer->train_minibatch(reader, lr, clip);
     }
     std::cout << "loss " << s << " " << loss << "\n";
+    if (BZ_CUDA::global_clip_flag) std::cout << "global_norm " << s << " " << BZ_CUDA::read_global_norm(gpu.ctx) << "\n";
   }
   if (trainer) std::cout << "abandoned " << trainer->abandoned_sweeps << "\n";
   devSynchAll(gpu.ctx);

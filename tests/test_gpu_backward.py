@@ -152,6 +152,73 @@ def test_sgd_update(ctx, n, clip):
         assert np.sqrt((((dW.get() - W) / lr) ** 2).sum()) == pytest.approx(clip, rel=1e-4)
 
 
+@pytest.mark.parametrize("threshold", [0.5, 1e6])
+def test_sgd_update_whole_model_clip(ctx, threshold):
+    """--whole-clip-gradients (norm_clip_GPU_v2_p1 / _p2, src/custom_kernels.h:1083-1135, src/model.hpp:1850-1892): the
+    squared norms of all scaled gradients are summed, and every gradient is shrunk by threshold / that norm when it is
+    larger.  Three gradients of different sizes (one not a multiple of four, one empty), checked against numpy in
+    float64: the accumulated sum, then each update."""
+    from zoph_rnn_amd import capi
+    g = synth.rng(114, 3)
+    sizes = [70001, 37, 0, 4096]
+    Ws = [U(g, (n,), -1, 1) for n in sizes]
+    Gs = [U(g, (n,), -3, 3) for n in sizes]
+    scale, lr = 1.0 / 16, 0.3
+    d_ss = ctx.array(np.array([123.0]))  # stale content: the first call resets
+    dGs = [ctx.array(G) if G.size else None for G in Gs]
+    for i, (G, dG) in enumerate(zip(Gs, dGs)):
+        ctx.grad_sumsq_accumulate(dG, G.size, scale, d_ss, reset=(i == 0))
+    ctx.sync()
+    want_ss = sum(((G.astype(np.float64) * scale) ** 2).sum() for G in Gs)
+    assert d_ss.get()[0] == pytest.approx(want_ss, rel=1e-12)
+    norm = np.sqrt(want_ss)
+    coef = threshold / norm if norm > threshold else 1.0
+    assert (coef < 1.0) == (threshold < 1.0)
+    for W, G, dG in zip(Ws, Gs, dGs):
+        if not G.size:
+            continue
+        dW = ctx.array(W)
+        ctx.sgd_update_clipped(dW, dG, G.size, scale, capi.ZR_CLIP_WHOLE_NORM, threshold, d_ss, lr)
+        ctx.sync()
+        assert np.allclose(dW.get(), W + lr * coef * scale * G.astype(np.float64), rtol=1e-5, atol=1e-6)
+    # reset with nothing to add clears the accumulator
+    ctx.grad_sumsq_accumulate(None, 0, 1.0, d_ss, reset=True)
+    ctx.sync()
+    assert d_ss.get()[0] == 0.0
+
+
+def test_sgd_update_element_clip(ctx):
+    """--ind-clip-gradients (clip_mat_kernel, src/custom_kernels.h:2220-2231): every element of the scaled gradient is
+    clamped to +-threshold, whatever the norm.  Elements on both sides of both bounds, and exactly on them."""
+    from zoph_rnn_amd import capi
+    g = synth.rng(115, 1)
+    n, thr, scale, lr = 5003, 0.1, 0.25, 0.7
+    W, G = U(g, (n,), -1, 1), U(g, (n,), -1, 1)
+    G[:4] = np.array([thr, -thr, 2 * thr, -2 * thr], np.float32) / scale
+    dW = ctx.array(W)
+    ctx.sgd_update_clipped(dW, ctx.array(G), n, scale, capi.ZR_CLIP_ELEMENT, thr, None, lr)
+    ctx.sync()
+    gs = np.clip(G * np.float32(scale), -np.float32(thr), np.float32(thr))
+    assert (np.abs(G * scale) > thr).sum() > n // 4 and (np.abs(G * scale) < thr).sum() > n // 4
+    assert np.allclose(dW.get(), W + np.float32(lr) * gs, rtol=1e-6, atol=1e-7)
+    # mode 0: no clipping at all
+    dW = ctx.array(W)
+    ctx.sgd_update_clipped(dW, ctx.array(G), n, scale, capi.ZR_CLIP_NONE, 0.0, None, lr)
+    ctx.sync()
+    assert np.allclose(dW.get(), W + lr * scale * G.astype(np.float64), rtol=1e-5, atol=1e-6)
+
+
+def test_sgd_update_clipped_rejects_bad_arguments(ctx):
+    from zoph_rnn_amd import capi
+    dW, dG = ctx.zeros((8,)), ctx.zeros((8,))
+    with pytest.raises(RuntimeError):
+        ctx.sgd_update_clipped(dW, dG, 8, 1.0, 7, 1.0, None, 0.1)
+    with pytest.raises(RuntimeError):  # whole-model clipping needs the accumulated sum
+        ctx.sgd_update_clipped(dW, dG, 8, 1.0, capi.ZR_CLIP_WHOLE_NORM, 1.0, None, 0.1)
+    with pytest.raises(RuntimeError):
+        ctx.sgd_update_clipped(dW, dG, 8, 1.0, capi.ZR_CLIP_ELEMENT, 0.0, None, 0.1)
+
+
 def test_language_model_training_step_gradients(ctx):
     """benchmark configuration 1 shape (1-layer LM, H=100, minibatch 8, T=20, V=10000): the full gradient of the summed
     log-likelihood -- output layer, LSTM matrices and biases, embedding -- from one forward/backward pass."""

@@ -67,16 +67,22 @@ def _read_model(path, n_head, L, H, Vs, Vt, lm):
     return m
 
 
-def _clip_update(W, grad, mb, clip, lr, clipped):
+def _clip_update(W, grad, mb, clip, lr, clipped, mode="matrix", whole_norm=None):
+    """mode "matrix": clip bounds this gradient's own norm; "whole": it bounds whole_norm, the norm of all gradients of
+    the model together; "element": every element is clamped to +-clip."""
     g = np.asarray(grad, np.float64) / mb
-    norm = np.sqrt((g * g).sum())
-    clipped.append(bool(norm > clip))
-    if norm > clip:
-        g = g * (clip / norm)
+    if mode == "element":
+        clipped.append(bool((np.abs(g) > clip).any()))
+        g = np.clip(g, -clip, clip)
+    else:
+        norm = np.sqrt((g * g).sum()) if mode == "matrix" else whole_norm
+        clipped.append(bool(norm > clip))
+        if norm > clip:
+            g = g * (clip / norm)
     return (np.asarray(W, np.float64) + lr * g).astype(np.float32)
 
 
-def _oracle_step(m, chunk, mb, lm, lr, clip, clipped):
+def _oracle_step(m, chunk, mb, lm, lr, clip, clipped, mode="matrix", norms=None):
     """One training step on the oracle; updates m in place and returns the log-likelihood before the update."""
     L = len(m["tgt_layers"])
     if lm:
@@ -107,7 +113,16 @@ def _oracle_step(m, chunk, mb, lm, lr, clip, clipped):
         zero_top = [np.zeros((H, mb), np.float32) for _ in range(S)]
         g_s, dW_s, _, _ = o.lstm_stack_backward(m["emb_s"], m["src_layers"], nn_s, m_s, zero_top, err_hT=eh0, err_cT=ec0)
         sides.append(("s", "src_layers", g_s, dW_s))
-    up = lambda W, g: _clip_update(W, g, mb, clip, lr, clipped)
+    whole = None
+    if mode == "whole":  # src/model.hpp:1850-1892: every gradient of the model, scaled by 1 / minibatch
+        ss = (np.asarray(dD, np.float64) ** 2).sum() + (np.asarray(dbd, np.float64) ** 2).sum()
+        for _, _, grads, dW in sides:
+            ss += (np.asarray(dW, np.float64) ** 2).sum()
+            for gr in grads:
+                ss += sum((np.asarray(gr[k][g], np.float64) ** 2).sum() for k in ("dM", "dWh", "db") for g in range(4))
+        whole = np.sqrt(ss) / mb
+        norms.append(whole)
+    up = lambda W, g: _clip_update(W, g, mb, clip, lr, clipped, mode, whole)
     m["D"], m["b_d"] = up(m["D"], dD), up(m["b_d"], dbd)
     for s, key, grads, dW in sides:
         m["emb_" + s] = up(m["emb_" + s], dW)
@@ -135,7 +150,7 @@ def test_abandoned_forward_sweep_is_repeated_before_the_update(tmp_path):
 @pytest.mark.parametrize("node_level", [False, True])
 @pytest.mark.parametrize("lm,L,H,mb,steps,clip", [(True, 2, 32, 4, 1, 0.4), (False, 2, 48, 3, 1, 0.25),
                                                   (False, 1, 32, 5, 3, 5.0), (True, 3, 64, 8, 2, 1.0)])
-def test_train_steps_match_oracle(tmp_path, lm, L, H, mb, steps, clip, node_level, abandon=False):
+def test_train_steps_match_oracle(tmp_path, lm, L, H, mb, steps, clip, node_level, abandon=False, mode="matrix"):
     """node_level: the same steps through the layer objects' back_prop_GPU / update_weights members
     (forward_model::compute_gradients) instead of model_trainer."""
     if not os.path.exists(DRIVER):
@@ -170,8 +185,9 @@ def test_train_steps_match_oracle(tmp_path, lm, L, H, mb, steps, clip, node_leve
             for k in range(4):
                 f.write(" ".join(str(v) for v in r[k]) + "\n")
     args = (["--sequence"] if lm else []) + (["--node-level"] if node_level else []) + \
-        (["--abandon-sweeps"] if abandon else []) + [str(model), str(data_path), str(mb), str(longest), str(lr), str(clip),
-                                             str(steps)]
+        (["--abandon-sweeps"] if abandon else []) + (["--whole-clip"] if mode == "whole" else []) + \
+        (["--ind-clip=%r" % clip] if mode == "element" else []) + \
+        [str(model), str(data_path), str(mb), str(longest), str(lr), str(clip), str(steps)]
     r = subprocess.run([DRIVER] + args, capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, r.stderr[-2000:]
     got_loss = [float(ln.split()[2]) for ln in r.stdout.splitlines() if ln.startswith("loss")]
@@ -179,14 +195,18 @@ def test_train_steps_match_oracle(tmp_path, lm, L, H, mb, steps, clip, node_leve
         n_abandoned = [int(ln.split()[1]) for ln in r.stdout.splitlines() if ln.startswith("abandoned")]
         assert n_abandoned == [steps], "every step's forward sweep should have been abandoned and repeated"
     chunks = [data[i:i + mb] for i in range(0, len(data), mb)]
-    clipped, want_loss = [], []
+    clipped, want_loss, want_norms = [], [], []
     for s in range(steps):
-        want_loss.append(_oracle_step(m, chunks[s % len(chunks)], mb, lm, lr, clip, clipped))
+        want_loss.append(_oracle_step(m, chunks[s % len(chunks)], mb, lm, lr, clip, clipped, mode, want_norms))
+    if mode == "whole":
+        got_norms = [float(ln.split()[2]) for ln in r.stdout.splitlines() if ln.startswith("global_norm")]
+        assert got_norms == pytest.approx(want_norms, rel=1e-4)
     assert len(got_loss) == steps
     for a, b in zip(got_loss, want_loss):
         assert a == pytest.approx(b, rel=1e-4, abs=1e-4)
     if clip < 5.0:
-        assert any(clipped) and not all(clipped), "pick norm_clip so that both branches of the clipping run"
+        assert any(clipped) and not all(clipped), "pick the threshold so that both branches of the clipping run: %s" % (
+            want_norms if mode == "whole" else clipped)
     new = _read_model(str(model) + ".trained", n_head, L, H, Vs, Vt, lm)
     _compare("D", new["D"], m["D"], orig["D"])
     _compare("b_d", new["b_d"], m["b_d"], orig["b_d"])
@@ -197,6 +217,17 @@ def test_train_steps_match_oracle(tmp_path, lm, L, H, mb, steps, clip, node_leve
                 for gate in range(4):
                     _compare("%s layer %d %s[%d]" % (key, l, k, gate), new[key][l][k][gate], m[key][l][k][gate],
                              orig[key][l][k][gate])
+
+
+@pytest.mark.parametrize("node_level", [False, True])
+@pytest.mark.parametrize("mode,lm,L,H,mb,steps,clip", [("whole", False, 2, 48, 3, 3, 3.5), ("whole", True, 2, 32, 4, 2, 1e3),
+                                                       ("element", False, 2, 48, 3, 2, 0.02),
+                                                       ("element", True, 1, 32, 5, 2, 0.05)])
+def test_train_steps_with_whole_model_and_element_clipping(tmp_path, mode, lm, L, H, mb, steps, clip, node_level):
+    """The reference's other two clipping modes (src/main.cu:495-511) through both training paths: norm_clip bounding
+    the norm of ALL gradients together (the first case clips in some steps and not in others, the second never), and a
+    clamp of every gradient element.  In whole-model mode the norm the driver reports is compared too."""
+    test_train_steps_match_oracle(tmp_path, lm, L, H, mb, steps, clip, node_level, mode=mode)
 
 
 def test_repeated_steps_on_one_minibatch_raise_its_likelihood(tmp_path):

@@ -310,24 +310,49 @@ __global__ void __launch_bounds__(1024) sumsq_partial_kernel(const float* __rest
   if (threadIdx.x == 0) partial[blockIdx.x] = s[0];
 }
 
-// W += lr * coef * scale * g, with coef = norm_clip / ||scale * g|| when that norm exceeds norm_clip (> 0), else 1
+// second stage of the whole-model norm (norm_clip_GPU_v2_p1, src/custom_kernels.h:1083-1099): the partial sums added in a
+// fixed order, times scale^2, into (or, with reset, over) the caller's accumulator
+__global__ void sumsq_accumulate_kernel(const double* __restrict__ partial, int n_partial, float scale,
+                                        double* __restrict__ sumsq, int reset) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  double ss = 0.0;
+  for (int i = 0; i < n_partial; ++i) ss += partial[i];
+  ss *= (double)scale * (double)scale;
+  *sumsq = reset ? ss : *sumsq + ss;
+}
+
+// W += lr * clip(scale * g).  mode ZR_CLIP_MATRIX_NORM: the gradient is shrunk by threshold / ||scale * g|| when that norm
+// (from `partial`) exceeds threshold; ZR_CLIP_WHOLE_NORM: the same with the norm sqrt(*sumsq) the caller accumulated
+// over every gradient of the model; ZR_CLIP_ELEMENT: every element of scale * g is clamped to +-threshold.
 __global__ void __launch_bounds__(256) sgd_apply_kernel(float* __restrict__ W, const float* __restrict__ g, long long n,
-                                                        float scale, float norm_clip, float lr,
-                                                        const double* __restrict__ partial, int n_partial) {
+                                                        float scale, int mode, float threshold, float lr,
+                                                        const double* __restrict__ partial, int n_partial,
+                                                        const double* __restrict__ sumsq) {
   __shared__ float coef_s;
   if (threadIdx.x == 0) {
     float coef = 1.0f;
-    if (norm_clip > 0.0f) {
+    if (mode == ZR_CLIP_MATRIX_NORM) {
       double ss = 0.0;
       for (int i = 0; i < n_partial; ++i) ss += partial[i];
       const float norm = (float)sqrt(ss) * fabsf(scale);
-      if (norm > norm_clip) coef = norm_clip / norm;
+      if (norm > threshold) coef = threshold / norm;
+    } else if (mode == ZR_CLIP_WHOLE_NORM) {
+      const float norm = (float)sqrt(*sumsq);
+      if (norm > threshold) coef = threshold / norm;
     }
     coef_s = coef;
   }
   __syncthreads();
+  const long long first = (long long)blockIdx.x * 256 + threadIdx.x, stride = (long long)gridDim.x * 256;
+  if (mode == ZR_CLIP_ELEMENT) {
+    for (long long i = first; i < n; i += stride) {
+      const float x = scale * g[i];
+      W[i] += lr * fminf(fmaxf(x, -threshold), threshold);
+    }
+    return;
+  }
   const float f = lr * coef_s * scale;
-  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) W[i] += f * g[i];
+  for (long long i = first; i < n; i += stride) W[i] += f * g[i];
 }
 
 
@@ -1153,25 +1178,52 @@ int zr_softmax_backward_accumulate(zr_ctx* ctx, const float* d_D, const float* d
   return softmax_backward(ctx, d_D, d_b_d, V, H, d_h, n, d_target, d_mask01, d_prob_scratch, d_err_h, d_dD, d_db, 1);
 }
 
-int zr_sgd_update(zr_ctx* ctx, float* d_W, const float* d_grad, long long n, float scale, float norm_clip,
-                  float learning_rate) {
+int zr_grad_sumsq_accumulate(zr_ctx* ctx, const float* d_grad, long long n, float scale, double* d_sumsq, int reset) {
   int rc = zr_bind_device(ctx);
   if (rc) return rc;
-  ZR_CHECK_ARG(n >= 0 && (n == 0 || (d_W && d_grad)), "zr_sgd_update: null pointer or n = %lld", n);
+  ZR_CHECK_ARG(n >= 0 && d_sumsq && (n == 0 || d_grad), "zr_grad_sumsq_accumulate: null pointer or n = %lld", n);
+  const int n_partial = n > 0 ? 256 : 0;
+  void* scratch = nullptr;
+  rc = zr_ctx_scratch(ctx, 1, sizeof(double) * 256, &scratch);
+  if (rc) return rc;
+  if (n > 0) {
+    sumsq_partial_kernel<<<n_partial, 1024, 0, ctx->stream>>>(d_grad, n, aligned16(d_grad) ? 1 : 0, (double*)scratch);
+    ZR_LAUNCH_CHECK("sumsq_partial_kernel");
+  }
+  sumsq_accumulate_kernel<<<1, 64, 0, ctx->stream>>>((const double*)scratch, n_partial, scale, d_sumsq, reset ? 1 : 0);
+  ZR_LAUNCH_CHECK("sumsq_accumulate_kernel");
+  return ZR_OK;
+}
+
+int zr_sgd_update_clipped(zr_ctx* ctx, float* d_W, const float* d_grad, long long n, float scale, int clip_mode,
+                          float threshold, const double* d_sumsq, float learning_rate) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(n >= 0 && (n == 0 || (d_W && d_grad)), "zr_sgd_update_clipped: null pointer or n = %lld", n);
+  ZR_CHECK_ARG(clip_mode >= ZR_CLIP_NONE && clip_mode <= ZR_CLIP_ELEMENT, "zr_sgd_update_clipped: clip_mode = %d",
+               clip_mode);
+  ZR_CHECK_ARG(clip_mode == ZR_CLIP_NONE || threshold > 0.0f, "zr_sgd_update_clipped: threshold = %g", (double)threshold);
+  ZR_CHECK_ARG(clip_mode != ZR_CLIP_WHOLE_NORM || d_sumsq, "zr_sgd_update_clipped: whole-model clipping without d_sumsq");
   if (n == 0) return ZR_OK;
   const int n_partial = 256;
   void* scratch = nullptr;
   rc = zr_ctx_scratch(ctx, 1, sizeof(double) * n_partial, &scratch);
   if (rc) return rc;
-  if (norm_clip > 0.0f) {
+  if (clip_mode == ZR_CLIP_MATRIX_NORM) {
     sumsq_partial_kernel<<<n_partial, 1024, 0, ctx->stream>>>(d_grad, n, aligned16(d_grad) ? 1 : 0, (double*)scratch);
     ZR_LAUNCH_CHECK("sumsq_partial_kernel");
   }
   const long long blocks = (n + 255) / 256;
   sgd_apply_kernel<<<(unsigned)(blocks < 2048 ? blocks : 2048), 256, 0, ctx->stream>>>(
-      d_W, d_grad, n, scale, norm_clip, learning_rate, (const double*)scratch, n_partial);
+      d_W, d_grad, n, scale, clip_mode, threshold, learning_rate, (const double*)scratch, n_partial, d_sumsq);
   ZR_LAUNCH_CHECK("sgd_apply_kernel");
   return ZR_OK;
+}
+
+int zr_sgd_update(zr_ctx* ctx, float* d_W, const float* d_grad, long long n, float scale, float norm_clip,
+                  float learning_rate) {
+  return zr_sgd_update_clipped(ctx, d_W, d_grad, n, scale, norm_clip > 0.0f ? ZR_CLIP_MATRIX_NORM : ZR_CLIP_NONE,
+                               norm_clip, nullptr, learning_rate);
 }
 
 }  // extern "C"

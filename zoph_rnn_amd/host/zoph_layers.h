@@ -27,6 +27,7 @@
 #ifndef ZOPH_LAYERS_H
 #define ZOPH_LAYERS_H
 
+#include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <fstream>
@@ -35,6 +36,7 @@
 #include <random>
 #include <sstream>
 #include <string>
+#include <utility>
 #include <vector>
 
 #include "../../include/zoph_rnn.h"
@@ -63,6 +65,49 @@ inline void refuse_backward_with_clip_cell(const char* who) {
                  "cannot run with BZ_CUDA::clip_cell set\n", who);
     std::exit(EXIT_FAILURE);
   }
+}
+// The three ways of clipping gradients (src/BZ_CUDA_UTIL.h:101-118), exclusive as src/main.cu:495-511 sets them: per
+// matrix (neither flag: the layers' clip_gradients / norm_clip), over the whole model (global_clip_flag, threshold =
+// the layers' norm_clip) and per element (individual_grad_clip, threshold = ind_norm_clip_thres).
+inline bool global_clip_flag = false;
+inline precision global_norm = 0;  // host copy of the last whole-model norm, fetched by read_global_norm only
+inline bool individual_grad_clip = false;
+inline precision ind_norm_clip_thres = 0.1f;
+// The whole-model sum of squares lives in device memory, one double per context: the updates read it there, so the
+// step needs no copy to the host and no wait (the reference copies every matrix's norm back, custom_kernels.h:1088).
+inline std::vector<std::pair<zr_ctx*, double*>> global_sumsq_slots;
+inline double* global_sumsq(zr_ctx* ctx) {
+  for (auto& s : global_sumsq_slots)
+    if (s.first == ctx) return s.second;
+  double* p = nullptr;
+  ZOPH_CALL(zr_malloc(ctx, sizeof(double), (void**)&p));
+  ZOPH_CALL(zr_memset_zero(ctx, p, sizeof(double)));
+  global_sumsq_slots.emplace_back(ctx, p);
+  return p;
+}
+inline void reset_global_norm(zr_ctx* ctx) {  // BZ_CUDA::global_norm = 0 (src/model.hpp:1852)
+  ZOPH_CALL(zr_grad_sumsq_accumulate(ctx, nullptr, 0, 1.0f, global_sumsq(ctx), 1));
+}
+inline void add_to_global_norm(zr_ctx* ctx, const float* grad, long long n, float scale) {  // norm_clip_GPU_v2_p1
+  ZOPH_CALL(zr_grad_sumsq_accumulate(ctx, grad, n, scale, global_sumsq(ctx), 0));
+}
+inline precision read_global_norm(zr_ctx* ctx) {  // waits for the stream (src/model.hpp:1892 takes the root on the host)
+  double ss = 0;
+  ZOPH_CALL(zr_d2h(ctx, &ss, global_sumsq(ctx), sizeof(double)));
+  global_norm = (precision)std::sqrt(ss);
+  return global_norm;
+}
+// One gradient's share of update_weights / update_global_params under the mode in force.  matrix_clip: the per-matrix
+// threshold, 0 for none; whole_threshold: the layer's norm_clip.
+inline void apply_update(zr_ctx* ctx, float* W, const float* grad, long long n, float scale, float matrix_clip,
+                         float whole_threshold, float learning_rate) {
+  if (individual_grad_clip)
+    ZOPH_CALL(zr_sgd_update_clipped(ctx, W, grad, n, scale, ZR_CLIP_ELEMENT, ind_norm_clip_thres, nullptr, learning_rate));
+  else if (global_clip_flag)
+    ZOPH_CALL(zr_sgd_update_clipped(ctx, W, grad, n, scale, ZR_CLIP_WHOLE_NORM, whole_threshold, global_sumsq(ctx),
+                                    learning_rate));
+  else
+    ZOPH_CALL(zr_sgd_update(ctx, W, grad, n, scale, matrix_clip, learning_rate));
 }
 inline precision lower = -0.08f;
 inline precision upper = 0.08f;
@@ -394,18 +439,27 @@ class attention_layer {  // src/attention_layer.h:14-143
     for (dType* e : h_total_hs_error) ZOPH_CALL(zr_memset_zero(ctx, e, n * sizeof(dType)));
     transfer_done = false;
   }
-  // scale_gradients, norm_clip_GPU_v2 per matrix, update_params (src/attention_layer.hpp:303-420); then the snapshots
-  // the forward kernels read are rebuilt
+  // norm_p1 (src/attention_layer.hpp): this layer's share of the whole-model gradient norm
+  void calculate_global_norm() {
+    zr_ctx* ctx = layer_info.ctx;
+    const float scale = 1.0f / (float)minibatch_size;
+    const long long hh = (long long)LSTM_size * LSTM_size;
+    for (const dType* g : {d_W_a_grad, d_W_p_grad, d_W_c_p1_grad, d_W_c_p2_grad}) BZ_CUDA::add_to_global_norm(ctx, g, hh, scale);
+    for (const dType* g : {d_v_p_grad, d_output_bias_grad}) BZ_CUDA::add_to_global_norm(ctx, g, LSTM_size, scale);
+  }
+  void update_global_params() { update_weights(); }  // norm_p2 + update_params
+  // scale_gradients, the clipping mode in force (norm_clip_GPU_v2 per matrix unless BZ_CUDA says otherwise),
+  // update_params (src/attention_layer.hpp:303-420); then the snapshots the forward kernels read are rebuilt
   void update_weights() {
     zr_ctx* ctx = layer_info.ctx;
     const float scale = 1.0f / (float)minibatch_size, clip = clip_gradients ? (float)norm_clip : 0.0f;
     const long long hh = (long long)LSTM_size * LSTM_size;
-    ZOPH_CALL(zr_sgd_update(ctx, d_W_a, d_W_a_grad, hh, scale, clip, learning_rate));
-    ZOPH_CALL(zr_sgd_update(ctx, d_W_p, d_W_p_grad, hh, scale, clip, learning_rate));
-    ZOPH_CALL(zr_sgd_update(ctx, d_v_p, d_v_p_grad, LSTM_size, scale, clip, learning_rate));
-    ZOPH_CALL(zr_sgd_update(ctx, d_output_bias, d_output_bias_grad, LSTM_size, scale, clip, learning_rate));
-    ZOPH_CALL(zr_sgd_update(ctx, d_W_c_p1, d_W_c_p1_grad, hh, scale, clip, learning_rate));
-    ZOPH_CALL(zr_sgd_update(ctx, d_W_c_p2, d_W_c_p2_grad, hh, scale, clip, learning_rate));
+    BZ_CUDA::apply_update(ctx, d_W_a, d_W_a_grad, hh, scale, clip, (float)norm_clip, learning_rate);
+    BZ_CUDA::apply_update(ctx, d_W_p, d_W_p_grad, hh, scale, clip, (float)norm_clip, learning_rate);
+    BZ_CUDA::apply_update(ctx, d_v_p, d_v_p_grad, LSTM_size, scale, clip, (float)norm_clip, learning_rate);
+    BZ_CUDA::apply_update(ctx, d_output_bias, d_output_bias_grad, LSTM_size, scale, clip, (float)norm_clip, learning_rate);
+    BZ_CUDA::apply_update(ctx, d_W_c_p1, d_W_c_p1_grad, hh, scale, clip, (float)norm_clip, learning_rate);
+    BZ_CUDA::apply_update(ctx, d_W_c_p2, d_W_c_p2_grad, hh, scale, clip, (float)norm_clip, learning_rate);
     if (BZ_CUDA::bf16_weights)
       ZOPH_CALL(zr_attn_use_bf16_weights(ctx, attn));
     else
@@ -708,12 +762,20 @@ class softmax_layer : public base_loss_layer<dType> {  // src/softmax.h:14-225
     lower_layer.send_error(index, nodes[index].d_d_ERRt_ht);
   }
   void back_prop2(int /*index*/) override {}
-  // scale by 1 / minibatch_size, clip each gradient to norm_clip in L2 norm, add (gradient ascent on log-likelihood)
+  void calculate_global_norm() {  // src/softmax.hpp calculate_global_norm
+    zr_ctx* ctx = s_layer_info.ctx;
+    const float scale = 1.0f / (float)minibatch_size;
+    BZ_CUDA::add_to_global_norm(ctx, d_D_grad, (long long)output_vocab_size * LSTM_size, scale);
+    BZ_CUDA::add_to_global_norm(ctx, d_b_d_grad, output_vocab_size, scale);
+  }
+  void update_global_params() { update_weights(); }
+  // scale by 1 / minibatch_size, clip (each gradient to norm_clip in L2 norm unless BZ_CUDA selects another mode), add
+  // (gradient ascent on log-likelihood)
   void update_weights() override {
     zr_ctx* ctx = s_layer_info.ctx;
     const float scale = 1.0f / (float)minibatch_size, clip = clip_gradients ? norm_clip : 0.0f;
-    ZOPH_CALL(zr_sgd_update(ctx, d_D, d_D_grad, (long long)output_vocab_size * LSTM_size, scale, clip, learning_rate));
-    ZOPH_CALL(zr_sgd_update(ctx, d_b_d, d_b_d_grad, output_vocab_size, scale, clip, learning_rate));
+    BZ_CUDA::apply_update(ctx, d_D, d_D_grad, (long long)output_vocab_size * LSTM_size, scale, clip, (float)norm_clip, learning_rate);
+    BZ_CUDA::apply_update(ctx, d_b_d, d_b_d_grad, output_vocab_size, scale, clip, (float)norm_clip, learning_rate);
     prepare_weights();
   }
   void update_learning_rate(dType lr) override { learning_rate = lr; }
@@ -797,7 +859,17 @@ struct lstm_layer_training {
     const float scale = 1.0f / (float)mb, clip = clip_gradients ? (float)norm_clip : 0.0f;
     dType* gQ[4] = {d_Q_i_grad, d_Q_f_grad, d_Q_c_grad, d_Q_o_grad};
     ZOPH_CALL(zr_unstack_gates(ctx, d_Q_grad_stack, H, gQ));
-    for (int g = 0; g < 4; g++) ZOPH_CALL(zr_sgd_update(ctx, Q[g], gQ[g], (long long)H * H, scale, clip, learning_rate));
+    for (int g = 0; g < 4; g++) BZ_CUDA::apply_update(ctx, Q[g], gQ[g], (long long)H * H, scale, clip, (float)norm_clip, learning_rate);
+  }
+  // calculate_global_norm (src/Hidden_To_Hidden_Layer.hpp:241-335): the gate matrices' gradients are summed as the
+  // stacks they are kept in
+  void add_gradient_norms(zr_ctx* ctx, int H, int mb) {
+    const float scale = 1.0f / (float)mb;
+    const long long hh4 = 4LL * H * H;
+    if (d_Q_grad_stack) BZ_CUDA::add_to_global_norm(ctx, d_Q_grad_stack, hh4, scale);
+    BZ_CUDA::add_to_global_norm(ctx, d_M_grad_stack, hh4, scale);
+    BZ_CUDA::add_to_global_norm(ctx, d_W_h_grad_stack, hh4, scale);
+    BZ_CUDA::add_to_global_norm(ctx, d_b_grad_stack, 4LL * H, scale);
   }
   void zero_gradients(zr_ctx* ctx, int H) {
     if (d_Q_grad_stack) ZOPH_CALL(zr_memset_zero(ctx, d_Q_grad_stack, 4 * (size_t)H * H * sizeof(dType)));
@@ -816,9 +888,9 @@ struct lstm_layer_training {
     ZOPH_CALL(zr_unstack_gates(ctx, d_M_grad_stack, H, gM));
     ZOPH_CALL(zr_unstack_gates(ctx, d_W_h_grad_stack, H, gWh));
     for (int g = 0; g < 4; g++) {
-      ZOPH_CALL(zr_sgd_update(ctx, M[g], gM[g], hh, scale, clip, learning_rate));
-      ZOPH_CALL(zr_sgd_update(ctx, Wh[g], gWh[g], hh, scale, clip, learning_rate));
-      ZOPH_CALL(zr_sgd_update(ctx, b[g], gb[g], H, scale, clip, learning_rate));
+      BZ_CUDA::apply_update(ctx, M[g], gM[g], hh, scale, clip, (float)norm_clip, learning_rate);
+      BZ_CUDA::apply_update(ctx, Wh[g], gWh[g], hh, scale, clip, (float)norm_clip, learning_rate);
+      BZ_CUDA::apply_update(ctx, b[g], gb[g], H, scale, clip, (float)norm_clip, learning_rate);
     }
   }
 };
@@ -999,6 +1071,8 @@ class Hidden_To_Hidden_Layer : public lstm_layer_training<dType> {  // src/Hidde
     this->zero_gradients(ctx, LSTM_size);
   }
   void clear_gradients_GPU(bool init) { clear_gradients(init); }
+  void calculate_global_norm() { this->add_gradient_norms(hh_layer_info.ctx, LSTM_size, minibatch_size); }
+  void update_global_params() { update_weights(); }  // src/Hidden_To_Hidden_Layer.hpp:353-382
   // src/Hidden_To_Hidden_Layer.hpp:497-560, then the snapshots the kernels read are rebuilt
   void update_weights() {
     zr_ctx* ctx = hh_layer_info.ctx;
@@ -1180,13 +1254,19 @@ class Input_To_Hidden_Layer : public lstm_layer_training<dType> {  // src/Input_
     ZOPH_CALL(zr_memset_zero(ctx, d_W_grad, (size_t)LSTM_size * input_vocab_size * sizeof(dType)));
   }
   void clear_gradients_GPU(bool init) { clear_gradients(init); }
+  void calculate_global_norm() {  // src/Input_To_Hidden_Layer.hpp calculate_global_norm (norm_clip_W_GPU_v2_p1 for W)
+    zr_ctx* ctx = ih_layer_info.ctx;
+    BZ_CUDA::add_to_global_norm(ctx, d_W_grad, (long long)LSTM_size * input_vocab_size, 1.0f / (float)minibatch_size);
+    this->add_gradient_norms(ctx, LSTM_size, minibatch_size);
+  }
+  void update_global_params() { update_weights(); }
   void update_weights() {  // src/Input_To_Hidden_Layer.hpp:690-790
     zr_ctx* ctx = ih_layer_info.ctx;
     dType* M[4] = {d_M_i, d_M_f, d_M_c, d_M_o};
     dType* Wh[4] = {d_W_hi, d_W_hf, d_W_hc, d_W_ho};
     dType* b[4] = {d_b_i, d_b_f, d_b_c, d_b_o};
-    ZOPH_CALL(zr_sgd_update(ctx, d_W, d_W_grad, (long long)LSTM_size * input_vocab_size, 1.0f / (float)minibatch_size,
-                            this->clip_gradients ? (float)this->norm_clip : 0.0f, this->learning_rate));
+    BZ_CUDA::apply_update(ctx, d_W, d_W_grad, (long long)LSTM_size * input_vocab_size, 1.0f / (float)minibatch_size,
+                          this->clip_gradients ? (float)this->norm_clip : 0.0f, (float)this->norm_clip, this->learning_rate);
     this->apply_gradients(ctx, LSTM_size, minibatch_size, M, Wh, b);
     if (feed_input && this->d_Q_grad_stack) {
       dType* Q[4] = {d_Q_i, d_Q_f, d_Q_c, d_Q_o};

@@ -646,7 +646,20 @@ class forward_model {
     softmax->clear_gradients();
     if (att) att->clear_gradients();
   }
-  void update_weights() {  // src/model.hpp:1845-1955, per-matrix clipping (no global norm)
+  // src/model.hpp:1845-1955.  With BZ_CUDA::global_clip_flag every layer first adds its gradients' squared norms to the
+  // whole-model sum (calculate_global_norm, :1850-1892), which the updates then read on the device.
+  void update_weights() {
+    if (BZ_CUDA::global_clip_flag && !BZ_CUDA::individual_grad_clip) {
+      BZ_CUDA::reset_global_norm(gpu.ctx);
+      softmax_obj.calculate_global_norm();
+      if (!info.LM) {
+        input_layer_source.calculate_global_norm();
+        for (auto& l : source_hidden_layers) l.calculate_global_norm();
+      }
+      input_layer_target.calculate_global_norm();
+      for (auto& l : target_hidden_layers) l.calculate_global_norm();
+      if (att) att->calculate_global_norm();
+    }
     softmax->update_weights();
     if (!info.LM) {
       input_layer_source.update_weights();
@@ -793,10 +806,11 @@ class model_trainer {
     dType* Wh[4] = {ly.d_W_hi, ly.d_W_hf, ly.d_W_hc, ly.d_W_ho};
     dType* b[4] = {ly.d_b_i, ly.d_b_f, ly.d_b_c, ly.d_b_o};
     ZOPH_CALL(zr_unstack_gates(ctx, s.dM[l], H, unst));
-    for (int g = 0; g < 4; g++) ZOPH_CALL(zr_sgd_update(ctx, M[g], unst[g], (long long)hh, scale, norm_clip, lr));
+    for (int g = 0; g < 4; g++) BZ_CUDA::apply_update(ctx, M[g], unst[g], (long long)hh, scale, norm_clip, norm_clip, lr);
     ZOPH_CALL(zr_unstack_gates(ctx, s.dWh[l], H, unst));
-    for (int g = 0; g < 4; g++) ZOPH_CALL(zr_sgd_update(ctx, Wh[g], unst[g], (long long)hh, scale, norm_clip, lr));
-    for (int g = 0; g < 4; g++) ZOPH_CALL(zr_sgd_update(ctx, b[g], s.db[l] + (size_t)g * H, H, scale, norm_clip, lr));
+    for (int g = 0; g < 4; g++) BZ_CUDA::apply_update(ctx, Wh[g], unst[g], (long long)hh, scale, norm_clip, norm_clip, lr);
+    for (int g = 0; g < 4; g++)
+      BZ_CUDA::apply_update(ctx, b[g], s.db[l] + (size_t)g * H, H, scale, norm_clip, norm_clip, lr);
     ly.repack();
     const dType *Mc[4], *Whc[4];
     gate_ptrs(ly, Mc, Whc);
@@ -871,13 +885,29 @@ class model_trainer {
       std::vector<const dType*> ehT(tgt.eh0.begin(), tgt.eh0.end()), ecT(tgt.ec0.begin(), tgt.ec0.end());
       backward_side(src, m.input_layer_source, m.source_hidden_layers, S, Vs, z, z, err_top, &ehT, &ecT);
     }
-    // update_weights
+    // update_weights (src/model.hpp:1845-1955) under the clipping mode BZ_CUDA names: norm_clip per matrix, or over the
+    // whole model (the squared norms of all gradients are summed on the device first), or a clamp per element
     const float scale = 1.0f / (float)mb;
-    ZOPH_CALL(zr_sgd_update(ctx, sm.d_D, dD, (long long)Vt * H, scale, norm_clip, learning_rate));
-    ZOPH_CALL(zr_sgd_update(ctx, sm.d_b_d, dbd, Vt, scale, norm_clip, learning_rate));
+    if (BZ_CUDA::global_clip_flag && !BZ_CUDA::individual_grad_clip) {
+      BZ_CUDA::reset_global_norm(ctx);
+      BZ_CUDA::add_to_global_norm(ctx, dD, (long long)Vt * H, scale);
+      BZ_CUDA::add_to_global_norm(ctx, dbd, Vt, scale);
+      auto norm_side = [&](side& s, int V) {
+        BZ_CUDA::add_to_global_norm(ctx, s.dW, (long long)H * V, scale);
+        for (int l = 0; l < L; l++) {
+          BZ_CUDA::add_to_global_norm(ctx, s.dM[l], 4LL * H * H, scale);
+          BZ_CUDA::add_to_global_norm(ctx, s.dWh[l], 4LL * H * H, scale);
+          BZ_CUDA::add_to_global_norm(ctx, s.db[l], 4LL * H, scale);
+        }
+      };
+      norm_side(tgt, Vt);
+      if (seq2seq) norm_side(src, Vs);
+    }
+    BZ_CUDA::apply_update(ctx, sm.d_D, dD, (long long)Vt * H, scale, norm_clip, norm_clip, learning_rate);
+    BZ_CUDA::apply_update(ctx, sm.d_b_d, dbd, Vt, scale, norm_clip, norm_clip, learning_rate);
     sm.prepare_weights();
     auto update_side = [&](side& s, Input_To_Hidden_Layer<dType>& in, std::vector<Hidden_To_Hidden_Layer<dType>>& hid, int V) {
-      ZOPH_CALL(zr_sgd_update(ctx, in.d_W, s.dW, (long long)H * V, scale, norm_clip, learning_rate));
+      BZ_CUDA::apply_update(ctx, in.d_W, s.dW, (long long)H * V, scale, norm_clip, norm_clip, learning_rate);
       update_layer(in, s, 0, scale, norm_clip, learning_rate);
       for (int l = 1; l < L; l++) update_layer(hid[l - 1], s, l, scale, norm_clip, learning_rate);
     };
