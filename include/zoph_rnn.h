@@ -115,6 +115,10 @@ int zr_memset_zero(zr_ctx* ctx, void* d_dst, size_t bytes);
 /* d_dst[i] += d_src[i] (add_two_mats_kernel, src/custom_kernels.h:1818-1822; e.g. the feed-input error added to an
  * attention node's error, src/attention_node.hpp:416). */
 int zr_add_inplace(zr_ctx* ctx, float* d_dst, const float* d_src, long long n);
+/* d_x[i] clamped to [-threshold, threshold] (clip_mat_kernel, src/custom_kernels.h:2220-2231: with BZ_CUDA::clip_cell the
+ * reference clamps the error a node sends to h_{t-1}, to the layer below and to the previous h~ to
+ * +-BZ_CUDA::error_clip_threshold, src/LSTM.hpp:792,861 and src/LSTM_HH.hpp:665,756).  A NaN stays a NaN. */
+int zr_clip_inplace(zr_ctx* ctx, float* d_x, long long n, float threshold);
 
 /* ---- A1: index preparation ---------------------------------------------------------------------------- */
 

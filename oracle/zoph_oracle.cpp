@@ -909,10 +909,31 @@ void orc_lstm_step_backward(int H, int mb, const float* gi, const float* gf, con
 //   loss layer (d_ERRt_ht).  err_hT / err_cT: L x (H*mb) errors arriving at the last time step from beyond (NULL = 0).
 //   Outputs (double accumulation, rounded once): grads[l][0..3] = dM_g, [4..7] = dWh_g (H x H), [8..11] = db_g (H);
 //   d_embed: H x V dense (zero where no token hit); err_h0 / err_c0: L x (H*mb) errors at the initial states.
+//   cell_clip > 0: BZ_CUDA::clip_cell with that cell_clip_threshold in the forward sweep (src/LSTM.hpp:369-371; the
+//   backward pass uses the clamped c_t and passes errors through the clamp unchanged), and err_clip as
+//   BZ_CUDA::error_clip_threshold: the error a node sends to h_{t-1} (src/LSTM.hpp:792, src/LSTM_HH.hpp:756) and the
+//   error a layer above the first sends to the layer below (src/LSTM_HH.hpp:665) are clamped to +-err_clip, each on
+//   its own, before they are added to anything.  (The reference's third clamp, of d_ERRnTOt_ct at src/LSTM.hpp:888 /
+//   src/LSTM_HH.hpp:774, is queued behind that array's last use in the node and changes no output: not restated.)
+void orc_lstm_stack_backward_clip(int L, int H, int mb, int T, int V, const float* embed, const float* const* weights,
+                                  const int* ids_nonneg, const int* mask01, const float* h0, const float* c0,
+                                  const float* err_top, const float* err_hT, const float* err_cT, float cell_clip,
+                                  float err_clip, float* const* grads, float* d_embed, float* err_h0, float* err_c0);
 void orc_lstm_stack_backward(int L, int H, int mb, int T, int V, const float* embed, const float* const* weights,
                              const int* ids_nonneg, const int* mask01, const float* h0, const float* c0,
                              const float* err_top, const float* err_hT, const float* err_cT, float* const* grads,
                              float* d_embed, float* err_h0, float* err_c0) {
+  orc_lstm_stack_backward_clip(L, H, mb, T, V, embed, weights, ids_nonneg, mask01, h0, c0, err_top, err_hT, err_cT, 0.0f,
+                               0.0f, grads, d_embed, err_h0, err_c0);
+}
+void orc_lstm_stack_backward_clip(int L, int H, int mb, int T, int V, const float* embed, const float* const* weights,
+                                  const int* ids_nonneg, const int* mask01, const float* h0, const float* c0,
+                                  const float* err_top, const float* err_hT, const float* err_cT, float cell_clip,
+                                  float err_clip, float* const* grads, float* d_embed, float* err_h0, float* err_c0) {
+  auto clamp_errors = [&](float* e, size_t count) {  // clip_mat_kernel, src/custom_kernels.h:2220-2231
+    if (!(cell_clip > 0.0f)) return;
+    for (size_t i = 0; i < count; ++i) e[i] = e[i] > err_clip ? err_clip : (e[i] < -err_clip ? -err_clip : e[i]);
+  };
   const size_t n = (size_t)H * mb;
   const size_t LT = (size_t)L * T;
   std::vector<float> h_all(LT * n), c_all(LT * n), g_all(LT * 4 * n), x_all((size_t)T * n);
@@ -930,9 +951,9 @@ void orc_lstm_stack_backward(int L, int H, int mb, int T, int V, const float* em
       const float* hp = (t == 0) ? h0 + (size_t)l * n : h_all.data() + ((size_t)l * T + t - 1) * n;
       const float* cp = (t == 0) ? c0 + (size_t)l * n : c_all.data() + ((size_t)l * T + t - 1) * n;
       float* g = g_all.data() + ((size_t)l * T + t) * 4 * n;
-      orc_lstm_step(1, H, mb, w, w + 4, nullptr, w + 8, in, hp, cp, nullptr, mask01 + (size_t)t * mb, 0, 0.0f, g,
-                    g + n, g + 2 * n, g + 3 * n, c_all.data() + ((size_t)l * T + t) * n,
-                    h_all.data() + ((size_t)l * T + t) * n);
+      orc_lstm_step(1, H, mb, w, w + 4, nullptr, w + 8, in, hp, cp, nullptr, mask01 + (size_t)t * mb,
+                    cell_clip > 0.0f ? 1 : 0, cell_clip, g, g + n, g + 2 * n, g + 3 * n,
+                    c_all.data() + ((size_t)l * T + t) * n, h_all.data() + ((size_t)l * T + t) * n);
     }
   // backward
   std::vector<double> acc((size_t)L * 8 * H * H, 0.0), accb((size_t)L * 4 * H, 0.0), acce((size_t)H * V, 0.0);
@@ -969,6 +990,8 @@ void orc_lstm_stack_backward(int L, int H, int mb, int T, int V, const float* em
         for (int col = 0; col < mb; ++col)
           for (int i = 0; i < H; ++i) accb[((size_t)l * 4 + q) * H + i] += dg[(size_t)q * n + IDX2C(i, col, H)];
       }
+      clamp_errors(eh_next.data() + (size_t)l * n, n);
+      if (l > 0) clamp_errors(below.data(), n);
       if (l == 0) {  // sparse embedding gradient (W_gradient kernels, src/custom_kernels.h:1297-1390), dense here
         for (int col = 0; col < mb; ++col) {
           if (mask01[(size_t)t * mb + col] != 1) continue;

@@ -372,10 +372,13 @@ def lstm_step_backward(gates, c, cprev, mask01, err_h, err_c_next=None):
     return {"i": outs[0], "f": outs[1], "c": outs[2], "o": outs[3]}, outs[4]
 
 
-def lstm_stack_backward(embed, layers, ids_nonneg, mask01, err_top, h0=None, c0=None, err_hT=None, err_cT=None):
+def lstm_stack_backward(embed, layers, ids_nonneg, mask01, err_top, h0=None, c0=None, err_hT=None, err_cT=None,
+                        cell_clip=0.0, err_clip=0.0):
     """Back-propagation through time of the stacked LSTM (gradients of a loss whose derivative with respect to the top
     layer's h_t is err_top[t], H x mb each).  Returns (grads, d_embed, err_h0, err_c0): grads[l] = dict with dM, dWh
-    (lists of 4 H x H) and db (list of 4 H); d_embed H x V; err_h0 / err_c0 lists of L (H x mb)."""
+    (lists of 4 H x H) and db (list of 4 H); d_embed H x V; err_h0 / err_c0 lists of L (H x mb).
+    cell_clip > 0: the reference's --clip-cell mode (cell clamp in the forward sweep, errors to h_{t-1} and to the layer
+    below clamped to +-err_clip)."""
     embed = F(embed)
     H, V = embed.shape
     ids_nonneg = np.ascontiguousarray(ids_nonneg, dtype=np.int32)
@@ -409,10 +412,10 @@ def lstm_stack_backward(embed, layers, ids_nonneg, mask01, err_top, h0=None, c0=
     et = np.concatenate([F(err_top[t]).reshape(-1, order="F") for t in range(T)])
     d_embed = np.zeros((H, V), dtype=np.float32, order="F")
     eh0, ec0 = np.empty(L * n, dtype=np.float32), np.empty(L * n, dtype=np.float32)
-    lib().orc_lstm_stack_backward(C.c_int(L), C.c_int(H), C.c_int(mb), C.c_int(T), C.c_int(V), _p(embed), wptrs,
-                                  _p(ids_nonneg, i32p), _p(mask01, i32p), _p(h0f), _p(c0f), _p(et),
-                                  _p(ehT) if ehT is not None else None, _p(ecT) if ecT is not None else None, gptrs,
-                                  _p(d_embed), _p(eh0), _p(ec0))
+    lib().orc_lstm_stack_backward_clip(C.c_int(L), C.c_int(H), C.c_int(mb), C.c_int(T), C.c_int(V), _p(embed), wptrs,
+                                       _p(ids_nonneg, i32p), _p(mask01, i32p), _p(h0f), _p(c0f), _p(et),
+                                       _p(ehT) if ehT is not None else None, _p(ecT) if ecT is not None else None,
+                                       C.c_float(cell_clip), C.c_float(err_clip), gptrs, _p(d_embed), _p(eh0), _p(ec0))
     grads = [{"dM": gl[0:4], "dWh": gl[4:8], "db": gl[8:12]} for gl in gmats]
     unflat = lambda f: [f[l * n:(l + 1) * n].reshape(H, mb, order="F") for l in range(L)]
     return grads, d_embed, unflat(eh0), unflat(ec0)

@@ -208,6 +208,21 @@ def test_sgd_update_element_clip(ctx):
     assert np.allclose(dW.get(), W + lr * scale * G.astype(np.float64), rtol=1e-5, atol=1e-6)
 
 
+def test_clip_inplace(ctx):
+    """clip_mat_kernel (src/custom_kernels.h:2220-2231): values beyond +-threshold are set to it, a NaN stays."""
+    g = synth.rng(116, 1)
+    x = U(g, (10007,), -3, 3)
+    x[:5] = np.array([1.5, -1.5, np.nan, np.inf, -np.inf], np.float32)
+    d = ctx.array(x)
+    ctx.clip_inplace(d, x.size, 1.5)
+    ctx.sync()
+    got = d.get()
+    assert np.isnan(got[2]) and got[3] == 1.5 and got[4] == -1.5
+    keep = np.ones(x.size, bool)
+    keep[2] = False
+    assert np.array_equal(got[keep], np.clip(x[keep], -1.5, 1.5))
+
+
 def test_sgd_update_clipped_rejects_bad_arguments(ctx):
     from zoph_rnn_amd import capi
     dW, dG = ctx.zeros((8,)), ctx.zeros((8,))

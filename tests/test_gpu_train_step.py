@@ -82,7 +82,7 @@ def _clip_update(W, grad, mb, clip, lr, clipped, mode="matrix", whole_norm=None)
     return (np.asarray(W, np.float64) + lr * g).astype(np.float32)
 
 
-def _oracle_step(m, chunk, mb, lm, lr, clip, clipped, mode="matrix", norms=None):
+def _oracle_step(m, chunk, mb, lm, lr, clip, clipped, mode="matrix", norms=None, cell=None):
     """One training step on the oracle; updates m in place and returns the log-likelihood before the update."""
     L = len(m["tgt_layers"])
     if lm:
@@ -92,12 +92,13 @@ def _oracle_step(m, chunk, mb, lm, lr, clip, clipped, mode="matrix", norms=None)
         src, tin, tout = (_time_major([c[k] for c in chunk], mb) for k in (0, 2, 3))
         S = src.shape[0]
         nn_s, m_s = o.vocab_prep(src)
-        hs_src, cs_src = o.lstm_stack_forward(m["emb_s"], m["src_layers"], nn_s, m_s)
+        hs_src, cs_src = o.lstm_stack_forward(m["emb_s"], m["src_layers"], nn_s, m_s, clip=cell[0] if cell else None)
         h0 = [np.asfortranarray(hs_src[l, S - 1]) for l in range(L)]
         c0 = [np.asfortranarray(cs_src[l, S - 1]) for l in range(L)]
     T = tin.shape[0]
     nn_t, m_t = o.vocab_prep(tin)
-    hs, _ = o.lstm_stack_forward(m["emb_t"], m["tgt_layers"], nn_t, m_t, h0=h0, c0=c0)
+    hs, _ = o.lstm_stack_forward(m["emb_t"], m["tgt_layers"], nn_t, m_t, h0=h0, c0=c0, clip=cell[0] if cell else None)
+    ck = dict(cell_clip=cell[0], err_clip=cell[1]) if cell else {}
     tgt, tmask, _ = o.vocab_softmax(tout)
     Vt, H = m["D"].shape
     dD, dbd = np.zeros((Vt, H), np.float64, order="F"), np.zeros(Vt, np.float64)
@@ -107,11 +108,12 @@ def _oracle_step(m, chunk, mb, lm, lr, clip, clipped, mode="matrix", norms=None)
         loss += o.softmax_loss(o.softmax_logprob_f64(o.softmax_logits(m["D"], m["b_d"], h)), tgt[t], tmask[t])
         e, dD, dbd = o.softmax_backward(m["D"], m["b_d"], h, tgt[t], tmask[t], dD, dbd)
         err_top.append(e)
-    g_t, dW_t, eh0, ec0 = o.lstm_stack_backward(m["emb_t"], m["tgt_layers"], nn_t, m_t, err_top, h0=h0, c0=c0)
+    g_t, dW_t, eh0, ec0 = o.lstm_stack_backward(m["emb_t"], m["tgt_layers"], nn_t, m_t, err_top, h0=h0, c0=c0, **ck)
     sides = [("t", "tgt_layers", g_t, dW_t)]
     if not lm:
         zero_top = [np.zeros((H, mb), np.float32) for _ in range(S)]
-        g_s, dW_s, _, _ = o.lstm_stack_backward(m["emb_s"], m["src_layers"], nn_s, m_s, zero_top, err_hT=eh0, err_cT=ec0)
+        g_s, dW_s, _, _ = o.lstm_stack_backward(m["emb_s"], m["src_layers"], nn_s, m_s, zero_top, err_hT=eh0, err_cT=ec0,
+                                                **ck)
         sides.append(("s", "src_layers", g_s, dW_s))
     whole = None
     if mode == "whole":  # src/model.hpp:1850-1892: every gradient of the model, scaled by 1 / minibatch
@@ -150,7 +152,8 @@ def test_abandoned_forward_sweep_is_repeated_before_the_update(tmp_path):
 @pytest.mark.parametrize("node_level", [False, True])
 @pytest.mark.parametrize("lm,L,H,mb,steps,clip", [(True, 2, 32, 4, 1, 0.4), (False, 2, 48, 3, 1, 0.25),
                                                   (False, 1, 32, 5, 3, 5.0), (True, 3, 64, 8, 2, 1.0)])
-def test_train_steps_match_oracle(tmp_path, lm, L, H, mb, steps, clip, node_level, abandon=False, mode="matrix"):
+def test_train_steps_match_oracle(tmp_path, lm, L, H, mb, steps, clip, node_level, abandon=False, mode="matrix",
+                                  cell=None):
     """node_level: the same steps through the layer objects' back_prop_GPU / update_weights members
     (forward_model::compute_gradients) instead of model_trainer."""
     if not os.path.exists(DRIVER):
@@ -187,6 +190,7 @@ def test_train_steps_match_oracle(tmp_path, lm, L, H, mb, steps, clip, node_leve
     args = (["--sequence"] if lm else []) + (["--node-level"] if node_level else []) + \
         (["--abandon-sweeps"] if abandon else []) + (["--whole-clip"] if mode == "whole" else []) + \
         (["--ind-clip=%r" % clip] if mode == "element" else []) + \
+        (["--clip-cell=%r,%r" % cell] if cell else []) + \
         [str(model), str(data_path), str(mb), str(longest), str(lr), str(clip), str(steps)]
     r = subprocess.run([DRIVER] + args, capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, r.stderr[-2000:]
@@ -196,8 +200,16 @@ def test_train_steps_match_oracle(tmp_path, lm, L, H, mb, steps, clip, node_leve
         assert n_abandoned == [steps], "every step's forward sweep should have been abandoned and repeated"
     chunks = [data[i:i + mb] for i in range(0, len(data), mb)]
     clipped, want_loss, want_norms = [], [], []
+    if cell:  # the clamps must matter: one step without them moves a recurrent matrix somewhere else
+        import copy
+        m_with, m_without = copy.deepcopy(m), copy.deepcopy(m)
+        _oracle_step(m_with, chunks[0], mb, lm, lr, clip, [], mode, [], cell)
+        _oracle_step(m_without, chunks[0], mb, lm, lr, clip, [], mode, [], None)
+        moved = np.abs(np.asarray(m_with["tgt_layers"][0]["Wh"][0]) - np.asarray(m["tgt_layers"][0]["Wh"][0])).max()
+        apart = np.abs(np.asarray(m_with["tgt_layers"][0]["Wh"][0]) - np.asarray(m_without["tgt_layers"][0]["Wh"][0])).max()
+        assert apart > 0.02 * moved, "thresholds too high to act (%g of %g)" % (apart, moved)
     for s in range(steps):
-        want_loss.append(_oracle_step(m, chunks[s % len(chunks)], mb, lm, lr, clip, clipped, mode, want_norms))
+        want_loss.append(_oracle_step(m, chunks[s % len(chunks)], mb, lm, lr, clip, clipped, mode, want_norms, cell))
     if mode == "whole":
         got_norms = [float(ln.split()[2]) for ln in r.stdout.splitlines() if ln.startswith("global_norm")]
         assert got_norms == pytest.approx(want_norms, rel=1e-4)
@@ -228,6 +240,16 @@ def test_train_steps_with_whole_model_and_element_clipping(tmp_path, mode, lm, L
     the norm of ALL gradients together (the first case clips in some steps and not in others, the second never), and a
     clamp of every gradient element.  In whole-model mode the norm the driver reports is compared too."""
     test_train_steps_match_oracle(tmp_path, lm, L, H, mb, steps, clip, node_level, mode=mode)
+
+
+@pytest.mark.parametrize("lm,L,H,mb,steps,cell", [(False, 2, 48, 3, 2, (0.2, 0.004)), (True, 3, 32, 4, 1, (0.15, 0.002))])
+def test_train_steps_with_cell_and_error_clamps(tmp_path, lm, L, H, mb, steps, cell):
+    """--clip-cell (src/main.cu:399-405): the cell clamped in the forward pass, and the errors sent to h_{t-1} and to the
+    layer below clamped in the backward pass, through the node classes (model_trainer hands such models to them).  The
+    thresholds are low enough to act: the same steps without them end at weights that differ by far more than the
+    tolerance (checked on the oracle)."""
+    test_train_steps_match_oracle(tmp_path, lm, L, H, mb, steps, 5.0, False, cell=cell)
+    test_train_steps_match_oracle(tmp_path, lm, L, H, mb, steps, 5.0, True, cell=cell)
 
 
 def test_repeated_steps_on_one_minibatch_raise_its_likelihood(tmp_path):

@@ -11,9 +11,23 @@ from zoph_rnn_amd import synth
 U = synth.uniform
 
 
-def _torch_stack(embed, layers, ids, mask, h0, c0, err_top, err_hT=None, err_cT=None):
+class _ClampGradient(torch.autograd.Function):
+    """Identity whose backward clamps the gradient passing through it to +-limit."""
+    @staticmethod
+    def forward(ctx, x, limit):
+        ctx.limit = limit
+        return x.view_as(x)
+
+    @staticmethod
+    def backward(ctx, grad):
+        return grad.clamp(-ctx.limit, ctx.limit), None
+
+
+def _torch_stack(embed, layers, ids, mask, h0, c0, err_top, err_hT=None, err_cT=None, cell_clip=0.0, err_clip=0.0):
     """The forward equations in torch float64; the scalar whose gradient is wanted is sum_t <err_top[t], h_top[t]>
-    (+ <err_hT, h_T> + <err_cT, c_T>)."""
+    (+ <err_hT, h_T> + <err_cT, c_T>).  cell_clip > 0 (the reference's --clip-cell): the cell is clamped in the forward
+    pass and the gradient passes the clamp unchanged; what flows back into h_{t-1} through the recurrent products, and
+    what flows into the layer below through the input products of a layer above the first, is clamped to +-err_clip."""
     td = lambda a: torch.tensor(np.asarray(a, dtype=np.float64), requires_grad=True)
     E = td(embed)
     W = [{"M": [td(m) for m in ly["M"]], "Wh": [td(m) for m in ly["Wh"]], "b": [td(b) for b in ly["b"]]} for ly in layers]
@@ -27,10 +41,18 @@ def _torch_stack(embed, layers, ids, mask, h0, c0, err_top, err_hT=None, err_cT=
         x = E[:, torch.tensor(np.maximum(ids[t], 0).astype(np.int64))]
         for l in range(L):
             w = W[l]
-            pre = [w["M"][g] @ x + w["Wh"][g] @ h[l] + w["b"][g][:, None] for g in range(4)]
+            hr = h[l]
+            if cell_clip > 0:
+                hr = _ClampGradient.apply(hr, err_clip)
+                if l > 0:
+                    x = _ClampGradient.apply(x, err_clip)
+            pre = [w["M"][g] @ x + w["Wh"][g] @ hr + w["b"][g][:, None] for g in range(4)]
             i, f, ct, og = torch.sigmoid(pre[0]), torch.sigmoid(pre[1]), torch.tanh(pre[2]), torch.sigmoid(pre[3])
-            cn = (f * c[l] + i * ct) * m
-            hn = og * torch.tanh(f * c[l] + i * ct) * m
+            cell = f * c[l] + i * ct
+            if cell_clip > 0:
+                cell = cell + (cell.clamp(-cell_clip, cell_clip) - cell).detach()
+            cn = cell * m
+            hn = og * torch.tanh(cell) * m
             h[l], c[l] = hn, cn
             x = hn
         loss = loss + (torch.tensor(np.asarray(err_top[t], np.float64)) * h[L - 1]).sum()
@@ -77,6 +99,48 @@ def test_stack_backward_matches_torch_autograd(L, H, mb, T, V, pad):
     for v in range(V):
         if v not in used:
             assert np.all(d_embed[:, v] == 0)
+
+
+@pytest.mark.parametrize("L,H,mb,T,V", [(1, 6, 3, 4, 9), (3, 10, 5, 6, 20)])
+def test_stack_backward_with_cell_and_error_clamps_matches_torch_autograd(L, H, mb, T, V):
+    """--clip-cell: thresholds small enough that the cell clamp and both error clamps act on a good share of the
+    elements (checked), so that a clamp applied at another place -- to the summed error of h_t, to the cell error, to the
+    embedding's error -- or left out changes the gradients."""
+    g = synth.rng(102, L * 100 + H)
+    embed = U(g, (H, V), -0.5, 0.5)
+    layers = [synth.lstm_layer(g, H) for _ in range(L)]
+    for ly in layers:
+        ly["M"] = [U(g, (H, H), -0.6, 0.6) for _ in range(4)]
+        ly["Wh"] = [U(g, (H, H), -0.6, 0.6) for _ in range(4)]
+        ly["b"] = [U(g, (H,), -0.3, 0.3) for _ in range(4)]
+    ids = g.integers(0, V, size=(T, mb)).astype(np.int32)
+    ids[:1, 1] = -1
+    nn, mask = o.vocab_prep(ids)
+    h0 = [U(g, (H, mb), -0.5, 0.5) for _ in range(L)]
+    c0 = [U(g, (H, mb), -0.9, 0.9) for _ in range(L)]
+    err_top = [U(g, (H, mb), -1, 1) for _ in range(T)]
+    cell_clip, err_clip = 0.35, 0.08
+    args = (embed, layers, nn, mask, err_top, h0, c0)
+    grads, d_embed, eh0, ec0 = o.lstm_stack_backward(*args, cell_clip=cell_clip, err_clip=err_clip)
+    plain = o.lstm_stack_backward(*args)
+    assert not np.allclose(plain[0][0]["dWh"][0], grads[0]["dWh"][0], rtol=1e-2, atol=1e-3), "the clamps never acted"
+    E, W, H0, C0 = _torch_stack(embed, layers, ids, mask, h0, c0, err_top, cell_clip=cell_clip, err_clip=err_clip)
+    tol = dict(rtol=2e-4, atol=2e-5)
+    for l in range(L):
+        for q in range(4):
+            assert np.allclose(grads[l]["dM"][q], W[l]["M"][q].grad.numpy(), **tol), (l, q, "dM")
+            assert np.allclose(grads[l]["dWh"][q], W[l]["Wh"][q].grad.numpy(), **tol), (l, q, "dWh")
+            assert np.allclose(grads[l]["db"][q], W[l]["b"][q].grad.numpy(), **tol), (l, q, "db")
+        assert np.allclose(eh0[l], H0[l].grad.numpy(), **tol)
+        assert np.allclose(ec0[l], C0[l].grad.numpy(), **tol)
+        assert np.abs(eh0[l]).max() <= err_clip + 1e-7
+    assert max((np.abs(e) >= err_clip - 1e-7).mean() for e in eh0) > 0.05, "no error of an initial state was clamped"
+    assert np.allclose(d_embed, E.grad.numpy(), **tol)
+    if L == 1:  # the error reaching the embedding is NOT clamped: some of it exceeds the bound
+        assert np.abs(d_embed).max() > err_clip
+    # a huge error bound and no cell clamp in reach: the plain gradients
+    same = o.lstm_stack_backward(*args, cell_clip=1e6, err_clip=1e6)
+    assert np.array_equal(same[1], plain[1]) and all(np.array_equal(a, b) for a, b in zip(same[2], plain[2]))
 
 
 def test_step_backward_closed_forms():

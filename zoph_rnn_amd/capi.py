@@ -44,7 +44,7 @@ SYMBOLS = [
     "zr_beam_hypotheses", "zr_beam_state",
     "zr_lstm_stack_forward_train", "zr_lstm_train_create", "zr_lstm_train_refresh", "zr_lstm_train_destroy",
     "zr_unstack_gates", "zr_lstm_stack_backward", "zr_lstm_weight_gradients", "zr_embed_gradient",
-    "zr_softmax_backward", "zr_sgd_update", "zr_grad_sumsq_accumulate", "zr_sgd_update_clipped", "zr_lstm_node_backward", "zr_lstm_node_gradients",
+    "zr_softmax_backward", "zr_sgd_update", "zr_grad_sumsq_accumulate", "zr_sgd_update_clipped", "zr_clip_inplace", "zr_lstm_node_backward", "zr_lstm_node_gradients",
     "zr_softmax_backward_accumulate", "zr_gather_columns_multi", "zr_softmax_backward_loss",
     "zr_softmax_forward_static", "zr_ctx_query", "zr_attn_prepare", "zr_lstm_step_embed", "zr_attn_viterbi", "zr_lstm_decoder_step", "zr_decoder_step", "zr_lstm_feed_backward", "zr_attn_set_error_tables",
     "zr_attn_backward", "zr_dropout_apply", "zr_uniform_fill", "zr_add_inplace",
@@ -342,6 +342,9 @@ class Context:
     def sgd_update(self, d_W, d_grad, n, scale, norm_clip, lr):
         _chk(load().zr_sgd_update(self.h, _vp(d_W), _vp(d_grad), C.c_longlong(n), C.c_float(scale), C.c_float(norm_clip),
                                   C.c_float(lr)))
+
+    def clip_inplace(self, d_x, n, threshold):
+        _chk(load().zr_clip_inplace(self.h, _vp(d_x), C.c_longlong(n), C.c_float(threshold)))
 
     def grad_sumsq_accumulate(self, d_grad, n, scale, d_sumsq, reset=False):
         """d_sumsq: device array of one float64"""

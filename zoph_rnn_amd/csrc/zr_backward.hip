@@ -347,7 +347,7 @@ __global__ void __launch_bounds__(256) sgd_apply_kernel(float* __restrict__ W, c
   if (mode == ZR_CLIP_ELEMENT) {
     for (long long i = first; i < n; i += stride) {
       const float x = scale * g[i];
-      W[i] += lr * fminf(fmaxf(x, -threshold), threshold);
+      W[i] += lr * (x > threshold ? threshold : (x < -threshold ? -threshold : x));  // a NaN stays a NaN (clip_mat_kernel)
     }
     return;
   }

@@ -205,9 +205,29 @@ __global__ void __launch_bounds__(256) add_inplace_kernel(float* __restrict__ ds
     dst[i] = dst[i] + src[i];
 }
 
+// clip_mat_kernel (src/custom_kernels.h:2220-2231)
+__global__ void __launch_bounds__(256) clip_inplace_kernel(float* __restrict__ x, long long n, float threshold) {
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) {
+    const float v = x[i];
+    x[i] = v > threshold ? threshold : (v < -threshold ? -threshold : v);  // a NaN stays a NaN, as in the reference
+  }
+}
+
 }  // namespace
 
 extern "C" {
+
+int zr_clip_inplace(zr_ctx* ctx, float* d_x, long long n, float threshold) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(n >= 0 && (n == 0 || d_x) && threshold >= 0.0f, "zr_clip_inplace: null pointer, n = %lld or threshold = %g",
+               n, (double)threshold);
+  if (n == 0) return ZR_OK;
+  const int blocks = (int)((n + 255) / 256 < 2048 ? (n + 255) / 256 : 2048);
+  clip_inplace_kernel<<<blocks, 256, 0, ctx->stream>>>(d_x, n, threshold);
+  ZR_LAUNCH_CHECK("clip_inplace_kernel");
+  return ZR_OK;
+}
 
 int zr_add_inplace(zr_ctx* ctx, float* d_dst, const float* d_src, long long n) {
   int rc = zr_bind_device(ctx);

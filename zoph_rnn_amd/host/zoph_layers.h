@@ -57,14 +57,12 @@ namespace BZ_CUDA {
 inline bool clip_cell = false;
 inline precision cell_clip_threshold = 50;
 // With clip_cell set the reference also clamps the back-propagated errors to +-error_clip_threshold
-// (src/LSTM.hpp:792,888; src/LSTM_HH.hpp:665,756,774).  The backward kernels here have no such clamp, so the backward
-// members refuse to run with clip_cell set rather than return gradients that differ from the reference's.
-inline void refuse_backward_with_clip_cell(const char* who) {
-  if (clip_cell) {
-    std::fprintf(stderr, "Error: %s: the backward pass does not clamp errors (BZ_CUDA::error_clip_threshold) and "
-                 "cannot run with BZ_CUDA::clip_cell set\n", who);
-    std::exit(EXIT_FAILURE);
-  }
+// (src/BZ_CUDA_UTIL.h:109; src/LSTM.hpp:792,861; src/LSTM_HH.hpp:665,756): the node classes' back_prop_GPU members do
+// the same.  (Its third clamp, of d_ERRnTOt_ct at src/LSTM.hpp:888 / src/LSTM_HH.hpp:774, is queued behind that
+// array's last use in the node and changes no output; it has no counterpart here.)
+inline precision error_clip_threshold = 1000;
+inline void clip_error(zr_ctx* ctx, float* d_err, long long n) {
+  if (clip_cell) ZOPH_CALL(zr_clip_inplace(ctx, d_err, n, error_clip_threshold));
 }
 // The three ways of clipping gradients (src/BZ_CUDA_UTIL.h:101-118), exclusive as src/main.cu:495-511 sets them: per
 // matrix (neither flag: the layers' clip_gradients / norm_clip), over the whole model (global_clip_flag, threshold =
@@ -1540,7 +1538,6 @@ void lower_transfer_layer<dType>::send_error(int index, dType* d_err) {
 // the driver passes to the next backprop_prep_GPU call, and the error for the layer below is handed down by pointer.
 template <typename dType>
 void LSTM_HH_Node<dType>::back_prop_GPU(int index) {
-  BZ_CUDA::refuse_backward_with_clip_cell("LSTM_HH_Node::back_prop_GPU");
   zr_ctx* ctx = model->hh_layer_info.ctx;
   if (!model->train_weights) model->clear_gradients(true);
   if (attention_model && model->attent_layer) {  // src/LSTM_HH.hpp:470-482: the error of h~ becomes the error of h_t
@@ -1553,6 +1550,8 @@ void LSTM_HH_Node<dType>::back_prop_GPU(int index) {
                                   d_input_vocab_indices_01, d_d_ERRt_ht, d_d_ERRnTOtp1_ht, d_d_ERRnTOtp1_ct,
                                   model->d_d_ERRnTOt_gates, model->d_d_ERRnTOt_htM1, model->d_d_ERRnTOt_ctM1,
                                   model->d_d_ERRnTOt_h_Below));
+  BZ_CUDA::clip_error(ctx, model->d_d_ERRnTOt_htM1, (long long)LSTM_size * minibatch_size);     // src/LSTM_HH.hpp:755-757
+  BZ_CUDA::clip_error(ctx, model->d_d_ERRnTOt_h_Below, (long long)LSTM_size * minibatch_size);  // src/LSTM_HH.hpp:665-667
   compute_gradients_GPU();
   if (d_input == d_h_t_below_drop && d_dropout_mask)  // src/LSTM_HH.hpp:673-675
     ZOPH_CALL(zr_dropout_apply(ctx, d_dropout_mask, dropout_rate, model->d_d_ERRnTOt_h_Below,
@@ -1569,7 +1568,6 @@ void LSTM_HH_Node<dType>::compute_gradients_GPU() {
 
 template <typename dType>
 void LSTM_IH_Node<dType>::back_prop_GPU(int /*index*/) {
-  BZ_CUDA::refuse_backward_with_clip_cell("LSTM_IH_Node::back_prop_GPU");
   zr_ctx* ctx = model->ih_layer_info.ctx;
   if (!model->train_weights) model->clear_gradients(true);
   if (attention_model && model->attent_layer) {  // src/LSTM.hpp:587-599: a one-layer model's attention sits on this layer
@@ -1582,10 +1580,13 @@ void LSTM_IH_Node<dType>::back_prop_GPU(int /*index*/) {
                                   d_input_vocab_indices_01, d_d_ERRt_ht, d_d_ERRnTOtp1_ht, d_d_ERRnTOtp1_ct,
                                   model->d_d_ERRnTOt_gates, model->d_d_ERRnTOt_htM1, model->d_d_ERRnTOt_ctM1,
                                   model->d_d_ERRnTOt_h_Below));
+  // src/LSTM.hpp:792-794 (the error that reaches the embedding through d_d_ERRnTOt_h_Below is not clamped there)
+  BZ_CUDA::clip_error(ctx, model->d_d_ERRnTOt_htM1, (long long)LSTM_size * minibatch_size);
   if (feed_input && index != 0) {  // src/LSTM.hpp:804-866 and :1014-1050
     const dType* Q[4] = {model->d_Q_i, model->d_Q_f, model->d_Q_c, model->d_Q_o};
     ZOPH_CALL(zr_lstm_feed_backward(ctx, Q, LSTM_size, minibatch_size, model->d_d_ERRnTOt_gates, d_h_tild,
                                     model->d_ERRnTOt_h_tild, model->d_Q_grad_stack));
+    BZ_CUDA::clip_error(ctx, model->d_ERRnTOt_h_tild, (long long)LSTM_size * minibatch_size);  // src/LSTM.hpp:861-863
     if (d_ERRnTOt_h_tild_cpy)
       ZOPH_CALL(zr_d2d(ctx, d_ERRnTOt_h_tild_cpy, model->d_ERRnTOt_h_tild,
                        (size_t)LSTM_size * minibatch_size * sizeof(dType)));

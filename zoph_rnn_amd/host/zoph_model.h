@@ -755,8 +755,8 @@ class model_trainer {
   }
 
   explicit model_trainer(forward_model<dType>& model) : m(model), ctx(model.gpu.ctx) {
-    BZ_CUDA::refuse_backward_with_clip_cell("model_trainer");
-    node_level = m.params.attent_params.attention_model || m.params.dropout;
+    // the stack-level backward sweep has no error clamp: with BZ_CUDA::clip_cell the step goes through the node classes
+    node_level = m.params.attent_params.attention_model || m.params.dropout || BZ_CUDA::clip_cell;
     H = m.info.LSTM_size;
     L = m.info.num_layers;
     mb = m.params.minibatch_size;
