@@ -74,7 +74,7 @@ def _zero_grads(ly, H):
     return g
 
 
-def _oracle_step(m, chunk, mb, lr, clip, clipped, D, longest, feed, masks):
+def _oracle_step(m, chunk, mb, lr, clip, clipped, D, longest, feed, masks, mode="matrix", norms=None):
     L, H = len(m["src_layers"]), m["emb_s"].shape[0]
     src, tin, tout = (_time_major([c[k] for c in chunk], mb) for k in (0, 2, 3))
     S, T = src.shape[0], tin.shape[0]
@@ -164,7 +164,16 @@ def _oracle_step(m, chunk, mb, lr, clip, clipped, D, longest, feed, masks):
                     if m_s[t][b] == 1:
                         dW_s[:, nn_s[t][b]] += below[:, b]
     # ---- update
-    up = lambda W, g: _clip_update(W, g, mb, clip, lr, clipped)
+    whole = None
+    if mode == "whole":  # the norm of every gradient of the model together (src/model.hpp:1850-1892)
+        sq = lambda x: (np.asarray(x, np.float64) ** 2).sum()
+        ss = sq(dD) + sq(dbd) + sq(dW_t) + sq(dW_s) + sum(sq(ag[k]) for k in ("W_a", "W_p", "v_p", "bias", "W_c1", "W_c2"))
+        for grads in (g_t, g_s):
+            for gr in grads:
+                ss += sum(sq(gr[k][q]) for k in gr for q in range(4))
+        whole = np.sqrt(ss) / mb
+        norms.append(whole)
+    up = lambda W, g: _clip_update(W, g, mb, clip, lr, clipped, mode, whole)
     m["D"], m["b_d"] = up(m["D"], dD), up(m["b_d"], dbd)
     m["emb_t"], m["emb_s"] = up(m["emb_t"], dW_t), up(m["emb_s"], dW_s)
     for layers, grads in ((m["tgt_layers"], g_t), (m["src_layers"], g_s)):
@@ -240,7 +249,7 @@ def _read_model(path, n_head, L, H, Vs, Vt, feed):
                          [(2, 32, 3, 2, True, 1.0, 1, 0.5, False), (1, 24, 4, 3, True, 1.0, 2, 5.0, False),
                           (2, 32, 3, 4, False, 1.0, 1, 5.0, False), (3, 40, 5, 2, True, 0.7, 2, 0.5, False),
                           (1, 24, 2, 2, False, 0.5, 1, 5.0, False), (2, 32, 3, 2, True, 0.8, 2, 0.5, True)])
-def test_attention_model_train_steps_match_oracle(tmp_path, L, H, mb, D, feed, rate, steps, clip, trainer):
+def test_attention_model_train_steps_match_oracle(tmp_path, L, H, mb, D, feed, rate, steps, clip, trainer, mode="matrix"):
     """trainer: through model_trainer::train_minibatch, which hands attention / dropout models to the node-level path."""
     if not os.path.exists(DRIVER):
         pytest.fail("tests/host/train_step is not built: run `python __graft_entry__.py build`")
@@ -272,7 +281,7 @@ def test_attention_model_train_steps_match_oracle(tmp_path, L, H, mb, D, feed, r
         for r in data:
             for k in range(4):
                 f.write(" ".join(str(v) for v in r[k]) + "\n")
-    args = ([] if trainer else ["--node-level"]) + ["--attention-D=%d" % D, "--dropout=%g" % rate, "--dropout-seed=%d" % seed, str(model),
+    args = ([] if trainer else ["--node-level"]) + (["--whole-clip"] if mode == "whole" else []) + ["--attention-D=%d" % D, "--dropout=%g" % rate, "--dropout-seed=%d" % seed, str(model),
             str(data_path), str(mb), str(longest), str(lr), str(clip), str(steps)]
     r = subprocess.run([DRIVER] + args, capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, r.stderr[-2000:]
@@ -281,16 +290,21 @@ def test_attention_model_train_steps_match_oracle(tmp_path, L, H, mb, D, feed, r
     try:
         masks = Masks(ctx, seed, H, mb, rate)
         chunks = [data[i:i + mb] for i in range(0, len(data), mb)]
-        clipped, want_loss = [], []
+        clipped, want_loss, want_norms = [], [], []
         for s in range(steps):
-            want_loss.append(_oracle_step(m, chunks[s % len(chunks)], mb, lr, clip, clipped, D, longest, feed, masks))
+            want_loss.append(_oracle_step(m, chunks[s % len(chunks)], mb, lr, clip, clipped, D, longest, feed, masks, mode,
+                                          want_norms))
     finally:
         ctx.close()
+    if mode == "whole":
+        got_norms = [float(ln.split()[2]) for ln in r.stdout.splitlines() if ln.startswith("global_norm")]
+        assert got_norms == pytest.approx(want_norms, rel=1e-4)
+        assert all(n > clip for n in want_norms), "the threshold should act: %s" % want_norms
     # the driver's loss line is the log-likelihood of the evaluation-mode forward pass (no dropout) before the update
     if rate >= 1.0:
         for x, y in zip(got_loss, want_loss):
             assert x == pytest.approx(y, rel=1e-4, abs=1e-4)
-    if clip < 5.0:
+    if clip < 5.0 and mode == "matrix":
         assert any(clipped) and not all(clipped), "pick norm_clip so that both branches of the clipping run"
     new = _read_model(str(model) + ".trained", n_head, L, H, Vs, Vt, feed)
     _compare("D", new["D"], m["D"], orig["D"])
@@ -304,3 +318,9 @@ def test_attention_model_train_steps_match_oracle(tmp_path, L, H, mb, D, feed, r
                 for gate in range(4):
                     _compare("%s layer %d %s[%d]" % (key, l, k, gate), new[key][l][k][gate], m[key][l][k][gate],
                              orig[key][l][k][gate])
+
+
+def test_attention_model_train_steps_with_whole_model_clipping(tmp_path):
+    """--whole-clip-gradients on a feed-input attention model: the attention layer's six gradients and the Q matrices'
+    take part in the model's norm (attention_layer::norm_p1 / norm_p2), which the driver reports."""
+    test_attention_model_train_steps_match_oracle(tmp_path, 2, 32, 3, 2, True, 1.0, 2, 1.0, False, mode="whole")
