@@ -354,6 +354,17 @@ int zr_beam_finish_logits(zr_ctx* ctx, zr_beam* b, const float* d_logits, const 
 /* Copies the finished hypotheses of sentence s to the host: returns their number (or a negative error);
  * h_words is n x max_len (row-major, -1 padded), h_len and h_score have n entries; at most cap are copied. */
 int zr_beam_hypotheses(zr_ctx* ctx, zr_beam* b, int sentence, int cap, int* h_words, int* h_len, float* h_score);
+/* Viterbi alignments through the beam, for unk replacement (decoder::top_sentences_viterbi and
+ * eigen_mat_wrapper::viterbi_alignments, src/decoder.h:126,230-231; initialised to -20, :1335).  With enable != 0 every
+ * later zr_beam_expand* / zr_beam_finish* call attaches to each candidate the alignment of the column it comes from,
+ * read from d_viterbi (n_sent*beam ints in device memory, e.g. zr_attn_viterbi's output, read when that call runs;
+ * NULL: -1 for every column, as the reference does when it is handed none, :1174-1179), a surviving hypothesis keeps
+ * its parent's alignments plus its own at position current_index+1 (:1281-1282), and a finished one likewise
+ * (:1266-1267, :683-684).  Switch it on before the first step of a sentence (the call then also runs zr_beam_init).
+ * zr_beam_hypotheses_viterbi copies the alignments of the finished hypotheses of sentence s, n x max_len like
+ * zr_beam_hypotheses' h_words and in the same order; returns their number. */
+int zr_beam_set_viterbi(zr_ctx* ctx, zr_beam* b, int enable, const int* d_viterbi);
+int zr_beam_hypotheses_viterbi(zr_ctx* ctx, zr_beam* b, int sentence, int cap, int* h_viterbi);
 /* Current beam state of sentence s (top_sentences_scores, current_indices). */
 int zr_beam_state(zr_ctx* ctx, zr_beam* b, int sentence, float* h_scores, int* h_words);
 

@@ -611,11 +611,13 @@ namespace {
 struct DecObj {
   float val;
   int vocab_index;
+  int viterbi_alignment;  // src/decoder.h:62: the column's alignment rides along with every candidate
 };
 struct DecGlobalObj {
   float val;
   int beam_index;
   int vocab_index;
+  int viterbi_alignment;  // src/decoder.h:35
 };
 struct PqCmp {
   bool operator()(const DecObj& a, const DecObj& b) const { return a.val < b.val; }
@@ -625,6 +627,7 @@ struct PqGlobalCmp {
 };
 struct Hypothesis {
   std::vector<int> words;
+  std::vector<int> viterbi;  // src/decoder.h:126: one source position per word (entry 0 keeps the initial -20)
   float score;
 };
 
@@ -634,6 +637,7 @@ struct OrcDecoder {
   int current_index;
   std::vector<int> current_indices, new_indicies_changes;
   std::vector<int> top_sentences, top_sentences_temp;  // beam x max_len, row-major here
+  std::vector<int> top_viterbi, top_viterbi_temp;      // top_sentences_viterbi (src/decoder.h:230-231), same shape
   std::vector<float> scores, scores_temp;
   std::vector<Hypothesis> hypotheses;
   std::priority_queue<DecObj, std::vector<DecObj>, PqCmp> pq;
@@ -658,6 +662,8 @@ void* orc_decoder_create(int beam, int vocab, int start_symbol, int end_symbol, 
   d->new_indicies_changes.assign(beam, 0);
   d->top_sentences.resize((size_t)beam * max_len);
   d->top_sentences_temp.resize((size_t)beam * max_len);
+  d->top_viterbi.resize((size_t)beam * max_len);
+  d->top_viterbi_temp.resize((size_t)beam * max_len);
   d->scores.resize(beam);
   d->scores_temp.resize(beam);
   d->current_index = 0;
@@ -674,11 +680,13 @@ void orc_decoder_init(void* p) {
   d->hypotheses.clear();
   for (int i = 0; i < d->beam; ++i) d->current_indices[i] = d->start_symbol;
   std::fill(d->top_sentences.begin(), d->top_sentences.end(), d->start_symbol);
+  std::fill(d->top_viterbi.begin(), d->top_viterbi.end(), -20);  // src/decoder.h:1335
 }
 
 // expand_hypothesis_without_fsa, src/decoder.h:1158-1315.  outputdist: vocab x beam probabilities,
-// column-major (column = beam entry).
-void orc_decoder_expand(void* p, const float* outputdist, int index) {
+// column-major (column = beam entry).  viterbi: the attention layer's Viterbi alignment of every column
+// (BZ_CUDA::viterbi_alignments), or NULL: the reference then fills in -1 for every column (:1174-1179).
+void orc_decoder_expand_viterbi(void* p, const float* outputdist, int index, const int* viterbi) {
   OrcDecoder* d = (OrcDecoder*)p;
   const int beam = d->beam, V = d->vocab, L = d->max_len;
   int cols = beam;
@@ -687,19 +695,20 @@ void orc_decoder_expand(void* p, const float* outputdist, int index) {
   for (int i = 0; i < cols; ++i) {
     while (!d->pq.empty()) d->pq.pop();
     if (d->current_indices[i] == -1) break;
+    const int vit = viterbi ? viterbi[i] : -1;
     for (int j = 0; j < V; ++j) {
       const float pr = outputdist[IDX2C(j, i, V)];
       if ((int)d->pq.size() < beam + 1) {
-        d->pq.push(DecObj{-pr, j});
+        d->pq.push(DecObj{-pr, j, vit});
       } else if (-pr < d->pq.top().val) {
         d->pq.pop();
-        d->pq.push(DecObj{-pr, j});
+        d->pq.push(DecObj{-pr, j, vit});
       }
     }
     while (!d->pq.empty()) {
       DecObj t = d->pq.top();
       d->pq.pop();
-      d->pq_global.push(DecGlobalObj{std::log(-t.val) + d->scores[i], i, t.vocab_index});
+      d->pq_global.push(DecGlobalObj{std::log(-t.val) + d->scores[i], i, t.vocab_index, t.viterbi_alignment});
     }
   }
   int i = 0;
@@ -707,6 +716,7 @@ void orc_decoder_expand(void* p, const float* outputdist, int index) {
     if (d->pq_global.empty()) {
       for (int c = 0; c < L; ++c) d->top_sentences_temp[(size_t)i * L + c] = d->top_sentences[c];
       d->top_sentences_temp[(size_t)i * L + d->current_index + 1] = d->start_symbol;
+      for (int c = 0; c < L; ++c) d->top_viterbi_temp[(size_t)i * L + c] = d->top_viterbi[c];  // :1237, row 0 as it is
       d->current_indices[i] = -1;
       d->new_indicies_changes[i] = 0;
       d->scores_temp[i] = 0;
@@ -721,12 +731,18 @@ void orc_decoder_expand(void* p, const float* outputdist, int index) {
         hy.words.assign(d->top_sentences.begin() + (size_t)t.beam_index * L,
                         d->top_sentences.begin() + (size_t)t.beam_index * L + d->current_index + 2);
         hy.words[d->current_index + 1] = d->end_symbol;
+        hy.viterbi.assign(d->top_viterbi.begin() + (size_t)t.beam_index * L,
+                          d->top_viterbi.begin() + (size_t)t.beam_index * L + d->current_index + 2);  // :1266-1267
+        hy.viterbi[d->current_index + 1] = t.viterbi_alignment;
         hy.score = t.val + d->penalty;
         d->hypotheses.push_back(hy);
       } else {
         for (int c = 0; c < L; ++c)
           d->top_sentences_temp[(size_t)i * L + c] = d->top_sentences[(size_t)t.beam_index * L + c];
         d->top_sentences_temp[(size_t)i * L + d->current_index + 1] = t.vocab_index;
+        for (int c = 0; c < L; ++c)
+          d->top_viterbi_temp[(size_t)i * L + c] = d->top_viterbi[(size_t)t.beam_index * L + c];  // :1281-1282
+        d->top_viterbi_temp[(size_t)i * L + d->current_index + 1] = t.viterbi_alignment;
         d->current_indices[i] = t.vocab_index;
         d->new_indicies_changes[i] = t.beam_index;
         d->scores_temp[i] = t.val + d->penalty;
@@ -735,12 +751,16 @@ void orc_decoder_expand(void* p, const float* outputdist, int index) {
     }
   }
   d->top_sentences = d->top_sentences_temp;
+  d->top_viterbi = d->top_viterbi_temp;  // :1301
   d->scores = d->scores_temp;
   d->current_index += 1;
 }
+void orc_decoder_expand(void* p, const float* outputdist, int index) {
+  orc_decoder_expand_viterbi(p, outputdist, index, nullptr);
+}
 
 // finish_current_hypotheses (non-FSA branch), src/decoder.h:672-688.
-void orc_decoder_finish(void* p, const float* outputdist) {
+void orc_decoder_finish_viterbi(void* p, const float* outputdist, const int* viterbi) {
   OrcDecoder* d = (OrcDecoder*)p;
   const int L = d->max_len, V = d->vocab;
   for (int i = 0; i < d->beam; ++i) {
@@ -750,10 +770,26 @@ void orc_decoder_finish(void* p, const float* outputdist) {
     Hypothesis hy;
     hy.words.assign(d->top_sentences.begin() + (size_t)i * L,
                     d->top_sentences.begin() + (size_t)i * L + d->current_index + 2);
+    hy.viterbi.assign(d->top_viterbi.begin() + (size_t)i * L,
+                      d->top_viterbi.begin() + (size_t)i * L + d->current_index + 2);  // :683-684
+    hy.viterbi[d->current_index + 1] = viterbi ? viterbi[i] : -1;
     hy.score = d->scores[i];
     d->hypotheses.push_back(hy);
   }
   d->current_index += 1;
+}
+void orc_decoder_finish(void* p, const float* outputdist) { orc_decoder_finish_viterbi(p, outputdist, nullptr); }
+
+// a finished hypothesis's alignments, one per word
+int orc_decoder_hypothesis_viterbi(void* p, int i, int* out, int cap) {
+  const Hypothesis& hy = ((OrcDecoder*)p)->hypotheses[i];
+  const int n = (int)hy.viterbi.size();
+  for (int k = 0; k < n && k < cap; ++k) out[k] = hy.viterbi[k];
+  return n;
+}
+void orc_decoder_top_viterbi(void* p, int* out) {
+  OrcDecoder* d = (OrcDecoder*)p;
+  memcpy(out, d->top_viterbi.data(), sizeof(int) * d->top_viterbi.size());
 }
 
 void orc_decoder_state(void* p, int* current_indices, int* new_indicies_changes, float* scores, int* top_sentences) {

@@ -40,6 +40,10 @@ def lib():
         _lib.orc_decoder_expand.argtypes = [C.c_void_p, f32p, C.c_int]
         _lib.orc_decoder_finish.argtypes = [C.c_void_p, f32p]
         _lib.orc_decoder_state.argtypes = [C.c_void_p, i32p, i32p, f32p, i32p]
+        _lib.orc_decoder_expand_viterbi.argtypes = [C.c_void_p, f32p, C.c_int, i32p]
+        _lib.orc_decoder_finish_viterbi.argtypes = [C.c_void_p, f32p, i32p]
+        _lib.orc_decoder_hypothesis_viterbi.argtypes = [C.c_void_p, C.c_int, i32p, C.c_int]
+        _lib.orc_decoder_top_viterbi.argtypes = [C.c_void_p, i32p]
         _lib.orc_decoder_current_index.argtypes = [C.c_void_p]
         _lib.orc_decoder_num_hypotheses.argtypes = [C.c_void_p]
         _lib.orc_decoder_hypothesis.argtypes = [C.c_void_p, C.c_int, i32p, C.c_int, f32p]
@@ -324,14 +328,38 @@ class Decoder:
     def init(self):
         lib().orc_decoder_init(self.h)
 
-    def expand(self, outputdist, index):
+    def expand(self, outputdist, index, viterbi=None):
+        """viterbi: the attention layer's Viterbi alignment of every beam column (None: the reference's -1)."""
         od = F(outputdist)
         assert od.shape == (self.vocab, self.beam)
-        lib().orc_decoder_expand(self.h, _p(od), index)
+        if viterbi is None:
+            lib().orc_decoder_expand(self.h, _p(od), index)
+        else:
+            v = np.ascontiguousarray(viterbi, dtype=np.int32)
+            assert v.shape == (self.beam,)
+            lib().orc_decoder_expand_viterbi(self.h, _p(od), index, _p(v, i32p))
 
-    def finish(self, outputdist):
+    def finish(self, outputdist, viterbi=None):
         od = F(outputdist)
-        lib().orc_decoder_finish(self.h, _p(od))
+        if viterbi is None:
+            lib().orc_decoder_finish(self.h, _p(od))
+        else:
+            v = np.ascontiguousarray(viterbi, dtype=np.int32)
+            lib().orc_decoder_finish_viterbi(self.h, _p(od), _p(v, i32p))
+
+    def hypotheses_viterbi(self):
+        """Per finished hypothesis: one alignment per word (entry 0 is the initial -20)."""
+        out = []
+        for i in range(lib().orc_decoder_num_hypotheses(self.h)):
+            v = np.empty(self.max_len + 2, dtype=np.int32)
+            n = lib().orc_decoder_hypothesis_viterbi(self.h, i, _p(v, i32p), v.size)
+            out.append(v[:n].copy())
+        return out
+
+    def top_viterbi(self):
+        v = np.empty((self.beam, self.max_len), dtype=np.int32)
+        lib().orc_decoder_top_viterbi(self.h, _p(v, i32p))
+        return v
 
     def state(self):
         ci = np.empty(self.beam, dtype=np.int32)

@@ -25,20 +25,33 @@ def _random_dist(g, V, cols, peaky=2.0, eof_boost=0.0):
     return np.asfortranarray((e / e.sum(axis=0)).astype(np.float32))
 
 
-def _decode_both(ctx, V, beam, n_sent, steps, max_len, penalty, seed, eof_boost):
+def _decode_both(ctx, V, beam, n_sent, steps, max_len, penalty, seed, eof_boost, viterbi=None):
+    """viterbi: None (not tracked), "given" (random alignments per column and step) or "absent" (tracked, but no
+    alignments handed over: the reference's -1)."""
     g = synth.rng(seed, 21)
     b = ctx.beam_create(beam, V, n_sent, max_len, penalty)
+    d_vit = ctx.empty(n_sent * beam, np.int32) if viterbi == "given" else None
+    if viterbi:
+        ctx.beam_set_viterbi(b, True, d_vit)
+
+    def alignments():
+        if viterbi != "given":
+            return [None] * n_sent
+        v = g.integers(0, 60, size=n_sent * beam).astype(np.int32)
+        d_vit.set(v)
+        return [v[s * beam:(s + 1) * beam] for s in range(n_sent)]
     decs = [o.Decoder(beam, V, max_len, penalty=penalty) for _ in range(n_sent)]
     d_words, d_back = ctx.empty(n_sent * beam, np.int32), ctx.empty(n_sent * beam, np.int32)
     d_prob = ctx.empty((V, n_sent * beam))
     for index in range(steps):
         P = _random_dist(g, V, n_sent * beam, eof_boost=eof_boost)
         d_prob.set(P)
+        vit = alignments()
         ctx.beam_expand(b, d_prob, index, d_words, d_back)
         ctx.sync()
         words, back = d_words.get(), d_back.get()
         for s in range(n_sent):
-            decs[s].expand(P[:, s * beam:(s + 1) * beam], index)
+            decs[s].expand(P[:, s * beam:(s + 1) * beam], index, vit[s])
             st = decs[s].state()
             assert np.array_equal(words[s * beam:(s + 1) * beam], st["current_indices"]), (index, s)
             assert np.array_equal(back[s * beam:(s + 1) * beam] - s * beam, st["new_indicies_changes"]), (index, s)
@@ -48,22 +61,41 @@ def _decode_both(ctx, V, beam, n_sent, steps, max_len, penalty, seed, eof_boost)
             assert np.array_equal(w2, st["current_indices"])
     P = _random_dist(g, V, n_sent * beam)
     d_prob.set(P)
+    vit = alignments()
     ctx.beam_finish(b, d_prob)
     ctx.sync()
     for s in range(n_sent):
-        decs[s].finish(P[:, s * beam:(s + 1) * beam])
+        decs[s].finish(P[:, s * beam:(s + 1) * beam], vit[s])
         want = decs[s].hypotheses()
         got, n = ctx.beam_hypotheses(b, s, cap=len(want) + 8, max_len=max_len)
         assert n == len(want), (s, n, len(want))
         for (gw, gs), (ww, ws) in zip(got, want):
             assert np.array_equal(gw, ww)
             assert gs == pytest.approx(ws, rel=1e-4, abs=1e-5)
+        if viterbi:
+            got_v, nv = ctx.beam_hypotheses_viterbi(b, s, cap=len(want) + 8, max_len=max_len)
+            want_v = decs[s].hypotheses_viterbi()
+            assert nv == len(want_v)
+            for gv, wv in zip(got_v, want_v):
+                assert np.array_equal(gv[:len(wv)], wv), (s, gv, wv)
+    if not viterbi:
+        with pytest.raises(capi.ZrError):
+            ctx.beam_hypotheses_viterbi(b, 0, cap=4, max_len=max_len)
     ctx.beam_destroy(b)
 
 
 @pytest.mark.parametrize("V,beam,n_sent,steps", [(50, 4, 1, 6), (500, 12, 3, 8), (97, 3, 5, 10), (40, 1, 2, 5)])
 def test_beam_against_reference_rules(ctx, V, beam, n_sent, steps):
     _decode_both(ctx, V, beam, n_sent, steps, max_len=steps + 4, penalty=0.0, seed=V + beam, eof_boost=0.0)
+
+
+@pytest.mark.parametrize("mode", ["given", "absent"])
+@pytest.mark.parametrize("V,beam,n_sent,steps,eof_boost", [(60, 5, 4, 9, 3.0), (500, 12, 3, 8, 0.0), (40, 1, 2, 5, 1.0)])
+def test_beam_carries_viterbi_alignments(ctx, V, beam, n_sent, steps, eof_boost, mode):
+    """The alignment histories of all finished hypotheses (those ended by an <EOF> candidate inside expand and those
+    ended by the forced finish), bit-exact against the oracle's decoder; words, scores and back-pointers as without."""
+    _decode_both(ctx, V, beam, n_sent, steps, max_len=steps + 4, penalty=0.2, seed=3 * V + beam, eof_boost=eof_boost,
+                 viterbi=mode)
 
 
 def test_beam_with_frequent_eof_and_penalty(ctx):

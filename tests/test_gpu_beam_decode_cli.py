@@ -31,14 +31,22 @@ def _parse_blocks(text):
     return sents
 
 
-@pytest.mark.parametrize("L,beam,batch", [(2, 4, 3), (1, 3, 8)])
-def test_beam_decode_cli_matches_per_sentence_oracle(tmp_path, L, beam, batch):
+@pytest.mark.parametrize("L,beam,batch,unk", [(2, 4, 3, False), (1, 3, 8, False), (2, 4, 3, True)])
+def test_beam_decode_cli_matches_per_sentence_oracle(tmp_path, L, beam, batch, unk):
+    """unk: with --UNK-decode the side file must hold, per printed hypothesis, the Viterbi alignment at position j+1 for
+    every <UNK> (id 2) at position j (src/decoder.h:1452-1459); the third of the target vocabulary's ids being <UNK>,
+    and the random model producing it now and then, some lines are non-empty (checked)."""
     g = synth.rng(95, L + beam)
     H, D, longest, K = 64, 3, 24, 3
     src_vocab = ["<UNK>"] + mf.make_vocab(79, "s")
     tgt_vocab = ["<START>", "<EOF>", "<UNK>"] + mf.make_vocab(397, "t")
     Vs, Vt = len(src_vocab), len(tgt_vocab)
     m = _model(g, H, Vs, Vt, L)
+    if unk:
+        m["b_soft"][2] += 7.0  # <UNK> likely enough to show up in the hypotheses
+        # window centres and scores that move from step to step, so that the alignments do
+        m["attn"]["v_p"] = m["attn"]["v_p"] * 60
+        m["attn"]["W_a"] = m["attn"]["W_a"] * 16
     model = tmp_path / "model.nn"
     with open(model, "w") as f:
         mf.write_header(f, L, H, tgt_vocab, src_vocab, True, True)
@@ -55,25 +63,38 @@ def test_beam_decode_cli_matches_per_sentence_oracle(tmp_path, L, beam, batch):
     src = [mf.random_sentences(g, src_vocab, 1, n, n)[0] for n in lens]
     sp, out = tmp_path / "src.txt", tmp_path / "out.txt"
     sp.write_text("".join(" ".join(s) + "\n" for s in src))
+    unk_path = tmp_path / "unk.txt"
     r = mf.run_program("beam_decode", ["--beam", beam, "--batch", batch, "--longest-sent", longest, "--attention-width",
-                                       D, "--num-best", K, "--print-score", "--ids", model, sp, out])
+                                       D, "--num-best", K, "--print-score", "--ids"] +
+                       (["--UNK-decode", unk_path] if unk else []) + [model, sp, out])
     assert r.returncode == 0, r.stderr[-2000:]
     got = _parse_blocks(out.read_text())
     assert len(got) == len(src)
+    unk_lines = unk_path.read_text().split("\n")[:-1] if unk else []
+    want_unk, shifted = [], 0
     smap = {w: i for i, w in enumerate(src_vocab)}
     for s, words in enumerate(src):
         ids = np.array([smap.get(w, 0) for w in words][::-1], np.int32)
         S = len(ids)
         steps = min(int(1.5 * S), longest - 2)
-        _, hyps, gap = _oracle_decode(m, ids, S, S, beam, steps, D, 0.0)
+        res = _oracle_decode(m, ids, S, S, beam, steps, D, 0.0, viterbi=unk)
+        hyps, gap = res[1], res[2]
+        vits = res[3] if unk else [None] * len(hyps)
         assert gap > 5e-6, "candidate scores nearly tie (gap %.2e): pick another seed" % gap
-        keep = [(w, sc) for (w, sc) in hyps if len(w) / S > 0.5]
+        keep = [(w, sc, v) for (w, sc), v in zip(hyps, vits) if len(w) / S > 0.5]
         keep.sort(key=lambda t: -t[1])
-        want = keep[:K]
+        want = [(w, sc) for w, sc, _ in keep[:K]]
+        for w, _, v in keep[:K]:
+            want_unk.append("".join("%d " % v[j + 1] for j in range(len(w) - 1) if w[j] == 2))
+            shifted += sum(1 for j in range(len(w) - 1) if w[j] == 2 and v[j] != v[j + 1])
         assert len(got[s]) == len(want), (s, len(got[s]), len(want))
         for (gw, gs), (ww, ws) in zip(got[s], want):
             assert gw == list(ww), (s, gw, list(ww))
             assert gs == pytest.approx(ws, rel=1e-4, abs=1e-4)
+    if unk:
+        assert unk_lines == want_unk
+        assert any(ln for ln in want_unk), "no <UNK> in any hypothesis: the side file shows nothing"
+        assert shifted >= 1, "every <UNK> has the same alignment before and after: position j would pass for j+1"
 
 
 def test_beam_decode_cli_default_output_is_words(tmp_path):

@@ -33,8 +33,10 @@ def _model(g, H, Vs, Vt, L):
     return m
 
 
-def _oracle_decode(m, src_col, src_len, S, beam, steps, D, penalty):
-    """One sentence, minibatch = beam, following forward_prop_source / forward_prop_target / swap_decoding_states."""
+def _oracle_decode(m, src_col, src_len, S, beam, steps, D, penalty, viterbi=False):
+    """One sentence, minibatch = beam, following forward_prop_source / forward_prop_target / swap_decoding_states.
+    viterbi: the attention layer's Viterbi alignments ride along (unk replacement); a fourth value, the alignments
+    of every finished hypothesis, is returned."""
     H, L, Vt = m["src_embed"].shape[0], len(m["src_layers"]), m["D_soft"].shape[0]
     nn, mk = o.vocab_prep(src_col.reshape(S, 1))
     hs, cs = o.lstm_stack_forward(m["src_embed"], m["src_layers"], nn, mk)
@@ -74,7 +76,7 @@ def _oracle_decode(m, src_col, src_len, S, beam, steps, D, penalty):
         n_hyp_before = len(dec.hypotheses())
         frac = att["p_t"] - np.floor(att["p_t"])
         assert np.all((frac > 1e-4) & (frac < 1 - 1e-4)), "p_t on an integer boundary; pick another seed"
-        dec.expand(P, index)
+        dec.expand(P, index, o.attention_viterbi(att["alignments"], att["indices"]) if viterbi else None)
         popped = beam + (len(dec.hypotheses()) - n_hyp_before) + 2  # survivors + <EOF> hypotheses (+ a <START>) + next
         min_gap = min(min_gap, np.min(-np.diff(cand[:popped + 1])))
         st = dec.state()
@@ -83,8 +85,10 @@ def _oracle_decode(m, src_col, src_len, S, beam, steps, D, penalty):
         hp = [np.asfortranarray(a[:, back]) for a in newh]
         cp = [np.asfortranarray(a[:, back]) for a in newc]
         h_tild = np.asfortranarray(att["h_tild"][:, back])
-    _, _, _, P = forward(steps)
-    dec.finish(P)
+    _, _, att, P = forward(steps)
+    dec.finish(P, o.attention_viterbi(att["alignments"], att["indices"]) if viterbi else None)
+    if viterbi:
+        return hist, dec.hypotheses(), min_gap, dec.hypotheses_viterbi()
     return hist, dec.hypotheses(), min_gap
 
 

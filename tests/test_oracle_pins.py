@@ -411,6 +411,62 @@ def test_beam_finish_and_k_best():
     assert [all_scores[i] for i in order] == sorted(all_scores, reverse=True)[:2]
 
 
+@pytest.mark.parametrize("V,beam,steps,seed", [(30, 3, 6, 1), (60, 5, 9, 2), (12, 2, 5, 3)])
+def test_beam_viterbi_histories_follow_the_back_pointers(V, beam, steps, seed):
+    """The alignments a hypothesis carries (src/decoder.h:1266-1282, 683-684), restated without row copies: the word at
+    position j of a hypothesis was chosen at expand step j-1 from some beam column; chase the back pointers
+    (new_indicies_changes) from the hypothesis's last column to find that column at every step, and the alignment at
+    position j must be the one the attention layer reported for THAT column at THAT step.  A history indexed by the new
+    slot instead of the parent column, or shifted by one position, fails.  Position 0 keeps the initial -20."""
+    rng = np.random.default_rng(seed)
+    dec = o.Decoder(beam, V, max_len=steps + 4, penalty=0.0)
+    vit_at, parent_at, words_at, n_hyp = [], [], [], [0]
+    for index in range(steps):
+        logits = rng.normal(0, 2.0, size=(V, beam))
+        logits[1] += 1.0  # <EOF> often near the top, so hypotheses finish at every length
+        P = (np.exp(logits) / np.exp(logits).sum(axis=0)).astype(np.float32)
+        vit = rng.integers(0, 50, size=beam).astype(np.int32)
+        dec.expand(P, index, vit)
+        st = dec.state()
+        vit_at.append(vit)
+        parent_at.append(st["new_indicies_changes"].copy())
+        words_at.append(st["current_indices"].copy())
+        n_hyp.append(len(dec.hypotheses()))
+        # live beam rows: chase from slot i at this step back to step 0
+        tv = dec.top_viterbi()
+        for i in range(beam):
+            if st["current_indices"][i] == -1:
+                continue
+            col = i
+            for j in range(index, -1, -1):
+                col_parent = parent_at[j][col]
+                assert tv[i, j + 1] == vit_at[j][col_parent], (index, i, j)
+                col = col_parent
+            assert tv[i, 0] == -20
+    fin_vit = rng.integers(0, 50, size=beam).astype(np.int32)
+    live = dec.state()["current_indices"].copy()
+    tv_before = dec.top_viterbi()
+    dec.finish(P, fin_vit)
+    hyps, hv = dec.hypotheses(), dec.hypotheses_viterbi()
+    assert len(hyps) == len(hv) > n_hyp[-1] - 1
+    # hypotheses finished by the forced <EOF>: the row of their slot, then the alignment of the last step
+    forced = [i for i in range(beam) if live[i] != -1]
+    for k, i in enumerate(forced):
+        v = hv[n_hyp[-1] + k]
+        assert len(v) == steps + 2 and v[-1] == fin_vit[i] and np.array_equal(v[:-1], tv_before[i, :steps + 1])
+    # hypotheses finished by an <EOF> candidate at step `index`: words identify the parent row unambiguously here only
+    # through the history, so check the invariants that do not need it: length, -20 at 0, every entry one of the
+    # alignments reported at its step
+    for (w, _), v in zip(hyps, hv):
+        assert len(v) == len(w) and v[0] == -20
+        for j in range(1, len(v) - (1 if len(v) == steps + 2 else 0)):
+            assert v[j] in set(vit_at[j - 1].tolist())
+    # no alignments given: the reference fills in -1
+    dec2 = o.Decoder(beam, V, max_len=8)
+    dec2.expand(P, 0)
+    assert set(dec2.top_viterbi()[:, 1].tolist()) <= {-1, -20} and (dec2.top_viterbi()[:, 1] == -1).any()
+
+
 # ----------------------------------------------------------------------------- A6/A7/A11 composition
 def test_stack_forward_is_composition_of_steps():
     H, mb, T, V, L = 8, 3, 4, 17, 2

@@ -41,7 +41,7 @@ SYMBOLS = [
     "zr_lstm_gates", "zr_lstm_stack_forward", "zr_gemm", "zr_softmax_prepare", "zr_softmax_prepare_bf16", "zr_softmax_release", "zr_softmax_forward", "zr_softmax_logprob_f64",
     "zr_softmax_loss", "zr_attn_create", "zr_attn_use_bf16_weights", "zr_attn_destroy", "zr_attn_step", "zr_gather_columns",
     "zr_broadcast_column", "zr_beam_create", "zr_beam_destroy", "zr_beam_init", "zr_beam_expand", "zr_beam_finish", "zr_beam_expand_logits", "zr_beam_finish_logits",
-    "zr_beam_hypotheses", "zr_beam_state",
+    "zr_beam_hypotheses", "zr_beam_state", "zr_beam_set_viterbi", "zr_beam_hypotheses_viterbi",
     "zr_lstm_stack_forward_train", "zr_lstm_train_create", "zr_lstm_train_refresh", "zr_lstm_train_destroy",
     "zr_unstack_gates", "zr_lstm_stack_backward", "zr_lstm_weight_gradients", "zr_embed_gradient",
     "zr_softmax_backward", "zr_sgd_update", "zr_grad_sumsq_accumulate", "zr_sgd_update_clipped", "zr_clip_inplace", "zr_lstm_node_backward", "zr_lstm_node_gradients",
@@ -450,6 +450,17 @@ class Context:
             _chk(n)
         k = min(n, cap)
         return [(words[i, :lens[i]].copy(), float(scores[i])) for i in range(k)], n
+
+    def beam_set_viterbi(self, b, enable, d_viterbi=None):
+        _chk(load().zr_beam_set_viterbi(self.h, b, C.c_int(1 if enable else 0), _vp(d_viterbi)))
+
+    def beam_hypotheses_viterbi(self, b, sentence, cap, max_len):
+        """Rows of max_len alignments, one row per finished hypothesis in beam_hypotheses' order; and their number."""
+        vit = np.full((cap, max_len), -1, dtype=np.int32)
+        n = load().zr_beam_hypotheses_viterbi(self.h, b, C.c_int(sentence), C.c_int(cap), vit.ctypes.data_as(C.c_void_p))
+        if n < 0:
+            _chk(n)
+        return vit[:min(n, cap)], n
 
     def beam_state(self, b, sentence, beam):
         scores = np.zeros(beam, dtype=np.float32)

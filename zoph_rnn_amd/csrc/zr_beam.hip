@@ -31,6 +31,13 @@ struct zr_beam {
   int* d_hyp_len;           // [n_sent][hyp_cap]
   float* d_hyp_score;       // [n_sent][hyp_cap]
   int* d_hyp_count;         // [n_sent]
+  // Viterbi alignments carried with the words (decoder::top_sentences_viterbi, src/decoder.h:230-231), in use once
+  // zr_beam_set_viterbi has switched them on
+  int* d_vit;               // [n_sent][beam][max_len]
+  int* d_vit_tmp;
+  int* d_hyp_vit;           // [n_sent][hyp_cap][max_len]
+  int track_viterbi;        // 0: the three arrays above are not touched
+  const int* d_viterbi_in;  // alignment of every column for the next expand / finish call (null: -1)
   // per step scratch
   float* d_cand_p;          // [n_sent*beam][beam+1]
   int* d_cand_w;            // [n_sent*beam][beam+1]
@@ -251,7 +258,8 @@ __global__ void __launch_bounds__(256)
 beam_merge_kernel(int beam, int K, int max_len, int hyp_cap, float penalty, int index, int current_index,
                   const float* __restrict__ cand_p, const int* __restrict__ cand_w, float* scores,
                   int* words, int* sent, int* sent_tmp, int* hyp_words, int* hyp_len, float* hyp_score,
-                  int* hyp_count, int* out_words, int* out_backptr) {
+                  int* hyp_count, int* out_words, int* out_backptr, const int* __restrict__ vit, int* vit_tmp,
+                  int* hyp_vit, const int* __restrict__ viterbi_in) {
   constexpr int MAXC = KMAX * KMAX;
   __shared__ float c_val[MAXC];
   __shared__ int c_col[MAXC];
@@ -345,6 +353,12 @@ beam_merge_kernel(int beam, int K, int max_len, int hyp_cap, float penalty, int 
     int* hw = hyp_words + ((size_t)s * hyp_cap + h) * max_len;
     const int* src = st + (size_t)s_fin_parent[f] * max_len;
     for (int c = tid; c < current_index + 2 && c < max_len; c += 256) hw[c] = (c == current_index + 1) ? 1 : src[c];
+    if (vit) {  // the parent's alignments, then the alignment of this step's column (src/decoder.h:1266-1267)
+      int* hv = hyp_vit + ((size_t)s * hyp_cap + h) * max_len;
+      const int* vsrc = vit + ((size_t)s * beam + s_fin_parent[f]) * max_len;
+      const int mine = viterbi_in ? viterbi_in[(size_t)s * beam + s_fin_parent[f]] : -1;
+      for (int c = tid; c < current_index + 2 && c < max_len; c += 256) hv[c] = (c == current_index + 1) ? mine : vsrc[c];
+    }
     if (tid == 0) {
       hyp_len[(size_t)s * hyp_cap + h] = current_index + 2;
       hyp_score[(size_t)s * hyp_cap + h] = s_fin_score[f];
@@ -361,6 +375,18 @@ beam_merge_kernel(int beam, int K, int max_len, int hyp_cap, float penalty, int 
     if (c == current_index + 1) v = (parent < 0) ? 0 : s_word[i];
     stt[(size_t)i * max_len + c] = v;
   }
+  if (vit) {
+    // src/decoder.h:1281-1282; an empty-heap filler slot takes row 0 as it is (:1237)
+    const int* vt = vit + (size_t)s * beam * max_len;
+    int* vtt = vit_tmp + (size_t)s * beam * max_len;
+    for (int e = tid; e < beam * lim; e += 256) {
+      const int i = e / lim, c = e % lim;
+      const int parent = s_parent[i];
+      int v = vt[(size_t)(parent < 0 ? 0 : parent) * max_len + c];
+      if (c == current_index + 1 && parent >= 0) v = viterbi_in ? viterbi_in[(size_t)s * beam + parent] : -1;
+      vtt[(size_t)i * max_len + c] = v;
+    }
+  }
   if (tid < beam) {
     const int parent = s_parent[tid];
     out_words[(size_t)s * beam + tid] = s_word[tid];
@@ -375,7 +401,8 @@ beam_merge_kernel(int beam, int K, int max_len, int hyp_cap, float penalty, int 
 __global__ void __launch_bounds__(256)
 beam_finish_kernel(int beam, int V, int max_len, int hyp_cap, float penalty, int current_index,
                    const float* __restrict__ prob, const float* __restrict__ colstats, float* scores, const int* words,
-                   int* sent, int* hyp_words, int* hyp_len, float* hyp_score, int* hyp_count) {
+                   int* sent, int* hyp_words, int* hyp_len, float* hyp_score, int* hyp_count,
+                   const int* __restrict__ vit, int* hyp_vit, const int* __restrict__ viterbi_in) {
   const int s = blockIdx.x;
   const int tid = threadIdx.x;
   int base = hyp_count[s];
@@ -391,6 +418,12 @@ beam_finish_kernel(int beam, int V, int max_len, int hyp_cap, float penalty, int
     if (h < hyp_cap) {
       int* hw = hyp_words + ((size_t)s * hyp_cap + h) * max_len;
       for (int c = tid; c < current_index + 2 && c < max_len; c += 256) hw[c] = (c == current_index + 1) ? 1 : row[c];
+      if (vit) {  // src/decoder.h:683-684
+        int* hv = hyp_vit + ((size_t)s * hyp_cap + h) * max_len;
+        const int* vrow = vit + ((size_t)s * beam + i) * max_len;
+        const int mine = viterbi_in ? viterbi_in[(size_t)s * beam + i] : -1;
+        for (int c = tid; c < current_index + 2 && c < max_len; c += 256) hv[c] = (c == current_index + 1) ? mine : vrow[c];
+      }
       if (tid == 0) {
         hyp_len[(size_t)s * hyp_cap + h] = current_index + 2;
         hyp_score[(size_t)s * hyp_cap + h] = sc;
@@ -407,7 +440,8 @@ beam_finish_kernel(int beam, int V, int max_len, int hyp_cap, float penalty, int
   if (tid == 0) hyp_count[s] = base + added;
 }
 
-__global__ void beam_init_kernel(int n_sent, int beam, int max_len, float* scores, int* words, int* sent, int* hyp_count) {
+__global__ void beam_init_kernel(int n_sent, int beam, int max_len, float* scores, int* words, int* sent, int* hyp_count,
+                                 int* vit) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n_sent * beam) {
     scores[i] = 0.0f;
@@ -415,6 +449,8 @@ __global__ void beam_init_kernel(int n_sent, int beam, int max_len, float* score
   }
   if (i < n_sent) hyp_count[i] = 0;
   for (int c = i; c < n_sent * beam * max_len; c += gridDim.x * blockDim.x) sent[c] = 0;
+  if (vit)
+    for (int c = i; c < n_sent * beam * max_len; c += gridDim.x * blockDim.x) vit[c] = -20;  // src/decoder.h:1335
 }
 
 }  // namespace
@@ -454,6 +490,8 @@ int zr_beam_create(zr_ctx* ctx, int beam, int vocab, int n_sent, int max_len, fl
   const size_t o_sent = take(nb * max_len * 4), o_sent_tmp = take(nb * max_len * 4);
   const size_t o_hw = take((size_t)n_sent * b->hyp_cap * max_len * 4), o_hl = take((size_t)n_sent * b->hyp_cap * 4);
   const size_t o_hs = take((size_t)n_sent * b->hyp_cap * 4), o_hc = take((size_t)n_sent * 4);
+  const size_t o_vit = take(nb * max_len * 4), o_vit_tmp = take(nb * max_len * 4);
+  const size_t o_hv = take((size_t)n_sent * b->hyp_cap * max_len * 4);
   const size_t o_cp = take(nb * K * 4), o_cw = take(nb * K * 4);
   const size_t n_chunks = ((size_t)vocab + kTopkChunk - 1) / kTopkChunk;  // K-lists per column from the first stage
   const size_t o_pp = take(nb * n_chunks * K * 4), o_pw = take(nb * n_chunks * K * 4);
@@ -472,6 +510,11 @@ int zr_beam_create(zr_ctx* ctx, int beam, int vocab, int n_sent, int max_len, fl
   b->d_hyp_len = (int*)(base + o_hl);
   b->d_hyp_score = (float*)(base + o_hs);
   b->d_hyp_count = (int*)(base + o_hc);
+  b->d_vit = (int*)(base + o_vit);
+  b->d_vit_tmp = (int*)(base + o_vit_tmp);
+  b->d_hyp_vit = (int*)(base + o_hv);
+  b->track_viterbi = 0;
+  b->d_viterbi_in = nullptr;
   b->d_cand_p = (float*)(base + o_cp);
   b->d_cand_w = (int*)(base + o_cw);
   b->d_part_p = (float*)(base + o_pp);
@@ -496,7 +539,7 @@ int zr_beam_init(zr_ctx* ctx, zr_beam* b) {
   ZR_CHECK_ARG(b != nullptr, "zr_beam_init: beam object is null");
   b->current_index = 0;
   beam_init_kernel<<<256, 256, 0, ctx->stream>>>(b->n_sent, b->beam, b->max_len, b->d_scores, b->d_words, b->d_sent,
-                                                b->d_hyp_count);
+                                                b->d_hyp_count, b->track_viterbi ? b->d_vit : nullptr);
   ZR_LAUNCH_CHECK("beam_init_kernel");
   return ZR_OK;
 }
@@ -525,11 +568,17 @@ static int beam_expand_impl(zr_ctx* ctx, const char* who, zr_beam* b, const floa
                                                         b->current_index, b->d_cand_p, b->d_cand_w, b->d_scores,
                                                         b->d_words, b->d_sent, b->d_sent_tmp,
                                                         b->d_hyp_words, b->d_hyp_len, b->d_hyp_score, b->d_hyp_count,
-                                                        d_words, d_backptr);
+                                                        d_words, d_backptr, b->track_viterbi ? b->d_vit : nullptr,
+                                                        b->d_vit_tmp, b->d_hyp_vit, b->d_viterbi_in);
   ZR_LAUNCH_CHECK("beam_merge_kernel");
   int* t = b->d_sent;  // the kernel wrote the new rows into d_sent_tmp
   b->d_sent = b->d_sent_tmp;
   b->d_sent_tmp = t;
+  if (b->track_viterbi) {
+    t = b->d_vit;
+    b->d_vit = b->d_vit_tmp;
+    b->d_vit_tmp = t;
+  }
   b->current_index += 1;
   return ZR_OK;
 }
@@ -541,7 +590,8 @@ static int beam_finish_impl(zr_ctx* ctx, const char* who, zr_beam* b, const floa
   beam_finish_kernel<<<b->n_sent, 256, 0, ctx->stream>>>(b->beam, b->vocab, b->max_len, b->hyp_cap, b->penalty,
                                                          b->current_index, d_values, d_colstats, b->d_scores, b->d_words,
                                                          b->d_sent, b->d_hyp_words, b->d_hyp_len, b->d_hyp_score,
-                                                         b->d_hyp_count);
+                                                         b->d_hyp_count, b->track_viterbi ? b->d_vit : nullptr,
+                                                         b->d_hyp_vit, b->d_viterbi_in);
   ZR_LAUNCH_CHECK("beam_finish_kernel");
   b->current_index += 1;
   return ZR_OK;
@@ -584,6 +634,43 @@ int zr_beam_hypotheses(zr_ctx* ctx, zr_beam* b, int sentence, int cap, int* h_wo
                           ctx->stream));
     ZR_HIP(hipMemcpyAsync(h_score, b->d_hyp_score + (size_t)sentence * b->hyp_cap, sizeof(float) * n,
                           hipMemcpyDeviceToHost, ctx->stream));
+    ZR_HIP(hipStreamSynchronize(ctx->stream));
+  }
+  return count;
+}
+
+int zr_beam_set_viterbi(zr_ctx* ctx, zr_beam* b, int enable, const int* d_viterbi) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(b != nullptr, "zr_beam_set_viterbi: beam object is null");
+  ZR_CHECK_ARG(enable || !d_viterbi, "zr_beam_set_viterbi: alignments given with tracking switched off");
+  if (enable && !b->track_viterbi) {
+    ZR_CHECK_ARG(b->current_index == 0, "zr_beam_set_viterbi: tracking can only be switched on before the first step");
+    b->track_viterbi = 1;
+    rc = zr_beam_init(ctx, b);  // fills the alignment rows with -20
+    if (rc) return rc;
+  }
+  if (!enable) b->track_viterbi = 0;
+  b->d_viterbi_in = d_viterbi;
+  return ZR_OK;
+}
+
+int zr_beam_hypotheses_viterbi(zr_ctx* ctx, zr_beam* b, int sentence, int cap, int* h_viterbi) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(b && sentence >= 0 && sentence < b->n_sent && cap >= 0, "zr_beam_hypotheses_viterbi: bad argument");
+  ZR_CHECK_ARG(b->track_viterbi, "zr_beam_hypotheses_viterbi: alignments are not being tracked (zr_beam_set_viterbi)");
+  int count = 0;
+  ZR_HIP(hipMemcpyAsync(&count, b->d_hyp_count + sentence, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
+  ZR_HIP(hipStreamSynchronize(ctx->stream));
+  if (count > b->hyp_cap)
+    return zr_set_error(ZR_EDATA, "zr_beam_hypotheses_viterbi: %d finished hypotheses exceed the capacity %d", count,
+                        b->hyp_cap);
+  const int n = count < cap ? count : cap;
+  if (n > 0) {
+    ZR_CHECK_ARG(h_viterbi != nullptr, "zr_beam_hypotheses_viterbi: null output");
+    ZR_HIP(hipMemcpyAsync(h_viterbi, b->d_hyp_vit + (size_t)sentence * b->hyp_cap * b->max_len,
+                          sizeof(int) * (size_t)n * b->max_len, hipMemcpyDeviceToHost, ctx->stream));
     ZR_HIP(hipStreamSynchronize(ctx->stream));
   }
   return count;

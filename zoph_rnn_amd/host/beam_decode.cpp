@@ -13,8 +13,13 @@
 // hypothesis an optional "-Score: s" line and the hypothesis (ids with --ids, <START> and <EOF> included, as the
 // reference's integer output; words otherwise).
 //
+// --UNK-decode FILE (attention models): the reference's unk-replacement side file (src/decoder.h:1452-1459) -- per
+// output hypothesis one line with, for every <UNK> (id 2) at position j of the hypothesis, the Viterbi alignment stored
+// at position j+1, i.e. a position in the reversed source sentence as the attention layer counts them.
+//
 // Options: --beam B (12)  --batch N (16 sentences side by side)  --longest-sent L (100)  --attention-width D (10)
 //          --penalty P (0)  --min-ratio R (0.5)  --max-ratio R (1.5)  --num-best K (1)  --print-score  --ids  --bf16
+//          --UNK-decode FILE
 #include <cstdio>
 #include <cstdlib>
 #include <iostream>
@@ -28,7 +33,7 @@ static int usage(const char* argv0) {
   std::fprintf(stderr,
                "usage: %s [--beam B] [--batch N] [--longest-sent L] [--attention-width D] [--penalty P]\n"
                "          [--min-ratio R] [--max-ratio R] [--num-best K] [--print-score] [--ids] [--bf16]\n"
-               "          model.nn source.txt output.txt\n",
+               "          [--UNK-decode FILE] model.nn source.txt output.txt\n",
                argv0);
   return 2;
 }
@@ -37,6 +42,7 @@ int main(int argc, char** argv) {
   int beam = 12, batch = 16, longest = 100, D = 10, num_best = 1;
   double penalty = 0, min_ratio = 0.5, max_ratio = 1.5;
   bool print_score = false, ids_out = false, bf16 = false;
+  std::string unk_file;
   std::vector<std::string> pos;
   for (int i = 1; i < argc; i++) {
     const std::string a = argv[i];
@@ -61,6 +67,10 @@ int main(int argc, char** argv) {
     else if (a == "--print-score") print_score = true;
     else if (a == "--ids") ids_out = true;
     else if (a == "--bf16") bf16 = true;
+    else if (a == "--UNK-decode") {
+      if (i + 1 >= argc) return usage(argv[0]);
+      unk_file = argv[++i];
+    }
     else if (a.rfind("--", 0) == 0) return usage(argv[0]);
     else pos.push_back(a);
   }
@@ -102,12 +112,17 @@ int main(int argc, char** argv) {
   for (size_t i = 0; i < sents.size(); i++) by_len[(int)sents[i].size()].push_back((int)i);
 
   BZ_CUDA::bf16_weights = bf16;
+  BZ_CUDA::unk_replacement = !unk_file.empty();  // src/main.cu:410-412
   layer_gpu_info gpu;
   gpu.init(0);
   forward_model<precision> m;
   m.initModel(gpu, info, 1, longest, D);
   m.load_weights(model);
   beam_decoder<precision> dec(m, beam, batch, longest, D, penalty);
+  if (BZ_CUDA::unk_replacement && !dec.track_viterbi) {
+    std::fprintf(stderr, "--UNK-decode needs an attention model\n");
+    return 1;
+  }
   dec.min_decoding_ratio = min_ratio;
   dec.max_decoding_ratio = max_ratio;
 
@@ -141,16 +156,37 @@ int main(int argc, char** argv) {
     }
     out << "\n";
   };
+  std::ofstream unk_out;
+  if (BZ_CUDA::unk_replacement) {
+    unk_out.open(unk_file);
+    if (!unk_out) {
+      std::fprintf(stderr, "cannot write %s\n", unk_file.c_str());
+      return 1;
+    }
+  }
+  auto put_unk = [&](const decoded_hypothesis& h) {  // src/decoder.h:1452-1459
+    if (!BZ_CUDA::unk_replacement) return;
+    for (size_t j = 0; j + 1 < h.words.size(); j++)
+      if (h.words[j] == 2) unk_out << h.viterbi[j + 1] << " ";
+    unk_out << "\n";
+  };
   const bool blocks = num_best > 1 || print_score;
   for (const auto& r : results) {
     if (!blocks) {
-      if (r.empty()) out << "\n"; else put(r[0], true);
+      if (r.empty()) {
+        out << "\n";
+        if (BZ_CUDA::unk_replacement) unk_out << "\n";
+      } else {
+        put(r[0], true);
+        put_unk(r[0]);
+      }
       continue;
     }
     out << "------------------------------------------------\n";
     for (const auto& h : r) {
       if (print_score) out << "-Score: " << h.score << "\n";
       put(h, false);
+      put_unk(h);
     }
     out << "\n";
   }

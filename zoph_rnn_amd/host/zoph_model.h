@@ -926,7 +926,8 @@ class model_trainer {
 // device-side beam directly (it normalises the entries it selects), so nothing vocabulary-sized is copied to the host.  As in the reference's decode path
 // every column runs with mask 1 and a dead beam slot (-1) is fed as word 0.
 struct decoded_hypothesis {
-  std::vector<int> words;  // target ids, <START> ... <EOF>
+  std::vector<int> words;    // target ids, <START> ... <EOF>
+  std::vector<int> viterbi;  // with BZ_CUDA::unk_replacement: one source position per word (entry 0 is -20)
   float score = 0;
 };
 
@@ -946,6 +947,11 @@ class beam_decoder {
   std::vector<dType*> enc_h, enc_c;           // encoder sweep outputs per layer, longest_sent * H * n_sent
   int *d_words = nullptr, *d_words_nn = nullptr, *d_back = nullptr, *d_ones = nullptr, *d_batch_info = nullptr,
       *d_src = nullptr, *d_src_nn = nullptr, *d_src_mask = nullptr, *d_rep = nullptr;
+  // unk replacement (BZ_CUDA::unk_replacement, attention models): the attention step's alignment weights and source
+  // indices of every column, and the Viterbi alignment taken from them (src/attention_node.hpp:225-234)
+  dType* d_align = nullptr;
+  int *d_align_idx = nullptr, *d_viterbi = nullptr;
+  bool track_viterbi = false;
   std::vector<const zr_lstm_weights*> src_w, tgt_w;
   int abandoned_launches = 0;  // batches decoded a second time because a single-launch sweep or step gave up a wait
 
@@ -1024,6 +1030,14 @@ class beam_decoder {
         ZOPH_CALL(zr_attn_prepare(ctx, attn));
     }
     ZOPH_CALL(zr_beam_create(ctx, beam, Vt, n_sent, longest_sent + 3, (float)penalty, &bm));
+    track_viterbi = BZ_CUDA::unk_replacement && attention;
+    if (track_viterbi) {
+      const size_t W = 2 * (size_t)D + 1;
+      d_align = dmalloc<dType>(W * cols);
+      d_align_idx = dmalloc<int>(W * cols);
+      d_viterbi = dmalloc<int>(cols);
+      ZOPH_CALL(zr_beam_set_viterbi(ctx, bm, 1, d_viterbi));
+    }
   }
 
   // forward_prop_target (src/model.hpp:2573-2688): state half p -> half q, logits and column statistics into logits
@@ -1036,8 +1050,10 @@ class beam_decoder {
     std::vector<const dType*> hp(h[p].begin(), h[p].end()), cp(c[p].begin(), c[p].end());
     ZOPH_CALL(zr_decoder_step(ctx, L, tgt_w.data(), m.input_layer_target.d_W, Vt, d_words_nn, hp.data(), cp.data(), feed,
                               d_ones, 0.0f, cols, h[q].data(), c[q].data(), attention ? attn : nullptr, d_batch_info,
-                              attention ? h_tild[q] : nullptr, nullptr, nullptr, nullptr, nullptr, m.softmax_obj.d_D,
+                              attention ? h_tild[q] : nullptr, d_align, d_align_idx, nullptr, nullptr, m.softmax_obj.d_D,
                               m.softmax_obj.d_b_d, Vt, ZR_SOFTMAX_LOGITS, logits));
+    // the alignment of every column, read by the beam call that follows (get_viterbi_alignment_kernel)
+    if (track_viterbi) ZOPH_CALL(zr_attn_viterbi(ctx, attn, d_align, d_align_idx, d_viterbi));
   }
 
   // Decodes up to n_sent sentences whose integerized sources (reversed, no padding) all have the same length S.
@@ -1121,10 +1137,11 @@ class beam_decoder {
 
     out.assign(real, {});
     const int cap = 4 * beam * (steps + 2), max_len = longest_sent + 3;
-    std::vector<int> words((size_t)cap * max_len), lens(cap);
+    std::vector<int> words((size_t)cap * max_len), lens(cap), vit(track_viterbi ? (size_t)cap * max_len : 0);
     std::vector<float> scores(cap);
     for (int s = 0; s < real; s++) {
       int n = zr_beam_hypotheses(ctx, bm, s, cap, words.data(), lens.data(), scores.data());
+      if (n >= 0 && track_viterbi) n = std::min(n, zr_beam_hypotheses_viterbi(ctx, bm, s, cap, vit.data()));
       if (n < 0) {
         std::fprintf(stderr, "zr_beam_hypotheses failed: %s\n", zr_last_error());
         std::exit(EXIT_FAILURE);
@@ -1139,6 +1156,7 @@ class beam_decoder {
       for (int i : order) {
         decoded_hypothesis hyp;
         hyp.words.assign(words.begin() + (size_t)i * max_len, words.begin() + (size_t)i * max_len + lens[i]);
+        if (track_viterbi) hyp.viterbi.assign(vit.begin() + (size_t)i * max_len, vit.begin() + (size_t)i * max_len + lens[i]);
         hyp.score = scores[i];
         out[s].push_back(hyp);
       }
