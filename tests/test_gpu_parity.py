@@ -419,7 +419,10 @@ def _run_attention(ctx, w, hs, batch_info, h_t, mask, D, prepared=False):
 
 @pytest.mark.parametrize("prepared", [False, True])
 @pytest.mark.parametrize("H,mb,S,D", [(64, 6, 9, 2), (100, 8, 20, 10), (52, 33, 12, 12), (30, 5, 7, 3), (1028, 70, 40, 100),
-                                      (2052, 9, 6, 1), (256, 3, 300, 255)])
+                                      (2052, 9, 6, 1), (256, 3, 300, 255),
+                                      # 1024 < H <= 2048: the eight-wave register-resident kernel up to 52 window slots
+                                      # (50 and exactly 52), the two-pass kernel beyond (53)
+                                      (2000, 20, 50, 50), (1500, 12, 52, 30), (2048, 5, 53, 40)])
 def test_attention_against_oracle(ctx, H, mb, S, D, prepared):
     g = synth.rng(13, H + S)
     w = synth.attention_weights(g, H)

@@ -230,26 +230,44 @@ attn_fused_kernel(const float* const* __restrict__ table, int longest_sent, cons
     }
   }
   __syncthreads();
-  // scores: the slots go round the four waves, two at a time per wave so that their loads overlap
+  // scores: the slots go round the four waves, eight at a time per wave and four 16-byte pieces of each per lane, so
+  // that 36 loads of a lane are in flight together (a column's source states are 4 * H * nvalid bytes that only this
+  // workgroup asks for: what it keeps in flight is what it gets per memory latency)
   {
+    constexpr int SG = 8;
     const zr_f32x4* qc = (const zr_f32x4*)(q + (size_t)b * H);
-    for (int j = wave * 2; j < nvalid; j += 8) {
-      const bool two = j + 1 < nvalid;
-      const zr_f32x4* h0 = (const zr_f32x4*)s_src[j];
-      const zr_f32x4* h1 = (const zr_f32x4*)s_src[two ? j + 1 : j];
-      float a0 = 0.0f, a1 = 0.0f;
-      for (int k4 = lane; k4 < H4; k4 += 64) {
-        const zr_f32x4 c = qc[k4];
-        const zr_f32x4 x0 = h0[k4];
-        const zr_f32x4 x1 = h1[k4];
-        a0 += x0.x * c.x + x0.y * c.y + x0.z * c.z + x0.w * c.w;
-        a1 += x1.x * c.x + x1.y * c.y + x1.z * c.z + x1.w * c.w;
+    const zr_f32x4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int j = wave * SG; j < nvalid; j += 4 * SG) {
+      const zr_f32x4* hsrc[SG];
+#pragma unroll
+      for (int u = 0; u < SG; ++u) hsrc[u] = (const zr_f32x4*)s_src[j + u < nvalid ? j + u : j];
+      float a[SG];
+#pragma unroll
+      for (int u = 0; u < SG; ++u) a[u] = 0.0f;
+      for (int k0 = 0; k0 < H4; k0 += 256) {
+        zr_f32x4 c[4], x[SG][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int k4 = k0 + 64 * i + lane;
+          const bool ok = k4 < H4;
+          c[i] = ok ? qc[k4] : zero4;
+#pragma unroll
+          for (int u = 0; u < SG; ++u) x[u][i] = ok ? hsrc[u][k4] : zero4;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (k0 + 64 * i + lane < H4) {
+#pragma unroll
+            for (int u = 0; u < SG; ++u)
+              a[u] += x[u][i].x * c[i].x + x[u][i].y * c[i].y + x[u][i].z * c[i].z + x[u][i].w * c[i].w;
+          }
       }
-      a0 = wave_sum(a0);
-      a1 = wave_sum(a1);
+#pragma unroll
+      for (int u = 0; u < SG; ++u) a[u] = wave_sum(a[u]);
       if (lane == 0) {
-        s_val[j] = a0;
-        if (two) s_val[j + 1] = a1;
+#pragma unroll
+        for (int u = 0; u < SG; ++u)
+          if (j + u < nvalid) s_val[j + u] = a[u];
       }
     }
   }
@@ -275,23 +293,41 @@ attn_fused_kernel(const float* const* __restrict__ table, int longest_sent, cons
     }
   }
   __syncthreads();
-  // context: c[:, b] = sum_j a_j h_s(slot j), four rows per thread, four slots in flight
-  for (int k4 = tid; k4 < H4; k4 += 256) {
-    zr_f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+  // context: c[:, b] = sum_j a_j h_s(slot j): four rows per thread at two places of the column, eight slots of each
+  // in flight (sixteen loads per lane)
+  for (int k0 = 0; k0 < H4; k0 += 512) {
+    const int ka = k0 + tid, kb = k0 + 256 + tid;
+    const bool oka = ka < H4, okb = kb < H4;
+    const zr_f32x4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+    zr_f32x4 acc_a = zero4, acc_b = zero4;
     int j = 0;
-    for (; j + 4 <= nvalid; j += 4) {
-      const zr_f32x4 x0 = ((const zr_f32x4*)s_src[j])[k4];
-      const zr_f32x4 x1 = ((const zr_f32x4*)s_src[j + 1])[k4];
-      const zr_f32x4 x2 = ((const zr_f32x4*)s_src[j + 2])[k4];
-      const zr_f32x4 x3 = ((const zr_f32x4*)s_src[j + 3])[k4];
-      acc += s_val[j] * x0;
-      acc += s_val[j + 1] * x1;
-      acc += s_val[j + 2] * x2;
-      acc += s_val[j + 3] * x3;
+    for (; j + 8 <= nvalid; j += 8) {
+      zr_f32x4 xa[8], xb[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const zr_f32x4* src = (const zr_f32x4*)s_src[j + u];
+        xa[u] = oka ? src[ka] : zero4;
+        xb[u] = okb ? src[kb] : zero4;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        acc_a += s_val[j + u] * xa[u];
+        acc_b += s_val[j + u] * xb[u];
+      }
     }
-    for (; j < nvalid; ++j) acc += s_val[j] * ((const zr_f32x4*)s_src[j])[k4];
-    ((zr_f32x4*)(ctx_out + (size_t)b * H))[k4] = acc;
-    if (ctx_pack) ((zr_f32x4*)ctx_pack)[(size_t)k4 * mb + b] = acc;
+    for (; j < nvalid; ++j) {
+      const zr_f32x4* src = (const zr_f32x4*)s_src[j];
+      if (oka) acc_a += s_val[j] * src[ka];
+      if (okb) acc_b += s_val[j] * src[kb];
+    }
+    if (oka) {
+      ((zr_f32x4*)(ctx_out + (size_t)b * H))[ka] = acc_a;
+      if (ctx_pack) ((zr_f32x4*)ctx_pack)[(size_t)ka * mb + b] = acc_a;
+    }
+    if (okb) {
+      ((zr_f32x4*)(ctx_out + (size_t)b * H))[kb] = acc_b;
+      if (ctx_pack) ((zr_f32x4*)ctx_pack)[(size_t)kb * mb + b] = acc_b;
+    }
   }
 }
 
@@ -339,15 +375,16 @@ __device__ __forceinline__ void wave_sum_many(float (&v)[N]) {
 // them, for every valid slot, in registers -- all loads of a column's source states are in flight together, the
 // scores are formed from the registers, and so is the context, so the source states are read exactly once and nothing
 // is read twice.  Also writes the context k-interleaved ([H/4][mb][4]) for the output product when ctx_pack is given.
-template <int MAXS>
-__global__ void __launch_bounds__(256)
+template <int MAXS, int NT = 256>
+__global__ void __launch_bounds__(NT)
 attn_fused_reg_kernel(const float* const* __restrict__ table, int longest_sent, const float* __restrict__ pre,
                       const float* __restrict__ q, const float* __restrict__ v_p, const int* __restrict__ batch_info,
                       const int* __restrict__ mask01, int H, int mb, int D, float sigma_sq, float* __restrict__ p_t,
                       int* __restrict__ indices, float* __restrict__ align, float* __restrict__ ctx_out,
                       float* __restrict__ ctx_pack, int* __restrict__ flags) {
-  __shared__ float s_red[4];
-  __shared__ float s_part[4][MAXS];
+  constexpr int NW = NT / 64;
+  __shared__ float s_red[NW];
+  __shared__ float s_part[NW][MAXS];
   __shared__ float s_val[MAXS];
   __shared__ const float* s_src[MAXS];
   const int b = blockIdx.x;
@@ -364,7 +401,12 @@ attn_fused_reg_kernel(const float* const* __restrict__ table, int longest_sent, 
     part = v.x * tanhf(t.x) + v.y * tanhf(t.y) + v.z * tanhf(t.z) + v.w * tanhf(t.w);
   }
   const zr_f32x4 qv = ((const zr_f32x4*)(q + (size_t)b * H))[k4];
-  const float sdot = block_sum_256(part, s_red, tid);
+  float sdot = wave_sum(part);
+  if (lane == 0) s_red[wave] = sdot;
+  __syncthreads();
+  sdot = s_red[0];
+#pragma unroll
+  for (int w = 1; w < NW; ++w) sdot += s_red[w];
   const float sig = (float)(1.0 / (1.0 + exp(-1.0 * (double)sdot)));
   const int len = batch_info[b], off = batch_info[mb + b];
   const float p = (float)len * sig;
@@ -376,7 +418,7 @@ attn_fused_reg_kernel(const float* const* __restrict__ table, int longest_sent, 
   nvalid = nvalid < 0 ? 0 : (nvalid > W ? W : nvalid);
   nvalid = nvalid > MAXS ? MAXS : nvalid;  // the host picks MAXS >= min(W, longest_sent)
   if (tid == 0) p_t[b] = p;
-  for (int j = tid; j < W; j += 256) indices[b + (size_t)mb * j] = j < nvalid ? lo + j : -1;
+  for (int j = tid; j < W; j += NT) indices[b + (size_t)mb * j] = j < nvalid ? lo + j : -1;
   if (tid < nvalid) {
     int t = len - 1 - (lo + tid) + off;
     if (t < 0 || t >= longest_sent) {
@@ -398,12 +440,16 @@ attn_fused_reg_kernel(const float* const* __restrict__ table, int longest_sent, 
     if (j0 < nvalid) {  // uniform over the workgroup
       float d[16];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) d[i] = x[j0 + i].x * qv.x + x[j0 + i].y * qv.y + x[j0 + i].z * qv.z + x[j0 + i].w * qv.w;
+      for (int i = 0; i < 16; ++i) {
+        constexpr int kLast = MAXS - 1;
+        const zr_f32x4& xv = x[j0 + i < MAXS ? j0 + i : kLast];  // (MAXS need not be a multiple of 16)
+        d[i] = xv.x * qv.x + xv.y * qv.y + xv.z * qv.z + xv.w * qv.w;
+      }
       wave_sum_many<16>(d);
       float dl = d[0];  // lane i keeps slot j0 + i
 #pragma unroll
       for (int i = 1; i < 16; ++i) dl = lane == i ? d[i] : dl;
-      if (lane < 16) s_part[wave][j0 + lane] = dl;
+      if (lane < 16 && j0 + lane < MAXS) s_part[wave][j0 + lane] = dl;
     }
   }
   __syncthreads();
@@ -412,7 +458,10 @@ attn_fused_reg_kernel(const float* const* __restrict__ table, int longest_sent, 
     float sc = 0.0f;
     const bool v = lane < nvalid;
     if (MAXS <= 64) {
-      if (v) sc = (s_part[0][lane] + s_part[1][lane]) + (s_part[2][lane] + s_part[3][lane]);
+      if (v) {
+        sc = (s_part[0][lane] + s_part[1][lane]) + (s_part[2][lane] + s_part[3][lane]);
+        if (NW == 8) sc += (s_part[4][lane] + s_part[5][lane]) + (s_part[6][lane] + s_part[7][lane]);
+      }
       const float max_val = wave_max(v ? fmaxf(sc, 0.0f) : 0.0f);
       const float e = v ? expf(sc - max_val) : 0.0f;
       const float sum = wave_sum(e);
@@ -650,6 +699,11 @@ static int launch_attn_middle(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, 
     attn_fused_reg_kernel<64><<<mb, 256, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_tanh1, a->d_q, a->v_p,
                                                            d_batch_info, d_mask01, H, mb, D, sigma_sq, pt, idx, align,
                                                            cctx, cpack, ctx->d_flags);
+  else if (H <= 2048 && max_slots <= 52)
+    // eight waves: every thread still holds one 16-byte piece of each slot (2 x 256 registers per lane pair of a SIMD)
+    attn_fused_reg_kernel<52, 512><<<mb, 512, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_tanh1, a->d_q, a->v_p,
+                                                                d_batch_info, d_mask01, H, mb, D, sigma_sq, pt, idx, align,
+                                                                cctx, cpack, ctx->d_flags);
   else
     attn_fused_kernel<<<mb, 256, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_tanh1, a->d_q, a->v_p, d_batch_info,
                                                    d_mask01, H, mb, D, sigma_sq, pt, idx, align, cctx, cpack,
@@ -777,39 +831,52 @@ static int attn_step_impl(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, cons
   // tanh itself) instead of four: bf16 weights, or matrices not registered with zr_attn_prepare.
   const bool vec = (H % 4 == 0) && a->tables_aligned && ((((uintptr_t)cctx | (uintptr_t)a->v_p) & 15u) == 0);
   g.epilogue = vec ? ZR_EPI_STORE : ZR_EPI_TANH;
+  // bf16 snapshots with the fused middle: W_p h and q = W_a^T h as one batch of two products (the snapshots of W_p and
+  // of W_a^T are neighbours, and so are d_tanh1 and d_q), each of which alone would leave half the chip idle
+  const bool both = vec && a->d_bf16 && mb > 32 && H < 8192 && a->d_q == a->d_tanh1 + (size_t)H * mb && per % 8 == 0;
+  if (both) {
+    g.batch = 2;
+    g.strideA = (long long)per;
+    g.strideC = (long long)H * mb;
+  }
   rc = zr_gemm_launch(ctx, g);
   if (rc) return rc;
-  if (!vec) {
-    attn_window_kernel<<<mb, 64, 0, ctx->stream>>>(a->d_tanh1, a->v_p, d_batch_info, d_mask01, H, mb, D, pt, idx);
-    ZR_LAUNCH_CHECK("attn_window_kernel");
-  }
-  // q = W_a^T h  (:195)
-  g.A[0] = a->W_a;
-  g.trans_a = 1;
-  if (a->d_bf16) {
-    g.A[0] = (const float*)(a->d_bf16 + per);  // already transposed
-    g.trans_a = 0;
-  }
-  g.C = a->d_q;
-  g.epilogue = ZR_EPI_STORE;
-  rc = zr_gemm_launch(ctx, g);
-  if (rc) return rc;
-  if (vec) {
+  if (both) {
     rc = launch_attn_middle(ctx, a, d_batch_info, d_mask01, pt, idx, align, cctx, nullptr);
     if (rc) return rc;
   } else {
-    const long long slots = (long long)mb * W;
-    const unsigned sgrid = (unsigned)((slots + 3) / 4);
-    attn_score_kernel<false><<<sgrid, 256, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_q, idx, d_batch_info, H,
-                                                             mb, W, align, ctx->d_flags);
-    ZR_LAUNCH_CHECK("attn_score_kernel");
-    const float sigma_sq = (float)((D * D) / 4.0);  // attention_node.hpp:50
-    attn_align_kernel<<<mb, 64, 0, ctx->stream>>>(align, idx, pt, mb, W, sigma_sq);
-    ZR_LAUNCH_CHECK("attn_align_kernel");
-    dim3 cg((H + 63) / 64, mb);
-    attn_context_kernel<false><<<cg, 64, 0, ctx->stream>>>(a->d_table, a->longest_sent, align, idx, d_batch_info, H, mb,
-                                                           W, cctx);
-    ZR_LAUNCH_CHECK("attn_context_kernel");
+    if (!vec) {
+      attn_window_kernel<<<mb, 64, 0, ctx->stream>>>(a->d_tanh1, a->v_p, d_batch_info, d_mask01, H, mb, D, pt, idx);
+      ZR_LAUNCH_CHECK("attn_window_kernel");
+    }
+    // q = W_a^T h  (:195)
+    g.A[0] = a->W_a;
+    g.trans_a = 1;
+    if (a->d_bf16) {
+      g.A[0] = (const float*)(a->d_bf16 + per);  // already transposed
+      g.trans_a = 0;
+    }
+    g.C = a->d_q;
+    g.epilogue = ZR_EPI_STORE;
+    rc = zr_gemm_launch(ctx, g);
+    if (rc) return rc;
+    if (vec) {
+      rc = launch_attn_middle(ctx, a, d_batch_info, d_mask01, pt, idx, align, cctx, nullptr);
+      if (rc) return rc;
+    } else {
+      const long long slots = (long long)mb * W;
+      const unsigned sgrid = (unsigned)((slots + 3) / 4);
+      attn_score_kernel<false><<<sgrid, 256, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_q, idx, d_batch_info, H,
+                                                               mb, W, align, ctx->d_flags);
+      ZR_LAUNCH_CHECK("attn_score_kernel");
+      const float sigma_sq = (float)((D * D) / 4.0);  // attention_node.hpp:50
+      attn_align_kernel<<<mb, 64, 0, ctx->stream>>>(align, idx, pt, mb, W, sigma_sq);
+      ZR_LAUNCH_CHECK("attn_align_kernel");
+      dim3 cg((H + 63) / 64, mb);
+      attn_context_kernel<false><<<cg, 64, 0, ctx->stream>>>(a->d_table, a->longest_sent, align, idx, d_batch_info, H, mb,
+                                                             W, cctx);
+      ZR_LAUNCH_CHECK("attn_context_kernel");
+    }
   }
   // h~ = tanh(W_c1 c + W_c2 h + b) * mask  (:354-379) as one two-segment GEMM with a fused epilogue
   ZrGemmDesc o = {};

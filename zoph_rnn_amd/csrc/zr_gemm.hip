@@ -181,7 +181,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& a, int m0, int n0, boo
       const float* xcol[TN];
 #pragma unroll
       for (int tm = 0; tm < TM; ++tm) {
-        wbase[tm] = (const unsigned short*)a.A[s];
+        wbase[tm] = (const unsigned short*)a.A[s] + (long long)z * a.strideA;  // (strideA counts bf16 elements here)
         woff[tm] = (unsigned)(8LL * rows[tm] + 8LL * half * a.lda[s]);
       }
       const unsigned short* xlo[TN];
@@ -1181,9 +1181,12 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
       ZR_CHECK_ARG(d.K[s] > 0, "gemm: K[%d] = %d", s, d.K[s]);
       ZR_CHECK_ARG(d.groups > 0 || (d.A[s] && d.B[s]), "gemm: null operand in segment %d", s);
       ZR_CHECK_ARG(d.lda[s] >= (d.trans_a ? d.K[s] : d.M), "gemm: lda[%d] = %d too small", s, d.lda[s]);
-      ZR_CHECK_ARG(!d.a_pack || (!d.trans_a && (d.batch == 1 || d.a_pack == 1) && d.lda[s] % 32 == 0 &&
-                                 8LL * d.lda[s] + 8LL * d.M < (1LL << 31)),
-                   "gemm: packed operand A of segment %d: needs no transpose, lda a multiple of 32 (bf16: one batch)", s);
+      ZR_CHECK_ARG(!d.a_pack || (!d.trans_a && d.lda[s] % 32 == 0 && 8LL * d.lda[s] + 8LL * d.M < (1LL << 31)),
+                   "gemm: packed operand A of segment %d: needs no transpose, lda a multiple of 32", s);
+      // a batch over bf16 matrices: one segment, plain store, and a shape the tile kernel serves (strideA in bf16 elements)
+      ZR_CHECK_ARG(d.a_pack != 2 || d.batch == 1 ||
+                       (d.nseg == 1 && d.epilogue == ZR_EPI_STORE && d.M < 8192 && d.strideA % 8 == 0),
+                   "gemm: a batch of bf16 products needs one segment, the store epilogue and M < 8192");
       ZR_CHECK_ARG(d.a_pack != 2 || d.K[s] % 16 == 0, "gemm: bf16 operand A needs K %% 16 == 0 (K[%d] = %d)", s, d.K[s]);
       ZR_CHECK_ARG(d.ldb[s] >= d.K[s], "gemm: ldb[%d] = %d < K = %d", s, d.ldb[s], d.K[s]);
       // per-lane weight offsets are 32-bit element indices
@@ -1275,16 +1278,20 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
       if (tn == 3) return launch_rows<3, ZR_A_PACK8_BF16>(ctx, ga, d.epilogue, n_tiles);
       return launch_rows<4, ZR_A_PACK8_BF16>(ctx, ga, d.epilogue, n_tiles);
     }
-    if (d.N <= 32) {
+    // 64 x 32 tiles for a narrow batch, and where 64 x 64 tiles would leave more than a third of the chip idle (the
+    // attention output product at 2000 x 256: 128 tiles of 64 x 64 against 256 of 64 x 32)
+    const long long wide_tiles = (long long)((ga.M + 63) / 64) * ((ga.N + 63) / 64) * d.batch;
+    const int cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
+    if (d.N <= 32 || wide_tiles * 3 <= 2LL * cus) {
       ga.m_tiles = (ga.M + 63) / 64;
       ga.n_tiles = (ga.N + 31) / 32;
-      if (one_term) return launch_epi<2, 1, 4, 1, ZR_A_PACK8_BF16_1T, true, 2>(ctx, ga, 1, d.epilogue);
-      return launch_epi<2, 1, 4, 1, ZR_A_PACK8_BF16, true, 2>(ctx, ga, 1, d.epilogue);
+      if (one_term) return launch_epi<2, 1, 4, 1, ZR_A_PACK8_BF16_1T, true, 2>(ctx, ga, d.batch, d.epilogue);
+      return launch_epi<2, 1, 4, 1, ZR_A_PACK8_BF16, true, 2>(ctx, ga, d.batch, d.epilogue);
     }
     ga.m_tiles = (ga.M + 63) / 64;
     ga.n_tiles = (ga.N + 63) / 64;
-    if (one_term) return launch_epi<2, 2, 4, 1, ZR_A_PACK8_BF16_1T, true, 2>(ctx, ga, 1, d.epilogue);
-    return launch_epi<2, 2, 4, 1, ZR_A_PACK8_BF16, true, 2>(ctx, ga, 1, d.epilogue);
+    if (one_term) return launch_epi<2, 2, 4, 1, ZR_A_PACK8_BF16_1T, true, 2>(ctx, ga, d.batch, d.epilogue);
+    return launch_epi<2, 2, 4, 1, ZR_A_PACK8_BF16, true, 2>(ctx, ga, d.batch, d.epilogue);
   }
   if (d.a_pack) {
     // Activations too: a k-interleaved copy in scratch turns their loads (16 bytes from each of 32 lines per

@@ -116,7 +116,7 @@ struct ZrGemmDesc {
   int ldb[3];
   float* C;
   int ldc;
-  // batch (blockIdx.z): A/C/bias advance by these strides (elements); B is shared
+  // batch (blockIdx.z): A/C/bias advance by these strides (elements; bf16 elements for a bf16 A); B is shared
   int batch;
   long long strideA, strideC, strideBias;
   const float* bias;  // per row m (may be NULL)
