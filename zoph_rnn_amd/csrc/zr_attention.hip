@@ -7,6 +7,7 @@
 #include <math.h>
 
 #include "zr_internal.h"
+#include "zr_mfma_core.h"
 
 
 namespace {
@@ -171,6 +172,19 @@ attn_context_kernel(const float* const* __restrict__ table, int longest_sent, co
     o[0] = acc[0];
 }
 
+// The four consecutive rows 4*k4 .. 4*k4+3 of column b as bf16 terms, into arrays laid out [H/8][mb][8] (what the bf16
+// products read: zr_split_pack_x_kernel's layout and its hi / lo split).  lo may be null (single-term mode).
+__device__ __forceinline__ void store_bf16_terms(const zr_f32x4& v, int k4, int b, int mb, unsigned short* hi,
+                                                 unsigned short* lo) {
+  typedef unsigned zr_u32x2 __attribute__((ext_vector_type(2)));
+  unsigned h0, l0, h1, l1;
+  zr_split_bf16_pair(v.x, v.y, h0, l0);
+  zr_split_bf16_pair(v.z, v.w, h1, l1);
+  const size_t o = ((size_t)(k4 >> 1) * mb + b) * 8 + (size_t)(k4 & 1) * 4;
+  *(zr_u32x2*)(hi + o) = zr_u32x2{h0, h1};
+  if (lo) *(zr_u32x2*)(lo + o) = zr_u32x2{l0, l1};
+}
+
 __device__ __forceinline__ float block_sum_256(float v, float* s_red, int tid) {
   v = wave_sum(v);
   __syncthreads();  // the previous use of s_red is over
@@ -190,7 +204,8 @@ attn_fused_kernel(const float* const* __restrict__ table, int longest_sent, cons
                   const float* __restrict__ q, const float* __restrict__ v_p, const int* __restrict__ batch_info,
                   const int* __restrict__ mask01, int H, int mb, int D, float sigma_sq, float* __restrict__ p_t,
                   int* __restrict__ indices, float* __restrict__ align, float* __restrict__ ctx_out,
-                  float* __restrict__ ctx_pack, int* __restrict__ flags) {
+                  float* __restrict__ ctx_pack, unsigned short* __restrict__ ctx_hi,
+                  unsigned short* __restrict__ ctx_lo, int* __restrict__ flags) {
   constexpr int kMaxSlots = 512;
   __shared__ float s_red[4];
   __shared__ float s_val[kMaxSlots];         // scores, then alignment weights, of the valid slots
@@ -323,10 +338,12 @@ attn_fused_kernel(const float* const* __restrict__ table, int longest_sent, cons
     if (oka) {
       ((zr_f32x4*)(ctx_out + (size_t)b * H))[ka] = acc_a;
       if (ctx_pack) ((zr_f32x4*)ctx_pack)[(size_t)ka * mb + b] = acc_a;
+      if (ctx_hi) store_bf16_terms(acc_a, ka, b, mb, ctx_hi, ctx_lo);
     }
     if (okb) {
       ((zr_f32x4*)(ctx_out + (size_t)b * H))[kb] = acc_b;
       if (ctx_pack) ((zr_f32x4*)ctx_pack)[(size_t)kb * mb + b] = acc_b;
+      if (ctx_hi) store_bf16_terms(acc_b, kb, b, mb, ctx_hi, ctx_lo);
     }
   }
 }
@@ -381,7 +398,8 @@ attn_fused_reg_kernel(const float* const* __restrict__ table, int longest_sent, 
                       const float* __restrict__ q, const float* __restrict__ v_p, const int* __restrict__ batch_info,
                       const int* __restrict__ mask01, int H, int mb, int D, float sigma_sq, float* __restrict__ p_t,
                       int* __restrict__ indices, float* __restrict__ align, float* __restrict__ ctx_out,
-                      float* __restrict__ ctx_pack, int* __restrict__ flags) {
+                      float* __restrict__ ctx_pack, unsigned short* __restrict__ ctx_hi,
+                      unsigned short* __restrict__ ctx_lo, int* __restrict__ flags) {
   constexpr int NW = NT / 64;
   __shared__ float s_red[NW];
   __shared__ float s_part[NW][MAXS];
@@ -483,6 +501,7 @@ attn_fused_reg_kernel(const float* const* __restrict__ table, int longest_sent, 
       if (j < nvalid) acc += s_val[j] * x[j];
     ((zr_f32x4*)(ctx_out + (size_t)b * H))[k4] = acc;
     if (ctx_pack) ((zr_f32x4*)ctx_pack)[(size_t)k4 * mb + b] = acc;
+    if (ctx_hi) store_bf16_terms(acc, k4, b, mb, ctx_hi, ctx_lo);
   }
 }
 
@@ -563,7 +582,7 @@ int zr_attn_use_bf16_weights(zr_ctx* ctx, zr_attn* a) {
   const size_t per = (size_t)H * ldp;
   if (!a->d_bf16) {
     // the four matrices, then room for h_t as two bf16 terms (split once per step for its three products)
-    if (hipMalloc((void**)&a->d_bf16, sizeof(unsigned short) * (4 * per + 2 * (size_t)H * a->mb)) != hipSuccess) {
+    if (hipMalloc((void**)&a->d_bf16, sizeof(unsigned short) * (4 * per + 4 * (size_t)H * a->mb)) != hipSuccess) {
       (void)hipGetLastError();
       a->d_bf16 = nullptr;
       return zr_set_error(ZR_ENOMEM, "zr_attn_use_bf16_weights: allocation failed");
@@ -683,30 +702,31 @@ int zr_decoder_step(zr_ctx* ctx, int nl, const zr_lstm_weights* const layers[], 
 // Everything between the projections and the output product in one launch (d_tanh1 holds W_p h BEFORE the tanh, d_q
 // holds W_a^T h): the register-resident kernel up to H = 1024 and 64 window slots, the two-pass one beyond.
 static int launch_attn_middle(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, const int* d_mask01, float* pt, int* idx,
-                              float* align, float* cctx, float* cpack) {
+                              float* align, float* cctx, float* cpack, unsigned short* chi = nullptr,
+                              unsigned short* clo = nullptr) {
   const int H = a->H, mb = a->mb, D = a->D, W = 2 * D + 1;
   const float sigma_sq = (float)((D * D) / 4.0);  // attention_node.hpp:50
   const int max_slots = W < a->longest_sent ? W : a->longest_sent;
   if (H <= 1024 && max_slots <= 16)
     attn_fused_reg_kernel<16><<<mb, 256, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_tanh1, a->d_q, a->v_p,
                                                            d_batch_info, d_mask01, H, mb, D, sigma_sq, pt, idx, align,
-                                                           cctx, cpack, ctx->d_flags);
+                                                           cctx, cpack, chi, clo, ctx->d_flags);
   else if (H <= 1024 && max_slots <= 32)
     attn_fused_reg_kernel<32><<<mb, 256, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_tanh1, a->d_q, a->v_p,
                                                            d_batch_info, d_mask01, H, mb, D, sigma_sq, pt, idx, align,
-                                                           cctx, cpack, ctx->d_flags);
+                                                           cctx, cpack, chi, clo, ctx->d_flags);
   else if (H <= 1024 && max_slots <= 64)
     attn_fused_reg_kernel<64><<<mb, 256, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_tanh1, a->d_q, a->v_p,
                                                            d_batch_info, d_mask01, H, mb, D, sigma_sq, pt, idx, align,
-                                                           cctx, cpack, ctx->d_flags);
+                                                           cctx, cpack, chi, clo, ctx->d_flags);
   else if (H <= 2048 && max_slots <= 52)
     // eight waves: every thread still holds one 16-byte piece of each slot (2 x 256 registers per lane pair of a SIMD)
     attn_fused_reg_kernel<52, 512><<<mb, 512, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_tanh1, a->d_q, a->v_p,
                                                                 d_batch_info, d_mask01, H, mb, D, sigma_sq, pt, idx, align,
-                                                                cctx, cpack, ctx->d_flags);
+                                                                cctx, cpack, chi, clo, ctx->d_flags);
   else
     attn_fused_kernel<<<mb, 256, 0, ctx->stream>>>(a->d_table, a->longest_sent, a->d_tanh1, a->d_q, a->v_p, d_batch_info,
-                                                   d_mask01, H, mb, D, sigma_sq, pt, idx, align, cctx, cpack,
+                                                   d_mask01, H, mb, D, sigma_sq, pt, idx, align, cctx, cpack, chi, clo,
                                                    ctx->d_flags);
   ZR_LAUNCH_CHECK("attn_fused_kernel");
   return ZR_OK;
@@ -841,8 +861,15 @@ static int attn_step_impl(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, cons
   }
   rc = zr_gemm_launch(ctx, g);
   if (rc) return rc;
+  // with bf16 matrices the fused middle also leaves the context as bf16 terms for the output product
+  unsigned short* c_hi = nullptr;
+  unsigned short* c_lo = nullptr;
+  if (vec && h_hi && H % 8 == 0) {
+    c_hi = a->d_bf16 + 4 * per + 2 * (size_t)H * mb;
+    c_lo = h_lo ? c_hi + (size_t)H * mb : nullptr;
+  }
   if (both) {
-    rc = launch_attn_middle(ctx, a, d_batch_info, d_mask01, pt, idx, align, cctx, nullptr);
+    rc = launch_attn_middle(ctx, a, d_batch_info, d_mask01, pt, idx, align, cctx, nullptr, c_hi, c_lo);
     if (rc) return rc;
   } else {
     if (!vec) {
@@ -861,7 +888,7 @@ static int attn_step_impl(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, cons
     rc = zr_gemm_launch(ctx, g);
     if (rc) return rc;
     if (vec) {
-      rc = launch_attn_middle(ctx, a, d_batch_info, d_mask01, pt, idx, align, cctx, nullptr);
+      rc = launch_attn_middle(ctx, a, d_batch_info, d_mask01, pt, idx, align, cctx, nullptr, c_hi, c_lo);
       if (rc) return rc;
     } else {
       const long long slots = (long long)mb * W;
@@ -899,6 +926,8 @@ static int attn_step_impl(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, cons
   }
   o.B[1] = d_h_t;
   o.ldb[1] = H;
+  o.Bhi[0] = c_hi;
+  o.Blo[0] = c_lo;
   o.Bhi[1] = h_hi;
   o.Blo[1] = h_lo;
   o.C = d_htild;
