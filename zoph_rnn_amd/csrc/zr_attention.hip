@@ -582,7 +582,7 @@ int zr_attn_use_bf16_weights(zr_ctx* ctx, zr_attn* a) {
   const size_t per = (size_t)H * ldp;
   if (!a->d_bf16) {
     // the four matrices, then room for h_t as two bf16 terms (split once per step for its three products)
-    if (hipMalloc((void**)&a->d_bf16, sizeof(unsigned short) * (4 * per + 4 * (size_t)H * a->mb)) != hipSuccess) {
+    if (hipMalloc((void**)&a->d_bf16, sizeof(unsigned short) * (4 * per + 6 * (size_t)H * a->mb)) != hipSuccess) {
       (void)hipGetLastError();
       a->d_bf16 = nullptr;
       return zr_set_error(ZR_ENOMEM, "zr_attn_use_bf16_weights: allocation failed");
@@ -696,7 +696,7 @@ int zr_decoder_step(zr_ctx* ctx, int nl, const zr_lstm_weights* const layers[], 
                       (pack32 || split16) && wrote, packed ? attn->d_htpack : nullptr);
   if (rc) return rc;
   return zr_softmax_forward_packed(ctx, d_D, d_b_d, V_out, attn->H, d_htild, packed ? attn->d_htpack : nullptr, mb, mode,
-                                   d_out, nullptr);
+                                   d_out, nullptr, attn->htild_hi, attn->htild_lo);
 }
 
 // Everything between the projections and the output product in one launch (d_tanh1 holds W_p h BEFORE the tanh, d_q
@@ -739,6 +739,7 @@ static int attn_step_impl(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, cons
   if (rc) return rc;
   ZR_CHECK_ARG(a != nullptr, "zr_attn_step: attention object is null");
   ZR_CHECK_ARG(d_batch_info && d_h_t && d_mask01 && d_htild, "zr_attn_step: null pointer");
+  a->htild_hi = a->htild_lo = nullptr;
   const int H = a->H, mb = a->mb, D = a->D, W = 2 * D + 1;
   float* align = d_alignments ? d_alignments : a->d_align;
   int* idx = d_indices ? d_indices : a->d_idx;
@@ -936,6 +937,12 @@ static int attn_step_impl(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, cons
   o.bias = a->out_bias;
   o.mask = d_mask01;
   o.epilogue = ZR_EPI_TANH_BIAS_MASK;
+  if (c_hi) {  // bf16 matrices: h~ also as bf16 terms, for a bf16 output layer behind this step
+    o.Chi = a->d_bf16 + 4 * per + 4 * (size_t)H * mb;
+    o.Clo = c_lo ? o.Chi + (size_t)H * mb : nullptr;
+    a->htild_hi = o.Chi;
+    a->htild_lo = o.Clo;
+  }
   return zr_gemm_launch(ctx, o);
 }
 

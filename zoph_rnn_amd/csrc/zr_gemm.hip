@@ -22,6 +22,8 @@ struct GemmArgs {
   const int* mask;
   float* partials;
   float* Cpack;          // ZR_EPI_TANH_BIAS_MASK: second, k-interleaved copy of the result (null: none)
+  unsigned short* Chi;   // ZR_EPI_TANH_BIAS_MASK: the result as bf16 terms, [M/8][N][8] (null: none); Clo may be null
+  unsigned short* Clo;
   int m_tiles, n_tiles;  // wave tiles along M and N
   int b_pack4;           // B segments are k-interleaved copies: element (k, n) at ((k/4)*N + n)*4 + k%4
   // bf16 weights: B[s] is the bf16 "hi" array and Blo[s] the "lo" array of the split activations, both
@@ -288,6 +290,12 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& a, int m0, int n0, boo
           const float t = tanhf(v + bias[m]) * (float)a.mask[n];
           C[(long long)n * a.ldc + m] = t;
           if (a.Cpack) a.Cpack[((long long)(m >> 2) * a.N + n) * 4 + (m & 3)] = t;
+          if (a.Chi) {  // the split of zr_split_bf16_pair, element by element
+            const __bf16 hb = (__bf16)t;
+            const long long o = ((long long)(m >> 3) * a.N + n) * 8 + (m & 7);
+            a.Chi[o] = __builtin_bit_cast(unsigned short, hb);
+            if (a.Clo) a.Clo[o] = __builtin_bit_cast(unsigned short, (__bf16)(t - (float)hb));
+          }
         }
       }
     }
@@ -1221,6 +1229,11 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
   ga.mask = d.mask;
   ga.partials = d.partials;
   ga.Cpack = d.Cpack;
+  ga.Chi = d.Chi;
+  ga.Clo = d.Clo;
+  ZR_CHECK_ARG(!d.Chi || (d.epilogue == ZR_EPI_TANH_BIAS_MASK && d.batch <= 1 && d.groups == 0 && d.M % 8 == 0),
+               "gemm: bf16 terms of the result need the tanh-bias-mask epilogue, one batch and M %% 8 == 0");
+  ZR_CHECK_ARG(!d.Clo || d.Chi, "gemm: Clo without Chi");
   ZR_CHECK_ARG(!d.Cpack || (d.epilogue == ZR_EPI_TANH_BIAS_MASK && d.batch <= 1 && d.groups == 0),
                "gemm: a k-interleaved second result needs the tanh-bias-mask epilogue and a single problem");
   ga.accum = d.accumulate;

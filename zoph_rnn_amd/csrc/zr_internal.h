@@ -125,6 +125,10 @@ struct ZrGemmDesc {
   float* partials;  // ZR_EPI_SOFTMAX_PARTIAL: [N][ceil(M/32)][2] floats (contiguous per column)
   float* Cpack;     // ZR_EPI_TANH_BIAS_MASK, single batch: the result is also stored k-interleaved, element (m, n) at
                     // ((m/4)*N + n)*4 + m%4 -- the layout a following product with b_packed reads (null: not wanted)
+  // ZR_EPI_TANH_BIAS_MASK, single batch, M % 8 == 0: the result also as bf16 terms (hi, and lo = the residue, or null),
+  // each laid out [M/8][N][8] -- what a following product on bf16 weights reads as Bhi / Blo (null: not wanted)
+  unsigned short* Chi;
+  unsigned short* Clo;
   int accumulate;   // ZR_EPI_STORE only: C += product (+ bias) instead of C = ...
   // groups > 0: that many independent problems of the same shape in one launch (at most 8; one segment, plain store
   // epilogue, no bias): problem g multiplies gA[g] (instead of A[0]) with gB[g] (instead of B[0]) into gC[g]
@@ -189,7 +193,8 @@ int zr_lstm_decoder_step_packed(zr_ctx* ctx, int nl, const zr_lstm_weights* cons
                                 const float* d_htild, const int* d_mask01, float clip_threshold, int mb,
                                 float* const d_h[], float* const d_c[], float* d_hp_top, int* wrote_hp_top);
 int zr_softmax_forward_packed(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h,
-                              const float* d_h_packed, int mb, int mode, float* d_out, float* d_logits_scratch);
+                              const float* d_h_packed, int mb, int mode, float* d_out, float* d_logits_scratch,
+                              const unsigned short* d_h_hi = nullptr, const unsigned short* d_h_lo = nullptr);
 
 // The attention layer's handle (zr_attention.hip; the backward pass lives in zr_backward.hip).
 struct zr_attn {
@@ -208,6 +213,10 @@ struct zr_attn {
   int ldp32, kp32;
   float *d_hpack, *d_cpack;  // k-interleaved copies ([H/4][mb][4]) of h_t and of the context (inside d_pack32's block)
   float* d_htpack;           // the same of h~, written by the output product for zr_decoder_step (same block)
+  // bf16 matrices: h~ of the last step as bf16 terms ([H/8][mb][8], inside d_bf16's block), written by the output
+  // product for a bf16 output layer behind it in zr_decoder_step; null when the last step did not write them
+  const unsigned short* htild_hi;
+  const unsigned short* htild_lo;
   float** d_err_table;       // zr_attn_set_error_tables: device copy of the source-state error pointers (null: none)
 };
 

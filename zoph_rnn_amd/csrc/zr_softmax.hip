@@ -167,7 +167,8 @@ softmax_loss_kernel(const float* __restrict__ logits, int V, int mb, const doubl
 // d_h_packed: optional k-interleaved copy of d_h ([H/4][mb][4]); used when the product runs on the registered fp32 copy
 // of D and H % 8 == 0 (the product then skips its own re-layout of d_h).
 int logits_with_partials(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int mb,
-                         float* d_logits, float** partials_out, int* nblocks_out, const float* d_h_packed = nullptr) {
+                         float* d_logits, float** partials_out, int* nblocks_out, const float* d_h_packed = nullptr,
+                         const unsigned short* d_h_hi = nullptr, const unsigned short* d_h_lo = nullptr) {
   const int nblocks = zr_softmax_partial_blocks(V);
   void* scratch = nullptr;
   // partials [mb][nblocks][2] followed by column stats (2 doubles per column, also used as 2 floats)
@@ -198,6 +199,10 @@ int logits_with_partials(zr_ctx* ctx, const float* d_D, const float* d_b_d, int 
   if (d_h_packed && d.a_pack == 1 && H % 8 == 0 && (((uintptr_t)d_h_packed & 15u) == 0)) {
     d.B[0] = d_h_packed;
     d.b_packed = 1;
+  }
+  if (d_h_hi && d.a_pack == 2) {  // the producer of h has left its bf16 terms (the GEMM takes them when they suffice)
+    d.Bhi[0] = d_h_hi;
+    d.Blo[0] = d_h_lo;
   }
   d.C = d_logits;
   d.ldc = V;
@@ -301,7 +306,8 @@ int zr_softmax_forward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V,
 }  // extern "C"
 
 int zr_softmax_forward_packed(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h,
-                              const float* d_h_packed, int mb, int mode, float* d_out, float* d_logits_scratch) {
+                              const float* d_h_packed, int mb, int mode, float* d_out, float* d_logits_scratch,
+                              const unsigned short* d_h_hi, const unsigned short* d_h_lo) {
   int rc = zr_bind_device(ctx);
   if (rc) return rc;
   rc = check_softmax_args("zr_softmax_forward", d_D, d_b_d, V, H, d_h, mb);
@@ -315,7 +321,7 @@ int zr_softmax_forward_packed(zr_ctx* ctx, const float* d_D, const float* d_b_d,
   float* logits = (d_logits_scratch && !logits_only) ? d_logits_scratch : d_out;
   float* partials = nullptr;
   int nblocks = 0;
-  rc = logits_with_partials(ctx, d_D, d_b_d, V, H, d_h, mb, logits, &partials, &nblocks, d_h_packed);
+  rc = logits_with_partials(ctx, d_D, d_b_d, V, H, d_h, mb, logits, &partials, &nblocks, d_h_packed, d_h_hi, d_h_lo);
   if (rc) return rc;
   // ZR_SOFTMAX_LOGITS: the column statistics go behind the logits in the caller's buffer and no normalised matrix is
   // written -- a consumer that needs only a few entries per column (the beam search) normalises those itself
