@@ -410,7 +410,9 @@ __global__ void __launch_bounds__(256) gemm_rows_kernel(GemmArgs a, int row_chun
 // tiles and the column tiles of one row tile run side by side on it.
 // Big tile of gemm_tall_kernel: 32*TM rows x 32*TN columns, operand ring PF deep, OCC workgroups per CU.  Measured on the 50000 x 128 x 1000 logits product (kernel time, us): one workgroup per CU with a six-deep
 // ring (all 512 registers) 134-136; two per CU with a ring of two 119, of three 122, of one 122; 32 x 128 tiles at two
-// per CU 123; 64 x 64 tiles at three per CU 123.
+// per CU 123; 64 x 64 tiles at three per CU 123.  Giving every resident workgroup the same share of the rows (512
+// workgroups of one 64-row and one 32-row tile each, all resident from start to end, instead of 768 tiles of which the
+// last 256 run one to a CU) changed nothing: 123.9 us for the whole output layer either way.
 // Minibatches that are a multiple of 64 but not of 128 columns wide (192 beam columns) take 64 x 64 tiles at three
 // workgroups per CU.
 template <int EPI, int TM, int TN, int PF, int OCC>
