@@ -416,6 +416,11 @@ def main():
         out = {"hbm_kernels": bench_hbm_kernels(ctx, n),
                "config3_decoder_step": {k: v for k, v in bench_decoder_step(ctx, n, 1).items() if k.endswith("_us")},
                "config4_beam_decode": bench_beam_decode(ctx, n)}
+        # the config-5 step as well (single-term mode): its attention kernel streams 102 MB of source states
+        ctx.set_option(capi.ZR_OPT_BF16_ACTIVATION_TERMS, 1)
+        out["config5_decoder_step_bf16_single_term"] = {
+            k: v for k, v in bench_decoder_step(ctx, n, 1, H=2000, mb=256, V=80000, bf16=True).items() if k.endswith("_us")}
+        ctx.set_option(capi.ZR_OPT_BF16_ACTIVATION_TERMS, 2)
         print(json.dumps(out))
         ctx.close()
         return
