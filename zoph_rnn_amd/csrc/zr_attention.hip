@@ -392,6 +392,10 @@ __device__ __forceinline__ void wave_sum_many(float (&v)[N]) {
 // them, for every valid slot, in registers -- all loads of a column's source states are in flight together, the
 // scores are formed from the registers, and so is the context, so the source states are read exactly once and nothing
 // is read twice.  Also writes the context k-interleaved ([H/4][mb][4]) for the output product when ctx_pack is given.
+// (With global attention -- D at least the sentence length -- the window does not depend on p_t, and requesting the
+// source states before p_t is computed was tried: the registers they occupy while the tanh, the reduction and the
+// double-precision sigmoid run push those computations into scratch; 47.9 us against 44.3 for the config-3 attention
+// step, and twice the time at H = 2000.)
 template <int MAXS, int NT = 256>
 __global__ void __launch_bounds__(NT)
 attn_fused_reg_kernel(const float* const* __restrict__ table, int longest_sent, const float* __restrict__ pre,
