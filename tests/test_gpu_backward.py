@@ -185,6 +185,12 @@ def test_sgd_update_whole_model_clip(ctx, threshold):
     ctx.grad_sumsq_accumulate(None, 0, 1.0, d_ss, reset=True)
     ctx.sync()
     assert d_ss.get()[0] == 0.0
+    # a gradient that does not start on a 16-byte boundary (the vector path must not be taken)
+    G = U(g, (1001,), -2, 2)
+    dG = ctx.array(G)
+    ctx.grad_sumsq_accumulate(dG.at(1), 1000, 0.5, d_ss, reset=True)
+    ctx.sync()
+    assert d_ss.get()[0] == pytest.approx(((G[1:].astype(np.float64) * 0.5) ** 2).sum(), rel=1e-12)
 
 
 def test_sgd_update_element_clip(ctx):
