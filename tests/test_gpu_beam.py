@@ -90,7 +90,8 @@ def test_beam_against_reference_rules(ctx, V, beam, n_sent, steps):
 
 
 @pytest.mark.parametrize("mode", ["given", "absent"])
-@pytest.mark.parametrize("V,beam,n_sent,steps,eof_boost", [(60, 5, 4, 9, 3.0), (500, 12, 3, 8, 0.0), (40, 1, 2, 5, 1.0)])
+@pytest.mark.parametrize("V,beam,n_sent,steps,eof_boost", [(60, 5, 4, 9, 3.0), (500, 12, 3, 8, 0.0), (40, 1, 2, 5, 1.0),
+                                                          (50000, 12, 4, 6, 6.0)])
 def test_beam_carries_viterbi_alignments(ctx, V, beam, n_sent, steps, eof_boost, mode):
     """The alignment histories of all finished hypotheses (those ended by an <EOF> candidate inside expand and those
     ended by the forced finish), bit-exact against the oracle's decoder; words, scores and back-pointers as without."""
