@@ -116,8 +116,72 @@ def beam_fixture():
             "max_len": np.int32(max_len), "penalty": np.float32(0.25)}
 
 
+def beam_viterbi_fixture():
+    """The same decode with the attention layer's Viterbi alignment of every column handed to each step (unk
+    replacement): the alignments every finished hypothesis ends up with."""
+    g = synth.rng(2024, 5)
+    V, beam, steps, max_len = 41, 5, 6, 10
+    dec = o.Decoder(beam, V, max_len, penalty=0.1)
+    probs, vits = [], []
+    for index in range(steps + 1):
+        lg = g.standard_normal(size=(V, beam)) * 2.0
+        lg[1, :] += 2.5
+        e = np.exp(lg - lg.max(axis=0))
+        P = np.asfortranarray((e / e.sum(axis=0)).astype(np.float32))
+        vit = g.integers(0, 30, size=beam).astype(np.int32)
+        probs.append(P)
+        vits.append(vit)
+        if index == steps:
+            dec.finish(P, vit)
+        else:
+            dec.expand(P, index, vit)
+    hyps, hv = dec.hypotheses(), dec.hypotheses_viterbi()
+    width = max(len(wd) for wd, _ in hyps)
+    hw = np.full((len(hyps), width), -1, np.int32)
+    hvit = np.full((len(hyps), width), -1, np.int32)
+    for i, ((wd, _), v) in enumerate(zip(hyps, hv)):
+        hw[i, :len(wd)] = wd
+        hvit[i, :len(v)] = v
+    return {"prob": np.stack(probs), "viterbi": np.stack(vits), "hyp_words": hw, "hyp_viterbi": hvit,
+            "hyp_len": np.array([len(wd) for wd, _ in hyps], np.int32), "beam": np.int32(beam),
+            "max_len": np.int32(max_len), "penalty": np.float32(0.1)}
+
+
+def backward_clamped_fixture():
+    """Back-propagation through a two-layer stack with the cell clamp and the error clamps of --clip-cell acting
+    (thresholds far below the values they meet): gradients of one recurrent and one input matrix, the embedding
+    gradient and the errors of the initial states."""
+    g = synth.rng(2024, 6)
+    L, H, mb, T, V = 2, 12, 4, 5, 15
+    embed = U(g, (H, V), -0.5, 0.5)
+    layers = [synth.lstm_layer(g, H) for _ in range(L)]
+    for ly in layers:
+        ly["M"] = [U(g, (H, H), -0.6, 0.6) for _ in range(4)]
+        ly["Wh"] = [U(g, (H, H), -0.6, 0.6) for _ in range(4)]
+    ids = g.integers(0, V, size=(T, mb)).astype(np.int32)
+    ids[0, 2] = -1
+    nn, mask = o.vocab_prep(ids)
+    h0 = [U(g, (H, mb), -0.5, 0.5) for _ in range(L)]
+    c0 = [U(g, (H, mb), -0.9, 0.9) for _ in range(L)]
+    err_top = [U(g, (H, mb), -1, 1) for _ in range(T)]
+    grads, d_embed, eh0, ec0 = o.lstm_stack_backward(embed, layers, nn, mask, err_top, h0, c0, cell_clip=0.35,
+                                                     err_clip=0.08)
+    out = {"embed": embed, "ids": ids, "err_top": np.stack(err_top), "h0": np.stack(h0), "c0": np.stack(c0),
+           "cell_clip": np.float32(0.35), "err_clip": np.float32(0.08), "d_embed": d_embed,
+           "err_h0": np.stack(eh0), "err_c0": np.stack(ec0)}
+    for l, ly in enumerate(layers):
+        for k in ("M", "Wh", "b"):
+            for q in range(4):
+                out["l%d_%s%d" % (l, k, q)] = ly[k][q]
+        out["l%d_dWh0" % l] = grads[l]["dWh"][0]
+        out["l%d_dM2" % l] = grads[l]["dM"][2]
+        out["l%d_db3" % l] = grads[l]["db"][3]
+    return out
+
+
 FIXTURES = {"lstm_two_layers": lstm_fixture, "attention_local_p": attention_fixture, "softmax_output_layer": softmax_fixture,
-            "beam_one_sentence": beam_fixture}
+            "beam_one_sentence": beam_fixture, "beam_viterbi_one_sentence": beam_viterbi_fixture,
+            "lstm_stack_backward_clamped": backward_clamped_fixture}
 
 if __name__ == "__main__":
     for name, fn in FIXTURES.items():

@@ -26,7 +26,8 @@ def _generator():
     return mod
 
 
-@pytest.mark.parametrize("name", ["lstm_two_layers", "attention_local_p", "softmax_output_layer", "beam_one_sentence"])
+@pytest.mark.parametrize("name", ["lstm_two_layers", "attention_local_p", "softmax_output_layer", "beam_one_sentence",
+                                  "beam_viterbi_one_sentence", "lstm_stack_backward_clamped"])
 def test_oracle_reproduces_the_committed_fixture(name):
     want = _load(name)
     got = _generator().FIXTURES[name]()
@@ -148,4 +149,30 @@ def test_gpu_beam_matches_the_fixture(ctx):
         want = f["hyp_words"][i]
         assert np.array_equal(gw, want[want != -1])
         assert gs == pytest.approx(float(f["hyp_scores"][i]), rel=1e-4, abs=1e-5)
+    ctx.beam_destroy(b)
+
+
+@pytest.mark.gpu
+def test_gpu_beam_viterbi_alignments_match_the_fixture(ctx):
+    f = _load("beam_viterbi_one_sentence")
+    beam, max_len = int(f["beam"]), int(f["max_len"])
+    steps, V = f["prob"].shape[0] - 1, f["prob"].shape[1]
+    b = ctx.beam_create(beam, V, 1, max_len, float(f["penalty"]))
+    d_vit = ctx.empty(beam, np.int32)
+    ctx.beam_set_viterbi(b, True, d_vit)
+    d_words, d_back = ctx.empty(beam, np.int32), ctx.empty(beam, np.int32)
+    for index in range(steps):
+        d_vit.set(f["viterbi"][index])
+        ctx.beam_expand(b, ctx.array(np.asfortranarray(f["prob"][index])), index, d_words, d_back)
+    d_vit.set(f["viterbi"][steps])
+    ctx.beam_finish(b, ctx.array(np.asfortranarray(f["prob"][steps])))
+    ctx.sync()
+    n_want = f["hyp_words"].shape[0]
+    got, n = ctx.beam_hypotheses(b, 0, cap=n_want + 4, max_len=max_len)
+    vit, nv = ctx.beam_hypotheses_viterbi(b, 0, cap=n_want + 4, max_len=max_len)
+    assert n == nv == n_want
+    for i in range(n_want):
+        ln = int(f["hyp_len"][i])
+        assert np.array_equal(got[i][0], f["hyp_words"][i, :ln])
+        assert np.array_equal(vit[i, :ln], f["hyp_viterbi"][i, :ln])
     ctx.beam_destroy(b)
