@@ -403,6 +403,16 @@ int zr_lstm_stack_backward(zr_ctx* ctx, int L, const zr_lstm_train* const layers
                            const float* const d_gates_all[], const float* d_err_top, const float* const d_err_hT[],
                            const float* const d_err_cT[], float* const d_dgates_all[], float* d_err_below0,
                            float* const d_err_h0[], float* const d_err_c0[]);
+/* The same with the error clamps of BZ_CUDA::clip_cell (src/LSTM.hpp:792-794, src/LSTM_HH.hpp:665-667,755-757): the error
+ * a node sends to h_{t-1}, and the error a layer above the first sends to the layer below, are clamped to +-err_clip,
+ * each on its own, before they are added to anything; d_err_h0 is clamped likewise (and d_err_hT on arrival: it is
+ * the same kind of error, from a node beyond the last step), d_err_below0 (the embedding's error) is not.
+ * err_clip <= 0: no clamp (zr_lstm_stack_backward). */
+int zr_lstm_stack_backward_clamped(zr_ctx* ctx, int L, const zr_lstm_train* const layers[], int T, int mb,
+                           const int* d_mask01, const float* const d_c0[], const float* const d_c_all[],
+                           const float* const d_gates_all[], const float* d_err_top, const float* const d_err_hT[],
+                           const float* const d_err_cT[], float* const d_dgates_all[], float* d_err_below0,
+                           float* const d_err_h0[], float* const d_err_c0[], float err_clip);
 
 /* One layer's weight gradients from the kept errors: compute_gradients_GPU (src/LSTM.hpp:1000-1270) summed over
  * all nodes in one product each.  d_in_all: the layer's inputs, H x (T*mb) (the layer below's h, or the gathered

@@ -53,6 +53,8 @@ def test_null_context_and_bad_arguments_return_errors():
     assert lib.zr_unstack_gates(None, None, 8, None) == -1
     assert lib.zr_lstm_stack_backward(None, 1, None, 1, 1, None, None, None, None, None, None, None, None, None, None,
                                       None) == -1
+    assert lib.zr_lstm_stack_backward_clamped(None, 1, None, 1, 1, None, None, None, None, None, None, None, None, None,
+                                              None, None, C.c_float(1)) == -1
     assert lib.zr_lstm_weight_gradients(None, 8, 1, 1, None, None, None, None, None, None, None) == -1
     assert lib.zr_embed_gradient(None, 8, 8, None, None, None, 1, None) == -1
     assert lib.zr_softmax_backward(None, None, None, 8, 8, None, 1, None, None, None, None, None, None) == -1

@@ -36,7 +36,7 @@ def _unstack(ctx, d_stack, H):
     return [a.get() for a in outs]
 
 
-def _gpu_stack_backward(ctx, embed, layers_np, ids, h0, c0, err_top, err_hT, err_cT):
+def _gpu_stack_backward(ctx, embed, layers_np, ids, h0, c0, err_top, err_hT, err_cT, cell_clip=0.0, err_clip=0.0):
     H, V = embed.shape
     T, mb = ids.shape
     L = len(layers_np)
@@ -49,14 +49,16 @@ def _gpu_stack_backward(ctx, embed, layers_np, ids, h0, c0, err_top, err_hT, err
     h_all = [ctx.empty((n * T,)) for _ in range(L)]
     c_all = [ctx.empty((n * T,)) for _ in range(L)]
     g_all = [ctx.empty((4 * n * T,)) for _ in range(L)]
-    ctx.lstm_stack_forward_train([ly.w for ly in layers], d_embed, V, d_nn, d_m, T, mb, d_h0, d_c0, h_all, c_all, g_all)
+    ctx.lstm_stack_forward_train([ly.w for ly in layers], d_embed, V, d_nn, d_m, T, mb, d_h0, d_c0, h_all, c_all, g_all,
+                                 clip=cell_clip)
     d_err_top = ctx.array(np.concatenate([np.asfortranarray(e).reshape(-1, order="F") for e in err_top]))
     dg_all = [ctx.empty((4 * n * T,)) for _ in range(L)]
     eh0, ec0 = [ctx.empty((H, mb)) for _ in range(L)], [ctx.empty((H, mb)) for _ in range(L)]
     d_below0 = ctx.empty((n * T,))
     ctx.lstm_stack_backward([ly.t for ly in layers], T, mb, d_m, d_c0, c_all, g_all, d_err_top, dg_all, eh0, ec0,
                             err_hT=[ctx.array(a) for a in err_hT] if err_hT else None,
-                            err_cT=[ctx.array(a) for a in err_cT] if err_cT else None, d_err_below0=d_below0)
+                            err_cT=[ctx.array(a) for a in err_cT] if err_cT else None, d_err_below0=d_below0,
+                            err_clip=err_clip)
     # weight gradients, layer by layer
     x_all = ctx.empty((n * T,))
     ctx.embed_gather(d_embed, H, V, d_nn, T * mb, x_all)
@@ -110,6 +112,42 @@ def test_stack_backward_and_gradients(ctx, L, H, mb, T, V, pad, tail):
     used = set(int(v) for v in ids[ids >= 0])
     unused = [v for v in range(V) if v not in used]
     assert np.all(got_e[:, unused] == 0)
+
+
+@pytest.mark.parametrize("L,H,mb,T,V", [(1, 32, 8, 5, 40), (3, 48, 33, 7, 90)])
+def test_stack_backward_with_cell_and_error_clamps(ctx, L, H, mb, T, V):
+    """zr_lstm_stack_backward_clamped behind a forward sweep with the cell clamp (the reference's --clip-cell): both
+    thresholds low enough to act on a good share of the values (the oracle's gradients with and without them differ
+    by far more than the tolerance)."""
+    g = synth.rng(117, L * 1000 + H + mb)
+    embed = U(g, (H, V), -0.5, 0.5)
+    layers = [synth.lstm_layer(g, H) for _ in range(L)]
+    for ly in layers:
+        ly["M"] = [U(g, (H, H), -0.3, 0.3) for _ in range(4)]
+        ly["Wh"] = [U(g, (H, H), -0.3, 0.3) for _ in range(4)]
+    ids = g.integers(0, V, size=(T, mb)).astype(np.int32)
+    ids[:2, 1] = -1
+    nn, mask = o.vocab_prep(ids)
+    h0 = [U(g, (H, mb), -0.5, 0.5) for _ in range(L)]
+    c0 = [U(g, (H, mb), -0.9, 0.9) for _ in range(L)]
+    err_top = [U(g, (H, mb), -1, 1) for _ in range(T)]
+    cell_clip, err_clip = 0.4, 0.15
+    want_g, want_e, want_eh0, want_ec0 = o.lstm_stack_backward(embed, layers, nn, mask, err_top, h0, c0,
+                                                               cell_clip=cell_clip, err_clip=err_clip)
+    plain_g = o.lstm_stack_backward(embed, layers, nn, mask, err_top, h0, c0)[0]
+    assert np.abs(plain_g[0]["dWh"][0] - want_g[0]["dWh"][0]).max() > 0.1 * np.abs(want_g[0]["dWh"][0]).max()
+    got_g, got_e, got_eh0, got_ec0 = _gpu_stack_backward(ctx, embed, layers, ids, h0, c0, err_top, None, None,
+                                                         cell_clip=cell_clip, err_clip=err_clip)
+    wfloor = 0.05 * np.sqrt(T * mb)
+    for l in range(L):
+        assert_close(got_eh0[l], want_eh0[l], what="err_h0 layer %d" % l)
+        assert np.abs(got_eh0[l]).max() <= err_clip
+        assert_close(got_ec0[l], want_ec0[l], what="err_c0 layer %d" % l)
+        for q in range(4):
+            assert_close(got_g[l]["dM"][q], want_g[l]["dM"][q], floor=wfloor, what="dM layer %d gate %d" % (l, q))
+            assert_close(got_g[l]["dWh"][q], want_g[l]["dWh"][q], floor=wfloor, what="dWh layer %d gate %d" % (l, q))
+            assert_close(got_g[l]["db"][q], want_g[l]["db"][q], floor=wfloor, what="db layer %d gate %d" % (l, q))
+    assert_close(got_e, want_e, floor=0.05 * np.sqrt(T), what="embedding gradient")
 
 
 @pytest.mark.parametrize("V,H,n", [(211, 16, 6), (1003, 48, 70), (5000, 64, 160), (1000, 32, 1056), (1003, 40, 1030)])

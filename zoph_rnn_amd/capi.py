@@ -44,7 +44,7 @@ SYMBOLS = [
     "zr_beam_hypotheses", "zr_beam_state", "zr_beam_set_viterbi", "zr_beam_hypotheses_viterbi",
     "zr_lstm_stack_forward_train", "zr_lstm_train_create", "zr_lstm_train_refresh", "zr_lstm_train_destroy",
     "zr_unstack_gates", "zr_lstm_stack_backward", "zr_lstm_weight_gradients", "zr_embed_gradient",
-    "zr_softmax_backward", "zr_sgd_update", "zr_grad_sumsq_accumulate", "zr_sgd_update_clipped", "zr_clip_inplace", "zr_lstm_node_backward", "zr_lstm_node_gradients",
+    "zr_softmax_backward", "zr_sgd_update", "zr_grad_sumsq_accumulate", "zr_sgd_update_clipped", "zr_clip_inplace", "zr_lstm_stack_backward_clamped", "zr_lstm_node_backward", "zr_lstm_node_gradients",
     "zr_softmax_backward_accumulate", "zr_gather_columns_multi", "zr_softmax_backward_loss",
     "zr_softmax_forward_static", "zr_ctx_query", "zr_attn_prepare", "zr_lstm_step_embed", "zr_attn_viterbi", "zr_lstm_decoder_step", "zr_decoder_step", "zr_lstm_feed_backward", "zr_attn_set_error_tables",
     "zr_attn_backward", "zr_dropout_apply", "zr_uniform_fill", "zr_add_inplace",
@@ -275,14 +275,16 @@ class Context:
         _chk(load().zr_unstack_gates(self.h, _vp(d_stack), C.c_int(H), _ptr_array(outs)))
 
     def lstm_stack_backward(self, layers, T, mb, d_mask, c0, c_all, gates_all, d_err_top, dgates_all, err_h0, err_c0,
-                            err_hT=None, err_cT=None, d_err_below0=None):
+                            err_hT=None, err_cT=None, d_err_below0=None, err_clip=0.0):
+        """err_clip > 0: the error clamps of the reference's --clip-cell mode (zr_lstm_stack_backward_clamped)."""
         L = len(layers)
         larr = (C.c_void_p * L)(*[w.value for w in layers])
-        _chk(load().zr_lstm_stack_backward(self.h, C.c_int(L), larr, C.c_int(T), C.c_int(mb), _vp(d_mask),
-                                           _ptr_array(c0), _ptr_array(c_all), _ptr_array(gates_all), _vp(d_err_top),
-                                           _ptr_array(err_hT) if err_hT else None,
-                                           _ptr_array(err_cT) if err_cT else None, _ptr_array(dgates_all),
-                                           _vp(d_err_below0), _ptr_array(err_h0), _ptr_array(err_c0)))
+        _chk(load().zr_lstm_stack_backward_clamped(self.h, C.c_int(L), larr, C.c_int(T), C.c_int(mb), _vp(d_mask),
+                                                   _ptr_array(c0), _ptr_array(c_all), _ptr_array(gates_all),
+                                                   _vp(d_err_top), _ptr_array(err_hT) if err_hT else None,
+                                                   _ptr_array(err_cT) if err_cT else None, _ptr_array(dgates_all),
+                                                   _vp(d_err_below0), _ptr_array(err_h0), _ptr_array(err_c0),
+                                                   C.c_float(err_clip)))
 
     def lstm_weight_gradients(self, H, T, mb, d_dgates, d_in_all, d_h0, d_h_all, d_dM, d_dWh, d_db):
         _chk(load().zr_lstm_weight_gradients(self.h, C.c_int(H), C.c_int(T), C.c_int(mb), _vp(d_dgates), _vp(d_in_all),

@@ -104,8 +104,14 @@ struct NodeBackwardGroup {
   float* ec[8];               // cell error, updated in place
   float* dg[8];
   float* dgp[8];              // non-null: second copy of dg, k-interleaved [4H/4][mb][4] (the grouped product's right side)
+  int clamp_above[8];         // err_above is an error product of the layer above (clamped like err_next), not the loss layer's
 };
-__global__ void __launch_bounds__(256) lstm_node_backward_group_kernel(NodeBackwardGroup G, int H, int mb) {
+// err_clip > 0: the error products a node receives are clamped to +-err_clip on arrival (clip_mat_kernel on
+// d_ERRnTOt_htM1 and d_ERRnTOt_h_Below, src/LSTM.hpp:792, src/LSTM_HH.hpp:665,756; a NaN stays a NaN)
+__device__ __forceinline__ float clamp_error(float v, float err_clip) {
+  return v > err_clip ? err_clip : (v < -err_clip ? -err_clip : v);
+}
+__global__ void __launch_bounds__(256) lstm_node_backward_group_kernel(NodeBackwardGroup G, int H, int mb, float err_clip) {
   const int u = blockIdx.z;
   const int b = blockIdx.y;
   const int j = blockIdx.x * 256 + threadIdx.x;
@@ -114,8 +120,14 @@ __global__ void __launch_bounds__(256) lstm_node_backward_group_kernel(NodeBackw
   const size_t ix = (size_t)b * H + j;
   const float m = (float)G.mask01[u][b];
   float eh = 0.0f;
-  if (G.err_above[u]) eh += G.err_above[u][ix];
-  if (G.err_next[u]) eh += G.err_next[u][ix];
+  if (G.err_above[u]) {
+    const float e = G.err_above[u][ix];
+    eh += (err_clip > 0.0f && G.clamp_above[u]) ? clamp_error(e, err_clip) : e;
+  }
+  if (G.err_next[u]) {
+    const float e = G.err_next[u][ix];
+    eh += err_clip > 0.0f ? clamp_error(e, err_clip) : e;
+  }
   eh *= m;
   const float* gt = G.gates[u];
   const float gi = gt[ix], gf = gt[n + ix], gc = gt[2 * n + ix], go = gt[3 * n + ix];
@@ -640,6 +652,16 @@ int zr_lstm_stack_backward(zr_ctx* ctx, int nl, const zr_lstm_train* const layer
                            const float* const d_gates_all[], const float* d_err_top, const float* const d_err_hT[],
                            const float* const d_err_cT[], float* const d_dgates_all[], float* d_err_below0,
                            float* const d_err_h0[], float* const d_err_c0[]) {
+  return zr_lstm_stack_backward_clamped(ctx, nl, layers, T, mb, d_mask01, d_c0, d_c_all, d_gates_all, d_err_top, d_err_hT,
+                                        d_err_cT, d_dgates_all, d_err_below0, d_err_h0, d_err_c0, 0.0f);
+}
+
+int zr_lstm_stack_backward_clamped(zr_ctx* ctx, int nl, const zr_lstm_train* const layers[], int T, int mb,
+                                   const int* d_mask01, const float* const d_c0[], const float* const d_c_all[],
+                                   const float* const d_gates_all[], const float* d_err_top,
+                                   const float* const d_err_hT[], const float* const d_err_cT[],
+                                   float* const d_dgates_all[], float* d_err_below0, float* const d_err_h0[],
+                                   float* const d_err_c0[], float err_clip) {
   int rc = zr_bind_device(ctx);
   if (rc) return rc;
   ZR_CHECK_ARG(nl > 0 && nl <= 16 && T > 0 && mb > 0, "zr_lstm_stack_backward: L = %d, T = %d, mb = %d", nl, T, mb);
@@ -698,6 +720,7 @@ int zr_lstm_stack_backward(zr_ctx* ctx, int nl, const zr_lstm_train* const layer
         G.cprev[nu] = (t == 0) ? d_c0[l] : d_c_all[l] + (size_t)(t - 1) * n;
         G.mask01[nu] = d_mask01 + (size_t)t * mb;
         G.err_above[nu] = (l == nl - 1) ? d_err_top + (size_t)t * n : wk(d + 1, l + 1) + n;
+        G.clamp_above[nu] = (l == nl - 1) ? 0 : 1;
         G.err_next[nu] = wk(d + 1, l);
         G.ec[nu] = d_err_c0[l];
         G.dg[nu] = d_dgates_all[l] + (size_t)t * 4 * n;
@@ -709,7 +732,7 @@ int zr_lstm_stack_backward(zr_ctx* ctx, int nl, const zr_lstm_train* const layer
       }
       if (nu == 0) continue;
       dim3 egrid((H + 255) / 256, mb, nu);
-      lstm_node_backward_group_kernel<<<egrid, 256, 0, ctx->stream>>>(G, H, mb);
+      lstm_node_backward_group_kernel<<<egrid, 256, 0, ctx->stream>>>(G, H, mb, err_clip);
       ZR_LAUNCH_CHECK("lstm_node_backward_group_kernel");
       // (error to h_{t-1}, error to below) = (Wh_stack^T, M_stack^T) * dg for every node: batch of 2 inside a group
       g.groups = nu;
@@ -740,8 +763,13 @@ int zr_lstm_stack_backward(zr_ctx* ctx, int nl, const zr_lstm_train* const layer
                             ctx->stream));
   }
   // node (l, 0) is on diagonal l
-  for (int l = 0; l < nl; ++l)
+  for (int l = 0; l < nl; ++l) {
     ZR_HIP(hipMemcpyAsync(d_err_h0[l], wk(l, l), sizeof(float) * n, hipMemcpyDeviceToDevice, ctx->stream));
+    if (err_clip > 0.0f) {  // node (l, 0)'s error to its initial state is an error to h_{t-1} like any other
+      rc = zr_clip_inplace(ctx, d_err_h0[l], (long long)n, err_clip);
+      if (rc) return rc;
+    }
+  }
   return ZR_OK;
 }
 

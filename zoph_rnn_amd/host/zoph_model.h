@@ -755,8 +755,7 @@ class model_trainer {
   }
 
   explicit model_trainer(forward_model<dType>& model) : m(model), ctx(model.gpu.ctx) {
-    // the stack-level backward sweep has no error clamp: with BZ_CUDA::clip_cell the step goes through the node classes
-    node_level = m.params.attent_params.attention_model || m.params.dropout || BZ_CUDA::clip_cell;
+    node_level = m.params.attent_params.attention_model || m.params.dropout;
     H = m.info.LSTM_size;
     L = m.info.num_layers;
     mb = m.params.minibatch_size;
@@ -795,8 +794,9 @@ class model_trainer {
       if (!l.packed) l.repack();
       w.push_back(l.packed);
     }
-    ZOPH_CALL(zr_lstm_stack_forward_train(ctx, L, w.data(), in.d_W, V, s.d_nn, s.d_mask, T, mb, h0.data(), c0.data(), 0.0f,
-                                          s.h_all.data(), s.c_all.data(), s.g_all.data()));
+    ZOPH_CALL(zr_lstm_stack_forward_train(ctx, L, w.data(), in.d_W, V, s.d_nn, s.d_mask, T, mb, h0.data(), c0.data(),
+                                          BZ_CUDA::clip_cell ? BZ_CUDA::cell_clip_threshold : 0.0f, s.h_all.data(),
+                                          s.c_all.data(), s.g_all.data()));
   }
 
   template <typename LayerT>
@@ -821,9 +821,11 @@ class model_trainer {
                      int V, const std::vector<const dType*>& h0, const std::vector<const dType*>& c0, const dType* top,
                      const std::vector<const dType*>* ehT, const std::vector<const dType*>* ecT) {
     std::vector<const dType*> c_all(s.c_all.begin(), s.c_all.end()), g_all(s.g_all.begin(), s.g_all.end());
-    ZOPH_CALL(zr_lstm_stack_backward(ctx, L, s.train.data(), T, mb, s.d_mask, c0.data(), c_all.data(), g_all.data(), top,
-                                     ehT ? ehT->data() : nullptr, ecT ? ecT->data() : nullptr, s.dg_all.data(),
-                                     s.below0, s.eh0.data(), s.ec0.data()));
+    // with BZ_CUDA::clip_cell the back-propagated errors are clamped as the node classes clamp them
+    ZOPH_CALL(zr_lstm_stack_backward_clamped(ctx, L, s.train.data(), T, mb, s.d_mask, c0.data(), c_all.data(), g_all.data(),
+                                             top, ehT ? ehT->data() : nullptr, ecT ? ecT->data() : nullptr,
+                                             s.dg_all.data(), s.below0, s.eh0.data(), s.ec0.data(),
+                                             BZ_CUDA::clip_cell ? BZ_CUDA::error_clip_threshold : 0.0f));
     ZOPH_CALL(zr_embed_gather(ctx, in.d_W, H, V, s.d_nn, T * mb, s.x_all));
     for (int l = 0; l < L; l++)
       ZOPH_CALL(zr_lstm_weight_gradients(ctx, H, T, mb, s.dg_all[l], l == 0 ? s.x_all : s.h_all[l - 1], h0[l],
