@@ -99,6 +99,31 @@ def test_beam_carries_viterbi_alignments(ctx, V, beam, n_sent, steps, eof_boost,
                  viterbi=mode)
 
 
+def test_beam_viterbi_tracking_must_start_before_the_first_step(ctx):
+    """Alignments of steps already taken cannot be made up: switching the tracking on after an expand is refused, and
+    so are alignments handed over with the tracking off; switching it off and on again before a sentence is fine."""
+    V, beam = 50, 3
+    g = synth.rng(5, 21)
+    b = ctx.beam_create(beam, V, 1, 8, 0.0)
+    d_words, d_back = ctx.empty(beam, np.int32), ctx.empty(beam, np.int32)
+    d_vit = ctx.zeros(beam, np.int32)
+    with pytest.raises(capi.ZrError):
+        ctx.beam_set_viterbi(b, False, d_vit)
+    ctx.beam_expand(b, ctx.array(_random_dist(g, V, beam)), 0, d_words, d_back)
+    with pytest.raises(capi.ZrError):
+        ctx.beam_set_viterbi(b, True, d_vit)
+    ctx.beam_init(b)
+    ctx.beam_set_viterbi(b, True, d_vit)
+    ctx.beam_set_viterbi(b, False)
+    ctx.beam_set_viterbi(b, True, None)
+    ctx.beam_expand(b, ctx.array(_random_dist(g, V, beam)), 0, d_words, d_back)
+    ctx.beam_finish(b, ctx.array(_random_dist(g, V, beam)))
+    ctx.sync()
+    vit, n = ctx.beam_hypotheses_viterbi(b, 0, cap=16, max_len=8)
+    assert n >= 1 and np.all(vit[:, 0] == -20) and np.all(vit[:, 1] == -1)
+    ctx.beam_destroy(b)
+
+
 def test_beam_with_frequent_eof_and_penalty(ctx):
     """<EOF> made likely: hypotheses finish inside expand without consuming beam slots; a word penalty is added."""
     _decode_both(ctx, 60, 5, 4, 7, max_len=12, penalty=0.3, seed=7, eof_boost=4.0)
