@@ -354,6 +354,10 @@ int zr_beam_finish_logits(zr_ctx* ctx, zr_beam* b, const float* d_logits, const 
 /* Copies the finished hypotheses of sentence s to the host: returns their number (or a negative error);
  * h_words is n x max_len (row-major, -1 padded), h_len and h_score have n entries; at most cap are copied. */
 int zr_beam_hypotheses(zr_ctx* ctx, zr_beam* b, int sentence, int cap, int* h_words, int* h_len, float* h_score);
+/* ensemble_factory::ensembles_models (src/ensemble_factory.hpp:767-793): d_out = the element-wise mean of n_models
+ * (<= 16) output distributions (V x cols each, summed in double), every column then divided by its sum.  d_out may be
+ * one of the inputs.  The result feeds zr_beam_expand / zr_beam_finish. */
+int zr_ensemble_average(zr_ctx* ctx, int n_models, const float* const d_probs[], int V, int cols, float* d_out);
 /* Viterbi alignments through the beam, for unk replacement (decoder::top_sentences_viterbi and
  * eigen_mat_wrapper::viterbi_alignments, src/decoder.h:126,230-231; initialised to -20, :1335).  With enable != 0 every
  * later zr_beam_expand* / zr_beam_finish* call attaches to each candidate the alignment of the column it comes from,

@@ -327,3 +327,33 @@ def test_beam_on_logits_equals_beam_on_probabilities(ctx, V, H, beam, n_sent, pr
         ctx.softmax_release(dD)
     ctx.beam_destroy(ba)
     ctx.beam_destroy(bb)
+
+
+@pytest.mark.parametrize("K,V,cols", [(1, 37, 3), (2, 400, 12), (5, 50000, 192), (8, 1025, 1)])
+def test_ensemble_average_is_the_renormalised_mean(ctx, K, V, cols):
+    """zr_ensemble_average: out(:, c) = mean_k p_k(:, c) divided by its own sum (src/ensemble_factory.hpp:767-793,
+    which sums the models' distributions in double, divides by their number and renormalises each column).  The
+    models' columns here deliberately do not sum to one (scaled by 0.5 .. 1.5), so a kernel that skipped the
+    renormalisation, or divided by a constant, fails; one column holds zeros in all models but one."""
+    g = synth.rng(77, K + cols)
+    ps = [np.asfortranarray(_random_dist(g, V, cols) * g.uniform(0.5, 1.5, size=(1, cols)).astype(np.float32))
+          for _ in range(K)]
+    if K > 1:
+        for p in ps[1:]:
+            p[:, 0] = 0.0
+    avg = (np.sum([p.astype(np.float64) for p in ps], axis=0) / K)
+    want = avg / avg.sum(axis=0)
+    d_ps = [ctx.array(p) for p in ps]
+    d_out = ctx.empty((V, cols))
+    ctx.ensemble_average(d_ps, V, cols, d_out)
+    got = d_out.get()
+    np.testing.assert_allclose(got, want, rtol=3e-6, atol=1e-12)
+    np.testing.assert_allclose(got.astype(np.float64).sum(axis=0), 1.0, rtol=1e-5)
+    if K == 1:
+        # one model: the result is that model's distribution, renormalised; in place is allowed
+        ctx.ensemble_average(d_ps, V, cols, d_ps[0])
+        np.testing.assert_array_equal(d_ps[0].get(), got)
+    with pytest.raises(capi.ZrError):
+        ctx.ensemble_average(d_ps * 17, V, cols, d_out)
+    for d in d_ps + [d_out]:
+        d.free()

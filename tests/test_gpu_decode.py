@@ -92,6 +92,68 @@ def _oracle_decode(m, src_col, src_len, S, beam, steps, D, penalty, viterbi=Fals
     return hist, dec.hypotheses(), min_gap
 
 
+def _oracle_ensemble_decode(ms, src_cols, S, beam, steps, D):
+    """One sentence through several models behind one beam (src/ensemble_factory.hpp:767-793): every model runs its
+    own encoder and decoder step, the step's output distributions are averaged (sum in double, divided by the number of
+    models) and each column divided by its sum, the one beam expands on that, and every model's states follow the
+    same back-pointers.  Returns the finished hypotheses and the smallest gap between candidate scores a step popped."""
+    K, Vt = len(ms), ms[0]["D_soft"].shape[0]
+    L = len(ms[0]["src_layers"])
+    ones = np.ones(beam, np.int32)
+    binfo = np.concatenate([np.full(beam, S, np.int32), np.zeros(beam, np.int32)])
+    st = []
+    for m, col in zip(ms, src_cols):
+        nn, mk = o.vocab_prep(col.reshape(S, 1))
+        hs, cs = o.lstm_stack_forward(m["src_embed"], m["src_layers"], nn, mk)
+        st.append({"table": np.repeat(hs[L - 1], beam, axis=2),
+                   "hp": [np.repeat(np.asfortranarray(hs[l, S - 1]), beam, axis=1) for l in range(L)],
+                   "cp": [np.repeat(np.asfortranarray(cs[l, S - 1]), beam, axis=1) for l in range(L)], "h_tild": None})
+    dec = o.Decoder(beam, Vt, steps + 3, penalty=0.0)
+    words = np.zeros(beam, np.int32)
+    min_gap = np.inf
+
+    def forward(k, index):
+        m, s = ms[k], st[k]
+        below = o.embed_gather(m["tgt_embed"], np.maximum(words, 0))
+        newh, newc = [], []
+        for l in range(L):
+            ly = m["tgt_layers"][l]
+            feed = l == 0 and index > 0
+            r = o.lstm_step(ly["M"], ly["Wh"], ly["b"], below, s["hp"][l], s["cp"][l], ones,
+                            Q=ly["Q"] if feed else None, htild=s["h_tild"] if feed else None)
+            newh.append(r["h"])
+            newc.append(r["c"])
+            below = r["h"]
+        att = o.attention_forward(hs_table=s["table"], batch_info=binfo, h_t=below, mask01=ones, D=D, **m["attn"])
+        P = o.softmax_dist(o.softmax_logits(m["D_soft"], m["b_soft"], att["h_tild"]))
+        return newh, newc, att, P
+
+    def mean_dist(outs):
+        avg = (np.sum([r[3].astype(np.float64) for r in outs], axis=0) / K).astype(np.float32)
+        norm = avg.astype(np.float64).sum(axis=0).astype(np.float32)
+        return np.asfortranarray((avg / norm[None, :]).astype(np.float32))
+
+    for index in range(steps):
+        outs = [forward(k, index) for k in range(K)]
+        P = mean_dist(outs)
+        cols = 1 if index == 0 else beam
+        sc = dec.state()["scores"]
+        cand = np.sort(np.concatenate([np.log(np.sort(P[:, i])[-(beam + 2):]) + sc[i] for i in range(cols)]))[::-1]
+        n_hyp_before = len(dec.hypotheses())
+        dec.expand(P, index)
+        popped = beam + (len(dec.hypotheses()) - n_hyp_before) + 2
+        min_gap = min(min_gap, np.min(-np.diff(cand[:popped + 1])))
+        d = dec.state()
+        words, back = d["current_indices"].copy(), d["new_indicies_changes"].copy()
+        for k in range(K):
+            newh, newc, att, _ = outs[k]
+            st[k]["hp"] = [np.asfortranarray(a[:, back]) for a in newh]
+            st[k]["cp"] = [np.asfortranarray(a[:, back]) for a in newc]
+            st[k]["h_tild"] = np.asfortranarray(att["h_tild"][:, back])
+    dec.finish(mean_dist([forward(k, steps) for k in range(K)]))
+    return dec.hypotheses(), min_gap
+
+
 @pytest.mark.parametrize("H,L,beam,n_sent,S,steps,D", [(64, 2, 4, 3, 7, 6, 3), (48, 1, 3, 2, 5, 5, 10), (100, 3, 12, 2, 9, 4, 10)])
 def test_batched_beam_decode_matches_per_sentence_reference(ctx, H, L, beam, n_sent, S, steps, D):
     g = synth.rng(61, H + beam)

@@ -41,7 +41,7 @@ SYMBOLS = [
     "zr_lstm_gates", "zr_lstm_stack_forward", "zr_gemm", "zr_softmax_prepare", "zr_softmax_prepare_bf16", "zr_softmax_release", "zr_softmax_forward", "zr_softmax_logprob_f64",
     "zr_softmax_loss", "zr_attn_create", "zr_attn_use_bf16_weights", "zr_attn_destroy", "zr_attn_step", "zr_gather_columns",
     "zr_broadcast_column", "zr_beam_create", "zr_beam_destroy", "zr_beam_init", "zr_beam_expand", "zr_beam_finish", "zr_beam_expand_logits", "zr_beam_finish_logits",
-    "zr_beam_hypotheses", "zr_beam_state", "zr_beam_set_viterbi", "zr_beam_hypotheses_viterbi",
+    "zr_beam_hypotheses", "zr_beam_state", "zr_beam_set_viterbi", "zr_beam_hypotheses_viterbi", "zr_ensemble_average",
     "zr_lstm_stack_forward_train", "zr_lstm_train_create", "zr_lstm_train_refresh", "zr_lstm_train_destroy",
     "zr_unstack_gates", "zr_lstm_stack_backward", "zr_lstm_weight_gradients", "zr_embed_gradient",
     "zr_softmax_backward", "zr_sgd_update", "zr_grad_sumsq_accumulate", "zr_sgd_update_clipped", "zr_clip_inplace", "zr_lstm_stack_backward_clamped", "zr_lstm_node_backward", "zr_lstm_node_gradients",
@@ -452,6 +452,10 @@ class Context:
             _chk(n)
         k = min(n, cap)
         return [(words[i, :lens[i]].copy(), float(scores[i])) for i in range(k)], n
+
+    def ensemble_average(self, d_probs, V, cols, d_out):
+        _chk(load().zr_ensemble_average(self.h, C.c_int(len(d_probs)), _ptr_array(d_probs), C.c_int(V), C.c_int(cols),
+                                        _vp(d_out)))
 
     def beam_set_viterbi(self, b, enable, d_viterbi=None):
         _chk(load().zr_beam_set_viterbi(self.h, b, C.c_int(1 if enable else 0), _vp(d_viterbi)))

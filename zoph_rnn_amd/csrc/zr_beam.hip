@@ -440,6 +440,35 @@ beam_finish_kernel(int beam, int V, int max_len, int hyp_cap, float penalty, int
   if (tid == 0) hyp_count[s] = base + added;
 }
 
+// ensemble_factory::ensembles_models (src/ensemble_factory.hpp:767-793): the models' output distributions are averaged
+// element by element (summed in double, divided by the number of models) and every column is divided by its sum again.
+// One workgroup per column: a pass that writes the averages and adds them up (double, fixed order), a pass that divides.
+constexpr int kMaxEnsemble = 16;
+struct EnsembleArgs {
+  const float* p[kMaxEnsemble];
+};
+__global__ void __launch_bounds__(256) ensemble_average_kernel(EnsembleArgs a, int n_models, int V, float* out) {
+  __shared__ double s_sum[256];
+  const int col = blockIdx.x, tid = threadIdx.x;
+  float* o = out + (size_t)col * V;
+  double colsum = 0.0;
+  for (int v = tid; v < V; v += 256) {
+    double t = 0.0;
+    for (int k = 0; k < n_models; ++k) t += (double)a.p[k][(size_t)col * V + v];
+    const float avg = (float)(t / (double)n_models);
+    o[v] = avg;
+    colsum += (double)avg;
+  }
+  s_sum[tid] = colsum;
+  __syncthreads();
+  for (int st = 128; st > 0; st >>= 1) {
+    if (tid < st) s_sum[tid] += s_sum[tid + st];
+    __syncthreads();
+  }
+  const float norm = (float)s_sum[0];
+  for (int v = tid; v < V; v += 256) o[v] = o[v] / norm;
+}
+
 __global__ void beam_init_kernel(int n_sent, int beam, int max_len, float* scores, int* words, int* sent, int* hyp_count,
                                  int* vit) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -637,6 +666,22 @@ int zr_beam_hypotheses(zr_ctx* ctx, zr_beam* b, int sentence, int cap, int* h_wo
     ZR_HIP(hipStreamSynchronize(ctx->stream));
   }
   return count;
+}
+
+int zr_ensemble_average(zr_ctx* ctx, int n_models, const float* const d_probs[], int V, int cols, float* d_out) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(n_models >= 1 && n_models <= kMaxEnsemble && V > 0 && cols > 0 && cols <= 65535 && d_probs && d_out,
+               "zr_ensemble_average: %d models (at most %d), V = %d, cols = %d, or a null pointer", n_models, kMaxEnsemble,
+               V, cols);
+  EnsembleArgs a = {};
+  for (int k = 0; k < n_models; ++k) {
+    ZR_CHECK_ARG(d_probs[k] != nullptr, "zr_ensemble_average: distribution %d is null", k);
+    a.p[k] = d_probs[k];
+  }
+  ensemble_average_kernel<<<cols, 256, 0, ctx->stream>>>(a, n_models, V, d_out);
+  ZR_LAUNCH_CHECK("ensemble_average_kernel");
+  return ZR_OK;
 }
 
 int zr_beam_set_viterbi(zr_ctx* ctx, zr_beam* b, int enable, const int* d_viterbi) {

@@ -13,6 +13,10 @@
 // hypothesis an optional "-Score: s" line and the hypothesis (ids with --ids, <START> and <EOF> included, as the
 // reference's integer output; words otherwise).
 //
+// model.nn may be a comma-separated list of model files: an ensemble (src/ensemble_factory.hpp:767-793).  Every model
+// integerizes the source with its own source vocabulary; the target vocabularies must be the same size (the first
+// model's words are printed); the models' output distributions are averaged and renormalised before the one beam picks
+// from them.  At most 8 models; not together with --UNK-decode.
 // --UNK-decode FILE (attention models): the reference's unk-replacement side file (src/decoder.h:1452-1459) -- per
 // output hypothesis one line with, for every <UNK> (id 2) at position j of the hypothesis, the Viterbi alignment stored
 // at position j+1, i.e. a position in the reversed source sentence as the attention layer counts them.
@@ -76,65 +80,100 @@ int main(int argc, char** argv) {
   }
   if (pos.size() != 3 || beam > 31) return usage(argv[0]);
 
-  std::ifstream model(pos[0]);
-  if (!model) {
-    std::fprintf(stderr, "cannot open %s\n", pos[0].c_str());
-    return 1;
+  std::vector<std::string> model_paths;
+  for (size_t from = 0; from <= pos[0].size();) {
+    const size_t comma = pos[0].find(',', from);
+    const size_t to = comma == std::string::npos ? pos[0].size() : comma;
+    if (to > from) model_paths.push_back(pos[0].substr(from, to - from));
+    from = to + 1;
   }
-  model_file_info info;
+  const int K = (int)model_paths.size();
+  if (K < 1 || K > 8 || (K > 1 && !unk_file.empty())) return usage(argv[0]);
+
+  std::vector<std::ifstream> model_files(K);
+  std::vector<model_file_info> infos(K);
   std::string err;
-  if (!read_model_file_info(model, false, info, err)) {
-    std::fprintf(stderr, "%s: %s\n", pos[0].c_str(), err.c_str());
-    return 1;
-  }
-  // integerize the source side: vocabulary lookup, reversed (src/input_file_prep.h:405-416)
-  std::unordered_map<std::string, int> smap;
-  for (size_t i = 0; i < info.source_vocab.size(); i++) smap[info.source_vocab[i]] = (int)i;
-  const int unk = smap.count("<UNK>") ? smap["<UNK>"] : 0;
-  std::ifstream src(pos[1]);
-  if (!src) {
-    std::fprintf(stderr, "cannot open %s\n", pos[1].c_str());
-    return 1;
-  }
-  std::vector<std::vector<int>> sents;
-  std::string line;
-  while (std::getline(src, line)) {
-    std::vector<int> v;
-    for (const auto& w : zoph_split_words(line)) v.push_back(smap.count(w) ? smap[w] : unk);
-    std::reverse(v.begin(), v.end());
-    if (v.empty() || (int)v.size() > longest - 2) {
-      std::fprintf(stderr, "source sentence %zu is empty or longer than longest-sent - 2\n", sents.size() + 1);
+  for (int k = 0; k < K; k++) {
+    model_files[k].open(model_paths[k]);
+    if (!model_files[k]) {
+      std::fprintf(stderr, "cannot open %s\n", model_paths[k].c_str());
       return 1;
     }
-    sents.push_back(v);
+    if (!read_model_file_info(model_files[k], false, infos[k], err)) {
+      std::fprintf(stderr, "%s: %s\n", model_paths[k].c_str(), err.c_str());
+      return 1;
+    }
+    if (infos[k].target_vocab_size != infos[0].target_vocab_size) {
+      std::fprintf(stderr, "%s: the models of an ensemble must have target vocabularies of one size\n",
+                   model_paths[k].c_str());
+      return 1;
+    }
   }
+  const model_file_info& info = infos[0];
+  // integerize the source side once per model: vocabulary lookup, reversed (src/input_file_prep.h:405-416)
+  std::vector<std::vector<std::vector<int>>> sents(K);  // [model][sentence]
+  for (int k = 0; k < K; k++) {
+    std::unordered_map<std::string, int> smap;
+    for (size_t i = 0; i < infos[k].source_vocab.size(); i++) smap[infos[k].source_vocab[i]] = (int)i;
+    const int unk = smap.count("<UNK>") ? smap["<UNK>"] : 0;
+    std::ifstream src(pos[1]);
+    if (!src) {
+      std::fprintf(stderr, "cannot open %s\n", pos[1].c_str());
+      return 1;
+    }
+    std::string line;
+    while (std::getline(src, line)) {
+      std::vector<int> v;
+      for (const auto& w : zoph_split_words(line)) v.push_back(smap.count(w) ? smap[w] : unk);
+      std::reverse(v.begin(), v.end());
+      if (v.empty() || (int)v.size() > longest - 2) {
+        std::fprintf(stderr, "source sentence %zu is empty or longer than longest-sent - 2\n", sents[k].size() + 1);
+        return 1;
+      }
+      sents[k].push_back(v);
+    }
+  }
+  const size_t n_sents = sents[0].size();
   std::map<int, std::vector<int>> by_len;  // source length -> sentence numbers, in input order
-  for (size_t i = 0; i < sents.size(); i++) by_len[(int)sents[i].size()].push_back((int)i);
+  for (size_t i = 0; i < n_sents; i++) by_len[(int)sents[0][i].size()].push_back((int)i);
 
   BZ_CUDA::bf16_weights = bf16;
   BZ_CUDA::unk_replacement = !unk_file.empty();  // src/main.cu:410-412
   layer_gpu_info gpu;
   gpu.init(0);
-  forward_model<precision> m;
-  m.initModel(gpu, info, 1, longest, D);
-  m.load_weights(model);
-  beam_decoder<precision> dec(m, beam, batch, longest, D, penalty);
+  std::vector<forward_model<precision>> models(K);
+  std::vector<beam_decoder<precision>*> decs;
+  for (int k = 0; k < K; k++) {
+    models[k].initModel(gpu, infos[k], 1, longest, D);
+    models[k].load_weights(model_files[k]);
+    decs.push_back(new beam_decoder<precision>(models[k], beam, batch, longest, D, penalty));
+    decs.back()->min_decoding_ratio = min_ratio;
+    decs.back()->max_decoding_ratio = max_ratio;
+  }
+  beam_decoder<precision>& dec = *decs[0];
   if (BZ_CUDA::unk_replacement && !dec.track_viterbi) {
     std::fprintf(stderr, "--UNK-decode needs an attention model\n");
     return 1;
   }
-  dec.min_decoding_ratio = min_ratio;
-  dec.max_decoding_ratio = max_ratio;
+  ensemble_beam_decoder<precision>* ensemble = K > 1 ? new ensemble_beam_decoder<precision>(decs) : nullptr;
 
-  std::vector<std::vector<decoded_hypothesis>> results(sents.size());
+  std::vector<std::vector<decoded_hypothesis>> results(n_sents);
   for (const auto& kv : by_len) {
     const auto& idx = kv.second;
     for (size_t base = 0; base < idx.size(); base += batch) {
-      std::vector<std::vector<int>> group;
-      for (size_t j = base; j < std::min(idx.size(), base + (size_t)batch); j++) group.push_back(sents[idx[j]]);
+      const size_t end = std::min(idx.size(), base + (size_t)batch);
       std::vector<std::vector<decoded_hypothesis>> out;
-      dec.decode_batch(group, num_best, out);
-      for (size_t j = 0; j < group.size(); j++) results[idx[base + j]] = out[j];
+      if (ensemble) {
+        std::vector<std::vector<std::vector<int>>> group(K);
+        for (int k = 0; k < K; k++)
+          for (size_t j = base; j < end; j++) group[k].push_back(sents[k][idx[j]]);
+        ensemble->decode_batch(group, num_best, out);
+      } else {
+        std::vector<std::vector<int>> group;
+        for (size_t j = base; j < end; j++) group.push_back(sents[0][idx[j]]);
+        dec.decode_batch(group, num_best, out);
+      }
+      for (size_t j = 0; j < end - base; j++) results[idx[base + j]] = out[j];
     }
   }
 
@@ -190,6 +229,6 @@ int main(int argc, char** argv) {
     }
     out << "\n";
   }
-  std::cout << "Sentences: " << sents.size() << "\n";
+  std::cout << "Sentences: " << n_sents << "\n";
   return 0;
 }

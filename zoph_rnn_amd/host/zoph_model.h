@@ -1042,6 +1042,10 @@ class beam_decoder {
     }
   }
 
+  // An ensemble member hands its output distribution on as probabilities (they are averaged over the models before the
+  // beam sees them); a decoder on its own leaves logits and column statistics for the beam to normalise what it picks.
+  bool prob_mode = false;
+
   // forward_prop_target (src/model.hpp:2573-2688): state half p -> half q, logits and column statistics into logits
   void forward_target(int p, int step_index) {
     const int q = 1 - p;
@@ -1053,18 +1057,17 @@ class beam_decoder {
     ZOPH_CALL(zr_decoder_step(ctx, L, tgt_w.data(), m.input_layer_target.d_W, Vt, d_words_nn, hp.data(), cp.data(), feed,
                               d_ones, 0.0f, cols, h[q].data(), c[q].data(), attention ? attn : nullptr, d_batch_info,
                               attention ? h_tild[q] : nullptr, d_align, d_align_idx, nullptr, nullptr, m.softmax_obj.d_D,
-                              m.softmax_obj.d_b_d, Vt, ZR_SOFTMAX_LOGITS, logits));
+                              m.softmax_obj.d_b_d, Vt, prob_mode ? ZR_SOFTMAX_PROB : ZR_SOFTMAX_LOGITS, logits));
     // the alignment of every column, read by the beam call that follows (get_viterbi_alignment_kernel)
     if (track_viterbi) ZOPH_CALL(zr_attn_viterbi(ctx, attn, d_align, d_align_idx, d_viterbi));
   }
 
-  // Decodes up to n_sent sentences whose integerized sources (reversed, no padding) all have the same length S.
-  // out[s] receives the num_best best finished hypotheses of sentence s, best first
-  // (decoder::output_k_best_hypotheses, src/decoder.h:1386-1413).
-  void decode_batch(const std::vector<std::vector<int>>& sources, int num_best,
-                    std::vector<std::vector<decoded_hypothesis>>& out) {
+  // forward_prop_source (src/model.hpp:2367-2452) for up to n_sent sentences whose integerized sources (reversed, no
+  // padding) all have the same length: the encoder sweep, every sentence's states replicated over its beam columns,
+  // <START> in every column.  Returns the source length.
+  int encode(const std::vector<std::vector<int>>& sources) {
     const int real = (int)sources.size();
-    const int S = (int)sources[0].size();
+    const int S = real > 0 ? (int)sources[0].size() : 0;
     if (real < 1 || real > n_sent || S < 1 || S > longest_sent) {
       std::fprintf(stderr, "beam_decoder::decode_batch: %d sentences of source length %d do not fit\n", real, S);
       std::exit(EXIT_FAILURE);
@@ -1101,59 +1104,56 @@ class beam_decoder {
     ZOPH_CALL(zr_h2d(ctx, d_batch_info, binfo.data(), binfo.size() * sizeof(int)));
     std::vector<int> start(cols, 0);  // <START>
     ZOPH_CALL(zr_h2d(ctx, d_words, start.data(), cols * sizeof(int)));
-    ZOPH_CALL(zr_beam_init(ctx, bm));
+    return S;
+  }
 
-    const int steps = std::min((int)(max_decoding_ratio * S), longest_sent - 2);
-    int p = 0, index = 0;
-    for (; index < steps; index++) {
-      forward_target(p, index);
-      ZOPH_CALL(zr_beam_expand_logits(ctx, bm, logits, logits + (size_t)Vt * cols, index, d_words, d_back));
-      // swap_decoding_states + target_copy_prev_states (src/model.hpp:2691-2726)
-      const int q = 1 - p;
-      std::vector<const dType*> from(h[q].begin(), h[q].end());
-      from.insert(from.end(), c[q].begin(), c[q].end());
-      std::vector<dType*> to(h[p].begin(), h[p].end());
-      to.insert(to.end(), c[p].begin(), c[p].end());
-      if (attention) {
-        from.push_back(h_tild[q]);
-        to.push_back(h_tild[p]);
-      }
-      ZOPH_CALL(zr_gather_columns_multi(ctx, (int)from.size(), from.data(), H, d_back, cols, cols, to.data()));
+  // swap_decoding_states + target_copy_prev_states (src/model.hpp:2691-2726): the new states (half 1 - p), reordered by
+  // the beam's back-pointers, become the previous states (half p) of the next step
+  void reorder_states(int p, const int* d_backptr) {
+    const int q = 1 - p;
+    std::vector<const dType*> from(h[q].begin(), h[q].end());
+    from.insert(from.end(), c[q].begin(), c[q].end());
+    std::vector<dType*> to(h[p].begin(), h[p].end());
+    to.insert(to.end(), c[p].begin(), c[p].end());
+    if (attention) {
+      from.push_back(h_tild[q]);
+      to.push_back(h_tild[p]);
     }
-    // one last step and forced <EOF> on every live hypothesis (src/ensemble_factory.hpp:727-743)
-    forward_target(p, index);
-    ZOPH_CALL(zr_beam_finish_logits(ctx, bm, logits, logits + (size_t)Vt * cols));
-    {
-      // A single-launch encoder sweep or decoder step that gave up a wait left NaN in its outputs: the batch is
-      // decoded again with one launch per node (and so is every later batch of this decoder).
-      int abandoned = 0;
-      ZOPH_CALL(zr_ctx_query(ctx, ZR_QUERY_LSTM_SWEEP_ABANDONED, &abandoned));
-      if (abandoned) {
-        abandoned_launches++;
-        ZOPH_CALL(zr_ctx_set_option(ctx, ZR_OPT_LSTM_SWEEP, 1));
-        decode_batch(sources, num_best, out);
-        return;
-      }
-    }
-    ZOPH_CALL(zr_ctx_sync(ctx));
+    ZOPH_CALL(zr_gather_columns_multi(ctx, (int)from.size(), from.data(), H, d_backptr, cols, cols, to.data()));
+  }
 
+  int decode_steps(int S) const { return std::min((int)(max_decoding_ratio * S), longest_sent - 2); }
+
+  // True when a single-launch encoder sweep or decoder step gave up a wait (its outputs hold NaN): every later launch of
+  // this context then goes out one per node, and the caller decodes the batch again.
+  bool launches_abandoned() {
+    int abandoned = 0;
+    ZOPH_CALL(zr_ctx_query(ctx, ZR_QUERY_LSTM_SWEEP_ABANDONED, &abandoned));
+    if (!abandoned) return false;
+    abandoned_launches++;
+    ZOPH_CALL(zr_ctx_set_option(ctx, ZR_OPT_LSTM_SWEEP, 1));
+    return true;
+  }
+
+  // output_k_best_hypotheses (src/decoder.h:1386-1413) for the first `real` sentences of beam object b: length ratio
+  // filter, then the num_best best scores, best first
+  void collect(zr_beam* b, int real, int S, int steps, int num_best, std::vector<std::vector<decoded_hypothesis>>& out) {
     out.assign(real, {});
     const int cap = 4 * beam * (steps + 2), max_len = longest_sent + 3;
     std::vector<int> words((size_t)cap * max_len), lens(cap), vit(track_viterbi ? (size_t)cap * max_len : 0);
     std::vector<float> scores(cap);
     for (int s = 0; s < real; s++) {
-      int n = zr_beam_hypotheses(ctx, bm, s, cap, words.data(), lens.data(), scores.data());
-      if (n >= 0 && track_viterbi) n = std::min(n, zr_beam_hypotheses_viterbi(ctx, bm, s, cap, vit.data()));
+      int n = zr_beam_hypotheses(ctx, b, s, cap, words.data(), lens.data(), scores.data());
+      if (n >= 0 && track_viterbi) n = std::min(n, zr_beam_hypotheses_viterbi(ctx, b, s, cap, vit.data()));
       if (n < 0) {
         std::fprintf(stderr, "zr_beam_hypotheses failed: %s\n", zr_last_error());
         std::exit(EXIT_FAILURE);
       }
       n = std::min(n, cap);
-      // output_k_best_hypotheses: length ratio filter, then the num_best best scores, best first
       std::vector<int> order;
       for (int i = 0; i < n; i++)
         if ((float)lens[i] / (float)S > (float)min_decoding_ratio) order.push_back(i);
-      std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return scores[a] > scores[b]; });
+      std::stable_sort(order.begin(), order.end(), [&](int a, int b2) { return scores[a] > scores[b2]; });
       if ((int)order.size() > num_best) order.resize(num_best);
       for (int i : order) {
         decoded_hypothesis hyp;
@@ -1163,6 +1163,96 @@ class beam_decoder {
         out[s].push_back(hyp);
       }
     }
+  }
+
+  // Decodes up to n_sent sentences whose integerized sources (reversed, no padding) all have the same length S.
+  // out[s] receives the num_best best finished hypotheses of sentence s, best first
+  // (decoder::output_k_best_hypotheses, src/decoder.h:1386-1413).
+  void decode_batch(const std::vector<std::vector<int>>& sources, int num_best,
+                    std::vector<std::vector<decoded_hypothesis>>& out) {
+    const int real = (int)sources.size();
+    const int S = encode(sources);
+    ZOPH_CALL(zr_beam_init(ctx, bm));
+    const int steps = decode_steps(S);
+    int p = 0, index = 0;
+    for (; index < steps; index++) {
+      forward_target(p, index);
+      ZOPH_CALL(zr_beam_expand_logits(ctx, bm, logits, logits + (size_t)Vt * cols, index, d_words, d_back));
+      reorder_states(p, d_back);
+    }
+    // one last step and forced <EOF> on every live hypothesis (src/ensemble_factory.hpp:727-743)
+    forward_target(p, index);
+    ZOPH_CALL(zr_beam_finish_logits(ctx, bm, logits, logits + (size_t)Vt * cols));
+    if (launches_abandoned()) {  // the batch is decoded again with one launch per node
+      decode_batch(sources, num_best, out);
+      return;
+    }
+    ZOPH_CALL(zr_ctx_sync(ctx));
+    collect(bm, real, S, steps, num_best, out);
+  }
+};
+
+// Several models decoded together (ensemble_factory::decode_file_batch with more than one model,
+// src/ensemble_factory.hpp:583-765): every model runs its own encoder and decoder step on its own weights and states,
+// the output distributions are averaged and renormalised (ensembles_models, :767-793), ONE beam picks the words from
+// the average, and every model reorders its states by that beam's back-pointers.  The members are beam_decoders over
+// one context with the same beam, batch and target vocabulary; each has its own source vocabulary, so a sentence
+// arrives integerized once per member.  (The reference's vote over the members' alignment scores for unk
+// replacement is not built: Viterbi tracking stays off here.)
+template <typename dType>
+class ensemble_beam_decoder {
+ public:
+  std::vector<beam_decoder<dType>*> members;
+  zr_ctx* ctx;
+  dType* mean = nullptr;  // V x cols: the averaged distribution
+
+  explicit ensemble_beam_decoder(const std::vector<beam_decoder<dType>*>& mem) : members(mem), ctx(mem.at(0)->ctx) {
+    auto& first = *members[0];
+    for (auto* d : members) {
+      if (d->ctx != ctx || d->beam != first.beam || d->n_sent != first.n_sent || d->Vt != first.Vt ||
+          d->longest_sent != first.longest_sent) {
+        std::fprintf(stderr, "ensemble_beam_decoder: the members must share the context, beam, batch, longest_sent and "
+                     "target vocabulary size\n");
+        std::exit(EXIT_FAILURE);
+      }
+      d->prob_mode = true;
+    }
+    ZOPH_CALL(zr_malloc(ctx, (size_t)first.Vt * first.cols * sizeof(dType), (void**)&mean));
+  }
+
+  // sources[k]: the batch's sentences integerized with member k's source vocabulary (reversed, equal lengths)
+  void decode_batch(const std::vector<std::vector<std::vector<int>>>& sources, int num_best,
+                    std::vector<std::vector<decoded_hypothesis>>& out) {
+    auto& first = *members[0];
+    const int K = (int)members.size(), real = (int)sources.at(0).size();
+    int S = 0;
+    for (int k = 0; k < K; k++) S = members[k]->encode(sources.at(k));
+    ZOPH_CALL(zr_beam_init(ctx, first.bm));
+    const int steps = first.decode_steps(S);
+    std::vector<const dType*> dists(K);
+    for (int k = 0; k < K; k++) dists[k] = members[k]->logits;
+    auto step = [&](int index) {
+      for (int k = 0; k < K; k++) {
+        // every member is fed the words the shared beam chose
+        if (k > 0) ZOPH_CALL(zr_d2d(ctx, members[k]->d_words, first.d_words, (size_t)first.cols * sizeof(int)));
+        members[k]->forward_target(0, index);
+      }
+      ZOPH_CALL(zr_ensemble_average(ctx, K, dists.data(), first.Vt, first.cols, mean));
+    };
+    int index = 0;
+    for (; index < steps; index++) {
+      step(index);
+      ZOPH_CALL(zr_beam_expand(ctx, first.bm, mean, index, first.d_words, first.d_back));
+      for (int k = 0; k < K; k++) members[k]->reorder_states(0, first.d_back);
+    }
+    step(index);
+    ZOPH_CALL(zr_beam_finish(ctx, first.bm, mean));
+    if (first.launches_abandoned()) {
+      decode_batch(sources, num_best, out);
+      return;
+    }
+    ZOPH_CALL(zr_ctx_sync(ctx));
+    first.collect(first.bm, real, S, steps, num_best, out);
   }
 };
 
