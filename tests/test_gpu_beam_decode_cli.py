@@ -110,13 +110,27 @@ def _write_model(path, m, L, H, tgt_vocab, src_vocab):
         _write_matrix(f, m["b_soft"].reshape(-1, 1))
 
 
-@pytest.mark.parametrize("n_models,L", [(2, 2), (3, 1)])
-def test_beam_decode_cli_ensemble_matches_per_sentence_oracle(tmp_path, n_models, L):
+def _round_matrices_to_bf16(m):
+    """Every matrix the decoder streams (LSTM, attention, output layer) rounded to bf16, so that bf16 storage is exact."""
+    from gpu_util import round_bf16
+    rb = lambda a: np.asfortranarray(round_bf16(a))
+    for ly in m["src_layers"] + m["tgt_layers"]:
+        for k in ("M", "Wh", "Q"):
+            if k in ly:
+                ly[k] = [rb(x) for x in ly[k]]
+    for k in ("W_a", "W_p", "W_c1", "W_c2"):
+        m["attn"][k] = rb(m["attn"][k])
+    m["D_soft"] = rb(m["D_soft"])
+
+
+@pytest.mark.parametrize("n_models,L,bf16", [(2, 2, False), (3, 1, False), (2, 2, True)])
+def test_beam_decode_cli_ensemble_matches_per_sentence_oracle(tmp_path, n_models, L, bf16):
     """A comma-separated list of model files decodes as an ensemble (src/ensemble_factory.hpp:767-793): the models'
     output distributions are averaged and renormalised at every step, one beam picks the words, every model's states
     are reordered by that beam's back-pointers.  The models differ in every weight and in their source vocabularies
     (same words, another order: each model integerizes the source text with its own mapping); an ensemble that read
-    only its first model, or fed every model the first model's source ids, fails."""
+    only its first model, or fed every model the first model's source ids, fails.  bf16: the members store their matrices
+    as bf16 (--bf16; the matrices are bf16-representable, so the fp32 oracle on the same matrices is the bar)."""
     g = synth.rng(98, n_models)
     H, D, longest, K, beam = 64, 3, 24, 3, 4
     base_src = mf.make_vocab(79, "s")
@@ -125,6 +139,8 @@ def test_beam_decode_cli_ensemble_matches_per_sentence_oracle(tmp_path, n_models
     for k in range(n_models):
         sv = ["<UNK>"] + [base_src[i] for i in g.permutation(len(base_src))]
         m = _model(g, H, len(sv), len(tgt_vocab), L)
+        if bf16:
+            _round_matrices_to_bf16(m)
         p = tmp_path / ("model%d.nn" % k)
         _write_model(p, m, L, H, tgt_vocab, sv)
         ms.append(m)
@@ -134,8 +150,9 @@ def test_beam_decode_cli_ensemble_matches_per_sentence_oracle(tmp_path, n_models
     src = [mf.random_sentences(g, src_vocabs[0], 1, n, n)[0] for n in lens]
     sp, out = tmp_path / "src.txt", tmp_path / "out.txt"
     sp.write_text("".join(" ".join(s) + "\n" for s in src))
-    r = mf.run_program("beam_decode", ["--beam", beam, "--batch", 3, "--longest-sent", longest, "--attention-width", D,
-                                       "--num-best", K, "--print-score", "--ids", ",".join(paths), sp, out])
+    r = mf.run_program("beam_decode", (["--bf16"] if bf16 else []) +
+                       ["--beam", beam, "--batch", 3, "--longest-sent", longest, "--attention-width", D,
+                        "--num-best", K, "--print-score", "--ids", ",".join(paths), sp, out])
     assert r.returncode == 0, r.stderr[-2000:]
     got = _parse_blocks(out.read_text())
     assert len(got) == len(src)
@@ -146,14 +163,14 @@ def test_beam_decode_cli_ensemble_matches_per_sentence_oracle(tmp_path, n_models
         S = len(words)
         steps = min(int(1.5 * S), longest - 2)
         hyps, gap = _oracle_ensemble_decode(ms, cols, S, beam, steps, D)
-        assert gap > 5e-6, "candidate scores nearly tie (gap %.2e): pick another seed" % gap
+        assert gap > (5e-5 if bf16 else 5e-6), "candidate scores nearly tie (gap %.2e): pick another seed" % gap
         keep = [(w, sc) for (w, sc) in hyps if len(w) / S > 0.5]
         keep.sort(key=lambda t: -t[1])
         want = keep[:K]
         assert len(got[s]) == len(want), (s, len(got[s]), len(want))
         for (gw, gs), (ww, ws) in zip(got[s], want):
             assert gw == list(ww), (s, gw, list(ww))
-            assert gs == pytest.approx(ws, rel=1e-4, abs=1e-4)
+            assert gs == pytest.approx(ws, rel=1e-4, abs=2e-4 if bf16 else 1e-4)
         alone = _oracle_decode(ms[0], cols[0], S, S, beam, steps, D, 0.0)[1]
         alone = sorted([(w, sc) for (w, sc) in alone if len(w) / S > 0.5], key=lambda t: -t[1])[:K]
         differs_from_first += [list(w) for w, _ in alone] != [list(w) for w, _ in want]
@@ -206,20 +223,12 @@ def test_beam_decode_cli_with_bf16_weight_storage(tmp_path):
     through the bf16 decoder step (the step's inputs split into bf16 terms in one launch, every LSTM node leaving its h as
     bf16 terms for the next product).  The model's matrices are bf16-representable, so the storage is exact and the
     fp32 oracle on the same matrices is the bar: same words, scores to 1e-4."""
-    from gpu_util import round_bf16
     g = synth.rng(97, 3)
     H, L, D, longest, K, beam = 64, 2, 3, 24, 2, 4
     src_vocab = ["<UNK>"] + mf.make_vocab(79, "s")
     tgt_vocab = ["<START>", "<EOF>", "<UNK>"] + mf.make_vocab(397, "t")
     m = _model(g, H, len(src_vocab), len(tgt_vocab), L)
-    rb = lambda a: np.asfortranarray(round_bf16(a))
-    for ly in m["src_layers"] + m["tgt_layers"]:
-        for k in ("M", "Wh", "Q"):
-            if k in ly:
-                ly[k] = [rb(x) for x in ly[k]]
-    for k in ("W_a", "W_p", "W_c1", "W_c2"):
-        m["attn"][k] = rb(m["attn"][k])
-    m["D_soft"] = rb(m["D_soft"])
+    _round_matrices_to_bf16(m)
     model = tmp_path / "model.nn"
     with open(model, "w") as f:
         mf.write_header(f, L, H, tgt_vocab, src_vocab, True, True)
