@@ -313,6 +313,14 @@ int zr_attn_step(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, const float* 
  * the object's internal arrays. */
 int zr_attn_viterbi(zr_ctx* ctx, const zr_attn* a, const float* d_alignments, const int* d_indices, int* d_viterbi);
 
+/* The alignment vote of an ensemble under unk replacement (ensemble_factory::ensembles_models,
+ * src/ensemble_factory.hpp:797-834, on the per-model rows filled at src/attention_node.hpp:236-268): every model's
+ * window weights (d_alignments[k], d_indices[k]: slots x cols as zr_attn_step leaves them, element (b, j) at b + cols*j;
+ * index -1 = no source position) are spread over longest_sent (<= 8192) source positions, summed over the n_models
+ * (<= 16) models in order, and d_viterbi[b] = the first position with the largest sum, -1 when no sum is positive. */
+int zr_attn_viterbi_ensemble(zr_ctx* ctx, int n_models, const float* const d_alignments[], const int* const d_indices[],
+                             int slots, int cols, int longest_sent, int* d_viterbi);
+
 /* ---- A12: decoder state shuffles ------------------------------------------------------------------------- */
 
 /* swap_states_decoding (src/Input_To_Hidden_Layer.hpp:1231-1242, src/Hidden_To_Hidden_Layer.hpp:780-791):
@@ -356,7 +364,9 @@ int zr_beam_finish_logits(zr_ctx* ctx, zr_beam* b, const float* d_logits, const 
 int zr_beam_hypotheses(zr_ctx* ctx, zr_beam* b, int sentence, int cap, int* h_words, int* h_len, float* h_score);
 /* ensemble_factory::ensembles_models (src/ensemble_factory.hpp:767-793): d_out = the element-wise mean of n_models
  * (<= 16) output distributions (V x cols each, summed in double), every column then divided by its sum.  d_out may be
- * one of the inputs.  The result feeds zr_beam_expand / zr_beam_finish. */
+ * one of the inputs.  The result feeds zr_beam_expand / zr_beam_finish.  The reference accumulates the column sums in
+ * float, row after row, and takes a single model's distribution as it is (no renormalisation); here the sums are in
+ * double for any number of models, which moves a column's log-probabilities by a common ~1e-5 at most. */
 int zr_ensemble_average(zr_ctx* ctx, int n_models, const float* const d_probs[], int V, int cols, float* d_out);
 /* Viterbi alignments through the beam, for unk replacement (decoder::top_sentences_viterbi and
  * eigen_mat_wrapper::viterbi_alignments, src/decoder.h:126,230-231; initialised to -20, :1335).  With enable != 0 every

@@ -61,6 +61,7 @@ def test_null_context_and_bad_arguments_return_errors():
     assert lib.zr_sgd_update(None, None, None, C.c_longlong(4), C.c_float(1), C.c_float(0), C.c_float(0.1)) == -1
     assert lib.zr_beam_set_viterbi(None, None, 1, None) == -1
     assert lib.zr_ensemble_average(None, 2, None, 8, 8, None) == -1
+    assert lib.zr_attn_viterbi_ensemble(None, 2, None, None, 7, 8, 20, None) == -1
     assert lib.zr_beam_hypotheses_viterbi(None, None, 0, 0, None) == -1
     assert lib.zr_clip_inplace(None, None, C.c_longlong(4), C.c_float(1)) == -1
     assert lib.zr_grad_sumsq_accumulate(None, None, C.c_longlong(4), C.c_float(1), None, 1) == -1

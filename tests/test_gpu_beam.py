@@ -357,3 +357,50 @@ def test_ensemble_average_is_the_renormalised_mean(ctx, K, V, cols):
         ctx.ensemble_average(d_ps * 17, V, cols, d_out)
     for d in d_ps + [d_out]:
         d.free()
+
+
+def test_ensemble_alignment_vote_known_answer_and_brute_force(ctx):
+    """zr_attn_viterbi_ensemble (src/ensemble_factory.hpp:797-834).  A hand-worked case first: model A puts 0.4375,
+    0.375, 0.1875 on source positions 2, 3, 4 (its own best: 2), model B 0.375, 0.1875, 0.4375 on positions 3, 4, 5 (its
+    own best: 5); the sums are 0.4375, 0.75, 0.375, 0.4375, so the vote is position 3, which neither model picks alone.
+    A second column ties exactly (0.625 at positions 3 and 5): the first wins.  A third has no source position at all
+    (-1).  Then random windows against the restatement in test_gpu_decode.ensemble_alignment_vote."""
+    from test_gpu_decode import ensemble_alignment_vote
+    f, i = np.float32, np.int32
+    alA = np.asfortranarray(np.array([[0.4375, 0.375, 0.1875], [0.25, 0.5, 0.25], [0.3, 0.3, 0.4]], f))
+    ixA = np.asfortranarray(np.array([[2, 3, 4], [2, 3, 4], [-1, -1, -1]], i))
+    alB = np.asfortranarray(np.array([[0.375, 0.1875, 0.4375], [0.125, 0.25, 0.625], [0.5, 0.2, 0.3]], f))
+    ixB = np.asfortranarray(np.array([[3, 4, 5], [3, 4, 5], [-1, -1, -1]], i))
+    d = [ctx.array(x) for x in (alA, alB)], [ctx.array(x) for x in (ixA, ixB)]
+    d_out = ctx.empty(3, np.int32)
+    ctx.attn_viterbi_ensemble(d[0], d[1], 3, 3, 9, d_out)
+    assert d_out.get().tolist() == [3, 3, -1]
+    assert ensemble_alignment_vote([alA, alB], [ixA, ixB], 9).tolist() == [3, 3, -1]
+    g = synth.rng(78, 5)
+    for K, D, cols, longest in [(1, 2, 7, 12), (3, 10, 192, 54), (8, 50, 24, 104), (16, 3, 5, 700)]:
+        W = 2 * D + 1
+        als, ixs = [], []
+        centre = g.integers(0, longest, size=cols)
+        for k in range(K):
+            c = np.clip(centre + g.integers(-2, 3, size=cols), 0, longest - 1)
+            ix = c[:, None] + np.arange(-D, D + 1)[None, :]
+            ix = np.where((ix < 0) | (ix >= longest - 4), -1, ix).astype(i)
+            al = g.uniform(0.0, 1.0, size=(cols, W)).astype(f)
+            al[ix == -1] = 0.0
+            al /= np.maximum(al.sum(axis=1, keepdims=True), 1e-9)
+            als.append(np.asfortranarray(al.astype(f)))
+            ixs.append(np.asfortranarray(ix))
+        d_al, d_ix = [ctx.array(x) for x in als], [ctx.array(x) for x in ixs]
+        d_o = ctx.empty(cols, np.int32)
+        ctx.attn_viterbi_ensemble(d_al, d_ix, W, cols, longest, d_o)
+        want = ensemble_alignment_vote(als, ixs, longest)
+        assert np.array_equal(d_o.get(), want), (K, D, cols, longest)
+        if K > 1:
+            own = ensemble_alignment_vote(als[:1], ixs[:1], longest)
+            assert np.any(own != want), "the vote equals the first model's choice everywhere"
+        for x in d_al + d_ix + [d_o]:
+            x.free()
+    with pytest.raises(capi.ZrError):
+        ctx.attn_viterbi_ensemble(d[0], d[1], 3, 3, 9000, d_out)
+    for x in d[0] + d[1] + [d_out]:
+        x.free()

@@ -123,14 +123,17 @@ def _round_matrices_to_bf16(m):
     m["D_soft"] = rb(m["D_soft"])
 
 
-@pytest.mark.parametrize("n_models,L,bf16", [(2, 2, False), (3, 1, False), (2, 2, True)])
-def test_beam_decode_cli_ensemble_matches_per_sentence_oracle(tmp_path, n_models, L, bf16):
+@pytest.mark.parametrize("n_models,L,bf16,unk", [(2, 2, False, False), (3, 1, False, False), (2, 2, True, False),
+                                                 (2, 2, False, True), (3, 1, False, True)])
+def test_beam_decode_cli_ensemble_matches_per_sentence_oracle(tmp_path, n_models, L, bf16, unk):
     """A comma-separated list of model files decodes as an ensemble (src/ensemble_factory.hpp:767-793): the models'
     output distributions are averaged and renormalised at every step, one beam picks the words, every model's states
     are reordered by that beam's back-pointers.  The models differ in every weight and in their source vocabularies
     (same words, another order: each model integerizes the source text with its own mapping); an ensemble that read
     only its first model, or fed every model the first model's source ids, fails.  bf16: the members store their matrices
-    as bf16 (--bf16; the matrices are bf16-representable, so the fp32 oracle on the same matrices is the bar)."""
+    as bf16 (--bf16; the matrices are bf16-representable, so the fp32 oracle on the same matrices is the bar).
+    unk: with --UNK-decode the side file holds the models' alignment VOTE (src/ensemble_factory.hpp:797-834), which must
+    differ from the first model's own alignment somewhere for the comparison to show anything (checked)."""
     g = synth.rng(98, n_models)
     H, D, longest, K, beam = 64, 3, 24, 3, 4
     base_src = mf.make_vocab(79, "s")
@@ -141,6 +144,10 @@ def test_beam_decode_cli_ensemble_matches_per_sentence_oracle(tmp_path, n_models
         m = _model(g, H, len(sv), len(tgt_vocab), L)
         if bf16:
             _round_matrices_to_bf16(m)
+        if unk:
+            m["b_soft"][2] += 7.0  # <UNK> likely enough to show up; alignments that move from step to step
+            m["attn"]["v_p"] = m["attn"]["v_p"] * 60
+            m["attn"]["W_a"] = m["attn"]["W_a"] * 16
         p = tmp_path / ("model%d.nn" % k)
         _write_model(p, m, L, H, tgt_vocab, sv)
         ms.append(m)
@@ -150,23 +157,30 @@ def test_beam_decode_cli_ensemble_matches_per_sentence_oracle(tmp_path, n_models
     src = [mf.random_sentences(g, src_vocabs[0], 1, n, n)[0] for n in lens]
     sp, out = tmp_path / "src.txt", tmp_path / "out.txt"
     sp.write_text("".join(" ".join(s) + "\n" for s in src))
-    r = mf.run_program("beam_decode", (["--bf16"] if bf16 else []) +
+    unk_path = tmp_path / "unk.txt"
+    r = mf.run_program("beam_decode", (["--bf16"] if bf16 else []) + (["--UNK-decode", unk_path] if unk else []) +
                        ["--beam", beam, "--batch", 3, "--longest-sent", longest, "--attention-width", D,
                         "--num-best", K, "--print-score", "--ids", ",".join(paths), sp, out])
     assert r.returncode == 0, r.stderr[-2000:]
     got = _parse_blocks(out.read_text())
     assert len(got) == len(src)
     smaps = [{w: i for i, w in enumerate(sv)} for sv in src_vocabs]
-    differs_from_first = 0
+    differs_from_first = vote_differs = 0
+    want_unk = []
     for s, words in enumerate(src):
         cols = [np.array([sm.get(w, 0) for w in words][::-1], np.int32) for sm in smaps]
         S = len(words)
         steps = min(int(1.5 * S), longest - 2)
-        hyps, gap = _oracle_ensemble_decode(ms, cols, S, beam, steps, D)
+        res = _oracle_ensemble_decode(ms, cols, S, beam, steps, D, viterbi=unk)
+        hyps, gap = res[0], res[1]
+        vits = res[2] if unk else [None] * len(hyps)
+        vote_differs += res[3] if unk else 0
         assert gap > (5e-5 if bf16 else 5e-6), "candidate scores nearly tie (gap %.2e): pick another seed" % gap
-        keep = [(w, sc) for (w, sc) in hyps if len(w) / S > 0.5]
+        keep = [(w, sc, v) for (w, sc), v in zip(hyps, vits) if len(w) / S > 0.5]
         keep.sort(key=lambda t: -t[1])
-        want = keep[:K]
+        want = [(w, sc) for w, sc, _ in keep[:K]]
+        for w, _, v in keep[:K]:
+            want_unk.append("".join("%d " % v[j + 1] for j in range(len(w) - 1) if w[j] == 2))
         assert len(got[s]) == len(want), (s, len(got[s]), len(want))
         for (gw, gs), (ww, ws) in zip(got[s], want):
             assert gw == list(ww), (s, gw, list(ww))
@@ -175,6 +189,10 @@ def test_beam_decode_cli_ensemble_matches_per_sentence_oracle(tmp_path, n_models
         alone = sorted([(w, sc) for (w, sc) in alone if len(w) / S > 0.5], key=lambda t: -t[1])[:K]
         differs_from_first += [list(w) for w, _ in alone] != [list(w) for w, _ in want]
     assert differs_from_first >= 1, "the ensemble's output equals the first model's alone: the test shows nothing"
+    if unk:
+        assert unk_path.read_text().split("\n")[:-1] == want_unk
+        assert any(ln for ln in want_unk), "no <UNK> in any hypothesis: the side file shows nothing"
+        assert vote_differs >= 1, "the vote always equals the first model's own alignment: the test shows nothing"
 
 
 def test_beam_decode_cli_ensemble_refuses_mismatched_models(tmp_path):

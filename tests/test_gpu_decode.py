@@ -92,12 +92,47 @@ def _oracle_decode(m, src_col, src_len, S, beam, steps, D, penalty, viterbi=Fals
     return hist, dec.hypotheses(), min_gap
 
 
-def _oracle_ensemble_decode(ms, src_cols, S, beam, steps, D):
+def ensemble_alignment_vote(aligns, indices, longest):
+    """The ensemble's alignment per column (src/ensemble_factory.hpp:797-834): every model's window weights spread over
+    a row of `longest` source positions (zero elsewhere, src/attention_node.hpp:236-268), the rows added in model order
+    in float32, then the first position whose sum exceeds every earlier one, starting from 0 (-1 if none is positive).
+    aligns, indices: per model a (columns, 2D+1) array."""
+    cols, W = aligns[0].shape
+    out = np.empty(cols, np.int32)
+    for b in range(cols):
+        total = np.zeros(longest, np.float32)
+        for al, ix in zip(aligns, indices):
+            row = np.zeros(longest, np.float32)
+            for j in range(W):
+                if ix[b, j] != -1:
+                    row[ix[b, j]] = al[b, j]
+            total = (total + row).astype(np.float32)
+        best, pos = np.float32(0), -1
+        for j in range(longest):
+            if total[j] > best:
+                best, pos = total[j], j
+        out[b] = pos
+    return out
+
+
+def _oracle_ensemble_decode(ms, src_cols, S, beam, steps, D, viterbi=False):
     """One sentence through several models behind one beam (src/ensemble_factory.hpp:767-793): every model runs its
     own encoder and decoder step, the step's output distributions are averaged (sum in double, divided by the number of
     models) and each column divided by its sum, the one beam expands on that, and every model's states follow the
-    same back-pointers.  Returns the finished hypotheses and the smallest gap between candidate scores a step popped."""
+    same back-pointers.  Returns the finished hypotheses and the smallest gap between candidate scores a step popped.
+    viterbi: the beam carries the models' alignment vote; returns in addition the finished hypotheses' alignments and
+    how many (step, column) pairs had a vote different from the first model's own alignment."""
     K, Vt = len(ms), ms[0]["D_soft"].shape[0]
+    vote_differs = 0
+
+    def vote(outs):
+        nonlocal vote_differs
+        if not viterbi:
+            return None
+        v = ensemble_alignment_vote([r[2]["alignments"] for r in outs], [r[2]["indices"] for r in outs], S + 4)
+        vote_differs += int(np.sum(v != o.attention_viterbi(outs[0][2]["alignments"], outs[0][2]["indices"])))
+        return v
+
     L = len(ms[0]["src_layers"])
     ones = np.ones(beam, np.int32)
     binfo = np.concatenate([np.full(beam, S, np.int32), np.zeros(beam, np.int32)])
@@ -140,7 +175,7 @@ def _oracle_ensemble_decode(ms, src_cols, S, beam, steps, D):
         sc = dec.state()["scores"]
         cand = np.sort(np.concatenate([np.log(np.sort(P[:, i])[-(beam + 2):]) + sc[i] for i in range(cols)]))[::-1]
         n_hyp_before = len(dec.hypotheses())
-        dec.expand(P, index)
+        dec.expand(P, index, vote(outs))
         popped = beam + (len(dec.hypotheses()) - n_hyp_before) + 2
         min_gap = min(min_gap, np.min(-np.diff(cand[:popped + 1])))
         d = dec.state()
@@ -150,7 +185,10 @@ def _oracle_ensemble_decode(ms, src_cols, S, beam, steps, D):
             st[k]["hp"] = [np.asfortranarray(a[:, back]) for a in newh]
             st[k]["cp"] = [np.asfortranarray(a[:, back]) for a in newc]
             st[k]["h_tild"] = np.asfortranarray(att["h_tild"][:, back])
-    dec.finish(mean_dist([forward(k, steps) for k in range(K)]))
+    outs = [forward(k, steps) for k in range(K)]
+    dec.finish(mean_dist(outs), vote(outs))
+    if viterbi:
+        return dec.hypotheses(), min_gap, dec.hypotheses_viterbi(), vote_differs
     return dec.hypotheses(), min_gap
 
 

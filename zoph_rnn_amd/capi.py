@@ -42,6 +42,7 @@ SYMBOLS = [
     "zr_softmax_loss", "zr_attn_create", "zr_attn_use_bf16_weights", "zr_attn_destroy", "zr_attn_step", "zr_gather_columns",
     "zr_broadcast_column", "zr_beam_create", "zr_beam_destroy", "zr_beam_init", "zr_beam_expand", "zr_beam_finish", "zr_beam_expand_logits", "zr_beam_finish_logits",
     "zr_beam_hypotheses", "zr_beam_state", "zr_beam_set_viterbi", "zr_beam_hypotheses_viterbi", "zr_ensemble_average",
+    "zr_attn_viterbi_ensemble",
     "zr_lstm_stack_forward_train", "zr_lstm_train_create", "zr_lstm_train_refresh", "zr_lstm_train_destroy",
     "zr_unstack_gates", "zr_lstm_stack_backward", "zr_lstm_weight_gradients", "zr_embed_gradient",
     "zr_softmax_backward", "zr_sgd_update", "zr_grad_sumsq_accumulate", "zr_sgd_update_clipped", "zr_clip_inplace", "zr_lstm_stack_backward_clamped", "zr_lstm_node_backward", "zr_lstm_node_gradients",
@@ -456,6 +457,11 @@ class Context:
     def ensemble_average(self, d_probs, V, cols, d_out):
         _chk(load().zr_ensemble_average(self.h, C.c_int(len(d_probs)), _ptr_array(d_probs), C.c_int(V), C.c_int(cols),
                                         _vp(d_out)))
+
+    def attn_viterbi_ensemble(self, d_alignments, d_indices, slots, cols, longest_sent, d_viterbi):
+        _chk(load().zr_attn_viterbi_ensemble(self.h, C.c_int(len(d_alignments)), _ptr_array(d_alignments),
+                                             _ptr_array(d_indices), C.c_int(slots), C.c_int(cols),
+                                             C.c_int(longest_sent), _vp(d_viterbi)))
 
     def beam_set_viterbi(self, b, enable, d_viterbi=None):
         _chk(load().zr_beam_set_viterbi(self.h, b, C.c_int(1 if enable else 0), _vp(d_viterbi)))

@@ -379,6 +379,58 @@ attn_viterbi_kernel(const float* __restrict__ align, const int* __restrict__ ind
   if (lane == 0) out[b] = slot == 0x7fffffff ? -1 : indices[b + (size_t)mb * slot];
 }
 
+// The alignment vote of an ensemble (ensemble_factory::ensembles_models, src/ensemble_factory.hpp:797-834): every model
+// spreads its window's alignment weights over a row of longest_sent source positions (zero elsewhere,
+// src/attention_node.hpp:236-268), the rows are added in model order, and the column's alignment is the first position
+// whose sum is strictly larger than every earlier one, starting from 0 (so -1 when no sum is positive).  One workgroup
+// per column; the row lives in LDS, each model's window is added behind a barrier (a window's positions are distinct,
+// so no two lanes meet on one element and the sum keeps the reference's order of additions).
+constexpr int kMaxEnsembleAlign = 16;
+struct EnsembleAlignArgs {
+  const float* align[kMaxEnsembleAlign];
+  const int* idx[kMaxEnsembleAlign];
+};
+__global__ void __launch_bounds__(256)
+attn_viterbi_ensemble_kernel(EnsembleAlignArgs a, int n_models, int mb, int W, int longest, int* __restrict__ out) {
+  extern __shared__ float s_score[];
+  __shared__ float s_best[256];
+  __shared__ int s_pos[256];
+  const int b = blockIdx.x, tid = threadIdx.x;
+  for (int j = tid; j < longest; j += 256) s_score[j] = 0.0f;
+  __syncthreads();
+  for (int k = 0; k < n_models; ++k) {
+    for (int j = tid; j < W; j += 256) {
+      const int ix = a.idx[k][b + (size_t)mb * j];
+      if (ix >= 0 && ix < longest) s_score[ix] += a.align[k][b + (size_t)mb * j];
+    }
+    __syncthreads();
+  }
+  float best = 0.0f;
+  int pos = -1;
+  for (int j = tid; j < longest; j += 256) {
+    const float v = s_score[j];
+    if (v > best) {
+      best = v;
+      pos = j;
+    }
+  }
+  s_best[tid] = best;
+  s_pos[tid] = pos;
+  __syncthreads();
+  for (int st = 128; st > 0; st >>= 1) {
+    if (tid < st) {
+      const float ob = s_best[tid + st];
+      const int op = s_pos[tid + st];
+      if (ob > s_best[tid] || (ob == s_best[tid] && op < s_pos[tid])) {
+        s_best[tid] = ob;
+        s_pos[tid] = op;
+      }
+    }
+    __syncthreads();
+  }
+  if (tid == 0) out[b] = s_pos[0];
+}
+
 // Sum over the 64 lanes of each of N values held one per register: lanes end up with the totals in all lanes.
 template <int N>
 __device__ __forceinline__ void wave_sum_many(float (&v)[N]) {
@@ -609,6 +661,26 @@ int zr_attn_viterbi(zr_ctx* ctx, const zr_attn* a, const float* d_alignments, co
   const int* ix = d_indices ? d_indices : a->d_idx;
   attn_viterbi_kernel<<<a->mb, 64, 0, ctx->stream>>>(al, ix, a->mb, 2 * a->D + 1, d_viterbi);
   ZR_LAUNCH_CHECK("attn_viterbi_kernel");
+  return ZR_OK;
+}
+
+int zr_attn_viterbi_ensemble(zr_ctx* ctx, int n_models, const float* const d_alignments[], const int* const d_indices[],
+                             int slots, int cols, int longest_sent, int* d_viterbi) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(n_models >= 1 && n_models <= kMaxEnsembleAlign && slots > 0 && cols > 0 && cols <= 65535 &&
+                   longest_sent > 0 && longest_sent <= 8192 && d_alignments && d_indices && d_viterbi,
+               "zr_attn_viterbi_ensemble: %d models (at most %d), %d slots, %d columns, longest_sent = %d (at most 8192), "
+               "or a null pointer", n_models, kMaxEnsembleAlign, slots, cols, longest_sent);
+  EnsembleAlignArgs a{};
+  for (int k = 0; k < n_models; ++k) {
+    ZR_CHECK_ARG(d_alignments[k] && d_indices[k], "zr_attn_viterbi_ensemble: model %d has a null array", k);
+    a.align[k] = d_alignments[k];
+    a.idx[k] = d_indices[k];
+  }
+  attn_viterbi_ensemble_kernel<<<cols, 256, (size_t)longest_sent * sizeof(float), ctx->stream>>>(a, n_models, cols, slots,
+                                                                                                longest_sent, d_viterbi);
+  ZR_LAUNCH_CHECK("attn_viterbi_ensemble_kernel");
   return ZR_OK;
 }
 

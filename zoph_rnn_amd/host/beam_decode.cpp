@@ -16,7 +16,8 @@
 // model.nn may be a comma-separated list of model files: an ensemble (src/ensemble_factory.hpp:767-793).  Every model
 // integerizes the source with its own source vocabulary; the target vocabularies must be the same size (the first
 // model's words are printed); the models' output distributions are averaged and renormalised before the one beam picks
-// from them.  At most 8 models; not together with --UNK-decode.
+// from them.  At most 8 models.  With --UNK-decode the alignments written are the models' vote (their alignment weights
+// summed per source position, src/ensemble_factory.hpp:797-834).
 // --UNK-decode FILE (attention models): the reference's unk-replacement side file (src/decoder.h:1452-1459) -- per
 // output hypothesis one line with, for every <UNK> (id 2) at position j of the hypothesis, the Viterbi alignment stored
 // at position j+1, i.e. a position in the reversed source sentence as the attention layer counts them.
@@ -88,7 +89,7 @@ int main(int argc, char** argv) {
     from = to + 1;
   }
   const int K = (int)model_paths.size();
-  if (K < 1 || K > 8 || (K > 1 && !unk_file.empty())) return usage(argv[0]);
+  if (K < 1 || K > 8) return usage(argv[0]);
 
   std::vector<std::ifstream> model_files(K);
   std::vector<model_file_info> infos(K);
@@ -151,10 +152,11 @@ int main(int argc, char** argv) {
     decs.back()->max_decoding_ratio = max_ratio;
   }
   beam_decoder<precision>& dec = *decs[0];
-  if (BZ_CUDA::unk_replacement && !dec.track_viterbi) {
-    std::fprintf(stderr, "--UNK-decode needs an attention model\n");
-    return 1;
-  }
+  for (auto* d : decs)
+    if (BZ_CUDA::unk_replacement && !d->track_viterbi) {
+      std::fprintf(stderr, "--UNK-decode needs an attention model\n");
+      return 1;
+    }
   ensemble_beam_decoder<precision>* ensemble = K > 1 ? new ensemble_beam_decoder<precision>(decs) : nullptr;
 
   std::vector<std::vector<decoded_hypothesis>> results(n_sents);

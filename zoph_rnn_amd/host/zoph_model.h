@@ -1197,8 +1197,9 @@ class beam_decoder {
 // the output distributions are averaged and renormalised (ensembles_models, :767-793), ONE beam picks the words from
 // the average, and every model reorders its states by that beam's back-pointers.  The members are beam_decoders over
 // one context with the same beam, batch and target vocabulary; each has its own source vocabulary, so a sentence
-// arrives integerized once per member.  (The reference's vote over the members' alignment scores for unk
-// replacement is not built: Viterbi tracking stays off here.)
+// arrives integerized once per member.  Under unk replacement the column's alignment is the members' vote: their
+// alignment weights summed per source position, the first largest sum wins (:797-834; zr_attn_viterbi_ensemble), and
+// the shared beam carries that alignment.
 template <typename dType>
 class ensemble_beam_decoder {
  public:
@@ -1210,9 +1211,10 @@ class ensemble_beam_decoder {
     auto& first = *members[0];
     for (auto* d : members) {
       if (d->ctx != ctx || d->beam != first.beam || d->n_sent != first.n_sent || d->Vt != first.Vt ||
-          d->longest_sent != first.longest_sent) {
+          d->longest_sent != first.longest_sent || d->track_viterbi != first.track_viterbi ||
+          (first.track_viterbi && d->D != first.D)) {
         std::fprintf(stderr, "ensemble_beam_decoder: the members must share the context, beam, batch, longest_sent and "
-                     "target vocabulary size\n");
+                     "target vocabulary size (and, under unk replacement, all have attention of one width)\n");
         std::exit(EXIT_FAILURE);
       }
       d->prob_mode = true;
@@ -1229,8 +1231,13 @@ class ensemble_beam_decoder {
     for (int k = 0; k < K; k++) S = members[k]->encode(sources.at(k));
     ZOPH_CALL(zr_beam_init(ctx, first.bm));
     const int steps = first.decode_steps(S);
-    std::vector<const dType*> dists(K);
-    for (int k = 0; k < K; k++) dists[k] = members[k]->logits;
+    std::vector<const dType*> dists(K), aligns(K);
+    std::vector<const int*> align_idx(K);
+    for (int k = 0; k < K; k++) {
+      dists[k] = members[k]->logits;
+      aligns[k] = members[k]->d_align;
+      align_idx[k] = members[k]->d_align_idx;
+    }
     auto step = [&](int index) {
       for (int k = 0; k < K; k++) {
         // every member is fed the words the shared beam chose
@@ -1238,6 +1245,10 @@ class ensemble_beam_decoder {
         members[k]->forward_target(0, index);
       }
       ZOPH_CALL(zr_ensemble_average(ctx, K, dists.data(), first.Vt, first.cols, mean));
+      // the beam call that follows reads first.d_viterbi: the members' vote replaces the first member's own alignment
+      if (first.track_viterbi)
+        ZOPH_CALL(zr_attn_viterbi_ensemble(ctx, K, aligns.data(), align_idx.data(), 2 * first.D + 1, first.cols,
+                                           first.longest_sent, first.d_viterbi));
     };
     int index = 0;
     for (; index < steps; index++) {
