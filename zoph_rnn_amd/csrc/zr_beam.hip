@@ -442,31 +442,80 @@ beam_finish_kernel(int beam, int V, int max_len, int hyp_cap, float penalty, int
 
 // ensemble_factory::ensembles_models (src/ensemble_factory.hpp:767-793): the models' output distributions are averaged
 // element by element (summed in double, divided by the number of models) and every column is divided by its sum again.
-// One workgroup per column: a pass that writes the averages and adds them up (double, fixed order), a pass that divides.
+// Two launches over (chunk of 4096 rows, column) workgroups, so that a few hundred columns still fill the chip: the
+// first writes the averages and one partial sum (double) per workgroup; the second adds a column's partials in chunk
+// order (every workgroup of the column gets the same total) and divides its chunk.  VEC: 16-byte accesses when the
+// columns are 16-byte aligned.
 constexpr int kMaxEnsemble = 16;
+constexpr int kEnsembleChunk = 4096;
 struct EnsembleArgs {
   const float* p[kMaxEnsemble];
 };
-__global__ void __launch_bounds__(256) ensemble_average_kernel(EnsembleArgs a, int n_models, int V, float* out) {
+template <bool VEC>
+__global__ void __launch_bounds__(256)
+ensemble_mean_kernel(EnsembleArgs a, int n_models, int V, float* out, double* partials) {
   __shared__ double s_sum[256];
-  const int col = blockIdx.x, tid = threadIdx.x;
-  float* o = out + (size_t)col * V;
-  double colsum = 0.0;
-  for (int v = tid; v < V; v += 256) {
-    double t = 0.0;
-    for (int k = 0; k < n_models; ++k) t += (double)a.p[k][(size_t)col * V + v];
-    const float avg = (float)(t / (double)n_models);
-    o[v] = avg;
-    colsum += (double)avg;
+  const int chunk = blockIdx.x, col = blockIdx.y, tid = threadIdx.x;
+  const size_t base = (size_t)col * V;
+  const int v0 = chunk * kEnsembleChunk, v1 = min(V, v0 + kEnsembleChunk);
+  const double inv = (double)n_models;
+  double sum = 0.0;
+  if (VEC) {
+    for (int v = v0 + 4 * tid; v < v1; v += 1024) {  // V % 4 == 0: a group of four never straddles v1
+      double t[4] = {0.0, 0.0, 0.0, 0.0};
+      for (int k = 0; k < n_models; ++k) {
+        const float4 x = *(const float4*)(a.p[k] + base + v);
+        t[0] += (double)x.x;
+        t[1] += (double)x.y;
+        t[2] += (double)x.z;
+        t[3] += (double)x.w;
+      }
+      float4 r;
+      r.x = (float)(t[0] / inv);
+      r.y = (float)(t[1] / inv);
+      r.z = (float)(t[2] / inv);
+      r.w = (float)(t[3] / inv);
+      *(float4*)(out + base + v) = r;
+      sum += ((double)r.x + (double)r.y) + ((double)r.z + (double)r.w);
+    }
+  } else {
+    for (int v = v0 + tid; v < v1; v += 256) {
+      double t = 0.0;
+      for (int k = 0; k < n_models; ++k) t += (double)a.p[k][base + v];
+      const float avg = (float)(t / inv);
+      out[base + v] = avg;
+      sum += (double)avg;
+    }
   }
-  s_sum[tid] = colsum;
+  s_sum[tid] = sum;
   __syncthreads();
   for (int st = 128; st > 0; st >>= 1) {
     if (tid < st) s_sum[tid] += s_sum[tid + st];
     __syncthreads();
   }
-  const float norm = (float)s_sum[0];
-  for (int v = tid; v < V; v += 256) o[v] = o[v] / norm;
+  if (tid == 0) partials[(size_t)col * gridDim.x + chunk] = s_sum[0];
+}
+
+template <bool VEC>
+__global__ void __launch_bounds__(256) ensemble_normalize_kernel(int V, float* out, const double* partials) {
+  const int chunk = blockIdx.x, col = blockIdx.y, tid = threadIdx.x;
+  double total = 0.0;
+  for (int c = 0; c < (int)gridDim.x; ++c) total += partials[(size_t)col * gridDim.x + c];
+  const float norm = (float)total;
+  const size_t base = (size_t)col * V;
+  const int v0 = chunk * kEnsembleChunk, v1 = min(V, v0 + kEnsembleChunk);
+  if (VEC) {
+    for (int v = v0 + 4 * tid; v < v1; v += 1024) {
+      float4 x = *(float4*)(out + base + v);
+      x.x = x.x / norm;
+      x.y = x.y / norm;
+      x.z = x.z / norm;
+      x.w = x.w / norm;
+      *(float4*)(out + base + v) = x;
+    }
+  } else {
+    for (int v = v0 + tid; v < v1; v += 256) out[base + v] = out[base + v] / norm;
+  }
 }
 
 __global__ void beam_init_kernel(int n_sent, int beam, int max_len, float* scores, int* words, int* sent, int* hyp_count,
@@ -679,8 +728,23 @@ int zr_ensemble_average(zr_ctx* ctx, int n_models, const float* const d_probs[],
     ZR_CHECK_ARG(d_probs[k] != nullptr, "zr_ensemble_average: distribution %d is null", k);
     a.p[k] = d_probs[k];
   }
-  ensemble_average_kernel<<<cols, 256, 0, ctx->stream>>>(a, n_models, V, d_out);
-  ZR_LAUNCH_CHECK("ensemble_average_kernel");
+  const int chunks = (V + kEnsembleChunk - 1) / kEnsembleChunk;
+  void* ws = nullptr;
+  rc = zr_ctx_scratch(ctx, 0, (size_t)chunks * cols * sizeof(double), &ws);
+  if (rc) return rc;
+  bool vec = V % 4 == 0 && ((uintptr_t)d_out & 15) == 0;
+  for (int k = 0; k < n_models; ++k) vec = vec && ((uintptr_t)d_probs[k] & 15) == 0;
+  const dim3 grid(chunks, cols);
+  if (vec) {
+    ensemble_mean_kernel<true><<<grid, 256, 0, ctx->stream>>>(a, n_models, V, d_out, (double*)ws);
+    ZR_LAUNCH_CHECK("ensemble_mean_kernel");
+    ensemble_normalize_kernel<true><<<grid, 256, 0, ctx->stream>>>(V, d_out, (const double*)ws);
+  } else {
+    ensemble_mean_kernel<false><<<grid, 256, 0, ctx->stream>>>(a, n_models, V, d_out, (double*)ws);
+    ZR_LAUNCH_CHECK("ensemble_mean_kernel");
+    ensemble_normalize_kernel<false><<<grid, 256, 0, ctx->stream>>>(V, d_out, (const double*)ws);
+  }
+  ZR_LAUNCH_CHECK("ensemble_normalize_kernel");
   return ZR_OK;
 }
 
