@@ -61,10 +61,17 @@ int zr_ctx_set_option(zr_ctx* ctx, int option, int value);
  *     ZR_LSTM_STACK_PATH_STEP_PER_LAYER (zr_lstm_decoder_step).  Does not wait.
  *   ZR_QUERY_LSTM_SWEEP_ABANDONED: waits for the stream; 1 if a single-launch sweep or decoder step since the last look
  *     gave up a wait (its outputs were then overwritten with NaN; run it again with ZR_OPT_LSTM_SWEEP = 1), else 0.  Clears
- *     the flag, so a following zr_ctx_sync no longer reports it. */
+ *     the flag, so a following zr_ctx_sync no longer reports it.
+ *   ZR_QUERY_ATTN_PATH: which schedule the last zr_attn_step (or the attention part of zr_decoder_step) on this
+ *     context took -- 0 none yet, ZR_ATTN_PATH_SINGLE_LAUNCH, ZR_ATTN_PATH_THREE_LAUNCHES or ZR_ATTN_PATH_SEPARATE.
+ *     Does not wait. */
 int zr_ctx_query(zr_ctx* ctx, int what, int* h_value);
 #define ZR_QUERY_LSTM_STACK_PATH 1
 #define ZR_QUERY_LSTM_SWEEP_ABANDONED 2
+#define ZR_QUERY_ATTN_PATH 3
+#define ZR_ATTN_PATH_SINGLE_LAUNCH 1  /* projections, window / scores / context and output product in one launch */
+#define ZR_ATTN_PATH_THREE_LAUNCHES 2 /* the same three stages as one launch each */
+#define ZR_ATTN_PATH_SEPARATE 3       /* unprepared or bf16 matrices: products and the middle as separate launches */
 #define ZR_LSTM_STACK_PATH_SWEEP 1
 #define ZR_LSTM_STACK_PATH_DIAGONALS 2
 #define ZR_LSTM_STACK_PATH_STEP_SINGLE_LAUNCH 3 /* zr_lstm_decoder_step: all layers in one launch */
@@ -103,6 +110,12 @@ const char* zr_version(void);
                                         waits of a layer for the layer below expect this many arrivals more than there
                                         will be, so each of them runs to ZR_OPT_LSTM_SWEEP_SPIN polls and gives up
                                         whatever the timing (0 = off, the default) */
+#define ZR_OPT_ATTN_SINGLE_LAUNCH 11 /* the attention step as ONE launch whose workgroups hand over through device
+                                        memory (prepared fp32 matrices, H a multiple of 8 up to 1024, at most 64 window
+                                        slots, all workgroups resident at once, own stream, only context on the
+                                        device): 0 auto (taken whenever it applies; ZR_OPT_LSTM_SWEEP = 1 also
+                                        switches it off), 1 never (three launches).  Its waits are bounded like the
+                                        single-launch LSTM schedules' and reported the same way */
 
 /* full_matrix_setup / cudaMalloc / cudaMemcpy / cudaMemset call sites (src/BZ_CUDA_UTIL.h:358-399 and the
  * layer constructors, e.g. src/LSTM.hpp:23-42). */

@@ -451,6 +451,64 @@ def test_attention_against_oracle(ctx, H, mb, S, D, prepared):
     assert np.all(got["h_tild"][:, mask == 0] == 0)
 
 
+@pytest.mark.parametrize("H,mb,S,D", [(1000, 128, 50, 50), (64, 6, 9, 2), (200, 70, 40, 10), (1024, 33, 64, 31),
+                                      (512, 12, 21, 10), (96, 1, 5, 7), (1000, 12, 50, 10)])
+def test_attention_step_in_one_launch(ctx, H, mb, S, D):
+    """The attention step as one launch (projections, per-column middle and output product handing over through device
+    memory): against the oracle, against the three-launch schedule on the same inputs, and twice in a row on one
+    attention object (the counters go back to zero inside the launch)."""
+    g = synth.rng(17, H + S + mb)
+    w = synth.attention_weights(g, H)
+    hs = (g.standard_normal(size=(S, H, mb), dtype=np.float32) * np.float32(0.5 if H <= 128 else 0.1))
+    lens = g.integers(1, S + 1, size=mb).astype(np.int32)
+    lens[0] = S
+    batch_info = np.concatenate([lens, S - lens]).astype(np.int32)
+    mask = (g.random(mb) > 0.15).astype(np.int32)
+    mask[0] = 1
+    h_t = U(g, (H, mb), -1, 1)
+    want = o.attention_forward(hs_table=hs, batch_info=batch_info, h_t=h_t, mask01=mask, D=D, **w)
+    frac = want["p_t"] - np.floor(want["p_t"])
+    assert ((frac > 1e-4) & (frac < 1 - 1e-4)).all(), "test inputs put p_t on an integer boundary; pick another seed"
+    tables = [ctx.array(np.asfortranarray(hs[t])) for t in range(S)]
+    dw = {k: ctx.array(v) for k, v in w.items()}
+    a = ctx.attn_create(H, mb, D, dw["W_a"], dw["W_p"], dw["v_p"], dw["out_bias"], dw["W_c1"], dw["W_c2"], tables)
+    ctx.attn_prepare(a)
+    Wn = 2 * D + 1
+    d_bi, d_h, d_m = ctx.array(batch_info), ctx.array(h_t), ctx.array(mask)
+
+    def run():
+        outs = (ctx.empty((H, mb)), ctx.empty((mb, Wn)), ctx.empty((mb, Wn), np.int32), ctx.empty((mb,)),
+                ctx.empty((H, mb)))
+        ctx.attn_step(a, d_bi, d_h, d_m, *outs)
+        ctx.sync()
+        return [x.get() for x in outs]
+
+    try:
+        one = run()
+        assert ctx.query(capi.ZR_QUERY_ATTN_PATH) == capi.ZR_ATTN_PATH_SINGLE_LAUNCH
+        again = run()
+        ctx.set_option(capi.ZR_OPT_ATTN_SINGLE_LAUNCH, 1)
+        three = run()
+        assert ctx.query(capi.ZR_QUERY_ATTN_PATH) == capi.ZR_ATTN_PATH_THREE_LAUNCHES
+    finally:
+        ctx.set_option(capi.ZR_OPT_ATTN_SINGLE_LAUNCH, 0)
+        ctx.attn_destroy(a)
+    names = ("h_tild", "alignments", "indices", "p_t", "c_ctx")
+    for name, x, y in zip(names, one, again):
+        assert np.array_equal(x, y), name + " differs between two launches"
+    got = dict(zip(names, one))
+    assert_close(got["p_t"], want["p_t"], what="p_t")
+    assert np.array_equal(got["indices"], want["indices"])
+    assert_close(got["alignments"], want["alignments"], floor=1e-4, what="alignments")
+    assert_close(got["c_ctx"], want["c_ctx"], what="context")
+    assert_close(got["h_tild"], want["h_tild"], what="h_tild")
+    assert np.all(got["h_tild"][:, mask == 0] == 0)
+    other = dict(zip(names, three))
+    assert np.array_equal(got["indices"], other["indices"])
+    assert_close(got["h_tild"], other["h_tild"], what="h_tild, one launch against three")
+    assert_close(got["c_ctx"], other["c_ctx"], what="context, one launch against three")
+
+
 @pytest.mark.parametrize("mb,D", [(7, 4), (130, 50), (3, 255)])
 def test_attention_viterbi_alignment_bit_exact(ctx, mb, D):
     """zr_attn_viterbi against the oracle on crafted weights: ties (first maximum wins), all-zero live columns, masked

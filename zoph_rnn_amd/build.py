@@ -8,7 +8,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libzoph_rnn_hip.so")
 SOURCES = ["zr_runtime.hip", "zr_elementwise.hip", "zr_gemm.hip", "zr_lstm.hip", "zr_softmax.hip",
-           "zr_attention.hip", "zr_beam.hip", "zr_backward.hip"]
+           "zr_attention.hip", "zr_attn_step.hip", "zr_beam.hip", "zr_backward.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
          # packed fp32 VALU forms are kept out of the generated code on this hardware pool

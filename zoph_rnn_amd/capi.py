@@ -22,8 +22,13 @@ ZR_OPT_LSTM_SWEEP = 7
 ZR_OPT_LSTM_SWEEP_SPIN = 8
 ZR_OPT_BF16_ACTIVATION_TERMS = 9
 ZR_OPT_LSTM_STEP_WAIT_EXTRA = 10
+ZR_OPT_ATTN_SINGLE_LAUNCH = 11
 ZR_QUERY_LSTM_STACK_PATH = 1
 ZR_QUERY_LSTM_SWEEP_ABANDONED = 2
+ZR_QUERY_ATTN_PATH = 3
+ZR_ATTN_PATH_SINGLE_LAUNCH = 1
+ZR_ATTN_PATH_THREE_LAUNCHES = 2
+ZR_ATTN_PATH_SEPARATE = 3
 ZR_LSTM_STACK_PATH_SWEEP = 1
 ZR_LSTM_STACK_PATH_DIAGONALS = 2
 ZR_LSTM_STACK_PATH_STEP_SINGLE_LAUNCH = 3

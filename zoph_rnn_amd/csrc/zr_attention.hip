@@ -597,6 +597,7 @@ int zr_attn_create(zr_ctx* ctx, int H, int mb, int D, const float* d_W_a, const 
   a->d_bf16 = nullptr;
   a->ldp = 0;
   a->d_pack32 = nullptr;
+  a->d_pq = nullptr;
   a->d_err_table = nullptr;
   a->ldp32 = a->kp32 = 0;
   const size_t n = (size_t)H * mb, W = 2 * (size_t)D + 1;
@@ -692,7 +693,8 @@ int zr_attn_prepare(zr_ctx* ctx, zr_attn* a) {
   const int ldp = (H + 31) / 32 * 32, kp = (H + 7) / 8 * 8;
   const size_t per = (size_t)kp * ldp;
   if (!a->d_pack32) {
-    if (hipMalloc((void**)&a->d_pack32, sizeof(float) * (4 * per + 3 * (size_t)H * a->mb)) != hipSuccess) {
+    if (hipMalloc((void**)&a->d_pack32, sizeof(float) * (4 * per + 3 * (size_t)H * a->mb + 3 * (size_t)ldp * a->mb + 32)) !=
+        hipSuccess) {
       (void)hipGetLastError();
       a->d_pack32 = nullptr;
       return zr_set_error(ZR_ENOMEM, "zr_attn_prepare: allocation failed");
@@ -705,6 +707,8 @@ int zr_attn_prepare(zr_ctx* ctx, zr_attn* a) {
   a->d_cpack = a->d_pack32 + 4 * per;
   a->d_hpack = a->d_cpack + (size_t)H * a->mb;
   a->d_htpack = a->d_hpack + (size_t)H * a->mb;
+  // (every column of these two starts a 128-byte line, so that a line has one producing tile and one consuming column)
+  a->d_pq = a->d_pack32 + (4 * per + 3 * (size_t)H * a->mb + 31) / 32 * 32;
   rc = zr_pack4_launch(ctx, a->W_p, H, H, H, ldp, kp, a->d_pack32);
   if (rc) return rc;
   rc = zr_pack4_trans_launch(ctx, a->W_a, H, H, H, ldp, kp, a->d_pack32 + per);  // W_a^T
@@ -843,6 +847,16 @@ static int attn_step_impl(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, cons
       rc = zr_pack4_x_launch(ctx, d_h_t, H, mb, H, a->d_hpack);
       if (rc) return rc;
     }
+    if (bp && ctx->attn_single != 1) {
+      int took = 0;
+      rc = zr_attn_step_single_launch(ctx, a, d_batch_info, d_mask01, d_htild, d_htild_pack, align, idx, pt, cctx, &took);
+      if (rc) return rc;
+      if (took) {
+        ctx->last_attn_path = ZR_ATTN_PATH_SINGLE_LAUNCH;
+        return ZR_OK;
+      }
+    }
+    ctx->last_attn_path = ZR_ATTN_PATH_THREE_LAUNCHES;
     g.B[0] = bp ? a->d_hpack : d_h_t;
     g.b_packed = bp ? 1 : 0;
     g.ldb[0] = H;
@@ -890,6 +904,7 @@ static int attn_step_impl(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, cons
     return zr_gemm_launch(ctx, o);
   }
 
+  ctx->last_attn_path = ZR_ATTN_PATH_SEPARATE;
   // tanh(W_p h)  (reference: attention_node.hpp:132-141)
   ZrGemmDesc g = {};
   g.M = H;

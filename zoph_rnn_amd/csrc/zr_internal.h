@@ -30,6 +30,9 @@ struct zr_ctx {
   int cu_count;      // compute units of the device (filled with sweep_capacity)
   int sweep_capacity[3];  // resident workgroups of lstm_sweep_kernel<TN> (0: not asked yet, -1: unknown)
   int stack_step_capacity;  // the same for lstm_decoder_stack_kernel (the lesser of its two tile widths)
+  int attn_step_capacity[3];  // the same for attn_step_kernel<8 / 16 / 32>
+  int attn_single;      // ZR_OPT_ATTN_SINGLE_LAUNCH
+  int last_attn_path;   // ZR_ATTN_PATH_* of the last attention step (0: none yet)
   int gemm_cfg;
   int bf16_terms;       // bf16-weight products: 2 (default, 0 = 2) = activations as two bf16 terms, 1 = rounded to bf16 once
   int last_stack_path;  // ZR_LSTM_STACK_PATH_* of the last zr_lstm_stack_forward(_train) call (0: none yet)
@@ -196,6 +199,12 @@ int zr_softmax_forward_packed(zr_ctx* ctx, const float* d_D, const float* d_b_d,
                               const float* d_h_packed, int mb, int mode, float* d_out, float* d_logits_scratch,
                               const unsigned short* d_h_hi = nullptr, const unsigned short* d_h_lo = nullptr);
 
+// The attention step in one launch (zr_attn_step.hip).  a->d_hpack must hold h_t k-interleaved.  *took = 0: the
+// conditions do not hold and nothing was launched (the caller goes on with one launch per stage).
+struct zr_attn;
+int zr_attn_step_single_launch(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, const int* d_mask01, float* d_htild,
+                               float* d_htild_pack, float* align, int* idx, float* pt, float* cctx, int* took);
+
 // The attention layer's handle (zr_attention.hip; the backward pass lives in zr_backward.hip).
 struct zr_attn {
   int H, mb, D, longest_sent;
@@ -213,6 +222,8 @@ struct zr_attn {
   int ldp32, kp32;
   float *d_hpack, *d_cpack;  // k-interleaved copies ([H/4][mb][4]) of h_t and of the context (inside d_pack32's block)
   float* d_htpack;           // the same of h~, written by the output product for zr_decoder_step (same block)
+  float* d_pq;               // single-launch step: W_p h_t, W_a^T h_t and the context in padded columns (3 x ldp32 x mb,
+                             // same block, 128-byte aligned)
   // bf16 matrices: h~ of the last step as bf16 terms ([H/8][mb][8], inside d_bf16's block), written by the output
   // product for a bf16 output layer behind it in zr_decoder_step; null when the last step did not write them
   const unsigned short* htild_hi;

@@ -176,6 +176,9 @@ int zr_ctx_query(zr_ctx* ctx, int what, int* h_value) {
     case ZR_QUERY_LSTM_STACK_PATH:
       *h_value = ctx->last_stack_path;
       return ZR_OK;
+    case ZR_QUERY_ATTN_PATH:
+      *h_value = ctx->last_attn_path;
+      return ZR_OK;
     case ZR_QUERY_LSTM_SWEEP_ABANDONED: {
       int rc = zr_bind_device(ctx);
       if (rc) return rc;
@@ -230,6 +233,10 @@ int zr_ctx_set_option(zr_ctx* ctx, int option, int value) {
     case ZR_OPT_LSTM_STEP_WAIT_EXTRA:
       ZR_CHECK_ARG(value >= 0 && value <= 1024, "ZR_OPT_LSTM_STEP_WAIT_EXTRA must be in [0, 1024]");
       ctx->step_wait_extra = value;
+      return ZR_OK;
+    case ZR_OPT_ATTN_SINGLE_LAUNCH:
+      ZR_CHECK_ARG(value == 0 || value == 1, "ZR_OPT_ATTN_SINGLE_LAUNCH must be 0 or 1");
+      ctx->attn_single = value;
       return ZR_OK;
     case ZR_OPT_BF16_ACTIVATION_TERMS:
       ZR_CHECK_ARG(value == 1 || value == 2, "ZR_OPT_BF16_ACTIVATION_TERMS must be 1 or 2");
