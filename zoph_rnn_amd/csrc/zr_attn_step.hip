@@ -183,7 +183,7 @@ __global__ void __launch_bounds__(512) attn_step_kernel(AttnStep P) {
         const unsigned wsoff[1] = {0u};
         const unsigned xoffb[1] = {16u * (unsigned)(col + half * mb)};
         const unsigned woffb = 16u * (unsigned)(j0 + jl + half * P.ldp);
-        zr_mma_segment_u<1, 1, KS, PF>(acc, zr_make_rsrc(P.wpack + (long long)pr * P.per), wsoff, woffb,
+        zr_mma_segment_ring<1, 1, KS, PF>(acc, zr_make_rsrc(P.wpack + (long long)pr * P.per), wsoff, woffb,
                                        32u * (unsigned)P.ldp, zr_make_rsrc(P.hpack), xoffb, 32u * (unsigned)mb, H, wave);
         float* out = pr == 0 ? P.pre : P.q;
         zr_reduce_visit<1, 1, KS>(acc, red, wave, lane, [&](const float(&v)[1], int, int r, int) {
@@ -402,7 +402,7 @@ __global__ void __launch_bounds__(512) attn_step_kernel(AttnStep P) {
       const unsigned xoffb[1] = {16u * (unsigned)(col + half * mb)};
       const unsigned woffb = 16u * (unsigned)(j0 + jl + half * P.ldp);
       const unsigned wstep = 32u * (unsigned)P.ldp, xstep = 32u * (unsigned)mb;
-      zr_mma_segment_u<1, 1, KS, PF>(acc, zr_make_rsrc(P.wpack + 3 * P.per), wsoff, woffb, wstep, zr_make_rsrc(P.hpack),
+      zr_mma_segment_ring<1, 1, KS, PF>(acc, zr_make_rsrc(P.wpack + 3 * P.per), wsoff, woffb, wstep, zr_make_rsrc(P.hpack),
                                      xoffb, xstep, H, wave);
       ZR_STAMP(9);
 #pragma unroll

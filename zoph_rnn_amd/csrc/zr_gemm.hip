@@ -30,6 +30,7 @@ struct GemmArgs {
   // k-interleaved by 8 ([K/8][N][8]); see zr_split_pack_x_kernel
   const unsigned short* Blo[3];
   int accum;  // ZR_EPI_STORE only: C += result instead of C = result
+  int stream_a;  // the weights are fetched with the streaming hint (ZrGemmDesc::stream_a)
   // groups > 0: blockIdx.z = group * batch + batch index; the group picks A, B and C from these tables
   int groups, batch;
   const float* gA[8];
@@ -121,7 +122,7 @@ __device__ __forceinline__ void softmax_partial_epilogue(const GemmArgs& a, floa
 // epilogue.  `active` false: same control flow (barriers), nothing stored.  PF = prefetch distance in k-groups.
 // BUF (k-interleaved fp32 operands on both sides, K % 8 == 0, every row and column of the tile in range, operands below
 // 4 GiB): the K loop fetches through buffer descriptors with the pinned schedule of zr_mma_segment_u.
-template <int TM, int TN, int KS, int AMODE, bool VEC, int EPI, int PF, bool BUF = false>
+template <int TM, int TN, int KS, int AMODE, bool VEC, int EPI, int PF, bool BUF = false, int WAUX = 0>
 __device__ __forceinline__ void gemm_tile(const GemmArgs& a, int m0, int n0, bool active, int z, float* redp,
                                           int kslice, int lane) {
   const int jl = lane & 31;
@@ -175,7 +176,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& a, int m0, int n0, boo
 #pragma unroll
       for (int tn = 0; tn < TN; ++tn) xoffb[tn] = 16u * (unsigned)(n0 + tn * 32 + jl + half * a.N);
       const unsigned woffb = 16u * (unsigned)(m0 + jl + half * (int)a.lda[s]);
-      zr_mma_segment_u<TM, TN, KS, PF>(acc, zr_make_rsrc(a.A[s]), wsoff, woffb, 32u * (unsigned)a.lda[s],
+      zr_mma_segment_ring<TM, TN, KS, PF, WAUX>(acc, zr_make_rsrc(a.A[s]), wsoff, woffb, 32u * (unsigned)a.lda[s],
                                        zr_make_rsrc(a.B[s]), xoffb, 32u * (unsigned)a.N, a.K[s], kslice);
     } else if constexpr (zr_is_bf16_mode(AMODE)) {
       const unsigned short* wbase[TM];
@@ -415,7 +416,7 @@ __global__ void __launch_bounds__(256) gemm_rows_kernel(GemmArgs a, int row_chun
 // last 256 run one to a CU) changed nothing: 123.9 us for the whole output layer either way.
 // Minibatches that are a multiple of 64 but not of 128 columns wide (192 beam columns) take 64 x 64 tiles at three
 // workgroups per CU.
-template <int EPI, int TM, int TN, int PF, int OCC>
+template <int EPI, int TM, int TN, int PF, int OCC, int WAUX>
 __global__ void __launch_bounds__(256, OCC) gemm_tall_kernel(GemmArgs a, int big_rows, int n_col_tiles, int n_big) {
   __shared__ float red[4 * TN * 16 * 64];
   const int tid = threadIdx.x;
@@ -427,7 +428,7 @@ __global__ void __launch_bounds__(256, OCC) gemm_tall_kernel(GemmArgs a, int big
     const int mpx = big_rows >> 3;  // big_rows is a multiple of 8
     const int nt = q % n_col_tiles;
     const int mt = r8 * mpx + q / n_col_tiles;
-    gemm_tile<TM, TN, 4, ZR_A_PACK4, true, EPI, PF, true>(a, mt * 32 * TM, nt * 32 * TN, true, 0, red, kslice, lane);
+    gemm_tile<TM, TN, 4, ZR_A_PACK4, true, EPI, PF, true, WAUX>(a, mt * 32 * TM, nt * 32 * TN, true, 0, red, kslice, lane);
   } else {
     const int idx = bid - n_big;
     const int n32 = (a.N + 31) >> 5;
@@ -994,10 +995,13 @@ bool launch_tall_v(zr_ctx* ctx, GemmArgs& ga, int epi, int* rc) {
   const int n_big = (int)(big_rows * n_col_tiles);
   const unsigned grid = (unsigned)(n_big + small);
   if (epi == ZR_EPI_STORE)
-    gemm_tall_kernel<ZR_EPI_STORE, TM, TN, PF, OCC><<<grid, 256, 0, ctx->stream>>>(ga, (int)big_rows, n_col_tiles, n_big);
+    gemm_tall_kernel<ZR_EPI_STORE, TM, TN, PF, OCC, 0><<<grid, 256, 0, ctx->stream>>>(ga, (int)big_rows, n_col_tiles, n_big);
+  else if (ga.stream_a)
+    gemm_tall_kernel<ZR_EPI_SOFTMAX_PARTIAL, TM, TN, PF, OCC, ZR_AUX_STREAM><<<grid, 256, 0, ctx->stream>>>(
+        ga, (int)big_rows, n_col_tiles, n_big);
   else
-    gemm_tall_kernel<ZR_EPI_SOFTMAX_PARTIAL, TM, TN, PF, OCC><<<grid, 256, 0, ctx->stream>>>(ga, (int)big_rows, n_col_tiles,
-                                                                                            n_big);
+    gemm_tall_kernel<ZR_EPI_SOFTMAX_PARTIAL, TM, TN, PF, OCC, 0><<<grid, 256, 0, ctx->stream>>>(ga, (int)big_rows,
+                                                                                               n_col_tiles, n_big);
   hipError_t e = hipGetLastError();
   *rc = e == hipSuccess ? ZR_OK : zr_set_error(ZR_EHIP, "launch of gemm_tall_kernel failed: %s", hipGetErrorString(e));
   return true;
@@ -1239,6 +1243,7 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
   ZR_CHECK_ARG(!d.Cpack || (d.epilogue == ZR_EPI_TANH_BIAS_MASK && d.batch <= 1 && d.groups == 0),
                "gemm: a k-interleaved second result needs the tanh-bias-mask epilogue and a single problem");
   ga.accum = d.accumulate;
+  ga.stream_a = d.stream_a;
   if (d.epilogue == ZR_EPI_TANH_BIAS_MASK) ZR_CHECK_ARG(d.bias && d.mask, "gemm: bias/mask required");
   ZR_CHECK_ARG(!d.accumulate || d.epilogue == ZR_EPI_STORE, "gemm: accumulate needs the plain store epilogue");
   if (d.epilogue == ZR_EPI_SOFTMAX_PARTIAL) ZR_CHECK_ARG(d.bias && d.partials, "gemm: bias/partials required");

@@ -133,6 +133,9 @@ struct ZrGemmDesc {
   unsigned short* Chi;
   unsigned short* Clo;
   int accumulate;   // ZR_EPI_STORE only: C += product (+ bias) instead of C = ...
+  // A is read once per step and is a large part of the memory-side cache: fetch it with the non-temporal hint so that
+  // it does not push out what the rest of the step reads again (honoured by the kernel of the output layer's product)
+  int stream_a;
   // groups > 0: that many independent problems of the same shape in one launch (at most 8; one segment, plain store
   // epilogue, no bias): problem g multiplies gA[g] (instead of A[0]) with gB[g] (instead of B[0]) into gC[g]
   // (instead of C); lda/ldb/ldc, the batch count and its strides apply inside every problem.

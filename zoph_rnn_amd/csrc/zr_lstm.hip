@@ -207,9 +207,9 @@ __global__ void __launch_bounds__(64 * KS) lstm_fused_kernel(LstmLaunch L) {
         xoffb[tn] = packed ? 16u * ((unsigned)cols[tn] + (unsigned)(half * L.mb)) : 4u * (c * (unsigned)H + 4u * half);
       }
       const float* xb = packed ? U.inp[s] + (long long)g0 * 8 * L.mb : U.in[s] + g0 * 8;
-      zr_mma_segment_u<4, TN, KS, lstm_prefetch_depth(TN, KS)>(acc, zr_make_rsrc(U.W), wsoff, woffb, 32u * (unsigned)L.ldw,
-                                                               zr_make_rsrc(xb), xoffb,
-                                                               packed ? 32u * (unsigned)L.mb : 32u, (g1 - g0) * 8, kslice);
+      zr_mma_segment_ring<4, TN, KS, lstm_prefetch_depth(TN, KS)>(acc, zr_make_rsrc(U.W), wsoff, woffb, 32u * (unsigned)L.ldw,
+                                                                  zr_make_rsrc(xb), xoffb,
+                                                                  packed ? 32u * (unsigned)L.mb : 32u, (g1 - g0) * 8, kslice);
     } else {
       const float* wbase[4];
       unsigned woff[4];

@@ -199,6 +199,11 @@ __device__ __forceinline__ void zr_mma_segment(zr_f32x16 (&acc)[TM][TN], const f
 //   wstep / xstep: bytes per k-group of 8 (weights: 32*lda; activations: 32 for a plain column, 32*mb k-interleaved)
 // Every offset sum must stay below 4 GiB (the host checks the extents).
 typedef unsigned zr_u32x4v __attribute__((ext_vector_type(4)));
+// Cache policy operand of the weight fetches (the buffer-load builtin's last argument): 0 = default, ZR_AUX_STREAM =
+// the non-temporal hint.  A matrix that is read once per step and is a large part of the memory-side cache (the output
+// layer's: 200 MB of its 256 MB at 50 000 x 1000) otherwise pushes out everything the rest of the step re-reads -- the
+// LSTM and attention matrices, the source states -- and every step fetches all of it from memory again.
+constexpr int ZR_AUX_STREAM = 2;
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t zr_make_rsrc(const void* base) {
   // raw buffer, no bounds limit to speak of, 32-bit data format (descriptor word 3 for this GPU family)
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0xFFFFFFFF, 0x00020000);
@@ -207,7 +212,7 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t zr_make_rsrc(const void* base)
 // The weight halves of the first PF ring stages of a segment, issued ahead of time (zr_mma_segment_u with WPRE then
 // fetches only the activation halves in its prologue): weights depend on nothing, so a caller that must wait for its
 // activations can have them in flight during the wait.
-template <int TM, int TN, int KS, int PF>
+template <int TM, int TN, int KS, int PF, int WAUX = 0>
 __device__ __forceinline__ void zr_preload_w(ZrFrag<TM, TN> (&f)[PF + 1], __amdgpu_buffer_rsrc_t wrsrc,
                                              const unsigned (&wsoff)[TM], unsigned woffb, unsigned wstep, int K,
                                              int kslice) {
@@ -219,7 +224,7 @@ __device__ __forceinline__ void zr_preload_w(ZrFrag<TM, TN> (&f)[PF + 1], __amdg
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) {
       const zr_u32x4v v =
-          __builtin_amdgcn_raw_buffer_load_b128(wrsrc, (int)woffb, (int)(wsoff[tm] + (unsigned)gl * wstep), 0);
+          __builtin_amdgcn_raw_buffer_load_b128(wrsrc, (int)woffb, (int)(wsoff[tm] + (unsigned)gl * wstep), WAUX);
       f[s].w[tm][0] = __uint_as_float(v.x);
       f[s].w[tm][1] = __uint_as_float(v.y);
       f[s].w[tm][2] = __uint_as_float(v.z);
@@ -228,7 +233,7 @@ __device__ __forceinline__ void zr_preload_w(ZrFrag<TM, TN> (&f)[PF + 1], __amdg
   }
 }
 
-template <int TM, int TN, int KS, int PF, bool WPRE = false>
+template <int TM, int TN, int KS, int PF, bool WPRE = false, int WAUX = 0>
 __device__ __forceinline__ void zr_mma_segment_u(zr_f32x16 (&acc)[TM][TN], __amdgpu_buffer_rsrc_t wrsrc,
                                                  const unsigned (&wsoff)[TM], unsigned woffb, unsigned wstep,
                                                  __amdgpu_buffer_rsrc_t xrsrc, const unsigned (&xoffb)[TN],
@@ -251,7 +256,7 @@ __device__ __forceinline__ void zr_mma_segment_u(zr_f32x16 (&acc)[TM][TN], __amd
     load_x(f, g);
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) {
-      const zr_u32x4v v = __builtin_amdgcn_raw_buffer_load_b128(wrsrc, (int)woffb, (int)(wsoff[tm] + ug * wstep), 0);
+      const zr_u32x4v v = __builtin_amdgcn_raw_buffer_load_b128(wrsrc, (int)woffb, (int)(wsoff[tm] + ug * wstep), WAUX);
       f.w[tm][0] = __uint_as_float(v.x);
       f.w[tm][1] = __uint_as_float(v.y);
       f.w[tm][2] = __uint_as_float(v.z);
@@ -306,13 +311,13 @@ __device__ __forceinline__ void zr_mma_segment_u(zr_f32x16 (&acc)[TM][TN], __amd
 }
 
 // The same with a ring of its own (no weights fetched ahead).
-template <int TM, int TN, int KS, int PF>
-__device__ __forceinline__ void zr_mma_segment_u(zr_f32x16 (&acc)[TM][TN], __amdgpu_buffer_rsrc_t wrsrc,
+template <int TM, int TN, int KS, int PF, int WAUX = 0>
+__device__ __forceinline__ void zr_mma_segment_ring(zr_f32x16 (&acc)[TM][TN], __amdgpu_buffer_rsrc_t wrsrc,
                                                  const unsigned (&wsoff)[TM], unsigned woffb, unsigned wstep,
                                                  __amdgpu_buffer_rsrc_t xrsrc, const unsigned (&xoffb)[TN],
                                                  unsigned xstep, int K, int kslice) {
   ZrFrag<TM, TN> f[PF + 1];
-  zr_mma_segment_u<TM, TN, KS, PF, false>(acc, wrsrc, wsoff, woffb, wstep, xrsrc, xoffb, xstep, K, kslice, f);
+  zr_mma_segment_u<TM, TN, KS, PF, false, WAUX>(acc, wrsrc, wsoff, woffb, wstep, xrsrc, xoffb, xstep, K, kslice, f);
 }
 
 // Workgroup barrier that also publishes: when it returns, every store any thread of the workgroup issued before it

@@ -209,6 +209,7 @@ int logits_with_partials(zr_ctx* ctx, const float* d_D, const float* d_b_d, int 
   d.batch = 1;
   d.bias = d_b_d;
   d.epilogue = ZR_EPI_SOFTMAX_PARTIAL;
+  d.stream_a = (size_t)V * H * (d.a_pack == 2 ? 2 : 4) >= ((size_t)64 << 20) ? 1 : 0;
   d.partials = (float*)scratch;
   rc = zr_gemm_launch(ctx, d);
   if (rc) return rc;
