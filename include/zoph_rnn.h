@@ -61,7 +61,11 @@ int zr_ctx_set_option(zr_ctx* ctx, int option, int value);
  *     ZR_LSTM_STACK_PATH_STEP_PER_LAYER (zr_lstm_decoder_step).  Does not wait.
  *   ZR_QUERY_LSTM_SWEEP_ABANDONED: waits for the stream; 1 if a single-launch sweep or decoder step since the last look
  *     gave up a wait (its outputs were then overwritten with NaN; run it again with ZR_OPT_LSTM_SWEEP = 1), else 0.  Clears
- *     the flag, so a following zr_ctx_sync no longer reports it.
+ *     the flag -- and with it the data flags that launches queued behind the abandoned one raised on its NaN outputs --
+ *     so a following zr_ctx_sync no longer reports it.  A decoder step called with d_c[l] == d_cprev[l] (cell state
+ *     updated in place) has overwritten its own input by then: running it again needs the caller's copy of c_{t-1}.
+ *   ZR_QUERY_SCRATCH_KIB: device memory the context has allocated for scratch buffers so far, in KiB (0 for a context
+ *     that has only served calls that allocate nothing).  Does not wait.
  *   ZR_QUERY_ATTN_PATH: which schedule the last zr_attn_step (or the attention part of zr_decoder_step) on this
  *     context took -- 0 none yet, ZR_ATTN_PATH_SINGLE_LAUNCH, ZR_ATTN_PATH_THREE_LAUNCHES or ZR_ATTN_PATH_SEPARATE.
  *     Does not wait. */
@@ -69,6 +73,7 @@ int zr_ctx_query(zr_ctx* ctx, int what, int* h_value);
 #define ZR_QUERY_LSTM_STACK_PATH 1
 #define ZR_QUERY_LSTM_SWEEP_ABANDONED 2
 #define ZR_QUERY_ATTN_PATH 3
+#define ZR_QUERY_SCRATCH_KIB 4
 #define ZR_ATTN_PATH_SINGLE_LAUNCH 1  /* projections, window / scores / context and output product in one launch */
 #define ZR_ATTN_PATH_THREE_LAUNCHES 2 /* the same three stages as one launch each */
 #define ZR_ATTN_PATH_SEPARATE 3       /* unprepared or bf16 matrices: products and the middle as separate launches */
@@ -272,7 +277,9 @@ int zr_softmax_forward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V,
  * GPU it runs on, so the call itself allocates and frees nothing.  Limits (ZR_EINVAL beyond them, message in
  * zr_last_error): H*mb*4 <= 8 MiB and ceil(V/32)*mb*8 + 16*mb + 64 <= 24 MiB -- e.g. V = 80000 with 256 columns
  * of H = 2000 fits, 6400 columns of V = 50000 do not.  Every call on one GPU shares that GPU's array: calls that overlap
- * on one GPU (two contexts, two streams) race; calls on one context are ordered by its stream and safe. */
+ * on one GPU (two contexts, two streams) race; calls on one context are ordered by its stream and safe.  Like every
+ * entry point, it must not be called on one context from two host threads at once (a context is single-threaded: for
+ * the duration of this call its scratch requests are redirected to the static array). */
 int zr_softmax_forward_static(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h,
                               int mb, int mode, float* d_out, float* d_logits_scratch);
 /* softmax_layer::get_perplexity_GPU (src/softmax.hpp:636-692) with outputdist_perplexity_kernel

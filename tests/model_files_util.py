@@ -87,11 +87,15 @@ def run_force_decode(args, timeout=300):
     return subprocess.run([exe] + [str(a) for a in args], capture_output=True, text=True, timeout=timeout)
 
 
-def run_program(name, args, timeout=300):
-    """Runs zoph_rnn_amd/host/<name> (built by `python __graft_entry__.py build`)."""
+def run_program(name, args, timeout=300, env=None):
+    """Runs zoph_rnn_amd/host/<name> (built by `python __graft_entry__.py build`); env: extra environment variables."""
     exe = os.path.join(ROOT, "zoph_rnn_amd", "host", name)
     assert os.path.exists(exe), "%s is not built: run `python __graft_entry__.py build`" % exe
-    return subprocess.run([exe] + [str(a) for a in args], capture_output=True, text=True, timeout=timeout)
+    full_env = None
+    if env:
+        full_env = dict(os.environ)
+        full_env.update({k: str(v) for k, v in env.items()})
+    return subprocess.run([exe] + [str(a) for a in args], capture_output=True, text=True, timeout=timeout, env=full_env)
 
 
 def random_sentences(g, vocab, n, min_len, max_len, oov_rate=0.1, oov_prefix="oov"):

@@ -212,6 +212,42 @@ def test_beam_decode_cli_ensemble_refuses_mismatched_models(tmp_path):
     assert r.returncode != 0 and "vocabular" in r.stderr
 
 
+def test_beam_decode_cli_decodes_a_batch_again_after_an_abandoned_launch(tmp_path):
+    """The decoder's context is put on the single-launch schedules whenever they fit, with waits that expect one arrival
+    more than will come and a poll limit of 64 (every kernel still exits normally): the first decoder step's launch gives
+    up, the program notices after that step, switches the context to one launch per layer and decodes the batch again.
+    The output must be that of an ordinary run, and the program says how often it started over."""
+    g = synth.rng(97, 1)
+    H, L, beam, batch, longest, D, K = 64, 2, 4, 3, 24, 3, 2
+    src_vocab = ["<UNK>"] + mf.make_vocab(60, "s")
+    tgt_vocab = ["<START>", "<EOF>", "<UNK>"] + mf.make_vocab(300, "t")
+    m = _model(g, H, len(src_vocab), len(tgt_vocab), L)
+    model = tmp_path / "model.nn"
+    _write_model(model, m, L, H, tgt_vocab, src_vocab)
+    src = [mf.random_sentences(g, src_vocab, 1, n, n)[0] for n in (5, 6, 5, 5, 6)]
+    sp = tmp_path / "src.txt"
+    sp.write_text("".join(" ".join(s) + "\n" for s in src))
+    outs = []
+    for name, env in (("plain", None),
+                      ("abandon", {"ZR_LSTM_SWEEP": 2, "ZR_LSTM_SWEEP_SPIN": 64, "ZR_LSTM_STEP_WAIT_EXTRA": 1})):
+        out = tmp_path / (name + ".txt")
+        r = mf.run_program("beam_decode", ["--beam", beam, "--batch", batch, "--longest-sent", longest,
+                                           "--attention-width", D, "--num-best", K, "--print-score", "--ids", model, sp,
+                                           out], env=env)
+        assert r.returncode == 0, (name, r.stderr[-2000:])
+        outs.append((_parse_blocks(out.read_text()), r.stdout))
+    (plain, plain_log), (again, again_log) = outs
+    assert "decoded again" not in plain_log
+    counts = [int(ln.split(":")[1]) for ln in again_log.split("\n") if "decoded again" in ln]
+    # two source lengths -> two batches of 3 and of 2 sentences; the first gives up and switches the context over for good
+    assert counts == [1], again_log
+    assert len(plain) == len(again) == len(src)
+    for a, b in zip(plain, again):
+        assert [w for w, _ in a] == [w for w, _ in b]
+        for (_, sa), (_, sb) in zip(a, b):
+            assert sa == pytest.approx(sb, rel=1e-4, abs=1e-4)
+
+
 def test_beam_decode_cli_default_output_is_words(tmp_path):
     g = synth.rng(96, 1)
     H, L = 48, 1

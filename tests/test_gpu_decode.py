@@ -76,7 +76,7 @@ def _oracle_decode(m, src_col, src_len, S, beam, steps, D, penalty, viterbi=Fals
         n_hyp_before = len(dec.hypotheses())
         frac = att["p_t"] - np.floor(att["p_t"])
         assert np.all((frac > 1e-4) & (frac < 1 - 1e-4)), "p_t on an integer boundary; pick another seed"
-        dec.expand(P, index, o.attention_viterbi(att["alignments"], att["indices"]) if viterbi else None)
+        dec.expand(P, index, _single_model_vote(att, S) if viterbi else None)
         popped = beam + (len(dec.hypotheses()) - n_hyp_before) + 2  # survivors + <EOF> hypotheses (+ a <START>) + next
         min_gap = min(min_gap, np.min(-np.diff(cand[:popped + 1])))
         st = dec.state()
@@ -86,10 +86,18 @@ def _oracle_decode(m, src_col, src_len, S, beam, steps, D, penalty, viterbi=Fals
         cp = [np.asfortranarray(a[:, back]) for a in newc]
         h_tild = np.asfortranarray(att["h_tild"][:, back])
     _, _, att, P = forward(steps)
-    dec.finish(P, o.attention_viterbi(att["alignments"], att["indices"]) if viterbi else None)
+    dec.finish(P, _single_model_vote(att, S) if viterbi else None)
     if viterbi:
         return hist, dec.hypotheses(), min_gap, dec.hypotheses_viterbi()
     return hist, dec.hypotheses(), min_gap
+
+
+def _single_model_vote(att, S):
+    """The alignment the reference's driver hands its decoder: also for one model it is the vote of
+    ensemble_factory::ensembles_models (src/ensemble_factory.hpp:797-834), which overwrites the attention layer's own
+    Viterbi alignment -- the two differ where no weight of a column's window is positive (-1 instead of the first
+    slot's position)."""
+    return ensemble_alignment_vote([att["alignments"]], [att["indices"]], S + 4)
 
 
 def ensemble_alignment_vote(aligns, indices, longest):

@@ -873,12 +873,17 @@ def test_decoder_step_single_launch_abandoned_wait_is_reported(ctx, H, mb, L):
 
 @pytest.mark.parametrize("H,mb,L,S,D,V,prepared", [(1000, 128, 4, 20, 10, 5000, True), (64, 5, 2, 9, 3, 301, True),
                                                    (1000, 128, 2, 12, 12, 2000, False), (100, 8, 1, 7, 2, 333, True),
-                                                   (256, 64, 3, 30, 50, 40000, True)])
+                                                   (256, 64, 3, 30, 50, 40000, True),
+                                                   # v_p at a 4-byte offset (see below)
+                                                   (1000, 128, 4, 20, 10, 5000, "v_p off by 4 bytes"),
+                                                   (64, 5, 2, 9, 3, 301, "v_p off by 4 bytes")])
 def test_decoder_step_as_one_call_matches_the_three_calls(ctx, H, mb, L, S, D, V, prepared):
     """zr_decoder_step (forward_prop_target as one call, hand-overs kept in the matrix cores' layout) against
     zr_lstm_decoder_step + zr_attn_step + zr_softmax_forward on the same inputs: the same kernels read the same numbers,
     so every output is the same bit for bit -- with and without the prepared snapshots, with an LSTM stack that takes
-    the single launch and one that does not, with a layer size the packed layout does not cover."""
+    the single launch and one that does not, with a layer size the packed layout does not cover.  With v_p misaligned
+    the attention step cannot run on its snapshots and writes no k-interleaved h~: the output layer must then read the
+    plain one."""
     g = synth.rng(35, H + mb + L)
     case = _decoder_step_case(g, H, mb, L, True, V=V)
     layers, embed, ids, hp, cp, ht, mask = case
@@ -890,7 +895,11 @@ def test_decoder_step_as_one_call_matches_the_three_calls(ctx, H, mb, L, S, D, V
     lys = [Layer(ctx, ly) for ly in layers]
     tables = [ctx.array(np.asfortranarray(hs[t])) for t in range(S)]
     dw = {k: ctx.array(v) for k, v in w.items()}
-    a = ctx.attn_create(H, mb, D, dw["W_a"], dw["W_p"], dw["v_p"], dw["out_bias"], dw["W_c1"], dw["W_c2"], tables)
+    v_p = dw["v_p"]
+    if prepared == "v_p off by 4 bytes":
+        d_vp_shifted = ctx.array(np.concatenate([np.zeros(1, np.float32), w["v_p"].reshape(-1)]))
+        v_p = d_vp_shifted.at(1)
+    a = ctx.attn_create(H, mb, D, dw["W_a"], dw["W_p"], v_p, dw["out_bias"], dw["W_c1"], dw["W_c2"], tables)
     dD, dbd = ctx.array(Dm), ctx.array(bd)
     if prepared:
         ctx.attn_prepare(a)

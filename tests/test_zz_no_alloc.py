@@ -32,8 +32,13 @@ def test_static_scratch_entry_point_matches_allocating_one_twice_in_a_row(prepar
         # first call: a large product (the prepared path re-lays-out the activations: both scratch slots in use);
         # second call: a smaller one on the same array, whose stale contents must not leak into the result
         for (V, H, mb, mode, seed) in [(20000, 256, 96, capi.ZR_SOFTMAX_PROB, 1), (4100, 64, 24, capi.ZR_SOFTMAX_LOGPROB, 2)]:
+            before = ctx.query(capi.ZR_QUERY_SCRATCH_KIB)
             got, (D, bd, h) = _run(ctx, V, H, mb, mode, prepared, seed, static=True)
+            # the static call allocates nothing: the context's own scratch is what it was (nothing at all the first time)
+            assert ctx.query(capi.ZR_QUERY_SCRATCH_KIB) == before
+            assert before > 0 or seed != 1 or ctx.query(capi.ZR_QUERY_SCRATCH_KIB) == 0
             want, _ = _run(ctx, V, H, mb, mode, prepared, seed, static=False)
+            assert ctx.query(capi.ZR_QUERY_SCRATCH_KIB) > 0  # (the allocating entry point did grow it)
             assert got.tobytes() == want.tobytes(), "static-scratch result differs from the allocating entry point"
             # and both are the oracle's soft-max
             logits = oracle.softmax_logits(D, bd, h)
@@ -59,6 +64,18 @@ def test_static_scratch_entry_point_rejects_what_does_not_fit():
         with pytest.raises(capi.ZrError) as e:
             ctx.softmax_forward(dD, db, V, H, dh, mb, capi.ZR_SOFTMAX_PROB, out, static=True)
         assert e.value.code == -1 and "allocation-free" in str(e.value)
+        ctx.sync()
+        # the other buffer's limit: 2304 x 1000 re-laid-out activations are 9.2 MB > 8 MiB (prepared matrix)
+        V, H, mb = 2048, 2304, 1000  # (the re-lay-out is taken from 2048 rows on)
+        dD, db = ctx.array(synth.uniform(g, (V, H))), ctx.array(synth.uniform(g, (V,)))
+        dh = ctx.array(synth.uniform(g, (H, mb)))
+        ctx.softmax_prepare(dD, V, H)
+        out = ctx.empty((V, mb))
+        with pytest.raises(capi.ZrError) as e:
+            ctx.softmax_forward(dD, db, V, H, dh, mb, capi.ZR_SOFTMAX_PROB, out, static=True)
+        assert e.value.code == -1 and "allocation-free" in str(e.value) and "re-laid-out" in str(e.value)
+        assert ctx.query(capi.ZR_QUERY_SCRATCH_KIB) == 0
+        ctx.softmax_release(dD)
         ctx.sync()
     finally:
         ctx.close()

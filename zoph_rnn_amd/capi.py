@@ -26,6 +26,7 @@ ZR_OPT_ATTN_SINGLE_LAUNCH = 11
 ZR_QUERY_LSTM_STACK_PATH = 1
 ZR_QUERY_LSTM_SWEEP_ABANDONED = 2
 ZR_QUERY_ATTN_PATH = 3
+ZR_QUERY_SCRATCH_KIB = 4
 ZR_ATTN_PATH_SINGLE_LAUNCH = 1
 ZR_ATTN_PATH_THREE_LAUNCHES = 2
 ZR_ATTN_PATH_SEPARATE = 3

@@ -741,11 +741,17 @@ int zr_attn_step(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, const float* 
                         nullptr);
 }
 
-// True when zr_attn_step on these operands takes the path that reads a->d_hpack (and can write h~ k-interleaved).
-static bool attn_reads_packed_h(const zr_attn* a, const float* d_h_t, const float* d_c_ctx) {
+// True when zr_attn_step on these operands runs on the k-interleaved fp32 snapshots (the single launch or the three
+// launches): prepared matrices and everything it reads with 16-byte accesses aligned.  The one predicate for both the
+// step itself and zr_decoder_step's choice of hand-over layout.
+static bool attn_on_snapshots(const zr_attn* a, const float* d_h_t, const float* d_c_ctx) {
   const float* cctx = d_c_ctx ? d_c_ctx : a->d_ctx;
-  return a->d_pack32 && !a->d_bf16 && (a->H % 8 == 0) && a->tables_aligned && (((uintptr_t)cctx & 15u) == 0) &&
-         (((uintptr_t)d_h_t & 15u) == 0);
+  return a->d_pack32 && !a->d_bf16 && (a->H % 4 == 0) && a->tables_aligned &&
+         ((((uintptr_t)cctx | (uintptr_t)d_h_t | (uintptr_t)a->v_p) & 15u) == 0);
+}
+// ... and reads h_t from a->d_hpack (and can write h~ k-interleaved)
+static bool attn_reads_packed_h(const zr_attn* a, const float* d_h_t, const float* d_c_ctx) {
+  return attn_on_snapshots(a, d_h_t, d_c_ctx) && a->H % 8 == 0;
 }
 
 int zr_decoder_step(zr_ctx* ctx, int nl, const zr_lstm_weights* const layers[], const float* d_embed, int V_in,
@@ -775,8 +781,10 @@ int zr_decoder_step(zr_ctx* ctx, int nl, const zr_lstm_weights* const layers[], 
   rc = attn_step_impl(ctx, attn, d_batch_info, top, d_mask01, d_htild, d_alignments, d_indices, d_p_t, d_c_ctx,
                       (pack32 || split16) && wrote, packed ? attn->d_htpack : nullptr);
   if (rc) return rc;
-  return zr_softmax_forward_packed(ctx, d_D, d_b_d, V_out, attn->H, d_htild, packed ? attn->d_htpack : nullptr, mb, mode,
-                                   d_out, nullptr, attn->htild_hi, attn->htild_lo);
+  // (the k-interleaved h~ only if the attention step says it wrote it)
+  return zr_softmax_forward_packed(ctx, d_D, d_b_d, V_out, attn->H, d_htild,
+                                   attn->wrote_htild_pack ? attn->d_htpack : nullptr, mb, mode, d_out, nullptr,
+                                   attn->htild_hi, attn->htild_lo);
 }
 
 // Everything between the projections and the output product in one launch (d_tanh1 holds W_p h BEFORE the tanh, d_q
@@ -826,9 +834,10 @@ static int attn_step_impl(zr_ctx* ctx, zr_attn* a, const int* d_batch_info, cons
   float* pt = d_p_t ? d_p_t : a->d_pt;
   float* cctx = d_c_ctx ? d_c_ctx : a->d_ctx;
 
-  const bool fast = a->d_pack32 && !a->d_bf16 && (H % 4 == 0) && a->tables_aligned &&
-                    ((((uintptr_t)cctx | (uintptr_t)d_h_t | (uintptr_t)a->v_p) & 15u) == 0);
+  a->wrote_htild_pack = false;
+  const bool fast = attn_on_snapshots(a, d_h_t, d_c_ctx);
   if (fast) {
+    a->wrote_htild_pack = d_htild_pack != nullptr && H % 8 == 0;
     // Three launches.  (1) W_p h (before the tanh) and q = W_a^T h as one batch of two products on the k-interleaved
     // snapshots; d_tanh1 and d_q are neighbours in the object's allocation (stride H*mb).
     const size_t per = (size_t)a->kp32 * a->ldp32;

@@ -547,8 +547,8 @@ int zr_beam_create(zr_ctx* ctx, int beam, int vocab, int n_sent, int max_len, fl
   const int kTopkChunk = topk_chunk(topk_e4_for(vocab));
   ZR_CHECK_ARG(vocab > beam + 1 && n_sent >= 1 && max_len >= 3, "zr_beam_create: vocab = %d, n_sent = %d, max_len = %d",
                vocab, n_sent, max_len);
-  // the reference caps the beam at floor(sqrt(V)) (src/ensemble_factory.hpp:19-21)
-  ZR_CHECK_ARG((long long)beam * beam <= vocab, "zr_beam_create: beam %d exceeds sqrt(vocab %d)", beam, vocab);
+  // (the reference's driver caps the beam at floor(sqrt(V)) before it builds its decoder, src/ensemble_factory.hpp:19-21;
+  // that is the caller's rule, as there: beam_decoder in host/zoph_model.h applies it)
   zr_beam* b = new zr_beam();
   b->beam = beam;
   b->vocab = vocab;

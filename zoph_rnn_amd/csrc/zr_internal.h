@@ -225,6 +225,7 @@ struct zr_attn {
   int ldp32, kp32;
   float *d_hpack, *d_cpack;  // k-interleaved copies ([H/4][mb][4]) of h_t and of the context (inside d_pack32's block)
   float* d_htpack;           // the same of h~, written by the output product for zr_decoder_step (same block)
+  bool wrote_htild_pack;     // the last attention step wrote d_htpack
   float* d_pq;               // single-launch step: W_p h_t, W_a^T h_t and the context in padded columns (3 x ldp32 x mb,
                              // same block, 128-byte aligned)
   // bf16 matrices: h~ of the last step as bf16 terms ([H/8][mb][8], inside d_bf16's block), written by the output

@@ -1577,9 +1577,15 @@ int zr_lstm_decoder_step_packed(zr_ctx* ctx, int nl, const zr_lstm_weights* cons
     ZR_CHECK_ARG(layers[l]->bf16 == layers[0]->bf16, "zr_lstm_decoder_step: layers mix fp32 and bf16 weights");
     ZR_CHECK_ARG(d_hprev[l] && d_cprev[l] && d_h[l] && d_c[l], "zr_lstm_decoder_step: null state for layer %d", l);
     ZR_CHECK_ARG(d_h[l] != d_htild, "zr_lstm_decoder_step: d_h[%d] aliases d_htild", l);
-    for (int m = 0; m < nl; ++m)
+    for (int m = 0; m < nl; ++m) {
       ZR_CHECK_ARG(d_h[l] != d_hprev[m] && (l == m || d_h[l] != d_h[m]),
                    "zr_lstm_decoder_step: d_h[%d] aliases another state array", l);
+      // the cell state may be updated in place (d_c[l] == d_cprev[l]: each element is read and written by one thread);
+      // anything else a workgroup of another tile or layer reads while this one writes may not be d_c[l]
+      ZR_CHECK_ARG(d_c[l] != d_hprev[m] && d_c[l] != d_h[m] && (l == m || (d_c[l] != d_c[m] && d_c[l] != d_cprev[m])),
+                   "zr_lstm_decoder_step: d_c[%d] aliases another state array", l);
+    }
+    ZR_CHECK_ARG(d_c[l] != d_htild, "zr_lstm_decoder_step: d_c[%d] aliases d_htild", l);
     vec = vec && aligned16(d_hprev[l]);
   }
   ZR_CHECK_ARG(!d_htild || layers[0]->nseg == 3, "zr_lstm_decoder_step: d_htild given but layer 0 was packed without Q");

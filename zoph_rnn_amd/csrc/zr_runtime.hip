@@ -126,6 +126,15 @@ int zr_ctx_create(int device, zr_ctx** out) {
     const int v = atoi(e);
     if (v >= 0 && v <= 2) c->lstm_sweep = v;
   }
+  // the same for ZR_OPT_LSTM_SWEEP_SPIN and ZR_OPT_LSTM_STEP_WAIT_EXTRA (tests of a whole program's give-up handling)
+  if (const char* e = getenv("ZR_LSTM_SWEEP_SPIN")) {
+    const int v = atoi(e);
+    if (v >= 0) c->sweep_spin = v;
+  }
+  if (const char* e = getenv("ZR_LSTM_STEP_WAIT_EXTRA")) {
+    const int v = atoi(e);
+    if (v >= 0 && v <= 1024) c->step_wait_extra = v;
+  }
   if (device < 64) g_live[device].fetch_add(1);
   *out = c;
   return ZR_OK;
@@ -176,6 +185,9 @@ int zr_ctx_query(zr_ctx* ctx, int what, int* h_value) {
     case ZR_QUERY_LSTM_STACK_PATH:
       *h_value = ctx->last_stack_path;
       return ZR_OK;
+    case ZR_QUERY_SCRATCH_KIB:
+      *h_value = (int)((ctx->scratch_bytes + ctx->scratch2_bytes + 1023) / 1024);
+      return ZR_OK;
     case ZR_QUERY_ATTN_PATH:
       *h_value = ctx->last_attn_path;
       return ZR_OK;
@@ -185,7 +197,10 @@ int zr_ctx_query(zr_ctx* ctx, int what, int* h_value) {
       ZR_HIP(hipStreamSynchronize(ctx->stream));
       int flag = 0;
       ZR_HIP(hipMemcpy(&flag, ctx->d_flags + 2, sizeof(int), hipMemcpyDeviceToHost));
-      if (flag != 0) ZR_HIP(hipMemset(ctx->d_flags + 2, 0, sizeof(int)));
+      // Everything queued behind the abandoned launch ran on its NaN outputs: the word ids picked from them and the
+      // window positions derived from them are out of range, so the data flags are up as well.  They say nothing about
+      // the caller's data; all four go down together, and the caller's re-run starts from a clean slate.
+      if (flag != 0) ZR_HIP(hipMemset(ctx->d_flags, 0, 4 * sizeof(int)));
       *h_value = flag != 0 ? 1 : 0;
       return ZR_OK;
     }

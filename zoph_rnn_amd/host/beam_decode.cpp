@@ -232,5 +232,7 @@ int main(int argc, char** argv) {
     out << "\n";
   }
   std::cout << "Sentences: " << n_sents << "\n";
+  if (dec.abandoned_launches)
+    std::cout << "Batches decoded again after a single-launch schedule gave up a wait: " << dec.abandoned_launches << "\n";
   return 0;
 }

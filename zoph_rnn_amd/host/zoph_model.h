@@ -967,6 +967,16 @@ class beam_decoder {
   beam_decoder(forward_model<dType>& model, int beam, int n_sent, int longest_sent, int attention_D, double penalty)
       : m(model), ctx(model.gpu.ctx), beam(beam), n_sent(n_sent), cols(beam * n_sent), longest_sent(longest_sent),
         D(attention_D), penalty(penalty) {
+    // "to make sure beam search does halt": the beam is silently capped at floor(sqrt(target vocabulary))
+    // (src/ensemble_factory.hpp:19-21)
+    {
+      const int cap = std::max(1, (int)std::sqrt((double)m.info.target_vocab_size));
+      if (this->beam > cap) {
+        this->beam = cap;
+        cols = this->beam * n_sent;
+      }
+      beam = this->beam;
+    }
     if (m.info.LM) {
       std::fprintf(stderr, "beam_decoder: a sequence model has no source side to decode from\n");
       std::exit(EXIT_FAILURE);
@@ -1058,8 +1068,16 @@ class beam_decoder {
                               d_ones, 0.0f, cols, h[q].data(), c[q].data(), attention ? attn : nullptr, d_batch_info,
                               attention ? h_tild[q] : nullptr, d_align, d_align_idx, nullptr, nullptr, m.softmax_obj.d_D,
                               m.softmax_obj.d_b_d, Vt, prob_mode ? ZR_SOFTMAX_PROB : ZR_SOFTMAX_LOGITS, logits));
-    // the alignment of every column, read by the beam call that follows (get_viterbi_alignment_kernel)
-    if (track_viterbi) ZOPH_CALL(zr_attn_viterbi(ctx, attn, d_align, d_align_idx, d_viterbi));
+    // The alignment of every column, read by the beam call that follows.  The reference's driver passes every step
+    // through ensembles_models, also with one model, and that overwrites the attention layer's own Viterbi alignment
+    // (get_viterbi_alignment_kernel) with the vote over the window weights (src/ensemble_factory.hpp:797-834): the same
+    // position wherever a weight is positive, -1 instead of the first slot's position where none is.  A member of an
+    // ensemble leaves this to the ensemble's vote.
+    if (track_viterbi && !prob_mode) {
+      const dType* al[1] = {d_align};
+      const int* ix[1] = {d_align_idx};
+      ZOPH_CALL(zr_attn_viterbi_ensemble(ctx, 1, al, ix, 2 * D + 1, cols, longest_sent, d_viterbi));
+    }
   }
 
   // forward_prop_source (src/model.hpp:2367-2452) for up to n_sent sentences whose integerized sources (reversed, no
@@ -1175,15 +1193,23 @@ class beam_decoder {
     ZOPH_CALL(zr_beam_init(ctx, bm));
     const int steps = decode_steps(S);
     int p = 0, index = 0;
-    for (; index < steps; index++) {
+    bool again = false;
+    for (; index < steps && !again; index++) {
       forward_target(p, index);
+      // (a look costs a wait for the stream: after the first step, which has then run the encoder sweep and one decoder
+      // step, and every 32 steps after that -- a launch that gives up takes about a second per step)
+      if (index % 32 == 0 && launches_abandoned()) again = true;
+      if (again) break;
       ZOPH_CALL(zr_beam_expand_logits(ctx, bm, logits, logits + (size_t)Vt * cols, index, d_words, d_back));
       reorder_states(p, d_back);
     }
-    // one last step and forced <EOF> on every live hypothesis (src/ensemble_factory.hpp:727-743)
-    forward_target(p, index);
-    ZOPH_CALL(zr_beam_finish_logits(ctx, bm, logits, logits + (size_t)Vt * cols));
-    if (launches_abandoned()) {  // the batch is decoded again with one launch per node
+    if (!again) {
+      // one last step and forced <EOF> on every live hypothesis (src/ensemble_factory.hpp:727-743)
+      forward_target(p, index);
+      ZOPH_CALL(zr_beam_finish_logits(ctx, bm, logits, logits + (size_t)Vt * cols));
+      again = launches_abandoned();
+    }
+    if (again) {  // the batch is decoded again with one launch per node (launches_abandoned has switched the context over)
       decode_batch(sources, num_best, out);
       return;
     }
@@ -1251,14 +1277,22 @@ class ensemble_beam_decoder {
                                            first.longest_sent, first.d_viterbi));
     };
     int index = 0;
+    bool again = false;
     for (; index < steps; index++) {
       step(index);
+      if (index % 32 == 0 && first.launches_abandoned()) {
+        again = true;
+        break;
+      }
       ZOPH_CALL(zr_beam_expand(ctx, first.bm, mean, index, first.d_words, first.d_back));
       for (int k = 0; k < K; k++) members[k]->reorder_states(0, first.d_back);
     }
-    step(index);
-    ZOPH_CALL(zr_beam_finish(ctx, first.bm, mean));
-    if (first.launches_abandoned()) {
+    if (!again) {
+      step(index);
+      ZOPH_CALL(zr_beam_finish(ctx, first.bm, mean));
+      again = first.launches_abandoned();
+    }
+    if (again) {
       decode_batch(sources, num_best, out);
       return;
     }
