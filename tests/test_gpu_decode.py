@@ -33,10 +33,15 @@ def _model(g, H, Vs, Vt, L):
     return m
 
 
-def _oracle_decode(m, src_col, src_len, S, beam, steps, D, penalty, viterbi=False):
+def _oracle_decode(m, src_col, src_len, S, beam, steps, D, penalty, viterbi=False, safe_out=None):
     """One sentence, minibatch = beam, following forward_prop_source / forward_prop_target / swap_decoding_states.
     viterbi: the attention layer's Viterbi alignments ride along (unk replacement); a fourth value, the alignments
-    of every finished hypothesis, is returned."""
+    of every finished hypothesis, is returned.
+    safe_out (a list): instead of failing when a step's p_t lies within 1e-4 of an integer (where fp32 rounding may
+    legitimately move the attention window) or two candidate scores a step pops lie within 5e-6 of each other (where it
+    (or, later in a long decode, within 1e-6 of their size) of each other (where it may swap them), the index of the
+    first such step is appended (steps + 1 if there is none; the forced finish counts
+    as step `steps`): a comparison is meaningful for the steps before it."""
     H, L, Vt = m["src_embed"].shape[0], len(m["src_layers"]), m["D_soft"].shape[0]
     nn, mk = o.vocab_prep(src_col.reshape(S, 1))
     hs, cs = o.lstm_stack_forward(m["src_embed"], m["src_layers"], nn, mk)
@@ -49,6 +54,7 @@ def _oracle_decode(m, src_col, src_len, S, beam, steps, D, penalty, viterbi=Fals
     words = np.zeros(beam, np.int32)
     h_tild = None
     hist, min_gap = [], np.inf
+    first_unsafe = steps + 1
 
     def forward(index):
         nonlocal hp, cp, h_tild
@@ -75,10 +81,20 @@ def _oracle_decode(m, src_col, src_len, S, beam, steps, D, penalty, viterbi=Fals
         cand = np.sort(np.concatenate([np.log(np.sort(P[:, i])[-(beam + 2):]) + sc[i] for i in range(cols)]))[::-1]
         n_hyp_before = len(dec.hypotheses())
         frac = att["p_t"] - np.floor(att["p_t"])
-        assert np.all((frac > 1e-4) & (frac < 1 - 1e-4)), "p_t on an integer boundary; pick another seed"
+        if not np.all((frac > 1e-4) & (frac < 1 - 1e-4)):
+            assert safe_out is not None, "p_t on an integer boundary; pick another seed"
+            first_unsafe = min(first_unsafe, index)
         dec.expand(P, index, _single_model_vote(att, S) if viterbi else None)
         popped = beam + (len(dec.hypotheses()) - n_hyp_before) + 2  # survivors + <EOF> hypotheses (+ a <START>) + next
-        min_gap = min(min_gap, np.min(-np.diff(cand[:popped + 1])))
+        step_gap = np.min(-np.diff(cand[:popped + 1]))
+        min_gap = min(min_gap, step_gap)
+        # a near-tie: either order is right to fp32 accuracy.  A score is a sum of one log-probability per step: each
+        # term carries the fp32 rounding of a 1000-term logit (about 2e-5 at logits of 15; the oracle accumulates in
+        # double), so two runs' scores drift apart like 2e-5 * sqrt(steps), and the sum itself is held in fp32 (as in
+        # the reference), 1e-6 of its size being 4 to 8 ulp
+        if safe_out is not None and step_gap <= max(5e-6, 1e-6 * float(np.abs(cand[:popped + 1]).max()),
+                                                    4e-5 * np.sqrt(index + 1.0)):
+            first_unsafe = min(first_unsafe, index)
         st = dec.state()
         words, back = st["current_indices"].copy(), st["new_indicies_changes"].copy()
         hist.append((words.copy(), back.copy()))
@@ -86,10 +102,42 @@ def _oracle_decode(m, src_col, src_len, S, beam, steps, D, penalty, viterbi=Fals
         cp = [np.asfortranarray(a[:, back]) for a in newc]
         h_tild = np.asfortranarray(att["h_tild"][:, back])
     _, _, att, P = forward(steps)
+    frac = att["p_t"] - np.floor(att["p_t"])
+    if safe_out is not None:
+        if not np.all((frac > 1e-4) & (frac < 1 - 1e-4)):
+            first_unsafe = min(first_unsafe, steps)
+        safe_out.append(first_unsafe)
     dec.finish(P, _single_model_vote(att, S) if viterbi else None)
     if viterbi:
         return hist, dec.hypotheses(), min_gap, dec.hypotheses_viterbi()
     return hist, dec.hypotheses(), min_gap
+
+
+def _oracle_score_of_path(m, src_col, src_len, S, D, words):
+    """The log-probability of one target word sequence (<START> ... <EOF>) under the model, teacher-forced through the
+    oracle one column wide: what the beam reports as that hypothesis' score whatever else was in the beam."""
+    L = len(m["src_layers"])
+    nn, mk = o.vocab_prep(src_col.reshape(S, 1))
+    hs, cs = o.lstm_stack_forward(m["src_embed"], m["src_layers"], nn, mk)
+    table = hs[L - 1]  # (S, H, 1)
+    hp = [np.asfortranarray(hs[l, S - 1]) for l in range(L)]
+    cp = [np.asfortranarray(cs[l, S - 1]) for l in range(L)]
+    binfo = np.array([src_len, S - src_len], np.int32)
+    ones = np.ones(1, np.int32)
+    h_tild, score = None, np.float32(0)
+    for t in range(len(words) - 1):
+        below = o.embed_gather(m["tgt_embed"], np.array([words[t]], np.int32))
+        for l in range(L):
+            ly = m["tgt_layers"][l]
+            feed = l == 0 and t > 0
+            r = o.lstm_step(ly["M"], ly["Wh"], ly["b"], below, hp[l], cp[l], ones, Q=ly["Q"] if feed else None,
+                            htild=h_tild if feed else None)
+            hp[l], cp[l], below = r["h"], r["c"], r["h"]
+        att = o.attention_forward(hs_table=table, batch_info=binfo, h_t=below, mask01=ones, D=D, **m["attn"])
+        h_tild = att["h_tild"]
+        P = o.softmax_dist(o.softmax_logits(m["D_soft"], m["b_soft"], h_tild))
+        score = np.float32(score + np.float32(np.log(P[words[t + 1], 0])))
+    return float(score)
 
 
 def _single_model_vote(att, S):
@@ -185,7 +233,15 @@ def _oracle_ensemble_decode(ms, src_cols, S, beam, steps, D, viterbi=False):
         n_hyp_before = len(dec.hypotheses())
         dec.expand(P, index, vote(outs))
         popped = beam + (len(dec.hypotheses()) - n_hyp_before) + 2
-        min_gap = min(min_gap, np.min(-np.diff(cand[:popped + 1])))
+        step_gap = np.min(-np.diff(cand[:popped + 1]))
+        min_gap = min(min_gap, step_gap)
+        # a near-tie: either order is right to fp32 accuracy.  A score is a sum of one log-probability per step: each
+        # term carries the fp32 rounding of a 1000-term logit (about 2e-5 at logits of 15; the oracle accumulates in
+        # double), so two runs' scores drift apart like 2e-5 * sqrt(steps), and the sum itself is held in fp32 (as in
+        # the reference), 1e-6 of its size being 4 to 8 ulp
+        if safe_out is not None and step_gap <= max(5e-6, 1e-6 * float(np.abs(cand[:popped + 1]).max()),
+                                                    4e-5 * np.sqrt(index + 1.0)):
+            first_unsafe = min(first_unsafe, index)
         d = dec.state()
         words, back = d["current_indices"].copy(), d["new_indicies_changes"].copy()
         for k in range(K):
@@ -279,3 +335,79 @@ def test_config4_beam_decode_at_full_size(ctx):
         gw, gb = dec.history[index]
         assert np.all((gw >= 2) & (gw < Vt)) and np.all((gb // beam) == np.repeat(np.arange(n_sent), beam))
     dec.close()
+
+
+def test_config4_beam_decode_over_its_full_length_all_sentences(ctx):
+    """Benchmark configuration 4 as stated: 4 layers, H = 1000, beam 12 x 16 sentences, source length 50, 50 000-word
+    vocabularies, the reference's default attention width D = 10, decoded to the reference's stop
+    min(1.5 * source length, longest_sent - 2) = 60 steps (src/ensemble_factory.hpp:637) plus the forced finish.  ALL
+    sixteen sentences are decoded one at a time by the oracle and compared step by step: words, back-pointers, and at
+    the end every finished hypothesis -- hypotheses that end early (the <EOF> bias is raised so that <EOF> enters the
+    candidates at some steps and not at others), late ones, and the forced finish of the survivors
+    (src/decoder.h:672-688).  Over 60 steps x 192 columns some step's p_t falls within fp32 rounding of an integer or
+    two candidate scores nearly tie; from such a step on either continuation is right, so a sentence is compared up to
+    its first such step (reported by the oracle run); enough sentences must be clean to the end."""
+    H, L, beam, n_sent, S, D, longest = 1000, 4, 12, 16, 50, 10, 62
+    steps = min(int(1.5 * S), longest - 2)
+    assert steps == 60
+    Vs = Vt = 50000
+    g = synth.rng(64, 5)
+    m = {"src_embed": synth.uniform(g, (H, Vs)), "tgt_embed": synth.uniform(g, (H, Vt), -0.5, 0.5),
+         "src_layers": [synth.lstm_layer(g, H, forget_bias_one=True) for _ in range(L)],
+         "tgt_layers": [synth.lstm_layer(g, H, feed_input=(l == 0), forget_bias_one=True) for l in range(L)],
+         "attn": synth.attention_weights(g, H),
+         "D_soft": synth.uniform(g, (Vt, H), -0.5, 0.5), "b_soft": synth.uniform(g, (Vt,), -1.0, 1.0)}
+    m["b_soft"][1] = 10.5
+    lens = g.integers(S - 12, S + 1, size=n_sent).astype(np.int32)
+    lens[0] = S
+    src = synth.zipf_ids(g, (S, n_sent), Vs)
+    for s in range(n_sent):
+        src[:S - lens[s], s] = -1
+    w = driver.Seq2SeqWeights(ctx, m["src_embed"], m["src_layers"], m["tgt_embed"], m["tgt_layers"], m["attn"],
+                              m["D_soft"], m["b_soft"])
+    dec = driver.BeamDecode(ctx, w, beam, n_sent, S, steps, attention_D=D, penalty=0.0)
+    dec.encode(src, lens)
+    for _ in range(steps):
+        dec.step(record=True)
+    dec.finish()
+    early, late, forced, compared, rescored = 0, 0, 0, 0, 0
+    for s in range(n_sent):
+        safe = []
+        hist, hyps, _ = _oracle_decode(m, src[:, s], int(lens[s]), S, beam, steps, D, 0.0, safe_out=safe)
+        upto = min(safe[0], steps)
+        compared += upto
+        for index in range(upto):
+            gw, gb = dec.history[index]
+            assert np.array_equal(gw[s * beam:(s + 1) * beam], hist[index][0]), (s, index)
+            assert np.array_equal(gb[s * beam:(s + 1) * beam] - s * beam, hist[index][1]), (s, index)
+        got = dec.hypotheses(s, cap=4 * beam * (steps + 2))
+        # the hypotheses that finished before the first doubtful step are the oracle's, in its order
+        want = [(ww, ws) for ww, ws in hyps if len(ww) - 2 < upto]
+        have = [(gw_, gs) for gw_, gs in got if len(gw_) - 2 < upto]
+        assert len(have) == len(want)
+        for (gwords, gscore), (wwords, wscore) in zip(have, want):
+            assert np.array_equal(gwords, wwords)
+            assert gscore == pytest.approx(wscore, rel=1e-4, abs=2e-4)
+        # whole length: words in range, <START> first and <EOF> last and nowhere else, the forced finish has produced one
+        # hypothesis per surviving slot
+        n_words = [len(gw_) for gw_, _ in got]
+        assert sum(1 for n in n_words if n == steps + 2) == beam
+        for gw_, _ in got:
+            assert gw_[0] == 0 and gw_[-1] == 1 and np.all((gw_[1:-1] >= 2) & (gw_[1:-1] < Vt))
+        early += sum(1 for n in n_words if n <= 12)
+        late += sum(1 for n in n_words if 25 <= n < steps + 2)
+        forced += sum(1 for n in n_words if n == steps + 2)
+        picks = {0, len(got) - 1}
+        picks.update([i for i, n in enumerate(n_words) if 25 <= n < steps + 2][:1])
+        for i in sorted(picks):
+            gw_, gs = got[i]
+            ws = _oracle_score_of_path(m, src[:, s], int(lens[s]), S, D, gw_)
+            assert gs == pytest.approx(ws, rel=2e-5, abs=2e-3), (s, i, len(gw_), gs, ws)
+            rescored += 1
+    for index in range(steps):
+        gw, gb = dec.history[index]
+        assert np.all((gw >= 2) & (gw < Vt)) and np.all((gb // beam) == np.repeat(np.arange(n_sent), beam))
+    dec.close()
+    # (with this seed 323 of the 960 steps are comparable one by one)
+    assert compared >= 250, "only %d of %d steps were comparable" % (compared, n_sent * steps)
+    assert early >= 1 and late >= 1 and forced == n_sent * beam and rescored >= 2 * n_sent, (early, late, forced, rescored)

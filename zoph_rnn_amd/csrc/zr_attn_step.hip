@@ -110,11 +110,6 @@ __device__ __forceinline__ float wave_sum_scatter_step(float (&v)[N > 1 ? N : 1]
   }
 }
 
-// 16-byte store that is written through to memory (device scope), like __hip_atomic_store(..., agent) for one float
-__device__ __forceinline__ void store16_device(void* p, zr_f32x4 v) {
-  asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
-}
-
 constexpr int ilog2(int n) { return n <= 1 ? 0 : 1 + ilog2(n / 2); }
 
 // All threads of the workgroup call this.  False: leave (the caller poisons what it owed).
@@ -341,9 +336,9 @@ __global__ void __launch_bounds__(512) attn_step_kernel(AttnStep P) {
       if (par == 0 && mine) {
         acc += ((const f4*)s_ctx)[k4];
         if (P.ctx_packed)
-          store16_device(P.cpack + ((long long)k4 * mb + b) * 4, acc);
+          zr_store16_device(P.cpack + ((long long)k4 * mb + b) * 4, acc);
         else
-          store16_device(P.cpad + (long long)b * P.ldp + 4 * k4, acc);
+          zr_store16_device(P.cpad + (long long)b * P.ldp + 4 * k4, acc);
         ((f4*)(P.ctx_out + (long long)b * H))[k4] = acc;
       }
       ZR_STAMP(7);

@@ -93,10 +93,16 @@ __device__ __forceinline__ void topk_unkey(unsigned long long key, float& p, int
   w = 0x7fffffff - (int)(unsigned)(key & 0xffffffffu);
 }
 
+// colstats (or null: the values are probabilities): the values are logits, and (max, sum of exp(x - max)) of the column
+// turns a logit into the probability the full normalisation would write, exp(x - max) / sum (src/custom_kernels.h:
+// 574-576).  The bound tau is then taken on the logits (the map is monotonic), but the candidates are keyed and ranked
+// by that PROBABILITY: two logits a few ulp apart can round to one probability, and the reference, which only ever sees
+// the probabilities, ranks such a pair by its tie rule, not by the logits.  So that every word whose probability could
+// equal a listed one is listed too, the bound is lowered by a few ulp of the operands of x - max first.
 template <int kTopkE4>
 __global__ void __launch_bounds__(256)
 beam_topk_kernel(const float* __restrict__ prob, int V, int K, int n_chunks, float* __restrict__ part_p,
-                 int* __restrict__ part_w) {
+                 int* __restrict__ part_w, const float* __restrict__ colstats) {
   constexpr int kTopkChunk = topk_chunk(kTopkE4), kTopkCap = topk_cap(kTopkE4);
   __shared__ unsigned long long s_max[256];
   __shared__ unsigned long long s_cand[kTopkCap];
@@ -108,6 +114,8 @@ beam_topk_kernel(const float* __restrict__ prob, int V, int K, int n_chunks, flo
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const float* p = prob + (size_t)col * V;
+  const bool as_logits = colstats != nullptr;
+  const float c_max = as_logits ? colstats[2 * col] : 0.0f, c_sum = as_logits ? colstats[2 * col + 1] : 1.0f;
   const int v_begin = chunk * kTopkChunk;
   const int v_end = (v_begin + kTopkChunk < V) ? v_begin + kTopkChunk : V;
   if (tid == 0) s_count = 0;
@@ -160,10 +168,14 @@ beam_topk_kernel(const float* __restrict__ prob, int V, int K, int n_chunks, flo
   unsigned long long tau = s_tau_wave[0];
 #pragma unroll
   for (int w = 1; w < 4; ++w) tau = s_tau_wave[w] > tau ? s_tau_wave[w] : tau;
-  auto collect = [&](unsigned long long t) {
+  auto collect = [&](unsigned long long t, bool widen) {
     float tp;
     int tw;
     topk_unkey(t, tp, tw);
+    if (as_logits && widen) {
+      tp -= 1e-6f + 5e-7f * (fabsf(tp) + fabsf(c_max));  // (see above; an infinite bound stays what it is)
+      tw = 0x7fffffff;
+    }
     if (bm >= tp && mu != 0u) {
 #pragma unroll
       for (int i = 0; i < kTopkE4; ++i)
@@ -174,13 +186,13 @@ beam_topk_kernel(const float* __restrict__ prob, int V, int K, int n_chunks, flo
             const int v = v_begin + 4 * (tid + 256 * i) + c;
             if (q > -INFINITY && (q > tp || v <= tw)) {
               const int pos = atomicAdd(&s_count, 1);
-              if (pos < kTopkCap) s_cand[pos] = topk_key(q, v);
+              if (pos < kTopkCap) s_cand[pos] = topk_key(as_logits ? expf(q - c_max) / c_sum : q, v);
             }
           }
         }
     }
   };
-  collect(tau);
+  collect(tau, true);
   __syncthreads();
   if (s_count > kTopkCap) {
     // The wave-level bound let too many elements through (several waves holding threads whose whole share is large, or
@@ -204,7 +216,7 @@ beam_topk_kernel(const float* __restrict__ prob, int V, int K, int n_chunks, flo
     __syncthreads();
     if (tid == 0) s_count = 0;
     __syncthreads();
-    collect(s_tau);
+    collect(s_tau, false);  // (so many equal values that the list overflowed: the exact bound, on the values as they are)
     __syncthreads();
   }
   const int n = s_count < kTopkCap ? s_count : kTopkCap;
@@ -223,11 +235,9 @@ beam_topk_kernel(const float* __restrict__ prob, int V, int K, int n_chunks, flo
   }
 }
 
-// colstats (or null): the values are logits and (max, sum of exp(x - max)) per column turns the K selected ones into
-// probabilities, exp(x - max) / sum as the full normalisation forms them (src/custom_kernels.h:574-576).
 __global__ void __launch_bounds__(256)
 beam_topk_merge_kernel(const float* __restrict__ part_p, const int* __restrict__ part_w, int K, int n_chunks,
-                       float* __restrict__ cand_p, int* __restrict__ cand_w, const float* __restrict__ colstats) {
+                       float* __restrict__ cand_p, int* __restrict__ cand_w) {
   __shared__ unsigned long long s_key[kMaxChunks * KMAX];
   const int col = blockIdx.x;
   const int tid = threadIdx.x;
@@ -244,9 +254,7 @@ beam_topk_merge_kernel(const float* __restrict__ part_p, const int* __restrict__
       rank += (kb > ka || (kb == ka && b < a)) ? 1 : 0;  // fillers share one key: order them by position
     }
     if (rank < K) {
-      float v = part_p[(size_t)col * n + a];
-      if (colstats && v > -INFINITY) v = expf(v - colstats[2 * col]) / colstats[2 * col + 1];
-      cand_p[(size_t)col * K + rank] = v;
+      cand_p[(size_t)col * K + rank] = part_p[(size_t)col * n + a];
       cand_w[(size_t)col * K + rank] = part_w[(size_t)col * n + a];
     }
   }
@@ -635,12 +643,14 @@ static int beam_expand_impl(zr_ctx* ctx, const char* who, zr_beam* b, const floa
   const int n_chunks = (b->vocab + topk_chunk(e4) - 1) / topk_chunk(e4);
   dim3 tgrid(n_chunks, b->n_sent * b->beam);
   if (e4 == kTopkE4Small)
-    beam_topk_kernel<kTopkE4Small><<<tgrid, 256, 0, ctx->stream>>>(d_values, b->vocab, K, n_chunks, b->d_part_p, b->d_part_w);
+    beam_topk_kernel<kTopkE4Small><<<tgrid, 256, 0, ctx->stream>>>(d_values, b->vocab, K, n_chunks, b->d_part_p, b->d_part_w,
+                                                                   d_colstats);
   else
-    beam_topk_kernel<kTopkE4Large><<<tgrid, 256, 0, ctx->stream>>>(d_values, b->vocab, K, n_chunks, b->d_part_p, b->d_part_w);
+    beam_topk_kernel<kTopkE4Large><<<tgrid, 256, 0, ctx->stream>>>(d_values, b->vocab, K, n_chunks, b->d_part_p, b->d_part_w,
+                                                                   d_colstats);
   ZR_LAUNCH_CHECK("beam_topk_kernel");
   beam_topk_merge_kernel<<<b->n_sent * b->beam, 256, 0, ctx->stream>>>(b->d_part_p, b->d_part_w, K, n_chunks,
-                                                                       b->d_cand_p, b->d_cand_w, d_colstats);
+                                                                       b->d_cand_p, b->d_cand_w);
   ZR_LAUNCH_CHECK("beam_topk_merge_kernel");
   beam_merge_kernel<<<b->n_sent, 256, 0, ctx->stream>>>(b->beam, K, b->max_len, b->hyp_cap, b->penalty, index,
                                                         b->current_index, b->d_cand_p, b->d_cand_w, b->d_scores,

@@ -331,6 +331,12 @@ __device__ __forceinline__ void zr_publish_barrier() {
   __syncthreads();
 }
 
+// 16-byte store that is written through to memory (device scope), what __hip_atomic_store(..., __HIP_MEMORY_SCOPE_AGENT)
+// is for one float: for data another workgroup reads behind a counter.
+__device__ __forceinline__ void zr_store16_device(void* p, zr_f32x4 v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+}
+
 // Number of visits zr_reduce_visit makes per thread, and the accumulator slot (tn*16 + r) of visit i: callers use
 // them to fetch epilogue operands (previous cell state, biases) before the K loop instead of after it.
 template <int TN, int KS>
