@@ -404,3 +404,40 @@ def test_ensemble_alignment_vote_known_answer_and_brute_force(ctx):
         ctx.attn_viterbi_ensemble(d[0], d[1], 3, 3, 9000, d_out)
     for x in d[0] + d[1] + [d_out]:
         x.free()
+
+
+def test_beam_on_logits_ranks_words_of_equal_probability_as_the_probability_matrix_would(ctx):
+    """Three words whose logits differ by one and two ulp but whose probabilities, exp(x - max) / sum, round to the same
+    float.  The reference only ever sees probabilities and ranks such words by its rule for equal values (here: lower
+    word id first); selection on the logits must do the same -- ranking them by logit would put the highest id first.
+    Checked against the expansion of a probability matrix that holds the three equal values."""
+    V, beam, n_sent = 5000, 3, 1
+    cols = beam * n_sent
+    g = synth.rng(48, 1)
+    lg = np.asfortranarray(g.uniform(-3, -2, size=(V, cols)).astype(np.float32))
+    top = np.float32(0.2)
+    below1 = np.nextafter(top, np.float32(-1))
+    below2 = np.nextafter(below1, np.float32(-1))
+    assert top > below1 > below2
+    lg[4000, 0], lg[10, 0], lg[700, 0] = top, below1, below2
+    mx = lg.max(axis=0)
+    sums = np.exp(lg.astype(np.float64) - mx.astype(np.float64)).sum(axis=0).astype(np.float32)
+    prob = np.asfortranarray((np.exp((lg - mx).astype(np.float32)) / sums).astype(np.float32))
+    assert prob[4000, 0] == prob[10, 0] == prob[700, 0]  # (exp of minus one or two ulp of 0.2 is 1 in fp32)
+    flat = np.concatenate([lg.reshape(-1, order="F"), np.stack([mx, sums], axis=1).reshape(-1)]).astype(np.float32)
+    d_lg = ctx.array(flat)
+    d_stats = d_lg.at(V * cols)
+    d_prob = ctx.array(prob)
+    ba, bb = ctx.beam_create(beam, V, n_sent, 8, 0.0), ctx.beam_create(beam, V, n_sent, 8, 0.0)
+    wa, ka = ctx.empty(cols, np.int32), ctx.empty(cols, np.int32)
+    wb, kb = ctx.empty(cols, np.int32), ctx.empty(cols, np.int32)
+    ctx.beam_expand(ba, d_prob, 0, wa, ka)
+    ctx.beam_expand_logits(bb, d_lg, d_stats, 0, wb, kb)
+    ctx.sync()
+    assert wa.get().tolist() == [10, 700, 4000]
+    assert wb.get().tolist() == [10, 700, 4000]
+    sa, _ = ctx.beam_state(ba, 0, beam)
+    sb, _ = ctx.beam_state(bb, 0, beam)
+    assert sa[0] == sa[1] == sa[2] and np.array_equal(sa, sb)
+    ctx.beam_destroy(ba)
+    ctx.beam_destroy(bb)
