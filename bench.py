@@ -103,6 +103,28 @@ def measure_steady_state_step(ctx, steps, warmup, H=1000, mb=128, T=50, V=50000,
     return us, L * 2.0 * 4 * H * mb * (2 * H)
 
 
+PEAK_BF16_MFMA_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak
+
+
+def roofline_entry(kernel, bound, us, flops=None, nbytes=None, peak_tflops=PEAK_FP32_MFMA_TFLOPS, note=None):
+    """One kernel (or stage) of a step against the roofline that bounds it: algorithmic flops and / or bytes, measured
+    time, achieved rate and fraction of the MI355X peak."""
+    e = {"kernel": kernel, "bound": bound, "us": round(us, 2)}
+    if flops is not None:
+        e["gflop"] = round(flops / 1e9, 3)
+        e["tflops"] = round(flops / (us * 1e-6) / 1e12, 2)
+    if nbytes is not None:
+        e["mbytes"] = round(nbytes / 1e6, 2)
+        e["gbytes_per_s"] = round(nbytes / (us * 1e-6) / 1e9, 1)
+    if bound == "mfma":
+        e["peak"], e["unit"], e["frac"] = peak_tflops, "TFLOP/s", round(e["tflops"] / peak_tflops, 4)
+    else:
+        e["peak"], e["unit"], e["frac"] = PEAK_HBM_GBS, "GB/s", round(e["gbytes_per_s"] / PEAK_HBM_GBS, 4)
+    if note:
+        e["note"] = note
+    return e
+
+
 def bench_decoder_step(ctx, steps, warmup, H=1000, mb=128, S=50, V=50000, L=4, D=50, bf16=False):
     """Config 3: gather, 4 LSTM layers (feed-input on layer 0), attention (D >= S: every source position has a
     slot), full softmax to probabilities."""
@@ -129,6 +151,11 @@ def bench_decoder_step(ctx, steps, warmup, H=1000, mb=128, S=50, V=50000, L=4, D
     d_c = [ctx.empty((H, mb)) for _ in range(L)]
     d_ht = ctx.empty((H, mb))
     d_prob = ctx.empty((V, mb))
+    d_logit = ctx.empty((V * mb + 2 * mb,))
+
+    def logits_part():
+        # the logits product and the column statistics alone (what the normalisation pass comes on top of)
+        ctx.softmax_forward(dD, dbd, V, H, d_ht, mb, capi.ZR_SOFTMAX_LOGITS, d_logit)
 
     def lstm_part():
         # all layers of the step in one call; layer 0 looks its input columns up in the embedding itself
@@ -147,16 +174,38 @@ def bench_decoder_step(ctx, steps, warmup, H=1000, mb=128, S=50, V=50000, L=4, D
 
     wall_ms, ev_ms = time_region(ctx, step, steps, warmup)
     parts = {}
-    for name, fn in (("lstm_stack", lstm_part), ("attention", attn_part), ("softmax", softmax_part)):
+    for name, fn in (("lstm_stack", lstm_part), ("attention", attn_part), ("softmax", softmax_part),
+                     ("logits_and_colstats", logits_part)):
         _, ms = time_region(ctx, fn, steps, 1)
         parts[name + "_us"] = round(ms * 1e3 / steps, 2)
-    flops = 2.0 * 4 * H * mb * (3 * H) + (L - 1) * 2.0 * 4 * H * mb * (2 * H) + 4 * 2.0 * H * H * mb + 2.0 * V * H * mb
+    f_lstm = 2.0 * 4 * H * mb * (3 * H) + (L - 1) * 2.0 * 4 * H * mb * (2 * H)
+    f_attn, f_logits = 4 * 2.0 * H * H * mb, 2.0 * V * H * mb
+    flops = f_lstm + f_attn + f_logits
     res = {"ms_per_step": ev_ms / steps, "wall_ms_per_step": wall_ms / steps, "tokens_per_s": mb * steps / (ev_ms * 1e-3),
            "gflop_per_step": flops / 1e9, "tflops": flops * steps / (ev_ms * 1e-3) / 1e12, "attention_D": D}
     res.update(parts)
     if not bf16:
         res["frac_of_fp32_matrix_peak"] = round(res["tflops"] / PEAK_FP32_MFMA_TFLOPS, 4)
     res["softmax_gemm_plus_normalise_tflops"] = round(2.0 * V * H * mb / (parts["softmax_us"] * 1e-6) / 1e12, 2)
+    # Every stage of the step against the roofline that bounds it.  Stages are timed on their own, back to back with
+    # themselves (a stage repeated alone keeps its matrices in the memory-side cache: the step's own time is the figure
+    # above); bytes and flops are algorithmic.
+    wb = 2 if bf16 else 4
+    peak = PEAK_BF16_MFMA_TFLOPS if bf16 else PEAK_FP32_MFMA_TFLOPS
+    slots = min(2 * D + 1, S)
+    norm_us = max(parts["softmax_us"] - parts["logits_and_colstats_us"], 0.01)
+    res["roofline"] = [
+        roofline_entry("LSTM stack, %d layers (lstm_decoder_stack_kernel or one lstm_fused_kernel per layer)" % L, "mfma",
+                       parts["lstm_stack_us"], flops=f_lstm, nbytes=(12 + 8 * (L - 1)) * H * H * wb, peak_tflops=peak),
+        roofline_entry("attention step (attn_step_kernel, or projections + fused middle + output product)", "mfma",
+                       parts["attention_us"], flops=f_attn, nbytes=4 * H * H * wb + slots * H * mb * 4, peak_tflops=peak,
+                       note="a chain of dependent stages: %.0f MB of source states and matrices, %.2f GFLOP"
+                            % ((4 * H * H * wb + slots * H * mb * 4) / 1e6, f_attn / 1e9)),
+        roofline_entry("output-layer logits + column statistics (gemm_tall_kernel / gemm_bf16_lds_kernel, "
+                       "softmax_colstats_kernel)", "hbm" if bf16 else "mfma", parts["logits_and_colstats_us"],
+                       flops=f_logits, nbytes=V * H * wb + V * mb * 4, peak_tflops=peak),
+        roofline_entry("softmax_normalize_kernel", "hbm", norm_us, nbytes=2.0 * V * mb * 4),
+    ]
     ctx.attn_destroy(attn)
     ctx.softmax_release(dD)
     return res
@@ -302,6 +351,15 @@ def bench_beam_decode(ctx, steps, H=1000, L=4, beam=12, n_sent=16, S=50, V=50000
     res = {"columns": beam * n_sent, "ms_per_decode_step": round(ms / steps, 4),
            "hypotheses_per_s": round(beam * n_sent * steps / (ms * 1e-3), 1), "encode_ms": round(enc_ms, 3),
            "attention_D": D}
+    # the beam's three launches on their own (selection over the V x columns logits, merges, bookkeeping)
+    bm = ctx.beam_create(beam, V, n_sent, steps + 40, 0.0)
+    d_w, d_b = ctx.empty(beam * n_sent, np.int32), ctx.empty(beam * n_sent, np.int32)
+    ctx.beam_expand_logits(bm, dec.logits, dec.colstats, 0, d_w, d_b)
+    _, bms = time_region(ctx, lambda: ctx.beam_expand_logits(bm, dec.logits, dec.colstats, 1, d_w, d_b), 20, 2)
+    ctx.beam_destroy(bm)
+    res["beam_us"] = round(bms * 1e3 / 20, 2)
+    res["beam_roofline"] = roofline_entry("beam_topk_kernel + beam_topk_merge_kernel + beam_merge_kernel", "hbm",
+                                          bms * 1e3 / 20, nbytes=float(V) * beam * n_sent * 4)
     dec.close()
     return res
 
@@ -479,9 +537,14 @@ def main():
         log("training step:", extra["lm_training_step"])
         extra["hbm_kernels"] = bench_hbm_kernels(ctx, args.steps)
         extra["config4_beam_decode"] = bench_beam_decode(ctx, max(args.steps * 5, 100))
+        # its forward stages at 192 columns and the reference's window (D = 10), each against its roofline
+        c4 = bench_decoder_step(ctx, short_steps // 2, short_warm, mb=192, D=10)
+        extra["config4_beam_decode"]["roofline"] = c4["roofline"] + [extra["config4_beam_decode"].pop("beam_roofline")]
+        extra["config4_beam_decode"]["forward_stages_ms_per_step"] = round(c4["ms_per_step"], 4)
         log("config4:", extra["config4_beam_decode"])
         # the reference decodes one sentence per pass: the same step with 12 columns
         extra["config4_single_sentence_beam12"] = bench_beam_decode(ctx, max(args.steps * 5, 100), n_sent=1)
+        extra["config4_single_sentence_beam12"].pop("beam_roofline", None)
         log("config4, one sentence:", extra["config4_single_sentence_beam12"])
         log("hbm kernels:", extra["hbm_kernels"])
     cpu = None

@@ -174,7 +174,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& a, int m0, int n0, boo
 #pragma unroll
       for (int tm = 0; tm < TM; ++tm) wsoff[tm] = 512u * (unsigned)tm;  // 32 rows of 16 bytes
 #pragma unroll
-      for (int tn = 0; tn < TN; ++tn) xoffb[tn] = 16u * (unsigned)(n0 + tn * 32 + jl + half * a.N);
+      for (int tn = 0; tn < TN; ++tn) xoffb[tn] = 16u * (unsigned)(cols[tn] + half * a.N);
       const unsigned woffb = 16u * (unsigned)(m0 + jl + half * (int)a.lda[s]);
       zr_mma_segment_ring<TM, TN, KS, PF, WAUX>(acc, zr_make_rsrc(a.A[s]), wsoff, woffb, 32u * (unsigned)a.lda[s],
                                        zr_make_rsrc(a.B[s]), xoffb, 32u * (unsigned)a.N, a.K[s], kslice);
@@ -397,6 +397,23 @@ __global__ void __launch_bounds__(256) gemm_rows_kernel(GemmArgs a, int row_chun
       gemm_tile<1, 1, 4, AMODE, true, EPI, PF4 + 2>(a, blk * 32, n0 + sub * 32, true, 0, red, kslice, lane);
     __syncthreads();
   }
+}
+
+// Tall weight matrix (k-interleaved) times at most 32 columns: the output layer at the width the reference decodes at
+// (one sentence, minibatch = beam).  The product is a stream of the matrix through the chip -- 200 MB for 1.2 GFLOP at
+// 50 000 x 1000 x 12 -- so the only thing that matters is bytes in flight, and everything that stands between two
+// fetches costs: K split over the waves of a workgroup means a cross-wave sum through LDS and a ramp per pass (the
+// row-range kernel: 50 us, 3.9 TB/s).  Here every WAVE takes whole 32-row blocks over all of K on its own, a ring of 12
+// fetch stages deep, three workgroups per compute unit (3072 waves for 1563 blocks): no LDS, no barrier, and the soft-max
+// partials of a block are the wave's own 32 rows.  K % 8 == 0, k-interleaved activations.
+template <int EPI, int WAUX>
+__global__ void __launch_bounds__(256, 3) gemm_stream_kernel(GemmArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * 4 + (threadIdx.x >> 6)));
+  const int n_waves = (int)gridDim.x * 4;
+  const int blocks = (a.M + 31) >> 5;
+  for (int b = wave; b < blocks; b += n_waves)
+    gemm_tile<1, 1, 1, ZR_A_PACK4, true, EPI, 12, true, WAUX>(a, b * 32, 0, true, 0, nullptr, 0, lane);
 }
 
 // Tall weight matrix (k-interleaved) times a minibatch that is a multiple of 128 columns wide, balanced over the
@@ -1349,6 +1366,23 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
       if ((d.N % 64 == 0 || d.N % 96 == 0) && ga.b_pack4 && ctx->gemm_cfg == 0) {
         int rc = ZR_OK;
         if (launch_tall(ctx, ga, d.epilogue, &rc)) return rc;
+      }
+      if (d.N <= 32 && ga.b_pack4 && d.K[0] % 8 == 0 && ctx->gemm_cfg == 0 &&
+          (long long)d.K[0] * ga.lda[0] * 4 + 4096 < (1LL << 32)) {
+        // one 32-row block per wave while there are waves (three workgroups per compute unit), more beyond that
+        const int blocks = (d.M + 31) / 32;
+        const int cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
+        int wgs = (blocks + 3) / 4;
+        if (wgs > 3 * cus) wgs = 3 * cus;
+        ga.m_tiles = ga.n_tiles = 0;
+        if (d.epilogue == ZR_EPI_STORE)
+          gemm_stream_kernel<ZR_EPI_STORE, 0><<<wgs, 256, 0, ctx->stream>>>(ga);
+        else if (ga.stream_a)
+          gemm_stream_kernel<ZR_EPI_SOFTMAX_PARTIAL, ZR_AUX_STREAM><<<wgs, 256, 0, ctx->stream>>>(ga);
+        else
+          gemm_stream_kernel<ZR_EPI_SOFTMAX_PARTIAL, 0><<<wgs, 256, 0, ctx->stream>>>(ga);
+        ZR_LAUNCH_CHECK("gemm_stream_kernel");
+        return ZR_OK;
       }
       const int n_tiles = (n32 + 3) / 4;
       const int tn = (n32 + n_tiles - 1) / n_tiles;
