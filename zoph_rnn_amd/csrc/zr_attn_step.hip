@@ -489,7 +489,14 @@ int zr_attn_step_single_launch(zr_ctx* ctx, zr_attn* a, const int* d_batch_info,
   const int cap = cached > 0 ? cached : 0;
   const int j_tiles = (H + 31) / 32, n_tiles = (mb + 31) / 32;
   const int n_o = j_tiles * n_tiles, n_o_pad = (n_o + 7) / 8 * 8;
-  const long long wgs = (long long)n_o_pad + mb;
+  // one workgroup per output tile and one per column; with few columns, further workgroups that only take projection
+  // tiles, so that the 2 * n_o of those are one round (12 columns of H = 1000: 64 tiles on 44 workgroups otherwise)
+  long long wgs = (long long)n_o_pad + mb;
+  {
+    const long long p_tiles = (2LL * n_o + 7) / 8 * 8;
+    const long long want = p_tiles < cap ? p_tiles : cap;
+    if (wgs < want) wgs = want;
+  }
   const bool alone = zr_live_contexts(ctx->device) == 1 && ctx->stream == ctx->own_stream;
   const long long lim = 1LL << 32;
   const bool offsets_fit = 4LL * a->kp32 * a->ldp32 * 4 < lim && (long long)a->ldp32 * mb * 4 < lim;

@@ -401,19 +401,26 @@ __global__ void __launch_bounds__(256) gemm_rows_kernel(GemmArgs a, int row_chun
 
 // Tall weight matrix (k-interleaved) times at most 32 columns: the output layer at the width the reference decodes at
 // (one sentence, minibatch = beam).  The product is a stream of the matrix through the chip -- 200 MB for 1.2 GFLOP at
-// 50 000 x 1000 x 12 -- so the only thing that matters is bytes in flight, and everything that stands between two
-// fetches costs: K split over the waves of a workgroup means a cross-wave sum through LDS and a ramp per pass (the
-// row-range kernel: 50 us, 3.9 TB/s).  Here every WAVE takes whole 32-row blocks over all of K on its own, a ring of 12
-// fetch stages deep, three workgroups per compute unit (3072 waves for 1563 blocks): no LDS, no barrier, and the soft-max
-// partials of a block are the wave's own 32 rows.  K % 8 == 0, k-interleaved activations.
+// 50 000 x 1000 x 12 -- so what matters is bytes in flight and how memory sees the fetches.  K split over the waves of a
+// workgroup means a cross-wave sum through LDS and a ramp per pass (the row-range kernel: 50 us, 3.9 TB/s).  Here every
+// WAVE takes two neighbouring 32-row blocks over all of K on its own, a ring of 10 fetch stages deep, two workgroups per
+// compute unit: no LDS, no barrier, and the soft-max partials of a block are the wave's own rows.  Measured at
+// 50 000 x 12 x 1000 (kernel time): one block per wave, ring of 12: 49.6 us; two blocks, ring of 10: 40.2 us (5.0 TB/s;
+// a wave's two weight fetches of a stage are 1 KB of contiguous memory instead of 512 bytes); two blocks, ring of 14:
+// 51.9; three blocks, ring of 8: 57.4; four blocks, ring of 6: 73.3 (too few bytes in flight).
+// K % 8 == 0, k-interleaved activations.
 template <int EPI, int WAUX>
-__global__ void __launch_bounds__(256, 3) gemm_stream_kernel(GemmArgs a) {
+__global__ void __launch_bounds__(256, 2) gemm_stream_kernel(GemmArgs a) {
+  constexpr int PF = 10;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * 4 + (threadIdx.x >> 6)));
   const int n_waves = (int)gridDim.x * 4;
-  const int blocks = (a.M + 31) >> 5;
-  for (int b = wave; b < blocks; b += n_waves)
-    gemm_tile<1, 1, 1, ZR_A_PACK4, true, EPI, 12, true, WAUX>(a, b * 32, 0, true, 0, nullptr, 0, lane);
+  const int blocks = (a.M + 31) >> 5;  // (the packed matrix holds exactly these rows: nothing beyond them is fetched)
+  const int pairs = blocks >> 1;
+  for (int b = wave; b < pairs; b += n_waves)
+    gemm_tile<2, 1, 1, ZR_A_PACK4, true, EPI, PF, true, WAUX>(a, b * 64, 0, true, 0, nullptr, 0, lane);
+  if ((blocks & 1) && wave == pairs % n_waves)  // an odd block at the end, on its own
+    gemm_tile<1, 1, 1, ZR_A_PACK4, true, EPI, PF, true, WAUX>(a, (blocks - 1) * 32, 0, true, 0, nullptr, 0, lane);
 }
 
 // Tall weight matrix (k-interleaved) times a minibatch that is a multiple of 128 columns wide, balanced over the
@@ -1370,10 +1377,12 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
       if (d.N <= 32 && ga.b_pack4 && d.K[0] % 8 == 0 && ctx->gemm_cfg == 0 &&
           (long long)d.K[0] * ga.lda[0] * 4 + 4096 < (1LL << 32)) {
         // one 32-row block per wave while there are waves (three workgroups per compute unit), more beyond that
-        const int blocks = (d.M + 31) / 32;
+        // two neighbouring 32-row blocks per wave (their fetches are 1 KB of contiguous memory), two workgroups per
+        // compute unit, one pair per wave while there are waves
+        const int pairs = ((d.M + 31) / 32 + 1) / 2;
         const int cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
-        int wgs = (blocks + 3) / 4;
-        if (wgs > 3 * cus) wgs = 3 * cus;
+        int wgs = (pairs + 3) / 4;
+        if (wgs > 2 * cus) wgs = 2 * cus;
         ga.m_tiles = ga.n_tiles = 0;
         if (d.epilogue == ZR_EPI_STORE)
           gemm_stream_kernel<ZR_EPI_STORE, 0><<<wgs, 256, 0, ctx->stream>>>(ga);
