@@ -398,6 +398,12 @@ int zr_ensemble_average(zr_ctx* ctx, int n_models, const float* const d_probs[],
  * zr_beam_hypotheses_viterbi copies the alignments of the finished hypotheses of sentence s, n x max_len like
  * zr_beam_hypotheses' h_words and in the same order; returns their number. */
 int zr_beam_set_viterbi(zr_ctx* ctx, zr_beam* b, int enable, const int* d_viterbi);
+/* The words a step selects are the next step's input ids, after the -1 of a dead slot has become 0 (vocab_to_nonM1,
+ * src/custom_kernels.h:23-34, which the reference runs on the decoder's current_indices in
+ * Input_To_Hidden_Layer::prep_GPU_vocab_indices).  With d_words_nonneg set (n_sent*beam ints in device memory; NULL
+ * switches it off) every later zr_beam_expand* call writes them there as well, in the launch that writes d_words, so
+ * the caller needs no zr_vocab_prep launch between the steps. */
+int zr_beam_set_input_ids(zr_ctx* ctx, zr_beam* b, int* d_words_nonneg);
 int zr_beam_hypotheses_viterbi(zr_ctx* ctx, zr_beam* b, int sentence, int cap, int* h_viterbi);
 /* Current beam state of sentence s (top_sentences_scores, current_indices). */
 int zr_beam_state(zr_ctx* ctx, zr_beam* b, int sentence, float* h_scores, int* h_words);

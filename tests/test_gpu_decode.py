@@ -233,15 +233,7 @@ def _oracle_ensemble_decode(ms, src_cols, S, beam, steps, D, viterbi=False):
         n_hyp_before = len(dec.hypotheses())
         dec.expand(P, index, vote(outs))
         popped = beam + (len(dec.hypotheses()) - n_hyp_before) + 2
-        step_gap = np.min(-np.diff(cand[:popped + 1]))
-        min_gap = min(min_gap, step_gap)
-        # a near-tie: either order is right to fp32 accuracy.  A score is a sum of one log-probability per step: each
-        # term carries the fp32 rounding of a 1000-term logit (about 2e-5 at logits of 15; the oracle accumulates in
-        # double), so two runs' scores drift apart like 2e-5 * sqrt(steps), and the sum itself is held in fp32 (as in
-        # the reference), 1e-6 of its size being 4 to 8 ulp
-        if safe_out is not None and step_gap <= max(5e-6, 1e-6 * float(np.abs(cand[:popped + 1]).max()),
-                                                    4e-5 * np.sqrt(index + 1.0)):
-            first_unsafe = min(first_unsafe, index)
+        min_gap = min(min_gap, np.min(-np.diff(cand[:popped + 1])))
         d = dec.state()
         words, back = d["current_indices"].copy(), d["new_indicies_changes"].copy()
         for k in range(K):

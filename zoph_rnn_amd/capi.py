@@ -469,6 +469,9 @@ class Context:
                                              _ptr_array(d_indices), C.c_int(slots), C.c_int(cols),
                                              C.c_int(longest_sent), _vp(d_viterbi)))
 
+    def beam_set_input_ids(self, b, d_words_nonneg):
+        _chk(load().zr_beam_set_input_ids(self.h, b, _vp(d_words_nonneg)))
+
     def beam_set_viterbi(self, b, enable, d_viterbi=None):
         _chk(load().zr_beam_set_viterbi(self.h, b, C.c_int(1 if enable else 0), _vp(d_viterbi)))
 

@@ -38,6 +38,7 @@ struct zr_beam {
   int* d_hyp_vit;           // [n_sent][hyp_cap][max_len]
   int track_viterbi;        // 0: the three arrays above are not touched
   const int* d_viterbi_in;  // alignment of every column for the next expand / finish call (null: -1)
+  int* d_words_nn_out;      // zr_beam_set_input_ids: every expand call also writes max(word, 0) per slot here (null: no)
   // per step scratch
   float* d_cand_p;          // [n_sent*beam][beam+1]
   int* d_cand_w;            // [n_sent*beam][beam+1]
@@ -266,7 +267,8 @@ __global__ void __launch_bounds__(256)
 beam_merge_kernel(int beam, int K, int max_len, int hyp_cap, float penalty, int index, int current_index,
                   const float* __restrict__ cand_p, const int* __restrict__ cand_w, float* scores,
                   int* words, int* sent, int* sent_tmp, int* hyp_words, int* hyp_len, float* hyp_score,
-                  int* hyp_count, int* out_words, int* out_backptr, const int* __restrict__ vit, int* vit_tmp,
+                  int* hyp_count, int* out_words, int* out_words_nn, int* out_backptr, const int* __restrict__ vit,
+                  int* vit_tmp,
                   int* hyp_vit, const int* __restrict__ viterbi_in) {
   constexpr int MAXC = KMAX * KMAX;
   __shared__ float c_val[MAXC];
@@ -398,6 +400,7 @@ beam_merge_kernel(int beam, int K, int max_len, int hyp_cap, float penalty, int 
   if (tid < beam) {
     const int parent = s_parent[tid];
     out_words[(size_t)s * beam + tid] = s_word[tid];
+    if (out_words_nn) out_words_nn[(size_t)s * beam + tid] = s_word[tid] < 0 ? 0 : s_word[tid];
     out_backptr[(size_t)s * beam + tid] = s * beam + (parent < 0 ? 0 : parent);
     sc[tid] = s_score[tid];  // s_score was filled from the old scores before the last barrier
     wd[tid] = s_word[tid];
@@ -656,7 +659,8 @@ static int beam_expand_impl(zr_ctx* ctx, const char* who, zr_beam* b, const floa
                                                         b->current_index, b->d_cand_p, b->d_cand_w, b->d_scores,
                                                         b->d_words, b->d_sent, b->d_sent_tmp,
                                                         b->d_hyp_words, b->d_hyp_len, b->d_hyp_score, b->d_hyp_count,
-                                                        d_words, d_backptr, b->track_viterbi ? b->d_vit : nullptr,
+                                                        d_words, b->d_words_nn_out, d_backptr,
+                                                        b->track_viterbi ? b->d_vit : nullptr,
                                                         b->d_vit_tmp, b->d_hyp_vit, b->d_viterbi_in);
   ZR_LAUNCH_CHECK("beam_merge_kernel");
   int* t = b->d_sent;  // the kernel wrote the new rows into d_sent_tmp
@@ -755,6 +759,13 @@ int zr_ensemble_average(zr_ctx* ctx, int n_models, const float* const d_probs[],
     ensemble_normalize_kernel<false><<<grid, 256, 0, ctx->stream>>>(V, d_out, (const double*)ws);
   }
   ZR_LAUNCH_CHECK("ensemble_normalize_kernel");
+  return ZR_OK;
+}
+
+int zr_beam_set_input_ids(zr_ctx* ctx, zr_beam* b, int* d_words_nonneg) {
+  (void)ctx;
+  ZR_CHECK_ARG(b != nullptr, "zr_beam_set_input_ids: beam object is null");
+  b->d_words_nn_out = d_words_nonneg;
   return ZR_OK;
 }
 

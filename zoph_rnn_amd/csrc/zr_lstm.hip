@@ -1436,7 +1436,7 @@ static int lstm_step_impl(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_
                           const float* d_hprev, const float* d_cprev, const float* d_htild, const int* d_mask01,
                           float clip_threshold, int mb, float* d_h, float* d_c, float* const d_gates[4],
                           const unsigned short* const* pre_hi = nullptr, const unsigned short* const* pre_lo = nullptr,
-                          unsigned short* out_hi = nullptr, unsigned short* out_lo = nullptr);
+                          unsigned short* out_hi = nullptr, unsigned short* out_lo = nullptr, float* out_hp = nullptr);
 
 int zr_lstm_step(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_in, const float* d_hprev,
                  const float* d_cprev, const float* d_htild, const int* d_mask01, float clip_threshold, int mb,
@@ -1456,12 +1456,13 @@ int zr_lstm_step_embed(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_emb
 // d_gather_ids non-null: d_in is the H x V embedding and column b of the input is d_in[:, d_gather_ids[b]].
 // pre_hi / pre_lo (or null; bf16 weights only): segment s's input already split into bf16 terms and k-interleaved by 8
 // (pre_lo[s] null in single-term mode); such a segment is neither gathered nor split here.  out_hi / out_lo (or null):
-// h is also written in that form, for the product that reads it next.
+// h is also written in that form, for the product that reads it next.  out_hp (or null; fp32 weights, fused epilogue):
+// h is also written k-interleaved ([H/4][mb][4]).
 static int lstm_step_impl(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_in, const int* d_gather_ids, int V,
                           const float* d_hprev, const float* d_cprev, const float* d_htild, const int* d_mask01,
                           float clip_threshold, int mb, float* d_h, float* d_c, float* const d_gates[4],
                           const unsigned short* const* pre_hi, const unsigned short* const* pre_lo,
-                          unsigned short* out_hi, unsigned short* out_lo) {
+                          unsigned short* out_hi, unsigned short* out_lo, float* out_hp) {
   int rc = zr_bind_device(ctx);
   if (rc) return rc;
   ZR_CHECK_ARG(w != nullptr, "zr_lstm_step: weights are null");
@@ -1508,6 +1509,7 @@ static int lstm_step_impl(zr_ctx* ctx, const zr_lstm_weights* w, const float* d_
   U.mask01 = d_mask01;
   U.h = d_h;
   U.c = d_c;
+  U.hp = (ctx->lstm_fused && !w->bf16) ? out_hp : nullptr;
   U.hsplit_hi = (ctx->lstm_fused && H % 8 == 0) ? out_hi : nullptr;
   U.hsplit_lo = U.hsplit_hi ? out_lo : nullptr;
   for (int g = 0; g < 4; ++g) U.gates[g] = d_gates ? d_gates[g] : nullptr;
@@ -1702,15 +1704,19 @@ int zr_lstm_decoder_step_packed(zr_ctx* ctx, int nl, const zr_lstm_weights* cons
     if (wrote_hp_top && top_hi) *wrote_hp_top = 1;
     return ZR_OK;
   }
+  // (the top layer also leaves its h k-interleaved for the caller's next product, as the single launch does)
+  float* top_hp = (!layers[0]->bf16 && ctx->lstm_fused && H % 8 == 0) ? d_hp_top : nullptr;
   for (int l = 0; l < nl; ++l) {
+    float* hp_out = l == nl - 1 ? top_hp : nullptr;
     if (l == 0)
       rc = lstm_step_impl(ctx, layers[0], d_embed, d_ids_nonneg, V, d_hprev[0], d_cprev[0], d_htild, d_mask01,
-                          clip_threshold, mb, d_h[0], d_c[0], nullptr);
+                          clip_threshold, mb, d_h[0], d_c[0], nullptr, nullptr, nullptr, nullptr, nullptr, hp_out);
     else
       rc = lstm_step_impl(ctx, layers[l], d_h[l - 1], nullptr, 0, d_hprev[l], d_cprev[l], nullptr, d_mask01,
-                          clip_threshold, mb, d_h[l], d_c[l], nullptr);
+                          clip_threshold, mb, d_h[l], d_c[l], nullptr, nullptr, nullptr, nullptr, nullptr, hp_out);
     if (rc) return rc;
   }
+  if (wrote_hp_top && top_hp) *wrote_hp_top = 1;
   return ZR_OK;
 }
 

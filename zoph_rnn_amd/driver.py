@@ -65,7 +65,8 @@ class BeamDecode:
         self.logits = ctx.empty((w.Vt * cols + 2 * cols,))
         self.colstats = self.logits.at(w.Vt * cols)
         self.d_words = ctx.array(np.zeros(cols, np.int32))  # <START> = 0
-        self.d_words_nn = ctx.empty(cols, np.int32)
+        self.d_words_nn = ctx.array(np.zeros(cols, np.int32))
+        ctx.beam_set_input_ids(self.bm, self.d_words_nn)
         self.d_back = ctx.empty(cols, np.int32)
         self.d_ones = ctx.array(np.ones(cols, np.int32))
         self.cur = 0
@@ -102,7 +103,7 @@ class BeamDecode:
         ctx, w, cols = self.ctx, self.w, self.cols
         H, L = w.H, w.L
         p, q = self.cur, 1 - self.cur
-        ctx.vocab_prep(self.d_words, cols, w.Vt, self.d_words_nn, None)
+        # (the input ids -- the words of the last step with a dead slot's -1 turned into 0 -- come from the beam itself)
         feed = self.h_tild[p] if self.step_index > 0 else None
         ctx.decoder_step(w.tgt, w.tgt_embed, w.Vt, self.d_words_nn, self.h[p], self.c[p], self.d_ones, cols, self.h[q],
                          self.c[q], self.attn, self.d_batch_info, self.h_tild[q], w.D_soft, w.b_soft, w.Vt,

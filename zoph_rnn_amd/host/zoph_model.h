@@ -1042,6 +1042,7 @@ class beam_decoder {
         ZOPH_CALL(zr_attn_prepare(ctx, attn));
     }
     ZOPH_CALL(zr_beam_create(ctx, beam, Vt, n_sent, longest_sent + 3, (float)penalty, &bm));
+    ZOPH_CALL(zr_beam_set_input_ids(ctx, bm, d_words_nn));
     track_viterbi = BZ_CUDA::unk_replacement && attention;
     if (track_viterbi) {
       const size_t W = 2 * (size_t)D + 1;
@@ -1059,7 +1060,7 @@ class beam_decoder {
   // forward_prop_target (src/model.hpp:2573-2688): state half p -> half q, logits and column statistics into logits
   void forward_target(int p, int step_index) {
     const int q = 1 - p;
-    ZOPH_CALL(zr_vocab_prep(ctx, d_words, cols, Vt, d_words_nn, nullptr));
+    // (d_words_nn, the input ids, are written by the beam call that chose the words: zr_beam_set_input_ids)
     // the whole step in one call: all LSTM layers (layer 0 looks its input columns up in the embedding itself), the
     // attention step on the top layer's h_t, the output distribution of h~
     const dType* feed = (feed_input && step_index > 0) ? h_tild[p] : nullptr;
@@ -1122,6 +1123,7 @@ class beam_decoder {
     ZOPH_CALL(zr_h2d(ctx, d_batch_info, binfo.data(), binfo.size() * sizeof(int)));
     std::vector<int> start(cols, 0);  // <START>
     ZOPH_CALL(zr_h2d(ctx, d_words, start.data(), cols * sizeof(int)));
+    ZOPH_CALL(zr_h2d(ctx, d_words_nn, start.data(), cols * sizeof(int)));
     return S;
   }
 
@@ -1267,7 +1269,7 @@ class ensemble_beam_decoder {
     auto step = [&](int index) {
       for (int k = 0; k < K; k++) {
         // every member is fed the words the shared beam chose
-        if (k > 0) ZOPH_CALL(zr_d2d(ctx, members[k]->d_words, first.d_words, (size_t)first.cols * sizeof(int)));
+        if (k > 0) ZOPH_CALL(zr_d2d(ctx, members[k]->d_words_nn, first.d_words_nn, (size_t)first.cols * sizeof(int)));
         members[k]->forward_target(0, index);
       }
       ZOPH_CALL(zr_ensemble_average(ctx, K, dists.data(), first.Vt, first.cols, mean));
