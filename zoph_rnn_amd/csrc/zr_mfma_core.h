@@ -333,8 +333,11 @@ __device__ __forceinline__ void zr_publish_barrier() {
 
 // 16-byte store that is written through to memory (device scope), what __hip_atomic_store(..., __HIP_MEMORY_SCOPE_AGENT)
 // is for one float: for data another workgroup reads behind a counter.
+// The instruction is followed by one idle cycle: a store of more than 8 bytes reads its data registers one cycle after
+// it issues, and the compiler, which inserts that cycle behind its own stores, does not look inside an asm statement
+// (without it the first register was seen overwritten by the next instruction).
 __device__ __forceinline__ void zr_store16_device(void* p, zr_f32x4 v) {
-  asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+  asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 0" ::"v"(p), "v"(v) : "memory");
 }
 
 // Number of visits zr_reduce_visit makes per thread, and the accumulator slot (tn*16 + r) of visit i: callers use
