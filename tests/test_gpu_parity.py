@@ -798,14 +798,19 @@ def _oracle_decoder_step(case, clip=0.8):
 @pytest.mark.parametrize("H,mb,L,feed", [(64, 5, 3, True), (1000, 128, 4, True), (200, 70, 2, True), (72, 33, 1, False),
                                          (128, 128, 4, False), (256, 192, 4, True), (1000, 12, 4, True),
                                          (104, 40, 8, False), (1000, 192, 4, True), (520, 200, 3, True),
-                                         (776, 250, 2, False)])
+                                         (1000, 160, 4, True), (776, 250, 2, False)])
 def test_decoder_step_all_layers_in_one_launch(ctx, H, mb, L, feed):
     """zr_lstm_decoder_step as ONE launch (two resident workgroups per state tile: one streams the W_h / Q products of
     every layer, the other walks up the chain of layers) against the oracle's node-by-node step and against one launch
     per layer: feed-input on layer 0, duplicate and extreme ids, a masked column, cell clipping, row and column tails,
     a batch width that is not a multiple of 8 (consumers then invalidate their caches), one to eight layers.  The last
-    three shapes have more 32-column tiles than the device holds workgroup pairs for and take 64-column tiles (192
-    columns of H = 1000: the batched beam decode; a last column tile of 8 columns; exactly 256 workgroups)."""
+    four shapes have more 32-column tiles than the device holds workgroup pairs for.  Three of them keep 32-column
+    tiles and hand the W_h products of the upper layers, and the upper part of Q, to helper workgroups of several tiles
+    each, while the chain workgroups compute the W_h products of the lower layers themselves: 192 columns of H = 1000,
+    the batched beam decode, with 64 helpers of three tiles for layers 2 and 3; 200 columns of H = 520 with a last
+    column tile of 8 columns, 88 helpers of two tiles or one, layers 1 and 2; 160 columns with 96 helpers of two tiles
+    or one for layers 1 to 3.  The last has exactly as many 32-column tiles as the device holds workgroups and takes
+    64-column tiles."""
     g = synth.rng(31, H + mb + L)
     case = _decoder_step_case(g, H, mb, L, feed)
     ctx.set_option(capi.ZR_OPT_LSTM_SWEEP, 2)
@@ -837,12 +842,13 @@ def test_decoder_step_picks_the_single_launch_at_benchmark_size_and_repeats_bit_
         assert h1[l].tobytes() == h2[l].tobytes() and c1[l].tobytes() == c2[l].tobytes()
 
 
-@pytest.mark.parametrize("H,mb,L", [(128, 40, 3), (128, 520, 3)])
+@pytest.mark.parametrize("H,mb,L", [(128, 40, 3), (128, 520, 3), (128, 1000, 3)])
 def test_decoder_step_single_launch_abandoned_wait_is_reported(ctx, H, mb, L):
     """The waits for the layer below are told to expect one arrival more than will come and given 64 polls: the layers
     above the first give up whatever the timing, every workgroup still leaves the kernel, the query reports it, the
     unfinished outputs hold NaN, and the next step with the default settings is complete again (the last workgroup out
-    of the abandoned launch returned the counters to zero).  Both tile widths."""
+    of the abandoned launch returned the counters to zero).  32-column tiles in pairs, 32-column tiles with helper
+    workgroups, 64-column tiles in pairs."""
     g = synth.rng(33, 1)
     case = _decoder_step_case(g, H, mb, L, True)
     ctx.set_option(capi.ZR_OPT_LSTM_SWEEP, 2)

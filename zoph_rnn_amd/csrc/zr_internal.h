@@ -27,6 +27,7 @@ struct zr_ctx {
   int lstm_sweep;    // whole-sweep LSTM kernel: 0 auto, 1 never, 2 whenever the launch fits on the device
   int sweep_spin;    // polls before a waiting workgroup of that kernel gives up (0: default)
   int step_wait_extra;  // arrivals the decoder step's layer waits expect beyond the real ones (tests of giving up)
+  int stack_helpers;    // 1 (default): the decoder step may run 32-column tiles with helper workgroups (zr_lstm.hip)
   int cu_count;      // compute units of the device (filled with sweep_capacity)
   int sweep_capacity[3];  // resident workgroups of lstm_sweep_kernel<TN> (0: not asked yet, -1: unknown)
   int stack_step_capacity;  // the same for lstm_decoder_stack_kernel (the lesser of its two tile widths)

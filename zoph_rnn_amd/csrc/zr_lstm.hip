@@ -843,6 +843,14 @@ __global__ void __launch_bounds__(256) lstm_sweep_kernel(LstmSweep P) {
 //          not depend on timing), runs the gate / cell epilogue, writes h and c, publishes a k-interleaved copy of
 //          h for the layer above, and goes on to M_{l+1} . h_t^l as soon as all row tiles of its column tile have
 //          arrived (the weights of that product are already in flight while it waits).
+// Two workgroups per tile need twice as many resident workgroups as there are 32-column tiles; past that (more than 128
+// columns of H = 1000 on 256 compute units) 64-column tiles halve the number of workgroups but leave compute units idle
+// (192 columns: 192 workgroups) and double every link of the chain.  Between the two, while the 32-column tiles alone
+// still fit, the schedule keeps them and fills the remaining compute units with HELPERS: a role-0 workgroup computes
+// the W_h product of the lower layers itself (before M . x, so the wait for the layer below comes last), and each
+// helper streams, for several tiles, first the upper part of Q and then the W_h products of the upper layers, layer by
+// layer, in the order the chains will come for them (192 columns: 192 chains, 64 helpers of three tiles for layers 2
+// and 3 -- 146 us against 168).
 // (Four workgroups per tile at two per compute unit -- the chain sharing each compute unit with the backlog of
 // independent products -- measured slower: 115 us against 106 at H = 1000, 128 columns, 4 layers; the epilogues and
 // hand-overs of the chain take three times as long next to a wave that keeps the matrix pipe busy.)
@@ -874,6 +882,10 @@ struct LstmDecStack {
   int spin_limit;
   int fence;                      // as in LstmSweep
   int wait_extra;                 // arrivals a layer's wait for the layer below expects beyond the real ones (tests)
+  int helpers;                    // 0: every tile has a role-1 workgroup of its own (grid.y = 2); else the number of
+                                  // role-1 workgroups behind the chain slots of a one-dimensional grid
+  int l_split;                    // role 1 delivers the independent products of layers l_split and up; below that a
+                                  // role-0 workgroup computes its own
 };
 
 // All threads of the workgroup call this.  False: leave the kernel.
@@ -908,55 +920,73 @@ __global__ void __launch_bounds__(256) lstm_decoder_stack_kernel(LstmDecStack P)
   const int tid = threadIdx.x;
 
   auto work = [&]() {
-    // die-aware placement as in lstm_fused_kernel; both roles of a tile land on the same die (gridDim.x % 8 == 0)
-    const int id = blockIdx.x;
-    const int r8 = id & 7;
-    const int q8 = id >> 3;
-    const int nt = q8 % P.n_tiles;
+    // Chain slots are placed die-aware as in lstm_fused_kernel; a tile's role-1 workgroup lands on the die of its
+    // role-0 workgroup (gridDim.x % 8 == 0, helpers % 8 == 0).
+    const int slots = P.helpers ? (int)gridDim.x - P.helpers : (int)gridDim.x;
+    const int role = P.helpers ? ((int)blockIdx.x >= slots ? 1 : 0) : (int)blockIdx.y;
     const int per_die = (P.j_tiles + 7) >> 3;
-    const int jt = r8 * per_die + q8 / P.n_tiles;
-    if (q8 / P.n_tiles >= per_die || jt >= P.j_tiles) return;
-    const int role = blockIdx.y;
-
     const int lane = tid & 63;
     const int kslice = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int H = P.H, mb = P.mb;
-    const int j0 = jt * 32;
-    const int n0 = nt * 32 * TN;
     const long long n_el = (long long)H * mb;
     const long long HH = (long long)P.kp * P.ldw;
     const int kgroups = H >> 3;
-    // Q's K range: role 0 takes 9/16 of it, so that role 1's sums of layer 0 (which still have to travel) are there
-    // when role 0 comes for them
+    // Q's K range is shared by the two roles: role 0 takes 9/16, so that role 1's sums of layer 0 (which still have
+    // to travel) are there when role 0 comes for them
     const int q_split = (kgroups * 9) >> 4;
     const int tiles = P.j_tiles * P.n_tiles;
-    const int tile = jt * P.n_tiles + nt;
     int* layer_ctr = P.counters + P.nl * tiles;
-    auto visit_col = [&](int i, int half) {
-      const int slot = zr_wide_visit_slot<KS>(kslice, i);
-      const int tn = slot >> 4, r = slot & 15;
-      const int n = n0 + tn * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-      return n < mb ? n : mb - 1;
-    };
 
-    // A finishing workgroup that abandons a wait in layer l0 leaves NaN in its tile of h and c from that layer up
-    // (role 1 never waits): whatever of the step's outputs was not finished cannot pass for a result.
-    auto abandon = [&](int l0) {
-      const float nan = __builtin_nanf("");
-      for (int l = l0; l < P.nl; ++l)
-        for (int e = tid; e < 32 * 32 * TN; e += 256) {
-          const int j = j0 + (e & 31), n = n0 + (e >> 5);
-          if (j < H && n < mb) P.h[l][(long long)n * H + j] = nan, P.c[l][(long long)n * H + j] = nan;
-        }
-    };
-    for (int l = 0; l < P.nl; ++l) {
-      // per-lane values are derived afresh in every layer (see lstm_sweep_kernel)
+    // Jobs.  Role 0: its tile, layer after layer.  Role 1: the independent products of layers l_split and up --
+    // without helpers for its own tile (l_split = 0), as a helper for the tiles of chain slots w, w + helpers,
+    // w + 2 helpers, ..., layer by layer, in the order the chain will come for them.
+    const int first_slot = role == 0 ? (int)blockIdx.x : (P.helpers ? (int)blockIdx.x - slots : (int)blockIdx.x);
+    const int slot_step = P.helpers ? P.helpers : slots;
+    const int my_slots = role == 0 ? 1 : (slots - first_slot + slot_step - 1) / slot_step;
+    const int l_first = role == 0 ? 0 : P.l_split;
+    // (a helper's first jobs: the upper part of Q's K range for each of its tiles, when layer 0 has a Q)
+    const int q_jobs = (role == 1 && P.helpers && P.htild) ? my_slots : 0;
+    const int n_jobs = q_jobs + (P.nl - l_first) * my_slots;
+    for (int job = 0; job < n_jobs; ++job) {
+      const bool q_only = job < q_jobs;
+      const int l = q_only ? 0 : l_first + (job - q_jobs) / my_slots;
+      const int id = first_slot + ((q_only ? job : job - q_jobs) % my_slots) * slot_step;
+      const int r8 = id & 7;
+      const int q8 = id >> 3;
+      const int nt = q8 % P.n_tiles;
+      const int jt = r8 * per_die + q8 / P.n_tiles;
+      if (q8 / P.n_tiles >= per_die || jt >= P.j_tiles) {  // a padding slot
+        if (role == 0) return;
+        continue;
+      }
+      const int j0 = jt * 32;
+      const int n0 = nt * 32 * TN;
+      const int tile = jt * P.n_tiles + nt;
+      const bool covered = l >= P.l_split;  // role 1 (or a helper) delivers this layer's independent products
+
+      // per-lane values are derived afresh in every job (see lstm_sweep_kernel)
       int lane_t = lane;
       asm volatile("" : "+v"(lane_t));
       const int jl = lane_t & 31, half = lane_t >> 5;
       const int j = j0 + jl;
       const bool j_ok = j < H;
       const int jc = j_ok ? j : H - 1;
+      auto visit_col = [&](int i) {
+        const int slot = zr_wide_visit_slot<KS>(kslice, i);
+        const int tn = slot >> 4, r = slot & 15;
+        const int n = n0 + tn * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+        return n < mb ? n : mb - 1;
+      };
+      // A finishing workgroup that abandons a wait in layer l0 leaves NaN in its tile of h and c from that layer up
+      // (role 1 never waits): whatever of the step's outputs was not finished cannot pass for a result.
+      auto abandon = [&](int l0) {
+        const float nan = __builtin_nanf("");
+        for (int l2 = l0; l2 < P.nl; ++l2)
+          for (int e = tid; e < 32 * 32 * TN; e += 256) {
+            const int j2 = j0 + (e & 31), n2 = n0 + (e >> 5);
+            if (j2 < H && n2 < mb) P.h[l2][(long long)n2 * H + j2] = nan, P.c[l2][(long long)n2 * H + j2] = nan;
+          }
+      };
       int cols[TN];
 #pragma unroll
       for (int tn = 0; tn < TN; ++tn) {
@@ -974,7 +1004,7 @@ __global__ void __launch_bounds__(256) lstm_decoder_stack_kernel(LstmDecStack P)
         bi = bias[jc], bf = bias[H + jc], bc = bias[2 * H + jc], bo = bias[3 * H + jc];
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
-          const int n = visit_col(i, half);
+          const int n = visit_col(i);
           cprev_v[i] = P.cprev[l][(long long)n * H + jc];
           mask_v[i] = (float)P.mask01[n];
         }
@@ -988,17 +1018,24 @@ __global__ void __launch_bounds__(256) lstm_decoder_stack_kernel(LstmDecStack P)
 #pragma unroll
           for (int r = 0; r < 16; ++r) acc[g][tn][r] = 0.0f;
 
-      const int nq = (l == 0 && P.htild) ? 2 : 1;
+      // The products of this job, the one that may have to wait (M_l . h_t^{l-1}) last:
+      //   role 1:                 W_h . h_{t-1}  [+ the upper part of Q's K range in layer 0]  (a helper's Q jobs: Q alone)
+      //   role 0, covered layer:  [the lower part of Q]  + M . x
+      //   role 0, layer it has to itself:  W_h . h_{t-1}  [+ the lower part of Q]  + M . x
+      const bool has_q = l == 0 && P.htild != nullptr;
+      const bool own_wh = role == 0 && !covered;
+      const int n_wh = role == 1 ? (q_only ? 0 : 1) : (own_wh ? 1 : 0);
+      const int nq = n_wh + (has_q ? 1 : 0) + (role == 0 ? 1 : 0);
       for (int q = 0; q < nq; ++q) {
-        // q = 0: this role's own matrix (0 = M, 1 = W_h) over all of K; q = 1: its part of Q's K range
-        const int s = (q == 1) ? 2 : role;
+        // s: the matrix (0 = M, 1 = W_h, 2 = Q)
+        const int s = q < n_wh ? 1 : ((role == 0 && q == nq - 1) ? 0 : 2);
         int g0 = 0, g1 = kgroups;
-        if (q == 1) {
+        if (s == 2) {
           g0 = role ? q_split : 0;
           g1 = role ? kgroups : q_split;
         }
         const int K = (g1 - g0) * 8;
-        const bool packed = role == 0 && q == 0 && l > 0;
+        const bool packed = s == 0 && l > 0;
         unsigned wsoff[4];
 #pragma unroll
         for (int g = 0; g < 4; ++g) wsoff[g] = (unsigned)((((long long)s * 4 + g) * HH + (long long)g0 * 8 * P.ldw) * 4);
@@ -1019,8 +1056,8 @@ __global__ void __launch_bounds__(256) lstm_decoder_stack_kernel(LstmDecStack P)
 #pragma unroll
           for (int tn = 0; tn < TN; ++tn) xoffb[tn] = 16u * ((unsigned)cols[tn] + (unsigned)(half * mb));
         } else {
-          xb = (q == 1) ? P.htild + g0 * 8 : (role == 1 ? P.hprev[l] : P.in0);
-          const bool gather = q == 0 && role == 0 && P.ids != nullptr;
+          xb = s == 2 ? P.htild + g0 * 8 : (s == 1 ? P.hprev[l] : P.in0);
+          const bool gather = s == 0 && P.ids != nullptr;
 #pragma unroll
           for (int tn = 0; tn < TN; ++tn) {
             unsigned c = (unsigned)cols[tn];
@@ -1049,16 +1086,23 @@ __global__ void __launch_bounds__(256) lstm_decoder_stack_kernel(LstmDecStack P)
       }
 
       // role 0: the other role's sums (normally long there), fetched while this workgroup's partial tiles are summed
-      if (!stack_wait(P, flag, 1, &s_go[1])) {
-        abandon(l);
-        return;
-      }
       float other[NV][4];
+      if (covered || has_q) {
+        if (!stack_wait(P, flag, 1, &s_go[1])) {
+          abandon(l);
+          return;
+        }
 #pragma unroll
-      for (int vi = 0; vi < NV; ++vi)
+        for (int vi = 0; vi < NV; ++vi)
 #pragma unroll
-        for (int g = 0; g < 4; ++g)
-          other[vi][g] = __hip_atomic_load(part + (vi * 4 + g) * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          for (int g = 0; g < 4; ++g)
+            other[vi][g] = __hip_atomic_load(part + (vi * 4 + g) * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      } else {
+#pragma unroll
+        for (int vi = 0; vi < NV; ++vi)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) other[vi][g] = 0.0f;
+      }
       const bool hand_on = l + 1 < P.nl;
       float* hp_out = P.hp + (long long)l * n_el;
       float h_v[NV], c_v[NV];
@@ -1601,10 +1645,28 @@ int zr_lstm_decoder_step_packed(zr_ctx* ctx, int nl, const zr_lstm_weights* cons
     const int cap = stack_step_capacity(ctx);
     // 32-column tiles while two workgroups per tile fit on the device together, 64-column tiles beyond that (192 columns
     // of H = 1000: 384 workgroups against 192)
-    const int tn = (2LL * padded * ((mb + 31) / 32) <= cap) ? 1 : 2;
+    // (or, between the two: 32-column tiles whose role-1 work of the UPPER layers goes to as many helper workgroups
+    // as still fit, several tiles each, while a role-0 workgroup computes the independent products of the lower layers
+    // itself -- at 192 columns 192 chains and 64 helpers of three tiles x two layers fill the 256 compute units that 192
+    // workgroups on 64-column tiles leave a quarter of idle)
+    const int slots1 = padded * ((mb + 31) / 32);
+    int tn = (2LL * slots1 <= cap) ? 1 : 2;
+    int helpers = 0, l_split = 0;
+    if (tn == 2 && slots1 < cap && ctx->stack_helpers) {
+      int hn = cap - slots1 < slots1 ? cap - slots1 : slots1;
+      hn &= ~7;
+      const int covered = hn > 0 ? (2 * nl * hn) / (slots1 + hn) : 0;
+      // (only when the helpers take at least half of the layers: at 224 columns, 32 helpers of seven tiles for the top
+      // layer alone, the step measured 206 us against 168 on 64-column tiles; at 160 and 192 columns 136 and 146)
+      if (covered >= 1 && 2 * covered >= nl) {
+        tn = 1;
+        helpers = hn;
+        l_split = nl - (covered < nl ? covered : nl);
+      }
+    }
     const int n_tiles = (mb + 32 * tn - 1) / (32 * tn);
     const long long tiles = (long long)j_tiles * n_tiles;
-    const long long wgs = 2LL * padded * n_tiles;
+    const long long wgs = helpers ? (long long)padded * n_tiles + helpers : 2LL * padded * n_tiles;
     const bool fills = wgs * 10 >= 6LL * ctx->cu_count && zr_live_contexts(ctx->device) == 1 &&
                        ctx->stream == ctx->own_stream;
     const long long lim = 1LL << 32;
@@ -1650,8 +1712,10 @@ int zr_lstm_decoder_step_packed(zr_ctx* ctx, int nl, const zr_lstm_weights* cons
       P.spin_limit = ctx->sweep_spin > 0 ? ctx->sweep_spin : (1 << 20);
       P.fence = (mb % 8 == 0) ? 0 : 1;
       P.wait_extra = ctx->step_wait_extra;
+      P.helpers = helpers;
+      P.l_split = l_split;
       ctx->last_stack_path = ZR_LSTM_STACK_PATH_STEP_SINGLE_LAUNCH;
-      const dim3 grid((unsigned)(padded * n_tiles), 2u);
+      const dim3 grid((unsigned)(padded * n_tiles + helpers), helpers ? 1u : 2u);
       if (tn == 1)
         lstm_decoder_stack_kernel<1><<<grid, 256, 0, ctx->stream>>>(P);
       else

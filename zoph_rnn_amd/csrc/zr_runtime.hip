@@ -135,6 +135,9 @@ int zr_ctx_create(int device, zr_ctx** out) {
     const int v = atoi(e);
     if (v >= 0 && v <= 1024) c->step_wait_extra = v;
   }
+  // ZR_LSTM_STACK_HELPERS=0 keeps the decoder step on its two-workgroups-per-tile schedules (timing comparisons)
+  c->stack_helpers = 1;
+  if (const char* e = getenv("ZR_LSTM_STACK_HELPERS")) c->stack_helpers = atoi(e) != 0 ? 1 : 0;
   if (device < 64) g_live[device].fetch_add(1);
   *out = c;
   return ZR_OK;
