@@ -47,7 +47,7 @@ SYMBOLS = [
     "zr_lstm_gates", "zr_lstm_stack_forward", "zr_gemm", "zr_softmax_prepare", "zr_softmax_prepare_bf16", "zr_softmax_release", "zr_softmax_forward", "zr_softmax_logprob_f64",
     "zr_softmax_loss", "zr_attn_create", "zr_attn_use_bf16_weights", "zr_attn_destroy", "zr_attn_step", "zr_gather_columns",
     "zr_broadcast_column", "zr_beam_create", "zr_beam_destroy", "zr_beam_init", "zr_beam_expand", "zr_beam_finish", "zr_beam_expand_logits", "zr_beam_finish_logits",
-    "zr_beam_hypotheses", "zr_beam_state", "zr_beam_set_viterbi", "zr_beam_hypotheses_viterbi", "zr_ensemble_average",
+    "zr_beam_hypotheses", "zr_beam_state", "zr_beam_set_viterbi", "zr_beam_set_input_ids", "zr_beam_hypotheses_viterbi", "zr_ensemble_average",
     "zr_attn_viterbi_ensemble",
     "zr_lstm_stack_forward_train", "zr_lstm_train_create", "zr_lstm_train_refresh", "zr_lstm_train_destroy",
     "zr_unstack_gates", "zr_lstm_stack_backward", "zr_lstm_weight_gradients", "zr_embed_gradient",
