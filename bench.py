@@ -335,7 +335,7 @@ def bench_hbm_kernels(ctx, steps, H=1000, mb=128, V=50000):
 def bench_beam_decode(ctx, steps, H=1000, L=4, beam=12, n_sent=16, S=50, V=50000, D=10):
     """Config 4: batched beam decode (16 sentences x beam 12 = 192 columns), per decode step: gather, 4 LSTM layers
     with feed-input, attention (reference default width D=10), full softmax, device-side beam, state reorder."""
-    from zoph_rnn_amd import driver, synth
+    from zoph_rnn_amd import capi, driver, synth
     g = synth.rng(1234, 4)
     src_layers = [synth.lstm_layer(g, H) for _ in range(L)]
     tgt_layers = [synth.lstm_layer(g, H, feed_input=(l == 0)) for l in range(L)]
@@ -351,15 +351,18 @@ def bench_beam_decode(ctx, steps, H=1000, L=4, beam=12, n_sent=16, S=50, V=50000
     res = {"columns": beam * n_sent, "ms_per_decode_step": round(ms / steps, 4),
            "hypotheses_per_s": round(beam * n_sent * steps / (ms * 1e-3), 1), "encode_ms": round(enc_ms, 3),
            "attention_D": D}
-    # the beam's three launches on their own (selection over the V x columns logits, merges, bookkeeping)
+    # the beam's two launches on their own: the per-column selection on the output product's per-block pairs (folds the
+    # pairs, reads only the blocks that can hold one of a column's beam + 1 largest logits) and the per-sentence merge.
+    # Algorithmic bytes: the pairs (8 bytes per 32 rows and column) -- the V x columns logits are not read again.
     bm = ctx.beam_create(beam, V, n_sent, steps + 40, 0.0)
     d_w, d_b = ctx.empty(beam * n_sent, np.int32), ctx.empty(beam * n_sent, np.int32)
-    ctx.beam_expand_logits(bm, dec.logits, dec.colstats, 0, d_w, d_b)
-    _, bms = time_region(ctx, lambda: ctx.beam_expand_logits(bm, dec.logits, dec.colstats, 1, d_w, d_b), 20, 2)
+    ctx.beam_expand_blocks(bm, dec.logits, dec.blocks, 0, d_w, d_b)
+    _, bms = time_region(ctx, lambda: ctx.beam_expand_blocks(bm, dec.logits, dec.blocks, 1, d_w, d_b), 20, 2)
     ctx.beam_destroy(bm)
     res["beam_us"] = round(bms * 1e3 / 20, 2)
-    res["beam_roofline"] = roofline_entry("beam_topk_kernel + beam_topk_merge_kernel + beam_merge_kernel", "hbm",
-                                          bms * 1e3 / 20, nbytes=float(V) * beam * n_sent * 4)
+    res["beam_roofline"] = roofline_entry("beam_select_blocks_kernel + beam_merge_kernel (latency-bound: two small "
+                                          "launches)", "hbm", bms * 1e3 / 20,
+                                          nbytes=float(capi.softmax_block_count(V)) * 8 * beam * n_sent)
     dec.close()
     return res
 

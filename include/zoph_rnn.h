@@ -263,10 +263,20 @@ int zr_softmax_release(zr_ctx* ctx, const float* d_D);
  * exp(x - max) / sum for the few entries a decode step needs, so the V x mb matrix is written once and read once per
  * step instead of written twice and read twice.  d_logits_scratch must be NULL in this mode. */
 #define ZR_SOFTMAX_LOGITS 2
+/* As ZR_SOFTMAX_LOGITS, but instead of two statistics per column d_out receives what the product's epilogue already
+ * has: one (max, sum of exp(x - max)) pair per block of 32 vocabulary rows and column, [mb][zr_softmax_block_count(V)][2]
+ * floats starting zr_softmax_blocks_offset(V, mb) floats into d_out (d_out holds that offset + 2 * blocks * mb floats).
+ * Nothing folds them: zr_beam_expand_blocks / zr_beam_finish_blocks do, and use the block maxima to find the few blocks
+ * of a column that can hold one of its beam + 1 largest entries, so a decode step reads the V x mb logits it has just
+ * written only there.  No counterpart in the reference (its decoder copies the whole normalised matrix to the host,
+ * src/decoder_model_wrapper.hpp:418).  d_logits_scratch must be NULL in this mode. */
+#define ZR_SOFTMAX_LOGITS_BLOCKS 3
+int zr_softmax_block_count(int V);
+long long zr_softmax_blocks_offset(int V, int cols);
 
 /* D h + b_d on MFMA (cublasSgemm + matrix_bias_kernel, src/softmax.hpp:539-547) followed by the per-column
  * max / exp / sum / normalise of outputdist_overflow_prevention_kernel (src/custom_kernels.h:503-577).
- * d_out: V x mb (V*mb + 2*mb floats in mode ZR_SOFTMAX_LOGITS).  d_logits_scratch: V x mb scratch for the logits, or
+ * d_out: V x mb (more in the two logits modes, see above).  d_logits_scratch: V x mb scratch for the logits, or
  * NULL to use d_out in place. */
 int zr_softmax_forward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int mb,
                        int mode, float* d_out, float* d_logits_scratch);
@@ -373,12 +383,20 @@ int zr_beam_finish(zr_ctx* ctx, zr_beam* b, const float* d_prob);
 /* zr_beam_expand / zr_beam_finish on the output of ZR_SOFTMAX_LOGITS: d_logits V x (n_sent*beam), d_colstats 2 floats
  * per column (max, sum of exp(x - max)) -- d_out and d_out + V*cols of that call.  The per-column selection runs on the
  * logits (the soft-max is monotonic within a column) and only the beam+1 selected entries of a column are normalised,
- * with the same expression as the full matrix, so candidates, scores, words and back-pointers are those of
- * zr_beam_expand on the probabilities; the one difference: two words whose logits differ but whose probabilities
- * round to the same float rank by logit here and by word id there. */
+ * with the same expression as the full matrix, and the candidates are ranked by those probabilities (words whose
+ * probabilities round to one float follow the tie rule, whatever their logits), so candidates, scores, words and
+ * back-pointers are those of zr_beam_expand on the probabilities. */
 int zr_beam_expand_logits(zr_ctx* ctx, zr_beam* b, const float* d_logits, const float* d_colstats, int index,
                           int* d_words, int* d_backptr);
 int zr_beam_finish_logits(zr_ctx* ctx, zr_beam* b, const float* d_logits, const float* d_colstats);
+/* The same on the output of ZR_SOFTMAX_LOGITS_BLOCKS: d_logits V x (n_sent*beam), d_blocks the per-block pairs behind
+ * them (d_out and d_out + zr_softmax_blocks_offset(V, cols) of that call).  One launch per step folds a column's pairs
+ * into its statistics (in the order zr_softmax_forward does: the same bits), bounds the beam + 1 largest entries from
+ * below by the block maxima, reads only the blocks that reach the bound and ranks what it finds there; results are
+ * those of zr_beam_expand_logits bit for bit. */
+int zr_beam_expand_blocks(zr_ctx* ctx, zr_beam* b, const float* d_logits, const float* d_blocks, int index,
+                          int* d_words, int* d_backptr);
+int zr_beam_finish_blocks(zr_ctx* ctx, zr_beam* b, const float* d_logits, const float* d_blocks);
 /* Copies the finished hypotheses of sentence s to the host: returns their number (or a negative error);
  * h_words is n x max_len (row-major, -1 padded), h_len and h_score have n entries; at most cap are copied. */
 int zr_beam_hypotheses(zr_ctx* ctx, zr_beam* b, int sentence, int cap, int* h_words, int* h_len, float* h_score);

@@ -267,8 +267,9 @@ def test_beam_selection_on_adversarial_layouts(ctx, V, beam):
 @pytest.mark.parametrize("V,H,beam,n_sent,prepared", [(5000, 32, 5, 3, False), (50000, 64, 12, 16, True),
                                                       (8193, 16, 31, 2, False), (70001, 24, 7, 4, True)])
 def test_beam_on_logits_equals_beam_on_probabilities(ctx, V, H, beam, n_sent, prepared):
-    """ZR_SOFTMAX_LOGITS + zr_beam_expand_logits / zr_beam_finish_logits against ZR_SOFTMAX_PROB + zr_beam_expand /
-    zr_beam_finish on the same activations: the logits are the same bits, the column statistics are the column's maximum
+    """ZR_SOFTMAX_LOGITS + zr_beam_expand_logits / zr_beam_finish_logits, and ZR_SOFTMAX_LOGITS_BLOCKS +
+    zr_beam_expand_blocks / zr_beam_finish_blocks (one selection launch on the product's per-block pairs, which must hold
+    the block maxima), against ZR_SOFTMAX_PROB + zr_beam_expand / zr_beam_finish on the same activations: the logits are the same bits, the column statistics are the column's maximum
     and its sum of exp(x - max), and every word, back-pointer, beam score and finished hypothesis is identical, scores
     to the bit (the selected entries are normalised with the expression the full matrix is normalised with).  <EOF> is
     made likely so that hypotheses finish inside the steps."""
@@ -284,41 +285,59 @@ def test_beam_on_logits_equals_beam_on_probabilities(ctx, V, H, beam, n_sent, pr
     d_lg = ctx.empty((V * cols + 2 * cols,))
     d_stats = d_lg.at(V * cols)
     ba, bb = ctx.beam_create(beam, V, n_sent, max_len, 0.1), ctx.beam_create(beam, V, n_sent, max_len, 0.1)
+    bc = ctx.beam_create(beam, V, n_sent, max_len, 0.1)
     wa, ka = ctx.empty(cols, np.int32), ctx.empty(cols, np.int32)
     wb, kb = ctx.empty(cols, np.int32), ctx.empty(cols, np.int32)
+    wc, kc = ctx.empty(cols, np.int32), ctx.empty(cols, np.int32)
+    off, nblk = capi.softmax_blocks_offset(V, cols), capi.softmax_block_count(V)
+    assert nblk == (V + 31) // 32 and off >= V * cols and off % 4 == 0
+    d_lb = ctx.empty((off + 2 * nblk * cols,))
+    d_blocks = d_lb.at(off)
     for index in range(steps + 1):
         h = np.asfortranarray(g.uniform(-1, 1, size=(H, cols)).astype(np.float32))
         dh = ctx.array(h)
         ctx.softmax_forward(dD, dbd, V, H, dh, cols, capi.ZR_SOFTMAX_PROB, d_prob, d_scr)
         ctx.softmax_forward(dD, dbd, V, H, dh, cols, capi.ZR_SOFTMAX_LOGITS, d_lg)
+        ctx.softmax_forward(dD, dbd, V, H, dh, cols, capi.ZR_SOFTMAX_LOGITS_BLOCKS, d_lb)
         ctx.sync()
         out = d_lg.get()
         lg, stats = out[:V * cols].reshape((V, cols), order="F"), out[V * cols:].reshape(cols, 2)
         assert np.array_equal(lg, d_scr.get())
+        outb = d_lb.get()
+        assert np.array_equal(outb[:V * cols], out[:V * cols])
+        pairs = outb[off:].reshape(cols, nblk, 2)
+        pad = np.full((nblk * 32, cols), -np.inf, np.float32)
+        pad[:V] = lg
+        assert np.array_equal(pairs[:, :, 0], pad.reshape(nblk, 32, cols).max(axis=1).T)  # the block maxima
         assert np.array_equal(stats[:, 0], lg.max(axis=0))
         want_sum = np.exp(lg.astype(np.float64) - lg.max(axis=0).astype(np.float64)).sum(axis=0)
         assert np.allclose(stats[:, 1], want_sum, rtol=2e-6, atol=0)
         if index == steps:
             ctx.beam_finish(ba, d_prob)
             ctx.beam_finish_logits(bb, d_lg, d_stats)
+            ctx.beam_finish_blocks(bc, d_lb, d_blocks)
             break
         ctx.beam_expand(ba, d_prob, index, wa, ka)
         ctx.beam_expand_logits(bb, d_lg, d_stats, index, wb, kb)
+        ctx.beam_expand_blocks(bc, d_lb, d_blocks, index, wc, kc)
         ctx.sync()
-        assert np.array_equal(wa.get(), wb.get()), index
-        assert np.array_equal(ka.get(), kb.get()), index
+        assert np.array_equal(wa.get(), wb.get()) and np.array_equal(wa.get(), wc.get()), index
+        assert np.array_equal(ka.get(), kb.get()) and np.array_equal(ka.get(), kc.get()), index
         for s in range(n_sent):
             sa, xa = ctx.beam_state(ba, s, beam)
             sb, xb = ctx.beam_state(bb, s, beam)
+            sc, xc = ctx.beam_state(bc, s, beam)
             assert np.array_equal(xa, xb) and np.array_equal(sa[xa != -1], sb[xb != -1]), (index, s)
+            assert np.array_equal(xa, xc) and np.array_equal(sa[xa != -1], sc[xc != -1]), (index, s)
     ctx.sync()
     finished = 0
     for s in range(n_sent):
         ga, na = ctx.beam_hypotheses(ba, s, cap=256, max_len=max_len)
         gb, nb = ctx.beam_hypotheses(bb, s, cap=256, max_len=max_len)
-        assert na == nb and na >= 1
-        for (w1, s1), (w2, s2) in zip(ga, gb):
-            assert np.array_equal(w1, w2) and s1 == s2
+        gc, nc = ctx.beam_hypotheses(bc, s, cap=256, max_len=max_len)
+        assert na == nb and na == nc and na >= 1
+        for (w1, s1), (w2, s2), (w3, s3) in zip(ga, gb, gc):
+            assert np.array_equal(w1, w2) and s1 == s2 and np.array_equal(w1, w3) and s1 == s3
         finished += na
     assert finished > n_sent * beam  # some hypotheses finished inside the steps, not only at the forced end
     with pytest.raises(capi.ZrError):
@@ -327,6 +346,7 @@ def test_beam_on_logits_equals_beam_on_probabilities(ctx, V, H, beam, n_sent, pr
         ctx.softmax_release(dD)
     ctx.beam_destroy(ba)
     ctx.beam_destroy(bb)
+    ctx.beam_destroy(bc)
 
 
 @pytest.mark.parametrize("K,V,cols", [(1, 37, 3), (2, 400, 12), (5, 50000, 192), (8, 1025, 1)])
@@ -404,6 +424,64 @@ def test_ensemble_alignment_vote_known_answer_and_brute_force(ctx):
         ctx.attn_viterbi_ensemble(d[0], d[1], 3, 3, 9000, d_out)
     for x in d[0] + d[1] + [d_out]:
         x.free()
+
+
+@pytest.mark.parametrize("V,beam,n_sent", [(50000, 12, 1), (8193, 12, 2), (40, 5, 1), (50017, 30, 1)])
+def test_beam_on_blocks_with_hostile_columns(ctx, V, beam, n_sent):
+    """zr_beam_expand_blocks against zr_beam_expand_logits and zr_beam_expand on logits built to stress the selection on
+    block maxima: a constant column (every block reaches the bound: the exact K-pass path), thousands of copies of the
+    largest value (candidate list overflows), copies of the K-th largest value spread over hundreds of blocks, the K
+    largest in one block, one per block, a column of very negative numbers, the three-words-one-probability case, a last
+    block of one row, a vocabulary of two blocks.  The logits are produced by the output product itself from a matrix
+    that holds them and one-hot activations (exact), so the three paths see the same bits."""
+    g = synth.rng(49, V + beam)
+    cols, K = beam * n_sent, beam + 1
+    lg = np.asfortranarray(g.uniform(-3, -2, size=(V, cols)).astype(np.float32))
+
+    def col(i):
+        return i % cols
+
+    lg[:, col(0)] = 0.5                                                  # constant column
+    many = g.choice(V, size=min(3000, V // 2), replace=False)
+    lg[many, col(1)] = 1.0                                               # thousands of copies of the maximum
+    top = np.float32(0.2)
+    b1 = np.nextafter(top, np.float32(-1))
+    b2 = np.nextafter(b1, np.float32(-1))
+    lg[V - 1, col(2)], lg[3, col(2)], lg[V // 2, col(2)] = top, b1, b2   # one probability, three logits
+    if V >= 64 * K:
+        lg[32 * 7:32 * 7 + K, col(3)] = np.linspace(2.0, 1.0, K, dtype=np.float32)      # the K largest in one block
+        lg[np.arange(K + 20) * 32 + 5, col(4)] = np.linspace(3.0, 1.0, K + 20, dtype=np.float32)  # one per block
+        idx = g.choice(V, size=min(700 * 32, V) // 32, replace=False)
+        lg[idx[:K - 1], col(6)] = 4.0 + np.arange(K - 1, dtype=np.float32)
+        lg[idx[K - 1:], col(6)] = 1.5                                     # the K-th largest, hundreds of times
+    lg[:, col(5)] = -1e30
+    lg[[2 % V, (V - 1)], col(5)] = [-5.0, -6.0]
+    H = cols
+    dD, dbd = ctx.array(lg), ctx.array(np.zeros(V, np.float32))
+    dh = ctx.array(np.asfortranarray(np.eye(H, dtype=np.float32)))
+    off, nblk = capi.softmax_blocks_offset(V, cols), capi.softmax_block_count(V)
+    d_prob, d_lg, d_lb = ctx.empty((V, cols)), ctx.empty((V * cols + 2 * cols,)), ctx.empty((off + 2 * nblk * cols,))
+    ctx.softmax_forward(dD, dbd, V, H, dh, cols, capi.ZR_SOFTMAX_PROB, d_prob)
+    ctx.softmax_forward(dD, dbd, V, H, dh, cols, capi.ZR_SOFTMAX_LOGITS, d_lg)
+    ctx.softmax_forward(dD, dbd, V, H, dh, cols, capi.ZR_SOFTMAX_LOGITS_BLOCKS, d_lb)
+    ctx.sync()
+    assert np.array_equal(d_lg.get()[:V * cols].reshape((V, cols), order="F"), lg)  # the product reproduced the logits
+    beams = [ctx.beam_create(beam, V, n_sent, 8, 0.0) for _ in range(3)]
+    outs = [(ctx.empty(cols, np.int32), ctx.empty(cols, np.int32)) for _ in range(3)]
+    for index in range(2):
+        ctx.beam_expand(beams[0], d_prob, index, *outs[0])
+        ctx.beam_expand_logits(beams[1], d_lg, d_lg.at(V * cols), index, *outs[1])
+        ctx.beam_expand_blocks(beams[2], d_lb, d_lb.at(off), index, *outs[2])
+        ctx.sync()
+        for k in (1, 2):
+            assert np.array_equal(outs[0][0].get(), outs[k][0].get()), (index, k)
+            assert np.array_equal(outs[0][1].get(), outs[k][1].get()), (index, k)
+            for s_ in range(n_sent):
+                sa, xa = ctx.beam_state(beams[0], s_, beam)
+                sk, xk = ctx.beam_state(beams[k], s_, beam)
+                assert np.array_equal(xa, xk) and np.array_equal(sa[xa != -1], sk[xk != -1]), (index, k, s_)
+    for b in beams:
+        ctx.beam_destroy(b)
 
 
 def test_beam_on_logits_ranks_words_of_equal_probability_as_the_probability_matrix_would(ctx):

@@ -38,6 +38,7 @@ ZR_SOFTMAX_PROB = 0
 ZR_SOFTMAX_LOGPROB = 1
 ZR_CLIP_NONE, ZR_CLIP_MATRIX_NORM, ZR_CLIP_WHOLE_NORM, ZR_CLIP_ELEMENT = 0, 1, 2, 3
 ZR_SOFTMAX_LOGITS = 2  # d_out: V*mb logits followed by 2*mb column statistics (max, sum of exp(x - max))
+ZR_SOFTMAX_LOGITS_BLOCKS = 3  # d_out: the logits, then (max, sum exp) per 32-row block and column at softmax_blocks_offset
 
 # every symbol include/zoph_rnn.h declares
 SYMBOLS = [
@@ -47,6 +48,7 @@ SYMBOLS = [
     "zr_lstm_gates", "zr_lstm_stack_forward", "zr_gemm", "zr_softmax_prepare", "zr_softmax_prepare_bf16", "zr_softmax_release", "zr_softmax_forward", "zr_softmax_logprob_f64",
     "zr_softmax_loss", "zr_attn_create", "zr_attn_use_bf16_weights", "zr_attn_destroy", "zr_attn_step", "zr_gather_columns",
     "zr_broadcast_column", "zr_beam_create", "zr_beam_destroy", "zr_beam_init", "zr_beam_expand", "zr_beam_finish", "zr_beam_expand_logits", "zr_beam_finish_logits",
+    "zr_beam_expand_blocks", "zr_beam_finish_blocks", "zr_softmax_block_count", "zr_softmax_blocks_offset",
     "zr_beam_hypotheses", "zr_beam_state", "zr_beam_set_viterbi", "zr_beam_set_input_ids", "zr_beam_hypotheses_viterbi", "zr_ensemble_average",
     "zr_attn_viterbi_ensemble",
     "zr_lstm_stack_forward_train", "zr_lstm_train_create", "zr_lstm_train_refresh", "zr_lstm_train_destroy",
@@ -76,7 +78,17 @@ def load():
         _lib = C.CDLL(LIB_PATH)
         _lib.zr_last_error.restype = C.c_char_p
         _lib.zr_version.restype = C.c_char_p
+        _lib.zr_softmax_blocks_offset.restype = C.c_longlong
     return _lib
+
+
+def softmax_block_count(V):
+    return int(load().zr_softmax_block_count(C.c_int(V)))
+
+
+def softmax_blocks_offset(V, cols):
+    """ZR_SOFTMAX_LOGITS_BLOCKS: where the per-block pairs start in d_out, in floats."""
+    return int(load().zr_softmax_blocks_offset(C.c_int(V), C.c_int(cols)))
 
 
 def _chk(rc):
@@ -448,6 +460,13 @@ class Context:
 
     def beam_finish_logits(self, b, d_logits, d_colstats):
         _chk(load().zr_beam_finish_logits(self.h, b, _vp(d_logits), _vp(d_colstats)))
+
+    def beam_expand_blocks(self, b, d_logits, d_blocks, index, d_words, d_backptr):
+        _chk(load().zr_beam_expand_blocks(self.h, b, _vp(d_logits), _vp(d_blocks), C.c_int(index), _vp(d_words),
+                                          _vp(d_backptr)))
+
+    def beam_finish_blocks(self, b, d_logits, d_blocks):
+        _chk(load().zr_beam_finish_blocks(self.h, b, _vp(d_logits), _vp(d_blocks)))
 
     def beam_hypotheses(self, b, sentence, cap, max_len):
         words = np.full((cap, max_len), -1, dtype=np.int32)

@@ -17,6 +17,7 @@
 #include <math.h>
 
 #include "zr_internal.h"
+#include "zr_softmax_fold.h"
 
 struct zr_beam {
   int beam, vocab, n_sent, max_len, hyp_cap;
@@ -44,6 +45,7 @@ struct zr_beam {
   int* d_cand_w;            // [n_sent*beam][beam+1]
   float* d_part_p;          // [n_sent*beam][chunks][beam+1] per-chunk candidates of the first top-K stage
   int* d_part_w;
+  float* d_colstats;        // [n_sent*beam][2] column statistics the selection on blocks leaves for zr_beam_finish_blocks
   void* d_block;            // the single allocation behind all of the above
 };
 
@@ -258,6 +260,148 @@ beam_topk_merge_kernel(const float* __restrict__ part_p, const int* __restrict__
       cand_p[(size_t)col * K + rank] = part_p[(size_t)col * n + a];
       cand_w[(size_t)col * K + rank] = part_w[(size_t)col * n + a];
     }
+  }
+}
+
+// Per-column top-K straight from the output product's per-block pairs (ZR_SOFTMAX_LOGITS_BLOCKS): one workgroup per
+// column does what softmax_colstats_kernel, beam_topk_kernel and beam_topk_merge_kernel do in three launches, and reads
+// of the column's V logits only the 32-row blocks that can hold one of its K largest entries.
+//   1. The column's pairs ([nblocks][2], 12.5 KB at 50 000 words) are folded into (max, sum) exactly as
+//      softmax_colstats_kernel folds them (zr_softmax_fold.h: the same bits, hence the same probabilities).
+//   2. A thread's largest block maximum is the maximum of a group of the column's logits, so the K-th largest of the
+//      threads' values (taken per wave, the largest of the four waves' results) is a lower bound of the K-th largest
+//      logit; it is lowered by a few ulp as in beam_topk_kernel, so that every word whose PROBABILITY could equal a
+//      listed one is listed.
+//   3. The blocks whose maximum reaches the bound are listed (a second pass over the pairs, which are in cache), their
+//      logits are read, 32 at a time per half-wave, and those at or above the bound go on the candidate list keyed by
+//      probability and word id; the list is ranked by counting and the first K written out.
+// Either list overflowing (hundreds of blocks within a few ulp of the K-th largest logit: constant columns) sends the
+// workgroup down an exact path that needs no bound: K passes over the whole column, each taking the largest key below
+// the previous one.  Keys, tie rule and fillers are those of the two-stage selection: the K-lists are the same bit for
+// bit.
+constexpr int kSelBlockCap = 512;   // candidate blocks per column
+constexpr int kSelCandCap = 1024;   // candidate words per column
+
+__global__ void __launch_bounds__(256)
+beam_select_blocks_kernel(const float* __restrict__ logits, const float* __restrict__ blocks, int V, int K, int nblocks,
+                          float* __restrict__ cand_p, int* __restrict__ cand_w, float* __restrict__ colstats_out) {
+  __shared__ float s_m[4], s_s[4];
+  __shared__ float s_stats[2];
+  __shared__ unsigned s_tau_wave[4];
+  __shared__ int s_blk[kSelBlockCap];
+  __shared__ unsigned long long s_cand[kSelCandCap];
+  __shared__ unsigned long long s_best[4];
+  __shared__ int s_nblk, s_count;
+  const int col = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const float* x = logits + (size_t)col * V;
+  const float* pairs = blocks + (size_t)col * nblocks * 2;
+  if (tid == 0) s_nblk = 0, s_count = 0;
+  float mx, sum, bm;
+  zr_softmax_fold_column(pairs, nblocks, s_m, s_s, mx, sum, &bm);
+  if (tid == 0) {
+    s_stats[0] = mx;
+    s_stats[1] = sum;
+    colstats_out[2 * col] = mx;
+    colstats_out[2 * col + 1] = sum;
+  }
+  // the bound: K-th largest thread value inside each wave (bitonic sort of the 64 lanes), largest of the four waves
+  {
+    unsigned v = bm > -INFINITY ? (unsigned)(topk_key(bm, 0) >> 32) : 0u;
+#pragma unroll
+    for (int k = 2; k <= 64; k <<= 1)
+#pragma unroll
+      for (int j = k >> 1; j > 0; j >>= 1) {
+        const unsigned o = (unsigned)__shfl_xor((int)v, j, 64);
+        const bool keep_max = ((lane & j) == 0) == ((lane & k) == 0);
+        v = keep_max ? (v > o ? v : o) : (v < o ? v : o);
+      }
+    if (lane == K - 1) s_tau_wave[wave] = v;
+  }
+  __syncthreads();
+  const float c_max = s_stats[0], c_sum = s_stats[1];
+  unsigned tu = s_tau_wave[0];
+#pragma unroll
+  for (int w = 1; w < 4; ++w) tu = s_tau_wave[w] > tu ? s_tau_wave[w] : tu;
+  float tp;
+  {
+    int tw;
+    topk_unkey((unsigned long long)tu << 32, tp, tw);  // (no thread value at all: -inf, which lists every block)
+    tp -= 1e-6f + 5e-7f * (fabsf(tp) + fabsf(c_max));
+  }
+  // candidate blocks (the maxima again, eight loads in flight per thread)
+  for (int b0 = 0; b0 < nblocks; b0 += 2048) {
+    float pm[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int b = b0 + tid + 256 * u;
+      pm[u] = b < nblocks ? pairs[2 * b] : -INFINITY;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (pm[u] >= tp && pm[u] > -INFINITY) {
+        const int pos = atomicAdd(&s_nblk, 1);
+        if (pos < kSelBlockCap) s_blk[pos] = b0 + tid + 256 * u;
+      }
+    }
+  }
+  __syncthreads();
+  const int nblk = s_nblk;
+  bool exact = nblk > kSelBlockCap;
+  if (!exact) {
+    // candidate words: a half-wave per block
+    const int hw = tid >> 5, l32 = tid & 31;
+    for (int i = hw; i < nblk; i += 8) {
+      const int v = s_blk[i] * 32 + l32;
+      const float q = v < V ? x[v] : -INFINITY;
+      if (q >= tp && q > -INFINITY) {
+        const int pos = atomicAdd(&s_count, 1);
+        if (pos < kSelCandCap) s_cand[pos] = topk_key(expf(q - c_max) / c_sum, v);
+      }
+    }
+    __syncthreads();
+    exact = s_count > kSelCandCap;
+  }
+  float* out_p = cand_p + (size_t)col * K;
+  int* out_w = cand_w + (size_t)col * K;
+  if (exact) {
+    // K passes over the column: the largest key below the previous pass's
+    unsigned long long prev = ~0ull;
+    for (int r = 0; r < K; ++r) {
+      unsigned long long best = 0ull;
+      for (int v = tid; v < V; v += 256) {
+        const float q = x[v];
+        const unsigned long long key = q > -INFINITY ? topk_key(expf(q - c_max) / c_sum, v) : 0ull;
+        best = (key < prev && key > best) ? key : best;
+      }
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) {
+        const unsigned long long o = __shfl_xor(best, off, 64);
+        best = o > best ? o : best;
+      }
+      __syncthreads();  // (s_best of the previous pass has been read)
+      if (lane == 0) s_best[wave] = best;
+      __syncthreads();
+      best = s_best[0];
+#pragma unroll
+      for (int w = 1; w < 4; ++w) best = s_best[w] > best ? s_best[w] : best;
+      if (tid == 0) topk_unkey(best, out_p[r], out_w[r]);  // key 0 (nothing left): the filler (-inf, 0x7fffffff)
+      prev = best != 0ull ? best : 0ull;
+    }
+    return;
+  }
+  const int n = s_count;
+  for (int a = tid; a < n; a += 256) {
+    const unsigned long long ka = s_cand[a];
+    int rank = 0;
+#pragma unroll 8
+    for (int b = 0; b < n; ++b) rank += s_cand[b] > ka ? 1 : 0;
+    if (rank < K) topk_unkey(ka, out_p[rank], out_w[rank]);
+  }
+  if (tid < K && tid >= n) {  // fewer than K words in the column
+    out_p[tid] = -INFINITY;
+    out_w[tid] = 0x7fffffff;
   }
 }
 
@@ -584,6 +728,7 @@ int zr_beam_create(zr_ctx* ctx, int beam, int vocab, int n_sent, int max_len, fl
   const size_t o_cp = take(nb * K * 4), o_cw = take(nb * K * 4);
   const size_t n_chunks = ((size_t)vocab + kTopkChunk - 1) / kTopkChunk;  // K-lists per column from the first stage
   const size_t o_pp = take(nb * n_chunks * K * 4), o_pw = take(nb * n_chunks * K * 4);
+  const size_t o_cs = take(nb * 2 * 4);
   char* base = nullptr;
   if (hipMalloc((void**)&base, off) != hipSuccess) {
     (void)hipGetLastError();
@@ -608,6 +753,7 @@ int zr_beam_create(zr_ctx* ctx, int beam, int vocab, int n_sent, int max_len, fl
   b->d_cand_w = (int*)(base + o_cw);
   b->d_part_p = (float*)(base + o_pp);
   b->d_part_w = (int*)(base + o_pw);
+  b->d_colstats = (float*)(base + o_cs);
   *out = b;
   return zr_beam_init(ctx, b);
 }
@@ -634,27 +780,35 @@ int zr_beam_init(zr_ctx* ctx, zr_beam* b) {
 }
 
 // d_colstats null: d_values are probabilities; otherwise logits with their column statistics
+// d_blocks: the values are logits with their per-block pairs behind them (one fused selection launch)
 static int beam_expand_impl(zr_ctx* ctx, const char* who, zr_beam* b, const float* d_values, const float* d_colstats,
-                            int index, int* d_words, int* d_backptr) {
+                            int index, int* d_words, int* d_backptr, const float* d_blocks = nullptr) {
   int rc = zr_bind_device(ctx);
   if (rc) return rc;
   ZR_CHECK_ARG(b && d_values && d_words && d_backptr, "%s: null pointer", who);
   ZR_CHECK_ARG(index >= 0, "%s: index = %d", who, index);
   ZR_CHECK_ARG(b->current_index + 2 < b->max_len, "%s: hypotheses reached max_len = %d", who, b->max_len);
   const int K = b->beam + 1;
-  const int e4 = topk_e4_for(b->vocab);
-  const int n_chunks = (b->vocab + topk_chunk(e4) - 1) / topk_chunk(e4);
-  dim3 tgrid(n_chunks, b->n_sent * b->beam);
-  if (e4 == kTopkE4Small)
-    beam_topk_kernel<kTopkE4Small><<<tgrid, 256, 0, ctx->stream>>>(d_values, b->vocab, K, n_chunks, b->d_part_p, b->d_part_w,
-                                                                   d_colstats);
-  else
-    beam_topk_kernel<kTopkE4Large><<<tgrid, 256, 0, ctx->stream>>>(d_values, b->vocab, K, n_chunks, b->d_part_p, b->d_part_w,
-                                                                   d_colstats);
-  ZR_LAUNCH_CHECK("beam_topk_kernel");
-  beam_topk_merge_kernel<<<b->n_sent * b->beam, 256, 0, ctx->stream>>>(b->d_part_p, b->d_part_w, K, n_chunks,
-                                                                       b->d_cand_p, b->d_cand_w);
-  ZR_LAUNCH_CHECK("beam_topk_merge_kernel");
+  if (d_blocks) {
+    beam_select_blocks_kernel<<<b->n_sent * b->beam, 256, 0, ctx->stream>>>(d_values, d_blocks, b->vocab, K,
+                                                                            zr_softmax_partial_blocks(b->vocab),
+                                                                            b->d_cand_p, b->d_cand_w, b->d_colstats);
+    ZR_LAUNCH_CHECK("beam_select_blocks_kernel");
+  } else {
+    const int e4 = topk_e4_for(b->vocab);
+    const int n_chunks = (b->vocab + topk_chunk(e4) - 1) / topk_chunk(e4);
+    dim3 tgrid(n_chunks, b->n_sent * b->beam);
+    if (e4 == kTopkE4Small)
+      beam_topk_kernel<kTopkE4Small><<<tgrid, 256, 0, ctx->stream>>>(d_values, b->vocab, K, n_chunks, b->d_part_p,
+                                                                     b->d_part_w, d_colstats);
+    else
+      beam_topk_kernel<kTopkE4Large><<<tgrid, 256, 0, ctx->stream>>>(d_values, b->vocab, K, n_chunks, b->d_part_p,
+                                                                     b->d_part_w, d_colstats);
+    ZR_LAUNCH_CHECK("beam_topk_kernel");
+    beam_topk_merge_kernel<<<b->n_sent * b->beam, 256, 0, ctx->stream>>>(b->d_part_p, b->d_part_w, K, n_chunks,
+                                                                         b->d_cand_p, b->d_cand_w);
+    ZR_LAUNCH_CHECK("beam_topk_merge_kernel");
+  }
   beam_merge_kernel<<<b->n_sent, 256, 0, ctx->stream>>>(b->beam, K, b->max_len, b->hyp_cap, b->penalty, index,
                                                         b->current_index, b->d_cand_p, b->d_cand_w, b->d_scores,
                                                         b->d_words, b->d_sent, b->d_sent_tmp,
@@ -706,6 +860,21 @@ int zr_beam_finish(zr_ctx* ctx, zr_beam* b, const float* d_prob) {
 int zr_beam_finish_logits(zr_ctx* ctx, zr_beam* b, const float* d_logits, const float* d_colstats) {
   ZR_CHECK_ARG(d_colstats != nullptr, "zr_beam_finish_logits: d_colstats is null");
   return beam_finish_impl(ctx, "zr_beam_finish_logits", b, d_logits, d_colstats);
+}
+
+int zr_beam_expand_blocks(zr_ctx* ctx, zr_beam* b, const float* d_logits, const float* d_blocks, int index,
+                          int* d_words, int* d_backptr) {
+  ZR_CHECK_ARG(d_blocks != nullptr, "zr_beam_expand_blocks: d_blocks is null");
+  return beam_expand_impl(ctx, "zr_beam_expand_blocks", b, d_logits, nullptr, index, d_words, d_backptr, d_blocks);
+}
+
+int zr_beam_finish_blocks(zr_ctx* ctx, zr_beam* b, const float* d_logits, const float* d_blocks) {
+  int rc = zr_bind_device(ctx);
+  if (rc) return rc;
+  ZR_CHECK_ARG(b && d_logits && d_blocks, "zr_beam_finish_blocks: null pointer");
+  rc = zr_softmax_colstats_launch(ctx, d_blocks, zr_softmax_partial_blocks(b->vocab), b->n_sent * b->beam, b->d_colstats);
+  if (rc) return rc;
+  return beam_finish_impl(ctx, "zr_beam_finish_blocks", b, d_logits, b->d_colstats);
 }
 
 int zr_beam_hypotheses(zr_ctx* ctx, zr_beam* b, int sentence, int cap, int* h_words, int* h_len, float* h_score) {

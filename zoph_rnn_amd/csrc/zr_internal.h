@@ -175,6 +175,10 @@ int zr_pack8_bf16_launch(zr_ctx* ctx, const float* src, int M, int K, long long 
                          unsigned short* dst, int trans = 0);
 // number of 32-row partial blocks the SOFTMAX_PARTIAL epilogue writes for M rows
 static inline int zr_softmax_partial_blocks(int M) { return (M + 31) / 32; }
+// ZR_SOFTMAX_LOGITS_BLOCKS: where the block pairs start in d_out (floats; a multiple of 4 behind the V x cols logits)
+static inline size_t zr_softmax_blocks_offset_floats(int V, int cols) { return ((size_t)V * cols + 3) & ~(size_t)3; }
+// softmax_colstats_kernel on [cols][nblocks][2] pairs -> colstats[cols][2] (zr_softmax.hip)
+int zr_softmax_colstats_launch(zr_ctx* ctx, const float* d_partials, int nblocks, int cols, float* d_colstats);
 
 struct zr_lstm_weights {
   int H;

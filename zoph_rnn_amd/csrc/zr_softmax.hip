@@ -3,59 +3,19 @@
 #include <math.h>
 
 #include "zr_internal.h"
+#include "zr_softmax_fold.h"
 
 namespace {
 
 // Folds the per-32-row partials of one column ([N][nblocks][2] floats: contiguous per column, nblocks
-// (max, sum exp(x - max)) pairs) into the column's (max, sum).  One workgroup per column; every thread folds its pairs
-// into one running pair -- eight loads at a time, all in flight together -- then the threads' pairs are folded
-// across the wave and the four waves, always in the same order.
-__device__ __forceinline__ void softmax_fold(float& m, float& sm, float pm, float ps) {
-  const float mn = fmaxf(m, pm);
-  sm = (m == mn ? sm : sm * expf(m - mn)) + (pm == mn ? ps : ps * expf(pm - mn));
-  m = mn;
-}
-
+// (max, sum exp(x - max)) pairs) into the column's (max, sum).  One workgroup per column (zr_softmax_fold.h).
 __global__ void __launch_bounds__(256)
 softmax_colstats_kernel(const float* __restrict__ partials, int nblocks, float* __restrict__ colstats) {
-  typedef float zr_f32x2 __attribute__((ext_vector_type(2)));
   __shared__ float s_m[4], s_s[4];
   const int n = blockIdx.x;
-  const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
-  const zr_f32x2* pp = (const zr_f32x2*)(partials + (size_t)n * nblocks * 2);
-  float mx = -INFINITY, sum = 0.0f;
-  for (int b0 = 0; b0 < nblocks; b0 += 2048) {
-    zr_f32x2 pr[8];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int b = b0 + tid + 256 * u;
-      pr[u] = zr_f32x2{-INFINITY, 0.0f};
-      if (b < nblocks) pr[u] = pp[b];
-    }
-#pragma unroll
-    for (int u = 0; u < 8; ++u) softmax_fold(mx, sum, pr[u].x, pr[u].y);
-  }
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    const float om = __shfl_xor(mx, off, 64), os = __shfl_xor(sum, off, 64);
-    // both partners add in the same order, so every lane ends with the same bits
-    float a_m = (lane & off) ? om : mx, a_s = (lane & off) ? os : sum;
-    const float b_m = (lane & off) ? mx : om, b_s = (lane & off) ? sum : os;
-    softmax_fold(a_m, a_s, b_m, b_s);
-    mx = a_m;
-    sum = a_s;
-  }
-  if (lane == 0) {
-    s_m[wave] = mx;
-    s_s[wave] = sum;
-  }
-  __syncthreads();
-  if (tid == 0) {
-    mx = s_m[0];
-    sum = s_s[0];
-#pragma unroll
-    for (int w = 1; w < 4; ++w) softmax_fold(mx, sum, s_m[w], s_s[w]);
+  float mx, sum;
+  zr_softmax_fold_column(partials + (size_t)n * nblocks * 2, nblocks, s_m, s_s, mx, sum, nullptr);
+  if (threadIdx.x == 0) {
     colstats[2 * n] = mx;
     colstats[2 * n + 1] = sum;
   }
@@ -166,15 +126,21 @@ softmax_loss_kernel(const float* __restrict__ logits, int V, int mb, const doubl
 
 // d_h_packed: optional k-interleaved copy of d_h ([H/4][mb][4]); used when the product runs on the registered fp32 copy
 // of D and H % 8 == 0 (the product then skips its own re-layout of d_h).
+// d_partials_ext: where the [mb][nblocks][2] pairs go instead of context scratch (ZR_SOFTMAX_LOGITS_BLOCKS: the caller's
+// buffer; no column statistics follow them there).
 int logits_with_partials(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h, int mb,
                          float* d_logits, float** partials_out, int* nblocks_out, const float* d_h_packed = nullptr,
-                         const unsigned short* d_h_hi = nullptr, const unsigned short* d_h_lo = nullptr) {
+                         const unsigned short* d_h_hi = nullptr, const unsigned short* d_h_lo = nullptr,
+                         float* d_partials_ext = nullptr) {
   const int nblocks = zr_softmax_partial_blocks(V);
-  void* scratch = nullptr;
-  // partials [mb][nblocks][2] followed by column stats (2 doubles per column, also used as 2 floats)
-  const size_t pbytes = sizeof(float) * 2 * (size_t)nblocks * mb;
-  int rc = zr_ctx_scratch(ctx, 1, pbytes + sizeof(double) * 2 * (size_t)mb + 64, &scratch);
-  if (rc) return rc;
+  void* scratch = d_partials_ext;
+  int rc = ZR_OK;
+  if (!scratch) {
+    // partials [mb][nblocks][2] followed by column stats (2 doubles per column, also used as 2 floats)
+    const size_t pbytes = sizeof(float) * 2 * (size_t)nblocks * mb;
+    rc = zr_ctx_scratch(ctx, 1, pbytes + sizeof(double) * 2 * (size_t)mb + 64, &scratch);
+    if (rc) return rc;
+  }
   ZrGemmDesc d = {};
   d.M = V;
   d.N = mb;
@@ -304,7 +270,19 @@ int zr_softmax_forward(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V,
   return zr_softmax_forward_packed(ctx, d_D, d_b_d, V, H, d_h, nullptr, mb, mode, d_out, d_logits_scratch);
 }
 
+int zr_softmax_block_count(int V) { return V > 0 ? zr_softmax_partial_blocks(V) : 0; }
+
+long long zr_softmax_blocks_offset(int V, int cols) {
+  return (V > 0 && cols > 0) ? (long long)zr_softmax_blocks_offset_floats(V, cols) : 0;
+}
+
 }  // extern "C"
+
+int zr_softmax_colstats_launch(zr_ctx* ctx, const float* d_partials, int nblocks, int cols, float* d_colstats) {
+  softmax_colstats_kernel<<<cols, 256, 0, ctx->stream>>>(d_partials, nblocks, d_colstats);
+  ZR_LAUNCH_CHECK("softmax_colstats_kernel");
+  return ZR_OK;
+}
 
 int zr_softmax_forward_packed(zr_ctx* ctx, const float* d_D, const float* d_b_d, int V, int H, const float* d_h,
                               const float* d_h_packed, int mb, int mode, float* d_out, float* d_logits_scratch,
@@ -314,16 +292,22 @@ int zr_softmax_forward_packed(zr_ctx* ctx, const float* d_D, const float* d_b_d,
   rc = check_softmax_args("zr_softmax_forward", d_D, d_b_d, V, H, d_h, mb);
   if (rc) return rc;
   ZR_CHECK_ARG(d_out != nullptr, "zr_softmax_forward: d_out is null");
-  ZR_CHECK_ARG(mode == ZR_SOFTMAX_PROB || mode == ZR_SOFTMAX_LOGPROB || mode == ZR_SOFTMAX_LOGITS,
+  ZR_CHECK_ARG(mode == ZR_SOFTMAX_PROB || mode == ZR_SOFTMAX_LOGPROB || mode == ZR_SOFTMAX_LOGITS ||
+                   mode == ZR_SOFTMAX_LOGITS_BLOCKS,
                "zr_softmax_forward: mode = %d", mode);
-  const bool logits_only = mode == ZR_SOFTMAX_LOGITS;
+  const bool with_blocks = mode == ZR_SOFTMAX_LOGITS_BLOCKS;
+  const bool logits_only = mode == ZR_SOFTMAX_LOGITS || with_blocks;
   ZR_CHECK_ARG(!logits_only || d_logits_scratch == nullptr,
-               "zr_softmax_forward: ZR_SOFTMAX_LOGITS writes the logits to d_out and takes no d_logits_scratch");
+               "zr_softmax_forward: ZR_SOFTMAX_LOGITS(_BLOCKS) writes the logits to d_out and takes no d_logits_scratch");
   float* logits = (d_logits_scratch && !logits_only) ? d_logits_scratch : d_out;
   float* partials = nullptr;
   int nblocks = 0;
-  rc = logits_with_partials(ctx, d_D, d_b_d, V, H, d_h, mb, logits, &partials, &nblocks, d_h_packed, d_h_hi, d_h_lo);
+  // ZR_SOFTMAX_LOGITS_BLOCKS: the product's per-block pairs go straight into the caller's buffer behind the logits and
+  // that is all -- no launch folds them; the consumer (zr_beam_expand_blocks) does that itself
+  rc = logits_with_partials(ctx, d_D, d_b_d, V, H, d_h, mb, logits, &partials, &nblocks, d_h_packed, d_h_hi, d_h_lo,
+                            with_blocks ? d_out + zr_softmax_blocks_offset_floats(V, mb) : nullptr);
   if (rc) return rc;
+  if (with_blocks) return ZR_OK;
   // ZR_SOFTMAX_LOGITS: the column statistics go behind the logits in the caller's buffer and no normalised matrix is
   // written -- a consumer that needs only a few entries per column (the beam search) normalises those itself
   float* colstats = logits_only ? d_out + (size_t)V * mb : (float*)stats_ptr(partials, nblocks, mb);

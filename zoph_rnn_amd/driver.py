@@ -60,10 +60,13 @@ class BeamDecode:
         self.c = [[ctx.empty((H, cols)) for _ in range(L)] for _ in range(2)]
         self.h_tild = [ctx.empty((H, cols)) for _ in range(2)]
         self.x = ctx.empty((H, cols))
-        # the logits and, behind them, two statistics per column (ZR_SOFTMAX_LOGITS): the beam normalises only the
-        # entries it selects, so no probability matrix is written or read
-        self.logits = ctx.empty((w.Vt * cols + 2 * cols,))
-        self.colstats = self.logits.at(w.Vt * cols)
+        # the logits and, behind them, the output product's (max, sum exp) pair per 32-row block and column
+        # (ZR_SOFTMAX_LOGITS_BLOCKS): the beam folds the pairs itself, reads only the blocks that can hold one of a
+        # column's beam + 1 largest entries and normalises only what it selects -- no probability matrix is written,
+        # and the logits are not read again as a whole
+        off = capi.softmax_blocks_offset(w.Vt, cols)
+        self.logits = ctx.empty((off + 2 * capi.softmax_block_count(w.Vt) * cols,))
+        self.blocks = self.logits.at(off)
         self.d_words = ctx.array(np.zeros(cols, np.int32))  # <START> = 0
         self.d_words_nn = ctx.array(np.zeros(cols, np.int32))
         ctx.beam_set_input_ids(self.bm, self.d_words_nn)
@@ -99,7 +102,7 @@ class BeamDecode:
         self._enc_keep = (h_all, c_all, d_nn, d_m, z, rep)
 
     def _forward(self):
-        """forward_prop_target (src/model.hpp:2573-2688): new state into the other ping-pong half, logits and column statistics."""
+        """forward_prop_target (src/model.hpp:2573-2688): new state into the other ping-pong half, logits and their per-block pairs."""
         ctx, w, cols = self.ctx, self.w, self.cols
         H, L = w.H, w.L
         p, q = self.cur, 1 - self.cur
@@ -107,14 +110,14 @@ class BeamDecode:
         feed = self.h_tild[p] if self.step_index > 0 else None
         ctx.decoder_step(w.tgt, w.tgt_embed, w.Vt, self.d_words_nn, self.h[p], self.c[p], self.d_ones, cols, self.h[q],
                          self.c[q], self.attn, self.d_batch_info, self.h_tild[q], w.D_soft, w.b_soft, w.Vt,
-                         capi.ZR_SOFTMAX_LOGITS, self.logits, d_htild_prev=feed)
+                         capi.ZR_SOFTMAX_LOGITS_BLOCKS, self.logits, d_htild_prev=feed)
 
     def step(self, record=False):
         """One decode step: forward, expand the beam, reorder the states by the back-pointers."""
         ctx, w, cols = self.ctx, self.w, self.cols
         H, L = w.H, w.L
         self._forward()
-        ctx.beam_expand_logits(self.bm, self.logits, self.colstats, self.step_index, self.d_words, self.d_back)
+        ctx.beam_expand_blocks(self.bm, self.logits, self.blocks, self.step_index, self.d_words, self.d_back)
         # swap_decoding_states + target_copy_prev_states (src/model.hpp:2691-2726): the new state, permuted, becomes
         # the previous state of the next step
         p, q = self.cur, 1 - self.cur
@@ -128,7 +131,7 @@ class BeamDecode:
     def finish(self):
         """Last forward step and forced <EOF> on every live hypothesis (src/ensemble_factory.hpp:727-743)."""
         self._forward()
-        self.ctx.beam_finish_logits(self.bm, self.logits, self.colstats)
+        self.ctx.beam_finish_blocks(self.bm, self.logits, self.blocks)
         self.ctx.sync()
 
     def hypotheses(self, sentence, cap=256):

@@ -1006,8 +1006,10 @@ class beam_decoder {
       h_tild[i] = dmalloc<dType>(n);
     }
     x = dmalloc<dType>(n);
-    // logits, then two statistics per column (ZR_SOFTMAX_LOGITS): the beam normalises only what it selects
-    logits = dmalloc<dType>((size_t)Vt * cols + 2 * (size_t)cols);
+    // logits, then the output product's (max, sum exp) pair per 32-row block and column (ZR_SOFTMAX_LOGITS_BLOCKS): the
+    // beam folds the pairs, reads only the blocks that can hold one of a column's beam + 1 largest entries and
+    // normalises only what it selects (a member of an ensemble writes V x cols probabilities there instead)
+    logits = dmalloc<dType>((size_t)zr_softmax_blocks_offset(Vt, cols) + 2 * (size_t)zr_softmax_block_count(Vt) * cols);
     zeros = dmalloc<dType>((size_t)H * n_sent);
     ZOPH_CALL(zr_memset_zero(ctx, zeros, (size_t)H * n_sent * sizeof(dType)));
     for (int l = 0; l < L; l++) {
@@ -1054,10 +1056,10 @@ class beam_decoder {
   }
 
   // An ensemble member hands its output distribution on as probabilities (they are averaged over the models before the
-  // beam sees them); a decoder on its own leaves logits and column statistics for the beam to normalise what it picks.
+  // beam sees them); a decoder on its own leaves logits and their per-block pairs for the beam to select from and normalise what it picks.
   bool prob_mode = false;
 
-  // forward_prop_target (src/model.hpp:2573-2688): state half p -> half q, logits and column statistics into logits
+  // forward_prop_target (src/model.hpp:2573-2688): state half p -> half q, logits and their per-block pairs into logits
   void forward_target(int p, int step_index) {
     const int q = 1 - p;
     // (d_words_nn, the input ids, are written by the beam call that chose the words: zr_beam_set_input_ids)
@@ -1068,7 +1070,7 @@ class beam_decoder {
     ZOPH_CALL(zr_decoder_step(ctx, L, tgt_w.data(), m.input_layer_target.d_W, Vt, d_words_nn, hp.data(), cp.data(), feed,
                               d_ones, 0.0f, cols, h[q].data(), c[q].data(), attention ? attn : nullptr, d_batch_info,
                               attention ? h_tild[q] : nullptr, d_align, d_align_idx, nullptr, nullptr, m.softmax_obj.d_D,
-                              m.softmax_obj.d_b_d, Vt, prob_mode ? ZR_SOFTMAX_PROB : ZR_SOFTMAX_LOGITS, logits));
+                              m.softmax_obj.d_b_d, Vt, prob_mode ? ZR_SOFTMAX_PROB : ZR_SOFTMAX_LOGITS_BLOCKS, logits));
     // The alignment of every column, read by the beam call that follows.  The reference's driver passes every step
     // through ensembles_models, also with one model, and that overwrites the attention layer's own Viterbi alignment
     // (get_viterbi_alignment_kernel) with the vote over the window weights (src/ensemble_factory.hpp:797-834): the same
@@ -1202,13 +1204,13 @@ class beam_decoder {
       // step, and every 32 steps after that -- a launch that gives up takes about a second per step)
       if (index % 32 == 0 && launches_abandoned()) again = true;
       if (again) break;
-      ZOPH_CALL(zr_beam_expand_logits(ctx, bm, logits, logits + (size_t)Vt * cols, index, d_words, d_back));
+      ZOPH_CALL(zr_beam_expand_blocks(ctx, bm, logits, logits + zr_softmax_blocks_offset(Vt, cols), index, d_words, d_back));
       reorder_states(p, d_back);
     }
     if (!again) {
       // one last step and forced <EOF> on every live hypothesis (src/ensemble_factory.hpp:727-743)
       forward_target(p, index);
-      ZOPH_CALL(zr_beam_finish_logits(ctx, bm, logits, logits + (size_t)Vt * cols));
+      ZOPH_CALL(zr_beam_finish_blocks(ctx, bm, logits, logits + zr_softmax_blocks_offset(Vt, cols)));
       again = launches_abandoned();
     }
     if (again) {  // the batch is decoded again with one launch per node (launches_abandoned has switched the context over)
