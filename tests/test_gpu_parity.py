@@ -477,7 +477,8 @@ def test_attention_against_oracle(ctx, H, mb, S, D, prepared):
 
 
 @pytest.mark.parametrize("H,mb,S,D", [(1000, 128, 50, 50), (64, 6, 9, 2), (200, 70, 40, 10), (1024, 33, 64, 31),
-                                      (512, 12, 21, 10), (96, 1, 5, 7), (1000, 12, 50, 10), (1000, 1, 50, 10)])
+                                      (512, 12, 21, 10), (96, 1, 5, 7), (1000, 12, 50, 10), (1000, 1, 50, 10),
+                                      (1000, 192, 30, 10), (256, 250, 20, 5)])
 def test_attention_step_in_one_launch(ctx, H, mb, S, D):
     """The attention step as one launch (projections, per-column middle and output product handing over through device
     memory): against the oracle, against the three-launch schedule on the same inputs, and twice in a row on one
