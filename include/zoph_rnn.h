@@ -321,9 +321,11 @@ int zr_attn_use_bf16_weights(zr_ctx* ctx, zr_attn* a);
 /* Optional preparation for repeated use (no counterpart in the reference, which hands d_W_p, d_W_a, d_W_c_p1 and
  * d_W_c_p2 to cublasSgemm as they are, src/attention_node.hpp:132,195,354,360): snapshots the four matrices in the
  * layout the matrix cores read fastest (W_a transposed; 4*H*H*4 more bytes).  Later zr_attn_step calls then run as
- * three launches -- both projections of h_t as one batch, one kernel for p_t, window, scores, alignment weights and
- * context that reads each valid source state from memory once, and the output product -- instead of eight.  Results
- * agree with the unprepared path to rounding (different summation order).  Call again after changing the matrices. */
+ * one launch whose workgroups hand the projections and the contexts over through device memory (fp32, H % 8 == 0,
+ * 32 <= H <= 1024, at most 64 window slots, the context's own stream: ZR_OPT_ATTN_SINGLE_LAUNCH), otherwise as three --
+ * both projections of h_t as one batch, one kernel for p_t, window, scores, alignment weights and context that reads
+ * each valid source state from memory once, and the output product -- instead of eight.  Results agree with the
+ * unprepared path to rounding (different summation order).  Call again after changing the matrices. */
 int zr_attn_prepare(zr_ctx* ctx, zr_attn* a);
 int zr_attn_destroy(zr_ctx* ctx, zr_attn* a);
 /* attention_node::forward_prop (src/attention_node.hpp:73-394), single-source branch: p_t, window, scores

@@ -1643,12 +1643,11 @@ int zr_lstm_decoder_step_packed(zr_ctx* ctx, int nl, const zr_lstm_weights* cons
     const int j_tiles = (H + 31) / 32;
     const int padded = (j_tiles + 7) / 8 * 8;
     const int cap = stack_step_capacity(ctx);
-    // 32-column tiles while two workgroups per tile fit on the device together, 64-column tiles beyond that (192 columns
-    // of H = 1000: 384 workgroups against 192)
-    // (or, between the two: 32-column tiles whose role-1 work of the UPPER layers goes to as many helper workgroups
-    // as still fit, several tiles each, while a role-0 workgroup computes the independent products of the lower layers
-    // itself -- at 192 columns 192 chains and 64 helpers of three tiles x two layers fill the 256 compute units that 192
-    // workgroups on 64-column tiles leave a quarter of idle)
+    // 32-column tiles while two workgroups per tile fit on the device together; beyond that, while the 32-column tiles
+    // alone still fit, 32-column tiles whose role-1 work of the UPPER layers goes to as many helper workgroups as still
+    // fit, several tiles each, while a role-0 workgroup computes the independent products of the lower layers itself
+    // (192 columns of H = 1000: 192 chains and 64 helpers of three tiles x two layers fill the 256 compute units);
+    // else 64-column tiles in pairs
     const int slots1 = padded * ((mb + 31) / 32);
     int tn = (2LL * slots1 <= cap) ? 1 : 2;
     int helpers = 0, l_split = 0;
