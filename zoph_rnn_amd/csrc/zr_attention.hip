@@ -173,7 +173,7 @@ attn_context_kernel(const float* const* __restrict__ table, int longest_sent, co
 }
 
 // The four consecutive rows 4*k4 .. 4*k4+3 of column b as bf16 terms, into arrays laid out [H/8][mb][8] (what the bf16
-// products read: zr_split_pack_x_kernel's layout and its hi / lo split).  lo may be null (single-term mode).
+// products read: zr_split_pack_multi_kernel's layout and its hi / lo split).  lo may be null (single-term mode).
 __device__ __forceinline__ void store_bf16_terms(const zr_f32x4& v, int k4, int b, int mb, unsigned short* hi,
                                                  unsigned short* lo) {
   typedef unsigned zr_u32x2 __attribute__((ext_vector_type(2)));

@@ -27,7 +27,7 @@ struct GemmArgs {
   int m_tiles, n_tiles;  // wave tiles along M and N
   int b_pack4;           // B segments are k-interleaved copies: element (k, n) at ((k/4)*N + n)*4 + k%4
   // bf16 weights: B[s] is the bf16 "hi" array and Blo[s] the "lo" array of the split activations, both
-  // k-interleaved by 8 ([K/8][N][8]); see zr_split_pack_x_kernel
+  // k-interleaved by 8 ([K/8][N][8]); see zr_split_pack_multi_kernel
   const unsigned short* Blo[3];
   int accum;  // ZR_EPI_STORE only: C += result instead of C = result
   int stream_a;  // the weights are fetched with the streaming hint (ZrGemmDesc::stream_a)
@@ -557,7 +557,7 @@ __device__ __forceinline__ void softmax_partial_epilogue_t(const GemmArgs& a, co
 // n_main); every 64-row block left over goes to one further workgroup whose four waves split the columns instead
 // (the same staging; the weights of those few blocks are fetched by four waves each).
 // ---------------------------------------------------------------------------------------------------------
-// LO: two-term mode -- the activations come as two bf16 arrays (hi and lo, see zr_split_pack_x_kernel) and every weight
+// LO: two-term mode -- the activations come as two bf16 arrays (hi and lo, see zr_split_pack_multi_kernel) and every weight
 // operand is multiplied with both (a chunk then holds CG k-groups of each term).
 // PD: how many chunks ahead the weight fetches run (a ring of PD + 1 register sets; 1 with the LDS double buffer).
 template <int TM, int TNW, int NB, int CG, bool LO, int PD>
@@ -1041,32 +1041,16 @@ bool launch_tall(zr_ctx* ctx, GemmArgs& ga, int epi, int* rc) {
 }
 
 // Activations X (K x N fp32, column n at src + n*ld, K % 8 == 0) -> two bf16 arrays hi and lo with x = hi + lo up
-// to 2^-16 |x|, each k-interleaved by 8: element (k, n) at ((k/8)*N + n)*8 + k%8.  One thread per 8 values.
-__global__ void __launch_bounds__(256) zr_split_pack_x_kernel(const float* __restrict__ src, int K, int N, int ld,
-                                                              unsigned short* __restrict__ hi,
-                                                              unsigned short* __restrict__ lo) {
-  const int i = blockIdx.x * 256 + threadIdx.x;
-  const int kb = K >> 3;
-  if (i >= kb * N) return;
-  const int n = i / kb, b = i - n * kb;
-  const zr_f32x4 v0 = *(const zr_f32x4*)(src + (long long)n * ld + 8 * b);
-  const zr_f32x4 v1 = *(const zr_f32x4*)(src + (long long)n * ld + 8 * b + 4);
-  zr_u32x4 h, l;
-  unsigned a, c;
-  zr_split_bf16_pair(v0.x, v0.y, a, c); h.x = a; l.x = c;
-  zr_split_bf16_pair(v0.z, v0.w, a, c); h.y = a; l.y = c;
-  zr_split_bf16_pair(v1.x, v1.y, a, c); h.z = a; l.z = c;
-  zr_split_bf16_pair(v1.z, v1.w, a, c); h.w = a; l.w = c;
-  const long long o = ((long long)b * N + n) * 8;
-  *(zr_u32x4*)(hi + o) = h;
-  if (lo) *(zr_u32x4*)(lo + o) = l;  // null: single-term mode, the residues are dropped
-}
-
-// The same for up to kSplitMultiMax matrices of one shape in one launch (blockIdx.y picks the matrix): a decoder step
-// splits the previous state of every layer, the previous attention output and the embedding columns of the current
-// words at its start, and each of them as a launch of its own costs more in launch latency than in work.  Matrix i goes
-// to hi + i*stride (lo + i*stride); ids (or null) turns matrix 0 into a gather, column n read from src[0] + ids[n]*ld
-// (ids outside [0, V) are clamped, as the gather kernel does).
+// to 2^-16 |x|, each k-interleaved by 8: element (k, n) at ((k/8)*N + n)*8 + k%8.
+// A workgroup takes 32 columns x 32 k-groups and turns them through LDS: it reads with 32 consecutive lanes on 32
+// consecutive k-groups of one column (1 KB contiguous) and writes with 32 consecutive lanes on 32 consecutive columns of
+// one k-group (512 bytes contiguous).  With one thread per k-group writing its 16 bytes where they belong, consecutive
+// lanes stored 16-byte pieces N*16 bytes apart: 11 us for the six 2000 x 256 arrays of a config-5 step.
+// Up to kSplitMultiMax matrices of one shape per launch (blockIdx.z picks the matrix): a decoder step splits the previous
+// state of every layer, the previous attention output and the embedding columns of the current words at its start, and
+// each of them as a launch of its own costs more in launch latency than in work.  Matrix i goes to hi + i*stride
+// (lo + i*stride); ids (or null) turns matrix 0 into a gather, column n read from src[0] + ids[n]*ld (ids outside
+// [0, V) are clamped, as the gather kernel does).
 constexpr int kSplitMultiMax = 12;
 struct SplitMulti {
   const float* src[kSplitMultiMax];
@@ -1076,28 +1060,46 @@ struct SplitMulti {
 __global__ void __launch_bounds__(256) zr_split_pack_multi_kernel(SplitMulti m, int K, int N, int ld,
                                                                   unsigned short* __restrict__ hi,
                                                                   unsigned short* __restrict__ lo, long long stride) {
-  const int i = blockIdx.x * 256 + threadIdx.x;
+  __shared__ zr_u32x4 s_hi[32][33], s_lo[32][33];  // [column][k-group], a row padded by one item
+  const int tid = threadIdx.x;
   const int kb = K >> 3;
-  if (i >= kb * N) return;
-  const int which = blockIdx.y;
-  const int n = i / kb, b = i - n * kb;
-  long long col = n;
-  if (which == 0 && m.ids) {
-    const int v = m.ids[n];
-    col = v < 0 ? 0 : (v >= m.V ? m.V - 1 : v);
+  const int b0 = blockIdx.x * 32, n0 = blockIdx.y * 32;
+  const int which = blockIdx.z;
+  const int lb = tid & 31;
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int c = u * 8 + (tid >> 5);
+    const int n = n0 + c, b = b0 + lb;
+    if (n < N && b < kb) {
+      long long col = n;
+      if (which == 0 && m.ids) {
+        const int v = m.ids[n];
+        col = v < 0 ? 0 : (v >= m.V ? m.V - 1 : v);
+      }
+      const float* src = m.src[which] + col * ld + 8 * b;
+      const zr_f32x4 v0 = *(const zr_f32x4*)src;
+      const zr_f32x4 v1 = *(const zr_f32x4*)(src + 4);
+      zr_u32x4 h, l;
+      unsigned x, y;
+      zr_split_bf16_pair(v0.x, v0.y, x, y); h.x = x; l.x = y;
+      zr_split_bf16_pair(v0.z, v0.w, x, y); h.y = x; l.y = y;
+      zr_split_bf16_pair(v1.x, v1.y, x, y); h.z = x; l.z = y;
+      zr_split_bf16_pair(v1.z, v1.w, x, y); h.w = x; l.w = y;
+      s_hi[c][lb] = h;
+      if (lo) s_lo[c][lb] = l;
+    }
   }
-  const float* src = m.src[which] + col * ld + 8 * b;
-  const zr_f32x4 v0 = *(const zr_f32x4*)src;
-  const zr_f32x4 v1 = *(const zr_f32x4*)(src + 4);
-  zr_u32x4 h, l;
-  unsigned a, c;
-  zr_split_bf16_pair(v0.x, v0.y, a, c); h.x = a; l.x = c;
-  zr_split_bf16_pair(v0.z, v0.w, a, c); h.y = a; l.y = c;
-  zr_split_bf16_pair(v1.x, v1.y, a, c); h.z = a; l.z = c;
-  zr_split_bf16_pair(v1.z, v1.w, a, c); h.w = a; l.w = c;
-  const long long o = which * stride + ((long long)b * N + n) * 8;
-  *(zr_u32x4*)(hi + o) = h;
-  if (lo) *(zr_u32x4*)(lo + o) = l;
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int bl = u * 8 + (tid >> 5);
+    const int n = n0 + lb, b = b0 + bl;
+    if (n < N && b < kb) {
+      const long long o = which * stride + ((long long)b * N + n) * 8;
+      *(zr_u32x4*)(hi + o) = s_hi[lb][bl];
+      if (lo) *(zr_u32x4*)(lo + o) = s_lo[lb][bl];  // null: single-term mode, the residues are dropped
+    }
+  }
 }
 
 __global__ void __launch_bounds__(256) pack4_kernel(const float* __restrict__ src, int M, int K, long long ld,
@@ -1145,14 +1147,6 @@ int zr_pack8_bf16_launch(zr_ctx* ctx, const float* src, int M, int K, long long 
   return ZR_OK;
 }
 
-int zr_split_pack_x_launch(zr_ctx* ctx, const float* src, int K, int N, int ld, unsigned short* hi,
-                           unsigned short* lo) {
-  const int n8 = (K / 8) * N;
-  zr_split_pack_x_kernel<<<(n8 + 255) / 256, 256, 0, ctx->stream>>>(src, K, N, ld, hi, lo);
-  ZR_LAUNCH_CHECK("zr_split_pack_x_kernel");
-  return ZR_OK;
-}
-
 int zr_split_pack_multi_launch(zr_ctx* ctx, int n_src, const float* const* srcs, const int* d_ids, int V, int K, int N,
                                int ld, unsigned short* hi, unsigned short* lo, long long stride) {
   if (n_src < 1 || n_src > kSplitMultiMax) return zr_set_error(ZR_EINVAL, "split: %d matrices in one launch", n_src);
@@ -1160,11 +1154,17 @@ int zr_split_pack_multi_launch(zr_ctx* ctx, int n_src, const float* const* srcs,
   for (int i = 0; i < n_src; ++i) m.src[i] = srcs[i];
   m.ids = d_ids;
   m.V = V;
-  const int n8 = (K / 8) * N;
-  zr_split_pack_multi_kernel<<<dim3((unsigned)((n8 + 255) / 256), (unsigned)n_src), 256, 0, ctx->stream>>>(m, K, N, ld, hi,
-                                                                                                          lo, stride);
+  const dim3 grid((unsigned)((K / 8 + 31) / 32), (unsigned)((N + 31) / 32), (unsigned)n_src);
+  if (grid.y > 65535) return zr_set_error(ZR_EINVAL, "split: %d columns", N);
+  zr_split_pack_multi_kernel<<<grid, 256, 0, ctx->stream>>>(m, K, N, ld, hi, lo, stride);
   ZR_LAUNCH_CHECK("zr_split_pack_multi_kernel");
   return ZR_OK;
+}
+
+int zr_split_pack_x_launch(zr_ctx* ctx, const float* src, int K, int N, int ld, unsigned short* hi,
+                           unsigned short* lo) {
+  const float* srcs[1] = {src};
+  return zr_split_pack_multi_launch(ctx, 1, srcs, nullptr, 0, K, N, ld, hi, lo, 0);
 }
 
 int zr_pack4_launch(zr_ctx* ctx, const float* src, int M, int K, long long ld, int ldp, int kp, float* dst) {
@@ -1287,16 +1287,14 @@ int zr_gemm_launch(zr_ctx* ctx, const ZrGemmDesc& d) {
       unsigned short* hi = (unsigned short*)p;
       for (int s = 0; s < d.nseg; ++s) {
         const size_t e = (size_t)d.K[s] * d.N;
-        const int n8 = (d.K[s] / 8) * d.N;
         const bool lo = !one_term;
         if (d.Bhi[s] && (one_term || d.Blo[s])) {  // the caller has split this segment already
           ga.B[s] = (const float*)d.Bhi[s];
           ga.Blo[s] = lo ? d.Blo[s] : nullptr;
           continue;
         }
-        zr_split_pack_x_kernel<<<(n8 + 255) / 256, 256, 0, ctx->stream>>>(d.B[s], d.K[s], d.N, d.ldb[s], hi,
-                                                                          lo ? hi + e : nullptr);
-        ZR_LAUNCH_CHECK("zr_split_pack_x_kernel");
+        rc = zr_split_pack_x_launch(ctx, d.B[s], d.K[s], d.N, d.ldb[s], hi, lo ? hi + e : nullptr);
+        if (rc) return rc;
         ga.B[s] = (const float*)hi;
         ga.Blo[s] = lo ? hi + e : nullptr;
         hi += 2 * e;

@@ -28,7 +28,7 @@ struct LstmUnit {
   float* hp;                // optional: h is also written packed as [H/4][mb][4] for the units that consume it
   unsigned short* hsplit_hi;  // optional: h is also written as bf16 terms, k-interleaved by 8 ([H/8][mb][8]), the layout
   unsigned short* hsplit_lo;  // products against bf16 weights read (hsplit_lo null: single term); same rounding as
-                              // zr_split_pack_x_kernel
+                              // zr_split_pack_multi_kernel
   const int* gather_ids;    // non-null: column n of segment 0 is in[0] + ids[n]*H (embedding gather)
   const float* cprev;
   const int* mask01;

@@ -503,7 +503,7 @@ __device__ __forceinline__ void zr_half_wave_softmax_stats(const float (&v)[G], 
 // the split.  Two bf16 instructions replace eight fp32 ones.
 //   woff[tm]:  8*row + 8*half*lda   (bf16 elements)
 //   xcol[tn]:  this lane's activation column advanced by 8*half
-// XPK: the activations were split and packed beforehand (zr_split_pack_x_kernel): two bf16 arrays hi and lo, each
+// XPK: the activations were split and packed beforehand (zr_split_pack_multi_kernel): two bf16 arrays hi and lo, each
 // k-interleaved like the weights ([K/8][N][8]); xcol[tn] / xlo[tn] then point at this lane's first block
 // (base + 8*(col + half*N)), xstride = N, and the loop body has no conversion arithmetic and only contiguous loads.
 // ---------------------------------------------------------------------------------------------------------
