@@ -1042,9 +1042,10 @@ bool launch_tall(zr_ctx* ctx, GemmArgs& ga, int epi, int* rc) {
 
 // Activations X (K x N fp32, column n at src + n*ld, K % 8 == 0) -> two bf16 arrays hi and lo with x = hi + lo up
 // to 2^-16 |x|, each k-interleaved by 8: element (k, n) at ((k/8)*N + n)*8 + k%8.
-// A workgroup takes 32 columns x 32 k-groups and turns them through LDS: it reads with 32 consecutive lanes on 32
-// consecutive k-groups of one column (1 KB contiguous) and writes with 32 consecutive lanes on 32 consecutive columns of
-// one k-group (512 bytes contiguous).  With one thread per k-group writing its 16 bytes where they belong, consecutive
+// A workgroup takes 16 columns x 16 k-groups, one per thread, and turns them through LDS: it reads with 16 consecutive
+// lanes on 16 consecutive k-groups of one column (512 bytes contiguous) and writes with 16 consecutive lanes on 16
+// consecutive columns of one k-group (256 bytes contiguous); small tiles, because a single 2000 x 256 array must still
+// spread over the chip (250 workgroups).  With one thread per k-group writing its 16 bytes where they belong, consecutive
 // lanes stored 16-byte pieces N*16 bytes apart: 11 us for the six 2000 x 256 arrays of a config-5 step.
 // Up to kSplitMultiMax matrices of one shape per launch (blockIdx.z picks the matrix): a decoder step splits the previous
 // state of every layer, the previous attention output and the embedding columns of the current words at its start, and
@@ -1060,16 +1061,14 @@ struct SplitMulti {
 __global__ void __launch_bounds__(256) zr_split_pack_multi_kernel(SplitMulti m, int K, int N, int ld,
                                                                   unsigned short* __restrict__ hi,
                                                                   unsigned short* __restrict__ lo, long long stride) {
-  __shared__ zr_u32x4 s_hi[32][33], s_lo[32][33];  // [column][k-group], a row padded by one item
+  __shared__ zr_u32x4 s_hi[16][17], s_lo[16][17];  // [column][k-group], a row padded by one item
   const int tid = threadIdx.x;
   const int kb = K >> 3;
-  const int b0 = blockIdx.x * 32, n0 = blockIdx.y * 32;
+  const int b0 = blockIdx.x * 16, n0 = blockIdx.y * 16;
   const int which = blockIdx.z;
-  const int lb = tid & 31;
-#pragma unroll
-  for (int u = 0; u < 4; ++u) {
-    const int c = u * 8 + (tid >> 5);
-    const int n = n0 + c, b = b0 + lb;
+  const int lx = tid & 15, ly = tid >> 4;
+  {
+    const int n = n0 + ly, b = b0 + lx;
     if (n < N && b < kb) {
       long long col = n;
       if (which == 0 && m.ids) {
@@ -1085,19 +1084,17 @@ __global__ void __launch_bounds__(256) zr_split_pack_multi_kernel(SplitMulti m, 
       zr_split_bf16_pair(v0.z, v0.w, x, y); h.y = x; l.y = y;
       zr_split_bf16_pair(v1.x, v1.y, x, y); h.z = x; l.z = y;
       zr_split_bf16_pair(v1.z, v1.w, x, y); h.w = x; l.w = y;
-      s_hi[c][lb] = h;
-      if (lo) s_lo[c][lb] = l;
+      s_hi[ly][lx] = h;
+      if (lo) s_lo[ly][lx] = l;
     }
   }
   __syncthreads();
-#pragma unroll
-  for (int u = 0; u < 4; ++u) {
-    const int bl = u * 8 + (tid >> 5);
-    const int n = n0 + lb, b = b0 + bl;
+  {
+    const int n = n0 + lx, b = b0 + ly;
     if (n < N && b < kb) {
       const long long o = which * stride + ((long long)b * N + n) * 8;
-      *(zr_u32x4*)(hi + o) = s_hi[lb][bl];
-      if (lo) *(zr_u32x4*)(lo + o) = s_lo[lb][bl];  // null: single-term mode, the residues are dropped
+      *(zr_u32x4*)(hi + o) = s_hi[lx][ly];
+      if (lo) *(zr_u32x4*)(lo + o) = s_lo[lx][ly];  // null: single-term mode, the residues are dropped
     }
   }
 }
@@ -1154,7 +1151,7 @@ int zr_split_pack_multi_launch(zr_ctx* ctx, int n_src, const float* const* srcs,
   for (int i = 0; i < n_src; ++i) m.src[i] = srcs[i];
   m.ids = d_ids;
   m.V = V;
-  const dim3 grid((unsigned)((K / 8 + 31) / 32), (unsigned)((N + 31) / 32), (unsigned)n_src);
+  const dim3 grid((unsigned)((K / 8 + 15) / 16), (unsigned)((N + 15) / 16), (unsigned)n_src);
   if (grid.y > 65535) return zr_set_error(ZR_EINVAL, "split: %d columns", N);
   zr_split_pack_multi_kernel<<<grid, 256, 0, ctx->stream>>>(m, K, N, ld, hi, lo, stride);
   ZR_LAUNCH_CHECK("zr_split_pack_multi_kernel");
